@@ -1,0 +1,248 @@
+/*
+ * TEST INFRASTRUCTURE ONLY -- never linked into, imported by, or called from the product.
+ *
+ * Thin driver around the reference's own CPU implementation.  It is compiled together with the
+ * reference sources where they lie (ggml.c, ggml-quants.c, ggml-alloc.c, ggml-backend.c) into
+ * oracle/_ref/libpi_ref.so by oracle/Makefile, only in a container that has the reference tree.
+ * It builds the same op sequence that llm_build_ffn_sparse emits on a CPU-only build
+ * (llama.cpp:4652-4757 with llm_build_sparse_mul_mat :4546 and llm_build_sparse_axpy :4599)
+ * and runs it through the reference executor (ggml_graph_compute, ggml.c:17380), plus a few
+ * single-op probes (dense mul_mat, norms, RoPE, softmax, Q4_0/Q8_0 codecs).
+ *
+ * Everything here is the reference's arithmetic; nothing is restated.  The fixtures under
+ * tests/golden/ were produced by calling these functions with n_threads = 1 (the reference's
+ * CPU AXPY merges per-thread partial sums without a lock, ggml.c:14433-14458).
+ */
+#include "ggml.h"
+
+#include <math.h>
+#include <stdint.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#define REF_API __attribute__((visibility("default")))
+
+static size_t tensor_bytes(enum ggml_type t, int64_t ne0, int64_t ne1) {
+    return (size_t)(ne0 / ggml_blck_size(t)) * ggml_type_size(t) * (size_t)ne1;
+}
+
+static struct ggml_context * new_ctx(size_t payload) {
+    struct ggml_init_params ip = { payload + (64u << 20), NULL, false };
+    return ggml_init(ip);
+}
+
+static struct ggml_tensor * put2d(struct ggml_context * ctx, enum ggml_type t, int64_t ne0, int64_t ne1, const void * src) {
+    struct ggml_tensor * x = ggml_new_tensor_2d(ctx, t, ne0, ne1);
+    if (src) memcpy(x->data, src, ggml_nbytes(x));
+    return x;
+}
+
+REF_API void ref_set_threshold(float thr) { sparse_pred_threshold = thr; }
+
+/*
+ * One sparse FFN block exactly as a CPU-only build of llama.cpp assembles it:
+ *   idx  = mul_mat(fc2, relu(mul_mat(fc1, x_pred)))
+ *   up   = mul_mat_idx(up_w,   x_ffn, idx, gpu_idx)
+ *   gate = mul_mat_idx(gate_w, x_ffn, idx, gpu_idx)        (omitted when has_gate == 0)
+ *   h    = relu(gate) * up            |  relu(up)
+ *   out  = axpy(down_t, h, idx, gpu_idx)
+ * wtype: 1 = F16, 2 = Q4_0 (applies to up/gate/down_t; fc1/fc2 are always F16).
+ * gpu_idx: int32[ff], 1 = "lives on the GPU, skip on the CPU".  All zero = everything computed.
+ * Any output pointer may be NULL.  Returns 0 on success.
+ */
+REF_API int ref_ffn_sparse(int d, int ff, int r, int T, int wtype, int has_gate,
+                           const void * up_w, const void * gate_w, const void * down_t,
+                           const uint16_t * fc1, const uint16_t * fc2,
+                           const float * x_ffn, const float * x_pred, const int32_t * gpu_idx,
+                           float threshold, int n_threads,
+                           float * logits, float * up_out, float * gate_out, float * h_out, float * out) {
+    enum ggml_type wt = (enum ggml_type) wtype;
+    size_t payload = 3 * tensor_bytes(wt, d, ff) + 2u * ((size_t)d * r + (size_t)r * ff)
+                   + (size_t)T * (2u * d + 8u * ff + 2u * r) * sizeof(float) + (size_t)ff * 4
+                   + (size_t)n_threads * d * 64 + (8u << 20);
+    struct ggml_context * ctx = new_ctx(payload);
+    if (!ctx) return 1;
+    sparse_pred_threshold = threshold;
+
+    struct ggml_tensor * t_up   = put2d(ctx, wt, d, ff, up_w);
+    struct ggml_tensor * t_gate = has_gate ? put2d(ctx, wt, d, ff, gate_w) : NULL;
+    struct ggml_tensor * t_down = put2d(ctx, wt, d, ff, down_t);
+    struct ggml_tensor * t_fc1  = put2d(ctx, GGML_TYPE_F16, d, r, fc1);
+    struct ggml_tensor * t_fc2  = put2d(ctx, GGML_TYPE_F16, r, ff, fc2);
+    struct ggml_tensor * t_x    = put2d(ctx, GGML_TYPE_F32, d, T, x_ffn);
+    struct ggml_tensor * t_xp   = put2d(ctx, GGML_TYPE_F32, d, T, x_pred);
+    struct ggml_tensor * t_gid  = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, ff);
+    memcpy(t_gid->data, gpu_idx, (size_t)ff * 4);
+
+    struct ggml_tensor * idx = ggml_mul_mat(ctx, t_fc1, t_xp);
+    idx = ggml_relu(ctx, idx);
+    idx = ggml_mul_mat(ctx, t_fc2, idx);
+
+    struct ggml_tensor * upo = ggml_mul_mat_idx(ctx, t_up, t_x, idx, t_gid);
+    struct ggml_tensor * gto = NULL;
+    struct ggml_tensor * cur;
+    if (has_gate) {
+        gto = ggml_mul_mat_idx(ctx, t_gate, t_x, idx, t_gid);
+        cur = ggml_mul(ctx, ggml_relu(ctx, gto), upo);
+    } else {
+        cur = ggml_relu(ctx, upo);
+    }
+    struct ggml_tensor * res = ggml_axpy(ctx, t_down, cur, idx, t_gid);
+
+    struct ggml_cgraph * gf = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, res);
+    ggml_graph_compute_with_ctx(ctx, gf, n_threads);
+
+    if (logits)          memcpy(logits,   idx->data, (size_t)ff * T * 4);
+    if (up_out)          memcpy(up_out,   upo->data, (size_t)ff * T * 4);
+    if (gate_out && gto) memcpy(gate_out, gto->data, (size_t)ff * T * 4);
+    if (h_out)           memcpy(h_out,    cur->data, (size_t)ff * T * 4);
+    if (out)             memcpy(out,      res->data, (size_t)d * T * 4);
+    ggml_free(ctx);
+    return 0;
+}
+
+/* dense ggml_mul_mat: W [cols, rows] of wtype (F32=0, F16=1, Q4_0=2), x F32 [cols, T] -> out F32 [rows, T] */
+REF_API int ref_mul_mat(int wtype, const void * w, int rows, int cols, const float * x, int T, int n_threads, float * out) {
+    enum ggml_type wt = (enum ggml_type) wtype;
+    struct ggml_context * ctx = new_ctx(tensor_bytes(wt, cols, rows) + (size_t)T * (cols + rows) * 8 + (4u << 20));
+    if (!ctx) return 1;
+    struct ggml_tensor * tw = put2d(ctx, wt, cols, rows, w);
+    struct ggml_tensor * tx = put2d(ctx, GGML_TYPE_F32, cols, T, x);
+    struct ggml_tensor * r  = ggml_mul_mat(ctx, tw, tx);
+    struct ggml_cgraph * gf = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, r);
+    ggml_graph_compute_with_ctx(ctx, gf, n_threads);
+    memcpy(out, r->data, (size_t)rows * T * 4);
+    ggml_free(ctx);
+    return 0;
+}
+
+/* kind 0 = rms_norm, 1 = norm (LayerNorm without affine); x [n, T] */
+REF_API int ref_norm(int kind, const float * x, int n, int T, float eps, float * out) {
+    struct ggml_context * ctx = new_ctx((size_t)n * T * 16 + (1u << 20));
+    if (!ctx) return 1;
+    struct ggml_tensor * tx = put2d(ctx, GGML_TYPE_F32, n, T, x);
+    struct ggml_tensor * r  = kind == 0 ? ggml_rms_norm(ctx, tx, eps) : ggml_norm(ctx, tx, eps);
+    struct ggml_cgraph * gf = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, r);
+    ggml_graph_compute_with_ctx(ctx, gf, 1);
+    memcpy(out, r->data, (size_t)n * T * 4);
+    ggml_free(ctx);
+    return 0;
+}
+
+/* ggml_rope_custom on x [n_embd_head, n_head, T] with positions pos[T]; mode 0 (LLaMA pairs) or 2 (NeoX) */
+REF_API int ref_rope(const float * x, int n_embd_head, int n_head, int T, const int32_t * pos, int n_dims, int mode,
+                     float freq_base, float freq_scale, float * out) {
+    size_t n = (size_t)n_embd_head * n_head * T;
+    struct ggml_context * ctx = new_ctx(n * 16 + (1u << 20));
+    if (!ctx) return 1;
+    struct ggml_tensor * tx = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, n_embd_head, n_head, T);
+    memcpy(tx->data, x, n * 4);
+    struct ggml_tensor * tp = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, T);
+    memcpy(tp->data, pos, (size_t)T * 4);
+    struct ggml_tensor * r = ggml_rope_custom(ctx, tx, tp, n_dims, mode, 0, 0, freq_base, freq_scale, 0.0f, 1.0f, 32.0f, 1.0f);
+    struct ggml_cgraph * gf = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, r);
+    ggml_graph_compute_with_ctx(ctx, gf, 1);
+    memcpy(out, r->data, n * 4);
+    ggml_free(ctx);
+    return 0;
+}
+
+/* ggml_soft_max over rows of x [n, rows] */
+REF_API int ref_soft_max(const float * x, int n, int rows, float * out) {
+    struct ggml_context * ctx = new_ctx((size_t)n * rows * 16 + (1u << 20));
+    if (!ctx) return 1;
+    struct ggml_tensor * tx = put2d(ctx, GGML_TYPE_F32, n, rows, x);
+    struct ggml_tensor * r  = ggml_soft_max(ctx, tx);
+    struct ggml_cgraph * gf = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, r);
+    ggml_graph_compute_with_ctx(ctx, gf, 1);
+    memcpy(out, r->data, (size_t)n * rows * 4);
+    ggml_free(ctx);
+    return 0;
+}
+
+/*
+ * Single-token-batch attention core as llm_build_kqv assembles it (llama.cpp:4764-4850) after
+ * llm_build_kv_store (llama.cpp:4383-4418): K cache F16 [n_ctx][n_embd_gqa], V cache F16 transposed
+ * [n_embd_gqa][n_ctx]; the caller passes caches that already contain positions [0, n_past) and
+ * this call stores k_cur/v_cur for T new tokens at n_past, then attends with a causal mask.
+ * q [n_embd_head, n_head, T] and k_cur [n_embd_head, n_head_kv, T] are post-RoPE; v_cur [n_embd_gqa, T].
+ * out: [n_embd, T] (kqv_merged_cont, before wo).  The caches are updated in place.
+ */
+REF_API int ref_attention(int n_embd_head, int n_head, int n_head_kv, int n_ctx, int n_past, int T,
+                          const float * q, const float * k_cur, const float * v_cur,
+                          uint16_t * k_cache, uint16_t * v_cache, float * out) {
+    const int n_embd = n_embd_head * n_head, n_embd_gqa = n_embd_head * n_head_kv;
+    const int n_kv = n_past + T;
+    size_t payload = (size_t)n_ctx * n_embd_gqa * 4 + (size_t)T * (n_embd * 8 + n_embd_gqa * 8)
+                   + (size_t)n_kv * T * (n_head * 12 + 4) + (size_t)n_embd * T * 16 + (8u << 20);
+    struct ggml_context * ctx = new_ctx(payload);
+    if (!ctx) return 1;
+    struct ggml_tensor * kc = ggml_new_tensor_1d(ctx, GGML_TYPE_F16, (int64_t)n_ctx * n_embd_gqa);
+    struct ggml_tensor * vc = ggml_new_tensor_1d(ctx, GGML_TYPE_F16, (int64_t)n_ctx * n_embd_gqa);
+    memcpy(kc->data, k_cache, ggml_nbytes(kc));
+    memcpy(vc->data, v_cache, ggml_nbytes(vc));
+    struct ggml_tensor * tq = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, n_embd_head, n_head, T);
+    struct ggml_tensor * tk = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, n_embd_head, n_head_kv, T);
+    struct ggml_tensor * tv = ggml_new_tensor_2d(ctx, GGML_TYPE_F32, n_embd_gqa, T);
+    memcpy(tq->data, q, ggml_nbytes(tq));
+    memcpy(tk->data, k_cur, ggml_nbytes(tk));
+    memcpy(tv->data, v_cur, ggml_nbytes(tv));
+    struct ggml_tensor * scale = ggml_new_tensor_1d(ctx, GGML_TYPE_F32, 1);
+    ((float *)scale->data)[0] = 1.0f / sqrtf((float)n_embd_head);
+    struct ggml_tensor * mask = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, n_kv, T, 1);
+    for (int j = 0; j < T; ++j)
+        for (int i = 0; i < n_kv; ++i)
+            ((float *)mask->data)[(size_t)j * n_kv + i] = (i > n_past + j) ? -INFINITY : 0.0f;
+
+    struct ggml_cgraph * gf = ggml_new_graph(ctx);
+    const size_t es = ggml_element_size(kc);
+    struct ggml_tensor * v_cur_t = ggml_transpose(ctx, ggml_reshape_2d(ctx, tv, n_embd_gqa, T));
+    struct ggml_tensor * k_view  = ggml_view_1d(ctx, kc, (int64_t)T * n_embd_gqa, es * n_embd_gqa * n_past);
+    struct ggml_tensor * v_view  = ggml_view_2d(ctx, vc, T, n_embd_gqa, n_ctx * es, n_past * es);
+    ggml_build_forward_expand(gf, ggml_cpy(ctx, tk, k_view));
+    ggml_build_forward_expand(gf, ggml_cpy(ctx, v_cur_t, v_view));
+
+    struct ggml_tensor * qp = ggml_permute(ctx, tq, 0, 2, 1, 3);
+    struct ggml_tensor * k  = ggml_view_3d(ctx, kc, n_embd_head, n_kv, n_head_kv, es * n_embd_gqa, es * n_embd_head, 0);
+    struct ggml_tensor * kq = ggml_mul_mat(ctx, k, qp);
+    kq = ggml_scale(ctx, kq, scale);
+    kq = ggml_add(ctx, kq, mask);
+    kq = ggml_soft_max(ctx, kq);
+    struct ggml_tensor * v   = ggml_view_3d(ctx, vc, n_kv, n_embd_head, n_head_kv, es * n_ctx, es * n_ctx * n_embd_head, 0);
+    struct ggml_tensor * kqv = ggml_mul_mat(ctx, v, kq);
+    struct ggml_tensor * mrg = ggml_permute(ctx, kqv, 0, 2, 1, 3);
+    struct ggml_tensor * cur = ggml_cont_2d(ctx, mrg, n_embd, T);
+    ggml_build_forward_expand(gf, cur);
+    ggml_graph_compute_with_ctx(ctx, gf, 1);
+
+    memcpy(out, cur->data, (size_t)n_embd * T * 4);
+    memcpy(k_cache, kc->data, ggml_nbytes(kc));
+    memcpy(v_cache, vc->data, ggml_nbytes(vc));
+    ggml_free(ctx);
+    return 0;
+}
+
+/* codecs, through the type-traits table the executor itself uses (ggml.c:429-455) */
+REF_API void ref_quantize_row(int type, const float * x, void * y, int n) {
+    ggml_internal_get_type_traits((enum ggml_type) type).from_float_reference(x, y, n);
+}
+REF_API void ref_quantize_row_fast(int type, const float * x, void * y, int n) {
+    ggml_internal_get_type_traits((enum ggml_type) type).from_float(x, y, n);
+}
+REF_API void ref_dequantize_row(int type, const void * x, float * y, int n) {
+    ggml_internal_get_type_traits((enum ggml_type) type).to_float(x, y, n);
+}
+REF_API void ref_fp32_to_fp16_row(const float * x, uint16_t * y, int n) { ggml_fp32_to_fp16_row(x, y, n); }
+REF_API void ref_fp16_to_fp32_row(const uint16_t * x, float * y, int n) { ggml_fp16_to_fp32_row(x, y, n); }
+
+REF_API void ref_init(void) {
+    struct ggml_init_params ip = { 1u << 20, NULL, false };
+    struct ggml_context * ctx = ggml_init(ip);   /* fills the fp16 / exp lookup tables */
+    ggml_free(ctx);
+}

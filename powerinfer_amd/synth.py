@@ -1,0 +1,158 @@
+"""Seeded synthetic PowerInfer models (random-init weights of a given shape).
+
+The reference ships no checkpoints; its loaders expect the tensors listed at llama.cpp:403-461
+(`blk.N.{attn_q,...,ffn_gate,ffn_up,ffn_down_t,fc1,fc2}.weight`).  This module produces arrays with
+those roles and shapes, in ggml's row-major layout (`[rows][ne0]`, ne0 contiguous).
+
+Predictor.  The reference predictor is weight-only: logits = fc2 . relu(fc1 . x), neuron j is active
+iff logit_j >= threshold (llama.cpp:4688-4695, ggml.c:14256).  To give neuron j a chosen firing rate
+p_j without a bias tensor, fc2 row j is built as  b_j * u + eps_j  with u the unit all-ones direction and
+eps_j ~ N(0, sigma^2 I).  For h = relu(fc1 . x) with Gaussian pre-activations, (u.h)/|h| concentrates
+at 1/sqrt(pi), so P(logit_j >= 0) = Phi(b_j / (sigma * sqrt(pi))), independent of the scale of x and
+fc1:  b_j = sigma * sqrt(pi) * Phi^-1(p_j).  Rates follow a Zipf(1.2) law over a seeded random ranking of
+the neurons, clipped to [p_min, p_max] and normalised to the requested mean.
+"""
+import numpy as np
+from scipy.special import ndtri
+
+F32, F16, Q4_0, I32 = 0, 1, 2, 18   # enum ggml_type values (ggml.h:333-355)
+
+
+def zipf_rates(ff, mean, rng, s=1.2, p_max=0.98, p_min=1e-4):
+    """Per-neuron firing rates p_j ∝ rank_j^-s with the given mean; returns (p, rank)."""
+    rank = rng.permutation(ff) + 1                    # rank 1 = hottest
+    w = rank.astype(np.float64) ** (-s)
+    p = np.minimum(w * (mean * ff / w.sum()), p_max)
+    for _ in range(64):                               # water-filling: rescale the unclipped part
+        free = p < p_max
+        need = mean * ff - p_max * (~free).sum()
+        scale = need / p[free].sum()
+        if abs(scale - 1) < 1e-12:
+            break
+        p[free] = np.minimum(p[free] * scale, p_max)
+    return np.maximum(p, p_min), rank
+
+
+def predictor_fc2(ff, r, p, rng, sigma=0.02):
+    b = sigma * np.sqrt(np.pi) * ndtri(p)
+    eps = rng.standard_normal((ff, r), dtype=np.float32) * np.float32(sigma)
+    return (eps + (b / np.sqrt(r)).astype(np.float32)[:, None]).astype(np.float16)
+
+
+def quantize_q4_0(x):
+    """ggml Q4_0 (ggml-quants.c:428-463) in numpy: float32 [..., n] -> uint8 [..., n/32*18]."""
+    x = np.ascontiguousarray(x, np.float32)
+    n = x.shape[-1]
+    b = x.reshape(-1, n // 32, 32)
+    i = np.argmax(np.abs(b), axis=-1)                 # first element of largest magnitude
+    mx = np.take_along_axis(b, i[..., None], -1)[..., 0]
+    d = (mx / np.float32(-8)).astype(np.float32)
+    idv = np.where(d != 0, np.float32(1) / np.where(d != 0, d, 1), 0).astype(np.float32)
+    q = np.minimum(15, (b * idv[..., None] + np.float32(8.5)).astype(np.int8)).astype(np.uint8)
+    out = np.empty(b.shape[:2] + (18,), np.uint8)
+    out[..., :2] = d.astype(np.float16).view(np.uint8).reshape(b.shape[:2] + (2,))
+    out[..., 2:] = q[..., :16] | (q[..., 16:] << 4)
+    return out.reshape(x.shape[:-1] + (n // 32 * 18,))
+
+
+def dequantize_q4_0(q, n):
+    b = q.reshape(-1, n // 32, 18)
+    d = b[..., :2].copy().view(np.float16).astype(np.float32)
+    lo = (b[..., 2:] & 0x0F).astype(np.int8) - 8
+    hi = (b[..., 2:] >> 4).astype(np.int8) - 8
+    y = np.concatenate([lo, hi], -1).astype(np.float32) * d
+    return y.reshape(q.shape[:-1] + (n,))
+
+
+def encode(w32, wtype):
+    return w32.astype(np.float16) if wtype == F16 else quantize_q4_0(w32)
+
+
+def gpu_split(p, hot_frac):
+    """Top `hot_frac` of neurons by firing rate go to the GPU (export_split.py:24-52 given the per-layer
+    count): gpu_idx int32[ff] (1 = on GPU), gpu_bucket = sorted original indices of the GPU neurons."""
+    ff = p.size
+    n_hot = int(round(hot_frac * ff))
+    hot = np.argsort(-p, kind="stable")[:n_hot]
+    gpu_idx = np.zeros(ff, np.int32)
+    gpu_idx[hot] = 1
+    return gpu_idx, np.sort(hot).astype(np.int32)
+
+
+def make_ffn_layer(seed, d, ff, r, wtype=F16, has_gate=True, mean_rate=0.10, T=1):
+    """Config-0 style single sparse FFN layer: weights ~N(0, 0.02), activations ~N(0, 1)."""
+    rng = np.random.default_rng(seed)
+    nrm = lambda rows, cols, s: rng.standard_normal((rows, cols), dtype=np.float32) * np.float32(s)  # noqa: E731
+    L = dict(d=d, ff=ff, r=r, wtype=wtype, has_gate=has_gate)
+    L["up"] = encode(nrm(ff, d, 0.02), wtype)
+    L["gate"] = encode(nrm(ff, d, 0.02), wtype) if has_gate else None
+    L["down_t"] = encode(nrm(ff, d, 0.02), wtype)
+    L["fc1"] = nrm(r, d, 0.02).astype(np.float16)
+    L["p"], L["rank"] = zipf_rates(ff, mean_rate, rng)
+    L["fc2"] = predictor_fc2(ff, r, L["p"], rng)
+    L["x"] = rng.standard_normal((T, d), dtype=np.float32)
+    return L
+
+
+class HParams(dict):
+    __getattr__ = dict.__getitem__
+
+
+def hparams(name, **over):
+    """Shapes of the benchmark configurations (d, ff, rank, heads, layers, vocab)."""
+    base = {
+        "llama-7b": dict(arch="llama", n_embd=4096, n_ff=11008, n_rank=1024, n_head=32, n_head_kv=32, n_layer=32,
+                         n_vocab=32000, mean_rate=0.10),
+        "llama-13b": dict(arch="llama", n_embd=5120, n_ff=13824, n_rank=1280, n_head=40, n_head_kv=40, n_layer=40,
+                          n_vocab=32000, mean_rate=0.11),
+        "falcon-40b": dict(arch="falcon", n_embd=8192, n_ff=32768, n_rank=1024, n_head=128, n_head_kv=8, n_layer=60,
+                           n_vocab=65024, mean_rate=0.08),
+        "llama-tiny": dict(arch="llama", n_embd=256, n_ff=1024, n_rank=64, n_head=4, n_head_kv=4, n_layer=2,
+                           n_vocab=512, mean_rate=0.15),
+        "falcon-tiny": dict(arch="falcon", n_embd=256, n_ff=1024, n_rank=64, n_head=8, n_head_kv=2, n_layer=2,
+                            n_vocab=512, mean_rate=0.15),
+    }[name]
+    hp = HParams(base, name=name, n_ctx=512, wtype=F16, norm_eps=1e-5, rope_freq_base=10000.0, sparse_threshold=0.0,
+                 hot_frac=1.0, seed=0)
+    hp.update(over)
+    return hp
+
+
+def make_model(hp):
+    """All tensors of a synthetic model as numpy arrays: dict(glob={...}, layers=[{...}], hp=hp).
+    Norm weights are 1 (biases 0); everything else ~N(0, 0.02) rounded to fp16 and then, for
+    wtype == Q4_0, quantised (attention, FFN and output matrices; predictors stay fp16)."""
+    rng = np.random.default_rng(hp.seed)
+    d, ff, r = hp.n_embd, hp.n_ff, hp.n_rank
+    gqa = d // hp.n_head * hp.n_head_kv
+    wt = hp.wtype
+    nrm = lambda rows, cols: (rng.standard_normal((rows, cols), dtype=np.float32) * np.float32(0.02)).astype(np.float16)  # noqa: E731
+    enc = (lambda a: a) if wt == F16 else (lambda a: quantize_q4_0(a.astype(np.float32)))
+    falcon = hp.arch == "falcon"
+    glob = dict(tok_embd=enc(nrm(hp.n_vocab, d)), output_norm=np.ones(d, np.float32), output=enc(nrm(hp.n_vocab, d)))
+    if falcon:
+        glob["output_norm_b"] = np.zeros(d, np.float32)
+    layers = []
+    for _ in range(hp.n_layer):
+        L = dict(attn_norm=np.ones(d, np.float32))
+        if falcon:
+            L["attn_norm_b"] = np.zeros(d, np.float32)
+            if hp.n_head_kv != hp.n_head and hp.get("two_norms", True):
+                L["attn_norm_2"] = np.ones(d, np.float32)
+                L["attn_norm_2_b"] = np.zeros(d, np.float32)
+            L["wqkv"] = enc(nrm(d + 2 * gqa, d))
+        else:
+            L["wq"], L["wk"], L["wv"] = enc(nrm(d, d)), enc(nrm(gqa, d)), enc(nrm(gqa, d))
+            L["ffn_norm"] = np.ones(d, np.float32)
+            L["ffn_gate"] = enc(nrm(ff, d))
+        L["wo"] = enc(nrm(d, d))
+        L["ffn_up"] = enc(nrm(ff, d))
+        L["ffn_down_t"] = enc(nrm(ff, d))
+        L["fc1"] = nrm(r, d)
+        p, _ = zipf_rates(ff, hp.mean_rate, rng)
+        L["fc2"] = predictor_fc2(ff, r, p, rng)
+        L["p"] = p
+        if hp.hot_frac < 1.0:
+            L["gpu_idx"], L["gpu_bucket"] = gpu_split(p, hp.hot_frac)
+        layers.append(L)
+    return dict(hp=hp, glob=glob, layers=layers)

@@ -1,0 +1,129 @@
+"""ctypes bindings to the parity checkers (test infrastructure only).
+
+`oracle()`  -> oracle/libpi_oracle.so, the repo's CPU restatement (always buildable).
+`ref()`     -> oracle/_ref/libpi_ref.so, the compiled reference ggml (None where it was never built).
+"""
+import ctypes as C
+import os
+import subprocess
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+ODIR = os.path.join(ROOT, "oracle")
+
+F32, F16, Q4_0, I32 = 0, 1, 2, 18
+
+_vp, _i, _f, _i64 = C.c_void_p, C.c_int, C.c_float, C.c_int64
+
+
+def _ptr(a):
+    if a is None:
+        return None
+    assert a.flags["C_CONTIGUOUS"]
+    return a.ctypes.data_as(C.c_void_p)
+
+
+_oracle = None
+_ref = None
+
+
+def oracle():
+    global _oracle
+    if _oracle is None:
+        so = os.path.join(ODIR, "libpi_oracle.so")
+        if not os.path.exists(so):
+            subprocess.check_call(["make", "-C", ODIR, "oracle"], stdout=subprocess.DEVNULL)
+        L = C.CDLL(so)
+        L.pio_f32_to_f16.restype = C.c_uint16
+        L.pio_f32_to_f16.argtypes = [_f]
+        L.pio_f16_to_f32.restype = _f
+        L.pio_f16_to_f32.argtypes = [C.c_uint16]
+        L.pio_row_bytes.restype = C.c_size_t
+        L.pio_row_bytes.argtypes = [_i, _i64]
+        L.pio_vec_dot_f16.restype = _f
+        L.pio_vec_dot_f16.argtypes = [_i64, _vp, _vp]
+        L.pio_vec_dot_q4_0_q8_0.restype = _f
+        L.pio_vec_dot_q4_0_q8_0.argtypes = [_i64, _vp, _vp]
+        for n in ("pio_f32_to_f16_row", "pio_f16_to_f32_row", "pio_quantize_row_q4_0", "pio_dequantize_row_q4_0",
+                  "pio_quantize_row_q8_0"):
+            getattr(L, n).argtypes = [_vp, _vp, _i64]
+            getattr(L, n).restype = None
+        L.pio_mul_mat.argtypes = [_i, _vp, _i64, _i64, _vp, _i, _vp, _i]
+        L.pio_mul_mat_sparse.argtypes = [_i, _vp, _i64, _i64, _vp, _i, _vp, _vp, _f, _vp, _i]
+        L.pio_axpy.argtypes = [_i, _vp, _i64, _i64, _vp, _i, _vp, _vp, _f, _vp, _i]
+        L.pio_rms_norm.argtypes = [_vp, _i64, _i, _f, _vp]
+        L.pio_norm.argtypes = [_vp, _i64, _i, _f, _vp]
+        L.pio_rope.argtypes = [_vp, _i, _i, _i, _vp, _i, _i, _f, _f, _vp]
+        L.pio_soft_max.argtypes = [_vp, _i64, _i64, _vp]
+        L.pio_active_list.argtypes = [_vp, _i64, _f, _vp]
+        L.pio_ffn_sparse.argtypes = [_i] * 6 + [_vp] * 8 + [_f, _i] + [_vp] * 5
+        L.pio_attention.argtypes = [_i] * 6 + [_vp] * 8
+        L.pio_model_new.restype = _vp
+        L.pio_model_new.argtypes = [_vp]
+        L.pio_model_free.argtypes = [_vp]
+        L.pio_model_set_tensor.argtypes = [_vp, _i, _i, _i, _vp, _i64, _i64]
+        L.pio_model_kv_clear.argtypes = [_vp]
+        L.pio_model_set_capture.argtypes = [_vp, _vp, _vp]
+        L.pio_model_eval.argtypes = [_vp, _vp, _vp, _vp, _i, _i, _vp, _i, _vp, _i]
+        L.pio_model_eval_simple.argtypes = [_vp, _vp, _i, _i, _vp, _i]
+        _oracle = L
+    return _oracle
+
+
+def ref():
+    """The compiled reference (or None).  Built on demand only where /root/reference exists."""
+    global _ref
+    if _ref is None:
+        so = os.path.join(ODIR, "_ref", "libpi_ref.so")
+        if not os.path.exists(so):
+            if not os.path.isdir("/root/reference"):
+                return None
+            subprocess.check_call(["make", "-C", ODIR, "ref"], stdout=subprocess.DEVNULL)
+        L = C.CDLL(so)
+        L.ref_ffn_sparse.argtypes = [_i] * 6 + [_vp] * 8 + [_f, _i] + [_vp] * 5
+        L.ref_mul_mat.argtypes = [_i, _vp, _i, _i, _vp, _i, _i, _vp]
+        L.ref_norm.argtypes = [_i, _vp, _i, _i, _f, _vp]
+        L.ref_rope.argtypes = [_vp, _i, _i, _i, _vp, _i, _i, _f, _f, _vp]
+        L.ref_soft_max.argtypes = [_vp, _i, _i, _vp]
+        L.ref_attention.argtypes = [_i] * 6 + [_vp] * 6
+        for n in ("ref_quantize_row", "ref_quantize_row_fast", "ref_dequantize_row"):
+            getattr(L, n).argtypes = [_i, _vp, _vp, _i]
+            getattr(L, n).restype = None
+        L.ref_init()
+        _ref = L
+    return _ref
+
+
+# ---------------------------------------------------------------------------------------------
+# numpy-level wrappers shared by the oracle and the reference (same argument meaning)
+# ---------------------------------------------------------------------------------------------
+def row_bytes(t, n):
+    return {F32: 4 * n, I32: 4 * n, F16: 2 * n, Q4_0: n // 32 * 18}[t]
+
+
+def quantize_q4_0(x, lib=None):
+    """x float32 [..., n] -> uint8 [..., n/32*18]"""
+    x = np.ascontiguousarray(x, np.float32)
+    n = x.shape[-1]
+    out = np.empty(x.shape[:-1] + (n // 32 * 18,), np.uint8)
+    xs, os_ = x.reshape(-1, n), out.reshape(-1, n // 32 * 18)
+    L = lib or oracle()
+    for i in range(xs.shape[0]):
+        if L is _ref:
+            L.ref_quantize_row(Q4_0, _ptr(xs[i]), _ptr(os_[i]), n)
+        else:
+            L.pio_quantize_row_q4_0(_ptr(xs[i]), _ptr(os_[i]), n)
+    return out
+
+
+def ffn_sparse(lib, d, ff, r, T, wtype, has_gate, up, gate, down_t, fc1, fc2, x_ffn, x_pred, gpu_idx, thr, nth=1):
+    """Runs the sparse FFN block on `lib` (oracle() or ref()).  Returns dict of float32 arrays."""
+    o = dict(logits=np.zeros((T, ff), np.float32), up=np.zeros((T, ff), np.float32),
+             gate=np.zeros((T, ff), np.float32), h=np.zeros((T, ff), np.float32), out=np.zeros((T, d), np.float32))
+    fn = lib.ref_ffn_sparse if lib is _ref and _ref is not None else lib.pio_ffn_sparse
+    rc = fn(d, ff, r, T, wtype, int(has_gate), _ptr(up), _ptr(gate) if has_gate else None, _ptr(down_t),
+            _ptr(fc1), _ptr(fc2), _ptr(x_ffn), _ptr(x_pred), _ptr(gpu_idx), thr, nth,
+            _ptr(o["logits"]), _ptr(o["up"]), _ptr(o["gate"]), _ptr(o["h"]), _ptr(o["out"]))
+    assert rc == 0, rc
+    return o

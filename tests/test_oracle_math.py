@@ -186,7 +186,7 @@ def test_norms_and_softmax_closed_form():
     O.pio_soft_max(P(s), 100, 3, P(p))
     e = np.exp(s.astype(np.float64) - s.max(-1, keepdims=True))
     np.testing.assert_allclose(p.sum(-1), 1, rtol=1e-6)
-    np.testing.assert_allclose(p, e / e.sum(-1, keepdims=True), rtol=2e-3, atol=1e-6)   # fp16 exp table: ~2^-11 per term, subnormal below 6e-5
+    np.testing.assert_allclose(p, e / e.sum(-1, keepdims=True), rtol=1.5e-2, atol=1e-6)   # exp table indexed by fp16(x - max): error grows as |x - max| * 2^-11
 
 
 def test_active_list_is_ascending_compaction():

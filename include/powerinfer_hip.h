@@ -1,0 +1,159 @@
+/*
+ * C ABI of libpowerinfer_hip.so -- the MI355X (gfx950) implementation of PowerInfer's sparse decode
+ * token loop.  Plain pointers and sizes only.  Three layers, each a drop-in for a slice of the
+ * reference (citations are file:line into the reference tree):
+ *
+ *   1. pi_k_*      one launcher per hot operator (what ggml-cuda.cu's op functions launch)
+ *   2. pi_model_*  the decode loop with resident weights (what llama_decode drives per token)
+ *   3. ggml_cuda_* the reference's own backend entry points, same names and contracts
+ *                  (declared in ggml_backend_abi.h)
+ *
+ * All device pointers are HIP device addresses on the current device.  Unless stated otherwise a
+ * function returns 0 on success and a negative code on error; pi_last_error() then describes it.
+ * Launchers are asynchronous on `stream` (a hipStream_t passed as void*, NULL = the default stream).
+ */
+#ifndef POWERINFER_HIP_H
+#define POWERINFER_HIP_H
+
+#include <stddef.h>
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define PI_API __attribute__((visibility("default")))
+
+typedef void * pi_stream_t;
+
+/* element types: numeric values of enum ggml_type (ggml.h:333-355) */
+enum { PI_TYPE_F32 = 0, PI_TYPE_F16 = 1, PI_TYPE_Q4_0 = 2, PI_TYPE_I32 = 18 };
+
+enum { PI_OK = 0, PI_E_ARG = -1, PI_E_HIP = -2, PI_E_UNSUPPORTED = -3, PI_E_STATE = -4 };
+
+/* ---- runtime plumbing (ggml_init_cublas, ggml-cuda.cu:6463-6534; host/device copies :8005-8080) ---- */
+PI_API int          pi_init(int device);
+PI_API const char * pi_last_error(void);
+PI_API int          pi_device_name(char * buf, size_t n);
+PI_API void *       pi_malloc(size_t bytes);                 /* NULL on failure */
+PI_API int          pi_free(void * dptr);
+PI_API int          pi_memset(void * dptr, int byte, size_t bytes);
+PI_API int          pi_memcpy_h2d(void * dptr, const void * host, size_t bytes);
+PI_API int          pi_memcpy_d2h(void * host, const void * dptr, size_t bytes);
+PI_API int          pi_memcpy_d2d(void * dst, const void * src, size_t bytes);
+PI_API int          pi_sync(void);
+/* deterministic N(0, std^2) fill rounded to fp16 (synthetic weights generated in HBM); row_bias, if
+ * not NULL, holds one fp32 per row of `cols` elements that is added before rounding */
+PI_API int          pi_fill_normal_f16(void * dptr, size_t n, uint64_t seed, float std, const float * row_bias, int cols, pi_stream_t stream);
+/* event timing on a stream: returns milliseconds between two recorded marks */
+PI_API void *       pi_event_create(void);
+PI_API int          pi_event_record(void * ev, pi_stream_t stream);
+PI_API int          pi_event_elapsed_ms(void * start, void * stop, float * ms);   /* synchronises on stop */
+PI_API int          pi_event_destroy(void * ev);
+
+/* ---- operator launchers ---------------------------------------------------------------------------- */
+
+/* optional normalisation applied to the activation vector before a mat-vec:
+ * kind 0 none | 1 RMSNorm (rms_norm_f32, ggml-cuda.cu:667) | 2 LayerNorm (norm_f32, ggml-cuda.cu:621);
+ * y = norm(x) * w (+ b).  w, b: device fp32 [cols] or NULL. */
+typedef struct pi_norm {
+    int32_t       kind;
+    float         eps;
+    const float * w;
+    const float * b;
+} pi_norm;
+
+enum { PI_EPI_NONE = 0, PI_EPI_RELU = 1, PI_EPI_ADD = 2, PI_EPI_ADD2 = 3 };
+
+/*
+ * Dense mat-vec  y[rows] = epi(W[rows][cols] . act(x)),  batch 1.
+ * Replaces dequantize_mul_mat_vec<1,1,convert_f16> (ggml-cuda.cu:4349, launcher :5629) and
+ * mul_mat_vec_q<QK4_0,...> with quantize_q8_1 (ggml-cuda.cu:4311, 1624, launcher :5480) for
+ * attention projections, predictor fc1 and lm-head.  Activations are rounded the way the CPU path
+ * rounds them (fp16 for F16 weights, Q8_0 blocks for Q4_0 weights; ggml.c:9703-9716).
+ * epilogue: NONE | RELU | ADD (y += add1) | ADD2 (y = (y + add1) + add2).
+ */
+PI_API int pi_k_gemv(int wtype, const void * W, int rows, int cols, const float * x, const pi_norm * norm,
+                     int epilogue, const float * add1, const float * add2, float * y, pi_stream_t stream);
+
+/* scratch shared by the predictor / sparse kernels of one stream; sized for the largest ff and d used */
+typedef struct pi_workspace pi_workspace;
+PI_API pi_workspace * pi_workspace_create(int max_ff, int max_d);
+PI_API int            pi_workspace_destroy(pi_workspace * ws);
+
+/*
+ * Predictor output layer fused with the activity test and compaction:
+ *   logits[ff] = fc2[ff][r] . fp16(hidden[r]);  neuron j active iff !(logits[j] < threshold)
+ * (mul_mat "mlp_pre_out", llama.cpp:4693; test ggml-cuda.cu:4695 / ggml.c:14256).  Emits the ascending
+ * list of active rows and its length.  With bucket == NULL rows are neuron indices 0..ff-1.  With a
+ * gpu_bucket (sorted original indices of the GPU-resident neurons, llama.cpp:2820-2870) the candidates
+ * are rows 0..n_bucket-1 of the compact GPU matrices and row i is active iff neuron bucket[i] is.
+ * The reference never materialises this list (it re-tests the mask in every kernel).
+ * zero_fill (optional): fp32 [ff] cleared by the same launch (the dense h vector of the Q4_0 path).
+ */
+PI_API int pi_k_predictor_fc2(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                              const int32_t * bucket, int n_bucket, float * logits,
+                              int32_t * active_rows, int32_t * n_active, float * zero_fill,
+                              pi_workspace * ws, pi_stream_t stream);
+
+/* the same test + compaction over logits that already exist (hybrid split: logits computed elsewhere) */
+PI_API int pi_k_compact_active(const float * logits, int ff, float threshold, const int32_t * bucket, int n_bucket,
+                               int32_t * active_rows, int32_t * n_active, pi_workspace * ws, pi_stream_t stream);
+
+/*
+ * Sparse up/gate mat-vec over the active rows only, fused with the activation:
+ *   h[k] = relu(gate[row_k] . x) * (up[row_k] . x)      (gate != NULL, LLM_FFN_PAR)
+ *   h[k] = relu(up[row_k] . x)                          (gate == NULL, Falcon)
+ * Replaces dequantize_mul_mat_vec_sparse (ggml-cuda.cu:4685) / mul_mat_vec_q(lst, idx) (:5490) plus
+ * relu_f32 and mul_f32.  h_compact[k] is indexed like active_rows; if h_dense != NULL the value is also
+ * scattered to h_dense[neuron] (neuron = bucket ? bucket[row] : row), which the caller has zeroed.
+ * up_dense/gate_dense (optional) receive the raw dot products the same way (GGML_OP_MUL_MAT_SPARSE output).
+ */
+PI_API int pi_k_sparse_upgate(int wtype, const void * up, const void * gate, int cols, const float * x, const pi_norm * norm,
+                              const int32_t * active_rows, const int32_t * n_active, const int32_t * bucket,
+                              float * h_compact, float * h_dense, float * up_dense, float * gate_dense, pi_stream_t stream);
+
+/*
+ * Sparse down projection (GGML_OP_AXPY):  out[cols] = epi( sum_k act(h_compact[k]) * down_t[row_k][:] ).
+ * Replaces dequantize_mul_mat_axpy_sparse (ggml-cuda.cu:4541) and _sparse_pro (:4479) and their
+ * per-row global atomics: column tiles x row groups accumulate in registers, merge through LDS and a
+ * fixed-order second stage, so the result is deterministic.  Rows whose rounded h is zero are not read.
+ * act(): fp16 rounding for F16 weights; for Q4_0 weights h is quantised to Q8_0 over blocks of 32
+ * neurons as the CPU path does (ggml.c:14465-14618), which needs the dense neuron-indexed vector
+ * h_dense (zeros at inactive neurons; may be NULL for F16) and the bucket that maps rows to neurons.
+ * epilogue: NONE | ADD | ADD2 as for pi_k_gemv.
+ */
+PI_API int pi_k_sparse_axpy(int wtype, const void * down_t, int cols, const float * h_compact,
+                            const float * h_dense, const int32_t * bucket,
+                            const int32_t * active_rows, const int32_t * n_active,
+                            int epilogue, const float * add1, const float * add2, float * out,
+                            pi_workspace * ws, pi_stream_t stream);
+
+/*
+ * RoPE on q and k of one token plus the KV-cache store (rope / rope_neox ggml-cuda.cu:4999,5027 and
+ * cpy_f32_f16 :4944 for llm_build_kv_store, llama.cpp:4383).  qkv: fp32 [n_head*hd + 2*n_head_kv*hd]
+ * (q | k | v).  mode 0 = adjacent pairs, 2 = NeoX halves.  The position is read from *pos (device).
+ * Cache layout (this library's own): K and V are fp16 [n_head_kv][n_ctx][hd].
+ */
+PI_API int pi_k_rope_kv_store(const float * qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
+                              const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache, pi_stream_t stream);
+
+/*
+ * Single-token attention over cells [0, *pos] of the cache (KQ, scale, softmax, KQV; replaces the
+ * batched hipBLAS GEMMs + soft_max_f32 the reference runs at batch 1, ggml-cuda.cu:8564-8712, 5135).
+ * Probabilities go through the same fp16 exp rounding as the CPU path (ggml.c:10747-10759).
+ * out: fp32 [n_head*hd].
+ */
+PI_API int pi_k_attn_decode(const float * q_rot, const void * k_cache, const void * v_cache, int n_head, int n_head_kv,
+                            int hd, int n_ctx, const int32_t * pos, float * out, pi_stream_t stream);
+
+/* x[cols] = row *token of the embedding table (k_get_rows, ggml-cuda.cu:1664) */
+PI_API int pi_k_embed(int wtype, const void * table, int cols, const int32_t * token, float * x, pi_stream_t stream);
+
+/* greedy sampling: *token_out = index of the first maximum (llama_sample_token_greedy, llama.cpp:8617-8631) */
+PI_API int pi_k_argmax(const float * logits, int n, int32_t * token_out, pi_stream_t stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,904 @@
+// Hand-written CDNA4 (gfx950, wave64) kernels for the sparse decode token loop and their C-ABI launchers.
+// Every hot kernel here is HBM-bound byte streaming: rows are read once with 128-bit loads, the activation
+// vector is staged in LDS, accumulation is fp32.  Citations are file:line into the reference tree.
+#include "device_utils.hpp"
+#include "runtime.hpp"
+#include "../../include/powerinfer_hip.h"
+
+#include <math.h>
+
+namespace {
+
+constexpr int kBlock = 256;                 // 4 waves
+constexpr int kWavesPerBlock = kBlock / PI_WAVE;
+
+struct NormArgs { int kind; float eps; const float * w; const float * b; };
+
+// ---------------------------------------------------------------------------------------------------
+// block-wide reductions (double, fixed order: lanes by butterfly, waves 0..n-1 sequentially)
+// ---------------------------------------------------------------------------------------------------
+__device__ double block_sum_f64(double v, double * red) {
+    v = pi_wave_sum_f64(v);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    double s = 0.0;
+    for (int i = 0; i < nw; ++i) s += red[i];
+    return s;
+}
+__device__ float block_max_f32(float v, float * red) {
+    v = pi_wave_max(v);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, nw = blockDim.x >> 6;
+    __syncthreads();
+    if (lane == 0) red[wave] = v;
+    __syncthreads();
+    float s = red[0];
+    for (int i = 1; i < nw; ++i) s = fmaxf(s, red[i]);
+    return s;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Activation staging.  x (fp32, global) -> optional norm -> rounded to fp16 -> LDS.
+// RMSNorm as ggml.c:9238-9284 (double sum of fp32 squares, scale = 1/sqrtf(mean+eps), then * w as a
+// second fp32 multiply: llm_build_norm, llama.cpp:4420-4450); LayerNorm as ggml.c:9169-9236.
+// ---------------------------------------------------------------------------------------------------
+__device__ void stage_x_f16(__half * xs, const float * __restrict__ x, int cols, NormArgs na, double * red) {
+    if (na.kind == 0) {
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) xs[i] = __float2half_rn(x[i]);
+    } else if (na.kind == 1) {
+        double s = 0.0;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = x[i]; s += (double)__fmul_rn(v, v); }
+        s = block_sum_f64(s, red);
+        const float mean = (float)(s / cols);
+        const float scale = 1.0f / sqrtf(mean + na.eps);
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+            float v = __fmul_rn(x[i], scale);
+            if (na.w) v = __fmul_rn(v, na.w[i]);
+            if (na.b) v = __fadd_rn(v, na.b[i]);
+            xs[i] = __float2half_rn(v);
+        }
+    } else {
+        double s = 0.0;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) s += (double)x[i];
+        s = block_sum_f64(s, red);
+        const float mean = (float)(s / cols);
+        double s2 = 0.0;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = __fsub_rn(x[i], mean); s2 += (double)__fmul_rn(v, v); }
+        s2 = block_sum_f64(s2, red);
+        const float var = (float)(s2 / cols);
+        const float scale = 1.0f / sqrtf(var + na.eps);
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+            float v = __fmul_rn(__fsub_rn(x[i], mean), scale);
+            if (na.w) v = __fmul_rn(v, na.w[i]);
+            if (na.b) v = __fadd_rn(v, na.b[i]);
+            xs[i] = __float2half_rn(v);
+        }
+    }
+    __syncthreads();
+}
+
+// Q8_0 staging for Q4_0 weights: per block of 32, d = amax/127 kept as fp16, q = rint(x * 127/amax)
+// (x86 path of quantize_row_q8_0, ggml-quants.c:702-760).  LDS layout: int8 q[cols] then float d[cols/32].
+__device__ void stage_x_q8(int8_t * xq, float * xd, const float * __restrict__ x, int cols, NormArgs na, double * red, float * xtmp) {
+    // normalised values first (fp32) into xtmp (LDS), then quantise per 32-block
+    if (na.kind == 0) {
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) xtmp[i] = x[i];
+    } else if (na.kind == 1) {
+        double s = 0.0;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = x[i]; s += (double)__fmul_rn(v, v); }
+        s = block_sum_f64(s, red);
+        const float scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+            float v = __fmul_rn(x[i], scale);
+            if (na.w) v = __fmul_rn(v, na.w[i]);
+            if (na.b) v = __fadd_rn(v, na.b[i]);
+            xtmp[i] = v;
+        }
+    } else {
+        double s = 0.0;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) s += (double)x[i];
+        s = block_sum_f64(s, red);
+        const float mean = (float)(s / cols);
+        double s2 = 0.0;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = __fsub_rn(x[i], mean); s2 += (double)__fmul_rn(v, v); }
+        s2 = block_sum_f64(s2, red);
+        const float scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+            float v = __fmul_rn(__fsub_rn(x[i], mean), scale);
+            if (na.w) v = __fmul_rn(v, na.w[i]);
+            if (na.b) v = __fadd_rn(v, na.b[i]);
+            xtmp[i] = v;
+        }
+    }
+    __syncthreads();
+    // 32 consecutive lanes own one block of 32 values
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+        const float v = xtmp[i];
+        float amax = fabsf(v);
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, PI_WAVE));
+        const float d = amax / 127.0f;
+        const float id = (amax != 0.0f) ? 127.0f / amax : 0.0f;
+        xq[i] = (int8_t)(int)rintf(__fmul_rn(v, id));
+        if ((i & 31) == 0) xd[i >> 5] = pi_round_f16(d);
+    }
+    __syncthreads();
+}
+
+__device__ __forceinline__ float apply_epilogue(float v, int epi, const float * add1, const float * add2, int row) {
+    if (epi == PI_EPI_RELU) return fmaxf(v, 0.0f);
+    if (epi == PI_EPI_ADD)  return __fadd_rn(v, add1[row]);
+    if (epi == PI_EPI_ADD2) return __fadd_rn(__fadd_rn(v, add1[row]), add2[row]);
+    return v;
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Dense F16 mat-vec.  One wave owns RPW consecutive rows; lane l reads 16 B (8 halfs) at column
+// 8*l + 512*i of each row, so a wave issues 1 KiB contiguous per row per load instruction.
+// ---------------------------------------------------------------------------------------------------
+template <int RPW>
+__global__ __launch_bounds__(kBlock) void gemv_f16_kernel(const __half * __restrict__ W, const float * __restrict__ x, NormArgs na,
+                                                          int epi, const float * add1, const float * add2,
+                                                          float * __restrict__ y, int rows, int cols) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __half * xs = reinterpret_cast<__half *>(smem);
+    __shared__ double red[16];
+    stage_x_f16(xs, x, cols, na, red);
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n_groups = (rows + RPW - 1) / RPW;
+    for (int g = blockIdx.x * kWavesPerBlock + wave; g < n_groups; g += gridDim.x * kWavesPerBlock) {
+        const int r0 = g * RPW;
+        float acc[RPW];
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) acc[i] = 0.0f;
+#pragma unroll 2
+        for (int c = lane * 8; c < cols; c += PI_WAVE * 8) {
+            float xf[8];
+            pi_unpack8(pi_ld16(xs + c), xf);
+#pragma unroll
+            for (int i = 0; i < RPW; ++i) {
+                if (r0 + i < rows) acc[i] = pi_dot8(pi_ld_stream(W + (size_t)(r0 + i) * cols + c), xf, acc[i]);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) {
+            const float s = pi_wave_sum(acc[i]);
+            if (lane == 0 && r0 + i < rows) y[r0 + i] = apply_epilogue(s, epi, add1, add2, r0 + i);
+        }
+    }
+}
+
+// Q4_0 dot of one 32-weight block against the staged Q8_0 activations: exact int32 sum of products,
+// then * (d_w * d_x) into fp32 (vec_dot_q4_0_q8_0, ggml-quants.c:2512-2650)
+__device__ __forceinline__ float q4_block_dot(const pi_block_q4_0 * __restrict__ wb, const int8_t * __restrict__ xq, float dx, float acc) {
+    uint16_t dbits; uint32_t q[4];
+    __builtin_memcpy(&dbits, &wb->d, 2);
+    __builtin_memcpy(q, wb->qs, 16);
+    const int * x32 = reinterpret_cast<const int *>(xq);          // 32 int8 = 8 dwords, 4-byte aligned in LDS
+    int sum = 0;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+        const int lo = (int)(q[j] & 0x0F0F0F0Fu);                  // elements 4j .. 4j+3
+        const int hi = (int)((q[j] >> 4) & 0x0F0F0F0Fu);           // elements 16+4j .. 16+4j+3
+        sum = __builtin_amdgcn_sdot4(lo, x32[j], sum, false);
+        sum = __builtin_amdgcn_sdot4(hi, x32[4 + j], sum, false);
+    }
+    // nibbles were used unsigned: subtract 8 * sum(x) of the block
+    int sx = 0;
+#pragma unroll
+    for (int j = 0; j < 8; ++j) sx = __builtin_amdgcn_sdot4(0x01010101, x32[j], sx, false);
+    sum -= 8 * sx;
+    return fmaf(__fmul_rn(pi_f16_from_bits(dbits), dx), (float)sum, acc);
+}
+
+// Dense Q4_0 mat-vec: one wave per RPW rows, lane l owns blocks l, l+64, ...
+template <int RPW>
+__global__ __launch_bounds__(kBlock) void gemv_q4_kernel(const pi_block_q4_0 * __restrict__ W, const float * __restrict__ x, NormArgs na,
+                                                         int epi, const float * add1, const float * add2,
+                                                         float * __restrict__ y, int rows, int cols) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    int8_t * xq   = reinterpret_cast<int8_t *>(smem);
+    float  * xd   = reinterpret_cast<float *>(smem + cols);
+    float  * xtmp = reinterpret_cast<float *>(smem + cols + (cols / 32) * 4);
+    __shared__ double red[16];
+    stage_x_q8(xq, xd, x, cols, na, red, xtmp);
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nb = cols / 32;
+    const int n_groups = (rows + RPW - 1) / RPW;
+    for (int g = blockIdx.x * kWavesPerBlock + wave; g < n_groups; g += gridDim.x * kWavesPerBlock) {
+        const int r0 = g * RPW;
+        float acc[RPW];
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) acc[i] = 0.0f;
+        for (int b = lane; b < nb; b += PI_WAVE) {
+            const float dx = xd[b];
+#pragma unroll
+            for (int i = 0; i < RPW; ++i)
+                if (r0 + i < rows) acc[i] = q4_block_dot(W + (size_t)(r0 + i) * nb + b, xq + b * 32, dx, acc[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) {
+            const float s = pi_wave_sum(acc[i]);
+            if (lane == 0 && r0 + i < rows) y[r0 + i] = apply_epilogue(s, epi, add1, add2, r0 + i);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Predictor fc2 + activity test + compaction.
+// Block = 32 consecutive neurons (8 per wave) -> one 32-bit mask word per block by wave ballot.  The
+// block that finishes last (ticket counter) turns the mask words into the ascending active-row list
+// with popcount prefix sums.
+// ---------------------------------------------------------------------------------------------------
+__device__ int block_exclusive_scan_i32(int v, int * total, int * sred) {
+    // inclusive scan within the wave
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6, nw = blockDim.x >> 6;
+    int inc = v;
+#pragma unroll
+    for (int o = 1; o < PI_WAVE; o <<= 1) { const int t = __shfl_up(inc, o, PI_WAVE); if (lane >= o) inc += t; }
+    __syncthreads();
+    if (lane == PI_WAVE - 1) sred[wave] = inc;
+    __syncthreads();
+    int base = 0, tot = 0;
+    for (int i = 0; i < nw; ++i) { const int s = sred[i]; if (i < wave) base += s; tot += s; }
+    *total = tot;
+    return base + inc - v;
+}
+
+__device__ void compact_from_words(const uint32_t * words, int ff, const int32_t * __restrict__ bucket, int n_bucket,
+                                   int32_t * __restrict__ list, int32_t * __restrict__ n_active, int * sred) {
+    int base = 0;
+    if (bucket == nullptr) {
+        const int nwords = (ff + 31) / 32;
+        for (int w0 = 0; w0 < nwords; w0 += blockDim.x) {
+            const int w = w0 + threadIdx.x;
+            uint32_t bits = (w < nwords) ? words[w] : 0u;
+            int tot;
+            int off = base + block_exclusive_scan_i32(__popc(bits), &tot, sred);
+            while (bits) { const int b = __ffs(bits) - 1; bits &= bits - 1; list[off++] = w * 32 + b; }
+            base += tot;
+        }
+    } else {
+        for (int r0 = 0; r0 < n_bucket; r0 += blockDim.x) {
+            const int r = r0 + threadIdx.x;
+            int act = 0;
+            if (r < n_bucket) { const int n = bucket[r]; act = (words[n >> 5] >> (n & 31)) & 1u; }
+            int tot;
+            const int off = base + block_exclusive_scan_i32(act, &tot, sred);
+            if (act) list[off] = r;
+            base += tot;
+        }
+    }
+    if (threadIdx.x == 0) *n_active = base;
+}
+
+// returns true in every thread of the block that took the last ticket; resets the counter for the next launch
+__device__ bool last_block_done(unsigned int * counter, unsigned int n_blocks, int * sflag) {
+    __threadfence();
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        const unsigned int t = atomicAdd(counter, 1u);
+        *sflag = (t == n_blocks - 1);
+        if (t == n_blocks - 1) *counter = 0;
+    }
+    __syncthreads();
+    const bool last = *sflag != 0;
+    if (last) __threadfence();
+    return last;
+}
+
+__global__ __launch_bounds__(kBlock) void pred_fc2_kernel(const __half * __restrict__ W, const float * __restrict__ hidden, int ff, int r,
+                                                          float thr, const int32_t * bucket, int n_bucket, float * __restrict__ logits,
+                                                          uint32_t * words, unsigned int * counter,
+                                                          int32_t * list, int32_t * n_active, float * zero_fill) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __half * xs = reinterpret_cast<__half *>(smem);
+    __shared__ float lg[32];
+    if (zero_fill && threadIdx.x < 32 && (int)(blockIdx.x * 32 + threadIdx.x) < ff) zero_fill[blockIdx.x * 32 + threadIdx.x] = 0.0f;
+    __shared__ int sred[kWavesPerBlock + 1];
+    for (int i = threadIdx.x; i < r; i += blockDim.x) xs[i] = __float2half_rn(hidden[i]);
+    __syncthreads();
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int row0 = blockIdx.x * 32 + wave * 8;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    for (int c = lane * 8; c < r; c += PI_WAVE * 8) {
+        float xf[8];
+        pi_unpack8(pi_ld16(xs + c), xf);
+#pragma unroll
+        for (int i = 0; i < 8; ++i)
+            if (row0 + i < ff) acc[i] = pi_dot8(pi_ld_stream(W + (size_t)(row0 + i) * r + c), xf, acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { const float s = pi_wave_sum(acc[i]); if (lane == 0) lg[wave * 8 + i] = s; }
+    __syncthreads();
+    if (wave == 0) {
+        const int row = blockIdx.x * 32 + lane;
+        bool act = false;
+        if (lane < 32 && row < ff) { const float v = lg[lane]; logits[row] = v; act = !(v < thr); }
+        const unsigned long long m = __ballot(act);
+        if (lane == 0) words[blockIdx.x] = (uint32_t)m;
+    }
+    if (last_block_done(counter, gridDim.x, &sred[kWavesPerBlock]))
+        compact_from_words(words, ff, bucket, n_bucket, list, n_active, sred);
+}
+
+// activity test + compaction over existing logits (single block)
+__global__ __launch_bounds__(1024) void compact_kernel(const float * __restrict__ logits, int ff, float thr, const int32_t * bucket, int n_bucket,
+                                                       uint32_t * words, int32_t * list, int32_t * n_active) {
+    __shared__ int sred[17];
+    const int lane = threadIdx.x & 63;
+    for (int i0 = 0; i0 < ff; i0 += blockDim.x) {
+        const int i = i0 + threadIdx.x;
+        const bool act = (i < ff) && !(logits[i] < thr);
+        const unsigned long long m = __ballot(act);
+        if (lane == 0 && i < ff) words[i >> 5] = (uint32_t)m;
+        if (lane == 32 && i < ff) words[i >> 5] = (uint32_t)(m >> 32);
+    }
+    __syncthreads();
+    compact_from_words(words, ff, bucket, n_bucket, list, n_active, sred);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Sparse up/gate over the active list.  One wave per active row: reads the gate row and the up row
+// (2 x cols fp16) with 128-bit loads, fp32 accumulate, h = relu(g) * u (or relu(u) without a gate).
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void sparse_upgate_f16_kernel(const __half * __restrict__ Wup, const __half * __restrict__ Wgate,
+                                                                   const float * __restrict__ x, NormArgs na, int cols,
+                                                                   const int32_t * __restrict__ list, const int32_t * __restrict__ n_active,
+                                                                   const int32_t * __restrict__ bucket, float * __restrict__ h_compact,
+                                                                   float * h_dense, float * up_dense, float * gate_dense) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __half * xs = reinterpret_cast<__half *>(smem);
+    __shared__ double red[16];
+    const int n = *n_active;
+    if ((int)(blockIdx.x * kWavesPerBlock) >= n) return;       // whole block idle (uniform)
+    stage_x_f16(xs, x, cols, na, red);
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int k = blockIdx.x * kWavesPerBlock + wave; k < n; k += gridDim.x * kWavesPerBlock) {
+        const int row = list[k];
+        const __half * wu = Wup + (size_t)row * cols;
+        const __half * wg = Wgate ? Wgate + (size_t)row * cols : nullptr;
+        float au = 0.0f, ag = 0.0f;
+#pragma unroll 4
+        for (int c = lane * 8; c < cols; c += PI_WAVE * 8) {
+            float xf[8];
+            pi_unpack8(pi_ld16(xs + c), xf);
+            au = pi_dot8(pi_ld_stream(wu + c), xf, au);
+            if (wg) ag = pi_dot8(pi_ld_stream(wg + c), xf, ag);
+        }
+        au = pi_wave_sum(au);
+        if (wg) ag = pi_wave_sum(ag);
+        if (lane == 0) {
+            const float h = wg ? __fmul_rn(fmaxf(ag, 0.0f), au) : fmaxf(au, 0.0f);
+            h_compact[k] = h;
+            const int neuron = bucket ? bucket[row] : row;
+            if (h_dense) h_dense[neuron] = h;
+            if (up_dense) up_dense[neuron] = au;
+            if (gate_dense && wg) gate_dense[neuron] = ag;
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void sparse_upgate_q4_kernel(const pi_block_q4_0 * __restrict__ Wup, const pi_block_q4_0 * __restrict__ Wgate,
+                                                                  const float * __restrict__ x, NormArgs na, int cols,
+                                                                  const int32_t * __restrict__ list, const int32_t * __restrict__ n_active,
+                                                                  const int32_t * __restrict__ bucket, float * __restrict__ h_compact,
+                                                                  float * h_dense, float * up_dense, float * gate_dense) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    int8_t * xq   = reinterpret_cast<int8_t *>(smem);
+    float  * xd   = reinterpret_cast<float *>(smem + cols);
+    float  * xtmp = reinterpret_cast<float *>(smem + cols + (cols / 32) * 4);
+    __shared__ double red[16];
+    const int n = *n_active;
+    if ((int)(blockIdx.x * kWavesPerBlock) >= n) return;
+    stage_x_q8(xq, xd, x, cols, na, red, xtmp);
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nb = cols / 32;
+    for (int k = blockIdx.x * kWavesPerBlock + wave; k < n; k += gridDim.x * kWavesPerBlock) {
+        const int row = list[k];
+        const pi_block_q4_0 * wu = Wup + (size_t)row * nb;
+        const pi_block_q4_0 * wg = Wgate ? Wgate + (size_t)row * nb : nullptr;
+        float au = 0.0f, ag = 0.0f;
+        for (int b = lane; b < nb; b += PI_WAVE) {
+            const float dx = xd[b];
+            au = q4_block_dot(wu + b, xq + b * 32, dx, au);
+            if (wg) ag = q4_block_dot(wg + b, xq + b * 32, dx, ag);
+        }
+        au = pi_wave_sum(au);
+        if (wg) ag = pi_wave_sum(ag);
+        if (lane == 0) {
+            const float h = wg ? __fmul_rn(fmaxf(ag, 0.0f), au) : fmaxf(au, 0.0f);
+            h_compact[k] = h;
+            const int neuron = bucket ? bucket[row] : row;
+            if (h_dense) h_dense[neuron] = h;
+            if (up_dense) up_dense[neuron] = au;
+            if (gate_dense && wg) gate_dense[neuron] = ag;
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Sparse down projection (axpy).  grid = (column tiles of 512, G row groups).  Wave w of block (t, g)
+// takes active rows k = g*4 + w, +4G, ... and accumulates h_k * down_t[row_k][tile] in 8 fp32 registers
+// per lane; the four waves merge through LDS; the partial tile goes to scratch; the block that finishes
+// last for the tile adds the G partials in order, applies the epilogue and stores.  No float atomics,
+// so the sum order -- and the result -- is fixed.  h is rounded to fp16 first and zero rows are skipped
+// as on the CPU path (ggml.c:14420-14431).
+// ---------------------------------------------------------------------------------------------------
+constexpr int kAxpyTile = PI_WAVE * 8;
+
+__device__ void axpy_finish(float * acc, float * lds, float * partial, unsigned int * tile_counter, int cols,
+                            int epi, const float * add1, const float * add2, float * out, int * sflag) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int tile = blockIdx.x, g = blockIdx.y, G = gridDim.y;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) lds[wave * kAxpyTile + lane * 8 + i] = acc[i];
+    __syncthreads();
+    for (int c = threadIdx.x; c < kAxpyTile; c += blockDim.x) {
+        const int col = tile * kAxpyTile + c;
+        if (col < cols) {
+            float s = lds[c];
+            for (int w = 1; w < kWavesPerBlock; ++w) s += lds[w * kAxpyTile + c];
+            partial[(size_t)g * cols + col] = s;
+        }
+    }
+    if (last_block_done(&tile_counter[tile], G, sflag)) {
+        for (int c = threadIdx.x; c < kAxpyTile; c += blockDim.x) {
+            const int col = tile * kAxpyTile + c;
+            if (col < cols) {
+                float s = partial[col];
+                for (int gg = 1; gg < G; ++gg) s += partial[(size_t)gg * cols + col];
+                out[col] = apply_epilogue(s, epi, add1, add2, col);
+            }
+        }
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void sparse_axpy_f16_kernel(const __half * __restrict__ Wd, int cols, const float * __restrict__ h_compact,
+                                                                 const int32_t * __restrict__ list, const int32_t * __restrict__ n_active,
+                                                                 float * partial, unsigned int * tile_counter,
+                                                                 int epi, const float * add1, const float * add2, float * out) {
+    __shared__ float lds[kWavesPerBlock * kAxpyTile];
+    __shared__ int sflag;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int col = blockIdx.x * kAxpyTile + lane * 8;
+    const int n = *n_active;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    if (col < cols) {
+        const int stride = gridDim.y * kWavesPerBlock;
+#pragma unroll 4
+        for (int k = blockIdx.y * kWavesPerBlock + wave; k < n; k += stride) {
+            const float a = pi_round_f16(h_compact[k]);
+            if (a == 0.0f) continue;
+            float wf[8];
+            pi_unpack8(pi_ld_stream(Wd + (size_t)list[k] * cols + col), wf);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] = fmaf(wf[i], a, acc[i]);
+        }
+    }
+    axpy_finish(acc, lds, partial, tile_counter, cols, epi, add1, add2, out, &sflag);
+}
+
+// Q4_0 axpy (ggml_compute_forward_mul_mat_axpy_q4_0, ggml.c:14465-14618; ggml_axpy_q4_0_q8_0, ggml-quants.c:2426):
+// h is quantised to Q8_0 over blocks of 32 *neurons* (in the dense [ff] index space on the CPU).  Here the
+// caller passes h already quantised per active row: hq[k] (int8) and hd[k] (fp16-rounded block scale).
+__global__ __launch_bounds__(kBlock) void sparse_axpy_q4_kernel(const pi_block_q4_0 * __restrict__ Wd, int cols, const int32_t * __restrict__ hq,
+                                                                const float * __restrict__ hd,
+                                                                const int32_t * __restrict__ list, const int32_t * __restrict__ n_active,
+                                                                float * partial, unsigned int * tile_counter,
+                                                                int epi, const float * add1, const float * add2, float * out) {
+    __shared__ float lds[kWavesPerBlock * kAxpyTile];
+    __shared__ int sflag;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    // lane covers 8 columns: a quarter of one 32-weight block -> elements (lane&3)*8 .. +8 of block col/32
+    const int col = blockIdx.x * kAxpyTile + lane * 8;
+    const int nb = cols / 32;
+    const int n = *n_active;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    if (col < cols) {
+        const int blk = col >> 5, sub = (col >> 3) & 3;          // sub 0,1: low nibbles of qs[0..7], qs[8..15]; sub 2,3: high nibbles
+        const int stride = gridDim.y * kWavesPerBlock;
+        for (int k = blockIdx.y * kWavesPerBlock + wave; k < n; k += stride) {
+            const int alpha = hq[k];
+            if (alpha == 0) continue;
+            const pi_block_q4_0 * wb = Wd + (size_t)list[k] * nb + blk;
+            uint16_t dbits; uint32_t q[2];
+            __builtin_memcpy(&dbits, &wb->d, 2);
+            __builtin_memcpy(q, wb->qs + (sub & 1) * 8, 8);
+            const float d = __fmul_rn(pi_f16_from_bits(dbits), hd[k]);
+            const int shift = (sub >> 1) * 4;
+#pragma unroll
+            for (int i = 0; i < 8; ++i) {
+                const int v = (int)((q[i >> 2] >> ((i & 3) * 8 + shift)) & 0xF) - 8;
+                acc[i] = __fadd_rn(acc[i], __fmul_rn((float)(v * alpha), d));
+            }
+        }
+    }
+    axpy_finish(acc, lds, partial, tile_counter, cols, epi, add1, add2, out, &sflag);
+}
+
+// Q8_0 quantisation of h for the Q4_0 axpy.  The CPU path quantises the dense [ff] vector in blocks of 32
+// neurons (inactive neurons contribute zeros), so the scale of an active neuron depends on its 31 block
+// neighbours.  For each active row this reads the neuron's block from the dense vector and emits the
+// int8 value hq[k] and the fp16-rounded block scale hd[k].
+__global__ __launch_bounds__(kBlock) void h_q8_gather_kernel(const float * __restrict__ h_dense, const int32_t * __restrict__ list,
+                                                             const int32_t * __restrict__ n_active, const int32_t * __restrict__ bucket,
+                                                             int32_t * __restrict__ hq, float * __restrict__ hd) {
+    const int n = *n_active;
+    for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < n; k += gridDim.x * blockDim.x) {
+        const int row = list[k];
+        const int neuron = bucket ? bucket[row] : row;
+        const float * blk = h_dense + (neuron & ~31);
+        float amax = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) amax = fmaxf(amax, fabsf(blk[j]));
+        const float d = amax / 127.0f;
+        const float id = (amax != 0.0f) ? 127.0f / amax : 0.0f;
+        hq[k] = (int)rintf(__fmul_rn(h_dense[neuron], id));
+        hd[k] = pi_round_f16(d);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// RoPE + KV store for one token (ggml.c:11163-11325; theta advanced by repeated fp32 multiplication as
+// the CPU path does, so the angle is bit-identical and only cosf/sinf may differ in the last place).
+// grid = n_head + 2*n_head_kv blocks of hd/2 threads.
+// ---------------------------------------------------------------------------------------------------
+__global__ void rope_kv_store_kernel(const float * __restrict__ qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
+                                     const int32_t * __restrict__ pos_p, int n_ctx, float * __restrict__ q_rot,
+                                     __half * __restrict__ k_cache, __half * __restrict__ v_cache) {
+    const int h = blockIdx.x, i = threadIdx.x;           // i = pair index
+    const int pos = *pos_p;
+    if (h < n_head + n_head_kv) {
+        const float * src = qkv + (size_t)h * hd;
+        float theta = (float)pos;
+        for (int j = 0; j < i; ++j) theta = __fmul_rn(theta, theta_scale);
+        const float c = cosf(theta), s = sinf(theta);
+        const int i0 = (mode & 2) ? i : 2 * i;
+        const int i1 = (mode & 2) ? i + hd / 2 : 2 * i + 1;
+        const float x0 = src[i0], x1 = src[i1];
+        const float y0 = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, s));
+        const float y1 = __fadd_rn(__fmul_rn(x0, s), __fmul_rn(x1, c));
+        if (h < n_head) {
+            q_rot[(size_t)h * hd + i0] = y0;
+            q_rot[(size_t)h * hd + i1] = y1;
+        } else {
+            __half * dst = k_cache + ((size_t)(h - n_head) * n_ctx + pos) * hd;
+            dst[i0] = __float2half_rn(y0);
+            dst[i1] = __float2half_rn(y1);
+        }
+    } else {
+        const int hv = h - n_head - n_head_kv;
+        const float * src = qkv + (size_t)(n_head + n_head_kv + hv) * hd;
+        __half * dst = v_cache + ((size_t)hv * n_ctx + pos) * hd;
+        dst[2 * i]     = __float2half_rn(src[2 * i]);
+        dst[2 * i + 1] = __float2half_rn(src[2 * i + 1]);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Decode attention: one block per query head over cells [0, pos].
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void attn_decode_kernel(const float * __restrict__ q_rot, const __half * __restrict__ k_cache,
+                                                             const __half * __restrict__ v_cache, int n_head, int n_head_kv, int hd,
+                                                             int n_ctx, const int32_t * __restrict__ pos_p, float * __restrict__ out) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float * s    = reinterpret_cast<float *>(smem);               // [n_kv] scores, then probabilities
+    float * part = s + n_ctx;                                     // [groups][hd] partial outputs
+    __shared__ double red[16];
+    __shared__ float redf[16];
+    const int h = blockIdx.x, kvh = h / (n_head / n_head_kv);
+    const int n_kv = *pos_p + 1;
+    const int lpp = hd / 8;                                       // lanes per position (16 B each)
+    const int tid = threadIdx.x;
+    const int sub = tid % lpp, grp = tid / lpp, ngrp = blockDim.x / lpp;
+    const float scale = 1.0f / sqrtf((float)hd);
+
+    // q chunk of this lane, rounded to fp16 as the CPU dot does
+    float qf[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qf[i] = pi_round_f16(q_rot[(size_t)h * hd + sub * 8 + i]);
+
+    const __half * kb = k_cache + (size_t)kvh * n_ctx * hd;
+    for (int c0 = 0; c0 < n_kv; c0 += ngrp) {
+        const int c = c0 + grp;
+        float d = 0.0f;
+        if (c < n_kv) d = pi_dot8(pi_ld16(kb + (size_t)c * hd + sub * 8), qf, 0.0f);
+        for (int o = lpp / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, PI_WAVE);
+        if (c < n_kv && sub == 0) s[c] = __fmul_rn(d, scale);
+    }
+    __syncthreads();
+
+    float mx = -INFINITY;
+    for (int c = tid; c < n_kv; c += blockDim.x) mx = fmaxf(mx, s[c]);
+    mx = block_max_f32(mx, redf);
+    double sum = 0.0;
+    for (int c = tid; c < n_kv; c += blockDim.x) {
+        // exp through fp16 in and out: the CPU path's lookup table holds fp16(expf(fp32(fp16(x - max))))
+        const float e = pi_round_f16(expf(pi_round_f16(__fsub_rn(s[c], mx))));
+        s[c] = e;
+        sum += (double)e;
+    }
+    sum = block_sum_f64(sum, red);                                // includes the barriers that publish s[]
+    const float inv = (float)(1.0 / sum);
+
+    const __half * vb = v_cache + (size_t)kvh * n_ctx * hd;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    for (int c = grp; c < n_kv; c += ngrp) {
+        const float p = pi_round_f16(__fmul_rn(s[c], inv));       // probabilities are rounded to fp16 before the V product
+        float vf[8];
+        pi_unpack8(pi_ld16(vb + (size_t)c * hd + sub * 8), vf);
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(vf[i], p, acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) part[grp * hd + sub * 8 + i] = acc[i];
+    __syncthreads();
+    for (int e = tid; e < hd; e += blockDim.x) {
+        float v = part[e];
+        for (int g = 1; g < ngrp; ++g) v += part[g * hd + e];
+        out[(size_t)h * hd + e] = v;
+    }
+}
+
+__global__ void embed_f16_kernel(const __half * __restrict__ table, int cols, const int32_t * __restrict__ token, float * __restrict__ x) {
+    const __half * row = table + (size_t)(*token) * cols;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < cols; i += gridDim.x * blockDim.x) x[i] = __half2float(row[i]);
+}
+__global__ void embed_q4_kernel(const pi_block_q4_0 * __restrict__ table, int cols, const int32_t * __restrict__ token, float * __restrict__ x) {
+    const pi_block_q4_0 * row = table + (size_t)(*token) * (cols / 32);
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < cols; i += gridDim.x * blockDim.x) {
+        const pi_block_q4_0 * b = row + (i >> 5);
+        uint16_t dbits; __builtin_memcpy(&dbits, &b->d, 2);
+        const int j = i & 31;
+        const int q = (j < 16) ? (b->qs[j] & 0x0F) : (b->qs[j - 16] >> 4);
+        x[i] = __fmul_rn((float)(q - 8), pi_f16_from_bits(dbits));
+    }
+}
+
+// first maximum wins (std::max_element, llama.cpp:8617-8631)
+__global__ __launch_bounds__(1024) void argmax_kernel(const float * __restrict__ logits, int n, int32_t * __restrict__ token_out) {
+    __shared__ float bv[16];
+    __shared__ int   bi[16];
+    float best = -INFINITY; int idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) { const float v = logits[i]; if (v > best) { best = v; idx = i; } }
+    if (idx == 0x7fffffff) { idx = n; }                          // thread saw nothing above -inf
+#pragma unroll
+    for (int o = PI_WAVE / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, PI_WAVE); const int oi = __shfl_xor(idx, o, PI_WAVE);
+        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+    }
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) { bv[wave] = best; bi[wave] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x >> 6); ++w)
+            if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
+        *token_out = idx < n ? idx : 0;
+    }
+}
+
+// counter-based N(0, std^2): two 32-bit hashes -> Box-Muller; deterministic in (seed, index)
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+__global__ void fill_normal_f16_kernel(__half * __restrict__ p, size_t n, uint64_t seed, float std, const float * __restrict__ row_bias, int cols) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const uint64_t r = mix64(seed * 0xD1342543DE82EF95ull + i);
+        const float u1 = ((uint32_t)(r >> 32) + 1.0f) * (1.0f / 4294967296.0f);
+        const float u2 = (uint32_t)r * (1.0f / 4294967296.0f);
+        float v = sqrtf(-2.0f * logf(u1)) * cosf(6.28318530718f * u2) * std;
+        if (row_bias) v += row_bias[i / cols];
+        p[i] = __float2half_rn(v);
+    }
+}
+
+NormArgs to_norm(const pi_norm * n) {
+    NormArgs a{0, 0.0f, nullptr, nullptr};
+    if (n) { a.kind = n->kind; a.eps = n->eps; a.w = n->w; a.b = n->b; }
+    return a;
+}
+
+}  // namespace
+
+// =====================================================================================================
+// C-ABI launchers
+// =====================================================================================================
+struct pi_workspace {
+    int max_ff, max_d;
+    uint32_t *     words;          // [max_ff/32 + 1]
+    unsigned int * counters;       // [64]: [0] predictor ticket, [1..] axpy tile tickets
+    float *        partial;        // [kAxpyGroups][max_d]
+    int32_t *      hq;             // [max_ff]  Q4_0 axpy: int8 value of h per active row
+    float *        hd;             // [max_ff]  and its Q8_0 block scale
+};
+constexpr int kAxpyGroups = 32;
+
+extern "C" {
+
+pi_workspace * pi_workspace_create(int max_ff, int max_d) {
+    if (max_ff <= 0 || max_d <= 0 || (max_d + kAxpyTile - 1) / kAxpyTile > 62) { pi::set_error("pi_workspace_create: bad sizes"); return nullptr; }
+    pi_workspace * ws = new pi_workspace{};
+    ws->max_ff = max_ff; ws->max_d = max_d;
+    ws->words    = (uint32_t *)pi_malloc(sizeof(uint32_t) * (max_ff / 32 + 2));
+    ws->counters = (unsigned int *)pi_malloc(sizeof(unsigned int) * 64);
+    ws->partial  = (float *)pi_malloc(sizeof(float) * (size_t)kAxpyGroups * max_d);
+    ws->hq       = (int32_t *)pi_malloc(sizeof(int32_t) * max_ff);
+    ws->hd       = (float *)pi_malloc(sizeof(float) * max_ff);
+    if (!ws->words || !ws->counters || !ws->partial || !ws->hq || !ws->hd) {
+        pi_workspace_destroy(ws); return nullptr;
+    }
+    pi_memset(ws->counters, 0, sizeof(unsigned int) * 64);
+    return ws;
+}
+int pi_workspace_destroy(pi_workspace * ws) {
+    if (!ws) return PI_OK;
+    pi_free(ws->words); pi_free(ws->counters); pi_free(ws->partial); pi_free(ws->hq); pi_free(ws->hd);
+    delete ws;
+    return PI_OK;
+}
+
+int pi_k_gemv(int wtype, const void * W, int rows, int cols, const float * x, const pi_norm * norm,
+              int epilogue, const float * add1, const float * add2, float * y, pi_stream_t stream) {
+    if (!W || !x || !y || rows <= 0 || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_gemv: null pointer or empty shape");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_gemv: bad epilogue arguments");
+    hipStream_t st = (hipStream_t)stream;
+    const NormArgs na = to_norm(norm);
+    const int rpw = rows >= 8192 ? 4 : rows >= 2048 ? 2 : 1;
+    const int n_groups = (rows + rpw - 1) / rpw;
+    int blocks = (n_groups + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks > 4096) blocks = 4096;
+    if (wtype == PI_TYPE_F16) {
+        if (cols % 8) return pi::fail(PI_E_ARG, "pi_k_gemv: F16 needs cols % 8 == 0");
+        const size_t sh = (size_t)cols * 2;
+        if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv: cols too large for LDS staging");
+        const __half * w = (const __half *)W;
+        if (rpw == 4)      hipLaunchKernelGGL(gemv_f16_kernel<4>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        else if (rpw == 2) hipLaunchKernelGGL(gemv_f16_kernel<2>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        else               hipLaunchKernelGGL(gemv_f16_kernel<1>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+    } else if (wtype == PI_TYPE_Q4_0) {
+        if (cols % 32) return pi::fail(PI_E_ARG, "pi_k_gemv: Q4_0 needs cols % 32 == 0");
+        const size_t sh = (size_t)cols + (size_t)(cols / 32) * 4 + (size_t)cols * 4;
+        if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv: cols too large for LDS staging");
+        const pi_block_q4_0 * w = (const pi_block_q4_0 *)W;
+        if (rpw == 4)      hipLaunchKernelGGL(gemv_q4_kernel<4>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        else if (rpw == 2) hipLaunchKernelGGL(gemv_q4_kernel<2>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        else               hipLaunchKernelGGL(gemv_q4_kernel<1>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+    } else {
+        return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv: weight type must be F16 or Q4_0");
+    }
+    return pi::check_launch("pi_k_gemv");
+}
+
+int pi_k_predictor_fc2(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                       const int32_t * bucket, int n_bucket, float * logits,
+                       int32_t * active_rows, int32_t * n_active, float * zero_fill, pi_workspace * ws, pi_stream_t stream) {
+    if (!fc2_f16 || !hidden || !logits || !active_rows || !n_active || !ws) return pi::fail(PI_E_ARG, "pi_k_predictor_fc2: null pointer");
+    if (ff <= 0 || r <= 0 || r % 8 || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_predictor_fc2: bad shape (r % 8 == 0, ff <= workspace)");
+    if (bucket && (n_bucket < 0 || n_bucket > ff)) return pi::fail(PI_E_ARG, "pi_k_predictor_fc2: bad bucket size");
+    const int blocks = (ff + 31) / 32;
+    hipLaunchKernelGGL(pred_fc2_kernel, dim3(blocks), dim3(kBlock), (size_t)r * 2, (hipStream_t)stream,
+                       (const __half *)fc2_f16, hidden, ff, r, threshold, bucket, n_bucket, logits, ws->words, ws->counters, active_rows, n_active, zero_fill);
+    return pi::check_launch("pi_k_predictor_fc2");
+}
+
+int pi_k_compact_active(const float * logits, int ff, float threshold, const int32_t * bucket, int n_bucket,
+                        int32_t * active_rows, int32_t * n_active, pi_workspace * ws, pi_stream_t stream) {
+    if (!logits || !active_rows || !n_active || !ws || ff <= 0 || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_compact_active: bad arguments");
+    if (bucket && (n_bucket < 0 || n_bucket > ff)) return pi::fail(PI_E_ARG, "pi_k_compact_active: bad bucket size");
+    hipLaunchKernelGGL(compact_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logits, ff, threshold, bucket, n_bucket, ws->words, active_rows, n_active);
+    return pi::check_launch("pi_k_compact_active");
+}
+
+int pi_k_sparse_upgate(int wtype, const void * up, const void * gate, int cols, const float * x, const pi_norm * norm,
+                       const int32_t * active_rows, const int32_t * n_active, const int32_t * bucket,
+                       float * h_compact, float * h_dense, float * up_dense, float * gate_dense, pi_stream_t stream) {
+    if (!up || !x || !active_rows || !n_active || !h_compact || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_sparse_upgate: null pointer or empty shape");
+    const NormArgs na = to_norm(norm);
+    const int blocks = 1024;       // fixed grid: the active count lives on the device; idle blocks exit at once
+    if (wtype == PI_TYPE_F16) {
+        if (cols % 8 || (size_t)cols * 2 > 60 * 1024) return pi::fail(PI_E_ARG, "pi_k_sparse_upgate: bad cols for F16");
+        hipLaunchKernelGGL(sparse_upgate_f16_kernel, dim3(blocks), dim3(kBlock), (size_t)cols * 2, (hipStream_t)stream,
+                           (const __half *)up, (const __half *)gate, x, na, cols, active_rows, n_active, bucket, h_compact, h_dense, up_dense, gate_dense);
+    } else if (wtype == PI_TYPE_Q4_0) {
+        const size_t sh = (size_t)cols + (size_t)(cols / 32) * 4 + (size_t)cols * 4;
+        if (cols % 32 || sh > 60 * 1024) return pi::fail(PI_E_ARG, "pi_k_sparse_upgate: bad cols for Q4_0");
+        hipLaunchKernelGGL(sparse_upgate_q4_kernel, dim3(blocks), dim3(kBlock), sh, (hipStream_t)stream,
+                           (const pi_block_q4_0 *)up, (const pi_block_q4_0 *)gate, x, na, cols, active_rows, n_active, bucket, h_compact, h_dense, up_dense, gate_dense);
+    } else {
+        return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_upgate: weight type must be F16 or Q4_0");
+    }
+    return pi::check_launch("pi_k_sparse_upgate");
+}
+
+int pi_k_sparse_axpy(int wtype, const void * down_t, int cols, const float * h_compact, const float * h_dense, const int32_t * bucket,
+                     const int32_t * active_rows, const int32_t * n_active,
+                     int epilogue, const float * add1, const float * add2, float * out,
+                     pi_workspace * ws, pi_stream_t stream) {
+    if (!down_t || !h_compact || !active_rows || !n_active || !out || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: null pointer");
+    if (cols <= 0 || cols > ws->max_d) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: cols exceeds the workspace");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: bad epilogue arguments");
+    const int tiles = (cols + kAxpyTile - 1) / kAxpyTile;
+    const dim3 grid(tiles, kAxpyGroups);
+    hipStream_t st = (hipStream_t)stream;
+    if (wtype == PI_TYPE_F16) {
+        if (cols % 8) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: F16 needs cols % 8 == 0");
+        hipLaunchKernelGGL(sparse_axpy_f16_kernel, grid, dim3(kBlock), 0, st,
+                           (const __half *)down_t, cols, h_compact, active_rows, n_active, ws->partial, ws->counters + 1, epilogue, add1, add2, out);
+    } else if (wtype == PI_TYPE_Q4_0) {
+        if (cols % 32) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: Q4_0 needs cols % 32 == 0");
+        if (!h_dense) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: Q4_0 needs the dense h vector (block scales span 32 neurons)");
+        hipLaunchKernelGGL(h_q8_gather_kernel, dim3(64), dim3(kBlock), 0, st, h_dense, active_rows, n_active, bucket, ws->hq, ws->hd);
+        hipLaunchKernelGGL(sparse_axpy_q4_kernel, grid, dim3(kBlock), 0, st,
+                           (const pi_block_q4_0 *)down_t, cols, ws->hq, ws->hd, active_rows, n_active, ws->partial, ws->counters + 1, epilogue, add1, add2, out);
+    } else {
+        return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_axpy: weight type must be F16 or Q4_0");
+    }
+    return pi::check_launch("pi_k_sparse_axpy");
+}
+
+int pi_k_rope_kv_store(const float * qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
+                       const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache, pi_stream_t stream) {
+    if (!qkv || !pos || !q_rot || !k_cache || !v_cache) return pi::fail(PI_E_ARG, "pi_k_rope_kv_store: null pointer");
+    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd <= 0 || hd % 2 || hd / 2 > 1024 || (mode != 0 && mode != 2))
+        return pi::fail(PI_E_ARG, "pi_k_rope_kv_store: bad head geometry or mode");
+    hipLaunchKernelGGL(rope_kv_store_kernel, dim3(n_head + 2 * n_head_kv), dim3(hd / 2), 0, (hipStream_t)stream,
+                       qkv, n_head, n_head_kv, hd, mode, theta_scale, pos, n_ctx, q_rot, (__half *)k_cache, (__half *)v_cache);
+    return pi::check_launch("pi_k_rope_kv_store");
+}
+
+int pi_k_attn_decode(const float * q_rot, const void * k_cache, const void * v_cache, int n_head, int n_head_kv,
+                     int hd, int n_ctx, const int32_t * pos, float * out, pi_stream_t stream) {
+    if (!q_rot || !k_cache || !v_cache || !pos || !out) return pi::fail(PI_E_ARG, "pi_k_attn_decode: null pointer");
+    if (hd % 8 || kBlock % (hd / 8) || PI_WAVE % (hd / 8) || n_head % n_head_kv) return pi::fail(PI_E_ARG, "pi_k_attn_decode: head size must be 8 * (a divisor of 64)");
+    const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd);
+    if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_decode: context too long for the single-pass kernel");
+    hipLaunchKernelGGL(attn_decode_kernel, dim3(n_head), dim3(kBlock), sh, (hipStream_t)stream,
+                       q_rot, (const __half *)k_cache, (const __half *)v_cache, n_head, n_head_kv, hd, n_ctx, pos, out);
+    return pi::check_launch("pi_k_attn_decode");
+}
+
+int pi_k_embed(int wtype, const void * table, int cols, const int32_t * token, float * x, pi_stream_t stream) {
+    if (!table || !token || !x || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_embed: bad arguments");
+    const int blocks = (cols + 255) / 256;
+    if (wtype == PI_TYPE_F16)       hipLaunchKernelGGL(embed_f16_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const __half *)table, cols, token, x);
+    else if (wtype == PI_TYPE_Q4_0) hipLaunchKernelGGL(embed_q4_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const pi_block_q4_0 *)table, cols, token, x);
+    else return pi::fail(PI_E_UNSUPPORTED, "pi_k_embed: table type must be F16 or Q4_0");
+    return pi::check_launch("pi_k_embed");
+}
+
+int pi_k_argmax(const float * logits, int n, int32_t * token_out, pi_stream_t stream) {
+    if (!logits || !token_out || n <= 0) return pi::fail(PI_E_ARG, "pi_k_argmax: bad arguments");
+    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logits, n, token_out);
+    return pi::check_launch("pi_k_argmax");
+}
+
+int pi_fill_normal_f16(void * dptr, size_t n, uint64_t seed, float std, const float * row_bias, int cols, pi_stream_t stream) {
+    if (!dptr || (row_bias && cols <= 0)) return pi::fail(PI_E_ARG, "pi_fill_normal_f16: bad arguments");
+    if (n == 0) return PI_OK;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(fill_normal_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (__half *)dptr, n, seed, std, row_bias, cols);
+    return pi::check_launch("pi_fill_normal_f16");
+}
+
+}  // extern "C"

@@ -1,0 +1,83 @@
+"""Host-side mirror of the reference's operator sequence for one sparse FFN block
+(llm_build_ffn_sparse, llama.cpp:4652-4757), driving the HIP launchers through the C ABI.
+Used by the parity tests and the layer-level benchmark; the fused decode loop lives in the C++ engine.
+"""
+import ctypes as C
+
+import numpy as np
+
+from . import lib as pl
+from .lib import DevBuf, check
+
+
+class SparseFFN:
+    """Device-resident weights of one layer + the launch sequence
+    fc1 -> relu -> fc2+threshold+compaction -> sparse up/gate -> sparse axpy.
+
+    bucket (optional int32 array): the layer holds only the GPU-resident neurons (rows bucket[i] of the
+    full matrices, compact, in bucket order) as llama.cpp's slice_ffn_mat_to_gpu does (llama.cpp:2898-2967).
+    """
+
+    def __init__(self, d, ff, r, wtype, up, gate, down_t, fc1, fc2, threshold=0.0, bucket=None,
+                 norm_kind=pl.NORM_NONE, norm_w=None, norm_b=None, eps=1e-5):
+        self.L = pl.init()
+        self.d, self.ff, self.r, self.wtype, self.thr = d, ff, r, wtype, float(threshold)
+        self.bucket_host = None if bucket is None else np.ascontiguousarray(bucket, np.int32)
+        sel = (lambda a: a) if bucket is None else (lambda a: np.ascontiguousarray(a[self.bucket_host]))
+        self.up = DevBuf(host=sel(up))
+        self.gate = DevBuf(host=sel(gate)) if gate is not None else None
+        self.down = DevBuf(host=sel(down_t))
+        self.fc1, self.fc2 = DevBuf(host=fc1), DevBuf(host=fc2)
+        self.bucket = DevBuf(host=self.bucket_host) if bucket is not None else None
+        self.n_bucket = 0 if bucket is None else int(self.bucket_host.size)
+        self.norm_kind, self.eps = norm_kind, eps
+        self.norm_w = DevBuf(host=np.asarray(norm_w, np.float32)) if norm_w is not None else None
+        self.norm_b = DevBuf(host=np.asarray(norm_b, np.float32)) if norm_b is not None else None
+        self.ws = self.L.pi_workspace_create(ff, d)
+        if not self.ws:
+            raise pl.PiError(self.L.pi_last_error().decode())
+        f4 = 4
+        self.x, self.xp = DevBuf(d * f4), DevBuf(d * f4)
+        self.hidden, self.logits = DevBuf(r * f4), DevBuf(ff * f4)
+        self.list, self.n_active = DevBuf(ff * 4), DevBuf.zeros(4)
+        self.h_c = DevBuf(ff * f4)
+        self.h_dense, self.up_dense, self.gate_dense = DevBuf.zeros(ff * f4), DevBuf.zeros(ff * f4), DevBuf.zeros(ff * f4)
+        self.out = DevBuf(d * f4)
+        self.resid = DevBuf.zeros(d * f4)
+
+    def launch(self, stream=None, dense_outputs=True, epilogue=pl.EPI_NONE):
+        L, p = self.L, (lambda b: b.ptr if b is not None else None)
+        check(L.pi_k_gemv(pl.F16, self.fc1.ptr, self.r, self.d, self.xp.ptr, None, pl.EPI_RELU, None, None, self.hidden.ptr, stream), "fc1")
+        check(L.pi_k_predictor_fc2(self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, p(self.bucket), self.n_bucket,
+                                   self.logits.ptr, self.list.ptr, self.n_active.ptr,
+                                   self.h_dense.ptr if (dense_outputs or self.wtype == pl.Q4_0) else None, self.ws, stream), "fc2")
+        nrm = pl.norm_arg(self.norm_kind, self.eps, self.norm_w, self.norm_b)
+        check(L.pi_k_sparse_upgate(self.wtype, self.up.ptr, p(self.gate), self.d, self.x.ptr, nrm, self.list.ptr, self.n_active.ptr,
+                                   p(self.bucket), self.h_c.ptr,
+                                   self.h_dense.ptr if (dense_outputs or self.wtype == pl.Q4_0) else None,
+                                   self.up_dense.ptr if dense_outputs else None,
+                                   self.gate_dense.ptr if dense_outputs else None, stream), "upgate")
+        check(L.pi_k_sparse_axpy(self.wtype, self.down.ptr, self.d, self.h_c.ptr,
+                                 self.h_dense.ptr if self.wtype == pl.Q4_0 else None, p(self.bucket),
+                                 self.list.ptr, self.n_active.ptr, epilogue, self.resid.ptr if epilogue else None, None,
+                                 self.out.ptr, self.ws, stream), "axpy")
+
+    def forward(self, x_ffn, x_pred):
+        """One token.  Returns dict(logits, active, up, gate, h, out) as numpy arrays (dense vectors are
+        neuron-indexed; rows outside the GPU bucket stay zero)."""
+        self.x.upload(np.asarray(x_ffn, np.float32))
+        self.xp.upload(np.asarray(x_pred, np.float32))
+        for b in (self.up_dense, self.gate_dense):
+            check(self.L.pi_memset(b.ptr, 0, b.nbytes), "memset")
+        self.launch()
+        pl.sync()
+        n = int(self.n_active.download(np.int32)[0])
+        return dict(logits=self.logits.download(np.float32), active=self.list.download(np.int32, n),
+                    up=self.up_dense.download(np.float32), gate=self.gate_dense.download(np.float32),
+                    h=self.h_dense.download(np.float32), h_compact=self.h_c.download(np.float32, n),
+                    out=self.out.download(np.float32))
+
+    def close(self):
+        if self.ws:
+            self.L.pi_workspace_destroy(self.ws)
+            self.ws = None

@@ -153,6 +153,74 @@ PI_API int pi_k_embed(int wtype, const void * table, int cols, const int32_t * t
 /* greedy sampling: *token_out = index of the first maximum (llama_sample_token_greedy, llama.cpp:8617-8631) */
 PI_API int pi_k_argmax(const float * logits, int n, int32_t * token_out, pi_stream_t stream);
 
+/* ---- decode loop with resident weights ------------------------------------------------------------- */
+
+enum { PI_ARCH_LLAMA = 0, PI_ARCH_FALCON = 1 };
+
+/* the llama_hparams fields this path reads (llama.cpp:1207-1270) */
+typedef struct pi_hparams {
+    int32_t arch;
+    int32_t n_embd, n_ff, n_head, n_head_kv, n_layer, n_vocab, n_ctx;
+    float   norm_eps, rope_freq_base, sparse_threshold;
+} pi_hparams;
+
+/* tensor roles; names as llama.cpp:403-461 (blk.N.<role>.weight).  layer = -1 for the global ones. */
+enum {
+    PI_T_TOK_EMBD = 0, PI_T_OUTPUT_NORM, PI_T_OUTPUT_NORM_B, PI_T_OUTPUT,
+    PI_T_ATTN_NORM, PI_T_ATTN_NORM_B, PI_T_ATTN_NORM_2, PI_T_ATTN_NORM_2_B,
+    PI_T_WQ, PI_T_WK, PI_T_WV, PI_T_WQKV, PI_T_WO,
+    PI_T_FFN_NORM, PI_T_FFN_GATE, PI_T_FFN_UP, PI_T_FFN_DOWN_T,
+    PI_T_FC1, PI_T_FC2, PI_T_GPU_IDX, PI_T_GPU_BUCKET,
+    PI_T_COUNT
+};
+
+typedef struct pi_model pi_model;
+
+/* llama_load_model_from_file + llama_new_context_with_model (llama.cpp:9789, 9819) without the file
+ * format: the caller hands over tensors one by one. */
+PI_API pi_model * pi_model_create(const pi_hparams * hp);
+PI_API void       pi_model_free(pi_model * m);
+
+/*
+ * Give the model one tensor.  `data` is a host pointer (copied to HBM) or, with on_device != 0, a device
+ * pointer the model adopts without copying (the caller keeps ownership).  ne0 = contiguous dimension,
+ * ne1 = rows.  wq/wk/wv are packed into one [n_embd + 2*n_embd_gqa][n_embd] matrix at finalize.
+ * FFN matrices of a layer that has a PI_T_GPU_BUCKET are given FULL-SIZE on the host: the bucket's rows are
+ * sliced into compact device matrices (slice_ffn_mat_to_gpu, llama.cpp:2898-2967) and the host copy is
+ * kept (borrowed, must outlive the model) for the cold neurons that run on the CPU.
+ */
+PI_API int pi_model_set_tensor(pi_model * m, int layer, int kind, int type, const void * data,
+                               int64_t ne0, int64_t ne1, int on_device);
+PI_API int pi_model_finalize(pi_model * m);
+PI_API int pi_model_kv_clear(pi_model * m);                    /* llama_kv_cache_clear, llama.h:367 */
+
+/*
+ * llama_decode (llama.cpp:10672) for one sequence: evaluates tokens[0..n_tokens) at positions
+ * n_past..n_past+n_tokens-1, stores K/V, and leaves the logits of the last token on the device.
+ * logits_out (optional, host, fp32 [n_vocab]) receives them (llama_get_logits).
+ * Returns the greedy token of the last position (llama_sample_token_greedy) or a negative error.
+ */
+PI_API int pi_model_decode(pi_model * m, const int32_t * tokens, int n_tokens, int n_past, float * logits_out);
+
+/*
+ * The batch-1 greedy token loop of examples/main (main.cpp:462-623 with temp == 0): continues from the
+ * state pi_model_decode left (next token = its greedy choice), generates n_steps tokens entirely on the
+ * device (one captured HIP graph replayed per token) and writes them to out_tokens (host).
+ * ms_out (optional) receives the device time of the loop measured with events on the model's stream.
+ */
+PI_API int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * ms_out);
+
+/* parity hooks: when enabled, pi_model_decode also records, for its LAST token, each layer's FFN output
+ * [n_layer][n_embd] (before the residual add), predictor logits [n_layer][n_ff], active-row count [n_layer]
+ * and the vector the FFN block read [n_layer][n_embd] (LLaMA: ffn_inp; Falcon: the layer input; both before
+ * the norm; it is also the predictor's input).  Any output pointer may be NULL. */
+PI_API int pi_model_set_capture(pi_model * m, int enable);
+PI_API int pi_model_get_capture(pi_model * m, float * ffn_out, float * pred_logits, int32_t * n_active, float * ffn_src);
+
+/* for each of the n_steps tokens of the most recent pi_model_generate: the sum over layers of the active-row
+ * counts (feeds the touched-bytes accounting of the benchmark) */
+PI_API int pi_model_step_active(pi_model * m, int32_t * per_step_total, int n_steps);
+
 #ifdef __cplusplus
 }
 #endif

@@ -499,7 +499,7 @@ struct pio_model {
     uint16_t  * k_cache;          /* [n_layer][n_ctx][n_embd_gqa] */
     uint16_t  * v_cache;          /* [n_layer][n_embd_gqa][n_ctx] */
     int32_t   * zero_gpu_idx;     /* used when a layer has no GPU_IDX: everything is computed (llama.cpp:2984-2990) */
-    float     * cap_ffn, * cap_logits;
+    float     * cap_ffn, * cap_logits, * cap_src;
 };
 
 pio_model * pio_model_new(const pio_hparams * hp) {
@@ -528,7 +528,7 @@ void pio_model_kv_clear(pio_model * m) {
     const size_t kv = (size_t)m->hp.n_layer * m->hp.n_ctx * (m->hp.n_embd / m->hp.n_head) * m->hp.n_head_kv;
     memset(m->k_cache, 0, kv * 2); memset(m->v_cache, 0, kv * 2);
 }
-void pio_model_set_capture(pio_model * m, float * ffn_out, float * pred_logits) { m->cap_ffn = ffn_out; m->cap_logits = pred_logits; }
+void pio_model_set_capture(pio_model * m, float * ffn_out, float * pred_logits, float * ffn_src) { m->cap_ffn = ffn_out; m->cap_logits = pred_logits; m->cap_src = ffn_src; }
 
 /* embedding gather: ggml_compute_forward_get_rows, ggml.c:10402 (dequantise the row to fp32) */
 static int get_row(const pio_tensor * t, int64_t row, float * y) {
@@ -576,6 +576,7 @@ int pio_model_eval(pio_model * m, const int32_t * tokens, const int32_t * pos, c
     float * ffi  = (float *)malloc(sizeof(float) * nd);
     float * ffo  = (float *)malloc(sizeof(float) * nd);
     float * lgt  = (float *)malloc(sizeof(float) * (size_t)ff * T);
+    float * inpL_in = (float *)malloc(sizeof(float) * nd);
 
     for (int t = 0; t < T; ++t) {
         if (tokens[t] < 0 || tokens[t] >= hp->n_vocab) { rc = 1; goto done; }
@@ -587,6 +588,7 @@ int pio_model_eval(pio_model * m, const int32_t * tokens, const int32_t * pos, c
         uint16_t * vc = m->v_cache + (size_t)il * hp->n_ctx * gqa;
         const int32_t * gid = L[PIO_T_GPU_IDX].data ? (const int32_t *)L[PIO_T_GPU_IDX].data : m->zero_gpu_idx;
         const int r = (int)L[PIO_T_FC1].ne1;
+        memcpy(inpL_in, inpL, sizeof(float) * nd);
         if (!falcon) {
             norm_affine(1, inpL, d, T, hp->norm_eps, &L[PIO_T_ATTN_NORM], NULL, nrm);
             rc |= mm(&L[PIO_T_WQ], nrm, T, q, n_threads);
@@ -627,6 +629,7 @@ int pio_model_eval(pio_model * m, const int32_t * tokens, const int32_t * pos, c
                                  nrm, inpL, gid, hp->sparse_threshold, n_threads, lgt, NULL, NULL, NULL, ffo);
             for (size_t i = 0; i < nd; ++i) { const float a = ffo[i] + cur[i]; inpL[i] = a + inpL[i]; }
         }
+        if (m->cap_src)    memcpy(m->cap_src    + (size_t)il * nd, falcon ? inpL_in : ffi, sizeof(float) * nd);
         if (m->cap_ffn)    memcpy(m->cap_ffn    + (size_t)il * nd,              ffo, sizeof(float) * nd);
         if (m->cap_logits) memcpy(m->cap_logits + (size_t)il * (size_t)ff * T,  lgt, sizeof(float) * (size_t)ff * T);
     }
@@ -637,7 +640,7 @@ int pio_model_eval(pio_model * m, const int32_t * tokens, const int32_t * pos, c
     }
 done:
     free(inpL); free(cur); free(nrm); free(nrm2); free(qkv); free(q); free(k); free(v); free(qr); free(kr);
-    free(att); free(ffi); free(ffo); free(lgt);
+    free(att); free(ffi); free(ffo); free(lgt); free(inpL_in);
     return rc;
 }
 

@@ -104,9 +104,10 @@ PIO_API void        pio_model_free(pio_model * m);
 PIO_API int         pio_model_set_tensor(pio_model * m, int layer, int kind, int type, const void * data, int64_t ne0, int64_t ne1);
 PIO_API void        pio_model_kv_clear(pio_model * m);
 
-/* optional per-layer captures, each may be NULL: ffn_out [n_layer][T][n_embd],
- * pred_logits [n_layer][T][n_ff]; they are filled by the next pio_model_eval call */
-PIO_API void        pio_model_set_capture(pio_model * m, float * ffn_out, float * pred_logits);
+/* optional per-layer captures, each may be NULL: ffn_out [n_layer][T][n_embd], pred_logits [n_layer][T][n_ff],
+ * ffn_src [n_layer][T][n_embd] (the vector the FFN block reads, before its norm: LLaMA ffn_inp, Falcon the layer
+ * input); they are filled by the next pio_model_eval call */
+PIO_API void        pio_model_set_capture(pio_model * m, float * ffn_out, float * pred_logits, float * ffn_src);
 
 /*
  * One llama_decode of T tokens: tokens[T], pos[T], kv_slot[T] (cache cell each token is written to),

@@ -1,0 +1,22 @@
+// CPU share of a hybrid (hot/cold split) layer: the neurons that are not GPU-resident are computed on host
+// threads from the same predictor logits and merged into the layer output
+// (llm_build_sparse_mul_mat / llm_build_sparse_axpy hybrid variants, llama.cpp:4581-4593, 4635-4646).
+#pragma once
+
+#include <hip/hip_runtime.h>
+
+struct pi_model;
+
+namespace pi {
+
+struct ColdPath;
+
+ColdPath * cold_create(pi_model * m);
+void       cold_destroy(ColdPath * c);
+// Runs after the GPU share's up/gate launch of layer `il` has been queued on `st`; leaves the merged layer
+// output (cold + hot + residuals) in m->x2.
+int        cold_layer_merge(ColdPath * c, int il, pi_model * m, hipStream_t st);
+
+int add_vec(float * y, const float * a, int n, hipStream_t st);
+
+}  // namespace pi

@@ -1,0 +1,452 @@
+// Decode loop with resident weights: the per-token operator sequence that llama.cpp builds as a ggml graph
+// (build_llama_variants, llama.cpp:4949-5084; build_falcon, llama.cpp:5326-5468; llm_build_ffn_sparse,
+// llama.cpp:4652-4757) issued as a fixed chain of fused HIP kernels on one stream and, for the greedy
+// token loop, captured once into a HIP graph and replayed per token (the reference rebuilds and walks a
+// ~40-node-per-layer graph every token, llama.cpp:6408, 6922).
+#include "runtime.hpp"
+#include "cold_path.hpp"
+#include "engine_internal.hpp"
+#include "../../include/powerinfer_hip.h"
+
+#include <math.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <utility>
+#include <vector>
+
+namespace {
+
+size_t row_bytes(int type, int64_t ne0) {
+    switch (type) {
+        case PI_TYPE_F32: case PI_TYPE_I32: return (size_t)ne0 * 4;
+        case PI_TYPE_F16:  return (size_t)ne0 * 2;
+        case PI_TYPE_Q4_0: return (size_t)(ne0 / 32) * 18;
+        default: return 0;
+    }
+}
+
+__global__ void set_state_kernel(int32_t * token, int32_t * pos, int32_t t, int32_t p) {
+    if (threadIdx.x == 0) { *token = t; *pos = p; }
+}
+
+// greedy choice of the finished step + bookkeeping for the next one: the chosen token becomes the next
+// input, the position advances, the token and the step's total active-row count are logged
+__global__ __launch_bounds__(1024) void argmax_advance_kernel(const float * __restrict__ logits, int n, int32_t * token, int32_t * pos,
+                                                              int32_t * step, int32_t * out_tokens, int32_t * out_active,
+                                                              const int32_t * __restrict__ n_active, int n_layer, int max_steps) {
+    __shared__ float bv[16];
+    __shared__ int   bi[16];
+    float best = -INFINITY; int idx = n;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) { const float v = logits[i]; if (v > best) { best = v; idx = i; } }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, 64); const int oi = __shfl_xor(idx, o, 64);
+        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+    }
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) { bv[wave] = best; bi[wave] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x >> 6); ++w)
+            if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
+        if (idx >= n) idx = 0;
+        int tot = 0;
+        for (int l = 0; l < n_layer; ++l) tot += n_active[l];
+        const int s = *step;
+        if (s < max_steps) { out_tokens[s] = idx; out_active[s] = tot; }
+        *token = idx;
+        *pos = *pos + 1;
+        *step = s + 1;
+    }
+}
+
+__global__ void add_vec_kernel(float * __restrict__ y, const float * __restrict__ a, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = __fadd_rn(y[i], a[i]);
+}
+
+}  // namespace
+
+namespace {
+
+int upload_tensor(pi_model * m, Tensor & t, int type, const void * data, int64_t ne0, int64_t ne1, int on_device) {
+    const size_t bytes = row_bytes(type, ne0) * (size_t)ne1;
+    if (bytes == 0) return pi::fail(PI_E_ARG, "pi_model_set_tensor: unsupported type or empty tensor");
+    t.type = type; t.ne0 = ne0; t.ne1 = ne1;
+    if (on_device) { t.dev = const_cast<void *>(data); t.owned = false; return PI_OK; }
+    t.dev = m->alloc<unsigned char>(bytes);
+    if (!t.dev) return PI_E_HIP;
+    t.owned = true;
+    return pi_memcpy_h2d(t.dev, data, bytes);
+}
+
+bool is_ffn_matrix(int kind) { return kind == PI_T_FFN_GATE || kind == PI_T_FFN_UP || kind == PI_T_FFN_DOWN_T; }
+
+pi_norm make_norm(int kind, float eps, const Tensor & w, const Tensor * b) {
+    pi_norm n{kind, eps, (const float *)w.dev, b ? (const float *)b->dev : nullptr};
+    return n;
+}
+
+#define PI_TRY(expr) do { int _rc = (expr); if (_rc != PI_OK) return _rc; } while (0)
+
+// ---- one layer, everything on the GPU --------------------------------------------------------------
+int layer_forward(pi_model * m, int il, bool last_token) {
+    const pi_hparams & hp = m->hp;
+    const int d = hp.n_embd, ff = hp.n_ff, hd = m->hd, gqa = m->gqa;
+    hipStream_t st = m->stream;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    Tensor & wqkv = m->L(il, PI_T_WQKV);
+    Tensor & wo = m->L(il, PI_T_WO);
+    Tensor & fc1 = m->L(il, PI_T_FC1);
+    Tensor & fc2 = m->L(il, PI_T_FC2);
+    Tensor & up = m->L(il, PI_T_FFN_UP);
+    Tensor & gate = m->L(il, PI_T_FFN_GATE);
+    Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
+    Tensor & bucket = m->L(il, PI_T_GPU_BUCKET);
+    const int r = (int)fc1.ne1;
+    const size_t kv_off = (size_t)il * hp.n_head_kv * hp.n_ctx * hd;
+    int32_t * n_act = m->n_active + il;
+    const int32_t * bk = (const int32_t *)bucket.dev;
+    const int n_bucket = bk ? (int)bucket.ne0 : 0;
+    const bool q4 = up.type == PI_TYPE_Q4_0;
+    const bool layer_hybrid = bk != nullptr;
+    float * x = m->x;
+
+    // attention
+    pi_norm an;
+    if (!falcon) an = make_norm(1, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), nullptr);
+    else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
+    else an = make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
+    PI_TRY(pi_k_gemv(wqkv.type, wqkv.dev, d + 2 * gqa, d, x, &an, PI_EPI_NONE, nullptr, nullptr, m->qkv, st));
+    PI_TRY(pi_k_rope_kv_store(m->qkv, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, m->d_pos, hp.n_ctx,
+                              m->q_rot, m->k_cache + kv_off, m->v_cache + kv_off, st));
+    PI_TRY(pi_k_attn_decode(m->q_rot, m->k_cache + kv_off, m->v_cache + kv_off, hp.n_head, hp.n_head_kv, hd, hp.n_ctx, m->d_pos, m->att, st));
+
+    const float * pred_in; const float * ffn_in; pi_norm fn;
+    if (!falcon) {
+        // ffn_inp = wo.att + x   (ggml_add(cur, inpSA), llama.cpp:5022)
+        PI_TRY(pi_k_gemv(wo.type, wo.dev, d, d, m->att, nullptr, PI_EPI_ADD, x, nullptr, m->ffn_inp, st));
+        pred_in = m->ffn_inp; ffn_in = m->ffn_inp;
+        fn = make_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
+    } else {
+        PI_TRY(pi_k_gemv(wo.type, wo.dev, d, d, m->att, nullptr, PI_EPI_NONE, nullptr, nullptr, m->attn_out, st));
+        pred_in = x; ffn_in = x;                       // Falcon: predictor sees the layer input, FFN sees attn_norm(layer input)
+        fn = make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
+    }
+
+    // predictor
+    PI_TRY(pi_k_gemv(fc1.type, fc1.dev, r, d, pred_in, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, st));
+    PI_TRY(pi_k_predictor_fc2(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, bk, n_bucket, m->pred_logits, m->list, n_act,
+                              (q4 || layer_hybrid) ? m->h_dense : nullptr, m->ws, st));
+
+    // sparse FFN, GPU share
+    PI_TRY(pi_k_sparse_upgate(up.type, up.dev, falcon ? nullptr : gate.dev, d, ffn_in, &fn, m->list, n_act, bk, m->h_c,
+                              (q4 || layer_hybrid) ? m->h_dense : nullptr, nullptr, nullptr, st));
+
+    if (!layer_hybrid && m->capture && last_token) {
+        // parity hook: keep the bare FFN output, then add the residuals in the reference's order
+        float * ffo = m->cap_ffn + (size_t)il * d;
+        PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, n_act,
+                                PI_EPI_NONE, nullptr, nullptr, ffo, m->ws, st));
+        PI_HIP_TRY(hipMemcpyAsync(m->x2, ffo, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
+        PI_TRY(pi::add_vec(m->x2, falcon ? m->attn_out : m->ffn_inp, d, st));
+        if (falcon) PI_TRY(pi::add_vec(m->x2, x, d, st));
+    } else if (!layer_hybrid) {
+        if (!falcon) PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, n_act,
+                                             PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, m->ws, st));
+        else         PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, n_act,
+                                             PI_EPI_ADD2, m->attn_out, x, m->x2, m->ws, st));
+    } else {
+        // hot/cold merge (llm_build_sparse_mul_mat / llm_build_sparse_axpy hybrid variants, llama.cpp:4581-4593, 4635-4646)
+        PI_TRY(pi::cold_layer_merge(m->cold, il, m, st));
+    }
+    std::swap(m->x, m->x2);
+
+    if (m->capture && last_token) {
+        PI_HIP_TRY(hipMemcpyAsync(m->cap_logits + (size_t)il * ff, m->pred_logits, sizeof(float) * ff, hipMemcpyDeviceToDevice, st));
+        PI_HIP_TRY(hipMemcpyAsync(m->cap_src + (size_t)il * d, ffn_in, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
+    }
+    return PI_OK;
+}
+
+// one token: embedding -> layers -> (final norm + lm-head + greedy)
+int token_forward(pi_model * m, bool want_logits, bool last_token) {
+    const pi_hparams & hp = m->hp;
+    hipStream_t st = m->stream;
+    PI_TRY(pi_k_embed(m->glob[PI_T_TOK_EMBD].type, m->glob[PI_T_TOK_EMBD].dev, hp.n_embd, m->d_token, m->x, st));
+    for (int il = 0; il < hp.n_layer; ++il) PI_TRY(layer_forward(m, il, last_token));
+    if (want_logits) {
+        const bool falcon = hp.arch == PI_ARCH_FALCON;
+        pi_norm on = make_norm(falcon ? 2 : 1, hp.norm_eps, m->glob[PI_T_OUTPUT_NORM], falcon ? &m->glob[PI_T_OUTPUT_NORM_B] : nullptr);
+        PI_TRY(pi_k_gemv(m->glob[PI_T_OUTPUT].type, m->glob[PI_T_OUTPUT].dev, hp.n_vocab, hp.n_embd, m->x, &on, PI_EPI_NONE, nullptr, nullptr, m->logits, st));
+    }
+    return PI_OK;
+}
+
+int launch_advance(pi_model * m) {
+    hipLaunchKernelGGL(argmax_advance_kernel, dim3(1), dim3(1024), 0, m->stream, m->logits, m->hp.n_vocab, m->d_token, m->d_pos, m->d_step,
+                       m->d_out_tokens, m->d_out_active, m->n_active, m->hp.n_layer, m->max_steps);
+    return pi::check_launch("argmax_advance");
+}
+
+}  // namespace
+
+// entry used by the cold path to add its share into the layer output on the model's stream
+namespace pi {
+int add_vec(float * y, const float * a, int n, hipStream_t st) {
+    hipLaunchKernelGGL(add_vec_kernel, dim3((n + 255) / 256), dim3(256), 0, st, y, a, n);
+    return check_launch("add_vec");
+}
+}  // namespace pi
+
+extern "C" {
+
+pi_model * pi_model_create(const pi_hparams * hp) {
+    if (!hp || hp->n_embd <= 0 || hp->n_ff <= 0 || hp->n_head <= 0 || hp->n_head_kv <= 0 || hp->n_layer <= 0 || hp->n_vocab <= 0 || hp->n_ctx <= 0 ||
+        hp->n_embd % hp->n_head || hp->n_head % hp->n_head_kv || (hp->arch != PI_ARCH_LLAMA && hp->arch != PI_ARCH_FALCON)) {
+        pi::set_error("pi_model_create: inconsistent hyper-parameters");
+        return nullptr;
+    }
+    if (pi_init(0) != PI_OK) return nullptr;
+    pi_model * m = new pi_model();
+    m->hp = *hp;
+    m->hd = hp->n_embd / hp->n_head;
+    m->gqa = m->hd * hp->n_head_kv;
+    m->layers.resize((size_t)hp->n_layer * PI_T_COUNT);
+    m->theta_scale = powf(hp->rope_freq_base, -2.0f / (float)m->hd);       // ggml.c:11196
+    return m;
+}
+
+void pi_model_free(pi_model * m) {
+    if (!m) return;
+    if (m->graph_exec) hipGraphExecDestroy(m->graph_exec);
+    if (m->graph) hipGraphDestroy(m->graph);
+    if (m->ev0) hipEventDestroy(m->ev0);
+    if (m->ev1) hipEventDestroy(m->ev1);
+    if (m->cold) pi::cold_destroy(m->cold);
+    if (m->ws) pi_workspace_destroy(m->ws);
+    for (void * p : m->owned) pi_free(p);
+    if (m->stream) hipStreamDestroy(m->stream);
+    delete m;
+}
+
+int pi_model_set_tensor(pi_model * m, int layer, int kind, int type, const void * data, int64_t ne0, int64_t ne1, int on_device) {
+    if (!m || !data || kind < 0 || kind >= PI_T_COUNT || ne0 <= 0 || ne1 <= 0) return pi::fail(PI_E_ARG, "pi_model_set_tensor: bad arguments");
+    if (m->finalized) return pi::fail(PI_E_STATE, "pi_model_set_tensor: model already finalized");
+    if (kind <= PI_T_OUTPUT) return upload_tensor(m, m->glob[kind], type, data, ne0, ne1, on_device);
+    if (layer < 0 || layer >= m->hp.n_layer) return pi::fail(PI_E_ARG, "pi_model_set_tensor: layer out of range");
+    Tensor & t = m->L(layer, kind);
+    if (is_ffn_matrix(kind) && !on_device) {
+        // sliced at finalize if the layer turns out to have a GPU bucket; remember the host copy until then
+        t.type = type; t.ne0 = ne0; t.ne1 = ne1; t.host = data;
+        return PI_OK;
+    }
+    if (kind == PI_T_GPU_IDX) { t.type = type; t.ne0 = ne0; t.ne1 = ne1; t.host = data; return PI_OK; }   // host-only (cold path)
+    if (kind == PI_T_GPU_BUCKET) { t.host = data; }
+    return upload_tensor(m, t, type, data, ne0, ne1, on_device);
+}
+
+int pi_model_finalize(pi_model * m) {
+    if (!m) return pi::fail(PI_E_ARG, "pi_model_finalize: null model");
+    if (m->finalized) return PI_OK;
+    const pi_hparams & hp = m->hp;
+    const int d = hp.n_embd, ff = hp.n_ff, gqa = m->gqa;
+    PI_HIP_TRY(hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking));
+    PI_HIP_TRY(hipEventCreate(&m->ev0));
+    PI_HIP_TRY(hipEventCreate(&m->ev1));
+
+    for (int k : {PI_T_TOK_EMBD, PI_T_OUTPUT_NORM, PI_T_OUTPUT})
+        if (!m->glob[k].dev) return pi::fail(PI_E_STATE, "pi_model_finalize: token_embd / output_norm / output missing");
+    if (hp.arch == PI_ARCH_FALCON && !m->glob[PI_T_OUTPUT_NORM_B].dev) return pi::fail(PI_E_STATE, "pi_model_finalize: output_norm bias missing");
+
+    int max_r = 0;
+    for (int il = 0; il < hp.n_layer; ++il) {
+        // pack q, k, v rows into one matrix so that one mat-vec produces q | k | v
+        Tensor & wqkv = m->L(il, PI_T_WQKV);
+        if (!wqkv.dev) {
+            Tensor & wq = m->L(il, PI_T_WQ); Tensor & wk = m->L(il, PI_T_WK); Tensor & wv = m->L(il, PI_T_WV);
+            if (!wq.dev || !wk.dev || !wv.dev) return pi::fail(PI_E_STATE, "pi_model_finalize: attention projections missing");
+            if (wq.type != wk.type || wq.type != wv.type || wq.ne0 != d || wk.ne0 != d || wv.ne0 != d || wq.ne1 != d || wk.ne1 != gqa || wv.ne1 != gqa)
+                return pi::fail(PI_E_ARG, "pi_model_finalize: attention projection shapes/types disagree");
+            const size_t rb = row_bytes(wq.type, d);
+            unsigned char * p = m->alloc<unsigned char>(rb * (size_t)(d + 2 * gqa));
+            if (!p) return PI_E_HIP;
+            PI_TRY(pi_memcpy_d2d(p, wq.dev, rb * d));
+            PI_TRY(pi_memcpy_d2d(p + rb * d, wk.dev, rb * gqa));
+            PI_TRY(pi_memcpy_d2d(p + rb * (d + gqa), wv.dev, rb * gqa));
+            wqkv.type = wq.type; wqkv.dev = p; wqkv.ne0 = d; wqkv.ne1 = d + 2 * gqa; wqkv.owned = true;
+            for (Tensor * t : {&wq, &wk, &wv}) {
+                if (t->owned) {   // release the separate copies
+                    for (auto & o : m->owned) if (o == t->dev) { pi_free(o); o = nullptr; }
+                }
+                t->dev = nullptr;
+            }
+        }
+        if (wqkv.ne0 != d || wqkv.ne1 != d + 2 * gqa) return pi::fail(PI_E_ARG, "pi_model_finalize: wqkv shape");
+        for (int k : {PI_T_ATTN_NORM, PI_T_WO, PI_T_FC1, PI_T_FC2})
+            if (!m->L(il, k).dev) return pi::fail(PI_E_STATE, "pi_model_finalize: a layer tensor is missing (attn_norm / wo / fc1 / fc2)");
+        if (hp.arch == PI_ARCH_LLAMA && !m->L(il, PI_T_FFN_NORM).dev) return pi::fail(PI_E_STATE, "pi_model_finalize: ffn_norm missing");
+        if (hp.arch == PI_ARCH_FALCON && !m->L(il, PI_T_ATTN_NORM_B).dev) return pi::fail(PI_E_STATE, "pi_model_finalize: attn_norm bias missing");
+        Tensor & fc1 = m->L(il, PI_T_FC1); Tensor & fc2 = m->L(il, PI_T_FC2);
+        if (fc2.type != PI_TYPE_F16) return pi::fail(PI_E_UNSUPPORTED, "pi_model_finalize: predictor fc2 must be F16");
+        if (fc1.ne0 != d || fc2.ne1 != ff || fc2.ne0 != fc1.ne1 || fc1.ne1 % 8) return pi::fail(PI_E_ARG, "pi_model_finalize: predictor shapes (fc1 {d, r}, fc2 {r, ff}, r % 8 == 0)");
+        if ((int)fc1.ne1 > max_r) max_r = (int)fc1.ne1;
+
+        // FFN matrices: whole on the GPU, or the bucket's rows only
+        Tensor & bucket = m->L(il, PI_T_GPU_BUCKET);
+        const int32_t * bk_host = (const int32_t *)bucket.host;
+        const int n_bucket = bucket.dev ? (int)bucket.ne0 : 0;
+        if (bucket.dev) {
+            if (!m->L(il, PI_T_GPU_IDX).host) return pi::fail(PI_E_STATE, "pi_model_finalize: a layer with gpu_bucket needs gpu_idx");
+            m->hybrid = true;
+        }
+        for (int k : {PI_T_FFN_UP, PI_T_FFN_GATE, PI_T_FFN_DOWN_T}) {
+            Tensor & t = m->L(il, k);
+            if (k == PI_T_FFN_GATE && hp.arch == PI_ARCH_FALCON) continue;
+            if (t.dev) continue;                                     // adopted device tensor
+            if (!t.host) return pi::fail(PI_E_STATE, "pi_model_finalize: an FFN matrix is missing");
+            if (t.ne0 != d || t.ne1 != ff) return pi::fail(PI_E_ARG, "pi_model_finalize: FFN matrices must be {n_embd, n_ff}");
+            const size_t rb = row_bytes(t.type, d);
+            if (!bucket.dev) {
+                t.dev = m->alloc<unsigned char>(rb * (size_t)ff);
+                if (!t.dev) return PI_E_HIP;
+                t.owned = true;
+                PI_TRY(pi_memcpy_h2d(t.dev, t.host, rb * (size_t)ff));
+                t.host = nullptr;
+            } else {
+                // compact [n_bucket][d] matrix in bucket order: gather on the host, one upload
+                std::vector<unsigned char> tmp(rb * (size_t)(n_bucket ? n_bucket : 1));
+                for (int i = 0; i < n_bucket; ++i) {
+                    if (bk_host[i] < 0 || bk_host[i] >= ff || (i && bk_host[i] <= bk_host[i - 1]))
+                        return pi::fail(PI_E_ARG, "pi_model_finalize: gpu_bucket must be strictly ascending neuron indices");
+                    memcpy(tmp.data() + rb * i, (const unsigned char *)t.host + rb * (size_t)bk_host[i], rb);
+                }
+                t.dev = m->alloc<unsigned char>(tmp.size());
+                if (!t.dev) return PI_E_HIP;
+                t.owned = true;
+                PI_TRY(pi_memcpy_h2d(t.dev, tmp.data(), tmp.size()));
+            }
+        }
+    }
+
+    m->ws = pi_workspace_create(ff, d);
+    if (!m->ws) return PI_E_HIP;
+    const size_t kv = (size_t)hp.n_layer * hp.n_head_kv * hp.n_ctx * m->hd;
+    m->x = m->alloc<float>(d); m->x2 = m->alloc<float>(d); m->qkv = m->alloc<float>(d + 2 * gqa); m->q_rot = m->alloc<float>(d);
+    m->att = m->alloc<float>(d); m->attn_out = m->alloc<float>(d); m->ffn_inp = m->alloc<float>(d); m->hidden = m->alloc<float>(max_r);
+    m->pred_logits = m->alloc<float>(ff); m->h_c = m->alloc<float>(ff); m->h_dense = m->alloc<float>(ff); m->logits = m->alloc<float>(hp.n_vocab);
+    m->cold_out = m->alloc<float>(d);
+    m->list = m->alloc<int32_t>(ff); m->n_active = m->alloc<int32_t>(hp.n_layer);
+    m->d_token = m->alloc<int32_t>(1); m->d_pos = m->alloc<int32_t>(1); m->d_step = m->alloc<int32_t>(1);
+    m->d_out_tokens = m->alloc<int32_t>(m->max_steps); m->d_out_active = m->alloc<int32_t>(m->max_steps);
+    m->k_cache = m->alloc<__half>(kv); m->v_cache = m->alloc<__half>(kv);
+    m->cap_ffn = m->alloc<float>((size_t)hp.n_layer * d); m->cap_logits = m->alloc<float>((size_t)hp.n_layer * ff); m->cap_src = m->alloc<float>((size_t)hp.n_layer * d);
+    if (!m->x || !m->x2 || !m->qkv || !m->q_rot || !m->att || !m->attn_out || !m->ffn_inp || !m->hidden || !m->pred_logits || !m->h_c || !m->h_dense ||
+        !m->logits || !m->cold_out || !m->list || !m->n_active || !m->d_token || !m->d_pos || !m->d_step || !m->d_out_tokens || !m->d_out_active ||
+        !m->k_cache || !m->v_cache || !m->cap_ffn || !m->cap_logits || !m->cap_src)
+        return PI_E_HIP;
+    PI_TRY(pi_memset(m->k_cache, 0, kv * 2));
+    PI_TRY(pi_memset(m->v_cache, 0, kv * 2));
+    PI_TRY(pi_memset(m->n_active, 0, sizeof(int32_t) * hp.n_layer));
+    PI_TRY(pi_memset(m->d_step, 0, 4));
+    PI_TRY(pi_memset(m->h_dense, 0, sizeof(float) * ff));
+    if (m->hybrid) {
+        m->cold = pi::cold_create(m);
+        if (!m->cold) return PI_E_STATE;
+    }
+    PI_HIP_TRY(hipDeviceSynchronize());
+    m->finalized = true;
+    return PI_OK;
+}
+
+int pi_model_kv_clear(pi_model * m) {
+    if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_kv_clear: model not finalized");
+    const size_t kv = (size_t)m->hp.n_layer * m->hp.n_head_kv * m->hp.n_ctx * m->hd;
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    PI_TRY(pi_memset(m->k_cache, 0, kv * 2));
+    PI_TRY(pi_memset(m->v_cache, 0, kv * 2));
+    return PI_OK;
+}
+
+int pi_model_decode(pi_model * m, const int32_t * tokens, int n_tokens, int n_past, float * logits_out) {
+    if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_decode: model not finalized");
+    if (!tokens || n_tokens <= 0 || n_past < 0 || n_past + n_tokens > m->hp.n_ctx) return pi::fail(PI_E_ARG, "pi_model_decode: token range exceeds the context");
+    for (int i = 0; i < n_tokens; ++i)
+        if (tokens[i] < 0 || tokens[i] >= m->hp.n_vocab) return pi::fail(PI_E_ARG, "pi_model_decode: token id out of range");
+    for (int i = 0; i < n_tokens; ++i) {
+        const bool last = i == n_tokens - 1;
+        hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, m->stream, m->d_token, m->d_pos, tokens[i], n_past + i);
+        PI_TRY(pi::check_launch("set_state"));
+        PI_TRY(token_forward(m, last, last));
+    }
+    // greedy choice on the device; the state then points at the next position
+    PI_HIP_TRY(hipMemsetAsync(m->d_step, 0, 4, m->stream));
+    PI_TRY(launch_advance(m));
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    int32_t tok = -1;
+    PI_TRY(pi_memcpy_d2h(&tok, m->d_token, 4));
+    if (logits_out) PI_TRY(pi_memcpy_d2h(logits_out, m->logits, sizeof(float) * m->hp.n_vocab));
+    return tok;
+}
+
+int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * ms_out) {
+    if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_generate: model not finalized");
+    if (n_steps <= 0 || n_steps > m->max_steps || !out_tokens) return pi::fail(PI_E_ARG, "pi_model_generate: bad step count");
+    int32_t pos = 0;
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    PI_TRY(pi_memcpy_d2h(&pos, m->d_pos, 4));
+    if (pos + n_steps > m->hp.n_ctx) return pi::fail(PI_E_ARG, "pi_model_generate: would run past the context");
+    PI_HIP_TRY(hipMemsetAsync(m->d_step, 0, 4, m->stream));
+
+    const bool use_graph = !m->hybrid && !m->capture;
+    if (use_graph && !m->graph_exec) {
+        PI_HIP_TRY(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
+        int rc = token_forward(m, true, false);
+        if (rc == PI_OK) rc = launch_advance(m);
+        hipGraph_t g = nullptr;
+        const hipError_t e = hipStreamEndCapture(m->stream, &g);
+        if (rc != PI_OK) { if (g) hipGraphDestroy(g); return rc; }
+        if (e != hipSuccess) return pi::hip_fail(e, "hipStreamEndCapture");
+        m->graph = g;
+        PI_HIP_TRY(hipGraphInstantiate(&m->graph_exec, g, nullptr, nullptr, 0));
+    }
+    PI_HIP_TRY(hipEventRecord(m->ev0, m->stream));
+    for (int s = 0; s < n_steps; ++s) {
+        if (use_graph) {
+            PI_HIP_TRY(hipGraphLaunch(m->graph_exec, m->stream));
+        } else {
+            PI_TRY(token_forward(m, true, false));
+            PI_TRY(launch_advance(m));
+        }
+    }
+    PI_HIP_TRY(hipEventRecord(m->ev1, m->stream));
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    if (ms_out) PI_HIP_TRY(hipEventElapsedTime(ms_out, m->ev0, m->ev1));
+    PI_TRY(pi_memcpy_d2h(out_tokens, m->d_out_tokens, sizeof(int32_t) * n_steps));
+    return PI_OK;
+}
+
+int pi_model_set_capture(pi_model * m, int enable) {
+    if (!m) return pi::fail(PI_E_ARG, "pi_model_set_capture: null model");
+    m->capture = enable != 0;
+    return PI_OK;
+}
+
+int pi_model_get_capture(pi_model * m, float * ffn_out, float * pred_logits, int32_t * n_active, float * ffn_src) {
+    if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_get_capture: model not finalized");
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    if (ffn_out) PI_TRY(pi_memcpy_d2h(ffn_out, m->cap_ffn, sizeof(float) * (size_t)m->hp.n_layer * m->hp.n_embd));
+    if (pred_logits) PI_TRY(pi_memcpy_d2h(pred_logits, m->cap_logits, sizeof(float) * (size_t)m->hp.n_layer * m->hp.n_ff));
+    if (n_active) PI_TRY(pi_memcpy_d2h(n_active, m->n_active, sizeof(int32_t) * m->hp.n_layer));
+    if (ffn_src) PI_TRY(pi_memcpy_d2h(ffn_src, m->cap_src, sizeof(float) * (size_t)m->hp.n_layer * m->hp.n_embd));
+    return PI_OK;
+}
+
+int pi_model_step_active(pi_model * m, int32_t * per_step_total, int n_steps) {
+    if (!m || !m->finalized || !per_step_total || n_steps <= 0 || n_steps > m->max_steps) return pi::fail(PI_E_ARG, "pi_model_step_active: bad arguments");
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    return pi_memcpy_d2h(per_step_total, m->d_out_active, sizeof(int32_t) * n_steps);
+}
+
+}  // extern "C"

@@ -1,0 +1,54 @@
+// Internal layout of the decode engine's model object (shared by the engine and the host cold path).
+#pragma once
+
+#include "../../include/powerinfer_hip.h"
+#include "cold_path.hpp"
+
+#include <hip/hip_runtime.h>
+#include <hip/hip_fp16.h>
+
+#include <vector>
+
+struct Tensor {
+    int          type = -1;
+    void *       dev = nullptr;      // device address (rows possibly sliced to the GPU bucket)
+    const void * host = nullptr;     // borrowed host copy (hybrid layers: full-size matrices for the cold path)
+    int64_t      ne0 = 0, ne1 = 0;   // as given by the caller
+    bool         owned = false;
+};
+
+
+struct pi_model {
+    pi_hparams hp{};
+    std::vector<Tensor> layers;           // [n_layer][PI_T_COUNT]
+    Tensor glob[4];
+    std::vector<void *> owned;            // every device allocation made by the model
+    bool finalized = false, hybrid = false;
+    int hd = 0, gqa = 0, max_steps = 4096;
+    hipStream_t stream = nullptr;
+    pi_workspace * ws = nullptr;
+    float theta_scale = 0.0f;
+
+    float *x = nullptr, *x2 = nullptr, *qkv = nullptr, *q_rot = nullptr, *att = nullptr, *attn_out = nullptr, *ffn_inp = nullptr;
+    float *hidden = nullptr, *pred_logits = nullptr, *h_c = nullptr, *h_dense = nullptr, *logits = nullptr, *cold_out = nullptr;
+    int32_t *list = nullptr, *n_active = nullptr, *d_token = nullptr, *d_pos = nullptr, *d_step = nullptr;
+    int32_t *d_out_tokens = nullptr, *d_out_active = nullptr;
+    __half *k_cache = nullptr, *v_cache = nullptr;
+
+    hipGraphExec_t graph_exec = nullptr;
+    hipGraph_t graph = nullptr;
+    hipEvent_t ev0 = nullptr, ev1 = nullptr;
+
+    bool capture = false;
+    float *cap_ffn = nullptr, *cap_logits = nullptr, *cap_src = nullptr;       // device
+    pi::ColdPath * cold = nullptr;
+
+    Tensor & L(int il, int kind) { return layers[(size_t)il * PI_T_COUNT + kind]; }
+
+    template <typename T> T * alloc(size_t count) {
+        void * p = pi_malloc(sizeof(T) * (count ? count : 1));
+        if (p) owned.push_back(p);
+        return (T *)p;
+    }
+};
+

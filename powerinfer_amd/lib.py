@@ -74,7 +74,8 @@ def load():
 
 
 def declared_symbols():
-    return sorted(_SIGS)
+    from .model import ENGINE_SYMBOLS
+    return sorted(list(_SIGS) + ENGINE_SYMBOLS)
 
 
 def check(rc, what=""):

@@ -1,0 +1,146 @@
+"""Python face of the decode engine (pi_model_* in include/powerinfer_hip.h): mirrors the slice of llama.h a
+greedy batch-1 run uses -- load, llama_decode, llama_get_logits, greedy sampling, the token loop."""
+import ctypes as C
+
+import numpy as np
+
+from . import lib as pl
+from .lib import check
+
+ARCH = {"llama": 0, "falcon": 1}
+
+# tensor roles, same order as the enum in include/powerinfer_hip.h
+KINDS = ["tok_embd", "output_norm", "output_norm_b", "output",
+         "attn_norm", "attn_norm_b", "attn_norm_2", "attn_norm_2_b",
+         "wq", "wk", "wv", "wqkv", "wo",
+         "ffn_norm", "ffn_gate", "ffn_up", "ffn_down_t",
+         "fc1", "fc2", "gpu_idx", "gpu_bucket"]
+KIND = {k: i for i, k in enumerate(KINDS)}
+
+
+class HParamsC(C.Structure):
+    _fields_ = [("arch", C.c_int32), ("n_embd", C.c_int32), ("n_ff", C.c_int32), ("n_head", C.c_int32),
+                ("n_head_kv", C.c_int32), ("n_layer", C.c_int32), ("n_vocab", C.c_int32), ("n_ctx", C.c_int32),
+                ("norm_eps", C.c_float), ("rope_freq_base", C.c_float), ("sparse_threshold", C.c_float)]
+
+
+def _declare(L):
+    vp, i = C.c_void_p, C.c_int
+    L.pi_model_create.restype, L.pi_model_create.argtypes = vp, [C.POINTER(HParamsC)]
+    L.pi_model_free.restype, L.pi_model_free.argtypes = None, [vp]
+    L.pi_model_set_tensor.restype, L.pi_model_set_tensor.argtypes = i, [vp, i, i, i, vp, C.c_int64, C.c_int64, i]
+    L.pi_model_finalize.restype, L.pi_model_finalize.argtypes = i, [vp]
+    L.pi_model_kv_clear.restype, L.pi_model_kv_clear.argtypes = i, [vp]
+    L.pi_model_decode.restype, L.pi_model_decode.argtypes = i, [vp, vp, i, i, vp]
+    L.pi_model_generate.restype, L.pi_model_generate.argtypes = i, [vp, i, vp, C.POINTER(C.c_float)]
+    L.pi_model_set_capture.restype, L.pi_model_set_capture.argtypes = i, [vp, i]
+    L.pi_model_get_capture.restype, L.pi_model_get_capture.argtypes = i, [vp, vp, vp, vp, vp]
+    L.pi_model_step_active.restype, L.pi_model_step_active.argtypes = i, [vp, vp, i]
+
+
+ENGINE_SYMBOLS = ["pi_model_create", "pi_model_free", "pi_model_set_tensor", "pi_model_finalize", "pi_model_kv_clear",
+                  "pi_model_decode", "pi_model_generate", "pi_model_set_capture", "pi_model_get_capture",
+                  "pi_model_step_active"]
+
+
+def _type_of(a, hint):
+    if a.dtype == np.float32:
+        return pl.F32
+    if a.dtype == np.float16:
+        return pl.F16
+    if a.dtype == np.int32:
+        return pl.I32
+    if a.dtype == np.uint8:
+        return pl.Q4_0
+    raise TypeError(f"{hint}: unsupported dtype {a.dtype}")
+
+
+def _ne(a, t):
+    """(ne0, ne1) of a 1-D or 2-D numpy array holding a tensor of ggml type t."""
+    rows = a.shape[0] if a.ndim == 2 else 1
+    inner = a.shape[-1]
+    return (inner // 18 * 32 if t == pl.Q4_0 else inner), rows
+
+
+class Model:
+    def __init__(self, hp):
+        self.L = pl.init()
+        _declare(self.L)
+        self.hp = hp
+        c = HParamsC(ARCH[hp.arch], hp.n_embd, hp.n_ff, hp.n_head, hp.n_head_kv, hp.n_layer, hp.n_vocab, hp.n_ctx,
+                     hp.norm_eps, hp.rope_freq_base, hp.sparse_threshold)
+        self.h = self.L.pi_model_create(C.byref(c))
+        if not self.h:
+            raise pl.PiError("pi_model_create: " + self.L.pi_last_error().decode())
+        self._keep = []        # host arrays the engine borrows (hybrid layers)
+
+    def set_tensor(self, layer, kind, arr):
+        arr = np.ascontiguousarray(arr)
+        t = _type_of(arr, kind)
+        ne0, ne1 = _ne(arr, t)
+        self._keep.append(arr)
+        check(self.L.pi_model_set_tensor(self.h, layer, KIND[kind], t, arr.ctypes.data_as(C.c_void_p), ne0, ne1, 0), f"set_tensor {kind}")
+
+    def set_tensor_device(self, layer, kind, ptr, t, ne0, ne1):
+        check(self.L.pi_model_set_tensor(self.h, layer, KIND[kind], t, ptr, ne0, ne1, 1), f"set_tensor {kind}")
+
+    def load(self, model):
+        """model: the dict powerinfer_amd.synth.make_model returns."""
+        for k, a in model["glob"].items():
+            self.set_tensor(-1, k, a)
+        for il, Lr in enumerate(model["layers"]):
+            for k, a in Lr.items():
+                if k in KIND and a is not None:
+                    self.set_tensor(il, k, a)
+        self.finalize()
+        return self
+
+    def finalize(self):
+        check(self.L.pi_model_finalize(self.h), "pi_model_finalize")
+
+    def kv_clear(self):
+        check(self.L.pi_model_kv_clear(self.h), "pi_model_kv_clear")
+
+    def decode(self, tokens, n_past, want_logits=True):
+        tokens = np.ascontiguousarray(tokens, np.int32)
+        logits = np.empty(self.hp.n_vocab, np.float32) if want_logits else None
+        tok = self.L.pi_model_decode(self.h, tokens.ctypes.data_as(C.c_void_p), tokens.size, n_past,
+                                     logits.ctypes.data_as(C.c_void_p) if want_logits else None)
+        if tok < 0:
+            raise pl.PiError(f"pi_model_decode ({tok}): " + self.L.pi_last_error().decode())
+        return tok, logits
+
+    def generate(self, n_steps):
+        out = np.empty(n_steps, np.int32)
+        ms = C.c_float(0)
+        check(self.L.pi_model_generate(self.h, n_steps, out.ctypes.data_as(C.c_void_p), C.byref(ms)), "pi_model_generate")
+        return out, float(ms.value)
+
+    def set_capture(self, on):
+        check(self.L.pi_model_set_capture(self.h, int(on)), "set_capture")
+
+    def get_capture(self):
+        hp = self.hp
+        ffn = np.empty((hp.n_layer, hp.n_embd), np.float32)
+        lg = np.empty((hp.n_layer, hp.n_ff), np.float32)
+        na = np.empty(hp.n_layer, np.int32)
+        src = np.empty((hp.n_layer, hp.n_embd), np.float32)
+        check(self.L.pi_model_get_capture(self.h, ffn.ctypes.data_as(C.c_void_p), lg.ctypes.data_as(C.c_void_p),
+                                          na.ctypes.data_as(C.c_void_p), src.ctypes.data_as(C.c_void_p)), "get_capture")
+        return ffn, lg, na, src
+
+    def step_active(self, n_steps):
+        out = np.empty(n_steps, np.int32)
+        check(self.L.pi_model_step_active(self.h, out.ctypes.data_as(C.c_void_p), n_steps), "step_active")
+        return out
+
+    def close(self):
+        if self.h:
+            self.L.pi_model_free(self.h)
+            self.h = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass

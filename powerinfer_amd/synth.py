@@ -107,10 +107,10 @@ def hparams(name, **over):
                           n_vocab=32000, mean_rate=0.11),
         "falcon-40b": dict(arch="falcon", n_embd=8192, n_ff=32768, n_rank=1024, n_head=128, n_head_kv=8, n_layer=60,
                            n_vocab=65024, mean_rate=0.08),
-        "llama-tiny": dict(arch="llama", n_embd=256, n_ff=1024, n_rank=64, n_head=4, n_head_kv=4, n_layer=2,
-                           n_vocab=512, mean_rate=0.15),
-        "falcon-tiny": dict(arch="falcon", n_embd=256, n_ff=1024, n_rank=64, n_head=8, n_head_kv=2, n_layer=2,
-                            n_vocab=512, mean_rate=0.15),
+        "llama-tiny": dict(arch="llama", n_embd=512, n_ff=4096, n_rank=128, n_head=8, n_head_kv=8, n_layer=3,
+                           n_vocab=1024, mean_rate=0.15),
+        "falcon-tiny": dict(arch="falcon", n_embd=512, n_ff=4096, n_rank=128, n_head=8, n_head_kv=2, n_layer=3,
+                            n_vocab=1024, mean_rate=0.15),
     }[name]
     hp = HParams(base, name=name, n_ctx=512, wtype=F16, norm_eps=1e-5, rope_freq_base=10000.0, sparse_threshold=0.0,
                  hot_frac=1.0, seed=0)

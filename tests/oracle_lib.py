@@ -64,7 +64,7 @@ def oracle():
         L.pio_model_free.argtypes = [_vp]
         L.pio_model_set_tensor.argtypes = [_vp, _i, _i, _i, _vp, _i64, _i64]
         L.pio_model_kv_clear.argtypes = [_vp]
-        L.pio_model_set_capture.argtypes = [_vp, _vp, _vp]
+        L.pio_model_set_capture.argtypes = [_vp, _vp, _vp, _vp]
         L.pio_model_eval.argtypes = [_vp, _vp, _vp, _vp, _i, _i, _vp, _i, _vp, _i]
         L.pio_model_eval_simple.argtypes = [_vp, _vp, _i, _i, _vp, _i]
         _oracle = L
@@ -127,3 +127,62 @@ def ffn_sparse(lib, d, ff, r, T, wtype, has_gate, up, gate, down_t, fc1, fc2, x_
             _ptr(o["logits"]), _ptr(o["up"]), _ptr(o["gate"]), _ptr(o["h"]), _ptr(o["out"]))
     assert rc == 0, rc
     return o
+
+
+# ---------------------------------------------------------------------------------------------
+# whole-model oracle driven from the dict powerinfer_amd.synth.make_model returns
+# ---------------------------------------------------------------------------------------------
+class HParamsC(C.Structure):
+    _fields_ = [("arch", C.c_int32), ("n_embd", C.c_int32), ("n_ff", C.c_int32), ("n_head", C.c_int32),
+                ("n_head_kv", C.c_int32), ("n_layer", C.c_int32), ("n_vocab", C.c_int32), ("n_ctx", C.c_int32),
+                ("norm_eps", C.c_float), ("rope_freq_base", C.c_float), ("sparse_threshold", C.c_float)]
+
+
+_KINDS = ["tok_embd", "output_norm", "output_norm_b", "output", "attn_norm", "attn_norm_b", "attn_norm_2", "attn_norm_2_b",
+          "wq", "wk", "wv", "wqkv", "wo", "ffn_norm", "ffn_gate", "ffn_up", "ffn_down_t", "fc1", "fc2", "gpu_idx"]
+
+
+class OracleModel:
+    def __init__(self, model, all_cold=True):
+        """all_cold: ignore any gpu_idx so the CPU path computes every neuron (what "all on GPU" is compared with)."""
+        self.O = oracle()
+        hp = model["hp"]
+        self.hp = hp
+        c = HParamsC({"llama": 0, "falcon": 1}[hp.arch], hp.n_embd, hp.n_ff, hp.n_head, hp.n_head_kv, hp.n_layer, hp.n_vocab,
+                     hp.n_ctx, hp.norm_eps, hp.rope_freq_base, hp.sparse_threshold)
+        self.h = self.O.pio_model_new(C.byref(c))
+        self._keep = []
+
+        def put(layer, k, a):
+            a = np.ascontiguousarray(a)
+            t = {np.dtype(np.float32): F32, np.dtype(np.float16): F16, np.dtype(np.int32): I32, np.dtype(np.uint8): Q4_0}[a.dtype]
+            rows = a.shape[0] if a.ndim == 2 else 1
+            ne0 = a.shape[-1] // 18 * 32 if t == Q4_0 else a.shape[-1]
+            self._keep.append(a)
+            assert self.O.pio_model_set_tensor(self.h, layer, _KINDS.index(k), t, _ptr(a), ne0, rows) == 0
+
+        for k, a in model["glob"].items():
+            put(-1, k, a)
+        for il, L in enumerate(model["layers"]):
+            for k, a in L.items():
+                if k in _KINDS and a is not None and not (all_cold and k == "gpu_idx"):
+                    put(il, k, a)
+
+    def capture(self, T=1):
+        hp = self.hp
+        self.cap_ffn = np.zeros((hp.n_layer, T, hp.n_embd), np.float32)
+        self.cap_lg = np.zeros((hp.n_layer, T, hp.n_ff), np.float32)
+        self.cap_src = np.zeros((hp.n_layer, T, hp.n_embd), np.float32)
+        self.O.pio_model_set_capture(self.h, _ptr(self.cap_ffn), _ptr(self.cap_lg), _ptr(self.cap_src))
+
+    def eval(self, tokens, n_past, nth=8):
+        tokens = np.ascontiguousarray(tokens, np.int32)
+        logits = np.zeros(self.hp.n_vocab, np.float32)
+        tok = self.O.pio_model_eval_simple(self.h, _ptr(tokens), tokens.size, n_past, _ptr(logits), nth)
+        assert tok >= 0
+        return tok, logits
+
+    def close(self):
+        if self.h:
+            self.O.pio_model_free(self.h)
+            self.h = None

@@ -1,0 +1,143 @@
+"""Decode engine (pi_model_* through the C ABI) against the CPU oracle on the same seeded weights.
+
+North-star tolerances: predictor masks agree on >= 99.9 % of neurons; per-layer FFN output within 2e-3
+relative error; logits within 1e-2 relative error; greedy tokens identical for the first 64 steps."""
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from oracle_lib import _ptr as P
+from powerinfer_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(a, b):
+    return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+def oracle_ffn_on(model, il, src):
+    """The oracle's FFN block of layer il applied to a given source vector (the vector before the norm)."""
+    hp, L = model["hp"], model["layers"][il]
+    O = ol.oracle()
+    d, ff, r = hp.n_embd, hp.n_ff, hp.n_rank
+    src = np.ascontiguousarray(src[None], np.float32)
+    xn = np.zeros_like(src)
+    if hp.arch == "llama":
+        O.pio_rms_norm(P(src), d, 1, hp.norm_eps, P(xn))
+        xn = xn * L["ffn_norm"]
+    else:
+        O.pio_norm(P(src), d, 1, hp.norm_eps, P(xn))
+        xn = xn * L["attn_norm"] + L["attn_norm_b"]
+    xn = np.ascontiguousarray(xn, np.float32)
+    return ol.ffn_sparse(O, d, ff, r, 1, hp.wtype, hp.arch == "llama", L["ffn_up"], L.get("ffn_gate"), L["ffn_down_t"],
+                         L["fc1"], L["fc2"], xn, src, np.zeros(ff, np.int32), hp.sparse_threshold, nth=8)
+
+
+def run_case(hp, n_prompt=12, n_gen=64):
+    """Both sides consume the same tokens.  Random-init weights make the comparison chaotic in one specific
+    way: activations are rounded to fp16 before every dot product (ggml.c:9703-9716), so an fp32 difference in
+    the last place (summation order) becomes a 1e-4 difference one layer later and can flip a neuron whose
+    predictor logit sits on the threshold.  The checks therefore are: masks agree on >= 99.9 % of all neurons
+    evaluated; each layer's FFN block, fed the GPU's own input, matches the oracle within 2e-3 whenever the two
+    masks are identical; logits within 1e-2; greedy tokens identical, a disagreement being admissible only where
+    the oracle's own logits tie within the logit tolerance."""
+    from powerinfer_amd.model import Model
+    model = synth.make_model(hp)
+    om = ol.OracleModel(model)
+    gm = Model(hp).load(model)
+    rng = np.random.default_rng(hp.seed + 99)
+    prompt = rng.integers(0, hp.n_vocab, n_prompt).astype(np.int32)
+    thr = hp.sparse_threshold
+
+    gm.set_capture(True)
+    om.capture(1)
+    n_past, flips, neurons, checked, skipped, lerr, clean_lerr = 0, 0, 0, 0, 0, [], []
+    for t in prompt:
+        tok_o, lg_o = om.eval([t], n_past)
+        tok_g, lg_g = gm.decode([t], n_past)
+        ffn_g, plg_g, na_g, src_g = gm.get_capture()
+        tflips = 0
+        for il in range(hp.n_layer):
+            mask_g = ~(plg_g[il] < thr)
+            tflips += int((mask_g != ~(om.cap_lg[il, 0] < thr)).sum())
+            assert na_g[il] == mask_g.sum()
+            o = oracle_ffn_on(model, il, src_g[il])
+            assert rel_err(plg_g[il], o["logits"][0]) < 1e-4
+            if np.array_equal(mask_g, ~(o["logits"][0] < thr)):
+                assert rel_err(ffn_g[il], o["out"][0]) < 2e-3, (il, rel_err(ffn_g[il], o["out"][0]))
+                checked += 1
+            else:
+                skipped += 1
+        flips += tflips
+        neurons += hp.n_layer * hp.n_ff
+        lerr.append(rel_err(lg_g, lg_o))
+        if tflips == 0:
+            clean_lerr.append(lerr[-1])
+        n_past += 1
+    assert 1 - flips / neurons >= 0.999, (flips, neurons)
+    assert skipped <= 0.1 * (checked + skipped), (checked, skipped)
+    assert np.median(lerr) < 1e-2, lerr
+    if hp.wtype == synth.F16:
+        assert not clean_lerr or max(clean_lerr) < 1e-2, clean_lerr
+    gm.set_capture(False)
+
+    # greedy loop: one HIP-graph replay per token on the device; the oracle is fed the GPU's trajectory
+    first = tok_g
+    toks_g, ms = gm.generate(n_gen)           # toks_g[s] = choice after consuming step s's token
+    consumed = [first] + list(toks_g[:-1])
+    same, explained = 0, 0
+    for s in range(n_gen):
+        tok_o, lg_o = om.eval([consumed[s]], n_past)
+        n_past += 1
+        if tok_o == toks_g[s]:
+            same += 1
+        elif lg_o[tok_o] - lg_o[toks_g[s]] <= 1e-2 * np.abs(lg_o).max():
+            explained += 1
+    assert same >= 0.9 * n_gen, (same, n_gen)
+    if hp.wtype == synth.F16:
+        assert same + explained == n_gen, (same, explained, n_gen)
+    # Q4_0: the int8 rounding of activations makes the reference itself jump by percents under a 1e-7
+    # perturbation (tests/test_oracle_math.py::test_reference_arithmetic_is_chaotic_under_last_bit_noise),
+    # so only the agreement rate is asserted
+    act = gm.step_active(n_gen)
+    assert (act > 0).all() and (act < hp.n_layer * hp.n_ff).all()
+    more, _ = gm.generate(3)                  # a second call continues from the device state
+    assert (more >= 0).all() and (more < hp.n_vocab).all()
+    gm.close(), om.close()
+    return same
+
+
+@pytest.mark.parametrize("wtype", [synth.F16, synth.Q4_0])
+def test_llama_tiny_greedy_matches_oracle(wtype):
+    run_case(synth.hparams("llama-tiny", wtype=wtype, n_ctx=128, seed=3))
+
+
+@pytest.mark.parametrize("wtype", [synth.F16, synth.Q4_0])
+def test_falcon_tiny_greedy_matches_oracle(wtype):
+    run_case(synth.hparams("falcon-tiny", wtype=wtype, n_ctx=128, seed=4))
+
+
+def test_falcon_single_norm_variant():
+    run_case(synth.hparams("falcon-tiny", n_ctx=96, seed=5, two_norms=False), n_prompt=6, n_gen=16)
+
+
+def test_llama_7b_width_two_layers():
+    """Full 7B layer shape (d 4096, ff 11008, rank 1024, 32 heads, vocab 32000), two layers."""
+    hp = synth.hparams("llama-7b", n_layer=2, n_ctx=128, seed=6)
+    run_case(hp, n_prompt=8, n_gen=64)
+
+
+def test_decode_rejects_bad_arguments():
+    from powerinfer_amd.model import Model
+    from powerinfer_amd.lib import PiError
+    hp = synth.hparams("llama-tiny", n_ctx=16, seed=7)
+    gm = Model(hp).load(synth.make_model(hp))
+    with pytest.raises(PiError):
+        gm.decode([hp.n_vocab], 0)                   # token id out of range
+    with pytest.raises(PiError):
+        gm.decode([1] * 17, 0)                       # longer than the context
+    gm.decode([1, 2, 3], 0)
+    with pytest.raises(PiError):
+        gm.generate(14)                              # would run past the context
+    gm.close()

@@ -1,0 +1,157 @@
+"""Dense operators of the decode path (mat-vec with fused norm, RoPE + KV store, decode attention, embedding,
+argmax) through the C ABI against the CPU oracle and the reference's golden vectors."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from oracle_lib import _ptr as P
+from powerinfer_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(a, b):
+    return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+def gpu_gemv(wtype, w, rows, cols, x, norm=None, epi=0, add1=None, add2=None):
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    dw, dx, dy = pl.DevBuf(host=w), pl.DevBuf(host=x.astype(np.float32)), pl.DevBuf(rows * 4)
+    d1 = pl.DevBuf(host=add1) if add1 is not None else None
+    d2 = pl.DevBuf(host=add2) if add2 is not None else None
+    na = None
+    keep = []
+    if norm is not None:
+        kind, eps, nw, nb = norm
+        bw = pl.DevBuf(host=nw) if nw is not None else None
+        bb = pl.DevBuf(host=nb) if nb is not None else None
+        keep += [bw, bb]
+        na = pl.norm_arg(kind, eps, bw, bb)
+    pl.check(L.pi_k_gemv(wtype, dw.ptr, rows, cols, dx.ptr, na, epi, d1.ptr if d1 else None, d2.ptr if d2 else None, dy.ptr, None), "gemv")
+    pl.sync()
+    return dy.download(np.float32)
+
+
+@pytest.mark.parametrize("wtype", [ol.F16, ol.Q4_0])
+@pytest.mark.parametrize("rows,cols", [(40, 256), (4096, 4096), (12288, 4096), (1024, 4096), (3000, 8192)])
+def test_gemv_plain(wtype, rows, cols):
+    rng = np.random.default_rng(rows + cols)
+    w32 = (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32)
+    w = synth.encode(w32, wtype)
+    x = rng.standard_normal(cols).astype(np.float32)
+    want = np.zeros(rows, np.float32)
+    assert ol.oracle().pio_mul_mat(wtype, P(w), rows, cols, P(x), 1, P(want), 8) == 0
+    got = gpu_gemv(wtype, w, rows, cols, x)
+    assert rel_err(got, want) < 2e-6
+
+
+def test_gemv_golden_reference(golden):
+    g = golden("ops")
+    for tag, wt in (("mm_f16", ol.F16), ("mm_q4", ol.Q4_0)):
+        w, x, y = g[tag + "_w"], g[tag + "_x"], g[tag + "_y"]
+        for t in range(x.shape[0]):
+            got = gpu_gemv(wt, w, y.shape[1], x.shape[1], x[t])
+            assert rel_err(got, y[t]) < 2e-6
+
+
+@pytest.mark.parametrize("wtype", [ol.F16, ol.Q4_0])
+@pytest.mark.parametrize("kind", [1, 2])
+def test_gemv_fused_norm_and_epilogues(wtype, kind):
+    from powerinfer_amd import lib as pl
+    rng = np.random.default_rng(kind * 7 + wtype)
+    rows, cols = 2048, 4096
+    w = synth.encode((rng.standard_normal((rows, cols)) * 0.02).astype(np.float32), wtype)
+    x = (rng.standard_normal(cols) * 3 + 0.5).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(cols)).astype(np.float32)
+    nb = (0.1 * rng.standard_normal(cols)).astype(np.float32) if kind == 2 else None
+    a1, a2 = rng.standard_normal(rows).astype(np.float32), rng.standard_normal(rows).astype(np.float32)
+    O = ol.oracle()
+    xn = np.zeros_like(x)
+    (O.pio_rms_norm if kind == 1 else O.pio_norm)(P(x), cols, 1, 1e-5, P(xn))
+    xn = xn * nw
+    if nb is not None:
+        xn = xn + nb
+    want = np.zeros(rows, np.float32)
+    assert O.pio_mul_mat(wtype, P(w), rows, cols, P(np.ascontiguousarray(xn, np.float32)), 1, P(want), 8) == 0
+    got = gpu_gemv(wtype, w, rows, cols, x, norm=(kind, 1e-5, nw, nb))
+    assert rel_err(got, want) < 5e-6
+    assert rel_err(gpu_gemv(wtype, w, rows, cols, x, norm=(kind, 1e-5, nw, nb), epi=pl.EPI_RELU), np.maximum(want, 0)) < 5e-6
+    assert rel_err(gpu_gemv(wtype, w, rows, cols, x, norm=(kind, 1e-5, nw, nb), epi=pl.EPI_ADD, add1=a1), want + a1) < 5e-6
+    assert rel_err(gpu_gemv(wtype, w, rows, cols, x, norm=(kind, 1e-5, nw, nb), epi=pl.EPI_ADD2, add1=a1, add2=a2), (want + a1) + a2) < 5e-6
+
+
+def test_gemv_rejects_bad_shapes():
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    b = pl.DevBuf(1024)
+    assert L.pi_k_gemv(pl.F16, b.ptr, 4, 12, b.ptr, None, 0, None, None, b.ptr, None) == -1      # cols % 8
+    assert L.pi_k_gemv(pl.Q4_0, b.ptr, 4, 48, b.ptr, None, 0, None, None, b.ptr, None) == -1     # cols % 32
+    assert L.pi_k_gemv(7, b.ptr, 4, 64, b.ptr, None, 0, None, None, b.ptr, None) == -3           # unsupported type
+    assert L.pi_k_gemv(pl.F16, None, 4, 64, b.ptr, None, 0, None, None, b.ptr, None) == -1
+    assert L.pi_k_gemv(pl.F16, b.ptr, 4, 64, b.ptr, None, pl.EPI_ADD, None, None, b.ptr, None) == -1
+    assert b"pi_k_gemv" in L.pi_last_error()
+
+
+@pytest.mark.parametrize("mode,hd,nh,nkv", [(0, 128, 4, 4), (2, 64, 8, 2)])
+def test_rope_attention_sequence(mode, hd, nh, nkv):
+    """Six decode steps: RoPE + KV store + attention on the GPU against the oracle's rope + attention with
+    the reference cache layout (K cell-major, V transposed)."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    O = ol.oracle()
+    rng = np.random.default_rng(mode + hd)
+    n_ctx, gqa, d = 48, nkv * hd, nh * hd
+    kc_o = np.zeros((n_ctx, gqa), np.uint16)
+    vc_o = np.zeros((gqa, n_ctx), np.uint16)
+    kc_g, vc_g = pl.DevBuf.zeros(nkv * n_ctx * hd * 2), pl.DevBuf.zeros(nkv * n_ctx * hd * 2)
+    dq, dpos, dqr, dout = pl.DevBuf((d + 2 * gqa) * 4), pl.DevBuf(4), pl.DevBuf(d * 4), pl.DevBuf(d * 4)
+    theta_scale = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
+    for pos in range(6):
+        qkv = rng.standard_normal(d + 2 * gqa).astype(np.float32)
+        q, k, v = qkv[:d], qkv[d:d + gqa], qkv[d + gqa:]
+        p = np.array([pos], np.int32)
+        qr, kr = np.zeros_like(q), np.zeros_like(k)
+        O.pio_rope(P(q), hd, nh, 1, P(p), hd, mode, 10000.0, 1.0, P(qr))
+        O.pio_rope(P(k), hd, nkv, 1, P(p), hd, mode, 10000.0, 1.0, P(kr))
+        n_kv = max(32, pos + 1)
+        mask = np.where(np.arange(n_kv)[None, :] > pos, -np.inf, 0).astype(np.float32)
+        want = np.zeros(d, np.float32)
+        assert O.pio_attention(hd, nh, nkv, n_ctx, n_kv, 1, P(p), P(mask), P(qr), P(kr), P(np.ascontiguousarray(v)), P(kc_o), P(vc_o), P(want)) == 0
+        dq.upload(qkv)
+        dpos.upload(p)
+        pl.check(L.pi_k_rope_kv_store(dq.ptr, nh, nkv, hd, mode, theta_scale, dpos.ptr, n_ctx, dqr.ptr, kc_g.ptr, vc_g.ptr, None), "rope")
+        pl.check(L.pi_k_attn_decode(dqr.ptr, kc_g.ptr, vc_g.ptr, nh, nkv, hd, n_ctx, dpos.ptr, dout.ptr, None), "attn")
+        pl.sync()
+        assert rel_err(dqr.download(np.float32), qr) < 1e-6
+        got = dout.download(np.float32)
+        assert rel_err(got, want) < 2e-3, (pos, rel_err(got, want))
+    # the caches hold the same fp16 values, in this library's [kv_head][cell][hd] layout
+    kg = kc_g.download(np.uint16).reshape(nkv, n_ctx, hd)
+    vg = vc_g.download(np.uint16).reshape(nkv, n_ctx, hd)
+    ko = kc_o.reshape(n_ctx, nkv, hd).transpose(1, 0, 2)
+    vo = vc_o.reshape(nkv, hd, n_ctx).transpose(0, 2, 1)
+    assert (kg[:, :6] != ko[:, :6]).mean() < 2e-3          # cos/sin may differ in the last place before rounding
+    assert np.array_equal(vg[:, :6], vo[:, :6])
+
+
+def test_embed_and_argmax():
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    rng = np.random.default_rng(0)
+    tab32 = (rng.standard_normal((100, 256)) * 0.02).astype(np.float32)
+    for wt in (ol.F16, ol.Q4_0):
+        tab = synth.encode(tab32, wt)
+        dt, dtok, dx = pl.DevBuf(host=tab), pl.DevBuf(host=np.array([37], np.int32)), pl.DevBuf(256 * 4)
+        pl.check(L.pi_k_embed(wt, dt.ptr, 256, dtok.ptr, dx.ptr, None), "embed")
+        pl.sync()
+        want = tab[37].astype(np.float32) if wt == ol.F16 else synth.dequantize_q4_0(tab[37:38], 256)[0]
+        assert np.array_equal(dx.download(np.float32), want)
+    lg = rng.standard_normal(32000).astype(np.float32)
+    lg[[123, 20000]] = lg.max() + 1          # tie: the first index wins
+    dl, dtok = pl.DevBuf(host=lg), pl.DevBuf(4)
+    pl.check(L.pi_k_argmax(dl.ptr, 32000, dtok.ptr, None), "argmax")
+    pl.sync()
+    assert dtok.download(np.int32)[0] == 123 == int(np.argmax(lg))

@@ -210,3 +210,28 @@ def test_zipf_predictor_hits_target_rate():
     assert 0.07 < rate < 0.13
     hot = np.argsort(-L["p"])[:100]
     assert (o["logits"][:, hot] >= 0).mean() > 0.8
+
+
+def test_reference_arithmetic_is_chaotic_under_last_bit_noise():
+    """Why model-level parity is statistical.  The CPU path rounds activations to fp16 (F16 weights) or to
+    int8 blocks (Q4_0 weights) before every dot product, so a perturbation in the LAST BIT of one fp32 input
+    is amplified by many orders of magnitude within a couple of layers, and flips neurons whose predictor
+    logit sits on the threshold.  Any implementation that sums in a different order than the scalar CPU loop
+    differs by more than that last bit, so per-token bit-level agreement of a whole model is not attainable;
+    agreement is asserted per operator (tight), per layer on identical inputs (tight) and statistically over
+    trajectories."""
+    for wt, floor in ((ol.F16, 1e-5), (ol.Q4_0, 1e-4)):
+        hp = synth.hparams("llama-tiny", n_ctx=32, seed=3, wtype=wt)
+        m = synth.make_model(hp)
+        m2 = dict(hp=hp, glob=m["glob"], layers=[dict(L) for L in m["layers"]])
+        noise = np.random.default_rng(0).standard_normal(hp.n_embd)
+        m2["layers"][0]["attn_norm"] = (m["layers"][0]["attn_norm"] * (1 + 1e-7 * noise)).astype(np.float32)
+        a, b = ol.OracleModel(m), ol.OracleModel(m2)
+        worst, n = 0.0, 0
+        for t in np.random.default_rng(1).integers(0, hp.n_vocab, 6):
+            _, la = a.eval([int(t)], n, nth=4)
+            _, lb = b.eval([int(t)], n, nth=4)
+            n += 1
+            worst = max(worst, float(np.abs(la - lb).max() / np.abs(la).max()))
+        assert worst > floor, (wt, worst)       # 1e-7 in, > 1e-5 (F16) / > 1e-4 (Q4_0) out
+        a.close(), b.close()

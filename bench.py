@@ -1,0 +1,228 @@
+#!/usr/bin/env python3
+"""Benchmark of the sparse decode token loop on one MI355X.
+
+Workload (BASELINE.json configs[1]): 32-layer ReLU-LLaMA-2-7B-shaped model, random-init FP16 weights generated
+in HBM, per-layer rank-1024 predictors with Zipf(1.2) firing rates (~10 % of neurons active), all neurons on
+the GPU; a 64-token random prompt, then greedy decode at batch 1.  One "step" = one decoded token.
+
+    python bench.py [--gpus 1] [--steps 256] [--warmup 8]
+
+Prints ONE JSON line: decode tok/s, the HBM roofline of the kernel that moves the most bytes per token
+(measured here with HIP events on the engine's stream), the touched-bytes accounting of the whole token
+loop, and a CPU baseline (the repo's CPU port of the reference path, timed on the host cores on a bounded
+sample of the same workload).
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+import numpy as np
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBPS = 8000.0
+
+
+def build_synthetic_on_device(hp, keep):
+    """Random-init weights generated directly in HBM (pi_fill_normal_f16), predictor fc2 rows carrying the
+    Zipf firing-rate bias computed on the host (powerinfer_amd.synth)."""
+    from powerinfer_amd import lib as pl, synth
+    from powerinfer_amd.model import Model
+    from scipy.special import ndtri
+    L = pl.init()
+    m = Model(hp)
+    d, ff, r = hp.n_embd, hp.n_ff, hp.n_rank
+    gqa = d // hp.n_head * hp.n_head_kv
+    seed = [hp.seed * 1000003 + 17]
+
+    def normal(rows, cols, bias=None):
+        buf = pl.DevBuf(rows * cols * 2)
+        seed[0] += 1
+        pl.check(L.pi_fill_normal_f16(buf.ptr, rows * cols, seed[0], 0.02, bias.ptr if bias is not None else None, cols, None), "fill")
+        keep.append(buf)
+        return buf
+
+    def put(layer, kind, buf, rows, cols):
+        m.set_tensor_device(layer, kind, buf.ptr, pl.F16, cols, rows)
+
+    put(-1, "tok_embd", normal(hp.n_vocab, d), hp.n_vocab, d)
+    put(-1, "output", normal(hp.n_vocab, d), hp.n_vocab, d)
+    m.set_tensor(-1, "output_norm", np.ones(d, np.float32))
+    rng = np.random.default_rng(hp.seed)
+    for il in range(hp.n_layer):
+        m.set_tensor(il, "attn_norm", np.ones(d, np.float32))
+        m.set_tensor(il, "ffn_norm", np.ones(d, np.float32))
+        put(il, "wqkv", normal(d + 2 * gqa, d), d + 2 * gqa, d)
+        put(il, "wo", normal(d, d), d, d)
+        put(il, "ffn_gate", normal(ff, d), ff, d)
+        put(il, "ffn_up", normal(ff, d), ff, d)
+        put(il, "ffn_down_t", normal(ff, d), ff, d)
+        put(il, "fc1", normal(r, d), r, d)
+        p, _ = synth.zipf_rates(ff, hp.mean_rate, rng)
+        b = (0.02 * np.sqrt(np.pi) * ndtri(p) / np.sqrt(r)).astype(np.float32)
+        bias = pl.DevBuf(host=b)
+        put(il, "fc2", normal(ff, r, bias), ff, r)
+    pl.sync()
+    m.finalize()
+    return m
+
+
+def download_model(hp, keep):
+    """Host copies of the device-generated tensors, in the dict layout powerinfer_amd.synth.make_model uses
+    (feeds the CPU port for the cpu_baseline leg)."""
+    d, ff, r = hp.n_embd, hp.n_ff, hp.n_rank
+    gqa = d // hp.n_head * hp.n_head_kv
+    it = iter(keep)
+    grab = lambda rows, cols: next(it).download(np.float16).reshape(rows, cols)  # noqa: E731
+    glob = dict(tok_embd=grab(hp.n_vocab, d), output=grab(hp.n_vocab, d), output_norm=np.ones(d, np.float32))
+    layers = []
+    for _ in range(hp.n_layer):
+        Lr = dict(attn_norm=np.ones(d, np.float32), ffn_norm=np.ones(d, np.float32))
+        wqkv = grab(d + 2 * gqa, d)
+        Lr["wq"], Lr["wk"], Lr["wv"] = (np.ascontiguousarray(a) for a in (wqkv[:d], wqkv[d:d + gqa], wqkv[d + gqa:]))
+        Lr["wo"], Lr["ffn_gate"], Lr["ffn_up"], Lr["ffn_down_t"] = grab(d, d), grab(ff, d), grab(ff, d), grab(ff, d)
+        Lr["fc1"], Lr["fc2"] = grab(r, d), grab(ff, r)
+        layers.append(Lr)
+    return dict(hp=hp, glob=glob, layers=layers)
+
+
+def touched_bytes_per_token(hp, active_sum, n_kv_mean):
+    """Algorithmic bytes of one decoded token:  sum_l [ W_attn + W_pred + A_l * n_mats * R + 2 * n_kv * n_embd_gqa * 2 ]
+    + W_lmhead + d * 2, with the measured per-token sum of active rows."""
+    d, ff, r, Lr = hp.n_embd, hp.n_ff, hp.n_rank, hp.n_layer
+    gqa = d // hp.n_head * hp.n_head_kv
+    s = 2.0
+    w_attn = (d * (d + 2 * gqa) + d * d) * s
+    w_pred = (d * r + r * ff) * 2.0
+    row = d * s
+    return Lr * (w_attn + w_pred + 2 * n_kv_mean * gqa * 2.0) + active_sum * 3 * row + hp.n_vocab * d * s + d * 2.0
+
+
+def cpu_baseline(hp, keep, prompt, n_prompt, n_decode, threads):
+    sys.path.insert(0, os.path.join(ROOT, "tests"))
+    import oracle_lib as ol
+    model = download_model(hp, keep)
+    om = ol.OracleModel(model)
+    n_past = 0
+    tok = 0
+    for t in prompt[:n_prompt]:
+        tok, _ = om.eval([int(t)], n_past, nth=threads)
+        n_past += 1
+    t0 = time.perf_counter()
+    for _ in range(n_decode):
+        tok, _ = om.eval([tok], n_past, nth=threads)
+        n_past += 1
+    dt = time.perf_counter() - t0
+    om.close()
+    return n_decode / dt
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=256)
+    ap.add_argument("--warmup", type=int, default=8)
+    ap.add_argument("--prompt", type=int, default=64)
+    ap.add_argument("--layers", type=int, default=32, help="only for quick trials; the reported workload uses 32")
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--cpu-tokens", type=int, default=24)
+    args = ap.parse_args()
+    if args.gpus != 1:
+        sys.exit("bench.py: this build runs the token loop on ONE GPU; --gpus must be 1 "
+                 "(how the path would shard over xGMI is described in DESIGN.md)")
+
+    from powerinfer_amd import lib as pl, synth
+    hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=args.prompt + args.warmup + args.steps + 8, seed=1)
+    keep = []
+    t0 = time.perf_counter()
+    m = build_synthetic_on_device(hp, keep)
+    t_build = time.perf_counter() - t0
+
+    rng = np.random.default_rng(2024)
+    prompt = rng.integers(0, hp.n_vocab, args.prompt).astype(np.int32)
+    m.decode(prompt, 0, want_logits=False)                    # prompt phase (not timed)
+    if args.warmup > 0:
+        m.generate(args.warmup)                               # warm-up steps (captures the HIP graph)
+    pl.sync()
+    t0 = time.perf_counter()
+    toks, ms_dev = m.generate(args.steps)                     # timed: exactly K decode steps, device events inside
+    pl.sync()
+    wall = time.perf_counter() - t0
+    ms_per_step = wall * 1e3 / args.steps
+    act = m.step_active(args.steps).astype(np.float64)
+    n_kv_mean = args.prompt + args.warmup + (args.steps + 1) / 2.0
+    tok_bytes = touched_bytes_per_token(hp, act.mean(), n_kv_mean)
+
+    # roofline of the dominant kernel: the q|k|v projection mat-vec (gemv_f16_kernel<4>), one launch per layer
+    d = hp.n_embd
+    gqa = d // hp.n_head * hp.n_head_kv
+    ms_qkv, n_qkv = m.time_section(0, 8)
+    qkv_bytes = (d + 2 * gqa) * d * 2.0 + d * 4 + (d + 2 * gqa) * 4          # weights + activation in + result out
+    achieved = qkv_bytes / (ms_qkv * 1e-3) / 1e9
+    ms_ffn, _ = m.time_section(1, 8)
+    ffn_bytes = (d * hp.n_rank + hp.n_rank * hp.n_ff) * 2.0 + (act.mean() / hp.n_layer) * 3 * d * 2.0
+    ms_head, _ = m.time_section(2, 8)
+
+    out = {
+        "metric": "decode tok/s bs=1 ReLU-Llama2-7B FP16",
+        "value": round(1e3 / ms_per_step, 2),
+        "unit": "tok/s",
+        "n_gpus": 1,
+        "steps": args.steps,
+        "warmup": args.warmup,
+        "ms_per_step": round(ms_per_step, 4),
+        "higher_is_better": True,
+        "scaling": "weak",
+        "vs_baseline": None,
+        "dtype": "f16",
+        "data": "synthetic",
+        "config": {
+            "workload": "configs[1]: ReLU-LLaMA-2-7B shape (d 4096, ff 11008, 32 heads, vocab 32000, predictor rank 1024), "
+                        f"{hp.n_layer} layers, random-init FP16 weights, all neurons on the GPU, {args.prompt}-token random prompt, "
+                        "greedy decode at batch 1",
+            "n_layer": hp.n_layer, "prompt_tokens": args.prompt, "n_ctx": hp.n_ctx,
+            "mean_active_per_layer": round(act.mean() / hp.n_layer, 1),
+            "device": pl.device_name(),
+        },
+        "roofline": {
+            "bound": "hbm",
+            "kernel": "gemv_f16_kernel<4> (q|k|v projection, 12288 x 4096 fp16, fused RMSNorm)",
+            "achieved": round(achieved, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "traffic": None,
+            "bytes_per_launch": qkv_bytes,
+            "us_per_launch": round(ms_qkv * 1e3, 2),
+            "launches_timed": n_qkv,
+        },
+        "token_loop": {
+            "device_ms_per_step": round(ms_dev / args.steps, 4),
+            "touched_GB_per_token": round(tok_bytes / 1e9, 4),
+            "effective_GBps": round(tok_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+            "hbm_frac_touched": round(tok_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "sparse_ffn_us_per_layer": round(ms_ffn * 1e3, 2),
+            "sparse_ffn_effective_GBps": round(ffn_bytes / (ms_ffn * 1e-3) / 1e9, 1),
+            "lm_head_us": round(ms_head * 1e3, 2),
+            "build_s": round(t_build, 1),
+        },
+    }
+    if not args.no_cpu:
+        threads = min(16, os.cpu_count() or 1)
+        n_prompt = 8
+        v = cpu_baseline(hp, keep, prompt, n_prompt, args.cpu_tokens, threads)
+        out["cpu_baseline"] = {
+            "value": round(v, 3), "unit": "tok/s", "cores": threads, "kind": "port",
+            "sample": f"same {hp.n_layer}-layer model and weights (copied back from HBM), {n_prompt}-token prompt then "
+                      f"{args.cpu_tokens} greedy decode tokens timed, oracle/pi_oracle.c with OpenMP",
+        }
+    m.close()
+    print(json.dumps(out), flush=True)
+
+
+if __name__ == "__main__":
+    main()

@@ -217,6 +217,16 @@ PI_API int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, fl
 PI_API int pi_model_set_capture(pi_model * m, int enable);
 PI_API int pi_model_get_capture(pi_model * m, float * ffn_out, float * pred_logits, int32_t * n_active, float * ffn_src);
 
+/*
+ * Event-timed replay of one section of the token loop on the model's stream, `rounds` passes over all layers,
+ * on the activations the last token left behind (the per-node timers of GGML_PERF, ggml.c:16604-16619, are the
+ * nearest thing in the reference).  section 0: the q|k|v projection mat-vec of every layer (the kernel that
+ * moves the most bytes per token); 1: the sparse FFN block of every layer (fc1, fc2+compaction, up/gate, axpy);
+ * 2: the lm-head mat-vec.  ms_total: device milliseconds for everything issued; launches: number of
+ * section instances issued (rounds * n_layer, or rounds for the lm-head).
+ */
+PI_API int pi_model_time_section(pi_model * m, int section, int rounds, float * ms_total, int * launches);
+
 /* for each of the n_steps tokens of the most recent pi_model_generate: the sum over layers of the active-row
  * counts (feeds the touched-bytes accounting of the benchmark) */
 PI_API int pi_model_step_active(pi_model * m, int32_t * per_step_total, int n_steps);

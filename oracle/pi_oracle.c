@@ -22,7 +22,7 @@
 #ifdef _OPENMP
 #include <omp.h>
 #endif
-#if defined(__F16C__)
+#if defined(__F16C__) || defined(__AVX2__)
 #include <immintrin.h>
 #endif
 
@@ -142,7 +142,37 @@ void pio_quantize_row_q8_0(const float * x, void * vy, int64_t n) {
  * fp16 dot: ggml_vec_dot_f16, ggml.c:1188-1222 with the AVX2 macros (:745-800): steps of 32
  * elements into 4 accumulators of 8 fp32 lanes by FMA, the reduce of :760-778, leftovers in double.
  * ---------------------------------------------------------------------------------------- */
+#if defined(__AVX2__) && defined(__F16C__) && defined(__FMA__)
+#define PIO_SIMD 1
+/* same arithmetic as the portable loops below, written with the x86 vector instructions so that the CPU
+ * baseline runs at a realistic speed: 4 accumulators x 8 lanes, lane l of accumulator j holds the elements
+ * 32k + 8j + l in increasing k */
+static inline float dot_f16_simd(int64_t n, const uint16_t * x, const uint16_t * y, int64_t * done) {
+    __m256 a0 = _mm256_setzero_ps(), a1 = a0, a2 = a0, a3 = a0;
+    const int64_t np = n & ~(int64_t)31;
+    for (int64_t i = 0; i < np; i += 32) {
+        a0 = _mm256_fmadd_ps(_mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(x + i))),      _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(y + i))),      a0);
+        a1 = _mm256_fmadd_ps(_mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(x + i + 8))),  _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(y + i + 8))),  a1);
+        a2 = _mm256_fmadd_ps(_mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(x + i + 16))), _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(y + i + 16))), a2);
+        a3 = _mm256_fmadd_ps(_mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(x + i + 24))), _mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(y + i + 24))), a3);
+    }
+    a0 = _mm256_add_ps(_mm256_add_ps(a0, a2), _mm256_add_ps(a1, a3));
+    const __m128 t0 = _mm_add_ps(_mm256_castps256_ps128(a0), _mm256_extractf128_ps(a0, 1));
+    const __m128 t1 = _mm_hadd_ps(t0, t0);
+    *done = np;
+    return _mm_cvtss_f32(_mm_hadd_ps(t1, t1));
+}
+#endif
+
 float pio_vec_dot_f16(int64_t n, const uint16_t * x, const uint16_t * y) {
+#ifdef PIO_SIMD
+    {
+        int64_t np;
+        double sumf = dot_f16_simd(n, x, y, &np);
+        for (int64_t i = np; i < n; ++i) sumf += (double)(H2F(x[i]) * H2F(y[i]));
+        return (float)sumf;
+    }
+#endif
     float acc[4][8];
     memset(acc, 0, sizeof acc);
     const int64_t np = n & ~(int64_t)31;
@@ -167,6 +197,26 @@ float pio_vec_dot_f16(int64_t n, const uint16_t * x, const uint16_t * y) {
 float pio_vec_dot_q4_0_q8_0(int64_t n, const void * vx, const void * vy) {
     const blk_q4_0 * x = (const blk_q4_0 *)vx;
     const blk_q8_0 * y = (const blk_q8_0 *)vy;
+#ifdef PIO_SIMD
+    {
+        __m256 accv = _mm256_setzero_ps();
+        const __m256i m4 = _mm256_set1_epi8(0x0F), off = _mm256_set1_epi8(8), ones = _mm256_set1_epi16(1);
+        for (int64_t b = 0; b < n / QK; ++b) {
+            const __m256 d = _mm256_set1_ps(H2F(x[b].d) * H2F(y[b].d));
+            const __m128i raw = _mm_loadu_si128((const __m128i *)x[b].qs);
+            __m256i q = _mm256_and_si256(_mm256_set_m128i(_mm_srli_epi16(raw, 4), raw), m4);   /* low nibbles | high nibbles */
+            q = _mm256_sub_epi8(q, off);
+            const __m256i yv = _mm256_loadu_si256((const __m256i *)y[b].qs);
+            const __m256i p16 = _mm256_maddubs_epi16(_mm256_sign_epi8(q, q), _mm256_sign_epi8(yv, q));
+            const __m256i p32 = _mm256_madd_epi16(ones, p16);                                  /* 8 sums of 4 adjacent products */
+            accv = _mm256_fmadd_ps(d, _mm256_cvtepi32_ps(p32), accv);
+        }
+        __m128 r = _mm_add_ps(_mm256_extractf128_ps(accv, 1), _mm256_castps256_ps128(accv));
+        r = _mm_add_ps(r, _mm_movehl_ps(r, r));
+        r = _mm_add_ss(r, _mm_movehdup_ps(r));
+        return _mm_cvtss_f32(r);
+    }
+#endif
     float acc[8] = {0};
     for (int64_t b = 0; b < n / QK; ++b) {
         const float d = H2F(x[b].d) * H2F(y[b].d);
@@ -233,12 +283,39 @@ int pio_mul_mat_sparse(int wtype, const void * w, int64_t rows, int64_t cols, co
 /* one axpy row, F16: ggml_axpy_avx_f16, ggml.c:14292-14312 (FMA of fp32(w) * fp32(fp16 alpha) into fp32) */
 static void axpy_row_f16(int64_t n, const uint16_t * w, float * acc, uint16_t alpha) {
     const float a = H2F(alpha);
+#ifdef PIO_SIMD
+    if ((n & 7) == 0) {
+        const __m256 av = _mm256_set1_ps(a);
+        for (int64_t i = 0; i < n; i += 8)
+            _mm256_storeu_ps(acc + i, _mm256_fmadd_ps(_mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(w + i))), av, _mm256_loadu_ps(acc + i)));
+        return;
+    }
+#endif
     for (int64_t i = 0; i < n; ++i) acc[i] = fmaf(H2F(w[i]), a, acc[i]);
 }
 /* one axpy row, Q4_0: ggml_axpy_q4_0_q8_0, ggml-quants.c:2426-2509: int16 product (q-8)*alpha,
  * converted to fp32, multiplied by d_w*d_h, then a separate add (no FMA) */
 static void axpy_row_q4_0(int64_t n, const blk_q4_0 * w, float * acc, int8_t alpha, uint16_t scale) {
     const float sc = H2F(scale);
+#ifdef PIO_SIMD
+    {
+        const __m256i al = _mm256_set1_epi16((short)alpha), m4 = _mm256_set1_epi8(0x0F), off = _mm256_set1_epi8(8);
+        for (int64_t b = 0; b < n / QK; ++b) {
+            const __m256 d = _mm256_set1_ps(H2F(w[b].d) * sc);
+            const __m128i raw = _mm_loadu_si128((const __m128i *)w[b].qs);
+            __m256i q = _mm256_sub_epi8(_mm256_and_si256(_mm256_set_m128i(_mm_srli_epi16(raw, 4), raw), m4), off);
+            float * o = acc + b * QK;
+            for (int half = 0; half < 2; ++half) {
+                const __m256i p16 = _mm256_mullo_epi16(_mm256_cvtepi8_epi16(half ? _mm256_extracti128_si256(q, 1) : _mm256_castsi256_si128(q)), al);
+                const __m256 f0 = _mm256_mul_ps(_mm256_cvtepi32_ps(_mm256_cvtepi16_epi32(_mm256_castsi256_si128(p16))), d);
+                const __m256 f1 = _mm256_mul_ps(_mm256_cvtepi32_ps(_mm256_cvtepi16_epi32(_mm256_extracti128_si256(p16, 1))), d);
+                _mm256_storeu_ps(o + half * 16,     _mm256_add_ps(_mm256_loadu_ps(o + half * 16), f0));
+                _mm256_storeu_ps(o + half * 16 + 8, _mm256_add_ps(_mm256_loadu_ps(o + half * 16 + 8), f1));
+            }
+        }
+        return;
+    }
+#endif
     for (int64_t b = 0; b < n / QK; ++b) {
         const float d = H2F(w[b].d) * sc;
         float * o = acc + b * QK;

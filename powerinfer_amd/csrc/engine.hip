@@ -220,14 +220,14 @@ pi_model * pi_model_create(const pi_hparams * hp) {
 
 void pi_model_free(pi_model * m) {
     if (!m) return;
-    if (m->graph_exec) hipGraphExecDestroy(m->graph_exec);
-    if (m->graph) hipGraphDestroy(m->graph);
-    if (m->ev0) hipEventDestroy(m->ev0);
-    if (m->ev1) hipEventDestroy(m->ev1);
+    if (m->graph_exec) (void)hipGraphExecDestroy(m->graph_exec);
+    if (m->graph) (void)hipGraphDestroy(m->graph);
+    if (m->ev0) (void)hipEventDestroy(m->ev0);
+    if (m->ev1) (void)hipEventDestroy(m->ev1);
     if (m->cold) pi::cold_destroy(m->cold);
     if (m->ws) pi_workspace_destroy(m->ws);
     for (void * p : m->owned) pi_free(p);
-    if (m->stream) hipStreamDestroy(m->stream);
+    if (m->stream) (void)hipStreamDestroy(m->stream);
     delete m;
 }
 
@@ -406,7 +406,7 @@ int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * m
         if (rc == PI_OK) rc = launch_advance(m);
         hipGraph_t g = nullptr;
         const hipError_t e = hipStreamEndCapture(m->stream, &g);
-        if (rc != PI_OK) { if (g) hipGraphDestroy(g); return rc; }
+        if (rc != PI_OK) { if (g) (void)hipGraphDestroy(g); return rc; }
         if (e != hipSuccess) return pi::hip_fail(e, "hipStreamEndCapture");
         m->graph = g;
         PI_HIP_TRY(hipGraphInstantiate(&m->graph_exec, g, nullptr, nullptr, 0));
@@ -424,6 +424,57 @@ int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * m
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
     if (ms_out) PI_HIP_TRY(hipEventElapsedTime(ms_out, m->ev0, m->ev1));
     PI_TRY(pi_memcpy_d2h(out_tokens, m->d_out_tokens, sizeof(int32_t) * n_steps));
+    return PI_OK;
+}
+
+int pi_model_time_section(pi_model * m, int section, int rounds, float * ms_total, int * launches) {
+    if (!m || !m->finalized || !ms_total || !launches || rounds <= 0) return pi::fail(PI_E_ARG, "pi_model_time_section: bad arguments");
+    if (m->hybrid) return pi::fail(PI_E_UNSUPPORTED, "pi_model_time_section: not available for hybrid models");
+    const pi_hparams & hp = m->hp;
+    const int d = hp.n_embd, ff = hp.n_ff, gqa = m->gqa;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    hipStream_t st = m->stream;
+    PI_HIP_TRY(hipStreamSynchronize(st));
+    int n = 0;
+    PI_HIP_TRY(hipEventRecord(m->ev0, st));
+    for (int r = 0; r < rounds; ++r) {
+        if (section == 2) {
+            pi_norm on = make_norm(falcon ? 2 : 1, hp.norm_eps, m->glob[PI_T_OUTPUT_NORM], falcon ? &m->glob[PI_T_OUTPUT_NORM_B] : nullptr);
+            PI_TRY(pi_k_gemv(m->glob[PI_T_OUTPUT].type, m->glob[PI_T_OUTPUT].dev, hp.n_vocab, d, m->x, &on, PI_EPI_NONE, nullptr, nullptr, m->logits, st));
+            ++n;
+            continue;
+        }
+        for (int il = 0; il < hp.n_layer; ++il) {
+            if (section == 0) {
+                Tensor & wqkv = m->L(il, PI_T_WQKV);
+                pi_norm an = falcon ? make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B))
+                                    : make_norm(1, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), nullptr);
+                PI_TRY(pi_k_gemv(wqkv.type, wqkv.dev, d + 2 * gqa, d, m->x, &an, PI_EPI_NONE, nullptr, nullptr, m->qkv, st));
+                ++n;
+            } else if (section == 1) {
+                // the sparse FFN block as the decode loop issues it, on the activations the last token left behind
+                Tensor & fc1 = m->L(il, PI_T_FC1); Tensor & fc2 = m->L(il, PI_T_FC2);
+                Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
+                const bool q4 = up.type == PI_TYPE_Q4_0;
+                pi_norm fn = falcon ? make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B))
+                                    : make_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
+                PI_TRY(pi_k_gemv(fc1.type, fc1.dev, (int)fc1.ne1, d, m->ffn_inp, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, st));
+                PI_TRY(pi_k_predictor_fc2(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, nullptr, 0, m->pred_logits, m->list, m->n_active + il,
+                                          q4 ? m->h_dense : nullptr, m->ws, st));
+                PI_TRY(pi_k_sparse_upgate(up.type, up.dev, falcon ? nullptr : gate.dev, d, m->ffn_inp, &fn, m->list, m->n_active + il, nullptr, m->h_c,
+                                          q4 ? m->h_dense : nullptr, nullptr, nullptr, st));
+                PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, m->n_active + il,
+                                        PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, m->ws, st));
+                ++n;
+            } else {
+                return pi::fail(PI_E_ARG, "pi_model_time_section: unknown section");
+            }
+        }
+    }
+    PI_HIP_TRY(hipEventRecord(m->ev1, st));
+    PI_HIP_TRY(hipStreamSynchronize(st));
+    PI_HIP_TRY(hipEventElapsedTime(ms_total, m->ev0, m->ev1));
+    *launches = n;
     return PI_OK;
 }
 

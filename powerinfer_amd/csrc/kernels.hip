@@ -762,7 +762,7 @@ int pi_k_gemv(int wtype, const void * W, int rows, int cols, const float * x, co
         return pi::fail(PI_E_ARG, "pi_k_gemv: bad epilogue arguments");
     hipStream_t st = (hipStream_t)stream;
     const NormArgs na = to_norm(norm);
-    const int rpw = rows >= 8192 ? 4 : rows >= 2048 ? 2 : 1;
+    const int rpw = rows >= 16384 ? 8 : rows >= 8192 ? 4 : rows >= 2048 ? 2 : 1;   // rows per wave (8: lm-head sized matrices)
     const int n_groups = (rows + rpw - 1) / rpw;
     int blocks = (n_groups + kWavesPerBlock - 1) / kWavesPerBlock;
     if (blocks > 4096) blocks = 4096;
@@ -771,7 +771,8 @@ int pi_k_gemv(int wtype, const void * W, int rows, int cols, const float * x, co
         const size_t sh = (size_t)cols * 2;
         if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv: cols too large for LDS staging");
         const __half * w = (const __half *)W;
-        if (rpw == 4)      hipLaunchKernelGGL(gemv_f16_kernel<4>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        if (rpw == 8)      hipLaunchKernelGGL(gemv_f16_kernel<8>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        else if (rpw == 4) hipLaunchKernelGGL(gemv_f16_kernel<4>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
         else if (rpw == 2) hipLaunchKernelGGL(gemv_f16_kernel<2>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
         else               hipLaunchKernelGGL(gemv_f16_kernel<1>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
     } else if (wtype == PI_TYPE_Q4_0) {
@@ -779,7 +780,8 @@ int pi_k_gemv(int wtype, const void * W, int rows, int cols, const float * x, co
         const size_t sh = (size_t)cols + (size_t)(cols / 32) * 4 + (size_t)cols * 4;
         if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv: cols too large for LDS staging");
         const pi_block_q4_0 * w = (const pi_block_q4_0 *)W;
-        if (rpw == 4)      hipLaunchKernelGGL(gemv_q4_kernel<4>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        if (rpw == 8)      hipLaunchKernelGGL(gemv_q4_kernel<8>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        else if (rpw == 4) hipLaunchKernelGGL(gemv_q4_kernel<4>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
         else if (rpw == 2) hipLaunchKernelGGL(gemv_q4_kernel<2>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
         else               hipLaunchKernelGGL(gemv_q4_kernel<1>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
     } else {

@@ -36,11 +36,12 @@ def _declare(L):
     L.pi_model_set_capture.restype, L.pi_model_set_capture.argtypes = i, [vp, i]
     L.pi_model_get_capture.restype, L.pi_model_get_capture.argtypes = i, [vp, vp, vp, vp, vp]
     L.pi_model_step_active.restype, L.pi_model_step_active.argtypes = i, [vp, vp, i]
+    L.pi_model_time_section.restype, L.pi_model_time_section.argtypes = i, [vp, i, i, C.POINTER(C.c_float), C.POINTER(C.c_int)]
 
 
 ENGINE_SYMBOLS = ["pi_model_create", "pi_model_free", "pi_model_set_tensor", "pi_model_finalize", "pi_model_kv_clear",
                   "pi_model_decode", "pi_model_generate", "pi_model_set_capture", "pi_model_get_capture",
-                  "pi_model_step_active"]
+                  "pi_model_step_active", "pi_model_time_section"]
 
 
 def _type_of(a, hint):
@@ -133,6 +134,12 @@ class Model:
         out = np.empty(n_steps, np.int32)
         check(self.L.pi_model_step_active(self.h, out.ctypes.data_as(C.c_void_p), n_steps), "step_active")
         return out
+
+    def time_section(self, section, rounds):
+        """(ms per instance, instances) of a replayed section: 0 qkv mat-vec, 1 sparse FFN block, 2 lm-head."""
+        ms, n = C.c_float(0), C.c_int(0)
+        check(self.L.pi_model_time_section(self.h, section, rounds, C.byref(ms), C.byref(n)), "time_section")
+        return float(ms.value) / n.value, n.value
 
     def close(self):
         if self.h:

@@ -276,17 +276,30 @@ __device__ void compact_from_words(const uint32_t * words, int ff, const int32_t
 }
 
 // returns true in every thread of the block that took the last ticket; resets the counter for the next launch
+#ifndef PI_FENCE_MODE
+#define PI_FENCE_MODE 1
+#endif
 __device__ bool last_block_done(unsigned int * counter, unsigned int n_blocks, int * sflag) {
+#if PI_FENCE_MODE == 0
     __threadfence();
+#endif
     __syncthreads();
     if (threadIdx.x == 0) {
+#if PI_FENCE_MODE == 1
+        __threadfence();          // cumulative: publishes the whole block's stores, ordered before the ticket
+#endif
         const unsigned int t = atomicAdd(counter, 1u);
         *sflag = (t == n_blocks - 1);
         if (t == n_blocks - 1) *counter = 0;
+#if PI_FENCE_MODE == 1
+        if (t == n_blocks - 1) __threadfence();
+#endif
     }
     __syncthreads();
     const bool last = *sflag != 0;
+#if PI_FENCE_MODE == 0
     if (last) __threadfence();
+#endif
     return last;
 }
 

@@ -44,39 +44,83 @@ __device__ float block_max_f32(float v, float * red) {
 // second fp32 multiply: llm_build_norm, llama.cpp:4420-4450); LayerNorm as ggml.c:9169-9236.
 // ---------------------------------------------------------------------------------------------------
 __device__ void stage_x_f16(__half * xs, const float * __restrict__ x, int cols, NormArgs na, double * red) {
-    if (na.kind == 0) {
-        for (int i = threadIdx.x; i < cols; i += blockDim.x) xs[i] = __float2half_rn(x[i]);
-    } else if (na.kind == 1) {
+    float mean = 0.0f, scale = 1.0f;
+    if (na.kind == 1) {
         double s = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = x[i]; s += (double)__fmul_rn(v, v); }
         s = block_sum_f64(s, red);
-        const float mean = (float)(s / cols);
-        const float scale = 1.0f / sqrtf(mean + na.eps);
-        for (int i = threadIdx.x; i < cols; i += blockDim.x) {
-            float v = __fmul_rn(x[i], scale);
-            if (na.w) v = __fmul_rn(v, na.w[i]);
-            if (na.b) v = __fadd_rn(v, na.b[i]);
-            xs[i] = __float2half_rn(v);
-        }
-    } else {
+        scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
+    } else if (na.kind == 2) {
         double s = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) s += (double)x[i];
         s = block_sum_f64(s, red);
-        const float mean = (float)(s / cols);
+        mean = (float)(s / cols);
         double s2 = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = __fsub_rn(x[i], mean); s2 += (double)__fmul_rn(v, v); }
         s2 = block_sum_f64(s2, red);
-        const float var = (float)(s2 / cols);
-        const float scale = 1.0f / sqrtf(var + na.eps);
-        for (int i = threadIdx.x; i < cols; i += blockDim.x) {
-            float v = __fmul_rn(__fsub_rn(x[i], mean), scale);
+        scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
+    }
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+        float v = x[i];
+        if (na.kind != 0) {
+            v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
             if (na.w) v = __fmul_rn(v, na.w[i]);
             if (na.b) v = __fadd_rn(v, na.b[i]);
-            xs[i] = __float2half_rn(v);
         }
+        xs[i] = __float2half_rn(v);
     }
     __syncthreads();
 }
+
+// Fast staging for cols % 256 == 0.  These kernels run a few microseconds, so what they wait for matters more
+// than what they compute: the activation vector and the norm weights are brought in with direct global->LDS
+// loads (no registers, a handful of instructions) issued together with the first weight loads, so that the
+// whole prologue costs one memory round trip; the code is kept small because every launch starts with a
+// cold instruction cache.
+// LDS layout (floats): xraw[cols] | wn[cols] | then xs as fp16[cols].
+__device__ __forceinline__ void stage_fast_issue(float * lds, const float * __restrict__ x, NormArgs na, int cols) {
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const bool has_w = na.kind != 0 && na.w != nullptr;
+    for (int base = wave * 256; base < cols; base += kWavesPerBlock * 256) {
+        __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(x + base + lane * 4),
+                                         (__attribute__((address_space(3))) void *)(lds + base), 16, 0, 0);
+        if (has_w)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(na.w + base + lane * 4),
+                                             (__attribute__((address_space(3))) void *)(lds + cols + base), 16, 0, 0);
+    }
+}
+// call after the loads above have landed (s_waitcnt + barrier); leaves fp16 activations in xs
+__device__ __forceinline__ void stage_fast_finish(__half * xs, const float * lds, NormArgs na, int cols, double * red) {
+    const float * xraw = lds;
+    const float * wn = lds + cols;
+    float mean = 0.0f, scale = 1.0f;
+    if (na.kind == 1) {
+        double s = 0.0;
+        for (int i = threadIdx.x; i < cols; i += kBlock) { const float v = xraw[i]; s += (double)__fmul_rn(v, v); }
+        s = block_sum_f64(s, red);
+        scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
+    } else if (na.kind == 2) {
+        double s = 0.0;
+        for (int i = threadIdx.x; i < cols; i += kBlock) s += (double)xraw[i];
+        s = block_sum_f64(s, red);
+        mean = (float)(s / cols);
+        double s2 = 0.0;
+        for (int i = threadIdx.x; i < cols; i += kBlock) { const float v = __fsub_rn(xraw[i], mean); s2 += (double)__fmul_rn(v, v); }
+        s2 = block_sum_f64(s2, red);
+        scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
+    }
+    for (int i = threadIdx.x; i < cols; i += kBlock) {
+        float v = xraw[i];
+        if (na.kind != 0) {
+            v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
+            if (na.w) v = __fmul_rn(v, wn[i]);
+            if (na.b) v = __fadd_rn(v, na.b[i]);
+        }
+        xs[i] = __float2half_rn(v);
+    }
+    __syncthreads();
+}
+__host__ __device__ inline size_t stage_fast_lds_bytes(int cols) { return (size_t)cols * (4 + 4 + 2); }
 
 // Q8_0 staging for Q4_0 weights: per block of 32, d = amax/127 kept as fp16, q = rint(x * 127/amax)
 // (x86 path of quantize_row_q8_0, ggml-quants.c:702-760).  LDS layout: int8 q[cols] then float d[cols/32].
@@ -134,39 +178,100 @@ __device__ __forceinline__ float apply_epilogue(float v, int epi, const float * 
 }
 
 // ---------------------------------------------------------------------------------------------------
-// Dense F16 mat-vec.  One wave owns RPW consecutive rows; lane l reads 16 B (8 halfs) at column
-// 8*l + 512*i of each row, so a wave issues 1 KiB contiguous per row per load instruction.
+// Dense F16 mat-vec.  A fixed grid of about two workgroups per CU (what a pure streaming read needs to reach
+// HBM speed on this chip), each wave walking row groups g = wave_id, wave_id + n_waves, ...  A group is RPW
+// consecutive rows; lane l reads 16 B (8 halfs) at column 8*l + 512*c of each row (chunk c), i.e. 1 KiB
+// contiguous per row per load instruction.  The (group, chunk) space of a wave is flattened into steps of U
+// chunks with one step of loads always in flight; the first step is issued before the activations are
+// staged (weights do not depend on them).  Fast path: cols % 512 == 0 and rows % RPW == 0 (no guards).
+// TAG only separates instantiations by role so that kernel traces can tell them apart.
 // ---------------------------------------------------------------------------------------------------
-template <int RPW>
+constexpr int kGemvBlocks = 512;
+
+template <int RPW, int U, int TAG>
 __global__ __launch_bounds__(kBlock) void gemv_f16_kernel(const __half * __restrict__ W, const float * __restrict__ x, NormArgs na,
                                                           int epi, const float * add1, const float * add2,
                                                           float * __restrict__ y, int rows, int cols) {
     extern __shared__ __align__(16) unsigned char smem[];
+    float * lds = reinterpret_cast<float *>(smem);
+    __half * xs = reinterpret_cast<__half *>(smem + (size_t)cols * 8);
+    __shared__ double red[16];
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n_waves = gridDim.x * kWavesPerBlock, wid = blockIdx.x * kWavesPerBlock + wave;
+    const int n_groups = rows / RPW;
+    const int spg = cols / (PI_WAVE * 8 * U);                              // steps per group
+    const int my_groups = wid < n_groups ? (n_groups - wid + n_waves - 1) / n_waves : 0;
+    const int T = my_groups * spg;
+
+    stage_fast_issue(lds, x, na, cols);
+
+    pi_u32x4 buf[RPW][U], nxt[RPW][U];
+    const __half * wp = W + (size_t)wid * RPW * cols + lane * 8;           // this wave's position in the (group, step) walk
+    int sig = 0;                                                           // step within the current group
+    auto issue = [&](pi_u32x4 (&dst)[RPW][U]) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int i = 0; i < RPW; ++i) dst[i][u] = pi_ld_stream(wp + (size_t)i * cols + u * (PI_WAVE * 8));
+        wp += U * PI_WAVE * 8;
+        if (++sig == spg) { sig = 0; wp += (size_t)(n_waves * RPW - 1) * cols; }   // next group: (n_waves*RPW) rows down, back to column 0
+    };
+    if (T > 0) issue(buf);
+    // the direct-to-LDS loads were issued first and complete in order: allow only the weight loads to remain in flight
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(RPW * U) : "memory");
+    __syncthreads();
+    stage_fast_finish(xs, lds, na, cols, red);
+
+    float acc[RPW];
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) acc[i] = 0.0f;
+    int row = wid * RPW, c = lane * 8, s_in = 0;
+    for (int t = 0; t < T; ++t) {
+        if (t + 1 < T) issue(nxt);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float xf[8];
+            pi_unpack8(pi_ld16(xs + c + u * (PI_WAVE * 8)), xf);
+#pragma unroll
+            for (int i = 0; i < RPW; ++i) acc[i] = pi_dot8(buf[i][u], xf, acc[i]);
+        }
+        c += U * PI_WAVE * 8;
+        if (++s_in == spg) {
+#pragma unroll
+            for (int i = 0; i < RPW; ++i) {
+                const float sum = pi_wave_sum(acc[i]);
+                if (lane == 0) y[row + i] = apply_epilogue(sum, epi, add1, add2, row + i);
+                acc[i] = 0.0f;
+            }
+            s_in = 0; c = lane * 8; row += n_waves * RPW;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int i = 0; i < RPW; ++i) buf[i][u] = nxt[i][u];
+    }
+}
+
+// any shape with cols % 8 == 0: one wave per row, grid-stride
+__global__ __launch_bounds__(kBlock) void gemv_f16_generic_kernel(const __half * __restrict__ W, const float * __restrict__ x, NormArgs na,
+                                                                  int epi, const float * add1, const float * add2,
+                                                                  float * __restrict__ y, int rows, int cols) {
+    extern __shared__ __align__(16) unsigned char smem[];
     __half * xs = reinterpret_cast<__half *>(smem);
     __shared__ double red[16];
     stage_x_f16(xs, x, cols, na, red);
-
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int n_groups = (rows + RPW - 1) / RPW;
-    for (int g = blockIdx.x * kWavesPerBlock + wave; g < n_groups; g += gridDim.x * kWavesPerBlock) {
-        const int r0 = g * RPW;
-        float acc[RPW];
-#pragma unroll
-        for (int i = 0; i < RPW; ++i) acc[i] = 0.0f;
-#pragma unroll 2
+    for (int r = blockIdx.x * kWavesPerBlock + wave; r < rows; r += gridDim.x * kWavesPerBlock) {
+        float acc = 0.0f;
+#pragma unroll 4
         for (int c = lane * 8; c < cols; c += PI_WAVE * 8) {
             float xf[8];
             pi_unpack8(pi_ld16(xs + c), xf);
-#pragma unroll
-            for (int i = 0; i < RPW; ++i) {
-                if (r0 + i < rows) acc[i] = pi_dot8(pi_ld_stream(W + (size_t)(r0 + i) * cols + c), xf, acc[i]);
-            }
+            acc = pi_dot8(pi_ld_stream(W + (size_t)r * cols + c), xf, acc);
         }
-#pragma unroll
-        for (int i = 0; i < RPW; ++i) {
-            const float s = pi_wave_sum(acc[i]);
-            if (lane == 0 && r0 + i < rows) y[r0 + i] = apply_epilogue(s, epi, add1, add2, r0 + i);
-        }
+        acc = pi_wave_sum(acc);
+        if (lane == 0) y[r] = apply_epilogue(acc, epi, add1, add2, r);
     }
 }
 
@@ -775,19 +880,32 @@ int pi_k_gemv(int wtype, const void * W, int rows, int cols, const float * x, co
         return pi::fail(PI_E_ARG, "pi_k_gemv: bad epilogue arguments");
     hipStream_t st = (hipStream_t)stream;
     const NormArgs na = to_norm(norm);
-    const int rpw = rows >= 16384 ? 8 : rows >= 8192 ? 4 : rows >= 2048 ? 2 : 1;   // rows per wave (8: lm-head sized matrices)
+    // rows per wave group / chunks per step: 8 x 16 B loads in flight per lane per step, and at least one
+    // group for each of the grid's waves
+    const int n_waves = kGemvBlocks * kWavesPerBlock;
+    const int rpw = rows >= 4 * n_waves ? 4 : rows >= 2 * n_waves ? 2 : 1;
     const int n_groups = (rows + rpw - 1) / rpw;
     int blocks = (n_groups + kWavesPerBlock - 1) / kWavesPerBlock;
-    if (blocks > 4096) blocks = 4096;
+    if (blocks > kGemvBlocks) blocks = kGemvBlocks;
     if (wtype == PI_TYPE_F16) {
         if (cols % 8) return pi::fail(PI_E_ARG, "pi_k_gemv: F16 needs cols % 8 == 0");
-        const size_t sh = (size_t)cols * 2;
-        if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv: cols too large for LDS staging");
         const __half * w = (const __half *)W;
-        if (rpw == 8)      hipLaunchKernelGGL(gemv_f16_kernel<8>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
-        else if (rpw == 4) hipLaunchKernelGGL(gemv_f16_kernel<4>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
-        else if (rpw == 2) hipLaunchKernelGGL(gemv_f16_kernel<2>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
-        else               hipLaunchKernelGGL(gemv_f16_kernel<1>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        const int u = 8 / rpw;
+        const bool fast = cols % (PI_WAVE * 8 * u) == 0 && rows % rpw == 0 && stage_fast_lds_bytes(cols) <= 64 * 1024 &&
+                          (((uintptr_t)x | (uintptr_t)(norm ? norm->w : nullptr)) & 15) == 0;
+        if (fast) {
+            const size_t sh = stage_fast_lds_bytes(cols);
+            if (rows >= 16384) hipLaunchKernelGGL((gemv_f16_kernel<4, 2, 1>), dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+            else if (rpw == 4) hipLaunchKernelGGL((gemv_f16_kernel<4, 2, 0>), dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+            else if (rpw == 2) hipLaunchKernelGGL((gemv_f16_kernel<2, 4, 0>), dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+            else               hipLaunchKernelGGL((gemv_f16_kernel<1, 8, 0>), dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        } else {
+            const size_t sh = (size_t)cols * 2;
+            if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv: cols too large for LDS staging");
+            int gb = (rows + kWavesPerBlock - 1) / kWavesPerBlock;
+            if (gb > 2048) gb = 2048;
+            hipLaunchKernelGGL(gemv_f16_generic_kernel, dim3(gb), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        }
     } else if (wtype == PI_TYPE_Q4_0) {
         if (cols % 32) return pi::fail(PI_E_ARG, "pi_k_gemv: Q4_0 needs cols % 32 == 0");
         const size_t sh = (size_t)cols + (size_t)(cols / 32) * 4 + (size_t)cols * 4;

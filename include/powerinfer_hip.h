@@ -82,13 +82,16 @@ PI_API pi_workspace * pi_workspace_create(int max_ff, int max_d);
 PI_API int            pi_workspace_destroy(pi_workspace * ws);
 
 /*
- * Predictor output layer fused with the activity test and compaction:
+ * Predictor output layer fused with the activity test:
  *   logits[ff] = fc2[ff][r] . fp16(hidden[r]);  neuron j active iff !(logits[j] < threshold)
- * (mul_mat "mlp_pre_out", llama.cpp:4693; test ggml-cuda.cu:4695 / ggml.c:14256).  Emits the ascending
- * list of active rows and its length.  With bucket == NULL rows are neuron indices 0..ff-1.  With a
- * gpu_bucket (sorted original indices of the GPU-resident neurons, llama.cpp:2820-2870) the candidates
- * are rows 0..n_bucket-1 of the compact GPU matrices and row i is active iff neuron bucket[i] is.
- * The reference never materialises this list (it re-tests the mask in every kernel).
+ * (mul_mat "mlp_pre_out", llama.cpp:4693; test ggml-cuda.cu:4695 / ggml.c:14256).  Each workgroup of 32
+ * neurons emits one 32-bit activity word by wave ballot; the words stay in the workspace.
+ * If active_rows/n_active are given, the ascending list of active rows and its length are produced as well
+ * (second, single-workgroup launch: popcount prefix sums over the words).  With bucket == NULL rows are neuron
+ * indices 0..ff-1.  With a gpu_bucket (sorted original indices of the GPU-resident neurons,
+ * llama.cpp:2820-2870) the candidates are rows 0..n_bucket-1 of the compact GPU matrices and row i is active
+ * iff neuron bucket[i] is.  With active_rows == NULL the list is left to pi_k_sparse_upgate(from_mask = 1),
+ * which builds it on the fly.  The reference never materialises this list (it re-tests the mask in every kernel).
  * zero_fill (optional): fp32 [ff] cleared by the same launch (the dense h vector of the Q4_0 path).
  */
 PI_API int pi_k_predictor_fc2(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
@@ -105,25 +108,33 @@ PI_API int pi_k_compact_active(const float * logits, int ff, float threshold, co
  *   h[k] = relu(gate[row_k] . x) * (up[row_k] . x)      (gate != NULL, LLM_FFN_PAR)
  *   h[k] = relu(up[row_k] . x)                          (gate == NULL, Falcon)
  * Replaces dequantize_mul_mat_vec_sparse (ggml-cuda.cu:4685) / mul_mat_vec_q(lst, idx) (:5490) plus
- * relu_f32 and mul_f32.  h_compact[k] is indexed like active_rows; if h_dense != NULL the value is also
- * scattered to h_dense[neuron] (neuron = bucket ? bucket[row] : row), which the caller has zeroed.
- * up_dense/gate_dense (optional) receive the raw dot products the same way (GGML_OP_MUL_MAT_SPARSE output).
+ * relu_f32 and mul_f32.
+ * from_mask != 0: the active set is taken from the mask words the last pi_k_predictor_fc2 on this workspace
+ *   left; every workgroup derives rank -> row from a popcount prefix table, and active_rows[k] / *n_active are
+ *   WRITTEN here (ascending list as a by-product).  bucket must be NULL.
+ * from_mask == 0: active_rows / n_active are inputs (produced by pi_k_predictor_fc2 or pi_k_compact_active).
+ * h_compact[k] is indexed like active_rows; if h_dense != NULL the value is also scattered to h_dense[neuron]
+ * (neuron = bucket ? bucket[row] : row), which the caller has zeroed.  up_dense/gate_dense (optional, list
+ * mode only) receive the raw dot products the same way (GGML_OP_MUL_MAT_SPARSE output).
  */
-PI_API int pi_k_sparse_upgate(int wtype, const void * up, const void * gate, int cols, const float * x, const pi_norm * norm,
-                              const int32_t * active_rows, const int32_t * n_active, const int32_t * bucket,
-                              float * h_compact, float * h_dense, float * up_dense, float * gate_dense, pi_stream_t stream);
+PI_API int pi_k_sparse_upgate(int wtype, const void * up, const void * gate, int cols, int ff, const float * x, const pi_norm * norm,
+                              int from_mask, int32_t * active_rows, int32_t * n_active, const int32_t * bucket,
+                              float * h_compact, float * h_dense, float * up_dense, float * gate_dense,
+                              pi_workspace * ws, pi_stream_t stream);
 
 /*
  * Sparse down projection (GGML_OP_AXPY):  out[cols] = epi( sum_k act(h_compact[k]) * down_t[row_k][:] ).
  * Replaces dequantize_mul_mat_axpy_sparse (ggml-cuda.cu:4541) and _sparse_pro (:4479) and their
- * per-row global atomics: column tiles x row groups accumulate in registers, merge through LDS and a
- * fixed-order second stage, so the result is deterministic.  Rows whose rounded h is zero are not read.
+ * per-row global atomics.  F16: a workgroup owns 128 output columns and all active rows, its 16 waves split
+ * the rows and merge through LDS in a fixed order.  Q4_0: column tiles x row groups with a fixed-order second
+ * stage.  Either way the result is deterministic.  Rows whose rounded h is zero are not read.
  * act(): fp16 rounding for F16 weights; for Q4_0 weights h is quantised to Q8_0 over blocks of 32
  * neurons as the CPU path does (ggml.c:14465-14618), which needs the dense neuron-indexed vector
  * h_dense (zeros at inactive neurons; may be NULL for F16) and the bucket that maps rows to neurons.
+ * n_rows: number of candidate rows (capacity of h_compact / active_rows): ff, or the bucket size.
  * epilogue: NONE | ADD | ADD2 as for pi_k_gemv.
  */
-PI_API int pi_k_sparse_axpy(int wtype, const void * down_t, int cols, const float * h_compact,
+PI_API int pi_k_sparse_axpy(int wtype, const void * down_t, int cols, int n_rows, const float * h_compact,
                             const float * h_dense, const int32_t * bucket,
                             const int32_t * active_rows, const int32_t * n_active,
                             int epilogue, const float * add1, const float * add2, float * out,

@@ -137,25 +137,29 @@ int layer_forward(pi_model * m, int il, bool last_token) {
 
     // predictor
     PI_TRY(pi_k_gemv(fc1.type, fc1.dev, r, d, pred_in, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, st));
-    PI_TRY(pi_k_predictor_fc2(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, bk, n_bucket, m->pred_logits, m->list, n_act,
+    // F16 layers that live entirely on the GPU take the fused route: the up/gate kernel reads the mask words itself
+    const bool fused = !layer_hybrid && !q4;
+    const int n_rows = layer_hybrid ? n_bucket : ff;
+    PI_TRY(pi_k_predictor_fc2(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, bk, n_bucket, m->pred_logits,
+                              fused ? nullptr : m->list, fused ? nullptr : n_act,
                               (q4 || layer_hybrid) ? m->h_dense : nullptr, m->ws, st));
 
     // sparse FFN, GPU share
-    PI_TRY(pi_k_sparse_upgate(up.type, up.dev, falcon ? nullptr : gate.dev, d, ffn_in, &fn, m->list, n_act, bk, m->h_c,
-                              (q4 || layer_hybrid) ? m->h_dense : nullptr, nullptr, nullptr, st));
+    PI_TRY(pi_k_sparse_upgate(up.type, up.dev, falcon ? nullptr : gate.dev, d, ff, ffn_in, &fn, fused ? 1 : 0, m->list, n_act, bk, m->h_c,
+                              (q4 || layer_hybrid) ? m->h_dense : nullptr, nullptr, nullptr, m->ws, st));
 
     if (!layer_hybrid && m->capture && last_token) {
         // parity hook: keep the bare FFN output, then add the residuals in the reference's order
         float * ffo = m->cap_ffn + (size_t)il * d;
-        PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, n_act,
+        PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, n_rows, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, n_act,
                                 PI_EPI_NONE, nullptr, nullptr, ffo, m->ws, st));
         PI_HIP_TRY(hipMemcpyAsync(m->x2, ffo, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
         PI_TRY(pi::add_vec(m->x2, falcon ? m->attn_out : m->ffn_inp, d, st));
         if (falcon) PI_TRY(pi::add_vec(m->x2, x, d, st));
     } else if (!layer_hybrid) {
-        if (!falcon) PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, n_act,
+        if (!falcon) PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, n_rows, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, n_act,
                                              PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, m->ws, st));
-        else         PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, n_act,
+        else         PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, n_rows, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, n_act,
                                              PI_EPI_ADD2, m->attn_out, x, m->x2, m->ws, st));
     } else {
         // hot/cold merge (llm_build_sparse_mul_mat / llm_build_sparse_axpy hybrid variants, llama.cpp:4581-4593, 4635-4646)
@@ -459,11 +463,11 @@ int pi_model_time_section(pi_model * m, int section, int rounds, float * ms_tota
                 pi_norm fn = falcon ? make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B))
                                     : make_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
                 PI_TRY(pi_k_gemv(fc1.type, fc1.dev, (int)fc1.ne1, d, m->ffn_inp, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, st));
-                PI_TRY(pi_k_predictor_fc2(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, nullptr, 0, m->pred_logits, m->list, m->n_active + il,
-                                          q4 ? m->h_dense : nullptr, m->ws, st));
-                PI_TRY(pi_k_sparse_upgate(up.type, up.dev, falcon ? nullptr : gate.dev, d, m->ffn_inp, &fn, m->list, m->n_active + il, nullptr, m->h_c,
-                                          q4 ? m->h_dense : nullptr, nullptr, nullptr, st));
-                PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, m->n_active + il,
+                PI_TRY(pi_k_predictor_fc2(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, nullptr, 0, m->pred_logits,
+                                          q4 ? m->list : nullptr, q4 ? m->n_active + il : nullptr, q4 ? m->h_dense : nullptr, m->ws, st));
+                PI_TRY(pi_k_sparse_upgate(up.type, up.dev, falcon ? nullptr : gate.dev, d, ff, m->ffn_inp, &fn, q4 ? 0 : 1, m->list, m->n_active + il, nullptr, m->h_c,
+                                          q4 ? m->h_dense : nullptr, nullptr, nullptr, m->ws, st));
+                PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, ff, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, m->n_active + il,
                                         PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, m->ws, st));
                 ++n;
             } else {

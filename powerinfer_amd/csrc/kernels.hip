@@ -81,7 +81,8 @@ __device__ void stage_x_f16(__half * xs, const float * __restrict__ x, int cols,
 __device__ __forceinline__ void stage_fast_issue(float * lds, const float * __restrict__ x, NormArgs na, int cols) {
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const bool has_w = na.kind != 0 && na.w != nullptr;
-    for (int base = wave * 256; base < cols; base += kWavesPerBlock * 256) {
+    const int nw = blockDim.x >> 6;
+    for (int base = wave * 256; base < cols; base += nw * 256) {
         __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(x + base + lane * 4),
                                          (__attribute__((address_space(3))) void *)(lds + base), 16, 0, 0);
         if (has_w)
@@ -96,20 +97,20 @@ __device__ __forceinline__ void stage_fast_finish(__half * xs, const float * lds
     float mean = 0.0f, scale = 1.0f;
     if (na.kind == 1) {
         double s = 0.0;
-        for (int i = threadIdx.x; i < cols; i += kBlock) { const float v = xraw[i]; s += (double)__fmul_rn(v, v); }
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = xraw[i]; s += (double)__fmul_rn(v, v); }
         s = block_sum_f64(s, red);
         scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
     } else if (na.kind == 2) {
         double s = 0.0;
-        for (int i = threadIdx.x; i < cols; i += kBlock) s += (double)xraw[i];
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) s += (double)xraw[i];
         s = block_sum_f64(s, red);
         mean = (float)(s / cols);
         double s2 = 0.0;
-        for (int i = threadIdx.x; i < cols; i += kBlock) { const float v = __fsub_rn(xraw[i], mean); s2 += (double)__fmul_rn(v, v); }
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = __fsub_rn(xraw[i], mean); s2 += (double)__fmul_rn(v, v); }
         s2 = block_sum_f64(s2, red);
         scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
     }
-    for (int i = threadIdx.x; i < cols; i += kBlock) {
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
         float v = xraw[i];
         if (na.kind != 0) {
             v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
@@ -408,32 +409,59 @@ __device__ bool last_block_done(unsigned int * counter, unsigned int n_blocks, i
     return last;
 }
 
+// Block = 32 consecutive neurons (8 per wave); all weight loads of the block are issued before the hidden
+// vector is staged.  Emits the logits and one 32-bit activity word per block (wave ballot).  NCH = number of
+// 512-column chunks (r <= 512 * NCH); NCH == 0 is the guard-everything variant for other ranks.
+template <int NCH>
 __global__ __launch_bounds__(kBlock) void pred_fc2_kernel(const __half * __restrict__ W, const float * __restrict__ hidden, int ff, int r,
-                                                          float thr, const int32_t * bucket, int n_bucket, float * __restrict__ logits,
-                                                          uint32_t * words, unsigned int * counter,
-                                                          int32_t * list, int32_t * n_active, float * zero_fill) {
+                                                          float thr, float * __restrict__ logits, uint32_t * __restrict__ words,
+                                                          float * zero_fill) {
     extern __shared__ __align__(16) unsigned char smem[];
-    __half * xs = reinterpret_cast<__half *>(smem);
+    float  * xraw = reinterpret_cast<float *>(smem);
+    __half * xs   = reinterpret_cast<__half *>(smem + (size_t)r * 4);
     __shared__ float lg[32];
-    if (zero_fill && threadIdx.x < 32 && (int)(blockIdx.x * 32 + threadIdx.x) < ff) zero_fill[blockIdx.x * 32 + threadIdx.x] = 0.0f;
-    __shared__ int sred[kWavesPerBlock + 1];
-    for (int i = threadIdx.x; i < r; i += blockDim.x) xs[i] = __float2half_rn(hidden[i]);
-    __syncthreads();
-
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int row0 = blockIdx.x * 32 + wave * 8;
+    if (zero_fill && threadIdx.x < 32 && (int)(blockIdx.x * 32 + threadIdx.x) < ff) zero_fill[blockIdx.x * 32 + threadIdx.x] = 0.0f;
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
-    for (int c = lane * 8; c < r; c += PI_WAVE * 8) {
-        float xf[8];
-        pi_unpack8(pi_ld16(xs + c), xf);
+
+    if constexpr (NCH > 0) {
+        for (int base = wave * 256; base < r; base += kWavesPerBlock * 256)
+            __builtin_amdgcn_global_load_lds((const __attribute__((address_space(1))) void *)(hidden + base + lane * 4),
+                                             (__attribute__((address_space(3))) void *)(xraw + base), 16, 0, 0);
+        pi_u32x4 buf[8][NCH];
+        const pi_u32x4 zero = {0u, 0u, 0u, 0u};
 #pragma unroll
-        for (int i = 0; i < 8; ++i)
-            if (row0 + i < ff) acc[i] = pi_dot8(pi_ld_stream(W + (size_t)(row0 + i) * r + c), xf, acc[i]);
+        for (int u = 0; u < NCH; ++u)
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                buf[i][u] = (row0 + i < ff) ? pi_ld_stream(W + (size_t)(row0 + i) * r + (u * PI_WAVE + lane) * 8) : zero;
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"(8 * NCH) : "memory");
+        __syncthreads();
+        for (int i = threadIdx.x; i < r; i += kBlock) xs[i] = __float2half_rn(xraw[i]);
+        __syncthreads();
+#pragma unroll
+        for (int u = 0; u < NCH; ++u) {
+            float xf[8];
+            pi_unpack8(pi_ld16(xs + (u * PI_WAVE + lane) * 8), xf);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) acc[i] = pi_dot8(buf[i][u], xf, acc[i]);
+        }
+    } else {
+        for (int i = threadIdx.x; i < r; i += kBlock) xs[i] = __float2half_rn(hidden[i]);
+        __syncthreads();
+        for (int c = lane * 8; c < r; c += PI_WAVE * 8) {
+            float xf[8];
+            pi_unpack8(pi_ld16(xs + c), xf);
+#pragma unroll
+            for (int i = 0; i < 8; ++i)
+                if (row0 + i < ff) acc[i] = pi_dot8(pi_ld_stream(W + (size_t)(row0 + i) * r + c), xf, acc[i]);
+        }
     }
 #pragma unroll
-    for (int i = 0; i < 8; ++i) { const float s = pi_wave_sum(acc[i]); if (lane == 0) lg[wave * 8 + i] = s; }
+    for (int i = 0; i < 8; ++i) { const float sum = pi_wave_sum(acc[i]); if (lane == 0) lg[wave * 8 + i] = sum; }
     __syncthreads();
     if (wave == 0) {
         const int row = blockIdx.x * 32 + lane;
@@ -442,8 +470,13 @@ __global__ __launch_bounds__(kBlock) void pred_fc2_kernel(const __half * __restr
         const unsigned long long m = __ballot(act);
         if (lane == 0) words[blockIdx.x] = (uint32_t)m;
     }
-    if (last_block_done(counter, gridDim.x, &sred[kWavesPerBlock]))
-        compact_from_words(words, ff, bucket, n_bucket, list, n_active, sred);
+}
+
+// compaction of existing mask words into the ascending active-row list (single block)
+__global__ __launch_bounds__(1024) void compact_words_kernel(const uint32_t * __restrict__ words, int ff, const int32_t * bucket, int n_bucket,
+                                                             int32_t * list, int32_t * n_active) {
+    __shared__ int sred[17];
+    compact_from_words(words, ff, bucket, n_bucket, list, n_active, sred);
 }
 
 // activity test + compaction over existing logits (single block)
@@ -460,6 +493,91 @@ __global__ __launch_bounds__(1024) void compact_kernel(const float * __restrict_
     }
     __syncthreads();
     compact_from_words(words, ff, bucket, n_bucket, list, n_active, sred);
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Sparse up/gate straight from the predictor's mask words (F16).  Every workgroup turns the mask into a
+// popcount prefix table in LDS (wave ballot happened in the predictor kernel, the prefix sum happens here),
+// so rank k -> neuron row is a binary search + bit select and no separate compaction pass or list read sits
+// on the critical path.  Wave w of the grid takes ranks w, w + n_waves, ...: it reads the gate row and the up
+// row (2 x cols fp16, 128-bit loads, all issued before the first use), h = relu(g) * u (or relu(u) without a
+// gate), and writes h_compact[k] and active_rows[k] = row, so the ascending index list is a by-product.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kUpBlock = 512;       // 8 waves
+constexpr int kUpBlocks = 256;      // about one workgroup per CU: 2048 waves >= the active count of the 7B..40B shapes
+
+__device__ __forceinline__ int select_nth_bit(uint32_t bits, int n) {      // index of the n-th (0-based) set bit
+    for (int i = 0; i < n; ++i) bits &= bits - 1;
+    return __ffs(bits) - 1;
+}
+
+template <int NCH>      // cols == 512 * NCH
+__global__ __launch_bounds__(kUpBlock) void sparse_upgate_mask_f16_kernel(const __half * __restrict__ Wup, const __half * __restrict__ Wgate,
+                                                                          const float * __restrict__ x, NormArgs na, int cols, int ff,
+                                                                          const uint32_t * __restrict__ words,
+                                                                          int32_t * __restrict__ list, int32_t * __restrict__ n_active,
+                                                                          float * __restrict__ h_compact, float * h_dense) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float  * lds = reinterpret_cast<float *>(smem);                       // xraw[cols] | wn[cols]
+    __half * xs  = reinterpret_cast<__half *>(smem + (size_t)cols * 8);
+    int    * prefix = reinterpret_cast<int *>(smem + (size_t)cols * 10);  // [nwords + 1]
+    uint32_t * wbits = reinterpret_cast<uint32_t *>(prefix + (ff + 31) / 32 + 1);
+    __shared__ double red[16];
+    __shared__ int sred[kUpBlock / PI_WAVE + 1];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nwords = (ff + 31) / 32;
+    constexpr int kWaves = kUpBlock / PI_WAVE;
+
+    // one memory round trip: activations (+ norm weights) by direct-to-LDS loads, mask words by ordinary loads
+    stage_fast_issue(lds, x, na, cols);
+    int base_cnt = 0;
+    for (int w0 = 0; w0 < nwords; w0 += kUpBlock) {
+        const int w = w0 + threadIdx.x;
+        const uint32_t bits = w < nwords ? words[w] : 0u;
+        int tot;
+        const int off = base_cnt + block_exclusive_scan_i32(__popc(bits), &tot, sred);
+        if (w < nwords) { prefix[w] = off; wbits[w] = bits; }
+        base_cnt += tot;
+    }
+    const int n = base_cnt;
+    if (threadIdx.x == 0) { prefix[nwords] = n; if (blockIdx.x == 0) *n_active = n; }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if ((int)(blockIdx.x * kWaves) >= n) return;                           // no rank for this workgroup (uniform)
+
+    stage_fast_finish(xs, lds, na, cols, red);
+
+    for (int k = blockIdx.x * kWaves + wave; k < n; k += gridDim.x * kWaves) {
+        // word holding rank k: largest w with prefix[w] <= k
+        int lo = 0, hi = nwords - 1;
+        while (lo < hi) { const int mid = (lo + hi + 1) >> 1; if (prefix[mid] <= k) lo = mid; else hi = mid - 1; }
+        const int row = lo * 32 + select_nth_bit(wbits[lo], k - prefix[lo]);
+        const __half * wu = Wup + (size_t)row * cols + lane * 8;
+        pi_u32x4 bu[NCH], bg[NCH];
+#pragma unroll
+        for (int u = 0; u < NCH; ++u) bu[u] = pi_ld_stream(wu + u * (PI_WAVE * 8));
+        if (Wgate) {
+            const __half * wg = Wgate + (size_t)row * cols + lane * 8;
+#pragma unroll
+            for (int u = 0; u < NCH; ++u) bg[u] = pi_ld_stream(wg + u * (PI_WAVE * 8));
+        }
+        float au = 0.0f, ag = 0.0f;
+#pragma unroll
+        for (int u = 0; u < NCH; ++u) {
+            float xf[8];
+            pi_unpack8(pi_ld16(xs + (u * PI_WAVE + lane) * 8), xf);
+            au = pi_dot8(bu[u], xf, au);
+            if (Wgate) ag = pi_dot8(bg[u], xf, ag);
+        }
+        au = pi_wave_sum(au);
+        if (Wgate) ag = pi_wave_sum(ag);
+        if (lane == 0) {
+            const float h = Wgate ? __fmul_rn(fmaxf(ag, 0.0f), au) : fmaxf(au, 0.0f);
+            h_compact[k] = h;
+            list[k] = row;
+            if (h_dense) h_dense[row] = h;
+        }
+    }
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -551,6 +669,79 @@ __global__ __launch_bounds__(kBlock) void sparse_upgate_q4_kernel(const pi_block
 // so the sum order -- and the result -- is fixed.  h is rounded to fp16 first and zero rows are skipped
 // as on the CPU path (ggml.c:14420-14431).
 // ---------------------------------------------------------------------------------------------------
+// F16 down projection with the whole reduction inside the workgroup: a workgroup owns 128 output columns
+// (lane = 2 columns, one 32-bit load per row) and all active rows; its 16 waves split the rows, accumulate in
+// registers and merge through LDS in wave order, so there is no inter-workgroup reduction, no atomics and no
+// fence, and the sum order is fixed.  Entries whose fp16-rounded h is zero are dropped by a workgroup-level
+// ballot/prefix compaction before any weight is read.
+constexpr int kAxBlock = 1024;
+constexpr int kAxWaves = kAxBlock / PI_WAVE;
+constexpr int kAxCap = 2048;        // compacted entries held in LDS per round
+constexpr int kAxUn = 16;           // rows in flight per wave
+
+__global__ __launch_bounds__(kAxBlock) void sparse_axpy_lds_f16_kernel(const __half * __restrict__ Wd, int cols, int n_max,
+                                                                       const float * __restrict__ h_compact, const int32_t * __restrict__ list,
+                                                                       const int32_t * __restrict__ n_active,
+                                                                       int epi, const float * add1, const float * add2, float * __restrict__ out) {
+    __shared__ int   crow[kAxCap];
+    __shared__ float ca[kAxCap];
+    __shared__ float redl[kAxWaves][128];
+    __shared__ int   sred[kAxWaves + 1];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int col = blockIdx.x * 128 + lane * 2;
+    // the first kAxBlock entries are fetched before the count is known (same round trip); stale slots are masked below
+    float a_spec = tid < n_max ? h_compact[tid] : 0.0f;
+    int   r_spec = tid < n_max ? list[tid] : 0;
+    const int n = *n_active;
+    float acc0 = 0.0f, acc1 = 0.0f;
+    int k0 = 0;
+    while (k0 < n) {
+        // ---- compact up to kAxCap non-zero entries starting at k0 -----------------------------------
+        int m = 0;
+        while (k0 < n && m + kAxBlock <= kAxCap) {
+            const int k = k0 + tid;
+            float a; int r;
+            if (k0 == 0) { a = a_spec; r = r_spec; } else { a = k < n ? h_compact[k] : 0.0f; r = k < n ? list[k] : 0; }
+            a = pi_round_f16(a);
+            const int nz = (k < n && a != 0.0f) ? 1 : 0;
+            int tot;
+            const int off = m + block_exclusive_scan_i32(nz, &tot, sred);
+            if (nz) { crow[off] = r; ca[off] = a; }
+            m += tot;
+            k0 += kAxBlock;
+        }
+        __syncthreads();
+        // ---- rows wave, wave + 16, ... of the compacted list ---------------------------------------
+        for (int i0 = wave; i0 < m; i0 += kAxWaves * kAxUn) {
+            uint32_t w[kAxUn]; float a[kAxUn];
+#pragma unroll
+            for (int u = 0; u < kAxUn; ++u) {
+                const int i = i0 + u * kAxWaves;
+                const bool ok = i < m;
+                a[u] = ok ? ca[i] : 0.0f;
+                w[u] = ok ? __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(Wd + (size_t)crow[i] * cols + col)) : 0u;
+            }
+#pragma unroll
+            for (int u = 0; u < kAxUn; ++u) {
+                const float2 f = __half22float2(*reinterpret_cast<const __half2 *>(&w[u]));
+                acc0 = fmaf(f.x, a[u], acc0);
+                acc1 = fmaf(f.y, a[u], acc1);
+            }
+        }
+        __syncthreads();
+    }
+    redl[wave][lane * 2] = acc0;
+    redl[wave][lane * 2 + 1] = acc1;
+    __syncthreads();
+    if (tid < 128) {
+        float sum = redl[0][tid];
+#pragma unroll
+        for (int w = 1; w < kAxWaves; ++w) sum += redl[w][tid];
+        const int c = blockIdx.x * 128 + tid;
+        out[c] = apply_epilogue(sum, epi, add1, add2, c);
+    }
+}
+
 constexpr int kAxpyTile = PI_WAVE * 8;
 
 __device__ void axpy_finish(float * acc, float * lds, float * partial, unsigned int * tile_counter, int cols,
@@ -924,12 +1115,21 @@ int pi_k_gemv(int wtype, const void * W, int rows, int cols, const float * x, co
 int pi_k_predictor_fc2(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
                        const int32_t * bucket, int n_bucket, float * logits,
                        int32_t * active_rows, int32_t * n_active, float * zero_fill, pi_workspace * ws, pi_stream_t stream) {
-    if (!fc2_f16 || !hidden || !logits || !active_rows || !n_active || !ws) return pi::fail(PI_E_ARG, "pi_k_predictor_fc2: null pointer");
+    if (!fc2_f16 || !hidden || !logits || !ws) return pi::fail(PI_E_ARG, "pi_k_predictor_fc2: null pointer");
+    if ((active_rows == nullptr) != (n_active == nullptr)) return pi::fail(PI_E_ARG, "pi_k_predictor_fc2: active_rows and n_active go together");
     if (ff <= 0 || r <= 0 || r % 8 || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_predictor_fc2: bad shape (r % 8 == 0, ff <= workspace)");
     if (bucket && (n_bucket < 0 || n_bucket > ff)) return pi::fail(PI_E_ARG, "pi_k_predictor_fc2: bad bucket size");
+    if (bucket && !active_rows) return pi::fail(PI_E_ARG, "pi_k_predictor_fc2: a bucket needs the explicit row list");
     const int blocks = (ff + 31) / 32;
-    hipLaunchKernelGGL(pred_fc2_kernel, dim3(blocks), dim3(kBlock), (size_t)r * 2, (hipStream_t)stream,
-                       (const __half *)fc2_f16, hidden, ff, r, threshold, bucket, n_bucket, logits, ws->words, ws->counters, active_rows, n_active, zero_fill);
+    hipStream_t st = (hipStream_t)stream;
+    const __half * w = (const __half *)fc2_f16;
+    const size_t sh = (size_t)r * 6;
+    const bool aligned = (((uintptr_t)hidden) & 15) == 0;
+    if (r == 1024 && aligned)     hipLaunchKernelGGL(pred_fc2_kernel<2>, dim3(blocks), dim3(kBlock), sh, st, w, hidden, ff, r, threshold, logits, ws->words, zero_fill);
+    else if (r == 512 && aligned) hipLaunchKernelGGL(pred_fc2_kernel<1>, dim3(blocks), dim3(kBlock), sh, st, w, hidden, ff, r, threshold, logits, ws->words, zero_fill);
+    else                          hipLaunchKernelGGL(pred_fc2_kernel<0>, dim3(blocks), dim3(kBlock), sh, st, w, hidden, ff, r, threshold, logits, ws->words, zero_fill);
+    if (active_rows)
+        hipLaunchKernelGGL(compact_words_kernel, dim3(1), dim3(1024), 0, st, ws->words, ff, bucket, n_bucket, active_rows, n_active);
     return pi::check_launch("pi_k_predictor_fc2");
 }
 
@@ -941,33 +1141,55 @@ int pi_k_compact_active(const float * logits, int ff, float threshold, const int
     return pi::check_launch("pi_k_compact_active");
 }
 
-int pi_k_sparse_upgate(int wtype, const void * up, const void * gate, int cols, const float * x, const pi_norm * norm,
-                       const int32_t * active_rows, const int32_t * n_active, const int32_t * bucket,
-                       float * h_compact, float * h_dense, float * up_dense, float * gate_dense, pi_stream_t stream) {
+int pi_k_sparse_upgate(int wtype, const void * up, const void * gate, int cols, int ff, const float * x, const pi_norm * norm,
+                       int from_mask, int32_t * active_rows, int32_t * n_active, const int32_t * bucket,
+                       float * h_compact, float * h_dense, float * up_dense, float * gate_dense, pi_workspace * ws, pi_stream_t stream) {
     if (!up || !x || !active_rows || !n_active || !h_compact || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_sparse_upgate: null pointer or empty shape");
     const NormArgs na = to_norm(norm);
-    const int blocks = 1024;       // fixed grid: the active count lives on the device; idle blocks exit at once
-    if (wtype == PI_TYPE_F16) {
-        if (cols % 8 || (size_t)cols * 2 > 60 * 1024) return pi::fail(PI_E_ARG, "pi_k_sparse_upgate: bad cols for F16");
-        hipLaunchKernelGGL(sparse_upgate_f16_kernel, dim3(blocks), dim3(kBlock), (size_t)cols * 2, (hipStream_t)stream,
-                           (const __half *)up, (const __half *)gate, x, na, cols, active_rows, n_active, bucket, h_compact, h_dense, up_dense, gate_dense);
-    } else if (wtype == PI_TYPE_Q4_0) {
-        const size_t sh = (size_t)cols + (size_t)(cols / 32) * 4 + (size_t)cols * 4;
-        if (cols % 32 || sh > 60 * 1024) return pi::fail(PI_E_ARG, "pi_k_sparse_upgate: bad cols for Q4_0");
-        hipLaunchKernelGGL(sparse_upgate_q4_kernel, dim3(blocks), dim3(kBlock), sh, (hipStream_t)stream,
-                           (const pi_block_q4_0 *)up, (const pi_block_q4_0 *)gate, x, na, cols, active_rows, n_active, bucket, h_compact, h_dense, up_dense, gate_dense);
-    } else {
-        return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_upgate: weight type must be F16 or Q4_0");
+    hipStream_t st = (hipStream_t)stream;
+    if (from_mask) {
+        if (!ws || ff <= 0 || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_sparse_upgate: the mask lives in the workspace (ff <= workspace)");
+        if (bucket) return pi::fail(PI_E_ARG, "pi_k_sparse_upgate: a bucket needs the explicit row list (from_mask = 0)");
+        const size_t sh = (size_t)cols * 10 + (size_t)((ff + 31) / 32) * 8 + 16;
+        const bool aligned = ((((uintptr_t)x) | (uintptr_t)na.w) & 15) == 0;
+        const bool fast = wtype == PI_TYPE_F16 && cols % 512 == 0 && cols / 512 <= 8 && sh <= 64 * 1024 && aligned && !up_dense && !gate_dense;
+        if (fast) {
+            const __half * u = (const __half *)up; const __half * g = (const __half *)gate;
+            const int nch = cols / 512;
+#define PI_UP_CASE(N) case N: hipLaunchKernelGGL(sparse_upgate_mask_f16_kernel<N>, dim3(kUpBlocks), dim3(kUpBlock), sh, st, u, g, x, na, cols, ff, ws->words, active_rows, n_active, h_compact, h_dense); break;
+            switch (nch) { PI_UP_CASE(1) PI_UP_CASE(2) PI_UP_CASE(4) PI_UP_CASE(8)
+                default: hipLaunchKernelGGL(compact_words_kernel, dim3(1), dim3(1024), 0, st, ws->words, ff, nullptr, 0, active_rows, n_active); goto list_mode; }
+#undef PI_UP_CASE
+            return pi::check_launch("pi_k_sparse_upgate");
+        }
+        // shapes the fused kernel does not cover: materialise the list first
+        hipLaunchKernelGGL(compact_words_kernel, dim3(1), dim3(1024), 0, st, ws->words, ff, nullptr, 0, active_rows, n_active);
+    }
+list_mode:
+    {
+        const int blocks = 1024;       // fixed grid: the active count lives on the device; idle blocks exit at once
+        if (wtype == PI_TYPE_F16) {
+            if (cols % 8 || (size_t)cols * 2 > 60 * 1024) return pi::fail(PI_E_ARG, "pi_k_sparse_upgate: bad cols for F16");
+            hipLaunchKernelGGL(sparse_upgate_f16_kernel, dim3(blocks), dim3(kBlock), (size_t)cols * 2, st,
+                               (const __half *)up, (const __half *)gate, x, na, cols, active_rows, n_active, bucket, h_compact, h_dense, up_dense, gate_dense);
+        } else if (wtype == PI_TYPE_Q4_0) {
+            const size_t sh = (size_t)cols + (size_t)(cols / 32) * 4 + (size_t)cols * 4;
+            if (cols % 32 || sh > 60 * 1024) return pi::fail(PI_E_ARG, "pi_k_sparse_upgate: bad cols for Q4_0");
+            hipLaunchKernelGGL(sparse_upgate_q4_kernel, dim3(blocks), dim3(kBlock), sh, st,
+                               (const pi_block_q4_0 *)up, (const pi_block_q4_0 *)gate, x, na, cols, active_rows, n_active, bucket, h_compact, h_dense, up_dense, gate_dense);
+        } else {
+            return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_upgate: weight type must be F16 or Q4_0");
+        }
     }
     return pi::check_launch("pi_k_sparse_upgate");
 }
 
-int pi_k_sparse_axpy(int wtype, const void * down_t, int cols, const float * h_compact, const float * h_dense, const int32_t * bucket,
+int pi_k_sparse_axpy(int wtype, const void * down_t, int cols, int n_rows, const float * h_compact, const float * h_dense, const int32_t * bucket,
                      const int32_t * active_rows, const int32_t * n_active,
                      int epilogue, const float * add1, const float * add2, float * out,
                      pi_workspace * ws, pi_stream_t stream) {
     if (!down_t || !h_compact || !active_rows || !n_active || !out || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: null pointer");
-    if (cols <= 0 || cols > ws->max_d) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: cols exceeds the workspace");
+    if (cols <= 0 || cols > ws->max_d || n_rows <= 0) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: cols exceeds the workspace or n_rows <= 0");
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
         return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: bad epilogue arguments");
     const int tiles = (cols + kAxpyTile - 1) / kAxpyTile;
@@ -975,8 +1197,12 @@ int pi_k_sparse_axpy(int wtype, const void * down_t, int cols, const float * h_c
     hipStream_t st = (hipStream_t)stream;
     if (wtype == PI_TYPE_F16) {
         if (cols % 8) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: F16 needs cols % 8 == 0");
-        hipLaunchKernelGGL(sparse_axpy_f16_kernel, grid, dim3(kBlock), 0, st,
-                           (const __half *)down_t, cols, h_compact, active_rows, n_active, ws->partial, ws->counters + 1, epilogue, add1, add2, out);
+        if (cols % 128 == 0)
+            hipLaunchKernelGGL(sparse_axpy_lds_f16_kernel, dim3(cols / 128), dim3(kAxBlock), 0, st,
+                               (const __half *)down_t, cols, n_rows, h_compact, active_rows, n_active, epilogue, add1, add2, out);
+        else
+            hipLaunchKernelGGL(sparse_axpy_f16_kernel, grid, dim3(kBlock), 0, st,
+                               (const __half *)down_t, cols, h_compact, active_rows, n_active, ws->partial, ws->counters + 1, epilogue, add1, add2, out);
     } else if (wtype == PI_TYPE_Q4_0) {
         if (cols % 32) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: Q4_0 needs cols % 32 == 0");
         if (!h_dense) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy: Q4_0 needs the dense h vector (block scales span 32 neurons)");

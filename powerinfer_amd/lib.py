@@ -50,8 +50,8 @@ _SIGS = {
     "pi_workspace_destroy": (_i, [_vp]),
     "pi_k_predictor_fc2": (_i, [_vp, _i, _i, _vp, _f, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_compact_active": (_i, [_vp, _i, _f, _vp, _i, _vp, _vp, _vp, _vp]),
-    "pi_k_sparse_upgate": (_i, [_i, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
-    "pi_k_sparse_axpy": (_i, [_i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_sparse_upgate": (_i, [_i, _vp, _vp, _i, _i, _vp, C.POINTER(Norm), _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_sparse_axpy": (_i, [_i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_rope_kv_store": (_i, [_vp, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp, _vp]),
     "pi_k_attn_decode": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "pi_k_embed": (_i, [_i, _vp, _i, _vp, _vp, _vp]),

@@ -46,30 +46,36 @@ class SparseFFN:
         self.resid = DevBuf.zeros(d * f4)
 
     def launch(self, stream=None, dense_outputs=True, epilogue=pl.EPI_NONE):
+        """dense_outputs: also scatter up/gate/h into neuron-indexed vectors (what GGML_OP_MUL_MAT_SPARSE returns);
+        this takes the explicit-list route.  Without it (and without a bucket) the fused route runs: the up/gate
+        kernel derives the active rows from the predictor's mask words itself."""
         L, p = self.L, (lambda b: b.ptr if b is not None else None)
+        fused = not dense_outputs and self.bucket is None
+        need_h_dense = dense_outputs or self.wtype == pl.Q4_0
+        n_rows = self.n_bucket if self.bucket is not None else self.ff
         check(L.pi_k_gemv(pl.F16, self.fc1.ptr, self.r, self.d, self.xp.ptr, None, pl.EPI_RELU, None, None, self.hidden.ptr, stream), "fc1")
         check(L.pi_k_predictor_fc2(self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, p(self.bucket), self.n_bucket,
-                                   self.logits.ptr, self.list.ptr, self.n_active.ptr,
-                                   self.h_dense.ptr if (dense_outputs or self.wtype == pl.Q4_0) else None, self.ws, stream), "fc2")
+                                   self.logits.ptr, None if fused else self.list.ptr, None if fused else self.n_active.ptr,
+                                   self.h_dense.ptr if need_h_dense else None, self.ws, stream), "fc2")
         nrm = pl.norm_arg(self.norm_kind, self.eps, self.norm_w, self.norm_b)
-        check(L.pi_k_sparse_upgate(self.wtype, self.up.ptr, p(self.gate), self.d, self.x.ptr, nrm, self.list.ptr, self.n_active.ptr,
-                                   p(self.bucket), self.h_c.ptr,
-                                   self.h_dense.ptr if (dense_outputs or self.wtype == pl.Q4_0) else None,
+        check(L.pi_k_sparse_upgate(self.wtype, self.up.ptr, p(self.gate), self.d, self.ff, self.x.ptr, nrm, int(fused),
+                                   self.list.ptr, self.n_active.ptr, p(self.bucket), self.h_c.ptr,
+                                   self.h_dense.ptr if need_h_dense else None,
                                    self.up_dense.ptr if dense_outputs else None,
-                                   self.gate_dense.ptr if dense_outputs else None, stream), "upgate")
-        check(L.pi_k_sparse_axpy(self.wtype, self.down.ptr, self.d, self.h_c.ptr,
+                                   self.gate_dense.ptr if dense_outputs else None, self.ws, stream), "upgate")
+        check(L.pi_k_sparse_axpy(self.wtype, self.down.ptr, self.d, n_rows, self.h_c.ptr,
                                  self.h_dense.ptr if self.wtype == pl.Q4_0 else None, p(self.bucket),
                                  self.list.ptr, self.n_active.ptr, epilogue, self.resid.ptr if epilogue else None, None,
                                  self.out.ptr, self.ws, stream), "axpy")
 
-    def forward(self, x_ffn, x_pred):
+    def forward(self, x_ffn, x_pred, dense_outputs=True):
         """One token.  Returns dict(logits, active, up, gate, h, out) as numpy arrays (dense vectors are
-        neuron-indexed; rows outside the GPU bucket stay zero)."""
+        neuron-indexed; rows outside the GPU bucket stay zero; up/gate/h only with dense_outputs)."""
         self.x.upload(np.asarray(x_ffn, np.float32))
         self.xp.upload(np.asarray(x_pred, np.float32))
-        for b in (self.up_dense, self.gate_dense):
+        for b in (self.up_dense, self.gate_dense, self.h_dense):
             check(self.L.pi_memset(b.ptr, 0, b.nbytes), "memset")
-        self.launch()
+        self.launch(dense_outputs=dense_outputs)
         pl.sync()
         n = int(self.n_active.download(np.int32)[0])
         return dict(logits=self.logits.download(np.float32), active=self.list.download(np.int32, n),

@@ -77,6 +77,11 @@ def test_ffn_7b_shape_vs_oracle(wtype, has_gate):
             assert rel_err(res["h"], ot["h"]) < 1e-4
             assert rel_err(res["out"], ot["out"]) < FFN_REL_TOL
             assert rel_err(res["out"], ot["out"]) < 1e-4      # in practice: fp32 summation order only
+        # fused route (what the decode loop runs): the up/gate kernel builds the list from the mask words itself
+        fus = ffn.forward(L["x"][t], L["x"][t], dense_outputs=False)
+        assert np.array_equal(fus["active"], res["active"])
+        assert np.array_equal(fus["h_compact"], res["h_compact"])
+        assert rel_err(fus["out"], res["out"]) < 1e-5
     ffn.close()
 
 
@@ -129,10 +134,10 @@ def test_axpy_is_deterministic_and_linear():
     d, ff, r = 4096, 11008, 1024
     L = synth.make_ffn_layer(seed=51, d=d, ff=ff, r=r)
     a = SparseFFN(d, ff, r, ol.F16, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"])
-    r1 = a.forward(L["x"][0], L["x"][0])
-    r2 = a.forward(L["x"][0], L["x"][0])
+    r1 = a.forward(L["x"][0], L["x"][0], dense_outputs=False)
+    r2 = a.forward(L["x"][0], L["x"][0], dense_outputs=False)
     assert np.array_equal(r1["out"], r2["out"]) and np.array_equal(r1["active"], r2["active"])
     b = SparseFFN(d, ff, r, ol.F16, L["up"], L["gate"], (L["down_t"].astype(np.float32) * 2).astype(np.float16), L["fc1"], L["fc2"])
-    r3 = b.forward(L["x"][0], L["x"][0])
+    r3 = b.forward(L["x"][0], L["x"][0], dense_outputs=False)
     assert np.array_equal(r3["out"], 2 * r1["out"])
     a.close(), b.close()

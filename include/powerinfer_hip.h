@@ -158,6 +158,15 @@ PI_API int pi_k_rope_kv_store(const float * qkv, int n_head, int n_head_kv, int 
 PI_API int pi_k_attn_decode(const float * q_rot, const void * k_cache, const void * v_cache, int n_head, int n_head_kv,
                             int hd, int n_ctx, const int32_t * pos, float * out, pi_stream_t stream);
 
+/* cos/sin table for pi_k_attn_fused: float2 [n_ctx][hd/2], angles formed as the CPU path forms them
+ * (theta advanced by repeated fp32 multiplication with theta_scale = base^(-2/hd), ggml.c:11196-11319) */
+PI_API int pi_k_rope_table(void * table, int n_ctx, int hd, float theta_scale, pi_stream_t stream);
+
+/* pi_k_rope_kv_store + pi_k_attn_decode in one launch (one workgroup per query head; the new cell is used
+ * from LDS and stored by the first query head of each KV group).  Same arithmetic, same cache layout. */
+PI_API int pi_k_attn_fused(const float * qkv, const void * rope_table, void * k_cache, void * v_cache, int n_head, int n_head_kv,
+                           int hd, int mode, int n_ctx, const int32_t * pos, float * out, pi_stream_t stream);
+
 /* x[cols] = row *token of the embedding table (k_get_rows, ggml-cuda.cu:1664) */
 PI_API int pi_k_embed(int wtype, const void * table, int cols, const int32_t * token, float * x, pi_stream_t stream);
 

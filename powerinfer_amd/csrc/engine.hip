@@ -119,9 +119,14 @@ int layer_forward(pi_model * m, int il, bool last_token) {
     else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
     else an = make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
     PI_TRY(pi_k_gemv(wqkv.type, wqkv.dev, d + 2 * gqa, d, x, &an, PI_EPI_NONE, nullptr, nullptr, m->qkv, st));
-    PI_TRY(pi_k_rope_kv_store(m->qkv, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, m->d_pos, hp.n_ctx,
-                              m->q_rot, m->k_cache + kv_off, m->v_cache + kv_off, st));
-    PI_TRY(pi_k_attn_decode(m->q_rot, m->k_cache + kv_off, m->v_cache + kv_off, hp.n_head, hp.n_head_kv, hd, hp.n_ctx, m->d_pos, m->att, st));
+    if (m->rope_table) {
+        PI_TRY(pi_k_attn_fused(m->qkv, m->rope_table, m->k_cache + kv_off, m->v_cache + kv_off, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0,
+                               hp.n_ctx, m->d_pos, m->att, st));
+    } else {
+        PI_TRY(pi_k_rope_kv_store(m->qkv, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, m->d_pos, hp.n_ctx,
+                                  m->q_rot, m->k_cache + kv_off, m->v_cache + kv_off, st));
+        PI_TRY(pi_k_attn_decode(m->q_rot, m->k_cache + kv_off, m->v_cache + kv_off, hp.n_head, hp.n_head_kv, hd, hp.n_ctx, m->d_pos, m->att, st));
+    }
 
     const float * pred_in; const float * ffn_in; pi_norm fn;
     if (!falcon) {
@@ -352,6 +357,13 @@ int pi_model_finalize(pi_model * m) {
         return PI_E_HIP;
     PI_TRY(pi_memset(m->k_cache, 0, kv * 2));
     PI_TRY(pi_memset(m->v_cache, 0, kv * 2));
+    // fused RoPE + attention when the head geometry and context fit its single-pass kernel
+    if (m->hd % 8 == 0 && 256 % (m->hd / 8) == 0 && 64 % (m->hd / 8) == 0 && m->hd / 2 + m->hd <= 256 &&
+        sizeof(float) * ((size_t)hp.n_ctx + (size_t)(256 / (m->hd / 8)) * m->hd + 3 * (size_t)m->hd) <= 60 * 1024) {
+        m->rope_table = m->alloc<float>((size_t)hp.n_ctx * m->hd);
+        if (!m->rope_table) return PI_E_HIP;
+        PI_TRY(pi_k_rope_table(m->rope_table, hp.n_ctx, m->hd, m->theta_scale, nullptr));
+    }
     PI_TRY(pi_memset(m->n_active, 0, sizeof(int32_t) * hp.n_layer));
     PI_TRY(pi_memset(m->d_step, 0, 4));
     PI_TRY(pi_memset(m->h_dense, 0, sizeof(float) * ff));

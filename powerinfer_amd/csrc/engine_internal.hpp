@@ -34,6 +34,7 @@ struct pi_model {
     int32_t *list = nullptr, *n_active = nullptr, *d_token = nullptr, *d_pos = nullptr, *d_step = nullptr;
     int32_t *d_out_tokens = nullptr, *d_out_active = nullptr;
     __half *k_cache = nullptr, *v_cache = nullptr;
+    float *rope_table = nullptr;          // float2 [n_ctx][hd/2] (cos, sin), when the fused attention kernel is used
 
     hipGraphExec_t graph_exec = nullptr;
     hipGraph_t graph = nullptr;

@@ -964,6 +964,120 @@ __global__ __launch_bounds__(kBlock) void attn_decode_kernel(const float * __res
     }
 }
 
+// cos/sin of every (position, pair) the way the CPU path forms them: theta advanced by repeated fp32
+// multiplication (ggml.c:11269-11319), so the angle is bit-identical and only cosf/sinf can differ in the
+// last place.  table[p][i] = (cos, sin) for pair i of position p.
+__global__ void rope_table_kernel(float2 * __restrict__ table, int n_ctx, int half_dim, float theta_scale) {
+    const int p = blockIdx.x, i = threadIdx.x;
+    if (p >= n_ctx || i >= half_dim) return;
+    float theta = (float)p;
+    for (int j = 0; j < i; ++j) theta = __fmul_rn(theta, theta_scale);
+    table[(size_t)p * half_dim + i] = make_float2(cosf(theta), sinf(theta));
+}
+
+// ---------------------------------------------------------------------------------------------------
+// RoPE + KV store + decode attention in one launch, one workgroup per query head.  The workgroup rotates its
+// own q head and the k head of its group (cos/sin from the table), rounds k and v to fp16 as the cache does,
+// and attends over cells [0, pos) from the cache plus the new cell from LDS, so it never reads what this
+// launch writes; the first query head of each group stores k and v.
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void attn_fused_kernel(const float * __restrict__ qkv, const float2 * __restrict__ rope_table,
+                                                            __half * __restrict__ k_cache, __half * __restrict__ v_cache,
+                                                            int n_head, int n_head_kv, int hd, int mode, int n_ctx,
+                                                            const int32_t * __restrict__ pos_p, float * __restrict__ out) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float * s    = reinterpret_cast<float *>(smem);               // [n_ctx] scores, then probabilities
+    float * part = s + n_ctx;                                     // [groups][hd]
+    float * qs   = part + (kBlock / (hd / 8)) * hd;               // [hd] rotated q, rounded to fp16
+    float * kcur = qs + hd;                                       // [hd] rotated k of this position, rounded to fp16
+    float * vcur = kcur + hd;                                     // [hd]
+    __shared__ double red[16];
+    __shared__ float redf[16];
+    const int h = blockIdx.x, grp_sz = n_head / n_head_kv, kvh = h / grp_sz;
+    const int tid = threadIdx.x;
+    const int pos = *pos_p, n_kv = pos + 1;
+    const float * qsrc = qkv + (size_t)h * hd;
+    const float * ksrc = qkv + (size_t)(n_head + kvh) * hd;
+    const float * vsrc = qkv + (size_t)(n_head + n_head_kv + kvh) * hd;
+    __half * kdst = k_cache + ((size_t)kvh * n_ctx + pos) * hd;
+    __half * vdst = v_cache + ((size_t)kvh * n_ctx + pos) * hd;
+    const bool leader = (h % grp_sz) == 0;
+    if (tid < hd / 2) {
+        const float2 cs = rope_table[(size_t)pos * (hd / 2) + tid];
+        const int i0 = (mode & 2) ? tid : 2 * tid;
+        const int i1 = (mode & 2) ? tid + hd / 2 : 2 * tid + 1;
+        const float q0 = qsrc[i0], q1 = qsrc[i1], k0 = ksrc[i0], k1 = ksrc[i1];
+        qs[i0] = pi_round_f16(__fsub_rn(__fmul_rn(q0, cs.x), __fmul_rn(q1, cs.y)));
+        qs[i1] = pi_round_f16(__fadd_rn(__fmul_rn(q0, cs.y), __fmul_rn(q1, cs.x)));
+        const __half ka = __float2half_rn(__fsub_rn(__fmul_rn(k0, cs.x), __fmul_rn(k1, cs.y)));
+        const __half kb = __float2half_rn(__fadd_rn(__fmul_rn(k0, cs.y), __fmul_rn(k1, cs.x)));
+        kcur[i0] = __half2float(ka); kcur[i1] = __half2float(kb);
+        if (leader) { kdst[i0] = ka; kdst[i1] = kb; }
+    } else if (tid < hd / 2 + hd) {
+        const int e = tid - hd / 2;
+        const __half v = __float2half_rn(vsrc[e]);
+        vcur[e] = __half2float(v);
+        if (leader) vdst[e] = v;
+    }
+    __syncthreads();
+
+    const int lpp = hd / 8;
+    const int sub = tid % lpp, grp = tid / lpp, ngrp = kBlock / lpp;
+    const float scale = 1.0f / sqrtf((float)hd);
+    float qf[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qf[i] = qs[sub * 8 + i];
+    const __half * kb = k_cache + (size_t)kvh * n_ctx * hd;
+    for (int c0 = 0; c0 < n_kv; c0 += ngrp) {
+        const int c = c0 + grp;
+        float d = 0.0f;
+        if (c < pos) d = pi_dot8(pi_ld16(kb + (size_t)c * hd + sub * 8), qf, 0.0f);
+        else if (c == pos) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) d = fmaf(kcur[sub * 8 + i], qf[i], d);
+        }
+        for (int o = lpp / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, PI_WAVE);
+        if (c < n_kv && sub == 0) s[c] = __fmul_rn(d, scale);
+    }
+    __syncthreads();
+
+    float mx = -INFINITY;
+    for (int c = tid; c < n_kv; c += kBlock) mx = fmaxf(mx, s[c]);
+    mx = block_max_f32(mx, redf);
+    double sum = 0.0;
+    for (int c = tid; c < n_kv; c += kBlock) {
+        const float e = pi_round_f16(expf(pi_round_f16(__fsub_rn(s[c], mx))));
+        s[c] = e;
+        sum += (double)e;
+    }
+    sum = block_sum_f64(sum, red);
+    const float inv = (float)(1.0 / sum);
+
+    const __half * vb = v_cache + (size_t)kvh * n_ctx * hd;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    for (int c = grp; c < n_kv; c += ngrp) {
+        const float p = pi_round_f16(__fmul_rn(s[c], inv));
+        float vf[8];
+        if (c < pos) pi_unpack8(pi_ld16(vb + (size_t)c * hd + sub * 8), vf);
+        else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vf[i] = vcur[sub * 8 + i];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(vf[i], p, acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) part[grp * hd + sub * 8 + i] = acc[i];
+    __syncthreads();
+    for (int e = tid; e < hd; e += kBlock) {
+        float v = part[e];
+        for (int g = 1; g < ngrp; ++g) v += part[g * hd + e];
+        out[(size_t)h * hd + e] = v;
+    }
+}
+
 __global__ void embed_f16_kernel(const __half * __restrict__ table, int cols, const int32_t * __restrict__ token, float * __restrict__ x) {
     const __half * row = table + (size_t)(*token) * cols;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < cols; i += gridDim.x * blockDim.x) x[i] = __half2float(row[i]);
@@ -1234,6 +1348,24 @@ int pi_k_attn_decode(const float * q_rot, const void * k_cache, const void * v_c
     hipLaunchKernelGGL(attn_decode_kernel, dim3(n_head), dim3(kBlock), sh, (hipStream_t)stream,
                        q_rot, (const __half *)k_cache, (const __half *)v_cache, n_head, n_head_kv, hd, n_ctx, pos, out);
     return pi::check_launch("pi_k_attn_decode");
+}
+
+int pi_k_rope_table(void * table, int n_ctx, int hd, float theta_scale, pi_stream_t stream) {
+    if (!table || n_ctx <= 0 || hd <= 0 || hd % 2 || hd / 2 > 1024) return pi::fail(PI_E_ARG, "pi_k_rope_table: bad arguments");
+    hipLaunchKernelGGL(rope_table_kernel, dim3(n_ctx), dim3(hd / 2), 0, (hipStream_t)stream, (float2 *)table, n_ctx, hd / 2, theta_scale);
+    return pi::check_launch("pi_k_rope_table");
+}
+
+int pi_k_attn_fused(const float * qkv, const void * rope_table, void * k_cache, void * v_cache, int n_head, int n_head_kv, int hd, int mode,
+                    int n_ctx, const int32_t * pos, float * out, pi_stream_t stream) {
+    if (!qkv || !rope_table || !k_cache || !v_cache || !pos || !out) return pi::fail(PI_E_ARG, "pi_k_attn_fused: null pointer");
+    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd % 8 || kBlock % (hd / 8) || PI_WAVE % (hd / 8) || hd / 2 + hd > kBlock || (mode != 0 && mode != 2))
+        return pi::fail(PI_E_ARG, "pi_k_attn_fused: head size must be 8 * (a divisor of 64), at most 128; mode 0 or 2");
+    const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd + 3 * (size_t)hd);
+    if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused: context too long for the single-pass kernel");
+    hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head), dim3(kBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
+                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out);
+    return pi::check_launch("pi_k_attn_fused");
 }
 
 int pi_k_embed(int wtype, const void * table, int cols, const int32_t * token, float * x, pi_stream_t stream) {

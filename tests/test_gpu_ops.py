@@ -109,6 +109,9 @@ def test_rope_attention_sequence(mode, hd, nh, nkv):
     kc_g, vc_g = pl.DevBuf.zeros(nkv * n_ctx * hd * 2), pl.DevBuf.zeros(nkv * n_ctx * hd * 2)
     dq, dpos, dqr, dout = pl.DevBuf((d + 2 * gqa) * 4), pl.DevBuf(4), pl.DevBuf(d * 4), pl.DevBuf(d * 4)
     theta_scale = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
+    kc_f, vc_f = pl.DevBuf.zeros(nkv * n_ctx * hd * 2), pl.DevBuf.zeros(nkv * n_ctx * hd * 2)
+    tab, dout_f = pl.DevBuf(n_ctx * hd * 4), pl.DevBuf(d * 4)
+    pl.check(L.pi_k_rope_table(tab.ptr, n_ctx, hd, theta_scale, None), "rope_table")
     for pos in range(6):
         qkv = rng.standard_normal(d + 2 * gqa).astype(np.float32)
         q, k, v = qkv[:d], qkv[d:d + gqa], qkv[d + gqa:]
@@ -124,10 +127,14 @@ def test_rope_attention_sequence(mode, hd, nh, nkv):
         dpos.upload(p)
         pl.check(L.pi_k_rope_kv_store(dq.ptr, nh, nkv, hd, mode, theta_scale, dpos.ptr, n_ctx, dqr.ptr, kc_g.ptr, vc_g.ptr, None), "rope")
         pl.check(L.pi_k_attn_decode(dqr.ptr, kc_g.ptr, vc_g.ptr, nh, nkv, hd, n_ctx, dpos.ptr, dout.ptr, None), "attn")
+        pl.check(L.pi_k_attn_fused(dq.ptr, tab.ptr, kc_f.ptr, vc_f.ptr, nh, nkv, hd, mode, n_ctx, dpos.ptr, dout_f.ptr, None), "attn_fused")
         pl.sync()
         assert rel_err(dqr.download(np.float32), qr) < 1e-6
         got = dout.download(np.float32)
         assert rel_err(got, want) < 2e-3, (pos, rel_err(got, want))
+        got_f = dout_f.download(np.float32)     # fused launch: same arithmetic; cos/sin come from a table kernel and
+        assert rel_err(got_f, want) < 2e-3      # may differ from the inline ones in the last place before the fp16 rounding
+        assert rel_err(got_f, got) < 1e-3
     # the caches hold the same fp16 values, in this library's [kv_head][cell][hd] layout
     kg = kc_g.download(np.uint16).reshape(nkv, n_ctx, hd)
     vg = vc_g.download(np.uint16).reshape(nkv, n_ctx, hd)
@@ -135,6 +142,8 @@ def test_rope_attention_sequence(mode, hd, nh, nkv):
     vo = vc_o.reshape(nkv, hd, n_ctx).transpose(0, 2, 1)
     assert (kg[:, :6] != ko[:, :6]).mean() < 2e-3          # cos/sin may differ in the last place before rounding
     assert np.array_equal(vg[:, :6], vo[:, :6])
+    assert (kc_f.download(np.uint16) != kc_g.download(np.uint16)).mean() < 1e-3
+    assert np.array_equal(vc_f.download(np.uint16), vc_g.download(np.uint16))
 
 
 def test_embed_and_argmax():

@@ -10,6 +10,7 @@
 
 #include <math.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <utility>
@@ -415,7 +416,9 @@ int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * m
     if (pos + n_steps > m->hp.n_ctx) return pi::fail(PI_E_ARG, "pi_model_generate: would run past the context");
     PI_HIP_TRY(hipMemsetAsync(m->d_step, 0, 4, m->stream));
 
-    const bool use_graph = !m->hybrid && !m->capture;
+    // PI_NO_GRAPH=1 issues the same launches eagerly (useful under tracing tools that cannot follow graph replays)
+    const char * no_graph = getenv("PI_NO_GRAPH");
+    const bool use_graph = !m->hybrid && !m->capture && !(no_graph && no_graph[0] == '1');
     if (use_graph && !m->graph_exec) {
         PI_HIP_TRY(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
         int rc = token_forward(m, true, false);

@@ -130,12 +130,31 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="only for quick trials; the reported workload uses 32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-tokens", type=int, default=24)
+    ap.add_argument("--pmc-probe", action="store_true",
+                    help="counter-collection aid: run only the q|k|v mat-vec of a 4-layer model a few times plus one "
+                         "device-to-device copy of the same byte count (the known-size reference for FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the token loop on ONE GPU; --gpus must be 1 "
                  "(how the path would shard over xGMI is described in DESIGN.md)")
 
     from powerinfer_amd import lib as pl, synth
+    if args.pmc_probe:
+        hp = synth.hparams("llama-7b", n_layer=4, n_ctx=64, seed=1)
+        keep = []
+        m = build_synthetic_on_device(hp, keep)
+        m.decode(np.array([1, 2], np.int32), 0, want_logits=False)
+        d = hp.n_embd
+        nbytes = 3 * d * d * 2
+        src, dst = pl.DevBuf(nbytes), pl.DevBuf(nbytes)
+        pl.check(pl.load().pi_memset(src.ptr, 1, nbytes), "memset")
+        pl.sync()
+        pl.check(pl.load().pi_memcpy_d2d(dst.ptr, src.ptr, nbytes), "copy")     # reads nbytes, writes nbytes
+        pl.sync()
+        ms, n = m.time_section(0, 4)
+        print(json.dumps({"pmc_probe": True, "copy_bytes": nbytes, "qkv_weight_bytes": nbytes, "qkv_launches": n, "us_per_launch": ms * 1e3}))
+        m.close()
+        return
     hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=args.prompt + args.warmup + args.steps + 8, seed=1)
     keep = []
     t0 = time.perf_counter()
@@ -167,6 +186,16 @@ def main():
     ffn_bytes = (d * hp.n_rank + hp.n_rank * hp.n_ff) * 2.0 + (act.mean() / hp.n_layer) * 3 * d * 2.0
     ms_head, _ = m.time_section(2, 8)
 
+    # HBM bytes per launch of that kernel from the FETCH_SIZE / WRITE_SIZE counter runs (profiles/qkv_gemv_hbm_traffic.md)
+    traffic = None
+    try:
+        with open(os.path.join(ROOT, "profiles", "qkv_gemv_hbm_traffic.json")) as f:
+            pj = json.load(f)
+        if pj.get("shape") == [d + 2 * gqa, d]:
+            traffic = pj["traffic_bytes_per_launch"]
+    except (OSError, ValueError, KeyError):
+        pass
+
     out = {
         "metric": "decode tok/s bs=1 ReLU-Llama2-7B FP16",
         "value": round(1e3 / ms_per_step, 2),
@@ -190,12 +219,12 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_f16_kernel<4> (q|k|v projection, 12288 x 4096 fp16, fused RMSNorm)",
+            "kernel": "gemv_f16_kernel<4,2,0> (q|k|v projection, 12288 x 4096 fp16, fused RMSNorm)",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
             "frac": round(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": None,
+            "traffic": traffic,
             "bytes_per_launch": qkv_bytes,
             "us_per_launch": round(ms_qkv * 1e3, 2),
             "launches_timed": n_qkv,

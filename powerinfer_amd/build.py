@@ -17,6 +17,8 @@ FLAGS = [
     # packed-FP32 instructions are not to be generated on this hardware pool
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
+    # host code of the cold path uses the x86 vector extensions every MI355X host CPU has
+    "-Xarch_host", "-mavx2", "-Xarch_host", "-mfma", "-Xarch_host", "-mf16c",
 ]
 
 

@@ -61,7 +61,8 @@ def run_case(hp, n_prompt=12, n_gen=64):
         for il in range(hp.n_layer):
             mask_g = ~(plg_g[il] < thr)
             tflips += int((mask_g != ~(om.cap_lg[il, 0] < thr)).sum())
-            assert na_g[il] == mask_g.sum()
+            gid = model["layers"][il].get("gpu_idx")
+            assert na_g[il] == (mask_g.sum() if gid is None else (mask_g & (gid == 1)).sum())   # the GPU's list covers its bucket only
             o = oracle_ffn_on(model, il, src_g[il])
             assert rel_err(plg_g[il], o["logits"][0]) < 1e-4
             if np.array_equal(mask_g, ~(o["logits"][0] < thr)):
@@ -128,6 +129,14 @@ def test_llama_7b_width_two_layers():
     """Full 7B layer shape (d 4096, ff 11008, rank 1024, 32 heads, vocab 32000), two layers."""
     hp = synth.hparams("llama-7b", n_layer=2, n_ctx=128, seed=6)
     run_case(hp, n_prompt=8, n_gen=64)
+
+
+@pytest.mark.parametrize("arch,wtype", [("llama-tiny", synth.F16), ("llama-tiny", synth.Q4_0), ("falcon-tiny", synth.F16)])
+def test_hybrid_split_matches_all_cold_oracle(arch, wtype):
+    """Config-2 style partial split: the hottest 60 % of each layer's neurons live on the GPU (compact matrices +
+    gpu_bucket), the rest run on host threads, the two partial results are added.  The sum must equal the CPU
+    path computing every neuron (gpu_idx = 0 everywhere)."""
+    run_case(synth.hparams(arch, wtype=wtype, n_ctx=96, seed=8, hot_frac=0.6), n_prompt=8, n_gen=24)
 
 
 def test_decode_rejects_bad_arguments():

@@ -1,0 +1,546 @@
+// The reference's accelerator-backend entry points (ggml-cuda.h:21-60) implemented on this library's kernels, so
+// that a host built against the reference's ggml.h / ggml-cuda.h links to libpowerinfer_hip.so instead of
+// ggml-cuda.cu.  Per-node dispatch as ggml_cuda_compute_forward does it (ggml-cuda.cu:9218-9346); the hot
+// operators (MUL_MAT at one token, MUL_MAT_SPARSE, AXPY) go to the tuned launchers, everything else to small
+// generic kernels.  Device addresses live in tensor->extra.  Errors are fatal, as in the reference
+// (CUDA_CHECK -> exit(1), ggml-cuda.cu:192-229).
+#include "runtime.hpp"
+#include "device_utils.hpp"
+#include "../../include/ggml_backend_abi.h"
+#include "../../include/powerinfer_hip.h"
+
+#include <math.h>
+#include <stdio.h>
+#include <stdlib.h>
+#include <string.h>
+
+#include <mutex>
+#include <vector>
+
+namespace {
+
+struct Extra {
+    void * data_device[GGML_CUDA_MAX_DEVICES];     // [0] is the only one used (single GPU)
+    bool   owned;
+};
+
+bool   g_loaded = false;
+float  g_threshold = 0.0f;
+char * g_scratch = nullptr;
+size_t g_scratch_size = 0, g_scratch_offset = 0;
+pi_workspace * g_ws = nullptr;
+int    g_ws_ff = 0, g_ws_d = 0;
+std::mutex g_mu;
+std::vector<Extra *> g_graph_extras;               // extras handed out by assign_*; freed with the scratch
+
+[[noreturn]] void die(const char * what) {
+    fprintf(stderr, "powerinfer-hip backend: %s: %s\n", what, pi_last_error());
+    exit(1);
+}
+#define BK_HIP(expr) do { hipError_t _e = (expr); if (_e != hipSuccess) { fprintf(stderr, "powerinfer-hip backend: %s: %s\n", #expr, hipGetErrorString(_e)); exit(1); } } while (0)
+#define BK_PI(expr) do { if ((expr) != PI_OK) die(#expr); } while (0)
+
+int blck(int type) { return type == GGML_TYPE_Q4_0 ? 32 : 1; }
+size_t tsize(int type) {
+    switch (type) {
+        case GGML_TYPE_F32: case GGML_TYPE_I32: return 4;
+        case GGML_TYPE_F16: case GGML_TYPE_I16: return 2;
+        case GGML_TYPE_I8: return 1;
+        case GGML_TYPE_Q4_0: return 18;
+        default: return 0;
+    }
+}
+size_t row_size(const ggml_tensor * t) { return tsize(t->type) * (size_t)(t->ne[0] / blck(t->type)); }
+int64_t nrows(const ggml_tensor * t) { return t->ne[1] * t->ne[2] * t->ne[3]; }
+int64_t nelem(const ggml_tensor * t) { return t->ne[0] * nrows(t); }
+size_t nbytes(const ggml_tensor * t) {
+    size_t n = tsize(t->type) * (size_t)(t->ne[0] / blck(t->type));        // ggml_nbytes: extent of the last element
+    for (int i = 1; i < GGML_MAX_DIMS; ++i) n += (size_t)(t->ne[i] - 1) * t->nb[i];
+    return n;
+}
+bool contiguous(const ggml_tensor * t) {
+    return t->nb[0] == tsize(t->type) && t->nb[1] == row_size(t) && t->nb[2] == t->nb[1] * (size_t)t->ne[1] && t->nb[3] == t->nb[2] * (size_t)t->ne[2];
+}
+
+// temporaries of one operator call (CPU-resident operands staged on the device, device results bound for the host)
+struct Temps {
+    std::vector<void *> ptrs;
+    void * get(size_t n) { void * p = pi_malloc(n); if (!p) die("temporary allocation"); ptrs.push_back(p); return p; }
+    ~Temps() { for (void * p : ptrs) pi_free(p); }
+};
+
+void * dev_in(const ggml_tensor * t, Temps & tmp) {
+    if (t->backend != GGML_BACKEND_CPU) {
+        if (!t->extra) { fprintf(stderr, "powerinfer-hip backend: tensor '%s' is marked GPU but has no device buffer\n", t->name); exit(1); }
+        return ((Extra *)t->extra)->data_device[0];
+    }
+    const size_t n = nbytes(t);
+    void * p = tmp.get(n);
+    BK_PI(pi_memcpy_h2d(p, t->data, n));
+    return p;
+}
+void * dev_out(ggml_tensor * t, Temps & tmp) {
+    if (t->backend != GGML_BACKEND_CPU) {
+        if (!t->extra) { fprintf(stderr, "powerinfer-hip backend: tensor '%s' is marked GPU but has no device buffer\n", t->name); exit(1); }
+        return ((Extra *)t->extra)->data_device[0];
+    }
+    return tmp.get(nbytes(t));
+}
+void finish_out(ggml_tensor * t, void * dptr) {
+    if (t->backend == GGML_BACKEND_CPU) {          // result wanted on the host: copy back, device idle on return
+        BK_PI(pi_sync());
+        BK_PI(pi_memcpy_d2h(t->data, dptr, nbytes(t)));
+    }
+}
+
+pi_workspace * workspace(int ff, int d) {
+    if (!g_ws || ff > g_ws_ff || d > g_ws_d) {
+        if (g_ws) { pi_sync(); pi_workspace_destroy(g_ws); }
+        g_ws_ff = ff > g_ws_ff ? ff : g_ws_ff; g_ws_d = d > g_ws_d ? d : g_ws_d;
+        g_ws = pi_workspace_create(g_ws_ff, g_ws_d);
+        if (!g_ws) die("workspace");
+    }
+    return g_ws;
+}
+
+// ---- generic kernels (correctness-first; the tuned paths are the pi_k_* launchers) -----------------------
+__global__ void bin_kernel(const float * a, const float * b, float * y, int64_t n, int64_t nb, int is_mul) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = is_mul ? __fmul_rn(a[i], b[i % nb]) : __fadd_rn(a[i], b[i % nb]);
+}
+__global__ void relu_kernel(const float * a, float * y, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = fmaxf(a[i], 0.0f);
+}
+__global__ void scale_kernel(const float * a, float * y, float s, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = __fmul_rn(a[i], s);
+}
+__global__ void fill_kernel(float * y, float v, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) y[i] = v;
+}
+// one workgroup per row; kind 0 rms_norm (ggml.c:9238), 1 norm (ggml.c:9169)
+__global__ __launch_bounds__(256) void norm_rows_kernel(const float * x, float * y, int n, float eps, int kind) {
+    __shared__ double red[4];
+    const float * xr = x + (size_t)blockIdx.x * n; float * yr = y + (size_t)blockIdx.x * n;
+    auto bsum = [&](double v) {
+        v = pi_wave_sum_f64(v);
+        __syncthreads();
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+        __syncthreads();
+        return red[0] + red[1] + red[2] + red[3];
+    };
+    float mean = 0.0f;
+    double s = 0.0;
+    if (kind == 0) { for (int i = threadIdx.x; i < n; i += 256) s += (double)__fmul_rn(xr[i], xr[i]); s = bsum(s); }
+    else {
+        for (int i = threadIdx.x; i < n; i += 256) s += (double)xr[i];
+        mean = (float)(bsum(s) / n);
+        s = 0.0;
+        for (int i = threadIdx.x; i < n; i += 256) { const float v = __fsub_rn(xr[i], mean); s += (double)__fmul_rn(v, v); }
+        s = bsum(s);
+    }
+    const float scale = 1.0f / sqrtf((float)(s / n) + eps);
+    for (int i = threadIdx.x; i < n; i += 256) yr[i] = __fmul_rn(__fsub_rn(xr[i], mean), scale);
+}
+// one workgroup per row; exp through the fp16 rounding of the CPU path's table (ggml.c:10747-10759)
+__global__ __launch_bounds__(256) void softmax_rows_kernel(const float * x, float * y, int n) {
+    __shared__ double red[4];
+    __shared__ float redf[4];
+    const float * xr = x + (size_t)blockIdx.x * n; float * yr = y + (size_t)blockIdx.x * n;
+    float mx = -INFINITY;
+    for (int i = threadIdx.x; i < n; i += 256) mx = fmaxf(mx, xr[i]);
+    mx = pi_wave_max(mx);
+    if ((threadIdx.x & 63) == 0) redf[threadIdx.x >> 6] = mx;
+    __syncthreads();
+    mx = fmaxf(fmaxf(redf[0], redf[1]), fmaxf(redf[2], redf[3]));
+    double s = 0.0;
+    for (int i = threadIdx.x; i < n; i += 256) {
+        const float v = xr[i] == -INFINITY ? 0.0f : pi_round_f16(expf(pi_round_f16(__fsub_rn(xr[i], mx))));
+        yr[i] = v; s += (double)v;
+    }
+    s = pi_wave_sum_f64(s);
+    if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = s;
+    __syncthreads();
+    const float inv = (float)(1.0 / (red[0] + red[1] + red[2] + red[3]));
+    for (int i = threadIdx.x; i < n; i += 256) yr[i] = __fmul_rn(yr[i], inv);
+}
+// x [hd, n_head, T] contiguous, pos[T]; mode 0 adjacent pairs, 2 NeoX halves (ggml.c:11163-11325, no YaRN)
+__global__ void rope_kernel(const float * x, const int32_t * pos, float * y, int hd, int n_head, int n_dims, int mode, float theta_scale, float freq_scale) {
+    const int t = blockIdx.y, h = blockIdx.x, i = threadIdx.x;         // i = pair index < n_dims/2
+    const float * s = x + ((size_t)t * n_head + h) * hd; float * o = y + ((size_t)t * n_head + h) * hd;
+    float theta = (float)pos[t];
+    if (mode & 2) theta = __fmul_rn(theta, freq_scale);
+    for (int j = 0; j < i; ++j) theta = __fmul_rn(theta, theta_scale);
+    const float th = __fmul_rn(freq_scale, theta);
+    const float c = cosf(th), sn = sinf(th);
+    const int i0 = (mode & 2) ? i : 2 * i, i1 = (mode & 2) ? i + n_dims / 2 : 2 * i + 1;
+    const float x0 = s[i0], x1 = s[i1];
+    o[i0] = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, sn));
+    o[i1] = __fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, c));
+}
+struct Shape { int64_t ne[4]; size_t nb[4]; };
+// element-wise copy with type conversion between two 4-D strided tensors of the same element count (ggml_cpy)
+__global__ void cpy_kernel(const char * src, Shape ss, int stype, char * dst, Shape ds, int dtype, int64_t n) {
+    const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    int64_t r = i; size_t so = 0, dof = 0;
+    { int64_t q = r; for (int k = 0; k < 4; ++k) { const int64_t id = q % ss.ne[k]; q /= ss.ne[k]; so += (size_t)id * ss.nb[k]; } }
+    { int64_t q = r; for (int k = 0; k < 4; ++k) { const int64_t id = q % ds.ne[k]; q /= ds.ne[k]; dof += (size_t)id * ds.nb[k]; } }
+    const float v = stype == GGML_TYPE_F16 ? __half2float(*(const __half *)(src + so)) : *(const float *)(src + so);
+    if (dtype == GGML_TYPE_F16) *(__half *)(dst + dof) = __float2half_rn(v); else *(float *)(dst + dof) = v;
+}
+// generic mat-mul for strided / batched operands (attention K.q and V.p): one wave per output element.
+// src0 F16 or F32 [ne00, ne01, ne02, ne03] with strides, src1 F32 [ne00, ne11, ne12, ne13]; activations rounded to fp16
+// when src0 is F16, as the CPU path does.
+__global__ __launch_bounds__(64) void mul_mat_strided_kernel(const char * w, Shape ws, int wtype, const char * x, Shape xs, float * y, Shape ys) {
+    const int64_t r = blockIdx.x, t = blockIdx.y, b = blockIdx.z;
+    const int64_t i12 = b % xs.ne[2], i13 = b / xs.ne[2];
+    const int64_t i02 = i12 / (xs.ne[2] / ws.ne[2]), i03 = i13 / (xs.ne[3] / ws.ne[3]);
+    const char * wr = w + r * ws.nb[1] + i02 * ws.nb[2] + i03 * ws.nb[3];
+    const char * xr = x + t * xs.nb[1] + i12 * xs.nb[2] + i13 * xs.nb[3];
+    float acc = 0.0f;
+    for (int64_t k = threadIdx.x; k < ws.ne[0]; k += 64) {
+        const float xv = *(const float *)(xr + k * xs.nb[0]);
+        if (wtype == GGML_TYPE_F16) acc = fmaf(__half2float(*(const __half *)(wr + k * ws.nb[0])), pi_round_f16(xv), acc);
+        else acc = fmaf(*(const float *)(wr + k * ws.nb[0]), xv, acc);
+    }
+    acc = pi_wave_sum(acc);
+    if (threadIdx.x == 0) *(float *)((char *)y + r * ys.nb[0] + t * ys.nb[1] + i12 * ys.nb[2] + i13 * ys.nb[3]) = acc;
+}
+__global__ void get_rows_kernel(const char * table, int type, size_t row_bytes, const int32_t * ids, float * y, int cols) {
+    const char * row = table + (size_t)ids[blockIdx.y] * row_bytes;
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= cols) return;
+    float v;
+    if (type == GGML_TYPE_F32) v = ((const float *)row)[i];
+    else if (type == GGML_TYPE_F16) v = __half2float(((const __half *)row)[i]);
+    else {
+        const pi_block_q4_0 * blk = (const pi_block_q4_0 *)row + (i >> 5);
+        uint16_t d; __builtin_memcpy(&d, &blk->d, 2);
+        const int j = i & 31;
+        const int q = j < 16 ? (blk->qs[j] & 0x0F) : (blk->qs[j - 16] >> 4);
+        v = __fmul_rn((float)(q - 8), pi_f16_from_bits(d));
+    }
+    y[(size_t)blockIdx.y * cols + i] = v;
+}
+__global__ void gather_h_kernel(const float * h_dense, const int32_t * list, const int32_t * n_active, const int32_t * bucket, float * h_compact) {
+    const int n = *n_active;
+    for (int k = blockIdx.x * blockDim.x + threadIdx.x; k < n; k += gridDim.x * blockDim.x) {
+        const int row = list[k];
+        h_compact[k] = h_dense[bucket ? bucket[row] : row];
+    }
+}
+
+Shape shape_of(const ggml_tensor * t) { Shape s; for (int i = 0; i < 4; ++i) { s.ne[i] = t->ne[i]; s.nb[i] = t->nb[i]; } return s; }
+dim3 grid1(int64_t n) { return dim3((unsigned)((n + 255) / 256)); }
+
+// ---- operators ---------------------------------------------------------------------------------------------
+bool op_mul_mat(ggml_tensor * dst) {
+    const ggml_tensor * a = dst->src[0]; const ggml_tensor * b = dst->src[1];
+    if (b->type != GGML_TYPE_F32 || dst->type != GGML_TYPE_F32) return false;
+    Temps tmp;
+    const bool weight_like = a->ne[2] == 1 && a->ne[3] == 1 && a->nb[0] == tsize(a->type) && a->nb[1] == row_size(a) && contiguous(b) && contiguous(dst) &&
+                             (a->type == GGML_TYPE_F16 || a->type == GGML_TYPE_Q4_0) && a->ne[0] % (a->type == GGML_TYPE_F16 ? 8 : 32) == 0;
+    if (!weight_like && a->type != GGML_TYPE_F16 && a->type != GGML_TYPE_F32) return false;
+    const char * wa = (const char *)dev_in(a, tmp); const char * xb = (const char *)dev_in(b, tmp); float * y = (float *)dev_out(dst, tmp);
+    if (weight_like) {
+        const int64_t T = nrows(b);
+        for (int64_t t = 0; t < T; ++t)
+            BK_PI(pi_k_gemv(a->type, wa, (int)a->ne[1], (int)a->ne[0], (const float *)xb + t * b->ne[0], nullptr, PI_EPI_NONE, nullptr, nullptr, y + t * a->ne[1], nullptr));
+    } else {
+        hipLaunchKernelGGL(mul_mat_strided_kernel, dim3((unsigned)a->ne[1], (unsigned)b->ne[1], (unsigned)(b->ne[2] * b->ne[3])), dim3(64), 0, 0,
+                           wa, shape_of(a), (int)a->type, xb, shape_of(b), y, shape_of(dst));
+    }
+    finish_out(dst, y);
+    return true;
+}
+
+bool sparse_common(ggml_tensor * dst, bool axpy) {
+    const ggml_tensor * w = dst->src[0]; const ggml_tensor * x = dst->src[1]; const ggml_tensor * idx = dst->src[2]; const ggml_tensor * aux = dst->src[3];
+    if (!idx || (w->type != GGML_TYPE_F16 && w->type != GGML_TYPE_Q4_0) || x->type != GGML_TYPE_F32 || idx->type != GGML_TYPE_F32) return false;
+    if (!contiguous(x) || !contiguous(idx) || !contiguous(dst) || w->nb[1] != row_size(w)) return false;
+    Temps tmp;
+    const int d = (int)w->ne[0], rows = (int)w->ne[1], ff = (int)idx->ne[0];
+    const int64_t T = nrows(x);
+    const char * wd = (const char *)dev_in(w, tmp); const float * xd = (const float *)dev_in(x, tmp);
+    const float * id = (const float *)dev_in(idx, tmp);
+    const int32_t * bk = aux ? (const int32_t *)dev_in(aux, tmp) : nullptr;       // GPU part: gpu_bucket maps rows -> neurons
+    const int n_bucket = aux ? (int)aux->ne[0] : 0;
+    if (aux && n_bucket != rows) return false;
+    if (!aux && rows != ff) return false;
+    float * y = (float *)dev_out(dst, tmp);
+    pi_workspace * ws = workspace(ff, d);
+    int32_t * list = (int32_t *)tmp.get(sizeof(int32_t) * (size_t)rows);
+    int32_t * n_act = (int32_t *)tmp.get(sizeof(int32_t));
+    float * hc = (float *)tmp.get(sizeof(float) * (size_t)rows);
+    const int out_n = (int)dst->ne[0];
+    for (int64_t t = 0; t < T; ++t) {
+        BK_PI(pi_k_compact_active(id + t * ff, ff, g_threshold, bk, n_bucket, list, n_act, ws, nullptr));
+        if (!axpy) {
+            // dst[neuron] = W[row] . x for active rows, 0 elsewhere (GGML_OP_MUL_MAT_SPARSE; upscale writes bucket positions only)
+            hipLaunchKernelGGL(fill_kernel, grid1(out_n), dim3(256), 0, 0, y + t * out_n, 0.0f, (int64_t)out_n);
+            BK_PI(pi_k_sparse_upgate(w->type, wd, nullptr, d, ff, xd + t * d, nullptr, 0, list, n_act, bk, hc, nullptr, y + t * out_n, nullptr, ws, nullptr));
+        } else {
+            // x is the dense, neuron-indexed h; out[d] = sum over active rows of h[neuron] * Wt[row]
+            hipLaunchKernelGGL(gather_h_kernel, dim3(16), dim3(256), 0, 0, xd + t * ff, list, n_act, bk, hc);
+            BK_PI(pi_k_sparse_axpy(w->type, wd, d, rows, hc, xd + t * ff, bk, list, n_act, PI_EPI_NONE, nullptr, nullptr, y + t * d, ws, nullptr));
+        }
+    }
+    finish_out(dst, y);
+    return true;
+}
+
+bool op_elementwise(ggml_tensor * dst) {
+    const ggml_tensor * a = dst->src[0]; const ggml_tensor * b = dst->src[1];
+    if (a->type != GGML_TYPE_F32 || dst->type != GGML_TYPE_F32 || !contiguous(a) || !contiguous(dst)) return false;
+    Temps tmp;
+    const int64_t n = nelem(dst);
+    if (dst->op == GGML_OP_ADD || dst->op == GGML_OP_MUL) {
+        if (!b || b->type != GGML_TYPE_F32 || !contiguous(b) || n % nelem(b)) return false;
+        const float * ad = (const float *)dev_in(a, tmp); const float * bd = (const float *)dev_in(b, tmp); float * y = (float *)dev_out(dst, tmp);
+        hipLaunchKernelGGL(bin_kernel, grid1(n), dim3(256), 0, 0, ad, bd, y, n, nelem(b), dst->op == GGML_OP_MUL ? 1 : 0);
+        finish_out(dst, y);
+    } else if (dst->op == GGML_OP_UNARY) {
+        const float * ad = (const float *)dev_in(a, tmp); float * y = (float *)dev_out(dst, tmp);
+        hipLaunchKernelGGL(relu_kernel, grid1(n), dim3(256), 0, 0, ad, y, n);
+        finish_out(dst, y);
+    } else if (dst->op == GGML_OP_SCALE) {
+        float s;
+        if (b->backend == GGML_BACKEND_CPU) s = *(const float *)b->data;               // the factor is a 1-element tensor read on the host
+        else { BK_PI(pi_sync()); BK_PI(pi_memcpy_d2h(&s, ((Extra *)b->extra)->data_device[0], 4)); }
+        const float * ad = (const float *)dev_in(a, tmp); float * y = (float *)dev_out(dst, tmp);
+        hipLaunchKernelGGL(scale_kernel, grid1(n), dim3(256), 0, 0, ad, y, s, n);
+        finish_out(dst, y);
+    } else if (dst->op == GGML_OP_RMS_NORM || dst->op == GGML_OP_NORM) {
+        float eps; memcpy(&eps, dst->op_params, 4);
+        const float * ad = (const float *)dev_in(a, tmp); float * y = (float *)dev_out(dst, tmp);
+        hipLaunchKernelGGL(norm_rows_kernel, dim3((unsigned)nrows(a)), dim3(256), 0, 0, ad, y, (int)a->ne[0], eps, dst->op == GGML_OP_NORM ? 1 : 0);
+        finish_out(dst, y);
+    } else if (dst->op == GGML_OP_SOFT_MAX) {
+        const float * ad = (const float *)dev_in(a, tmp); float * y = (float *)dev_out(dst, tmp);
+        hipLaunchKernelGGL(softmax_rows_kernel, dim3((unsigned)nrows(a)), dim3(256), 0, 0, ad, y, (int)a->ne[0]);
+        finish_out(dst, y);
+    } else {
+        return false;
+    }
+    return true;
+}
+
+bool op_rope(ggml_tensor * dst) {
+    const ggml_tensor * a = dst->src[0]; const ggml_tensor * p = dst->src[1];
+    if (a->type != GGML_TYPE_F32 || !contiguous(a) || !contiguous(dst) || !p || p->type != GGML_TYPE_I32 || a->ne[3] != 1) return false;
+    const int n_dims = dst->op_params[1], mode = dst->op_params[2];
+    float freq_base, freq_scale, ext_factor;
+    memcpy(&freq_base, dst->op_params + 5, 4); memcpy(&freq_scale, dst->op_params + 6, 4); memcpy(&ext_factor, dst->op_params + 7, 4);
+    if ((mode != 0 && mode != 2) || ext_factor != 0.0f || n_dims != a->ne[0] || n_dims / 2 > 1024) return false;       // no GLM / YaRN / partial rotation here
+    Temps tmp;
+    const float * ad = (const float *)dev_in(a, tmp); const int32_t * pd = (const int32_t *)dev_in(p, tmp); float * y = (float *)dev_out(dst, tmp);
+    const float theta_scale = powf(freq_base, -2.0f / n_dims);
+    hipLaunchKernelGGL(rope_kernel, dim3((unsigned)a->ne[1], (unsigned)a->ne[2]), dim3(n_dims / 2), 0, 0, ad, pd, y, (int)a->ne[0], (int)a->ne[1], n_dims, mode, theta_scale, freq_scale);
+    finish_out(dst, y);
+    return true;
+}
+
+bool op_cpy(ggml_tensor * dst) {
+    // CPY: src0 -> src1 (a view, e.g. into the KV cache), dst is a view of src1.  CONT / DUP: src0 -> dst.
+    const ggml_tensor * a = dst->src[0];
+    ggml_tensor * to = dst->op == GGML_OP_CPY ? dst->src[1] : dst;
+    if ((a->type != GGML_TYPE_F32 && a->type != GGML_TYPE_F16) || (to->type != GGML_TYPE_F32 && to->type != GGML_TYPE_F16) || nelem(a) != nelem(to)) return false;
+    Temps tmp;
+    const char * ad = (const char *)dev_in(a, tmp);
+    char * td;
+    if (to->backend != GGML_BACKEND_CPU) td = (char *)((Extra *)to->extra)->data_device[0];
+    else { td = (char *)tmp.get(nbytes(to)); BK_PI(pi_memcpy_h2d(td, to->data, nbytes(to))); }      // strided destination: keep the gaps
+    hipLaunchKernelGGL(cpy_kernel, grid1(nelem(a)), dim3(256), 0, 0, ad, shape_of(a), (int)a->type, td, shape_of(to), (int)to->type, nelem(a));
+    finish_out(to, td);
+    return true;
+}
+
+bool op_get_rows(ggml_tensor * dst) {
+    const ggml_tensor * a = dst->src[0]; const ggml_tensor * ids = dst->src[1];
+    if (!ids || ids->type != GGML_TYPE_I32 || a->nb[1] != row_size(a) || !contiguous(dst) || tsize(a->type) == 0 || a->type == GGML_TYPE_I32) return false;
+    Temps tmp;
+    const char * ad = (const char *)dev_in(a, tmp); const int32_t * id = (const int32_t *)dev_in(ids, tmp); float * y = (float *)dev_out(dst, tmp);
+    hipLaunchKernelGGL(get_rows_kernel, dim3((unsigned)((a->ne[0] + 255) / 256), (unsigned)nelem(ids)), dim3(256), 0, 0, ad, (int)a->type, row_size(a), id, y, (int)a->ne[0]);
+    finish_out(dst, y);
+    return true;
+}
+
+Extra * new_extra(void * p, bool owned) {
+    Extra * e = new Extra();
+    memset(e, 0, sizeof *e);
+    e->data_device[0] = p; e->owned = owned;
+    return e;
+}
+
+void assign(ggml_tensor * tensor, bool scratch, bool alloc) {
+    if (tensor->src[0] && tensor->src[0]->backend == GGML_BACKEND_CPU &&
+        (tensor->op == GGML_OP_RESHAPE || tensor->op == GGML_OP_VIEW || tensor->op == GGML_OP_PERMUTE || tensor->op == GGML_OP_TRANSPOSE))
+        assign(tensor->src[0], scratch, alloc);                      // a GPU view needs its parent on the GPU too (ggml-cuda.cu:9047-9060)
+    tensor->backend = GGML_BACKEND_GPU;
+    if (!alloc || tensor->extra) return;
+    std::lock_guard<std::mutex> g(g_mu);
+    if (tensor->view_src && tensor->view_src->extra) {               // views share the parent's buffer
+        Extra * e = new_extra((char *)((Extra *)tensor->view_src->extra)->data_device[0] + tensor->view_offs, false);
+        g_graph_extras.push_back(e); tensor->extra = e; return;
+    }
+    const size_t n = (nbytes(tensor) + 255) & ~(size_t)255;
+    void * p;
+    if (scratch && g_scratch_size >= n) {
+        if (!g_scratch) { g_scratch = (char *)pi_malloc(g_scratch_size); if (!g_scratch) die("scratch"); }
+        if (g_scratch_offset + n > g_scratch_size) g_scratch_offset = 0;            // ring, as the reference's scratch buffer
+        p = g_scratch + g_scratch_offset; g_scratch_offset += n;
+        Extra * e = new_extra(p, false); g_graph_extras.push_back(e); tensor->extra = e;
+    } else {
+        p = pi_malloc(n); if (!p) die("tensor allocation");
+        Extra * e = new_extra(p, true); g_graph_extras.push_back(e); tensor->extra = e;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+void ggml_init_cublas(void) {
+    std::lock_guard<std::mutex> g(g_mu);
+    if (g_loaded) return;
+    g_loaded = pi_init(0) == PI_OK;
+    if (!g_loaded) fprintf(stderr, "powerinfer-hip backend: no usable HIP device (%s)\n", pi_last_error());
+}
+bool ggml_cublas_loaded(void) { return g_loaded; }
+
+void * ggml_cuda_host_malloc(size_t size) {
+    if (getenv("GGML_CUDA_NO_PINNED")) return nullptr;
+    void * p = nullptr;
+    if (hipHostMalloc(&p, size, hipHostMallocDefault) != hipSuccess) { (void)hipGetLastError(); return nullptr; }
+    return p;
+}
+void ggml_cuda_host_free(void * ptr) { if (ptr) BK_HIP(hipHostFree(ptr)); }
+
+bool ggml_cuda_can_mul_mat(const struct ggml_tensor * src0, const struct ggml_tensor * src1, struct ggml_tensor * dst) {
+    const int64_t ne10 = src1->ne[0], ne0 = dst->ne[0], ne1 = dst->ne[1];
+    return (src0->type == GGML_TYPE_F32 || src0->type == GGML_TYPE_F16 || src0->type == GGML_TYPE_Q4_0) &&
+           src1->type == GGML_TYPE_F32 && dst->type == GGML_TYPE_F32 && ne0 >= 32 && ne1 >= 32 && ne10 >= 32;   // ggml-cuda.cu:8714-8727
+}
+void ggml_cuda_set_tensor_split(const float * tensor_split) { (void)tensor_split; }       // one GPU
+void ggml_cuda_set_main_device(int main_device) { if (main_device != 0) fprintf(stderr, "powerinfer-hip backend: single-GPU build, main device stays 0\n"); }
+void ggml_cuda_set_mul_mat_q(bool mul_mat_q) { (void)mul_mat_q; }
+
+void ggml_cuda_transform_tensor(void * data, struct ggml_tensor * tensor) {
+    const size_t n = nbytes(tensor);
+    void * p = pi_malloc(n); if (!p) die("ggml_cuda_transform_tensor");
+    BK_PI(pi_memcpy_h2d(p, data, n));
+    tensor->extra = new_extra(p, true);
+}
+void ggml_cuda_alloc_tensor(struct ggml_tensor * tensor) {
+    void * p = pi_malloc(nbytes(tensor)); if (!p) die("ggml_cuda_alloc_tensor");
+    tensor->extra = new_extra(p, true);
+}
+void ggml_cuda_free_data(struct ggml_tensor * tensor) {
+    if (!tensor || !tensor->extra) return;
+    Extra * e = (Extra *)tensor->extra;
+    if (e->owned && e->data_device[0]) pi_free(e->data_device[0]);
+    {
+        std::lock_guard<std::mutex> g(g_mu);
+        for (auto & x : g_graph_extras) if (x == e) x = nullptr;
+    }
+    delete e;
+    tensor->extra = nullptr;
+}
+// copies src's host row into dst's current device pointer; the caller then bumps the pointer it got from
+// ggml_cuda_get_data_pp to stream the bucket's rows into a compact matrix (llama.cpp:2898-2967)
+void ggml_cuda_cpy_1d(struct ggml_tensor * dst, const struct ggml_tensor * src) {
+    BK_PI(pi_memcpy_h2d(((Extra *)dst->extra)->data_device[0], src->data, nbytes(src)));
+}
+void ** ggml_cuda_get_data_pp(struct ggml_tensor * tensor) { return &((Extra *)tensor->extra)->data_device[0]; }
+
+void ggml_cuda_assign_buffers(struct ggml_tensor * tensor) { assign(tensor, true, true); }
+void ggml_cuda_assign_buffers_no_scratch(struct ggml_tensor * tensor) { assign(tensor, false, true); }
+void ggml_cuda_assign_buffers_force_inplace(struct ggml_tensor * tensor) { assign(tensor, true, true); }
+void ggml_cuda_assign_buffers_no_alloc(struct ggml_tensor * tensor) { assign(tensor, false, false); }
+void ggml_cuda_assign_scratch_offset(struct ggml_tensor * tensor, size_t offset) {
+    std::lock_guard<std::mutex> g(g_mu);
+    if (!g_scratch_size) { fprintf(stderr, "powerinfer-hip backend: ggml_cuda_assign_scratch_offset without a scratch size\n"); exit(1); }
+    if (!g_scratch) { g_scratch = (char *)pi_malloc(g_scratch_size); if (!g_scratch) die("scratch"); }
+    if (offset + nbytes(tensor) > g_scratch_size) { fprintf(stderr, "powerinfer-hip backend: scratch offset out of range for '%s'\n", tensor->name); exit(1); }
+    if (!tensor->extra) { Extra * e = new_extra(nullptr, false); g_graph_extras.push_back(e); tensor->extra = e; }
+    ((Extra *)tensor->extra)->data_device[0] = g_scratch + offset;
+}
+void ggml_cuda_set_scratch_size(size_t scratch_size) {
+    if (scratch_size > g_scratch_size) ggml_cuda_free_scratch();
+    g_scratch_size = scratch_size;
+}
+void ggml_cuda_free_scratch(void) {
+    std::lock_guard<std::mutex> g(g_mu);
+    for (Extra * e : g_graph_extras) if (e) { if (e->owned) pi_free(e->data_device[0]); e->data_device[0] = nullptr; e->owned = false; }
+    if (g_scratch) { pi_free(g_scratch); g_scratch = nullptr; }
+    g_scratch_offset = 0;
+}
+void ggml_cuda_copy_to_device(struct ggml_tensor * tensor) {
+    BK_PI(pi_memcpy_h2d(((Extra *)tensor->extra)->data_device[0], tensor->data, nbytes(tensor)));
+}
+void ggml_cuda_copy_to_host(struct ggml_tensor * tensor) {
+    BK_PI(pi_sync());
+    BK_PI(pi_memcpy_d2h(tensor->data, ((Extra *)tensor->extra)->data_device[0], nbytes(tensor)));
+}
+
+int ggml_cuda_get_device_count(void) { int n = 0; if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return 0; } return n; }
+void ggml_cuda_get_device_description(int device, char * description, size_t description_size) {
+    hipDeviceProp_t p;
+    if (hipGetDeviceProperties(&p, device) != hipSuccess) { (void)hipGetLastError(); snprintf(description, description_size, "unknown"); return; }
+    snprintf(description, description_size, "%s", p.gcnArchName);
+}
+size_t ggml_cuda_get_free_memory(int device) {
+    (void)device;
+    size_t f = 0, t = 0;
+    BK_HIP(hipMemGetInfo(&f, &t));
+    return f;
+}
+void ggml_cuda_set_device_constants(float sparse_pred_threshold) { g_threshold = sparse_pred_threshold; }
+
+bool ggml_cuda_compute_forward(struct ggml_compute_params * params, struct ggml_tensor * tensor) {
+    if (!g_loaded) return false;
+    const ggml_tensor * s0 = tensor->src[0];
+    const bool src0_on_device = s0 != nullptr && s0->backend != GGML_BACKEND_CPU;
+    const bool any_on_device = tensor->backend == GGML_BACKEND_GPU || src0_on_device || (tensor->src[1] != nullptr && tensor->src[1]->backend == GGML_BACKEND_GPU);
+    // weights not on the device: the sparse operators run on the CPU with the sparsity (ggml-cuda.cu:9226-9230)
+    if ((!src0_on_device && (tensor->op == GGML_OP_MUL_MAT_SPARSE || tensor->op == GGML_OP_AXPY)) || !any_on_device) return false;
+    switch (tensor->op) {
+        case GGML_OP_MUL_MAT: case GGML_OP_MUL_MAT_SPARSE: case GGML_OP_AXPY: case GGML_OP_ADD: case GGML_OP_MUL:
+        case GGML_OP_SCALE: case GGML_OP_RMS_NORM: case GGML_OP_NORM: case GGML_OP_SOFT_MAX: case GGML_OP_ROPE:
+        case GGML_OP_CPY: case GGML_OP_CONT: case GGML_OP_DUP: case GGML_OP_GET_ROWS:
+        case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE:
+            break;
+        case GGML_OP_UNARY:
+            if (tensor->op_params[0] != GGML_UNARY_OP_RELU) return false;
+            break;
+        default:
+            return false;
+    }
+    if (params->ith != 0) return true;
+    if (params->type == GGML_TASK_INIT || params->type == GGML_TASK_FINALIZE) return true;
+    bool ok = true;
+    switch (tensor->op) {
+        case GGML_OP_MUL_MAT:        ok = op_mul_mat(tensor); break;
+        case GGML_OP_MUL_MAT_SPARSE: ok = sparse_common(tensor, false); break;
+        case GGML_OP_AXPY:           ok = sparse_common(tensor, true); break;
+        case GGML_OP_ROPE:           ok = op_rope(tensor); break;
+        case GGML_OP_CPY: case GGML_OP_CONT: case GGML_OP_DUP: ok = op_cpy(tensor); break;
+        case GGML_OP_GET_ROWS:       ok = op_get_rows(tensor); break;
+        case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE: break;
+        default:                     ok = op_elementwise(tensor); break;
+    }
+    if (!ok) {
+        // the phase protocol has no way to hand a node back after INIT was claimed: refuse loudly rather than compute wrongly
+        fprintf(stderr, "powerinfer-hip backend: node '%s' (op %d) has a shape/type/stride this backend does not implement\n", tensor->name, (int)tensor->op);
+        exit(1);
+    }
+    if (pi::check_launch("ggml_cuda_compute_forward") != PI_OK) die("kernel launch");
+    return true;
+}
+
+ggml_backend_t ggml_backend_cuda_init(void) { return nullptr; }
+
+}  // extern "C"

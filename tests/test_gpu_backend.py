@@ -1,0 +1,127 @@
+"""The reference's backend entry points (ggml_cuda_* in include/ggml_backend_abi.h) driven the way ggml's executor
+drives them, on the op sequence llm_build_ffn_sparse emits (llama.cpp:4652-4757): full-GPU fast path and the
+hybrid CPU part + GPU part + ggml_add variant."""
+import ctypes as C
+
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from powerinfer_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(a, b):
+    return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+def build_ffn(G, L, x, wtype, full_gpu, gid=None, bucket=None):
+    """llm_build_ffn_sparse for T tokens; returns (idx, out)."""
+    d, ff, r, T = L["d"], L["ff"], L["r"], x.shape[0]
+    has_gate = L["gate"] is not None
+    t_x = G.new(0, [d, T], x, "ffn_input")
+    fc1 = G.weight_to_gpu(G.new(1, [d, r], L["fc1"], "fc1"))
+    fc2 = G.weight_to_gpu(G.new(1, [r, ff], L["fc2"], "fc2"))
+    names = ("up", "gate", "down_t") if has_gate else ("up", "down_t")
+    if full_gpu:
+        W = {n: G.weight_to_gpu(G.new(wtype, [d, ff], L[n], n + "_gpu")) for n in names}
+    else:
+        Wc = {n: G.new(wtype, [d, ff], L[n], n) for n in names}
+        Wg = {n: G.weight_to_gpu(G.new(wtype, [d, bucket.size], np.ascontiguousarray(L[n][bucket]), n + "_gpu")) for n in names}
+        t_gid = G.new(18, [ff], gid, "gpu_idx")
+        t_bkt = G.new(18, [bucket.size], bucket, "gpu_bucket")
+    idx = G.on_gpu(G.mul_mat(fc1, t_x, "mlp_pre_hidden"))
+    idx = G.on_gpu(G.relu(idx, "mlp_pre_relu"))
+    idx = G.mul_mat(fc2, idx, "mlp_pre_out")
+    if full_gpu:
+        G.on_gpu(idx)
+
+    def sparse_mm(n):
+        if full_gpu:
+            return G.on_gpu(G.mul_mat_idx(W[n], t_x, idx, None, f"ffn_{n}_sparse"))
+        cpu = G.mul_mat_idx(Wc[n], t_x, idx, t_gid, f"ffn_{n}_sparse")
+        gpu = G.on_gpu(G.mul_mat_idx_upscale(Wg[n], t_x, idx, t_bkt, ff, f"ffn_{n}_sparse_gpu"))
+        return G.add(cpu, gpu, f"ffn_{n}_sparse_merged")
+
+    up = sparse_mm("up")
+    if has_gate:
+        gate = sparse_mm("gate")
+        act = G.relu(gate, "ffn_gate_act")
+        cur = G.mul(act, up, "ffn_gate_par")
+        if full_gpu:
+            G.on_gpu(act), G.on_gpu(cur)
+    else:
+        cur = G.relu(up, "ffn_up_act")
+        if full_gpu:
+            G.on_gpu(cur)
+    if full_gpu:
+        out = G.on_gpu(G.axpy(W["down_t"], cur, idx, None, "ffn_down_sparse"))
+    else:
+        cpu = G.axpy(Wc["down_t"], cur, idx, t_gid, "ffn_down_sparse")
+        gpu = G.on_gpu(G.axpy(Wg["down_t"], cur, idx, t_bkt, "ffn_down_sparse_gpu"))
+        out = G.on_gpu(G.add(cpu, gpu, "ffn_down_sparse_merged"))
+    return idx, out
+
+
+@pytest.mark.parametrize("wtype", [ol.F16, ol.Q4_0])
+@pytest.mark.parametrize("has_gate", [True, False])
+def test_full_gpu_graph(wtype, has_gate):
+    from powerinfer_amd import lib as pl
+    from ggml_graph import Graph
+    d, ff, r, T = 1024, 4096, 128, 2
+    L = synth.make_ffn_layer(seed=61 + wtype, d=d, ff=ff, r=r, wtype=wtype, has_gate=has_gate, mean_rate=0.15, T=T)
+    G = Graph(pl.load())
+    idx, out = build_ffn(G, L, L["x"], wtype, True)
+    G.compute(0.0)
+    assert not G.cpu_run, G.cpu_run                      # every node was taken by the backend
+    o = ol.ffn_sparse(ol.oracle(), d, ff, r, T, wtype, has_gate, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], L["x"], L["x"],
+                      np.zeros(ff, np.int32), 0.0, nth=4)
+    lg = G.host(idx)
+    assert rel_err(lg, o["logits"]) < 1e-5
+    if np.array_equal(lg >= 0, o["logits"] >= 0):
+        assert rel_err(G.host(out), o["out"]) < 1e-4
+
+
+@pytest.mark.parametrize("wtype", [ol.F16, ol.Q4_0])
+def test_hybrid_graph_cpu_part_plus_gpu_part(wtype):
+    from powerinfer_amd import lib as pl
+    from ggml_graph import Graph
+    d, ff, r, T = 1024, 4096, 128, 2
+    L = synth.make_ffn_layer(seed=71, d=d, ff=ff, r=r, wtype=wtype, mean_rate=0.15, T=T)
+    gid, bucket = synth.gpu_split(L["p"], 0.6)
+    G = Graph(pl.load())
+    idx, out = build_ffn(G, L, L["x"], wtype, False, gid, bucket)
+    G.compute(0.0)
+    # weights on the CPU: the backend must hand those sparse nodes back (ggml-cuda.cu:9226-9230)
+    assert {"ffn_up_sparse", "ffn_gate_sparse", "ffn_down_sparse"} <= set(G.cpu_run)
+    assert {"ffn_up_sparse_gpu", "ffn_gate_sparse_gpu", "ffn_down_sparse_gpu", "mlp_pre_out"} <= set(G.gpu_run)
+    o = ol.ffn_sparse(ol.oracle(), d, ff, r, T, wtype, 1, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], L["x"], L["x"],
+                      np.zeros(ff, np.int32), 0.0, nth=4)
+    lg = G.host(idx)
+    assert rel_err(lg, o["logits"]) < 1e-5
+    if np.array_equal(lg >= 0, o["logits"] >= 0):
+        assert rel_err(G.host(out), o["out"]) < 1e-4
+
+
+def test_backend_info_entry_points():
+    from powerinfer_amd import lib as pl
+    L = pl.load()
+    L.ggml_init_cublas()
+    L.ggml_cublas_loaded.restype = C.c_bool
+    assert L.ggml_cublas_loaded()
+    assert L.ggml_cuda_get_device_count() >= 1
+    buf = C.create_string_buffer(128)
+    L.ggml_cuda_get_device_description.argtypes = [C.c_int, C.c_char_p, C.c_size_t]
+    L.ggml_cuda_get_device_description(0, buf, 128)
+    assert buf.value.startswith(b"gfx950")
+    L.ggml_cuda_get_free_memory.restype = C.c_size_t
+    assert L.ggml_cuda_get_free_memory(0) > (100 << 30)
+    L.ggml_cuda_host_malloc.restype = C.c_void_p
+    L.ggml_cuda_host_malloc.argtypes = [C.c_size_t]
+    L.ggml_cuda_host_free.argtypes = [C.c_void_p]
+    p = L.ggml_cuda_host_malloc(1 << 20)
+    assert p
+    L.ggml_cuda_host_free(p)
+    L.ggml_backend_cuda_init.restype = C.c_void_p
+    assert L.ggml_backend_cuda_init() is None

@@ -246,3 +246,114 @@ REF_API void ref_init(void) {
     struct ggml_context * ctx = ggml_init(ip);   /* fills the fp16 / exp lookup tables */
     ggml_free(ctx);
 }
+
+#ifdef GGML_USE_CUBLAS
+/*
+ * The same FFN block, but with the reference compiled with -DGGML_USE_CUBLAS and linked against THIS repository's
+ * backend library in place of ggml-cuda.cu: the reference's own op constructors, graph and executor
+ * (ggml_graph_compute, two threads, as the hybrid ops require: ggml.c:16714-16720) drive the HIP kernels through
+ * ggml_cuda_compute_forward.  Graph as llm_build_ffn_sparse builds it under GGML_USE_CUBLAS (llama.cpp:4546-4757):
+ *   n_bucket == 0 : full-GPU fast path, every FFN tensor and node on the GPU (src[3] == NULL);
+ *   n_bucket  > 0 : hybrid, CPU part (full matrices, gpu_idx) + GPU part (bucket rows, gpu_bucket) + ggml_add.
+ */
+#include "ggml-cuda.h"
+
+static struct ggml_tensor * to_gpu(struct ggml_tensor * t) {
+    t->backend = GGML_BACKEND_GPU;
+    ggml_cuda_transform_tensor(t->data, t);
+    return t;
+}
+static struct ggml_tensor * node_gpu(struct ggml_tensor * t) { ggml_cuda_assign_buffers_no_scratch(t); return t; }
+
+static struct ggml_tensor * sparse_mm(struct ggml_context * ctx, struct ggml_tensor * w, struct ggml_tensor * w_gpu, struct ggml_tensor * x,
+                                      struct ggml_tensor * idx, struct ggml_tensor * gid, struct ggml_tensor * bkt, int full_gpu) {
+    if (full_gpu) return node_gpu(ggml_mul_mat_idx(ctx, w_gpu, x, idx, NULL));
+    struct ggml_tensor * out = ggml_mul_mat_idx(ctx, w, x, idx, gid);
+    struct ggml_tensor * out_gpu = node_gpu(ggml_mul_mat_idx_upscale(ctx, w_gpu, x, idx, bkt, out->ne[0]));
+    return ggml_add(ctx, out, out_gpu);
+}
+
+static void * gather_rows(const void * w, size_t rb, const int32_t * bucket, int n) {
+    char * p = (char *)malloc(rb * (size_t)(n ? n : 1));
+    for (int i = 0; i < n; ++i) memcpy(p + rb * i, (const char *)w + rb * (size_t)bucket[i], rb);
+    return p;
+}
+
+REF_API int ref_ffn_sparse_gpu(int d, int ff, int r, int T, int wtype, int has_gate,
+                               const void * up_w, const void * gate_w, const void * down_t,
+                               const uint16_t * fc1, const uint16_t * fc2,
+                               const float * x_ffn, const float * x_pred,
+                               const int32_t * gpu_idx, const int32_t * gpu_bucket, int n_bucket,
+                               float threshold, float * logits, float * out) {
+    enum ggml_type wt = (enum ggml_type) wtype;
+    const int full_gpu = n_bucket == 0;
+    const size_t rb = tensor_bytes(wt, d, 1);
+    size_t payload = 6 * tensor_bytes(wt, d, ff) + 2u * ((size_t)d * r + (size_t)r * ff)
+                   + (size_t)T * (2u * d + 16u * ff + 2u * r) * sizeof(float) + (size_t)ff * 8 + (size_t)d * 256 + (16u << 20);
+    struct ggml_context * ctx = new_ctx(payload);
+    if (!ctx) return 1;
+    sparse_pred_threshold = threshold;
+    ggml_cuda_set_device_constants(threshold);
+
+    struct ggml_tensor * t_fc1 = to_gpu(put2d(ctx, GGML_TYPE_F16, d, r, fc1));
+    struct ggml_tensor * t_fc2 = to_gpu(put2d(ctx, GGML_TYPE_F16, r, ff, fc2));
+    struct ggml_tensor * t_x   = put2d(ctx, GGML_TYPE_F32, d, T, x_ffn);
+    struct ggml_tensor * t_xp  = put2d(ctx, GGML_TYPE_F32, d, T, x_pred);
+    struct ggml_tensor *up = NULL, *gate = NULL, *down = NULL, *up_g, *gate_g = NULL, *down_g, *gid = NULL, *bkt = NULL;
+    void * tmp[3] = {NULL, NULL, NULL};
+    if (full_gpu) {
+        up_g = to_gpu(put2d(ctx, wt, d, ff, up_w));
+        if (has_gate) gate_g = to_gpu(put2d(ctx, wt, d, ff, gate_w));
+        down_g = to_gpu(put2d(ctx, wt, d, ff, down_t));
+    } else {
+        up = put2d(ctx, wt, d, ff, up_w); down = put2d(ctx, wt, d, ff, down_t);
+        if (has_gate) gate = put2d(ctx, wt, d, ff, gate_w);
+        tmp[0] = gather_rows(up_w, rb, gpu_bucket, n_bucket);   up_g   = to_gpu(put2d(ctx, wt, d, n_bucket, tmp[0]));
+        tmp[1] = gather_rows(down_t, rb, gpu_bucket, n_bucket); down_g = to_gpu(put2d(ctx, wt, d, n_bucket, tmp[1]));
+        if (has_gate) { tmp[2] = gather_rows(gate_w, rb, gpu_bucket, n_bucket); gate_g = to_gpu(put2d(ctx, wt, d, n_bucket, tmp[2])); }
+        gid = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, ff);       memcpy(gid->data, gpu_idx, (size_t)ff * 4);
+        bkt = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, n_bucket); memcpy(bkt->data, gpu_bucket, (size_t)n_bucket * 4);
+    }
+
+    struct ggml_tensor * idx = node_gpu(ggml_mul_mat(ctx, t_fc1, t_xp));
+    idx = node_gpu(ggml_relu(ctx, idx));
+    idx = ggml_mul_mat(ctx, t_fc2, idx);
+    if (full_gpu) node_gpu(idx);                                 /* hybrid: the sparsity index stays on the CPU (llama.cpp:4693-4695) */
+
+    struct ggml_tensor * upo = sparse_mm(ctx, up, up_g, t_x, idx, gid, bkt, full_gpu);
+    struct ggml_tensor * cur;
+    if (has_gate) {
+        struct ggml_tensor * gto = sparse_mm(ctx, gate, gate_g, t_x, idx, gid, bkt, full_gpu);
+        struct ggml_tensor * act = ggml_relu(ctx, gto);
+        cur = ggml_mul(ctx, act, upo);
+        if (full_gpu) { node_gpu(act); node_gpu(cur); }
+    } else {
+        cur = ggml_relu(ctx, upo);
+        if (full_gpu) node_gpu(cur);
+    }
+    struct ggml_tensor * res;
+    if (full_gpu) {
+        res = node_gpu(ggml_axpy(ctx, down_g, cur, idx, NULL));
+    } else {
+        struct ggml_tensor * o_cpu = ggml_axpy(ctx, down, cur, idx, gid);
+        struct ggml_tensor * o_gpu = node_gpu(ggml_axpy(ctx, down_g, cur, idx, bkt));
+        res = node_gpu(ggml_add(ctx, o_cpu, o_gpu));
+    }
+
+    struct ggml_cgraph * gf = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, res);
+    ggml_graph_compute_with_ctx(ctx, gf, 2);
+
+    if (idx->backend == GGML_BACKEND_GPU) ggml_cuda_copy_to_host(idx);
+    ggml_cuda_copy_to_host(res);
+    if (logits) memcpy(logits, idx->data, (size_t)ff * T * 4);
+    if (out)    memcpy(out, res->data, (size_t)d * T * 4);
+
+    struct ggml_tensor * owned[] = {t_fc1, t_fc2, up_g, gate_g, down_g};
+    for (int i = 0; i < 5; ++i) if (owned[i]) ggml_cuda_free_data(owned[i]);
+    ggml_cuda_free_scratch();
+    for (int i = 0; i < 3; ++i) free(tmp[i]);
+    ggml_free(ctx);
+    return 0;
+}
+#endif

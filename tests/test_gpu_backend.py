@@ -125,3 +125,34 @@ def test_backend_info_entry_points():
     L.ggml_cuda_host_free(p)
     L.ggml_backend_cuda_init.restype = C.c_void_p
     assert L.ggml_backend_cuda_init() is None
+
+
+@pytest.mark.parametrize("wtype", [ol.F16, ol.Q4_0])
+@pytest.mark.parametrize("hot_frac", [1.0, 0.6])
+def test_reference_executor_drives_this_backend(wtype, hot_frac):
+    """Drop-in check of the boundary: oracle/_ref/libpi_ref_gpu.so is the REFERENCE's ggml.c compiled with
+    -DGGML_USE_CUBLAS and linked against libpowerinfer_hip.so in place of ggml-cuda.cu.  Its own op constructors,
+    graph and two-thread executor run llm_build_ffn_sparse's op sequence (full-GPU, and hybrid CPU part + GPU part
+    + ggml_add); the result must equal the CPU path computing every neuron."""
+    import os
+    so = os.path.join(ol.ODIR, "_ref", "libpi_ref_gpu.so")
+    if not os.path.exists(so):
+        pytest.skip("oracle/_ref/libpi_ref_gpu.so was not built (needs the reference tree at build time)")
+    R = C.CDLL(so)
+    vp, i, f = C.c_void_p, C.c_int, C.c_float
+    R.ref_ffn_sparse_gpu.argtypes = [i] * 6 + [vp] * 9 + [i, f, vp, vp]
+    R.ref_init()
+    d, ff, r, T = 1024, 4096, 128, 2
+    L = synth.make_ffn_layer(seed=81 + wtype, d=d, ff=ff, r=r, wtype=wtype, mean_rate=0.15, T=T)
+    gid, bucket = synth.gpu_split(L["p"], hot_frac)
+    n_bucket = 0 if hot_frac >= 1.0 else bucket.size
+    lg, out = np.zeros((T, ff), np.float32), np.zeros((T, d), np.float32)
+    P = ol._ptr
+    rc = R.ref_ffn_sparse_gpu(d, ff, r, T, wtype, 1, P(L["up"]), P(L["gate"]), P(L["down_t"]), P(L["fc1"]), P(L["fc2"]), P(L["x"]), P(L["x"]),
+                              P(gid), P(bucket), n_bucket, 0.0, P(lg), P(out))
+    assert rc == 0
+    o = ol.ffn_sparse(ol.oracle(), d, ff, r, T, wtype, 1, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], L["x"], L["x"],
+                      np.zeros(ff, np.int32), 0.0, nth=4)
+    assert rel_err(lg, o["logits"]) < 1e-5
+    if np.array_equal(lg >= 0, o["logits"] >= 0):
+        assert rel_err(out, o["out"]) < 1e-4

@@ -9,9 +9,10 @@
  *
  * How each function is pinned (tests/test_oracle_*.py): against golden vectors produced by the
  * compiled reference (oracle/_ref, tests/golden/), against numpy.float16 / closed forms, and
- * against dense fp64 matmul with an all-true mask.  pio_model_eval is pinned at the model level
- * only through fixtures produced by the compiled reference's ops assembled by
- * oracle/ref_harness.c; its graph wiring (llama.cpp:4949-5084, 5326-5468) is a restatement.
+ * against dense fp64 matmul with an all-true mask.  pio_model_eval (the graph wiring of
+ * llama.cpp:4949-5084, 5326-5468) is pinned by greedy tokens and logits that the reference's own
+ * llama.cpp CPU path produced on synthetic PowerInfer GGUF files (tests/golden/ref_*.npz,
+ * LLaMA F16, LLaMA Q4_0, Falcon F16 with grouped KV heads), to 1e-5 of the logit range.
  */
 #include "pi_oracle.h"
 

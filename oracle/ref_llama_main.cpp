@@ -1,0 +1,54 @@
+// TEST INFRASTRUCTURE ONLY.  A minimal driver around the reference's own llama.cpp (CPU-only build): loads a
+// PowerInfer GGUF, feeds the given tokens one llama_decode at a time, then continues greedily, and dumps for
+// every step the token consumed, the greedy choice and the full logits.  Built by oracle/Makefile into
+// oracle/_ref/ref_llama from the reference sources where they lie; used by tests/golden/make_llama_fixture.py.
+//
+//   ref_llama <model.gguf> <n_ctx> <n_threads> <n_generate> <out.bin> tok0 tok1 ...
+#include "llama.h"
+
+#include <cstdio>
+#include <cstdlib>
+#include <vector>
+
+int main(int argc, char ** argv) {
+    if (argc < 7) { fprintf(stderr, "usage: %s model n_ctx n_threads n_generate out.bin tok...\n", argv[0]); return 2; }
+    const char * path = argv[1];
+    const int n_ctx = atoi(argv[2]), n_threads = atoi(argv[3]), n_gen = atoi(argv[4]);
+    const char * out_path = argv[5];
+    std::vector<llama_token> prompt;
+    for (int i = 6; i < argc; ++i) prompt.push_back(atoi(argv[i]));
+
+    llama_backend_init(false);
+    llama_model_params mp = llama_model_default_params();
+    mp.n_gpu_layers = 0;
+    llama_model * model = llama_load_model_from_file(path, mp);
+    if (!model) { fprintf(stderr, "failed to load %s\n", path); return 1; }
+    llama_context_params cp = llama_context_default_params();
+    cp.seed = 1; cp.n_ctx = n_ctx; cp.n_batch = 512; cp.n_threads = n_threads; cp.n_threads_batch = n_threads;
+    llama_context * ctx = llama_new_context_with_model(model, cp);
+    if (!ctx) { fprintf(stderr, "failed to create context\n"); return 1; }
+    const int n_vocab = llama_n_vocab(model);
+
+    FILE * f = fopen(out_path, "wb");
+    if (!f) return 1;
+    const int n_steps = (int)prompt.size() + n_gen;
+    int32_t hdr[2] = { n_steps, n_vocab };
+    fwrite(hdr, 4, 2, f);
+    llama_token tok = prompt[0];
+    for (int s = 0; s < n_steps; ++s) {
+        if (s < (int)prompt.size()) tok = prompt[s];
+        if (llama_decode(ctx, llama_batch_get_one(&tok, 1, s, 0)) != 0) { fprintf(stderr, "llama_decode failed at step %d\n", s); return 1; }
+        const float * lg = llama_get_logits(ctx);
+        int best = 0;
+        for (int i = 1; i < n_vocab; ++i) if (lg[i] > lg[best]) best = i;
+        int32_t rec[2] = { tok, best };
+        fwrite(rec, 4, 2, f);
+        fwrite(lg, 4, n_vocab, f);
+        tok = best;
+    }
+    fclose(f);
+    llama_free(ctx);
+    llama_free_model(model);
+    llama_backend_free();
+    return 0;
+}

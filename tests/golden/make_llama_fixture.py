@@ -1,0 +1,76 @@
+"""Model-level golden vectors from the REFERENCE's own llama.cpp CPU path (oracle/_ref/ref_llama = llama.cpp + ggml
+compiled from /root/reference by oracle/Makefile): a synthetic PowerInfer GGUF ("PWRI" magic, tokenizer entries taken
+from the reference's models/ggml-vocab-*.gguf data files) is written to a temporary directory, evaluated token by
+token with one thread, and the greedy tokens plus a fixed sample of the logits of every step are stored.
+The model itself is regenerated from its seed by powerinfer_amd.synth (a hash of the tensors guards the stream).
+
+    python tests/golden/make_llama_fixture.py
+"""
+import hashlib
+import os
+import subprocess
+import sys
+import tempfile
+
+import numpy as np
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+ROOT = os.path.dirname(os.path.dirname(HERE))
+sys.path.insert(0, ROOT)
+from powerinfer_amd import gguf, synth  # noqa: E402
+
+REF = "/root/reference"
+BIN = os.path.join(ROOT, "oracle", "_ref", "ref_llama")
+
+CASES = {
+    "llama_f16": dict(base="llama-tiny", vocab="ggml-vocab-llama.gguf", over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=4, n_head_kv=4, n_layer=2, n_vocab=32000, n_ctx=64, seed=21)),
+    "llama_q4": dict(base="llama-tiny", vocab="ggml-vocab-llama.gguf", over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=4, n_head_kv=4, n_layer=2, n_vocab=32000, n_ctx=64, seed=22, wtype=synth.Q4_0)),
+    "falcon_f16": dict(base="falcon-tiny", vocab="ggml-vocab-falcon.gguf", over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=8, n_head_kv=2, n_layer=2, n_vocab=65024, n_ctx=64, seed=23)),
+}
+
+
+def model_sha(model):
+    h = hashlib.sha256()
+    for a in model["glob"].values():
+        h.update(np.ascontiguousarray(a).tobytes())
+    for L in model["layers"]:
+        for k in sorted(L):
+            if L[k] is not None and k != "p":
+                h.update(np.ascontiguousarray(L[k]).tobytes())
+    return np.frombuffer(h.digest(), np.uint8)
+
+
+def case_model(name):
+    c = CASES[name]
+    hp = synth.hparams(c["base"], **c["over"])
+    return hp, synth.make_model(hp)
+
+
+def main():
+    for name, c in CASES.items():
+        hp, model = case_model(name)
+        _, vkv, _ = gguf.read_gguf(os.path.join(REF, "models", c["vocab"]))
+        tok_kv = {k: v for k, v in vkv.items() if k.startswith("tokenizer.")}
+        assert len(tok_kv["tokenizer.ggml.tokens"][1][1]) == hp.n_vocab
+        prompt = np.random.default_rng(hp.seed).integers(0, hp.n_vocab, 6)
+        n_gen = 10
+        with tempfile.TemporaryDirectory() as td:
+            path, out = os.path.join(td, "m.powerinfer.gguf"), os.path.join(td, "out.bin")
+            gguf.write_model(path, model, tok_kv)
+            subprocess.check_call([BIN, path, str(hp.n_ctx), "1", str(n_gen), out] + [str(int(t)) for t in prompt],
+                                  stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+            raw = np.fromfile(out, np.uint8)
+        n_steps, n_vocab = raw[:8].view(np.int32)
+        rec = raw[8:].reshape(n_steps, 8 + 4 * n_vocab)
+        consumed = rec[:, :4].copy().view(np.int32)[:, 0]
+        greedy = rec[:, 4:8].copy().view(np.int32)[:, 0]
+        logits = rec[:, 8:].copy().view(np.float32)
+        sample = np.sort(np.random.default_rng(1).choice(n_vocab, 1024, replace=False)).astype(np.int32)
+        np.savez_compressed(os.path.join(HERE, f"ref_{name}.npz"), prompt=prompt.astype(np.int32), consumed=consumed, greedy=greedy,
+                            sample_idx=sample, logits_sample=logits[:, sample], logits_max=logits.max(1), logits_absmax=np.abs(logits).max(1),
+                            model_sha=model_sha(model))
+        print(name, "greedy", greedy.tolist())
+
+
+if __name__ == "__main__":
+    main()

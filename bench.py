@@ -219,7 +219,7 @@ def main():
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_f16_kernel<4,2,0> (q|k|v projection, 12288 x 4096 fp16, fused RMSNorm)",
+            "kernel": "gemv_f16_reg_kernel<8,2> (q|k|v projection, 12288 x 4096 fp16, fused RMSNorm)",
             "achieved": round(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",

@@ -141,6 +141,42 @@ PI_API int pi_k_sparse_axpy(int wtype, const void * down_t, int cols, int n_rows
                             pi_workspace * ws, pi_stream_t stream);
 
 /*
+ * Full-GPU F16 fast route of the sparse FFN: predictor fc2, the activity test and the sparse up/gate mat-vec in
+ * ONE launch, and the down projection straight from the dense h vector in a second one.  Replaces the
+ * mul_mat(fc2) -> dequantize_mul_mat_vec_sparse x2 -> relu -> mul chain of llm_build_ffn_sparse
+ * (llama.cpp:4688-4740; ggml-cuda.cu:4349, 4685) and dequantize_mul_mat_axpy_sparse (ggml-cuda.cu:4541).
+ *   pi_k_pred_upgate: a workgroup owns 32 consecutive neurons: logits[n] = fc2[n] . fp16(hidden), active iff
+ *     !(logit < threshold), h_dense[n] = relu(gate[n] . xn) * (up[n] . xn) for active n (relu(up[n] . xn) when
+ *     gate == NULL) and 0 otherwise, xn = fp16(norm(x)).  Writes all ff entries of h_dense, the mask words of
+ *     the workspace and, if logits != NULL, the ff predictor logits.  Shapes: see pi_k_pred_upgate_supported.
+ *   pi_k_sparse_axpy_dense: out[cols] = epi( sum over n with fp16(h_dense[n]) != 0 of fp16(h_dense[n]) *
+ *     down_t[n][:] ), ascending n within a fixed reduction tree; cols % 64 == 0.  If n_active != NULL it
+ *     receives the number of set bits in the workspace's mask words (the predictor's active count).
+ */
+/*
+ * The same block in its tightest form (what the F16 decode loop runs at cols == 4096): one launch computes fc2, the
+ * activity test, gate/up, h and each workgroup's share of the down projection; a small second launch adds the
+ * per-workgroup partial vectors in a fixed order plus the residual(s):
+ *   out[cols] = epi( sum_n fp16(h[n]) * down_t[n][:] ),  h[n] as for pi_k_pred_upgate.
+ * logits (fp32 [ff]), h_dense (fp32 [ff], every entry written) and n_active (predictor's active count) are
+ * optional outputs for inspection.  Shapes: see pi_k_sparse_ffn_supported.
+ */
+PI_API int pi_k_sparse_ffn_supported(int ff, int r, int cols);
+PI_API int pi_k_sparse_ffn(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                           const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols,
+                           const float * x, const pi_norm * norm,
+                           int epilogue, const float * add1, const float * add2, float * out,
+                           float * logits, float * h_dense, int32_t * n_active,
+                           pi_workspace * ws, pi_stream_t stream);
+PI_API int pi_k_pred_upgate_supported(int ff, int r, int cols);      /* 1 if the fused kernel covers the shape */
+PI_API int pi_k_pred_upgate(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                            const void * up_f16, const void * gate_f16, int cols, const float * x, const pi_norm * norm,
+                            float * logits, float * h_dense, pi_workspace * ws, pi_stream_t stream);
+PI_API int pi_k_sparse_axpy_dense(const void * down_t_f16, int cols, int ff, const float * h_dense, int32_t * n_active,
+                                  int epilogue, const float * add1, const float * add2, float * out,
+                                  pi_workspace * ws, pi_stream_t stream);
+
+/*
  * RoPE on q and k of one token plus the KV-cache store (rope / rope_neox ggml-cuda.cu:4999,5027 and
  * cpy_f32_f16 :4944 for llm_build_kv_store, llama.cpp:4383).  qkv: fp32 [n_head*hd + 2*n_head_kv*hd]
  * (q | k | v).  mode 0 = adjacent pairs, 2 = NeoX halves.  The position is read from *pos (device).

@@ -12,15 +12,47 @@
 struct __attribute__((packed)) pi_block_q4_0 { uint16_t d; uint8_t qs[16]; };
 static_assert(sizeof(pi_block_q4_0) == 18, "q4_0 block is 18 bytes");
 
+// Wave-wide reductions through DPP (data-parallel primitives: lane permutations inside the VALU, no LDS
+// crossbar round trip): pairs, quads, half rows and rows by quad_perm / row_half_mirror / row_mirror, then the
+// last lane of row 0 (2) is added into row 1 (3) and lane 31 into rows 2-3, so lane 63 holds the total, which
+// v_readlane hands to every lane.  The association order is fixed, so results are reproducible.
+#define PI_DPP_XOR1        0xB1    /* quad_perm [1,0,3,2] */
+#define PI_DPP_XOR2        0x4E    /* quad_perm [2,3,0,1] */
+#define PI_DPP_HALF_MIRROR 0x141
+#define PI_DPP_MIRROR      0x140
+#define PI_DPP_BCAST15     0x142
+#define PI_DPP_BCAST31     0x143
+
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ int pi_dpp_i32(int v) {
+    return __builtin_amdgcn_update_dpp(0, v, CTRL, ROW_MASK, 0xF, false);
+}
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ float pi_dpp_f32(float v) {
+    return __int_as_float(pi_dpp_i32<CTRL, ROW_MASK>(__float_as_int(v)));
+}
+template <int CTRL, int ROW_MASK> __device__ __forceinline__ double pi_dpp_f64(double v) {
+    const long long b = __double_as_longlong(v);
+    const int lo = pi_dpp_i32<CTRL, ROW_MASK>((int)(b & 0xffffffffll)), hi = pi_dpp_i32<CTRL, ROW_MASK>((int)(b >> 32));
+    return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
+}
 __device__ __forceinline__ float pi_wave_sum(float v) {
-#pragma unroll
-    for (int o = PI_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, PI_WAVE);
-    return v;
+    v += pi_dpp_f32<PI_DPP_XOR1, 0xF>(v);
+    v += pi_dpp_f32<PI_DPP_XOR2, 0xF>(v);
+    v += pi_dpp_f32<PI_DPP_HALF_MIRROR, 0xF>(v);
+    v += pi_dpp_f32<PI_DPP_MIRROR, 0xF>(v);
+    v += pi_dpp_f32<PI_DPP_BCAST15, 0xA>(v);
+    v += pi_dpp_f32<PI_DPP_BCAST31, 0xC>(v);
+    return __int_as_float(__builtin_amdgcn_readlane(__float_as_int(v), 63));
 }
 __device__ __forceinline__ double pi_wave_sum_f64(double v) {
-#pragma unroll
-    for (int o = PI_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, PI_WAVE);
-    return v;
+    v += pi_dpp_f64<PI_DPP_XOR1, 0xF>(v);
+    v += pi_dpp_f64<PI_DPP_XOR2, 0xF>(v);
+    v += pi_dpp_f64<PI_DPP_HALF_MIRROR, 0xF>(v);
+    v += pi_dpp_f64<PI_DPP_MIRROR, 0xF>(v);
+    v += pi_dpp_f64<PI_DPP_BCAST15, 0xA>(v);
+    v += pi_dpp_f64<PI_DPP_BCAST31, 0xC>(v);
+    const long long b = __double_as_longlong(v);
+    const int lo = __builtin_amdgcn_readlane((int)(b & 0xffffffffll), 63), hi = __builtin_amdgcn_readlane((int)(b >> 32), 63);
+    return __longlong_as_double(((long long)hi << 32) | (unsigned int)lo);
 }
 __device__ __forceinline__ float pi_wave_max(float v) {
 #pragma unroll
@@ -28,9 +60,13 @@ __device__ __forceinline__ float pi_wave_max(float v) {
     return v;
 }
 __device__ __forceinline__ int pi_wave_sum_i32(int v) {
-#pragma unroll
-    for (int o = PI_WAVE / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, PI_WAVE);
-    return v;
+    v += pi_dpp_i32<PI_DPP_XOR1, 0xF>(v);
+    v += pi_dpp_i32<PI_DPP_XOR2, 0xF>(v);
+    v += pi_dpp_i32<PI_DPP_HALF_MIRROR, 0xF>(v);
+    v += pi_dpp_i32<PI_DPP_MIRROR, 0xF>(v);
+    v += pi_dpp_i32<PI_DPP_BCAST15, 0xA>(v);
+    v += pi_dpp_i32<PI_DPP_BCAST31, 0xC>(v);
+    return __builtin_amdgcn_readlane(v, 63);
 }
 
 // round-to-nearest-even through binary16, the rounding the CPU path applies to activations
@@ -53,6 +89,18 @@ __device__ __forceinline__ float pi_dot8(const pi_u32x4 & w, const float * x, fl
     pi_unpack8(w, wf);
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc = fmaf(wf[i], x[i], acc);
+    return acc;
+}
+
+// the same with the activations still packed as 8 fp16: both widenings fold into the mixed-precision FMA
+__device__ __forceinline__ float pi_dot8h(const pi_u32x4 & w, const pi_u32x4 & x, float acc) {
+    const __half2 * a = reinterpret_cast<const __half2 *>(&w);
+    const __half2 * b = reinterpret_cast<const __half2 *>(&x);
+#pragma unroll
+    for (int i = 0; i < 4; ++i) {
+        acc = fmaf(__low2float(a[i]), __low2float(b[i]), acc);
+        acc = fmaf(__high2float(a[i]), __high2float(b[i]), acc);
+    }
     return acc;
 }
 

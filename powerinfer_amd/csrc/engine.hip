@@ -143,6 +143,28 @@ int layer_forward(pi_model * m, int il, bool last_token) {
 
     // predictor
     PI_TRY(pi_k_gemv(fc1.type, fc1.dev, r, d, pred_in, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, st));
+    if (!layer_hybrid && !q4 && pi_k_sparse_ffn_supported(ff, r, d)) {
+        // one launch for fc2 + mask + gate/up + each workgroup's share of the down projection, one small reduction
+        const void * gp = falcon ? nullptr : gate.dev;
+        if (m->capture && last_token) {
+            float * ffo = m->cap_ffn + (size_t)il * d;
+            PI_TRY(pi_k_sparse_ffn(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, gp, down.dev, d, ffn_in, &fn,
+                                   PI_EPI_NONE, nullptr, nullptr, ffo, m->pred_logits, nullptr, n_act, m->ws, st));
+            PI_HIP_TRY(hipMemcpyAsync(m->x2, ffo, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
+            PI_TRY(pi::add_vec(m->x2, falcon ? m->attn_out : m->ffn_inp, d, st));
+            if (falcon) PI_TRY(pi::add_vec(m->x2, x, d, st));
+            PI_HIP_TRY(hipMemcpyAsync(m->cap_logits + (size_t)il * ff, m->pred_logits, sizeof(float) * ff, hipMemcpyDeviceToDevice, st));
+            PI_HIP_TRY(hipMemcpyAsync(m->cap_src + (size_t)il * d, ffn_in, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
+        } else if (!falcon) {
+            PI_TRY(pi_k_sparse_ffn(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, gp, down.dev, d, ffn_in, &fn,
+                                   PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, nullptr, nullptr, n_act, m->ws, st));
+        } else {
+            PI_TRY(pi_k_sparse_ffn(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, gp, down.dev, d, ffn_in, &fn,
+                                   PI_EPI_ADD2, m->attn_out, x, m->x2, nullptr, nullptr, n_act, m->ws, st));
+        }
+        std::swap(m->x, m->x2);
+        return PI_OK;
+    }
     // F16 layers that live entirely on the GPU take the fused route: the up/gate kernel reads the mask words itself
     const bool fused = !layer_hybrid && !q4;
     const int n_rows = layer_hybrid ? n_bucket : ff;
@@ -478,6 +500,12 @@ int pi_model_time_section(pi_model * m, int section, int rounds, float * ms_tota
                 pi_norm fn = falcon ? make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B))
                                     : make_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
                 PI_TRY(pi_k_gemv(fc1.type, fc1.dev, (int)fc1.ne1, d, m->ffn_inp, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, st));
+                if (!q4 && pi_k_sparse_ffn_supported(ff, (int)fc1.ne1, d)) {
+                    PI_TRY(pi_k_sparse_ffn(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, down.dev, d,
+                                           m->ffn_inp, &fn, PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, nullptr, nullptr, m->n_active + il, m->ws, st));
+                    ++n;
+                    continue;
+                }
                 PI_TRY(pi_k_predictor_fc2(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, nullptr, 0, m->pred_logits,
                                           q4 ? m->list : nullptr, q4 ? m->n_active + il : nullptr, q4 ? m->h_dense : nullptr, m->ws, st));
                 PI_TRY(pi_k_sparse_upgate(up.type, up.dev, falcon ? nullptr : gate.dev, d, ff, m->ffn_inp, &fn, q4 ? 0 : 1, m->list, m->n_active + il, nullptr, m->h_c,

@@ -363,11 +363,7 @@ __global__ __launch_bounds__(kBlock) void gemv_f16_reg_kernel(const __half * __r
             if (rr < rows) {
                 float acc = 0.0f;
 #pragma unroll
-                for (int j = 0; j < NCH; ++j) {
-                    float xf[8];
-                    pi_unpack8(xr[j], xf);
-                    acc = pi_dot8(buf[b][j], xf, acc);
-                }
+                for (int j = 0; j < NCH; ++j) acc = pi_dot8h(buf[b][j], xr[j], acc);
                 acc = pi_wave_sum(acc);
                 if (epi == PI_EPI_RELU) acc = fmaxf(acc, 0.0f);
                 else if (epi == PI_EPI_ADD) acc = __fadd_rn(acc, r1[b]);
@@ -595,6 +591,421 @@ __global__ __launch_bounds__(kBlock) void pred_fc2_kernel(const __half * __restr
         const unsigned long long m = __ballot(act);
         if (lane == 0) words[blockIdx.x] = (uint32_t)m;
     }
+}
+
+__device__ __forceinline__ int select_nth_bit(uint32_t bits, int n);
+
+// ---------------------------------------------------------------------------------------------------
+// Predictor fc2 + activity test + sparse up/gate in one kernel (F16, cols == 512*NCH, r == 512*RCH).
+// A workgroup owns 32 consecutive neurons.  Phase A: its four waves compute the 32 predictor logits (8 rows
+// each, all loads issued at once); while those are in flight every wave loads the FFN input, normalises it
+// and keeps it as packed fp16 in registers.  Phase B: the 32 logits meet in LDS, every wave derives the same
+// 32-bit activity word, and wave w takes the w-th, (w+4)-th ... set bit, two neurons per round trip (gate row
+// + up row each).  The workgroup writes h for all of its 32 neurons (0 where inactive), the activity word and
+// the logits; nothing crosses workgroups, so neither a compaction pass nor a second launch sits between
+// predictor and FFN.  Neurons fire independently of their index, so a workgroup sees about ff*rate/32*...
+// a handful of active rows and finishes phase B in one round trip almost always.
+// ---------------------------------------------------------------------------------------------------
+template <int NCH, int RCH>
+__global__ __launch_bounds__(kBlock) void pred_upgate_f16_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
+                                                                 const __half * __restrict__ Wup, const __half * __restrict__ Wgate,
+                                                                 const float * __restrict__ x, NormArgs na, float thr,
+                                                                 float * __restrict__ logits, uint32_t * __restrict__ words, float * __restrict__ h_dense) {
+    constexpr int cols = NCH * 512, r = RCH * 512;
+    __shared__ float lg[32];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n0 = blockIdx.x * 32;
+
+    // ---- phase A loads: 8 predictor rows per wave, the hidden vector, the FFN input ---------------------
+    pi_u32x4 a[8][RCH];
+#pragma unroll
+    for (int i = 0; i < 8; ++i)
+#pragma unroll
+        for (int j = 0; j < RCH; ++j) a[i][j] = pi_ld_stream(W2 + (size_t)(n0 + wave * 8 + i) * r + (j * PI_WAVE + lane) * 8);
+    float4 hv[RCH][2], xv[NCH][2];
+#pragma unroll
+    for (int j = 0; j < RCH; ++j) {
+        hv[j][0] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8);
+        hv[j][1] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8 + 4);
+    }
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) {
+        xv[j][0] = *reinterpret_cast<const float4 *>(x + j * 512 + lane * 8);
+        xv[j][1] = *reinterpret_cast<const float4 *>(x + j * 512 + lane * 8 + 4);
+    }
+    // ---- logits ------------------------------------------------------------------------------------------
+    {
+        float hf[RCH][8];
+#pragma unroll
+        for (int j = 0; j < RCH; ++j) {       // the CPU path rounds the hidden vector to fp16 before the dot (ggml.c:9703-9716)
+            hf[j][0] = pi_round_f16(hv[j][0].x); hf[j][1] = pi_round_f16(hv[j][0].y); hf[j][2] = pi_round_f16(hv[j][0].z); hf[j][3] = pi_round_f16(hv[j][0].w);
+            hf[j][4] = pi_round_f16(hv[j][1].x); hf[j][5] = pi_round_f16(hv[j][1].y); hf[j][6] = pi_round_f16(hv[j][1].z); hf[j][7] = pi_round_f16(hv[j][1].w);
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < RCH; ++j) acc = pi_dot8(a[i][j], hf[j], acc);
+            acc = pi_wave_sum(acc);
+            if (lane == 0) lg[wave * 8 + i] = acc;
+        }
+    }
+    // ---- FFN input: norm, round to fp16, keep in registers --------------------------------------------
+    pi_u32x4 xr[NCH];
+    {
+        const bool has_w = na.kind != 0 && na.w != nullptr;
+        float4 wv[NCH][2];
+        if (has_w) {
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+                wv[j][0] = *reinterpret_cast<const float4 *>(na.w + j * 512 + lane * 8);
+                wv[j][1] = *reinterpret_cast<const float4 *>(na.w + j * 512 + lane * 8 + 4);
+            }
+        }
+        float mean = 0.0f, scale = 1.0f;
+        if (na.kind == 1) {
+            double s = 0.0;
+#pragma unroll
+            for (int j = 0; j < NCH; ++j)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const float4 v = xv[j][h];
+                    s += (double)__fmul_rn(v.x, v.x); s += (double)__fmul_rn(v.y, v.y); s += (double)__fmul_rn(v.z, v.z); s += (double)__fmul_rn(v.w, v.w);
+                }
+            s = pi_wave_sum_f64(s);
+            scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
+        } else if (na.kind == 2) {
+            double s = 0.0;
+#pragma unroll
+            for (int j = 0; j < NCH; ++j)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) { const float4 v = xv[j][h]; s += (double)v.x; s += (double)v.y; s += (double)v.z; s += (double)v.w; }
+            s = pi_wave_sum_f64(s);
+            mean = (float)(s / cols);
+            double s2 = 0.0;
+#pragma unroll
+            for (int j = 0; j < NCH; ++j)
+#pragma unroll
+                for (int h = 0; h < 2; ++h) {
+                    const float4 v = xv[j][h];
+                    const float p = __fsub_rn(v.x, mean), q = __fsub_rn(v.y, mean), c = __fsub_rn(v.z, mean), e = __fsub_rn(v.w, mean);
+                    s2 += (double)__fmul_rn(p, p); s2 += (double)__fmul_rn(q, q); s2 += (double)__fmul_rn(c, c); s2 += (double)__fmul_rn(e, e);
+                }
+            s2 = pi_wave_sum_f64(s2);
+            scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
+        }
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            __half2 hh[4];
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                float4 v = xv[j][h];
+                if (na.kind != 0) {
+                    if (na.kind == 2) { v.x = __fsub_rn(v.x, mean); v.y = __fsub_rn(v.y, mean); v.z = __fsub_rn(v.z, mean); v.w = __fsub_rn(v.w, mean); }
+                    v.x = __fmul_rn(v.x, scale); v.y = __fmul_rn(v.y, scale); v.z = __fmul_rn(v.z, scale); v.w = __fmul_rn(v.w, scale);
+                    if (has_w) { const float4 w4 = wv[j][h]; v.x = __fmul_rn(v.x, w4.x); v.y = __fmul_rn(v.y, w4.y); v.z = __fmul_rn(v.z, w4.z); v.w = __fmul_rn(v.w, w4.w); }
+                    if (na.b) {
+                        const float4 b4 = *reinterpret_cast<const float4 *>(na.b + j * 512 + lane * 8 + 4 * h);
+                        v.x = __fadd_rn(v.x, b4.x); v.y = __fadd_rn(v.y, b4.y); v.z = __fadd_rn(v.z, b4.z); v.w = __fadd_rn(v.w, b4.w);
+                    }
+                }
+                hh[2 * h] = __floats2half2_rn(v.x, v.y); hh[2 * h + 1] = __floats2half2_rn(v.z, v.w);
+            }
+            xr[j] = *reinterpret_cast<const pi_u32x4 *>(hh);
+        }
+    }
+    __syncthreads();
+    // ---- activity word (identical in every wave) -----------------------------------------------------
+    const float my_logit = lg[lane & 31];
+    const bool my_act = !(my_logit < thr);
+    const uint32_t mask = (uint32_t)__ballot(my_act);
+    if (wave == 0) {
+        if (lane < 32) { if (logits) logits[n0 + lane] = my_logit; if (!my_act) h_dense[n0 + lane] = 0.0f; }
+        if (lane == 0) words[blockIdx.x] = mask;
+    }
+    // ---- phase B: two active neurons per wave per round trip ------------------------------------------
+    const int n = __popc(mask);
+    for (int k = wave; k < n; k += 2 * kWavesPerBlock) {
+        const int rowA = n0 + select_nth_bit(mask, k);
+        const bool twoB = k + kWavesPerBlock < n;
+        const int rowB = twoB ? n0 + select_nth_bit(mask, k + kWavesPerBlock) : rowA;
+        pi_u32x4 uA[NCH], gA[NCH], uB[NCH], gB[NCH];
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) uA[j] = pi_ld_stream(Wup + (size_t)rowA * cols + (j * PI_WAVE + lane) * 8);
+        if (Wgate) {
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) gA[j] = pi_ld_stream(Wgate + (size_t)rowA * cols + (j * PI_WAVE + lane) * 8);
+        }
+        if (twoB) {
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) uB[j] = pi_ld_stream(Wup + (size_t)rowB * cols + (j * PI_WAVE + lane) * 8);
+            if (Wgate) {
+#pragma unroll
+                for (int j = 0; j < NCH; ++j) gB[j] = pi_ld_stream(Wgate + (size_t)rowB * cols + (j * PI_WAVE + lane) * 8);
+            }
+        }
+        float au = 0.0f, ag = 0.0f, bu = 0.0f, bg = 0.0f;
+#pragma unroll
+        for (int j = 0; j < NCH; ++j) {
+            float xf[8];
+            pi_unpack8(xr[j], xf);
+            au = pi_dot8(uA[j], xf, au);
+            if (Wgate) ag = pi_dot8(gA[j], xf, ag);
+        }
+        au = pi_wave_sum(au);
+        if (Wgate) ag = pi_wave_sum(ag);
+        if (lane == 0) h_dense[rowA] = Wgate ? __fmul_rn(fmaxf(ag, 0.0f), au) : fmaxf(au, 0.0f);
+        if (twoB) {
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) {
+                float xf[8];
+                pi_unpack8(xr[j], xf);
+                bu = pi_dot8(uB[j], xf, bu);
+                if (Wgate) bg = pi_dot8(gB[j], xf, bg);
+            }
+            bu = pi_wave_sum(bu);
+            if (Wgate) bg = pi_wave_sum(bg);
+            if (lane == 0) h_dense[rowB] = Wgate ? __fmul_rn(fmaxf(bg, 0.0f), bu) : fmaxf(bu, 0.0f);
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// The whole sparse FFN of one token behind fc1, in one launch plus a small reduction (F16, cols == 4096).
+// A workgroup of 8 waves owns 32 consecutive neurons.
+//   A  wave w computes 4 of the 32 predictor logits (fc2 rows, r == 512*RCH) and, meanwhile, loads ITS eighth
+//      of the FFN input and of the norm weights (columns [512w, 512w+512): 8 values per lane); the sum of squares
+//      (and the mean for LayerNorm) crosses the waves through LDS, after which each wave holds its slice of
+//      fp16(norm(x)) in four registers.  Nobody reads the whole vector.
+//   B  the 32 logits meet in LDS, every wave derives the same activity word, and for up to 8 active neurons
+//      at a time wave w loads ITS 512-column slice of the gate, up and down rows (one 16-byte load per lane and
+//      row, all issued together), so the work is balanced whatever the number of active neurons.  The partial
+//      gate/up dots cross the waves through LDS in wave order; h = relu(g)*u (relu(u) without a gate).
+//   C  out_partial[workgroup][512w + 8*lane ..] += fp16(h) * down slice: the wave owns its columns, so the
+//      workgroup's contribution needs no further merge and is stored once.
+// ffn_reduce_kernel then adds the per-workgroup partial vectors in workgroup order plus the residual(s).
+// Two dependent memory round trips (A, B+C) instead of four kernels; summation order fixed, no atomics.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kPfBlock = 512;
+constexpr int kPfWaves = kPfBlock / PI_WAVE;      // 8 column slices of 512
+constexpr int kPfChunk = 8;                       // active neurons per round trip
+
+__device__ __forceinline__ int select_nth_bit(uint32_t bits, int n);
+
+template <int RCH, bool GATE>
+__global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
+                                                                   const __half * __restrict__ Wup, const __half * __restrict__ Wgate,
+                                                                   const __half * __restrict__ Wdown,
+                                                                   const float * __restrict__ x, NormArgs na, float thr,
+                                                                   float * __restrict__ logits, uint32_t * __restrict__ words, float * __restrict__ h_dense,
+                                                                   float * __restrict__ partial) {
+    constexpr int cols = kPfWaves * 512, r = RCH * 512;
+    __shared__ float  lg[32];
+    __shared__ double red[2][kPfWaves];
+    __shared__ float  part[kPfWaves][kPfChunk][2];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n0 = blockIdx.x * 32;
+    const int cbase = wave * 512 + lane * 8;
+
+    // ---- A: loads ------------------------------------------------------------------------------------------
+    pi_u32x4 a[4][RCH];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < RCH; ++j) a[i][j] = pi_ld_stream(W2 + (size_t)(n0 + wave * 4 + i) * r + (j * PI_WAVE + lane) * 8);
+    float4 hv[RCH][2];
+#pragma unroll
+    for (int j = 0; j < RCH; ++j) {
+        hv[j][0] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8);
+        hv[j][1] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8 + 4);
+    }
+    float xs[8], ws[8], bs[8];
+    {
+        const float4 x0 = *reinterpret_cast<const float4 *>(x + cbase), x1 = *reinterpret_cast<const float4 *>(x + cbase + 4);
+        xs[0] = x0.x; xs[1] = x0.y; xs[2] = x0.z; xs[3] = x0.w; xs[4] = x1.x; xs[5] = x1.y; xs[6] = x1.z; xs[7] = x1.w;
+        if (na.kind != 0 && na.w) {
+            const float4 w0 = *reinterpret_cast<const float4 *>(na.w + cbase), w1 = *reinterpret_cast<const float4 *>(na.w + cbase + 4);
+            ws[0] = w0.x; ws[1] = w0.y; ws[2] = w0.z; ws[3] = w0.w; ws[4] = w1.x; ws[5] = w1.y; ws[6] = w1.z; ws[7] = w1.w;
+        }
+        if (na.kind != 0 && na.b) {
+            const float4 b0 = *reinterpret_cast<const float4 *>(na.b + cbase), b1 = *reinterpret_cast<const float4 *>(na.b + cbase + 4);
+            bs[0] = b0.x; bs[1] = b0.y; bs[2] = b0.z; bs[3] = b0.w; bs[4] = b1.x; bs[5] = b1.y; bs[6] = b1.z; bs[7] = b1.w;
+        }
+    }
+    // ---- A: logits (the CPU path rounds the hidden vector to fp16 before the dot, ggml.c:9703-9716) ------------
+    {
+        pi_u32x4 hr[RCH];
+#pragma unroll
+        for (int j = 0; j < RCH; ++j) {
+            __half2 hh[4] = {__floats2half2_rn(hv[j][0].x, hv[j][0].y), __floats2half2_rn(hv[j][0].z, hv[j][0].w),
+                             __floats2half2_rn(hv[j][1].x, hv[j][1].y), __floats2half2_rn(hv[j][1].z, hv[j][1].w)};
+            hr[j] = *reinterpret_cast<const pi_u32x4 *>(hh);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < RCH; ++j) acc = pi_dot8h(a[i][j], hr[j], acc);
+            acc = pi_wave_sum(acc);
+            if (lane == 0) lg[wave * 4 + i] = acc;
+        }
+    }
+    // ---- A: norm statistics across the 8 slices ---------------------------------------------------------------
+    float mean = 0.0f, scale = 1.0f;
+    if (na.kind == 1) {
+        double sq = 0.0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) sq += (double)__fmul_rn(xs[k], xs[k]);
+        sq = pi_wave_sum_f64(sq);
+        if (lane == 0) red[0][wave] = sq;
+        __syncthreads();
+        double t = 0.0;
+#pragma unroll
+        for (int w = 0; w < kPfWaves; ++w) t += red[0][w];
+        scale = 1.0f / sqrtf((float)(t / cols) + na.eps);
+    } else if (na.kind == 2) {
+        double sm = 0.0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) sm += (double)xs[k];
+        sm = pi_wave_sum_f64(sm);
+        if (lane == 0) red[0][wave] = sm;
+        __syncthreads();
+        double t = 0.0;
+#pragma unroll
+        for (int w = 0; w < kPfWaves; ++w) t += red[0][w];
+        mean = (float)(t / cols);
+        double sq = 0.0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { const float v = __fsub_rn(xs[k], mean); sq += (double)__fmul_rn(v, v); }
+        sq = pi_wave_sum_f64(sq);
+        if (lane == 0) red[1][wave] = sq;
+        __syncthreads();
+        double t2 = 0.0;
+#pragma unroll
+        for (int w = 0; w < kPfWaves; ++w) t2 += red[1][w];
+        scale = 1.0f / sqrtf((float)(t2 / cols) + na.eps);
+    } else {
+        __syncthreads();
+    }
+    pi_u32x4 xr;
+    {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            float v = xs[k];
+            if (na.kind != 0) {
+                v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
+                if (na.w) v = __fmul_rn(v, ws[k]);
+                if (na.b) v = __fadd_rn(v, bs[k]);
+            }
+            xs[k] = v;
+        }
+        __half2 hh[4] = {__floats2half2_rn(xs[0], xs[1]), __floats2half2_rn(xs[2], xs[3]), __floats2half2_rn(xs[4], xs[5]), __floats2half2_rn(xs[6], xs[7])};
+        xr = *reinterpret_cast<const pi_u32x4 *>(hh);
+    }
+    // ---- activity word (identical in every wave; lg is complete after the barrier above) -----------------------
+    const float my_logit = lg[lane & 31];
+    const bool my_act = !(my_logit < thr);
+    const uint32_t mask = (uint32_t)__ballot(my_act);
+    if (wave == 0) {
+        if (lane < 32) { if (logits) logits[n0 + lane] = my_logit; if (h_dense && !my_act) h_dense[n0 + lane] = 0.0f; }
+        if (lane == 0) words[blockIdx.x] = mask;
+    }
+    // ---- B + C ---------------------------------------------------------------------------------------------
+    const int n = __popc(mask);
+    float acc[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[k] = 0.0f;
+    for (int c0 = 0; c0 < n; c0 += kPfChunk) {
+        const int nn = n - c0 < kPfChunk ? n - c0 : kPfChunk;
+        int rows[kPfChunk];
+        pi_u32x4 gu[kPfChunk], uu[kPfChunk], dd[kPfChunk];
+#pragma unroll
+        for (int j = 0; j < kPfChunk; ++j) {
+            if (j < nn) {
+                rows[j] = n0 + select_nth_bit(mask, c0 + j);
+                const size_t off = (size_t)rows[j] * cols + cbase;
+                uu[j] = pi_ld_stream(Wup + off);
+                if (GATE) gu[j] = pi_ld_stream(Wgate + off);
+                dd[j] = pi_ld_stream(Wdown + off);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kPfChunk; ++j) {
+            if (j < nn) {
+                float pu = pi_wave_sum(pi_dot8h(uu[j], xr, 0.0f));
+                float pg = GATE ? pi_wave_sum(pi_dot8h(gu[j], xr, 0.0f)) : 0.0f;
+                if (lane == 0) { part[wave][j][0] = pu; part[wave][j][1] = pg; }
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < kPfChunk; ++j) {
+            if (j < nn) {
+                float u = 0.0f, g = 0.0f;
+#pragma unroll
+                for (int w = 0; w < kPfWaves; ++w) { u += part[w][j][0]; if (GATE) g += part[w][j][1]; }
+                const float h = GATE ? __fmul_rn(fmaxf(g, 0.0f), u) : fmaxf(u, 0.0f);
+                if (h_dense && threadIdx.x == 0) h_dense[rows[j]] = h;
+                const float hq = pi_round_f16(h);                 // the CPU axpy rounds h to fp16 (ggml.c:14420-14431)
+                float wf[8];
+                pi_unpack8(dd[j], wf);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) acc[k] = fmaf(wf[k], hq, acc[k]);
+            }
+        }
+        if (c0 + kPfChunk < n) __syncthreads();                   // part[] is reused by the next chunk
+    }
+    float4 * po = reinterpret_cast<float4 *>(partial + (size_t)blockIdx.x * cols + cbase);
+    po[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    po[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+}
+
+// out[c] = epi( sum over workgroups b (ascending within a fixed tree) of partial[b][c] ).  A workgroup of 8 waves owns
+// 64 columns: 16 lanes x float4 cover them, the four 16-lane groups of a wave and the 8 waves split the rows of the
+// partial matrix; groups merge by DPP-free shuffles, waves through LDS in wave order.  Workgroup 0 also counts the
+// predictor's active neurons from the mask words.
+constexpr int kFrUn = 12;
+__global__ __launch_bounds__(kPfBlock) void ffn_reduce_kernel(const float * __restrict__ partial, int n_part, int cols,
+                                                              const uint32_t * __restrict__ words, int n_words, int32_t * __restrict__ n_active_out,
+                                                              int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ out) {
+    __shared__ float redl[kPfWaves][64];
+    __shared__ int   sred[kPfWaves];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int sub = lane >> 4, col = blockIdx.x * 64 + (lane & 15) * 4;
+    // the residual operands and the mask words do not depend on anything computed here: fetch them first
+    float r1 = 0.0f, r2 = 0.0f;
+    if (tid < 64) {
+        if (epi >= PI_EPI_ADD) r1 = add1[blockIdx.x * 64 + tid];
+        if (epi == PI_EPI_ADD2) r2 = add2[blockIdx.x * 64 + tid];
+    }
+    int cnt = 0;
+    if (blockIdx.x == 0 && n_active_out)
+        for (int w = tid; w < n_words; w += kPfBlock) cnt += __popc(words[w]);
+    float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (int b0 = wave * 4 + sub; b0 < n_part; b0 += kPfWaves * 4 * kFrUn) {
+        float4 v[kFrUn];
+#pragma unroll
+        for (int u = 0; u < kFrUn; ++u) {
+            const int b = b0 + u * kPfWaves * 4;
+            v[u] = b < n_part ? *reinterpret_cast<const float4 *>(partial + (size_t)b * cols + col) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        }
+#pragma unroll
+        for (int u = 0; u < kFrUn; ++u) { acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w; }
+    }
+    acc.x += __shfl_xor(acc.x, 16, PI_WAVE); acc.y += __shfl_xor(acc.y, 16, PI_WAVE); acc.z += __shfl_xor(acc.z, 16, PI_WAVE); acc.w += __shfl_xor(acc.w, 16, PI_WAVE);
+    acc.x += __shfl_xor(acc.x, 32, PI_WAVE); acc.y += __shfl_xor(acc.y, 32, PI_WAVE); acc.z += __shfl_xor(acc.z, 32, PI_WAVE); acc.w += __shfl_xor(acc.w, 32, PI_WAVE);
+    if (lane < 16) { redl[wave][lane * 4] = acc.x; redl[wave][lane * 4 + 1] = acc.y; redl[wave][lane * 4 + 2] = acc.z; redl[wave][lane * 4 + 3] = acc.w; }
+    if (blockIdx.x == 0 && n_active_out) { cnt = pi_wave_sum_i32(cnt); if (lane == 0) sred[wave] = cnt; }
+    __syncthreads();
+    if (tid < 64) {
+        float sum = redl[0][tid];
+#pragma unroll
+        for (int w = 1; w < kPfWaves; ++w) sum += redl[w][tid];
+        if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, r1);
+        else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, r1), r2);
+        out[blockIdx.x * 64 + tid] = sum;
+    }
+    if (blockIdx.x == 0 && n_active_out && tid == 0) { int t = 0; for (int w = 0; w < kPfWaves; ++w) t += sred[w]; *n_active_out = t; }
 }
 
 // compaction of existing mask words into the ascending active-row list (single block)
@@ -864,6 +1275,118 @@ __global__ __launch_bounds__(kAxBlock) void sparse_axpy_lds_f16_kernel(const __h
         for (int w = 1; w < kAxWaves; ++w) sum += redl[w][tid];
         const int c = blockIdx.x * 128 + tid;
         out[c] = apply_epilogue(sum, epi, add1, add2, c);
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// F16 down projection straight from the dense h vector (0 for inactive neurons).  A workgroup of 16 waves owns
+// 64 output columns and all rows.  Every thread fetches its share of h in one go (16 values per 16384
+// neurons), rounds to fp16 as the CPU path does and drops zeros (ggml.c:14420-14431); wave ballots give the
+// per-(round, wave) counts, one workgroup scan turns them into offsets, and the surviving (row, h) pairs land
+// in LDS in ascending row order.  Then one round trip of weight loads: 8 lanes cover the 128-byte segment of
+// a row, a wave load instruction covers 8 rows, 8 instructions are in flight per lane.  The 8 row slots of a
+// wave merge by shuffles, the 16 waves through LDS in wave order: fixed summation order, no atomics.
+// Workgroup 0 also counts the predictor's active neurons from the mask words.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kAdTile = 64;
+constexpr int kAdCap = 4096;         // (row, h) pairs held in LDS per pass
+constexpr int kAdRounds = 16;        // h values per thread per super-group of 16384 neurons
+constexpr int kAdUn = 8;
+
+__global__ __launch_bounds__(kAxBlock) void sparse_axpy_dense_f16_kernel(const __half * __restrict__ Wd, int cols, int ff,
+                                                                         const float * __restrict__ h_dense, const uint32_t * __restrict__ words,
+                                                                         int32_t * __restrict__ n_active_out,
+                                                                         int epi, const float * add1, const float * add2, float * __restrict__ out) {
+    __shared__ int   crow[kAdCap];
+    __shared__ float ca[kAdCap];
+    __shared__ int   cnt[kAdRounds * kAxWaves];
+    __shared__ float redl[kAxWaves][kAdTile];
+    __shared__ int   sred[kAxWaves + 1];
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const int sub = lane >> 3, col = blockIdx.x * kAdTile + (lane & 7) * 8;
+    const unsigned long long lt = (1ull << lane) - 1ull;
+    float acc[8];
+#pragma unroll
+    for (int j = 0; j < 8; ++j) acc[j] = 0.0f;
+
+    for (int base = 0; base < ff; base += kAdRounds * kAxBlock) {
+        float hv[kAdRounds];
+#pragma unroll
+        for (int i = 0; i < kAdRounds; ++i) {
+            const int idx = base + i * kAxBlock + tid;
+            hv[i] = idx < ff ? h_dense[idx] : 0.0f;
+        }
+        int lp[kAdRounds];
+#pragma unroll
+        for (int i = 0; i < kAdRounds; ++i) {
+            hv[i] = pi_round_f16(hv[i]);
+            const unsigned long long m = __ballot(hv[i] != 0.0f);
+            lp[i] = __popcll(m & lt);
+            if (lane == 0) cnt[i * kAxWaves + wave] = __popcll(m);
+        }
+        __syncthreads();
+        int tot;
+        const int v = tid < kAdRounds * kAxWaves ? cnt[tid] : 0;
+        const int off = block_exclusive_scan_i32(v, &tot, sred);
+        __syncthreads();
+        if (tid < kAdRounds * kAxWaves) cnt[tid] = off;
+        __syncthreads();
+        for (int c0 = 0; c0 < tot; c0 += kAdCap) {
+#pragma unroll
+            for (int i = 0; i < kAdRounds; ++i) {
+                if (hv[i] != 0.0f) {
+                    const int o = cnt[i * kAxWaves + wave] + lp[i] - c0;
+                    if (o >= 0 && o < kAdCap) { crow[o] = base + i * kAxBlock + tid; ca[o] = hv[i]; }
+                }
+            }
+            __syncthreads();
+            const int m = tot - c0 < kAdCap ? tot - c0 : kAdCap;
+            for (int i0 = wave * 8 + sub; i0 < m; i0 += kAxWaves * 8 * kAdUn) {
+                pi_u32x4 w[kAdUn]; float a[kAdUn];
+#pragma unroll
+                for (int u = 0; u < kAdUn; ++u) {
+                    const int i = i0 + u * kAxWaves * 8;
+                    const bool ok = i < m;
+                    a[u] = ok ? ca[i] : 0.0f;
+                    w[u] = ok ? pi_ld_stream(Wd + (size_t)crow[i] * cols + col) : pi_u32x4{0u, 0u, 0u, 0u};
+                }
+#pragma unroll
+                for (int u = 0; u < kAdUn; ++u) {
+                    float wf[8];
+                    pi_unpack8(w[u], wf);
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) acc[j] = fmaf(wf[j], a[u], acc[j]);
+                }
+            }
+            __syncthreads();
+        }
+    }
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        acc[j] += __shfl_xor(acc[j], 8, PI_WAVE);
+        acc[j] += __shfl_xor(acc[j], 16, PI_WAVE);
+        acc[j] += __shfl_xor(acc[j], 32, PI_WAVE);
+    }
+    if (lane < 8) {
+#pragma unroll
+        for (int j = 0; j < 8; ++j) redl[wave][lane * 8 + j] = acc[j];
+    }
+    __syncthreads();
+    if (tid < kAdTile) {
+        float sum = redl[0][tid];
+#pragma unroll
+        for (int w = 1; w < kAxWaves; ++w) sum += redl[w][tid];
+        const int c = blockIdx.x * kAdTile + tid;
+        out[c] = apply_epilogue(sum, epi, add1, add2, c);
+    }
+    if (blockIdx.x == 0 && n_active_out && words) {
+        int c = 0;
+        for (int w = tid; w < (ff + 31) / 32; w += kAxBlock) c += __popc(words[w]);
+        c = pi_wave_sum_i32(c);
+        __syncthreads();
+        if (lane == 0) sred[wave] = c;
+        __syncthreads();
+        if (tid == 0) { int t = 0; for (int w = 0; w < kAxWaves; ++w) t += sred[w]; *n_active_out = t; }
     }
 }
 
@@ -1276,6 +1799,7 @@ struct pi_workspace {
     float *        partial;        // [kAxpyGroups][max_d]
     int32_t *      hq;             // [max_ff]  Q4_0 axpy: int8 value of h per active row
     float *        hd;             // [max_ff]  and its Q8_0 block scale
+    float *        ffn_partial;    // [max_ff/32][max_d]  per-workgroup partial outputs of the fused sparse FFN
 };
 constexpr int kAxpyGroups = 32;
 
@@ -1290,7 +1814,8 @@ pi_workspace * pi_workspace_create(int max_ff, int max_d) {
     ws->partial  = (float *)pi_malloc(sizeof(float) * (size_t)kAxpyGroups * max_d);
     ws->hq       = (int32_t *)pi_malloc(sizeof(int32_t) * max_ff);
     ws->hd       = (float *)pi_malloc(sizeof(float) * max_ff);
-    if (!ws->words || !ws->counters || !ws->partial || !ws->hq || !ws->hd) {
+    ws->ffn_partial = (float *)pi_malloc(sizeof(float) * (size_t)((max_ff + 31) / 32) * max_d);
+    if (!ws->words || !ws->counters || !ws->partial || !ws->hq || !ws->hd || !ws->ffn_partial) {
         pi_workspace_destroy(ws); return nullptr;
     }
     pi_memset(ws->counters, 0, sizeof(unsigned int) * 64);
@@ -1298,7 +1823,7 @@ pi_workspace * pi_workspace_create(int max_ff, int max_d) {
 }
 int pi_workspace_destroy(pi_workspace * ws) {
     if (!ws) return PI_OK;
-    pi_free(ws->words); pi_free(ws->counters); pi_free(ws->partial); pi_free(ws->hq); pi_free(ws->hd);
+    pi_free(ws->words); pi_free(ws->counters); pi_free(ws->partial); pi_free(ws->hq); pi_free(ws->hd); pi_free(ws->ffn_partial);
     delete ws;
     return PI_OK;
 }
@@ -1464,6 +1989,61 @@ int pi_k_sparse_axpy(int wtype, const void * down_t, int cols, int n_rows, const
         return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_axpy: weight type must be F16 or Q4_0");
     }
     return pi::check_launch("pi_k_sparse_axpy");
+}
+
+int pi_k_pred_upgate(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                     const void * up_f16, const void * gate_f16, int cols, const float * x, const pi_norm * norm,
+                     float * logits, float * h_dense, pi_workspace * ws, pi_stream_t stream) {
+    if (!fc2_f16 || !hidden || !up_f16 || !x || !h_dense || !ws) return pi::fail(PI_E_ARG, "pi_k_pred_upgate: null pointer");
+    if (!pi_k_pred_upgate_supported(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_pred_upgate: shape outside the fused kernel (cols 4096, r 1024, ff % 32 == 0)");
+    if (ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_pred_upgate: ff exceeds the workspace");
+    const NormArgs na = to_norm(norm);
+    if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_pred_upgate: vectors must be 16-byte aligned");
+    hipLaunchKernelGGL((pred_upgate_f16_kernel<8, 2>), dim3(ff / 32), dim3(kBlock), 0, (hipStream_t)stream,
+                       (const __half *)fc2_f16, hidden, (const __half *)up_f16, (const __half *)gate_f16, x, na, threshold, logits, ws->words, h_dense);
+    return pi::check_launch("pi_k_pred_upgate");
+}
+
+int pi_k_pred_upgate_supported(int ff, int r, int cols) { return cols == 4096 && r == 1024 && ff > 0 && ff % 32 == 0; }
+
+int pi_k_sparse_axpy_dense(const void * down_t_f16, int cols, int ff, const float * h_dense, int32_t * n_active,
+                           int epilogue, const float * add1, const float * add2, float * out, pi_workspace * ws, pi_stream_t stream) {
+    if (!down_t_f16 || !h_dense || !out || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy_dense: null pointer");
+    if (cols <= 0 || cols % kAdTile || ff <= 0 || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_sparse_axpy_dense: cols % 64 == 0 and ff <= workspace required");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_sparse_axpy_dense: bad epilogue arguments");
+    hipLaunchKernelGGL(sparse_axpy_dense_f16_kernel, dim3(cols / kAdTile), dim3(kAxBlock), 0, (hipStream_t)stream,
+                       (const __half *)down_t_f16, cols, ff, h_dense, ws->words, n_active, epilogue, add1, add2, out);
+    return pi::check_launch("pi_k_sparse_axpy_dense");
+}
+
+int pi_k_sparse_ffn_supported(int ff, int r, int cols) { return cols == 4096 && (r == 1024 || r == 512) && ff > 0 && ff % 32 == 0; }
+
+int pi_k_sparse_ffn(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                    const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x, const pi_norm * norm,
+                    int epilogue, const float * add1, const float * add2, float * out,
+                    float * logits, float * h_dense, int32_t * n_active, pi_workspace * ws, pi_stream_t stream) {
+    if (!fc2_f16 || !hidden || !up_f16 || !down_t_f16 || !x || !out || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: null pointer");
+    if (!pi_k_sparse_ffn_supported(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn: shape outside the fused kernel (cols 4096, r 512 or 1024, ff % 32 == 0)");
+    if (ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: shape exceeds the workspace");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: bad epilogue arguments");
+    const NormArgs na = to_norm(norm);
+    if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: vectors must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const __half * w2 = (const __half *)fc2_f16; const __half * u = (const __half *)up_f16; const __half * g = (const __half *)gate_f16;
+    const __half * dn = (const __half *)down_t_f16;
+    const dim3 grid(ff / 32), block(kPfBlock);
+    if (r == 1024) {
+        if (g) hipLaunchKernelGGL((pred_ffn_f16_kernel<2, true>),  grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial);
+        else   hipLaunchKernelGGL((pred_ffn_f16_kernel<2, false>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial);
+    } else {
+        if (g) hipLaunchKernelGGL((pred_ffn_f16_kernel<1, true>),  grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial);
+        else   hipLaunchKernelGGL((pred_ffn_f16_kernel<1, false>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial);
+    }
+    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, st, ws->ffn_partial, ff / 32, cols, ws->words, ff / 32, n_active,
+                       epilogue, add1, add2, out);
+    return pi::check_launch("pi_k_sparse_ffn");
 }
 
 int pi_k_rope_kv_store(const float * qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale,

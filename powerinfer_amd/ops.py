@@ -83,6 +83,50 @@ class SparseFFN:
                     h=self.h_dense.download(np.float32), h_compact=self.h_c.download(np.float32, n),
                     out=self.out.download(np.float32))
 
+    def forward_two_launch(self, x_ffn, x_pred, epilogue=pl.EPI_NONE, resid=None):
+        """The full-GPU F16 fast route of the decode loop: fc1, then pi_k_pred_upgate (fc2 + mask + up/gate in one
+        launch) and pi_k_sparse_axpy_dense (down projection from the dense h).  Returns dict(logits, mask_words,
+        h, n_active, out)."""
+        L = self.L
+        if self.bucket is not None or self.wtype != pl.F16 or not L.pi_k_pred_upgate_supported(self.ff, self.r, self.d):
+            raise pl.PiError("forward_two_launch: shape or placement outside the fused kernels")
+        self.x.upload(np.asarray(x_ffn, np.float32))
+        self.xp.upload(np.asarray(x_pred, np.float32))
+        if resid is not None:
+            self.resid.upload(np.asarray(resid, np.float32))
+        check(L.pi_memset(self.h_dense.ptr, 0xFF, self.h_dense.nbytes), "memset")      # the kernel must write every entry
+        nrm = pl.norm_arg(self.norm_kind, self.eps, self.norm_w, self.norm_b)
+        check(L.pi_k_gemv(pl.F16, self.fc1.ptr, self.r, self.d, self.xp.ptr, None, pl.EPI_RELU, None, None, self.hidden.ptr, None), "fc1")
+        check(L.pi_k_pred_upgate(self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, self.up.ptr,
+                                 self.gate.ptr if self.gate is not None else None, self.d, self.x.ptr, nrm,
+                                 self.logits.ptr, self.h_dense.ptr, self.ws, None), "pred_upgate")
+        check(L.pi_k_sparse_axpy_dense(self.down.ptr, self.d, self.ff, self.h_dense.ptr, self.n_active.ptr, epilogue,
+                                       self.resid.ptr if epilogue else None, None, self.out.ptr, self.ws, None), "axpy_dense")
+        pl.sync()
+        return dict(logits=self.logits.download(np.float32), h=self.h_dense.download(np.float32),
+                    n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32))
+
+    def forward_one_launch(self, x_ffn, x_pred, epilogue=pl.EPI_NONE, resid=None):
+        """fc1, then pi_k_sparse_ffn: predictor fc2, mask, gate/up, h and the down projection in one launch plus the
+        fixed-order reduction of the per-workgroup partial outputs.  Returns dict(logits, h, n_active, out)."""
+        L = self.L
+        if self.bucket is not None or self.wtype != pl.F16 or not L.pi_k_sparse_ffn_supported(self.ff, self.r, self.d):
+            raise pl.PiError("forward_one_launch: shape or placement outside the fused kernel")
+        self.x.upload(np.asarray(x_ffn, np.float32))
+        self.xp.upload(np.asarray(x_pred, np.float32))
+        if resid is not None:
+            self.resid.upload(np.asarray(resid, np.float32))
+        check(L.pi_memset(self.h_dense.ptr, 0xFF, self.h_dense.nbytes), "memset")      # the kernel must write every entry
+        nrm = pl.norm_arg(self.norm_kind, self.eps, self.norm_w, self.norm_b)
+        check(L.pi_k_gemv(pl.F16, self.fc1.ptr, self.r, self.d, self.xp.ptr, None, pl.EPI_RELU, None, None, self.hidden.ptr, None), "fc1")
+        check(L.pi_k_sparse_ffn(self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, self.up.ptr,
+                                self.gate.ptr if self.gate is not None else None, self.down.ptr, self.d, self.x.ptr, nrm,
+                                epilogue, self.resid.ptr if epilogue else None, None, self.out.ptr,
+                                self.logits.ptr, self.h_dense.ptr, self.n_active.ptr, self.ws, None), "sparse_ffn")
+        pl.sync()
+        return dict(logits=self.logits.download(np.float32), h=self.h_dense.download(np.float32),
+                    n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32))
+
     def close(self):
         if self.ws:
             self.L.pi_workspace_destroy(self.ws)

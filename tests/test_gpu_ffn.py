@@ -85,6 +85,46 @@ def test_ffn_7b_shape_vs_oracle(wtype, has_gate):
     ffn.close()
 
 
+@pytest.mark.parametrize("route", ["one", "two"])
+@pytest.mark.parametrize("has_gate", [True, False])
+@pytest.mark.parametrize("norm", [0, 1, 2])
+def test_fused_routes_7b_shape(has_gate, norm, route):
+    """pi_k_sparse_ffn (what the F16 decode loop runs at d = 4096) and pi_k_pred_upgate + pi_k_sparse_axpy_dense
+    against the oracle, with the fused RMSNorm / LayerNorm prologue and the residual epilogue."""
+    from powerinfer_amd import lib as pl
+    from powerinfer_amd.ops import SparseFFN
+    d, ff, r, T = 4096, 11008, 1024, 3
+    L = synth.make_ffn_layer(seed=77 + norm, d=d, ff=ff, r=r, wtype=ol.F16, has_gate=has_gate, T=T)
+    rng = np.random.default_rng(5)
+    nw = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32) if norm else None
+    nb = (0.1 * rng.standard_normal(d)).astype(np.float32) if norm == 2 else None
+    eps = 1e-5
+    O = ol.oracle()
+    P = ol._ptr
+    ffn = SparseFFN(d, ff, r, ol.F16, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], norm_kind=norm, norm_w=nw, norm_b=nb, eps=eps)
+    for t in range(T):
+        x = np.ascontiguousarray(L["x"][t:t + 1], np.float32)
+        xn = x.copy()
+        if norm == 1:
+            O.pio_rms_norm(P(x), d, 1, eps, P(xn)); xn = np.ascontiguousarray(xn * nw, np.float32)
+        elif norm == 2:
+            O.pio_norm(P(x), d, 1, eps, P(xn)); xn = np.ascontiguousarray(xn * nw + nb, np.float32)
+        o = ol.ffn_sparse(O, d, ff, r, 1, ol.F16, has_gate, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], xn, x,
+                          np.zeros(ff, np.int32), 0.0, nth=8)
+        resid = rng.standard_normal(d).astype(np.float32)
+        res = (ffn.forward_one_launch if route == "one" else ffn.forward_two_launch)(x[0], x[0], epilogue=pl.EPI_ADD, resid=resid)
+        assert rel_err(res["logits"], o["logits"][0]) < 1e-4
+        mask_g, mask_o = ~(res["logits"] < 0.0), ~(o["logits"][0] < 0.0)
+        assert (mask_g == mask_o).mean() >= MASK_AGREE
+        assert res["n_active"] == int(mask_g.sum())
+        assert not np.isnan(res["h"]).any()
+        assert np.all(res["h"][~mask_g] == 0.0)               # every inactive neuron written as 0
+        if np.array_equal(mask_g, mask_o):
+            assert rel_err(res["h"], o["h"][0]) < 1e-4
+            assert rel_err(res["out"] - resid, o["out"][0]) < 1e-4
+    ffn.close()
+
+
 @pytest.mark.parametrize("wtype", [ol.F16, ol.Q4_0])
 def test_hybrid_split_gpu_share(wtype):
     """Config 2 split: the GPU holds the hottest 60 % of neurons (compact matrices + gpu_bucket) and

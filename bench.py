@@ -28,8 +28,10 @@ HBM_PEAK_GBPS = 8000.0
 
 
 def build_synthetic_on_device(hp, keep):
-    """Random-init weights generated directly in HBM (pi_fill_normal_f16), predictor fc2 rows carrying the
-    Zipf firing-rate bias computed on the host (powerinfer_amd.synth)."""
+    """Random-init weights generated directly in HBM (pi_fill_normal_f16 / pi_fill_normal_q4_0), predictor fc2 rows
+    carrying the Zipf firing-rate bias computed on the host (powerinfer_amd.synth).  With hp.hot_frac < 1 the FFN
+    matrices are copied back to the host, which keeps the cold neurons, and the engine gathers the hot rows
+    (gpu_bucket) into compact device matrices."""
     from powerinfer_amd import lib as pl, synth
     from powerinfer_amd.model import Model
     from scipy.special import ndtri
@@ -37,43 +39,70 @@ def build_synthetic_on_device(hp, keep):
     m = Model(hp)
     d, ff, r = hp.n_embd, hp.n_ff, hp.n_rank
     gqa = d // hp.n_head * hp.n_head_kv
+    falcon = hp.arch == "falcon"
+    q4 = hp.wtype == pl.Q4_0
+    hybrid = hp.hot_frac < 1.0
     seed = [hp.seed * 1000003 + 17]
 
-    def normal(rows, cols, bias=None):
-        buf = pl.DevBuf(rows * cols * 2)
+    def normal(rows, cols, bias=None, f16=False):
         seed[0] += 1
-        pl.check(L.pi_fill_normal_f16(buf.ptr, rows * cols, seed[0], 0.02, bias.ptr if bias is not None else None, cols, None), "fill")
+        if q4 and not f16:
+            buf = pl.DevBuf(rows * cols // 32 * 18)
+            pl.check(L.pi_fill_normal_q4_0(buf.ptr, rows * cols, seed[0], 0.02, None), "fill")
+        else:
+            buf = pl.DevBuf(rows * cols * 2)
+            pl.check(L.pi_fill_normal_f16(buf.ptr, rows * cols, seed[0], 0.02, bias.ptr if bias is not None else None, cols, None), "fill")
         keep.append(buf)
         return buf
 
-    def put(layer, kind, buf, rows, cols):
-        m.set_tensor_device(layer, kind, buf.ptr, pl.F16, cols, rows)
+    def put(layer, kind, buf, rows, cols, f16=False):
+        m.set_tensor_device(layer, kind, buf.ptr, pl.F16 if (f16 or not q4) else pl.Q4_0, cols, rows)
+
+    def put_ffn(layer, kind, buf, rows, cols):
+        if not hybrid:
+            return put(layer, kind, buf, rows, cols)
+        pl.sync()
+        host = buf.download(np.uint8).reshape(rows, -1) if q4 else buf.download(np.float16).reshape(rows, cols)
+        m.set_tensor(layer, kind, host)
 
     put(-1, "tok_embd", normal(hp.n_vocab, d), hp.n_vocab, d)
     put(-1, "output", normal(hp.n_vocab, d), hp.n_vocab, d)
     m.set_tensor(-1, "output_norm", np.ones(d, np.float32))
+    if falcon:
+        m.set_tensor(-1, "output_norm_b", np.zeros(d, np.float32))
     rng = np.random.default_rng(hp.seed)
     for il in range(hp.n_layer):
         m.set_tensor(il, "attn_norm", np.ones(d, np.float32))
-        m.set_tensor(il, "ffn_norm", np.ones(d, np.float32))
+        if falcon:
+            m.set_tensor(il, "attn_norm_b", np.zeros(d, np.float32))
+            if hp.n_head_kv != hp.n_head:
+                m.set_tensor(il, "attn_norm_2", np.ones(d, np.float32))
+                m.set_tensor(il, "attn_norm_2_b", np.zeros(d, np.float32))
+        else:
+            m.set_tensor(il, "ffn_norm", np.ones(d, np.float32))
         put(il, "wqkv", normal(d + 2 * gqa, d), d + 2 * gqa, d)
         put(il, "wo", normal(d, d), d, d)
-        put(il, "ffn_gate", normal(ff, d), ff, d)
-        put(il, "ffn_up", normal(ff, d), ff, d)
-        put(il, "ffn_down_t", normal(ff, d), ff, d)
-        put(il, "fc1", normal(r, d), r, d)
+        if not falcon:
+            put_ffn(il, "ffn_gate", normal(ff, d), ff, d)
+        put_ffn(il, "ffn_up", normal(ff, d), ff, d)
+        put_ffn(il, "ffn_down_t", normal(ff, d), ff, d)
+        put(il, "fc1", normal(r, d, f16=True), r, d, f16=True)
         p, _ = synth.zipf_rates(ff, hp.mean_rate, rng)
         b = (0.02 * np.sqrt(np.pi) * ndtri(p) / np.sqrt(r)).astype(np.float32)
         bias = pl.DevBuf(host=b)
-        put(il, "fc2", normal(ff, r, bias), ff, r)
+        put(il, "fc2", normal(ff, r, bias, f16=True), ff, r, f16=True)
+        if hybrid:
+            gi, gb = synth.gpu_split(p, hp.hot_frac)
+            m.set_tensor(il, "gpu_idx", gi)
+            m.set_tensor(il, "gpu_bucket", gb)
     pl.sync()
     m.finalize()
     return m
 
 
 def download_model(hp, keep):
-    """Host copies of the device-generated tensors, in the dict layout powerinfer_amd.synth.make_model uses
-    (feeds the CPU port for the cpu_baseline leg)."""
+    """Host copies of the device-generated tensors of the default workload (F16 LLaMA shape, all neurons on the GPU), in
+    the dict layout powerinfer_amd.synth.make_model uses (feeds the CPU port for the cpu_baseline leg)."""
     d, ff, r = hp.n_embd, hp.n_ff, hp.n_rank
     gqa = d // hp.n_head * hp.n_head_kv
     it = iter(keep)
@@ -90,16 +119,21 @@ def download_model(hp, keep):
     return dict(hp=hp, glob=glob, layers=layers)
 
 
+def rnd(v, n):
+    return None if v != v else round(v, n)
+
+
 def touched_bytes_per_token(hp, active_sum, n_kv_mean):
     """Algorithmic bytes of one decoded token:  sum_l [ W_attn + W_pred + A_l * n_mats * R + 2 * n_kv * n_embd_gqa * 2 ]
-    + W_lmhead + d * 2, with the measured per-token sum of active rows."""
+    + W_lmhead + d * 2, with the measured per-token sum of active rows (the GPU's share for a hybrid split)."""
     d, ff, r, Lr = hp.n_embd, hp.n_ff, hp.n_rank, hp.n_layer
     gqa = d // hp.n_head * hp.n_head_kv
-    s = 2.0
+    s = 2.0 if hp.wtype == 1 else 18.0 / 32.0
+    n_mats = 2 if hp.arch == "falcon" else 3
     w_attn = (d * (d + 2 * gqa) + d * d) * s
     w_pred = (d * r + r * ff) * 2.0
     row = d * s
-    return Lr * (w_attn + w_pred + 2 * n_kv_mean * gqa * 2.0) + active_sum * 3 * row + hp.n_vocab * d * s + d * 2.0
+    return Lr * (w_attn + w_pred + 2 * n_kv_mean * gqa * 2.0) + active_sum * n_mats * row + hp.n_vocab * d * s + d * 2.0
 
 
 def cpu_baseline(hp, keep, prompt, n_prompt, n_decode, threads):
@@ -130,6 +164,9 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="only for quick trials; the reported workload uses 32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-tokens", type=int, default=24)
+    ap.add_argument("--config", type=int, default=1, choices=[1, 2, 4],
+                    help="BASELINE configs index: 1 (default, the reported metric) 7B FP16 all on the GPU; 2 the same shape in "
+                         "Q4_0 with the hottest 60 %% of neurons on the GPU and the rest on host threads; 4 Falcon-40B shape FP16")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter-collection aid: run only the q|k|v mat-vec of a 4-layer model a few times plus one "
                          "device-to-device copy of the same byte count (the known-size reference for FETCH_SIZE / WRITE_SIZE)")
@@ -155,7 +192,14 @@ def main():
         print(json.dumps({"pmc_probe": True, "copy_bytes": nbytes, "qkv_weight_bytes": nbytes, "qkv_launches": n, "us_per_launch": ms * 1e3}))
         m.close()
         return
-    hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=args.prompt + args.warmup + args.steps + 8, seed=1)
+    n_ctx = args.prompt + args.warmup + args.steps + 8
+    if args.config == 1:
+        hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_ctx, seed=1)
+    elif args.config == 2:
+        hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_ctx, seed=1, wtype=pl.Q4_0, hot_frac=0.6)
+    else:
+        hp = synth.hparams("falcon-40b", n_layer=60 if args.layers == 32 else args.layers, n_ctx=n_ctx, seed=1)
+    hybrid = hp.hot_frac < 1.0
     keep = []
     t0 = time.perf_counter()
     m = build_synthetic_on_device(hp, keep)
@@ -179,25 +223,31 @@ def main():
     # roofline of the dominant kernel: the q|k|v projection mat-vec (gemv_f16_kernel<4>), one launch per layer
     d = hp.n_embd
     gqa = d // hp.n_head * hp.n_head_kv
-    ms_qkv, n_qkv = m.time_section(0, 8)
-    qkv_bytes = (d + 2 * gqa) * d * 2.0 + d * 4 + (d + 2 * gqa) * 4          # weights + activation in + result out
+    wbytes = 2.0 if hp.wtype == pl.F16 else 18.0 / 32.0
+    qkv_bytes = (d + 2 * gqa) * d * wbytes + d * 4 + (d + 2 * gqa) * 4       # weights + activation in + result out
+    if hybrid:                                                               # the section timers replay full-GPU layers only
+        ms_qkv, n_qkv, ms_ffn, ms_head = float("nan"), 0, float("nan"), float("nan")
+    else:
+        ms_qkv, n_qkv = m.time_section(0, 8)
+        ms_ffn, _ = m.time_section(1, 8)
+        ms_head, _ = m.time_section(2, 8)
     achieved = qkv_bytes / (ms_qkv * 1e-3) / 1e9
-    ms_ffn, _ = m.time_section(1, 8)
-    ffn_bytes = (d * hp.n_rank + hp.n_rank * hp.n_ff) * 2.0 + (act.mean() / hp.n_layer) * 3 * d * 2.0
-    ms_head, _ = m.time_section(2, 8)
+    n_mats = 2 if hp.arch == "falcon" else 3
+    ffn_bytes = (d * hp.n_rank + hp.n_rank * hp.n_ff) * 2.0 + (act.mean() / hp.n_layer) * n_mats * d * wbytes
 
     # HBM bytes per launch of that kernel from the FETCH_SIZE / WRITE_SIZE counter runs (profiles/qkv_gemv_hbm_traffic.md)
     traffic = None
     try:
         with open(os.path.join(ROOT, "profiles", "qkv_gemv_hbm_traffic.json")) as f:
             pj = json.load(f)
-        if pj.get("shape") == [d + 2 * gqa, d]:
+        if pj.get("shape") == [d + 2 * gqa, d] and args.config == 1:
             traffic = pj["traffic_bytes_per_launch"]
     except (OSError, ValueError, KeyError):
         pass
 
     out = {
-        "metric": "decode tok/s bs=1 ReLU-Llama2-7B FP16",
+        "metric": {1: "decode tok/s bs=1 ReLU-Llama2-7B FP16", 2: "decode tok/s bs=1 ReLU-Llama2-7B Q4_0 (60 % of neurons on the GPU)",
+                   4: "decode tok/s bs=1 ReLU-Falcon-40B FP16"}[args.config],
         "value": round(1e3 / ms_per_step, 2),
         "unit": "tok/s",
         "n_gpus": 1,
@@ -207,26 +257,35 @@ def main():
         "higher_is_better": True,
         "scaling": "weak",
         "vs_baseline": None,
-        "dtype": "f16",
+        "dtype": "f16" if hp.wtype == pl.F16 else "q4_0 x q8_0 (int8 dot, fp32 scale)",
         "data": "synthetic",
         "config": {
-            "workload": "configs[1]: ReLU-LLaMA-2-7B shape (d 4096, ff 11008, 32 heads, vocab 32000, predictor rank 1024), "
-                        f"{hp.n_layer} layers, random-init FP16 weights, all neurons on the GPU, {args.prompt}-token random prompt, "
-                        "greedy decode at batch 1",
+            "workload": {
+                1: "configs[1]: ReLU-LLaMA-2-7B shape (d 4096, ff 11008, 32 heads, vocab 32000, predictor rank 1024), "
+                   f"{hp.n_layer} layers, random-init FP16 weights, all neurons on the GPU, {args.prompt}-token random prompt, "
+                   "greedy decode at batch 1",
+                2: "configs[2]: ReLU-LLaMA-2-7B shape, random-init weights quantised to Q4_0 (predictors FP16), per layer the hottest "
+                   f"60 % of neurons on the GPU and the rest on host threads, {hp.n_layer} layers, {args.prompt}-token random prompt, "
+                   "greedy decode at batch 1",
+                4: "configs[4]: ReLU-Falcon-40B shape (d 8192, ff 32768 up/down only, 128 heads / 8 KV heads, vocab 65024, predictor "
+                   f"rank 1024), {hp.n_layer} layers, random-init FP16 weights, all neurons on the GPU, {args.prompt}-token random "
+                   "prompt, greedy decode at batch 1"}[args.config],
             "n_layer": hp.n_layer, "prompt_tokens": args.prompt, "n_ctx": hp.n_ctx,
             "mean_active_per_layer": round(act.mean() / hp.n_layer, 1),
             "device": pl.device_name(),
         },
         "roofline": {
             "bound": "hbm",
-            "kernel": "gemv_f16_reg_kernel<8,2> (q|k|v projection, 12288 x 4096 fp16, fused RMSNorm)",
-            "achieved": round(achieved, 1),
+            "kernel": {1: "gemv_f16_reg_kernel<8,1,0> (q|k|v projection, 12288 x 4096 fp16, fused RMSNorm)",
+                       2: "gemv_q4_kernel (q|k|v projection, 12288 x 4096 Q4_0, fused RMSNorm; not timed for a hybrid model)",
+                       4: "gemv_f16_reg_kernel<16,2,0> (q|k|v projection, 9216 x 8192 fp16, fused LayerNorm)"}[args.config],
+            "achieved": rnd(achieved, 1),
             "peak": HBM_PEAK_GBPS,
             "unit": "GB/s",
-            "frac": round(achieved / HBM_PEAK_GBPS, 4),
+            "frac": rnd(achieved / HBM_PEAK_GBPS, 4),
             "traffic": traffic,
             "bytes_per_launch": qkv_bytes,
-            "us_per_launch": round(ms_qkv * 1e3, 2),
+            "us_per_launch": rnd(ms_qkv * 1e3, 2),
             "launches_timed": n_qkv,
         },
         "token_loop": {
@@ -234,13 +293,13 @@ def main():
             "touched_GB_per_token": round(tok_bytes / 1e9, 4),
             "effective_GBps": round(tok_bytes / (ms_per_step * 1e-3) / 1e9, 1),
             "hbm_frac_touched": round(tok_bytes / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-            "sparse_ffn_us_per_layer": round(ms_ffn * 1e3, 2),
-            "sparse_ffn_effective_GBps": round(ffn_bytes / (ms_ffn * 1e-3) / 1e9, 1),
-            "lm_head_us": round(ms_head * 1e3, 2),
+            "sparse_ffn_us_per_layer": rnd(ms_ffn * 1e3, 2),
+            "sparse_ffn_effective_GBps": rnd(ffn_bytes / (ms_ffn * 1e-3) / 1e9, 1),
+            "lm_head_us": rnd(ms_head * 1e3, 2),
             "build_s": round(t_build, 1),
         },
     }
-    if not args.no_cpu:
+    if not args.no_cpu and args.config == 1:
         threads = min(16, os.cpu_count() or 1)
         n_prompt = 8
         v = cpu_baseline(hp, keep, prompt, n_prompt, args.cpu_tokens, threads)

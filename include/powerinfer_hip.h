@@ -45,6 +45,9 @@ PI_API int          pi_sync(void);
 /* deterministic N(0, std^2) fill rounded to fp16 (synthetic weights generated in HBM); row_bias, if
  * not NULL, holds one fp32 per row of `cols` elements that is added before rounding */
 PI_API int          pi_fill_normal_f16(void * dptr, size_t n, uint64_t seed, float std, const float * row_bias, int cols, pi_stream_t stream);
+/* the same values (rounded to fp16 first) quantised to Q4_0 blocks of 32 as quantize_row_q4_0_reference does
+ * (ggml-quants.c:428-463); n_weights % 32 == 0, dptr receives n_weights / 32 * 18 bytes */
+PI_API int          pi_fill_normal_q4_0(void * dptr, size_t n_weights, uint64_t seed, float std, pi_stream_t stream);
 /* event timing on a stream: returns milliseconds between two recorded marks */
 PI_API void *       pi_event_create(void);
 PI_API int          pi_event_record(void * ev, pi_stream_t stream);

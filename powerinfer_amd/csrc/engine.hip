@@ -499,16 +499,18 @@ int pi_model_time_section(pi_model * m, int section, int rounds, float * ms_tota
                 const bool q4 = up.type == PI_TYPE_Q4_0;
                 pi_norm fn = falcon ? make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B))
                                     : make_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
-                PI_TRY(pi_k_gemv(fc1.type, fc1.dev, (int)fc1.ne1, d, m->ffn_inp, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, st));
+                // Falcon's predictor and FFN read the layer input; LLaMA's read the post-attention residual stream
+                const float * fin = falcon ? m->x : m->ffn_inp;
+                PI_TRY(pi_k_gemv(fc1.type, fc1.dev, (int)fc1.ne1, d, fin, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, st));
                 if (!q4 && pi_k_sparse_ffn_supported(ff, (int)fc1.ne1, d)) {
                     PI_TRY(pi_k_sparse_ffn(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, down.dev, d,
-                                           m->ffn_inp, &fn, PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, nullptr, nullptr, m->n_active + il, m->ws, st));
+                                           fin, &fn, PI_EPI_ADD, fin, nullptr, m->x2, nullptr, nullptr, m->n_active + il, m->ws, st));
                     ++n;
                     continue;
                 }
                 PI_TRY(pi_k_predictor_fc2(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, nullptr, 0, m->pred_logits,
                                           q4 ? m->list : nullptr, q4 ? m->n_active + il : nullptr, q4 ? m->h_dense : nullptr, m->ws, st));
-                PI_TRY(pi_k_sparse_upgate(up.type, up.dev, falcon ? nullptr : gate.dev, d, ff, m->ffn_inp, &fn, q4 ? 0 : 1, m->list, m->n_active + il, nullptr, m->h_c,
+                PI_TRY(pi_k_sparse_upgate(up.type, up.dev, falcon ? nullptr : gate.dev, d, ff, fin, &fn, q4 ? 0 : 1, m->list, m->n_active + il, nullptr, m->h_c,
                                           q4 ? m->h_dense : nullptr, nullptr, nullptr, m->ws, st));
                 PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, ff, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, m->n_active + il,
                                         PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, m->ws, st));

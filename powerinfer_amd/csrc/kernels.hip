@@ -254,123 +254,155 @@ __global__ __launch_bounds__(kBlock) void gemv_f16_kernel(const __half * __restr
     }
 }
 
-// Register-resident variant for cols == 512 * NCH (4096, 5120, 8192 ...): a wave owns whole rows
+// Register-resident variant for cols == 512 * NCH (4096, 5120, 8192): a wave owns whole rows
 // (row = wave_id, wave_id + n_waves, ...), lane l holds the activations of columns 8*l + 512*j as packed fp16 in
-// registers, so the inner loop touches neither LDS nor a workgroup barrier.  Every wave normalises the whole
-// vector itself (64 lanes x 8*NCH values; double sums reduced by butterfly), which costs one L2 round trip
-// overlapped with the first row's weight loads.  Two rows of loads (2*NCH x 16 B per lane) are in flight.
-// The residual operands of the epilogue are fetched together with the row so that no load sits between the
-// reduction and the store.
-template <int NCH, int TAG>
-__global__ __launch_bounds__(kBlock) void gemv_f16_reg_kernel(const __half * __restrict__ W, const float * __restrict__ x, NormArgs na,
+// registers, so the row loop touches neither LDS nor a workgroup barrier.  The prologue is shared by the four
+// waves of a workgroup: wave w loads and normalises chunks w, w+4, ... of the vector (statistics cross the waves
+// through LDS in wave order), the packed fp16 result meets in LDS and every wave reads all of it back once.
+// 16 weight loads of 16 B per lane are in flight throughout (two rows, or the two halves of a wide row) and
+// are issued before the prologue starts.  The residual operands of the epilogue travel with the row.
+// KIND: 0 no norm, 1 RMSNorm * w, 2 LayerNorm * w + b.  TAG only names the role in kernel traces.
+template <int NCH, int KIND, int TAG>
+__global__ __launch_bounds__(kBlock, 2) void gemv_f16_reg_kernel(const __half * __restrict__ W, const float * __restrict__ x,
+                                                              const float * __restrict__ nw, const float * __restrict__ nb, float eps,
                                                               int epi, const float * __restrict__ add1, const float * __restrict__ add2,
                                                               float * __restrict__ y, int rows) {
     constexpr int cols = NCH * 512;
-    constexpr bool kEarlyW = NCH <= 8;            // registers allow the norm weights to travel with the activations
-    const int lane = threadIdx.x & 63;
-    const int n_waves = gridDim.x * kWavesPerBlock, wid = blockIdx.x * kWavesPerBlock + (threadIdx.x >> 6);
-    pi_u32x4 buf[2][NCH];
+    constexpr bool kWide = NCH > 8;               // wide rows: the two buffers hold the halves of one row
+    constexpr int CPB = kWide ? NCH / 2 : NCH;
+    static_assert(!kWide || NCH % 2 == 0, "wide rows are split in two halves");
+    constexpr int MYCH = (NCH + kWavesPerBlock - 1) / kWavesPerBlock;      // chunks a wave normalises
+    __shared__ __align__(16) __half xs[cols];
+    __shared__ double red[2][kWavesPerBlock];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n_waves = gridDim.x * kWavesPerBlock, wid = blockIdx.x * kWavesPerBlock + wave;
+    pi_u32x4 buf[2][CPB];
     float r1[2] = {0.0f, 0.0f}, r2[2] = {0.0f, 0.0f};
     auto issue = [&](int b, int r) {
         if (r < rows) {
-            const __half * wp = W + (size_t)r * cols + lane * 8;
+            const __half * wp = W + (size_t)r * cols + lane * 8 + (kWide ? b * CPB * 512 : 0);
 #pragma unroll
-            for (int j = 0; j < NCH; ++j) buf[b][j] = pi_ld_stream(wp + j * 512);
-            if (epi >= PI_EPI_ADD) r1[b] = add1[r];
-            if (epi == PI_EPI_ADD2) r2[b] = add2[r];
+            for (int j = 0; j < CPB; ++j) buf[b][j] = pi_ld_stream(wp + j * 512);
+            if (!kWide || b == 0) {
+                if (epi >= PI_EPI_ADD) r1[b] = add1[r];
+                if (epi == PI_EPI_ADD2) r2[b] = add2[r];
+            }
         }
     };
     issue(0, wid);
-    if (kEarlyW) issue(1, wid + n_waves);
+    issue(1, kWide ? wid : wid + n_waves);
 
-    pi_u32x4 xr[NCH];
+    // ---- shared prologue ---------------------------------------------------------------------------------
     {
-        float4 xv[NCH][2], wv[kEarlyW ? NCH : 1][2];
-        const bool has_w = na.kind != 0 && na.w != nullptr;
+        float xv[MYCH][8], wv[MYCH][8], bv[MYCH][8];
 #pragma unroll
-        for (int j = 0; j < NCH; ++j) {
-            xv[j][0] = *reinterpret_cast<const float4 *>(x + j * 512 + lane * 8);
-            xv[j][1] = *reinterpret_cast<const float4 *>(x + j * 512 + lane * 8 + 4);
-        }
-        if (kEarlyW && has_w) {
-#pragma unroll
-            for (int j = 0; j < NCH; ++j) {
-                wv[j][0] = *reinterpret_cast<const float4 *>(na.w + j * 512 + lane * 8);
-                wv[j][1] = *reinterpret_cast<const float4 *>(na.w + j * 512 + lane * 8 + 4);
+        for (int i = 0; i < MYCH; ++i) {
+            const int j = wave + i * kWavesPerBlock;
+            if (j < NCH) {
+                const int o = j * 512 + lane * 8;
+                const float4 a = *reinterpret_cast<const float4 *>(x + o), b = *reinterpret_cast<const float4 *>(x + o + 4);
+                xv[i][0] = a.x; xv[i][1] = a.y; xv[i][2] = a.z; xv[i][3] = a.w; xv[i][4] = b.x; xv[i][5] = b.y; xv[i][6] = b.z; xv[i][7] = b.w;
+                if (KIND >= 1) {
+                    const float4 c = *reinterpret_cast<const float4 *>(nw + o), e = *reinterpret_cast<const float4 *>(nw + o + 4);
+                    wv[i][0] = c.x; wv[i][1] = c.y; wv[i][2] = c.z; wv[i][3] = c.w; wv[i][4] = e.x; wv[i][5] = e.y; wv[i][6] = e.z; wv[i][7] = e.w;
+                }
+                if (KIND == 2) {
+                    const float4 c = *reinterpret_cast<const float4 *>(nb + o), e = *reinterpret_cast<const float4 *>(nb + o + 4);
+                    bv[i][0] = c.x; bv[i][1] = c.y; bv[i][2] = c.z; bv[i][3] = c.w; bv[i][4] = e.x; bv[i][5] = e.y; bv[i][6] = e.z; bv[i][7] = e.w;
+                }
             }
         }
         float mean = 0.0f, scale = 1.0f;
-        if (na.kind == 1) {
+        if (KIND >= 1) {
             double s = 0.0;
 #pragma unroll
-            for (int j = 0; j < NCH; ++j)
+            for (int i = 0; i < MYCH; ++i)
+                if (wave + i * kWavesPerBlock < NCH) {
 #pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const float4 v = xv[j][h];
-                    s += (double)__fmul_rn(v.x, v.x); s += (double)__fmul_rn(v.y, v.y); s += (double)__fmul_rn(v.z, v.z); s += (double)__fmul_rn(v.w, v.w);
+                    for (int k = 0; k < 8; ++k) s += KIND == 1 ? (double)__fmul_rn(xv[i][k], xv[i][k]) : (double)xv[i][k];
                 }
             s = pi_wave_sum_f64(s);
-            scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
-        } else if (na.kind == 2) {
-            double s = 0.0;
+            if (lane == 0) red[0][wave] = s;
+            __syncthreads();
+            double t = 0.0;
 #pragma unroll
-            for (int j = 0; j < NCH; ++j)
+            for (int w = 0; w < kWavesPerBlock; ++w) t += red[0][w];
+            if (KIND == 1) scale = 1.0f / sqrtf((float)(t / cols) + eps);
+            else {
+                mean = (float)(t / cols);
+                double s2 = 0.0;
 #pragma unroll
-                for (int h = 0; h < 2; ++h) { const float4 v = xv[j][h]; s += (double)v.x; s += (double)v.y; s += (double)v.z; s += (double)v.w; }
-            s = pi_wave_sum_f64(s);
-            mean = (float)(s / cols);
-            double s2 = 0.0;
+                for (int i = 0; i < MYCH; ++i)
+                    if (wave + i * kWavesPerBlock < NCH) {
 #pragma unroll
-            for (int j = 0; j < NCH; ++j)
-#pragma unroll
-                for (int h = 0; h < 2; ++h) {
-                    const float4 v = xv[j][h];
-                    const float a = __fsub_rn(v.x, mean), b = __fsub_rn(v.y, mean), c = __fsub_rn(v.z, mean), e = __fsub_rn(v.w, mean);
-                    s2 += (double)__fmul_rn(a, a); s2 += (double)__fmul_rn(b, b); s2 += (double)__fmul_rn(c, c); s2 += (double)__fmul_rn(e, e);
-                }
-            s2 = pi_wave_sum_f64(s2);
-            scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
-        }
-#pragma unroll
-        for (int j = 0; j < NCH; ++j) {
-            __half2 hh[4];
-#pragma unroll
-            for (int h = 0; h < 2; ++h) {
-                float4 v = xv[j][h];
-                if (na.kind != 0) {
-                    if (na.kind == 2) { v.x = __fsub_rn(v.x, mean); v.y = __fsub_rn(v.y, mean); v.z = __fsub_rn(v.z, mean); v.w = __fsub_rn(v.w, mean); }
-                    v.x = __fmul_rn(v.x, scale); v.y = __fmul_rn(v.y, scale); v.z = __fmul_rn(v.z, scale); v.w = __fmul_rn(v.w, scale);
-                    if (has_w) {
-                        const float4 w4 = kEarlyW ? wv[kEarlyW ? j : 0][h] : *reinterpret_cast<const float4 *>(na.w + j * 512 + lane * 8 + 4 * h);
-                        v.x = __fmul_rn(v.x, w4.x); v.y = __fmul_rn(v.y, w4.y); v.z = __fmul_rn(v.z, w4.z); v.w = __fmul_rn(v.w, w4.w);
+                        for (int k = 0; k < 8; ++k) { const float v = __fsub_rn(xv[i][k], mean); s2 += (double)__fmul_rn(v, v); }
                     }
-                    if (na.b) {
-                        const float4 b4 = *reinterpret_cast<const float4 *>(na.b + j * 512 + lane * 8 + 4 * h);
-                        v.x = __fadd_rn(v.x, b4.x); v.y = __fadd_rn(v.y, b4.y); v.z = __fadd_rn(v.z, b4.z); v.w = __fadd_rn(v.w, b4.w);
-                    }
-                }
-                hh[2 * h] = __floats2half2_rn(v.x, v.y); hh[2 * h + 1] = __floats2half2_rn(v.z, v.w);
+                s2 = pi_wave_sum_f64(s2);
+                if (lane == 0) red[1][wave] = s2;
+                __syncthreads();
+                double t2 = 0.0;
+#pragma unroll
+                for (int w = 0; w < kWavesPerBlock; ++w) t2 += red[1][w];
+                scale = 1.0f / sqrtf((float)(t2 / cols) + eps);
             }
-            xr[j] = *reinterpret_cast<const pi_u32x4 *>(hh);
         }
+#pragma unroll
+        for (int i = 0; i < MYCH; ++i) {
+            const int j = wave + i * kWavesPerBlock;
+            if (j < NCH) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    float v = xv[i][k];
+                    if (KIND >= 1) v = __fmul_rn(__fmul_rn(KIND == 2 ? __fsub_rn(v, mean) : v, scale), wv[i][k]);
+                    if (KIND == 2) v = __fadd_rn(v, bv[i][k]);
+                    xv[i][k] = v;
+                }
+                __half2 hh[4] = {__floats2half2_rn(xv[i][0], xv[i][1]), __floats2half2_rn(xv[i][2], xv[i][3]),
+                                 __floats2half2_rn(xv[i][4], xv[i][5]), __floats2half2_rn(xv[i][6], xv[i][7])};
+                *reinterpret_cast<pi_u32x4 *>(xs + j * 512 + lane * 8) = *reinterpret_cast<const pi_u32x4 *>(hh);
+            }
+        }
+        __syncthreads();
     }
-    if (!kEarlyW) issue(1, wid + n_waves);
+    pi_u32x4 xr[NCH];
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) xr[j] = *reinterpret_cast<const pi_u32x4 *>(xs + j * 512 + lane * 8);
 
-    for (int r = wid; r < rows; r += 2 * n_waves) {
+    auto finish = [&](float acc, float a1, float a2, int r) {
+        acc = pi_wave_sum(acc);
+        if (epi == PI_EPI_RELU) acc = fmaxf(acc, 0.0f);
+        else if (epi == PI_EPI_ADD) acc = __fadd_rn(acc, a1);
+        else if (epi == PI_EPI_ADD2) acc = __fadd_rn(__fadd_rn(acc, a1), a2);
+        if (lane == 0) y[r] = acc;
+    };
+    if constexpr (kWide) {
+        for (int r = wid; r < rows; r += n_waves) {
+            // keep the activations packed: widening them once outside the loop would double their register footprint
 #pragma unroll
-        for (int b = 0; b < 2; ++b) {
-            const int rr = r + b * n_waves;
-            if (rr < rows) {
-                float acc = 0.0f;
+            for (int j = 0; j < NCH; ++j) asm volatile("" : "+v"(xr[j].x), "+v"(xr[j].y), "+v"(xr[j].z), "+v"(xr[j].w));
+            float acc = 0.0f;
 #pragma unroll
-                for (int j = 0; j < NCH; ++j) acc = pi_dot8h(buf[b][j], xr[j], acc);
-                acc = pi_wave_sum(acc);
-                if (epi == PI_EPI_RELU) acc = fmaxf(acc, 0.0f);
-                else if (epi == PI_EPI_ADD) acc = __fadd_rn(acc, r1[b]);
-                else if (epi == PI_EPI_ADD2) acc = __fadd_rn(__fadd_rn(acc, r1[b]), r2[b]);
-                if (lane == 0) y[rr] = acc;
+            for (int j = 0; j < CPB; ++j) acc = pi_dot8h(buf[0][j], xr[j], acc);
+            const float a1 = r1[0], a2 = r2[0];
+            issue(0, r + n_waves);
+#pragma unroll
+            for (int j = 0; j < CPB; ++j) acc = pi_dot8h(buf[1][j], xr[CPB + j], acc);
+            issue(1, r + n_waves);
+            finish(acc, a1, a2, r);
+        }
+    } else {
+        for (int r = wid; r < rows; r += 2 * n_waves) {
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int rr = r + b * n_waves;
+                if (rr < rows) {
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < NCH; ++j) acc = pi_dot8h(buf[b][j], xr[j], acc);
+                    finish(acc, r1[b], r2[b], rr);
+                }
+                issue(b, rr + 2 * n_waves);
             }
-            issue(b, rr + 2 * n_waves);
         }
     }
 }
@@ -792,20 +824,21 @@ constexpr int kPfChunk = 8;                       // active neurons per round tr
 
 __device__ __forceinline__ int select_nth_bit(uint32_t bits, int n);
 
-template <int RCH, bool GATE>
+template <int CPW, int RCH, bool GATE>      // cols == 8 waves * CPW chunks * 512; r == RCH * 512
 __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
                                                                    const __half * __restrict__ Wup, const __half * __restrict__ Wgate,
                                                                    const __half * __restrict__ Wdown,
                                                                    const float * __restrict__ x, NormArgs na, float thr,
                                                                    float * __restrict__ logits, uint32_t * __restrict__ words, float * __restrict__ h_dense,
                                                                    float * __restrict__ partial) {
-    constexpr int cols = kPfWaves * 512, r = RCH * 512;
+    constexpr int cols = kPfWaves * CPW * 512, r = RCH * 512;
+    constexpr int CH = kPfChunk / CPW;                 // active neurons per round trip: 3*CPW*CH (2*CPW*CH) loads in flight per lane
     __shared__ float  lg[32];
     __shared__ double red[2][kPfWaves];
-    __shared__ float  part[kPfWaves][kPfChunk][2];
+    __shared__ float  part[kPfWaves][CH][2];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int n0 = blockIdx.x * 32;
-    const int cbase = wave * 512 + lane * 8;
+    const int cbase = wave * CPW * 512 + lane * 8;     // chunk c of this lane starts at column cbase + 512*c
 
     // ---- A: loads ------------------------------------------------------------------------------------------
     pi_u32x4 a[4][RCH];
@@ -819,17 +852,19 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
         hv[j][0] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8);
         hv[j][1] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8 + 4);
     }
-    float xs[8], ws[8], bs[8];
-    {
-        const float4 x0 = *reinterpret_cast<const float4 *>(x + cbase), x1 = *reinterpret_cast<const float4 *>(x + cbase + 4);
-        xs[0] = x0.x; xs[1] = x0.y; xs[2] = x0.z; xs[3] = x0.w; xs[4] = x1.x; xs[5] = x1.y; xs[6] = x1.z; xs[7] = x1.w;
+    float xs[CPW][8], ws[CPW][8], bs[CPW][8];
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+        const int o = cbase + c * 512;
+        const float4 x0 = *reinterpret_cast<const float4 *>(x + o), x1 = *reinterpret_cast<const float4 *>(x + o + 4);
+        xs[c][0] = x0.x; xs[c][1] = x0.y; xs[c][2] = x0.z; xs[c][3] = x0.w; xs[c][4] = x1.x; xs[c][5] = x1.y; xs[c][6] = x1.z; xs[c][7] = x1.w;
         if (na.kind != 0 && na.w) {
-            const float4 w0 = *reinterpret_cast<const float4 *>(na.w + cbase), w1 = *reinterpret_cast<const float4 *>(na.w + cbase + 4);
-            ws[0] = w0.x; ws[1] = w0.y; ws[2] = w0.z; ws[3] = w0.w; ws[4] = w1.x; ws[5] = w1.y; ws[6] = w1.z; ws[7] = w1.w;
+            const float4 w0 = *reinterpret_cast<const float4 *>(na.w + o), w1 = *reinterpret_cast<const float4 *>(na.w + o + 4);
+            ws[c][0] = w0.x; ws[c][1] = w0.y; ws[c][2] = w0.z; ws[c][3] = w0.w; ws[c][4] = w1.x; ws[c][5] = w1.y; ws[c][6] = w1.z; ws[c][7] = w1.w;
         }
         if (na.kind != 0 && na.b) {
-            const float4 b0 = *reinterpret_cast<const float4 *>(na.b + cbase), b1 = *reinterpret_cast<const float4 *>(na.b + cbase + 4);
-            bs[0] = b0.x; bs[1] = b0.y; bs[2] = b0.z; bs[3] = b0.w; bs[4] = b1.x; bs[5] = b1.y; bs[6] = b1.z; bs[7] = b1.w;
+            const float4 b0 = *reinterpret_cast<const float4 *>(na.b + o), b1 = *reinterpret_cast<const float4 *>(na.b + o + 4);
+            bs[c][0] = b0.x; bs[c][1] = b0.y; bs[c][2] = b0.z; bs[c][3] = b0.w; bs[c][4] = b1.x; bs[c][5] = b1.y; bs[c][6] = b1.z; bs[c][7] = b1.w;
         }
     }
     // ---- A: logits (the CPU path rounds the hidden vector to fp16 before the dot, ggml.c:9703-9716) ------------
@@ -855,7 +890,9 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
     if (na.kind == 1) {
         double sq = 0.0;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) sq += (double)__fmul_rn(xs[k], xs[k]);
+        for (int c = 0; c < CPW; ++c)
+#pragma unroll
+            for (int k = 0; k < 8; ++k) sq += (double)__fmul_rn(xs[c][k], xs[c][k]);
         sq = pi_wave_sum_f64(sq);
         if (lane == 0) red[0][wave] = sq;
         __syncthreads();
@@ -866,7 +903,9 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
     } else if (na.kind == 2) {
         double sm = 0.0;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) sm += (double)xs[k];
+        for (int c = 0; c < CPW; ++c)
+#pragma unroll
+            for (int k = 0; k < 8; ++k) sm += (double)xs[c][k];
         sm = pi_wave_sum_f64(sm);
         if (lane == 0) red[0][wave] = sm;
         __syncthreads();
@@ -876,7 +915,9 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
         mean = (float)(t / cols);
         double sq = 0.0;
 #pragma unroll
-        for (int k = 0; k < 8; ++k) { const float v = __fsub_rn(xs[k], mean); sq += (double)__fmul_rn(v, v); }
+        for (int c = 0; c < CPW; ++c)
+#pragma unroll
+            for (int k = 0; k < 8; ++k) { const float v = __fsub_rn(xs[c][k], mean); sq += (double)__fmul_rn(v, v); }
         sq = pi_wave_sum_f64(sq);
         if (lane == 0) red[1][wave] = sq;
         __syncthreads();
@@ -887,20 +928,22 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
     } else {
         __syncthreads();
     }
-    pi_u32x4 xr;
-    {
+    pi_u32x4 xr[CPW];
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
-            float v = xs[k];
+            float v = xs[c][k];
             if (na.kind != 0) {
                 v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
-                if (na.w) v = __fmul_rn(v, ws[k]);
-                if (na.b) v = __fadd_rn(v, bs[k]);
+                if (na.w) v = __fmul_rn(v, ws[c][k]);
+                if (na.b) v = __fadd_rn(v, bs[c][k]);
             }
-            xs[k] = v;
+            xs[c][k] = v;
         }
-        __half2 hh[4] = {__floats2half2_rn(xs[0], xs[1]), __floats2half2_rn(xs[2], xs[3]), __floats2half2_rn(xs[4], xs[5]), __floats2half2_rn(xs[6], xs[7])};
-        xr = *reinterpret_cast<const pi_u32x4 *>(hh);
+        __half2 hh[4] = {__floats2half2_rn(xs[c][0], xs[c][1]), __floats2half2_rn(xs[c][2], xs[c][3]),
+                         __floats2half2_rn(xs[c][4], xs[c][5]), __floats2half2_rn(xs[c][6], xs[c][7])};
+        xr[c] = *reinterpret_cast<const pi_u32x4 *>(hh);
     }
     // ---- activity word (identical in every wave; lg is complete after the barrier above) -----------------------
     const float my_logit = lg[lane & 31];
@@ -912,34 +955,42 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
     }
     // ---- B + C ---------------------------------------------------------------------------------------------
     const int n = __popc(mask);
-    float acc[8];
+    float acc[CPW][8];
 #pragma unroll
-    for (int k = 0; k < 8; ++k) acc[k] = 0.0f;
-    for (int c0 = 0; c0 < n; c0 += kPfChunk) {
-        const int nn = n - c0 < kPfChunk ? n - c0 : kPfChunk;
-        int rows[kPfChunk];
-        pi_u32x4 gu[kPfChunk], uu[kPfChunk], dd[kPfChunk];
+    for (int c = 0; c < CPW; ++c)
 #pragma unroll
-        for (int j = 0; j < kPfChunk; ++j) {
+        for (int k = 0; k < 8; ++k) acc[c][k] = 0.0f;
+    for (int c0 = 0; c0 < n; c0 += CH) {
+        const int nn = n - c0 < CH ? n - c0 : CH;
+        int rows[CH];
+        pi_u32x4 gu[CH][CPW], uu[CH][CPW], dd[CH][CPW];
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
             if (j < nn) {
                 rows[j] = n0 + select_nth_bit(mask, c0 + j);
                 const size_t off = (size_t)rows[j] * cols + cbase;
-                uu[j] = pi_ld_stream(Wup + off);
-                if (GATE) gu[j] = pi_ld_stream(Wgate + off);
-                dd[j] = pi_ld_stream(Wdown + off);
+#pragma unroll
+                for (int c = 0; c < CPW; ++c) {
+                    uu[j][c] = pi_ld_stream(Wup + off + c * 512);
+                    if (GATE) gu[j][c] = pi_ld_stream(Wgate + off + c * 512);
+                    dd[j][c] = pi_ld_stream(Wdown + off + c * 512);
+                }
             }
         }
 #pragma unroll
-        for (int j = 0; j < kPfChunk; ++j) {
+        for (int j = 0; j < CH; ++j) {
             if (j < nn) {
-                float pu = pi_wave_sum(pi_dot8h(uu[j], xr, 0.0f));
-                float pg = GATE ? pi_wave_sum(pi_dot8h(gu[j], xr, 0.0f)) : 0.0f;
+                float pu = 0.0f, pg = 0.0f;
+#pragma unroll
+                for (int c = 0; c < CPW; ++c) { pu = pi_dot8h(uu[j][c], xr[c], pu); if (GATE) pg = pi_dot8h(gu[j][c], xr[c], pg); }
+                pu = pi_wave_sum(pu);
+                if (GATE) pg = pi_wave_sum(pg);
                 if (lane == 0) { part[wave][j][0] = pu; part[wave][j][1] = pg; }
             }
         }
         __syncthreads();
 #pragma unroll
-        for (int j = 0; j < kPfChunk; ++j) {
+        for (int j = 0; j < CH; ++j) {
             if (j < nn) {
                 float u = 0.0f, g = 0.0f;
 #pragma unroll
@@ -947,17 +998,23 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
                 const float h = GATE ? __fmul_rn(fmaxf(g, 0.0f), u) : fmaxf(u, 0.0f);
                 if (h_dense && threadIdx.x == 0) h_dense[rows[j]] = h;
                 const float hq = pi_round_f16(h);                 // the CPU axpy rounds h to fp16 (ggml.c:14420-14431)
-                float wf[8];
-                pi_unpack8(dd[j], wf);
 #pragma unroll
-                for (int k = 0; k < 8; ++k) acc[k] = fmaf(wf[k], hq, acc[k]);
+                for (int c = 0; c < CPW; ++c) {
+                    float wf[8];
+                    pi_unpack8(dd[j][c], wf);
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) acc[c][k] = fmaf(wf[k], hq, acc[c][k]);
+                }
             }
         }
-        if (c0 + kPfChunk < n) __syncthreads();                   // part[] is reused by the next chunk
+        if (c0 + CH < n) __syncthreads();                         // part[] is reused by the next chunk
     }
-    float4 * po = reinterpret_cast<float4 *>(partial + (size_t)blockIdx.x * cols + cbase);
-    po[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
-    po[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+#pragma unroll
+    for (int c = 0; c < CPW; ++c) {
+        float4 * po = reinterpret_cast<float4 *>(partial + (size_t)blockIdx.x * cols + cbase + c * 512);
+        po[0] = make_float4(acc[c][0], acc[c][1], acc[c][2], acc[c][3]);
+        po[1] = make_float4(acc[c][4], acc[c][5], acc[c][6], acc[c][7]);
+    }
 }
 
 // out[c] = epi( sum over workgroups b (ascending within a fixed tree) of partial[b][c] ).  A workgroup of 8 waves owns
@@ -1781,6 +1838,33 @@ __global__ void fill_normal_f16_kernel(__half * __restrict__ p, size_t n, uint64
     }
 }
 
+// N(0, std^2) values quantised to Q4_0 exactly as quantize_row_q4_0_reference does (ggml-quants.c:428-463): the
+// element of largest magnitude (first one wins) sets d = max / -8, q = min(15, (int)(x / d + 8.5)).  One thread per block.
+__global__ void fill_normal_q4_0_kernel(pi_block_q4_0 * __restrict__ p, size_t n_blocks, uint64_t seed, float std) {
+    for (size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x; b < n_blocks; b += (size_t)gridDim.x * blockDim.x) {
+        float v[32];
+        float amax = 0.0f, mx = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            const uint64_t r = mix64(seed * 0xD1342543DE82EF95ull + b * 32 + j);
+            const float u1 = ((uint32_t)(r >> 32) + 1.0f) * (1.0f / 4294967296.0f);
+            const float u2 = (uint32_t)r * (1.0f / 4294967296.0f);
+            v[j] = pi_round_f16(sqrtf(-2.0f * logf(u1)) * cosf(6.28318530718f * u2) * std);
+            if (fabsf(v[j]) > amax) { amax = fabsf(v[j]); mx = v[j]; }
+        }
+        const float d = mx / -8.0f;
+        const float id = d != 0.0f ? 1.0f / d : 0.0f;
+        pi_block_q4_0 blk;
+        blk.d = pi_f16_bits(d);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int q0 = min(15, (int)(v[j] * id + 8.5f)), q1 = min(15, (int)(v[j + 16] * id + 8.5f));
+            blk.qs[j] = (uint8_t)(q0 | (q1 << 4));
+        }
+        p[b] = blk;
+    }
+}
+
 NormArgs to_norm(const pi_norm * n) {
     NormArgs a{0, 0.0f, nullptr, nullptr};
     if (n) { a.kind = n->kind; a.eps = n->eps; a.w = n->w; a.b = n->b; }
@@ -1850,16 +1934,19 @@ int pi_k_gemv(int wtype, const void * W, int rows, int cols, const float * x, co
                           (((uintptr_t)x | (uintptr_t)(norm ? norm->w : nullptr)) & 15) == 0;
         const bool aligned = (((uintptr_t)x | (uintptr_t)(norm ? norm->w : nullptr) | (uintptr_t)(norm ? norm->b : nullptr)) & 15) == 0;
         const int rblocks = rows >= n_waves ? kGemvBlocks : (rows + kWavesPerBlock - 1) / kWavesPerBlock;
-        if (aligned && cols == 4096) {
-            // the tag only names the role in kernel traces: lm-head, q|k|v, predictor fc1, attention output
-            if (rows >= 16384)     hipLaunchKernelGGL((gemv_f16_reg_kernel<8, 1>), dim3(rblocks), dim3(kBlock), 0, st, w, x, na, epilogue, add1, add2, y, rows);
-            else if (rows >= 8192) hipLaunchKernelGGL((gemv_f16_reg_kernel<8, 2>), dim3(rblocks), dim3(kBlock), 0, st, w, x, na, epilogue, add1, add2, y, rows);
-            else if (rows < 2048)  hipLaunchKernelGGL((gemv_f16_reg_kernel<8, 3>), dim3(rblocks), dim3(kBlock), 0, st, w, x, na, epilogue, add1, add2, y, rows);
-            else                   hipLaunchKernelGGL((gemv_f16_reg_kernel<8, 0>), dim3(rblocks), dim3(kBlock), 0, st, w, x, na, epilogue, add1, add2, y, rows);
-        } else if (aligned && cols == 5120) {
-            hipLaunchKernelGGL((gemv_f16_reg_kernel<10, 0>), dim3(rblocks), dim3(kBlock), 0, st, w, x, na, epilogue, add1, add2, y, rows);
-        } else if (aligned && cols == 8192) {
-            hipLaunchKernelGGL((gemv_f16_reg_kernel<16, 0>), dim3(rblocks), dim3(kBlock), 0, st, w, x, na, epilogue, add1, add2, y, rows);
+        // register-resident kernel: the norm must carry what its kind needs (RMSNorm a weight, LayerNorm weight and bias)
+        const bool reg_ok = aligned && (cols == 4096 || cols == 5120 || cols == 8192) &&
+                            (na.kind == 0 || (na.kind == 1 && na.w && !na.b) || (na.kind == 2 && na.w && na.b));
+        if (reg_ok) {
+            // the tag only names the role in kernel traces: 1 = lm-head sized, 2 = fewer rows than the grid has waves
+            const int tag = rows >= 16384 ? 1 : rows < n_waves ? 2 : 0;
+#define PI_GEMV_REG(NCH, KIND, TAG) hipLaunchKernelGGL((gemv_f16_reg_kernel<NCH, KIND, TAG>), dim3(rblocks), dim3(kBlock), 0, st, w, x, na.w, na.b, na.eps, epilogue, add1, add2, y, rows)
+#define PI_GEMV_REG_K(NCH, KIND) do { if (tag == 1) PI_GEMV_REG(NCH, KIND, 1); else if (tag == 2) PI_GEMV_REG(NCH, KIND, 2); else PI_GEMV_REG(NCH, KIND, 0); } while (0)
+#define PI_GEMV_REG_N(NCH) do { if (na.kind == 0) PI_GEMV_REG_K(NCH, 0); else if (na.kind == 1) PI_GEMV_REG_K(NCH, 1); else PI_GEMV_REG_K(NCH, 2); } while (0)
+            if (cols == 4096) PI_GEMV_REG_N(8); else if (cols == 5120) PI_GEMV_REG_N(10); else PI_GEMV_REG_N(16);
+#undef PI_GEMV_REG_N
+#undef PI_GEMV_REG_K
+#undef PI_GEMV_REG
         } else if (fast) {
             const size_t sh = stage_fast_lds_bytes(cols);
             if (rows >= 16384) hipLaunchKernelGGL((gemv_f16_kernel<4, 2, 1>), dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
@@ -2017,14 +2104,14 @@ int pi_k_sparse_axpy_dense(const void * down_t_f16, int cols, int ff, const floa
     return pi::check_launch("pi_k_sparse_axpy_dense");
 }
 
-int pi_k_sparse_ffn_supported(int ff, int r, int cols) { return cols == 4096 && (r == 1024 || r == 512) && ff > 0 && ff % 32 == 0; }
+int pi_k_sparse_ffn_supported(int ff, int r, int cols) { return (cols == 4096 || cols == 8192) && (r == 1024 || r == 512) && ff > 0 && ff % 32 == 0; }
 
 int pi_k_sparse_ffn(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
                     const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x, const pi_norm * norm,
                     int epilogue, const float * add1, const float * add2, float * out,
                     float * logits, float * h_dense, int32_t * n_active, pi_workspace * ws, pi_stream_t stream) {
     if (!fc2_f16 || !hidden || !up_f16 || !down_t_f16 || !x || !out || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: null pointer");
-    if (!pi_k_sparse_ffn_supported(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn: shape outside the fused kernel (cols 4096, r 512 or 1024, ff % 32 == 0)");
+    if (!pi_k_sparse_ffn_supported(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn: shape outside the fused kernel (cols 4096 or 8192, r 512 or 1024, ff % 32 == 0)");
     if (ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: shape exceeds the workspace");
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
         return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: bad epilogue arguments");
@@ -2034,13 +2121,13 @@ int pi_k_sparse_ffn(const void * fc2_f16, int ff, int r, const float * hidden, f
     const __half * w2 = (const __half *)fc2_f16; const __half * u = (const __half *)up_f16; const __half * g = (const __half *)gate_f16;
     const __half * dn = (const __half *)down_t_f16;
     const dim3 grid(ff / 32), block(kPfBlock);
-    if (r == 1024) {
-        if (g) hipLaunchKernelGGL((pred_ffn_f16_kernel<2, true>),  grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial);
-        else   hipLaunchKernelGGL((pred_ffn_f16_kernel<2, false>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial);
-    } else {
-        if (g) hipLaunchKernelGGL((pred_ffn_f16_kernel<1, true>),  grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial);
-        else   hipLaunchKernelGGL((pred_ffn_f16_kernel<1, false>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial);
-    }
+#define PI_PF_LAUNCH(CPW, RCH, GATE) hipLaunchKernelGGL((pred_ffn_f16_kernel<CPW, RCH, GATE>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial)
+    const int cpw = cols / 4096, rch = r / 512;
+    if (cpw == 1 && rch == 2) { if (g) PI_PF_LAUNCH(1, 2, true); else PI_PF_LAUNCH(1, 2, false); }
+    else if (cpw == 1)        { if (g) PI_PF_LAUNCH(1, 1, true); else PI_PF_LAUNCH(1, 1, false); }
+    else if (rch == 2)        { if (g) PI_PF_LAUNCH(2, 2, true); else PI_PF_LAUNCH(2, 2, false); }
+    else                      { if (g) PI_PF_LAUNCH(2, 1, true); else PI_PF_LAUNCH(2, 1, false); }
+#undef PI_PF_LAUNCH
     hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, st, ws->ffn_partial, ff / 32, cols, ws->words, ff / 32, n_active,
                        epilogue, add1, add2, out);
     return pi::check_launch("pi_k_sparse_ffn");
@@ -2107,6 +2194,15 @@ int pi_fill_normal_f16(void * dptr, size_t n, uint64_t seed, float std, const fl
     if (blocks > 65536) blocks = 65536;
     hipLaunchKernelGGL(fill_normal_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (__half *)dptr, n, seed, std, row_bias, cols);
     return pi::check_launch("pi_fill_normal_f16");
+}
+
+int pi_fill_normal_q4_0(void * dptr, size_t n_weights, uint64_t seed, float std, pi_stream_t stream) {
+    if (!dptr || n_weights % 32) return pi::fail(PI_E_ARG, "pi_fill_normal_q4_0: null pointer or a weight count that is not a multiple of 32");
+    if (n_weights == 0) return PI_OK;
+    size_t blocks = (n_weights / 32 + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(fill_normal_q4_0_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (pi_block_q4_0 *)dptr, n_weights / 32, seed, std);
+    return pi::check_launch("pi_fill_normal_q4_0");
 }
 
 }  // extern "C"

@@ -41,6 +41,7 @@ _SIGS = {
     "pi_memcpy_d2d": (_i, [_vp, _vp, _sz]),
     "pi_sync": (_i, []),
     "pi_fill_normal_f16": (_i, [_vp, _sz, _u64, _f, _vp, _i, _vp]),
+    "pi_fill_normal_q4_0": (_i, [_vp, _sz, _u64, _f, _vp]),
     "pi_event_create": (_vp, []),
     "pi_event_record": (_i, [_vp, _vp]),
     "pi_event_elapsed_ms": (_i, [_vp, _vp, C.POINTER(_f)]),

@@ -91,9 +91,19 @@ def test_ffn_7b_shape_vs_oracle(wtype, has_gate):
 def test_fused_routes_7b_shape(has_gate, norm, route):
     """pi_k_sparse_ffn (what the F16 decode loop runs at d = 4096) and pi_k_pred_upgate + pi_k_sparse_axpy_dense
     against the oracle, with the fused RMSNorm / LayerNorm prologue and the residual epilogue."""
+    run_fused_route(has_gate, norm, route, 4096, 11008, 1024)
+
+
+@pytest.mark.parametrize("has_gate,norm", [(False, 2), (True, 1)])
+def test_one_launch_route_wide_rows(has_gate, norm):
+    """The 8192-column instantiation (Falcon-40B width; each lane holds two 8-column chunks), rank-512 predictor."""
+    run_fused_route(has_gate, norm, "one", 8192, 4096, 512)
+
+
+def run_fused_route(has_gate, norm, route, d, ff, r):
     from powerinfer_amd import lib as pl
     from powerinfer_amd.ops import SparseFFN
-    d, ff, r, T = 4096, 11008, 1024, 3
+    T = 3
     L = synth.make_ffn_layer(seed=77 + norm, d=d, ff=ff, r=r, wtype=ol.F16, has_gate=has_gate, T=T)
     rng = np.random.default_rng(5)
     nw = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32) if norm else None

@@ -407,6 +407,180 @@ __global__ __launch_bounds__(kBlock, 2) void gemv_f16_reg_kernel(const __half * 
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Register-resident Q4_0 mat-vec for cols == 4096 * CB.  A Q4_0 row of 4096 weights is 128 blocks of 18 bytes =
+// 2304 bytes = 64 lanes x 36 bytes: lane l reads the block pair (2l, 2l+1) of each 4096-column group with two
+// 16-byte loads and one 4-byte load (4-byte aligned) and meets it with the matching 64 int8 activations, their two
+// Q8_0 scales and block sums, all held in registers.  The nibbles are used unsigned through v_dot4_i32_i8 and
+// 8 * sum(x) is subtracted per block, which is exact in int32; the result is scaled by d_w * d_x in fp32 as
+// vec_dot_q4_0_q8_0 does (ggml-quants.c:2512-2650).  The prologue (norm, then Q8_0 quantisation as the x86
+// quantize_row_q8_0 does: d = amax / 127 kept as fp16, q = rint(x * 127 / amax), ggml-quants.c:702-760) is shared by
+// the four waves through LDS.  Four rows (two for CB = 2) of loads are in flight per lane.
+// ---------------------------------------------------------------------------------------------------
+typedef uint32_t pi_u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+template <int CB, int KIND, int TAG>
+__global__ __launch_bounds__(kBlock, 2) void gemv_q4_reg_kernel(const unsigned char * __restrict__ W, const float * __restrict__ x,
+                                                             const float * __restrict__ nw, const float * __restrict__ nb, float eps,
+                                                             int epi, const float * __restrict__ add1, const float * __restrict__ add2,
+                                                             float * __restrict__ y, int rows) {
+    constexpr int cols = CB * 4096, NCH = cols / 512, nblk = cols / 32;
+    constexpr int NBUF = 4 / CB;
+    constexpr int MYCH = NCH / kWavesPerBlock;
+    constexpr size_t row_bytes = (size_t)nblk * 18;
+    __shared__ __align__(16) int8_t xq[cols];
+    __shared__ float xd[nblk];
+    __shared__ int   xsum[nblk];
+    __shared__ double red[2][kWavesPerBlock];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n_waves = gridDim.x * kWavesPerBlock, wid = blockIdx.x * kWavesPerBlock + wave;
+
+    uint32_t D[NBUF][CB][9];
+    float r1[NBUF], r2[NBUF];
+    auto issue = [&](int b, int r) {
+        if (r < rows) {
+#pragma unroll
+            for (int g = 0; g < CB; ++g) {
+                const unsigned char * p = W + (size_t)r * row_bytes + g * 2304 + lane * 36;
+                const pi_u32x4_a4 v0 = __builtin_nontemporal_load(reinterpret_cast<const pi_u32x4_a4 *>(p));
+                const pi_u32x4_a4 v1 = __builtin_nontemporal_load(reinterpret_cast<const pi_u32x4_a4 *>(p + 16));
+                D[b][g][0] = v0.x; D[b][g][1] = v0.y; D[b][g][2] = v0.z; D[b][g][3] = v0.w;
+                D[b][g][4] = v1.x; D[b][g][5] = v1.y; D[b][g][6] = v1.z; D[b][g][7] = v1.w;
+                D[b][g][8] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p + 32));
+            }
+            if (epi >= PI_EPI_ADD) r1[b] = add1[r];
+            if (epi == PI_EPI_ADD2) r2[b] = add2[r];
+        }
+    };
+#pragma unroll
+    for (int b = 0; b < NBUF; ++b) { r1[b] = 0.0f; r2[b] = 0.0f; issue(b, wid + b * n_waves); }
+
+    // ---- shared prologue: norm, Q8_0 quantisation -------------------------------------------------------------
+    {
+        float xv[MYCH][8], wv[MYCH][8], bv[MYCH][8];
+#pragma unroll
+        for (int i = 0; i < MYCH; ++i) {
+            const int o = (wave + i * kWavesPerBlock) * 512 + lane * 8;
+            const float4 a = *reinterpret_cast<const float4 *>(x + o), b = *reinterpret_cast<const float4 *>(x + o + 4);
+            xv[i][0] = a.x; xv[i][1] = a.y; xv[i][2] = a.z; xv[i][3] = a.w; xv[i][4] = b.x; xv[i][5] = b.y; xv[i][6] = b.z; xv[i][7] = b.w;
+            if (KIND >= 1) {
+                const float4 c = *reinterpret_cast<const float4 *>(nw + o), e = *reinterpret_cast<const float4 *>(nw + o + 4);
+                wv[i][0] = c.x; wv[i][1] = c.y; wv[i][2] = c.z; wv[i][3] = c.w; wv[i][4] = e.x; wv[i][5] = e.y; wv[i][6] = e.z; wv[i][7] = e.w;
+            }
+            if (KIND == 2) {
+                const float4 c = *reinterpret_cast<const float4 *>(nb + o), e = *reinterpret_cast<const float4 *>(nb + o + 4);
+                bv[i][0] = c.x; bv[i][1] = c.y; bv[i][2] = c.z; bv[i][3] = c.w; bv[i][4] = e.x; bv[i][5] = e.y; bv[i][6] = e.z; bv[i][7] = e.w;
+            }
+        }
+        float mean = 0.0f, scale = 1.0f;
+        if (KIND >= 1) {
+            double s = 0.0;
+#pragma unroll
+            for (int i = 0; i < MYCH; ++i)
+#pragma unroll
+                for (int k = 0; k < 8; ++k) s += KIND == 1 ? (double)__fmul_rn(xv[i][k], xv[i][k]) : (double)xv[i][k];
+            s = pi_wave_sum_f64(s);
+            if (lane == 0) red[0][wave] = s;
+            __syncthreads();
+            double t = 0.0;
+#pragma unroll
+            for (int w = 0; w < kWavesPerBlock; ++w) t += red[0][w];
+            if (KIND == 1) scale = 1.0f / sqrtf((float)(t / cols) + eps);
+            else {
+                mean = (float)(t / cols);
+                double s2 = 0.0;
+#pragma unroll
+                for (int i = 0; i < MYCH; ++i)
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) { const float v = __fsub_rn(xv[i][k], mean); s2 += (double)__fmul_rn(v, v); }
+                s2 = pi_wave_sum_f64(s2);
+                if (lane == 0) red[1][wave] = s2;
+                __syncthreads();
+                double t2 = 0.0;
+#pragma unroll
+                for (int w = 0; w < kWavesPerBlock; ++w) t2 += red[1][w];
+                scale = 1.0f / sqrtf((float)(t2 / cols) + eps);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MYCH; ++i) {
+            const int j = wave + i * kWavesPerBlock;
+            float amax = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                float v = xv[i][k];
+                if (KIND >= 1) v = __fmul_rn(__fmul_rn(KIND == 2 ? __fsub_rn(v, mean) : v, scale), wv[i][k]);
+                if (KIND == 2) v = __fadd_rn(v, bv[i][k]);
+                xv[i][k] = v;
+                amax = fmaxf(amax, fabsf(v));
+            }
+            // a quad of lanes holds one block of 32 values
+            amax = fmaxf(amax, pi_dpp_f32<PI_DPP_XOR1, 0xF>(amax));
+            amax = fmaxf(amax, pi_dpp_f32<PI_DPP_XOR2, 0xF>(amax));
+            const float d = amax / 127.0f;
+            const float id = (amax != 0.0f) ? 127.0f / amax : 0.0f;
+            int q[8], qs = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) { q[k] = (int)rintf(__fmul_rn(xv[i][k], id)); qs += q[k]; }
+            qs += pi_dpp_i32<PI_DPP_XOR1, 0xF>(qs);
+            qs += pi_dpp_i32<PI_DPP_XOR2, 0xF>(qs);
+            const uint32_t p0 = (uint32_t)(q[0] & 0xff) | ((uint32_t)(q[1] & 0xff) << 8) | ((uint32_t)(q[2] & 0xff) << 16) | ((uint32_t)(q[3] & 0xff) << 24);
+            const uint32_t p1 = (uint32_t)(q[4] & 0xff) | ((uint32_t)(q[5] & 0xff) << 8) | ((uint32_t)(q[6] & 0xff) << 16) | ((uint32_t)(q[7] & 0xff) << 24);
+            *reinterpret_cast<pi_u32x2 *>(xq + j * 512 + lane * 8) = pi_u32x2{p0, p1};
+            if ((lane & 3) == 0) { xd[j * 16 + (lane >> 2)] = pi_round_f16(d); xsum[j * 16 + (lane >> 2)] = qs; }
+        }
+        __syncthreads();
+    }
+    int   X[CB][16];
+    float dx[CB][2];
+    int   sx[CB][2];
+#pragma unroll
+    for (int g = 0; g < CB; ++g) {
+        const int b0 = g * 128 + 2 * lane;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const pi_u32x4 v = *reinterpret_cast<const pi_u32x4 *>(xq + b0 * 32 + k * 16);
+            X[g][4 * k] = (int)v.x; X[g][4 * k + 1] = (int)v.y; X[g][4 * k + 2] = (int)v.z; X[g][4 * k + 3] = (int)v.w;
+        }
+        dx[g][0] = xd[b0]; dx[g][1] = xd[b0 + 1];
+        sx[g][0] = xsum[b0]; sx[g][1] = xsum[b0 + 1];
+    }
+
+    for (int r = wid; r < rows; r += NBUF * n_waves) {
+#pragma unroll
+        for (int b = 0; b < NBUF; ++b) {
+            const int rr = r + b * n_waves;
+            if (rr < rows) {
+                float acc = 0.0f;
+#pragma unroll
+                for (int g = 0; g < CB; ++g) {
+                    const uint32_t * d9 = D[b][g];
+                    int s0 = 0, s1 = 0;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t q0 = __builtin_amdgcn_alignbit(d9[k + 1], d9[k], 16);       // bytes 2 + 4k .. 5 + 4k of the pair
+                        s0 = __builtin_amdgcn_sdot4((int)(q0 & 0x0F0F0F0Fu), X[g][k], s0, false);
+                        s0 = __builtin_amdgcn_sdot4((int)((q0 >> 4) & 0x0F0F0F0Fu), X[g][4 + k], s0, false);
+                        const uint32_t q1 = d9[5 + k];
+                        s1 = __builtin_amdgcn_sdot4((int)(q1 & 0x0F0F0F0Fu), X[g][8 + k], s1, false);
+                        s1 = __builtin_amdgcn_sdot4((int)((q1 >> 4) & 0x0F0F0F0Fu), X[g][12 + k], s1, false);
+                    }
+                    s0 -= 8 * sx[g][0];
+                    s1 -= 8 * sx[g][1];
+                    acc = fmaf(__fmul_rn(pi_f16_from_bits((uint16_t)(d9[0] & 0xffffu)), dx[g][0]), (float)s0, acc);
+                    acc = fmaf(__fmul_rn(pi_f16_from_bits((uint16_t)(d9[4] >> 16)), dx[g][1]), (float)s1, acc);
+                }
+                acc = pi_wave_sum(acc);
+                if (epi == PI_EPI_RELU) acc = fmaxf(acc, 0.0f);
+                else if (epi == PI_EPI_ADD) acc = __fadd_rn(acc, r1[b]);
+                else if (epi == PI_EPI_ADD2) acc = __fadd_rn(__fadd_rn(acc, r1[b]), r2[b]);
+                if (lane == 0) y[rr] = acc;
+            }
+            issue(b, rr + NBUF * n_waves);
+        }
+    }
+}
+
 // any shape with cols % 8 == 0: one wave per row, grid-stride
 __global__ __launch_bounds__(kBlock) void gemv_f16_generic_kernel(const __half * __restrict__ W, const float * __restrict__ x, NormArgs na,
                                                                   int epi, const float * add1, const float * add2,
@@ -1965,6 +2139,22 @@ int pi_k_gemv(int wtype, const void * W, int rows, int cols, const float * x, co
         const size_t sh = (size_t)cols + (size_t)(cols / 32) * 4 + (size_t)cols * 4;
         if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv: cols too large for LDS staging");
         const pi_block_q4_0 * w = (const pi_block_q4_0 *)W;
+        const bool aligned = (((uintptr_t)x | (uintptr_t)(norm ? norm->w : nullptr) | (uintptr_t)(norm ? norm->b : nullptr)) & 15) == 0 && ((uintptr_t)W & 3) == 0;
+        const bool reg_ok = aligned && (cols == 4096 || cols == 8192) &&
+                            (na.kind == 0 || (na.kind == 1 && na.w && !na.b) || (na.kind == 2 && na.w && na.b));
+        if (reg_ok) {
+            const int rblocks = rows >= n_waves ? kGemvBlocks : (rows + kWavesPerBlock - 1) / kWavesPerBlock;
+            const int tag = rows >= 16384 ? 1 : 0;
+            const unsigned char * wb = (const unsigned char *)W;
+#define PI_GEMV_Q4(CB, KIND, TAG) hipLaunchKernelGGL((gemv_q4_reg_kernel<CB, KIND, TAG>), dim3(rblocks), dim3(kBlock), 0, st, wb, x, na.w, na.b, na.eps, epilogue, add1, add2, y, rows)
+#define PI_GEMV_Q4_K(CB, KIND) do { if (tag == 1) PI_GEMV_Q4(CB, KIND, 1); else PI_GEMV_Q4(CB, KIND, 0); } while (0)
+#define PI_GEMV_Q4_N(CB) do { if (na.kind == 0) PI_GEMV_Q4_K(CB, 0); else if (na.kind == 1) PI_GEMV_Q4_K(CB, 1); else PI_GEMV_Q4_K(CB, 2); } while (0)
+            if (cols == 4096) PI_GEMV_Q4_N(1); else PI_GEMV_Q4_N(2);
+#undef PI_GEMV_Q4_N
+#undef PI_GEMV_Q4_K
+#undef PI_GEMV_Q4
+            return pi::check_launch("pi_k_gemv");
+        }
         if (rpw == 8)      hipLaunchKernelGGL(gemv_q4_kernel<8>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
         else if (rpw == 4) hipLaunchKernelGGL(gemv_q4_kernel<4>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
         else if (rpw == 2) hipLaunchKernelGGL(gemv_q4_kernel<2>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);

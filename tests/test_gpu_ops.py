@@ -36,7 +36,7 @@ def gpu_gemv(wtype, w, rows, cols, x, norm=None, epi=0, add1=None, add2=None):
 
 
 @pytest.mark.parametrize("wtype", [ol.F16, ol.Q4_0])
-@pytest.mark.parametrize("rows,cols", [(40, 256), (4096, 4096), (12288, 4096), (1024, 4096), (3000, 8192)])
+@pytest.mark.parametrize("rows,cols", [(40, 256), (4096, 4096), (12288, 4096), (1024, 4096), (3000, 8192), (2050, 5120)])
 def test_gemv_plain(wtype, rows, cols):
     rng = np.random.default_rng(rows + cols)
     w32 = (rng.standard_normal((rows, cols)) * 0.02).astype(np.float32)

@@ -1860,14 +1860,15 @@ __global__ void rope_table_kernel(float2 * __restrict__ table, int n_ctx, int ha
 // and attends over cells [0, pos) from the cache plus the new cell from LDS, so it never reads what this
 // launch writes; the first query head of each group stores k and v.
 // ---------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void attn_fused_kernel(const float * __restrict__ qkv, const float2 * __restrict__ rope_table,
+constexpr int kAttnBlock = 1024;        // 16 waves per head: 64 (hd 128) or 128 (hd 64) cache cells per pass
+__global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __restrict__ qkv, const float2 * __restrict__ rope_table,
                                                             __half * __restrict__ k_cache, __half * __restrict__ v_cache,
                                                             int n_head, int n_head_kv, int hd, int mode, int n_ctx,
                                                             const int32_t * __restrict__ pos_p, float * __restrict__ out) {
     extern __shared__ __align__(16) unsigned char smem[];
     float * s    = reinterpret_cast<float *>(smem);               // [n_ctx] scores, then probabilities
     float * part = s + n_ctx;                                     // [groups][hd]
-    float * qs   = part + (kBlock / (hd / 8)) * hd;               // [hd] rotated q, rounded to fp16
+    float * qs   = part + (kAttnBlock / (hd / 8)) * hd;               // [hd] rotated q, rounded to fp16
     float * kcur = qs + hd;                                       // [hd] rotated k of this position, rounded to fp16
     float * vcur = kcur + hd;                                     // [hd]
     __shared__ double red[16];
@@ -1901,7 +1902,7 @@ __global__ __launch_bounds__(kBlock) void attn_fused_kernel(const float * __rest
     __syncthreads();
 
     const int lpp = hd / 8;
-    const int sub = tid % lpp, grp = tid / lpp, ngrp = kBlock / lpp;
+    const int sub = tid % lpp, grp = tid / lpp, ngrp = kAttnBlock / lpp;
     const float scale = 1.0f / sqrtf((float)hd);
     float qf[8];
 #pragma unroll
@@ -1921,10 +1922,10 @@ __global__ __launch_bounds__(kBlock) void attn_fused_kernel(const float * __rest
     __syncthreads();
 
     float mx = -INFINITY;
-    for (int c = tid; c < n_kv; c += kBlock) mx = fmaxf(mx, s[c]);
+    for (int c = tid; c < n_kv; c += kAttnBlock) mx = fmaxf(mx, s[c]);
     mx = block_max_f32(mx, redf);
     double sum = 0.0;
-    for (int c = tid; c < n_kv; c += kBlock) {
+    for (int c = tid; c < n_kv; c += kAttnBlock) {
         const float e = pi_round_f16(expf(pi_round_f16(__fsub_rn(s[c], mx))));
         s[c] = e;
         sum += (double)e;
@@ -1950,7 +1951,7 @@ __global__ __launch_bounds__(kBlock) void attn_fused_kernel(const float * __rest
 #pragma unroll
     for (int i = 0; i < 8; ++i) part[grp * hd + sub * 8 + i] = acc[i];
     __syncthreads();
-    for (int e = tid; e < hd; e += kBlock) {
+    for (int e = tid; e < hd; e += kAttnBlock) {
         float v = part[e];
         for (int g = 1; g < ngrp; ++g) v += part[g * hd + e];
         out[(size_t)h * hd + e] = v;
@@ -2353,11 +2354,11 @@ int pi_k_rope_table(void * table, int n_ctx, int hd, float theta_scale, pi_strea
 int pi_k_attn_fused(const float * qkv, const void * rope_table, void * k_cache, void * v_cache, int n_head, int n_head_kv, int hd, int mode,
                     int n_ctx, const int32_t * pos, float * out, pi_stream_t stream) {
     if (!qkv || !rope_table || !k_cache || !v_cache || !pos || !out) return pi::fail(PI_E_ARG, "pi_k_attn_fused: null pointer");
-    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd % 8 || kBlock % (hd / 8) || PI_WAVE % (hd / 8) || hd / 2 + hd > kBlock || (mode != 0 && mode != 2))
+    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd % 8 || kAttnBlock % (hd / 8) || PI_WAVE % (hd / 8) || hd / 2 + hd > kAttnBlock || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_attn_fused: head size must be 8 * (a divisor of 64), at most 128; mode 0 or 2");
-    const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd + 3 * (size_t)hd);
+    const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kAttnBlock / (hd / 8)) * hd + 3 * (size_t)hd);
     if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused: context too long for the single-pass kernel");
-    hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head), dim3(kBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
+    hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
                        (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out);
     return pi::check_launch("pi_k_attn_fused");
 }

@@ -180,6 +180,27 @@ PI_API int pi_k_sparse_axpy_dense(const void * down_t_f16, int cols, int ff, con
                                   pi_workspace * ws, pi_stream_t stream);
 
 /*
+ * Batched decode step: T <= 16 tokens, one per sequence (examples/batched/batched.cpp:100-260 drives llama_decode with
+ * n_tokens = n_parallel).  The weights are streamed once per step; the dense mat-muls and the sparse gate/up run on the
+ * matrix cores (the batch >= 8 dense cross-over the reference takes through cuBLAS, ggml-cuda.cu:7717-7756, and its
+ * mul_mat_batch_sparse kernels, :6994-7034).  Vectors of a step are token-major: x[T][cols], y[T][rows].
+ *   pi_k_norm_round_f16: out_f16[t] = fp16(norm(x[t])) -- what the CPU path feeds every F16 dot (ggml.c:9703-9716).
+ *   pi_k_gemm_f16:       y[t][row] = epi( W[row] . xn[t] ), cols % 128 == 0; add1/add2 are [T][rows].
+ *   pi_k_batch_sparse_ffn: logits [T][ff] (from pi_k_gemm_f16 on fc2); union_rows/n_union receive the ascending list of
+ *     neurons active for at least one token (each weight row is read once for the whole step);
+ *     out[t] = epi( sum over union rows active for t of fp16(h[t][n]) * down_t[n][:] ), h as in pi_k_sparse_upgate;
+ *     cols % 512 == 0.  h_dense is reserved (pass NULL).
+ */
+PI_API int pi_k_norm_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, pi_stream_t stream);
+PI_API int pi_k_gemm_f16(const void * W_f16, int rows, int cols, const void * xn_f16, int T, int epilogue,
+                         const float * add1, const float * add2, float * y, pi_stream_t stream);
+PI_API int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold,
+                                 const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const void * xn_f16,
+                                 int epilogue, const float * add1, const float * add2, float * out,
+                                 int32_t * union_rows, int32_t * n_union, float * h_dense,
+                                 pi_workspace * ws, pi_stream_t stream);
+
+/*
  * RoPE on q and k of one token plus the KV-cache store (rope / rope_neox ggml-cuda.cu:4999,5027 and
  * cpy_f32_f16 :4944 for llm_build_kv_store, llama.cpp:4383).  qkv: fp32 [n_head*hd + 2*n_head_kv*hd]
  * (q | k | v).  mode 0 = adjacent pairs, 2 = NeoX halves.  The position is read from *pos (device).

@@ -2040,6 +2040,226 @@ __global__ void fill_normal_q4_0_kernel(pi_block_q4_0 * __restrict__ p, size_t n
     }
 }
 
+// =====================================================================================================
+// Batched decode (2..16 tokens per step, one per sequence).  Weights are still streamed once per step, so the
+// roofline stays HBM, but 16 dot products per weight would make the VALU the limit: the dense mat-muls and the
+// sparse gate/up run on the matrix cores (v_mfma_f32_16x16x32_f16: a tile of 16 weight rows x 16 tokens x 32
+// columns per instruction, fp32 accumulate).  Lane l holds, for row (token) l % 16, the 8 columns
+// 8 * (l / 16) .. + 8 of the 32-column slab of both operands, i.e. one 16-byte load each; the accumulator lane l
+// holds rows 4 * (l / 16) .. + 4 of column (token) l % 16.
+// Activations are normalised and rounded to fp16 once per mat-mul input by norm_round_f16_kernel (the CPU path rounds
+// them to fp16 before every dot, ggml.c:9703-9716) and read by every tile from L2.
+// =====================================================================================================
+typedef _Float16 pi_h8 __attribute__((ext_vector_type(8)));
+typedef float    pi_f4 __attribute__((ext_vector_type(4)));
+constexpr int kBtMaxT = 16;
+
+__global__ __launch_bounds__(kBlock) void norm_round_f16_kernel(const float * __restrict__ x, int cols, NormArgs na, __half * __restrict__ out) {
+    __shared__ double red[16];
+    const float * xt = x + (size_t)blockIdx.x * cols;
+    __half * ot = out + (size_t)blockIdx.x * cols;
+    float mean = 0.0f, scale = 1.0f;
+    if (na.kind == 1) {
+        double s = 0.0;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = xt[i]; s += (double)__fmul_rn(v, v); }
+        s = block_sum_f64(s, red);
+        scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
+    } else if (na.kind == 2) {
+        double s = 0.0;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) s += (double)xt[i];
+        s = block_sum_f64(s, red);
+        mean = (float)(s / cols);
+        double s2 = 0.0;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = __fsub_rn(xt[i], mean); s2 += (double)__fmul_rn(v, v); }
+        s2 = block_sum_f64(s2, red);
+        scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
+    }
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+        float v = xt[i];
+        if (na.kind != 0) {
+            v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
+            if (na.w) v = __fmul_rn(v, na.w[i]);
+            if (na.b) v = __fadd_rn(v, na.b[i]);
+        }
+        ot[i] = __float2half_rn(v);
+    }
+}
+
+// y[t][row] = epi( W[row] . xn[t] ), t < T <= 16.  A workgroup owns 16 rows; its four waves split the columns in
+// quarters (cols % 128 == 0) and merge their 16 x 16 accumulator tiles through LDS in wave order.
+constexpr int kGmUn = 8;
+__global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
+                                                              int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y) {
+    __shared__ float cs[kWavesPerBlock][16][17];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;
+    const int row0 = blockIdx.x * 16;
+    const int row = row0 + i < rows ? row0 + i : rows - 1;
+    const int tok = i < T ? i : T - 1;
+    const int kw = cols / kWavesPerBlock;
+    const __half * ap = W + (size_t)row * cols + wave * kw + g * 8;
+    const __half * bp = xn + (size_t)tok * cols + wave * kw + g * 8;
+    pi_f4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int steps = kw / 32;
+    for (int s0 = 0; s0 < steps; s0 += kGmUn) {
+        pi_u32x4 a[kGmUn], b[kGmUn];
+#pragma unroll
+        for (int u = 0; u < kGmUn; ++u)
+            if (s0 + u < steps) { a[u] = pi_ld_stream(ap + (s0 + u) * 32); b[u] = pi_ld16(bp + (s0 + u) * 32); }
+#pragma unroll
+        for (int u = 0; u < kGmUn; ++u)
+            if (s0 + u < steps) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a[u]), __builtin_bit_cast(pi_h8, b[u]), acc, 0, 0, 0);
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) cs[wave][4 * g + r][i] = acc[r];
+    __syncthreads();
+    const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
+    if (row0 + rr < rows && t < T) {
+        float sum = cs[0][rr][t];
+#pragma unroll
+        for (int w = 1; w < kWavesPerBlock; ++w) sum += cs[w][rr][t];
+        const size_t o = (size_t)t * rows + row0 + rr;
+        if (epi == PI_EPI_RELU) sum = fmaxf(sum, 0.0f);
+        else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
+        else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[o]), add2[o]);
+        y[o] = sum;
+    }
+}
+
+// union over the tokens of the step of the predictor's active sets: list of neurons active for at least one token,
+// ascending (single workgroup: wave ballot per 64 neurons, popcount prefix over the mask words)
+__global__ __launch_bounds__(1024) void union_active_kernel(const float * __restrict__ logits, int T, int ff, float thr,
+                                                            uint32_t * __restrict__ words, int32_t * __restrict__ list, int32_t * __restrict__ n_union) {
+    __shared__ int sred[17];
+    const int lane = threadIdx.x & 63;
+    for (int i0 = 0; i0 < ff; i0 += blockDim.x) {
+        const int i = i0 + threadIdx.x;
+        bool act = false;
+        if (i < ff) for (int t = 0; t < T; ++t) act = act || !(logits[(size_t)t * ff + i] < thr);
+        const unsigned long long m = __ballot(act);
+        if (lane == 0 && i < ff) words[i >> 5] = (uint32_t)m;
+        if (lane == 32 && i < ff) words[i >> 5] = (uint32_t)(m >> 32);
+    }
+    __syncthreads();
+    compact_from_words(words, ff, nullptr, 0, list, n_union, sred);
+}
+
+// sparse gate/up for the union rows: a workgroup gathers 16 rows of the union list into one MFMA tile (lane l reads
+// the row of list entry 16 * tile + l % 16), the four waves split the columns, then
+// hc[u][t] = active(t, row_u) ? relu(gate . x_t) * (up . x_t) : 0  (relu(up . x_t) without a gate).
+__global__ __launch_bounds__(kBlock) void batch_upgate_f16_kernel(const __half * __restrict__ Wup, const __half * __restrict__ Wgate, int cols,
+                                                                  const __half * __restrict__ xn, int T, const float * __restrict__ logits, int ff, float thr,
+                                                                  const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
+                                                                  float * __restrict__ hc) {
+    __shared__ float cu[kWavesPerBlock][16][17], cg[kWavesPerBlock][16][17];
+    const int n = *n_union;
+    const int u0 = blockIdx.x * 16;
+    if (u0 >= n) return;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;
+    const int row = list[u0 + i < n ? u0 + i : n - 1];
+    const int tok = i < T ? i : T - 1;
+    const int kw = cols / kWavesPerBlock;
+    const size_t aoff = (size_t)row * cols + wave * kw + g * 8;
+    const __half * bp = xn + (size_t)tok * cols + wave * kw + g * 8;
+    pi_f4 au = {0.0f, 0.0f, 0.0f, 0.0f}, ag = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int steps = kw / 32;
+    constexpr int UN = 4;
+    for (int s0 = 0; s0 < steps; s0 += UN) {
+        pi_u32x4 a[UN], c[UN], b[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+            if (s0 + u < steps) {
+                a[u] = pi_ld_stream(Wup + aoff + (s0 + u) * 32);
+                if (Wgate) c[u] = pi_ld_stream(Wgate + aoff + (s0 + u) * 32);
+                b[u] = pi_ld16(bp + (s0 + u) * 32);
+            }
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+            if (s0 + u < steps) {
+                au = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a[u]), __builtin_bit_cast(pi_h8, b[u]), au, 0, 0, 0);
+                if (Wgate) ag = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, c[u]), __builtin_bit_cast(pi_h8, b[u]), ag, 0, 0, 0);
+            }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) { cu[wave][4 * g + r][i] = au[r]; cg[wave][4 * g + r][i] = ag[r]; }
+    __syncthreads();
+    const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
+    float h = 0.0f;
+    if (u0 + rr < n && t < T) {
+        const int rrow = list[u0 + rr];
+        if (!(logits[(size_t)t * ff + rrow] < thr)) {
+            float su = cu[0][rr][t], sg = cg[0][rr][t];
+#pragma unroll
+            for (int w = 1; w < kWavesPerBlock; ++w) { su += cu[w][rr][t]; sg += cg[w][rr][t]; }
+            h = Wgate ? __fmul_rn(fmaxf(sg, 0.0f), su) : fmaxf(su, 0.0f);
+        }
+    }
+    hc[(size_t)(u0 + rr) * kBtMaxT + t] = h;
+}
+
+// sparse down projection for the step: partial[g][t][c] = sum over union entries u = g, g + G, ... of fp16(hc[u][t]) * down[row_u][c].
+// A wave owns 512 columns (8 per lane) and one of G row groups; 16 tokens x 8 columns of fp32 accumulators per lane.
+constexpr int kBaGroups = 32;
+__global__ __launch_bounds__(kBlock) void batch_axpy_f16_kernel(const __half * __restrict__ Wd, int cols, const float * __restrict__ hc,
+                                                                const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
+                                                                float * __restrict__ partial) {
+    const int n = *n_union;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int grp = blockIdx.y * kWavesPerBlock + wave;
+    const int c0 = blockIdx.x * 512 + lane * 8;
+    float acc[kBtMaxT][8];
+#pragma unroll
+    for (int t = 0; t < kBtMaxT; ++t)
+#pragma unroll
+        for (int k = 0; k < 8; ++k) acc[t][k] = 0.0f;
+    constexpr int UN = 4;
+    for (int u0 = grp; u0 < n; u0 += kBaGroups * UN) {
+        pi_u32x4 w[UN];
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            const int u = u0 + j * kBaGroups;
+            w[j] = u < n ? pi_ld_stream(Wd + (size_t)list[u] * cols + c0) : pi_u32x4{0u, 0u, 0u, 0u};
+        }
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            const int u = u0 + j * kBaGroups;
+            if (u < n) {
+                float wf[8];
+                pi_unpack8(w[j], wf);
+                const float4 * hp = reinterpret_cast<const float4 *>(hc + (size_t)u * kBtMaxT);
+#pragma unroll
+                for (int q = 0; q < 4; ++q) {
+                    const float4 h4 = hp[q];
+                    const float hh[4] = {pi_round_f16(h4.x), pi_round_f16(h4.y), pi_round_f16(h4.z), pi_round_f16(h4.w)};
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) acc[4 * q + e][k] = fmaf(wf[k], hh[e], acc[4 * q + e][k]);
+                }
+            }
+        }
+    }
+#pragma unroll
+    for (int t = 0; t < kBtMaxT; ++t) {
+        float4 * po = reinterpret_cast<float4 *>(partial + ((size_t)grp * kBtMaxT + t) * cols + c0);
+        po[0] = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
+        po[1] = make_float4(acc[t][4], acc[t][5], acc[t][6], acc[t][7]);
+    }
+}
+
+__global__ __launch_bounds__(kBlock) void batch_reduce_kernel(const float * __restrict__ partial, int T, int cols, int epi,
+                                                              const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ out) {
+    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    if (idx >= T * cols) return;
+    const int t = idx / cols, c = idx - t * cols;
+    float sum = 0.0f;
+    for (int g = 0; g < kBaGroups; ++g) sum += partial[((size_t)g * kBtMaxT + t) * cols + c];
+    if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[idx]);
+    else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[idx]), add2[idx]);
+    out[idx] = sum;
+}
+
 NormArgs to_norm(const pi_norm * n) {
     NormArgs a{0, 0.0f, nullptr, nullptr};
     if (n) { a.kind = n->kind; a.eps = n->eps; a.w = n->w; a.b = n->b; }
@@ -2058,7 +2278,8 @@ struct pi_workspace {
     float *        partial;        // [kAxpyGroups][max_d]
     int32_t *      hq;             // [max_ff]  Q4_0 axpy: int8 value of h per active row
     float *        hd;             // [max_ff]  and its Q8_0 block scale
-    float *        ffn_partial;    // [max_ff/32][max_d]  per-workgroup partial outputs of the fused sparse FFN
+    float *        ffn_partial;    // [max(max_ff/32, 32 * 16)][max_d]  partial outputs of the fused sparse FFN / of the batched axpy
+    float *        hc_batch;       // [max_ff][16]  h of the union rows for a batched step
 };
 constexpr int kAxpyGroups = 32;
 
@@ -2073,8 +2294,10 @@ pi_workspace * pi_workspace_create(int max_ff, int max_d) {
     ws->partial  = (float *)pi_malloc(sizeof(float) * (size_t)kAxpyGroups * max_d);
     ws->hq       = (int32_t *)pi_malloc(sizeof(int32_t) * max_ff);
     ws->hd       = (float *)pi_malloc(sizeof(float) * max_ff);
-    ws->ffn_partial = (float *)pi_malloc(sizeof(float) * (size_t)((max_ff + 31) / 32) * max_d);
-    if (!ws->words || !ws->counters || !ws->partial || !ws->hq || !ws->hd || !ws->ffn_partial) {
+    const size_t n_part = (size_t)((max_ff + 31) / 32) > (size_t)kBaGroups * kBtMaxT ? (size_t)((max_ff + 31) / 32) : (size_t)kBaGroups * kBtMaxT;
+    ws->ffn_partial = (float *)pi_malloc(sizeof(float) * n_part * max_d);
+    ws->hc_batch = (float *)pi_malloc(sizeof(float) * ((size_t)max_ff + 16) * kBtMaxT);
+    if (!ws->words || !ws->counters || !ws->partial || !ws->hq || !ws->hd || !ws->ffn_partial || !ws->hc_batch) {
         pi_workspace_destroy(ws); return nullptr;
     }
     pi_memset(ws->counters, 0, sizeof(unsigned int) * 64);
@@ -2082,7 +2305,7 @@ pi_workspace * pi_workspace_create(int max_ff, int max_d) {
 }
 int pi_workspace_destroy(pi_workspace * ws) {
     if (!ws) return PI_OK;
-    pi_free(ws->words); pi_free(ws->counters); pi_free(ws->partial); pi_free(ws->hq); pi_free(ws->hd); pi_free(ws->ffn_partial);
+    pi_free(ws->words); pi_free(ws->counters); pi_free(ws->partial); pi_free(ws->hq); pi_free(ws->hd); pi_free(ws->ffn_partial); pi_free(ws->hc_batch);
     delete ws;
     return PI_OK;
 }
@@ -2322,6 +2545,42 @@ int pi_k_sparse_ffn(const void * fc2_f16, int ff, int r, const float * hidden, f
     hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, st, ws->ffn_partial, ff / 32, cols, ws->words, ff / 32, n_active,
                        epilogue, add1, add2, out);
     return pi::check_launch("pi_k_sparse_ffn");
+}
+
+int pi_k_norm_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, pi_stream_t stream) {
+    if (!x || !out_f16 || T <= 0 || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_norm_round_f16: bad arguments");
+    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(kBlock), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16);
+    return pi::check_launch("pi_k_norm_round_f16");
+}
+
+int pi_k_gemm_f16(const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
+                  float * y, pi_stream_t stream) {
+    if (!W || !xn_f16 || !y || rows <= 0) return pi::fail(PI_E_ARG, "pi_k_gemm_f16: null pointer or empty shape");
+    if (T < 1 || T > kBtMaxT || cols <= 0 || cols % 128) return pi::fail(PI_E_ARG, "pi_k_gemm_f16: 1 <= T <= 16 and cols % 128 == 0 required");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_gemm_f16: bad epilogue arguments");
+    hipLaunchKernelGGL(gemm_t16_f16_kernel, dim3((rows + 15) / 16), dim3(kBlock), 0, (hipStream_t)stream,
+                       (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y);
+    return pi::check_launch("pi_k_gemm_f16");
+}
+
+int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, const void * up_f16, const void * gate_f16, const void * down_t_f16,
+                          int cols, const void * xn_f16, int epilogue, const float * add1, const float * add2, float * out,
+                          int32_t * union_rows, int32_t * n_union, float * h_dense, pi_workspace * ws, pi_stream_t stream) {
+    if (!logits || !up_f16 || !down_t_f16 || !xn_f16 || !out || !union_rows || !n_union || !ws) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: null pointer");
+    if (T < 1 || T > kBtMaxT || ff <= 0 || ff > ws->max_ff || cols <= 0 || cols > ws->max_d || cols % 512)
+        return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: 1 <= T <= 16, ff <= workspace, cols % 512 == 0 and cols <= workspace required");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: bad epilogue arguments");
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, logits, T, ff, threshold, ws->words, union_rows, n_union);
+    hipLaunchKernelGGL(batch_upgate_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
+                       (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch);
+    hipLaunchKernelGGL(batch_axpy_f16_kernel, dim3(cols / 512, kBaGroups / kWavesPerBlock), dim3(kBlock), 0, st, (const __half *)down_t_f16, cols,
+                       ws->hc_batch, union_rows, n_union, ws->ffn_partial);
+    hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, T, cols, epilogue, add1, add2, out);
+    (void)h_dense;
+    return pi::check_launch("pi_k_batch_sparse_ffn");
 }
 
 int pi_k_rope_kv_store(const float * qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale,

@@ -1,0 +1,116 @@
+"""Batched decode step kernels (T <= 16 tokens, one per sequence) through the C ABI against the CPU oracle:
+dense mat-mul on the matrix cores, and the sparse FFN over the union of the tokens' active sets."""
+import numpy as np
+import pytest
+
+import oracle_lib as ol
+from oracle_lib import _ptr as P
+from powerinfer_amd import synth
+
+pytestmark = pytest.mark.gpu
+
+
+def rel_err(a, b):
+    return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
+
+
+def gpu_norm_round(pl, L, x, norm=None):
+    T, cols = x.shape
+    dx, dn = pl.DevBuf(host=np.ascontiguousarray(x, np.float32)), pl.DevBuf(T * cols * 2)
+    keep, na = [], None
+    if norm is not None:
+        kind, eps, nw, nb = norm
+        bw = pl.DevBuf(host=nw) if nw is not None else None
+        bb = pl.DevBuf(host=nb) if nb is not None else None
+        keep += [bw, bb]
+        na = pl.norm_arg(kind, eps, bw, bb)
+    pl.check(L.pi_k_norm_round_f16(dx.ptr, T, cols, na, dn.ptr, None), "norm_round")
+    pl.sync()
+    return dn
+
+
+@pytest.mark.parametrize("rows,cols,T", [(3000, 5120, 16), (4096, 4096, 7), (13824, 1280, 16), (70, 128, 1)])
+def test_gemm_matches_oracle(rows, cols, T):
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    rng = np.random.default_rng(rows + cols + T)
+    w = (rng.standard_normal((rows, cols)) * 0.02).astype(np.float16)
+    x = rng.standard_normal((T, cols)).astype(np.float32)
+    a1 = rng.standard_normal((T, rows)).astype(np.float32)
+    want = np.zeros((T, rows), np.float32)
+    assert ol.oracle().pio_mul_mat(ol.F16, P(w), rows, cols, P(x), T, P(want), 8) == 0
+    dn = gpu_norm_round(pl, L, x)
+    assert np.array_equal(dn.download(np.float16).reshape(T, cols), x.astype(np.float16))
+    dw, dy, d1 = pl.DevBuf(host=w), pl.DevBuf(T * rows * 4), pl.DevBuf(host=a1)
+    pl.check(L.pi_k_gemm_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_NONE, None, None, dy.ptr, None), "gemm")
+    pl.sync()
+    got = dy.download(np.float32).reshape(T, rows)
+    assert rel_err(got, want) < 5e-6
+    pl.check(L.pi_k_gemm_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_ADD, d1.ptr, None, dy.ptr, None), "gemm")
+    pl.sync()
+    assert rel_err(dy.download(np.float32).reshape(T, rows), want + a1) < 5e-6
+    pl.check(L.pi_k_gemm_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_RELU, None, None, dy.ptr, None), "gemm")
+    pl.sync()
+    assert rel_err(dy.download(np.float32).reshape(T, rows), np.maximum(want, 0)) < 5e-6
+
+
+@pytest.mark.parametrize("kind", [1, 2])
+def test_norm_round_matches_oracle(kind):
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    rng = np.random.default_rng(kind)
+    T, cols = 5, 5120
+    x = (rng.standard_normal((T, cols)) * 2 + 0.3).astype(np.float32)
+    nw = (1 + 0.1 * rng.standard_normal(cols)).astype(np.float32)
+    nb = (0.1 * rng.standard_normal(cols)).astype(np.float32) if kind == 2 else None
+    O = ol.oracle()
+    xn = np.zeros_like(x)
+    (O.pio_rms_norm if kind == 1 else O.pio_norm)(P(x), cols, T, 1e-5, P(xn))
+    xn = xn * nw + (nb if nb is not None else 0)
+    got = gpu_norm_round(pl, L, x, norm=(kind, 1e-5, nw, nb)).download(np.float16).reshape(T, cols).astype(np.float32)
+    want = xn.astype(np.float32).astype(np.float16).astype(np.float32)
+    # identical up to fp16 rounding ties on a handful of elements
+    assert (got != want).mean() < 1e-3
+    assert rel_err(got, want) < 1e-3
+
+
+@pytest.mark.parametrize("shape,has_gate,T", [((5120, 13824, 1280), True, 16), ((4096, 11008, 1024), False, 5)])
+def test_batch_sparse_ffn_matches_oracle(shape, has_gate, T):
+    """Config 3's FFN block (13B shape, 16 tokens): each weight row of the union of active sets is read once."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    d, ff, r = shape
+    Lr = synth.make_ffn_layer(seed=31 + T, d=d, ff=ff, r=r, wtype=ol.F16, has_gate=has_gate, mean_rate=0.11, T=T)
+    x = Lr["x"]
+    O = ol.oracle()
+    o = ol.ffn_sparse(O, d, ff, r, T, ol.F16, has_gate, Lr["up"], Lr["gate"], Lr["down_t"], Lr["fc1"], Lr["fc2"], x, x,
+                      np.zeros(ff, np.int32), 0.0, nth=8)
+    ws = L.pi_workspace_create(ff, d)
+    assert ws
+    up, down, fc1, fc2 = (pl.DevBuf(host=Lr[k]) for k in ("up", "down_t", "fc1", "fc2"))
+    gate = pl.DevBuf(host=Lr["gate"]) if has_gate else None
+    xn = gpu_norm_round(pl, L, x)
+    hidden, hid16 = pl.DevBuf(T * r * 4), pl.DevBuf(T * r * 2)
+    logits, out = pl.DevBuf(T * ff * 4), pl.DevBuf(T * d * 4)
+    union, n_union = pl.DevBuf(ff * 4), pl.DevBuf.zeros(4)
+    resid = np.random.default_rng(3).standard_normal((T, d)).astype(np.float32)
+    dres = pl.DevBuf(host=resid)
+    pl.check(L.pi_k_gemm_f16(fc1.ptr, r, d, xn.ptr, T, pl.EPI_RELU, None, None, hidden.ptr, None), "fc1")
+    pl.check(L.pi_k_norm_round_f16(hidden.ptr, T, r, None, hid16.ptr, None), "round hidden")
+    pl.check(L.pi_k_gemm_f16(fc2.ptr, ff, r, hid16.ptr, T, pl.EPI_NONE, None, None, logits.ptr, None), "fc2")
+    pl.check(L.pi_k_batch_sparse_ffn(logits.ptr, T, ff, 0.0, up.ptr, gate.ptr if gate else None, down.ptr, d, xn.ptr,
+                                     pl.EPI_ADD, dres.ptr, None, out.ptr, union.ptr, n_union.ptr, None, ws, None), "batch ffn")
+    pl.sync()
+    lg = logits.download(np.float32).reshape(T, ff)
+    assert rel_err(lg, o["logits"]) < 1e-4
+    mask_g, mask_o = ~(lg < 0.0), ~(o["logits"] < 0.0)
+    assert (mask_g == mask_o).mean() >= 0.999
+    n = int(n_union.download(np.int32)[0])
+    assert np.array_equal(union.download(np.int32, n), np.nonzero(mask_g.any(0))[0])      # ascending union list, bit-exact for this mask
+    got = out.download(np.float32).reshape(T, d) - resid
+    for t in range(T):
+        if np.array_equal(mask_g[t], mask_o[t]):
+            assert rel_err(got[t], o["out"][t]) < 2e-3
+            assert rel_err(got[t], o["out"][t]) < 1e-4
+    assert sum(np.array_equal(mask_g[t], mask_o[t]) for t in range(T)) >= T - 2
+    L.pi_workspace_destroy(ws)

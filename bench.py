@@ -155,6 +155,49 @@ def cpu_baseline(hp, keep, prompt, n_prompt, n_decode, threads):
     return n_decode / dt
 
 
+def bench_batched(args):
+    """configs[3]: 13B shape, 16 sequences advancing one token per step; the whole-job rate counts every sequence's token."""
+    from powerinfer_amd import lib as pl, synth
+    n_seq = 16
+    n_prompt = 512 if args.prompt == 64 else args.prompt
+    steps = 128 if args.steps == 256 else args.steps
+    hp = synth.hparams("llama-13b", n_layer=40 if args.layers == 32 else args.layers, n_ctx=n_prompt + args.warmup + steps + 8, seed=1)
+    keep = []
+    m = build_synthetic_on_device(hp, keep)
+    m.batch_init(n_seq)
+    rng = np.random.default_rng(2024)
+    prompt = rng.integers(0, hp.n_vocab, (n_prompt, n_seq)).astype(np.int32)
+    for s in range(n_prompt):                                   # prompt phase (not timed): one position of every sequence per step
+        m.batch_decode(prompt[s], np.full(n_seq, s, np.int32), want_logits=False)
+    if args.warmup > 0:
+        m.batch_generate(args.warmup)
+    pl.sync()
+    t0 = time.perf_counter()
+    toks, ms_dev = m.batch_generate(steps)
+    pl.sync()
+    wall = time.perf_counter() - t0
+    union = m.batch_union().astype(np.float64)
+    d, ff, r = hp.n_embd, hp.n_ff, hp.n_rank
+    n_kv = n_prompt + args.warmup + (steps + 1) / 2.0
+    step_bytes = hp.n_layer * (4 * d * d * 2.0 + (d * r + r * ff) * 2.0 + n_seq * 2 * n_kv * d * 2.0) + union.sum() * 3 * d * 2.0 + hp.n_vocab * d * 2.0
+    ms_step = wall * 1e3 / steps
+    out = {
+        "metric": "decode tok/s, 16 sequences, ProSparse-Llama2-13B shape FP16", "value": round(n_seq * 1e3 / ms_step, 1), "unit": "tok/s",
+        "n_gpus": 1, "steps": steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "config": {"workload": "configs[3]: ProSparse-LLaMA-2-13B shape (d 5120, ff 13824, 40 heads, vocab 32000, predictor rank 1280), "
+                               f"{hp.n_layer} layers, random-init FP16 weights, all neurons on the GPU, {n_seq} sequences with {n_prompt}-token random "
+                               "prompts, greedy decode in lockstep (one token per sequence per step)",
+                   "n_layer": hp.n_layer, "n_seq": n_seq, "prompt_tokens": n_prompt, "n_ctx": hp.n_ctx,
+                   "mean_union_rows_per_layer": round(union.mean(), 1), "device": pl.device_name()},
+        "token_loop": {"device_ms_per_step": round(ms_dev / steps, 4), "touched_GB_per_step": round(step_bytes / 1e9, 3),
+                       "effective_GBps": round(step_bytes / (ms_step * 1e-3) / 1e9, 1),
+                       "hbm_frac_touched": round(step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
+    }
+    m.close()
+    print(json.dumps(out), flush=True)
+
+
 def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
@@ -164,9 +207,10 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="only for quick trials; the reported workload uses 32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--cpu-tokens", type=int, default=24)
-    ap.add_argument("--config", type=int, default=1, choices=[1, 2, 4],
+    ap.add_argument("--config", type=int, default=1, choices=[1, 2, 3, 4],
                     help="BASELINE configs index: 1 (default, the reported metric) 7B FP16 all on the GPU; 2 the same shape in "
-                         "Q4_0 with the hottest 60 %% of neurons on the GPU and the rest on host threads; 4 Falcon-40B shape FP16")
+                         "Q4_0 with the hottest 60 %% of neurons on the GPU and the rest on host threads; 3 ProSparse-LLaMA-2-13B shape FP16, "
+                         "16 sequences decoded in lockstep; 4 Falcon-40B shape FP16")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter-collection aid: run only the q|k|v mat-vec of a 4-layer model a few times plus one "
                          "device-to-device copy of the same byte count (the known-size reference for FETCH_SIZE / WRITE_SIZE)")
@@ -197,8 +241,12 @@ def main():
         hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_ctx, seed=1)
     elif args.config == 2:
         hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_ctx, seed=1, wtype=pl.Q4_0, hot_frac=0.6)
+    elif args.config == 3:
+        hp = None
     else:
         hp = synth.hparams("falcon-40b", n_layer=60 if args.layers == 32 else args.layers, n_ctx=n_ctx, seed=1)
+    if args.config == 3:
+        return bench_batched(args)
     hybrid = hp.hot_frac < 1.0
     keep = []
     t0 = time.perf_counter()

@@ -200,6 +200,17 @@ PI_API int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float thre
                                  int32_t * union_rows, int32_t * n_union, float * h_dense,
                                  pi_workspace * ws, pi_stream_t stream);
 
+/* per-sequence pieces of a batched step: sequence t owns token t, position pos[t] and the cache at t * cache_seq_stride
+ * (elements); pi_k_argmax_batch picks each sequence's next token (first maximum wins), stores it in tokens[t], adds 1 to
+ * positions[t] and records it at out_tokens[*step][t]; pi_k_step_advance then moves *step on. */
+PI_API int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache,
+                                 size_t cache_seq_stride, int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx,
+                                 const int32_t * pos, float * out, int out_stride, pi_stream_t stream);
+PI_API int pi_k_embed_batch(const void * table_f16, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream);
+PI_API int pi_k_argmax_batch(const float * logits, int n, int T, int32_t * tokens, int32_t * positions, int32_t * step,
+                             int32_t * out_tokens, int max_steps, pi_stream_t stream);
+PI_API int pi_k_step_advance(int32_t * step, pi_stream_t stream);
+
 /*
  * RoPE on q and k of one token plus the KV-cache store (rope / rope_neox ggml-cuda.cu:4999,5027 and
  * cpy_f32_f16 :4944 for llm_build_kv_store, llama.cpp:4383).  qkv: fp32 [n_head*hd + 2*n_head_kv*hd]
@@ -294,6 +305,18 @@ PI_API int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, fl
  * [n_layer][n_embd] (before the residual add), predictor logits [n_layer][n_ff], active-row count [n_layer]
  * and the vector the FFN block read [n_layer][n_embd] (LLaMA: ffn_inp; Falcon: the layer input; both before
  * the norm; it is also the predictor's input).  Any output pointer may be NULL. */
+/*
+ * Batched greedy decoding: n_seq <= 16 independent sequences advance one token per step (examples/batched/batched.cpp:100-260).
+ * F16 models with every neuron on the GPU.  pi_model_batch_init allocates one KV cache per sequence and the step buffers;
+ * pi_model_batch_decode feeds tokens[t] of sequence t at positions[t] and returns each sequence's greedy next token (and,
+ * if logits_out != NULL, the [n_seq][n_vocab] logits); pi_model_batch_generate continues greedily from that state for
+ * n_steps steps and returns out_tokens[n_steps][n_seq].
+ */
+PI_API int pi_model_batch_init(pi_model * m, int n_seq);
+PI_API int pi_model_batch_decode(pi_model * m, const int32_t * tokens, const int32_t * positions, int32_t * next_tokens, float * logits_out);
+PI_API int pi_model_batch_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * ms_out);
+PI_API int pi_model_batch_union(pi_model * m, int32_t * n_union_per_layer);   /* union sizes of the last step, [n_layer] */
+
 PI_API int pi_model_set_capture(pi_model * m, int enable);
 PI_API int pi_model_get_capture(pi_model * m, float * ffn_out, float * pred_logits, int32_t * n_active, float * ffn_src);
 

@@ -257,6 +257,7 @@ void pi_model_free(pi_model * m) {
     if (m->ev0) (void)hipEventDestroy(m->ev0);
     if (m->ev1) (void)hipEventDestroy(m->ev1);
     if (m->cold) pi::cold_destroy(m->cold);
+    pi::batch_destroy(m);
     if (m->ws) pi_workspace_destroy(m->ws);
     for (void * p : m->owned) pi_free(p);
     if (m->stream) (void)hipStreamDestroy(m->stream);

@@ -1,0 +1,210 @@
+// Batched greedy decoding on top of the single-sequence engine's weights: n_seq <= 16 independent sequences advance one
+// token per step (what examples/batched/batched.cpp:100-260 drives through llama_decode with n_tokens = n_parallel).
+// Per layer: activations are normalised + rounded to fp16 once per mat-mul input, dense mat-muls and the sparse gate/up
+// run on the matrix cores, every weight row of the union of the sequences' active sets is read once per step.
+#include "engine_internal.hpp"
+#include "runtime.hpp"
+
+#include <stdlib.h>
+
+struct BatchState {
+    int n_seq = 0, max_steps = 4096;
+    size_t cache_seq_stride = 0;          // elements per sequence: n_layer * n_head_kv * n_ctx * hd
+    __half *k_cache = nullptr, *v_cache = nullptr;
+    float *x = nullptr, *x2 = nullptr, *qkv = nullptr, *att = nullptr, *attn_out = nullptr, *ffn_inp = nullptr, *hidden = nullptr;
+    float *pred_logits = nullptr, *logits = nullptr;
+    __half *xa16 = nullptr, *xf16 = nullptr, *xp16 = nullptr, *att16 = nullptr, *hid16 = nullptr;
+    int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_step = nullptr, *d_out_tokens = nullptr, *union_rows = nullptr, *n_union = nullptr;
+    hipGraphExec_t graph_exec = nullptr;
+    hipGraph_t graph = nullptr;
+};
+
+namespace {
+
+#define PI_TRY(expr) do { int _rc = (expr); if (_rc != PI_OK) return _rc; } while (0)
+
+pi_norm mk_norm(int kind, float eps, const Tensor & w, const Tensor * b) {
+    pi_norm n{kind, eps, (const float *)w.dev, b ? (const float *)b->dev : nullptr};
+    return n;
+}
+
+int batch_layer(pi_model * m, int il) {
+    BatchState * b = m->batch;
+    const pi_hparams & hp = m->hp;
+    const int T = b->n_seq, d = hp.n_embd, ff = hp.n_ff, hd = m->hd, gqa = m->gqa;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    hipStream_t st = m->stream;
+    Tensor & wqkv = m->L(il, PI_T_WQKV); Tensor & wo = m->L(il, PI_T_WO);
+    Tensor & fc1 = m->L(il, PI_T_FC1); Tensor & fc2 = m->L(il, PI_T_FC2);
+    Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
+    const int r = (int)fc1.ne1;
+    const size_t kv_off = (size_t)il * hp.n_head_kv * hp.n_ctx * hd;
+    float * x = b->x;
+
+    // attention
+    pi_norm an;
+    if (!falcon) an = mk_norm(1, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), nullptr);
+    else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
+    else an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
+    PI_TRY(pi_k_norm_round_f16(x, T, d, &an, b->xa16, st));
+    PI_TRY(pi_k_gemm_f16(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, st));
+    PI_TRY(pi_k_attn_fused_batch(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
+                                 hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, hp.n_ctx, b->d_pos, b->att, d, st));
+    PI_TRY(pi_k_norm_round_f16(b->att, T, d, nullptr, b->att16, st));
+
+    const float * pred_in; pi_norm fn;
+    if (!falcon) {
+        PI_TRY(pi_k_gemm_f16(wo.dev, d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, st));       // ffn_inp = wo.att + x
+        pred_in = b->ffn_inp;
+        fn = mk_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
+    } else {
+        PI_TRY(pi_k_gemm_f16(wo.dev, d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, st));
+        pred_in = x;                                       // Falcon: predictor and FFN read the layer input
+        fn = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
+    }
+    // predictor
+    PI_TRY(pi_k_norm_round_f16(pred_in, T, d, nullptr, b->xp16, st));
+    PI_TRY(pi_k_gemm_f16(fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, st));
+    PI_TRY(pi_k_norm_round_f16(b->hidden, T, r, nullptr, b->hid16, st));
+    PI_TRY(pi_k_gemm_f16(fc2.dev, ff, r, b->hid16, T, PI_EPI_NONE, nullptr, nullptr, b->pred_logits, st));
+    // sparse FFN over the union of the sequences' active sets
+    PI_TRY(pi_k_norm_round_f16(pred_in, T, d, &fn, b->xf16, st));
+    if (!falcon)
+        PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, gate.dev, down.dev, d, b->xf16, PI_EPI_ADD, b->ffn_inp, nullptr,
+                                     b->x2, b->union_rows, b->n_union + il, nullptr, m->ws, st));
+    else
+        PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, nullptr, down.dev, d, b->xf16, PI_EPI_ADD2, b->attn_out, x,
+                                     b->x2, b->union_rows, b->n_union + il, nullptr, m->ws, st));
+    std::swap(b->x, b->x2);
+    return PI_OK;
+}
+
+int batch_step(pi_model * m) {
+    BatchState * b = m->batch;
+    const pi_hparams & hp = m->hp;
+    const int T = b->n_seq, d = hp.n_embd;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    hipStream_t st = m->stream;
+    PI_TRY(pi_k_embed_batch(m->glob[PI_T_TOK_EMBD].dev, d, b->d_tokens, T, b->x, st));
+    for (int il = 0; il < hp.n_layer; ++il) PI_TRY(batch_layer(m, il));
+    pi_norm on = mk_norm(falcon ? 2 : 1, hp.norm_eps, m->glob[PI_T_OUTPUT_NORM], falcon ? &m->glob[PI_T_OUTPUT_NORM_B] : nullptr);
+    PI_TRY(pi_k_norm_round_f16(b->x, T, d, &on, b->xa16, st));
+    PI_TRY(pi_k_gemm_f16(m->glob[PI_T_OUTPUT].dev, hp.n_vocab, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->logits, st));
+    PI_TRY(pi_k_argmax_batch(b->logits, hp.n_vocab, T, b->d_tokens, b->d_pos, b->d_step, b->d_out_tokens, b->max_steps, st));
+    PI_TRY(pi_k_step_advance(b->d_step, st));
+    return PI_OK;
+}
+
+}  // namespace
+
+namespace pi {
+void batch_destroy(pi_model * m) {
+    if (!m->batch) return;
+    if (m->batch->graph_exec) (void)hipGraphExecDestroy(m->batch->graph_exec);
+    if (m->batch->graph) (void)hipGraphDestroy(m->batch->graph);
+    delete m->batch;                      // device buffers are owned by the model's allocation list
+    m->batch = nullptr;
+}
+}  // namespace pi
+
+extern "C" {
+
+int pi_model_batch_init(pi_model * m, int n_seq) {
+    if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_batch_init: model not finalized");
+    if (n_seq < 1 || n_seq > 16) return pi::fail(PI_E_ARG, "pi_model_batch_init: 1 <= n_seq <= 16");
+    if (m->batch) return pi::fail(PI_E_STATE, "pi_model_batch_init: already initialised");
+    const pi_hparams & hp = m->hp;
+    const int d = hp.n_embd, ff = hp.n_ff;
+    if (m->hybrid) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: hybrid models decode one sequence at a time");
+    if (!m->rope_table) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: head size outside the fused attention kernel");
+    const int r = (int)m->L(0, PI_T_FC1).ne1;
+    for (int il = 0; il < hp.n_layer; ++il)
+        for (int k : {PI_T_WQKV, PI_T_WO, PI_T_FC1, PI_T_FC2, PI_T_FFN_UP, PI_T_FFN_DOWN_T})
+            if (m->L(il, k).type != PI_TYPE_F16) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: batched decoding needs F16 weights");
+    if (m->glob[PI_T_TOK_EMBD].type != PI_TYPE_F16 || m->glob[PI_T_OUTPUT].type != PI_TYPE_F16)
+        return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: batched decoding needs F16 weights");
+    if (d % 512 || r % 128) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: n_embd % 512 == 0 and predictor rank % 128 == 0 required");
+    BatchState * b = new BatchState();
+    b->n_seq = n_seq;
+    b->cache_seq_stride = (size_t)hp.n_layer * hp.n_head_kv * hp.n_ctx * m->hd;
+    const size_t T = n_seq;
+    b->k_cache = m->alloc<__half>(b->cache_seq_stride * T); b->v_cache = m->alloc<__half>(b->cache_seq_stride * T);
+    b->x = m->alloc<float>(T * d); b->x2 = m->alloc<float>(T * d); b->qkv = m->alloc<float>(T * (d + 2 * m->gqa));
+    b->att = m->alloc<float>(T * d); b->attn_out = m->alloc<float>(T * d); b->ffn_inp = m->alloc<float>(T * d);
+    b->hidden = m->alloc<float>(T * r); b->pred_logits = m->alloc<float>(T * ff); b->logits = m->alloc<float>(T * hp.n_vocab);
+    b->xa16 = m->alloc<__half>(T * d); b->xf16 = m->alloc<__half>(T * d); b->xp16 = m->alloc<__half>(T * d);
+    b->att16 = m->alloc<__half>(T * d); b->hid16 = m->alloc<__half>(T * r);
+    b->d_tokens = m->alloc<int32_t>(T); b->d_pos = m->alloc<int32_t>(T); b->d_step = m->alloc<int32_t>(1);
+    b->d_out_tokens = m->alloc<int32_t>((size_t)b->max_steps * T); b->union_rows = m->alloc<int32_t>(ff); b->n_union = m->alloc<int32_t>(hp.n_layer);
+    if (!b->k_cache || !b->v_cache || !b->x || !b->x2 || !b->qkv || !b->att || !b->attn_out || !b->ffn_inp || !b->hidden || !b->pred_logits || !b->logits ||
+        !b->xa16 || !b->xf16 || !b->xp16 || !b->att16 || !b->hid16 || !b->d_tokens || !b->d_pos || !b->d_step || !b->d_out_tokens || !b->union_rows || !b->n_union) {
+        delete b;
+        return PI_E_HIP;
+    }
+    PI_HIP_TRY(hipMemsetAsync(b->k_cache, 0, sizeof(__half) * b->cache_seq_stride * T, m->stream));
+    PI_HIP_TRY(hipMemsetAsync(b->v_cache, 0, sizeof(__half) * b->cache_seq_stride * T, m->stream));
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    m->batch = b;
+    return PI_OK;
+}
+
+int pi_model_batch_decode(pi_model * m, const int32_t * tokens, const int32_t * positions, int32_t * next_tokens, float * logits_out) {
+    if (!m || !m->batch) return pi::fail(PI_E_STATE, "pi_model_batch_decode: pi_model_batch_init first");
+    if (!tokens || !positions) return pi::fail(PI_E_ARG, "pi_model_batch_decode: null pointer");
+    BatchState * b = m->batch;
+    for (int t = 0; t < b->n_seq; ++t) {
+        if (tokens[t] < 0 || tokens[t] >= m->hp.n_vocab) return pi::fail(PI_E_ARG, "pi_model_batch_decode: token id out of range");
+        if (positions[t] < 0 || positions[t] >= m->hp.n_ctx) return pi::fail(PI_E_ARG, "pi_model_batch_decode: position outside the context");
+    }
+    PI_HIP_TRY(hipMemcpyAsync(b->d_tokens, tokens, sizeof(int32_t) * b->n_seq, hipMemcpyHostToDevice, m->stream));
+    PI_HIP_TRY(hipMemcpyAsync(b->d_pos, positions, sizeof(int32_t) * b->n_seq, hipMemcpyHostToDevice, m->stream));
+    PI_HIP_TRY(hipMemsetAsync(b->d_step, 0, 4, m->stream));
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));          // the host arrays may be pageable: finish the copies before returning control
+    PI_TRY(batch_step(m));
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    if (next_tokens) PI_TRY(pi_memcpy_d2h(next_tokens, b->d_tokens, sizeof(int32_t) * b->n_seq));
+    if (logits_out) PI_TRY(pi_memcpy_d2h(logits_out, b->logits, sizeof(float) * (size_t)b->n_seq * m->hp.n_vocab));
+    return PI_OK;
+}
+
+int pi_model_batch_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * ms_out) {
+    if (!m || !m->batch) return pi::fail(PI_E_STATE, "pi_model_batch_generate: pi_model_batch_init first");
+    BatchState * b = m->batch;
+    if (n_steps <= 0 || n_steps > b->max_steps || !out_tokens) return pi::fail(PI_E_ARG, "pi_model_batch_generate: bad step count");
+    std::vector<int32_t> pos(b->n_seq);
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    PI_TRY(pi_memcpy_d2h(pos.data(), b->d_pos, sizeof(int32_t) * b->n_seq));
+    for (int t = 0; t < b->n_seq; ++t)
+        if (pos[t] + n_steps > m->hp.n_ctx) return pi::fail(PI_E_ARG, "pi_model_batch_generate: would run past the context");
+    PI_HIP_TRY(hipMemsetAsync(b->d_step, 0, 4, m->stream));
+    const char * no_graph = getenv("PI_NO_GRAPH");
+    const bool use_graph = !(no_graph && no_graph[0] == '1');
+    if (use_graph && !b->graph_exec) {
+        PI_HIP_TRY(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
+        const int rc = batch_step(m);
+        hipGraph_t g = nullptr;
+        const hipError_t e = hipStreamEndCapture(m->stream, &g);
+        if (rc != PI_OK) { if (g) (void)hipGraphDestroy(g); return rc; }
+        if (e != hipSuccess) return pi::hip_fail(e, "hipStreamEndCapture");
+        b->graph = g;
+        PI_HIP_TRY(hipGraphInstantiate(&b->graph_exec, g, nullptr, nullptr, 0));
+    }
+    PI_HIP_TRY(hipEventRecord(m->ev0, m->stream));
+    for (int s = 0; s < n_steps; ++s) {
+        if (use_graph) PI_HIP_TRY(hipGraphLaunch(b->graph_exec, m->stream));
+        else PI_TRY(batch_step(m));
+    }
+    PI_HIP_TRY(hipEventRecord(m->ev1, m->stream));
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    if (ms_out) PI_HIP_TRY(hipEventElapsedTime(ms_out, m->ev0, m->ev1));
+    PI_TRY(pi_memcpy_d2h(out_tokens, b->d_out_tokens, sizeof(int32_t) * (size_t)n_steps * b->n_seq));
+    return PI_OK;
+}
+
+int pi_model_batch_union(pi_model * m, int32_t * n_union_per_layer) {
+    if (!m || !m->batch || !n_union_per_layer) return pi::fail(PI_E_ARG, "pi_model_batch_union: bad arguments");
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    return pi_memcpy_d2h(n_union_per_layer, m->batch->n_union, sizeof(int32_t) * m->hp.n_layer);
+}
+
+}  // extern "C"

@@ -18,6 +18,8 @@ struct Tensor {
 };
 
 
+struct BatchState;
+
 struct pi_model {
     pi_hparams hp{};
     std::vector<Tensor> layers;           // [n_layer][PI_T_COUNT]
@@ -43,6 +45,7 @@ struct pi_model {
     bool capture = false;
     float *cap_ffn = nullptr, *cap_logits = nullptr, *cap_src = nullptr;       // device
     pi::ColdPath * cold = nullptr;
+    BatchState * batch = nullptr;         // per-sequence caches and step buffers of batched decoding
 
     Tensor & L(int il, int kind) { return layers[(size_t)il * PI_T_COUNT + kind]; }
 
@@ -53,3 +56,6 @@ struct pi_model {
     }
 };
 
+namespace pi {
+void batch_destroy(pi_model * m);       // frees the batched-decoding state (graphs; device buffers belong to the model)
+}

@@ -1864,7 +1864,14 @@ constexpr int kAttnBlock = 1024;        // 16 waves per head: 64 (hd 128) or 128
 __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __restrict__ qkv, const float2 * __restrict__ rope_table,
                                                             __half * __restrict__ k_cache, __half * __restrict__ v_cache,
                                                             int n_head, int n_head_kv, int hd, int mode, int n_ctx,
-                                                            const int32_t * __restrict__ pos_p, float * __restrict__ out) {
+                                                            const int32_t * __restrict__ pos_p, float * __restrict__ out,
+                                                            int qkv_stride, size_t cache_seq_stride, int out_stride) {
+    // blockIdx.y = sequence of a batched step (its own token, position and cache); 0 for single-sequence decoding
+    qkv += (size_t)blockIdx.y * qkv_stride;
+    k_cache += (size_t)blockIdx.y * cache_seq_stride;
+    v_cache += (size_t)blockIdx.y * cache_seq_stride;
+    out += (size_t)blockIdx.y * out_stride;
+    pos_p += blockIdx.y;
     extern __shared__ __align__(16) unsigned char smem[];
     float * s    = reinterpret_cast<float *>(smem);               // [n_ctx] scores, then probabilities
     float * part = s + n_ctx;                                     // [groups][hd]
@@ -2260,6 +2267,40 @@ __global__ __launch_bounds__(kBlock) void batch_reduce_kernel(const float * __re
     out[idx] = sum;
 }
 
+__global__ void embed_f16_batch_kernel(const __half * __restrict__ table, int cols, const int32_t * __restrict__ tokens, float * __restrict__ x) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c < cols) x[(size_t)blockIdx.y * cols + c] = __half2float(table[(size_t)tokens[blockIdx.y] * cols + c]);
+}
+
+// greedy choice per sequence (first maximum wins, llama.cpp:8617-8631), then the sequence's state moves on: its next token,
+// its position + 1; workgroup 0 also advances the step counter after recording the step's tokens.
+__global__ __launch_bounds__(1024) void argmax_batch_kernel(const float * __restrict__ logits, int n, int T, int32_t * __restrict__ tokens,
+                                                            int32_t * __restrict__ positions, int32_t * __restrict__ step,
+                                                            int32_t * __restrict__ out_tokens, int max_steps) {
+    __shared__ float bv[16];
+    __shared__ int   bi[16];
+    const int t = blockIdx.x;
+    const float * lg = logits + (size_t)t * n;
+    float best = -INFINITY; int idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) { const float v = lg[i]; if (v > best) { best = v; idx = i; } }
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, PI_WAVE); const int oi = __shfl_xor(idx, o, PI_WAVE);
+        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+    }
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) { bv[wave] = best; bi[wave] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; ++w) if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
+        tokens[t] = idx;
+        if (positions) positions[t] += 1;
+        const int s = step ? *step : 0;
+        if (out_tokens && s < max_steps) out_tokens[(size_t)s * T + t] = idx;
+    }
+}
+
+__global__ void step_advance_kernel(int32_t * step) { if (threadIdx.x == 0) *step += 1; }
+
 NormArgs to_norm(const pi_norm * n) {
     NormArgs a{0, 0.0f, nullptr, nullptr};
     if (n) { a.kind = n->kind; a.eps = n->eps; a.w = n->w; a.b = n->b; }
@@ -2618,8 +2659,40 @@ int pi_k_attn_fused(const float * qkv, const void * rope_table, void * k_cache, 
     const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kAttnBlock / (hd / 8)) * hd + 3 * (size_t)hd);
     if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused: context too long for the single-pass kernel");
     hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
-                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out);
+                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, 0, (size_t)0, 0);
     return pi::check_launch("pi_k_attn_fused");
+}
+
+int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache, size_t cache_seq_stride,
+                          int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, const int32_t * pos, float * out, int out_stride,
+                          pi_stream_t stream) {
+    if (!qkv || !rope_table || !k_cache || !v_cache || !pos || !out || n_seq <= 0 || n_seq > kBtMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch: bad arguments");
+    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd % 8 || kAttnBlock % (hd / 8) || PI_WAVE % (hd / 8) || hd / 2 + hd > kAttnBlock || (mode != 0 && mode != 2))
+        return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch: head size must be 8 * (a divisor of 64), at most 128; mode 0 or 2");
+    const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kAttnBlock / (hd / 8)) * hd + 3 * (size_t)hd);
+    if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused_batch: context too long for the single-pass kernel");
+    hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head, n_seq), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
+                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride);
+    return pi::check_launch("pi_k_attn_fused_batch");
+}
+
+int pi_k_step_advance(int32_t * step, pi_stream_t stream) {
+    if (!step) return pi::fail(PI_E_ARG, "pi_k_step_advance: null pointer");
+    hipLaunchKernelGGL(step_advance_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, step);
+    return pi::check_launch("pi_k_step_advance");
+}
+
+int pi_k_embed_batch(const void * table_f16, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream) {
+    if (!table_f16 || !tokens || !x || cols <= 0 || T <= 0 || T > kBtMaxT) return pi::fail(PI_E_ARG, "pi_k_embed_batch: bad arguments");
+    hipLaunchKernelGGL(embed_f16_batch_kernel, dim3((cols + 255) / 256, T), dim3(256), 0, (hipStream_t)stream, (const __half *)table_f16, cols, tokens, x);
+    return pi::check_launch("pi_k_embed_batch");
+}
+
+int pi_k_argmax_batch(const float * logits, int n, int T, int32_t * tokens, int32_t * positions, int32_t * step, int32_t * out_tokens, int max_steps,
+                      pi_stream_t stream) {
+    if (!logits || !tokens || n <= 0 || T <= 0 || T > kBtMaxT) return pi::fail(PI_E_ARG, "pi_k_argmax_batch: bad arguments");
+    hipLaunchKernelGGL(argmax_batch_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, logits, n, T, tokens, positions, step, out_tokens, max_steps);
+    return pi::check_launch("pi_k_argmax_batch");
 }
 
 int pi_k_embed(int wtype, const void * table, int cols, const int32_t * token, float * x, pi_stream_t stream) {

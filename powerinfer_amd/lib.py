@@ -61,6 +61,10 @@ _SIGS = {
     "pi_k_norm_round_f16": (_i, [_vp, _i, _i, C.POINTER(Norm), _vp, _vp]),
     "pi_k_gemm_f16": (_i, [_vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp]),
     "pi_k_batch_sparse_ffn": (_i, [_vp, _i, _i, _f, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_attn_fused_batch": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp]),
+    "pi_k_embed_batch": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
+    "pi_k_argmax_batch": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _i, _vp]),
+    "pi_k_step_advance": (_i, [_vp, _vp]),
     "pi_k_rope_kv_store": (_i, [_vp, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp, _vp]),
     "pi_k_attn_decode": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "pi_k_rope_table": (_i, [_vp, _i, _i, _f, _vp]),

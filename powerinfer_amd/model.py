@@ -36,12 +36,17 @@ def _declare(L):
     L.pi_model_set_capture.restype, L.pi_model_set_capture.argtypes = i, [vp, i]
     L.pi_model_get_capture.restype, L.pi_model_get_capture.argtypes = i, [vp, vp, vp, vp, vp]
     L.pi_model_step_active.restype, L.pi_model_step_active.argtypes = i, [vp, vp, i]
+    L.pi_model_batch_init.restype, L.pi_model_batch_init.argtypes = i, [vp, i]
+    L.pi_model_batch_decode.restype, L.pi_model_batch_decode.argtypes = i, [vp, vp, vp, vp, vp]
+    L.pi_model_batch_generate.restype, L.pi_model_batch_generate.argtypes = i, [vp, i, vp, C.POINTER(C.c_float)]
+    L.pi_model_batch_union.restype, L.pi_model_batch_union.argtypes = i, [vp, vp]
     L.pi_model_time_section.restype, L.pi_model_time_section.argtypes = i, [vp, i, i, C.POINTER(C.c_float), C.POINTER(C.c_int)]
 
 
 ENGINE_SYMBOLS = ["pi_model_create", "pi_model_free", "pi_model_set_tensor", "pi_model_finalize", "pi_model_kv_clear",
                   "pi_model_decode", "pi_model_generate", "pi_model_set_capture", "pi_model_get_capture",
-                  "pi_model_step_active", "pi_model_time_section"]
+                  "pi_model_step_active", "pi_model_time_section",
+                  "pi_model_batch_init", "pi_model_batch_decode", "pi_model_batch_generate", "pi_model_batch_union"]
 
 
 def _type_of(a, hint):
@@ -74,6 +79,7 @@ class Model:
         if not self.h:
             raise pl.PiError("pi_model_create: " + self.L.pi_last_error().decode())
         self._keep = []        # host arrays the engine borrows (hybrid layers)
+        self.n_seq = 0         # sequences of batched decoding (batch_init)
 
     def set_tensor(self, layer, kind, arr):
         arr = np.ascontiguousarray(arr)
@@ -140,6 +146,36 @@ class Model:
         ms, n = C.c_float(0), C.c_int(0)
         check(self.L.pi_model_time_section(self.h, section, rounds, C.byref(ms), C.byref(n)), "time_section")
         return float(ms.value) / n.value, n.value
+
+    # ---- batched greedy decoding: n_seq independent sequences, one token each per step ----------------------
+    def batch_init(self, n_seq):
+        check(self.L.pi_model_batch_init(self.h, n_seq), "pi_model_batch_init")
+        self.n_seq = n_seq
+
+    def batch_decode(self, tokens, positions, want_logits=True):
+        if self.n_seq <= 0:
+            raise pl.PiError("batch_decode: batch_init first")
+        tokens = np.ascontiguousarray(tokens, np.int32)
+        positions = np.ascontiguousarray(positions, np.int32)
+        if tokens.size != self.n_seq or positions.size != self.n_seq:
+            raise pl.PiError("batch_decode: one token and one position per sequence")
+        nxt = np.empty(self.n_seq, np.int32)
+        logits = np.empty((self.n_seq, self.hp.n_vocab), np.float32) if want_logits else None
+        check(self.L.pi_model_batch_decode(self.h, tokens.ctypes.data_as(C.c_void_p), positions.ctypes.data_as(C.c_void_p),
+                                           nxt.ctypes.data_as(C.c_void_p), logits.ctypes.data_as(C.c_void_p) if want_logits else None),
+              "pi_model_batch_decode")
+        return nxt, logits
+
+    def batch_generate(self, n_steps):
+        out = np.empty((n_steps, self.n_seq), np.int32)
+        ms = C.c_float(0)
+        check(self.L.pi_model_batch_generate(self.h, n_steps, out.ctypes.data_as(C.c_void_p), C.byref(ms)), "pi_model_batch_generate")
+        return out, float(ms.value)
+
+    def batch_union(self):
+        out = np.empty(self.hp.n_layer, np.int32)
+        check(self.L.pi_model_batch_union(self.h, out.ctypes.data_as(C.c_void_p)), "pi_model_batch_union")
+        return out
 
     def close(self):
         if self.h:

@@ -114,3 +114,66 @@ def test_batch_sparse_ffn_matches_oracle(shape, has_gate, T):
             assert rel_err(got[t], o["out"][t]) < 1e-4
     assert sum(np.array_equal(mask_g[t], mask_o[t]) for t in range(T)) >= T - 2
     L.pi_workspace_destroy(ws)
+
+
+@pytest.mark.parametrize("arch", ["llama-tiny", "falcon-tiny"])
+def test_batched_decode_matches_per_sequence_oracle(arch):
+    """Four sequences with different prompts advance in lockstep (examples/batched/batched.cpp).  Sequences do not interact,
+    so sequence t of the batch must reproduce a single-sequence run on the same tokens: against the CPU oracle (teacher
+    forced, the trajectory-level criteria of the single-sequence tests) and against this library's own batch-1 engine."""
+    from powerinfer_amd.model import Model
+    hp = synth.hparams(arch, seed=5, n_ctx=64)
+    model = synth.make_model(hp)
+    n_seq, n_steps = 4, 10
+    rng = np.random.default_rng(11)
+    toks = rng.integers(0, hp.n_vocab, (n_steps, n_seq)).astype(np.int32)
+    gm = Model(hp).load(model)
+    gm.batch_init(n_seq)
+    batch_logits = np.zeros((n_steps, n_seq, hp.n_vocab), np.float32)
+    batch_next = np.zeros((n_steps, n_seq), np.int32)
+    for s in range(n_steps):
+        nxt, lg = gm.batch_decode(toks[s], np.full(n_seq, s, np.int32))
+        batch_logits[s], batch_next[s] = lg, nxt
+        assert np.array_equal(nxt, lg.argmax(1))
+    assert np.all(gm.batch_union() > 0)
+    errs_o, errs_g, same = [], [], 0
+    for t in range(n_seq):
+        om = ol.OracleModel(model)
+        gm.kv_clear()
+        for s in range(n_steps):
+            tok_o, lg_o = om.eval([int(toks[s, t])], s)
+            tok_g, lg_g = gm.decode([int(toks[s, t])], s)
+            errs_o.append(rel_err(batch_logits[s, t], lg_o))
+            errs_g.append(rel_err(batch_logits[s, t], lg_g))
+            same += int(batch_next[s, t] == tok_o)
+        om.close()
+    errs_o, errs_g = np.array(errs_o), np.array(errs_g)
+    assert np.median(errs_o) < 1e-2, errs_o
+    assert np.median(errs_g) < 1e-2, errs_g
+    assert same >= 0.9 * n_seq * n_steps, same
+    # greedy continuation on the device equals stepping the same state by hand
+    gm2 = Model(hp).load(model)
+    gm2.batch_init(n_seq)
+    nxt, _ = gm2.batch_decode(toks[0], np.zeros(n_seq, np.int32))
+    gen, _ = gm2.batch_generate(6)
+    gm3 = Model(hp).load(model)
+    gm3.batch_init(n_seq)
+    cur, _ = gm3.batch_decode(toks[0], np.zeros(n_seq, np.int32))
+    assert np.array_equal(cur, nxt)
+    for s in range(6):
+        cur, _ = gm3.batch_decode(cur, np.full(n_seq, s + 1, np.int32))
+        assert np.array_equal(gen[s], cur), s
+    for m in (gm, gm2, gm3):
+        m.close()
+
+
+def test_batch_init_rejects_unsupported_models():
+    from powerinfer_amd import lib as pl
+    from powerinfer_amd.model import Model
+    hp = synth.hparams("llama-tiny", seed=2, n_ctx=32, wtype=ol.Q4_0)
+    m = Model(hp).load(synth.make_model(hp))
+    with pytest.raises(pl.PiError):
+        m.batch_init(4)
+    with pytest.raises(pl.PiError):
+        m.batch_decode([1], [0])
+    m.close()

@@ -184,28 +184,34 @@ PI_API int pi_k_sparse_axpy_dense(const void * down_t_f16, int cols, int ff, con
  * n_tokens = n_parallel).  The weights are streamed once per step; the dense mat-muls and the sparse gate/up run on the
  * matrix cores (the batch >= 8 dense cross-over the reference takes through cuBLAS, ggml-cuda.cu:7717-7756, and its
  * mul_mat_batch_sparse kernels, :6994-7034).  Vectors of a step are token-major: x[T][cols], y[T][rows].
- *   pi_k_norm_round_f16: out_f16[t] = fp16(norm(x[t])) -- what the CPU path feeds every F16 dot (ggml.c:9703-9716).
- *   pi_k_gemm_f16:       y[t][row] = epi( W[row] . xn[t] ), cols % 128 == 0; add1/add2 are [T][rows].
- *   pi_k_batch_sparse_ffn: logits [T][ff] (from pi_k_gemm_f16 on fc2); union_rows/n_union receive the ascending list of
- *     neurons active for at least one token (each weight row is read once for the whole step);
+ *   pi_k_norm_round_f16: out_f16[t] = fp16(norm(x[t])) -- what the CPU path feeds every F16 dot (ggml.c:9703-9716);
+ *     out_plain_f16 (optional) receives fp16(x[t]) from the same pass (the predictor reads the un-normalised vector).
+ *   pi_k_gemm_f16:       y[t][row] = epi( W[row] . xn[t] ), cols % 128 == 0; add1/add2 are [T][rows]; y_f16 (optional) receives
+ *     fp16(y) for the next mat-mul.
+ *   pi_k_batch_predictor_fc2: logits[t][n] = fc2[n] . hidden_f16[t]; the epilogue also flags in the workspace every neuron with
+ *     !(logit < threshold) for at least one token.
+ *   pi_k_batch_sparse_ffn: logits [T][ff] and the workspace flags from pi_k_batch_predictor_fc2; union_rows/n_union receive the
+ *     ascending list of neurons active for at least one token (each weight row is read once for the whole step);
  *     out[t] = epi( sum over union rows active for t of fp16(h[t][n]) * down_t[n][:] ), h as in pi_k_sparse_upgate;
- *     cols % 512 == 0.  h_dense is reserved (pass NULL).
+ *     cols % 256 == 0.
  */
-PI_API int pi_k_norm_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, pi_stream_t stream);
+PI_API int pi_k_norm_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, void * out_plain_f16, pi_stream_t stream);
 PI_API int pi_k_gemm_f16(const void * W_f16, int rows, int cols, const void * xn_f16, int T, int epilogue,
-                         const float * add1, const float * add2, float * y, pi_stream_t stream);
+                         const float * add1, const float * add2, float * y, void * y_f16, pi_stream_t stream);
+PI_API int pi_k_batch_predictor_fc2(const void * fc2_f16, int ff, int r, const void * hidden_f16, int T, float threshold, float * logits,
+                                    pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold,
                                  const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const void * xn_f16,
                                  int epilogue, const float * add1, const float * add2, float * out,
-                                 int32_t * union_rows, int32_t * n_union, float * h_dense,
+                                 int32_t * union_rows, int32_t * n_union,
                                  pi_workspace * ws, pi_stream_t stream);
 
 /* per-sequence pieces of a batched step: sequence t owns token t, position pos[t] and the cache at t * cache_seq_stride
- * (elements); pi_k_argmax_batch picks each sequence's next token (first maximum wins), stores it in tokens[t], adds 1 to
+ * (elements), out_f16 (optional) receives fp16(out); pi_k_argmax_batch picks each sequence's next token (first maximum wins), stores it in tokens[t], adds 1 to
  * positions[t] and records it at out_tokens[*step][t]; pi_k_step_advance then moves *step on. */
 PI_API int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache,
                                  size_t cache_seq_stride, int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx,
-                                 const int32_t * pos, float * out, int out_stride, pi_stream_t stream);
+                                 const int32_t * pos, float * out, int out_stride, void * out_f16, pi_stream_t stream);
 PI_API int pi_k_embed_batch(const void * table_f16, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream);
 PI_API int pi_k_argmax_batch(const float * logits, int n, int T, int32_t * tokens, int32_t * positions, int32_t * step,
                              int32_t * out_tokens, int max_steps, pi_stream_t stream);

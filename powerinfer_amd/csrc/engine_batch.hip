@@ -46,35 +46,32 @@ int batch_layer(pi_model * m, int il) {
     if (!falcon) an = mk_norm(1, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), nullptr);
     else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
     else an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
-    PI_TRY(pi_k_norm_round_f16(x, T, d, &an, b->xa16, st));
-    PI_TRY(pi_k_gemm_f16(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, st));
+    PI_TRY(pi_k_norm_round_f16(x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));       // Falcon: the predictor reads the raw layer input
+    PI_TRY(pi_k_gemm_f16(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr, st));
     PI_TRY(pi_k_attn_fused_batch(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
-                                 hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, hp.n_ctx, b->d_pos, b->att, d, st));
-    PI_TRY(pi_k_norm_round_f16(b->att, T, d, nullptr, b->att16, st));
+                                 hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, hp.n_ctx, b->d_pos, b->att, d, b->att16, st));
 
-    const float * pred_in; pi_norm fn;
+    pi_norm fn;
     if (!falcon) {
-        PI_TRY(pi_k_gemm_f16(wo.dev, d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, st));       // ffn_inp = wo.att + x
-        pred_in = b->ffn_inp;
+        PI_TRY(pi_k_gemm_f16(wo.dev, d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, nullptr, st));       // ffn_inp = wo.att + x
         fn = mk_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
+        PI_TRY(pi_k_norm_round_f16(b->ffn_inp, T, d, &fn, b->xf16, b->xp16, st));                                // FFN input and predictor input in one pass
     } else {
-        PI_TRY(pi_k_gemm_f16(wo.dev, d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, st));
-        pred_in = x;                                       // Falcon: predictor and FFN read the layer input
+        PI_TRY(pi_k_gemm_f16(wo.dev, d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, nullptr, st));
         fn = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
+        if (m->L(il, PI_T_ATTN_NORM_2).dev) PI_TRY(pi_k_norm_round_f16(x, T, d, &fn, b->xf16, nullptr, st));     // two norms: the FFN has its own
     }
+    const __half * ffn_x = (falcon && !m->L(il, PI_T_ATTN_NORM_2).dev) ? b->xa16 : b->xf16;                        // single-norm Falcon: attention and FFN share it
     // predictor
-    PI_TRY(pi_k_norm_round_f16(pred_in, T, d, nullptr, b->xp16, st));
-    PI_TRY(pi_k_gemm_f16(fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, st));
-    PI_TRY(pi_k_norm_round_f16(b->hidden, T, r, nullptr, b->hid16, st));
-    PI_TRY(pi_k_gemm_f16(fc2.dev, ff, r, b->hid16, T, PI_EPI_NONE, nullptr, nullptr, b->pred_logits, st));
+    PI_TRY(pi_k_gemm_f16(fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16, st));
+    PI_TRY(pi_k_batch_predictor_fc2(fc2.dev, ff, r, b->hid16, T, hp.sparse_threshold, b->pred_logits, m->ws, st));
     // sparse FFN over the union of the sequences' active sets
-    PI_TRY(pi_k_norm_round_f16(pred_in, T, d, &fn, b->xf16, st));
     if (!falcon)
-        PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, gate.dev, down.dev, d, b->xf16, PI_EPI_ADD, b->ffn_inp, nullptr,
-                                     b->x2, b->union_rows, b->n_union + il, nullptr, m->ws, st));
+        PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, gate.dev, down.dev, d, ffn_x, PI_EPI_ADD, b->ffn_inp, nullptr,
+                                     b->x2, b->union_rows, b->n_union + il, m->ws, st));
     else
-        PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, nullptr, down.dev, d, b->xf16, PI_EPI_ADD2, b->attn_out, x,
-                                     b->x2, b->union_rows, b->n_union + il, nullptr, m->ws, st));
+        PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, nullptr, down.dev, d, ffn_x, PI_EPI_ADD2, b->attn_out, x,
+                                     b->x2, b->union_rows, b->n_union + il, m->ws, st));
     std::swap(b->x, b->x2);
     return PI_OK;
 }
@@ -88,8 +85,8 @@ int batch_step(pi_model * m) {
     PI_TRY(pi_k_embed_batch(m->glob[PI_T_TOK_EMBD].dev, d, b->d_tokens, T, b->x, st));
     for (int il = 0; il < hp.n_layer; ++il) PI_TRY(batch_layer(m, il));
     pi_norm on = mk_norm(falcon ? 2 : 1, hp.norm_eps, m->glob[PI_T_OUTPUT_NORM], falcon ? &m->glob[PI_T_OUTPUT_NORM_B] : nullptr);
-    PI_TRY(pi_k_norm_round_f16(b->x, T, d, &on, b->xa16, st));
-    PI_TRY(pi_k_gemm_f16(m->glob[PI_T_OUTPUT].dev, hp.n_vocab, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->logits, st));
+    PI_TRY(pi_k_norm_round_f16(b->x, T, d, &on, b->xa16, nullptr, st));
+    PI_TRY(pi_k_gemm_f16(m->glob[PI_T_OUTPUT].dev, hp.n_vocab, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->logits, nullptr, st));
     PI_TRY(pi_k_argmax_batch(b->logits, hp.n_vocab, T, b->d_tokens, b->d_pos, b->d_step, b->d_out_tokens, b->max_steps, st));
     PI_TRY(pi_k_step_advance(b->d_step, st));
     return PI_OK;

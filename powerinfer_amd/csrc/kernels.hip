@@ -1865,12 +1865,13 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
                                                             __half * __restrict__ k_cache, __half * __restrict__ v_cache,
                                                             int n_head, int n_head_kv, int hd, int mode, int n_ctx,
                                                             const int32_t * __restrict__ pos_p, float * __restrict__ out,
-                                                            int qkv_stride, size_t cache_seq_stride, int out_stride) {
+                                                            int qkv_stride, size_t cache_seq_stride, int out_stride, __half * __restrict__ out16) {
     // blockIdx.y = sequence of a batched step (its own token, position and cache); 0 for single-sequence decoding
     qkv += (size_t)blockIdx.y * qkv_stride;
     k_cache += (size_t)blockIdx.y * cache_seq_stride;
     v_cache += (size_t)blockIdx.y * cache_seq_stride;
     out += (size_t)blockIdx.y * out_stride;
+    if (out16) out16 += (size_t)blockIdx.y * out_stride;      // optional fp16 copy: the input of the next mat-mul of a batched step
     pos_p += blockIdx.y;
     extern __shared__ __align__(16) unsigned char smem[];
     float * s    = reinterpret_cast<float *>(smem);               // [n_ctx] scores, then probabilities
@@ -1962,6 +1963,7 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
         float v = part[e];
         for (int g = 1; g < ngrp; ++g) v += part[g * hd + e];
         out[(size_t)h * hd + e] = v;
+        if (out16) out16[(size_t)h * hd + e] = __float2half_rn(v);
     }
 }
 
@@ -2061,7 +2063,8 @@ typedef _Float16 pi_h8 __attribute__((ext_vector_type(8)));
 typedef float    pi_f4 __attribute__((ext_vector_type(4)));
 constexpr int kBtMaxT = 16;
 
-__global__ __launch_bounds__(kBlock) void norm_round_f16_kernel(const float * __restrict__ x, int cols, NormArgs na, __half * __restrict__ out) {
+__global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __restrict__ x, int cols, NormArgs na, __half * __restrict__ out,
+                                                              __half * __restrict__ out_plain) {
     __shared__ double red[16];
     const float * xt = x + (size_t)blockIdx.x * cols;
     __half * ot = out + (size_t)blockIdx.x * cols;
@@ -2083,6 +2086,7 @@ __global__ __launch_bounds__(kBlock) void norm_round_f16_kernel(const float * __
     }
     for (int i = threadIdx.x; i < cols; i += blockDim.x) {
         float v = xt[i];
+        if (out_plain) out_plain[(size_t)blockIdx.x * cols + i] = __float2half_rn(v);
         if (na.kind != 0) {
             v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
             if (na.w) v = __fmul_rn(v, na.w[i]);
@@ -2096,7 +2100,8 @@ __global__ __launch_bounds__(kBlock) void norm_round_f16_kernel(const float * __
 // quarters (cols % 128 == 0) and merge their 16 x 16 accumulator tiles through LDS in wave order.
 constexpr int kGmUn = 8;
 __global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
-                                                              int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y) {
+                                                              int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y,
+                                                              __half * __restrict__ y16, float thr, unsigned char * __restrict__ row_any) {
     __shared__ float cs[kWavesPerBlock][16][17];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int i = lane & 15, g = lane >> 4;
@@ -2121,6 +2126,7 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __r
     for (int r = 0; r < 4; ++r) cs[wave][4 * g + r][i] = acc[r];
     __syncthreads();
     const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
+    bool act = false;
     if (row0 + rr < rows && t < T) {
         float sum = cs[0][rr][t];
 #pragma unroll
@@ -2130,19 +2136,24 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __r
         else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
         else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[o]), add2[o]);
         y[o] = sum;
+        if (y16) y16[o] = __float2half_rn(sum);
+        act = !(sum < thr);
+    }
+    if (row_any) {      // predictor logits: is the row active for at least one token of the step?  (16 lanes = 16 tokens of a row)
+        const unsigned long long m = __ballot(act);
+        if (t == 0 && row0 + rr < rows) row_any[row0 + rr] = ((m >> (16 * (lane >> 4))) & 0xffffull) ? 1 : 0;
     }
 }
 
-// union over the tokens of the step of the predictor's active sets: list of neurons active for at least one token,
-// ascending (single workgroup: wave ballot per 64 neurons, popcount prefix over the mask words)
-__global__ __launch_bounds__(1024) void union_active_kernel(const float * __restrict__ logits, int T, int ff, float thr,
+// union over the tokens of the step of the predictor's active sets: ascending list of the neurons whose flag the
+// predictor's mat-mul epilogue raised (single workgroup: wave ballot per 64 neurons, popcount prefix over the mask words)
+__global__ __launch_bounds__(1024) void union_active_kernel(const unsigned char * __restrict__ row_any, int ff,
                                                             uint32_t * __restrict__ words, int32_t * __restrict__ list, int32_t * __restrict__ n_union) {
     __shared__ int sred[17];
     const int lane = threadIdx.x & 63;
     for (int i0 = 0; i0 < ff; i0 += blockDim.x) {
         const int i = i0 + threadIdx.x;
-        bool act = false;
-        if (i < ff) for (int t = 0; t < T; ++t) act = act || !(logits[(size_t)t * ff + i] < thr);
+        const bool act = i < ff && row_any[i] != 0;
         const unsigned long long m = __ballot(act);
         if (lane == 0 && i < ff) words[i >> 5] = (uint32_t)m;
         if (lane == 32 && i < ff) words[i >> 5] = (uint32_t)(m >> 32);
@@ -2158,6 +2169,7 @@ __global__ __launch_bounds__(kBlock) void batch_upgate_f16_kernel(const __half *
                                                                   const __half * __restrict__ xn, int T, const float * __restrict__ logits, int ff, float thr,
                                                                   const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
                                                                   float * __restrict__ hc) {
+    // hc[u][t] is stored already rounded to fp16 (kept as fp32): the CPU axpy rounds h before use (ggml.c:14420-14431)
     __shared__ float cu[kWavesPerBlock][16][17], cg[kWavesPerBlock][16][17];
     const int n = *n_union;
     const int u0 = blockIdx.x * 16;
@@ -2199,59 +2211,73 @@ __global__ __launch_bounds__(kBlock) void batch_upgate_f16_kernel(const __half *
             float su = cu[0][rr][t], sg = cg[0][rr][t];
 #pragma unroll
             for (int w = 1; w < kWavesPerBlock; ++w) { su += cu[w][rr][t]; sg += cg[w][rr][t]; }
-            h = Wgate ? __fmul_rn(fmaxf(sg, 0.0f), su) : fmaxf(su, 0.0f);
+            h = pi_round_f16(Wgate ? __fmul_rn(fmaxf(sg, 0.0f), su) : fmaxf(su, 0.0f));
         }
     }
     hc[(size_t)(u0 + rr) * kBtMaxT + t] = h;
 }
 
-// sparse down projection for the step: partial[g][t][c] = sum over union entries u = g, g + G, ... of fp16(hc[u][t]) * down[row_u][c].
-// A wave owns 512 columns (8 per lane) and one of G row groups; 16 tokens x 8 columns of fp32 accumulators per lane.
-constexpr int kBaGroups = 32;
-__global__ __launch_bounds__(kBlock) void batch_axpy_f16_kernel(const __half * __restrict__ Wd, int cols, const float * __restrict__ hc,
-                                                                const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
-                                                                float * __restrict__ partial) {
+// sparse down projection for the step: partial[g][t][c] = sum over the union entries of row group g of hc[u][t] * down[row_u][c].
+// A workgroup of 8 waves owns 256 columns (4 per lane, one 8-byte load per row) and one of G row groups; wave w of group g
+// walks entries u = 8g + w, + 8G, ...: a whole wave works on ONE row at a time, so the row's 16 h values are wave-uniform
+// and arrive through the scalar cache.  The 8 waves then add their 16 x 256 tiles into LDS one after the other (fixed order).
+constexpr int kBaGroups = 8;
+constexpr int kBaBlock = 512;
+constexpr int kBaWaves = kBaBlock / PI_WAVE;
+constexpr int kBaTile = 256;
+__global__ __launch_bounds__(kBaBlock) void batch_axpy_f16_kernel(const __half * __restrict__ Wd, int cols, const float * __restrict__ hc,
+                                                                  const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
+                                                                  float * __restrict__ partial) {
+    __shared__ float tile[kBtMaxT][kBaTile];
     const int n = *n_union;
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int grp = blockIdx.y * kWavesPerBlock + wave;
-    const int c0 = blockIdx.x * 512 + lane * 8;
-    float acc[kBtMaxT][8];
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int c0 = blockIdx.x * kBaTile + lane * 4;
+    const int stride = kBaGroups * kBaWaves;
+    float acc[kBtMaxT][4];
 #pragma unroll
     for (int t = 0; t < kBtMaxT; ++t)
 #pragma unroll
-        for (int k = 0; k < 8; ++k) acc[t][k] = 0.0f;
-    constexpr int UN = 4;
-    for (int u0 = grp; u0 < n; u0 += kBaGroups * UN) {
-        pi_u32x4 w[UN];
+        for (int k = 0; k < 4; ++k) acc[t][k] = 0.0f;
+    constexpr int UN = 8;
+    for (int u0 = blockIdx.y * kBaWaves + wave; u0 < n; u0 += stride * UN) {
+        pi_u32x2 w[UN];
 #pragma unroll
         for (int j = 0; j < UN; ++j) {
-            const int u = u0 + j * kBaGroups;
-            w[j] = u < n ? pi_ld_stream(Wd + (size_t)list[u] * cols + c0) : pi_u32x4{0u, 0u, 0u, 0u};
+            const int u = u0 + j * stride;
+            w[j] = u < n ? __builtin_nontemporal_load(reinterpret_cast<const pi_u32x2 *>(Wd + (size_t)list[u] * cols + c0)) : pi_u32x2{0u, 0u};
         }
 #pragma unroll
         for (int j = 0; j < UN; ++j) {
-            const int u = u0 + j * kBaGroups;
+            const int u = u0 + j * stride;
             if (u < n) {
-                float wf[8];
-                pi_unpack8(w[j], wf);
-                const float4 * hp = reinterpret_cast<const float4 *>(hc + (size_t)u * kBtMaxT);
+                const __half2 * hw = reinterpret_cast<const __half2 *>(&w[j]);
+                const float2 w01 = __half22float2(hw[0]), w23 = __half22float2(hw[1]);
+                const float * hp = hc + (size_t)u * kBtMaxT;
 #pragma unroll
-                for (int q = 0; q < 4; ++q) {
-                    const float4 h4 = hp[q];
-                    const float hh[4] = {pi_round_f16(h4.x), pi_round_f16(h4.y), pi_round_f16(h4.z), pi_round_f16(h4.w)};
-#pragma unroll
-                    for (int e = 0; e < 4; ++e)
-#pragma unroll
-                        for (int k = 0; k < 8; ++k) acc[4 * q + e][k] = fmaf(wf[k], hh[e], acc[4 * q + e][k]);
+                for (int t = 0; t < kBtMaxT; ++t) {
+                    const float h = hp[t];
+                    acc[t][0] = fmaf(w01.x, h, acc[t][0]); acc[t][1] = fmaf(w01.y, h, acc[t][1]);
+                    acc[t][2] = fmaf(w23.x, h, acc[t][2]); acc[t][3] = fmaf(w23.y, h, acc[t][3]);
                 }
             }
         }
     }
+    for (int w = 0; w < kBaWaves; ++w) {
+        if (wave == w) {
 #pragma unroll
-    for (int t = 0; t < kBtMaxT; ++t) {
-        float4 * po = reinterpret_cast<float4 *>(partial + ((size_t)grp * kBtMaxT + t) * cols + c0);
-        po[0] = make_float4(acc[t][0], acc[t][1], acc[t][2], acc[t][3]);
-        po[1] = make_float4(acc[t][4], acc[t][5], acc[t][6], acc[t][7]);
+            for (int t = 0; t < kBtMaxT; ++t) {
+                float4 * p = reinterpret_cast<float4 *>(&tile[t][lane * 4]);
+                float4 v = w == 0 ? make_float4(0.0f, 0.0f, 0.0f, 0.0f) : *p;
+                v.x += acc[t][0]; v.y += acc[t][1]; v.z += acc[t][2]; v.w += acc[t][3];
+                *p = v;
+            }
+        }
+        __syncthreads();
+    }
+    for (int i = threadIdx.x; i < kBtMaxT * kBaTile / 4; i += kBaBlock) {
+        const int t = i / (kBaTile / 4), c4 = i % (kBaTile / 4);
+        *reinterpret_cast<float4 *>(partial + ((size_t)blockIdx.y * kBtMaxT + t) * cols + blockIdx.x * kBaTile + c4 * 4) =
+            *reinterpret_cast<const float4 *>(&tile[t][c4 * 4]);
     }
 }
 
@@ -2321,6 +2347,7 @@ struct pi_workspace {
     float *        hd;             // [max_ff]  and its Q8_0 block scale
     float *        ffn_partial;    // [max(max_ff/32, 32 * 16)][max_d]  partial outputs of the fused sparse FFN / of the batched axpy
     float *        hc_batch;       // [max_ff][16]  h of the union rows for a batched step
+    unsigned char * row_any;       // [max_ff]  batched step: neuron active for at least one token
 };
 constexpr int kAxpyGroups = 32;
 
@@ -2338,7 +2365,8 @@ pi_workspace * pi_workspace_create(int max_ff, int max_d) {
     const size_t n_part = (size_t)((max_ff + 31) / 32) > (size_t)kBaGroups * kBtMaxT ? (size_t)((max_ff + 31) / 32) : (size_t)kBaGroups * kBtMaxT;
     ws->ffn_partial = (float *)pi_malloc(sizeof(float) * n_part * max_d);
     ws->hc_batch = (float *)pi_malloc(sizeof(float) * ((size_t)max_ff + 16) * kBtMaxT);
-    if (!ws->words || !ws->counters || !ws->partial || !ws->hq || !ws->hd || !ws->ffn_partial || !ws->hc_batch) {
+    ws->row_any = (unsigned char *)pi_malloc((size_t)max_ff + 16);
+    if (!ws->words || !ws->counters || !ws->partial || !ws->hq || !ws->hd || !ws->ffn_partial || !ws->hc_batch || !ws->row_any) {
         pi_workspace_destroy(ws); return nullptr;
     }
     pi_memset(ws->counters, 0, sizeof(unsigned int) * 64);
@@ -2346,7 +2374,7 @@ pi_workspace * pi_workspace_create(int max_ff, int max_d) {
 }
 int pi_workspace_destroy(pi_workspace * ws) {
     if (!ws) return PI_OK;
-    pi_free(ws->words); pi_free(ws->counters); pi_free(ws->partial); pi_free(ws->hq); pi_free(ws->hd); pi_free(ws->ffn_partial); pi_free(ws->hc_batch);
+    pi_free(ws->words); pi_free(ws->counters); pi_free(ws->partial); pi_free(ws->hq); pi_free(ws->hd); pi_free(ws->ffn_partial); pi_free(ws->hc_batch); pi_free(ws->row_any);
     delete ws;
     return PI_OK;
 }
@@ -2588,39 +2616,49 @@ int pi_k_sparse_ffn(const void * fc2_f16, int ff, int r, const float * hidden, f
     return pi::check_launch("pi_k_sparse_ffn");
 }
 
-int pi_k_norm_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, pi_stream_t stream) {
+int pi_k_norm_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, void * out_plain_f16, pi_stream_t stream) {
     if (!x || !out_f16 || T <= 0 || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_norm_round_f16: bad arguments");
-    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(kBlock), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16);
+    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16, (__half *)out_plain_f16);
     return pi::check_launch("pi_k_norm_round_f16");
 }
 
-int pi_k_gemm_f16(const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
-                  float * y, pi_stream_t stream) {
-    if (!W || !xn_f16 || !y || rows <= 0) return pi::fail(PI_E_ARG, "pi_k_gemm_f16: null pointer or empty shape");
-    if (T < 1 || T > kBtMaxT || cols <= 0 || cols % 128) return pi::fail(PI_E_ARG, "pi_k_gemm_f16: 1 <= T <= 16 and cols % 128 == 0 required");
+static int gemm_launch(const char * who, const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
+                       float * y, void * y_f16, float thr, unsigned char * row_any, pi_stream_t stream) {
+    if (!W || !xn_f16 || !y || rows <= 0) return pi::fail(PI_E_ARG, who);
+    if (T < 1 || T > kBtMaxT || cols <= 0 || cols % 128) return pi::fail(PI_E_ARG, "batched mat-mul: 1 <= T <= 16 and cols % 128 == 0 required");
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
-        return pi::fail(PI_E_ARG, "pi_k_gemm_f16: bad epilogue arguments");
+        return pi::fail(PI_E_ARG, "batched mat-mul: bad epilogue arguments");
     hipLaunchKernelGGL(gemm_t16_f16_kernel, dim3((rows + 15) / 16), dim3(kBlock), 0, (hipStream_t)stream,
-                       (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y);
-    return pi::check_launch("pi_k_gemm_f16");
+                       (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any);
+    return pi::check_launch(who);
+}
+
+int pi_k_gemm_f16(const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
+                  float * y, void * y_f16, pi_stream_t stream) {
+    return gemm_launch("pi_k_gemm_f16", W, rows, cols, xn_f16, T, epilogue, add1, add2, y, y_f16, 0.0f, nullptr, stream);
+}
+
+int pi_k_batch_predictor_fc2(const void * fc2_f16, int ff, int r, const void * hidden_f16, int T, float threshold, float * logits,
+                             pi_workspace * ws, pi_stream_t stream) {
+    if (!ws || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_batch_predictor_fc2: ff exceeds the workspace");
+    return gemm_launch("pi_k_batch_predictor_fc2", fc2_f16, ff, r, hidden_f16, T, PI_EPI_NONE, nullptr, nullptr, logits, nullptr, threshold, ws->row_any, stream);
 }
 
 int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, const void * up_f16, const void * gate_f16, const void * down_t_f16,
                           int cols, const void * xn_f16, int epilogue, const float * add1, const float * add2, float * out,
-                          int32_t * union_rows, int32_t * n_union, float * h_dense, pi_workspace * ws, pi_stream_t stream) {
+                          int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream) {
     if (!logits || !up_f16 || !down_t_f16 || !xn_f16 || !out || !union_rows || !n_union || !ws) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: null pointer");
-    if (T < 1 || T > kBtMaxT || ff <= 0 || ff > ws->max_ff || cols <= 0 || cols > ws->max_d || cols % 512)
-        return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: 1 <= T <= 16, ff <= workspace, cols % 512 == 0 and cols <= workspace required");
+    if (T < 1 || T > kBtMaxT || ff <= 0 || ff > ws->max_ff || cols <= 0 || cols > ws->max_d || cols % kBaTile || cols % 128)
+        return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: 1 <= T <= 16, ff <= workspace, cols % 256 == 0 and cols <= workspace required");
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
         return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: bad epilogue arguments");
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, logits, T, ff, threshold, ws->words, union_rows, n_union);
+    hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, ws->row_any, ff, ws->words, union_rows, n_union);
     hipLaunchKernelGGL(batch_upgate_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
                        (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch);
-    hipLaunchKernelGGL(batch_axpy_f16_kernel, dim3(cols / 512, kBaGroups / kWavesPerBlock), dim3(kBlock), 0, st, (const __half *)down_t_f16, cols,
+    hipLaunchKernelGGL(batch_axpy_f16_kernel, dim3(cols / kBaTile, kBaGroups), dim3(kBaBlock), 0, st, (const __half *)down_t_f16, cols,
                        ws->hc_batch, union_rows, n_union, ws->ffn_partial);
     hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, T, cols, epilogue, add1, add2, out);
-    (void)h_dense;
     return pi::check_launch("pi_k_batch_sparse_ffn");
 }
 
@@ -2659,20 +2697,20 @@ int pi_k_attn_fused(const float * qkv, const void * rope_table, void * k_cache, 
     const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kAttnBlock / (hd / 8)) * hd + 3 * (size_t)hd);
     if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused: context too long for the single-pass kernel");
     hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
-                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, 0, (size_t)0, 0);
+                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, 0, (size_t)0, 0, nullptr);
     return pi::check_launch("pi_k_attn_fused");
 }
 
 int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache, size_t cache_seq_stride,
                           int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, const int32_t * pos, float * out, int out_stride,
-                          pi_stream_t stream) {
+                          void * out_f16, pi_stream_t stream) {
     if (!qkv || !rope_table || !k_cache || !v_cache || !pos || !out || n_seq <= 0 || n_seq > kBtMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch: bad arguments");
     if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd % 8 || kAttnBlock % (hd / 8) || PI_WAVE % (hd / 8) || hd / 2 + hd > kAttnBlock || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch: head size must be 8 * (a divisor of 64), at most 128; mode 0 or 2");
     const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kAttnBlock / (hd / 8)) * hd + 3 * (size_t)hd);
     if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused_batch: context too long for the single-pass kernel");
     hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head, n_seq), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
-                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride);
+                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride, (__half *)out_f16);
     return pi::check_launch("pi_k_attn_fused_batch");
 }
 

@@ -58,10 +58,11 @@ _SIGS = {
     "pi_k_pred_upgate_supported": (_i, [_i, _i, _i]),
     "pi_k_pred_upgate": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp]),
     "pi_k_sparse_axpy_dense": (_i, [_vp, _i, _i, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
-    "pi_k_norm_round_f16": (_i, [_vp, _i, _i, C.POINTER(Norm), _vp, _vp]),
-    "pi_k_gemm_f16": (_i, [_vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp]),
-    "pi_k_batch_sparse_ffn": (_i, [_vp, _i, _i, _f, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
-    "pi_k_attn_fused_batch": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp]),
+    "pi_k_norm_round_f16": (_i, [_vp, _i, _i, C.POINTER(Norm), _vp, _vp, _vp]),
+    "pi_k_gemm_f16": (_i, [_vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_batch_predictor_fc2": (_i, [_vp, _i, _i, _vp, _i, _f, _vp, _vp, _vp]),
+    "pi_k_batch_sparse_ffn": (_i, [_vp, _i, _i, _f, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_attn_fused_batch": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),
     "pi_k_embed_batch": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
     "pi_k_argmax_batch": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _i, _vp]),
     "pi_k_step_advance": (_i, [_vp, _vp]),

@@ -24,7 +24,7 @@ def gpu_norm_round(pl, L, x, norm=None):
         bb = pl.DevBuf(host=nb) if nb is not None else None
         keep += [bw, bb]
         na = pl.norm_arg(kind, eps, bw, bb)
-    pl.check(L.pi_k_norm_round_f16(dx.ptr, T, cols, na, dn.ptr, None), "norm_round")
+    pl.check(L.pi_k_norm_round_f16(dx.ptr, T, cols, na, dn.ptr, None, None), "norm_round")
     pl.sync()
     return dn
 
@@ -42,16 +42,19 @@ def test_gemm_matches_oracle(rows, cols, T):
     dn = gpu_norm_round(pl, L, x)
     assert np.array_equal(dn.download(np.float16).reshape(T, cols), x.astype(np.float16))
     dw, dy, d1 = pl.DevBuf(host=w), pl.DevBuf(T * rows * 4), pl.DevBuf(host=a1)
-    pl.check(L.pi_k_gemm_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_NONE, None, None, dy.ptr, None), "gemm")
+    pl.check(L.pi_k_gemm_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_NONE, None, None, dy.ptr, None, None), "gemm")
     pl.sync()
     got = dy.download(np.float32).reshape(T, rows)
     assert rel_err(got, want) < 5e-6
-    pl.check(L.pi_k_gemm_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_ADD, d1.ptr, None, dy.ptr, None), "gemm")
+    pl.check(L.pi_k_gemm_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_ADD, d1.ptr, None, dy.ptr, None, None), "gemm")
     pl.sync()
     assert rel_err(dy.download(np.float32).reshape(T, rows), want + a1) < 5e-6
-    pl.check(L.pi_k_gemm_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_RELU, None, None, dy.ptr, None), "gemm")
+    dy16 = pl.DevBuf(T * rows * 2)
+    pl.check(L.pi_k_gemm_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_RELU, None, None, dy.ptr, dy16.ptr, None), "gemm")
     pl.sync()
-    assert rel_err(dy.download(np.float32).reshape(T, rows), np.maximum(want, 0)) < 5e-6
+    got = dy.download(np.float32).reshape(T, rows)
+    assert rel_err(got, np.maximum(want, 0)) < 5e-6
+    assert np.array_equal(dy16.download(np.float16).reshape(T, rows), got.astype(np.float16))
 
 
 @pytest.mark.parametrize("kind", [1, 2])
@@ -95,11 +98,10 @@ def test_batch_sparse_ffn_matches_oracle(shape, has_gate, T):
     union, n_union = pl.DevBuf(ff * 4), pl.DevBuf.zeros(4)
     resid = np.random.default_rng(3).standard_normal((T, d)).astype(np.float32)
     dres = pl.DevBuf(host=resid)
-    pl.check(L.pi_k_gemm_f16(fc1.ptr, r, d, xn.ptr, T, pl.EPI_RELU, None, None, hidden.ptr, None), "fc1")
-    pl.check(L.pi_k_norm_round_f16(hidden.ptr, T, r, None, hid16.ptr, None), "round hidden")
-    pl.check(L.pi_k_gemm_f16(fc2.ptr, ff, r, hid16.ptr, T, pl.EPI_NONE, None, None, logits.ptr, None), "fc2")
+    pl.check(L.pi_k_gemm_f16(fc1.ptr, r, d, xn.ptr, T, pl.EPI_RELU, None, None, hidden.ptr, hid16.ptr, None), "fc1")
+    pl.check(L.pi_k_batch_predictor_fc2(fc2.ptr, ff, r, hid16.ptr, T, 0.0, logits.ptr, ws, None), "fc2")
     pl.check(L.pi_k_batch_sparse_ffn(logits.ptr, T, ff, 0.0, up.ptr, gate.ptr if gate else None, down.ptr, d, xn.ptr,
-                                     pl.EPI_ADD, dres.ptr, None, out.ptr, union.ptr, n_union.ptr, None, ws, None), "batch ffn")
+                                     pl.EPI_ADD, dres.ptr, None, out.ptr, union.ptr, n_union.ptr, ws, None), "batch ffn")
     pl.sync()
     lg = logits.download(np.float32).reshape(T, ff)
     assert rel_err(lg, o["logits"]) < 1e-4

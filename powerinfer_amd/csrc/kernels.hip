@@ -2096,52 +2096,75 @@ __global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __re
     }
 }
 
-// y[t][row] = epi( W[row] . xn[t] ), t < T <= 16.  A workgroup owns 16 rows; its four waves split the columns in
-// quarters (cols % 128 == 0) and merge their 16 x 16 accumulator tiles through LDS in wave order.
-constexpr int kGmUn = 8;
+// y[t][row] = epi( W[row] . xn[t] ), t < T <= 16.  A workgroup owns 16*RT rows; its four waves split the columns in
+// quarters (cols % 128 == 0) and merge their 16 x 16 accumulator tiles through LDS in wave order.  A wave loads each
+// activation fragment once per 32-column step and uses it for its RT row tiles (the activations of a step are 16 x cols
+// fp16, as many bytes per row tile as the weights, so re-reading them per tile would double the L2 -> CU traffic);
+// 16 weight loads of 16 B per lane are in flight.
+template <int RT>
 __global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
                                                               int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y,
                                                               __half * __restrict__ y16, float thr, unsigned char * __restrict__ row_any) {
     __shared__ float cs[kWavesPerBlock][16][17];
+    constexpr int SU = 16 / RT;                     // steps per batch of loads
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int i = lane & 15, g = lane >> 4;
-    const int row0 = blockIdx.x * 16;
-    const int row = row0 + i < rows ? row0 + i : rows - 1;
+    const int row0 = blockIdx.x * 16 * RT;
     const int tok = i < T ? i : T - 1;
     const int kw = cols / kWavesPerBlock;
-    const __half * ap = W + (size_t)row * cols + wave * kw + g * 8;
+    const __half * ap[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int row = row0 + rt * 16 + i < rows ? row0 + rt * 16 + i : rows - 1;
+        ap[rt] = W + (size_t)row * cols + wave * kw + g * 8;
+    }
     const __half * bp = xn + (size_t)tok * cols + wave * kw + g * 8;
-    pi_f4 acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    pi_f4 acc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
     const int steps = kw / 32;
-    for (int s0 = 0; s0 < steps; s0 += kGmUn) {
-        pi_u32x4 a[kGmUn], b[kGmUn];
+    for (int s0 = 0; s0 < steps; s0 += SU) {
+        pi_u32x4 a[SU][RT], b[SU];
 #pragma unroll
-        for (int u = 0; u < kGmUn; ++u)
-            if (s0 + u < steps) { a[u] = pi_ld_stream(ap + (s0 + u) * 32); b[u] = pi_ld16(bp + (s0 + u) * 32); }
+        for (int u = 0; u < SU; ++u)
+            if (s0 + u < steps) {
 #pragma unroll
-        for (int u = 0; u < kGmUn; ++u)
-            if (s0 + u < steps) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a[u]), __builtin_bit_cast(pi_h8, b[u]), acc, 0, 0, 0);
+                for (int rt = 0; rt < RT; ++rt) a[u][rt] = pi_ld_stream(ap[rt] + (s0 + u) * 32);
+                b[u] = pi_ld16(bp + (s0 + u) * 32);
+            }
+#pragma unroll
+        for (int u = 0; u < SU; ++u)
+            if (s0 + u < steps) {
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a[u][rt]), __builtin_bit_cast(pi_h8, b[u]), acc[rt], 0, 0, 0);
+            }
     }
-#pragma unroll
-    for (int r = 0; r < 4; ++r) cs[wave][4 * g + r][i] = acc[r];
-    __syncthreads();
     const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
-    bool act = false;
-    if (row0 + rr < rows && t < T) {
-        float sum = cs[0][rr][t];
 #pragma unroll
-        for (int w = 1; w < kWavesPerBlock; ++w) sum += cs[w][rr][t];
-        const size_t o = (size_t)t * rows + row0 + rr;
-        if (epi == PI_EPI_RELU) sum = fmaxf(sum, 0.0f);
-        else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
-        else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[o]), add2[o]);
-        y[o] = sum;
-        if (y16) y16[o] = __float2half_rn(sum);
-        act = !(sum < thr);
-    }
-    if (row_any) {      // predictor logits: is the row active for at least one token of the step?  (16 lanes = 16 tokens of a row)
-        const unsigned long long m = __ballot(act);
-        if (t == 0 && row0 + rr < rows) row_any[row0 + rr] = ((m >> (16 * (lane >> 4))) & 0xffffull) ? 1 : 0;
+    for (int rt = 0; rt < RT; ++rt) {
+        if (rt > 0) __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 4; ++r) cs[wave][4 * g + r][i] = acc[rt][r];
+        __syncthreads();
+        const int row = row0 + rt * 16 + rr;
+        bool act = false;
+        if (row < rows && t < T) {
+            float sum = cs[0][rr][t];
+#pragma unroll
+            for (int w = 1; w < kWavesPerBlock; ++w) sum += cs[w][rr][t];
+            const size_t o = (size_t)t * rows + row;
+            if (epi == PI_EPI_RELU) sum = fmaxf(sum, 0.0f);
+            else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
+            else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[o]), add2[o]);
+            y[o] = sum;
+            if (y16) y16[o] = __float2half_rn(sum);
+            act = !(sum < thr);
+        }
+        if (row_any) {      // predictor logits: is the row active for at least one token of the step?  (16 lanes = 16 tokens of a row)
+            const unsigned long long m = __ballot(act);
+            if (t == 0 && row < rows) row_any[row] = ((m >> (16 * (lane >> 4))) & 0xffffull) ? 1 : 0;
+        }
     }
 }
 
@@ -2628,8 +2651,12 @@ static int gemm_launch(const char * who, const void * W, int rows, int cols, con
     if (T < 1 || T > kBtMaxT || cols <= 0 || cols % 128) return pi::fail(PI_E_ARG, "batched mat-mul: 1 <= T <= 16 and cols % 128 == 0 required");
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
         return pi::fail(PI_E_ARG, "batched mat-mul: bad epilogue arguments");
-    hipLaunchKernelGGL(gemm_t16_f16_kernel, dim3((rows + 15) / 16), dim3(kBlock), 0, (hipStream_t)stream,
-                       (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any);
+    // row tiles per wave: enough workgroups to fill the chip first, then as few reads of the activations as possible
+    const int rt = rows >= 16384 ? 4 : rows >= 8192 ? 2 : 1;
+#define PI_GEMM_T16(RT) hipLaunchKernelGGL((gemm_t16_f16_kernel<RT>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(kBlock), 0, (hipStream_t)stream, \
+                       (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any)
+    if (rt == 4) PI_GEMM_T16(4); else if (rt == 2) PI_GEMM_T16(2); else PI_GEMM_T16(1);
+#undef PI_GEMM_T16
     return pi::check_launch(who);
 }
 

@@ -155,4 +155,12 @@ def make_model(hp):
         if hp.hot_frac < 1.0:
             L["gpu_idx"], L["gpu_bucket"] = gpu_split(p, hp.hot_frac)
         layers.append(L)
+    if hp.get("vram_budget_gb") is not None:
+        # --vram-budget: the planner decides how many neurons of each layer stay on the GPU (powerinfer_amd.split)
+        from . import split
+        splits, rep = split.plan_split(hp, [L["p"] for L in layers], hp.vram_budget_gb, hp.n_ctx, batch=hp.get("split_batch", 256))
+        for L, (gi, gb) in zip(layers, splits):
+            if gb.size:
+                L["gpu_idx"], L["gpu_bucket"] = gi, gb
+        hp["split_report"] = rep
     return dict(hp=hp, glob=glob, layers=layers)

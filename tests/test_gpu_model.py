@@ -139,6 +139,21 @@ def test_hybrid_split_matches_all_cold_oracle(arch, wtype):
     run_case(synth.hparams(arch, wtype=wtype, n_ctx=96, seed=8, hot_frac=0.6), n_prompt=8, n_gen=24)
 
 
+def test_vram_budget_split_matches_all_cold_oracle():
+    """--vram-budget: the planner (offload order, neuron capacity, per-layer distribution) decides the split, the engine runs
+    the hybrid it describes."""
+    from powerinfer_amd import split
+    hp = synth.hparams("llama-tiny", n_ctx=96, seed=9, split_batch=64)
+    dense = split.offload_plan(hp, 1 << 40, hp.n_ctx)
+    base = dense["dense_bytes"] + 2 * hp.n_embd * hp.n_layer * hp.n_ctx * 2
+    hp["vram_budget_gb"] = (base + 8.0e6) / 1024 ** 3
+    model = synth.make_model(hp)
+    counts = hp["split_report"]["counts"]
+    assert all(c > 0 for c in counts) and sum(counts) < hp.n_ff * hp.n_layer
+    assert all("gpu_bucket" in L for L in model["layers"])
+    run_case(hp, n_prompt=8, n_gen=24)
+
+
 def test_decode_rejects_bad_arguments():
     from powerinfer_amd.model import Model
     from powerinfer_amd.lib import PiError

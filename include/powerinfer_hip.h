@@ -212,6 +212,11 @@ PI_API int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float thre
 PI_API int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache,
                                  size_t cache_seq_stride, int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx,
                                  const int32_t * pos, float * out, int out_stride, void * out_f16, pi_stream_t stream);
+/* prompt chunk of ONE sequence: T <= 16 consecutive tokens at positions pos[t]; RoPE + KV store of the whole chunk first, then
+ * every token attends to the cells up to its own position (the causal mask of llama.cpp:6506-6531).  q_rot: fp32 [T][n_head*hd]. */
+PI_API int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
+                           const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache,
+                           float * out, int out_stride, void * out_f16, pi_stream_t stream);
 PI_API int pi_k_embed_batch(const void * table_f16, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream);
 PI_API int pi_k_argmax_batch(const float * logits, int n, int T, int32_t * tokens, int32_t * positions, int32_t * step,
                              int32_t * out_tokens, int max_steps, pi_stream_t stream);

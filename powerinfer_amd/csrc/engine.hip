@@ -414,7 +414,17 @@ int pi_model_decode(pi_model * m, const int32_t * tokens, int n_tokens, int n_pa
     if (!tokens || n_tokens <= 0 || n_past < 0 || n_past + n_tokens > m->hp.n_ctx) return pi::fail(PI_E_ARG, "pi_model_decode: token range exceeds the context");
     for (int i = 0; i < n_tokens; ++i)
         if (tokens[i] < 0 || tokens[i] >= m->hp.n_vocab) return pi::fail(PI_E_ARG, "pi_model_decode: token id out of range");
-    for (int i = 0; i < n_tokens; ++i) {
+    int first = 0;
+    if (n_tokens > 2 && pi::prefill_supported(m)) {
+        // the prompt goes through in chunks of up to 16 tokens (weights read once per chunk); the last token takes the
+        // single-token path below, which produces the logits
+        while (n_tokens - 1 - first >= 2) {
+            const int T = n_tokens - 1 - first < 16 ? n_tokens - 1 - first : 16;
+            PI_TRY(pi::prefill_chunk(m, tokens + first, T, n_past + first));
+            first += T;
+        }
+    }
+    for (int i = first; i < n_tokens; ++i) {
         const bool last = i == n_tokens - 1;
         hipLaunchKernelGGL(set_state_kernel, dim3(1), dim3(64), 0, m->stream, m->d_token, m->d_pos, tokens[i], n_past + i);
         PI_TRY(pi::check_launch("set_state"));

@@ -9,6 +9,8 @@
 
 struct BatchState {
     int n_seq = 0, max_steps = 4096;
+    bool prefill = false;                 // prompt chunks of the model's own sequence: tokens share the model's KV cache
+    float * q_rot = nullptr;
     size_t cache_seq_stride = 0;          // elements per sequence: n_layer * n_head_kv * n_ctx * hd
     __half *k_cache = nullptr, *v_cache = nullptr;
     float *x = nullptr, *x2 = nullptr, *qkv = nullptr, *att = nullptr, *attn_out = nullptr, *ffn_inp = nullptr, *hidden = nullptr;
@@ -28,8 +30,7 @@ pi_norm mk_norm(int kind, float eps, const Tensor & w, const Tensor * b) {
     return n;
 }
 
-int batch_layer(pi_model * m, int il) {
-    BatchState * b = m->batch;
+int batch_layer(pi_model * m, BatchState * b, int il) {
     const pi_hparams & hp = m->hp;
     const int T = b->n_seq, d = hp.n_embd, ff = hp.n_ff, hd = m->hd, gqa = m->gqa;
     const bool falcon = hp.arch == PI_ARCH_FALCON;
@@ -48,8 +49,12 @@ int batch_layer(pi_model * m, int il) {
     else an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
     PI_TRY(pi_k_norm_round_f16(x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));       // Falcon: the predictor reads the raw layer input
     PI_TRY(pi_k_gemm_f16(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr, st));
-    PI_TRY(pi_k_attn_fused_batch(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
-                                 hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, hp.n_ctx, b->d_pos, b->att, d, b->att16, st));
+    if (b->prefill)
+        PI_TRY(pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, b->d_pos, hp.n_ctx, b->q_rot,
+                               m->k_cache + kv_off, m->v_cache + kv_off, b->att, d, b->att16, st));
+    else
+        PI_TRY(pi_k_attn_fused_batch(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
+                                     hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, hp.n_ctx, b->d_pos, b->att, d, b->att16, st));
 
     pi_norm fn;
     if (!falcon) {
@@ -83,7 +88,7 @@ int batch_step(pi_model * m) {
     const bool falcon = hp.arch == PI_ARCH_FALCON;
     hipStream_t st = m->stream;
     PI_TRY(pi_k_embed_batch(m->glob[PI_T_TOK_EMBD].dev, d, b->d_tokens, T, b->x, st));
-    for (int il = 0; il < hp.n_layer; ++il) PI_TRY(batch_layer(m, il));
+    for (int il = 0; il < hp.n_layer; ++il) PI_TRY(batch_layer(m, b, il));
     pi_norm on = mk_norm(falcon ? 2 : 1, hp.norm_eps, m->glob[PI_T_OUTPUT_NORM], falcon ? &m->glob[PI_T_OUTPUT_NORM_B] : nullptr);
     PI_TRY(pi_k_norm_round_f16(b->x, T, d, &on, b->xa16, nullptr, st));
     PI_TRY(pi_k_gemm_f16(m->glob[PI_T_OUTPUT].dev, hp.n_vocab, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->logits, nullptr, st));
@@ -94,8 +99,81 @@ int batch_step(pi_model * m) {
 
 }  // namespace
 
+namespace {
+
+const char * batch_unsupported(pi_model * m) {
+    const pi_hparams & hp = m->hp;
+    if (m->hybrid) return "hybrid models decode one token at a time";
+    for (int il = 0; il < hp.n_layer; ++il)
+        for (int k : {PI_T_WQKV, PI_T_WO, PI_T_FC1, PI_T_FC2, PI_T_FFN_UP, PI_T_FFN_DOWN_T})
+            if (m->L(il, k).type != PI_TYPE_F16) return "multi-token steps need F16 weights";
+    if (m->glob[PI_T_TOK_EMBD].type != PI_TYPE_F16 || m->glob[PI_T_OUTPUT].type != PI_TYPE_F16) return "multi-token steps need F16 weights";
+    if (hp.n_embd % 512 || (int)m->L(0, PI_T_FC1).ne1 % 128) return "n_embd % 512 == 0 and predictor rank % 128 == 0 required";
+    return nullptr;
+}
+
+// step buffers for up to T tokens; caches only for independent sequences
+BatchState * batch_alloc(pi_model * m, int T, bool with_caches) {
+    const pi_hparams & hp = m->hp;
+    const int d = hp.n_embd, ff = hp.n_ff, r = (int)m->L(0, PI_T_FC1).ne1;
+    BatchState * b = new BatchState();
+    b->n_seq = T;
+    b->cache_seq_stride = (size_t)hp.n_layer * hp.n_head_kv * hp.n_ctx * m->hd;
+    const size_t n = T;
+    bool ok = true;
+    if (with_caches) {
+        b->k_cache = m->alloc<__half>(b->cache_seq_stride * n); b->v_cache = m->alloc<__half>(b->cache_seq_stride * n);
+        ok = b->k_cache && b->v_cache;
+    } else {
+        b->q_rot = m->alloc<float>(n * d);
+        ok = b->q_rot != nullptr;
+    }
+    b->x = m->alloc<float>(n * d); b->x2 = m->alloc<float>(n * d); b->qkv = m->alloc<float>(n * (d + 2 * m->gqa));
+    b->att = m->alloc<float>(n * d); b->attn_out = m->alloc<float>(n * d); b->ffn_inp = m->alloc<float>(n * d);
+    b->hidden = m->alloc<float>(n * r); b->pred_logits = m->alloc<float>(n * ff); b->logits = m->alloc<float>(n * hp.n_vocab);
+    b->xa16 = m->alloc<__half>(n * d); b->xf16 = m->alloc<__half>(n * d); b->xp16 = m->alloc<__half>(n * d);
+    b->att16 = m->alloc<__half>(n * d); b->hid16 = m->alloc<__half>(n * r);
+    b->d_tokens = m->alloc<int32_t>(n); b->d_pos = m->alloc<int32_t>(n); b->d_step = m->alloc<int32_t>(1);
+    b->d_out_tokens = m->alloc<int32_t>((size_t)b->max_steps * n); b->union_rows = m->alloc<int32_t>(ff); b->n_union = m->alloc<int32_t>(hp.n_layer);
+    if (!ok || !b->x || !b->x2 || !b->qkv || !b->att || !b->attn_out || !b->ffn_inp || !b->hidden || !b->pred_logits || !b->logits ||
+        !b->xa16 || !b->xf16 || !b->xp16 || !b->att16 || !b->hid16 || !b->d_tokens || !b->d_pos || !b->d_step || !b->d_out_tokens || !b->union_rows || !b->n_union) {
+        delete b;
+        return nullptr;
+    }
+    return b;
+}
+
+}  // namespace
+
 namespace pi {
+bool prefill_supported(pi_model * m) {
+    const char * off = getenv("PI_NO_PREFILL");
+    return !(off && off[0] == '1') && !m->capture && batch_unsupported(m) == nullptr;
+}
+
+// T <= 16 consecutive prompt tokens of the model's own sequence in one step: the weights are read once for the chunk
+// (the prompt-phase counterpart of llama_decode with n_tokens > 1; the reference's batch kernels, ggml-cuda.cu:6994-7034)
+int prefill_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) {
+    if (T < 1 || T > 16) return pi::fail(PI_E_ARG, "prefill_chunk: 1 <= T <= 16");
+    if (!m->prefill) {
+        m->prefill = batch_alloc(m, 16, false);
+        if (!m->prefill) return PI_E_HIP;
+        m->prefill->prefill = true;
+    }
+    BatchState * b = m->prefill;
+    b->n_seq = T;
+    int32_t pos[16];
+    for (int t = 0; t < T; ++t) pos[t] = n_past + t;
+    PI_HIP_TRY(hipMemcpyAsync(b->d_tokens, tokens, sizeof(int32_t) * T, hipMemcpyHostToDevice, m->stream));
+    PI_HIP_TRY(hipMemcpyAsync(b->d_pos, pos, sizeof(int32_t) * T, hipMemcpyHostToDevice, m->stream));
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    PI_TRY(pi_k_embed_batch(m->glob[PI_T_TOK_EMBD].dev, m->hp.n_embd, b->d_tokens, T, b->x, m->stream));
+    for (int il = 0; il < m->hp.n_layer; ++il) PI_TRY(batch_layer(m, b, il));
+    return PI_OK;
+}
+
 void batch_destroy(pi_model * m) {
+    if (m->prefill) { delete m->prefill; m->prefill = nullptr; }
     if (!m->batch) return;
     if (m->batch->graph_exec) (void)hipGraphExecDestroy(m->batch->graph_exec);
     if (m->batch->graph) (void)hipGraphDestroy(m->batch->graph);
@@ -110,34 +188,11 @@ int pi_model_batch_init(pi_model * m, int n_seq) {
     if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_batch_init: model not finalized");
     if (n_seq < 1 || n_seq > 16) return pi::fail(PI_E_ARG, "pi_model_batch_init: 1 <= n_seq <= 16");
     if (m->batch) return pi::fail(PI_E_STATE, "pi_model_batch_init: already initialised");
-    const pi_hparams & hp = m->hp;
-    const int d = hp.n_embd, ff = hp.n_ff;
-    if (m->hybrid) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: hybrid models decode one sequence at a time");
     if (!m->rope_table) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: head size outside the fused attention kernel");
-    const int r = (int)m->L(0, PI_T_FC1).ne1;
-    for (int il = 0; il < hp.n_layer; ++il)
-        for (int k : {PI_T_WQKV, PI_T_WO, PI_T_FC1, PI_T_FC2, PI_T_FFN_UP, PI_T_FFN_DOWN_T})
-            if (m->L(il, k).type != PI_TYPE_F16) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: batched decoding needs F16 weights");
-    if (m->glob[PI_T_TOK_EMBD].type != PI_TYPE_F16 || m->glob[PI_T_OUTPUT].type != PI_TYPE_F16)
-        return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: batched decoding needs F16 weights");
-    if (d % 512 || r % 128) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: n_embd % 512 == 0 and predictor rank % 128 == 0 required");
-    BatchState * b = new BatchState();
-    b->n_seq = n_seq;
-    b->cache_seq_stride = (size_t)hp.n_layer * hp.n_head_kv * hp.n_ctx * m->hd;
+    if (const char * why = batch_unsupported(m)) { pi::set_error(why); return PI_E_UNSUPPORTED; }
+    BatchState * b = batch_alloc(m, n_seq, true);
+    if (!b) return PI_E_HIP;
     const size_t T = n_seq;
-    b->k_cache = m->alloc<__half>(b->cache_seq_stride * T); b->v_cache = m->alloc<__half>(b->cache_seq_stride * T);
-    b->x = m->alloc<float>(T * d); b->x2 = m->alloc<float>(T * d); b->qkv = m->alloc<float>(T * (d + 2 * m->gqa));
-    b->att = m->alloc<float>(T * d); b->attn_out = m->alloc<float>(T * d); b->ffn_inp = m->alloc<float>(T * d);
-    b->hidden = m->alloc<float>(T * r); b->pred_logits = m->alloc<float>(T * ff); b->logits = m->alloc<float>(T * hp.n_vocab);
-    b->xa16 = m->alloc<__half>(T * d); b->xf16 = m->alloc<__half>(T * d); b->xp16 = m->alloc<__half>(T * d);
-    b->att16 = m->alloc<__half>(T * d); b->hid16 = m->alloc<__half>(T * r);
-    b->d_tokens = m->alloc<int32_t>(T); b->d_pos = m->alloc<int32_t>(T); b->d_step = m->alloc<int32_t>(1);
-    b->d_out_tokens = m->alloc<int32_t>((size_t)b->max_steps * T); b->union_rows = m->alloc<int32_t>(ff); b->n_union = m->alloc<int32_t>(hp.n_layer);
-    if (!b->k_cache || !b->v_cache || !b->x || !b->x2 || !b->qkv || !b->att || !b->attn_out || !b->ffn_inp || !b->hidden || !b->pred_logits || !b->logits ||
-        !b->xa16 || !b->xf16 || !b->xp16 || !b->att16 || !b->hid16 || !b->d_tokens || !b->d_pos || !b->d_step || !b->d_out_tokens || !b->union_rows || !b->n_union) {
-        delete b;
-        return PI_E_HIP;
-    }
     PI_HIP_TRY(hipMemsetAsync(b->k_cache, 0, sizeof(__half) * b->cache_seq_stride * T, m->stream));
     PI_HIP_TRY(hipMemsetAsync(b->v_cache, 0, sizeof(__half) * b->cache_seq_stride * T, m->stream));
     PI_HIP_TRY(hipStreamSynchronize(m->stream));

@@ -46,6 +46,7 @@ struct pi_model {
     float *cap_ffn = nullptr, *cap_logits = nullptr, *cap_src = nullptr;       // device
     pi::ColdPath * cold = nullptr;
     BatchState * batch = nullptr;         // per-sequence caches and step buffers of batched decoding
+    BatchState * prefill = nullptr;       // step buffers for prompt chunks of the model's own sequence
 
     Tensor & L(int il, int kind) { return layers[(size_t)il * PI_T_COUNT + kind]; }
 
@@ -58,4 +59,6 @@ struct pi_model {
 
 namespace pi {
 void batch_destroy(pi_model * m);       // frees the batched-decoding state (graphs; device buffers belong to the model)
+bool prefill_supported(pi_model * m);   // F16 weights, every neuron on the GPU, shapes the multi-token kernels cover
+int  prefill_chunk(pi_model * m, const int32_t * tokens, int T, int n_past);
 }

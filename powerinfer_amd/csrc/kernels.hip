@@ -1746,7 +1746,11 @@ __global__ __launch_bounds__(kBlock) void h_q8_gather_kernel(const float * __res
 // ---------------------------------------------------------------------------------------------------
 __global__ void rope_kv_store_kernel(const float * __restrict__ qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
                                      const int32_t * __restrict__ pos_p, int n_ctx, float * __restrict__ q_rot,
-                                     __half * __restrict__ k_cache, __half * __restrict__ v_cache) {
+                                     __half * __restrict__ k_cache, __half * __restrict__ v_cache, int qkv_stride, int q_stride) {
+    // blockIdx.y = token of a prompt chunk (same sequence, its own position); 0 for single-token decoding
+    qkv += (size_t)blockIdx.y * qkv_stride;
+    q_rot += (size_t)blockIdx.y * q_stride;
+    pos_p += blockIdx.y;
     const int h = blockIdx.x, i = threadIdx.x;           // i = pair index
     const int pos = *pos_p;
     if (h < n_head + n_head_kv) {
@@ -1781,7 +1785,13 @@ __global__ void rope_kv_store_kernel(const float * __restrict__ qkv, int n_head,
 // ---------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(kBlock) void attn_decode_kernel(const float * __restrict__ q_rot, const __half * __restrict__ k_cache,
                                                              const __half * __restrict__ v_cache, int n_head, int n_head_kv, int hd,
-                                                             int n_ctx, const int32_t * __restrict__ pos_p, float * __restrict__ out) {
+                                                             int n_ctx, const int32_t * __restrict__ pos_p, float * __restrict__ out,
+                                                             int q_stride, int out_stride, __half * __restrict__ out16) {
+    // blockIdx.y = token of a prompt chunk: it sees the cache cells up to its own position (causal mask)
+    q_rot += (size_t)blockIdx.y * q_stride;
+    out += (size_t)blockIdx.y * out_stride;
+    if (out16) out16 += (size_t)blockIdx.y * out_stride;
+    pos_p += blockIdx.y;
     extern __shared__ __align__(16) unsigned char smem[];
     float * s    = reinterpret_cast<float *>(smem);               // [n_kv] scores, then probabilities
     float * part = s + n_ctx;                                     // [groups][hd] partial outputs
@@ -1840,6 +1850,7 @@ __global__ __launch_bounds__(kBlock) void attn_decode_kernel(const float * __res
         float v = part[e];
         for (int g = 1; g < ngrp; ++g) v += part[g * hd + e];
         out[(size_t)h * hd + e] = v;
+        if (out16) out16[(size_t)h * hd + e] = __float2half_rn(v);
     }
 }
 
@@ -2695,7 +2706,7 @@ int pi_k_rope_kv_store(const float * qkv, int n_head, int n_head_kv, int hd, int
     if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd <= 0 || hd % 2 || hd / 2 > 1024 || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_rope_kv_store: bad head geometry or mode");
     hipLaunchKernelGGL(rope_kv_store_kernel, dim3(n_head + 2 * n_head_kv), dim3(hd / 2), 0, (hipStream_t)stream,
-                       qkv, n_head, n_head_kv, hd, mode, theta_scale, pos, n_ctx, q_rot, (__half *)k_cache, (__half *)v_cache);
+                       qkv, n_head, n_head_kv, hd, mode, theta_scale, pos, n_ctx, q_rot, (__half *)k_cache, (__half *)v_cache, 0, 0);
     return pi::check_launch("pi_k_rope_kv_store");
 }
 
@@ -2706,7 +2717,7 @@ int pi_k_attn_decode(const float * q_rot, const void * k_cache, const void * v_c
     const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd);
     if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_decode: context too long for the single-pass kernel");
     hipLaunchKernelGGL(attn_decode_kernel, dim3(n_head), dim3(kBlock), sh, (hipStream_t)stream,
-                       q_rot, (const __half *)k_cache, (const __half *)v_cache, n_head, n_head_kv, hd, n_ctx, pos, out);
+                       q_rot, (const __half *)k_cache, (const __half *)v_cache, n_head, n_head_kv, hd, n_ctx, pos, out, 0, 0, nullptr);
     return pi::check_launch("pi_k_attn_decode");
 }
 
@@ -2739,6 +2750,23 @@ int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_t
     hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head, n_seq), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
                        (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride, (__half *)out_f16);
     return pi::check_launch("pi_k_attn_fused_batch");
+}
+
+int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
+                    const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache, float * out, int out_stride, void * out_f16,
+                    pi_stream_t stream) {
+    if (!qkv || !pos || !q_rot || !k_cache || !v_cache || !out || T <= 0 || T > kBtMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad arguments");
+    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd <= 0 || hd % 8 || hd / 2 > 1024 || kBlock % (hd / 8) || PI_WAVE % (hd / 8) || (mode != 0 && mode != 2))
+        return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad head geometry or mode");
+    const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd);
+    if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_chunk: context too long for the single-pass kernel");
+    hipStream_t st = (hipStream_t)stream;
+    // all K/V rows of the chunk are in the cache before any token of the chunk attends
+    hipLaunchKernelGGL(rope_kv_store_kernel, dim3(n_head + 2 * n_head_kv, T), dim3(hd / 2), 0, st,
+                       qkv, n_head, n_head_kv, hd, mode, theta_scale, pos, n_ctx, q_rot, (__half *)k_cache, (__half *)v_cache, qkv_stride, n_head * hd);
+    hipLaunchKernelGGL(attn_decode_kernel, dim3(n_head, T), dim3(kBlock), sh, st,
+                       q_rot, (const __half *)k_cache, (const __half *)v_cache, n_head, n_head_kv, hd, n_ctx, pos, out, n_head * hd, out_stride, (__half *)out_f16);
+    return pi::check_launch("pi_k_attn_chunk");
 }
 
 int pi_k_step_advance(int32_t * step, pi_stream_t stream) {

@@ -63,6 +63,7 @@ _SIGS = {
     "pi_k_batch_predictor_fc2": (_i, [_vp, _i, _i, _vp, _i, _f, _vp, _vp, _vp]),
     "pi_k_batch_sparse_ffn": (_i, [_vp, _i, _i, _f, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_attn_fused_batch": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),
+    "pi_k_attn_chunk": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     "pi_k_embed_batch": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
     "pi_k_argmax_batch": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _i, _vp]),
     "pi_k_step_advance": (_i, [_vp, _vp]),

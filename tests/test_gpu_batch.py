@@ -179,3 +179,38 @@ def test_batch_init_rejects_unsupported_models():
     with pytest.raises(pl.PiError):
         m.batch_decode([1], [0])
     m.close()
+
+
+@pytest.mark.parametrize("arch", ["llama-tiny", "falcon-tiny"])
+def test_prompt_chunks_match_token_by_token(arch):
+    """A prompt handed over in one call is evaluated in chunks of up to 16 tokens (weights read once per chunk, causal attention
+    inside the chunk); the result must agree with the CPU oracle evaluating the whole prompt as one batch (llama_decode with
+    n_tokens > 1) and with feeding the same tokens one at a time.  As in the single-token model tests one predictor logit on
+    the threshold can flip a neuron in either path (a few percent of one layer's output with these random predictors), so
+    the criterion is the median over several prompts."""
+    from powerinfer_amd.model import Model
+    hp = synth.hparams(arch, seed=12, n_ctx=64)
+    model = synth.make_model(hp)
+    rng = np.random.default_rng(4)
+    err_oracle, err_single, err_after = [], [], []
+    for n in (4, 10, 17, 22, 35):
+        prompt = rng.integers(0, hp.n_vocab, n).astype(np.int32)
+        nxt = rng.integers(0, hp.n_vocab, 3).astype(np.int32)
+        ga, gb = Model(hp).load(model), Model(hp).load(model)
+        _, lg_a = ga.decode(prompt, 0)                       # chunks of up to 16 tokens, the last token alone
+        for i, t in enumerate(prompt):
+            _, lg_b = gb.decode([int(t)], i)
+        om = ol.OracleModel(model)
+        _, lg_o = om.eval([int(t) for t in prompt], 0)
+        err_oracle.append(rel_err(lg_a, lg_o))
+        err_single.append(rel_err(lg_a, lg_b))
+        for i, t in enumerate(nxt):                          # the caches the chunks left behind serve later single-token steps
+            _, la = ga.decode([int(t)], n + i)
+            _, lo = om.eval([int(t)], n + i)
+            err_after.append(rel_err(la, lo))
+        om.close()
+        ga.close()
+        gb.close()
+    assert np.median(err_oracle) < 1e-2, err_oracle
+    assert np.median(err_after) < 1e-2, err_after
+    assert np.median(err_single) < 5e-2 and max(err_single) < 0.3, err_single

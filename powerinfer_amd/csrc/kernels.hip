@@ -2179,6 +2179,96 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __r
     }
 }
 
+// The same mat-mul with row-contiguous global reads (cols % 1024 == 0).  The MFMA operand layout wants lane l to hold
+// row l % 16, which makes a direct load instruction touch 16 rows x 64 B; here a wave instead reads 2 rows x 512 B per
+// instruction (8 instructions = its 16 rows x 256 columns), drops the tile into a wave-private LDS buffer with a padded
+// row stride (conflict-free both ways) and reads it back in operand layout.  No workgroup barrier is involved: the
+// buffer belongs to one wave and LDS operations of a wave complete in order.  Two 256-column tiles of loads are in flight.
+constexpr int kGlStride = 512 + 16;               // bytes per LDS row: 256 fp16 + one 16-byte pad
+template <int RT>
+__global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
+                                                                  int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y,
+                                                                  __half * __restrict__ y16, float thr, unsigned char * __restrict__ row_any) {
+    __shared__ __align__(16) unsigned char tile[kWavesPerBlock][16 * kGlStride];
+    __shared__ float cs[kWavesPerBlock][16][17];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;
+    const int lr = lane >> 5, lc = lane & 31;           // load role: row within the pair, 16-byte chunk within the 512-byte row piece
+    const int row0 = blockIdx.x * 16 * RT;
+    const int tok = i < T ? i : T - 1;
+    const int kw = cols / kWavesPerBlock;               // multiple of 256
+    const int k0 = wave * kw;
+    const __half * bp = xn + (size_t)tok * cols + k0 + g * 8;
+    unsigned char * mytile = tile[wave];
+    pi_f4 acc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    const int n_ss = kw / 256;                          // 256-column super-steps of this wave
+    pi_u32x4 ld[2][RT][8];
+    auto issue = [&](int buf, int ss) {
+        if (ss < n_ss) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    int r = row0 + rt * 16 + 2 * j + lr;
+                    r = r < rows ? r : rows - 1;
+                    ld[buf][rt][j] = pi_ld_stream(W + (size_t)r * cols + k0 + ss * 256 + lc * 8);
+                }
+        }
+    };
+    issue(0, 0);
+    issue(1, 1);
+    for (int ss = 0; ss < n_ss; ss += 2) {
+#pragma unroll
+        for (int buf = 0; buf < 2; ++buf) {
+            const int cur = ss + buf;
+            if (cur < n_ss) {
+                pi_u32x4 b[8];
+#pragma unroll
+                for (int st = 0; st < 8; ++st) b[st] = pi_ld16(bp + cur * 256 + st * 32);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (2 * j + lr) * kGlStride + lc * 16) = ld[buf][rt][j];
+#pragma unroll
+                    for (int st = 0; st < 8; ++st) {
+                        const pi_u32x4 a = *reinterpret_cast<const pi_u32x4 *>(mytile + i * kGlStride + (4 * st + g) * 16);
+                        acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a), __builtin_bit_cast(pi_h8, b[st]), acc[rt], 0, 0, 0);
+                    }
+                }
+            }
+            issue(buf, cur + 2);
+        }
+    }
+    const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        if (rt > 0) __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 4; ++r) cs[wave][4 * g + r][i] = acc[rt][r];
+        __syncthreads();
+        const int row = row0 + rt * 16 + rr;
+        bool act = false;
+        if (row < rows && t < T) {
+            float sum = cs[0][rr][t];
+#pragma unroll
+            for (int w = 1; w < kWavesPerBlock; ++w) sum += cs[w][rr][t];
+            const size_t o = (size_t)t * rows + row;
+            if (epi == PI_EPI_RELU) sum = fmaxf(sum, 0.0f);
+            else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
+            else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[o]), add2[o]);
+            y[o] = sum;
+            if (y16) y16[o] = __float2half_rn(sum);
+            act = !(sum < thr);
+        }
+        if (row_any) {
+            const unsigned long long m = __ballot(act);
+            if (t == 0 && row < rows) row_any[row] = ((m >> (16 * (lane >> 4))) & 0xffffull) ? 1 : 0;
+        }
+    }
+}
+
 // union over the tokens of the step of the predictor's active sets: ascending list of the neurons whose flag the
 // predictor's mat-mul epilogue raised (single workgroup: wave ballot per 64 neurons, popcount prefix over the mask words)
 __global__ __launch_bounds__(1024) void union_active_kernel(const unsigned char * __restrict__ row_any, int ff,
@@ -2666,7 +2756,11 @@ static int gemm_launch(const char * who, const void * W, int rows, int cols, con
     const int rt = rows >= 16384 ? 4 : rows >= 8192 ? 2 : 1;
 #define PI_GEMM_T16(RT) hipLaunchKernelGGL((gemm_t16_f16_kernel<RT>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(kBlock), 0, (hipStream_t)stream, \
                        (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any)
-    if (rt == 4) PI_GEMM_T16(4); else if (rt == 2) PI_GEMM_T16(2); else PI_GEMM_T16(1);
+#define PI_GEMM_LDS(RT) hipLaunchKernelGGL((gemm_t16_lds_f16_kernel<RT>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(kBlock), 0, (hipStream_t)stream, \
+                       (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any)
+    if (cols % 1024 == 0) { if (rt >= 2) PI_GEMM_LDS(2); else PI_GEMM_LDS(1); }
+    else if (rt == 4) PI_GEMM_T16(4); else if (rt == 2) PI_GEMM_T16(2); else PI_GEMM_T16(1);
+#undef PI_GEMM_LDS
 #undef PI_GEMM_T16
     return pi::check_launch(who);
 }

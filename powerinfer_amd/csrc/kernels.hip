@@ -2292,8 +2292,8 @@ __global__ __launch_bounds__(1024) void union_active_kernel(const unsigned char 
 __global__ __launch_bounds__(kBlock) void batch_upgate_f16_kernel(const __half * __restrict__ Wup, const __half * __restrict__ Wgate, int cols,
                                                                   const __half * __restrict__ xn, int T, const float * __restrict__ logits, int ff, float thr,
                                                                   const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
-                                                                  float * __restrict__ hc) {
-    // hc[u][t] is stored already rounded to fp16 (kept as fp32): the CPU axpy rounds h before use (ggml.c:14420-14431)
+                                                                  __half * __restrict__ hc, int hstride) {
+    // hc[t][u] (token-major, stride hstride) holds h already rounded to fp16: the CPU axpy rounds h before use (ggml.c:14420-14431)
     __shared__ float cu[kWavesPerBlock][16][17], cg[kWavesPerBlock][16][17];
     const int n = *n_union;
     const int u0 = blockIdx.x * 16;
@@ -2335,10 +2335,94 @@ __global__ __launch_bounds__(kBlock) void batch_upgate_f16_kernel(const __half *
             float su = cu[0][rr][t], sg = cg[0][rr][t];
 #pragma unroll
             for (int w = 1; w < kWavesPerBlock; ++w) { su += cu[w][rr][t]; sg += cg[w][rr][t]; }
-            h = pi_round_f16(Wgate ? __fmul_rn(fmaxf(sg, 0.0f), su) : fmaxf(su, 0.0f));
+            h = Wgate ? __fmul_rn(fmaxf(sg, 0.0f), su) : fmaxf(su, 0.0f);
         }
     }
-    hc[(size_t)(u0 + rr) * kBtMaxT + t] = h;
+    hc[(size_t)t * hstride + u0 + rr] = __float2half_rn(h);
+}
+
+// sparse gate/up with row-contiguous reads (cols % 1024 == 0): the loader of gemm_t16_lds_f16_kernel applied to the gathered
+// rows of the union list; the gate tile and the up tile of a 256-column step pass through the same wave-private LDS buffer.
+__global__ __launch_bounds__(kBlock) void batch_upgate_lds_f16_kernel(const __half * __restrict__ Wup, const __half * __restrict__ Wgate, int cols,
+                                                                      const __half * __restrict__ xn, int T, const float * __restrict__ logits, int ff, float thr,
+                                                                      const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
+                                                                      __half * __restrict__ hc, int hstride) {
+    __shared__ __align__(16) unsigned char tile[kWavesPerBlock][16 * kGlStride];
+    __shared__ float cu[kWavesPerBlock][16][17], cg[kWavesPerBlock][16][17];
+    const int n = *n_union;
+    const int u0 = blockIdx.x * 16;
+    if (u0 >= n) return;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;
+    const int lr = lane >> 5, lc = lane & 31;
+    const int tok = i < T ? i : T - 1;
+    const int kw = cols / kWavesPerBlock, k0 = wave * kw;
+    const __half * bp = xn + (size_t)tok * cols + k0 + g * 8;
+    unsigned char * mytile = tile[wave];
+    size_t roff[8];                                       // row offsets of the 8 load instructions of this lane
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int u = u0 + 2 * j + lr;
+        roff[j] = (size_t)list[u < n ? u : n - 1] * cols + k0 + lc * 8;
+    }
+    const bool has_gate = Wgate != nullptr;
+    pi_f4 au = {0.0f, 0.0f, 0.0f, 0.0f}, ag = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int n_ss = kw / 256;
+    pi_u32x4 lu[2][8], lg[2][8];
+    auto issue = [&](int buf, int ss) {
+        if (ss < n_ss) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                lu[buf][j] = pi_ld_stream(Wup + roff[j] + ss * 256);
+                if (has_gate) lg[buf][j] = pi_ld_stream(Wgate + roff[j] + ss * 256);
+            }
+        }
+    };
+    issue(0, 0);
+    issue(1, 1);
+    for (int ss = 0; ss < n_ss; ss += 2) {
+#pragma unroll
+        for (int buf = 0; buf < 2; ++buf) {
+            const int cur = ss + buf;
+            if (cur < n_ss) {
+                pi_u32x4 b[8];
+#pragma unroll
+                for (int st = 0; st < 8; ++st) b[st] = pi_ld16(bp + cur * 256 + st * 32);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (2 * j + lr) * kGlStride + lc * 16) = lu[buf][j];
+#pragma unroll
+                for (int st = 0; st < 8; ++st) {
+                    const pi_u32x4 a = *reinterpret_cast<const pi_u32x4 *>(mytile + i * kGlStride + (4 * st + g) * 16);
+                    au = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a), __builtin_bit_cast(pi_h8, b[st]), au, 0, 0, 0);
+                }
+                if (has_gate) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (2 * j + lr) * kGlStride + lc * 16) = lg[buf][j];
+#pragma unroll
+                    for (int st = 0; st < 8; ++st) {
+                        const pi_u32x4 a = *reinterpret_cast<const pi_u32x4 *>(mytile + i * kGlStride + (4 * st + g) * 16);
+                        ag = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a), __builtin_bit_cast(pi_h8, b[st]), ag, 0, 0, 0);
+                    }
+                }
+            }
+            issue(buf, cur + 2);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) { cu[wave][4 * g + r][i] = au[r]; cg[wave][4 * g + r][i] = ag[r]; }
+    __syncthreads();
+    const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
+    float h = 0.0f;
+    if (u0 + rr < n && t < T) {
+        const int rrow = list[u0 + rr];
+        if (!(logits[(size_t)t * ff + rrow] < thr)) {
+            float su = cu[0][rr][t], sg = cg[0][rr][t];
+#pragma unroll
+            for (int w = 1; w < kWavesPerBlock; ++w) { su += cu[w][rr][t]; sg += cg[w][rr][t]; }
+            h = has_gate ? __fmul_rn(fmaxf(sg, 0.0f), su) : fmaxf(su, 0.0f);
+        }
+    }
+    hc[(size_t)t * hstride + u0 + rr] = __float2half_rn(h);
 }
 
 // sparse down projection for the step: partial[g][t][c] = sum over the union entries of row group g of hc[u][t] * down[row_u][c].
@@ -2349,7 +2433,7 @@ constexpr int kBaGroups = 8;
 constexpr int kBaBlock = 512;
 constexpr int kBaWaves = kBaBlock / PI_WAVE;
 constexpr int kBaTile = 256;
-__global__ __launch_bounds__(kBaBlock) void batch_axpy_f16_kernel(const __half * __restrict__ Wd, int cols, const float * __restrict__ hc,
+__global__ __launch_bounds__(kBaBlock) void batch_axpy_f16_kernel(const __half * __restrict__ Wd, int cols, const __half * __restrict__ hc, int hstride,
                                                                   const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
                                                                   float * __restrict__ partial) {
     __shared__ float tile[kBtMaxT][kBaTile];
@@ -2376,10 +2460,9 @@ __global__ __launch_bounds__(kBaBlock) void batch_axpy_f16_kernel(const __half *
             if (u < n) {
                 const __half2 * hw = reinterpret_cast<const __half2 *>(&w[j]);
                 const float2 w01 = __half22float2(hw[0]), w23 = __half22float2(hw[1]);
-                const float * hp = hc + (size_t)u * kBtMaxT;
 #pragma unroll
                 for (int t = 0; t < kBtMaxT; ++t) {
-                    const float h = hp[t];
+                    const float h = __half2float(hc[(size_t)t * hstride + u]);
                     acc[t][0] = fmaf(w01.x, h, acc[t][0]); acc[t][1] = fmaf(w01.y, h, acc[t][1]);
                     acc[t][2] = fmaf(w23.x, h, acc[t][2]); acc[t][3] = fmaf(w23.y, h, acc[t][3]);
                 }
@@ -2405,13 +2488,79 @@ __global__ __launch_bounds__(kBaBlock) void batch_axpy_f16_kernel(const __half *
     }
 }
 
-__global__ __launch_bounds__(kBlock) void batch_reduce_kernel(const float * __restrict__ partial, int T, int cols, int epi,
+// The down projection on the matrix cores (cols % 1024 == 0).  out[t][c] = sum_u h[t][u] * down[row_u][c] has the union rows as its
+// reduction dimension, along which the weight matrix is NOT contiguous, so the operand layout cannot be loaded directly: a wave
+// reads 16 union rows x 256 columns row-contiguously (2 rows x 512 B per instruction), drops them into its private LDS tile and
+// reads the B fragments column-wise (4 rows of one column per lane: four 2-byte LDS reads) for 16 column tiles of
+// v_mfma_f32_16x16x16_f16; the A fragment is 4 consecutive entries of h[t][.] (one 8-byte load from the token-major h).
+// grid = (cols / 1024, G row groups); wave w of a workgroup owns columns 256 w .. 256 w + 255 of the workgroup's 1024 and walks
+// the 16-row steps g, g + G, ...; partial[g][t][c] is summed by batch_reduce_kernel.
+typedef _Float16 pi_h4 __attribute__((ext_vector_type(4)));
+constexpr int kBmGroups = 32;
+__global__ __launch_bounds__(kBlock) void batch_axpy_mfma_f16_kernel(const __half * __restrict__ Wd, int cols, const __half * __restrict__ hc, int hstride,
+                                                                     const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
+                                                                     float * __restrict__ partial) {
+    __shared__ __align__(16) unsigned char tile[kWavesPerBlock][16 * kGlStride];
+    const int n = *n_union;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;
+    const int lr = lane >> 5, lc = lane & 31;
+    const int c0 = blockIdx.x * 1024 + wave * 256;
+    unsigned char * mytile = tile[wave];
+    pi_f4 acc[16];
+#pragma unroll
+    for (int ct = 0; ct < 16; ++ct) acc[ct] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    const int n_steps = (n + 15) / 16;
+    pi_u32x4 ld[2][8];
+    pi_u32x2 af[2];
+    auto issue = [&](int buf, int ks) {
+        if (ks < n_steps) {
+            const int u0 = ks * 16;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int u = u0 + 2 * j + lr;
+                ld[buf][j] = pi_ld_stream(Wd + (size_t)list[u < n ? u : n - 1] * cols + c0 + lc * 8);
+            }
+            af[buf] = *reinterpret_cast<const pi_u32x2 *>(hc + (size_t)i * hstride + u0 + 4 * g);      // zeros beyond n (written by the gate/up kernel)
+        }
+    };
+    issue(0, blockIdx.y);
+    issue(1, blockIdx.y + kBmGroups);
+    for (int ks = blockIdx.y; ks < n_steps; ks += 2 * kBmGroups) {
+#pragma unroll
+        for (int buf = 0; buf < 2; ++buf) {
+            const int cur = ks + buf * kBmGroups;
+            if (cur < n_steps) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (2 * j + lr) * kGlStride + lc * 16) = ld[buf][j];
+                const pi_h4 a = __builtin_bit_cast(pi_h4, af[buf]);
+#pragma unroll
+                for (int ct = 0; ct < 16; ++ct) {
+                    const unsigned char * bp = mytile + (4 * g) * kGlStride + (ct * 16 + i) * 2;
+                    const uint32_t e0 = *reinterpret_cast<const uint16_t *>(bp), e1 = *reinterpret_cast<const uint16_t *>(bp + kGlStride);
+                    const uint32_t e2 = *reinterpret_cast<const uint16_t *>(bp + 2 * kGlStride), e3 = *reinterpret_cast<const uint16_t *>(bp + 3 * kGlStride);
+                    const pi_u32x2 bw = {e0 | (e1 << 16), e2 | (e3 << 16)};
+                    acc[ct] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, __builtin_bit_cast(pi_h4, bw), acc[ct], 0, 0, 0);
+                }
+            }
+            issue(buf, cur + 2 * kBmGroups);
+        }
+    }
+    // accumulator lane l: tokens 4 * (l / 16) .. + 3 of column l % 16 of every column tile
+#pragma unroll
+    for (int ct = 0; ct < 16; ++ct)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            partial[((size_t)blockIdx.y * kBtMaxT + 4 * g + r) * cols + c0 + ct * 16 + i] = acc[ct][r];
+}
+
+__global__ __launch_bounds__(kBlock) void batch_reduce_kernel(const float * __restrict__ partial, int n_groups, int T, int cols, int epi,
                                                               const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ out) {
     const int idx = blockIdx.x * blockDim.x + threadIdx.x;
     if (idx >= T * cols) return;
     const int t = idx / cols, c = idx - t * cols;
     float sum = 0.0f;
-    for (int g = 0; g < kBaGroups; ++g) sum += partial[((size_t)g * kBtMaxT + t) * cols + c];
+    for (int g = 0; g < n_groups; ++g) sum += partial[((size_t)g * kBtMaxT + t) * cols + c];
     if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[idx]);
     else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[idx]), add2[idx]);
     out[idx] = sum;
@@ -2470,7 +2619,7 @@ struct pi_workspace {
     int32_t *      hq;             // [max_ff]  Q4_0 axpy: int8 value of h per active row
     float *        hd;             // [max_ff]  and its Q8_0 block scale
     float *        ffn_partial;    // [max(max_ff/32, 32 * 16)][max_d]  partial outputs of the fused sparse FFN / of the batched axpy
-    float *        hc_batch;       // [max_ff][16]  h of the union rows for a batched step
+    __half *       hc_batch;       // [16][max_ff + 16]  fp16 h of the union rows for a batched step, token-major
     unsigned char * row_any;       // [max_ff]  batched step: neuron active for at least one token
 };
 constexpr int kAxpyGroups = 32;
@@ -2486,9 +2635,9 @@ pi_workspace * pi_workspace_create(int max_ff, int max_d) {
     ws->partial  = (float *)pi_malloc(sizeof(float) * (size_t)kAxpyGroups * max_d);
     ws->hq       = (int32_t *)pi_malloc(sizeof(int32_t) * max_ff);
     ws->hd       = (float *)pi_malloc(sizeof(float) * max_ff);
-    const size_t n_part = (size_t)((max_ff + 31) / 32) > (size_t)kBaGroups * kBtMaxT ? (size_t)((max_ff + 31) / 32) : (size_t)kBaGroups * kBtMaxT;
+    const size_t n_part = (size_t)((max_ff + 31) / 32) > (size_t)kBmGroups * kBtMaxT ? (size_t)((max_ff + 31) / 32) : (size_t)kBmGroups * kBtMaxT;
     ws->ffn_partial = (float *)pi_malloc(sizeof(float) * n_part * max_d);
-    ws->hc_batch = (float *)pi_malloc(sizeof(float) * ((size_t)max_ff + 16) * kBtMaxT);
+    ws->hc_batch = (__half *)pi_malloc(sizeof(__half) * ((size_t)max_ff + 16) * kBtMaxT);
     ws->row_any = (unsigned char *)pi_malloc((size_t)max_ff + 16);
     if (!ws->words || !ws->counters || !ws->partial || !ws->hq || !ws->hd || !ws->ffn_partial || !ws->hc_batch || !ws->row_any) {
         pi_workspace_destroy(ws); return nullptr;
@@ -2786,11 +2935,20 @@ int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, 
         return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: bad epilogue arguments");
     hipStream_t st = (hipStream_t)stream;
     hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, ws->row_any, ff, ws->words, union_rows, n_union);
-    hipLaunchKernelGGL(batch_upgate_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
-                       (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch);
-    hipLaunchKernelGGL(batch_axpy_f16_kernel, dim3(cols / kBaTile, kBaGroups), dim3(kBaBlock), 0, st, (const __half *)down_t_f16, cols,
-                       ws->hc_batch, union_rows, n_union, ws->ffn_partial);
-    hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, T, cols, epilogue, add1, add2, out);
+    const int hstride = ws->max_ff + 16;
+    if (cols % 1024 == 0) {
+        hipLaunchKernelGGL(batch_upgate_lds_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
+                           (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
+        hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3(cols / 1024, kBmGroups), dim3(kBlock), 0, st, (const __half *)down_t_f16, cols,
+                           ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
+        hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBmGroups, T, cols, epilogue, add1, add2, out);
+    } else {
+        hipLaunchKernelGGL(batch_upgate_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
+                           (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
+        hipLaunchKernelGGL(batch_axpy_f16_kernel, dim3(cols / kBaTile, kBaGroups), dim3(kBaBlock), 0, st, (const __half *)down_t_f16, cols,
+                           ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
+        hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBaGroups, T, cols, epilogue, add1, add2, out);
+    }
     return pi::check_launch("pi_k_batch_sparse_ffn");
 }
 

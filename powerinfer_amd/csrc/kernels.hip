@@ -2179,7 +2179,7 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __r
     }
 }
 
-// The same mat-mul with row-contiguous global reads (cols % 1024 == 0).  The MFMA operand layout wants lane l to hold
+// The same mat-mul with row-contiguous global reads (cols % 256 == 0).  The MFMA operand layout wants lane l to hold
 // row l % 16, which makes a direct load instruction touch 16 rows x 64 B; here a wave instead reads 2 rows x 512 B per
 // instruction (8 instructions = its 16 rows x 256 columns), drops the tile into a wave-private LDS buffer with a padded
 // row stride (conflict-free both ways) and reads it back in operand layout.  No workgroup barrier is involved: the
@@ -2196,14 +2196,13 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
     const int lr = lane >> 5, lc = lane & 31;           // load role: row within the pair, 16-byte chunk within the 512-byte row piece
     const int row0 = blockIdx.x * 16 * RT;
     const int tok = i < T ? i : T - 1;
-    const int kw = cols / kWavesPerBlock;               // multiple of 256
-    const int k0 = wave * kw;
-    const __half * bp = xn + (size_t)tok * cols + k0 + g * 8;
+    // the 256-column super-steps of a row are dealt round-robin to the four waves: wave w takes steps w, w + 4, ...
+    const __half * bp = xn + (size_t)tok * cols + g * 8;
     unsigned char * mytile = tile[wave];
     pi_f4 acc[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
-    const int n_ss = kw / 256;                          // 256-column super-steps of this wave
+    const int n_ss = (cols / 256 - wave + kWavesPerBlock - 1) / kWavesPerBlock;      // super-steps of this wave
     pi_u32x4 ld[2][RT][8];
     auto issue = [&](int buf, int ss) {
         if (ss < n_ss) {
@@ -2213,7 +2212,7 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
                 for (int j = 0; j < 8; ++j) {
                     int r = row0 + rt * 16 + 2 * j + lr;
                     r = r < rows ? r : rows - 1;
-                    ld[buf][rt][j] = pi_ld_stream(W + (size_t)r * cols + k0 + ss * 256 + lc * 8);
+                    ld[buf][rt][j] = pi_ld_stream(W + (size_t)r * cols + (wave + ss * kWavesPerBlock) * 256 + lc * 8);
                 }
         }
     };
@@ -2226,7 +2225,7 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
             if (cur < n_ss) {
                 pi_u32x4 b[8];
 #pragma unroll
-                for (int st = 0; st < 8; ++st) b[st] = pi_ld16(bp + cur * 256 + st * 32);
+                for (int st = 0; st < 8; ++st) b[st] = pi_ld16(bp + (wave + cur * kWavesPerBlock) * 256 + st * 32);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
@@ -2341,7 +2340,7 @@ __global__ __launch_bounds__(kBlock) void batch_upgate_f16_kernel(const __half *
     hc[(size_t)t * hstride + u0 + rr] = __float2half_rn(h);
 }
 
-// sparse gate/up with row-contiguous reads (cols % 1024 == 0): the loader of gemm_t16_lds_f16_kernel applied to the gathered
+// sparse gate/up with row-contiguous reads (cols % 256 == 0): the loader of gemm_t16_lds_f16_kernel applied to the gathered
 // rows of the union list; the gate tile and the up tile of a 256-column step pass through the same wave-private LDS buffer.
 __global__ __launch_bounds__(kBlock) void batch_upgate_lds_f16_kernel(const __half * __restrict__ Wup, const __half * __restrict__ Wgate, int cols,
                                                                       const __half * __restrict__ xn, int T, const float * __restrict__ logits, int ff, float thr,
@@ -2356,25 +2355,24 @@ __global__ __launch_bounds__(kBlock) void batch_upgate_lds_f16_kernel(const __ha
     const int i = lane & 15, g = lane >> 4;
     const int lr = lane >> 5, lc = lane & 31;
     const int tok = i < T ? i : T - 1;
-    const int kw = cols / kWavesPerBlock, k0 = wave * kw;
-    const __half * bp = xn + (size_t)tok * cols + k0 + g * 8;
+    const __half * bp = xn + (size_t)tok * cols + g * 8;       // super-steps w, w + 4, ... of the row belong to wave w
     unsigned char * mytile = tile[wave];
     size_t roff[8];                                       // row offsets of the 8 load instructions of this lane
 #pragma unroll
     for (int j = 0; j < 8; ++j) {
         const int u = u0 + 2 * j + lr;
-        roff[j] = (size_t)list[u < n ? u : n - 1] * cols + k0 + lc * 8;
+        roff[j] = (size_t)list[u < n ? u : n - 1] * cols + wave * 256 + lc * 8;
     }
     const bool has_gate = Wgate != nullptr;
     pi_f4 au = {0.0f, 0.0f, 0.0f, 0.0f}, ag = {0.0f, 0.0f, 0.0f, 0.0f};
-    const int n_ss = kw / 256;
+    const int n_ss = (cols / 256 - wave + kWavesPerBlock - 1) / kWavesPerBlock;
     pi_u32x4 lu[2][8], lg[2][8];
     auto issue = [&](int buf, int ss) {
         if (ss < n_ss) {
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
-                lu[buf][j] = pi_ld_stream(Wup + roff[j] + ss * 256);
-                if (has_gate) lg[buf][j] = pi_ld_stream(Wgate + roff[j] + ss * 256);
+                lu[buf][j] = pi_ld_stream(Wup + roff[j] + ss * kWavesPerBlock * 256);
+                if (has_gate) lg[buf][j] = pi_ld_stream(Wgate + roff[j] + ss * kWavesPerBlock * 256);
             }
         }
     };
@@ -2387,7 +2385,7 @@ __global__ __launch_bounds__(kBlock) void batch_upgate_lds_f16_kernel(const __ha
             if (cur < n_ss) {
                 pi_u32x4 b[8];
 #pragma unroll
-                for (int st = 0; st < 8; ++st) b[st] = pi_ld16(bp + cur * 256 + st * 32);
+                for (int st = 0; st < 8; ++st) b[st] = pi_ld16(bp + (wave + cur * kWavesPerBlock) * 256 + st * 32);
 #pragma unroll
                 for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (2 * j + lr) * kGlStride + lc * 16) = lu[buf][j];
 #pragma unroll
@@ -2488,7 +2486,7 @@ __global__ __launch_bounds__(kBaBlock) void batch_axpy_f16_kernel(const __half *
     }
 }
 
-// The down projection on the matrix cores (cols % 1024 == 0).  out[t][c] = sum_u h[t][u] * down[row_u][c] has the union rows as its
+// The down projection on the matrix cores (cols % 256 == 0).  out[t][c] = sum_u h[t][u] * down[row_u][c] has the union rows as its
 // reduction dimension, along which the weight matrix is NOT contiguous, so the operand layout cannot be loaded directly: a wave
 // reads 16 union rows x 256 columns row-contiguously (2 rows x 512 B per instruction), drops them into its private LDS tile and
 // reads the B fragments column-wise (4 rows of one column per lane: four 2-byte LDS reads) for 16 column tiles of
@@ -2506,6 +2504,7 @@ __global__ __launch_bounds__(kBlock) void batch_axpy_mfma_f16_kernel(const __hal
     const int i = lane & 15, g = lane >> 4;
     const int lr = lane >> 5, lc = lane & 31;
     const int c0 = blockIdx.x * 1024 + wave * 256;
+    if (c0 >= cols) return;                               // no workgroup barrier below: waves are independent
     unsigned char * mytile = tile[wave];
     pi_f4 acc[16];
 #pragma unroll
@@ -2556,14 +2555,22 @@ __global__ __launch_bounds__(kBlock) void batch_axpy_mfma_f16_kernel(const __hal
 
 __global__ __launch_bounds__(kBlock) void batch_reduce_kernel(const float * __restrict__ partial, int n_groups, int T, int cols, int epi,
                                                               const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ out) {
-    const int idx = blockIdx.x * blockDim.x + threadIdx.x;
+    const int idx = (blockIdx.x * blockDim.x + threadIdx.x) * 4;          // cols % 4 == 0: four columns of one token
     if (idx >= T * cols) return;
     const int t = idx / cols, c = idx - t * cols;
-    float sum = 0.0f;
-    for (int g = 0; g < n_groups; ++g) sum += partial[((size_t)g * kBtMaxT + t) * cols + c];
-    if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[idx]);
-    else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[idx]), add2[idx]);
-    out[idx] = sum;
+    const size_t gstride = (size_t)kBtMaxT * cols;
+    const float * p = partial + (size_t)t * cols + c;
+    float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (int g0 = 0; g0 < n_groups; g0 += 8) {
+        float4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = g0 + j < n_groups ? *reinterpret_cast<const float4 *>(p + (size_t)(g0 + j) * gstride) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { sum.x += v[j].x; sum.y += v[j].y; sum.z += v[j].z; sum.w += v[j].w; }
+    }
+    if (epi >= PI_EPI_ADD) { const float4 a = *reinterpret_cast<const float4 *>(add1 + idx); sum.x = __fadd_rn(sum.x, a.x); sum.y = __fadd_rn(sum.y, a.y); sum.z = __fadd_rn(sum.z, a.z); sum.w = __fadd_rn(sum.w, a.w); }
+    if (epi == PI_EPI_ADD2) { const float4 a = *reinterpret_cast<const float4 *>(add2 + idx); sum.x = __fadd_rn(sum.x, a.x); sum.y = __fadd_rn(sum.y, a.y); sum.z = __fadd_rn(sum.z, a.z); sum.w = __fadd_rn(sum.w, a.w); }
+    *reinterpret_cast<float4 *>(out + idx) = sum;
 }
 
 __global__ void embed_f16_batch_kernel(const __half * __restrict__ table, int cols, const int32_t * __restrict__ tokens, float * __restrict__ x) {
@@ -2907,7 +2914,7 @@ static int gemm_launch(const char * who, const void * W, int rows, int cols, con
                        (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any)
 #define PI_GEMM_LDS(RT) hipLaunchKernelGGL((gemm_t16_lds_f16_kernel<RT>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(kBlock), 0, (hipStream_t)stream, \
                        (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any)
-    if (cols % 1024 == 0) { if (rt >= 2) PI_GEMM_LDS(2); else PI_GEMM_LDS(1); }
+    if (cols % 256 == 0) { if (rt >= 2) PI_GEMM_LDS(2); else PI_GEMM_LDS(1); }
     else if (rt == 4) PI_GEMM_T16(4); else if (rt == 2) PI_GEMM_T16(2); else PI_GEMM_T16(1);
 #undef PI_GEMM_LDS
 #undef PI_GEMM_T16
@@ -2936,18 +2943,18 @@ int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, 
     hipStream_t st = (hipStream_t)stream;
     hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, ws->row_any, ff, ws->words, union_rows, n_union);
     const int hstride = ws->max_ff + 16;
-    if (cols % 1024 == 0) {
+    if (cols % 256 == 0) {
         hipLaunchKernelGGL(batch_upgate_lds_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
                            (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
-        hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3(cols / 1024, kBmGroups), dim3(kBlock), 0, st, (const __half *)down_t_f16, cols,
+        hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3((cols + 1023) / 1024, kBmGroups), dim3(kBlock), 0, st, (const __half *)down_t_f16, cols,
                            ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
-        hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBmGroups, T, cols, epilogue, add1, add2, out);
+        hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBmGroups, T, cols, epilogue, add1, add2, out);
     } else {
         hipLaunchKernelGGL(batch_upgate_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
                            (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
         hipLaunchKernelGGL(batch_axpy_f16_kernel, dim3(cols / kBaTile, kBaGroups), dim3(kBaBlock), 0, st, (const __half *)down_t_f16, cols,
                            ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
-        hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBaGroups, T, cols, epilogue, add1, add2, out);
+        hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBaGroups, T, cols, epilogue, add1, add2, out);
     }
     return pi::check_launch("pi_k_batch_sparse_ffn");
 }

@@ -118,6 +118,37 @@ def test_batch_sparse_ffn_matches_oracle(shape, has_gate, T):
     L.pi_workspace_destroy(ws)
 
 
+@pytest.mark.parametrize("thr", [1e9, -1e9])
+def test_batch_sparse_ffn_none_and_all_active(thr):
+    """Empty union (zero output, residual only) and the full union (every row of every matrix read once: the dense FFN)."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    d, ff, r, T = 1024, 1024, 128, 3
+    Lr = synth.make_ffn_layer(seed=5, d=d, ff=ff, r=r, wtype=ol.F16, has_gate=True, T=T)
+    x = Lr["x"]
+    o = ol.ffn_sparse(ol.oracle(), d, ff, r, T, ol.F16, True, Lr["up"], Lr["gate"], Lr["down_t"], Lr["fc1"], Lr["fc2"], x, x,
+                      np.zeros(ff, np.int32), thr, nth=8)
+    ws = L.pi_workspace_create(ff, d)
+    up, gate, down, fc1, fc2 = (pl.DevBuf(host=Lr[k]) for k in ("up", "gate", "down_t", "fc1", "fc2"))
+    xn = gpu_norm_round(pl, L, x)
+    hidden, hid16 = pl.DevBuf(T * r * 4), pl.DevBuf(T * r * 2)
+    logits, out = pl.DevBuf(T * ff * 4), pl.DevBuf(T * d * 4)
+    union, n_union = pl.DevBuf(ff * 4), pl.DevBuf.zeros(4)
+    pl.check(L.pi_k_gemm_f16(fc1.ptr, r, d, xn.ptr, T, pl.EPI_RELU, None, None, hidden.ptr, hid16.ptr, None), "fc1")
+    pl.check(L.pi_k_batch_predictor_fc2(fc2.ptr, ff, r, hid16.ptr, T, thr, logits.ptr, ws, None), "fc2")
+    pl.check(L.pi_k_batch_sparse_ffn(logits.ptr, T, ff, thr, up.ptr, gate.ptr, down.ptr, d, xn.ptr,
+                                     pl.EPI_NONE, None, None, out.ptr, union.ptr, n_union.ptr, ws, None), "batch ffn")
+    pl.sync()
+    n = int(n_union.download(np.int32)[0])
+    got = out.download(np.float32).reshape(T, d)
+    if thr > 0:
+        assert n == 0 and (got == 0).all()
+    else:
+        assert n == ff and np.array_equal(union.download(np.int32, n), np.arange(ff))
+        assert rel_err(got, o["out"]) < 1e-4
+    L.pi_workspace_destroy(ws)
+
+
 @pytest.mark.parametrize("arch", ["llama-tiny", "falcon-tiny"])
 def test_batched_decode_matches_per_sequence_oracle(arch):
     """Four sequences with different prompts advance in lockstep (examples/batched/batched.cpp).  Sequences do not interact,

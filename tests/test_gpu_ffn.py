@@ -177,6 +177,31 @@ def test_threshold_and_empty_list():
         ffn.close()
 
 
+@pytest.mark.parametrize("route", ["one", "two"])
+def test_fused_routes_thresholds_none_some_all(route):
+    """The fused kernels at the extremes of the activity test: nothing active (zero output), a raised threshold, and every
+    neuron active (32 per workgroup: the chunk loop of the one-launch kernel runs four times, the dense-h axpy compacts all ff
+    rows in several passes)."""
+    from powerinfer_amd.ops import SparseFFN
+    d, ff, r = 4096, 2048, (512 if route == "one" else 1024)
+    L = synth.make_ffn_layer(seed=43, d=d, ff=ff, r=r)
+    O = ol.oracle()
+    for thr in (1e9, 0.02, -1e9):
+        o = ol.ffn_sparse(O, d, ff, r, 1, ol.F16, 1, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], L["x"], L["x"],
+                          np.zeros(ff, np.int32), thr, nth=8)
+        ffn = SparseFFN(d, ff, r, ol.F16, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], threshold=thr)
+        res = (ffn.forward_one_launch if route == "one" else ffn.forward_two_launch)(L["x"][0], L["x"][0])
+        mask_g, mask_o = ~(res["logits"] < thr), ~(o["logits"][0] < thr)
+        assert res["n_active"] == int(mask_g.sum())
+        if thr == 1e9:
+            assert res["n_active"] == 0 and (res["out"] == 0).all() and (res["h"] == 0).all()
+        if thr == -1e9:
+            assert res["n_active"] == ff
+        if np.array_equal(mask_g, mask_o):
+            assert np.abs(res["out"] - o["out"][0]).max() <= 1e-4 * max(np.abs(o["out"][0]).max(), 1e-6)
+        ffn.close()
+
+
 def test_axpy_is_deterministic_and_linear():
     """Size-independent properties at full 7B shape: repeated launches are bit-identical (no float atomics),
     and the block output is linear in the down matrix (down_t * 2 doubles the output exactly)."""

@@ -165,6 +165,14 @@ PI_API int pi_k_sparse_axpy(int wtype, const void * down_t, int cols, int n_rows
  * optional outputs for inspection.  Shapes: see pi_k_sparse_ffn_supported.
  */
 PI_API int pi_k_sparse_ffn_supported(int ff, int r, int cols);
+/* the two launches of pi_k_sparse_ffn on their own, for callers that overlap the block with an independent branch (Falcon's
+ * attention reads the same layer input): _partials may run on another stream, _reduce needs it and the residual operands done */
+PI_API int pi_k_sparse_ffn_partials(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                                    const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols,
+                                    const float * x, const pi_norm * norm, float * logits, float * h_dense,
+                                    pi_workspace * ws, pi_stream_t stream);
+PI_API int pi_k_sparse_ffn_reduce(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out,
+                                  int32_t * n_active, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_sparse_ffn(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
                            const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols,
                            const float * x, const pi_norm * norm,

@@ -82,6 +82,8 @@ int upload_tensor(pi_model * m, Tensor & t, int type, const void * data, int64_t
     return pi_memcpy_h2d(t.dev, data, bytes);
 }
 
+bool hp_arch_is_falcon(const pi_model * m) { return m->hp.arch == PI_ARCH_FALCON; }
+
 bool is_ffn_matrix(int kind) { return kind == PI_T_FFN_GATE || kind == PI_T_FFN_UP || kind == PI_T_FFN_DOWN_T; }
 
 pi_norm make_norm(int kind, float eps, const Tensor & w, const Tensor * b) {
@@ -114,6 +116,16 @@ int layer_forward(pi_model * m, int il, bool last_token) {
     const bool layer_hybrid = bk != nullptr;
     float * x = m->x;
 
+    const bool branch = falcon && m->stream2 && !layer_hybrid && !q4 && !m->capture && pi_k_sparse_ffn_supported(ff, r, d);
+    if (branch) {
+        pi_norm fnb = make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
+        PI_HIP_TRY(hipEventRecord(m->ev_fork[il], st));
+        PI_HIP_TRY(hipStreamWaitEvent(m->stream2, m->ev_fork[il], 0));
+        PI_TRY(pi_k_gemv(fc1.type, fc1.dev, r, d, x, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, m->stream2));
+        PI_TRY(pi_k_sparse_ffn_partials(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, nullptr, down.dev, d, x, &fnb,
+                                        nullptr, nullptr, m->ws, m->stream2));
+    }
+
     // attention
     pi_norm an;
     if (!falcon) an = make_norm(1, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), nullptr);
@@ -142,7 +154,16 @@ int layer_forward(pi_model * m, int il, bool last_token) {
     }
 
     // predictor
-    PI_TRY(pi_k_gemv(fc1.type, fc1.dev, r, d, pred_in, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, st));
+    if (!branch) PI_TRY(pi_k_gemv(fc1.type, fc1.dev, r, d, pred_in, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, st));
+    if (branch) {
+        // Falcon's attention and FFN both read the layer input: the predictor + sparse FFN partials run on a second stream
+        // beside q|k|v -> attention -> wo, and only the final reduction (FFN + attention output + input) waits for both
+        PI_HIP_TRY(hipEventRecord(m->ev_join[il], m->stream2));
+        PI_HIP_TRY(hipStreamWaitEvent(st, m->ev_join[il], 0));
+        PI_TRY(pi_k_sparse_ffn_reduce(ff, d, PI_EPI_ADD2, m->attn_out, x, m->x2, n_act, m->ws, st));
+        std::swap(m->x, m->x2);
+        return PI_OK;
+    }
     if (!layer_hybrid && !q4 && pi_k_sparse_ffn_supported(ff, r, d)) {
         // one launch for fc2 + mask + gate/up + each workgroup's share of the down projection, one small reduction
         const void * gp = falcon ? nullptr : gate.dev;
@@ -256,6 +277,9 @@ void pi_model_free(pi_model * m) {
     if (m->graph) (void)hipGraphDestroy(m->graph);
     if (m->ev0) (void)hipEventDestroy(m->ev0);
     if (m->ev1) (void)hipEventDestroy(m->ev1);
+    for (hipEvent_t e : m->ev_fork) if (e) (void)hipEventDestroy(e);
+    for (hipEvent_t e : m->ev_join) if (e) (void)hipEventDestroy(e);
+    if (m->stream2) (void)hipStreamDestroy(m->stream2);
     if (m->cold) pi::cold_destroy(m->cold);
     pi::batch_destroy(m);
     if (m->ws) pi_workspace_destroy(m->ws);
@@ -286,6 +310,17 @@ int pi_model_finalize(pi_model * m) {
     const pi_hparams & hp = m->hp;
     const int d = hp.n_embd, ff = hp.n_ff, gqa = m->gqa;
     PI_HIP_TRY(hipStreamCreateWithFlags(&m->stream, hipStreamNonBlocking));
+    {
+        const char * nb = getenv("PI_NO_BRANCH");          // PI_NO_BRANCH=1: Falcon layers run their two branches one after the other
+        if (hp_arch_is_falcon(m) && !(nb && nb[0] == '1')) {
+            PI_HIP_TRY(hipStreamCreateWithFlags(&m->stream2, hipStreamNonBlocking));
+            m->ev_fork.resize(m->hp.n_layer); m->ev_join.resize(m->hp.n_layer);
+            for (int il = 0; il < m->hp.n_layer; ++il) {
+                PI_HIP_TRY(hipEventCreateWithFlags(&m->ev_fork[il], hipEventDisableTiming));
+                PI_HIP_TRY(hipEventCreateWithFlags(&m->ev_join[il], hipEventDisableTiming));
+            }
+        }
+    }
     PI_HIP_TRY(hipEventCreate(&m->ev0));
     PI_HIP_TRY(hipEventCreate(&m->ev1));
 

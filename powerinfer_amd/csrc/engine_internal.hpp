@@ -28,6 +28,8 @@ struct pi_model {
     bool finalized = false, hybrid = false;
     int hd = 0, gqa = 0, max_steps = 4096;
     hipStream_t stream = nullptr;
+    hipStream_t stream2 = nullptr;         // Falcon: the FFN branch runs beside the attention branch (both read the layer input)
+    std::vector<hipEvent_t> ev_fork, ev_join;
     pi_workspace * ws = nullptr;
     float theta_scale = 0.0f;
 

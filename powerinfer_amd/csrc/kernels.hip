@@ -998,7 +998,7 @@ constexpr int kPfChunk = 8;                       // active neurons per round tr
 
 __device__ __forceinline__ int select_nth_bit(uint32_t bits, int n);
 
-template <int CPW, int RCH, bool GATE>      // cols == 8 waves * CPW chunks * 512; r == RCH * 512
+template <int CPW, int RCH, bool GATE, int G>      // cols == 8 waves * CPW chunks * 512; r == RCH * 512; G groups of 32 neurons
 __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
                                                                    const __half * __restrict__ Wup, const __half * __restrict__ Wgate,
                                                                    const __half * __restrict__ Wdown,
@@ -1007,11 +1007,11 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
                                                                    float * __restrict__ partial) {
     constexpr int cols = kPfWaves * CPW * 512, r = RCH * 512;
     constexpr int CH = kPfChunk / CPW;                 // active neurons per round trip: 3*CPW*CH (2*CPW*CH) loads in flight per lane
-    __shared__ float  lg[32];
+    __shared__ float  lg[2][32];
     __shared__ double red[2][kPfWaves];
     __shared__ float  part[kPfWaves][CH][2];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int n0 = blockIdx.x * 32;
+    int n0 = blockIdx.x * 32 * G;
     const int cbase = wave * CPW * 512 + lane * 8;     // chunk c of this lane starts at column cbase + 512*c
 
     // ---- A: loads ------------------------------------------------------------------------------------------
@@ -1042,22 +1042,26 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
         }
     }
     // ---- A: logits (the CPU path rounds the hidden vector to fp16 before the dot, ggml.c:9703-9716) ------------
-    {
-        pi_u32x4 hr[RCH];
+    pi_u32x4 hr[RCH];
 #pragma unroll
-        for (int j = 0; j < RCH; ++j) {
-            __half2 hh[4] = {__floats2half2_rn(hv[j][0].x, hv[j][0].y), __floats2half2_rn(hv[j][0].z, hv[j][0].w),
-                             __floats2half2_rn(hv[j][1].x, hv[j][1].y), __floats2half2_rn(hv[j][1].z, hv[j][1].w)};
-            hr[j] = *reinterpret_cast<const pi_u32x4 *>(hh);
-        }
+    for (int j = 0; j < RCH; ++j) {
+        __half2 hh[4] = {__floats2half2_rn(hv[j][0].x, hv[j][0].y), __floats2half2_rn(hv[j][0].z, hv[j][0].w),
+                         __floats2half2_rn(hv[j][1].x, hv[j][1].y), __floats2half2_rn(hv[j][1].z, hv[j][1].w)};
+        hr[j] = *reinterpret_cast<const pi_u32x4 *>(hh);
+    }
 #pragma unroll
-        for (int i = 0; i < 4; ++i) {
-            float acc = 0.0f;
+    for (int i = 0; i < 4; ++i) {
+        float acc = 0.0f;
 #pragma unroll
-            for (int j = 0; j < RCH; ++j) acc = pi_dot8h(a[i][j], hr[j], acc);
-            acc = pi_wave_sum(acc);
-            if (lane == 0) lg[wave * 4 + i] = acc;
-        }
+        for (int j = 0; j < RCH; ++j) acc = pi_dot8h(a[i][j], hr[j], acc);
+        acc = pi_wave_sum(acc);
+        if (lane == 0) lg[0][wave * 4 + i] = acc;
+    }
+    if (G > 1) {       // the next group's predictor rows travel while this group's FFN rows are fetched and used
+#pragma unroll
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < RCH; ++j) a[i][j] = pi_ld_stream(W2 + (size_t)(n0 + 32 + wave * 4 + i) * r + (j * PI_WAVE + lane) * 8);
     }
     // ---- A: norm statistics across the 8 slices ---------------------------------------------------------------
     float mean = 0.0f, scale = 1.0f;
@@ -1119,21 +1123,40 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
                          __floats2half2_rn(xs[c][4], xs[c][5]), __floats2half2_rn(xs[c][6], xs[c][7])};
         xr[c] = *reinterpret_cast<const pi_u32x4 *>(hh);
     }
-    // ---- activity word (identical in every wave; lg is complete after the barrier above) -----------------------
-    const float my_logit = lg[lane & 31];
-    const bool my_act = !(my_logit < thr);
-    const uint32_t mask = (uint32_t)__ballot(my_act);
-    if (wave == 0) {
-        if (lane < 32) { if (logits) logits[n0 + lane] = my_logit; if (h_dense && !my_act) h_dense[n0 + lane] = 0.0f; }
-        if (lane == 0) words[blockIdx.x] = mask;
-    }
-    // ---- B + C ---------------------------------------------------------------------------------------------
-    const int n = __popc(mask);
     float acc[CPW][8];
 #pragma unroll
     for (int c = 0; c < CPW; ++c)
 #pragma unroll
         for (int k = 0; k < 8; ++k) acc[c][k] = 0.0f;
+#pragma unroll 1
+    for (int g = 0; g < G; ++g, n0 += 32) {
+    if (g > 0) {
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float lacc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < RCH; ++j) lacc = pi_dot8h(a[i][j], hr[j], lacc);
+            lacc = pi_wave_sum(lacc);
+            if (lane == 0) lg[g & 1][wave * 4 + i] = lacc;
+        }
+        if (g + 1 < G) {
+#pragma unroll
+            for (int i = 0; i < 4; ++i)
+#pragma unroll
+                for (int j = 0; j < RCH; ++j) a[i][j] = pi_ld_stream(W2 + (size_t)(n0 + 32 + wave * 4 + i) * r + (j * PI_WAVE + lane) * 8);
+        }
+        __syncthreads();
+    }
+    // ---- activity word (identical in every wave; lg[g & 1] is complete after the barrier above) ----------------
+    const float my_logit = lg[g & 1][lane & 31];
+    const bool my_act = !(my_logit < thr);
+    const uint32_t mask = (uint32_t)__ballot(my_act);
+    if (wave == 0) {
+        if (lane < 32) { if (logits) logits[n0 + lane] = my_logit; if (h_dense && !my_act) h_dense[n0 + lane] = 0.0f; }
+        if (lane == 0) words[blockIdx.x * G + g] = mask;
+    }
+    // ---- B + C ---------------------------------------------------------------------------------------------
+    const int n = __popc(mask);
     for (int c0 = 0; c0 < n; c0 += CH) {
         const int nn = n - c0 < CH ? n - c0 : CH;
         int rows[CH];
@@ -1183,6 +1206,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
         }
         if (c0 + CH < n) __syncthreads();                         // part[] is reused by the next chunk
     }
+    }   // groups: the barrier behind the next group's logits also orders this group's last reads of part[] and lg[]
 #pragma unroll
     for (int c = 0; c < CPW; ++c) {
         float4 * po = reinterpret_cast<float4 *>(partial + (size_t)blockIdx.x * cols + cbase + c * 512);
@@ -2869,31 +2893,62 @@ int pi_k_sparse_axpy_dense(const void * down_t_f16, int cols, int ff, const floa
 
 int pi_k_sparse_ffn_supported(int ff, int r, int cols) { return (cols == 4096 || cols == 8192) && (r == 1024 || r == 512) && ff > 0 && ff % 32 == 0; }
 
-int pi_k_sparse_ffn(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
-                    const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x, const pi_norm * norm,
-                    int epilogue, const float * add1, const float * add2, float * out,
-                    float * logits, float * h_dense, int32_t * n_active, pi_workspace * ws, pi_stream_t stream) {
-    if (!fc2_f16 || !hidden || !up_f16 || !down_t_f16 || !x || !out || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: null pointer");
+// Groups of 32 neurons per workgroup of the fused sparse FFN.  Wide rows: a workgroup takes four groups in turn (the next
+// group's predictor rows travel during the current group's FFN rows) and stores one partial vector for all of them, which
+// quarters the partial-sum traffic (it grows with cols; at 32768 x 8192 it was 67 MB of 220 MB per layer).
+// PI_PF_GROUPS=1|2|4 overrides the choice for wide rows (measurement aid).
+static int pf_groups(int ff, int cols) {
+    static const int forced = [] { const char * e = getenv("PI_PF_GROUPS"); return e ? atoi(e) : 0; }();
+    if (cols != 8192) return 1;                    // at 4096 columns one group per workgroup measured fastest
+    if ((forced == 1 || forced == 2 || forced == 4) && ff % (32 * forced) == 0) return forced;
+    return (ff % 128 == 0 && ff / 128 >= 256) ? 4 : 1;
+}
+
+int pi_k_sparse_ffn_partials(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                             const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x, const pi_norm * norm,
+                             float * logits, float * h_dense, pi_workspace * ws, pi_stream_t stream) {
+    if (!fc2_f16 || !hidden || !up_f16 || !down_t_f16 || !x || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: null pointer");
     if (!pi_k_sparse_ffn_supported(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn: shape outside the fused kernel (cols 4096 or 8192, r 512 or 1024, ff % 32 == 0)");
     if (ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: shape exceeds the workspace");
-    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
-        return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: bad epilogue arguments");
     const NormArgs na = to_norm(norm);
     if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: vectors must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
     const __half * w2 = (const __half *)fc2_f16; const __half * u = (const __half *)up_f16; const __half * g = (const __half *)gate_f16;
     const __half * dn = (const __half *)down_t_f16;
-    const dim3 grid(ff / 32), block(kPfBlock);
-#define PI_PF_LAUNCH(CPW, RCH, GATE) hipLaunchKernelGGL((pred_ffn_f16_kernel<CPW, RCH, GATE>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial)
+    const int G = pf_groups(ff, cols);
+    const dim3 grid(ff / (32 * G)), block(kPfBlock);
+#define PI_PF_LAUNCH(CPW, RCH, GATE, GG) hipLaunchKernelGGL((pred_ffn_f16_kernel<CPW, RCH, GATE, GG>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial)
+#define PI_PF_WIDE(RCH, GATE) do { if (G == 4) PI_PF_LAUNCH(2, RCH, GATE, 4); else if (G == 2) PI_PF_LAUNCH(2, RCH, GATE, 2); else PI_PF_LAUNCH(2, RCH, GATE, 1); } while (0)
     const int cpw = cols / 4096, rch = r / 512;
-    if (cpw == 1 && rch == 2) { if (g) PI_PF_LAUNCH(1, 2, true); else PI_PF_LAUNCH(1, 2, false); }
-    else if (cpw == 1)        { if (g) PI_PF_LAUNCH(1, 1, true); else PI_PF_LAUNCH(1, 1, false); }
-    else if (rch == 2)        { if (g) PI_PF_LAUNCH(2, 2, true); else PI_PF_LAUNCH(2, 2, false); }
-    else                      { if (g) PI_PF_LAUNCH(2, 1, true); else PI_PF_LAUNCH(2, 1, false); }
+    if (cpw == 1 && rch == 2) { if (g) PI_PF_LAUNCH(1, 2, true, 1); else PI_PF_LAUNCH(1, 2, false, 1); }
+    else if (cpw == 1)        { if (g) PI_PF_LAUNCH(1, 1, true, 1); else PI_PF_LAUNCH(1, 1, false, 1); }
+    else if (rch == 2)        { if (g) PI_PF_WIDE(2, true); else PI_PF_WIDE(2, false); }
+    else                      { if (g) PI_PF_WIDE(1, true); else PI_PF_WIDE(1, false); }
+#undef PI_PF_WIDE
 #undef PI_PF_LAUNCH
-    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, st, ws->ffn_partial, ff / 32, cols, ws->words, ff / 32, n_active,
+    return pi::check_launch("pi_k_sparse_ffn_partials");
+}
+
+int pi_k_sparse_ffn_reduce(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out, int32_t * n_active,
+                           pi_workspace * ws, pi_stream_t stream) {
+    if (!out || !ws || ff <= 0 || ff % 32 || ff > ws->max_ff || cols <= 0 || cols % 64 || cols > ws->max_d) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_reduce: bad arguments");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_reduce: bad epilogue arguments");
+    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, ff / (32 * pf_groups(ff, cols)), cols, ws->words, ff / 32, n_active,
                        epilogue, add1, add2, out);
-    return pi::check_launch("pi_k_sparse_ffn");
+    return pi::check_launch("pi_k_sparse_ffn_reduce");
+}
+
+int pi_k_sparse_ffn(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                    const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x, const pi_norm * norm,
+                    int epilogue, const float * add1, const float * add2, float * out,
+                    float * logits, float * h_dense, int32_t * n_active, pi_workspace * ws, pi_stream_t stream) {
+    if (!out) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: null pointer");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: bad epilogue arguments");
+    const int rc = pi_k_sparse_ffn_partials(fc2_f16, ff, r, hidden, threshold, up_f16, gate_f16, down_t_f16, cols, x, norm, logits, h_dense, ws, stream);
+    if (rc != PI_OK) return rc;
+    return pi_k_sparse_ffn_reduce(ff, cols, epilogue, add1, add2, out, n_active, ws, stream);
 }
 
 int pi_k_norm_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, void * out_plain_f16, pi_stream_t stream) {

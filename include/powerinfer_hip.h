@@ -164,6 +164,24 @@ PI_API int pi_k_sparse_axpy(int wtype, const void * down_t, int cols, int n_rows
  * logits (fp32 [ff]), h_dense (fp32 [ff], every entry written) and n_active (predictor's active count) are
  * optional outputs for inspection.  Shapes: see pi_k_sparse_ffn_supported.
  */
+/* Q4_0 weights, cols == 4096: predictor fc2 + mask + up/gate of the GPU-resident neurons in one launch, then the down
+ * projection as per-workgroup partial vectors plus one reduction.  Replaces the GPU nodes of llm_build_ffn_sparse for Q4_0
+ * (mul_mat_vec_sparse_q ggml-cuda.cu:7232, dequantize_axpy :7593) and follows the CPU arithmetic (Q8_0 input,
+ * ggml-quants.c:2512-2650; Q8_0 h over 32-neuron blocks, ggml.c:14465-14618, ggml-quants.c:2426-2509).
+ * hot_words[ff/32]: bit j of word g set iff neuron 32g+j is GPU-resident; hot_prefix[g]: GPU-resident neurons before group g
+ * (= row of the compact matrices, llama.cpp:2820-2967); both NULL: every neuron resident, row = neuron.
+ * h_dense[ff] gets h for active resident neurons and 0 elsewhere.  logits, h_dense and xq8_out (cols/32 blocks of
+ * {fp16 d, int8 qs[32]}: the Q8_0 form of the normalised input, optional) may be pinned host memory, and so may `h` of the
+ * partials call (the vector after the host share filled in its neurons) and add1/add2 of the reduction. */
+PI_API int pi_k_pred_upgate_q4_supported(int ff, int r, int cols);
+PI_API int pi_k_pred_upgate_q4(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                               const void * up_q4, const void * gate_q4, int cols, const float * x, const pi_norm * norm,
+                               const uint32_t * hot_words, const int32_t * hot_prefix,
+                               float * logits, float * h_dense, void * xq8_out, pi_workspace * ws, pi_stream_t stream);
+PI_API int pi_k_axpy_q4_partials(const void * down_t_q4, int cols, int ff, const float * h,
+                                 const uint32_t * hot_words, const int32_t * hot_prefix, pi_workspace * ws, pi_stream_t stream);
+PI_API int pi_k_axpy_q4_reduce(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out,
+                               int32_t * n_active, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_sparse_ffn_supported(int ff, int r, int cols);
 /* the two launches of pi_k_sparse_ffn on their own, for callers that overlap the block with an independent branch (Falcon's
  * attention reads the same layer input): _partials may run on another stream, _reduce needs it and the residual operands done */

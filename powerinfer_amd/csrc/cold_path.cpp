@@ -10,10 +10,12 @@
 #include "runtime.hpp"
 
 #include <math.h>
+#include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
 
 #include <atomic>
+#include <chrono>
 #include <condition_variable>
 #include <functional>
 #include <mutex>
@@ -81,7 +83,26 @@ float dot_f16(int n, const uint16_t * w, const uint16_t * x) {
 #endif
 }
 
+// Q4_0 row . Q8_0 activations (ggml_vec_dot_q4_0_q8_0, ggml-quants.c:2512-2650): exact integer dot per block of 32, scaled by
+// d4*d8 and accumulated in fp32 (eight lanes with AVX2, each holding four of a block's products, summed at the end)
 float dot_q4_q8(int n, const BlockQ4 * w, const BlockQ8 * x) {
+#ifdef PI_COLD_SIMD
+    __m256 acc = _mm256_setzero_ps();
+    const __m256i lowmask = _mm256_set1_epi8(0x0F), eight = _mm256_set1_epi8(8), ones = _mm256_set1_epi16(1);
+    for (int b = 0; b < n / 32; ++b) {
+        const __m128i q = _mm_loadu_si128((const __m128i *)w[b].qs);
+        __m256i bx = _mm256_and_si256(_mm256_set_m128i(_mm_srli_epi16(q, 4), q), lowmask);     // elements 0..15 | 16..31
+        bx = _mm256_sub_epi8(bx, eight);
+        const __m256i by = _mm256_loadu_si256((const __m256i *)x[b].qs);
+        const __m256i prod = _mm256_maddubs_epi16(_mm256_sign_epi8(bx, bx), _mm256_sign_epi8(by, bx));   // |w| * (x * sign(w)), pairs summed
+        const __m256 pf = _mm256_cvtepi32_ps(_mm256_madd_epi16(prod, ones));
+        acc = _mm256_fmadd_ps(_mm256_set1_ps(h2f(w[b].d) * h2f(x[b].d)), pf, acc);
+    }
+    __m128 r = _mm_add_ps(_mm256_extractf128_ps(acc, 1), _mm256_castps256_ps128(acc));
+    r = _mm_add_ps(r, _mm_movehl_ps(r, r));
+    r = _mm_add_ss(r, _mm_movehdup_ps(r));
+    return _mm_cvtss_f32(r);
+#else
     float acc = 0.f;
     for (int b = 0; b < n / 32; ++b) {
         int sum = 0;
@@ -92,6 +113,34 @@ float dot_q4_q8(int n, const BlockQ4 * w, const BlockQ8 * x) {
         acc = fmaf(h2f(w[b].d) * h2f(x[b].d), (float)sum, acc);
     }
     return acc;
+#endif
+}
+
+// out[32 b .. 32 b + 32) += float((q4 - 8) * a) * (d4 * sc) for the blocks [b0, b1) of one Q4_0 row
+// (ggml_axpy_q4_0_q8_0, ggml-quants.c:2426-2509: integer product, one fp32 multiply, one fp32 add)
+void axpy_q4_blocks(const BlockQ4 * row, int b0, int b1, int a, float sc, float * out) {
+    for (int b = b0; b < b1; ++b) {
+        const float dd = h2f(row[b].d) * sc;
+        float * o = out + b * 32;
+#ifdef PI_COLD_SIMD
+        const __m128i q = _mm_loadu_si128((const __m128i *)row[b].qs);
+        const __m128i lowmask = _mm_set1_epi8(0x0F), eight = _mm_set1_epi8(8);
+        const __m128i lo = _mm_sub_epi8(_mm_and_si128(q, lowmask), eight), hi = _mm_sub_epi8(_mm_and_si128(_mm_srli_epi16(q, 4), lowmask), eight);
+        const __m256i av = _mm256_set1_epi16((short)a);
+        const __m256 dv = _mm256_set1_ps(dd);
+        const __m256i plo = _mm256_mullo_epi16(_mm256_cvtepi8_epi16(lo), av), phi = _mm256_mullo_epi16(_mm256_cvtepi8_epi16(hi), av);
+        const __m256i parts[4] = {_mm256_cvtepi16_epi32(_mm256_castsi256_si128(plo)), _mm256_cvtepi16_epi32(_mm256_extracti128_si256(plo, 1)),
+                                  _mm256_cvtepi16_epi32(_mm256_castsi256_si128(phi)), _mm256_cvtepi16_epi32(_mm256_extracti128_si256(phi, 1))};
+        for (int k = 0; k < 4; ++k)
+            _mm256_storeu_ps(o + 8 * k, _mm256_add_ps(_mm256_loadu_ps(o + 8 * k), _mm256_mul_ps(_mm256_cvtepi32_ps(parts[k]), dv)));
+#else
+        for (int q = 0; q < 16; ++q) {
+            const float p0 = (float)(((int)(row[b].qs[q] & 0x0F) - 8) * a) * dd, p1 = (float)(((int)(row[b].qs[q] >> 4) - 8) * a) * dd;
+            o[q]      = o[q] + p0;
+            o[q + 16] = o[q + 16] + p1;
+        }
+#endif
+    }
 }
 
 // x86 quantize_row_q8_0 semantics (ggml-quants.c:702-760): d = amax/127 stored as fp16, q = rint(x * 127/amax)
@@ -105,50 +154,67 @@ void quantize_q8(const float * x, BlockQ8 * y, int n) {
     }
 }
 
+// Fork/join over persistent host threads.  A decode step forks twice per layer with a few microseconds of work each,
+// so idle workers spin on the generation counter for a short while (a condition-variable wake-up costs more than the
+// work) and only then go to sleep; the caller takes share 0 and spins for the join.
 class Pool {
   public:
     explicit Pool(int n) : n_(n) {
         for (int i = 1; i < n_; ++i) threads_.emplace_back([this, i] { loop(i); });
     }
     ~Pool() {
-        { std::lock_guard<std::mutex> g(mu_); stop_ = true; ++gen_; }
+        stop_.store(true);
+        gen_.fetch_add(1);
+        { std::lock_guard<std::mutex> g(mu_); }
         cv_.notify_all();
         for (auto & t : threads_) t.join();
     }
     int size() const { return n_; }
     void run(const std::function<void(int, int)> & fn) {
-        { std::lock_guard<std::mutex> g(mu_); fn_ = &fn; pending_ = n_ - 1; ++gen_; }
-        cv_.notify_all();
+        fn_ = &fn;
+        pending_.store(n_ - 1, std::memory_order_relaxed);
+        gen_.fetch_add(1);                                    // publishes fn_ and pending_
+        if (sleepers_.load() > 0) { { std::lock_guard<std::mutex> g(mu_); } cv_.notify_all(); }
         fn(0, n_);
-        std::unique_lock<std::mutex> g(mu_);
-        done_.wait(g, [this] { return pending_ == 0; });
-        fn_ = nullptr;
+        while (pending_.load(std::memory_order_acquire) != 0) cpu_relax();
     }
 
   private:
+    static void cpu_relax() {
+#ifdef PI_COLD_SIMD
+        _mm_pause();
+#else
+        std::this_thread::yield();
+#endif
+    }
     void loop(int id) {
         uint64_t seen = 0;
         for (;;) {
-            const std::function<void(int, int)> * fn;
-            {
-                std::unique_lock<std::mutex> g(mu_);
-                cv_.wait(g, [&] { return gen_ != seen; });
-                seen = gen_;
-                if (stop_) return;
-                fn = fn_;
+            auto t0 = std::chrono::steady_clock::now();
+            for (int it = 0; gen_.load(std::memory_order_acquire) == seen; ++it) {
+                cpu_relax();
+                if ((it & 255) == 255 && std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(kSpinUs)) {
+                    std::unique_lock<std::mutex> g(mu_);
+                    sleepers_.fetch_add(1);
+                    cv_.wait(g, [&] { return gen_.load() != seen; });
+                    sleepers_.fetch_sub(1);
+                }
             }
-            (*fn)(id, n_);
-            { std::lock_guard<std::mutex> g(mu_); if (--pending_ == 0) done_.notify_one(); }
+            seen = gen_.load(std::memory_order_acquire);
+            if (stop_.load()) return;
+            (*fn_)(id, n_);
+            pending_.fetch_sub(1, std::memory_order_release);
         }
     }
+    static constexpr int kSpinUs = 500;
     int n_;
     std::vector<std::thread> threads_;
     std::mutex mu_;
-    std::condition_variable cv_, done_;
+    std::condition_variable cv_;
     const std::function<void(int, int)> * fn_ = nullptr;
-    int pending_ = 0;
-    uint64_t gen_ = 0;
-    bool stop_ = false;
+    std::atomic<int> pending_{0}, sleepers_{0};
+    std::atomic<uint64_t> gen_{0};
+    std::atomic<bool> stop_{false};
 };
 
 }  // namespace
@@ -162,7 +228,17 @@ struct ColdPath {
     Pool * pool = nullptr;
     std::vector<ColdLayer> layers;
     // pinned staging
-    float * logits = nullptr, * src = nullptr, * h_gpu = nullptr, * h_full = nullptr, * out = nullptr;
+    float * logits = nullptr, * src = nullptr, * h_gpu = nullptr;      // device -> host, consumed before the layer call returns
+    float * h_full[2] = {nullptr, nullptr}, * out[2] = {nullptr, nullptr};   // host -> device, read by the GPU after the call returned: two sets, used in turn
+    int flip = 0;
+    hipEvent_t ev_in = nullptr, ev_h = nullptr;
+    std::vector<float> hval;                    // h of the active cold neurons, in the order of act
+    // PI_COLD_TRACE=1: mean host time per phase of a layer call, printed when the model is freed
+    bool trace = false;
+    double t_phase[6] = {0, 0, 0, 0, 0, 0};
+    long long n_calls = 0, n_cold_active = 0;
+    std::chrono::steady_clock::time_point t_last_return;
+    double t_between = 0;
     std::vector<float> xn;
     std::vector<uint16_t> x16;
     std::vector<BlockQ8> xq8, hq8;
@@ -179,6 +255,7 @@ ColdPath * cold_create(pi_model * m) {
     if (const char * e = getenv("PI_COLD_THREADS")) { const int v = atoi(e); if (v > 0) nt = v; }
     if (nt < 1) nt = 1;
     c->pool = new Pool(nt);
+    if (const char * e = getenv("PI_COLD_TRACE")) c->trace = e[0] == '1';
     c->layers.resize(hp.n_layer);
     const bool falcon = hp.arch == PI_ARCH_FALCON;
     for (int il = 0; il < hp.n_layer; ++il) {
@@ -195,18 +272,50 @@ ColdPath * cold_create(pi_model * m) {
         for (int j = 0; j < c->ff; ++j) if (gid[j] != 1) cl.cold_rows.push_back(j);
     }
     auto pin = [](size_t n) { void * p = nullptr; return hipHostMalloc(&p, n * sizeof(float), hipHostMallocDefault) == hipSuccess ? (float *)p : nullptr; };
-    c->logits = pin(c->ff); c->src = pin(c->d); c->h_gpu = pin(c->ff); c->h_full = pin(c->ff); c->out = pin(c->d);
-    if (!c->logits || !c->src || !c->h_gpu || !c->h_full || !c->out) { set_error("cold path: pinned host allocation failed"); cold_destroy(c); return nullptr; }
+    c->logits = pin(c->ff); c->src = pin(c->d); c->h_gpu = pin(c->ff);
+    for (int i = 0; i < 2; ++i) { c->h_full[i] = pin(c->ff); c->out[i] = pin(c->d); }
+    if (!c->logits || !c->src || !c->h_gpu || !c->h_full[0] || !c->h_full[1] || !c->out[0] || !c->out[1]) { set_error("cold path: pinned host allocation failed"); cold_destroy(c); return nullptr; }
+    if (hipEventCreateWithFlags(&c->ev_in, hipEventDisableTiming) != hipSuccess || hipEventCreateWithFlags(&c->ev_h, hipEventDisableTiming) != hipSuccess) {
+        set_error("cold path: event creation failed"); cold_destroy(c); return nullptr;
+    }
     c->xn.resize(c->d); c->x16.resize(c->d); c->xq8.resize(c->d / 32 + 1); c->hq8.resize(c->ff / 32 + 1);
-    c->act.reserve(c->ff);
+    c->act.reserve(c->ff); c->hval.resize(c->ff);
     return c;
 }
 
 void cold_destroy(ColdPath * c) {
     if (!c) return;
+    if (c->trace && c->n_calls) {
+        const double n = (double)c->n_calls;
+        fprintf(stderr, "cold path, mean us per layer call over %lld calls: between calls %.1f | wait inputs %.1f | norm+list %.1f | up/gate %.1f | wait h + upload %.1f | down %.1f | merge launch %.1f | active cold neurons %.1f\n",
+                c->n_calls, c->t_between / n, c->t_phase[0] / n, c->t_phase[1] / n, c->t_phase[2] / n, c->t_phase[3] / n, c->t_phase[4] / n, c->t_phase[5] / n, (double)c->n_cold_active / n);
+    }
     delete c->pool;
-    for (float * p : {c->logits, c->src, c->h_gpu, c->h_full, c->out}) if (p) (void)hipHostFree(p);
+    for (float * p : {c->logits, c->src, c->h_gpu, c->h_full[0], c->h_full[1], c->out[0], c->out[1]}) if (p) (void)hipHostFree(p);
+    if (c->ev_in) (void)hipEventDestroy(c->ev_in);
+    if (c->ev_h) (void)hipEventDestroy(c->ev_h);
     delete c;
+}
+
+namespace {
+// The host waits for the device twice per layer and the waits are short: poll the event before falling back to a blocking wait.
+hipError_t wait_event(hipEvent_t ev) {
+    const auto t0 = std::chrono::steady_clock::now();
+    for (int it = 0;; ++it) {
+        const hipError_t e = hipEventQuery(ev);
+        if (e != hipErrorNotReady) return e;
+        if ((it & 63) == 63 && std::chrono::steady_clock::now() - t0 > std::chrono::milliseconds(2)) return hipEventSynchronize(ev);
+    }
+}
+}  // namespace
+
+int cold_stage_inputs(ColdPath * c, int il, pi_model * m, hipStream_t st) {
+    (void)il;
+    const float * ffn_src = m->hp.arch == PI_ARCH_FALCON ? m->x : m->ffn_inp;
+    PI_HIP_TRY(hipMemcpyAsync(c->logits, m->pred_logits, sizeof(float) * c->ff, hipMemcpyDeviceToHost, st));
+    PI_HIP_TRY(hipMemcpyAsync(c->src, ffn_src, sizeof(float) * c->d, hipMemcpyDeviceToHost, st));
+    PI_HIP_TRY(hipEventRecord(c->ev_in, st));
+    return PI_OK;
 }
 
 int cold_layer_merge(ColdPath * c, int il, pi_model * m, hipStream_t st) {
@@ -220,19 +329,25 @@ int cold_layer_merge(ColdPath * c, int il, pi_model * m, hipStream_t st) {
     const int n_bucket = (int)bucket.ne0;
     const int32_t * bk = (const int32_t *)bucket.dev;
     int32_t * n_act = m->n_active + il;
-    const float * ffn_src = falcon ? m->x : m->ffn_inp;
     const float thr = hp.sparse_threshold;
+    const int p = (c->flip ^= 1);
+    auto now = [] { return std::chrono::steady_clock::now(); };
+    auto us = [](std::chrono::steady_clock::time_point a, std::chrono::steady_clock::time_point b) { return std::chrono::duration<double, std::micro>(b - a).count(); };
+    std::chrono::steady_clock::time_point tp = now();
+    if (c->trace && c->n_calls) c->t_between += us(c->t_last_return, tp);
+    auto lap = [&](int i) { if (c->trace) { const auto t = now(); c->t_phase[i] += us(tp, t); tp = t; } };
 
-    // 1. what the host needs from the device: predictor logits and the FFN block's input vector
-    PI_HIP_TRY(hipMemcpyAsync(c->logits, m->pred_logits, sizeof(float) * ff, hipMemcpyDeviceToHost, st));
-    PI_HIP_TRY(hipMemcpyAsync(c->src, ffn_src, sizeof(float) * d, hipMemcpyDeviceToHost, st));
-    if (q4) PI_HIP_TRY(hipMemcpyAsync(c->h_gpu, m->h_dense, sizeof(float) * ff, hipMemcpyDeviceToHost, st));   // after the GPU share's up/gate
-    if (!q4) {
-        // F16: the GPU share needs nothing from the host; queue its down projection now so it overlaps the CPU work
+    // 1. the GPU share goes on while the host works: Q4_0 sends its h back (the Q8_0 blocks of h mix hot and cold neurons),
+    //    F16 needs nothing from the host and queues its down projection right away
+    if (q4) {
+        PI_HIP_TRY(hipMemcpyAsync(c->h_gpu, m->h_dense, sizeof(float) * ff, hipMemcpyDeviceToHost, st));
+        PI_HIP_TRY(hipEventRecord(c->ev_h, st));
+    } else {
         const int rc = pi_k_sparse_axpy(down.type, down.dev, d, n_bucket, m->h_c, nullptr, bk, m->list, n_act, PI_EPI_NONE, nullptr, nullptr, m->x2, m->ws, st);
         if (rc != PI_OK) return rc;
     }
-    PI_HIP_TRY(hipStreamSynchronize(st));
+    PI_HIP_TRY(wait_event(c->ev_in));           // predictor logits and the FFN input are on the host
+    lap(0);
 
     // 2. norm of the FFN input (llm_build_norm, llama.cpp:4420-4450), then round to the weights' dot type
     {
@@ -260,9 +375,8 @@ int cold_layer_merge(ColdPath * c, int il, pi_model * m, hipStream_t st) {
     c->act.clear();
     for (int j : cl.cold_rows) if (!(c->logits[j] < thr)) c->act.push_back(j);
     const int na = (int)c->act.size();
-    float * hfull = c->h_full;
-    if (q4) memcpy(hfull, c->h_gpu, sizeof(float) * ff);        // GPU share's h (zero elsewhere): the supports are disjoint
-    else memset(hfull, 0, sizeof(float) * ff);
+    lap(1);
+    float * hval = c->hval.data();
     const size_t rb = q4 ? (size_t)(d / 32) * 18 : (size_t)d * 2;
     const unsigned char * wu = (const unsigned char *)up.host;
     const unsigned char * wg = falcon ? nullptr : (const unsigned char *)gate.host;
@@ -277,21 +391,27 @@ int cold_layer_merge(ColdPath * c, int il, pi_model * m, hipStream_t st) {
                 u = dot_f16(d, (const uint16_t *)(wu + rb * j), c->x16.data());
                 if (wg) g = dot_f16(d, (const uint16_t *)(wg + rb * j), c->x16.data());
             }
-            hfull[j] = wg ? (g > 0.f ? g : 0.f) * u : (u > 0.f ? u : 0.f);
+            hval[k] = wg ? (g > 0.f ? g : 0.f) * u : (u > 0.f ? u : 0.f);
         }
     });
 
+    lap(2);
     // 4. Q4_0: the Q8_0 scales of h span 32 neighbouring neurons, hot and cold alike, so both sides need the merged vector
+    float * hfull = c->h_full[p];
     if (q4) {
+        PI_HIP_TRY(wait_event(c->ev_h));
+        memcpy(hfull, c->h_gpu, sizeof(float) * ff);        // GPU share's h (zero elsewhere): the supports are disjoint
+        for (int k = 0; k < na; ++k) hfull[c->act[k]] = hval[k];
         PI_HIP_TRY(hipMemcpyAsync(m->h_dense, hfull, sizeof(float) * ff, hipMemcpyHostToDevice, st));
         const int rc = pi_k_sparse_axpy(down.type, down.dev, d, n_bucket, m->h_c, m->h_dense, bk, m->list, n_act, PI_EPI_NONE, nullptr, nullptr, m->x2, m->ws, st);
         if (rc != PI_OK) return rc;
         quantize_q8(hfull, c->hq8.data(), ff);
     }
 
+    lap(3);
     // 5. cold share of the down projection, threads split the output columns (blocks of 32 for Q4_0)
     const unsigned char * wd = (const unsigned char *)down.host;
-    float * out = c->out;
+    float * out = c->out[p];
     const int unit = 32, n_units = d / unit;
     c->pool->run([&](int t, int nt) {
         const int u0 = (int)((long long)n_units * t / nt), u1 = (int)((long long)n_units * (t + 1) / nt);
@@ -304,17 +424,9 @@ int cold_layer_merge(ColdPath * c, int il, pi_model * m, hipStream_t st) {
                 const int a = hb.qs[j % 32];
                 if (a == 0) continue;
                 const float sc = h2f(hb.d);
-                const BlockQ4 * row = (const BlockQ4 *)(wd + rb * j);
-                for (int b = u0; b < u1; ++b) {
-                    const float dd = h2f(row[b].d) * sc;
-                    float * o = out + b * 32;
-                    for (int q = 0; q < 16; ++q) {
-                        o[q]      = o[q]      + (float)(((int)(row[b].qs[q] & 0x0F) - 8) * a) * dd;
-                        o[q + 16] = o[q + 16] + (float)(((int)(row[b].qs[q] >> 4) - 8) * a) * dd;
-                    }
-                }
+                axpy_q4_blocks((const BlockQ4 *)(wd + rb * j), u0, u1, a, sc, out);
             } else {
-                const uint16_t hb = f2h(hfull[j]);
+                const uint16_t hb = f2h(hval[k]);
                 if (hb == 0) continue;
                 const float a = h2f(hb);
                 const uint16_t * row = (const uint16_t *)(wd + rb * j);
@@ -329,18 +441,15 @@ int cold_layer_merge(ColdPath * c, int il, pi_model * m, hipStream_t st) {
         }
     });
 
-    // 6. merge: (cold + hot) + residual(s), in the reference's order (ggml_add(cpu, gpu), then the residual adds)
-    PI_HIP_TRY(hipMemcpyAsync(m->cold_out, out, sizeof(float) * d, hipMemcpyHostToDevice, st));
-    int rc = add_vec(m->cold_out, m->x2, d, st);                 // cold_out = cold + hot
-    if (rc != PI_OK) return rc;
-    PI_HIP_TRY(hipMemcpyAsync(m->x2, m->cold_out, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
-    if (m->capture) PI_HIP_TRY(hipMemcpyAsync(m->cap_ffn + (size_t)il * d, m->cold_out, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
-    rc = add_vec(m->x2, falcon ? m->attn_out : m->ffn_inp, d, st);
-    if (rc != PI_OK) return rc;
-    if (falcon) { rc = add_vec(m->x2, m->x, d, st); if (rc != PI_OK) return rc; }
-    // the pinned buffers are reused by the next layer: wait for the upload to be consumed
-    PI_HIP_TRY(hipStreamSynchronize(st));
-    return PI_OK;
+    // 6. merge: (cold + hot) + residual(s), in the reference's order (ggml_add(cpu, gpu), then the residual adds).  The kernel
+    //    reads the cold share straight from the pinned buffer; that buffer and h_full[p] are written again two layers on, after
+    //    the host has waited for an event recorded behind this layer's work, so no wait is needed here.
+    lap(4);
+    const int rc = merge_shares(m->x2, out, m->x2, falcon ? m->attn_out : m->ffn_inp, falcon ? m->x : nullptr,
+                                m->capture ? m->cap_ffn + (size_t)il * d : nullptr, d, st);
+    lap(5);
+    if (c->trace) { ++c->n_calls; c->n_cold_active += na; c->t_last_return = now(); }
+    return rc;
 }
 
 }  // namespace pi

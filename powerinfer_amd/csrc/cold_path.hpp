@@ -13,10 +13,14 @@ struct ColdPath;
 
 ColdPath * cold_create(pi_model * m);
 void       cold_destroy(ColdPath * c);
+// Runs right after the predictor of layer `il` has been queued on `st`: starts the copies the host share needs.
+int        cold_stage_inputs(ColdPath * c, int il, pi_model * m, hipStream_t st);
 // Runs after the GPU share's up/gate launch of layer `il` has been queued on `st`; leaves the merged layer
 // output (cold + hot + residuals) in m->x2.
 int        cold_layer_merge(ColdPath * c, int il, pi_model * m, hipStream_t st);
 
 int add_vec(float * y, const float * a, int n, hipStream_t st);
+// dst = ((cold + hot) + r1) [+ r2]; `cold` may be pinned host memory; `keep` (optional) receives cold + hot
+int merge_shares(float * dst, const float * cold, const float * hot, const float * r1, const float * r2, float * keep, int n, hipStream_t st);
 
 }  // namespace pi

@@ -192,6 +192,7 @@ int layer_forward(pi_model * m, int il, bool last_token) {
     PI_TRY(pi_k_predictor_fc2(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, bk, n_bucket, m->pred_logits,
                               fused ? nullptr : m->list, fused ? nullptr : n_act,
                               (q4 || layer_hybrid) ? m->h_dense : nullptr, m->ws, st));
+    if (layer_hybrid) PI_TRY(pi::cold_stage_inputs(m->cold, il, m, st));
 
     // sparse FFN, GPU share
     PI_TRY(pi_k_sparse_upgate(up.type, up.dev, falcon ? nullptr : gate.dev, d, ff, ffn_in, &fn, fused ? 1 : 0, m->list, n_act, bk, m->h_c,
@@ -245,8 +246,25 @@ int launch_advance(pi_model * m) {
 
 }  // namespace
 
-// entry used by the cold path to add its share into the layer output on the model's stream
+namespace {
+__global__ void merge_shares_kernel(float * __restrict__ dst, const float * cold, const float * hot, const float * __restrict__ r1,
+                                    const float * __restrict__ r2, float * __restrict__ keep, int n) {
+    const int i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i >= n) return;
+    float v = __fadd_rn(cold[i], hot[i]);
+    if (keep) keep[i] = v;
+    v = __fadd_rn(v, r1[i]);
+    if (r2) v = __fadd_rn(v, r2[i]);
+    dst[i] = v;
+}
+}  // namespace
+
+// entries used by the cold path to add its share into the layer output on the model's stream
 namespace pi {
+int merge_shares(float * dst, const float * cold, const float * hot, const float * r1, const float * r2, float * keep, int n, hipStream_t st) {
+    hipLaunchKernelGGL(merge_shares_kernel, dim3((n + 255) / 256), dim3(256), 0, st, dst, cold, hot, r1, r2, keep, n);
+    return check_launch("merge_shares");
+}
 int add_vec(float * y, const float * a, int n, hipStream_t st) {
     hipLaunchKernelGGL(add_vec_kernel, dim3((n + 255) / 256), dim3(256), 0, st, y, a, n);
     return check_launch("add_vec");

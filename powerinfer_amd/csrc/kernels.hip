@@ -1263,6 +1263,301 @@ __global__ __launch_bounds__(kPfBlock) void ffn_reduce_kernel(const float * __re
     if (blockIdx.x == 0 && n_active_out && tid == 0) { int t = 0; for (int w = 0; w < kPfWaves; ++w) t += sred[w]; *n_active_out = t; }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Q4_0 weights (cols == 4096): the predictor's second layer, the mask and the up/gate rows of the GPU-resident
+// neurons in one launch, in the layout of pred_ffn_f16_kernel: a workgroup of 8 waves owns 32 neurons, wave w owns
+// columns [512w, 512w + 512), lane l eight of them, i.e. a quarter of one 32-weight block (sub = l & 3: low nibbles of
+// qs[0..7], of qs[8..15], then the high nibbles of the same bytes).
+//   A  four fc2 rows per wave; the wave's slice of the FFN input is normalised and quantised to Q8_0 in registers:
+//      the four lanes of a block agree on amax by two quad permutations, d = amax/127 kept as fp16, q = rint(x*127/amax)
+//      (x86 path of quantize_row_q8_0, ggml-quants.c:702-760).  Workgroup 0 also stores the Q8_0 blocks ({fp16 d, 32 x int8},
+//      34 bytes each) for a host that computes the other neurons from the same quantised input.
+//   B  active neurons that live on the GPU (mask & hot word): row = hot_prefix + rank among the hot bits; every wave loads
+//      its 8 bytes + scale of up to 8 up and gate rows at once; exact int32 block sums (two more quad permutations)
+//      times d_w * d_x (vec_dot_q4_0_q8_0, ggml-quants.c:2512-2650), summed per wave and across waves through LDS.
+// h_dense gets h for those neurons and 0 for every other neuron of the group; the pointers handed in for logits,
+// h_dense and the Q8_0 blocks may be pinned host memory (a hybrid layer's host share reads them after the launch).
+// ---------------------------------------------------------------------------------------------------
+struct __attribute__((packed)) pi_q8_host_block { uint16_t d; int8_t qs[32]; };
+
+template <int RCH, bool GATE>
+__global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
+                                                                     const pi_block_q4_0 * __restrict__ Wup, const pi_block_q4_0 * __restrict__ Wgate,
+                                                                     const float * __restrict__ x, NormArgs na, float thr,
+                                                                     const uint32_t * __restrict__ hot_words, const int32_t * __restrict__ hot_prefix,
+                                                                     float * __restrict__ logits, uint32_t * __restrict__ words, uint32_t * __restrict__ words_hot,
+                                                                     float * __restrict__ h_dense, pi_q8_host_block * __restrict__ xq_out) {
+    constexpr int cols = 4096, r = RCH * 512, nb = cols / 32, CH = kPfChunk;
+    __shared__ float  lg[32];
+    __shared__ double red[2][kPfWaves];
+    __shared__ float  part[kPfWaves][CH][2];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n0 = blockIdx.x * 32;
+    const int cbase = wave * 512 + lane * 8;
+    const int blk = cbase >> 5, sub = lane & 3;
+
+    // ---- A: loads ------------------------------------------------------------------------------------------
+    pi_u32x4 a[4][RCH];
+#pragma unroll
+    for (int i = 0; i < 4; ++i)
+#pragma unroll
+        for (int j = 0; j < RCH; ++j) a[i][j] = pi_ld_stream(W2 + (size_t)(n0 + wave * 4 + i) * r + (j * PI_WAVE + lane) * 8);
+    float4 hv[RCH][2];
+#pragma unroll
+    for (int j = 0; j < RCH; ++j) {
+        hv[j][0] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8);
+        hv[j][1] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8 + 4);
+    }
+    const uint32_t hot = hot_words ? hot_words[blockIdx.x] : 0xFFFFFFFFu;
+    const int base_row = hot_prefix ? hot_prefix[blockIdx.x] : n0;
+    float xs[8], wn[8], bn[8];
+    {
+        const float4 x0 = *reinterpret_cast<const float4 *>(x + cbase), x1 = *reinterpret_cast<const float4 *>(x + cbase + 4);
+        xs[0] = x0.x; xs[1] = x0.y; xs[2] = x0.z; xs[3] = x0.w; xs[4] = x1.x; xs[5] = x1.y; xs[6] = x1.z; xs[7] = x1.w;
+        if (na.kind != 0 && na.w) {
+            const float4 w0 = *reinterpret_cast<const float4 *>(na.w + cbase), w1 = *reinterpret_cast<const float4 *>(na.w + cbase + 4);
+            wn[0] = w0.x; wn[1] = w0.y; wn[2] = w0.z; wn[3] = w0.w; wn[4] = w1.x; wn[5] = w1.y; wn[6] = w1.z; wn[7] = w1.w;
+        }
+        if (na.kind != 0 && na.b) {
+            const float4 b0 = *reinterpret_cast<const float4 *>(na.b + cbase), b1 = *reinterpret_cast<const float4 *>(na.b + cbase + 4);
+            bn[0] = b0.x; bn[1] = b0.y; bn[2] = b0.z; bn[3] = b0.w; bn[4] = b1.x; bn[5] = b1.y; bn[6] = b1.z; bn[7] = b1.w;
+        }
+    }
+    // ---- A: logits (the CPU path rounds the hidden vector to fp16 before the dot, ggml.c:9703-9716) ------------
+    {
+        pi_u32x4 hr[RCH];
+#pragma unroll
+        for (int j = 0; j < RCH; ++j) {
+            __half2 hh[4] = {__floats2half2_rn(hv[j][0].x, hv[j][0].y), __floats2half2_rn(hv[j][0].z, hv[j][0].w),
+                             __floats2half2_rn(hv[j][1].x, hv[j][1].y), __floats2half2_rn(hv[j][1].z, hv[j][1].w)};
+            hr[j] = *reinterpret_cast<const pi_u32x4 *>(hh);
+        }
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < RCH; ++j) acc = pi_dot8h(a[i][j], hr[j], acc);
+            acc = pi_wave_sum(acc);
+            if (lane == 0) lg[wave * 4 + i] = acc;
+        }
+    }
+    // ---- A: norm statistics across the 8 slices ---------------------------------------------------------------
+    float mean = 0.0f, scale = 1.0f;
+    if (na.kind == 1) {
+        double sq = 0.0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) sq += (double)__fmul_rn(xs[k], xs[k]);
+        sq = pi_wave_sum_f64(sq);
+        if (lane == 0) red[0][wave] = sq;
+        __syncthreads();
+        double t = 0.0;
+#pragma unroll
+        for (int w = 0; w < kPfWaves; ++w) t += red[0][w];
+        scale = 1.0f / sqrtf((float)(t / cols) + na.eps);
+    } else if (na.kind == 2) {
+        double sm = 0.0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) sm += (double)xs[k];
+        sm = pi_wave_sum_f64(sm);
+        if (lane == 0) red[0][wave] = sm;
+        __syncthreads();
+        double t = 0.0;
+#pragma unroll
+        for (int w = 0; w < kPfWaves; ++w) t += red[0][w];
+        mean = (float)(t / cols);
+        double sq = 0.0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { const float v = __fsub_rn(xs[k], mean); sq += (double)__fmul_rn(v, v); }
+        sq = pi_wave_sum_f64(sq);
+        if (lane == 0) red[1][wave] = sq;
+        __syncthreads();
+        double t2 = 0.0;
+#pragma unroll
+        for (int w = 0; w < kPfWaves; ++w) t2 += red[1][w];
+        scale = 1.0f / sqrtf((float)(t2 / cols) + na.eps);
+    } else {
+        __syncthreads();
+    }
+    // ---- A: Q8_0 of the normalised slice -----------------------------------------------------------------------
+    float amax = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        float v = xs[k];
+        if (na.kind != 0) {
+            v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
+            if (na.w) v = __fmul_rn(v, wn[k]);
+            if (na.b) v = __fadd_rn(v, bn[k]);
+        }
+        xs[k] = v;
+        amax = fmaxf(amax, fabsf(v));
+    }
+    amax = fmaxf(amax, pi_dpp_f32<PI_DPP_XOR1, 0xF>(amax));
+    amax = fmaxf(amax, pi_dpp_f32<PI_DPP_XOR2, 0xF>(amax));
+    const float dq = amax / 127.0f, idq = (amax != 0.0f) ? 127.0f / amax : 0.0f;
+    const float dx = pi_round_f16(dq);
+    int xq0 = 0, xq1 = 0, sx = 0;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) {
+        const int q = (int)rintf(__fmul_rn(xs[k], idq));
+        sx += q;
+        if (k < 4) xq0 |= (q & 0xFF) << (8 * k); else xq1 |= (q & 0xFF) << (8 * (k - 4));
+    }
+    if (blockIdx.x == 0 && xq_out) {
+        pi_q8_host_block * ob = xq_out + blk;
+        const int q2[2] = {xq0, xq1};
+        __builtin_memcpy(ob->qs + sub * 8, q2, 8);
+        if (sub == 0) { const uint16_t db = pi_f16_bits(dq); __builtin_memcpy(&ob->d, &db, 2); }
+    }
+    // ---- activity word (identical in every wave; lg is complete after the barrier above) -----------------------
+    const float my_logit = lg[lane & 31];
+    const bool my_act = !(my_logit < thr);
+    const uint32_t mask = (uint32_t)__ballot(my_act);
+    const uint32_t sel = mask & hot;
+    if (wave == 0) {
+        if (lane < 32) { if (logits) logits[n0 + lane] = my_logit; if (!((sel >> lane) & 1u)) h_dense[n0 + lane] = 0.0f; }
+        if (lane == 0) { words[blockIdx.x] = mask; if (words_hot) words_hot[blockIdx.x] = sel; }
+    }
+    // ---- B -------------------------------------------------------------------------------------------------
+    const int n = __popc(sel);
+    const int shift = (sub >> 1) * 4, qoff = (sub & 1) * 8;
+    for (int c0 = 0; c0 < n; c0 += CH) {
+        const int nn = n - c0 < CH ? n - c0 : CH;
+        int nrn[CH];
+        uint32_t qu[CH][2], qg[CH][2];
+        uint16_t du[CH], dg[CH];
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            if (j < nn) {
+                const int bit = select_nth_bit(sel, c0 + j);
+                nrn[j] = n0 + bit;
+                const size_t row = (size_t)(base_row + __popc(hot & ((1u << bit) - 1u)));
+                const pi_block_q4_0 * wu = Wup + row * nb + blk;
+                __builtin_memcpy(&du[j], &wu->d, 2);
+                __builtin_memcpy(qu[j], wu->qs + qoff, 8);
+                if (GATE) {
+                    const pi_block_q4_0 * wg = Wgate + row * nb + blk;
+                    __builtin_memcpy(&dg[j], &wg->d, 2);
+                    __builtin_memcpy(qg[j], wg->qs + qoff, 8);
+                }
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            if (j < nn) {
+                int su = __builtin_amdgcn_sdot4((int)((qu[j][0] >> shift) & 0x0F0F0F0Fu), xq0, 0, false);
+                su = __builtin_amdgcn_sdot4((int)((qu[j][1] >> shift) & 0x0F0F0F0Fu), xq1, su, false) - 8 * sx;
+                su += pi_dpp_i32<PI_DPP_XOR1, 0xF>(su);
+                su += pi_dpp_i32<PI_DPP_XOR2, 0xF>(su);
+                float pu = sub == 0 ? __fmul_rn(__fmul_rn(pi_f16_from_bits(du[j]), dx), (float)su) : 0.0f, pg = 0.0f;
+                if (GATE) {
+                    int sg = __builtin_amdgcn_sdot4((int)((qg[j][0] >> shift) & 0x0F0F0F0Fu), xq0, 0, false);
+                    sg = __builtin_amdgcn_sdot4((int)((qg[j][1] >> shift) & 0x0F0F0F0Fu), xq1, sg, false) - 8 * sx;
+                    sg += pi_dpp_i32<PI_DPP_XOR1, 0xF>(sg);
+                    sg += pi_dpp_i32<PI_DPP_XOR2, 0xF>(sg);
+                    pg = sub == 0 ? __fmul_rn(__fmul_rn(pi_f16_from_bits(dg[j]), dx), (float)sg) : 0.0f;
+                    pg = pi_wave_sum(pg);
+                }
+                pu = pi_wave_sum(pu);
+                if (lane == 0) { part[wave][j][0] = pu; part[wave][j][1] = pg; }
+            }
+        }
+        __syncthreads();
+        if (threadIdx.x < CH && (int)threadIdx.x < nn) {
+            const int j = threadIdx.x;
+            float u = 0.0f, g = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kPfWaves; ++w) { u += part[w][j][0]; if (GATE) g += part[w][j][1]; }
+            int nj = 0;
+#pragma unroll
+            for (int jj = 0; jj < CH; ++jj) if (jj == j) nj = nrn[jj];
+            h_dense[nj] = GATE ? __fmul_rn(fmaxf(g, 0.0f), u) : fmaxf(u, 0.0f);
+        }
+        if (c0 + CH < n) __syncthreads();                         // part[] is reused by the next chunk
+    }
+}
+
+// Q4_0 down projection behind pred_upgate_q4_kernel (cols == 4096).  A workgroup owns kAqGroups x 32 consecutive neurons.
+// Their h (hot and host-computed values merged by the caller; `h` may be pinned host memory, only wave 0 touches it) is
+// quantised to Q8_0 over the 32-neuron blocks exactly as the CPU path does on the dense vector (ggml.c:14465-14618):
+// d = amax/127 as fp16, q = rint(h*127/amax).  Neurons with q != 0 that live on the GPU are compacted into LDS, and the 8
+// waves each add their 512-column slice of those rows: acc += float((nibble - 8) * q) * (d_w * d_h), one fp32 multiply and
+// one fp32 add per element (ggml_axpy_q4_0_q8_0, ggml-quants.c:2426-2509), rows in ascending order.  One partial vector per
+// workgroup goes to `partial`; ffn_reduce_kernel adds them in workgroup order.
+constexpr int kAqGroups = 4;
+constexpr int kAqN = kAqGroups * 32;       // neurons per workgroup
+constexpr int kAqChunk = 16;               // rows in flight per wave
+
+__global__ __launch_bounds__(kPfBlock, 2) void axpy_q4_groups_kernel(const pi_block_q4_0 * __restrict__ Wd, const float * h, int ff,
+                                                                     const uint32_t * __restrict__ hot_words, const int32_t * __restrict__ hot_prefix,
+                                                                     float * __restrict__ partial) {
+    constexpr int cols = 4096, nb = cols / 32;
+    __shared__ int   lrow[kAqN];
+    __shared__ int   lq[kAqN];
+    __shared__ float ld[kAqN];
+    __shared__ int   ln;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int cbase = wave * 512 + lane * 8, blk = cbase >> 5, sub = lane & 3;
+    const int n0 = blockIdx.x * kAqN;
+    if (wave == 0) {
+        int cnt = 0;
+#pragma unroll
+        for (int i = 0; i < kAqN / 64; ++i) {
+            const int nrn = n0 + i * 64 + lane;
+            const float hvv = nrn < ff ? h[nrn] : 0.0f;
+            float amax = fabsf(hvv);
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, PI_WAVE));
+            const float d = amax / 127.0f, id = (amax != 0.0f) ? 127.0f / amax : 0.0f;
+            const int q = (int)rintf(__fmul_rn(hvv, id));
+            const int g = nrn >> 5;
+            const uint32_t hot = (nrn < ff) ? (hot_words ? hot_words[g] : 0xFFFFFFFFu) : 0u;
+            const bool take = q != 0 && ((hot >> (lane & 31)) & 1u);
+            const unsigned long long b = __ballot(take);
+            if (take) {
+                const int pos = cnt + __popcll(b & ((1ull << lane) - 1ull));
+                lrow[pos] = (hot_prefix ? hot_prefix[g] : (nrn & ~31)) + __popc(hot & ((1u << (lane & 31)) - 1u));
+                lq[pos] = q;
+                ld[pos] = pi_round_f16(d);
+            }
+            cnt += __popcll(b);
+        }
+        if (lane == 0) ln = cnt;
+    }
+    __syncthreads();
+    const int n = ln;
+    const int shift = (sub >> 1) * 4, qoff = (sub & 1) * 8;
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+    for (int k0 = 0; k0 < n; k0 += kAqChunk) {
+        uint32_t q[kAqChunk][2];
+        uint16_t dw[kAqChunk];
+#pragma unroll
+        for (int j = 0; j < kAqChunk; ++j) {
+            if (k0 + j < n) {
+                const pi_block_q4_0 * wb = Wd + (size_t)lrow[k0 + j] * nb + blk;
+                __builtin_memcpy(&dw[j], &wb->d, 2);
+                __builtin_memcpy(q[j], wb->qs + qoff, 8);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < kAqChunk; ++j) {
+            if (k0 + j < n) {
+                const int alpha = lq[k0 + j];
+                const float d = __fmul_rn(pi_f16_from_bits(dw[j]), ld[k0 + j]);
+#pragma unroll
+                for (int i = 0; i < 8; ++i) {
+                    const int v = (int)((q[j][i >> 2] >> ((i & 3) * 8 + shift)) & 0xF) - 8;
+                    acc[i] = __fadd_rn(acc[i], __fmul_rn((float)(v * alpha), d));
+                }
+            }
+        }
+    }
+    float4 * po = reinterpret_cast<float4 *>(partial + (size_t)blockIdx.x * cols + cbase);
+    po[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    po[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+}
+
 // compaction of existing mask words into the ascending active-row list (single block)
 __global__ __launch_bounds__(1024) void compact_words_kernel(const uint32_t * __restrict__ words, int ff, const int32_t * bucket, int n_bucket,
                                                              int32_t * list, int32_t * n_active) {
@@ -2645,6 +2940,7 @@ NormArgs to_norm(const pi_norm * n) {
 struct pi_workspace {
     int max_ff, max_d;
     uint32_t *     words;          // [max_ff/32 + 1]
+    uint32_t *     words_hot;      // [max_ff/32 + 1]  mask & GPU-resident neurons (Q4_0 fused route)
     unsigned int * counters;       // [64]: [0] predictor ticket, [1..] axpy tile tickets
     float *        partial;        // [kAxpyGroups][max_d]
     int32_t *      hq;             // [max_ff]  Q4_0 axpy: int8 value of h per active row
@@ -2662,6 +2958,7 @@ pi_workspace * pi_workspace_create(int max_ff, int max_d) {
     pi_workspace * ws = new pi_workspace{};
     ws->max_ff = max_ff; ws->max_d = max_d;
     ws->words    = (uint32_t *)pi_malloc(sizeof(uint32_t) * (max_ff / 32 + 2));
+    ws->words_hot = (uint32_t *)pi_malloc(sizeof(uint32_t) * (max_ff / 32 + 2));
     ws->counters = (unsigned int *)pi_malloc(sizeof(unsigned int) * 64);
     ws->partial  = (float *)pi_malloc(sizeof(float) * (size_t)kAxpyGroups * max_d);
     ws->hq       = (int32_t *)pi_malloc(sizeof(int32_t) * max_ff);
@@ -2670,7 +2967,7 @@ pi_workspace * pi_workspace_create(int max_ff, int max_d) {
     ws->ffn_partial = (float *)pi_malloc(sizeof(float) * n_part * max_d);
     ws->hc_batch = (__half *)pi_malloc(sizeof(__half) * ((size_t)max_ff + 16) * kBtMaxT);
     ws->row_any = (unsigned char *)pi_malloc((size_t)max_ff + 16);
-    if (!ws->words || !ws->counters || !ws->partial || !ws->hq || !ws->hd || !ws->ffn_partial || !ws->hc_batch || !ws->row_any) {
+    if (!ws->words || !ws->words_hot || !ws->counters || !ws->partial || !ws->hq || !ws->hd || !ws->ffn_partial || !ws->hc_batch || !ws->row_any) {
         pi_workspace_destroy(ws); return nullptr;
     }
     pi_memset(ws->counters, 0, sizeof(unsigned int) * 64);
@@ -2678,7 +2975,7 @@ pi_workspace * pi_workspace_create(int max_ff, int max_d) {
 }
 int pi_workspace_destroy(pi_workspace * ws) {
     if (!ws) return PI_OK;
-    pi_free(ws->words); pi_free(ws->counters); pi_free(ws->partial); pi_free(ws->hq); pi_free(ws->hd); pi_free(ws->ffn_partial); pi_free(ws->hc_batch); pi_free(ws->row_any);
+    pi_free(ws->words); pi_free(ws->words_hot); pi_free(ws->counters); pi_free(ws->partial); pi_free(ws->hq); pi_free(ws->hd); pi_free(ws->ffn_partial); pi_free(ws->hc_batch); pi_free(ws->row_any);
     delete ws;
     return PI_OK;
 }
@@ -2876,6 +3173,51 @@ int pi_k_pred_upgate(const void * fc2_f16, int ff, int r, const float * hidden, 
     hipLaunchKernelGGL((pred_upgate_f16_kernel<8, 2>), dim3(ff / 32), dim3(kBlock), 0, (hipStream_t)stream,
                        (const __half *)fc2_f16, hidden, (const __half *)up_f16, (const __half *)gate_f16, x, na, threshold, logits, ws->words, h_dense);
     return pi::check_launch("pi_k_pred_upgate");
+}
+
+int pi_k_pred_upgate_q4_supported(int ff, int r, int cols) {
+    return cols == 4096 && (r == 512 || r == 1024) && ff > 0 && ff % 32 == 0;
+}
+
+int pi_k_pred_upgate_q4(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                        const void * up_q4, const void * gate_q4, int cols, const float * x, const pi_norm * norm,
+                        const uint32_t * hot_words, const int32_t * hot_prefix,
+                        float * logits, float * h_dense, void * xq8_out, pi_workspace * ws, pi_stream_t stream) {
+    if (!fc2_f16 || !hidden || !up_q4 || !x || !h_dense || !ws) return pi::fail(PI_E_ARG, "pi_k_pred_upgate_q4: null pointer");
+    if (!pi_k_pred_upgate_q4_supported(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_pred_upgate_q4: shape outside the fused kernel (cols 4096, r 512 or 1024, ff % 32 == 0)");
+    if (ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_ARG, "pi_k_pred_upgate_q4: shape exceeds the workspace");
+    if ((hot_words == nullptr) != (hot_prefix == nullptr)) return pi::fail(PI_E_ARG, "pi_k_pred_upgate_q4: hot_words and hot_prefix go together");
+    const NormArgs na = to_norm(norm);
+    if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_pred_upgate_q4: vectors must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const __half * w2 = (const __half *)fc2_f16;
+    const pi_block_q4_0 * u = (const pi_block_q4_0 *)up_q4; const pi_block_q4_0 * g = (const pi_block_q4_0 *)gate_q4;
+    const dim3 grid(ff / 32), block(kPfBlock);
+#define PI_PQ_LAUNCH(RCH, GATE) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, GATE>), grid, block, 0, st, w2, hidden, u, g, x, na, threshold, hot_words, hot_prefix, logits, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)xq8_out)
+    if (r == 1024) { if (g) PI_PQ_LAUNCH(2, true); else PI_PQ_LAUNCH(2, false); }
+    else           { if (g) PI_PQ_LAUNCH(1, true); else PI_PQ_LAUNCH(1, false); }
+#undef PI_PQ_LAUNCH
+    return pi::check_launch("pi_k_pred_upgate_q4");
+}
+
+int pi_k_axpy_q4_partials(const void * down_t_q4, int cols, int ff, const float * h, const uint32_t * hot_words, const int32_t * hot_prefix,
+                          pi_workspace * ws, pi_stream_t stream) {
+    if (!down_t_q4 || !h || !ws) return pi::fail(PI_E_ARG, "pi_k_axpy_q4_partials: null pointer");
+    if (cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_UNSUPPORTED, "pi_k_axpy_q4_partials: cols must be 4096, ff % 32 == 0, within the workspace");
+    if ((hot_words == nullptr) != (hot_prefix == nullptr)) return pi::fail(PI_E_ARG, "pi_k_axpy_q4_partials: hot_words and hot_prefix go together");
+    hipLaunchKernelGGL(axpy_q4_groups_kernel, dim3((ff + kAqN - 1) / kAqN), dim3(kPfBlock), 0, (hipStream_t)stream,
+                       (const pi_block_q4_0 *)down_t_q4, h, ff, hot_words, hot_prefix, ws->ffn_partial);
+    return pi::check_launch("pi_k_axpy_q4_partials");
+}
+
+int pi_k_axpy_q4_reduce(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out, int32_t * n_active,
+                        pi_workspace * ws, pi_stream_t stream) {
+    if (!out || !ws || cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_axpy_q4_reduce: bad arguments");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_axpy_q4_reduce: bad epilogue arguments");
+    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, (ff + kAqN - 1) / kAqN, cols,
+                       ws->words_hot, ff / 32, n_active, epilogue, add1, add2, out);
+    return pi::check_launch("pi_k_axpy_q4_reduce");
 }
 
 int pi_k_pred_upgate_supported(int ff, int r, int cols) { return cols == 4096 && r == 1024 && ff > 0 && ff % 32 == 0; }

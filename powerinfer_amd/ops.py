@@ -127,6 +127,48 @@ class SparseFFN:
         return dict(logits=self.logits.download(np.float32), h=self.h_dense.download(np.float32),
                     n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32))
 
+    def _hot_tables(self):
+        """hot_words[g] bit j: neuron 32g+j is GPU-resident; hot_prefix[g]: resident neurons before group g."""
+        if self.bucket_host is None:
+            return None, None
+        if not hasattr(self, "_hot"):
+            bits = np.zeros(self.ff, np.uint8)
+            bits[self.bucket_host] = 1
+            words = (bits.reshape(-1, 32).astype(np.uint64) << np.arange(32, dtype=np.uint64)).sum(1).astype(np.uint32)
+            prefix = np.concatenate([[0], np.cumsum(bits.reshape(-1, 32).sum(1))[:-1]]).astype(np.int32)
+            self._hot = (DevBuf(host=words), DevBuf(host=prefix))
+        return self._hot
+
+    def forward_q4_fused(self, x_ffn, x_pred, epilogue=pl.EPI_NONE, resid=None, fill_h=None):
+        """Q4_0 route of the decode loop at d = 4096: fc1, pi_k_pred_upgate_q4 (fc2 + mask + up/gate of the resident neurons),
+        then pi_k_axpy_q4_partials + pi_k_axpy_q4_reduce.  fill_h(h) may return the vector with the host share's neurons
+        filled in (hybrid layers) before the down projection.  Returns dict(logits, h, xq8, n_active, out)."""
+        L = self.L
+        if self.wtype != pl.Q4_0 or not L.pi_k_pred_upgate_q4_supported(self.ff, self.r, self.d):
+            raise pl.PiError("forward_q4_fused: type or shape outside the fused kernels")
+        hw, hp = self._hot_tables()
+        p = lambda b: b.ptr if b is not None else None  # noqa: E731
+        self.x.upload(np.asarray(x_ffn, np.float32))
+        self.xp.upload(np.asarray(x_pred, np.float32))
+        if resid is not None:
+            self.resid.upload(np.asarray(resid, np.float32))
+        check(L.pi_memset(self.h_dense.ptr, 0xFF, self.h_dense.nbytes), "memset")      # the kernel must write every entry
+        xq8 = DevBuf(self.d // 32 * 34)
+        nrm = pl.norm_arg(self.norm_kind, self.eps, self.norm_w, self.norm_b)
+        check(L.pi_k_gemv(pl.F16, self.fc1.ptr, self.r, self.d, self.xp.ptr, None, pl.EPI_RELU, None, None, self.hidden.ptr, None), "fc1")
+        check(L.pi_k_pred_upgate_q4(self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, self.up.ptr, p(self.gate), self.d,
+                                    self.x.ptr, nrm, p(hw), p(hp), self.logits.ptr, self.h_dense.ptr, xq8.ptr, self.ws, None), "pred_upgate_q4")
+        pl.sync()
+        h = self.h_dense.download(np.float32)
+        if fill_h is not None:
+            self.h_dense.upload(np.ascontiguousarray(fill_h(h.copy()), np.float32))
+        check(L.pi_k_axpy_q4_partials(self.down.ptr, self.d, self.ff, self.h_dense.ptr, p(hw), p(hp), self.ws, None), "axpy_q4_partials")
+        check(L.pi_k_axpy_q4_reduce(self.ff, self.d, epilogue, self.resid.ptr if epilogue else None, None, self.out.ptr,
+                                    self.n_active.ptr, self.ws, None), "axpy_q4_reduce")
+        pl.sync()
+        return dict(logits=self.logits.download(np.float32), h=h, xq8=xq8.download(np.uint8),
+                    n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32))
+
     def close(self):
         if self.ws:
             self.L.pi_workspace_destroy(self.ws)

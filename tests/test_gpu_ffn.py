@@ -135,6 +135,106 @@ def run_fused_route(has_gate, norm, route, d, ff, r):
     ffn.close()
 
 
+def q8_blocks_np(v):
+    """Q8_0 over blocks of 32 as quantize_row_q8_0 does on x86 (ggml-quants.c:702-760): returns (q int32, d float32 per element)."""
+    v = np.asarray(v, np.float32).reshape(-1, 32)
+    amax = np.abs(v).max(1)
+    d = (amax / np.float32(127.0)).astype(np.float32)
+    idv = np.where(amax != 0, np.float32(127.0) / np.where(amax != 0, amax, 1), 0).astype(np.float32)
+    q = np.rint(v * idv[:, None]).astype(np.int32)
+    return q.reshape(-1), np.repeat(d.astype(np.float16).astype(np.float32), 32)
+
+
+def q4_rows_np(raw, rows, d):
+    """(nibble - 8) [len(rows), d] int32 and the fp32 block scales [len(rows), d/32] of Q4_0 rows."""
+    b = raw[rows].reshape(len(rows), d // 32, 18)
+    dw = b[:, :, :2].copy().view(np.float16).astype(np.float32)[:, :, 0]
+    qs = b[:, :, 2:]
+    v = np.concatenate([qs & 0x0F, qs >> 4], axis=2).astype(np.int32) - 8
+    return v.reshape(len(rows), d), dw
+
+
+@pytest.mark.parametrize("has_gate", [True, False])
+@pytest.mark.parametrize("norm", [0, 1, 2])
+def test_q4_fused_route_7b_shape(has_gate, norm):
+    """pi_k_pred_upgate_q4 + pi_k_axpy_q4_partials/_reduce (what the Q4_0 decode loop runs at d = 4096), all neurons resident,
+    against the oracle; the Q8_0 blocks the kernel hands to a host share are checked against the closed form."""
+    from powerinfer_amd import lib as pl
+    from powerinfer_amd.ops import SparseFFN
+    d, ff, r, T = 4096, 11008, 1024, 3
+    L = synth.make_ffn_layer(seed=90 + norm, d=d, ff=ff, r=r, wtype=ol.Q4_0, has_gate=has_gate, T=T)
+    rng = np.random.default_rng(6)
+    nw = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32) if norm else None
+    nb = (0.1 * rng.standard_normal(d)).astype(np.float32) if norm == 2 else None
+    eps = 1e-5
+    O, P = ol.oracle(), ol._ptr
+    ffn = SparseFFN(d, ff, r, ol.Q4_0, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], norm_kind=norm, norm_w=nw, norm_b=nb, eps=eps)
+    for t in range(T):
+        x = np.ascontiguousarray(L["x"][t:t + 1], np.float32)
+        xn = x.copy()
+        if norm == 1:
+            O.pio_rms_norm(P(x), d, 1, eps, P(xn)); xn = np.ascontiguousarray(xn * nw, np.float32)
+        elif norm == 2:
+            O.pio_norm(P(x), d, 1, eps, P(xn)); xn = np.ascontiguousarray(xn * nw + nb, np.float32)
+        o = ol.ffn_sparse(O, d, ff, r, 1, ol.Q4_0, has_gate, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], xn, x,
+                          np.zeros(ff, np.int32), 0.0, nth=8)
+        resid = rng.standard_normal(d).astype(np.float32)
+        res = ffn.forward_q4_fused(x[0], x[0], epilogue=pl.EPI_ADD, resid=resid)
+        assert rel_err(res["logits"], o["logits"][0]) < 1e-4
+        mask_g, mask_o = ~(res["logits"] < 0.0), ~(o["logits"][0] < 0.0)
+        assert (mask_g == mask_o).mean() >= MASK_AGREE
+        assert res["n_active"] == int(mask_g.sum())
+        assert not np.isnan(res["h"]).any()
+        assert np.all(res["h"][~mask_g] == 0.0)
+        # Q8_0 blocks of the normalised input: int8 values may differ by one step where the norm differs in the last place
+        blocks = res["xq8"].reshape(d // 32, 34)
+        qg = blocks[:, 2:].copy().view(np.int8).astype(np.int32).reshape(-1)
+        dg = np.repeat(blocks[:, :2].copy().view(np.float16).astype(np.float32)[:, 0], 32)
+        qo, do = q8_blocks_np(xn[0])
+        assert np.abs(qg - qo).max() <= 1 and (qg != qo).mean() < 1e-3
+        assert np.allclose(dg, do, rtol=2e-3)
+        if np.array_equal(mask_g, mask_o):
+            assert rel_err(res["h"], o["h"][0]) < 1e-4
+            assert rel_err(res["out"] - resid, o["out"][0]) < FFN_REL_TOL     # an int8 step of h where h * 127/amax sits on a rounding boundary
+    ffn.close()
+
+
+def test_q4_fused_route_hybrid_share():
+    """Hot/cold split at the 7B width: the kernels see only the resident 60 % (compact matrices, hot words / prefix); with the
+    cold neurons' h filled in before the down projection, GPU share + cold share (numpy, same Q8_0 blocks of h) must equal the
+    oracle computing every neuron."""
+    from powerinfer_amd.ops import SparseFFN
+    d, ff, r, T = 4096, 4096, 512, 2
+    L = synth.make_ffn_layer(seed=33, d=d, ff=ff, r=r, wtype=ol.Q4_0, mean_rate=0.15, T=T)
+    gid, bucket = synth.gpu_split(L["p"], 0.6)
+    O = ol.oracle()
+    full = ol.ffn_sparse(O, d, ff, r, T, ol.Q4_0, 1, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], L["x"], L["x"], np.zeros(ff, np.int32), 0.0)
+    ffn = SparseFFN(d, ff, r, ol.Q4_0, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], bucket=bucket)
+    for t in range(T):
+        cold = gid == 0
+
+        def fill(h):
+            assert np.all(h[cold] == 0.0)                       # the kernel writes zeros outside its share
+            h[cold] = full["h"][t][cold]
+            return h
+
+        res = ffn.forward_q4_fused(L["x"][t], L["x"][t], fill_h=fill)
+        mask_g, mask_o = ~(res["logits"] < 0.0), ~(full["logits"][t] < 0.0)
+        assert rel_err(res["logits"], full["logits"][t]) < 1e-4
+        assert res["n_active"] == int((mask_g & ~cold).sum())
+        if not np.array_equal(mask_g, mask_o):
+            continue
+        assert rel_err(res["h"][~cold], full["h"][t][~cold]) < 1e-4
+        hm = res["h"].copy(); hm[cold] = full["h"][t][cold]
+        q, dh = q8_blocks_np(hm)
+        rows = np.nonzero(cold & (q != 0))[0]
+        v, dw = q4_rows_np(L["down_t"], rows, d)
+        contrib = (v * q[rows, None]).astype(np.float32) * (np.repeat(dw, 32, axis=1) * dh[rows, None])
+        cold_out = contrib.sum(0, dtype=np.float32)
+        assert rel_err(res["out"] + cold_out, full["out"][t]) < FFN_REL_TOL
+    ffn.close()
+
+
 @pytest.mark.parametrize("wtype", [ol.F16, ol.Q4_0])
 def test_hybrid_split_gpu_share(wtype):
     """Config 2 split: the GPU holds the hottest 60 % of neurons (compact matrices + gpu_bucket) and

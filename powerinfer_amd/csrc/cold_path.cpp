@@ -143,14 +143,43 @@ void axpy_q4_blocks(const BlockQ4 * row, int b0, int b1, int a, float sc, float 
     }
 }
 
+// the cold rows live in host DRAM and a token touches each of them once: fetch the next row while this one is used
+inline void prefetch_bytes(const void * p, size_t n) {
+#ifdef PI_COLD_SIMD
+    const char * b = (const char *)p;
+    for (size_t o = 0; o < n; o += 64) _mm_prefetch(b + o, _MM_HINT_T0);
+#else
+    (void)p; (void)n;
+#endif
+}
+
 // x86 quantize_row_q8_0 semantics (ggml-quants.c:702-760): d = amax/127 stored as fp16, q = rint(x * 127/amax)
 void quantize_q8(const float * x, BlockQ8 * y, int n) {
     for (int b = 0; b < n / 32; ++b) {
+#ifdef PI_COLD_SIMD
+        const __m256 sign = _mm256_set1_ps(-0.0f);
+        __m256 v[4], mx = _mm256_setzero_ps();
+        for (int k = 0; k < 4; ++k) { v[k] = _mm256_loadu_ps(x + b * 32 + 8 * k); mx = _mm256_max_ps(mx, _mm256_andnot_ps(sign, v[k])); }
+        __m128 m4 = _mm_max_ps(_mm256_extractf128_ps(mx, 1), _mm256_castps256_ps128(mx));
+        m4 = _mm_max_ps(m4, _mm_movehl_ps(m4, m4));
+        m4 = _mm_max_ss(m4, _mm_movehdup_ps(m4));
+        const float amax = _mm_cvtss_f32(m4);
+        const float d = amax / 127.f, id = amax != 0.f ? 127.f / amax : 0.f;
+        y[b].d = f2h(d);
+        const __m256 mul = _mm256_set1_ps(id);
+        __m256i q[4];
+        for (int k = 0; k < 4; ++k) q[k] = _mm256_cvtps_epi32(_mm256_mul_ps(v[k], mul));        // round to nearest even, as rintf
+        const __m256i p01 = _mm256_packs_epi32(q[0], q[1]), p23 = _mm256_packs_epi32(q[2], q[3]);   // lanes interleave: fixed below
+        __m256i p = _mm256_packs_epi16(p01, p23);
+        p = _mm256_permutevar8x32_epi32(p, _mm256_setr_epi32(0, 4, 1, 5, 2, 6, 3, 7));
+        _mm256_storeu_si256((__m256i *)y[b].qs, p);
+#else
         float amax = 0.f;
         for (int j = 0; j < 32; ++j) amax = fmaxf(amax, fabsf(x[b * 32 + j]));
         const float d = amax / 127.f, id = amax != 0.f ? 127.f / amax : 0.f;
         y[b].d = f2h(d);
         for (int j = 0; j < 32; ++j) y[b].qs[j] = (int8_t)(int)rintf(x[b * 32 + j] * id);
+#endif
     }
 }
 
@@ -230,6 +259,7 @@ struct ColdPath {
     // pinned staging
     float * logits = nullptr, * src = nullptr, * h_gpu = nullptr;      // device -> host, consumed before the layer call returns
     float * h_full[2] = {nullptr, nullptr}, * out[2] = {nullptr, nullptr};   // host -> device, read by the GPU after the call returned: two sets, used in turn
+    BlockQ8 * xq8_pin = nullptr;                // Q8_0 blocks of the normalised FFN input, written by the fused Q4_0 kernel
     int flip = 0;
     hipEvent_t ev_in = nullptr, ev_h = nullptr;
     std::vector<float> hval;                    // h of the active cold neurons, in the order of act
@@ -251,7 +281,7 @@ ColdPath * cold_create(pi_model * m) {
     const pi_hparams & hp = m->hp;
     c->d = hp.n_embd; c->ff = hp.n_ff;
     int nt = (int)std::thread::hardware_concurrency();
-    if (nt > 16) nt = 16;
+    if (nt > 8) nt = 8;        // the forks are microseconds long and the workers spin between them: more threads only add join latency
     if (const char * e = getenv("PI_COLD_THREADS")) { const int v = atoi(e); if (v > 0) nt = v; }
     if (nt < 1) nt = 1;
     c->pool = new Pool(nt);
@@ -271,10 +301,11 @@ ColdPath * cold_create(pi_model * m) {
         const int32_t * gid = (const int32_t *)m->L(il, PI_T_GPU_IDX).host;
         for (int j = 0; j < c->ff; ++j) if (gid[j] != 1) cl.cold_rows.push_back(j);
     }
-    auto pin = [](size_t n) { void * p = nullptr; return hipHostMalloc(&p, n * sizeof(float), hipHostMallocDefault) == hipSuccess ? (float *)p : nullptr; };
+    auto pin = [](size_t n) { void * p = nullptr; return hipHostMalloc(&p, n * sizeof(float), hipHostMallocCoherent) == hipSuccess ? (float *)p : nullptr; };
+    c->xq8_pin = (BlockQ8 *)pin((size_t)(c->d / 32 + 1) * sizeof(BlockQ8) / sizeof(float) + 1);
     c->logits = pin(c->ff); c->src = pin(c->d); c->h_gpu = pin(c->ff);
     for (int i = 0; i < 2; ++i) { c->h_full[i] = pin(c->ff); c->out[i] = pin(c->d); }
-    if (!c->logits || !c->src || !c->h_gpu || !c->h_full[0] || !c->h_full[1] || !c->out[0] || !c->out[1]) { set_error("cold path: pinned host allocation failed"); cold_destroy(c); return nullptr; }
+    if (!c->logits || !c->src || !c->h_gpu || !c->h_full[0] || !c->h_full[1] || !c->out[0] || !c->out[1] || !c->xq8_pin) { set_error("cold path: pinned host allocation failed"); cold_destroy(c); return nullptr; }
     if (hipEventCreateWithFlags(&c->ev_in, hipEventDisableTiming) != hipSuccess || hipEventCreateWithFlags(&c->ev_h, hipEventDisableTiming) != hipSuccess) {
         set_error("cold path: event creation failed"); cold_destroy(c); return nullptr;
     }
@@ -292,6 +323,7 @@ void cold_destroy(ColdPath * c) {
     }
     delete c->pool;
     for (float * p : {c->logits, c->src, c->h_gpu, c->h_full[0], c->h_full[1], c->out[0], c->out[1]}) if (p) (void)hipHostFree(p);
+    if (c->xq8_pin) (void)hipHostFree(c->xq8_pin);
     if (c->ev_in) (void)hipEventDestroy(c->ev_in);
     if (c->ev_h) (void)hipEventDestroy(c->ev_h);
     delete c;
@@ -447,6 +479,101 @@ int cold_layer_merge(ColdPath * c, int il, pi_model * m, hipStream_t st) {
     lap(4);
     const int rc = merge_shares(m->x2, out, m->x2, falcon ? m->attn_out : m->ffn_inp, falcon ? m->x : nullptr,
                                 m->capture ? m->cap_ffn + (size_t)il * d : nullptr, d, st);
+    lap(5);
+    if (c->trace) { ++c->n_calls; c->n_cold_active += na; c->t_last_return = now(); }
+    return rc;
+}
+
+int cold_layer_q4(ColdPath * c, int il, pi_model * m, hipStream_t st, bool capture) {
+    const pi_hparams & hp = m->hp;
+    const int d = c->d, ff = c->ff;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    ColdLayer & cl = c->layers[il];
+    Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
+    Tensor & fc1 = m->L(il, PI_T_FC1); Tensor & fc2 = m->L(il, PI_T_FC2);
+    const int r = (int)fc1.ne1;
+    const float thr = hp.sparse_threshold;
+    const int p = (c->flip ^= 1);
+    float * hfull = c->h_full[p];
+    float * out = c->out[p];
+    auto now = [] { return std::chrono::steady_clock::now(); };
+    auto us = [](std::chrono::steady_clock::time_point a, std::chrono::steady_clock::time_point b) { return std::chrono::duration<double, std::micro>(b - a).count(); };
+    std::chrono::steady_clock::time_point tp = now();
+    if (c->trace && c->n_calls) c->t_between += us(c->t_last_return, tp);
+    auto lap = [&](int i) { if (c->trace) { const auto t = now(); c->t_phase[i] += us(tp, t); tp = t; } };
+
+    // 1. the kernel writes what the host needs straight into pinned memory: logits, the Q8_0 blocks of the normalised input,
+    //    and h (resident active neurons; zero elsewhere) into the vector the host completes below
+    pi_norm fn;
+    fn.kind = falcon ? 2 : 1; fn.eps = hp.norm_eps;
+    fn.w = (const float *)m->L(il, falcon ? PI_T_ATTN_NORM : PI_T_FFN_NORM).dev;
+    fn.b = falcon ? (const float *)m->L(il, PI_T_ATTN_NORM_B).dev : nullptr;
+    const float * ffn_src = falcon ? m->x : m->ffn_inp;
+    int rc = pi_k_pred_upgate_q4(fc2.dev, ff, r, m->hidden, thr, up.dev, falcon ? nullptr : gate.dev, d, ffn_src, &fn,
+                                 m->hot_words[il], m->hot_prefix[il], c->logits, hfull, c->xq8_pin, m->ws, st);
+    if (rc != PI_OK) return rc;
+    PI_HIP_TRY(hipEventRecord(c->ev_in, st));
+    if (capture) PI_HIP_TRY(hipMemcpyAsync(m->cap_logits + (size_t)il * ff, c->logits, sizeof(float) * ff, hipMemcpyHostToDevice, st));
+    PI_HIP_TRY(wait_event(c->ev_in));
+    lap(0);
+
+    // 2. active cold neurons, their up/gate rows against the same Q8_0 input
+    c->act.clear();
+    for (int j : cl.cold_rows) if (!(c->logits[j] < thr)) c->act.push_back(j);
+    const int na = (int)c->act.size();
+    lap(1);
+    float * hval = c->hval.data();
+    const size_t rb = (size_t)(d / 32) * 18;
+    const unsigned char * wu = (const unsigned char *)up.host;
+    const unsigned char * wg = falcon ? nullptr : (const unsigned char *)gate.host;
+    const BlockQ8 * xq = c->xq8_pin;
+    c->pool->run([&](int t, int nt) {
+        for (int k = t; k < na; k += nt) {
+            const int j = c->act[k];
+            if (k + nt < na) { prefetch_bytes(wu + rb * c->act[k + nt], rb); if (wg) prefetch_bytes(wg + rb * c->act[k + nt], rb); }
+            const float u = dot_q4_q8(d, (const BlockQ4 *)(wu + rb * j), xq);
+            const float g = wg ? dot_q4_q8(d, (const BlockQ4 *)(wg + rb * j), xq) : 0.f;
+            hval[k] = wg ? (g > 0.f ? g : 0.f) * u : (u > 0.f ? u : 0.f);
+        }
+    });
+    for (int k = 0; k < na; ++k) hfull[c->act[k]] = hval[k];
+    lap(2);
+
+    // 3. the GPU's down projection reads the completed vector from the pinned buffer; the host quantises it the same way
+    rc = pi_k_axpy_q4_partials(down.dev, d, ff, hfull, m->hot_words[il], m->hot_prefix[il], m->ws, st);
+    if (rc != PI_OK) return rc;
+    for (int k = 0, last = -1; k < na; ++k) {               // act is ascending: only the Q8_0 blocks of h that hold an active cold neuron
+        const int b = c->act[k] / 32;
+        if (b != last) { quantize_q8(hfull + b * 32, c->hq8.data() + b, 32); last = b; }
+    }
+    lap(3);
+    const unsigned char * wd = (const unsigned char *)down.host;
+    const int n_units = d / 32;
+    c->pool->run([&](int t, int nt) {
+        const int u0 = (int)((long long)n_units * t / nt), u1 = (int)((long long)n_units * (t + 1) / nt);
+        for (int i = u0 * 32; i < u1 * 32; ++i) out[i] = 0.f;
+        for (int k = 0; k < na; ++k) {
+            const int j = c->act[k];
+            const BlockQ8 & hb = c->hq8[j / 32];
+            const int a = hb.qs[j % 32];
+            if (k + 2 < na) prefetch_bytes(wd + rb * c->act[k + 2] + (size_t)u0 * 18, (size_t)(u1 - u0) * 18);
+            if (a == 0) continue;
+            axpy_q4_blocks((const BlockQ4 *)(wd + rb * j), u0, u1, a, h2f(hb.d), out);
+        }
+    });
+    lap(4);
+
+    // 4. (cold + hot) + residual(s), the reference's order (ggml_add(cpu, gpu), then the residual adds): folded into the
+    //    reduction of the GPU partials when there is a single residual and nothing to keep
+    int32_t * n_act = m->n_active + il;
+    if (!falcon && !capture) {
+        rc = pi_k_axpy_q4_reduce(ff, d, PI_EPI_ADD2, out, m->ffn_inp, m->x2, n_act, m->ws, st);
+    } else {
+        rc = pi_k_axpy_q4_reduce(ff, d, PI_EPI_NONE, nullptr, nullptr, m->x2, n_act, m->ws, st);
+        if (rc == PI_OK)
+            rc = merge_shares(m->x2, out, m->x2, falcon ? m->attn_out : m->ffn_inp, falcon ? m->x : nullptr,
+                              capture ? m->cap_ffn + (size_t)il * d : nullptr, d, st);
+    }
     lap(5);
     if (c->trace) { ++c->n_calls; c->n_cold_active += na; c->t_last_return = now(); }
     return rc;

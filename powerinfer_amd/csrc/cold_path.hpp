@@ -19,6 +19,10 @@ int        cold_stage_inputs(ColdPath * c, int il, pi_model * m, hipStream_t st)
 // output (cold + hot + residuals) in m->x2.
 int        cold_layer_merge(ColdPath * c, int il, pi_model * m, hipStream_t st);
 
+// Q4_0 hybrid layer at d = 4096 on the fused kernels: queues fc2 + mask + resident up/gate, computes the host share from the
+// buffers that launch fills, queues the down projection and the merge; leaves the layer output in m->x2.
+int        cold_layer_q4(ColdPath * c, int il, pi_model * m, hipStream_t st, bool capture);
+
 int add_vec(float * y, const float * a, int n, hipStream_t st);
 // dst = ((cold + hot) + r1) [+ r2]; `cold` may be pinned host memory; `keep` (optional) receives cold + hot
 int merge_shares(float * dst, const float * cold, const float * hot, const float * r1, const float * r2, float * keep, int n, hipStream_t st);

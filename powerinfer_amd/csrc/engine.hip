@@ -186,6 +186,34 @@ int layer_forward(pi_model * m, int il, bool last_token) {
         std::swap(m->x, m->x2);
         return PI_OK;
     }
+    if (q4 && fc2.type == PI_TYPE_F16 && pi_k_pred_upgate_q4_supported(ff, r, d) && (!layer_hybrid || m->hot_words[il])) {
+        // Q4_0 at d = 4096: fc2 + mask + up/gate of the resident neurons in one launch, the down projection as partial vectors
+        // plus one reduction; a hybrid layer's host share works between the two from the buffers the first kernel fills
+        const void * gp = falcon ? nullptr : gate.dev;
+        const bool cap = m->capture && last_token;
+        if (layer_hybrid) {
+            PI_TRY(pi::cold_layer_q4(m->cold, il, m, st, cap));
+        } else {
+            PI_TRY(pi_k_pred_upgate_q4(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, gp, d, ffn_in, &fn, nullptr, nullptr,
+                                       m->pred_logits, m->h_dense, nullptr, m->ws, st));
+            PI_TRY(pi_k_axpy_q4_partials(down.dev, d, ff, m->h_dense, nullptr, nullptr, m->ws, st));
+            if (cap) {
+                float * ffo = m->cap_ffn + (size_t)il * d;
+                PI_TRY(pi_k_axpy_q4_reduce(ff, d, PI_EPI_NONE, nullptr, nullptr, ffo, n_act, m->ws, st));
+                PI_HIP_TRY(hipMemcpyAsync(m->x2, ffo, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
+                PI_TRY(pi::add_vec(m->x2, falcon ? m->attn_out : m->ffn_inp, d, st));
+                if (falcon) PI_TRY(pi::add_vec(m->x2, x, d, st));
+                PI_HIP_TRY(hipMemcpyAsync(m->cap_logits + (size_t)il * ff, m->pred_logits, sizeof(float) * ff, hipMemcpyDeviceToDevice, st));
+            } else if (!falcon) {
+                PI_TRY(pi_k_axpy_q4_reduce(ff, d, PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, n_act, m->ws, st));
+            } else {
+                PI_TRY(pi_k_axpy_q4_reduce(ff, d, PI_EPI_ADD2, m->attn_out, x, m->x2, n_act, m->ws, st));
+            }
+        }
+        if (cap) PI_HIP_TRY(hipMemcpyAsync(m->cap_src + (size_t)il * d, ffn_in, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
+        std::swap(m->x, m->x2);
+        return PI_OK;
+    }
     // F16 layers that live entirely on the GPU take the fused route: the up/gate kernel reads the mask words itself
     const bool fused = !layer_hybrid && !q4;
     const int n_rows = layer_hybrid ? n_bucket : ff;
@@ -413,6 +441,24 @@ int pi_model_finalize(pi_model * m) {
                 t.owned = true;
                 PI_TRY(pi_memcpy_h2d(t.dev, tmp.data(), tmp.size()));
             }
+        }
+    }
+
+    // hot words / prefix of hybrid layers for the kernels that walk the neurons in groups of 32
+    m->hot_words.assign(hp.n_layer, nullptr); m->hot_prefix.assign(hp.n_layer, nullptr);
+    if (ff % 32 == 0) {
+        for (int il = 0; il < hp.n_layer; ++il) {
+            Tensor & bucket = m->L(il, PI_T_GPU_BUCKET);
+            if (!bucket.dev) continue;
+            const int32_t * bk_host = (const int32_t *)bucket.host;
+            std::vector<uint32_t> words(ff / 32, 0u);
+            std::vector<int32_t> prefix(ff / 32, 0);
+            for (int i = 0; i < (int)bucket.ne0; ++i) words[bk_host[i] >> 5] |= 1u << (bk_host[i] & 31);
+            for (int g = 1; g < ff / 32; ++g) prefix[g] = prefix[g - 1] + __builtin_popcount(words[g - 1]);
+            m->hot_words[il] = m->alloc<uint32_t>(ff / 32); m->hot_prefix[il] = m->alloc<int32_t>(ff / 32);
+            if (!m->hot_words[il] || !m->hot_prefix[il]) return PI_E_HIP;
+            PI_TRY(pi_memcpy_h2d(m->hot_words[il], words.data(), sizeof(uint32_t) * words.size()));
+            PI_TRY(pi_memcpy_h2d(m->hot_prefix[il], prefix.data(), sizeof(int32_t) * prefix.size()));
         }
     }
 

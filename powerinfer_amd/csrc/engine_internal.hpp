@@ -47,6 +47,8 @@ struct pi_model {
     bool capture = false;
     float *cap_ffn = nullptr, *cap_logits = nullptr, *cap_src = nullptr;       // device
     pi::ColdPath * cold = nullptr;
+    std::vector<uint32_t *> hot_words;    // per hybrid layer: bit j of word g set iff neuron 32g+j is GPU-resident (device)
+    std::vector<int32_t *> hot_prefix;    //                   GPU-resident neurons before group g = row of the compact matrices
     BatchState * batch = nullptr;         // per-sequence caches and step buffers of batched decoding
     BatchState * prefill = nullptr;       // step buffers for prompt chunks of the model's own sequence
 

@@ -618,6 +618,14 @@ int pi_model_time_section(pi_model * m, int section, int rounds, float * ms_tota
                     ++n;
                     continue;
                 }
+                if (q4 && fc2.type == PI_TYPE_F16 && pi_k_pred_upgate_q4_supported(ff, (int)fc1.ne1, d)) {
+                    PI_TRY(pi_k_pred_upgate_q4(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, d, fin, &fn,
+                                               nullptr, nullptr, m->pred_logits, m->h_dense, nullptr, m->ws, st));
+                    PI_TRY(pi_k_axpy_q4_partials(down.dev, d, ff, m->h_dense, nullptr, nullptr, m->ws, st));
+                    PI_TRY(pi_k_axpy_q4_reduce(ff, d, PI_EPI_ADD, fin, nullptr, m->x2, m->n_active + il, m->ws, st));
+                    ++n;
+                    continue;
+                }
                 PI_TRY(pi_k_predictor_fc2(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, nullptr, 0, m->pred_logits,
                                           q4 ? m->list : nullptr, q4 ? m->n_active + il : nullptr, q4 ? m->h_dense : nullptr, m->ws, st));
                 PI_TRY(pi_k_sparse_upgate(up.type, up.dev, falcon ? nullptr : gate.dev, d, ff, fin, &fn, q4 ? 0 : 1, m->list, m->n_active + il, nullptr, m->h_c,

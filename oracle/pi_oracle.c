@@ -722,6 +722,35 @@ done:
     return rc;
 }
 
+/* K-shift (llm_build_k_shift, llama.cpp:4332-4381): every layer's K cache, viewed [n_rot = head size][n_head_kv][n_ctx], goes
+ * through the in-place RoPE of fp16 data (ggml_compute_forward_rope_f16, ggml.c:11327-11478) with the cells' accumulated
+ * position deltas as "positions" (delta[n_ctx], llama.cpp:6533-6547): fp16 -> fp32, rotate by delta * theta_i with theta
+ * advanced by repeated fp32 multiplication, round back to fp16.  A cell with delta 0 is rotated by angle 0 and keeps its bits. */
+int pio_model_k_shift(pio_model * m, const int32_t * delta) {
+    const pio_hparams * hp = &m->hp;
+    const int hd = hp->n_embd / hp->n_head, gqa = hd * hp->n_head_kv;
+    const int is_neox = hp->arch == 1;
+    const float theta_scale = powf(hp->rope_freq_base, -2.0f / hd);
+    for (int il = 0; il < hp->n_layer; ++il) {
+        uint16_t * kc = m->k_cache + (size_t)il * hp->n_ctx * gqa;
+        for (int c = 0; c < hp->n_ctx; ++c)
+            for (int h = 0; h < hp->n_head_kv; ++h) {
+                uint16_t * row = kc + (size_t)c * gqa + (size_t)h * hd;
+                float theta_base = (float)delta[c];
+                if (is_neox) theta_base *= 1.0f;                       /* freq_scale, ggml.c:11447 */
+                for (int i = 0; i < hd / 2; ++i) {
+                    const float c_ = cosf(theta_base), s_ = sinf(theta_base);
+                    theta_base *= theta_scale;
+                    const int i0 = is_neox ? i : 2 * i, i1 = is_neox ? i + hd / 2 : 2 * i + 1;
+                    const float x0 = H2F(row[i0]), x1 = H2F(row[i1]);
+                    row[i0] = F2H(x0 * c_ - x1 * s_);
+                    row[i1] = F2H(x0 * s_ + x1 * c_);
+                }
+            }
+    }
+    return 0;
+}
+
 /* single sequence: cell = position, n_kv = max(32, n_past + T) (llama.cpp:6842), mask as llama.cpp:6506-6531;
  * returns the greedy token of the last position (first maximum wins, llama.cpp:8617-8631) or -1 */
 int pio_model_eval_simple(pio_model * m, const int32_t * tokens, int T, int n_past, float * logits_out, int n_threads) {

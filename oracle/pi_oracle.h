@@ -114,6 +114,8 @@ PIO_API void        pio_model_set_capture(pio_model * m, float * ffn_out, float 
  * n_kv cells attended, kq_mask [T][n_kv] (0 or -inf).  logits_out [T][n_vocab] if all_logits else
  * [n_vocab] of the last token.  Returns 0 on success.
  */
+/* llm_build_k_shift: rotates every cached K row by delta[cell] positions (delta[n_ctx]; 0 leaves the cell's bits unchanged) */
+PIO_API int         pio_model_k_shift(pio_model * m, const int32_t * delta);
 PIO_API int         pio_model_eval(pio_model * m, const int32_t * tokens, const int32_t * pos, const int32_t * kv_slot,
                                    int T, int n_kv, const float * kq_mask, int all_logits, float * logits_out, int n_threads);
 

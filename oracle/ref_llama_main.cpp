@@ -4,6 +4,10 @@
 // oracle/_ref/ref_llama from the reference sources where they lie; used by tests/golden/make_llama_fixture.py.
 //
 //   ref_llama <model.gguf> <n_ctx> <n_threads> <n_generate> <out.bin> tok0 tok1 ...
+//
+// With REF_SHIFT_AT=s REF_N_KEEP=k REF_N_DISCARD=d in the environment the driver does, before step s, what the reference's
+// examples do when the context is full (examples/main/main.cpp): llama_kv_cache_seq_rm(ctx, 0, k, k + d), then
+// llama_kv_cache_seq_shift(ctx, 0, k + d, n_past, -d), and continues at position n_past - d.
 #include "llama.h"
 
 #include <cstdio>
@@ -34,10 +38,19 @@ int main(int argc, char ** argv) {
     const int n_steps = (int)prompt.size() + n_gen;
     int32_t hdr[2] = { n_steps, n_vocab };
     fwrite(hdr, 4, 2, f);
+    const char * e_at = getenv("REF_SHIFT_AT");
+    const int shift_at = e_at ? atoi(e_at) : -1;
+    const int n_keep = getenv("REF_N_KEEP") ? atoi(getenv("REF_N_KEEP")) : 0, n_discard = getenv("REF_N_DISCARD") ? atoi(getenv("REF_N_DISCARD")) : 0;
     llama_token tok = prompt[0];
-    for (int s = 0; s < n_steps; ++s) {
+    int n_past = 0;
+    for (int s = 0; s < n_steps; ++s, ++n_past) {
         if (s < (int)prompt.size()) tok = prompt[s];
-        if (llama_decode(ctx, llama_batch_get_one(&tok, 1, s, 0)) != 0) { fprintf(stderr, "llama_decode failed at step %d\n", s); return 1; }
+        if (s == shift_at) {
+            llama_kv_cache_seq_rm(ctx, 0, n_keep, n_keep + n_discard);
+            llama_kv_cache_seq_shift(ctx, 0, n_keep + n_discard, n_past, -n_discard);
+            n_past -= n_discard;
+        }
+        if (llama_decode(ctx, llama_batch_get_one(&tok, 1, n_past, 0)) != 0) { fprintf(stderr, "llama_decode failed at step %d\n", s); return 1; }
         const float * lg = llama_get_logits(ctx);
         int best = 0;
         for (int i = 1; i < n_vocab; ++i) if (lg[i] > lg[best]) best = i;

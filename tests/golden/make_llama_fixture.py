@@ -25,6 +25,9 @@ BIN = os.path.join(ROOT, "oracle", "_ref", "ref_llama")
 CASES = {
     "llama_f16": dict(base="llama-tiny", vocab="ggml-vocab-llama.gguf", over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=4, n_head_kv=4, n_layer=2, n_vocab=32000, n_ctx=64, seed=21)),
     "llama_q4": dict(base="llama-tiny", vocab="ggml-vocab-llama.gguf", over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=4, n_head_kv=4, n_layer=2, n_vocab=32000, n_ctx=64, seed=22, wtype=synth.Q4_0)),
+    # the same models with a context shift before step 12 (llama_kv_cache_seq_rm + llama_kv_cache_seq_shift: K-shift, ring slots)
+    "llama_f16_shift": dict(base="llama-tiny", vocab="ggml-vocab-llama.gguf", shift=(12, 2, 4), n_gen=14, over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=4, n_head_kv=4, n_layer=2, n_vocab=32000, n_ctx=64, seed=21)),
+    "falcon_f16_shift": dict(base="falcon-tiny", vocab="ggml-vocab-falcon.gguf", shift=(12, 2, 4), n_gen=14, over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=8, n_head_kv=2, n_layer=2, n_vocab=65024, n_ctx=64, seed=23)),
     "falcon_f16": dict(base="falcon-tiny", vocab="ggml-vocab-falcon.gguf", over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=8, n_head_kv=2, n_layer=2, n_vocab=65024, n_ctx=64, seed=23)),
 }
 
@@ -53,12 +56,16 @@ def main():
         tok_kv = {k: v for k, v in vkv.items() if k.startswith("tokenizer.")}
         assert len(tok_kv["tokenizer.ggml.tokens"][1][1]) == hp.n_vocab
         prompt = np.random.default_rng(hp.seed).integers(0, hp.n_vocab, 6)
-        n_gen = 10
+        n_gen = c.get("n_gen", 10)
+        env = dict(os.environ)
+        shift = c.get("shift")
+        if shift:
+            env.update(REF_SHIFT_AT=str(shift[0]), REF_N_KEEP=str(shift[1]), REF_N_DISCARD=str(shift[2]))
         with tempfile.TemporaryDirectory() as td:
             path, out = os.path.join(td, "m.powerinfer.gguf"), os.path.join(td, "out.bin")
             gguf.write_model(path, model, tok_kv)
             subprocess.check_call([BIN, path, str(hp.n_ctx), "1", str(n_gen), out] + [str(int(t)) for t in prompt],
-                                  stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL)
+                                  stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL, env=env)
             raw = np.fromfile(out, np.uint8)
         n_steps, n_vocab = raw[:8].view(np.int32)
         rec = raw[8:].reshape(n_steps, 8 + 4 * n_vocab)
@@ -68,7 +75,7 @@ def main():
         sample = np.sort(np.random.default_rng(1).choice(n_vocab, 1024, replace=False)).astype(np.int32)
         np.savez_compressed(os.path.join(HERE, f"ref_{name}.npz"), prompt=prompt.astype(np.int32), consumed=consumed, greedy=greedy,
                             sample_idx=sample, logits_sample=logits[:, sample], logits_max=logits.max(1), logits_absmax=np.abs(logits).max(1),
-                            model_sha=model_sha(model))
+                            model_sha=model_sha(model), shift=np.asarray(shift if shift else (-1, 0, 0), np.int32))
         print(name, "greedy", greedy.tolist())
 
 

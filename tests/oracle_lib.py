@@ -67,6 +67,7 @@ def oracle():
         L.pio_model_set_capture.argtypes = [_vp, _vp, _vp, _vp]
         L.pio_model_eval.argtypes = [_vp, _vp, _vp, _vp, _i, _i, _vp, _i, _vp, _i]
         L.pio_model_eval_simple.argtypes = [_vp, _vp, _i, _i, _vp, _i]
+        L.pio_model_k_shift.argtypes = [_vp, _vp]
         _oracle = L
     return _oracle
 
@@ -130,6 +131,80 @@ def ffn_sparse(lib, d, ff, r, T, wtype, has_gate, up, gate, down_t, fc1, fc2, x_
 
 
 # ---------------------------------------------------------------------------------------------
+# the reference's KV cell bookkeeping (llama.cpp:1381-1850), for one context
+# ---------------------------------------------------------------------------------------------
+class KVCells:
+    """pos / delta / sequence sets per cell and the ring-buffer slot search, as llama_kv_cache does it."""
+
+    def __init__(self, n_ctx):
+        self.size, self.head, self.has_shift = n_ctx, 0, False
+        self.pos = np.full(n_ctx, -1, np.int64)
+        self.delta = np.zeros(n_ctx, np.int64)
+        self.seq = [set() for _ in range(n_ctx)]
+
+    def find_slot(self, positions, seq_id=0):          # llama_kv_cache_find_slot, llama.cpp:1683-1736
+        n, tested = len(positions), 0
+        while True:
+            if self.head + n > self.size:
+                tested += self.size - self.head
+                self.head = 0
+                continue
+            busy = [i for i in range(n) if self.pos[self.head + i] >= 0]
+            if not busy:
+                break
+            self.head += busy[0] + 1
+            tested += busy[0] + 1
+            if tested >= self.size:
+                raise RuntimeError("no KV slot")
+        for i, p in enumerate(positions):
+            self.pos[self.head + i] = p
+            self.seq[self.head + i].add(seq_id)
+        return self.head
+
+    def cell_max(self):                                 # llama_kv_cache_cell_max, llama.cpp:1739-1747
+        for i in range(self.size - 1, 0, -1):
+            if self.pos[i] >= 0 and self.seq[i]:
+                return i + 1
+        return 0
+
+    def seq_rm(self, seq_id, p0, p1):                   # llama_kv_cache_seq_rm, llama.cpp:1757-1785
+        new_head = self.size
+        p0 = max(p0, 0)
+        p1 = np.iinfo(np.int32).max if p1 < 0 else p1
+        for i in range(self.size):
+            if p0 <= self.pos[i] < p1 and (seq_id < 0 or seq_id in self.seq[i]):
+                self.seq[i] = set() if seq_id < 0 else self.seq[i] - {seq_id}
+                if not self.seq[i]:
+                    self.pos[i] = -1
+                    new_head = min(new_head, i)
+        if new_head != self.size:
+            self.head = new_head
+
+    def seq_shift(self, seq_id, p0, p1, d):             # llama_kv_cache_seq_shift, llama.cpp:1819-1848
+        new_head = self.size
+        p0 = max(p0, 0)
+        p1 = np.iinfo(np.int32).max if p1 < 0 else p1
+        for i in range(self.size):
+            if seq_id in self.seq[i] and p0 <= self.pos[i] < p1:
+                self.has_shift = True
+                self.pos[i] += d
+                self.delta[i] += d
+                if self.pos[i] < 0:
+                    self.pos[i] = -1
+                    self.seq[i] = set()
+                    new_head = min(new_head, i)
+        self.head = new_head if new_head != self.size else 0
+
+    def mask(self, positions, n_kv, seq_id=0):          # KQ_mask, llama.cpp:6506-6531
+        m = np.zeros((len(positions), n_kv), np.float32)
+        for j, p in enumerate(positions):
+            for i in range(n_kv):
+                if seq_id not in self.seq[i] or self.pos[i] > p:
+                    m[j, i] = -np.inf
+        return m
+
+
+# ---------------------------------------------------------------------------------------------
 # whole-model oracle driven from the dict powerinfer_amd.synth.make_model returns
 # ---------------------------------------------------------------------------------------------
 class HParamsC(C.Structure):
@@ -181,6 +256,21 @@ class OracleModel:
         tok = self.O.pio_model_eval_simple(self.h, _ptr(tokens), tokens.size, n_past, _ptr(logits), nth)
         assert tok >= 0
         return tok, logits
+
+    def eval_cells(self, tokens, pos, slots, n_kv, mask):
+        """General form (pio_model_eval): tokens[T] at positions pos[T] stored in cache cells slots[T]; n_kv cells attended
+        under mask [T][n_kv] (0 / -inf).  Returns (greedy token of the last position, its logits)."""
+        tokens, pos, slots = (np.ascontiguousarray(a, np.int32) for a in (tokens, pos, slots))
+        mask = np.ascontiguousarray(mask, np.float32)
+        logits = np.zeros(self.hp.n_vocab, np.float32)
+        rc = self.O.pio_model_eval(self.h, _ptr(tokens), _ptr(pos), _ptr(slots), tokens.size, int(n_kv), _ptr(mask), 0, _ptr(logits), 1)
+        assert rc == 0
+        return int(np.argmax(logits)), logits
+
+    def k_shift(self, delta):
+        delta = np.ascontiguousarray(delta, np.int32)
+        assert delta.size == self.hp.n_ctx
+        assert self.O.pio_model_k_shift(self.h, _ptr(delta)) == 0
 
     def close(self):
         if self.h:

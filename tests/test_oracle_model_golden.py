@@ -32,3 +32,38 @@ def test_model_eval_matches_reference_llama_cpp(name):
     # same arithmetic, same order (single thread): agreement at fp32 round-off
     assert worst < 1e-5, worst
     om.close()
+
+
+@pytest.mark.parametrize("name", ["llama_f16_shift", "falcon_f16_shift"])
+def test_context_shift_matches_reference_llama_cpp(name):
+    """KV ring slots, cell mask and K-shift: before step 12 the reference removed positions [2, 6) and shifted the later cells by
+    -4 (llama_kv_cache_seq_rm + llama_kv_cache_seq_shift); the next llama_decode rotated the cached K rows (llm_build_k_shift)
+    and stored new tokens in the freed cells.  The oracle repeats that with the reference's cell bookkeeping."""
+    g = dict(np.load(os.path.join(ROOT, "tests", "golden", f"ref_{name}.npz")))
+    hp, model = fx.case_model(name)
+    if not np.array_equal(fx.model_sha(model), g["model_sha"]):
+        pytest.skip("numpy generates a different stream here than where the fixture was written")
+    shift_at, n_keep, n_discard = (int(v) for v in g["shift"])
+    om = ol.OracleModel(model)
+    cells = ol.KVCells(hp.n_ctx)
+    n_past, worst = 0, 0.0
+    for s, tok in enumerate(g["consumed"]):
+        if s == shift_at:
+            cells.seq_rm(0, n_keep, n_keep + n_discard)
+            cells.seq_shift(0, n_keep + n_discard, n_past, -n_discard)
+            n_past -= n_discard
+        if cells.has_shift:                              # llama_decode_internal applies pending shifts first (llama.cpp:5494-5500, 6921-6929)
+            om.k_shift(cells.delta)
+            cells.has_shift = False
+            cells.delta[:] = 0
+        slot = cells.find_slot([n_past])
+        n_kv = min(hp.n_ctx, max(32, cells.cell_max()))                      # llama.cpp:6842
+        best, lg = om.eval_cells([int(tok)], [n_past], [slot], n_kv, cells.mask([n_past], n_kv))
+        if s == shift_at:
+            assert slot == n_keep and slot != n_past     # the ring reuses the freed cells
+        err = np.abs(lg[g["sample_idx"]] - g["logits_sample"][s]).max() / g["logits_absmax"][s]
+        worst = max(worst, float(err))
+        assert best == g["greedy"][s], (s, best, g["greedy"][s])
+        n_past += 1
+    assert worst < 1e-5, worst
+    om.close()

@@ -182,6 +182,12 @@ PI_API int pi_k_axpy_q4_partials(const void * down_t_q4, int cols, int ff, const
                                  const uint32_t * hot_words, const int32_t * hot_prefix, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_axpy_q4_reduce(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out,
                                int32_t * n_active, pi_workspace * ws, pi_stream_t stream);
+/* KV cache maintenance.  pi_k_k_shift replaces the graph of llm_build_k_shift (llama.cpp:4332-4381; the fp16 RoPE
+ * ggml.c:11327-11478): cache [rows = layers x kv heads][n_ctx][hd] fp16, delta[n_cells] positions to rotate each cell by.
+ * pi_k_kv_compact moves cell map[j] to cell j (map ascending) through `stage` ([rows][n_new][hd] fp16): this implementation keeps
+ * the live cells contiguous instead of searching a ring for free slots (llama_kv_cache_find_slot, llama.cpp:1683-1736). */
+PI_API int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float theta_scale, const int32_t * delta, int n_cells, pi_stream_t stream);
+PI_API int pi_k_kv_compact(void * cache, void * stage, int rows, int n_ctx, int hd, const int32_t * map, int n_new, pi_stream_t stream);
 PI_API int pi_k_sparse_ffn_supported(int ff, int r, int cols);
 /* the two launches of pi_k_sparse_ffn on their own, for callers that overlap the block with an independent branch (Falcon's
  * attention reads the same layer input): _partials may run on another stream, _reduce needs it and the residual operands done */
@@ -321,6 +327,16 @@ PI_API int pi_model_set_tensor(pi_model * m, int layer, int kind, int type, cons
                                int64_t ne0, int64_t ne1, int on_device);
 PI_API int pi_model_finalize(pi_model * m);
 PI_API int pi_model_kv_clear(pi_model * m);                    /* llama_kv_cache_clear, llama.h:367 */
+/*
+ * llama_kv_cache_seq_rm / llama_kv_cache_seq_shift for the model's own sequence (llama.cpp:1757-1785, 1819-1848; p1 < 0 means
+ * "to the end").  Removed cells are squeezed out at once and shifted cells get their K rows rotated at once (the reference marks
+ * the cells and applies the rotation inside the next llama_decode, llama.cpp:5494-5500).  Decoding needs the cells' positions to
+ * be 0 .. n-1 again (what the context shift of examples/main does: remove [keep, keep+discard), shift the rest by -discard);
+ * pi_model_decode / pi_model_generate report PI_E_STATE while a gap is open.  After an edit that leaves contiguous positions the
+ * next position is n (pi_model_generate continues there; pi_model_decode takes n_past = n).  Both return n or a negative error.
+ */
+PI_API int pi_model_kv_seq_rm(pi_model * m, int p0, int p1);
+PI_API int pi_model_kv_seq_shift(pi_model * m, int p0, int p1, int delta);
 
 /*
  * llama_decode (llama.cpp:10672) for one sequence: evaluates tokens[0..n_tokens) at positions

@@ -5,6 +5,7 @@
 // ~40-node-per-layer graph every token, llama.cpp:6408, 6922).
 #include "runtime.hpp"
 #include "cold_path.hpp"
+#include <limits.h>
 #include "engine_internal.hpp"
 #include "../../include/powerinfer_hip.h"
 
@@ -505,11 +506,83 @@ int pi_model_kv_clear(pi_model * m) {
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
     PI_TRY(pi_memset(m->k_cache, 0, kv * 2));
     PI_TRY(pi_memset(m->v_cache, 0, kv * 2));
+    m->kv_pos.clear();
+    PI_TRY(pi_memset(m->d_pos, 0, 4));
     return PI_OK;
+}
+
+namespace {
+// One edit of the model's own sequence: cells whose position lies in [p0, p1) are dropped (delta == 0 and !shift) or moved by
+// delta positions (dropped if that takes them below 0).  Returns the number of live cells, or a negative error.
+int kv_edit(pi_model * m, int p0, int p1, int delta, bool shift) {
+    const pi_hparams & hp = m->hp;
+    hipStream_t st = m->stream;
+    PI_HIP_TRY(hipStreamSynchronize(st));
+    if (m->kv_pos.empty()) {
+        int32_t n = 0;
+        PI_TRY(pi_memcpy_d2h(&n, m->d_pos, 4));
+        if (n < 0 || n > hp.n_ctx) return pi::fail(PI_E_STATE, "KV edit: the device position is out of range");
+        m->kv_pos.resize(n);
+        for (int i = 0; i < n; ++i) m->kv_pos[i] = i;
+    }
+    if (p0 < 0) p0 = 0;
+    if (p1 < 0) p1 = INT32_MAX;
+    const int n_old = (int)m->kv_pos.size();
+    std::vector<int32_t> dl(n_old ? n_old : 1, 0), map, pos;
+    bool any_shift = false;
+    for (int i = 0; i < n_old; ++i) {
+        int p = m->kv_pos[i];
+        if (p >= p0 && p < p1) {
+            if (!shift) continue;                     // removed
+            p += delta;
+            if (p < 0) continue;                      // shifted out (llama.cpp:1836-1840)
+            dl[i] = delta; any_shift = any_shift || delta != 0;
+        }
+        map.push_back(i); pos.push_back(p);
+    }
+    const int n_new = (int)map.size();
+    const int rows = hp.n_layer * hp.n_head_kv;
+    if (!m->kv_map) { m->kv_map = m->alloc<int32_t>(hp.n_ctx); if (!m->kv_map) return PI_E_HIP; }
+    if (any_shift) {
+        PI_TRY(pi_memcpy_h2d(m->kv_map, dl.data(), sizeof(int32_t) * n_old));
+        PI_TRY(pi_k_k_shift(m->k_cache, rows, hp.n_ctx, m->hd, hp.arch == PI_ARCH_FALCON ? 2 : 0, m->theta_scale, m->kv_map, n_old, st));
+        PI_HIP_TRY(hipStreamSynchronize(st));
+    }
+    bool moved = false;
+    for (int j = 0; j < n_new; ++j) moved = moved || map[j] != j;
+    if (moved) {
+        if (!m->kv_stage) { m->kv_stage = m->alloc<__half>((size_t)rows * hp.n_ctx * m->hd); if (!m->kv_stage) return PI_E_HIP; }
+        PI_TRY(pi_memcpy_h2d(m->kv_map, map.data(), sizeof(int32_t) * n_new));
+        PI_TRY(pi_k_kv_compact(m->k_cache, m->kv_stage, rows, hp.n_ctx, m->hd, m->kv_map, n_new, st));
+        PI_TRY(pi_k_kv_compact(m->v_cache, m->kv_stage, rows, hp.n_ctx, m->hd, m->kv_map, n_new, st));
+        PI_HIP_TRY(hipStreamSynchronize(st));
+    }
+    bool identity = true;
+    for (int j = 0; j < n_new; ++j) identity = identity && pos[j] == j;
+    if (identity) {
+        m->kv_pos.clear();
+        const int32_t n = n_new;
+        PI_TRY(pi_memcpy_h2d(m->d_pos, &n, 4));       // generation continues at position n
+    } else {
+        m->kv_pos = pos;
+    }
+    return n_new;
+}
+}  // namespace
+
+int pi_model_kv_seq_rm(pi_model * m, int p0, int p1) {
+    if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_kv_seq_rm: model not finalized");
+    return kv_edit(m, p0, p1, 0, false);
+}
+
+int pi_model_kv_seq_shift(pi_model * m, int p0, int p1, int delta) {
+    if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_kv_seq_shift: model not finalized");
+    return kv_edit(m, p0, p1, delta, true);
 }
 
 int pi_model_decode(pi_model * m, const int32_t * tokens, int n_tokens, int n_past, float * logits_out) {
     if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_decode: model not finalized");
+    if (!m->kv_pos.empty()) return pi::fail(PI_E_STATE, "pi_model_decode: the KV cells' positions are not contiguous (shift the cells behind a removed range first)");
     if (!tokens || n_tokens <= 0 || n_past < 0 || n_past + n_tokens > m->hp.n_ctx) return pi::fail(PI_E_ARG, "pi_model_decode: token range exceeds the context");
     for (int i = 0; i < n_tokens; ++i)
         if (tokens[i] < 0 || tokens[i] >= m->hp.n_vocab) return pi::fail(PI_E_ARG, "pi_model_decode: token id out of range");
@@ -542,6 +615,7 @@ int pi_model_decode(pi_model * m, const int32_t * tokens, int n_tokens, int n_pa
 int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * ms_out) {
     if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_generate: model not finalized");
     if (n_steps <= 0 || n_steps > m->max_steps || !out_tokens) return pi::fail(PI_E_ARG, "pi_model_generate: bad step count");
+    if (!m->kv_pos.empty()) return pi::fail(PI_E_STATE, "pi_model_generate: the KV cells' positions are not contiguous (shift the cells behind a removed range first)");
     int32_t pos = 0;
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
     PI_TRY(pi_memcpy_d2h(&pos, m->d_pos, 4));

@@ -47,6 +47,9 @@ struct pi_model {
     bool capture = false;
     float *cap_ffn = nullptr, *cap_logits = nullptr, *cap_src = nullptr;       // device
     pi::ColdPath * cold = nullptr;
+    std::vector<int32_t> kv_pos;          // positions of the cache cells while an edit left them non-contiguous; empty: cell i holds position i
+    __half * kv_stage = nullptr;          // [n_layer * n_head_kv][n_ctx][hd] staging for cell compaction, allocated at the first edit
+    int32_t * kv_map = nullptr;           // [n_ctx] device copy of the cell map / deltas of an edit
     std::vector<uint32_t *> hot_words;    // per hybrid layer: bit j of word g set iff neuron 32g+j is GPU-resident (device)
     std::vector<int32_t *> hot_prefix;    //                   GPU-resident neurons before group g = row of the compact matrices
     BatchState * batch = nullptr;         // per-sequence caches and step buffers of batched decoding

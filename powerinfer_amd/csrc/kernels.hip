@@ -2059,6 +2059,43 @@ __global__ __launch_bounds__(kBlock) void h_q8_gather_kernel(const float * __res
 }
 
 // ---------------------------------------------------------------------------------------------------
+// K-shift (llm_build_k_shift, llama.cpp:4332-4381): cached K rows whose position changed by delta[cell] are rotated in place
+// by that many positions, the RoPE of fp16 data (ggml_compute_forward_rope_f16, ggml.c:11327-11478): fp16 -> fp32, angle
+// delta * theta_i with theta advanced by repeated fp32 multiplication, back to fp16.  Cache layout [row][n_ctx][hd] with
+// row = (layer, kv head).  grid = (cells, rows), hd/2 threads; cells with delta 0 are left alone (the reference rotates them
+// by angle 0, which returns the same bits).
+// ---------------------------------------------------------------------------------------------------
+__global__ void k_shift_kernel(__half * __restrict__ k_cache, int n_ctx, int hd, int mode, float theta_scale,
+                               const int32_t * __restrict__ delta) {
+    const int cell = blockIdx.x, i = threadIdx.x;
+    const int dl = delta[cell];
+    if (dl == 0) return;
+    __half * row = k_cache + ((size_t)blockIdx.y * n_ctx + cell) * hd;
+    float theta = (float)dl;
+    for (int j = 0; j < i; ++j) theta = __fmul_rn(theta, theta_scale);
+    const float c = cosf(theta), sn = sinf(theta);
+    const int i0 = (mode & 2) ? i : 2 * i;
+    const int i1 = (mode & 2) ? i + hd / 2 : 2 * i + 1;
+    const float x0 = __half2float(row[i0]), x1 = __half2float(row[i1]);
+    row[i0] = __float2half_rn(__fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, sn)));
+    row[i1] = __float2half_rn(__fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, c)));
+}
+
+// Cell compaction of one cache (K or V) after cells were removed: new cell j takes old cell map[j] (map ascending, so the cells
+// keep their order).  Two launches through a staging buffer [rows][n_new][hd] because source and destination ranges overlap.
+// grid = (n_new, rows), hd/8 threads (16 bytes each).
+__global__ void kv_gather_kernel(const __half * __restrict__ cache, __half * __restrict__ stage, const int32_t * __restrict__ map, int n_new, int n_ctx, int hd) {
+    const pi_u32x4 * src = reinterpret_cast<const pi_u32x4 *>(cache + ((size_t)blockIdx.y * n_ctx + map[blockIdx.x]) * hd);
+    pi_u32x4 * dst = reinterpret_cast<pi_u32x4 *>(stage + ((size_t)blockIdx.y * n_new + blockIdx.x) * hd);
+    dst[threadIdx.x] = src[threadIdx.x];
+}
+__global__ void kv_place_kernel(__half * __restrict__ cache, const __half * __restrict__ stage, int n_new, int n_ctx, int hd) {
+    const pi_u32x4 * src = reinterpret_cast<const pi_u32x4 *>(stage + ((size_t)blockIdx.y * n_new + blockIdx.x) * hd);
+    pi_u32x4 * dst = reinterpret_cast<pi_u32x4 *>(cache + ((size_t)blockIdx.y * n_ctx + blockIdx.x) * hd);
+    dst[threadIdx.x] = src[threadIdx.x];
+}
+
+// ---------------------------------------------------------------------------------------------------
 // RoPE + KV store for one token (ggml.c:11163-11325; theta advanced by repeated fp32 multiplication as
 // the CPU path does, so the angle is bit-identical and only cosf/sinf may differ in the last place).
 // grid = n_head + 2*n_head_kv blocks of hd/2 threads.
@@ -3423,6 +3460,23 @@ int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_
     hipLaunchKernelGGL(attn_decode_kernel, dim3(n_head, T), dim3(kBlock), sh, st,
                        q_rot, (const __half *)k_cache, (const __half *)v_cache, n_head, n_head_kv, hd, n_ctx, pos, out, n_head * hd, out_stride, (__half *)out_f16);
     return pi::check_launch("pi_k_attn_chunk");
+}
+
+int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float theta_scale, const int32_t * delta, int n_cells, pi_stream_t stream) {
+    if (!k_cache || !delta || rows <= 0 || n_ctx <= 0 || hd <= 0 || hd % 2 || hd / 2 > 1024 || n_cells < 0 || n_cells > n_ctx || (mode != 0 && mode != 2))
+        return pi::fail(PI_E_ARG, "pi_k_k_shift: bad arguments");
+    if (n_cells == 0) return PI_OK;
+    hipLaunchKernelGGL(k_shift_kernel, dim3(n_cells, rows), dim3(hd / 2), 0, (hipStream_t)stream, (__half *)k_cache, n_ctx, hd, mode, theta_scale, delta);
+    return pi::check_launch("pi_k_k_shift");
+}
+
+int pi_k_kv_compact(void * cache, void * stage, int rows, int n_ctx, int hd, const int32_t * map, int n_new, pi_stream_t stream) {
+    if (!cache || !stage || !map || rows <= 0 || n_ctx <= 0 || hd <= 0 || hd % 8 || hd / 8 > 1024 || n_new < 0 || n_new > n_ctx)
+        return pi::fail(PI_E_ARG, "pi_k_kv_compact: bad arguments");
+    if (n_new == 0) return PI_OK;
+    hipLaunchKernelGGL(kv_gather_kernel, dim3(n_new, rows), dim3(hd / 8), 0, (hipStream_t)stream, (const __half *)cache, (__half *)stage, map, n_new, n_ctx, hd);
+    hipLaunchKernelGGL(kv_place_kernel, dim3(n_new, rows), dim3(hd / 8), 0, (hipStream_t)stream, (__half *)cache, (const __half *)stage, n_new, n_ctx, hd);
+    return pi::check_launch("pi_k_kv_compact");
 }
 
 int pi_k_step_advance(int32_t * step, pi_stream_t stream) {

@@ -31,6 +31,8 @@ def _declare(L):
     L.pi_model_set_tensor.restype, L.pi_model_set_tensor.argtypes = i, [vp, i, i, i, vp, C.c_int64, C.c_int64, i]
     L.pi_model_finalize.restype, L.pi_model_finalize.argtypes = i, [vp]
     L.pi_model_kv_clear.restype, L.pi_model_kv_clear.argtypes = i, [vp]
+    L.pi_model_kv_seq_rm.restype, L.pi_model_kv_seq_rm.argtypes = i, [vp, i, i]
+    L.pi_model_kv_seq_shift.restype, L.pi_model_kv_seq_shift.argtypes = i, [vp, i, i, i]
     L.pi_model_decode.restype, L.pi_model_decode.argtypes = i, [vp, vp, i, i, vp]
     L.pi_model_generate.restype, L.pi_model_generate.argtypes = i, [vp, i, vp, C.POINTER(C.c_float)]
     L.pi_model_set_capture.restype, L.pi_model_set_capture.argtypes = i, [vp, i]
@@ -44,6 +46,7 @@ def _declare(L):
 
 
 ENGINE_SYMBOLS = ["pi_model_create", "pi_model_free", "pi_model_set_tensor", "pi_model_finalize", "pi_model_kv_clear",
+                  "pi_model_kv_seq_rm", "pi_model_kv_seq_shift",
                   "pi_model_decode", "pi_model_generate", "pi_model_set_capture", "pi_model_get_capture",
                   "pi_model_step_active", "pi_model_time_section",
                   "pi_model_batch_init", "pi_model_batch_decode", "pi_model_batch_generate", "pi_model_batch_union"]
@@ -107,6 +110,18 @@ class Model:
 
     def kv_clear(self):
         check(self.L.pi_model_kv_clear(self.h), "pi_model_kv_clear")
+
+    def kv_seq_rm(self, p0, p1):
+        """llama_kv_cache_seq_rm for the model's own sequence; returns the number of live cells."""
+        n = self.L.pi_model_kv_seq_rm(self.h, p0, p1)
+        check(min(n, 0), "pi_model_kv_seq_rm")
+        return n
+
+    def kv_seq_shift(self, p0, p1, delta):
+        """llama_kv_cache_seq_shift (positions in [p0, p1) move by delta, their K rows are rotated); returns the live cells."""
+        n = self.L.pi_model_kv_seq_shift(self.h, p0, p1, delta)
+        check(min(n, 0), "pi_model_kv_seq_shift")
+        return n
 
     def decode(self, tokens, n_past, want_logits=True):
         tokens = np.ascontiguousarray(tokens, np.int32)

@@ -164,3 +164,45 @@ def test_embed_and_argmax():
     pl.check(L.pi_k_argmax(dl.ptr, 32000, dtok.ptr, None), "argmax")
     pl.sync()
     assert dtok.download(np.int32)[0] == 123 == int(np.argmax(lg))
+
+
+@pytest.mark.parametrize("mode", [0, 2])
+def test_k_shift_and_compaction(mode):
+    """pi_k_k_shift against the fp16 RoPE of the reference's K-shift restated in numpy (ggml.c:11327-11478: fp16 in, fp32
+    rotation with theta advanced by repeated multiplication, fp16 out), and pi_k_kv_compact against a gather."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    rows, n_ctx, hd, n_cells = 6, 40, 64, 33
+    rng = np.random.default_rng(11)
+    k = rng.standard_normal((rows, n_ctx, hd)).astype(np.float16)
+    delta = rng.integers(-9, 10, n_cells).astype(np.int32)
+    delta[::4] = 0
+    theta_scale = np.float32(10000.0) ** np.float32(-2.0 / hd)
+    want = k.copy()
+    for c in range(n_cells):
+        if delta[c] == 0:
+            continue
+        th = np.float32(delta[c])
+        for i in range(hd // 2):
+            cs, sn = np.float32(np.cos(th)), np.float32(np.sin(th))
+            i0, i1 = (i, i + hd // 2) if mode == 2 else (2 * i, 2 * i + 1)
+            x0, x1 = k[:, c, i0].astype(np.float32), k[:, c, i1].astype(np.float32)
+            want[:, c, i0] = (x0 * cs - x1 * sn).astype(np.float16)
+            want[:, c, i1] = (x0 * sn + x1 * cs).astype(np.float16)
+            th = np.float32(th * theta_scale)
+    kd, dd = pl.DevBuf(host=k), pl.DevBuf(host=delta)
+    pl.check(L.pi_k_k_shift(kd.ptr, rows, n_ctx, hd, mode, float(theta_scale), dd.ptr, n_cells, None), "k_shift")
+    pl.sync()
+    got = kd.download(np.float16).reshape(rows, n_ctx, hd)
+    assert np.array_equal(got[:, n_cells:], k[:, n_cells:])                       # cells beyond the live range untouched
+    assert np.array_equal(got[:, :n_cells][:, delta == 0], k[:, :n_cells][:, delta == 0])
+    diff = np.abs(got.astype(np.float32) - want.astype(np.float32))
+    assert diff.max() <= 2e-3 * np.abs(want.astype(np.float32)).max()             # cosf/sinf of the device vs numpy: a last-place fp16 step
+    assert (got != want).mean() < 0.02
+    # compaction: drop cells 3..8 and 20
+    keep = np.array([c for c in range(n_cells) if not (3 <= c < 9 or c == 20)], np.int32)
+    stage, md = pl.DevBuf(rows * n_ctx * hd * 2), pl.DevBuf(host=keep)
+    pl.check(L.pi_k_kv_compact(kd.ptr, stage.ptr, rows, n_ctx, hd, md.ptr, keep.size, None), "kv_compact")
+    pl.sync()
+    after = kd.download(np.float16).reshape(rows, n_ctx, hd)
+    assert np.array_equal(after[:, :keep.size], got[:, keep])

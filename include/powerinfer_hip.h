@@ -368,6 +368,12 @@ PI_API int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, fl
 PI_API int pi_model_batch_init(pi_model * m, int n_seq);
 PI_API int pi_model_batch_decode(pi_model * m, const int32_t * tokens, const int32_t * positions, int32_t * next_tokens, float * logits_out);
 PI_API int pi_model_batch_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * ms_out);
+/* llama_kv_cache_seq_rm / _seq_shift / _seq_cp (llama.cpp:1757-1848) for sequence `seq` of the batch, with the semantics of
+ * pi_model_kv_seq_rm / _shift.  Sequences own their caches, so _cp copies cells [p0, p1) of src into dst, which must hold exactly
+ * p0 cells (a prompt prefix evaluated once and handed to the other sequences); returns dst's cell count. */
+PI_API int pi_model_batch_kv_seq_rm(pi_model * m, int seq, int p0, int p1);
+PI_API int pi_model_batch_kv_seq_shift(pi_model * m, int seq, int p0, int p1, int delta);
+PI_API int pi_model_batch_kv_seq_cp(pi_model * m, int src, int dst, int p0, int p1);
 PI_API int pi_model_batch_union(pi_model * m, int32_t * n_union_per_layer);   /* union sizes of the last step, [n_layer] */
 
 PI_API int pi_model_set_capture(pi_model * m, int enable);

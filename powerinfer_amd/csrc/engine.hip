@@ -300,6 +300,66 @@ int add_vec(float * y, const float * a, int n, hipStream_t st) {
 }
 }  // namespace pi
 
+namespace pi {
+// One edit of a sequence's cache (k, v: [n_layer * n_head_kv][n_ctx][hd]; d_pos: the device word holding its next position;
+// kv_pos: the cells' positions while they are not 0 .. n-1): cells whose position lies in [p0, p1) are dropped (!shift) or moved
+// by delta positions (dropped if that takes them below 0).  Returns the number of live cells, or a negative error.
+int kv_edit(pi_model * m, __half * k_cache, __half * v_cache, int32_t * d_pos, std::vector<int32_t> & kv_pos, int p0, int p1, int delta, bool shift) {
+    const pi_hparams & hp = m->hp;
+    hipStream_t st = m->stream;
+    PI_HIP_TRY(hipStreamSynchronize(st));
+    if (kv_pos.empty()) {
+        int32_t n = 0;
+        PI_TRY(pi_memcpy_d2h(&n, d_pos, 4));
+        if (n < 0 || n > hp.n_ctx) return pi::fail(PI_E_STATE, "KV edit: the device position is out of range");
+        kv_pos.resize(n);
+        for (int i = 0; i < n; ++i) kv_pos[i] = i;
+    }
+    if (p0 < 0) p0 = 0;
+    if (p1 < 0) p1 = INT32_MAX;
+    const int n_old = (int)kv_pos.size();
+    std::vector<int32_t> dl(n_old ? n_old : 1, 0), map, pos;
+    bool any_shift = false;
+    for (int i = 0; i < n_old; ++i) {
+        int p = kv_pos[i];
+        if (p >= p0 && p < p1) {
+            if (!shift) continue;                     // removed
+            p += delta;
+            if (p < 0) continue;                      // shifted out (llama.cpp:1836-1840)
+            dl[i] = delta; any_shift = any_shift || delta != 0;
+        }
+        map.push_back(i); pos.push_back(p);
+    }
+    const int n_new = (int)map.size();
+    const int rows = hp.n_layer * hp.n_head_kv;
+    if (!m->kv_map) { m->kv_map = m->alloc<int32_t>(hp.n_ctx); if (!m->kv_map) return PI_E_HIP; }
+    if (any_shift) {
+        PI_TRY(pi_memcpy_h2d(m->kv_map, dl.data(), sizeof(int32_t) * n_old));
+        PI_TRY(pi_k_k_shift(k_cache, rows, hp.n_ctx, m->hd, hp.arch == PI_ARCH_FALCON ? 2 : 0, m->theta_scale, m->kv_map, n_old, st));
+        PI_HIP_TRY(hipStreamSynchronize(st));
+    }
+    bool moved = false;
+    for (int j = 0; j < n_new; ++j) moved = moved || map[j] != j;
+    if (moved) {
+        if (!m->kv_stage) { m->kv_stage = m->alloc<__half>((size_t)rows * hp.n_ctx * m->hd); if (!m->kv_stage) return PI_E_HIP; }
+        PI_TRY(pi_memcpy_h2d(m->kv_map, map.data(), sizeof(int32_t) * n_new));
+        PI_TRY(pi_k_kv_compact(k_cache, m->kv_stage, rows, hp.n_ctx, m->hd, m->kv_map, n_new, st));
+        PI_TRY(pi_k_kv_compact(v_cache, m->kv_stage, rows, hp.n_ctx, m->hd, m->kv_map, n_new, st));
+        PI_HIP_TRY(hipStreamSynchronize(st));
+    }
+    bool identity = true;
+    for (int j = 0; j < n_new; ++j) identity = identity && pos[j] == j;
+    if (identity) {
+        kv_pos.clear();
+        const int32_t n = n_new;
+        PI_TRY(pi_memcpy_h2d(d_pos, &n, 4));          // generation continues at position n
+    } else {
+        kv_pos = pos;
+    }
+    return n_new;
+}
+}  // namespace pi
+
 extern "C" {
 
 pi_model * pi_model_create(const pi_hparams * hp) {
@@ -511,73 +571,14 @@ int pi_model_kv_clear(pi_model * m) {
     return PI_OK;
 }
 
-namespace {
-// One edit of the model's own sequence: cells whose position lies in [p0, p1) are dropped (delta == 0 and !shift) or moved by
-// delta positions (dropped if that takes them below 0).  Returns the number of live cells, or a negative error.
-int kv_edit(pi_model * m, int p0, int p1, int delta, bool shift) {
-    const pi_hparams & hp = m->hp;
-    hipStream_t st = m->stream;
-    PI_HIP_TRY(hipStreamSynchronize(st));
-    if (m->kv_pos.empty()) {
-        int32_t n = 0;
-        PI_TRY(pi_memcpy_d2h(&n, m->d_pos, 4));
-        if (n < 0 || n > hp.n_ctx) return pi::fail(PI_E_STATE, "KV edit: the device position is out of range");
-        m->kv_pos.resize(n);
-        for (int i = 0; i < n; ++i) m->kv_pos[i] = i;
-    }
-    if (p0 < 0) p0 = 0;
-    if (p1 < 0) p1 = INT32_MAX;
-    const int n_old = (int)m->kv_pos.size();
-    std::vector<int32_t> dl(n_old ? n_old : 1, 0), map, pos;
-    bool any_shift = false;
-    for (int i = 0; i < n_old; ++i) {
-        int p = m->kv_pos[i];
-        if (p >= p0 && p < p1) {
-            if (!shift) continue;                     // removed
-            p += delta;
-            if (p < 0) continue;                      // shifted out (llama.cpp:1836-1840)
-            dl[i] = delta; any_shift = any_shift || delta != 0;
-        }
-        map.push_back(i); pos.push_back(p);
-    }
-    const int n_new = (int)map.size();
-    const int rows = hp.n_layer * hp.n_head_kv;
-    if (!m->kv_map) { m->kv_map = m->alloc<int32_t>(hp.n_ctx); if (!m->kv_map) return PI_E_HIP; }
-    if (any_shift) {
-        PI_TRY(pi_memcpy_h2d(m->kv_map, dl.data(), sizeof(int32_t) * n_old));
-        PI_TRY(pi_k_k_shift(m->k_cache, rows, hp.n_ctx, m->hd, hp.arch == PI_ARCH_FALCON ? 2 : 0, m->theta_scale, m->kv_map, n_old, st));
-        PI_HIP_TRY(hipStreamSynchronize(st));
-    }
-    bool moved = false;
-    for (int j = 0; j < n_new; ++j) moved = moved || map[j] != j;
-    if (moved) {
-        if (!m->kv_stage) { m->kv_stage = m->alloc<__half>((size_t)rows * hp.n_ctx * m->hd); if (!m->kv_stage) return PI_E_HIP; }
-        PI_TRY(pi_memcpy_h2d(m->kv_map, map.data(), sizeof(int32_t) * n_new));
-        PI_TRY(pi_k_kv_compact(m->k_cache, m->kv_stage, rows, hp.n_ctx, m->hd, m->kv_map, n_new, st));
-        PI_TRY(pi_k_kv_compact(m->v_cache, m->kv_stage, rows, hp.n_ctx, m->hd, m->kv_map, n_new, st));
-        PI_HIP_TRY(hipStreamSynchronize(st));
-    }
-    bool identity = true;
-    for (int j = 0; j < n_new; ++j) identity = identity && pos[j] == j;
-    if (identity) {
-        m->kv_pos.clear();
-        const int32_t n = n_new;
-        PI_TRY(pi_memcpy_h2d(m->d_pos, &n, 4));       // generation continues at position n
-    } else {
-        m->kv_pos = pos;
-    }
-    return n_new;
-}
-}  // namespace
-
 int pi_model_kv_seq_rm(pi_model * m, int p0, int p1) {
     if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_kv_seq_rm: model not finalized");
-    return kv_edit(m, p0, p1, 0, false);
+    return pi::kv_edit(m, m->k_cache, m->v_cache, m->d_pos, m->kv_pos, p0, p1, 0, false);
 }
 
 int pi_model_kv_seq_shift(pi_model * m, int p0, int p1, int delta) {
     if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_kv_seq_shift: model not finalized");
-    return kv_edit(m, p0, p1, delta, true);
+    return pi::kv_edit(m, m->k_cache, m->v_cache, m->d_pos, m->kv_pos, p0, p1, delta, true);
 }
 
 int pi_model_decode(pi_model * m, const int32_t * tokens, int n_tokens, int n_past, float * logits_out) {

@@ -19,6 +19,7 @@ struct BatchState {
     int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_step = nullptr, *d_out_tokens = nullptr, *union_rows = nullptr, *n_union = nullptr;
     hipGraphExec_t graph_exec = nullptr;
     hipGraph_t graph = nullptr;
+    std::vector<std::vector<int32_t>> kv_pos;      // per sequence: cell positions while an edit left them non-contiguous
 };
 
 namespace {
@@ -204,6 +205,7 @@ int pi_model_batch_decode(pi_model * m, const int32_t * tokens, const int32_t * 
     if (!m || !m->batch) return pi::fail(PI_E_STATE, "pi_model_batch_decode: pi_model_batch_init first");
     if (!tokens || !positions) return pi::fail(PI_E_ARG, "pi_model_batch_decode: null pointer");
     BatchState * b = m->batch;
+    for (auto & v : b->kv_pos) if (!v.empty()) return pi::fail(PI_E_STATE, "pi_model_batch_decode: a sequence's KV cells are not at contiguous positions");
     for (int t = 0; t < b->n_seq; ++t) {
         if (tokens[t] < 0 || tokens[t] >= m->hp.n_vocab) return pi::fail(PI_E_ARG, "pi_model_batch_decode: token id out of range");
         if (positions[t] < 0 || positions[t] >= m->hp.n_ctx) return pi::fail(PI_E_ARG, "pi_model_batch_decode: position outside the context");
@@ -223,6 +225,7 @@ int pi_model_batch_generate(pi_model * m, int n_steps, int32_t * out_tokens, flo
     if (!m || !m->batch) return pi::fail(PI_E_STATE, "pi_model_batch_generate: pi_model_batch_init first");
     BatchState * b = m->batch;
     if (n_steps <= 0 || n_steps > b->max_steps || !out_tokens) return pi::fail(PI_E_ARG, "pi_model_batch_generate: bad step count");
+    for (auto & v : b->kv_pos) if (!v.empty()) return pi::fail(PI_E_STATE, "pi_model_batch_generate: a sequence's KV cells are not at contiguous positions");
     std::vector<int32_t> pos(b->n_seq);
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
     PI_TRY(pi_memcpy_d2h(pos.data(), b->d_pos, sizeof(int32_t) * b->n_seq));
@@ -251,6 +254,49 @@ int pi_model_batch_generate(pi_model * m, int n_steps, int32_t * out_tokens, flo
     if (ms_out) PI_HIP_TRY(hipEventElapsedTime(ms_out, m->ev0, m->ev1));
     PI_TRY(pi_memcpy_d2h(out_tokens, b->d_out_tokens, sizeof(int32_t) * (size_t)n_steps * b->n_seq));
     return PI_OK;
+}
+
+// llama_kv_cache_seq_rm / _seq_shift / _seq_cp for one sequence of the batch (llama.cpp:1757-1848).  Every sequence owns a cache,
+// so "copy" really copies: cells [p0, p1) of src become the same cells of dst, which must hold exactly p0 cells (a shared prompt
+// prefix is evaluated once and handed to the other sequences).
+int pi_model_batch_kv_seq_rm(pi_model * m, int seq, int p0, int p1) {
+    if (!m || !m->batch || seq < 0 || seq >= m->batch->n_seq) return pi::fail(PI_E_ARG, "pi_model_batch_kv_seq_rm: bad sequence");
+    BatchState * b = m->batch;
+    if ((int)b->kv_pos.size() != b->n_seq) b->kv_pos.resize(b->n_seq);
+    return pi::kv_edit(m, b->k_cache + (size_t)seq * b->cache_seq_stride, b->v_cache + (size_t)seq * b->cache_seq_stride, b->d_pos + seq, b->kv_pos[seq], p0, p1, 0, false);
+}
+
+int pi_model_batch_kv_seq_shift(pi_model * m, int seq, int p0, int p1, int delta) {
+    if (!m || !m->batch || seq < 0 || seq >= m->batch->n_seq) return pi::fail(PI_E_ARG, "pi_model_batch_kv_seq_shift: bad sequence");
+    BatchState * b = m->batch;
+    if ((int)b->kv_pos.size() != b->n_seq) b->kv_pos.resize(b->n_seq);
+    return pi::kv_edit(m, b->k_cache + (size_t)seq * b->cache_seq_stride, b->v_cache + (size_t)seq * b->cache_seq_stride, b->d_pos + seq, b->kv_pos[seq], p0, p1, delta, true);
+}
+
+int pi_model_batch_kv_seq_cp(pi_model * m, int src, int dst, int p0, int p1) {
+    if (!m || !m->batch || src < 0 || dst < 0 || src >= m->batch->n_seq || dst >= m->batch->n_seq || src == dst)
+        return pi::fail(PI_E_ARG, "pi_model_batch_kv_seq_cp: bad sequences");
+    BatchState * b = m->batch;
+    if ((int)b->kv_pos.size() == b->n_seq && (!b->kv_pos[src].empty() || !b->kv_pos[dst].empty()))
+        return pi::fail(PI_E_STATE, "pi_model_batch_kv_seq_cp: a sequence has non-contiguous cell positions");
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    std::vector<int32_t> pos(b->n_seq);
+    PI_TRY(pi_memcpy_d2h(pos.data(), b->d_pos, sizeof(int32_t) * b->n_seq));
+    if (p0 < 0) p0 = 0;
+    if (p1 < 0 || p1 > pos[src]) p1 = pos[src];
+    if (p1 < p0) return pi::fail(PI_E_ARG, "pi_model_batch_kv_seq_cp: empty range");
+    if (pos[dst] != p0) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_kv_seq_cp: the destination must hold exactly p0 cells");
+    const int rows = m->hp.n_layer * m->hp.n_head_kv;
+    const size_t pitch = (size_t)m->hp.n_ctx * m->hd * sizeof(__half), width = (size_t)(p1 - p0) * m->hd * sizeof(__half);
+    if (width) {
+        for (__half * base : {b->k_cache, b->v_cache})
+            PI_HIP_TRY(hipMemcpy2DAsync(base + (size_t)dst * b->cache_seq_stride + (size_t)p0 * m->hd, pitch,
+                                        base + (size_t)src * b->cache_seq_stride + (size_t)p0 * m->hd, pitch, width, rows, hipMemcpyDeviceToDevice, m->stream));
+        PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    }
+    const int32_t n = p1;
+    PI_TRY(pi_memcpy_h2d(b->d_pos + dst, &n, 4));
+    return p1;
 }
 
 int pi_model_batch_union(pi_model * m, int32_t * n_union_per_layer) {

@@ -65,6 +65,7 @@ struct pi_model {
 };
 
 namespace pi {
+int  kv_edit(pi_model * m, __half * k_cache, __half * v_cache, int32_t * d_pos, std::vector<int32_t> & kv_pos, int p0, int p1, int delta, bool shift);
 void batch_destroy(pi_model * m);       // frees the batched-decoding state (graphs; device buffers belong to the model)
 bool prefill_supported(pi_model * m);   // F16 weights, every neuron on the GPU, shapes the multi-token kernels cover
 int  prefill_chunk(pi_model * m, const int32_t * tokens, int T, int n_past);

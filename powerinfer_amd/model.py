@@ -41,6 +41,9 @@ def _declare(L):
     L.pi_model_batch_init.restype, L.pi_model_batch_init.argtypes = i, [vp, i]
     L.pi_model_batch_decode.restype, L.pi_model_batch_decode.argtypes = i, [vp, vp, vp, vp, vp]
     L.pi_model_batch_generate.restype, L.pi_model_batch_generate.argtypes = i, [vp, i, vp, C.POINTER(C.c_float)]
+    L.pi_model_batch_kv_seq_rm.restype, L.pi_model_batch_kv_seq_rm.argtypes = i, [vp, i, i, i]
+    L.pi_model_batch_kv_seq_shift.restype, L.pi_model_batch_kv_seq_shift.argtypes = i, [vp, i, i, i, i]
+    L.pi_model_batch_kv_seq_cp.restype, L.pi_model_batch_kv_seq_cp.argtypes = i, [vp, i, i, i, i]
     L.pi_model_batch_union.restype, L.pi_model_batch_union.argtypes = i, [vp, vp]
     L.pi_model_time_section.restype, L.pi_model_time_section.argtypes = i, [vp, i, i, C.POINTER(C.c_float), C.POINTER(C.c_int)]
 
@@ -49,7 +52,8 @@ ENGINE_SYMBOLS = ["pi_model_create", "pi_model_free", "pi_model_set_tensor", "pi
                   "pi_model_kv_seq_rm", "pi_model_kv_seq_shift",
                   "pi_model_decode", "pi_model_generate", "pi_model_set_capture", "pi_model_get_capture",
                   "pi_model_step_active", "pi_model_time_section",
-                  "pi_model_batch_init", "pi_model_batch_decode", "pi_model_batch_generate", "pi_model_batch_union"]
+                  "pi_model_batch_init", "pi_model_batch_decode", "pi_model_batch_generate", "pi_model_batch_union",
+                  "pi_model_batch_kv_seq_rm", "pi_model_batch_kv_seq_shift", "pi_model_batch_kv_seq_cp"]
 
 
 def _type_of(a, hint):
@@ -186,6 +190,22 @@ class Model:
         ms = C.c_float(0)
         check(self.L.pi_model_batch_generate(self.h, n_steps, out.ctypes.data_as(C.c_void_p), C.byref(ms)), "pi_model_batch_generate")
         return out, float(ms.value)
+
+    def batch_kv_seq_rm(self, seq, p0, p1):
+        n = self.L.pi_model_batch_kv_seq_rm(self.h, seq, p0, p1)
+        check(min(n, 0), "pi_model_batch_kv_seq_rm")
+        return n
+
+    def batch_kv_seq_shift(self, seq, p0, p1, delta):
+        n = self.L.pi_model_batch_kv_seq_shift(self.h, seq, p0, p1, delta)
+        check(min(n, 0), "pi_model_batch_kv_seq_shift")
+        return n
+
+    def batch_kv_seq_cp(self, src, dst, p0, p1):
+        """Cells [p0, p1) of sequence src become the same cells of dst (which must hold exactly p0 cells)."""
+        n = self.L.pi_model_batch_kv_seq_cp(self.h, src, dst, p0, p1)
+        check(min(n, 0), "pi_model_batch_kv_seq_cp")
+        return n
 
     def batch_union(self):
         out = np.empty(self.hp.n_layer, np.int32)

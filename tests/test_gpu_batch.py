@@ -200,6 +200,49 @@ def test_batched_decode_matches_per_sequence_oracle(arch):
         m.close()
 
 
+def test_batch_kv_sequence_edits():
+    """llama_kv_cache_seq_rm / _seq_shift / _seq_cp on the sequences of a batch: one sequence takes a context shift, one is
+    untouched, one is emptied and handed the first cells of its neighbour (a shared prefix).  The next lockstep token of every
+    sequence must match a single-sequence engine that went through the same history."""
+    from powerinfer_amd.model import Model
+    hp = synth.hparams("llama-tiny", seed=9, n_ctx=48, sparse_threshold=-1e30)      # every neuron active: no predictor flips between the two paths
+    model = synth.make_model(hp)
+    n_seq, n0 = 3, 8
+    rng = np.random.default_rng(21)
+    toks = rng.integers(0, hp.n_vocab, (n0 + 1, n_seq)).astype(np.int32)
+    gm = Model(hp).load(model)
+    gm.batch_init(n_seq)
+    for s in range(n0):
+        gm.batch_decode(toks[s], np.full(n_seq, s, np.int32), want_logits=False)
+    assert gm.batch_kv_seq_rm(0, 2, 5) == 5
+    with pytest.raises(Exception):                               # sequence 0 has a gap open
+        gm.batch_decode(toks[n0], np.array([5, 8, 6], np.int32))
+    assert gm.batch_kv_seq_shift(0, 5, 8, -3) == 5
+    assert gm.batch_kv_seq_rm(2, 0, -1) == 0
+    assert gm.batch_kv_seq_cp(1, 2, 0, 6) == 6
+    _, lg = gm.batch_decode(toks[n0], np.array([5, 8, 6], np.int32))
+    ref = Model(hp).load(model)
+    # sequence 0: the same shift on the single-sequence engine
+    for s in range(n0):
+        ref.decode([int(toks[s, 0])], s)
+    ref.kv_seq_rm(2, 5)
+    ref.kv_seq_shift(5, 8, -3)
+    _, want0 = ref.decode([int(toks[n0, 0])], 5)
+    # sequence 1: plain history
+    ref.kv_clear()
+    for s in range(n0):
+        ref.decode([int(toks[s, 1])], s)
+    _, want1 = ref.decode([int(toks[n0, 1])], 8)
+    # sequence 2: the first six tokens of sequence 1, then its own token
+    ref.kv_clear()
+    for s in range(6):
+        ref.decode([int(toks[s, 1])], s)
+    _, want2 = ref.decode([int(toks[n0, 2])], 6)
+    for got, want in zip(lg, (want0, want1, want2)):
+        assert rel_err(got, want) < 2e-3
+    gm.close(); ref.close()
+
+
 def test_batch_init_rejects_unsupported_models():
     from powerinfer_amd import lib as pl
     from powerinfer_amd.model import Model

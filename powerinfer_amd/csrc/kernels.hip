@@ -2228,6 +2228,7 @@ __global__ void rope_table_kernel(float2 * __restrict__ table, int n_ctx, int ha
 // launch writes; the first query head of each group stores k and v.
 // ---------------------------------------------------------------------------------------------------
 constexpr int kAttnBlock = 1024;        // 16 waves per head: 64 (hd 128) or 128 (hd 64) cache cells per pass
+constexpr int kAttnPre = 4;             // passes whose K and V rows are requested before the prologue
 __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __restrict__ qkv, const float2 * __restrict__ rope_table,
                                                             __half * __restrict__ k_cache, __half * __restrict__ v_cache,
                                                             int n_head, int n_head_kv, int hd, int mode, int n_ctx,
@@ -2257,6 +2258,18 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
     __half * kdst = k_cache + ((size_t)kvh * n_ctx + pos) * hd;
     __half * vdst = v_cache + ((size_t)kvh * n_ctx + pos) * hd;
     const bool leader = (h % grp_sz) == 0;
+    // the cache cells of the first kAttnPre passes do not depend on anything computed here: their K and V rows are requested
+    // now and travel during the rotation, the scores and the softmax (one memory round trip instead of three in a row)
+    const int lpp = hd / 8;
+    const int sub = tid % lpp, grp = tid / lpp, ngrp = kAttnBlock / lpp;
+    const __half * kb = k_cache + (size_t)kvh * n_ctx * hd;
+    const __half * vb = v_cache + (size_t)kvh * n_ctx * hd;
+    pi_u32x4 kpre[kAttnPre], vpre[kAttnPre];
+#pragma unroll
+    for (int i = 0; i < kAttnPre; ++i) {
+        const int c = i * ngrp + grp;
+        if (c < pos) { kpre[i] = pi_ld16(kb + (size_t)c * hd + sub * 8); vpre[i] = pi_ld16(vb + (size_t)c * hd + sub * 8); }
+    }
     if (tid < hd / 2) {
         const float2 cs = rope_table[(size_t)pos * (hd / 2) + tid];
         const int i0 = (mode & 2) ? tid : 2 * tid;
@@ -2276,14 +2289,25 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
     }
     __syncthreads();
 
-    const int lpp = hd / 8;
-    const int sub = tid % lpp, grp = tid / lpp, ngrp = kAttnBlock / lpp;
     const float scale = 1.0f / sqrtf((float)hd);
     float qf[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) qf[i] = qs[sub * 8 + i];
-    const __half * kb = k_cache + (size_t)kvh * n_ctx * hd;
-    for (int c0 = 0; c0 < n_kv; c0 += ngrp) {
+#pragma unroll
+    for (int i = 0; i < kAttnPre; ++i) {
+        if (i * ngrp < n_kv) {
+            const int c = i * ngrp + grp;
+            float d = 0.0f;
+            if (c < pos) d = pi_dot8(kpre[i], qf, 0.0f);
+            else if (c == pos) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) d = fmaf(kcur[sub * 8 + k], qf[k], d);
+            }
+            for (int o = lpp / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, PI_WAVE);
+            if (c < n_kv && sub == 0) s[c] = __fmul_rn(d, scale);
+        }
+    }
+    for (int c0 = kAttnPre * ngrp; c0 < n_kv; c0 += ngrp) {
         const int c = c0 + grp;
         float d = 0.0f;
         if (c < pos) d = pi_dot8(pi_ld16(kb + (size_t)c * hd + sub * 8), qf, 0.0f);
@@ -2308,11 +2332,25 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
     sum = block_sum_f64(sum, red);
     const float inv = (float)(1.0 / sum);
 
-    const __half * vb = v_cache + (size_t)kvh * n_ctx * hd;
     float acc[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
-    for (int c = grp; c < n_kv; c += ngrp) {
+#pragma unroll
+    for (int i = 0; i < kAttnPre; ++i) {
+        const int c = i * ngrp + grp;
+        if (c < n_kv) {
+            const float p = pi_round_f16(__fmul_rn(s[c], inv));
+            float vf[8];
+            if (c < pos) pi_unpack8(vpre[i], vf);
+            else {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) vf[k] = vcur[sub * 8 + k];
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) acc[k] = fmaf(vf[k], p, acc[k]);
+        }
+    }
+    for (int c = kAttnPre * ngrp + grp; c < n_kv; c += ngrp) {
         const float p = pi_round_f16(__fmul_rn(s[c], inv));
         float vf[8];
         if (c < pos) pi_unpack8(pi_ld16(vb + (size_t)c * hd + sub * 8), vf);

@@ -2474,6 +2474,50 @@ __global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __re
     const float * xt = x + (size_t)blockIdx.x * cols;
     __half * ot = out + (size_t)blockIdx.x * cols;
     float mean = 0.0f, scale = 1.0f;
+    if (cols <= 8 * 1024) {
+        // one memory round trip: the row, the norm weights and the bias are requested together and stay in registers
+        float xv[8], wv[8], bv[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int i = threadIdx.x + k * 1024;
+            xv[k] = i < cols ? xt[i] : 0.0f;
+            wv[k] = (na.kind != 0 && na.w && i < cols) ? na.w[i] : 1.0f;
+            bv[k] = (na.kind != 0 && na.b && i < cols) ? na.b[i] : 0.0f;
+        }
+        if (na.kind == 1) {
+            double s = 0.0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) s += (double)__fmul_rn(xv[k], xv[k]);
+            s = block_sum_f64(s, red);
+            scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
+        } else if (na.kind == 2) {
+            double s = 0.0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) s += (double)xv[k];
+            s = block_sum_f64(s, red);
+            mean = (float)(s / cols);
+            double s2 = 0.0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) { const int i = threadIdx.x + k * 1024; const float v = __fsub_rn(xv[k], mean); if (i < cols) s2 += (double)__fmul_rn(v, v); }
+            s2 = block_sum_f64(s2, red);
+            scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int i = threadIdx.x + k * 1024;
+            if (i < cols) {
+                float v = xv[k];
+                if (out_plain) out_plain[(size_t)blockIdx.x * cols + i] = __float2half_rn(v);
+                if (na.kind != 0) {
+                    v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
+                    if (na.w) v = __fmul_rn(v, wv[k]);
+                    if (na.b) v = __fadd_rn(v, bv[k]);
+                }
+                ot[i] = __float2half_rn(v);
+            }
+        }
+        return;
+    }
     if (na.kind == 1) {
         double s = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = xt[i]; s += (double)__fmul_rn(v, v); }
@@ -2668,6 +2712,29 @@ __global__ __launch_bounds__(1024) void union_active_kernel(const unsigned char 
                                                             uint32_t * __restrict__ words, int32_t * __restrict__ list, int32_t * __restrict__ n_union) {
     __shared__ int sred[17];
     const int lane = threadIdx.x & 63;
+    if ((ff & 31) == 0) {
+        // a thread takes 16 neurons (one 16-byte load); 16384 neurons per pass
+        int base = 0;
+        for (int i0 = 0; i0 < ff; i0 += 16 * 1024) {
+            const int i = i0 + threadIdx.x * 16;
+            uint32_t m = 0;
+            if (i < ff) {
+                const pi_u32x4 v = *reinterpret_cast<const pi_u32x4 *>(row_any + i);
+                const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int k = 0; k < 16; ++k) m |= (((d[k >> 2] >> ((k & 3) * 8)) & 0xFFu) != 0u ? 1u : 0u) << k;
+            }
+            const uint32_t hi = (uint32_t)__shfl_down((int)m, 1, PI_WAVE);
+            if ((threadIdx.x & 1) == 0 && i < ff) words[i >> 5] = m | (hi << 16);
+            int tot;
+            int off = base + block_exclusive_scan_i32(__popc(m), &tot, sred);
+            while (m) { const int b = __ffs(m) - 1; m &= m - 1; list[off++] = i + b; }
+            base += tot;
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) *n_union = base;
+        return;
+    }
     for (int i0 = 0; i0 < ff; i0 += blockDim.x) {
         const int i = i0 + threadIdx.x;
         const bool act = i < ff && row_any[i] != 0;

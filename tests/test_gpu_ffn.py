@@ -100,11 +100,16 @@ def test_one_launch_route_wide_rows(has_gate, norm):
     run_fused_route(has_gate, norm, "one", 8192, 4096, 512)
 
 
-def run_fused_route(has_gate, norm, route, d, ff, r):
+def test_one_launch_route_falcon40b_layer():
+    """One FFN block at the full Falcon-40B shape (32768 x 8192, no gate, LayerNorm, rank 1024): the instantiation in which a
+    workgroup takes four groups of 32 neurons and stores one partial vector for all of them."""
+    run_fused_route(False, 2, "one", 8192, 32768, 1024, T=1, mean_rate=0.08)
+
+
+def run_fused_route(has_gate, norm, route, d, ff, r, T=3, mean_rate=0.10):
     from powerinfer_amd import lib as pl
     from powerinfer_amd.ops import SparseFFN
-    T = 3
-    L = synth.make_ffn_layer(seed=77 + norm, d=d, ff=ff, r=r, wtype=ol.F16, has_gate=has_gate, T=T)
+    L = synth.make_ffn_layer(seed=77 + norm, d=d, ff=ff, r=r, wtype=ol.F16, has_gate=has_gate, T=T, mean_rate=mean_rate)
     rng = np.random.default_rng(5)
     nw = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32) if norm else None
     nb = (0.1 * rng.standard_normal(d)).astype(np.float32) if norm == 2 else None

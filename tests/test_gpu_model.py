@@ -34,7 +34,7 @@ def oracle_ffn_on(model, il, src):
                          L["fc1"], L["fc2"], xn, src, np.zeros(ff, np.int32), hp.sparse_threshold, nth=8)
 
 
-def run_case(hp, n_prompt=12, n_gen=64):
+def run_case(hp, n_prompt=12, n_gen=64, logit_tol=1e-2, min_same=0.9):
     """Both sides consume the same tokens.  Random-init weights make the comparison chaotic in one specific
     way: activations are rounded to fp16 before every dot product (ggml.c:9703-9716), so an fp32 difference in
     the last place (summation order) becomes a 1e-4 difference one layer later and can flip a neuron whose
@@ -78,7 +78,7 @@ def run_case(hp, n_prompt=12, n_gen=64):
         n_past += 1
     assert 1 - flips / neurons >= 0.999, (flips, neurons)
     assert skipped <= 0.1 * (checked + skipped), (checked, skipped)
-    assert np.median(lerr) < 1e-2, lerr
+    assert np.median(lerr) < logit_tol, lerr
     if hp.wtype == synth.F16:
         assert not clean_lerr or max(clean_lerr) < 1e-2, clean_lerr
     gm.set_capture(False)
@@ -95,7 +95,7 @@ def run_case(hp, n_prompt=12, n_gen=64):
             same += 1
         elif lg_o[tok_o] - lg_o[toks_g[s]] <= 1e-2 * np.abs(lg_o).max():
             explained += 1
-    assert same >= 0.9 * n_gen, (same, n_gen)
+    assert same >= min_same * n_gen, (same, n_gen)
     if hp.wtype == synth.F16:
         # a remaining disagreement needs a flipped neuron upstream (its effect on the logits is a few percent, more
         # than a near-tie explains); those are rare
@@ -129,6 +129,18 @@ def test_llama_7b_width_two_layers():
     """Full 7B layer shape (d 4096, ff 11008, rank 1024, 32 heads, vocab 32000), two layers."""
     hp = synth.hparams("llama-7b", n_layer=2, n_ctx=128, seed=6)
     run_case(hp, n_prompt=8, n_gen=64)
+
+
+@pytest.mark.parametrize("hot_frac", [1.0, 0.6])
+def test_llama_7b_width_q4_two_layers(hot_frac):
+    """Q4_0 at the 7B layer shape: the fused Q4_0 kernels (predictor + mask + up/gate in one launch, grouped down projection);
+    with hot_frac 0.6 the host share works from the pinned buffers those kernels fill (logits, Q8_0 input, h)."""
+    hp = synth.hparams("llama-7b", n_layer=2, n_ctx=64, seed=12, wtype=synth.Q4_0, hot_frac=hot_frac)
+    # 4096 int8-rounded activations per dot: a last-place difference in a layer's input moves a few of them by one step, which
+    # is 1e-3 on the next layer's input and flips predictor neurons there (first token, first layer: 2e-7 on every quantity;
+    # second layer: 1.5e-3 and two flips).  The per-layer checks on the GPU's own inputs keep their bounds; the end-to-end
+    # bounds are the ones that have to absorb the reference arithmetic's own sensitivity.
+    run_case(hp, n_prompt=6, n_gen=24, logit_tol=1.5e-1, min_same=0.5)
 
 
 @pytest.mark.parametrize("arch,wtype", [("llama-tiny", synth.F16), ("llama-tiny", synth.Q4_0), ("falcon-tiny", synth.F16)])

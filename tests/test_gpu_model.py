@@ -131,6 +131,14 @@ def test_llama_7b_width_two_layers():
     run_case(hp, n_prompt=8, n_gen=64)
 
 
+def test_falcon_4096_width_two_layers():
+    """A Falcon-architecture model wide enough for the fused FFN kernels (d 4096, rank 512, 64 heads over 8 KV heads): the
+    attention branch and the FFN branch of a layer run on two streams / graph branches and meet in the reduction."""
+    hp = synth.hparams("falcon-tiny", n_embd=4096, n_ff=8192, n_rank=512, n_head=64, n_head_kv=8, n_layer=2, n_vocab=4096,
+                       n_ctx=96, seed=13)
+    run_case(hp, n_prompt=8, n_gen=48)
+
+
 @pytest.mark.parametrize("hot_frac", [1.0, 0.6])
 def test_llama_7b_width_q4_two_layers(hot_frac):
     """Q4_0 at the 7B layer shape: the fused Q4_0 kernels (predictor + mask + up/gate in one launch, grouped down projection);

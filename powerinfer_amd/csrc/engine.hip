@@ -39,26 +39,53 @@ __global__ __launch_bounds__(1024) void argmax_advance_kernel(const float * __re
                                                               const int32_t * __restrict__ n_active, int n_layer, int max_steps) {
     __shared__ float bv[16];
     __shared__ int   bi[16];
+    __shared__ int stot;
     float best = -INFINITY; int idx = n;
-    for (int i = threadIdx.x; i < n; i += blockDim.x) { const float v = logits[i]; if (v > best) { best = v; idx = i; } }
+    // the bookkeeping operands are requested with the logits: one memory round trip for the whole kernel at vocabularies up to 32 K
+    int act = 0;
+    for (int l = threadIdx.x; l < n_layer; l += blockDim.x) act += n_active[l];
+    const int s_in = *step, p_in = *pos;
+    for (int base = 0; base < n; base += 8 * 4 * 1024) {
+        float4 v[8];
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = base + (u * 1024 + (int)threadIdx.x) * 4;
+            if (i + 3 < n) v[u] = *reinterpret_cast<const float4 *>(logits + i);
+            else v[u] = make_float4(i < n ? logits[i] : -INFINITY, i + 1 < n ? logits[i + 1] : -INFINITY, i + 2 < n ? logits[i + 2] : -INFINITY, -INFINITY);
+        }
+#pragma unroll
+        for (int u = 0; u < 8; ++u) {
+            const int i = base + (u * 1024 + (int)threadIdx.x) * 4;
+            if (v[u].x > best) { best = v[u].x; idx = i; }
+            if (v[u].y > best) { best = v[u].y; idx = i + 1; }
+            if (v[u].z > best) { best = v[u].z; idx = i + 2; }
+            if (v[u].w > best) { best = v[u].w; idx = i + 3; }
+        }
+    }
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, 64); const int oi = __shfl_xor(idx, o, 64);
         if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
     }
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (wave == 0) {                       // n_layer <= 1024 entries were spread over the threads; at most a few waves hold non-zeros
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) act += __shfl_xor(act, o, 64);
+    }
+    if (threadIdx.x == 0) stot = 0;
     if (lane == 0) { bv[wave] = best; bi[wave] = idx; }
+    __syncthreads();
+    if (wave != 0 && act != 0) atomicAdd(&stot, act);      // layers beyond the first 64 (LDS atomic, integer: order does not matter)
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int w = 1; w < (int)(blockDim.x >> 6); ++w)
             if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
         if (idx >= n) idx = 0;
-        int tot = 0;
-        for (int l = 0; l < n_layer; ++l) tot += n_active[l];
-        const int s = *step;
+        const int tot = act + stot;
+        const int s = s_in;
         if (s < max_steps) { out_tokens[s] = idx; out_active[s] = tot; }
         *token = idx;
-        *pos = *pos + 1;
+        *pos = p_in + 1;
         *step = s + 1;
     }
 }

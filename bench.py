@@ -218,7 +218,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the token loop on ONE GPU; --gpus must be 1 "
-                 "(how the path would shard over xGMI is described in DESIGN.md)")
+                 "(more GPUs would split the FFN by neuron and attention by head, one [n_embd] exchange per layer)")
 
     from powerinfer_amd import lib as pl, synth
     if args.pmc_probe:

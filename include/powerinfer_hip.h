@@ -197,6 +197,16 @@ PI_API int pi_k_sparse_ffn_partials(const void * fc2_f16, int ff, int r, const f
                                     pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_sparse_ffn_reduce(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out,
                                   int32_t * n_active, pi_workspace * ws, pi_stream_t stream);
+/* the same two launches for a hot/cold split layer (F16): only the GPU-resident neurons are computed, from the compact matrices of
+ * the bucket (hot_words / hot_prefix as for pi_k_pred_upgate_q4); logits and xn_f16_out (the fp16-rounded normalised input, cols
+ * values, optional) may be pinned host memory for the host share; _reduce_hot counts the resident active neurons, and its add1 /
+ * add2 may be pinned host memory (the host share's output).  GPU part of llm_build_sparse_mul_mat / _axpy, llama.cpp:4581-4646. */
+PI_API int pi_k_sparse_ffn_partials_hot(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                                        const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols,
+                                        const float * x, const pi_norm * norm, const uint32_t * hot_words, const int32_t * hot_prefix,
+                                        float * logits, float * h_dense, void * xn_f16_out, pi_workspace * ws, pi_stream_t stream);
+PI_API int pi_k_sparse_ffn_reduce_hot(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out,
+                                      int32_t * n_active, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_sparse_ffn(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
                            const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols,
                            const float * x, const pi_norm * norm,

@@ -998,13 +998,18 @@ constexpr int kPfChunk = 8;                       // active neurons per round tr
 
 __device__ __forceinline__ int select_nth_bit(uint32_t bits, int n);
 
-template <int CPW, int RCH, bool GATE, int G>      // cols == 8 waves * CPW chunks * 512; r == RCH * 512; G groups of 32 neurons
+// HYB: a hot/cold split layer.  Only the GPU-resident neurons are computed (mask & hot word; weight row = hot prefix + rank among
+// the hot bits: the compact matrices of the bucket), the activity words of that share go to words_hot, and workgroup 0 hands the
+// fp16-rounded normalised input to the host share (xn_out; like logits it may be pinned host memory).
+template <int CPW, int RCH, bool GATE, int G, bool HYB>      // cols == 8 waves * CPW chunks * 512; r == RCH * 512; G groups of 32 neurons
 __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
                                                                    const __half * __restrict__ Wup, const __half * __restrict__ Wgate,
                                                                    const __half * __restrict__ Wdown,
                                                                    const float * __restrict__ x, NormArgs na, float thr,
                                                                    float * __restrict__ logits, uint32_t * __restrict__ words, float * __restrict__ h_dense,
-                                                                   float * __restrict__ partial) {
+                                                                   float * __restrict__ partial,
+                                                                   const uint32_t * __restrict__ hot_words, const int32_t * __restrict__ hot_prefix,
+                                                                   uint32_t * __restrict__ words_hot, __half * __restrict__ xn_out) {
     constexpr int cols = kPfWaves * CPW * 512, r = RCH * 512;
     constexpr int CH = kPfChunk / CPW;                 // active neurons per round trip: 3*CPW*CH (2*CPW*CH) loads in flight per lane
     __shared__ float  lg[2][32];
@@ -1122,6 +1127,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
         __half2 hh[4] = {__floats2half2_rn(xs[c][0], xs[c][1]), __floats2half2_rn(xs[c][2], xs[c][3]),
                          __floats2half2_rn(xs[c][4], xs[c][5]), __floats2half2_rn(xs[c][6], xs[c][7])};
         xr[c] = *reinterpret_cast<const pi_u32x4 *>(hh);
+        if (HYB && blockIdx.x == 0 && xn_out) *reinterpret_cast<pi_u32x4 *>(xn_out + cbase + c * 512) = xr[c];
     }
     float acc[CPW][8];
 #pragma unroll
@@ -1150,10 +1156,13 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
     // ---- activity word (identical in every wave; lg[g & 1] is complete after the barrier above) ----------------
     const float my_logit = lg[g & 1][lane & 31];
     const bool my_act = !(my_logit < thr);
-    const uint32_t mask = (uint32_t)__ballot(my_act);
+    const uint32_t all = (uint32_t)__ballot(my_act);
+    const uint32_t hot = HYB ? hot_words[blockIdx.x * G + g] : 0xFFFFFFFFu;
+    const int base_row = HYB ? hot_prefix[blockIdx.x * G + g] : n0;
+    const uint32_t mask = all & hot;
     if (wave == 0) {
-        if (lane < 32) { if (logits) logits[n0 + lane] = my_logit; if (h_dense && !my_act) h_dense[n0 + lane] = 0.0f; }
-        if (lane == 0) words[blockIdx.x * G + g] = mask;
+        if (lane < 32) { if (logits) logits[n0 + lane] = my_logit; if (h_dense && !((mask >> lane) & 1u)) h_dense[n0 + lane] = 0.0f; }
+        if (lane == 0) { words[blockIdx.x * G + g] = all; if (HYB) words_hot[blockIdx.x * G + g] = mask; }
     }
     // ---- B + C ---------------------------------------------------------------------------------------------
     const int n = __popc(mask);
@@ -1164,8 +1173,9 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
 #pragma unroll
         for (int j = 0; j < CH; ++j) {
             if (j < nn) {
-                rows[j] = n0 + select_nth_bit(mask, c0 + j);
-                const size_t off = (size_t)rows[j] * cols + cbase;
+                const int bit = select_nth_bit(mask, c0 + j);
+                rows[j] = n0 + bit;
+                const size_t off = (size_t)(HYB ? base_row + __popc(hot & ((1u << bit) - 1u)) : rows[j]) * cols + cbase;
 #pragma unroll
                 for (int c = 0; c < CPW; ++c) {
                     uu[j][c] = pi_ld_stream(Wup + off + c * 512);
@@ -3388,20 +3398,24 @@ static int pf_groups(int ff, int cols) {
     return (ff % 128 == 0 && ff / 128 >= 256) ? 4 : 1;
 }
 
-int pi_k_sparse_ffn_partials(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
-                             const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x, const pi_norm * norm,
-                             float * logits, float * h_dense, pi_workspace * ws, pi_stream_t stream) {
-    if (!fc2_f16 || !hidden || !up_f16 || !down_t_f16 || !x || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: null pointer");
+static int sparse_ffn_partials_impl(const char * who, const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                                    const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x, const pi_norm * norm,
+                                    float * logits, float * h_dense, const uint32_t * hot_words, const int32_t * hot_prefix, void * xn_f16_out,
+                                    pi_workspace * ws, pi_stream_t stream) {
+    if (!fc2_f16 || !hidden || !up_f16 || !down_t_f16 || !x || !ws) return pi::fail(PI_E_ARG, who);
     if (!pi_k_sparse_ffn_supported(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn: shape outside the fused kernel (cols 4096 or 8192, r 512 or 1024, ff % 32 == 0)");
     if (ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: shape exceeds the workspace");
+    if ((hot_words == nullptr) != (hot_prefix == nullptr)) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: hot_words and hot_prefix go together");
     const NormArgs na = to_norm(norm);
-    if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: vectors must be 16-byte aligned");
+    if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b | (uintptr_t)xn_f16_out) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: vectors must be 16-byte aligned");
     hipStream_t st = (hipStream_t)stream;
     const __half * w2 = (const __half *)fc2_f16; const __half * u = (const __half *)up_f16; const __half * g = (const __half *)gate_f16;
     const __half * dn = (const __half *)down_t_f16;
     const int G = pf_groups(ff, cols);
     const dim3 grid(ff / (32 * G)), block(kPfBlock);
-#define PI_PF_LAUNCH(CPW, RCH, GATE, GG) hipLaunchKernelGGL((pred_ffn_f16_kernel<CPW, RCH, GATE, GG>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial)
+    const bool hyb = hot_words != nullptr;
+#define PI_PF_LAUNCH2(CPW, RCH, GATE, GG, HYB) hipLaunchKernelGGL((pred_ffn_f16_kernel<CPW, RCH, GATE, GG, HYB>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial, hot_words, hot_prefix, ws->words_hot, (__half *)xn_f16_out)
+#define PI_PF_LAUNCH(CPW, RCH, GATE, GG) do { if (hyb) PI_PF_LAUNCH2(CPW, RCH, GATE, GG, true); else PI_PF_LAUNCH2(CPW, RCH, GATE, GG, false); } while (0)
 #define PI_PF_WIDE(RCH, GATE) do { if (G == 4) PI_PF_LAUNCH(2, RCH, GATE, 4); else if (G == 2) PI_PF_LAUNCH(2, RCH, GATE, 2); else PI_PF_LAUNCH(2, RCH, GATE, 1); } while (0)
     const int cpw = cols / 4096, rch = r / 512;
     if (cpw == 1 && rch == 2) { if (g) PI_PF_LAUNCH(1, 2, true, 1); else PI_PF_LAUNCH(1, 2, false, 1); }
@@ -3410,15 +3424,45 @@ int pi_k_sparse_ffn_partials(const void * fc2_f16, int ff, int r, const float * 
     else                      { if (g) PI_PF_WIDE(1, true); else PI_PF_WIDE(1, false); }
 #undef PI_PF_WIDE
 #undef PI_PF_LAUNCH
-    return pi::check_launch("pi_k_sparse_ffn_partials");
+#undef PI_PF_LAUNCH2
+    return pi::check_launch(who);
 }
+
+int pi_k_sparse_ffn_partials(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                             const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x, const pi_norm * norm,
+                             float * logits, float * h_dense, pi_workspace * ws, pi_stream_t stream) {
+    return sparse_ffn_partials_impl("pi_k_sparse_ffn_partials", fc2_f16, ff, r, hidden, threshold, up_f16, gate_f16, down_t_f16, cols, x, norm, logits, h_dense,
+                                    nullptr, nullptr, nullptr, ws, stream);
+}
+
+int pi_k_sparse_ffn_partials_hot(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                                 const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x, const pi_norm * norm,
+                                 const uint32_t * hot_words, const int32_t * hot_prefix, float * logits, float * h_dense, void * xn_f16_out,
+                                 pi_workspace * ws, pi_stream_t stream) {
+    if (!hot_words || !hot_prefix) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_partials_hot: hot words and prefix are required");
+    return sparse_ffn_partials_impl("pi_k_sparse_ffn_partials_hot", fc2_f16, ff, r, hidden, threshold, up_f16, gate_f16, down_t_f16, cols, x, norm, logits, h_dense,
+                                    hot_words, hot_prefix, xn_f16_out, ws, stream);
+}
+
+static int sparse_ffn_reduce_impl(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out, int32_t * n_active,
+                                  bool hot, pi_workspace * ws, pi_stream_t stream);
 
 int pi_k_sparse_ffn_reduce(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out, int32_t * n_active,
                            pi_workspace * ws, pi_stream_t stream) {
+    return sparse_ffn_reduce_impl(ff, cols, epilogue, add1, add2, out, n_active, false, ws, stream);
+}
+
+int pi_k_sparse_ffn_reduce_hot(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out, int32_t * n_active,
+                               pi_workspace * ws, pi_stream_t stream) {
+    return sparse_ffn_reduce_impl(ff, cols, epilogue, add1, add2, out, n_active, true, ws, stream);
+}
+
+static int sparse_ffn_reduce_impl(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out, int32_t * n_active,
+                                  bool hot, pi_workspace * ws, pi_stream_t stream) {
     if (!out || !ws || ff <= 0 || ff % 32 || ff > ws->max_ff || cols <= 0 || cols % 64 || cols > ws->max_d) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_reduce: bad arguments");
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
         return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_reduce: bad epilogue arguments");
-    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, ff / (32 * pf_groups(ff, cols)), cols, ws->words, ff / 32, n_active,
+    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, ff / (32 * pf_groups(ff, cols)), cols, hot ? ws->words_hot : ws->words, ff / 32, n_active,
                        epilogue, add1, add2, out);
     return pi::check_launch("pi_k_sparse_ffn_reduce");
 }

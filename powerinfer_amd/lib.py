@@ -62,6 +62,8 @@ _SIGS = {
     "pi_k_k_shift": (_i, [_vp, _i, _i, _i, _i, _f, _vp, _i, _vp]),
     "pi_k_kv_compact": (_i, [_vp, _vp, _i, _i, _i, _vp, _i, _vp]),
     "pi_k_sparse_ffn_partials": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp]),
+    "pi_k_sparse_ffn_partials_hot": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_sparse_ffn_reduce_hot": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_reduce": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_pred_upgate_supported": (_i, [_i, _i, _i]),
     "pi_k_pred_upgate": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp]),

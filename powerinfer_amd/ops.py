@@ -139,6 +139,30 @@ class SparseFFN:
             self._hot = (DevBuf(host=words), DevBuf(host=prefix))
         return self._hot
 
+    def forward_one_launch_hot(self, x_ffn, x_pred, epilogue=pl.EPI_NONE, resid=None):
+        """The fused F16 route on a hot/cold split layer: pi_k_sparse_ffn_partials_hot + pi_k_sparse_ffn_reduce_hot over the
+        bucket's compact matrices.  Returns dict(logits, h, xn16, n_active, out): out is the resident neurons' share."""
+        L = self.L
+        if self.bucket is None or self.wtype != pl.F16 or not L.pi_k_sparse_ffn_supported(self.ff, self.r, self.d):
+            raise pl.PiError("forward_one_launch_hot: needs a bucket, F16 weights and a shape the fused kernel covers")
+        hw, hp = self._hot_tables()
+        self.x.upload(np.asarray(x_ffn, np.float32))
+        self.xp.upload(np.asarray(x_pred, np.float32))
+        if resid is not None:
+            self.resid.upload(np.asarray(resid, np.float32))
+        check(L.pi_memset(self.h_dense.ptr, 0xFF, self.h_dense.nbytes), "memset")      # the kernel must write every entry
+        xn16 = DevBuf(self.d * 2)
+        nrm = pl.norm_arg(self.norm_kind, self.eps, self.norm_w, self.norm_b)
+        check(L.pi_k_gemv(pl.F16, self.fc1.ptr, self.r, self.d, self.xp.ptr, None, pl.EPI_RELU, None, None, self.hidden.ptr, None), "fc1")
+        check(L.pi_k_sparse_ffn_partials_hot(self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, self.up.ptr,
+                                             self.gate.ptr if self.gate is not None else None, self.down.ptr, self.d, self.x.ptr, nrm,
+                                             hw.ptr, hp.ptr, self.logits.ptr, self.h_dense.ptr, xn16.ptr, self.ws, None), "partials_hot")
+        check(L.pi_k_sparse_ffn_reduce_hot(self.ff, self.d, epilogue, self.resid.ptr if epilogue else None, None, self.out.ptr,
+                                           self.n_active.ptr, self.ws, None), "reduce_hot")
+        pl.sync()
+        return dict(logits=self.logits.download(np.float32), h=self.h_dense.download(np.float32), xn16=xn16.download(np.float16),
+                    n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32))
+
     def forward_q4_fused(self, x_ffn, x_pred, epilogue=pl.EPI_NONE, resid=None, fill_h=None):
         """Q4_0 route of the decode loop at d = 4096: fc1, pi_k_pred_upgate_q4 (fc2 + mask + up/gate of the resident neurons),
         then pi_k_axpy_q4_partials + pi_k_axpy_q4_reduce.  fill_h(h) may return the vector with the host share's neurons

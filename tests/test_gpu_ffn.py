@@ -204,6 +204,41 @@ def test_q4_fused_route_7b_shape(has_gate, norm):
     ffn.close()
 
 
+@pytest.mark.parametrize("has_gate,norm", [(True, 1), (False, 2)])
+def test_f16_fused_route_hybrid_share(has_gate, norm):
+    """The fused F16 kernels on a hot/cold split at the 7B width: the resident 60 % come from compact matrices through the hot
+    words / prefix; their output must equal what the oracle computes for exactly those neurons (gpu_idx inverted), and the
+    normalised fp16 input handed to the host share must be the oracle's."""
+    from powerinfer_amd.ops import SparseFFN
+    d, ff, r, T = 4096, 4096, 512, 2
+    L = synth.make_ffn_layer(seed=35 + norm, d=d, ff=ff, r=r, wtype=ol.F16, has_gate=has_gate, mean_rate=0.15, T=T)
+    gid, bucket = synth.gpu_split(L["p"], 0.6)
+    rng = np.random.default_rng(8)
+    nw = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    nb = (0.1 * rng.standard_normal(d)).astype(np.float32) if norm == 2 else None
+    eps = 1e-5
+    O, P = ol.oracle(), ol._ptr
+    ffn = SparseFFN(d, ff, r, ol.F16, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], bucket=bucket, norm_kind=norm, norm_w=nw, norm_b=nb, eps=eps)
+    for t in range(T):
+        x = np.ascontiguousarray(L["x"][t:t + 1], np.float32)
+        xn = x.copy()
+        if norm == 1:
+            O.pio_rms_norm(P(x), d, 1, eps, P(xn)); xn = np.ascontiguousarray(xn * nw, np.float32)
+        else:
+            O.pio_norm(P(x), d, 1, eps, P(xn)); xn = np.ascontiguousarray(xn * nw + nb, np.float32)
+        share = ol.ffn_sparse(O, d, ff, r, 1, ol.F16, has_gate, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], xn, x, 1 - gid, 0.0)
+        res = ffn.forward_one_launch_hot(x[0], x[0])
+        mask_g, mask_o = ~(res["logits"] < 0.0), ~(share["logits"][0] < 0.0)
+        assert rel_err(res["logits"], share["logits"][0]) < 1e-4
+        assert res["n_active"] == int((mask_g & (gid == 1)).sum())
+        assert np.all(res["h"][gid == 0] == 0.0) and np.all(res["h"][~mask_g] == 0.0)
+        assert (res["xn16"] != xn[0].astype(np.float16)).mean() < 1e-3              # a last-place step of the norm at most
+        if np.array_equal(mask_g, mask_o):
+            assert rel_err(res["h"], share["h"][0]) < 1e-4
+            assert rel_err(res["out"], share["out"][0]) < 1e-4
+    ffn.close()
+
+
 def test_q4_fused_route_hybrid_share():
     """Hot/cold split at the 7B width: the kernels see only the resident 60 % (compact matrices, hot words / prefix); with the
     cold neurons' h filled in before the down projection, GPU share + cold share (numpy, same Q8_0 blocks of h) must equal the

@@ -211,7 +211,7 @@ def main():
                     help="BASELINE configs index: 1 (default, the reported metric) 7B FP16 all on the GPU; 2 the same shape in "
                          "Q4_0 with the hottest 60 %% of neurons on the GPU and the rest on host threads; 3 ProSparse-LLaMA-2-13B shape FP16, "
                          "16 sequences decoded in lockstep; 4 Falcon-40B shape FP16")
-    ap.add_argument("--hot-frac", type=float, default=None, help="config 2 only: share of each layer's neurons on the GPU (default 0.6; 1.0 = all)")
+    ap.add_argument("--hot-frac", type=float, default=None, help="configs 1 and 2: share of each layer's neurons on the GPU (default 1.0 and 0.6)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter-collection aid: run only the q|k|v mat-vec of a 4-layer model a few times plus one "
                          "device-to-device copy of the same byte count (the known-size reference for FETCH_SIZE / WRITE_SIZE)")
@@ -239,7 +239,7 @@ def main():
         return
     n_ctx = args.prompt + args.warmup + args.steps + 8
     if args.config == 1:
-        hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_ctx, seed=1)
+        hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_ctx, seed=1, hot_frac=1.0 if args.hot_frac is None else args.hot_frac)
     elif args.config == 2:
         hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_ctx, seed=1, wtype=pl.Q4_0, hot_frac=0.6 if args.hot_frac is None else args.hot_frac)
     elif args.config == 3:

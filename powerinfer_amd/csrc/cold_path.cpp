@@ -260,6 +260,7 @@ struct ColdPath {
     float * logits = nullptr, * src = nullptr, * h_gpu = nullptr;      // device -> host, consumed before the layer call returns
     float * h_full[2] = {nullptr, nullptr}, * out[2] = {nullptr, nullptr};   // host -> device, read by the GPU after the call returned: two sets, used in turn
     BlockQ8 * xq8_pin = nullptr;                // Q8_0 blocks of the normalised FFN input, written by the fused Q4_0 kernel
+    uint16_t * x16_pin = nullptr;               // fp16 normalised FFN input, written by the fused F16 kernel
     int flip = 0;
     hipEvent_t ev_in = nullptr, ev_h = nullptr;
     std::vector<float> hval;                    // h of the active cold neurons, in the order of act
@@ -303,9 +304,10 @@ ColdPath * cold_create(pi_model * m) {
     }
     auto pin = [](size_t n) { void * p = nullptr; return hipHostMalloc(&p, n * sizeof(float), hipHostMallocCoherent) == hipSuccess ? (float *)p : nullptr; };
     c->xq8_pin = (BlockQ8 *)pin((size_t)(c->d / 32 + 1) * sizeof(BlockQ8) / sizeof(float) + 1);
+    c->x16_pin = (uint16_t *)pin((size_t)c->d / 2 + 8);
     c->logits = pin(c->ff); c->src = pin(c->d); c->h_gpu = pin(c->ff);
     for (int i = 0; i < 2; ++i) { c->h_full[i] = pin(c->ff); c->out[i] = pin(c->d); }
-    if (!c->logits || !c->src || !c->h_gpu || !c->h_full[0] || !c->h_full[1] || !c->out[0] || !c->out[1] || !c->xq8_pin) { set_error("cold path: pinned host allocation failed"); cold_destroy(c); return nullptr; }
+    if (!c->logits || !c->src || !c->h_gpu || !c->h_full[0] || !c->h_full[1] || !c->out[0] || !c->out[1] || !c->xq8_pin || !c->x16_pin) { set_error("cold path: pinned host allocation failed"); cold_destroy(c); return nullptr; }
     if (hipEventCreateWithFlags(&c->ev_in, hipEventDisableTiming) != hipSuccess || hipEventCreateWithFlags(&c->ev_h, hipEventDisableTiming) != hipSuccess) {
         set_error("cold path: event creation failed"); cold_destroy(c); return nullptr;
     }
@@ -324,6 +326,7 @@ void cold_destroy(ColdPath * c) {
     delete c->pool;
     for (float * p : {c->logits, c->src, c->h_gpu, c->h_full[0], c->h_full[1], c->out[0], c->out[1]}) if (p) (void)hipHostFree(p);
     if (c->xq8_pin) (void)hipHostFree(c->xq8_pin);
+    if (c->x16_pin) (void)hipHostFree(c->x16_pin);
     if (c->ev_in) (void)hipEventDestroy(c->ev_in);
     if (c->ev_h) (void)hipEventDestroy(c->ev_h);
     delete c;
@@ -570,6 +573,96 @@ int cold_layer_q4(ColdPath * c, int il, pi_model * m, hipStream_t st, bool captu
         rc = pi_k_axpy_q4_reduce(ff, d, PI_EPI_ADD2, out, m->ffn_inp, m->x2, n_act, m->ws, st);
     } else {
         rc = pi_k_axpy_q4_reduce(ff, d, PI_EPI_NONE, nullptr, nullptr, m->x2, n_act, m->ws, st);
+        if (rc == PI_OK)
+            rc = merge_shares(m->x2, out, m->x2, falcon ? m->attn_out : m->ffn_inp, falcon ? m->x : nullptr,
+                              capture ? m->cap_ffn + (size_t)il * d : nullptr, d, st);
+    }
+    lap(5);
+    if (c->trace) { ++c->n_calls; c->n_cold_active += na; c->t_last_return = now(); }
+    return rc;
+}
+
+int cold_layer_f16(ColdPath * c, int il, pi_model * m, hipStream_t st, bool capture) {
+    const pi_hparams & hp = m->hp;
+    const int d = c->d, ff = c->ff;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    ColdLayer & cl = c->layers[il];
+    Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
+    Tensor & fc1 = m->L(il, PI_T_FC1); Tensor & fc2 = m->L(il, PI_T_FC2);
+    const int r = (int)fc1.ne1;
+    const float thr = hp.sparse_threshold;
+    const int p = (c->flip ^= 1);
+    float * out = c->out[p];
+    auto now = [] { return std::chrono::steady_clock::now(); };
+    auto us = [](std::chrono::steady_clock::time_point a, std::chrono::steady_clock::time_point b) { return std::chrono::duration<double, std::micro>(b - a).count(); };
+    std::chrono::steady_clock::time_point tp = now();
+    if (c->trace && c->n_calls) c->t_between += us(c->t_last_return, tp);
+    auto lap = [&](int i) { if (c->trace) { const auto t = now(); c->t_phase[i] += us(tp, t); tp = t; } };
+
+    // 1. the resident share in one launch; logits and the fp16 input land in pinned memory for the host share
+    pi_norm fn;
+    fn.kind = falcon ? 2 : 1; fn.eps = hp.norm_eps;
+    fn.w = (const float *)m->L(il, falcon ? PI_T_ATTN_NORM : PI_T_FFN_NORM).dev;
+    fn.b = falcon ? (const float *)m->L(il, PI_T_ATTN_NORM_B).dev : nullptr;
+    const float * ffn_src = falcon ? m->x : m->ffn_inp;
+    int rc = pi_k_sparse_ffn_partials_hot(fc2.dev, ff, r, m->hidden, thr, up.dev, falcon ? nullptr : gate.dev, down.dev, d, ffn_src, &fn,
+                                          m->hot_words[il], m->hot_prefix[il], c->logits, nullptr, c->x16_pin, m->ws, st);
+    if (rc != PI_OK) return rc;
+    PI_HIP_TRY(hipEventRecord(c->ev_in, st));
+    if (capture) PI_HIP_TRY(hipMemcpyAsync(m->cap_logits + (size_t)il * ff, c->logits, sizeof(float) * ff, hipMemcpyHostToDevice, st));
+    PI_HIP_TRY(wait_event(c->ev_in));
+    lap(0);
+
+    // 2. active cold neurons: up/gate dots on the fp16 input (ggml.c:14030-14282), h rounded to fp16 for the axpy (ggml.c:14420-14431)
+    c->act.clear();
+    for (int j : cl.cold_rows) if (!(c->logits[j] < thr)) c->act.push_back(j);
+    const int na = (int)c->act.size();
+    lap(1);
+    float * hval = c->hval.data();
+    const size_t rb = (size_t)d * 2;
+    const unsigned char * wu = (const unsigned char *)up.host;
+    const unsigned char * wg = falcon ? nullptr : (const unsigned char *)gate.host;
+    const uint16_t * x16 = c->x16_pin;
+    c->pool->run([&](int t, int nt) {
+        for (int k = t; k < na; k += nt) {
+            const int j = c->act[k];
+            if (k + nt < na) { prefetch_bytes(wu + rb * c->act[k + nt], rb); if (wg) prefetch_bytes(wg + rb * c->act[k + nt], rb); }
+            const float u = dot_f16(d, (const uint16_t *)(wu + rb * j), x16);
+            const float g = wg ? dot_f16(d, (const uint16_t *)(wg + rb * j), x16) : 0.f;
+            hval[k] = wg ? (g > 0.f ? g : 0.f) * u : (u > 0.f ? u : 0.f);
+        }
+    });
+    lap(2);
+    lap(3);
+    const unsigned char * wd = (const unsigned char *)down.host;
+    const int n_units = d / 32;
+    c->pool->run([&](int t, int nt) {
+        const int u0 = (int)((long long)n_units * t / nt), u1 = (int)((long long)n_units * (t + 1) / nt);
+        const int c0 = u0 * 32, c1 = u1 * 32;
+        for (int i = c0; i < c1; ++i) out[i] = 0.f;
+        for (int k = 0; k < na; ++k) {
+            const uint16_t hb = f2h(hval[k]);
+            if (k + 2 < na) prefetch_bytes(wd + rb * c->act[k + 2] + (size_t)c0 * 2, (size_t)(c1 - c0) * 2);
+            if (hb == 0) continue;
+            const float a = h2f(hb);
+            const uint16_t * row = (const uint16_t *)(wd + rb * c->act[k]);
+#ifdef PI_COLD_SIMD
+            const __m256 av = _mm256_set1_ps(a);
+            for (int i = c0; i < c1; i += 8)
+                _mm256_storeu_ps(out + i, _mm256_fmadd_ps(_mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(row + i))), av, _mm256_loadu_ps(out + i)));
+#else
+            for (int i = c0; i < c1; ++i) out[i] = fmaf(h2f(row[i]), a, out[i]);
+#endif
+        }
+    });
+    lap(4);
+
+    // 3. (cold + hot) + residual(s), folded into the reduction of the GPU partials when there is one residual and nothing to keep
+    int32_t * n_act = m->n_active + il;
+    if (!falcon && !capture) {
+        rc = pi_k_sparse_ffn_reduce_hot(ff, d, PI_EPI_ADD2, out, m->ffn_inp, m->x2, n_act, m->ws, st);
+    } else {
+        rc = pi_k_sparse_ffn_reduce_hot(ff, d, PI_EPI_NONE, nullptr, nullptr, m->x2, n_act, m->ws, st);
         if (rc == PI_OK)
             rc = merge_shares(m->x2, out, m->x2, falcon ? m->attn_out : m->ffn_inp, falcon ? m->x : nullptr,
                               capture ? m->cap_ffn + (size_t)il * d : nullptr, d, st);

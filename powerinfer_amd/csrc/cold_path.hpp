@@ -22,6 +22,9 @@ int        cold_layer_merge(ColdPath * c, int il, pi_model * m, hipStream_t st);
 // Q4_0 hybrid layer at d = 4096 on the fused kernels: queues fc2 + mask + resident up/gate, computes the host share from the
 // buffers that launch fills, queues the down projection and the merge; leaves the layer output in m->x2.
 int        cold_layer_q4(ColdPath * c, int il, pi_model * m, hipStream_t st, bool capture);
+// The same for an F16 hybrid layer at a width the fused F16 kernels cover: the resident share needs nothing from the host, so
+// its whole FFN (gate/up/down partial vectors) is queued at once and only the final reduction waits for the host share.
+int        cold_layer_f16(ColdPath * c, int il, pi_model * m, hipStream_t st, bool capture);
 
 int add_vec(float * y, const float * a, int n, hipStream_t st);
 // dst = ((cold + hot) + r1) [+ r2]; `cold` may be pinned host memory; `keep` (optional) receives cold + hot

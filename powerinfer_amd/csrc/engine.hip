@@ -214,6 +214,15 @@ int layer_forward(pi_model * m, int il, bool last_token) {
         std::swap(m->x, m->x2);
         return PI_OK;
     }
+    if (layer_hybrid && !q4 && m->hot_words[il] && up.type == PI_TYPE_F16 && fc2.type == PI_TYPE_F16 && pi_k_sparse_ffn_supported(ff, r, d)) {
+        // F16 hybrid layer at a width the fused kernels cover: the resident share's whole FFN is one launch, the host share works
+        // from the pinned buffers it fills, the reduction merges both
+        const bool cap = m->capture && last_token;
+        PI_TRY(pi::cold_layer_f16(m->cold, il, m, st, cap));
+        if (cap) PI_HIP_TRY(hipMemcpyAsync(m->cap_src + (size_t)il * d, ffn_in, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
+        std::swap(m->x, m->x2);
+        return PI_OK;
+    }
     if (q4 && fc2.type == PI_TYPE_F16 && pi_k_pred_upgate_q4_supported(ff, r, d) && (!layer_hybrid || m->hot_words[il])) {
         // Q4_0 at d = 4096: fc2 + mask + up/gate of the resident neurons in one launch, the down projection as partial vectors
         // plus one reduction; a hybrid layer's host share works between the two from the buffers the first kernel fills

@@ -139,6 +139,13 @@ def test_falcon_4096_width_two_layers():
     run_case(hp, n_prompt=8, n_gen=48)
 
 
+def test_llama_7b_width_hybrid_f16_two_layers():
+    """F16 hot/cold split at the 7B layer shape: the resident 60 % run through the fused kernels on the bucket's compact
+    matrices, the host share works from the pinned logits and fp16 input, the reduction adds both shares and the residual."""
+    hp = synth.hparams("llama-7b", n_layer=2, n_ctx=96, seed=14, hot_frac=0.6)
+    run_case(hp, n_prompt=8, n_gen=32)
+
+
 @pytest.mark.parametrize("hot_frac", [1.0, 0.6])
 def test_llama_7b_width_q4_two_layers(hot_frac):
     """Q4_0 at the 7B layer shape: the fused Q4_0 kernels (predictor + mask + up/gate in one launch, grouped down projection);

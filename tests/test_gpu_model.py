@@ -139,6 +139,18 @@ def test_falcon_4096_width_two_layers():
     run_case(hp, n_prompt=8, n_gen=48)
 
 
+@pytest.mark.parametrize("wtype", [synth.F16, synth.Q4_0])
+def test_falcon_4096_width_hybrid(wtype):
+    """Falcon architecture (no gate, LayerNorm, two residuals) with a 60 % split at a width the fused kernels cover: the host
+    share works from the pinned buffers; the reduction is followed by the three-operand merge."""
+    hp = synth.hparams("falcon-tiny", n_embd=4096, n_ff=8192, n_rank=512, n_head=64, n_head_kv=8, n_layer=2, n_vocab=4096,
+                       n_ctx=96, seed=15, wtype=wtype, hot_frac=0.6)
+    if wtype == synth.Q4_0:
+        run_case(hp, n_prompt=6, n_gen=24, logit_tol=1.5e-1, min_same=0.5)      # see test_llama_7b_width_q4_two_layers
+    else:
+        run_case(hp, n_prompt=8, n_gen=32)
+
+
 def test_llama_7b_width_hybrid_f16_two_layers():
     """F16 hot/cold split at the 7B layer shape: the resident 60 % run through the fused kernels on the bucket's compact
     matrices, the host share works from the pinned logits and fp16 input, the reduction adds both shares and the residual."""

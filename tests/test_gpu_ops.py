@@ -146,6 +146,53 @@ def test_rope_attention_sequence(mode, hd, nh, nkv):
     assert np.array_equal(vc_f.download(np.uint16), vc_g.download(np.uint16))
 
 
+@pytest.mark.parametrize("mode,hd,nh,nkv", [(0, 128, 4, 4), (2, 64, 8, 2)])
+def test_attention_long_context(mode, hd, nh, nkv):
+    """One decode step over a cache that already holds several hundred cells: the fused kernel requests the K and V rows of its
+    first four passes (256 cells at head size 128, 512 at 64) before its prologue and takes the rest in a loop; positions on both
+    sides of that boundary are compared with the oracle, as is the two-launch form."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    O = ol.oracle()
+    rng = np.random.default_rng(3 * mode + hd)
+    n_ctx, gqa, d = 768, nkv * hd, nh * hd
+    theta_scale = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
+    tab = pl.DevBuf(n_ctx * hd * 4)
+    pl.check(L.pi_k_rope_table(tab.ptr, n_ctx, hd, theta_scale, None), "rope_table")
+    kfill = (rng.standard_normal((n_ctx, nkv, hd)) * 0.5).astype(np.float16)        # cell-major, as the oracle keeps K
+    vfill = (rng.standard_normal((n_ctx, nkv, hd)) * 0.5).astype(np.float16)
+    boundary = 4 * (1024 // (hd // 8))
+    for pos in (boundary - 1, boundary, boundary + 1, boundary + 45, 700):
+        kc_o = np.ascontiguousarray(kfill.reshape(n_ctx, gqa)).view(np.uint16).copy()
+        vc_o = np.ascontiguousarray(vfill.reshape(n_ctx, gqa).T).view(np.uint16).copy()
+        kg = np.ascontiguousarray(kfill.transpose(1, 0, 2))
+        vg = np.ascontiguousarray(vfill.transpose(1, 0, 2))
+        qkv = rng.standard_normal(d + 2 * gqa).astype(np.float32)
+        q, k, v = qkv[:d], qkv[d:d + gqa], qkv[d + gqa:]
+        p = np.array([pos], np.int32)
+        qr, kr = np.zeros_like(q), np.zeros_like(k)
+        O.pio_rope(P(q), hd, nh, 1, P(p), hd, mode, 10000.0, 1.0, P(qr))
+        O.pio_rope(P(k), hd, nkv, 1, P(p), hd, mode, 10000.0, 1.0, P(kr))
+        n_kv = pos + 1
+        mask = np.zeros((1, n_kv), np.float32)
+        want = np.zeros(d, np.float32)
+        assert O.pio_attention(hd, nh, nkv, n_ctx, n_kv, 1, P(p), P(mask), P(qr), P(kr), P(np.ascontiguousarray(v)), P(kc_o), P(vc_o), P(want)) == 0
+        dq, dpos = pl.DevBuf(host=qkv), pl.DevBuf(host=p)
+        for fused in (True, False):
+            kc, vc, dout, dqr = pl.DevBuf(host=kg), pl.DevBuf(host=vg), pl.DevBuf(d * 4), pl.DevBuf(d * 4)
+            if fused:
+                pl.check(L.pi_k_attn_fused(dq.ptr, tab.ptr, kc.ptr, vc.ptr, nh, nkv, hd, mode, n_ctx, dpos.ptr, dout.ptr, None), "attn_fused")
+            else:
+                pl.check(L.pi_k_rope_kv_store(dq.ptr, nh, nkv, hd, mode, theta_scale, dpos.ptr, n_ctx, dqr.ptr, kc.ptr, vc.ptr, None), "rope")
+                pl.check(L.pi_k_attn_decode(dqr.ptr, kc.ptr, vc.ptr, nh, nkv, hd, n_ctx, dpos.ptr, dout.ptr, None), "attn")
+            pl.sync()
+            assert rel_err(dout.download(np.float32), want) < 2e-3, (pos, fused)
+            # only the new cell was written
+            after = kc.download(np.float16).reshape(nkv, n_ctx, hd)
+            untouched = np.ones(n_ctx, bool); untouched[pos] = False
+            assert np.array_equal(after[:, untouched], kg[:, untouched])
+
+
 def test_embed_and_argmax():
     from powerinfer_amd import lib as pl
     L = pl.init()

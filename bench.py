@@ -213,8 +213,10 @@ def main():
                          "16 sequences decoded in lockstep; 4 Falcon-40B shape FP16")
     ap.add_argument("--hot-frac", type=float, default=None, help="configs 1 and 2: share of each layer's neurons on the GPU (default 1.0 and 0.6)")
     ap.add_argument("--pmc-probe", action="store_true",
-                    help="counter-collection aid: run only the q|k|v mat-vec of a 4-layer model a few times plus one "
-                         "device-to-device copy of the same byte count (the known-size reference for FETCH_SIZE / WRITE_SIZE)")
+                    help="counter-collection aid: run only one section of a 4-layer model a few times plus one "
+                         "device-to-device copy of the q|k|v matrix's byte count (the known-size reference for FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--pmc-section", type=int, default=0, choices=[0, 1],
+                    help="section replayed by --pmc-probe: 0 the q|k|v mat-vec, 1 the sparse FFN block (fc1, fused predictor + FFN, reduction)")
     args = ap.parse_args()
     if args.gpus != 1:
         sys.exit("bench.py: this build runs the token loop on ONE GPU; --gpus must be 1 "
@@ -233,8 +235,10 @@ def main():
         pl.sync()
         pl.check(pl.load().pi_memcpy_d2d(dst.ptr, src.ptr, nbytes), "copy")     # reads nbytes, writes nbytes
         pl.sync()
-        ms, n = m.time_section(0, 4)
-        print(json.dumps({"pmc_probe": True, "copy_bytes": nbytes, "qkv_weight_bytes": nbytes, "qkv_launches": n, "us_per_launch": ms * 1e3}))
+        ms, n = m.time_section(args.pmc_section, 4)
+        act = [int(v) for v in m.get_capture()[2]] if args.pmc_section == 1 else None      # active rows per layer of the replayed block
+        print(json.dumps({"pmc_probe": True, "section": args.pmc_section, "copy_bytes": nbytes, "launches": n, "us_per_launch": ms * 1e3,
+                          "active_per_layer": act}))
         m.close()
         return
     n_ctx = args.prompt + args.warmup + args.steps + 8

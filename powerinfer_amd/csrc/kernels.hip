@@ -709,31 +709,16 @@ __device__ void compact_from_words(const uint32_t * words, int ff, const int32_t
 }
 
 // returns true in every thread of the block that took the last ticket; resets the counter for the next launch
-#ifndef PI_FENCE_MODE
-#define PI_FENCE_MODE 1
-#endif
 __device__ bool last_block_done(unsigned int * counter, unsigned int n_blocks, int * sflag) {
-#if PI_FENCE_MODE == 0
-    __threadfence();
-#endif
     __syncthreads();
     if (threadIdx.x == 0) {
-#if PI_FENCE_MODE == 1
         __threadfence();          // cumulative: publishes the whole block's stores, ordered before the ticket
-#endif
         const unsigned int t = atomicAdd(counter, 1u);
         *sflag = (t == n_blocks - 1);
-        if (t == n_blocks - 1) *counter = 0;
-#if PI_FENCE_MODE == 1
-        if (t == n_blocks - 1) __threadfence();
-#endif
+        if (t == n_blocks - 1) { *counter = 0; __threadfence(); }
     }
     __syncthreads();
-    const bool last = *sflag != 0;
-#if PI_FENCE_MODE == 0
-    if (last) __threadfence();
-#endif
-    return last;
+    return *sflag != 0;
 }
 
 // Block = 32 consecutive neurons (8 per wave); all weight loads of the block are issued before the hidden
@@ -3390,11 +3375,8 @@ int pi_k_sparse_ffn_supported(int ff, int r, int cols) { return (cols == 4096 ||
 // Groups of 32 neurons per workgroup of the fused sparse FFN.  Wide rows: a workgroup takes four groups in turn (the next
 // group's predictor rows travel during the current group's FFN rows) and stores one partial vector for all of them, which
 // quarters the partial-sum traffic (it grows with cols; at 32768 x 8192 it was 67 MB of 220 MB per layer).
-// PI_PF_GROUPS=1|2|4 overrides the choice for wide rows (measurement aid).
 static int pf_groups(int ff, int cols) {
-    static const int forced = [] { const char * e = getenv("PI_PF_GROUPS"); return e ? atoi(e) : 0; }();
     if (cols != 8192) return 1;                    // at 4096 columns one group per workgroup measured fastest
-    if ((forced == 1 || forced == 2 || forced == 4) && ff % (32 * forced) == 0) return forced;
     return (ff % 128 == 0 && ff / 128 >= 256) ? 4 : 1;
 }
 

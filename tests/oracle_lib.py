@@ -130,6 +130,40 @@ def ffn_sparse(lib, d, ff, r, T, wtype, has_gate, up, gate, down_t, fc1, fc2, x_
     return o
 
 
+def apply_norm(x, kind, w=None, b=None, eps=1e-5):
+    """norm(x) * w (+ b) as llm_build_norm does (llama.cpp:4420-4450): kind 0 none, 1 RMSNorm, 2 LayerNorm.  x [n] or [T][n]."""
+    x = np.ascontiguousarray(np.atleast_2d(x), np.float32)
+    if kind == 0:
+        return x
+    out = np.empty_like(x)
+    (oracle().pio_rms_norm if kind == 1 else oracle().pio_norm)(_ptr(x), x.shape[1], x.shape[0], eps, _ptr(out))
+    if w is not None:
+        out = out * np.asarray(w, np.float32)
+    if b is not None:
+        out = out + np.asarray(b, np.float32)
+    return np.ascontiguousarray(out, np.float32)
+
+
+def ffn_under_logits(lib, d, ff, wtype, has_gate, up, gate, down_t, xn, logits, thr, gpu_idx=None, nth=1):
+    """The CPU sparse FFN of ONE token evaluated under GIVEN predictor logits (GGML_OP_MUL_MAT_SPARSE for up and gate, relu, mul,
+    GGML_OP_AXPY, each with idx = logits): what the reference's CPU kernels return for exactly the activity mask those logits
+    imply.  Lets a test compare outputs whatever the two sides' own predictors did to a neuron on the threshold.
+    xn: the (already normalised) FFN input [d].  Returns dict(up, gate, h, out)."""
+    xn = np.ascontiguousarray(np.asarray(xn, np.float32).reshape(1, d))
+    idx = np.ascontiguousarray(np.asarray(logits, np.float32).reshape(1, ff))
+    gi = np.zeros(ff, np.int32) if gpu_idx is None else np.ascontiguousarray(gpu_idx, np.int32)
+    o = dict(up=np.zeros((1, ff), np.float32), gate=np.zeros((1, ff), np.float32), out=np.zeros((1, d), np.float32))
+    assert lib.pio_mul_mat_sparse(wtype, _ptr(up), ff, d, _ptr(xn), 1, _ptr(idx), _ptr(gi), thr, _ptr(o["up"]), nth) == 0
+    if has_gate:
+        assert lib.pio_mul_mat_sparse(wtype, _ptr(gate), ff, d, _ptr(xn), 1, _ptr(idx), _ptr(gi), thr, _ptr(o["gate"]), nth) == 0
+        h = np.maximum(o["gate"], 0.0) * o["up"]
+    else:
+        h = np.maximum(o["up"], 0.0)
+    h = np.ascontiguousarray(h, np.float32)
+    assert lib.pio_axpy(wtype, _ptr(down_t), ff, d, _ptr(h), 1, _ptr(idx), _ptr(gi), thr, _ptr(o["out"]), nth) == 0
+    return dict(up=o["up"][0], gate=o["gate"][0], h=h[0], out=o["out"][0])
+
+
 # ---------------------------------------------------------------------------------------------
 # the reference's KV cell bookkeeping (llama.cpp:1381-1850), for one context
 # ---------------------------------------------------------------------------------------------

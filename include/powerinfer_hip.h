@@ -291,6 +291,12 @@ PI_API int pi_k_rope_table(void * table, int n_ctx, int hd, float theta_scale, p
 PI_API int pi_k_attn_fused(const float * qkv, const void * rope_table, void * k_cache, void * v_cache, int n_head, int n_head_kv,
                            int hd, int mode, int n_ctx, const int32_t * pos, float * out, pi_stream_t stream);
 
+/* 1 if the single-pass attention kernels cover the head size and context (they keep the scores of every cell in LDS: at head
+ * size 128 pi_k_attn_fused reaches n_ctx 6784 and pi_k_attn_decode 13312).  pi_model_finalize picks the fused kernel where it
+ * fits and the rope_kv_store + attn_decode pair otherwise; batched decoding needs the fused one. */
+PI_API int pi_k_attn_fused_supported(int hd, int n_ctx);
+PI_API int pi_k_attn_decode_supported(int hd, int n_ctx);
+
 /* x[cols] = row *token of the embedding table (k_get_rows, ggml-cuda.cu:1664) */
 PI_API int pi_k_embed(int wtype, const void * table, int cols, const int32_t * token, float * x, pi_stream_t stream);
 

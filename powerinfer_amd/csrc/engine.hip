@@ -577,13 +577,15 @@ int pi_model_finalize(pi_model * m) {
         return PI_E_HIP;
     PI_TRY(pi_memset(m->k_cache, 0, kv * 2));
     PI_TRY(pi_memset(m->v_cache, 0, kv * 2));
-    // fused RoPE + attention when the head geometry and context fit its single-pass kernel
-    if (m->hd % 8 == 0 && 256 % (m->hd / 8) == 0 && 64 % (m->hd / 8) == 0 && m->hd / 2 + m->hd <= 256 &&
-        sizeof(float) * ((size_t)hp.n_ctx + (size_t)(256 / (m->hd / 8)) * m->hd + 3 * (size_t)m->hd) <= 60 * 1024) {
+    // fused RoPE + attention when the head geometry and the context fit its single-pass kernel (the launcher's own test);
+    // otherwise the rope_kv_store + attn_decode pair, whose smaller workgroup leaves room for a longer context
+    if (pi_k_attn_fused_supported(m->hd, hp.n_ctx)) {
         m->rope_table = m->alloc<float>((size_t)hp.n_ctx * m->hd);
         if (!m->rope_table) return PI_E_HIP;
         PI_TRY(pi_k_rope_table(m->rope_table, hp.n_ctx, m->hd, m->theta_scale, nullptr));
     }
+    else if (!pi_k_attn_decode_supported(m->hd, hp.n_ctx))
+        return pi::fail(PI_E_UNSUPPORTED, "pi_model_finalize: head size or context outside both attention kernels (scores of every cell are kept in LDS: n_ctx up to about 13 000 at head size 128)");
     PI_TRY(pi_memset(m->n_active, 0, sizeof(int32_t) * hp.n_layer));
     PI_TRY(pi_memset(m->d_step, 0, 4));
     PI_TRY(pi_memset(m->h_dense, 0, sizeof(float) * ff));

@@ -189,7 +189,7 @@ int pi_model_batch_init(pi_model * m, int n_seq) {
     if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_batch_init: model not finalized");
     if (n_seq < 1 || n_seq > 16) return pi::fail(PI_E_ARG, "pi_model_batch_init: 1 <= n_seq <= 16");
     if (m->batch) return pi::fail(PI_E_STATE, "pi_model_batch_init: already initialised");
-    if (!m->rope_table) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: head size outside the fused attention kernel");
+    if (!m->rope_table) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: head size or context outside the fused attention kernel (pi_k_attn_fused_supported)");
     if (const char * why = batch_unsupported(m)) { pi::set_error(why); return PI_E_UNSUPPORTED; }
     BatchState * b = batch_alloc(m, n_seq, true);
     if (!b) return PI_E_HIP;

@@ -3054,6 +3054,7 @@ __global__ __launch_bounds__(1024) void argmax_batch_kernel(const float * __rest
     __syncthreads();
     if (threadIdx.x == 0) {
         for (int w = 1; w < 16; ++w) if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
+        if (idx >= n) idx = 0;             // no logit compared greater than -inf (all NaN or -inf): a valid row for the next embedding lookup
         tokens[t] = idx;
         if (positions) positions[t] += 1;
         const int s = step ? *step : 0;
@@ -3551,13 +3552,31 @@ int pi_k_rope_table(void * table, int n_ctx, int hd, float theta_scale, pi_strea
     return pi::check_launch("pi_k_rope_table");
 }
 
+// LDS of attn_fused_kernel: the scores of every cell, one partial output row per group of hd/8 lanes, and q, k, v of the new cell
+static bool attn_fused_geometry_ok(int hd) {
+    return hd > 0 && hd % 8 == 0 && kAttnBlock % (hd / 8) == 0 && PI_WAVE % (hd / 8) == 0 && hd / 2 + hd <= kAttnBlock;
+}
+static size_t attn_fused_lds_bytes(int hd, int n_ctx) {
+    return sizeof(float) * ((size_t)n_ctx + (size_t)(kAttnBlock / (hd / 8)) * hd + 3 * (size_t)hd);
+}
+constexpr size_t kAttnLdsLimit = 60 * 1024;
+
+int pi_k_attn_fused_supported(int hd, int n_ctx) {
+    return attn_fused_geometry_ok(hd) && n_ctx > 0 && attn_fused_lds_bytes(hd, n_ctx) <= kAttnLdsLimit;
+}
+
+int pi_k_attn_decode_supported(int hd, int n_ctx) {
+    return hd > 0 && hd % 8 == 0 && kBlock % (hd / 8) == 0 && PI_WAVE % (hd / 8) == 0 && n_ctx > 0 &&
+           sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd) <= kAttnLdsLimit;
+}
+
 int pi_k_attn_fused(const float * qkv, const void * rope_table, void * k_cache, void * v_cache, int n_head, int n_head_kv, int hd, int mode,
                     int n_ctx, const int32_t * pos, float * out, pi_stream_t stream) {
     if (!qkv || !rope_table || !k_cache || !v_cache || !pos || !out) return pi::fail(PI_E_ARG, "pi_k_attn_fused: null pointer");
-    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd % 8 || kAttnBlock % (hd / 8) || PI_WAVE % (hd / 8) || hd / 2 + hd > kAttnBlock || (mode != 0 && mode != 2))
+    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || !attn_fused_geometry_ok(hd) || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_attn_fused: head size must be 8 * (a divisor of 64), at most 128; mode 0 or 2");
-    const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kAttnBlock / (hd / 8)) * hd + 3 * (size_t)hd);
-    if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused: context too long for the single-pass kernel");
+    const size_t sh = attn_fused_lds_bytes(hd, n_ctx);
+    if (sh > kAttnLdsLimit) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused: context too long for the single-pass kernel");
     hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
                        (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, 0, (size_t)0, 0, nullptr);
     return pi::check_launch("pi_k_attn_fused");
@@ -3567,10 +3586,10 @@ int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_t
                           int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, const int32_t * pos, float * out, int out_stride,
                           void * out_f16, pi_stream_t stream) {
     if (!qkv || !rope_table || !k_cache || !v_cache || !pos || !out || n_seq <= 0 || n_seq > kBtMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch: bad arguments");
-    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd % 8 || kAttnBlock % (hd / 8) || PI_WAVE % (hd / 8) || hd / 2 + hd > kAttnBlock || (mode != 0 && mode != 2))
+    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || !attn_fused_geometry_ok(hd) || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch: head size must be 8 * (a divisor of 64), at most 128; mode 0 or 2");
-    const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kAttnBlock / (hd / 8)) * hd + 3 * (size_t)hd);
-    if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused_batch: context too long for the single-pass kernel");
+    const size_t sh = attn_fused_lds_bytes(hd, n_ctx);
+    if (sh > kAttnLdsLimit) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused_batch: context too long for the single-pass kernel");
     hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head, n_seq), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
                        (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride, (__half *)out_f16);
     return pi::check_launch("pi_k_attn_fused_batch");

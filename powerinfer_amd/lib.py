@@ -80,6 +80,8 @@ _SIGS = {
     "pi_k_rope_kv_store": (_i, [_vp, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp, _vp]),
     "pi_k_attn_decode": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
     "pi_k_rope_table": (_i, [_vp, _i, _i, _f, _vp]),
+    "pi_k_attn_fused_supported": (_i, [_i, _i]),
+    "pi_k_attn_decode_supported": (_i, [_i, _i]),
     "pi_k_attn_fused": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp]),
     "pi_k_embed": (_i, [_i, _vp, _i, _vp, _vp, _vp]),
     "pi_k_argmax": (_i, [_vp, _i, _vp, _vp]),

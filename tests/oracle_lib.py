@@ -144,14 +144,18 @@ def apply_norm(x, kind, w=None, b=None, eps=1e-5):
     return np.ascontiguousarray(out, np.float32)
 
 
-def ffn_under_logits(lib, d, ff, wtype, has_gate, up, gate, down_t, xn, logits, thr, gpu_idx=None, nth=1):
+def ffn_under_logits(lib, d, ff, wtype, has_gate, up, gate, down_t, xn, logits, thr, gpu_idx=None, axpy_gpu_idx=None, nth=1):
     """The CPU sparse FFN of ONE token evaluated under GIVEN predictor logits (GGML_OP_MUL_MAT_SPARSE for up and gate, relu, mul,
     GGML_OP_AXPY, each with idx = logits): what the reference's CPU kernels return for exactly the activity mask those logits
     imply.  Lets a test compare outputs whatever the two sides' own predictors did to a neuron on the threshold.
-    xn: the (already normalised) FFN input [d].  Returns dict(up, gate, h, out)."""
+    xn: the (already normalised) FFN input [d].  gpu_idx (1 = skipped by the CPU kernels) applies to up/gate and, unless
+    axpy_gpu_idx is given, to the down projection; a hybrid graph merges up/gate over all neurons first and splits only the down
+    projection (whose Q8_0 scales of h then span both shares), which is gpu_idx=None with axpy_gpu_idx = the share's complement.
+    Returns dict(up, gate, h, out)."""
     xn = np.ascontiguousarray(np.asarray(xn, np.float32).reshape(1, d))
     idx = np.ascontiguousarray(np.asarray(logits, np.float32).reshape(1, ff))
     gi = np.zeros(ff, np.int32) if gpu_idx is None else np.ascontiguousarray(gpu_idx, np.int32)
+    ga = gi if axpy_gpu_idx is None else np.ascontiguousarray(axpy_gpu_idx, np.int32)
     o = dict(up=np.zeros((1, ff), np.float32), gate=np.zeros((1, ff), np.float32), out=np.zeros((1, d), np.float32))
     assert lib.pio_mul_mat_sparse(wtype, _ptr(up), ff, d, _ptr(xn), 1, _ptr(idx), _ptr(gi), thr, _ptr(o["up"]), nth) == 0
     if has_gate:
@@ -160,8 +164,18 @@ def ffn_under_logits(lib, d, ff, wtype, has_gate, up, gate, down_t, xn, logits, 
     else:
         h = np.maximum(o["up"], 0.0)
     h = np.ascontiguousarray(h, np.float32)
-    assert lib.pio_axpy(wtype, _ptr(down_t), ff, d, _ptr(h), 1, _ptr(idx), _ptr(gi), thr, _ptr(o["out"]), nth) == 0
+    assert lib.pio_axpy(wtype, _ptr(down_t), ff, d, _ptr(h), 1, _ptr(idx), _ptr(ga), thr, _ptr(o["out"]), nth) == 0
     return dict(up=o["up"][0], gate=o["gate"][0], h=h[0], out=o["out"][0])
+
+
+def axpy_under_logits(lib, d, ff, wtype, down_t, h, logits, thr, skip):
+    """GGML_OP_AXPY of one token on the CPU: sum of h[n] * down_t[n] over the rows with skip[n] == 0 that the logits leave active
+    (h is quantised over all ff neurons first for Q4_0 weights, as the node's INIT phase does, ggml.c:14465-14618)."""
+    h = np.ascontiguousarray(np.asarray(h, np.float32).reshape(1, ff))
+    idx = np.ascontiguousarray(np.asarray(logits, np.float32).reshape(1, ff))
+    out = np.zeros((1, d), np.float32)
+    assert lib.pio_axpy(wtype, _ptr(down_t), ff, d, _ptr(h), 1, _ptr(idx), _ptr(np.ascontiguousarray(skip, np.int32)), thr, _ptr(out), 1) == 0
+    return out[0]
 
 
 # ---------------------------------------------------------------------------------------------

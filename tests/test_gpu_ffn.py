@@ -18,6 +18,12 @@ def rel_err(a, b):
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
 
 
+def under(L, d, ff, wtype, has_gate, xn, logits, thr=0.0, gpu_idx=None):
+    """The CPU oracle's FFN for the mask the GPU's own predictor logits imply: the output comparison then never depends on a
+    neuron whose logit sits on the threshold having fallen the same way on both sides."""
+    return ol.ffn_under_logits(ol.oracle(), d, ff, wtype, has_gate, L["up"], L["gate"], L["down_t"], xn, logits, thr, gpu_idx)
+
+
 def check_token(g, o, ff, thr=0.0, gid=None):
     """g: GPU result dict for one token, o: oracle dict rows for the same token."""
     mask_g = np.zeros(ff, bool)
@@ -71,12 +77,12 @@ def test_ffn_7b_shape_vs_oracle(wtype, has_gate):
     for t in range(T):
         res = ffn.forward(L["x"][t], L["x"][t])
         ot = {k: v[t] for k, v in o.items()}
-        same = check_token(res, ot, ff)
+        check_token(res, ot, ff)
         assert 600 < res["active"].size < 1700
-        if same.all():
-            assert rel_err(res["h"], ot["h"]) < 1e-4
-            assert rel_err(res["out"], ot["out"]) < FFN_REL_TOL
-            assert rel_err(res["out"], ot["out"]) < 1e-4      # in practice: fp32 summation order only
+        ou = under(L, d, ff, wtype, has_gate, L["x"][t], res["logits"])
+        assert rel_err(res["up"], ou["up"]) < 1e-5
+        assert rel_err(res["h"], ou["h"]) < 1e-4
+        assert rel_err(res["out"], ou["out"]) < (1e-4 if wtype == ol.F16 else FFN_REL_TOL)      # F16: fp32 summation order only
         # fused route (what the decode loop runs): the up/gate kernel builds the list from the mask words itself
         fus = ffn.forward(L["x"][t], L["x"][t], dense_outputs=False)
         assert np.array_equal(fus["active"], res["active"])
@@ -134,9 +140,9 @@ def run_fused_route(has_gate, norm, route, d, ff, r, T=3, mean_rate=0.10):
         assert res["n_active"] == int(mask_g.sum())
         assert not np.isnan(res["h"]).any()
         assert np.all(res["h"][~mask_g] == 0.0)               # every inactive neuron written as 0
-        if np.array_equal(mask_g, mask_o):
-            assert rel_err(res["h"], o["h"][0]) < 1e-4
-            assert rel_err(res["out"] - resid, o["out"][0]) < 1e-4
+        ou = under(L, d, ff, ol.F16, has_gate, xn, res["logits"])
+        assert rel_err(res["h"], ou["h"]) < 1e-4
+        assert rel_err(res["out"] - resid, ou["out"]) < 1e-4
     ffn.close()
 
 
@@ -198,9 +204,9 @@ def test_q4_fused_route_7b_shape(has_gate, norm):
         qo, do = q8_blocks_np(xn[0])
         assert np.abs(qg - qo).max() <= 1 and (qg != qo).mean() < 1e-3
         assert np.allclose(dg, do, rtol=2e-3)
-        if np.array_equal(mask_g, mask_o):
-            assert rel_err(res["h"], o["h"][0]) < 1e-4
-            assert rel_err(res["out"] - resid, o["out"][0]) < FFN_REL_TOL     # an int8 step of h where h * 127/amax sits on a rounding boundary
+        ou = under(L, d, ff, ol.Q4_0, has_gate, xn, res["logits"])
+        assert rel_err(res["h"], ou["h"]) < 1e-4
+        assert rel_err(res["out"] - resid, ou["out"]) < FFN_REL_TOL     # an int8 step of h where h * 127/amax sits on a rounding boundary
     ffn.close()
 
 
@@ -233,9 +239,10 @@ def test_f16_fused_route_hybrid_share(has_gate, norm):
         assert res["n_active"] == int((mask_g & (gid == 1)).sum())
         assert np.all(res["h"][gid == 0] == 0.0) and np.all(res["h"][~mask_g] == 0.0)
         assert (res["xn16"] != xn[0].astype(np.float16)).mean() < 1e-3              # a last-place step of the norm at most
-        if np.array_equal(mask_g, mask_o):
-            assert rel_err(res["h"], share["h"][0]) < 1e-4
-            assert rel_err(res["out"], share["out"][0]) < 1e-4
+        assert (mask_g == mask_o).mean() >= MASK_AGREE
+        su = under(L, d, ff, ol.F16, has_gate, xn, res["logits"], gpu_idx=1 - gid)      # the resident neurons only, under the GPU's mask
+        assert rel_err(res["h"], su["h"]) < 1e-4
+        assert rel_err(res["out"], su["out"]) < 1e-4
     ffn.close()
 
 
@@ -252,26 +259,29 @@ def test_q4_fused_route_hybrid_share():
     ffn = SparseFFN(d, ff, r, ol.Q4_0, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], bucket=bucket)
     for t in range(T):
         cold = gid == 0
+        got = {}
 
         def fill(h):
             assert np.all(h[cold] == 0.0)                       # the kernel writes zeros outside its share
-            h[cold] = full["h"][t][cold]
+            # every neuron on the CPU under the logits the GPU just produced: the cold neurons' h comes from there
+            got["full"] = under(L, d, ff, ol.Q4_0, True, L["x"][t], ffn.logits.download(np.float32))
+            h[cold] = got["full"]["h"][cold]
             return h
 
         res = ffn.forward_q4_fused(L["x"][t], L["x"][t], fill_h=fill)
+        fu = got["full"]
         mask_g, mask_o = ~(res["logits"] < 0.0), ~(full["logits"][t] < 0.0)
         assert rel_err(res["logits"], full["logits"][t]) < 1e-4
+        assert (mask_g == mask_o).mean() >= MASK_AGREE
         assert res["n_active"] == int((mask_g & ~cold).sum())
-        if not np.array_equal(mask_g, mask_o):
-            continue
-        assert rel_err(res["h"][~cold], full["h"][t][~cold]) < 1e-4
-        hm = res["h"].copy(); hm[cold] = full["h"][t][cold]
+        assert rel_err(res["h"][~cold], fu["h"][~cold]) < 1e-4
+        hm = res["h"].copy(); hm[cold] = fu["h"][cold]
         q, dh = q8_blocks_np(hm)
         rows = np.nonzero(cold & (q != 0))[0]
         v, dw = q4_rows_np(L["down_t"], rows, d)
         contrib = (v * q[rows, None]).astype(np.float32) * (np.repeat(dw, 32, axis=1) * dh[rows, None])
         cold_out = contrib.sum(0, dtype=np.float32)
-        assert rel_err(res["out"] + cold_out, full["out"][t]) < FFN_REL_TOL
+        assert rel_err(res["out"] + cold_out, fu["out"]) < FFN_REL_TOL
     ffn.close()
 
 
@@ -292,9 +302,11 @@ def test_hybrid_split_gpu_share(wtype):
         res = ffn.forward(L["x"][t], L["x"][t])
         check_token(res, {k: v[t] for k, v in full.items()}, ff, gid=bucket)
         assert (res["up"][gid == 0] == 0).all()                # upscale writes bucket positions only
-        assert rel_err(res["up"], gpu_share["up"][t]) < 1e-5
+        su = under(L, d, ff, wtype, True, L["x"][t], res["logits"], gpu_idx=1 - gid)      # the GPU's neurons under the GPU's mask
+        assert rel_err(res["up"], su["up"]) < 1e-5
+        assert rel_err(res["logits"], gpu_share["logits"][t]) < 1e-4
         if wtype == ol.F16:                                    # Q8_0 scales of h need the merged h (tested at model level)
-            assert rel_err(res["out"], gpu_share["out"][t]) < 1e-4
+            assert rel_err(res["out"], su["out"]) < 1e-4
     ffn.close()
 
 
@@ -337,8 +349,9 @@ def test_fused_routes_thresholds_none_some_all(route):
             assert res["n_active"] == 0 and (res["out"] == 0).all() and (res["h"] == 0).all()
         if thr == -1e9:
             assert res["n_active"] == ff
-        if np.array_equal(mask_g, mask_o):
-            assert np.abs(res["out"] - o["out"][0]).max() <= 1e-4 * max(np.abs(o["out"][0]).max(), 1e-6)
+        assert (mask_g == mask_o).mean() >= MASK_AGREE
+        ou = under(L, d, ff, ol.F16, True, L["x"][0], res["logits"], thr)
+        assert np.abs(res["out"] - ou["out"]).max() <= 1e-4 * max(np.abs(ou["out"]).max(), 1e-6)
         ffn.close()
 
 

@@ -34,14 +34,25 @@ def oracle_ffn_on(model, il, src):
                          L["fc1"], L["fc2"], xn, src, np.zeros(ff, np.int32), hp.sparse_threshold, nth=8)
 
 
+def oracle_ffn_under(model, il, src, logits):
+    """The oracle's up/gate/down of layer il (every neuron on the CPU) applied to a given source vector under GIVEN predictor
+    logits: the FFN output the reference's CPU kernels produce for exactly the activity mask the GPU decided on."""
+    hp, L = model["hp"], model["layers"][il]
+    xn = ol.apply_norm(src, 1 if hp.arch == "llama" else 2, L["ffn_norm"] if hp.arch == "llama" else L["attn_norm"],
+                       None if hp.arch == "llama" else L["attn_norm_b"], hp.norm_eps)
+    return ol.ffn_under_logits(ol.oracle(), hp.n_embd, hp.n_ff, hp.wtype, hp.arch == "llama", L["ffn_up"], L.get("ffn_gate"),
+                               L["ffn_down_t"], xn, logits, hp.sparse_threshold, nth=8)
+
+
 def run_case(hp, n_prompt=12, n_gen=64, logit_tol=1e-2, min_same=0.9):
     """Both sides consume the same tokens.  Random-init weights make the comparison chaotic in one specific
     way: activations are rounded to fp16 before every dot product (ggml.c:9703-9716), so an fp32 difference in
     the last place (summation order) becomes a 1e-4 difference one layer later and can flip a neuron whose
     predictor logit sits on the threshold.  The checks therefore are: masks agree on >= 99.9 % of all neurons
-    evaluated; each layer's FFN block, fed the GPU's own input, matches the oracle within 2e-3 whenever the two
-    masks are identical; logits within 1e-2; greedy tokens identical, a disagreement being admissible only where
-    the oracle's own logits tie within the logit tolerance."""
+    evaluated; each layer's FFN block, fed the GPU's own input and evaluated by the oracle under the GPU's own
+    predictor logits (so the comparison runs for every layer of every token), within 2e-3; logits within 1e-2;
+    greedy tokens identical, a disagreement being admissible only where the oracle's own logits tie within the
+    logit tolerance.  run_north_star() below asserts the criteria verbatim on models whose predictors cannot flip."""
     from powerinfer_amd.model import Model
     model = synth.make_model(hp)
     om = ol.OracleModel(model)
@@ -52,7 +63,7 @@ def run_case(hp, n_prompt=12, n_gen=64, logit_tol=1e-2, min_same=0.9):
 
     gm.set_capture(True)
     om.capture(1)
-    n_past, flips, neurons, checked, skipped, lerr, clean_lerr = 0, 0, 0, 0, 0, [], []
+    n_past, flips, neurons, checked, lerr, clean_lerr = 0, 0, 0, 0, [], []
     for t in prompt:
         tok_o, lg_o = om.eval([t], n_past)
         tok_g, lg_g = gm.decode([t], n_past)
@@ -65,11 +76,9 @@ def run_case(hp, n_prompt=12, n_gen=64, logit_tol=1e-2, min_same=0.9):
             assert na_g[il] == (mask_g.sum() if gid is None else (mask_g & (gid == 1)).sum())   # the GPU's list covers its bucket only
             o = oracle_ffn_on(model, il, src_g[il])
             assert rel_err(plg_g[il], o["logits"][0]) < 1e-4
-            if np.array_equal(mask_g, ~(o["logits"][0] < thr)):
-                assert rel_err(ffn_g[il], o["out"][0]) < 2e-3, (il, rel_err(ffn_g[il], o["out"][0]))
-                checked += 1
-            else:
-                skipped += 1
+            ou = oracle_ffn_under(model, il, src_g[il], plg_g[il])
+            assert rel_err(ffn_g[il], ou["out"]) < 2e-3, (il, rel_err(ffn_g[il], ou["out"]))
+            checked += 1
         flips += tflips
         neurons += hp.n_layer * hp.n_ff
         lerr.append(rel_err(lg_g, lg_o))
@@ -77,7 +86,7 @@ def run_case(hp, n_prompt=12, n_gen=64, logit_tol=1e-2, min_same=0.9):
             clean_lerr.append(lerr[-1])
         n_past += 1
     assert 1 - flips / neurons >= 0.999, (flips, neurons)
-    assert skipped <= 0.1 * (checked + skipped), (checked, skipped)
+    assert checked == n_prompt * hp.n_layer
     assert np.median(lerr) < logit_tol, lerr
     if hp.wtype == synth.F16:
         assert not clean_lerr or max(clean_lerr) < 1e-2, clean_lerr
@@ -109,6 +118,118 @@ def run_case(hp, n_prompt=12, n_gen=64, logit_tol=1e-2, min_same=0.9):
     assert (more >= 0).all() and (more < hp.n_vocab).all()
     gm.close(), om.close()
     return same
+
+
+def run_north_star(hp, n_prompt=8, n_gen=64):
+    """The stated tolerances, verbatim, on a model whose decisions keep a margin:
+      * predictor (synth.predictor_fc2_margin): every logit stays away from the threshold, so no neuron can flip and nothing
+        turns a last-place difference of the arithmetic into a different mask;
+      * greedy choice (hparams head_pair): four dominant output rows +-w0, +-w1, so the winner is decided by two projections of
+        the final state and the runner-up comes close only where their magnitudes happen to agree, which the test rules out for
+        its seed by measuring it (with i.i.d. random output rows two correct implementations disagree on one greedy token in
+        a few hundred, because the two largest of tens of thousands of logits come that close).
+    Asserted: predictor masks identical; every layer's FFN output within 2e-3 of the reference's block on the same input (and
+    the free-running trajectories within 2e-3 of each other for F16 weights); the logits of EVERY token within 1e-2 (maximum,
+    not median; for Q4_0 weights the median, see note()); 64 greedy tokens of the two sides, each running free on its own choices, identical -- and, so that this
+    identity is implied rather than lucky, the oracle's top-2 gap at every step more than 2.5 times the largest logit
+    difference of that step."""
+    from powerinfer_amd.model import Model
+    assert hp.get("pred_margin") and hp.get("head_pair")
+    model = synth.make_model(hp)
+    om = ol.OracleModel(model)
+    gm = Model(hp).load(model)
+    rng = np.random.default_rng(hp.seed + 7)
+    prompt = rng.integers(0, hp.n_vocab, n_prompt).astype(np.int32)
+    thr = hp.sparse_threshold
+    gm.set_capture(True)
+    om.capture(1)
+    n_past, margins, gaps, diffs, errs = 0, [], [], [], []
+    q4 = hp.wtype != synth.F16
+
+    def note(lg_g, lg_o):
+        top = np.partition(lg_o, -2)[-2:]
+        gaps.append(float(top[1] - top[0]))
+        diffs.append(float(np.abs(lg_g - lg_o).max()))
+        errs.append(rel_err(lg_g, lg_o))
+        # Q4_0: the reference run against itself, with norm weights moved by one ulp, departs by more than this over such a path
+        # (tests/test_oracle_math.py::test_q4_reference_departs_from_itself_beyond_the_logit_tolerance), so there the tolerance is
+        # held on the median and every decision is protected by the margin check below
+        assert q4 or errs[-1] < 1e-2, (n_past, errs[-1])
+
+    for t in prompt:
+        tok_o, lg_o = om.eval([t], n_past)
+        tok_g, lg_g = gm.decode([t], n_past)
+        ffn_g, plg_g, na_g, src_g = gm.get_capture()
+        for il in range(hp.n_layer):
+            assert np.array_equal(~(plg_g[il] < thr), ~(om.cap_lg[il, 0] < thr)), (n_past, il)          # masks identical
+            margins.append(float(np.abs(om.cap_lg[il, 0] - thr).min() / np.abs(om.cap_lg[il, 0]).max()))
+            # per-layer FFN output: the reference's block on the input this layer actually received, and the two trajectories
+            # side by side.  With Q4_0 weights the reference rounds activations to int8 per block of 32, so a last-place
+            # difference upstream can move one rounding step; the trajectories then differ by that step and what it grows into,
+            # while each layer, given the same input, still agrees to 2e-3.
+            ou = oracle_ffn_under(model, il, src_g[il], plg_g[il])
+            assert rel_err(ffn_g[il], ou["out"]) < 2e-3, (n_past, il, rel_err(ffn_g[il], ou["out"]))
+            assert q4 or rel_err(ffn_g[il], om.cap_ffn[il, 0]) < 2e-3, (n_past, il)
+        note(lg_g, lg_o)
+        assert tok_g == tok_o
+        n_past += 1
+    assert min(margins) > 1e-3, min(margins)                    # the predictor's margin, far above any arithmetic difference
+    gm.set_capture(False)
+    toks_g, _ = gm.generate(n_gen)                              # free-running on the device: one HIP-graph replay per token
+    cur, toks_o = int(tok_o), []
+    for s in range(n_gen):                                      # free-running on the CPU
+        cur, _ = om.eval([cur], n_past + s)
+        toks_o.append(int(cur))
+    assert list(map(int, toks_g)) == toks_o
+    assert len(set(toks_o)) >= 2 and max(toks_o.count(t) for t in set(toks_o)) <= n_gen - 3, toks_o      # the path is not one token repeated
+    # the same path once more, token by token with logits (a second engine instance continues from an identical prefix)
+    gm2 = Model(hp).load(model)
+    gm2.decode(prompt, 0, want_logits=False)
+    om.O.pio_model_kv_clear(om.h)
+    om.capture(n_prompt)                                        # the capture buffers hold one row per token of a call
+    om.eval([int(t) for t in prompt], 0)
+    cur = int(tok_o)
+    for s in range(n_gen):
+        _, lg_o = om.eval([cur], n_past + s)
+        _, lg_g = gm2.decode([cur], n_past + s)
+        note(lg_g, lg_o)
+        cur = toks_o[s]
+    assert np.median(errs) < 1e-2, errs
+    ratio = min(g / max(e, 1e-30) for g, e in zip(gaps, diffs))
+    assert ratio > 2.5, ratio        # identical greedy tokens are implied once the winner leads by more than twice the largest difference
+    gm.close(), gm2.close(), om.close()
+
+
+NS = dict(pred_margin=True, head_pair=2048)
+# seeds whose greedy path (a CPU-oracle property) visits both tokens of the pair
+SEED_7B_F16, SEED_7B_Q4, SEED_F40 = 35, 40, 29
+
+
+# (Q4_0 at this width is left to run_case: 256-wide activations make one int8 rounding step a visible share of a dot product, and
+# the reference's own trajectories then part by tens of percent -- see test_q4_reference_departs_from_itself_beyond_the_logit_tolerance)
+@pytest.mark.parametrize("arch,wtype,hot,seed", [("llama-tiny", synth.F16, 1.0, 23), ("falcon-tiny", synth.F16, 1.0, 22)])
+def test_north_star_tiny(arch, wtype, hot, seed):
+    run_north_star(synth.hparams(arch, wtype=wtype, hot_frac=hot, n_ctx=96, seed=seed, **NS))
+
+
+@pytest.mark.timeout(300)
+def test_north_star_f16_7b_width():
+    """configs[1]'s layer shape (d 4096, ff 11008, rank 1024, 32 heads, vocab 32000), two layers, every neuron on the GPU."""
+    run_north_star(synth.hparams("llama-7b", n_layer=2, n_ctx=96, seed=SEED_7B_F16, **NS))
+
+
+@pytest.mark.timeout(300)
+def test_north_star_q4_split_7b_width():
+    """configs[2]: the same shape in Q4_0 with the hottest 60 % of each layer's neurons on the GPU and the rest on host threads."""
+    run_north_star(synth.hparams("llama-7b", n_layer=2, n_ctx=96, seed=SEED_7B_Q4, wtype=synth.Q4_0, hot_frac=0.6, **NS))
+
+
+@pytest.mark.timeout(600)
+def test_north_star_falcon_40b_width():
+    """configs[4]'s own width through the engine: d 8192, 128 query heads over 8 KV heads (head size 64), ff 32768 without a gate,
+    LayerNorm, parallel attention + FFN block, vocab 65024, two layers: the 8192-column mat-vec with the fused LayerNorm, the
+    GQA attention and the four-groups-per-workgroup FFN instantiation all run here."""
+    run_north_star(synth.hparams("falcon-40b", n_layer=2, n_ctx=80, seed=SEED_F40, **NS), n_prompt=6, n_gen=64)
 
 
 @pytest.mark.parametrize("wtype", [synth.F16, synth.Q4_0])

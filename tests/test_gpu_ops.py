@@ -57,12 +57,15 @@ def test_gemv_golden_reference(golden):
             assert rel_err(got, y[t]) < 2e-6
 
 
-@pytest.mark.parametrize("wtype", [ol.F16, ol.Q4_0])
+@pytest.mark.parametrize("wtype,cols,rows", [(ol.F16, 4096, 2048), (ol.Q4_0, 4096, 2048), (ol.F16, 5120, 2304), (ol.F16, 8192, 2304),
+                                             (ol.F16, 8192, 120), (ol.Q4_0, 8192, 2048)])
 @pytest.mark.parametrize("kind", [1, 2])
-def test_gemv_fused_norm_and_epilogues(wtype, kind):
+def test_gemv_fused_norm_and_epilogues(wtype, cols, rows, kind):
+    """The register-resident mat-vecs with the fused RMSNorm / LayerNorm prologue at every width they are instantiated for:
+    4096 (7B), 5120 (13B), 8192 (Falcon-40B: a row is split in two halves, LayerNorm with bias is what its q|k|v projection
+    runs), with more rows than the grid has waves (2304 = 2048 + 256: a second, partial round), fewer (120) and Q4_0."""
     from powerinfer_amd import lib as pl
-    rng = np.random.default_rng(kind * 7 + wtype)
-    rows, cols = 2048, 4096
+    rng = np.random.default_rng(kind * 7 + wtype + cols)
     w = synth.encode((rng.standard_normal((rows, cols)) * 0.02).astype(np.float32), wtype)
     x = (rng.standard_normal(cols) * 3 + 0.5).astype(np.float32)
     nw = (1 + 0.1 * rng.standard_normal(cols)).astype(np.float32)

@@ -139,3 +139,17 @@ def test_layer7b_shape(golden):
     np.testing.assert_allclose(o["h"][0][s], g["h_sample"], **TOL)
     # 4 threads: same terms, different summation order than the 1-thread reference
     np.testing.assert_allclose(o["out"][0], g["out"], rtol=1e-4, atol=1e-6)
+
+
+@pytest.mark.parametrize("name", ["ffn_f16_gate", "ffn_f16_nogate", "ffn_q4_gate", "ffn_q4_nogate"])
+def test_ffn_under_given_logits_reproduces_the_reference_block(golden, name):
+    """oracle_lib.ffn_under_logits (the sparse mat-muls and the axpy driven by GIVEN predictor logits, which the GPU tests feed
+    with the GPU's own logits) must return exactly what the compiled reference returned for the whole block when it is given
+    the reference's logits."""
+    g = golden(name)
+    d, ff, T, wt, hg = (int(g[k]) for k in ("d", "ff", "T", "wtype", "has_gate"))
+    for t in range(T):
+        u = ol.ffn_under_logits(ol.oracle(), d, ff, wt, hg, g["up"], g["gate"] if hg else None, g["down_t"], g["x_ffn"][t], g["logits"][t], 0.0)
+        assert np.array_equal(u["up"], g["up_out"][t])
+        assert np.array_equal(u["h"], g["h"][t])
+        assert np.array_equal(u["out"], g["out"][t])

@@ -235,3 +235,34 @@ def test_reference_arithmetic_is_chaotic_under_last_bit_noise():
             worst = max(worst, float(np.abs(la - lb).max() / np.abs(la).max()))
         assert worst > floor, (wt, worst)       # 1e-7 in, > 1e-5 (F16) / > 1e-4 (Q4_0) out
         a.close(), b.close()
+
+
+def test_q4_reference_departs_from_itself_beyond_the_logit_tolerance():
+    """The 1e-2 logits tolerance is not a property the reference's Q4_0 path has against ITSELF over a 72-token trajectory: moving the
+    FFN norm weights by one fp32 ulp (less than any other summation order changes) moves some int8 roundings of the activations,
+    the difference stays in the KV cache and grows.  Both runs consume the same tokens.  With F16 weights the same experiment stays
+    near 1e-3.  Hence the model-level GPU tests hold Q4_0 logits to the tolerance on the median and protect every greedy decision
+    by its margin, and hold F16 logits to it on every token."""
+    worst = {}
+    for wt, seed in ((ol.Q4_0, 25), (ol.F16, 23)):
+        hp = synth.hparams("llama-tiny", seed=seed, wtype=wt, pred_margin=True, head_pair=2048)
+        m = synth.make_model(hp)
+        m2 = dict(hp=hp, glob=m["glob"], layers=[dict(L) for L in m["layers"]])
+        rng = np.random.default_rng(5)
+        for L in m2["layers"]:
+            w = L["ffn_norm"].copy()
+            bits = w.view(np.int32)
+            bits += rng.integers(-1, 2, bits.shape).astype(np.int32)
+            L["ffn_norm"] = w
+        a, b = ol.OracleModel(m), ol.OracleModel(m2)
+        prompt = np.random.default_rng(seed + 7).integers(0, hp.n_vocab, 8)
+        cur, w = None, 0.0
+        for s in range(72):
+            tok = int(prompt[s]) if s < 8 else cur
+            cur, la = a.eval([tok], s, nth=4)
+            _, lb = b.eval([tok], s, nth=4)
+            w = max(w, float(np.abs(la - lb).max() / np.abs(la).max()))
+        worst[wt] = w
+        a.close(), b.close()
+    assert worst[ol.Q4_0] > 1e-2, worst
+    assert worst[ol.F16] < 5e-3, worst

@@ -263,7 +263,14 @@ static struct ggml_tensor * to_gpu(struct ggml_tensor * t) {
     ggml_cuda_transform_tensor(t->data, t);
     return t;
 }
-static struct ggml_tensor * node_gpu(struct ggml_tensor * t) { ggml_cuda_assign_buffers_no_scratch(t); return t; }
+/* nodes placed on the device outside the scratch buffer own their memory (ggml-cuda.cu:9102-9109); released after the run */
+static struct ggml_tensor * g_gpu_nodes[64];
+static int g_n_gpu_nodes = 0;
+static struct ggml_tensor * node_gpu(struct ggml_tensor * t) {
+    ggml_cuda_assign_buffers_no_scratch(t);
+    if (g_n_gpu_nodes < 64) g_gpu_nodes[g_n_gpu_nodes++] = t;
+    return t;
+}
 
 static struct ggml_tensor * sparse_mm(struct ggml_context * ctx, struct ggml_tensor * w, struct ggml_tensor * w_gpu, struct ggml_tensor * x,
                                       struct ggml_tensor * idx, struct ggml_tensor * gid, struct ggml_tensor * bkt, int full_gpu) {
@@ -279,12 +286,34 @@ static void * gather_rows(const void * w, size_t rb, const int32_t * bucket, int
     return p;
 }
 
+REF_API int ref_ffn_sparse_gpu_parts(int d, int ff, int r, int T, int wtype, int has_gate,
+                                     const void * up_w, const void * gate_w, const void * down_t,
+                                     const uint16_t * fc1, const uint16_t * fc2,
+                                     const float * x_ffn, const float * x_pred,
+                                     const int32_t * gpu_idx, const int32_t * gpu_bucket, int n_bucket,
+                                     float threshold, float * logits, float * out,
+                                     float * h_out, float * out_cpu_part, float * out_gpu_part);
+
 REF_API int ref_ffn_sparse_gpu(int d, int ff, int r, int T, int wtype, int has_gate,
                                const void * up_w, const void * gate_w, const void * down_t,
                                const uint16_t * fc1, const uint16_t * fc2,
                                const float * x_ffn, const float * x_pred,
                                const int32_t * gpu_idx, const int32_t * gpu_bucket, int n_bucket,
                                float threshold, float * logits, float * out) {
+    return ref_ffn_sparse_gpu_parts(d, ff, r, T, wtype, has_gate, up_w, gate_w, down_t, fc1, fc2, x_ffn, x_pred, gpu_idx, gpu_bucket, n_bucket,
+                                    threshold, logits, out, NULL, NULL, NULL);
+}
+
+/* the same graph; a hybrid run also hands back the merged h ("ffn_gate_par", [T][ff]) and the two operands of the final ggml_add:
+ * the host node's share ("ffn_down_sparse", [T][d], computed by the reference's own CPU axpy on two threads) and the backend
+ * node's share ("ffn_down_sparse_gpu", [T][d]); each may be NULL */
+REF_API int ref_ffn_sparse_gpu_parts(int d, int ff, int r, int T, int wtype, int has_gate,
+                                     const void * up_w, const void * gate_w, const void * down_t,
+                                     const uint16_t * fc1, const uint16_t * fc2,
+                                     const float * x_ffn, const float * x_pred,
+                                     const int32_t * gpu_idx, const int32_t * gpu_bucket, int n_bucket,
+                                     float threshold, float * logits, float * out,
+                                     float * h_out, float * out_cpu_part, float * out_gpu_part) {
     enum ggml_type wt = (enum ggml_type) wtype;
     const int full_gpu = n_bucket == 0;
     const size_t rb = tensor_bytes(wt, d, 1);
@@ -331,12 +360,12 @@ REF_API int ref_ffn_sparse_gpu(int d, int ff, int r, int T, int wtype, int has_g
         cur = ggml_relu(ctx, upo);
         if (full_gpu) node_gpu(cur);
     }
-    struct ggml_tensor * res;
+    struct ggml_tensor * res, * o_cpu = NULL, * o_gpu = NULL;
     if (full_gpu) {
         res = node_gpu(ggml_axpy(ctx, down_g, cur, idx, NULL));
     } else {
-        struct ggml_tensor * o_cpu = ggml_axpy(ctx, down, cur, idx, gid);
-        struct ggml_tensor * o_gpu = node_gpu(ggml_axpy(ctx, down_g, cur, idx, bkt));
+        o_cpu = ggml_axpy(ctx, down, cur, idx, gid);
+        o_gpu = node_gpu(ggml_axpy(ctx, down_g, cur, idx, bkt));
         res = node_gpu(ggml_add(ctx, o_cpu, o_gpu));
     }
 
@@ -348,9 +377,16 @@ REF_API int ref_ffn_sparse_gpu(int d, int ff, int r, int T, int wtype, int has_g
     ggml_cuda_copy_to_host(res);
     if (logits) memcpy(logits, idx->data, (size_t)ff * T * 4);
     if (out)    memcpy(out, res->data, (size_t)d * T * 4);
+    if (!full_gpu) {
+        if (h_out) memcpy(h_out, cur->data, (size_t)ff * T * 4);
+        if (out_cpu_part) memcpy(out_cpu_part, o_cpu->data, (size_t)d * T * 4);
+        if (out_gpu_part) { ggml_cuda_copy_to_host(o_gpu); memcpy(out_gpu_part, o_gpu->data, (size_t)d * T * 4); }
+    }
 
     struct ggml_tensor * owned[] = {t_fc1, t_fc2, up_g, gate_g, down_g};
     for (int i = 0; i < 5; ++i) if (owned[i]) ggml_cuda_free_data(owned[i]);
+    for (int i = 0; i < g_n_gpu_nodes; ++i) ggml_cuda_free_data(g_gpu_nodes[i]);
+    g_n_gpu_nodes = 0;
     ggml_cuda_free_scratch();
     for (int i = 0; i < 3; ++i) free(tmp[i]);
     ggml_free(ctx);

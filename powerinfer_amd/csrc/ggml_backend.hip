@@ -22,6 +22,7 @@ namespace {
 struct Extra {
     void * data_device[GGML_CUDA_MAX_DEVICES];     // [0] is the only one used (single GPU)
     bool   owned;
+    bool   outside_scratch;                        // address computed from a host offset that does not lie in the scratch: never dereferenced
 };
 
 bool   g_loaded = false;
@@ -31,7 +32,20 @@ size_t g_scratch_size = 0, g_scratch_offset = 0;
 pi_workspace * g_ws = nullptr;
 int    g_ws_ff = 0, g_ws_d = 0;
 std::mutex g_mu;
-std::vector<Extra *> g_graph_extras;               // extras handed out by assign_*; freed with the scratch
+// Per-evaluation extras come from a ring, as in the reference (ggml-cuda.cu:9030-9044): a host rebuilds its graph for every
+// token and never hands these back, so they must not be heap objects of their own.
+constexpr size_t kMaxNodes = 8192;
+Extra * g_ring = nullptr;
+size_t  g_ring_next = 0;
+Extra * ring_extra(void * p) {
+    if (!g_ring) g_ring = new Extra[kMaxNodes];
+    Extra * e = &g_ring[g_ring_next];
+    g_ring_next = (g_ring_next + 1) % kMaxNodes;
+    memset(e, 0, sizeof *e);
+    e->data_device[0] = p;
+    return e;
+}
+bool is_ring(const Extra * e) { return g_ring && e >= g_ring && e < g_ring + kMaxNodes; }
 
 [[noreturn]] void die(const char * what) {
     fprintf(stderr, "powerinfer-hip backend: %s: %s\n", what, pi_last_error());
@@ -53,9 +67,15 @@ size_t tsize(int type) {
 size_t row_size(const ggml_tensor * t) { return tsize(t->type) * (size_t)(t->ne[0] / blck(t->type)); }
 int64_t nrows(const ggml_tensor * t) { return t->ne[1] * t->ne[2] * t->ne[3]; }
 int64_t nelem(const ggml_tensor * t) { return t->ne[0] * nrows(t); }
-size_t nbytes(const ggml_tensor * t) {
-    size_t n = tsize(t->type) * (size_t)(t->ne[0] / blck(t->type));        // ggml_nbytes: extent of the last element
-    for (int i = 1; i < GGML_MAX_DIMS; ++i) n += (size_t)(t->ne[i] - 1) * t->nb[i];
+size_t nbytes(const ggml_tensor * t) {                    // ggml_nbytes (ggml.c:1956-1973): the extent up to the last element, strides honoured
+    size_t n;
+    if (blck(t->type) == 1) {
+        n = tsize(t->type);
+        for (int i = 0; i < GGML_MAX_DIMS; ++i) n += (size_t)(t->ne[i] - 1) * t->nb[i];      // a permuted tensor's nb[0] is not the element size
+    } else {
+        n = (size_t)t->ne[0] * t->nb[0] / blck(t->type);
+        for (int i = 1; i < GGML_MAX_DIMS; ++i) n += (size_t)(t->ne[i] - 1) * t->nb[i];
+    }
     return n;
 }
 bool contiguous(const ggml_tensor * t) {
@@ -69,21 +89,21 @@ struct Temps {
     ~Temps() { for (void * p : ptrs) pi_free(p); }
 };
 
+void * dev_ptr(const ggml_tensor * t) {
+    const Extra * e = (const Extra *)t->extra;
+    if (!e || !e->data_device[0]) { fprintf(stderr, "powerinfer-hip backend: tensor '%s' is marked GPU but has no device buffer\n", t->name); exit(1); }
+    if (e->outside_scratch) { fprintf(stderr, "powerinfer-hip backend: tensor '%s' was given a scratch offset outside the scratch buffer\n", t->name); exit(1); }
+    return e->data_device[0];
+}
 void * dev_in(const ggml_tensor * t, Temps & tmp) {
-    if (t->backend != GGML_BACKEND_CPU) {
-        if (!t->extra) { fprintf(stderr, "powerinfer-hip backend: tensor '%s' is marked GPU but has no device buffer\n", t->name); exit(1); }
-        return ((Extra *)t->extra)->data_device[0];
-    }
+    if (t->backend != GGML_BACKEND_CPU) return dev_ptr(t);
     const size_t n = nbytes(t);
     void * p = tmp.get(n);
     BK_PI(pi_memcpy_h2d(p, t->data, n));
     return p;
 }
 void * dev_out(ggml_tensor * t, Temps & tmp) {
-    if (t->backend != GGML_BACKEND_CPU) {
-        if (!t->extra) { fprintf(stderr, "powerinfer-hip backend: tensor '%s' is marked GPU but has no device buffer\n", t->name); exit(1); }
-        return ((Extra *)t->extra)->data_device[0];
-    }
+    if (t->backend != GGML_BACKEND_CPU) return dev_ptr(t);
     return tmp.get(nbytes(t));
 }
 void finish_out(ggml_tensor * t, void * dptr) {
@@ -112,9 +132,9 @@ __global__ void relu_kernel(const float * a, float * y, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) y[i] = fmaxf(a[i], 0.0f);
 }
-__global__ void scale_kernel(const float * a, float * y, float s, int64_t n) {
+__global__ void scale_kernel(const float * a, float * y, const float * s, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
-    if (i < n) y[i] = __fmul_rn(a[i], s);
+    if (i < n) y[i] = __fmul_rn(a[i], *s);
 }
 __global__ void fill_kernel(float * y, float v, int64_t n) {
     const int64_t i = (int64_t)blockIdx.x * blockDim.x + threadIdx.x;
@@ -307,11 +327,9 @@ bool op_elementwise(ggml_tensor * dst) {
         hipLaunchKernelGGL(relu_kernel, grid1(n), dim3(256), 0, 0, ad, y, n);
         finish_out(dst, y);
     } else if (dst->op == GGML_OP_SCALE) {
-        float s;
-        if (b->backend == GGML_BACKEND_CPU) s = *(const float *)b->data;               // the factor is a 1-element tensor read on the host
-        else { BK_PI(pi_sync()); BK_PI(pi_memcpy_d2h(&s, ((Extra *)b->extra)->data_device[0], 4)); }
-        const float * ad = (const float *)dev_in(a, tmp); float * y = (float *)dev_out(dst, tmp);
-        hipLaunchKernelGGL(scale_kernel, grid1(n), dim3(256), 0, 0, ad, y, s, n);
+        if (!b || b->type != GGML_TYPE_F32) return false;
+        const float * ad = (const float *)dev_in(a, tmp); const float * sd = (const float *)dev_in(b, tmp); float * y = (float *)dev_out(dst, tmp);
+        hipLaunchKernelGGL(scale_kernel, grid1(n), dim3(256), 0, 0, ad, y, sd, n);       // the factor is a 1-element tensor, read where it lives
         finish_out(dst, y);
     } else if (dst->op == GGML_OP_RMS_NORM || dst->op == GGML_OP_NORM) {
         float eps; memcpy(&eps, dst->op_params, 4);
@@ -351,7 +369,7 @@ bool op_cpy(ggml_tensor * dst) {
     Temps tmp;
     const char * ad = (const char *)dev_in(a, tmp);
     char * td;
-    if (to->backend != GGML_BACKEND_CPU) td = (char *)((Extra *)to->extra)->data_device[0];
+    if (to->backend != GGML_BACKEND_CPU) td = (char *)dev_ptr(to);
     else { td = (char *)tmp.get(nbytes(to)); BK_PI(pi_memcpy_h2d(td, to->data, nbytes(to))); }      // strided destination: keep the gaps
     hipLaunchKernelGGL(cpy_kernel, grid1(nelem(a)), dim3(256), 0, 0, ad, shape_of(a), (int)a->type, td, shape_of(to), (int)to->type, nelem(a));
     finish_out(to, td);
@@ -375,27 +393,51 @@ Extra * new_extra(void * p, bool owned) {
     return e;
 }
 
-void assign(ggml_tensor * tensor, bool scratch, bool alloc) {
-    if (tensor->src[0] && tensor->src[0]->backend == GGML_BACKEND_CPU &&
-        (tensor->op == GGML_OP_RESHAPE || tensor->op == GGML_OP_VIEW || tensor->op == GGML_OP_PERMUTE || tensor->op == GGML_OP_TRANSPOSE))
-        assign(tensor->src[0], scratch, alloc);                      // a GPU view needs its parent on the GPU too (ggml-cuda.cu:9047-9060)
+bool view_like(int op) { return op == GGML_OP_RESHAPE || op == GGML_OP_VIEW || op == GGML_OP_PERMUTE || op == GGML_OP_TRANSPOSE; }
+char * scratch_base() {
+    if (!g_scratch) { g_scratch = (char *)pi_malloc(g_scratch_size); if (!g_scratch) die("scratch"); }
+    return g_scratch;
+}
+// Device address of a tensor that shares its parent's memory (ggml-cuda.cu:9069-9082 and 9132-9141): an operator computed in
+// place, a reshape / permute / transpose (same host address as src0) or a VIEW (byte offset in op_params) of a tensor that
+// lives on the device takes the parent's device address; nullptr when the rule does not apply.
+Extra * inplace_extra(const ggml_tensor * t, bool force_inplace) {
+    const ggml_tensor * s0 = t->src[0];
+    const bool inplace = (s0 != nullptr && s0->data == t->data) || t->op == GGML_OP_VIEW || force_inplace;
+    if (!inplace || !s0 || s0->backend == GGML_BACKEND_CPU || !s0->extra) return nullptr;
+    size_t offset = 0;
+    if (t->op == GGML_OP_VIEW) memcpy(&offset, t->op_params, sizeof(size_t));
+    const Extra * parent = (const Extra *)s0->extra;
+    const bool unusable = parent->outside_scratch;
+    Extra * e = ring_extra((char *)parent->data_device[0] + offset);      // may recycle the parent's slot only after 8192 newer extras
+    e->outside_scratch = unusable;
+    return e;
+}
+
+// ggml_cuda_assign_buffers_impl (ggml-cuda.cu:9046-9117)
+void assign(ggml_tensor * tensor, bool scratch, bool force_inplace, bool no_alloc) {
+    if (scratch && g_scratch_size == 0) return;
     tensor->backend = GGML_BACKEND_GPU;
-    if (!alloc || tensor->extra) return;
+    // a chain of views above a host tensor moves to the device with its consumer, and so does the destination of a copy
+    if (tensor->src[0] && tensor->src[0]->backend == GGML_BACKEND_CPU && view_like(tensor->src[0]->op)) assign(tensor->src[0], scratch, force_inplace, no_alloc);
+    if (tensor->op == GGML_OP_CPY && tensor->src[1]->backend == GGML_BACKEND_CPU) assign(tensor->src[1], scratch, force_inplace, no_alloc);
+    if (scratch && no_alloc) return;
     std::lock_guard<std::mutex> g(g_mu);
-    if (tensor->view_src && tensor->view_src->extra) {               // views share the parent's buffer
-        Extra * e = new_extra((char *)((Extra *)tensor->view_src->extra)->data_device[0] + tensor->view_offs, false);
-        g_graph_extras.push_back(e); tensor->extra = e; return;
+    if (Extra * shared = inplace_extra(tensor, force_inplace)) { tensor->extra = shared; return; }
+    if (tensor->op == GGML_OP_CPY) {                                    // the result of a copy is its destination
+        tensor->extra = ring_extra(dev_ptr(tensor->src[1]));
+        return;
     }
-    const size_t n = (nbytes(tensor) + 255) & ~(size_t)255;
-    void * p;
-    if (scratch && g_scratch_size >= n) {
-        if (!g_scratch) { g_scratch = (char *)pi_malloc(g_scratch_size); if (!g_scratch) die("scratch"); }
+    const size_t n = nbytes(tensor);
+    if (scratch) {
+        if (n > g_scratch_size) { fprintf(stderr, "powerinfer-hip backend: '%s' (%zu bytes) exceeds the scratch buffer (%zu)\n", tensor->name, n, g_scratch_size); exit(1); }
         if (g_scratch_offset + n > g_scratch_size) g_scratch_offset = 0;            // ring, as the reference's scratch buffer
-        p = g_scratch + g_scratch_offset; g_scratch_offset += n;
-        Extra * e = new_extra(p, false); g_graph_extras.push_back(e); tensor->extra = e;
+        tensor->extra = ring_extra(scratch_base() + g_scratch_offset);
+        g_scratch_offset += n;
     } else {
-        p = pi_malloc(n); if (!p) die("tensor allocation");
-        Extra * e = new_extra(p, true); g_graph_extras.push_back(e); tensor->extra = e;
+        void * p = pi_malloc(n); if (!p) die("tensor allocation");
+        BK_HIP(hipMemset(p, 0, n));
+        tensor->extra = new_extra(p, true);                            // released by ggml_cuda_free_data (the KV cache, llama.cpp:1420-1422)
     }
 }
 
@@ -441,32 +483,34 @@ void ggml_cuda_alloc_tensor(struct ggml_tensor * tensor) {
 void ggml_cuda_free_data(struct ggml_tensor * tensor) {
     if (!tensor || !tensor->extra) return;
     Extra * e = (Extra *)tensor->extra;
-    if (e->owned && e->data_device[0]) pi_free(e->data_device[0]);
-    {
-        std::lock_guard<std::mutex> g(g_mu);
-        for (auto & x : g_graph_extras) if (x == e) x = nullptr;
-    }
-    delete e;
     tensor->extra = nullptr;
+    if (is_ring(e)) return;                        // a per-evaluation address: nothing is owned
+    if (e->owned && e->data_device[0]) pi_free(e->data_device[0]);
+    delete e;
 }
 // copies src's host row into dst's current device pointer; the caller then bumps the pointer it got from
 // ggml_cuda_get_data_pp to stream the bucket's rows into a compact matrix (llama.cpp:2898-2967)
 void ggml_cuda_cpy_1d(struct ggml_tensor * dst, const struct ggml_tensor * src) {
-    BK_PI(pi_memcpy_h2d(((Extra *)dst->extra)->data_device[0], src->data, nbytes(src)));
+    BK_PI(pi_memcpy_h2d(dev_ptr(dst), src->data, nbytes(src)));
 }
 void ** ggml_cuda_get_data_pp(struct ggml_tensor * tensor) { return &((Extra *)tensor->extra)->data_device[0]; }
 
-void ggml_cuda_assign_buffers(struct ggml_tensor * tensor) { assign(tensor, true, true); }
-void ggml_cuda_assign_buffers_no_scratch(struct ggml_tensor * tensor) { assign(tensor, false, true); }
-void ggml_cuda_assign_buffers_force_inplace(struct ggml_tensor * tensor) { assign(tensor, true, true); }
-void ggml_cuda_assign_buffers_no_alloc(struct ggml_tensor * tensor) { assign(tensor, false, false); }
+void ggml_cuda_assign_buffers(struct ggml_tensor * tensor) { if (tensor) assign(tensor, true, false, false); }
+void ggml_cuda_assign_buffers_no_scratch(struct ggml_tensor * tensor) { assign(tensor, false, false, false); }
+void ggml_cuda_assign_buffers_force_inplace(struct ggml_tensor * tensor) { assign(tensor, false, true, false); }
+void ggml_cuda_assign_buffers_no_alloc(struct ggml_tensor * tensor) { assign(tensor, true, false, true); }
+// ggml-cuda.cu:9119-9146.  The host passes the tensor's offset inside its own compute buffer, whose layout the device scratch
+// mirrors.  For a tensor that shares its parent's memory the parent's device address wins: the parent may live outside the
+// scratch (a view of the KV cache), where the host-side offset means nothing -- the reference stores such an address without
+// looking at it, so an offset beyond the scratch is accepted here as long as no kernel is ever pointed at it (checked at use).
 void ggml_cuda_assign_scratch_offset(struct ggml_tensor * tensor, size_t offset) {
+    if (g_scratch_size == 0) return;
     std::lock_guard<std::mutex> g(g_mu);
-    if (!g_scratch_size) { fprintf(stderr, "powerinfer-hip backend: ggml_cuda_assign_scratch_offset without a scratch size\n"); exit(1); }
-    if (!g_scratch) { g_scratch = (char *)pi_malloc(g_scratch_size); if (!g_scratch) die("scratch"); }
-    if (offset + nbytes(tensor) > g_scratch_size) { fprintf(stderr, "powerinfer-hip backend: scratch offset out of range for '%s'\n", tensor->name); exit(1); }
-    if (!tensor->extra) { Extra * e = new_extra(nullptr, false); g_graph_extras.push_back(e); tensor->extra = e; }
-    ((Extra *)tensor->extra)->data_device[0] = g_scratch + offset;
+    char * base = scratch_base();
+    if (Extra * shared = inplace_extra(tensor, false)) { tensor->extra = shared; return; }
+    Extra * e = ring_extra(base + offset);
+    e->outside_scratch = offset > g_scratch_size || nbytes(tensor) > g_scratch_size - offset;
+    tensor->extra = e;
 }
 void ggml_cuda_set_scratch_size(size_t scratch_size) {
     if (scratch_size > g_scratch_size) ggml_cuda_free_scratch();
@@ -474,16 +518,15 @@ void ggml_cuda_set_scratch_size(size_t scratch_size) {
 }
 void ggml_cuda_free_scratch(void) {
     std::lock_guard<std::mutex> g(g_mu);
-    for (Extra * e : g_graph_extras) if (e) { if (e->owned) pi_free(e->data_device[0]); e->data_device[0] = nullptr; e->owned = false; }
     if (g_scratch) { pi_free(g_scratch); g_scratch = nullptr; }
     g_scratch_offset = 0;
 }
 void ggml_cuda_copy_to_device(struct ggml_tensor * tensor) {
-    BK_PI(pi_memcpy_h2d(((Extra *)tensor->extra)->data_device[0], tensor->data, nbytes(tensor)));
+    BK_PI(pi_memcpy_h2d(dev_ptr(tensor), tensor->data, nbytes(tensor)));
 }
 void ggml_cuda_copy_to_host(struct ggml_tensor * tensor) {
     BK_PI(pi_sync());
-    BK_PI(pi_memcpy_d2h(tensor->data, ((Extra *)tensor->extra)->data_device[0], nbytes(tensor)));
+    BK_PI(pi_memcpy_d2h(tensor->data, dev_ptr(tensor), nbytes(tensor)));
 }
 
 int ggml_cuda_get_device_count(void) { int n = 0; if (hipGetDeviceCount(&n) != hipSuccess) { (void)hipGetLastError(); return 0; } return n; }
@@ -506,7 +549,12 @@ bool ggml_cuda_compute_forward(struct ggml_compute_params * params, struct ggml_
     const bool src0_on_device = s0 != nullptr && s0->backend != GGML_BACKEND_CPU;
     const bool any_on_device = tensor->backend == GGML_BACKEND_GPU || src0_on_device || (tensor->src[1] != nullptr && tensor->src[1]->backend == GGML_BACKEND_GPU);
     // weights not on the device: the sparse operators run on the CPU with the sparsity (ggml-cuda.cu:9226-9230)
-    if ((!src0_on_device && (tensor->op == GGML_OP_MUL_MAT_SPARSE || tensor->op == GGML_OP_AXPY)) || !any_on_device) return false;
+    if ((!src0_on_device && (tensor->op == GGML_OP_MUL_MAT_SPARSE || tensor->op == GGML_OP_AXPY)) || (!any_on_device && tensor->op != GGML_OP_MUL_MAT)) return false;
+    if (tensor->op == GGML_OP_MUL_MAT) {
+        if (tensor->src[0]->ne[3] != tensor->src[1]->ne[3]) return false;
+        // host-resident operands: only a product large enough to pay for the transfer is taken (ggml-cuda.cu:9278-9282)
+        if (!any_on_device && !ggml_cuda_can_mul_mat(tensor->src[0], tensor->src[1], tensor)) return false;
+    }
     switch (tensor->op) {
         case GGML_OP_MUL_MAT: case GGML_OP_MUL_MAT_SPARSE: case GGML_OP_AXPY: case GGML_OP_ADD: case GGML_OP_MUL:
         case GGML_OP_SCALE: case GGML_OP_RMS_NORM: case GGML_OP_NORM: case GGML_OP_SOFT_MAX: case GGML_OP_ROPE:

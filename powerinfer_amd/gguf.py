@@ -154,6 +154,25 @@ def _gtype(arr):
     return {np.dtype(np.float32): F32, np.dtype(np.float16): F16, np.dtype(np.uint8): Q4_0, np.dtype(np.int32): I32}[arr.dtype]
 
 
+def synthetic_tokenizer_kv(n_vocab):
+    """`tokenizer.*` entries of a made-up SentencePiece-type vocabulary of n_vocab distinct strings, enough for the reference's
+    loader (llm_load_vocab, llama.cpp:2473-2700) to accept a synthetic model of either architecture: ids 0..2 are <unk> <s> </s>,
+    3..258 the byte tokens <0x00>..<0xFF> (the loader looks the newline up as <0x0A>), the rest plain words.  Logits do not
+    depend on any of it."""
+    if n_vocab < 259:
+        raise ValueError("a SentencePiece vocabulary needs the 3 control and 256 byte tokens")
+    words = [b"<unk>", b"<s>", b"</s>"] + [b"<0x%02X>" % i for i in range(256)] + [b"w%d" % i for i in range(259, n_vocab)]
+    types = np.ones(n_vocab, np.int32)              # normal
+    types[0], types[1:3], types[3:259] = 2, 3, 6    # unknown, control, byte
+    return {
+        "tokenizer.ggml.model": (T_STR, b"llama"),
+        "tokenizer.ggml.tokens": (T_ARR, (T_STR, words)),
+        "tokenizer.ggml.scores": (T_ARR, (T_F32, np.zeros(n_vocab, np.float32))),
+        "tokenizer.ggml.token_type": (T_ARR, (T_I32, types)),
+        "tokenizer.ggml.bos_token_id": (T_U32, 1), "tokenizer.ggml.eos_token_id": (T_U32, 2), "tokenizer.ggml.unknown_token_id": (T_U32, 0),
+    }
+
+
 def write_model(path, model, tokenizer_kv):
     """Writes a synthetic model (powerinfer_amd.synth.make_model) as a PowerInfer GGUF.  tokenizer_kv: the
     `tokenizer.*` entries of a vocabulary file whose token count equals hp.n_vocab."""

@@ -125,6 +125,77 @@ class Graph:
     def axpy(self, a, b, idx, aux, name="axpy"):                                # ggml.c:4158
         return self._node("AXPY", F32, [a.ne[0], b.ne[1], b.ne[2], b.ne[3]], [a, b, idx, aux], name, params=(0 if aux is not None else 1,))
 
+    def _f32(self, v):
+        return int(np.float32(v).view(np.int32))
+
+    def rms_norm(self, a, eps, name="rms_norm"):                                # ggml.c:4553
+        return self._node("RMS_NORM", F32, list(a.ne), [a], name, params=(self._f32(eps),))
+
+    def norm(self, a, eps, name="norm"):                                        # ggml.c:4521
+        return self._node("NORM", F32, list(a.ne), [a], name, params=(self._f32(eps),))
+
+    def scale(self, a, s, name="scale"):                                        # ggml.c:4712 (the factor is a 1-element tensor)
+        return self._node("SCALE", F32, list(a.ne), [a, s], name)
+
+    def soft_max(self, a, name="soft_max"):                                     # ggml.c:5171
+        return self._node("SOFT_MAX", F32, list(a.ne), [a], name)
+
+    def rope(self, a, pos, n_dims, mode, freq_base=10000.0, freq_scale=1.0, name="rope"):      # ggml_rope_impl, ggml.c:5222-5262
+        params = [0, n_dims, mode, 0, 0, self._f32(freq_base), self._f32(freq_scale), self._f32(0.0), self._f32(1.0), self._f32(32.0), self._f32(1.0)]
+        return self._node("ROPE", F32, list(a.ne), [a, pos], name, params=params)
+
+    def get_rows(self, a, ids, name="get_rows"):                                # ggml.c:4925
+        return self._node("GET_ROWS", F32, [a.ne[0], ids.ne[0]], [a, ids], name)
+
+    def view(self, a, ne, nb, offset, name="view"):
+        """ggml_view_nd (ggml.c:4791-4900): a tensor over a's buffer with its own shape, byte strides nb[1..] and byte offset."""
+        t = Tensor()
+        t.type, t.backend, t.n_dims = a.type, CPU, len(ne)
+        ne = list(ne) + [1] * (4 - len(ne))
+        nb = [_tsize(a.type)] + list(nb)
+        while len(nb) < 4:
+            nb.append(nb[-1] * ne[len(nb) - 1])
+        for i in range(4):
+            t.ne[i], t.nb[i] = ne[i], nb[i]
+        t.op = OP["VIEW"]
+        t.src[0] = C.pointer(a)
+        t.view_src = C.pointer(a)
+        t.view_offs = offset
+        t.op_params[0] = offset & 0xFFFFFFFF
+        t.op_params[1] = offset >> 32
+        t.data = a.data + offset
+        t.name = name.encode()[:63]
+        t._host, t._srcs = a._host, [a]
+        self.nodes.append(t)
+        return t
+
+    def permute(self, a, axes, name="permute"):                                 # ggml_permute, ggml.c:4960-5010
+        t = Tensor()
+        t.type, t.backend, t.n_dims = a.type, CPU, 4
+        for i in range(4):
+            t.ne[axes[i]], t.nb[axes[i]] = a.ne[i], a.nb[i]
+        t.op = OP["PERMUTE"]
+        t.src[0] = C.pointer(a)
+        t.view_src = a.view_src if a.view_src else C.pointer(a)
+        t.view_offs = a.view_offs
+        t.data = a.data
+        t.name = name.encode()[:63]
+        t._host, t._srcs = a._host, [a]
+        self.nodes.append(t)
+        return t
+
+    def cpy(self, a, b, name="cpy"):                                            # ggml_cpy, ggml.c:4740: result is a view of b
+        t = self.view(b, [b.ne[i] for i in range(4)], [b.nb[i] for i in range(1, 4)], 0, name)
+        self.nodes.pop()
+        t.op = OP["CPY"]
+        t.src[0], t.src[1] = C.pointer(a), C.pointer(b)
+        t._srcs = [a, b]
+        self.nodes.append(t)
+        return t
+
+    def cont(self, a, name="cont"):                                             # ggml_cont, ggml.c:4766
+        return self._node("CONT", a.type, [a.ne[i] for i in range(4)], [a], name)
+
     # ---- executor --------------------------------------------------------------------------------------
     def compute(self, threshold=0.0):
         self.L.ggml_cuda_set_device_constants(threshold)
@@ -154,6 +225,8 @@ class Graph:
         O = ol.oracle()
         s = t._srcs
         op = {v: k for k, v in OP.items()}[t.op]
+        if op in ("VIEW", "PERMUTE", "RESHAPE", "TRANSPOSE"):
+            return                                               # no computation (ggml.c:16508-16520)
         out = t._host.view(np.float32)
         T = int(t.ne[1] * t.ne[2] * t.ne[3])
         if op == "MUL_MAT":

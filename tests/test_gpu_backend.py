@@ -16,6 +16,12 @@ def rel_err(a, b):
     return float(np.abs(a - b).max() / max(np.abs(b).max(), 1e-30))
 
 
+def out_under(L, wtype, has_gate, x, lg, thr=0.0):
+    """[T][d] output of the CPU oracle for the masks the given predictor logits [T][ff] imply."""
+    return np.stack([ol.ffn_under_logits(ol.oracle(), L["d"], L["ff"], wtype, has_gate, L["up"], L["gate"], L["down_t"], x[t], lg[t], thr)["out"]
+                     for t in range(x.shape[0])])
+
+
 def build_ffn(G, L, x, wtype, full_gpu, gid=None, bucket=None):
     """llm_build_ffn_sparse for T tokens; returns (idx, out)."""
     d, ff, r, T = L["d"], L["ff"], L["r"], x.shape[0]
@@ -79,8 +85,8 @@ def test_full_gpu_graph(wtype, has_gate):
                       np.zeros(ff, np.int32), 0.0, nth=4)
     lg = G.host(idx)
     assert rel_err(lg, o["logits"]) < 1e-5
-    if np.array_equal(lg >= 0, o["logits"] >= 0):
-        assert rel_err(G.host(out), o["out"]) < 1e-4
+    assert ((lg >= 0) == (o["logits"] >= 0)).mean() >= 0.999
+    assert rel_err(G.host(out), out_under(L, wtype, has_gate, L["x"], lg)) < 1e-4
 
 
 @pytest.mark.parametrize("wtype", [ol.F16, ol.Q4_0])
@@ -100,8 +106,8 @@ def test_hybrid_graph_cpu_part_plus_gpu_part(wtype):
                       np.zeros(ff, np.int32), 0.0, nth=4)
     lg = G.host(idx)
     assert rel_err(lg, o["logits"]) < 1e-5
-    if np.array_equal(lg >= 0, o["logits"] >= 0):
-        assert rel_err(G.host(out), o["out"]) < 1e-4
+    assert ((lg >= 0) == (o["logits"] >= 0)).mean() >= 0.999
+    assert rel_err(G.host(out), out_under(L, wtype, True, L["x"], lg)) < 1e-4
 
 
 def test_backend_info_entry_points():
@@ -133,36 +139,56 @@ def test_reference_executor_drives_this_backend(wtype, hot_frac):
     """Drop-in check of the boundary: oracle/_ref/libpi_ref_gpu.so is the REFERENCE's ggml.c compiled with
     -DGGML_USE_CUBLAS and linked against libpowerinfer_hip.so in place of ggml-cuda.cu.  Its own op constructors,
     graph and two-thread executor run llm_build_ffn_sparse's op sequence (full-GPU, and hybrid CPU part + GPU part
-    + ggml_add); the result must equal the CPU path computing every neuron."""
+    + ggml_add), ONE evaluation each.
+
+    Every node this backend computes is deterministic and is checked strictly: the predictor logits, the backend's share of
+    the down projection and the final ggml_add of the two shares.  The hybrid graph's host share is computed by the reference's
+    own CPU axpy on two threads (the executor asserts n_threads > 1 for hybrid graphs), and that kernel adds each thread's
+    partial vector into the output without a lock, eight floats at a time (`res += tmp`, ggml.c:14433-14458): an 8-float
+    group of the HOST node may therefore hold the sum of both threads' rows or of either thread's rows alone.  Only that node
+    gets this three-way acceptance, per 8-float group, and the groups that lost a share are counted in the report."""
     import os
     so = os.path.join(ol.ODIR, "_ref", "libpi_ref_gpu.so")
     if not os.path.exists(so):
         pytest.skip("oracle/_ref/libpi_ref_gpu.so was not built (needs the reference tree at build time)")
     R = C.CDLL(so)
     vp, i, f = C.c_void_p, C.c_int, C.c_float
-    R.ref_ffn_sparse_gpu.argtypes = [i] * 6 + [vp] * 9 + [i, f, vp, vp]
+    R.ref_ffn_sparse_gpu_parts.argtypes = [i] * 6 + [vp] * 9 + [i, f] + [vp] * 5
     R.ref_init()
     d, ff, r, T = 1024, 4096, 128, 2
     L = synth.make_ffn_layer(seed=81 + wtype, d=d, ff=ff, r=r, wtype=wtype, mean_rate=0.15, T=T)
     gid, bucket = synth.gpu_split(L["p"], hot_frac)
-    n_bucket = 0 if hot_frac >= 1.0 else bucket.size
+    hybrid = hot_frac < 1.0
+    n_bucket = bucket.size if hybrid else 0
     lg, out = np.zeros((T, ff), np.float32), np.zeros((T, d), np.float32)
+    h, part_cpu, part_gpu = np.zeros((T, ff), np.float32), np.zeros((T, d), np.float32), np.zeros((T, d), np.float32)
     P = ol._ptr
-    o = ol.ffn_sparse(ol.oracle(), d, ff, r, T, wtype, 1, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], L["x"], L["x"],
-                      np.zeros(ff, np.int32), 0.0, nth=4)
-    # The hybrid graph runs the reference's own CPU axpy on two host threads, and that kernel adds each thread's partial
-    # sums into the output without a lock (ggml.c:14433-14458): now and then one thread's share is lost on the HOST side.
-    # The executor asserts n_threads > 1 for hybrid graphs, so the graph is evaluated up to three times and must agree once;
-    # the full-GPU graph has no host share and gets a single evaluation.
-    errs = []
-    for _ in range(1 if hot_frac >= 1.0 else 3):
-        rc = R.ref_ffn_sparse_gpu(d, ff, r, T, wtype, 1, P(L["up"]), P(L["gate"]), P(L["down_t"]), P(L["fc1"]), P(L["fc2"]), P(L["x"]), P(L["x"]),
-                                  P(gid), P(bucket), n_bucket, 0.0, P(lg), P(out))
-        assert rc == 0
-        assert rel_err(lg, o["logits"]) < 1e-5
-        if not np.array_equal(lg >= 0, o["logits"] >= 0):
-            return
-        errs.append(rel_err(out, o["out"]))
-        if errs[-1] < 1e-4:
-            break
-    assert min(errs) < 1e-4, errs
+    O = ol.oracle()
+    o = ol.ffn_sparse(O, d, ff, r, T, wtype, 1, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], L["x"], L["x"], np.zeros(ff, np.int32), 0.0, nth=4)
+    rc = R.ref_ffn_sparse_gpu_parts(d, ff, r, T, wtype, 1, P(L["up"]), P(L["gate"]), P(L["down_t"]), P(L["fc1"]), P(L["fc2"]), P(L["x"]), P(L["x"]),
+                                    P(gid), P(bucket), n_bucket, 0.0, P(lg), P(out), P(h), P(part_cpu), P(part_gpu))
+    assert rc == 0
+    assert rel_err(lg, o["logits"]) < 1e-5                                   # mlp_pre_out: a backend node
+    assert ((lg >= 0) == (o["logits"] >= 0)).mean() >= 0.999
+    if not hybrid:
+        assert rel_err(out, out_under(L, wtype, True, L["x"], lg)) < 1e-4    # every node ran on the backend
+        return
+    raced = 0
+    for t in range(T):
+        u = ol.ffn_under_logits(O, d, ff, wtype, True, L["up"], L["gate"], L["down_t"], L["x"][t], lg[t], 0.0)      # up/gate/h over all neurons
+        scale = np.abs(u["out"]).max()
+        assert rel_err(h[t], u["h"]) < 1e-4                                  # ffn_*_sparse (host) + ffn_*_sparse_gpu (backend) merged
+        # the backend's share of the down projection: rows of the bucket, h as the graph merged it
+        want_gpu = ol.axpy_under_logits(O, d, ff, wtype, L["down_t"], h[t], lg[t], 0.0, skip=1 - gid)
+        assert np.abs(part_gpu[t] - want_gpu).max() < 1e-4 * scale, "ffn_down_sparse_gpu (backend node)"
+        # the final ggml_add ran on the backend
+        assert np.abs(out[t] - (part_cpu[t] + part_gpu[t])).max() <= 1e-6 * scale, "ffn_down_sparse_merged (backend node)"
+        # the host node: both threads' rows, or (lost update) the rows of one thread only, per 8-float group
+        dr = (ff + 1) // 2
+        first = np.arange(ff) < dr
+        cands = [ol.axpy_under_logits(O, d, ff, wtype, L["down_t"], h[t], lg[t], 0.0, skip=sk)
+                 for sk in (gid, gid | (~first).astype(np.int32), gid | first.astype(np.int32))]
+        err = np.stack([np.abs(part_cpu[t] - c).reshape(-1, 8).max(1) for c in cands])      # [3][d/8]
+        assert (err.min(0) < 1e-4 * scale).all(), f"host node ffn_down_sparse: errors vs (both, thread 0, thread 1) {err.max(1) / scale}"
+        raced += int((err[0] >= 1e-4 * scale).sum())
+    print(f"host axpy groups of 8 floats that lost one thread's share: {raced} of {T * d // 8}")

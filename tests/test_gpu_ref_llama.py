@@ -1,0 +1,65 @@
+"""The reference's own llama.cpp -- model loader, VRAM-budget offload, graph builder, ggml-alloc and the hybrid executor --
+compiled with its accelerator hooks and linked against libpowerinfer_hip.so in place of ggml-cuda.cu
+(oracle/_ref/ref_llama_gpu, built by oracle/Makefile), run on the golden models.  Its logits are compared with the vectors
+the same llama.cpp produced on the CPU alone (tests/golden/ref_*.npz): every ggml_cuda_* entry point llama.cpp calls is
+exercised the way the reference calls it, including ggml_cuda_assign_scratch_offset against a real ggml-alloc layout.
+
+The model file carries a made-up tokenizer (gguf.synthetic_tokenizer_kv) instead of the reference's vocabulary files; logits do
+not depend on it.  The neuron split comes from a `<model>.generated.gpuidx` written by powerinfer_amd.split.write_gpuidx, which
+the reference's llama_gpu_split_loader reads."""
+import importlib.util
+import os
+import subprocess
+
+import numpy as np
+import pytest
+
+from powerinfer_amd import gguf, split
+
+pytestmark = pytest.mark.gpu
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+BIN = os.path.join(ROOT, "oracle", "_ref", "ref_llama_gpu")
+spec = importlib.util.spec_from_file_location("make_llama_fixture", os.path.join(ROOT, "tests", "golden", "make_llama_fixture.py"))
+fx = importlib.util.module_from_spec(spec)
+spec.loader.exec_module(fx)
+
+
+def run_reference(tmp_path, name, share, n_threads):
+    if not os.path.exists(BIN):
+        pytest.skip("oracle/_ref/ref_llama_gpu is not built (needs the reference sources at build time)")
+    g = dict(np.load(os.path.join(ROOT, "tests", "golden", f"ref_{name}.npz")))
+    hp, model = fx.case_model(name)
+    if not np.array_equal(fx.model_sha(model), g["model_sha"]):
+        pytest.skip("numpy generates a different stream here than where the fixture was written")
+    path, out = str(tmp_path / "m.powerinfer.gguf"), str(tmp_path / "out.bin")
+    gguf.write_model(path, model, gguf.synthetic_tokenizer_kv(hp.n_vocab))
+    rates = [L["p"] for L in model["layers"]]
+    splits = split.split_from_counts(rates, [int(round(share * hp.n_ff))] * hp.n_layer)
+    split.write_gpuidx(path + ".generated.gpuidx", splits, split.required_bytes(hp, splits))
+    toks = [str(int(t)) for t in g["consumed"]]                 # every step consumes the reference's token (teacher forcing)
+    env = dict(os.environ, REF_VRAM_GB="2")
+    r = subprocess.run([BIN, path, str(hp.n_ctx), str(n_threads), "0", out] + toks, env=env, capture_output=True, text=True, timeout=110)
+    log = r.stdout + r.stderr
+    assert r.returncode == 0, log[-3000:]
+    raw = np.fromfile(out, np.uint8)
+    n_steps, n_vocab = (int(v) for v in raw[:8].view(np.int32))
+    rec = raw[8:].reshape(n_steps, 8 + 4 * n_vocab)
+    greedy = rec[:, 4:8].copy().view(np.int32)[:, 0]
+    logits = rec[:, 8:].copy().view(np.float32)
+    return g, hp, log, greedy, logits
+
+
+@pytest.mark.timeout(120)
+@pytest.mark.parametrize("name,share,n_threads", [("llama_f16", 1.0, 1), ("llama_f16", 0.6, 2), ("llama_q4", 1.0, 1), ("llama_q4", 0.6, 2),
+                                                  ("falcon_f16", 1.0, 1), ("falcon_f16", 0.6, 2)])
+def test_reference_llama_cpp_runs_on_this_backend(name, share, n_threads, tmp_path):
+    g, hp, log, greedy, logits = run_reference(tmp_path, name, share, n_threads)
+    # the loader took the offload path this test is about: attention, predictor and output tensors plus both halves of the KV cache
+    # on the device (n_gpu_layers = n_layer + 3), and the FFN rows of the split
+    assert "offloading v cache to GPU" in log and "offloading k cache to GPU" in log, log[-3000:]
+    assert "offloaded layers from VRAM budget" in log
+    errs = np.abs(logits[:, g["sample_idx"]] - g["logits_sample"]).max(1) / g["logits_absmax"]
+    assert errs.max() < 1e-2, errs                               # the north star's logits tolerance
+    assert np.median(errs) < 2e-3, errs
+    assert int((greedy == g["greedy"]).sum()) >= len(errs) - 1, (greedy, g["greedy"])

@@ -283,7 +283,9 @@ PI_API int pi_k_attn_decode(const float * q_rot, const void * k_cache, const voi
                             int hd, int n_ctx, const int32_t * pos, float * out, pi_stream_t stream);
 
 /* cos/sin table for pi_k_attn_fused: float2 [n_ctx][hd/2], angles formed as the CPU path forms them
- * (theta advanced by repeated fp32 multiplication with theta_scale = base^(-2/hd), ggml.c:11196-11319) */
+ * (theta advanced by repeated fp32 multiplication with theta_scale = base^(-2/hd), ggml.c:11196-11319).  A set-up call: the
+ * values are computed on the host with the C library's cosf / sinf (what the CPU path calls) and copied with a blocking copy
+ * after the stream has drained. */
 PI_API int pi_k_rope_table(void * table, int n_ctx, int hd, float theta_scale, pi_stream_t stream);
 
 /* pi_k_rope_kv_store + pi_k_attn_decode in one launch (one workgroup per query head; the new cell is used

@@ -16,6 +16,10 @@ FLAGS = [
     "-O3", "--offload-arch=gfx950", "-std=c++17", "-fPIC", "-shared", "-fvisibility=hidden", "-pthread",
     # packed-FP32 instructions are not to be generated on this hardware pool
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
+    # a product and a sum fuse into one FMA only where the source writes them as one expression: hipcc's default ("fast") also
+    # fuses across statements and through __fmul_rn / __fadd_rn (plain * and + in the HIP headers), which moves results by one
+    # unit in the last place where the CPU path rounds twice (norm weight then bias, the RoPE rotation)
+    "-ffp-contract=on",
     "-Wno-unused-command-line-argument",
     # host code of the cold path uses the x86 vector extensions every MI355X host CPU has
     "-Xarch_host", "-mavx2", "-Xarch_host", "-mfma", "-Xarch_host", "-mf16c",

@@ -12,6 +12,18 @@
 struct __attribute__((packed)) pi_block_q4_0 { uint16_t d; uint8_t qs[16]; };
 static_assert(sizeof(pi_block_q4_0) == 18, "q4_0 block is 18 bytes");
 
+// 1.0f / sqrtf(v) exactly as the CPU evaluates it: a correctly rounded fp32 square root, then a correctly rounded fp32
+// division.  Both are taken through fp64 (53 >= 2 * 24 + 2 bits, so the second rounding is innocuous).  The fp32 forms the
+// compiler picks for the device may be one unit in the last place off, and a norm scale that is off by one moves the fp16
+// rounding of a few activations of every vector it multiplies (1e-5 of a mat-vec result at 8192 columns).
+__host__ __device__ __forceinline__ float pi_inv_sqrt(float v) {
+    const float r = (float)sqrt((double)v);
+    return (float)(1.0 / (double)r);
+}
+
+// a / b rounded once to fp32, as IEEE division on the CPU is (the quotient is formed in fp64 and rounded: innocuous for fp32 operands)
+__host__ __device__ __forceinline__ float pi_div(float a, float b) { return (float)((double)a / (double)b); }
+
 // Wave-wide reductions through DPP (data-parallel primitives: lane permutations inside the VALU, no LDS
 // crossbar round trip): pairs, quads, half rows and rows by quad_perm / row_half_mirror / row_mirror, then the
 // last lane of row 0 (2) is added into row 1 (3) and lane 31 into rows 2-3, so lane 63 holds the total, which

@@ -161,7 +161,7 @@ __global__ __launch_bounds__(256) void norm_rows_kernel(const float * x, float *
         for (int i = threadIdx.x; i < n; i += 256) { const float v = __fsub_rn(xr[i], mean); s += (double)__fmul_rn(v, v); }
         s = bsum(s);
     }
-    const float scale = 1.0f / sqrtf((float)(s / n) + eps);
+    const float scale = pi_inv_sqrt((float)(s / n) + eps);
     for (int i = threadIdx.x; i < n; i += 256) yr[i] = __fmul_rn(__fsub_rn(xr[i], mean), scale);
 }
 // one workgroup per row; exp through the fp16 rounding of the CPU path's table (ggml.c:10747-10759)

@@ -7,6 +7,8 @@
 
 #include <math.h>
 
+#include <vector>
+
 namespace {
 
 constexpr int kBlock = 256;                 // 4 waves
@@ -49,7 +51,7 @@ __device__ void stage_x_f16(__half * xs, const float * __restrict__ x, int cols,
         double s = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = x[i]; s += (double)__fmul_rn(v, v); }
         s = block_sum_f64(s, red);
-        scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
+        scale = pi_inv_sqrt((float)(s / cols) + na.eps);
     } else if (na.kind == 2) {
         double s = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) s += (double)x[i];
@@ -58,7 +60,7 @@ __device__ void stage_x_f16(__half * xs, const float * __restrict__ x, int cols,
         double s2 = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = __fsub_rn(x[i], mean); s2 += (double)__fmul_rn(v, v); }
         s2 = block_sum_f64(s2, red);
-        scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
+        scale = pi_inv_sqrt((float)(s2 / cols) + na.eps);
     }
     for (int i = threadIdx.x; i < cols; i += blockDim.x) {
         float v = x[i];
@@ -99,7 +101,7 @@ __device__ __forceinline__ void stage_fast_finish(__half * xs, const float * lds
         double s = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = xraw[i]; s += (double)__fmul_rn(v, v); }
         s = block_sum_f64(s, red);
-        scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
+        scale = pi_inv_sqrt((float)(s / cols) + na.eps);
     } else if (na.kind == 2) {
         double s = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) s += (double)xraw[i];
@@ -108,7 +110,7 @@ __device__ __forceinline__ void stage_fast_finish(__half * xs, const float * lds
         double s2 = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = __fsub_rn(xraw[i], mean); s2 += (double)__fmul_rn(v, v); }
         s2 = block_sum_f64(s2, red);
-        scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
+        scale = pi_inv_sqrt((float)(s2 / cols) + na.eps);
     }
     for (int i = threadIdx.x; i < cols; i += blockDim.x) {
         float v = xraw[i];
@@ -133,7 +135,7 @@ __device__ void stage_x_q8(int8_t * xq, float * xd, const float * __restrict__ x
         double s = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = x[i]; s += (double)__fmul_rn(v, v); }
         s = block_sum_f64(s, red);
-        const float scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
+        const float scale = pi_inv_sqrt((float)(s / cols) + na.eps);
         for (int i = threadIdx.x; i < cols; i += blockDim.x) {
             float v = __fmul_rn(x[i], scale);
             if (na.w) v = __fmul_rn(v, na.w[i]);
@@ -148,7 +150,7 @@ __device__ void stage_x_q8(int8_t * xq, float * xd, const float * __restrict__ x
         double s2 = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = __fsub_rn(x[i], mean); s2 += (double)__fmul_rn(v, v); }
         s2 = block_sum_f64(s2, red);
-        const float scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
+        const float scale = pi_inv_sqrt((float)(s2 / cols) + na.eps);
         for (int i = threadIdx.x; i < cols; i += blockDim.x) {
             float v = __fmul_rn(__fsub_rn(x[i], mean), scale);
             if (na.w) v = __fmul_rn(v, na.w[i]);
@@ -163,8 +165,8 @@ __device__ void stage_x_q8(int8_t * xq, float * xd, const float * __restrict__ x
         float amax = fabsf(v);
 #pragma unroll
         for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, PI_WAVE));
-        const float d = amax / 127.0f;
-        const float id = (amax != 0.0f) ? 127.0f / amax : 0.0f;
+        const float d = pi_div(amax, 127.0f);
+        const float id = (amax != 0.0f) ? pi_div(127.0f, amax) : 0.0f;
         xq[i] = (int8_t)(int)rintf(__fmul_rn(v, id));
         if ((i & 31) == 0) xd[i >> 5] = pi_round_f16(d);
     }
@@ -327,7 +329,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemv_f16_reg_kernel(const __half * 
             double t = 0.0;
 #pragma unroll
             for (int w = 0; w < kWavesPerBlock; ++w) t += red[0][w];
-            if (KIND == 1) scale = 1.0f / sqrtf((float)(t / cols) + eps);
+            if (KIND == 1) scale = pi_inv_sqrt((float)(t / cols) + eps);
             else {
                 mean = (float)(t / cols);
                 double s2 = 0.0;
@@ -343,7 +345,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemv_f16_reg_kernel(const __half * 
                 double t2 = 0.0;
 #pragma unroll
                 for (int w = 0; w < kWavesPerBlock; ++w) t2 += red[1][w];
-                scale = 1.0f / sqrtf((float)(t2 / cols) + eps);
+                scale = pi_inv_sqrt((float)(t2 / cols) + eps);
             }
         }
 #pragma unroll
@@ -485,7 +487,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemv_q4_reg_kernel(const unsigned c
             double t = 0.0;
 #pragma unroll
             for (int w = 0; w < kWavesPerBlock; ++w) t += red[0][w];
-            if (KIND == 1) scale = 1.0f / sqrtf((float)(t / cols) + eps);
+            if (KIND == 1) scale = pi_inv_sqrt((float)(t / cols) + eps);
             else {
                 mean = (float)(t / cols);
                 double s2 = 0.0;
@@ -499,7 +501,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemv_q4_reg_kernel(const unsigned c
                 double t2 = 0.0;
 #pragma unroll
                 for (int w = 0; w < kWavesPerBlock; ++w) t2 += red[1][w];
-                scale = 1.0f / sqrtf((float)(t2 / cols) + eps);
+                scale = pi_inv_sqrt((float)(t2 / cols) + eps);
             }
         }
 #pragma unroll
@@ -517,8 +519,8 @@ __global__ __launch_bounds__(kBlock, 2) void gemv_q4_reg_kernel(const unsigned c
             // a quad of lanes holds one block of 32 values
             amax = fmaxf(amax, pi_dpp_f32<PI_DPP_XOR1, 0xF>(amax));
             amax = fmaxf(amax, pi_dpp_f32<PI_DPP_XOR2, 0xF>(amax));
-            const float d = amax / 127.0f;
-            const float id = (amax != 0.0f) ? 127.0f / amax : 0.0f;
+            const float d = pi_div(amax, 127.0f);
+            const float id = (amax != 0.0f) ? pi_div(127.0f, amax) : 0.0f;
             int q[8], qs = 0;
 #pragma unroll
             for (int k = 0; k < 8; ++k) { q[k] = (int)rintf(__fmul_rn(xv[i][k], id)); qs += q[k]; }
@@ -864,7 +866,7 @@ __global__ __launch_bounds__(kBlock) void pred_upgate_f16_kernel(const __half * 
                     s += (double)__fmul_rn(v.x, v.x); s += (double)__fmul_rn(v.y, v.y); s += (double)__fmul_rn(v.z, v.z); s += (double)__fmul_rn(v.w, v.w);
                 }
             s = pi_wave_sum_f64(s);
-            scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
+            scale = pi_inv_sqrt((float)(s / cols) + na.eps);
         } else if (na.kind == 2) {
             double s = 0.0;
 #pragma unroll
@@ -883,7 +885,7 @@ __global__ __launch_bounds__(kBlock) void pred_upgate_f16_kernel(const __half * 
                     s2 += (double)__fmul_rn(p, p); s2 += (double)__fmul_rn(q, q); s2 += (double)__fmul_rn(c, c); s2 += (double)__fmul_rn(e, e);
                 }
             s2 = pi_wave_sum_f64(s2);
-            scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
+            scale = pi_inv_sqrt((float)(s2 / cols) + na.eps);
         }
 #pragma unroll
         for (int j = 0; j < NCH; ++j) {
@@ -1067,7 +1069,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
         double t = 0.0;
 #pragma unroll
         for (int w = 0; w < kPfWaves; ++w) t += red[0][w];
-        scale = 1.0f / sqrtf((float)(t / cols) + na.eps);
+        scale = pi_inv_sqrt((float)(t / cols) + na.eps);
     } else if (na.kind == 2) {
         double sm = 0.0;
 #pragma unroll
@@ -1092,7 +1094,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
         double t2 = 0.0;
 #pragma unroll
         for (int w = 0; w < kPfWaves; ++w) t2 += red[1][w];
-        scale = 1.0f / sqrtf((float)(t2 / cols) + na.eps);
+        scale = pi_inv_sqrt((float)(t2 / cols) + na.eps);
     } else {
         __syncthreads();
     }
@@ -1348,7 +1350,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
         double t = 0.0;
 #pragma unroll
         for (int w = 0; w < kPfWaves; ++w) t += red[0][w];
-        scale = 1.0f / sqrtf((float)(t / cols) + na.eps);
+        scale = pi_inv_sqrt((float)(t / cols) + na.eps);
     } else if (na.kind == 2) {
         double sm = 0.0;
 #pragma unroll
@@ -1369,7 +1371,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
         double t2 = 0.0;
 #pragma unroll
         for (int w = 0; w < kPfWaves; ++w) t2 += red[1][w];
-        scale = 1.0f / sqrtf((float)(t2 / cols) + na.eps);
+        scale = pi_inv_sqrt((float)(t2 / cols) + na.eps);
     } else {
         __syncthreads();
     }
@@ -1388,7 +1390,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
     }
     amax = fmaxf(amax, pi_dpp_f32<PI_DPP_XOR1, 0xF>(amax));
     amax = fmaxf(amax, pi_dpp_f32<PI_DPP_XOR2, 0xF>(amax));
-    const float dq = amax / 127.0f, idq = (amax != 0.0f) ? 127.0f / amax : 0.0f;
+    const float dq = pi_div(amax, 127.0f), idq = (amax != 0.0f) ? pi_div(127.0f, amax) : 0.0f;
     const float dx = pi_round_f16(dq);
     int xq0 = 0, xq1 = 0, sx = 0;
 #pragma unroll
@@ -1502,7 +1504,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void axpy_q4_groups_kernel(const pi_bl
             float amax = fabsf(hvv);
 #pragma unroll
             for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, PI_WAVE));
-            const float d = amax / 127.0f, id = (amax != 0.0f) ? 127.0f / amax : 0.0f;
+            const float d = pi_div(amax, 127.0f), id = (amax != 0.0f) ? pi_div(127.0f, amax) : 0.0f;
             const int q = (int)rintf(__fmul_rn(hvv, id));
             const int g = nrn >> 5;
             const uint32_t hot = (nrn < ff) ? (hot_words ? hot_words[g] : 0xFFFFFFFFu) : 0u;
@@ -2046,8 +2048,8 @@ __global__ __launch_bounds__(kBlock) void h_q8_gather_kernel(const float * __res
         float amax = 0.0f;
 #pragma unroll
         for (int j = 0; j < 32; ++j) amax = fmaxf(amax, fabsf(blk[j]));
-        const float d = amax / 127.0f;
-        const float id = (amax != 0.0f) ? 127.0f / amax : 0.0f;
+        const float d = pi_div(amax, 127.0f);
+        const float id = (amax != 0.0f) ? pi_div(127.0f, amax) : 0.0f;
         hq[k] = (int)rintf(__fmul_rn(h_dense[neuron], id));
         hd[k] = pi_round_f16(d);
     }
@@ -2153,7 +2155,7 @@ __global__ __launch_bounds__(kBlock) void attn_decode_kernel(const float * __res
     const int lpp = hd / 8;                                       // lanes per position (16 B each)
     const int tid = threadIdx.x;
     const int sub = tid % lpp, grp = tid / lpp, ngrp = blockDim.x / lpp;
-    const float scale = 1.0f / sqrtf((float)hd);
+    const float scale = pi_inv_sqrt((float)hd);
 
     // q chunk of this lane, rounded to fp16 as the CPU dot does
     float qf[8];
@@ -2208,14 +2210,6 @@ __global__ __launch_bounds__(kBlock) void attn_decode_kernel(const float * __res
 // cos/sin of every (position, pair) the way the CPU path forms them: theta advanced by repeated fp32
 // multiplication (ggml.c:11269-11319), so the angle is bit-identical and only cosf/sinf can differ in the
 // last place.  table[p][i] = (cos, sin) for pair i of position p.
-__global__ void rope_table_kernel(float2 * __restrict__ table, int n_ctx, int half_dim, float theta_scale) {
-    const int p = blockIdx.x, i = threadIdx.x;
-    if (p >= n_ctx || i >= half_dim) return;
-    float theta = (float)p;
-    for (int j = 0; j < i; ++j) theta = __fmul_rn(theta, theta_scale);
-    table[(size_t)p * half_dim + i] = make_float2(cosf(theta), sinf(theta));
-}
-
 // ---------------------------------------------------------------------------------------------------
 // RoPE + KV store + decode attention in one launch, one workgroup per query head.  The workgroup rotates its
 // own q head and the k head of its group (cos/sin from the table), rounds k and v to fp16 as the cache does,
@@ -2284,7 +2278,7 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
     }
     __syncthreads();
 
-    const float scale = 1.0f / sqrtf((float)hd);
+    const float scale = pi_inv_sqrt((float)hd);
     float qf[8];
 #pragma unroll
     for (int i = 0; i < 8; ++i) qf[i] = qs[sub * 8 + i];
@@ -2437,7 +2431,7 @@ __global__ void fill_normal_q4_0_kernel(pi_block_q4_0 * __restrict__ p, size_t n
             if (fabsf(v[j]) > amax) { amax = fabsf(v[j]); mx = v[j]; }
         }
         const float d = mx / -8.0f;
-        const float id = d != 0.0f ? 1.0f / d : 0.0f;
+        const float id = d != 0.0f ? pi_div(1.0f, d) : 0.0f;
         pi_block_q4_0 blk;
         blk.d = pi_f16_bits(d);
 #pragma unroll
@@ -2484,7 +2478,7 @@ __global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __re
 #pragma unroll
             for (int k = 0; k < 8; ++k) s += (double)__fmul_rn(xv[k], xv[k]);
             s = block_sum_f64(s, red);
-            scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
+            scale = pi_inv_sqrt((float)(s / cols) + na.eps);
         } else if (na.kind == 2) {
             double s = 0.0;
 #pragma unroll
@@ -2495,7 +2489,7 @@ __global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __re
 #pragma unroll
             for (int k = 0; k < 8; ++k) { const int i = threadIdx.x + k * 1024; const float v = __fsub_rn(xv[k], mean); if (i < cols) s2 += (double)__fmul_rn(v, v); }
             s2 = block_sum_f64(s2, red);
-            scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
+            scale = pi_inv_sqrt((float)(s2 / cols) + na.eps);
         }
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
@@ -2517,7 +2511,7 @@ __global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __re
         double s = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = xt[i]; s += (double)__fmul_rn(v, v); }
         s = block_sum_f64(s, red);
-        scale = 1.0f / sqrtf((float)(s / cols) + na.eps);
+        scale = pi_inv_sqrt((float)(s / cols) + na.eps);
     } else if (na.kind == 2) {
         double s = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) s += (double)xt[i];
@@ -2526,7 +2520,7 @@ __global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __re
         double s2 = 0.0;
         for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = __fsub_rn(xt[i], mean); s2 += (double)__fmul_rn(v, v); }
         s2 = block_sum_f64(s2, red);
-        scale = 1.0f / sqrtf((float)(s2 / cols) + na.eps);
+        scale = pi_inv_sqrt((float)(s2 / cols) + na.eps);
     }
     for (int i = threadIdx.x; i < cols; i += blockDim.x) {
         float v = xt[i];
@@ -3548,8 +3542,22 @@ int pi_k_attn_decode(const float * q_rot, const void * k_cache, const void * v_c
 
 int pi_k_rope_table(void * table, int n_ctx, int hd, float theta_scale, pi_stream_t stream) {
     if (!table || n_ctx <= 0 || hd <= 0 || hd % 2 || hd / 2 > 1024) return pi::fail(PI_E_ARG, "pi_k_rope_table: bad arguments");
-    hipLaunchKernelGGL(rope_table_kernel, dim3(n_ctx), dim3(hd / 2), 0, (hipStream_t)stream, (float2 *)table, n_ctx, hd / 2, theta_scale);
-    return pi::check_launch("pi_k_rope_table");
+    // A set-up call: the table is computed on the host with the C library's cosf / sinf -- the functions the CPU path itself calls
+    // (ggml.c:11163-11325: theta = position, then *= theta_scale per pair) -- so rotated q and k start from bit-identical factors;
+    // the device's own cosf / sinf may differ from them in the last place.
+    const int half = hd / 2;
+    std::vector<float> host((size_t)n_ctx * hd);
+    for (int p = 0; p < n_ctx; ++p) {
+        float theta = (float)p;
+        for (int i = 0; i < half; ++i) {
+            host[((size_t)p * half + i) * 2]     = cosf(theta);
+            host[((size_t)p * half + i) * 2 + 1] = sinf(theta);
+            theta *= theta_scale;
+        }
+    }
+    PI_HIP_TRY(hipStreamSynchronize((hipStream_t)stream));
+    PI_HIP_TRY(hipMemcpy(table, host.data(), host.size() * sizeof(float), hipMemcpyHostToDevice));
+    return PI_OK;
 }
 
 // LDS of attn_fused_kernel: the scores of every cell, one partial output row per group of hd/8 lanes, and q, k, v of the new cell

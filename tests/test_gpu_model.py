@@ -202,7 +202,7 @@ def run_north_star(hp, n_prompt=8, n_gen=64):
 
 NS = dict(pred_margin=True, head_pair=2048)
 # seeds whose greedy path (a CPU-oracle property) visits both tokens of the pair
-SEED_7B_F16, SEED_7B_Q4, SEED_F40 = 35, 40, 29
+SEED_7B_F16, SEED_7B_Q4, SEED_F40 = 35, 40, 44
 
 
 # (Q4_0 at this width is left to run_case: 256-wide activations make one int8 rounding step a visible share of a dot product, and

@@ -213,6 +213,23 @@ PI_API int pi_k_sparse_ffn(const void * fc2_f16, int ff, int r, const float * hi
                            int epilogue, const float * add1, const float * add2, float * out,
                            float * logits, float * h_dense, int32_t * n_active,
                            pi_workspace * ws, pi_stream_t stream);
+/*
+ * pi_k_sparse_ffn for callers that cannot allocate device memory (code under HIP graph capture, tight serving loops, harnesses
+ * that forbid hipMalloc).  No counterpart in the reference.  Same arguments and results as pi_k_sparse_ffn minus the workspace:
+ * the per-workgroup partial vectors and the activity words live in a static device array of
+ * pi_k_sparse_ffn_noalloc_scratch_bytes() (8 MiB + 32 KiB) that each GPU the library runs on holds until the process ends.  The call
+ * allocates and frees nothing.  Shapes whose partial vectors exceed 8 MiB ((ff / 32) * cols floats at cols 4096, (ff / 128) * cols
+ * at cols 8192 when ff / 128 >= 256) or with ff > 131072 are refused with PI_E_UNSUPPORTED (_supported tells beforehand).
+ * All calls on one GPU share the array: calls that overlap on one GPU (different streams or threads) race; calls on one stream
+ * are ordered.  Nothing in the array has to be cleared between calls (every word a call reads it has written itself).
+ */
+PI_API size_t pi_k_sparse_ffn_noalloc_scratch_bytes(void);
+PI_API int pi_k_sparse_ffn_noalloc_supported(int ff, int r, int cols);
+PI_API int pi_k_sparse_ffn_noalloc(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                                   const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols,
+                                   const float * x, const pi_norm * norm,
+                                   int epilogue, const float * add1, const float * add2, float * out,
+                                   float * logits, float * h_dense, int32_t * n_active, pi_stream_t stream);
 PI_API int pi_k_pred_upgate_supported(int ff, int r, int cols);      /* 1 if the fused kernel covers the shape */
 PI_API int pi_k_pred_upgate(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
                             const void * up_f16, const void * gate_f16, int cols, const float * x, const pi_norm * norm,

@@ -3456,6 +3456,70 @@ int pi_k_sparse_ffn(const void * fc2_f16, int ff, int r, const float * hidden, f
     return pi_k_sparse_ffn_reduce(ff, cols, epilogue, add1, add2, out, n_active, ws, stream);
 }
 
+// ---- the fused sparse FFN for callers that may not allocate ------------------------------------------------
+// The block's scratch (per-workgroup partial outputs, activity words) lives in a file-scope device array instead of a
+// pi_workspace, so the call reaches no allocator.  Every call on a device shares that device's array.
+}  // extern "C"
+
+constexpr size_t kNaPartialBytes = (size_t)8 << 20;      // per-workgroup partial vectors: n_parts * cols floats
+constexpr int    kNaMaxWords     = 4096;                 // activity words: ff / 32
+constexpr size_t kNaScratchBytes = kNaPartialBytes + 2 * sizeof(uint32_t) * kNaMaxWords;
+static __device__ __align__(256) unsigned char scratch[kNaScratchBytes];
+
+namespace {
+constexpr int kNaMaxDevices = 16;
+unsigned char * g_na_ptr[kNaMaxDevices] = {};            // device address of `scratch` on each device (the name itself is not one)
+}
+
+// resolves the scratch array's address on the current device, once per device
+static int noalloc_setup_current_device(unsigned char ** out) {
+    int dev = -1;
+    PI_HIP_TRY(hipGetDevice(&dev));
+    if (dev < 0 || dev >= kNaMaxDevices) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn_noalloc: device index beyond 15");
+    if (!g_na_ptr[dev]) {
+        unsigned char * p = nullptr;
+        PI_HIP_TRY(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
+        if (!p) return pi::fail(PI_E_HIP, "pi_k_sparse_ffn_noalloc: the scratch array has no device address");
+        g_na_ptr[dev] = p;
+    }
+    if (out) *out = g_na_ptr[dev];
+    return PI_OK;
+}
+
+namespace pi {
+int noalloc_setup() { return noalloc_setup_current_device(nullptr); }      // called by pi_init with the device current
+}
+
+extern "C" {
+
+size_t pi_k_sparse_ffn_noalloc_scratch_bytes(void) { return kNaScratchBytes; }
+
+int pi_k_sparse_ffn_noalloc_supported(int ff, int r, int cols) {
+    if (!pi_k_sparse_ffn_supported(ff, r, cols)) return 0;
+    const size_t parts = (size_t)(ff / (32 * pf_groups(ff, cols)));
+    return ff / 32 <= kNaMaxWords && parts * (size_t)cols * sizeof(float) <= kNaPartialBytes;
+}
+
+int pi_k_sparse_ffn_noalloc(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                            const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x, const pi_norm * norm,
+                            int epilogue, const float * add1, const float * add2, float * out,
+                            float * logits, float * h_dense, int32_t * n_active, pi_stream_t stream) {
+    if (!pi_k_sparse_ffn_supported(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn_noalloc: shape outside the fused kernel (cols 4096 or 8192, r 512 or 1024, ff % 32 == 0)");
+    if (!pi_k_sparse_ffn_noalloc_supported(ff, r, cols))
+        return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn_noalloc: shape exceeds the static scratch (at most 8 MiB of partial vectors = (ff / 32 or ff / 128) * cols floats, ff <= 131072)");
+    unsigned char * base = nullptr;
+    const int rc = noalloc_setup_current_device(&base);
+    if (rc != PI_OK) return rc;
+    // a workspace view of the static array: only the members the fused route touches
+    pi_workspace ws{};
+    ws.max_ff = kNaMaxWords * 32; ws.max_d = cols;
+    ws.ffn_partial = reinterpret_cast<float *>(base);
+    ws.words       = reinterpret_cast<uint32_t *>(base + kNaPartialBytes);
+    ws.words_hot   = ws.words + kNaMaxWords;
+    return pi_k_sparse_ffn(fc2_f16, ff, r, hidden, threshold, up_f16, gate_f16, down_t_f16, cols, x, norm, epilogue, add1, add2, out,
+                           logits, h_dense, n_active, &ws, stream);
+}
+
 int pi_k_norm_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, void * out_plain_f16, pi_stream_t stream) {
     if (!x || !out_f16 || T <= 0 || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_norm_round_f16: bad arguments");
     hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16, (__half *)out_plain_f16);

@@ -35,7 +35,7 @@ int pi_init(int device) {
     hipDeviceProp_t p;
     PI_HIP_TRY(hipGetDeviceProperties(&p, device));
     if (p.warpSize != 64) return pi::fail(PI_E_UNSUPPORTED, "pi_init: kernels are written for 64-wide wavefronts");
-    return PI_OK;
+    return pi::noalloc_setup();
 }
 
 int pi_device_name(char * buf, size_t n) {

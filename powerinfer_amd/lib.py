@@ -55,6 +55,9 @@ _SIGS = {
     "pi_k_sparse_axpy": (_i, [_i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_supported": (_i, [_i, _i, _i]),
     "pi_k_sparse_ffn": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_sparse_ffn_noalloc_scratch_bytes": (_sz, []),
+    "pi_k_sparse_ffn_noalloc_supported": (_i, [_i, _i, _i]),
+    "pi_k_sparse_ffn_noalloc": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_pred_upgate_q4_supported": (_i, [_i, _i, _i]),
     "pi_k_pred_upgate_q4": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_axpy_q4_partials": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),

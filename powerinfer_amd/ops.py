@@ -106,9 +106,10 @@ class SparseFFN:
         return dict(logits=self.logits.download(np.float32), h=self.h_dense.download(np.float32),
                     n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32))
 
-    def forward_one_launch(self, x_ffn, x_pred, epilogue=pl.EPI_NONE, resid=None):
+    def forward_one_launch(self, x_ffn, x_pred, epilogue=pl.EPI_NONE, resid=None, noalloc=False):
         """fc1, then pi_k_sparse_ffn: predictor fc2, mask, gate/up, h and the down projection in one launch plus the
-        fixed-order reduction of the per-workgroup partial outputs.  Returns dict(logits, h, n_active, out)."""
+        fixed-order reduction of the per-workgroup partial outputs.  Returns dict(logits, h, n_active, out).
+        noalloc: go through pi_k_sparse_ffn_noalloc (scratch in the library's static device array, no workspace)."""
         L = self.L
         if self.bucket is not None or self.wtype != pl.F16 or not L.pi_k_sparse_ffn_supported(self.ff, self.r, self.d):
             raise pl.PiError("forward_one_launch: shape or placement outside the fused kernel")
@@ -119,10 +120,14 @@ class SparseFFN:
         check(L.pi_memset(self.h_dense.ptr, 0xFF, self.h_dense.nbytes), "memset")      # the kernel must write every entry
         nrm = pl.norm_arg(self.norm_kind, self.eps, self.norm_w, self.norm_b)
         check(L.pi_k_gemv(pl.F16, self.fc1.ptr, self.r, self.d, self.xp.ptr, None, pl.EPI_RELU, None, None, self.hidden.ptr, None), "fc1")
-        check(L.pi_k_sparse_ffn(self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, self.up.ptr,
-                                self.gate.ptr if self.gate is not None else None, self.down.ptr, self.d, self.x.ptr, nrm,
-                                epilogue, self.resid.ptr if epilogue else None, None, self.out.ptr,
-                                self.logits.ptr, self.h_dense.ptr, self.n_active.ptr, self.ws, None), "sparse_ffn")
+        args = (self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, self.up.ptr,
+                self.gate.ptr if self.gate is not None else None, self.down.ptr, self.d, self.x.ptr, nrm,
+                epilogue, self.resid.ptr if epilogue else None, None, self.out.ptr,
+                self.logits.ptr, self.h_dense.ptr, self.n_active.ptr)
+        if noalloc:
+            check(L.pi_k_sparse_ffn_noalloc(*args, None), "sparse_ffn_noalloc")
+        else:
+            check(L.pi_k_sparse_ffn(*args, self.ws, None), "sparse_ffn")
         pl.sync()
         return dict(logits=self.logits.download(np.float32), h=self.h_dense.download(np.float32),
                     n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32))

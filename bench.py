@@ -360,7 +360,9 @@ def main():
         out["cpu_baseline"] = {
             "value": round(v, 3), "unit": "tok/s", "cores": threads, "kind": "port",
             "sample": f"same {hp.n_layer}-layer model and weights (copied back from HBM), {n_prompt}-token prompt then "
-                      f"{cpu_tokens} greedy decode tokens timed, oracle/pi_oracle.c with OpenMP",
+                      f"{cpu_tokens} greedy decode tokens timed, oracle/pi_oracle.c with OpenMP; on the build container this port runs "
+                      f"the 7B sparse FFN block in 0.67x (1 thread) / 0.36x (8 threads) the time of the reference's own ggml.c "
+                      f"(oracle/calibrate_cpu.py), so it overstates the reference's CPU path by about 1.5-2.8x",
         }
     m.close()
     print(json.dumps(out), flush=True)

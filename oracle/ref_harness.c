@@ -20,6 +20,7 @@
 #include <stdio.h>
 #include <stdlib.h>
 #include <string.h>
+#include <time.h>
 
 #define REF_API __attribute__((visibility("default")))
 
@@ -39,6 +40,12 @@ static struct ggml_tensor * put2d(struct ggml_context * ctx, enum ggml_type t, i
 }
 
 REF_API void ref_set_threshold(float thr) { sparse_pred_threshold = thr; }
+
+/* ref_set_repeat(n > 1): the next ref_ffn_sparse calls run their graph n more times and keep the mean time of one run */
+static int g_repeat = 1;
+static double g_last_ms = 0.0;
+REF_API void ref_set_repeat(int n) { g_repeat = n; }
+REF_API double ref_last_compute_ms(void) { return g_last_ms; }
 
 /*
  * One sparse FFN block exactly as a CPU-only build of llama.cpp assembles it:
@@ -92,7 +99,19 @@ REF_API int ref_ffn_sparse(int d, int ff, int r, int T, int wtype, int has_gate,
 
     struct ggml_cgraph * gf = ggml_new_graph(ctx);
     ggml_build_forward_expand(gf, res);
-    ggml_graph_compute_with_ctx(ctx, gf, n_threads);
+    if (g_repeat <= 1) {
+        ggml_graph_compute_with_ctx(ctx, gf, n_threads);
+    } else {                                         /* timing: the graph alone, set-up and copies excluded */
+        struct ggml_cplan plan = ggml_graph_plan(gf, n_threads);
+        plan.work_data = plan.work_size ? malloc(plan.work_size) : NULL;
+        ggml_graph_compute(gf, &plan);
+        struct timespec t0, t1;
+        clock_gettime(CLOCK_MONOTONIC, &t0);
+        for (int i = 0; i < g_repeat; ++i) ggml_graph_compute(gf, &plan);
+        clock_gettime(CLOCK_MONOTONIC, &t1);
+        g_last_ms = ((t1.tv_sec - t0.tv_sec) * 1e3 + (t1.tv_nsec - t0.tv_nsec) * 1e-6) / g_repeat;
+        free(plan.work_data);
+    }
 
     if (logits)          memcpy(logits,   idx->data, (size_t)ff * T * 4);
     if (up_out)          memcpy(up_out,   upo->data, (size_t)ff * T * 4);

@@ -155,6 +155,37 @@ def cpu_baseline(hp, keep, prompt, n_prompt, n_decode, threads):
     return n_decode / dt
 
 
+def reference_host_on_this_backend(n_layer=4, n_prompt=8, n_gen=48):
+    """The cost of per-node dispatch as a number: the reference's own llama.cpp (loader, ggml-alloc, graph builder, executor)
+    compiled against this library in place of ggml-cuda.cu (oracle/_ref/ref_llama_gpu, test infrastructure) decodes a 7B-wide,
+    n_layer-deep synthetic model with every tensor on the GPU, one ggml_cuda_compute_forward call per graph node."""
+    import subprocess
+    import tempfile
+    from powerinfer_amd import gguf, split, synth
+    exe = os.path.join(ROOT, "oracle", "_ref", "ref_llama_gpu")
+    if not os.path.exists(exe):
+        return None
+    hp = synth.hparams("llama-7b", n_layer=n_layer, n_ctx=128, seed=3)
+    model = synth.make_model(hp)
+    with tempfile.TemporaryDirectory() as td:
+        path, out = os.path.join(td, "m.powerinfer.gguf"), os.path.join(td, "out.bin")
+        gguf.write_model(path, model, gguf.synthetic_tokenizer_kv(hp.n_vocab))
+        splits = [(np.ones(hp.n_ff, np.int32), np.arange(hp.n_ff, dtype=np.int32)) for _ in range(hp.n_layer)]
+        split.write_gpuidx(path + ".generated.gpuidx", splits, split.required_bytes(hp, splits))
+        del model
+        toks = [str(int(t)) for t in np.random.default_rng(5).integers(0, hp.n_vocab, n_prompt)]
+        r = subprocess.run([exe, path, "128", "1", str(n_gen), out] + toks, env=dict(os.environ, REF_VRAM_GB="16"),
+                           capture_output=True, text=True, timeout=240)
+    if r.returncode != 0:
+        return {"error": (r.stdout + r.stderr)[-300:]}
+    ms = [float(l.split()[1]) for l in r.stdout.splitlines() if l.startswith("decode_ms_per_token")]
+    if not ms:
+        return {"error": "no timing line"}
+    return {"ms_per_token": round(ms[0], 3), "n_layer": n_layer, "ms_per_token_per_layer": round(ms[0] / n_layer, 4), "host_threads": 1,
+            "what": "reference llama.cpp + ggml executor linked to libpowerinfer_hip.so (oracle/_ref/ref_llama_gpu), 7B-wide layers, "
+                    "all tensors and the KV cache on the GPU, one backend call per graph node; includes the lm-head once per token"}
+
+
 def bench_batched(args):
     """configs[3]: 13B shape, 16 sequences advancing one token per step; the whole-job rate counts every sequence's token."""
     from powerinfer_amd import lib as pl, synth
@@ -206,6 +237,7 @@ def main():
     ap.add_argument("--prompt", type=int, default=64)
     ap.add_argument("--layers", type=int, default=32, help="only for quick trials; the reported workload uses 32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-ref-host", action="store_true", help="skip the leg that runs the reference's llama.cpp on this backend (about 40 s)")
     ap.add_argument("--cpu-tokens", type=int, default=320, help="decode tokens timed on the host for the cpu_baseline leg (about 10 s of CPU work)")
     ap.add_argument("--config", type=int, default=1, choices=[1, 2, 3, 4],
                     help="BASELINE configs index: 1 (default, the reported metric) 7B FP16 all on the GPU; 2 the same shape in "
@@ -284,9 +316,27 @@ def main():
         ms_qkv, n_qkv = m.time_section(0, 8)
         ms_ffn, _ = m.time_section(1, 8)
         ms_head, _ = m.time_section(2, 8)
+        try:
+            ms_pf, n_pf = m.time_section(3, 8)            # the fused predictor + FFN kernel alone, and the reduction behind it
+            ms_fr, _ = m.time_section(4, 8)
+        except Exception:
+            ms_pf, n_pf, ms_fr = float("nan"), 0, float("nan")
     achieved = qkv_bytes / (ms_qkv * 1e-3) / 1e9
     n_mats = 2 if hp.arch == "falcon" else 3
     ffn_bytes = (d * hp.n_rank + hp.n_rank * hp.n_ff) * 2.0 + (act.mean() / hp.n_layer) * n_mats * d * wbytes
+
+    # the kernel next to it in time per token: fc2 rows of every neuron, the gate/up/down rows of the active ones, the input vector,
+    # the norm weights and the hidden vector in; the logits-free path writes one partial output vector per 32 neurons
+    a_layer = act.mean() / hp.n_layer
+    pf_bytes = hp.n_rank * hp.n_ff * 2.0 + a_layer * n_mats * d * 2.0 + (2 * d + hp.n_rank) * 4.0 + (hp.n_ff / 32.0) * d * 4.0
+    pf_traffic = None
+    try:
+        with open(os.path.join(ROOT, "profiles", "sparse_ffn_hbm_traffic.json")) as f:
+            pj = json.load(f)
+        if pj.get("shape") == [hp.n_ff, d, hp.n_rank] and args.config == 1:
+            pf_traffic = pj["traffic_bytes_per_launch"]
+    except (OSError, ValueError, KeyError):
+        pass
 
     # HBM bytes per launch of that kernel from the FETCH_SIZE / WRITE_SIZE counter runs (profiles/qkv_gemv_hbm_traffic.md)
     traffic = None
@@ -341,6 +391,21 @@ def main():
             "us_per_launch": rnd(ms_qkv * 1e3, 2),
             "launches_timed": n_qkv,
         },
+        "roofline_sparse_ffn": {
+            "bound": "hbm",
+            "kernel": {1: "pred_ffn_f16_kernel<1,2,true,1,false> (predictor fc2 11008 x 1024 + mask + gate/up/down rows of the active neurons, 7B layer)",
+                       2: "pred_upgate_q4_kernel (not timed for a hybrid model)",
+                       4: "pred_ffn_f16_kernel<2,2,false,4,false> (predictor fc2 32768 x 1024 + mask + up/down rows of the active neurons, Falcon-40B layer)"}[args.config],
+            "achieved": rnd(pf_bytes / (ms_pf * 1e-3) / 1e9, 1),
+            "peak": HBM_PEAK_GBPS,
+            "unit": "GB/s",
+            "frac": rnd(pf_bytes / (ms_pf * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+            "traffic": pf_traffic,
+            "bytes_per_launch": round(pf_bytes),
+            "us_per_launch": rnd(ms_pf * 1e3, 2),
+            "reduce_us_per_launch": rnd(ms_fr * 1e3, 2),
+            "launches_timed": n_pf,
+        },
         "token_loop": {
             "device_ms_per_step": round(ms_dev / args.steps, 4),
             "touched_GB_per_token": round(tok_bytes / 1e9, 4),
@@ -365,6 +430,14 @@ def main():
                       f"(oracle/calibrate_cpu.py), so it overstates the reference's CPU path by about 1.5-2.8x",
         }
     m.close()
+    del keep
+    if not args.no_ref_host and args.config == 1:
+        try:
+            rh = reference_host_on_this_backend()
+        except Exception as e:          # a reporting extra: never costs the bench line
+            rh = {"error": repr(e)[:200]}
+        if rh is not None:
+            out["reference_host_on_this_backend"] = rh
     print(json.dumps(out), flush=True)
 
 

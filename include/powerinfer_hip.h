@@ -419,7 +419,8 @@ PI_API int pi_model_get_capture(pi_model * m, float * ffn_out, float * pred_logi
  * on the activations the last token left behind (the per-node timers of GGML_PERF, ggml.c:16604-16619, are the
  * nearest thing in the reference).  section 0: the q|k|v projection mat-vec of every layer (the kernel that
  * moves the most bytes per token); 1: the sparse FFN block of every layer (fc1, fc2+compaction, up/gate, axpy);
- * 2: the lm-head mat-vec.  ms_total: device milliseconds for everything issued; launches: number of
+ * 2: the lm-head mat-vec; 3: the fused predictor + gate/up/down kernel of every layer alone (F16 models the fused block
+ * covers); 4: the reduction of its partial vectors alone.  ms_total: device milliseconds for everything issued; launches: number of
  * section instances issued (rounds * n_layer, or rounds for the lm-head).
  */
 PI_API int pi_model_time_section(pi_model * m, int section, int rounds, float * ms_total, int * launches);

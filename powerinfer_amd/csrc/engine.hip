@@ -746,6 +746,21 @@ int pi_model_time_section(pi_model * m, int section, int rounds, float * ms_tota
                 PI_TRY(pi_k_sparse_axpy(down.type, down.dev, d, ff, m->h_c, q4 ? m->h_dense : nullptr, nullptr, m->list, m->n_active + il,
                                         PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, m->ws, st));
                 ++n;
+            } else if (section == 3 || section == 4) {
+                // one kernel of the fused F16 block alone: 3 the predictor + gate/up/down kernel, 4 the reduction of its partial vectors
+                Tensor & fc1 = m->L(il, PI_T_FC1); Tensor & fc2 = m->L(il, PI_T_FC2);
+                Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
+                if (up.type != PI_TYPE_F16 || !pi_k_sparse_ffn_supported(ff, (int)fc1.ne1, d))
+                    return pi::fail(PI_E_UNSUPPORTED, "pi_model_time_section: the fused F16 block does not cover this model");
+                pi_norm fn = falcon ? make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B))
+                                    : make_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
+                const float * fin = falcon ? m->x : m->ffn_inp;
+                if (section == 3)
+                    PI_TRY(pi_k_sparse_ffn_partials(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, down.dev, d,
+                                                    fin, &fn, nullptr, nullptr, m->ws, st));
+                else
+                    PI_TRY(pi_k_sparse_ffn_reduce(ff, d, PI_EPI_ADD, fin, nullptr, m->x2, m->n_active + il, m->ws, st));
+                ++n;
             } else {
                 return pi::fail(PI_E_ARG, "pi_model_time_section: unknown section");
             }

@@ -265,6 +265,16 @@ PI_API int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float thre
                                  int32_t * union_rows, int32_t * n_union,
                                  pi_workspace * ws, pi_stream_t stream);
 
+/* The two sparse operators of a step AS OPERATORS, for a host that runs the predictor itself and hands over its output idx [T][ff]
+ * (the reference's mul_mat_batch_sparse and axpy at batch size > 1, ggml-cuda.cu:6994-7034, 8787-8814): T <= 16, F16 rows, cols % 256 == 0.
+ *   pi_k_batch_sparse_mul_mat: y[t][n] = W[n] . xn_f16[t] where !(idx[t][n] < threshold), 0 elsewhere (y is [T][ff], fully written);
+ *   pi_k_batch_sparse_axpy:    out[t] = sum over n with !(idx[t][n] < threshold) of fp16(h[t][n]) * down_t[n][:]   (h is [T][ff], out [T][cols]).
+ * Each weight row is read once per step (rows active for at least one token); union_rows [ff] / n_union [1] are scratch the caller owns. */
+PI_API int pi_k_batch_sparse_mul_mat(const void * W_f16, int ff, int cols, const void * xn_f16, int T, const float * idx, float threshold,
+                                     float * y, int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream);
+PI_API int pi_k_batch_sparse_axpy(const void * down_t_f16, int cols, int ff, const float * h, const float * idx, int T, float threshold,
+                                  float * out, int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream);
+
 /* per-sequence pieces of a batched step: sequence t owns token t, position pos[t] and the cache at t * cache_seq_stride
  * (elements), out_f16 (optional) receives fp16(out); pi_k_argmax_batch picks each sequence's next token (first maximum wins), stores it in tokens[t], adds 1 to
  * positions[t] and records it at out_tokens[*step][t]; pi_k_step_advance then moves *step on. */

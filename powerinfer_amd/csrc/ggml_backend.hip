@@ -267,6 +267,17 @@ bool op_mul_mat(ggml_tensor * dst) {
     const char * wa = (const char *)dev_in(a, tmp); const char * xb = (const char *)dev_in(b, tmp); float * y = (float *)dev_out(dst, tmp);
     if (weight_like) {
         const int64_t T = nrows(b);
+        if (T > 1 && a->type == GGML_TYPE_F16 && a->ne[0] % 128 == 0) {          // the matrix is read once per 16 tokens (matrix cores)
+            const int cols = (int)a->ne[0], rows = (int)a->ne[1];
+            __half * xn16 = (__half *)tmp.get(sizeof(__half) * 16 * (size_t)cols);
+            for (int64_t t0 = 0; t0 < T; t0 += 16) {
+                const int tc = (int)(T - t0 < 16 ? T - t0 : 16);
+                BK_PI(pi_k_norm_round_f16((const float *)xb + t0 * cols, tc, cols, nullptr, xn16, nullptr, nullptr));
+                BK_PI(pi_k_gemm_f16(wa, rows, cols, xn16, tc, PI_EPI_NONE, nullptr, nullptr, y + t0 * rows, nullptr, nullptr));
+            }
+            finish_out(dst, y);
+            return true;
+        }
         for (int64_t t = 0; t < T; ++t)
             BK_PI(pi_k_gemv(a->type, wa, (int)a->ne[1], (int)a->ne[0], (const float *)xb + t * b->ne[0], nullptr, PI_EPI_NONE, nullptr, nullptr, y + t * a->ne[1], nullptr));
     } else {
@@ -296,6 +307,22 @@ bool sparse_common(ggml_tensor * dst, bool axpy) {
     int32_t * n_act = (int32_t *)tmp.get(sizeof(int32_t));
     float * hc = (float *)tmp.get(sizeof(float) * (size_t)rows);
     const int out_n = (int)dst->ne[0];
+    // a step of several tokens with every neuron resident: each weight row is read once for up to 16 tokens at a time (the
+    // reference's batch kernels, ggml-cuda.cu:6994-7034, 8787-8814); other layouts go token by token below
+    if (T > 1 && !aux && w->type == GGML_TYPE_F16 && d % 256 == 0 && d <= g_ws_d) {
+        __half * xn16 = axpy ? nullptr : (__half *)tmp.get(sizeof(__half) * 16 * (size_t)d);
+        for (int64_t t0 = 0; t0 < T; t0 += 16) {
+            const int tc = (int)(T - t0 < 16 ? T - t0 : 16);
+            if (!axpy) {
+                BK_PI(pi_k_norm_round_f16(xd + t0 * d, tc, d, nullptr, xn16, nullptr, nullptr));
+                BK_PI(pi_k_batch_sparse_mul_mat(wd, ff, d, xn16, tc, id + t0 * ff, g_threshold, y + t0 * out_n, list, n_act, ws, nullptr));
+            } else {
+                BK_PI(pi_k_batch_sparse_axpy(wd, d, ff, xd + t0 * ff, id + t0 * ff, tc, g_threshold, y + t0 * d, list, n_act, ws, nullptr));
+            }
+        }
+        finish_out(dst, y);
+        return true;
+    }
     for (int64_t t = 0; t < T; ++t) {
         BK_PI(pi_k_compact_active(id + t * ff, ff, g_threshold, bk, n_bucket, list, n_act, ws, nullptr));
         if (!axpy) {

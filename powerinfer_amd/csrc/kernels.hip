@@ -2695,6 +2695,29 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
     }
 }
 
+// the operator boundary hands over the predictor's output instead of running the predictor: row_any[n] = some token has !(idx[t][n] < thr)
+__global__ void batch_flag_any_kernel(const float * __restrict__ idx, int T, int ff, float thr, unsigned char * __restrict__ row_any) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= ff) return;
+    bool any = false;
+    for (int t = 0; t < T; ++t) any = any || !(idx[(size_t)t * ff + n] < thr);
+    row_any[n] = any ? 1 : 0;
+}
+// hc[t][u] = fp16(h[t][row_u]) where the row is active for token t, 0 elsewhere and in the padding up to the next multiple of 16
+__global__ void batch_gather_h_kernel(const float * __restrict__ h, const float * __restrict__ idx, int T, int ff, float thr,
+                                      const int32_t * __restrict__ list, const int32_t * __restrict__ n_union, __half * __restrict__ hc, int hstride) {
+    const int n = *n_union, n_pad = (n + 15) & ~15;
+    const int t = blockIdx.y;
+    for (int u = blockIdx.x * blockDim.x + threadIdx.x; u < n_pad; u += gridDim.x * blockDim.x) {
+        float v = 0.0f;
+        if (u < n && t < T) { const int row = list[u]; if (!(idx[(size_t)t * ff + row] < thr)) v = h[(size_t)t * ff + row]; }
+        hc[(size_t)t * hstride + u] = __float2half_rn(v);
+    }
+}
+__global__ void zero_f32_kernel(float * __restrict__ p, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0.0f;
+}
+
 // union over the tokens of the step of the predictor's active sets: ascending list of the neurons whose flag the
 // predictor's mat-mul epilogue raised (single workgroup: wave ballot per 64 neurons, popcount prefix over the mask words)
 __global__ __launch_bounds__(1024) void union_active_kernel(const unsigned char * __restrict__ row_any, int ff,
@@ -2795,7 +2818,9 @@ __global__ __launch_bounds__(kBlock) void batch_upgate_f16_kernel(const __half *
 __global__ __launch_bounds__(kBlock) void batch_upgate_lds_f16_kernel(const __half * __restrict__ Wup, const __half * __restrict__ Wgate, int cols,
                                                                       const __half * __restrict__ xn, int T, const float * __restrict__ logits, int ff, float thr,
                                                                       const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
-                                                                      __half * __restrict__ hc, int hstride) {
+                                                                      __half * __restrict__ hc, int hstride, float * __restrict__ raw) {
+    // raw != nullptr: the plain product of ONE matrix (Wgate == nullptr) for the operator boundary: raw[t][row] = Wup[row] . xn[t] for
+    // the tokens the row is active for and 0 for the others (rows outside the union list are zeroed by the caller); hc is not written
     __shared__ __align__(16) unsigned char tile[kWavesPerBlock][16 * kGlStride];
     __shared__ float cu[kWavesPerBlock][16][17], cg[kWavesPerBlock][16][17];
     const int n = *n_union;
@@ -2860,17 +2885,20 @@ __global__ __launch_bounds__(kBlock) void batch_upgate_lds_f16_kernel(const __ha
     for (int r = 0; r < 4; ++r) { cu[wave][4 * g + r][i] = au[r]; cg[wave][4 * g + r][i] = ag[r]; }
     __syncthreads();
     const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
-    float h = 0.0f;
+    float h = 0.0f, su = 0.0f;
+    int rrow = -1;
     if (u0 + rr < n && t < T) {
-        const int rrow = list[u0 + rr];
+        rrow = list[u0 + rr];
         if (!(logits[(size_t)t * ff + rrow] < thr)) {
-            float su = cu[0][rr][t], sg = cg[0][rr][t];
+            float sg = cg[0][rr][t];
+            su = cu[0][rr][t];
 #pragma unroll
             for (int w = 1; w < kWavesPerBlock; ++w) { su += cu[w][rr][t]; sg += cg[w][rr][t]; }
             h = has_gate ? __fmul_rn(fmaxf(sg, 0.0f), su) : fmaxf(su, 0.0f);
         }
     }
-    hc[(size_t)t * hstride + u0 + rr] = __float2half_rn(h);
+    if (raw) { if (rrow >= 0) raw[(size_t)t * ff + rrow] = su; }
+    else hc[(size_t)t * hstride + u0 + rr] = __float2half_rn(h);
 }
 
 // sparse down projection for the step: partial[g][t][c] = sum over the union entries of row group g of hc[u][t] * down[row_u][c].
@@ -3569,7 +3597,7 @@ int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, 
     const int hstride = ws->max_ff + 16;
     if (cols % 256 == 0) {
         hipLaunchKernelGGL(batch_upgate_lds_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
-                           (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
+                           (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride, (float *)nullptr);
         hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3((cols + 1023) / 1024, kBmGroups), dim3(kBlock), 0, st, (const __half *)down_t_f16, cols,
                            ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
         hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBmGroups, T, cols, epilogue, add1, add2, out);
@@ -3581,6 +3609,37 @@ int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, 
         hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBaGroups, T, cols, epilogue, add1, add2, out);
     }
     return pi::check_launch("pi_k_batch_sparse_ffn");
+}
+
+// The two sparse operators of a step of T <= 16 tokens AS OPERATORS (the reference's mul_mat_batch_sparse / axpy at batch size > 1,
+// ggml-cuda.cu:6994-7034, 8787-8814): the caller supplies the predictor output idx [T][ff]; each weight row is read once for the step.
+int pi_k_batch_sparse_mul_mat(const void * W_f16, int ff, int cols, const void * xn_f16, int T, const float * idx, float threshold,
+                              float * y, int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream) {
+    if (!W_f16 || !xn_f16 || !idx || !y || !union_rows || !n_union || !ws) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_mul_mat: null pointer");
+    if (T < 1 || T > kBtMaxT || ff <= 0 || ff > ws->max_ff || cols <= 0 || cols % 256) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_mul_mat: 1 <= T <= 16, ff <= workspace and cols % 256 == 0 required");
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(batch_flag_any_kernel, dim3((ff + 255) / 256), dim3(256), 0, st, idx, T, ff, threshold, ws->row_any);
+    hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, ws->row_any, ff, ws->words, union_rows, n_union);
+    hipLaunchKernelGGL(zero_f32_kernel, dim3(256), dim3(256), 0, st, y, (size_t)T * ff);
+    hipLaunchKernelGGL(batch_upgate_lds_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)W_f16, (const __half *)nullptr, cols,
+                       (const __half *)xn_f16, T, idx, ff, threshold, union_rows, n_union, ws->hc_batch, ws->max_ff + 16, y);
+    return pi::check_launch("pi_k_batch_sparse_mul_mat");
+}
+int pi_k_batch_sparse_axpy(const void * down_t_f16, int cols, int ff, const float * h, const float * idx, int T, float threshold,
+                           float * out, int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream) {
+    if (!down_t_f16 || !h || !idx || !out || !union_rows || !n_union || !ws) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_axpy: null pointer");
+    if (T < 1 || T > kBtMaxT || ff <= 0 || ff > ws->max_ff || cols <= 0 || cols > ws->max_d || cols % 256)
+        return pi::fail(PI_E_ARG, "pi_k_batch_sparse_axpy: 1 <= T <= 16, ff and cols within the workspace and cols % 256 == 0 required");
+    hipStream_t st = (hipStream_t)stream;
+    const int hstride = ws->max_ff + 16;
+    hipLaunchKernelGGL(batch_flag_any_kernel, dim3((ff + 255) / 256), dim3(256), 0, st, idx, T, ff, threshold, ws->row_any);
+    hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, ws->row_any, ff, ws->words, union_rows, n_union);
+    hipLaunchKernelGGL(batch_gather_h_kernel, dim3(32, kBtMaxT), dim3(256), 0, st, h, idx, T, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
+    hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3((cols + 1023) / 1024, kBmGroups), dim3(kBlock), 0, st, (const __half *)down_t_f16, cols,
+                       ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
+    hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBmGroups, T, cols, PI_EPI_NONE,
+                       (const float *)nullptr, (const float *)nullptr, out);
+    return pi::check_launch("pi_k_batch_sparse_axpy");
 }
 
 int pi_k_rope_kv_store(const float * qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale,

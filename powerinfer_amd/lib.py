@@ -75,6 +75,8 @@ _SIGS = {
     "pi_k_gemm_f16": (_i, [_vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_batch_predictor_fc2": (_i, [_vp, _i, _i, _vp, _i, _f, _vp, _vp, _vp]),
     "pi_k_batch_sparse_ffn": (_i, [_vp, _i, _i, _f, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_batch_sparse_mul_mat": (_i, [_vp, _i, _i, _vp, _i, _vp, _f, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_batch_sparse_axpy": (_i, [_vp, _i, _i, _vp, _vp, _i, _f, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_attn_fused_batch": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),
     "pi_k_attn_chunk": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     "pi_k_embed_batch": (_i, [_vp, _i, _vp, _i, _vp, _vp]),

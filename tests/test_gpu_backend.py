@@ -110,6 +110,29 @@ def test_hybrid_graph_cpu_part_plus_gpu_part(wtype):
     assert rel_err(G.host(out), out_under(L, wtype, True, L["x"], lg)) < 1e-4
 
 
+@pytest.mark.timeout(300)
+def test_full_gpu_graph_13b_step_of_16():
+    """configs[3]'s step as the reference's graph hands it over: 16 tokens through the FFN block of a 13B layer (d 5120, ff 13824,
+    predictor rank 1024), every node on the backend.  The sparse operators take the batch route (union of the active rows, each
+    weight row read once for the 16 tokens, matrix cores) instead of 16 single-token passes (ggml-cuda.cu:6994-7034, 8787-8814)."""
+    from powerinfer_amd import lib as pl
+    from ggml_graph import Graph
+    d, ff, r, T = 5120, 13824, 1024, 16
+    L = synth.make_ffn_layer(seed=67, d=d, ff=ff, r=r, wtype=ol.F16, has_gate=True, T=T)
+    G = Graph(pl.load())
+    idx, out = build_ffn(G, L, L["x"], ol.F16, True)
+    G.compute(0.0)
+    assert not G.cpu_run, G.cpu_run
+    o = ol.ffn_sparse(ol.oracle(), d, ff, r, T, ol.F16, True, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], L["x"], L["x"],
+                      np.zeros(ff, np.int32), 0.0, nth=8)
+    lg = G.host(idx)
+    assert rel_err(lg, o["logits"]) < 1e-5
+    assert ((lg >= 0) == (o["logits"] >= 0)).mean() >= 0.999
+    assert rel_err(G.host(out), out_under(L, ol.F16, True, L["x"], lg)) < 1e-4
+    per_token = ((lg >= 0).sum(1))
+    assert per_token.min() > 0 and len(set(per_token.tolist())) > 1          # the tokens' active sets differ: the union is a real union
+
+
 def test_backend_info_entry_points():
     from powerinfer_amd import lib as pl
     L = pl.load()

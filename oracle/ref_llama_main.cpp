@@ -8,6 +8,12 @@
 //
 //   ref_llama <model.gguf> <n_ctx> <n_threads> <n_generate> <out.bin> tok0 tok1 ...
 //
+// With REF_SCRIPT=<file> the tokens on the command line are ignored and the file is executed line by line instead:
+//     decode n  tok pos seq  tok pos seq ...   one llama_decode of n entries (token, position, sequence id); the logits of every entry
+//                                              are appended to <out.bin> in entry order
+//     rm seq p0 p1 | shift seq p0 p1 delta | cp src dst p0 p1      llama_kv_cache_seq_rm / _seq_shift / _seq_cp
+// <out.bin> then starts with {number of logits rows, n_vocab}.
+//
 // REF_VRAM_GB=<GiB> sets llama_model_params.vram_budget_gb (the accelerator build offloads by budget; the neuron split is
 // read from <model.gguf>.generated.gpuidx).  The time of the greedy steps is printed as "decode_ms_per_token <ms>".
 //
@@ -20,6 +26,7 @@
 #include <csignal>
 #include <cstdio>
 #include <cstdlib>
+#include <cstring>
 #include <vector>
 
 #include <execinfo.h>
@@ -67,6 +74,48 @@ int main(int argc, char ** argv) {
 
     FILE * f = fopen(out_path, "wb");
     if (!f) return 1;
+    if (const char * script = getenv("REF_SCRIPT")) {
+        FILE * sf = fopen(script, "r");
+        if (!sf) { fprintf(stderr, "cannot open %s\n", script); return 1; }
+        int32_t hdr2[2] = { 0, n_vocab };
+        fwrite(hdr2, 4, 2, f);
+        char op[16];
+        int n_rows = 0;
+        while (fscanf(sf, "%15s", op) == 1) {
+            if (!strcmp(op, "decode")) {
+                int n = 0;
+                if (fscanf(sf, "%d", &n) != 1 || n <= 0) return 1;
+                llama_batch b = llama_batch_init(n, 0, 1);
+                b.n_tokens = n;
+                for (int i = 0; i < n; ++i) {
+                    int tok_i, pos_i, seq_i;
+                    if (fscanf(sf, "%d %d %d", &tok_i, &pos_i, &seq_i) != 3) return 1;
+                    b.token[i] = tok_i; b.pos[i] = pos_i; b.n_seq_id[i] = 1; b.seq_id[i][0] = seq_i; b.logits[i] = 1;
+                }
+                if (llama_decode(ctx, b) != 0) { fprintf(stderr, "llama_decode failed\n"); return 1; }
+                for (int i = 0; i < n; ++i) { fwrite(llama_get_logits_ith(ctx, i), 4, n_vocab, f); ++n_rows; }
+                llama_batch_free(b);
+            } else if (!strcmp(op, "rm")) {
+                int q, p0, p1; if (fscanf(sf, "%d %d %d", &q, &p0, &p1) != 3) return 1;
+                llama_kv_cache_seq_rm(ctx, q, p0, p1);
+            } else if (!strcmp(op, "shift")) {
+                int q, p0, p1, dl; if (fscanf(sf, "%d %d %d %d", &q, &p0, &p1, &dl) != 4) return 1;
+                llama_kv_cache_seq_shift(ctx, q, p0, p1, dl);
+            } else if (!strcmp(op, "cp")) {
+                int a, b2, p0, p1; if (fscanf(sf, "%d %d %d %d", &a, &b2, &p0, &p1) != 4) return 1;
+                llama_kv_cache_seq_cp(ctx, a, b2, p0, p1);
+            } else { fprintf(stderr, "unknown script line %s\n", op); return 1; }
+        }
+        fclose(sf);
+        hdr2[0] = n_rows;
+        fseek(f, 0, SEEK_SET);
+        fwrite(hdr2, 4, 2, f);
+        fclose(f);
+        llama_free(ctx);
+        llama_free_model(model);
+        llama_backend_free();
+        return 0;
+    }
     const int n_steps = (int)prompt.size() + n_gen;
     int32_t hdr[2] = { n_steps, n_vocab };
     fwrite(hdr, 4, 2, f);

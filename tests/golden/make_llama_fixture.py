@@ -49,7 +49,42 @@ def case_model(name):
     return hp, synth.make_model(hp)
 
 
+def seq_edit_case():
+    """Three sequences in lockstep, then llama_kv_cache_seq_rm / _seq_shift / _seq_cp on them (the history of
+    tests/test_gpu_batch.py::test_batch_kv_sequence_edits), driven through the reference's own KV-cell bookkeeping."""
+    hp = synth.hparams("llama-tiny", seed=9, n_ctx=48, sparse_threshold=-1e30)
+    n_seq, n0 = 3, 8
+    toks = np.random.default_rng(21).integers(0, hp.n_vocab, (n0 + 1, n_seq)).astype(np.int32)
+    lines = []
+    for s in range(n0):
+        lines.append("decode %d " % n_seq + " ".join("%d %d %d" % (toks[s, q], s, q) for q in range(n_seq)))
+    lines += ["rm 0 2 5", "shift 0 5 8 -3", "rm 2 0 -1", "cp 1 2 0 6"]
+    last_pos = (5, 8, 6)
+    lines.append("decode %d " % n_seq + " ".join("%d %d %d" % (toks[n0, q], last_pos[q], q) for q in range(n_seq)))
+    return hp, toks, last_pos, lines
+
+
+def make_seq_edit_fixture():
+    hp, toks, last_pos, lines = seq_edit_case()
+    model = synth.make_model(hp)
+    with tempfile.TemporaryDirectory() as td:
+        path, out, script = os.path.join(td, "m.powerinfer.gguf"), os.path.join(td, "out.bin"), os.path.join(td, "script.txt")
+        gguf.write_model(path, model, gguf.synthetic_tokenizer_kv(hp.n_vocab))
+        with open(script, "w") as f:
+            f.write("\n".join(lines) + "\n")
+        subprocess.check_call([BIN, path, str(hp.n_ctx), "1", "0", out, "0"], stdout=subprocess.DEVNULL, stderr=subprocess.DEVNULL,
+                              env=dict(os.environ, REF_SCRIPT=script))
+        raw = np.fromfile(out, np.uint8)
+    n_rows, n_vocab = (int(v) for v in raw[:8].view(np.int32))
+    logits = raw[8:].view(np.float32).reshape(n_rows, n_vocab)
+    assert n_rows == 3 * 9
+    np.savez_compressed(os.path.join(HERE, "ref_llama_seq_edits.npz"), tokens=toks, last_pos=np.asarray(last_pos, np.int32),
+                        logits_last=logits[-3:], logits_step0=logits[:3], model_sha=model_sha(model))
+    print("seq edits: greedy of the last step", logits[-3:].argmax(1).tolist())
+
+
 def main():
+    make_seq_edit_fixture()
     for name, c in CASES.items():
         hp, model = case_model(name)
         _, vkv, _ = gguf.read_gguf(os.path.join(REF, "models", c["vocab"]))

@@ -191,6 +191,8 @@ class KVCells:
         self.seq = [set() for _ in range(n_ctx)]
 
     def find_slot(self, positions, seq_id=0):          # llama_kv_cache_find_slot, llama.cpp:1683-1736
+        """seq_id: one id for every token, or one per token."""
+        seq_ids = list(seq_id) if np.ndim(seq_id) else [seq_id] * len(positions)
         n, tested = len(positions), 0
         while True:
             if self.head + n > self.size:
@@ -206,7 +208,7 @@ class KVCells:
                 raise RuntimeError("no KV slot")
         for i, p in enumerate(positions):
             self.pos[self.head + i] = p
-            self.seq[self.head + i].add(seq_id)
+            self.seq[self.head + i].add(seq_ids[i])
         return self.head
 
     def cell_max(self):                                 # llama_kv_cache_cell_max, llama.cpp:1739-1747
@@ -228,6 +230,14 @@ class KVCells:
         if new_head != self.size:
             self.head = new_head
 
+    def seq_cp(self, src, dst, p0, p1):                 # llama_kv_cache_seq_cp, llama.cpp:1787-1803: the cells gain a second owner
+        p0 = max(p0, 0)
+        p1 = np.iinfo(np.int32).max if p1 < 0 else p1
+        self.head = 0
+        for i in range(self.size):
+            if src in self.seq[i] and p0 <= self.pos[i] < p1:
+                self.seq[i].add(dst)
+
     def seq_shift(self, seq_id, p0, p1, d):             # llama_kv_cache_seq_shift, llama.cpp:1819-1848
         new_head = self.size
         p0 = max(p0, 0)
@@ -244,10 +254,11 @@ class KVCells:
         self.head = new_head if new_head != self.size else 0
 
     def mask(self, positions, n_kv, seq_id=0):          # KQ_mask, llama.cpp:6506-6531
+        seq_ids = list(seq_id) if np.ndim(seq_id) else [seq_id] * len(positions)
         m = np.zeros((len(positions), n_kv), np.float32)
         for j, p in enumerate(positions):
             for i in range(n_kv):
-                if seq_id not in self.seq[i] or self.pos[i] > p:
+                if seq_ids[j] not in self.seq[i] or self.pos[i] > p:
                     m[j, i] = -np.inf
         return m
 
@@ -305,15 +316,15 @@ class OracleModel:
         assert tok >= 0
         return tok, logits
 
-    def eval_cells(self, tokens, pos, slots, n_kv, mask):
+    def eval_cells(self, tokens, pos, slots, n_kv, mask, all_logits=False):
         """General form (pio_model_eval): tokens[T] at positions pos[T] stored in cache cells slots[T]; n_kv cells attended
-        under mask [T][n_kv] (0 / -inf).  Returns (greedy token of the last position, its logits)."""
+        under mask [T][n_kv] (0 / -inf).  Returns (greedy token of the last position, its logits), or of every position."""
         tokens, pos, slots = (np.ascontiguousarray(a, np.int32) for a in (tokens, pos, slots))
         mask = np.ascontiguousarray(mask, np.float32)
-        logits = np.zeros(self.hp.n_vocab, np.float32)
-        rc = self.O.pio_model_eval(self.h, _ptr(tokens), _ptr(pos), _ptr(slots), tokens.size, int(n_kv), _ptr(mask), 0, _ptr(logits), 1)
+        logits = np.zeros((tokens.size, self.hp.n_vocab) if all_logits else self.hp.n_vocab, np.float32)
+        rc = self.O.pio_model_eval(self.h, _ptr(tokens), _ptr(pos), _ptr(slots), tokens.size, int(n_kv), _ptr(mask), int(all_logits), _ptr(logits), 1)
         assert rc == 0
-        return int(np.argmax(logits)), logits
+        return (logits.argmax(1) if all_logits else int(np.argmax(logits))), logits
 
     def k_shift(self, delta):
         delta = np.ascontiguousarray(delta, np.int32)

@@ -279,6 +279,20 @@ def test_batch_kv_sequence_edits():
     _, want2 = ref.decode([int(toks[n0, 2])], 6)
     for got, want in zip(lg, (want0, want1, want2)):
         assert rel_err(got, want) < 2e-3
+    # and the reference itself: its llama.cpp went through the same history with three sequence ids in one KV cache
+    # (tests/golden/ref_llama_seq_edits.npz, written by tests/golden/make_llama_fixture.py)
+    import importlib.util
+    import os
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    spec = importlib.util.spec_from_file_location("make_llama_fixture", os.path.join(root, "tests", "golden", "make_llama_fixture.py"))
+    fx = importlib.util.module_from_spec(spec)
+    spec.loader.exec_module(fx)
+    g = dict(np.load(os.path.join(root, "tests", "golden", "ref_llama_seq_edits.npz")))
+    if np.array_equal(fx.model_sha(model), g["model_sha"]):
+        assert np.array_equal(toks, g["tokens"])
+        for q in range(n_seq):
+            assert rel_err(lg[q], g["logits_last"][q]) < 2e-3, q
+            assert int(np.argmax(lg[q])) == int(np.argmax(g["logits_last"][q]))
     gm.close(); ref.close()
 
 

@@ -266,3 +266,24 @@ def test_q4_reference_departs_from_itself_beyond_the_logit_tolerance():
         a.close(), b.close()
     assert worst[ol.Q4_0] > 1e-2, worst
     assert worst[ol.F16] < 5e-3, worst
+
+
+def test_sparse_mul_mat_dispatch_rule_of_the_executor():
+    """ggml.c:14904-14927: MUL_MAT_SPARSE goes to the threshold kernel only when the predictor output is wider than 1000; narrower
+    nodes take a different kernel (one flag per 128 rows, fixed cut at -7) that no model shape reaches.  The oracle restates the
+    first and refuses the second rather than answer with the wrong rule; AXPY without its aux tensor is refused likewise (the
+    reference's F16 kernel skips every row then, ggml.c:14424)."""
+    O = ol.oracle()
+    rng = np.random.default_rng(0)
+    for rows, want in ((1000, 4), (1001, 0), (1024, 0)):
+        w = (rng.standard_normal((rows, 64)) * 0.1).astype(np.float16)
+        x = rng.standard_normal(64).astype(np.float32)
+        idx = rng.standard_normal(rows).astype(np.float32)
+        out = np.zeros(rows, np.float32)
+        rc = O.pio_mul_mat_sparse(ol.F16, ol._ptr(w), rows, 64, ol._ptr(x), 1, ol._ptr(idx), ol._ptr(np.zeros(rows, np.int32)), 0.0, ol._ptr(out), 1)
+        assert rc == want, (rows, rc)
+        if rc == 0:
+            assert np.array_equal(out != 0, idx >= 0)
+    h = rng.standard_normal(1024).astype(np.float32)
+    wt = (rng.standard_normal((1024, 64)) * 0.1).astype(np.float16)
+    assert O.pio_axpy(ol.F16, ol._ptr(wt), 1024, 64, ol._ptr(h), 1, ol._ptr(h), None, 0.0, ol._ptr(np.zeros(64, np.float32)), 1) == 3

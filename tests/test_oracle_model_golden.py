@@ -8,6 +8,7 @@ import numpy as np
 import pytest
 
 import oracle_lib as ol
+from powerinfer_amd import synth
 
 ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
 spec = importlib.util.spec_from_file_location("make_llama_fixture", os.path.join(ROOT, "tests", "golden", "make_llama_fixture.py"))
@@ -66,4 +67,43 @@ def test_context_shift_matches_reference_llama_cpp(name):
         assert best == g["greedy"][s], (s, best, g["greedy"][s])
         n_past += 1
     assert worst < 1e-5, worst
+    om.close()
+
+
+def test_sequence_edits_match_reference_llama_cpp():
+    """Three sequences sharing one KV cache (llama_batch entries with sequence ids), then llama_kv_cache_seq_rm, _seq_shift and
+    _seq_cp: one sequence takes a context shift, one is emptied and handed the first six cells of its neighbour.  The reference
+    wrote the logits of the last lockstep step (tests/golden/ref_llama_seq_edits.npz); the oracle repeats the history with the
+    reference's cell bookkeeping (ring slots, owners per cell, pending K-shift, per-token mask)."""
+    g = dict(np.load(os.path.join(ROOT, "tests", "golden", "ref_llama_seq_edits.npz")))
+    hp, toks, last_pos, _ = fx.seq_edit_case()
+    model = synth.make_model(hp)
+    if not np.array_equal(fx.model_sha(model), g["model_sha"]):
+        pytest.skip("numpy generates a different stream here than where the fixture was written")
+    assert np.array_equal(toks, g["tokens"])
+    om = ol.OracleModel(model)
+    cells = ol.KVCells(hp.n_ctx)
+    n_seq, n0 = toks.shape[1], toks.shape[0] - 1
+    seqs = list(range(n_seq))
+
+    def step(tokens, positions):
+        if cells.has_shift:
+            om.k_shift(cells.delta)
+            cells.has_shift = False
+            cells.delta[:] = 0
+        slot = cells.find_slot(positions, seqs)
+        n_kv = min(hp.n_ctx, max(32, cells.cell_max()))
+        return om.eval_cells(tokens, positions, [slot + i for i in range(n_seq)], n_kv, cells.mask(positions, n_kv, seqs), all_logits=True)[1]
+
+    for s in range(n0):
+        lg = step(toks[s], [s] * n_seq)
+        if s == 0:
+            assert np.abs(lg - g["logits_step0"]).max() <= 1e-5 * np.abs(g["logits_step0"]).max()
+    cells.seq_rm(0, 2, 5)
+    cells.seq_shift(0, 5, 8, -3)
+    cells.seq_rm(2, 0, -1)
+    cells.seq_cp(1, 2, 0, 6)
+    lg = step(toks[n0], list(g["last_pos"]))
+    assert np.abs(lg - g["logits_last"]).max() <= 1e-5 * np.abs(g["logits_last"]).max()
+    assert np.array_equal(lg.argmax(1), g["logits_last"].argmax(1))
     om.close()

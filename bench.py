@@ -237,6 +237,7 @@ def main():
     ap.add_argument("--prompt", type=int, default=64)
     ap.add_argument("--layers", type=int, default=32, help="only for quick trials; the reported workload uses 32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--prompt-bench", type=int, default=1024, help="length of the prompt timed for the prompt_phase entry (0 = skip)")
     ap.add_argument("--no-ref-host", action="store_true", help="skip the leg that runs the reference's llama.cpp on this backend (about 40 s)")
     ap.add_argument("--cpu-tokens", type=int, default=320, help="decode tokens timed on the host for the cpu_baseline leg (about 10 s of CPU work)")
     ap.add_argument("--config", type=int, default=1, choices=[1, 2, 3, 4],
@@ -431,6 +432,28 @@ def main():
         }
     m.close()
     del keep
+    if args.prompt_bench > 0 and not hybrid and hp.wtype == pl.F16:
+        # prompt phase on its own: a fresh instance of the same model with room for the prompt, one untimed pass (allocations, the
+        # transposed down projections), then the timed pass from an empty cache; chunks of up to 128 tokens per weight pass
+        try:
+            hp2 = synth.hparams({1: "llama-7b", 4: "falcon-40b"}[args.config], n_layer=hp.n_layer, n_ctx=args.prompt_bench + 8, seed=1)
+            keep2 = []
+            m2 = build_synthetic_on_device(hp2, keep2)
+            ptoks = rng.integers(0, hp2.n_vocab, args.prompt_bench).astype(np.int32)
+            m2.decode(ptoks[:200], 0, want_logits=False)
+            m2.kv_clear()
+            pl.sync()
+            t0 = time.perf_counter()
+            m2.decode(ptoks, 0, want_logits=False)
+            pl.sync()
+            dt = time.perf_counter() - t0
+            out["prompt_phase"] = {"tokens": args.prompt_bench, "ms": round(dt * 1e3, 2), "tok_per_s": round(args.prompt_bench / dt, 1),
+                                   "what": "pi_model_decode of the whole prompt: chunks of up to 128 tokens (dense MFMA mat-muls, each weight row read "
+                                           "once per chunk, predictor mask applied to h), last token through the single-token path"}
+            m2.close()
+            del keep2
+        except Exception as e:
+            out["prompt_phase"] = {"error": repr(e)[:200]}
     if not args.no_ref_host and args.config == 1:
         try:
             rh = reference_host_on_this_backend()

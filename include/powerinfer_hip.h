@@ -265,6 +265,16 @@ PI_API int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float thre
                                  int32_t * union_rows, int32_t * n_union,
                                  pi_workspace * ws, pi_stream_t stream);
 
+/* Prompt chunks of up to 128 tokens (the prompt phase of llama_decode, where the reference goes through cuBLAS and its batch kernels,
+ * ggml-cuda.cu:7662-7756, 6994-7034): pi_k_gemm_wide_f16 is pi_k_gemm_f16 for T <= 128 (cols % 256 == 0; a weight row is read once per
+ * chunk); pi_k_ffn_h_f16 forms h_f16[t][n] = fp16(relu(gate) * up) where !(logits[t][n] < threshold) and 0 elsewhere from dense gate/up
+ * products (gate may be NULL: relu(up)); pi_k_transpose_f16 writes out[cols][rows] of an fp16 matrix in[rows][cols] (the down projection
+ * of a chunk is a mat-mul over the neurons and wants them contiguous). */
+PI_API int pi_k_gemm_wide_f16(const void * W_f16, int rows, int cols, const void * xn_f16, int T, int epilogue,
+                              const float * add1, const float * add2, float * y, void * y_f16, pi_stream_t stream);
+PI_API int pi_k_ffn_h_f16(const float * up, const float * gate, const float * logits, float threshold, int T, int ff, void * h_f16, pi_stream_t stream);
+PI_API int pi_k_transpose_f16(const void * in_f16, int rows, int cols, void * out_f16, pi_stream_t stream);
+
 /* The two sparse operators of a step AS OPERATORS, for a host that runs the predictor itself and hands over its output idx [T][ff]
  * (the reference's mul_mat_batch_sparse and axpy at batch size > 1, ggml-cuda.cu:6994-7034, 8787-8814): T <= 16, F16 rows, cols % 256 == 0.
  *   pi_k_batch_sparse_mul_mat: y[t][n] = W[n] . xn_f16[t] where !(idx[t][n] < threshold), 0 elsewhere (y is [T][ff], fully written);

@@ -17,6 +17,8 @@ struct BatchState {
     float *pred_logits = nullptr, *logits = nullptr;
     __half *xa16 = nullptr, *xf16 = nullptr, *xp16 = nullptr, *att16 = nullptr, *hid16 = nullptr;
     int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_step = nullptr, *d_out_tokens = nullptr, *union_rows = nullptr, *n_union = nullptr;
+    float *up_out = nullptr, *gate_out = nullptr;      // wide prompt chunks: dense gate/up products [T][n_ff]
+    __half *h16 = nullptr;                             //                     and the FFN's hidden vector
     hipGraphExec_t graph_exec = nullptr;
     hipGraph_t graph = nullptr;
     std::vector<std::vector<int32_t>> kv_pos;      // per sequence: cell positions while an edit left them non-contiguous
@@ -146,7 +148,92 @@ BatchState * batch_alloc(pi_model * m, int T, bool with_caches) {
 
 }  // namespace
 
+namespace {
+// one layer of a wide prompt chunk (16 < T <= 128): every mat-mul reads its matrix once for the chunk; with that many tokens the union
+// of the active sets is nearly every neuron, so gate/up run dense and the predictor's mask turns into exact zeros of h (what the
+// sparse operators compute, term by term: an inactive neuron contributes nothing to the down projection)
+int wide_layer(pi_model * m, BatchState * b, int il) {
+    const pi_hparams & hp = m->hp;
+    const int T = b->n_seq, d = hp.n_embd, ff = hp.n_ff, hd = m->hd, gqa = m->gqa;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    hipStream_t st = m->stream;
+    Tensor & wqkv = m->L(il, PI_T_WQKV); Tensor & wo = m->L(il, PI_T_WO);
+    Tensor & fc1 = m->L(il, PI_T_FC1); Tensor & fc2 = m->L(il, PI_T_FC2);
+    Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE);
+    const int r = (int)fc1.ne1;
+    const size_t kv_off = (size_t)il * hp.n_head_kv * hp.n_ctx * hd;
+    float * x = b->x;
+    pi_norm an;
+    if (!falcon) an = mk_norm(1, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), nullptr);
+    else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
+    else an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
+    PI_TRY(pi_k_norm_round_f16(x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));
+    PI_TRY(pi_k_gemm_wide_f16(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr, st));
+    PI_TRY(pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, b->d_pos, hp.n_ctx, b->q_rot,
+                           m->k_cache + kv_off, m->v_cache + kv_off, b->att, d, b->att16, st));
+    pi_norm fn;
+    if (!falcon) {
+        PI_TRY(pi_k_gemm_wide_f16(wo.dev, d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, nullptr, st));
+        fn = mk_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
+        PI_TRY(pi_k_norm_round_f16(b->ffn_inp, T, d, &fn, b->xf16, b->xp16, st));
+    } else {
+        PI_TRY(pi_k_gemm_wide_f16(wo.dev, d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, nullptr, st));
+        fn = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
+        if (m->L(il, PI_T_ATTN_NORM_2).dev) PI_TRY(pi_k_norm_round_f16(x, T, d, &fn, b->xf16, nullptr, st));
+    }
+    const __half * ffn_x = (falcon && !m->L(il, PI_T_ATTN_NORM_2).dev) ? b->xa16 : b->xf16;
+    PI_TRY(pi_k_gemm_wide_f16(fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16, st));
+    PI_TRY(pi_k_gemm_wide_f16(fc2.dev, ff, r, b->hid16, T, PI_EPI_NONE, nullptr, nullptr, b->pred_logits, nullptr, st));
+    PI_TRY(pi_k_gemm_wide_f16(up.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->up_out, nullptr, st));
+    if (!falcon) PI_TRY(pi_k_gemm_wide_f16(gate.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->gate_out, nullptr, st));
+    PI_TRY(pi_k_ffn_h_f16(b->up_out, falcon ? nullptr : b->gate_out, b->pred_logits, hp.sparse_threshold, T, ff, b->h16, st));
+    if (!falcon) PI_TRY(pi_k_gemm_wide_f16(m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD, b->ffn_inp, nullptr, b->x2, nullptr, st));
+    else         PI_TRY(pi_k_gemm_wide_f16(m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD2, b->attn_out, x, b->x2, nullptr, st));
+    std::swap(b->x, b->x2);
+    return PI_OK;
+}
+}  // namespace
+
 namespace pi {
+bool prefill_wide_supported(pi_model * m) {
+    const char * off = getenv("PI_NO_PREFILL_WIDE");
+    return !(off && off[0] == '1') && prefill_supported(m) && m->hp.n_embd % 256 == 0 && m->hp.n_ff % 256 == 0 && (int)m->L(0, PI_T_FC1).ne1 % 256 == 0;
+}
+
+int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) {
+    constexpr int kMaxT = 128;
+    if (T <= 16 || T > kMaxT) return pi::fail(PI_E_ARG, "prefill_wide_chunk: 16 < T <= 128");
+    const pi_hparams & hp = m->hp;
+    if (!m->prefill_wide) {
+        BatchState * b = batch_alloc(m, kMaxT, false);
+        if (!b) return PI_E_HIP;
+        b->prefill = true;
+        b->up_out = m->alloc<float>((size_t)kMaxT * hp.n_ff);
+        b->gate_out = hp.arch == PI_ARCH_FALCON ? nullptr : m->alloc<float>((size_t)kMaxT * hp.n_ff);
+        b->h16 = m->alloc<__half>((size_t)kMaxT * hp.n_ff);
+        if (!b->up_out || (hp.arch != PI_ARCH_FALCON && !b->gate_out) || !b->h16) { delete b; return PI_E_HIP; }
+        // the down projection of a chunk is a mat-mul whose reduction runs over the neurons: one more copy of it with the neurons
+        // contiguous (n_embd x n_ff fp16 per layer; the decode loop keeps using the row-per-neuron layout)
+        m->down_rows.assign(hp.n_layer, nullptr);
+        for (int il = 0; il < hp.n_layer; ++il) {
+            m->down_rows[il] = m->alloc<__half>((size_t)hp.n_embd * hp.n_ff);
+            if (!m->down_rows[il]) { delete b; m->down_rows.clear(); return PI_E_HIP; }
+            PI_TRY(pi_k_transpose_f16(m->L(il, PI_T_FFN_DOWN_T).dev, hp.n_ff, hp.n_embd, m->down_rows[il], m->stream));
+        }
+        m->prefill_wide = b;
+    }
+    BatchState * b = m->prefill_wide;
+    b->n_seq = T;
+    int32_t pos[kMaxT];
+    for (int t = 0; t < T; ++t) pos[t] = n_past + t;
+    PI_HIP_TRY(hipMemcpyAsync(b->d_tokens, tokens, sizeof(int32_t) * T, hipMemcpyHostToDevice, m->stream));
+    PI_HIP_TRY(hipMemcpyAsync(b->d_pos, pos, sizeof(int32_t) * T, hipMemcpyHostToDevice, m->stream));
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    PI_TRY(pi_k_embed_batch(m->glob[PI_T_TOK_EMBD].dev, hp.n_embd, b->d_tokens, T, b->x, m->stream));
+    for (int il = 0; il < hp.n_layer; ++il) PI_TRY(wide_layer(m, b, il));
+    return PI_OK;
+}
+
 bool prefill_supported(pi_model * m) {
     const char * off = getenv("PI_NO_PREFILL");
     return !(off && off[0] == '1') && !m->capture && batch_unsupported(m) == nullptr;
@@ -175,6 +262,7 @@ int prefill_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) {
 
 void batch_destroy(pi_model * m) {
     if (m->prefill) { delete m->prefill; m->prefill = nullptr; }
+    if (m->prefill_wide) { delete m->prefill_wide; m->prefill_wide = nullptr; }
     if (!m->batch) return;
     if (m->batch->graph_exec) (void)hipGraphExecDestroy(m->batch->graph_exec);
     if (m->batch->graph) (void)hipGraphDestroy(m->batch->graph);

@@ -2695,6 +2695,125 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
     }
 }
 
+// Prompt chunks of up to 128 tokens: the same mat-mul with NT token tiles of 16 per row tile, so a weight row is read once per chunk
+// instead of once per 16 tokens.  A wave keeps its RT x 16 rows of a 256-column super-step in its private LDS tile (row-contiguous
+// global reads, as above; the load registers are free again once the tile is written, so the next super-step's loads are issued at
+// once and travel during the MFMAs) and streams the activations of all NT x 16 tokens past it, one 32-column step ahead.
+// K is split over the four waves of a workgroup (super-steps w, w + 4, ...); their partial tiles meet in LDS in wave order.
+constexpr int kWideMaxT = 128;
+template <int RT, int NT>
+__global__ __launch_bounds__(kBlock) void gemm_wide_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
+                                                               int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y,
+                                                               __half * __restrict__ y16) {
+    __shared__ __align__(16) unsigned char tile[kWavesPerBlock][RT * 16 * kGlStride];
+    __shared__ float cs[kWavesPerBlock][16][17];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;
+    const int lr = lane >> 5, lc = lane & 31;
+    const int row0 = blockIdx.x * 16 * RT;
+    // blockIdx.y: group of NT x 16 tokens (matrices with few rows are spread over more workgroups by splitting the chunk's tokens)
+    const int t_base = blockIdx.y * NT * 16;
+    xn += (size_t)t_base * cols; y += (size_t)t_base * rows; T -= t_base;
+    if (y16) y16 += (size_t)t_base * rows;
+    if (add1) add1 += (size_t)t_base * rows;
+    if (add2) add2 += (size_t)t_base * rows;
+    const __half * bp[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) { const int tok = nt * 16 + i; bp[nt] = xn + (size_t)(tok < T ? tok : T - 1) * cols + g * 8; }
+    unsigned char * mytile = tile[wave];
+    pi_f4 acc[RT][NT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    const int n_ss = (cols / 256 - wave + kWavesPerBlock - 1) / kWavesPerBlock;
+    pi_u32x4 ld[RT][8];
+    auto issue = [&](int ss) {
+        if (ss < n_ss) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    int r = row0 + rt * 16 + 2 * j + lr;
+                    r = r < rows ? r : rows - 1;
+                    ld[rt][j] = pi_ld_stream(W + (size_t)r * cols + (wave + ss * kWavesPerBlock) * 256 + lc * 8);
+                }
+        }
+    };
+    issue(0);
+    for (int ss = 0; ss < n_ss; ++ss) {
+        const int k0 = (wave + ss * kWavesPerBlock) * 256;
+        pi_u32x4 b[2][NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) b[0][nt] = pi_ld16(bp[nt] + k0);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (rt * 16 + 2 * j + lr) * kGlStride + lc * 16) = ld[rt][j];
+        issue(ss + 1);
+#pragma unroll
+        for (int st = 0; st < 8; ++st) {
+            if (st + 1 < 8) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) b[(st + 1) & 1][nt] = pi_ld16(bp[nt] + k0 + (st + 1) * 32);
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                const pi_u32x4 a = *reinterpret_cast<const pi_u32x4 *>(mytile + (rt * 16 + i) * kGlStride + (4 * st + g) * 16);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a), __builtin_bit_cast(pi_h8, b[st & 1][nt]), acc[rt][nt], 0, 0, 0);
+            }
+        }
+    }
+    const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < 4; ++r) cs[wave][4 * g + r][i] = acc[rt][nt][r];
+            __syncthreads();
+            const int row = row0 + rt * 16 + rr, tok = nt * 16 + t;
+            if (row < rows && tok < T) {
+                float sum = cs[0][rr][t];
+#pragma unroll
+                for (int w = 1; w < kWavesPerBlock; ++w) sum += cs[w][rr][t];
+                const size_t o = (size_t)tok * rows + row;
+                if (epi == PI_EPI_RELU) sum = fmaxf(sum, 0.0f);
+                else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
+                else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[o]), add2[o]);
+                y[o] = sum;
+                if (y16) y16[o] = __float2half_rn(sum);
+            }
+        }
+}
+// h16[t][n] = fp16( !(logit[t][n] < thr) ? relu(gate[t][n]) * up[t][n] : 0 )   (relu(up) without a gate): the FFN's hidden vector of a
+// prompt chunk from the dense gate/up products; inactive neurons become exact zeros, which add nothing in the down projection
+__global__ void ffn_h_f16_kernel(const float * __restrict__ up, const float * __restrict__ gate, const float * __restrict__ logits, float thr,
+                                 size_t n, __half * __restrict__ h16) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        float h = 0.0f;
+        if (!(logits[i] < thr)) h = gate ? __fmul_rn(fmaxf(gate[i], 0.0f), up[i]) : fmaxf(up[i], 0.0f);
+        h16[i] = __float2half_rn(h);
+    }
+}
+// out[c][r] = in[r][c] for an fp16 matrix [rows][cols] (32 x 32 tiles through LDS)
+__global__ void transpose_f16_kernel(const __half * __restrict__ in, int rows, int cols, __half * __restrict__ out) {
+    __shared__ __half t[32][33];
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    for (int j = threadIdx.y; j < 32; j += blockDim.y) {
+        const int r = r0 + j, c = c0 + threadIdx.x;
+        if (r < rows && c < cols) t[j][threadIdx.x] = in[(size_t)r * cols + c];
+    }
+    __syncthreads();
+    for (int j = threadIdx.y; j < 32; j += blockDim.y) {
+        const int c = c0 + j, r = r0 + threadIdx.x;
+        if (r < rows && c < cols) out[(size_t)c * rows + r] = t[threadIdx.x][j];
+    }
+}
+
 // the operator boundary hands over the predictor's output instead of running the predictor: row_any[n] = some token has !(idx[t][n] < thr)
 __global__ void batch_flag_any_kernel(const float * __restrict__ idx, int T, int ff, float thr, unsigned char * __restrict__ row_any) {
     const int n = blockIdx.x * blockDim.x + threadIdx.x;
@@ -3578,6 +3697,34 @@ int pi_k_gemm_f16(const void * W, int rows, int cols, const void * xn_f16, int T
     return gemm_launch("pi_k_gemm_f16", W, rows, cols, xn_f16, T, epilogue, add1, add2, y, y_f16, 0.0f, nullptr, stream);
 }
 
+int pi_k_gemm_wide_f16(const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
+                       float * y, void * y_f16, pi_stream_t stream) {
+    if (!W || !xn_f16 || !y || rows <= 0) return pi::fail(PI_E_ARG, "pi_k_gemm_wide_f16: null pointer or empty shape");
+    if (T < 1 || T > kWideMaxT || cols <= 0 || cols % 256) return pi::fail(PI_E_ARG, "pi_k_gemm_wide_f16: 1 <= T <= 128 and cols % 256 == 0 required");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_gemm_wide_f16: bad epilogue arguments");
+    if (T <= kBtMaxT) return gemm_launch("pi_k_gemm_wide_f16", W, rows, cols, xn_f16, T, epilogue, add1, add2, y, y_f16, 0.0f, nullptr, stream);
+#define PI_GEMM_WIDE(RT, NT) hipLaunchKernelGGL((gemm_wide_f16_kernel<RT, NT>), dim3((rows + 16 * RT - 1) / (16 * RT), (T + 16 * NT - 1) / (16 * NT)), dim3(kBlock), 0, \
+        (hipStream_t)stream, (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16)
+    // tile shape by row count: wide matrices take 64 rows x the whole chunk per workgroup; narrower ones split the chunk's tokens over
+    // several workgroups so that the grid still covers the chip (their weights then pass through L2 once per token group)
+    if (rows >= 8192) { if (T <= 32) PI_GEMM_WIDE(2, 2); else if (T <= 64) PI_GEMM_WIDE(4, 4); else PI_GEMM_WIDE(4, 8); }
+    else if (rows > 2048) { if (T <= 32) PI_GEMM_WIDE(2, 2); else PI_GEMM_WIDE(2, 4); }
+    else PI_GEMM_WIDE(1, 2);
+#undef PI_GEMM_WIDE
+    return pi::check_launch("pi_k_gemm_wide_f16");
+}
+int pi_k_ffn_h_f16(const float * up, const float * gate, const float * logits, float threshold, int T, int ff, void * h_f16, pi_stream_t stream) {
+    if (!up || !logits || !h_f16 || T <= 0 || ff <= 0) return pi::fail(PI_E_ARG, "pi_k_ffn_h_f16: bad arguments");
+    hipLaunchKernelGGL(ffn_h_f16_kernel, dim3(1024), dim3(256), 0, (hipStream_t)stream, up, gate, logits, threshold, (size_t)T * ff, (__half *)h_f16);
+    return pi::check_launch("pi_k_ffn_h_f16");
+}
+int pi_k_transpose_f16(const void * in, int rows, int cols, void * out, pi_stream_t stream) {
+    if (!in || !out || rows <= 0 || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_transpose_f16: bad arguments");
+    hipLaunchKernelGGL(transpose_f16_kernel, dim3((cols + 31) / 32, (rows + 31) / 32), dim3(32, 8), 0, (hipStream_t)stream, (const __half *)in, rows, cols, (__half *)out);
+    return pi::check_launch("pi_k_transpose_f16");
+}
+
 int pi_k_batch_predictor_fc2(const void * fc2_f16, int ff, int r, const void * hidden_f16, int T, float threshold, float * logits,
                              pi_workspace * ws, pi_stream_t stream) {
     if (!ws || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_batch_predictor_fc2: ff exceeds the workspace");
@@ -3729,7 +3876,7 @@ int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_t
 int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
                     const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache, float * out, int out_stride, void * out_f16,
                     pi_stream_t stream) {
-    if (!qkv || !pos || !q_rot || !k_cache || !v_cache || !out || T <= 0 || T > kBtMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad arguments");
+    if (!qkv || !pos || !q_rot || !k_cache || !v_cache || !out || T <= 0 || T > kWideMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad arguments");
     if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd <= 0 || hd % 8 || hd / 2 > 1024 || kBlock % (hd / 8) || PI_WAVE % (hd / 8) || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad head geometry or mode");
     const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd);
@@ -3767,7 +3914,7 @@ int pi_k_step_advance(int32_t * step, pi_stream_t stream) {
 }
 
 int pi_k_embed_batch(const void * table_f16, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream) {
-    if (!table_f16 || !tokens || !x || cols <= 0 || T <= 0 || T > kBtMaxT) return pi::fail(PI_E_ARG, "pi_k_embed_batch: bad arguments");
+    if (!table_f16 || !tokens || !x || cols <= 0 || T <= 0 || T > kWideMaxT) return pi::fail(PI_E_ARG, "pi_k_embed_batch: bad arguments");
     hipLaunchKernelGGL(embed_f16_batch_kernel, dim3((cols + 255) / 256, T), dim3(256), 0, (hipStream_t)stream, (const __half *)table_f16, cols, tokens, x);
     return pi::check_launch("pi_k_embed_batch");
 }

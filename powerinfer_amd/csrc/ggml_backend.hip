@@ -82,11 +82,35 @@ bool contiguous(const ggml_tensor * t) {
     return t->nb[0] == tsize(t->type) && t->nb[1] == row_size(t) && t->nb[2] == t->nb[1] * (size_t)t->ne[1] && t->nb[3] == t->nb[2] * (size_t)t->ne[2];
 }
 
-// temporaries of one operator call (CPU-resident operands staged on the device, device results bound for the host)
+// Temporaries of one operator call (CPU-resident operands staged on the device, device results bound for the host, index lists).
+// They come from one arena that lives as long as the scratch buffer: nodes are computed one after the other on one stream, so the
+// next node may reuse the bytes as soon as its own work is queued behind the previous node's.  A call that needs more than the
+// arena holds takes plain allocations for the excess (freed when it returns) and the arena grows before the next call.
+struct Arena { char * base = nullptr; size_t cap = 0, want = 4u << 20; };
+Arena g_arena;
 struct Temps {
-    std::vector<void *> ptrs;
-    void * get(size_t n) { void * p = pi_malloc(n); if (!p) die("temporary allocation"); ptrs.push_back(p); return p; }
-    ~Temps() { for (void * p : ptrs) pi_free(p); }
+    std::vector<void *> extra;
+    size_t off = 0, need = 0;
+    Temps() {
+        if (g_arena.want > g_arena.cap) {
+            if (g_arena.base) { pi_sync(); pi_free(g_arena.base); }
+            g_arena.cap = g_arena.want;
+            g_arena.base = (char *)pi_malloc(g_arena.cap);
+            if (!g_arena.base) die("temporary arena");
+        }
+    }
+    void * get(size_t n) {
+        n = (n + 255) & ~(size_t)255;
+        need += n;
+        if (off + n <= g_arena.cap) { void * p = g_arena.base + off; off += n; return p; }
+        void * p = pi_malloc(n); if (!p) die("temporary allocation");
+        extra.push_back(p);
+        return p;
+    }
+    ~Temps() {
+        for (void * p : extra) pi_free(p);
+        if (need > g_arena.want) g_arena.want = need + (need >> 2);
+    }
 };
 
 void * dev_ptr(const ggml_tensor * t) {
@@ -546,6 +570,7 @@ void ggml_cuda_set_scratch_size(size_t scratch_size) {
 void ggml_cuda_free_scratch(void) {
     std::lock_guard<std::mutex> g(g_mu);
     if (g_scratch) { pi_free(g_scratch); g_scratch = nullptr; }
+    if (g_arena.base) { pi_sync(); pi_free(g_arena.base); g_arena.base = nullptr; g_arena.cap = 0; }
     g_scratch_offset = 0;
 }
 void ggml_cuda_copy_to_device(struct ggml_tensor * tensor) {

@@ -34,8 +34,25 @@ def run_reference(tmp_path, name, share, n_threads):
         pytest.skip("numpy generates a different stream here than where the fixture was written")
     path, out = str(tmp_path / "m.powerinfer.gguf"), str(tmp_path / "out.bin")
     gguf.write_model(path, model, gguf.synthetic_tokenizer_kv(hp.n_vocab))
-    rates = [L["p"] for L in model["layers"]]
-    splits = split.split_from_counts(rates, [int(round(share * hp.n_ff))] * hp.n_layer)
+    if share >= 1.0:
+        splits = [(np.ones(hp.n_ff, np.int32), np.arange(hp.n_ff, dtype=np.int32)) for _ in range(hp.n_layer)]
+    else:
+        # The reference's CPU half of the down projection lets each thread add its partial result into the output without a lock
+        # (ggml.c:14436-14452), and hybrid execution insists on two threads (ggml.c:16719): run CPU-only on these models with two
+        # threads it departs from its own single-thread logits by 7e-2 .. 4.5e-1 in a quarter of the runs.  To compare against the
+        # single-thread vectors the split keeps every host-resident neuron in the first half of the index range: the second
+        # thread's rows (ggml.c:14390, rows / n_threads each) are then all GPU-resident, it skips them and adds its zeros long
+        # before the first thread adds its sum.  The share on the GPU is still `share`: the whole second half plus the hottest
+        # neurons of the first.
+        splits = []
+        for L in model["layers"]:
+            half = hp.n_ff // 2
+            k = int(round(share * hp.n_ff)) - (hp.n_ff - half)
+            assert 0 < k < half
+            gi = np.zeros(hp.n_ff, np.int32)
+            gi[half:] = 1
+            gi[np.argsort(-np.asarray(L["p"][:half]), kind="stable")[:k]] = 1
+            splits.append((gi, np.flatnonzero(gi).astype(np.int32)))
     split.write_gpuidx(path + ".generated.gpuidx", splits, split.required_bytes(hp, splits))
     toks = [str(int(t)) for t in g["consumed"]]                 # every step consumes the reference's token (teacher forcing)
     env = dict(os.environ, REF_VRAM_GB="2")
@@ -60,19 +77,7 @@ def test_reference_llama_cpp_runs_on_this_backend(name, share, n_threads, tmp_pa
     assert "offloading v cache to GPU" in log and "offloading k cache to GPU" in log, log[-3000:]
     assert "offloaded layers from VRAM budget" in log
     errs = np.abs(logits[:, g["sample_idx"]] - g["logits_sample"]).max(1) / g["logits_absmax"]
-    if share >= 1.0:
-        # every neuron on the device, one host thread: the north star's logits tolerance on every step
-        assert errs.max() < 1e-2, errs
-        assert np.median(errs) < 2e-3, errs
-        assert int((greedy == g["greedy"]).sum()) >= len(errs) - 1, (greedy, g["greedy"])
-        return
-    # Split runs.  The reference's CPU half of the down projection lets each thread add its partial result into the output without
-    # a lock (ggml.c:14436-14452; hybrid execution insists on two threads, ggml.c:16719), so now and then a step loses one thread's
-    # share of eight outputs -- in the reference's own arithmetic, before this backend sees the tensor -- and the damaged state
-    # stays in the KV cache, fading over the following steps.  Up to the first such step the tolerance holds as above (observed:
-    # 1e-7 .. 1e-4); a hit shows as a jump of orders of magnitude.  Hits are rare, so: at most two steps beyond the tolerance,
-    # none beyond 0.1, and the typical step well inside it.
-    assert int((errs >= 1e-2).sum()) <= 2 and errs.max() < 0.1, errs
-    assert np.median(errs) < 5e-3, errs
-    first_hit = int(np.argmax(errs >= 1e-2)) if (errs >= 1e-2).any() else len(errs)
-    assert (greedy[:first_hit] == g["greedy"][:first_hit]).sum() >= first_hit - 1, (greedy, g["greedy"])
+    # the north star's logits tolerance on every step, full and split alike
+    assert errs.max() < 1e-2, errs
+    assert np.median(errs) < 2e-3, errs
+    assert int((greedy == g["greedy"]).sum()) >= len(errs) - 1, (greedy, g["greedy"])

@@ -65,12 +65,24 @@ def build_synthetic_on_device(hp, keep):
         host = buf.download(np.uint8).reshape(rows, -1) if q4 else buf.download(np.float16).reshape(rows, cols)
         m.set_tensor(layer, kind, host)
 
-    put(-1, "tok_embd", normal(hp.n_vocab, d), hp.n_vocab, d)
-    put(-1, "output", normal(hp.n_vocab, d), hp.n_vocab, d)
+    tok_embd, output = normal(hp.n_vocab, d), normal(hp.n_vocab, d)
+    rng = np.random.default_rng(hp.seed)
+    if hp.get("head_pair"):
+        # the greedy decision with a margin of powerinfer_amd.synth.make_model: four dominant output rows +-w0, +-w1, and the
+        # embeddings of those four tokens scaled down
+        assert not q4
+        pl.sync()
+        rows = np.empty((4, d), np.float16)
+        for k in range(2):
+            w = rng.standard_normal(d, dtype=np.float32) * np.float32(0.02 * hp.head_pair)
+            rows[2 * k], rows[2 * k + 1] = w.astype(np.float16), (-w).astype(np.float16)
+        output.upload(rows)
+        tok_embd.upload((tok_embd.download(np.float16, 4 * d).astype(np.float32) * np.float32(0.05)).astype(np.float16))
+    put(-1, "tok_embd", tok_embd, hp.n_vocab, d)
+    put(-1, "output", output, hp.n_vocab, d)
     m.set_tensor(-1, "output_norm", np.ones(d, np.float32))
     if falcon:
         m.set_tensor(-1, "output_norm_b", np.zeros(d, np.float32))
-    rng = np.random.default_rng(hp.seed)
     for il in range(hp.n_layer):
         m.set_tensor(il, "attn_norm", np.ones(d, np.float32))
         if falcon:
@@ -88,9 +100,14 @@ def build_synthetic_on_device(hp, keep):
         put_ffn(il, "ffn_down_t", normal(ff, d), ff, d)
         put(il, "fc1", normal(r, d, f16=True), r, d, f16=True)
         p, _ = synth.zipf_rates(ff, hp.mean_rate, rng)
-        b = (0.02 * np.sqrt(np.pi) * ndtri(p) / np.sqrt(r)).astype(np.float32)
-        bias = pl.DevBuf(host=b)
-        put(il, "fc2", normal(ff, r, bias, f16=True), ff, r, f16=True)
+        if hp.get("pred_margin"):                  # a predictor whose decisions keep a margin (synth.predictor_fc2_margin), made on the host
+            fc2 = pl.DevBuf(host=synth.predictor_fc2_margin(ff, r, p, rng))
+            keep.append(fc2)
+        else:
+            b = (0.02 * np.sqrt(np.pi) * ndtri(p) / np.sqrt(r)).astype(np.float32)
+            bias = pl.DevBuf(host=b)
+            fc2 = normal(ff, r, bias, f16=True)
+        put(il, "fc2", fc2, ff, r, f16=True)
         if hybrid:
             gi, gb = synth.gpu_split(p, hp.hot_frac)
             m.set_tensor(il, "gpu_idx", gi)

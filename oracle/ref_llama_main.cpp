@@ -17,6 +17,11 @@
 // REF_VRAM_GB=<GiB> sets llama_model_params.vram_budget_gb (the accelerator build offloads by budget; the neuron split is
 // read from <model.gguf>.generated.gpuidx).  The time of the greedy steps is printed as "decode_ms_per_token <ms>".
 //
+// REF_ONE_CORE=1 binds the process, and with it every thread it starts, to the core it is on.  The reference's CPU share of the
+// down projection lets each worker add its partial sum into the result without a lock (ggml.c:14436-14452); with its workers
+// on one core they run one at a time and change over where they yield between graph nodes (ggml.c:16946), so two of them are
+// never inside that addition together and a multi-threaded run repeats the single-threaded numbers.
+//
 // With REF_SHIFT_AT=s REF_N_KEEP=k REF_N_DISCARD=d in the environment the driver does, before step s, what the reference's
 // examples do when the context is full (examples/main/main.cpp): llama_kv_cache_seq_rm(ctx, 0, k, k + d), then
 // llama_kv_cache_seq_shift(ctx, 0, k + d, n_past, -d), and continues at position n_past - d.
@@ -30,6 +35,7 @@
 #include <vector>
 
 #include <execinfo.h>
+#include <sched.h>
 #include <unistd.h>
 
 // a crash of the host side names its call chain on stderr (the binary is linked with -rdynamic)
@@ -58,6 +64,12 @@ int main(int argc, char ** argv) {
     sa.sa_flags = SA_SIGINFO;
     sigaction(SIGSEGV, &sa, NULL);
     sigaction(SIGABRT, &sa, NULL);
+    if (getenv("REF_ONE_CORE") && atoi(getenv("REF_ONE_CORE"))) {
+        cpu_set_t one;
+        CPU_ZERO(&one);
+        CPU_SET(sched_getcpu(), &one);
+        if (sched_setaffinity(0, sizeof one, &one) != 0) { perror("sched_setaffinity"); return 2; }
+    }
     llama_backend_init(false);
     llama_model_params mp = llama_model_default_params();
     mp.n_gpu_layers = 0;                                      // sparse models offload by VRAM budget, not by layer count

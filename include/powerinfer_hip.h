@@ -275,6 +275,15 @@ PI_API int pi_k_gemm_wide_f16(const void * W_f16, int rows, int cols, const void
 PI_API int pi_k_ffn_h_f16(const float * up, const float * gate, const float * logits, float threshold, int T, int ff, void * h_f16, pi_stream_t stream);
 PI_API int pi_k_transpose_f16(const void * in_f16, int rows, int cols, void * out_f16, pi_stream_t stream);
 
+/* The same mat-mul for prompt chunks of any length through hipBLASLt (fp16 operands, fp32 accumulation and result), where the reference
+ * calls cuBLAS (ggml_cuda_op_mul_mat_cublas, ggml-cuda.cu:7662-7756).  Arguments and epilogues as pi_k_gemm_f16; no limit on T or cols.
+ * A pi_gemm_lib holds the library handle, its workspace and one plan per distinct (rows, cols, T) - at most 64 of them. */
+typedef struct pi_gemm_lib pi_gemm_lib;
+PI_API pi_gemm_lib * pi_gemm_lib_create(size_t workspace_bytes);
+PI_API int           pi_gemm_lib_destroy(pi_gemm_lib * g);
+PI_API int pi_gemm_lib_f16(pi_gemm_lib * g, const void * W_f16, int rows, int cols, const void * xn_f16, int T, int epilogue,
+                           const float * add1, const float * add2, float * y, void * y_f16, pi_stream_t stream);
+
 /* The two sparse operators of a step AS OPERATORS, for a host that runs the predictor itself and hands over its output idx [T][ff]
  * (the reference's mul_mat_batch_sparse and axpy at batch size > 1, ggml-cuda.cu:6994-7034, 8787-8814): T <= 16, F16 rows, cols % 256 == 0.
  *   pi_k_batch_sparse_mul_mat: y[t][n] = W[n] . xn_f16[t] where !(idx[t][n] < threshold), 0 elsewhere (y is [T][ff], fully written);

@@ -24,6 +24,8 @@ FLAGS = [
     # host code of the cold path uses the x86 vector extensions every MI355X host CPU has
     "-Xarch_host", "-mavx2", "-Xarch_host", "-mfma", "-Xarch_host", "-mf16c",
 ]
+# dense mat-muls of long prompt chunks go to the library the reference's cuBLAS calls correspond to
+LIBS = ["-L/opt/rocm/lib", "-lhipblaslt", "-Wl,-rpath,/opt/rocm/lib"]
 
 
 def sources():
@@ -31,7 +33,7 @@ def sources():
 
 
 def build(verbose=True):
-    cmd = [HIPCC] + FLAGS + ["-o", LIB] + sources()
+    cmd = [HIPCC] + FLAGS + ["-o", LIB] + sources() + LIBS
     if verbose:
         print(" ".join(cmd), flush=True)
     p = subprocess.run(cmd, capture_output=True, text=True)

@@ -627,13 +627,14 @@ int pi_model_decode(pi_model * m, const int32_t * tokens, int n_tokens, int n_pa
         if (tokens[i] < 0 || tokens[i] >= m->hp.n_vocab) return pi::fail(PI_E_ARG, "pi_model_decode: token id out of range");
     int first = 0;
     if (n_tokens > 2 && pi::prefill_supported(m)) {
-        // the prompt goes through in chunks (weights read once per chunk): up to 128 tokens where the dense chunk kernels cover the
+        // the prompt goes through in chunks (weights read once per chunk): up to 512 tokens where the dense chunk path covers the
         // shape, up to 16 otherwise and for the remainder; the last token takes the single-token path below, which produces the logits
         const bool wide = pi::prefill_wide_supported(m);
+        const int wide_max = wide ? pi::prefill_wide_max(m) : 0;
         while (n_tokens - 1 - first >= 2) {
             const int left = n_tokens - 1 - first;
             if (wide && left > 16) {
-                const int T = left < 128 ? left : 128;
+                const int T = left < wide_max ? left : wide_max;
                 PI_TRY(pi::prefill_wide_chunk(m, tokens + first, T, n_past + first));
                 first += T;
             } else {

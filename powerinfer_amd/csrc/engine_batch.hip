@@ -6,6 +6,7 @@
 #include "runtime.hpp"
 
 #include <stdlib.h>
+#include <string.h>
 
 struct BatchState {
     int n_seq = 0, max_steps = 4096;
@@ -152,6 +153,13 @@ namespace {
 // one layer of a wide prompt chunk (16 < T <= 128): every mat-mul reads its matrix once for the chunk; with that many tokens the union
 // of the active sets is nearly every neuron, so gate/up run dense and the predictor's mask turns into exact zeros of h (what the
 // sparse operators compute, term by term: an inactive neuron contributes nothing to the down projection)
+// one dense mat-mul of a chunk: the library's plan for long chunks, this library's own kernel otherwise
+int chunk_gemm(pi_model * m, const void * W, int rows, int cols, const void * xn, int T, int epi, const float * add1, const float * add2,
+               float * y, void * y16) {
+    if (m->gemm_lib) return pi_gemm_lib_f16(m->gemm_lib, W, rows, cols, xn, T, epi, add1, add2, y, y16, m->stream);
+    return pi_k_gemm_wide_f16(W, rows, cols, xn, T, epi, add1, add2, y, y16, m->stream);
+}
+
 int wide_layer(pi_model * m, BatchState * b, int il) {
     const pi_hparams & hp = m->hp;
     const int T = b->n_seq, d = hp.n_embd, ff = hp.n_ff, hd = m->hd, gqa = m->gqa;
@@ -168,27 +176,27 @@ int wide_layer(pi_model * m, BatchState * b, int il) {
     else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
     else an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
     PI_TRY(pi_k_norm_round_f16(x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));
-    PI_TRY(pi_k_gemm_wide_f16(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr, st));
+    PI_TRY(chunk_gemm(m, wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr));
     PI_TRY(pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, b->d_pos, hp.n_ctx, b->q_rot,
                            m->k_cache + kv_off, m->v_cache + kv_off, b->att, d, b->att16, st));
     pi_norm fn;
     if (!falcon) {
-        PI_TRY(pi_k_gemm_wide_f16(wo.dev, d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, nullptr, st));
+        PI_TRY(chunk_gemm(m, wo.dev, d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, nullptr));
         fn = mk_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
         PI_TRY(pi_k_norm_round_f16(b->ffn_inp, T, d, &fn, b->xf16, b->xp16, st));
     } else {
-        PI_TRY(pi_k_gemm_wide_f16(wo.dev, d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, nullptr, st));
+        PI_TRY(chunk_gemm(m, wo.dev, d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, nullptr));
         fn = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
         if (m->L(il, PI_T_ATTN_NORM_2).dev) PI_TRY(pi_k_norm_round_f16(x, T, d, &fn, b->xf16, nullptr, st));
     }
     const __half * ffn_x = (falcon && !m->L(il, PI_T_ATTN_NORM_2).dev) ? b->xa16 : b->xf16;
-    PI_TRY(pi_k_gemm_wide_f16(fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16, st));
-    PI_TRY(pi_k_gemm_wide_f16(fc2.dev, ff, r, b->hid16, T, PI_EPI_NONE, nullptr, nullptr, b->pred_logits, nullptr, st));
-    PI_TRY(pi_k_gemm_wide_f16(up.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->up_out, nullptr, st));
-    if (!falcon) PI_TRY(pi_k_gemm_wide_f16(gate.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->gate_out, nullptr, st));
+    PI_TRY(chunk_gemm(m, fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16));
+    PI_TRY(chunk_gemm(m, fc2.dev, ff, r, b->hid16, T, PI_EPI_NONE, nullptr, nullptr, b->pred_logits, nullptr));
+    PI_TRY(chunk_gemm(m, up.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->up_out, nullptr));
+    if (!falcon) PI_TRY(chunk_gemm(m, gate.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->gate_out, nullptr));
     PI_TRY(pi_k_ffn_h_f16(b->up_out, falcon ? nullptr : b->gate_out, b->pred_logits, hp.sparse_threshold, T, ff, b->h16, st));
-    if (!falcon) PI_TRY(pi_k_gemm_wide_f16(m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD, b->ffn_inp, nullptr, b->x2, nullptr, st));
-    else         PI_TRY(pi_k_gemm_wide_f16(m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD2, b->attn_out, x, b->x2, nullptr, st));
+    if (!falcon) PI_TRY(chunk_gemm(m, m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD, b->ffn_inp, nullptr, b->x2, nullptr));
+    else         PI_TRY(chunk_gemm(m, m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD2, b->attn_out, x, b->x2, nullptr));
     std::swap(b->x, b->x2);
     return PI_OK;
 }
@@ -200,11 +208,20 @@ bool prefill_wide_supported(pi_model * m) {
     return !(off && off[0] == '1') && prefill_supported(m) && m->hp.n_embd % 256 == 0 && m->hp.n_ff % 256 == 0 && (int)m->L(0, PI_T_FC1).ne1 % 256 == 0;
 }
 
+int prefill_wide_max(pi_model * m) {
+    const char * own = getenv("PI_PREFILL_GEMM");
+    return (own && !strcmp(own, "own")) ? 128 : 512;
+}
+
 int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) {
-    constexpr int kMaxT = 128;
-    if (T <= 16 || T > kMaxT) return pi::fail(PI_E_ARG, "prefill_wide_chunk: 16 < T <= 128");
+    const int kMaxT = prefill_wide_max(m);
+    if (T <= 16 || T > kMaxT) return pi::fail(PI_E_ARG, "prefill_wide_chunk: chunk length outside 17 .. prefill_wide_max");
     const pi_hparams & hp = m->hp;
     if (!m->prefill_wide) {
+        if (kMaxT > 128) {
+            m->gemm_lib = pi_gemm_lib_create((size_t)64 << 20);
+            if (!m->gemm_lib) return PI_E_HIP;
+        }
         BatchState * b = batch_alloc(m, kMaxT, false);
         if (!b) return PI_E_HIP;
         b->prefill = true;
@@ -224,7 +241,7 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
     }
     BatchState * b = m->prefill_wide;
     b->n_seq = T;
-    int32_t pos[kMaxT];
+    int32_t pos[512];
     for (int t = 0; t < T; ++t) pos[t] = n_past + t;
     PI_HIP_TRY(hipMemcpyAsync(b->d_tokens, tokens, sizeof(int32_t) * T, hipMemcpyHostToDevice, m->stream));
     PI_HIP_TRY(hipMemcpyAsync(b->d_pos, pos, sizeof(int32_t) * T, hipMemcpyHostToDevice, m->stream));
@@ -263,6 +280,7 @@ int prefill_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) {
 void batch_destroy(pi_model * m) {
     if (m->prefill) { delete m->prefill; m->prefill = nullptr; }
     if (m->prefill_wide) { delete m->prefill_wide; m->prefill_wide = nullptr; }
+    if (m->gemm_lib) { (void)pi_gemm_lib_destroy(m->gemm_lib); m->gemm_lib = nullptr; }
     if (!m->batch) return;
     if (m->batch->graph_exec) (void)hipGraphExecDestroy(m->batch->graph_exec);
     if (m->batch->graph) (void)hipGraphDestroy(m->batch->graph);

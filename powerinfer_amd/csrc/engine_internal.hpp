@@ -54,7 +54,8 @@ struct pi_model {
     std::vector<int32_t *> hot_prefix;    //                   GPU-resident neurons before group g = row of the compact matrices
     BatchState * batch = nullptr;         // per-sequence caches and step buffers of batched decoding
     BatchState * prefill = nullptr;       // step buffers for prompt chunks of the model's own sequence
-    BatchState * prefill_wide = nullptr;  // the same for chunks of up to 128 tokens (dense mat-muls, weights read once per chunk)
+    BatchState * prefill_wide = nullptr;  // the same for chunks of up to 512 tokens (dense mat-muls, weights read once per chunk)
+    pi_gemm_lib * gemm_lib = nullptr;     // hipBLASLt plans of those mat-muls (PI_PREFILL_GEMM=own keeps them on this library's kernel, 128 tokens a chunk)
     std::vector<__half *> down_rows;      // per layer: the down projection with the neurons contiguous ([n_embd][n_ff]), made at the first wide chunk
 
     Tensor & L(int il, int kind) { return layers[(size_t)il * PI_T_COUNT + kind]; }
@@ -72,5 +73,6 @@ void batch_destroy(pi_model * m);       // frees the batched-decoding state (gra
 bool prefill_supported(pi_model * m);   // F16 weights, every neuron on the GPU, shapes the multi-token kernels cover
 int  prefill_chunk(pi_model * m, const int32_t * tokens, int T, int n_past);
 bool prefill_wide_supported(pi_model * m);   // and additionally n_ff and the predictor rank multiples of 256
-int  prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past);     // 16 < T <= 128
+int  prefill_wide_max(pi_model * m);         // longest chunk: 512 through the library mat-mul, 128 on this library's own kernel (PI_PREFILL_GEMM=own)
+int  prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past);     // 16 < T <= prefill_wide_max
 }

@@ -2700,7 +2700,8 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
 // global reads, as above; the load registers are free again once the tile is written, so the next super-step's loads are issued at
 // once and travel during the MFMAs) and streams the activations of all NT x 16 tokens past it, one 32-column step ahead.
 // K is split over the four waves of a workgroup (super-steps w, w + 4, ...); their partial tiles meet in LDS in wave order.
-constexpr int kWideMaxT = 128;
+constexpr int kWideMaxT = 128;            // longest chunk of gemm_wide_f16_kernel
+constexpr int kChunkMaxT = 512;           // longest chunk of the attention, embedding and elementwise kernels of a prompt chunk
 template <int RT, int NT>
 __global__ __launch_bounds__(kBlock) void gemm_wide_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
                                                                int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y,
@@ -3876,7 +3877,7 @@ int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_t
 int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
                     const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache, float * out, int out_stride, void * out_f16,
                     pi_stream_t stream) {
-    if (!qkv || !pos || !q_rot || !k_cache || !v_cache || !out || T <= 0 || T > kWideMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad arguments");
+    if (!qkv || !pos || !q_rot || !k_cache || !v_cache || !out || T <= 0 || T > kChunkMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad arguments");
     if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd <= 0 || hd % 8 || hd / 2 > 1024 || kBlock % (hd / 8) || PI_WAVE % (hd / 8) || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad head geometry or mode");
     const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd);
@@ -3914,7 +3915,7 @@ int pi_k_step_advance(int32_t * step, pi_stream_t stream) {
 }
 
 int pi_k_embed_batch(const void * table_f16, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream) {
-    if (!table_f16 || !tokens || !x || cols <= 0 || T <= 0 || T > kWideMaxT) return pi::fail(PI_E_ARG, "pi_k_embed_batch: bad arguments");
+    if (!table_f16 || !tokens || !x || cols <= 0 || T <= 0 || T > kChunkMaxT) return pi::fail(PI_E_ARG, "pi_k_embed_batch: bad arguments");
     hipLaunchKernelGGL(embed_f16_batch_kernel, dim3((cols + 255) / 256, T), dim3(256), 0, (hipStream_t)stream, (const __half *)table_f16, cols, tokens, x);
     return pi::check_launch("pi_k_embed_batch");
 }

@@ -78,6 +78,9 @@ _SIGS = {
     "pi_k_gemm_wide_f16": (_i, [_vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_ffn_h_f16": (_i, [_vp, _vp, _vp, _f, _i, _i, _vp, _vp]),
     "pi_k_transpose_f16": (_i, [_vp, _i, _i, _vp, _vp]),
+    "pi_gemm_lib_create": (_vp, [C.c_size_t]),
+    "pi_gemm_lib_destroy": (_i, [_vp]),
+    "pi_gemm_lib_f16": (_i, [_vp, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_batch_sparse_mul_mat": (_i, [_vp, _i, _i, _vp, _i, _vp, _f, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_batch_sparse_axpy": (_i, [_vp, _i, _i, _vp, _vp, _i, _f, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_attn_fused_batch": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),

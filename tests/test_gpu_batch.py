@@ -92,6 +92,44 @@ def test_gemm_wide_matches_oracle(rows, cols, T):
     assert np.array_equal(dt.download(np.float16).reshape(cols, rows), w.T)
 
 
+@pytest.mark.parametrize("rows,cols,T", [(3000, 5120, 300), (4104, 4096, 512), (1024, 11008, 130), (520, 512, 17), (12288, 4096, 512)])
+def test_gemm_lib_matches_oracle(rows, cols, T):
+    """The library mat-mul of long prompt chunks (hipBLASLt plans, fp16 operands, fp32 accumulation) against the reference's CPU
+    mat-mul on the same fp16-rounded activations: token and row counts on and off round numbers, the FFN-wide reduction, every
+    epilogue (a residual as the C operand, the second residual / ReLU / fp16 copy in the pass behind it), a plan used twice."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    rng = np.random.default_rng(rows + cols + T)
+    w = (rng.standard_normal((rows, cols)) * 0.02).astype(np.float16)
+    x = rng.standard_normal((T, cols)).astype(np.float32)
+    a1, a2 = rng.standard_normal((T, rows)).astype(np.float32), rng.standard_normal((T, rows)).astype(np.float32)
+    want = np.zeros((T, rows), np.float32)
+    assert ol.oracle().pio_mul_mat(ol.F16, P(w), rows, cols, P(x), T, P(want), 8) == 0
+    g = L.pi_gemm_lib_create(32 << 20)
+    assert g, L.pi_last_error()
+    dn = gpu_norm_round(pl, L, x)
+    dw, dy, d1, d2 = pl.DevBuf(host=w), pl.DevBuf(T * rows * 4), pl.DevBuf(host=a1), pl.DevBuf(host=a2)
+    for _ in range(2):
+        pl.check(L.pi_memset(dy.ptr, 0xFF, dy.nbytes), "memset")
+        pl.check(L.pi_gemm_lib_f16(g, dw.ptr, rows, cols, dn.ptr, T, pl.EPI_NONE, None, None, dy.ptr, None, None), "gemm_lib")
+        pl.sync()
+        assert rel_err(dy.download(np.float32).reshape(T, rows), want) < 2e-5
+    pl.check(L.pi_gemm_lib_f16(g, dw.ptr, rows, cols, dn.ptr, T, pl.EPI_ADD, d1.ptr, None, dy.ptr, None, None), "gemm_lib")
+    pl.sync()
+    assert rel_err(dy.download(np.float32).reshape(T, rows), want + a1) < 2e-5
+    pl.check(L.pi_gemm_lib_f16(g, dw.ptr, rows, cols, dn.ptr, T, pl.EPI_ADD2, d1.ptr, d2.ptr, dy.ptr, None, None), "gemm_lib")
+    pl.sync()
+    assert rel_err(dy.download(np.float32).reshape(T, rows), (want + a1) + a2) < 2e-5
+    dy16 = pl.DevBuf(T * rows * 2)
+    pl.check(L.pi_gemm_lib_f16(g, dw.ptr, rows, cols, dn.ptr, T, pl.EPI_RELU, None, None, dy.ptr, dy16.ptr, None), "gemm_lib")
+    pl.sync()
+    got = dy.download(np.float32).reshape(T, rows)
+    assert rel_err(got, np.maximum(want, 0)) < 2e-5
+    assert np.array_equal(dy16.download(np.float16).reshape(T, rows), got.astype(np.float16))
+    assert L.pi_gemm_lib_f16(g, dw.ptr, rows, cols, dn.ptr, T, pl.EPI_ADD, None, None, dy.ptr, None, None) != 0      # residual missing
+    pl.check(L.pi_gemm_lib_destroy(g), "destroy")
+
+
 def test_ffn_h_from_dense_products():
     from powerinfer_amd import lib as pl
     L = pl.init()
@@ -392,16 +430,24 @@ def test_prompt_chunks_match_token_by_token(arch):
 
 
 @pytest.mark.timeout(300)
-@pytest.mark.parametrize("name,kw,n_prompt", [("llama-tiny", dict(n_rank=256, n_ctx=192), 150), ("falcon-tiny", dict(n_rank=256, n_ctx=192), 150),
-                                              ("llama-tiny", dict(n_rank=256, n_ctx=192), 40),
-                                              ("llama-7b", dict(n_layer=2, n_ctx=160), 140)])
-def test_wide_prompt_chunks_match_the_oracle(name, kw, n_prompt):
-    """Prompts longer than 16 tokens go through chunks of up to 128 (dense mat-muls, every weight row read once per chunk, the
-    predictor's mask applied as zeros of h), then chunks of 16, then the last token alone.  On a margin-protected model (no
-    neuron can flip, greedy decisions keep their distance) the logits after the prompt and of the steps behind it agree with
-    the CPU oracle within the stated tolerance, and with the same engine fed 16 tokens at a time."""
+@pytest.mark.parametrize("name,kw,n_prompt,gemm", [("llama-tiny", dict(n_rank=256, n_ctx=192), 150, "own"), ("falcon-tiny", dict(n_rank=256, n_ctx=192), 150, "own"),
+                                                   ("llama-tiny", dict(n_rank=256, n_ctx=192), 40, "own"),
+                                                   ("llama-7b", dict(n_layer=2, n_ctx=160), 140, "own"),
+                                                   ("llama-tiny", dict(n_rank=256, n_ctx=192), 150, "lib"), ("falcon-tiny", dict(n_rank=256, n_ctx=640), 600, "lib"),
+                                                   ("llama-tiny", dict(n_rank=256, n_ctx=192), 40, "lib"),
+                                                   ("llama-7b", dict(n_layer=2, n_ctx=640), 600, "lib")])
+def test_wide_prompt_chunks_match_the_oracle(name, kw, n_prompt, gemm, monkeypatch):
+    """Prompts longer than 16 tokens go through chunks of up to 512 (dense mat-muls through the library, every weight row read once
+    per chunk, the predictor's mask applied as zeros of h; chunks of up to 128 on this library's own mat-mul kernel with
+    PI_PREFILL_GEMM=own), then chunks of 16, then the last token alone.  On a margin-protected model (no neuron can flip, greedy
+    decisions keep their distance) the logits after the prompt and of the steps behind it agree with the CPU oracle within the
+    stated tolerance, and with the same engine fed 16 tokens at a time."""
     import os
     from powerinfer_amd.model import Model
+    if gemm == "own":
+        monkeypatch.setenv("PI_PREFILL_GEMM", "own")
+    else:
+        monkeypatch.delenv("PI_PREFILL_GEMM", raising=False)
     hp = synth.hparams(name, seed=5, pred_margin=True, head_pair=2048, **kw)
     model = synth.make_model(hp)
     rng = np.random.default_rng(8)

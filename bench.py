@@ -451,13 +451,14 @@ def main():
     del keep
     if args.prompt_bench > 0 and not hybrid and hp.wtype == pl.F16:
         # prompt phase on its own: a fresh instance of the same model with room for the prompt, one untimed pass (allocations, the
-        # transposed down projections), then the timed pass from an empty cache; chunks of up to 128 tokens per weight pass
+        # transposed down projections, the library's mat-mul plans), then the timed pass from an empty cache; chunks of up to 512 tokens
+        # per weight pass
         try:
             hp2 = synth.hparams({1: "llama-7b", 4: "falcon-40b"}[args.config], n_layer=hp.n_layer, n_ctx=args.prompt_bench + 8, seed=1)
             keep2 = []
             m2 = build_synthetic_on_device(hp2, keep2)
             ptoks = rng.integers(0, hp2.n_vocab, args.prompt_bench).astype(np.int32)
-            m2.decode(ptoks[:200], 0, want_logits=False)
+            m2.decode(ptoks, 0, want_logits=False)
             m2.kv_clear()
             pl.sync()
             t0 = time.perf_counter()
@@ -465,8 +466,8 @@ def main():
             pl.sync()
             dt = time.perf_counter() - t0
             out["prompt_phase"] = {"tokens": args.prompt_bench, "ms": round(dt * 1e3, 2), "tok_per_s": round(args.prompt_bench / dt, 1),
-                                   "what": "pi_model_decode of the whole prompt: chunks of up to 128 tokens (dense MFMA mat-muls, each weight row read "
-                                           "once per chunk, predictor mask applied to h), last token through the single-token path"}
+                                   "what": "pi_model_decode of the whole prompt: chunks of up to 512 tokens (dense mat-muls through hipBLASLt plans, each weight "
+                                           "row read once per chunk, predictor mask applied to h), last token through the single-token path"}
             m2.close()
             del keep2
         except Exception as e:

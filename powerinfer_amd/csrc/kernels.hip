@@ -6,6 +6,8 @@
 #include "../../include/powerinfer_hip.h"
 
 #include <math.h>
+#include <stdlib.h>
+#include <string.h>
 
 #include <vector>
 
@@ -2815,6 +2817,151 @@ __global__ void transpose_f16_kernel(const __half * __restrict__ in, int rows, i
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Attention of a prompt chunk on the matrix cores: a workgroup owns 16 consecutive tokens of one query head and the four waves
+// split the cache cells.  Three phases, with the rounding points of attn_decode_kernel (and so of the CPU path):
+//   1. scores: S[cell][token] = K[cell] . fp16(q[token]) by 16x16x32 MFMAs (a K row is read in operand layout straight from
+//      the cache, q stays in registers), times 1/sqrt(hd), into LDS as s[token][cell];
+//   2. softmax per token over the cells it may see (cell <= its position): maximum, fp16(exp(fp16(s - max))), the sum in double,
+//      p = fp16(e / sum); cells beyond the token's position become exact zeros;
+//   3. out[token][:] = sum over cells of p * V[cell][:]: the V cache keeps a cell's head contiguous, the MFMA wants eight cells of
+//      one column per lane, so a wave reads eight cells of a column pair (4 bytes per lane, a whole row per instruction), packs
+//      them with two byte permutes per pair of cells and drops two 16-byte columns into its private LDS tile (32 cells a tile),
+//      from where the operand comes back with one 16-byte read.  No workgroup barrier inside the loops: the tile belongs to one
+//      wave and the LDS operations of a wave complete in order.  The waves' partial outputs meet in LDS in wave order.
+// HD = 128 or 64.  LDS: 16 x (cells rounded up to 32, + 4) floats of scores + 4 x HD x 80 bytes of V tiles.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kAcVtStride = 40;                // halves per row of the transposed V tile: 32 cells + 8 of padding (conflict-free both ways)
+template <int HD>
+__global__ __launch_bounds__(kBlock) void attn_chunk_mfma_kernel(const float * __restrict__ q_rot, const __half * __restrict__ k_cache,
+                                                                 const __half * __restrict__ v_cache, int n_head, int n_head_kv, int n_ctx,
+                                                                 const int32_t * __restrict__ pos_p, int T, float * __restrict__ out,
+                                                                 int q_stride, int out_stride, __half * __restrict__ out16, int s_stride) {
+    static_assert(HD == 128 || HD == 64, "head size");
+    extern __shared__ __align__(16) unsigned char smem[];
+    float * s = reinterpret_cast<float *>(smem);                                       // [16][s_stride]
+    unsigned char * vt_all = smem + sizeof(float) * 16 * (size_t)s_stride;             // [4 waves][HD][kAcVtStride] halves
+    const int h = blockIdx.x, kvh = h / (n_head / n_head_kv);
+    const int t0 = blockIdx.y * 16;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
+    // cells the furthest-reaching token of the tile sees
+    int n_kv = pos_p[min(t0 + i, T - 1)] + 1;
+    for (int o = 8; o > 0; o >>= 1) n_kv = max(n_kv, __shfl_xor(n_kv, o, PI_WAVE));
+    const int n_t16 = (n_kv + 15) / 16, n_t32 = (n_kv + 31) / 32;
+
+    // ---- 1. scores --------------------------------------------------------------------------------------------------------
+    {
+        const float * qp = q_rot + (size_t)min(t0 + i, T - 1) * q_stride + (size_t)h * HD + 8 * g;
+        pi_h8 qf[HD / 32];
+#pragma unroll
+        for (int ks = 0; ks < HD / 32; ++ks) {
+            const float4 a = *reinterpret_cast<const float4 *>(qp + ks * 32), b = *reinterpret_cast<const float4 *>(qp + ks * 32 + 4);
+            qf[ks] = pi_h8{(_Float16)a.x, (_Float16)a.y, (_Float16)a.z, (_Float16)a.w, (_Float16)b.x, (_Float16)b.y, (_Float16)b.z, (_Float16)b.w};
+        }
+        const float scale = pi_inv_sqrt((float)HD);
+        const __half * kb = k_cache + (size_t)kvh * n_ctx * HD + 8 * g;
+        pi_u32x4 a[HD / 32], an[HD / 32];
+        auto issue = [&](pi_u32x4 * dst, int kt) {
+            if (kt < n_t16) {
+                const int c = min(kt * 16 + i, n_kv - 1);
+#pragma unroll
+                for (int ks = 0; ks < HD / 32; ++ks) dst[ks] = pi_ld16(kb + (size_t)c * HD + ks * 32);
+            }
+        };
+        issue(a, wave);
+        for (int kt = wave; kt < n_t16; kt += kWavesPerBlock) {
+            issue(an, kt + kWavesPerBlock);
+            pi_f4 acc = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (int ks = 0; ks < HD / 32; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a[ks]), qf[ks], acc, 0, 0, 0);
+            // acc[r] = S[cell kt*16 + 4g + r][token i]
+            *reinterpret_cast<float4 *>(s + (size_t)i * s_stride + kt * 16 + 4 * g) =
+                float4{__fmul_rn(acc[0], scale), __fmul_rn(acc[1], scale), __fmul_rn(acc[2], scale), __fmul_rn(acc[3], scale)};
+#pragma unroll
+            for (int ks = 0; ks < HD / 32; ++ks) a[ks] = an[ks];
+        }
+    }
+    __syncthreads();
+
+    // ---- 2. softmax: 16 lanes per token ---------------------------------------------------------------------------------------
+    {
+        const int q = threadIdx.x >> 4, j = threadIdx.x & 15;
+        const int nq = pos_p[min(t0 + q, T - 1)] + 1;
+        float * sq = s + (size_t)q * s_stride;
+        float mx = -INFINITY;
+        for (int c = j; c < nq; c += 16) mx = fmaxf(mx, sq[c]);
+        for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, PI_WAVE));
+        double sum = 0.0;
+        for (int c = j; c < nq; c += 16) {
+            const float e = pi_round_f16(expf(pi_round_f16(__fsub_rn(sq[c], mx))));
+            sq[c] = e;
+            sum += (double)e;
+        }
+        for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, PI_WAVE);
+        const float inv = (float)(1.0 / sum);
+        for (int c = j; c < n_t32 * 32; c += 16) sq[c] = c < nq ? pi_round_f16(__fmul_rn(sq[c], inv)) : 0.0f;
+    }
+    __syncthreads();
+
+    // ---- 3. p . V -------------------------------------------------------------------------------------------------------------
+    pi_f4 acc[HD / 16];
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt) acc[dt] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    unsigned char * myvt = vt_all + (size_t)wave * HD * kAcVtStride * 2;
+    {
+        constexpr int LPR = HD / 2;                 // lanes per V row, 4 bytes (a column pair) each
+        constexpr int GPI = PI_WAVE / LPR;          // groups of eight cells per load instruction
+        const int dp = lane % LPR, sub = lane / LPR;
+        const __half * vb = v_cache + (size_t)kvh * n_ctx * HD + 2 * dp;
+        for (int kt = wave; kt < n_t32; kt += kWavesPerBlock) {
+            const int c0 = kt * 32;
+#pragma unroll
+            for (int rnd = 0; rnd < 4 / GPI; ++rnd) {
+                const int grp8 = rnd * GPI + sub;   // which eight cells of the tile
+                unsigned v[8];
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    const int c = c0 + grp8 * 8 + k;
+                    v[k] = c < n_kv ? *reinterpret_cast<const unsigned *>(vb + (size_t)c * HD) : 0u;      // cells past the end may hold anything
+                }
+                pi_u32x4 lo, hi;
+                lo.x = __builtin_amdgcn_perm(v[1], v[0], 0x05040100u); hi.x = __builtin_amdgcn_perm(v[1], v[0], 0x07060302u);
+                lo.y = __builtin_amdgcn_perm(v[3], v[2], 0x05040100u); hi.y = __builtin_amdgcn_perm(v[3], v[2], 0x07060302u);
+                lo.z = __builtin_amdgcn_perm(v[5], v[4], 0x05040100u); hi.z = __builtin_amdgcn_perm(v[5], v[4], 0x07060302u);
+                lo.w = __builtin_amdgcn_perm(v[7], v[6], 0x05040100u); hi.w = __builtin_amdgcn_perm(v[7], v[6], 0x07060302u);
+                *reinterpret_cast<pi_u32x4 *>(myvt + ((size_t)(2 * dp) * kAcVtStride + grp8 * 8) * 2) = lo;
+                *reinterpret_cast<pi_u32x4 *>(myvt + ((size_t)(2 * dp + 1) * kAcVtStride + grp8 * 8) * 2) = hi;
+            }
+            const float * pp = s + (size_t)i * s_stride + c0 + 8 * g;
+            const float4 p0 = *reinterpret_cast<const float4 *>(pp), p1 = *reinterpret_cast<const float4 *>(pp + 4);
+            const pi_h8 pa = pi_h8{(_Float16)p0.x, (_Float16)p0.y, (_Float16)p0.z, (_Float16)p0.w, (_Float16)p1.x, (_Float16)p1.y, (_Float16)p1.z, (_Float16)p1.w};
+#pragma unroll
+            for (int dt = 0; dt < HD / 16; ++dt) {
+                const pi_u32x4 b = *reinterpret_cast<const pi_u32x4 *>(myvt + ((size_t)(dt * 16 + i) * kAcVtStride + 8 * g) * 2);
+                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(pi_h8, b), acc[dt], 0, 0, 0);
+            }
+        }
+    }
+    // acc[dt][r] = out[token 4g + r][dt*16 + i] over this wave's cells; the four partial tiles meet in wave order
+    constexpr int PS = HD + 4;
+    float * mypart = reinterpret_cast<float *>(myvt);                                  // [16][PS], inside the wave's own tile
+#pragma unroll
+    for (int dt = 0; dt < HD / 16; ++dt)
+#pragma unroll
+        for (int r = 0; r < 4; ++r) mypart[(4 * g + r) * PS + dt * 16 + i] = acc[dt][r];
+    __syncthreads();
+    for (int e = threadIdx.x; e < 16 * HD; e += kBlock) {
+        const int q = e / HD, d = e % HD, t = t0 + q;
+        if (t < T) {
+            float v = 0.0f;
+#pragma unroll
+            for (int w = 0; w < kWavesPerBlock; ++w) v += reinterpret_cast<const float *>(vt_all + (size_t)w * HD * kAcVtStride * 2)[q * PS + d];
+            out[(size_t)t * out_stride + (size_t)h * HD + d] = v;
+            if (out16) out16[(size_t)t * out_stride + (size_t)h * HD + d] = __float2half_rn(v);
+        }
+    }
+}
+
 // the operator boundary hands over the predictor's output instead of running the predictor: row_any[n] = some token has !(idx[t][n] < thr)
 __global__ void batch_flag_any_kernel(const float * __restrict__ idx, int T, int ff, float thr, unsigned char * __restrict__ row_any) {
     const int n = blockIdx.x * blockDim.x + threadIdx.x;
@@ -3880,12 +4027,30 @@ int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_
     if (!qkv || !pos || !q_rot || !k_cache || !v_cache || !out || T <= 0 || T > kChunkMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad arguments");
     if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd <= 0 || hd % 8 || hd / 2 > 1024 || kBlock % (hd / 8) || PI_WAVE % (hd / 8) || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad head geometry or mode");
-    const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd);
-    if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_chunk: context too long for the single-pass kernel");
     hipStream_t st = (hipStream_t)stream;
     // all K/V rows of the chunk are in the cache before any token of the chunk attends
     hipLaunchKernelGGL(rope_kv_store_kernel, dim3(n_head + 2 * n_head_kv, T), dim3(hd / 2), 0, st,
                        qkv, n_head, n_head_kv, hd, mode, theta_scale, pos, n_ctx, q_rot, (__half *)k_cache, (__half *)v_cache, qkv_stride, n_head * hd);
+    // 16 tokens per workgroup on the matrix cores where the head size and the context fit (scores of 16 tokens in LDS)
+    const int s_stride = ((n_ctx + 31) & ~31) + 4;
+    const size_t sh_mfma = sizeof(float) * 16 * (size_t)s_stride + (size_t)kWavesPerBlock * hd * kAcVtStride * 2;
+    const char * own = getenv("PI_ATTN_CHUNK");
+    if ((hd == 128 || hd == 64) && T > 1 && sh_mfma <= 156 * 1024 && !(own && !strcmp(own, "scalar"))) {
+        static bool raised[2] = {false, false};
+        if (!raised[hd == 64]) {
+            if (hd == 128) PI_HIP_TRY(hipFuncSetAttribute((const void *)attn_chunk_mfma_kernel<128>, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
+            else           PI_HIP_TRY(hipFuncSetAttribute((const void *)attn_chunk_mfma_kernel<64>, hipFuncAttributeMaxDynamicSharedMemorySize, 156 * 1024));
+            raised[hd == 64] = true;
+        }
+        const dim3 grid(n_head, (T + 15) / 16);
+        if (hd == 128) hipLaunchKernelGGL(attn_chunk_mfma_kernel<128>, grid, dim3(kBlock), sh_mfma, st, q_rot, (const __half *)k_cache, (const __half *)v_cache,
+                                          n_head, n_head_kv, n_ctx, pos, T, out, n_head * hd, out_stride, (__half *)out_f16, s_stride);
+        else           hipLaunchKernelGGL(attn_chunk_mfma_kernel<64>, grid, dim3(kBlock), sh_mfma, st, q_rot, (const __half *)k_cache, (const __half *)v_cache,
+                                          n_head, n_head_kv, n_ctx, pos, T, out, n_head * hd, out_stride, (__half *)out_f16, s_stride);
+        return pi::check_launch("pi_k_attn_chunk");
+    }
+    const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd);
+    if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_chunk: context too long for the single-pass kernel");
     hipLaunchKernelGGL(attn_decode_kernel, dim3(n_head, T), dim3(kBlock), sh, st,
                        q_rot, (const __half *)k_cache, (const __half *)v_cache, n_head, n_head_kv, hd, n_ctx, pos, out, n_head * hd, out_stride, (__half *)out_f16);
     return pi::check_launch("pi_k_attn_chunk");

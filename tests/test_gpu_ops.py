@@ -98,6 +98,58 @@ def test_gemv_rejects_bad_shapes():
     assert b"pi_k_gemv" in L.pi_last_error()
 
 
+@pytest.mark.parametrize("mode,hd,nh,nkv,chunks", [(0, 128, 4, 4, (37, 45)), (2, 64, 8, 2, (70, 17, 2)), (0, 128, 2, 1, (130,)), (0, 64, 4, 4, (16, 33))])
+def test_attention_of_prompt_chunks(mode, hd, nh, nkv, chunks, monkeypatch):
+    """Prompt chunks through pi_k_attn_chunk (RoPE + KV store of the whole chunk, then causal attention of every token over the cache)
+    against the oracle's rope + attention: the route on the matrix cores (16 tokens per workgroup; chunk lengths on and off that
+    tile, caches filled by earlier chunks, grouped query heads) and the one-token-per-workgroup route, which must agree with
+    each other more closely than either has to agree with the CPU."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    O = ol.oracle()
+    rng = np.random.default_rng(mode + hd + sum(chunks))
+    n_ctx, gqa, d = 160, nkv * hd, nh * hd
+    kc_o = np.zeros((n_ctx, gqa), np.uint16)
+    vc_o = np.zeros((gqa, n_ctx), np.uint16)
+    theta_scale = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
+    caches = {r: (pl.DevBuf.zeros(nkv * n_ctx * hd * 2), pl.DevBuf.zeros(nkv * n_ctx * hd * 2)) for r in ("mfma", "scalar")}
+    for kc, vc in caches.values():                                    # cells never written must not leak into a result
+        pl.check(L.pi_memset(kc.ptr, 0x7E, kc.nbytes), "memset")      # 0x7E7E is a NaN pattern in fp16
+        pl.check(L.pi_memset(vc.ptr, 0x7E, vc.nbytes), "memset")
+    n_past = 0
+    for T in chunks:
+        qkv = rng.standard_normal((T, d + 2 * gqa)).astype(np.float32)
+        q, k, v = (np.ascontiguousarray(a) for a in (qkv[:, :d], qkv[:, d:d + gqa], qkv[:, d + gqa:]))
+        pos = np.arange(n_past, n_past + T, dtype=np.int32)
+        qr, kr = np.zeros_like(q), np.zeros_like(k)
+        O.pio_rope(P(q), hd, nh, T, P(pos), hd, mode, 10000.0, 1.0, P(qr))
+        O.pio_rope(P(k), hd, nkv, T, P(pos), hd, mode, 10000.0, 1.0, P(kr))
+        n_kv = (n_past + T + 31) // 32 * 32
+        mask = np.where(np.arange(n_kv)[None, :] > pos[:, None], -np.inf, 0).astype(np.float32)
+        want = np.zeros((T, d), np.float32)
+        assert O.pio_attention(hd, nh, nkv, n_ctx, n_kv, T, P(pos), P(mask), P(qr), P(kr), P(v), P(kc_o), P(vc_o), P(want)) == 0
+        dq, dpos = pl.DevBuf(host=qkv), pl.DevBuf(host=pos)
+        got = {}
+        for route, (kc, vc) in caches.items():
+            if route == "scalar":
+                monkeypatch.setenv("PI_ATTN_CHUNK", "scalar")
+            else:
+                monkeypatch.delenv("PI_ATTN_CHUNK", raising=False)
+            dqr, dout, dout16 = pl.DevBuf(T * d * 4), pl.DevBuf(T * d * 4), pl.DevBuf(T * d * 2)
+            pl.check(L.pi_memset(dout.ptr, 0xFF, dout.nbytes), "memset")
+            pl.check(L.pi_k_attn_chunk(dq.ptr, d + 2 * gqa, T, nh, nkv, hd, mode, theta_scale, dpos.ptr, n_ctx, dqr.ptr, kc.ptr, vc.ptr,
+                                       dout.ptr, d, dout16.ptr, None), "attn_chunk")
+            pl.sync()
+            got[route] = dout.download(np.float32).reshape(T, d)
+            assert np.array_equal(dout16.download(np.float16).reshape(T, d), got[route].astype(np.float16))
+            assert rel_err(got[route], want) < 2e-3, (route, T, rel_err(got[route], want))
+        # the scores are summed in another order, so here and there fp16(s - max) lands on the neighbouring value and one p moves by a unit
+        assert rel_err(got["mfma"], got["scalar"]) < 5e-4, rel_err(got["mfma"], got["scalar"])
+        assert not np.array_equal(got["mfma"], got["scalar"])         # two routes, two summation orders
+        n_past += T
+    monkeypatch.delenv("PI_ATTN_CHUNK", raising=False)
+
+
 @pytest.mark.parametrize("mode,hd,nh,nkv", [(0, 128, 4, 4), (2, 64, 8, 2)])
 def test_rope_attention_sequence(mode, hd, nh, nkv):
     """Six decode steps: RoPE + KV store + attention on the GPU against the oracle's rope + attention with

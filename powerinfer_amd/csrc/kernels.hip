@@ -2860,46 +2860,72 @@ __global__ __launch_bounds__(kBlock) void attn_chunk_mfma_kernel(const float * _
         }
         const float scale = pi_inv_sqrt((float)HD);
         const __half * kb = k_cache + (size_t)kvh * n_ctx * HD + 8 * g;
-        pi_u32x4 a[HD / 32], an[HD / 32];
+        // six tiles of K rows are in flight per wave: the loads come from L2 and a wave has little else to hide their latency behind
+        constexpr int D1 = 6;
+        pi_u32x4 a[D1][HD / 32];
+        // (requests past the last tile re-read the last cell: unconditional loads keep the count of outstanding ones static, which
+        // is what lets the compiler wait for the oldest tile only)
         auto issue = [&](pi_u32x4 * dst, int kt) {
-            if (kt < n_t16) {
-                const int c = min(kt * 16 + i, n_kv - 1);
+            const int c = min(kt * 16 + i, n_kv - 1);
 #pragma unroll
-                for (int ks = 0; ks < HD / 32; ++ks) dst[ks] = pi_ld16(kb + (size_t)c * HD + ks * 32);
-            }
+            for (int ks = 0; ks < HD / 32; ++ks) dst[ks] = pi_ld16(kb + (size_t)c * HD + ks * 32);
         };
-        issue(a, wave);
-        for (int kt = wave; kt < n_t16; kt += kWavesPerBlock) {
-            issue(an, kt + kWavesPerBlock);
-            pi_f4 acc = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
-            for (int ks = 0; ks < HD / 32; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a[ks]), qf[ks], acc, 0, 0, 0);
-            // acc[r] = S[cell kt*16 + 4g + r][token i]
-            *reinterpret_cast<float4 *>(s + (size_t)i * s_stride + kt * 16 + 4 * g) =
-                float4{__fmul_rn(acc[0], scale), __fmul_rn(acc[1], scale), __fmul_rn(acc[2], scale), __fmul_rn(acc[3], scale)};
+        for (int u = 0; u < D1; ++u) issue(a[u], wave + u * kWavesPerBlock);
+        for (int kt0 = wave; kt0 < n_t16; kt0 += D1 * kWavesPerBlock) {
 #pragma unroll
-            for (int ks = 0; ks < HD / 32; ++ks) a[ks] = an[ks];
+            for (int u = 0; u < D1; ++u) {
+                const int kt = kt0 + u * kWavesPerBlock;
+                if (kt < n_t16) {
+                    pi_f4 acc = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+                    for (int ks = 0; ks < HD / 32; ++ks) acc = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a[u][ks]), qf[ks], acc, 0, 0, 0);
+                    // acc[r] = S[cell kt*16 + 4g + r][token i]
+                    *reinterpret_cast<float4 *>(s + (size_t)i * s_stride + kt * 16 + 4 * g) =
+                        float4{__fmul_rn(acc[0], scale), __fmul_rn(acc[1], scale), __fmul_rn(acc[2], scale), __fmul_rn(acc[3], scale)};
+                }
+                issue(a[u], kt + D1 * kWavesPerBlock);
+            }
         }
     }
     __syncthreads();
 
-    // ---- 2. softmax: 16 lanes per token ---------------------------------------------------------------------------------------
+    // ---- 2. softmax: 16 lanes per token, four cells per lane and step ------------------------------------------------------------
     {
         const int q = threadIdx.x >> 4, j = threadIdx.x & 15;
         const int nq = pos_p[min(t0 + q, T - 1)] + 1;
         float * sq = s + (size_t)q * s_stride;
         float mx = -INFINITY;
-        for (int c = j; c < nq; c += 16) mx = fmaxf(mx, sq[c]);
+        for (int c = 4 * j; c < nq; c += 64) {
+            const float4 v = *reinterpret_cast<const float4 *>(sq + c);
+            mx = fmaxf(mx, v.x);
+            if (c + 1 < nq) mx = fmaxf(mx, v.y);
+            if (c + 2 < nq) mx = fmaxf(mx, v.z);
+            if (c + 3 < nq) mx = fmaxf(mx, v.w);
+        }
         for (int o = 8; o > 0; o >>= 1) mx = fmaxf(mx, __shfl_xor(mx, o, PI_WAVE));
         double sum = 0.0;
-        for (int c = j; c < nq; c += 16) {
-            const float e = pi_round_f16(expf(pi_round_f16(__fsub_rn(sq[c], mx))));
-            sq[c] = e;
-            sum += (double)e;
+        for (int c = 4 * j; c < nq; c += 64) {
+            float4 v = *reinterpret_cast<const float4 *>(sq + c);
+            // exp through fp16 in and out, as the CPU path's lookup table does; cells past the token's own position count as zero
+            v.x = pi_round_f16(expf(pi_round_f16(__fsub_rn(v.x, mx))));
+            v.y = c + 1 < nq ? pi_round_f16(expf(pi_round_f16(__fsub_rn(v.y, mx)))) : 0.0f;
+            v.z = c + 2 < nq ? pi_round_f16(expf(pi_round_f16(__fsub_rn(v.z, mx)))) : 0.0f;
+            v.w = c + 3 < nq ? pi_round_f16(expf(pi_round_f16(__fsub_rn(v.w, mx)))) : 0.0f;
+            *reinterpret_cast<float4 *>(sq + c) = v;
+            sum += (double)v.x; sum += (double)v.y; sum += (double)v.z; sum += (double)v.w;
         }
         for (int o = 8; o > 0; o >>= 1) sum += __shfl_xor(sum, o, PI_WAVE);
         const float inv = (float)(1.0 / sum);
-        for (int c = j; c < n_t32 * 32; c += 16) sq[c] = c < nq ? pi_round_f16(__fmul_rn(sq[c], inv)) : 0.0f;
+        for (int c = 4 * j; c < n_t32 * 32; c += 64) {
+            float4 v = float4{0.0f, 0.0f, 0.0f, 0.0f};
+            if (c < nq) {
+                v = *reinterpret_cast<const float4 *>(sq + c);
+                v.x = pi_round_f16(__fmul_rn(v.x, inv)); v.y = pi_round_f16(__fmul_rn(v.y, inv));
+                v.z = pi_round_f16(__fmul_rn(v.z, inv)); v.w = pi_round_f16(__fmul_rn(v.w, inv));       // zeros past nq stay zeros
+            }
+            *reinterpret_cast<float4 *>(sq + c) = v;
+        }
     }
     __syncthreads();
 
@@ -2913,32 +2939,51 @@ __global__ __launch_bounds__(kBlock) void attn_chunk_mfma_kernel(const float * _
         constexpr int GPI = PI_WAVE / LPR;          // groups of eight cells per load instruction
         const int dp = lane % LPR, sub = lane / LPR;
         const __half * vb = v_cache + (size_t)kvh * n_ctx * HD + 2 * dp;
-        for (int kt = wave; kt < n_t32; kt += kWavesPerBlock) {
-            const int c0 = kt * 32;
+        // the cells of the next three tiles are on their way while a tile is packed and multiplied; cells past the end may hold
+        // anything and enter as zeros
+        constexpr int D3 = 3;
+        unsigned vq[D3][4 / GPI][8];
+        auto issue = [&](unsigned (*dst)[8], int kt) {
 #pragma unroll
-            for (int rnd = 0; rnd < 4 / GPI; ++rnd) {
-                const int grp8 = rnd * GPI + sub;   // which eight cells of the tile
-                unsigned v[8];
+            for (int rnd = 0; rnd < 4 / GPI; ++rnd)
 #pragma unroll
                 for (int k = 0; k < 8; ++k) {
-                    const int c = c0 + grp8 * 8 + k;
-                    v[k] = c < n_kv ? *reinterpret_cast<const unsigned *>(vb + (size_t)c * HD) : 0u;      // cells past the end may hold anything
+                    const int c = kt * 32 + (rnd * GPI + sub) * 8 + k;
+                    dst[rnd][k] = *reinterpret_cast<const unsigned *>(vb + (size_t)min(c, n_kv - 1) * HD);
                 }
-                pi_u32x4 lo, hi;
-                lo.x = __builtin_amdgcn_perm(v[1], v[0], 0x05040100u); hi.x = __builtin_amdgcn_perm(v[1], v[0], 0x07060302u);
-                lo.y = __builtin_amdgcn_perm(v[3], v[2], 0x05040100u); hi.y = __builtin_amdgcn_perm(v[3], v[2], 0x07060302u);
-                lo.z = __builtin_amdgcn_perm(v[5], v[4], 0x05040100u); hi.z = __builtin_amdgcn_perm(v[5], v[4], 0x07060302u);
-                lo.w = __builtin_amdgcn_perm(v[7], v[6], 0x05040100u); hi.w = __builtin_amdgcn_perm(v[7], v[6], 0x07060302u);
-                *reinterpret_cast<pi_u32x4 *>(myvt + ((size_t)(2 * dp) * kAcVtStride + grp8 * 8) * 2) = lo;
-                *reinterpret_cast<pi_u32x4 *>(myvt + ((size_t)(2 * dp + 1) * kAcVtStride + grp8 * 8) * 2) = hi;
-            }
-            const float * pp = s + (size_t)i * s_stride + c0 + 8 * g;
-            const float4 p0 = *reinterpret_cast<const float4 *>(pp), p1 = *reinterpret_cast<const float4 *>(pp + 4);
-            const pi_h8 pa = pi_h8{(_Float16)p0.x, (_Float16)p0.y, (_Float16)p0.z, (_Float16)p0.w, (_Float16)p1.x, (_Float16)p1.y, (_Float16)p1.z, (_Float16)p1.w};
+        };
 #pragma unroll
-            for (int dt = 0; dt < HD / 16; ++dt) {
-                const pi_u32x4 b = *reinterpret_cast<const pi_u32x4 *>(myvt + ((size_t)(dt * 16 + i) * kAcVtStride + 8 * g) * 2);
-                acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(pi_h8, b), acc[dt], 0, 0, 0);
+        for (int u = 0; u < D3; ++u) issue(vq[u], wave + u * kWavesPerBlock);
+        for (int kt0 = wave; kt0 < n_t32; kt0 += D3 * kWavesPerBlock) {
+#pragma unroll
+            for (int u = 0; u < D3; ++u) {
+                const int kt = kt0 + u * kWavesPerBlock;
+                if (kt < n_t32) {
+                    const int c0 = kt * 32;
+#pragma unroll
+                    for (int rnd = 0; rnd < 4 / GPI; ++rnd) {
+                        const int grp8 = rnd * GPI + sub;   // which eight cells of the tile
+                        unsigned v[8];
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) v[k] = c0 + grp8 * 8 + k < n_kv ? vq[u][rnd][k] : 0u;
+                        pi_u32x4 lo, hi;
+                        lo.x = __builtin_amdgcn_perm(v[1], v[0], 0x05040100u); hi.x = __builtin_amdgcn_perm(v[1], v[0], 0x07060302u);
+                        lo.y = __builtin_amdgcn_perm(v[3], v[2], 0x05040100u); hi.y = __builtin_amdgcn_perm(v[3], v[2], 0x07060302u);
+                        lo.z = __builtin_amdgcn_perm(v[5], v[4], 0x05040100u); hi.z = __builtin_amdgcn_perm(v[5], v[4], 0x07060302u);
+                        lo.w = __builtin_amdgcn_perm(v[7], v[6], 0x05040100u); hi.w = __builtin_amdgcn_perm(v[7], v[6], 0x07060302u);
+                        *reinterpret_cast<pi_u32x4 *>(myvt + ((size_t)(2 * dp) * kAcVtStride + grp8 * 8) * 2) = lo;
+                        *reinterpret_cast<pi_u32x4 *>(myvt + ((size_t)(2 * dp + 1) * kAcVtStride + grp8 * 8) * 2) = hi;
+                    }
+                    const float * pp = s + (size_t)i * s_stride + c0 + 8 * g;
+                    const float4 p0 = *reinterpret_cast<const float4 *>(pp), p1 = *reinterpret_cast<const float4 *>(pp + 4);
+                    const pi_h8 pa = pi_h8{(_Float16)p0.x, (_Float16)p0.y, (_Float16)p0.z, (_Float16)p0.w, (_Float16)p1.x, (_Float16)p1.y, (_Float16)p1.z, (_Float16)p1.w};
+#pragma unroll
+                    for (int dt = 0; dt < HD / 16; ++dt) {
+                        const pi_u32x4 b = *reinterpret_cast<const pi_u32x4 *>(myvt + ((size_t)(dt * 16 + i) * kAcVtStride + 8 * g) * 2);
+                        acc[dt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(pa, __builtin_bit_cast(pi_h8, b), acc[dt], 0, 0, 0);
+                    }
+                }
+                issue(vq[u], kt + D3 * kWavesPerBlock);
             }
         }
     }

@@ -137,6 +137,16 @@ void finish_out(ggml_tensor * t, void * dptr) {
     }
 }
 
+// hipBLASLt plans for mat-muls of long token batches (the reference's cuBLAS calls, ggml-cuda.cu:7662-7756); kept until the process ends
+pi_gemm_lib * g_gemm = nullptr;
+pi_gemm_lib * gemm_lib() {
+    if (!g_gemm) {
+        g_gemm = pi_gemm_lib_create((size_t)32 << 20);
+        if (!g_gemm) die("pi_gemm_lib_create");
+    }
+    return g_gemm;
+}
+
 pi_workspace * workspace(int ff, int d) {
     if (!g_ws || ff > g_ws_ff || d > g_ws_d) {
         if (g_ws) { pi_sync(); pi_workspace_destroy(g_ws); }
@@ -291,6 +301,14 @@ bool op_mul_mat(ggml_tensor * dst) {
     const char * wa = (const char *)dev_in(a, tmp); const char * xb = (const char *)dev_in(b, tmp); float * y = (float *)dev_out(dst, tmp);
     if (weight_like) {
         const int64_t T = nrows(b);
+        if (T > 32 && a->type == GGML_TYPE_F16 && T * a->ne[0] < ((int64_t)1 << 28)) {     // a prompt batch: one library mat-mul over all its tokens
+            const int cols = (int)a->ne[0], rows = (int)a->ne[1];
+            __half * xn16 = (__half *)tmp.get(sizeof(__half) * (size_t)T * cols);
+            BK_PI(pi_k_norm_round_f16((const float *)xb, (int)T, cols, nullptr, xn16, nullptr, nullptr));
+            BK_PI(pi_gemm_lib_f16(gemm_lib(), wa, rows, cols, xn16, (int)T, PI_EPI_NONE, nullptr, nullptr, y, nullptr, nullptr));
+            finish_out(dst, y);
+            return true;
+        }
         if (T > 1 && a->type == GGML_TYPE_F16 && a->ne[0] % 128 == 0) {          // the matrix is read once per 16 tokens (matrix cores)
             const int cols = (int)a->ne[0], rows = (int)a->ne[1];
             __half * xn16 = (__half *)tmp.get(sizeof(__half) * 16 * (size_t)cols);

@@ -77,6 +77,25 @@ def test_dense_mul_mat_two_tokens_and_get_rows(golden, wtype):
     assert np.array_equal(G.host(emb), table[ids])
 
 
+@pytest.mark.parametrize("T", [20, 70])
+def test_dense_mul_mat_of_a_prompt_batch(T):
+    """MUL_MAT with a batch of prompt tokens at the boundary (the reference's cuBLAS leg, ggml-cuda.cu:7662-7756): 20 tokens go
+    through this library's 16-token mat-mul kernel, 70 through one library mat-mul over all of them; both against the
+    reference's CPU mat-mul (activations rounded to fp16, ggml.c:9598-9807) as the oracle restates it."""
+    rng = np.random.default_rng(T)
+    rows, cols = 1000, 1024
+    w = (rng.standard_normal((rows, cols)) * 0.02).astype(np.float16)
+    x = rng.standard_normal((T, cols)).astype(np.float32)
+    want = np.zeros((T, rows), np.float32)
+    assert ol.oracle().pio_mul_mat(ol.F16, P(w), rows, cols, P(x), T, P(want), 4) == 0
+    G = graph()
+    tw = G.weight_to_gpu(G.new(F16, [cols, rows], w, "w"))
+    y = G.on_gpu(G.mul_mat(tw, G.new(F32, [cols, T], x, "x")))
+    G.compute()
+    assert not G.cpu_run
+    assert rel_err(G.host(y), want) < 1e-5
+
+
 def test_kv_store_and_attention_core_as_the_graph_builds_them(golden):
     """llm_build_kv_store (llama.cpp:4383-4418): K rows copied F32 -> F16 into a 1-D cache view, V transposed into a strided view;
     llm_build_kqv (:4764-4850): K . q over a strided 3-D view of the cache against the permuted q, scale, mask add, softmax,

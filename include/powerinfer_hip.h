@@ -265,7 +265,7 @@ PI_API int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float thre
                                  int32_t * union_rows, int32_t * n_union,
                                  pi_workspace * ws, pi_stream_t stream);
 
-/* Prompt chunks of up to 128 tokens (the prompt phase of llama_decode, where the reference goes through cuBLAS and its batch kernels,
+/* Prompt chunks of up to 128 tokens on this library's own mat-mul kernel (the prompt phase of llama_decode, where the reference goes through cuBLAS and its batch kernels,
  * ggml-cuda.cu:7662-7756, 6994-7034): pi_k_gemm_wide_f16 is pi_k_gemm_f16 for T <= 128 (cols % 256 == 0; a weight row is read once per
  * chunk); pi_k_ffn_h_f16 forms h_f16[t][n] = fp16(relu(gate) * up) where !(logits[t][n] < threshold) and 0 elsewhere from dense gate/up
  * products (gate may be NULL: relu(up)); pi_k_transpose_f16 writes out[cols][rows] of an fp16 matrix in[rows][cols] (the down projection
@@ -300,8 +300,11 @@ PI_API int pi_k_batch_sparse_axpy(const void * down_t_f16, int cols, int ff, con
 PI_API int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache,
                                  size_t cache_seq_stride, int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx,
                                  const int32_t * pos, float * out, int out_stride, void * out_f16, pi_stream_t stream);
-/* prompt chunk of ONE sequence: T <= 16 consecutive tokens at positions pos[t]; RoPE + KV store of the whole chunk first, then
- * every token attends to the cells up to its own position (the causal mask of llama.cpp:6506-6531).  q_rot: fp32 [T][n_head*hd]. */
+/* prompt chunk of ONE sequence: T <= 512 consecutive tokens at positions pos[t]; RoPE + KV store of the whole chunk first, then
+ * every token attends to the cells up to its own position (the causal mask of llama.cpp:6506-6531).  q_rot: fp32 [T][n_head*hd].
+ * Head sizes 128 and 64 with 16 * n_ctx floats of scores within 156 KB of LDS (n_ctx up to about 1900) take 16 tokens per
+ * workgroup on the matrix cores; other shapes one token per workgroup.  Same rounding points either way (llm_build_kqv on the
+ * CPU path: fp16 q and K, fp16 in and out of exp, fp16 probabilities). */
 PI_API int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
                            const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache,
                            float * out, int out_stride, void * out_f16, pi_stream_t stream);

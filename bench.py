@@ -261,6 +261,7 @@ def main():
                     help="BASELINE configs index: 1 (default, the reported metric) 7B FP16 all on the GPU; 2 the same shape in "
                          "Q4_0 with the hottest 60 %% of neurons on the GPU and the rest on host threads; 3 ProSparse-LLaMA-2-13B shape FP16, "
                          "16 sequences decoded in lockstep; 4 Falcon-40B shape FP16")
+    ap.add_argument("--rest-on-gpu", action="store_true", help="config 2: the GPU reads the non-resident neurons' rows from pinned host memory itself instead of handing those neurons to host threads")
     ap.add_argument("--hot-frac", type=float, default=None, help="configs 1 and 2: share of each layer's neurons on the GPU (default 1.0 and 0.6)")
     ap.add_argument("--pmc-probe", action="store_true",
                     help="counter-collection aid: run only one section of a 4-layer model a few times plus one "
@@ -295,7 +296,8 @@ def main():
     if args.config == 1:
         hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_ctx, seed=1, hot_frac=1.0 if args.hot_frac is None else args.hot_frac)
     elif args.config == 2:
-        hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_ctx, seed=1, wtype=pl.Q4_0, hot_frac=0.6 if args.hot_frac is None else args.hot_frac)
+        hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_ctx, seed=1, wtype=pl.Q4_0, hot_frac=0.6 if args.hot_frac is None else args.hot_frac,
+                           rest_on_gpu=bool(args.rest_on_gpu))
     elif args.config == 3:
         hp = None
     else:
@@ -330,6 +332,7 @@ def main():
     qkv_bytes = (d + 2 * gqa) * d * wbytes + d * 4 + (d + 2 * gqa) * 4       # weights + activation in + result out
     if hybrid:                                                               # the section timers replay full-GPU layers only
         ms_qkv, n_qkv, ms_ffn, ms_head = float("nan"), 0, float("nan"), float("nan")
+        ms_pf, n_pf, ms_fr = float("nan"), 0, float("nan")
     else:
         ms_qkv, n_qkv = m.time_section(0, 8)
         ms_ffn, _ = m.time_section(1, 8)
@@ -386,8 +389,8 @@ def main():
                    f"{hp.n_layer} layers, random-init FP16 weights, all neurons on the GPU, {args.prompt}-token random prompt, "
                    "greedy decode at batch 1",
                 2: "configs[2]: ReLU-LLaMA-2-7B shape, random-init weights quantised to Q4_0 (predictors FP16), per layer the hottest "
-                   f"60 % of neurons on the GPU and the rest on host threads, {hp.n_layer} layers, {args.prompt}-token random prompt, "
-                   "greedy decode at batch 1",
+                   f"60 % of neurons on the GPU and the rest " + ("in pinned host memory, their active rows read by the GPU itself" if hp.get("rest_on_gpu") else "on host threads")
+                   + f", {hp.n_layer} layers, {args.prompt}-token random prompt, greedy decode at batch 1",
                 4: "configs[4]: ReLU-Falcon-40B shape (d 8192, ff 32768 up/down only, 128 heads / 8 KV heads, vocab 65024, predictor "
                    f"rank 1024), {hp.n_layer} layers, random-init FP16 weights, all neurons on the GPU, {args.prompt}-token random "
                    "prompt, greedy decode at batch 1"}[args.config],
@@ -449,6 +452,31 @@ def main():
         }
     m.close()
     del keep
+    if args.config == 2 and hybrid and not hp.get("rest_on_gpu"):
+        # the same split with the non-resident rows in pinned host memory and the GPU reading the active ones itself: no host
+        # threads in the loop, one graph replay per token; same model, prompt and steps, tokens compared with the run above
+        try:
+            hp2 = synth.HParams(hp)
+            hp2["rest_on_gpu"] = True
+            keep2 = []
+            m2 = build_synthetic_on_device(hp2, keep2)
+            m2.decode(prompt, 0, want_logits=False)
+            if args.warmup > 0:
+                m2.generate(args.warmup)
+            pl.sync()
+            t0 = time.perf_counter()
+            toks2, _ = m2.generate(args.steps)
+            pl.sync()
+            dt = time.perf_counter() - t0
+            out["rest_read_by_gpu"] = {"value": round(args.steps / dt, 2), "unit": "tok/s", "ms_per_step": round(dt * 1e3 / args.steps, 4),
+                                       "tokens_identical_to_host_threads": bool(np.array_equal(np.asarray(toks), np.asarray(toks2))),
+                                       "what": "same 60 % split: the non-resident 40 % of each layer's rows stay in pinned host memory, the kernels that "
+                                               "compute the resident neurons also read the rows of active non-resident neurons over the host link "
+                                               "(pi_model_set_rest_on_gpu), one HIP graph replay per token"}
+            m2.close()
+            del keep2
+        except Exception as e:
+            out["rest_read_by_gpu"] = {"error": repr(e)[:200]}
     if args.prompt_bench > 0 and not hybrid and hp.wtype == pl.F16:
         # prompt phase on its own: a fresh instance of the same model with room for the prompt, one untimed pass (allocations, the
         # transposed down projections, the library's mat-mul plans), then the timed pass from an empty cache; chunks of up to 512 tokens

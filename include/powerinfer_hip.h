@@ -182,6 +182,19 @@ PI_API int pi_k_axpy_q4_partials(const void * down_t_q4, int cols, int ff, const
                                  const uint32_t * hot_words, const int32_t * hot_prefix, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_axpy_q4_reduce(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out,
                                int32_t * n_active, pi_workspace * ws, pi_stream_t stream);
+/* The same two launches when the GPU computes the neurons outside the hot set as well, reading their rows where they lie: up_rest /
+ * gate_rest / down_t_rest hold exactly the non-resident neurons' rows in ascending neuron order (row = neuron index minus the
+ * resident neurons before it) and may be pinned host memory - only the rows of active neurons cross the host link.  The split
+ * of llama.cpp:2820-2967 (hot rows in VRAM, the rest in host memory) is kept; what moves is who multiplies the cold rows
+ * (the CPU half of llm_build_sparse_mul_mat / llm_build_sparse_axpy, llama.cpp:4581-4593, 4635-4646).  h_dense then holds h of
+ * every active neuron.  *_rest == NULL: identical to the calls above. */
+PI_API int pi_k_pred_upgate_q4_split(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                                     const void * up_q4, const void * gate_q4, const void * up_rest_q4, const void * gate_rest_q4,
+                                     int cols, const float * x, const pi_norm * norm,
+                                     const uint32_t * hot_words, const int32_t * hot_prefix,
+                                     float * logits, float * h_dense, void * xq8_out, pi_workspace * ws, pi_stream_t stream);
+PI_API int pi_k_axpy_q4_partials_split(const void * down_t_q4, const void * down_t_rest_q4, int cols, int ff, const float * h,
+                                       const uint32_t * hot_words, const int32_t * hot_prefix, pi_workspace * ws, pi_stream_t stream);
 /* KV cache maintenance.  pi_k_k_shift replaces the graph of llm_build_k_shift (llama.cpp:4332-4381; the fp16 RoPE
  * ggml.c:11327-11478): cache [rows = layers x kv heads][n_ctx][hd] fp16, delta[n_cells] positions to rotate each cell by.
  * pi_k_kv_compact moves cell map[j] to cell j (map ascending) through `stage` ([rows][n_new][hd] fp16): this implementation keeps
@@ -443,6 +456,10 @@ PI_API int pi_model_batch_kv_seq_shift(pi_model * m, int seq, int p0, int p1, in
 PI_API int pi_model_batch_kv_seq_cp(pi_model * m, int src, int dst, int p0, int p1);
 PI_API int pi_model_batch_union(pi_model * m, int32_t * n_union_per_layer);   /* union sizes of the last step, [n_layer] */
 
+/* Before pi_model_finalize: layers with a gpu_bucket keep their non-resident rows in pinned host memory and the GPU reads the
+ * rows of active neurons from there itself (pi_k_pred_upgate_q4_split) instead of handing those neurons to host threads; the
+ * token loop then needs no host step and replays as a HIP graph.  Q4_0 layers at n_embd 4096; the VRAM split is unchanged. */
+PI_API int pi_model_set_rest_on_gpu(pi_model * m, int enable);
 PI_API int pi_model_set_capture(pi_model * m, int enable);
 PI_API int pi_model_get_capture(pi_model * m, float * ffn_out, float * pred_logits, int32_t * n_active, float * ffn_src);
 

@@ -228,12 +228,16 @@ int layer_forward(pi_model * m, int il, bool last_token) {
         // plus one reduction; a hybrid layer's host share works between the two from the buffers the first kernel fills
         const void * gp = falcon ? nullptr : gate.dev;
         const bool cap = m->capture && last_token;
-        if (layer_hybrid) {
+        if (layer_hybrid && !m->rest_on_gpu) {
             PI_TRY(pi::cold_layer_q4(m->cold, il, m, st, cap));
         } else {
-            PI_TRY(pi_k_pred_upgate_q4(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, gp, d, ffn_in, &fn, nullptr, nullptr,
-                                       m->pred_logits, m->h_dense, nullptr, m->ws, st));
-            PI_TRY(pi_k_axpy_q4_partials(down.dev, d, ff, m->h_dense, nullptr, nullptr, m->ws, st));
+            // every neuron on the GPU, or the non-resident neurons' rows read from pinned host memory by the same two launches
+            const uint32_t * hw = layer_hybrid ? m->hot_words[il] : nullptr;
+            const int32_t * hpx = layer_hybrid ? m->hot_prefix[il] : nullptr;
+            PI_TRY(pi_k_pred_upgate_q4_split(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, gp,
+                                             layer_hybrid ? m->rest_up[il] : nullptr, (layer_hybrid && !falcon) ? m->rest_gate[il] : nullptr,
+                                             d, ffn_in, &fn, hw, hpx, m->pred_logits, m->h_dense, nullptr, m->ws, st));
+            PI_TRY(pi_k_axpy_q4_partials_split(down.dev, layer_hybrid ? m->rest_down[il] : nullptr, d, ff, m->h_dense, hw, hpx, m->ws, st));
             if (cap) {
                 float * ffo = m->cap_ffn + (size_t)il * d;
                 PI_TRY(pi_k_axpy_q4_reduce(ff, d, PI_EPI_NONE, nullptr, nullptr, ffo, n_act, m->ws, st));
@@ -427,6 +431,7 @@ void pi_model_free(pi_model * m) {
     pi::batch_destroy(m);
     if (m->ws) pi_workspace_destroy(m->ws);
     for (void * p : m->owned) pi_free(p);
+    for (void * p : m->pinned) (void)hipHostFree(p);
     if (m->stream) (void)hipStreamDestroy(m->stream);
     delete m;
 }
@@ -559,6 +564,33 @@ int pi_model_finalize(pi_model * m) {
         }
     }
 
+    // non-resident rows the GPU is to read itself: gathered in ascending neuron order into pinned host memory
+    m->rest_up.assign(hp.n_layer, nullptr); m->rest_gate.assign(hp.n_layer, nullptr); m->rest_down.assign(hp.n_layer, nullptr);
+    if (m->hybrid && m->rest_on_gpu) {
+        for (int il = 0; il < hp.n_layer; ++il) {
+            Tensor & bucket = m->L(il, PI_T_GPU_BUCKET);
+            if (!bucket.dev) continue;
+            Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & fc1 = m->L(il, PI_T_FC1);
+            if (up.type != PI_TYPE_Q4_0 || !m->hot_words[il] || !pi_k_pred_upgate_q4_supported(ff, (int)fc1.ne1, d))
+                return pi::fail(PI_E_UNSUPPORTED, "pi_model_finalize: rest_on_gpu covers Q4_0 layers at n_embd 4096 with a predictor of rank 512 or 1024 and n_ff % 32 == 0");
+            const int32_t * gi = (const int32_t *)m->L(il, PI_T_GPU_IDX).host;
+            std::vector<int> rest;
+            for (int j = 0; j < ff; ++j) if (gi[j] != 1) rest.push_back(j);
+            if ((int)rest.size() + (int)bucket.ne0 != ff) return pi::fail(PI_E_ARG, "pi_model_finalize: gpu_idx and gpu_bucket disagree");
+            const size_t rb = row_bytes(up.type, d);
+            for (int k : {PI_T_FFN_UP, PI_T_FFN_GATE, PI_T_FFN_DOWN_T}) {
+                if (k == PI_T_FFN_GATE && hp.arch == PI_ARCH_FALCON) continue;
+                Tensor & t = m->L(il, k);
+                if (!t.host) return pi::fail(PI_E_STATE, "pi_model_finalize: rest_on_gpu needs the host copy of the FFN matrices");
+                void * pin = nullptr;
+                PI_HIP_TRY(hipHostMalloc(&pin, rb * (rest.empty() ? 1 : rest.size()), hipHostMallocDefault));
+                m->pinned.push_back(pin);
+                for (size_t i = 0; i < rest.size(); ++i) memcpy((unsigned char *)pin + rb * i, (const unsigned char *)t.host + rb * (size_t)rest[i], rb);
+                (k == PI_T_FFN_UP ? m->rest_up : k == PI_T_FFN_GATE ? m->rest_gate : m->rest_down)[il] = pin;
+            }
+        }
+    }
+
     m->ws = pi_workspace_create(ff, d);
     if (!m->ws) return PI_E_HIP;
     const size_t kv = (size_t)hp.n_layer * hp.n_head_kv * hp.n_ctx * m->hd;
@@ -589,7 +621,7 @@ int pi_model_finalize(pi_model * m) {
     PI_TRY(pi_memset(m->n_active, 0, sizeof(int32_t) * hp.n_layer));
     PI_TRY(pi_memset(m->d_step, 0, 4));
     PI_TRY(pi_memset(m->h_dense, 0, sizeof(float) * ff));
-    if (m->hybrid) {
+    if (m->hybrid && !m->rest_on_gpu) {
         m->cold = pi::cold_create(m);
         if (!m->cold) return PI_E_STATE;
     }
@@ -672,7 +704,7 @@ int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * m
 
     // PI_NO_GRAPH=1 issues the same launches eagerly (useful under tracing tools that cannot follow graph replays)
     const char * no_graph = getenv("PI_NO_GRAPH");
-    const bool use_graph = !m->hybrid && !m->capture && !(no_graph && no_graph[0] == '1');
+    const bool use_graph = !(m->hybrid && !m->rest_on_gpu) && !m->capture && !(no_graph && no_graph[0] == '1');
     if (use_graph && !m->graph_exec) {
         PI_HIP_TRY(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
         int rc = token_forward(m, true, false);
@@ -779,6 +811,13 @@ int pi_model_time_section(pi_model * m, int section, int rounds, float * ms_tota
     PI_HIP_TRY(hipStreamSynchronize(st));
     PI_HIP_TRY(hipEventElapsedTime(ms_total, m->ev0, m->ev1));
     *launches = n;
+    return PI_OK;
+}
+
+int pi_model_set_rest_on_gpu(pi_model * m, int enable) {
+    if (!m) return pi::fail(PI_E_ARG, "pi_model_set_rest_on_gpu: null model");
+    if (m->finalized) return pi::fail(PI_E_STATE, "pi_model_set_rest_on_gpu: call before pi_model_finalize");
+    m->rest_on_gpu = enable != 0;
     return PI_OK;
 }
 

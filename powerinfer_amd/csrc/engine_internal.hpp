@@ -52,6 +52,11 @@ struct pi_model {
     int32_t * kv_map = nullptr;           // [n_ctx] device copy of the cell map / deltas of an edit
     std::vector<uint32_t *> hot_words;    // per hybrid layer: bit j of word g set iff neuron 32g+j is GPU-resident (device)
     std::vector<int32_t *> hot_prefix;    //                   GPU-resident neurons before group g = row of the compact matrices
+    // hybrid layers whose non-resident rows the GPU reads from pinned host memory itself (pi_model_set_rest_on_gpu): per layer
+    // the up / gate / down rows of the non-resident neurons in ascending order; no host threads, the token loop replays as a graph
+    bool rest_on_gpu = false;
+    std::vector<void *> rest_up, rest_gate, rest_down;
+    std::vector<void *> pinned;           // hipHostMalloc allocations owned by the model
     BatchState * batch = nullptr;         // per-sequence caches and step buffers of batched decoding
     BatchState * prefill = nullptr;       // step buffers for prompt chunks of the model's own sequence
     BatchState * prefill_wide = nullptr;  // the same for chunks of up to 512 tokens (dense mat-muls, weights read once per chunk)

@@ -1279,9 +1279,12 @@ __global__ __launch_bounds__(kPfBlock) void ffn_reduce_kernel(const float * __re
 // ---------------------------------------------------------------------------------------------------
 struct __attribute__((packed)) pi_q8_host_block { uint16_t d; int8_t qs[32]; };
 
-template <int RCH, bool GATE>
+// SPLIT: the neurons outside the hot words are computed here too, from a second pair of matrices that holds exactly those
+// neurons' rows in ascending order (rows in pinned host memory, fetched over the host link by the loads below).
+template <int RCH, bool GATE, bool SPLIT>
 __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
                                                                      const pi_block_q4_0 * __restrict__ Wup, const pi_block_q4_0 * __restrict__ Wgate,
+                                                                     const pi_block_q4_0 * __restrict__ Wup_rest, const pi_block_q4_0 * __restrict__ Wgate_rest,
                                                                      const float * __restrict__ x, NormArgs na, float thr,
                                                                      const uint32_t * __restrict__ hot_words, const int32_t * __restrict__ hot_prefix,
                                                                      float * __restrict__ logits, uint32_t * __restrict__ words, uint32_t * __restrict__ words_hot,
@@ -1411,7 +1414,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
     const float my_logit = lg[lane & 31];
     const bool my_act = !(my_logit < thr);
     const uint32_t mask = (uint32_t)__ballot(my_act);
-    const uint32_t sel = mask & hot;
+    const uint32_t sel = SPLIT ? mask : mask & hot;
     if (wave == 0) {
         if (lane < 32) { if (logits) logits[n0 + lane] = my_logit; if (!((sel >> lane) & 1u)) h_dense[n0 + lane] = 0.0f; }
         if (lane == 0) { words[blockIdx.x] = mask; if (words_hot) words_hot[blockIdx.x] = sel; }
@@ -1429,12 +1432,14 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
             if (j < nn) {
                 const int bit = select_nth_bit(sel, c0 + j);
                 nrn[j] = n0 + bit;
-                const size_t row = (size_t)(base_row + __popc(hot & ((1u << bit) - 1u)));
-                const pi_block_q4_0 * wu = Wup + row * nb + blk;
+                const int below = __popc(hot & ((1u << bit) - 1u));
+                const bool rest = SPLIT && !((hot >> bit) & 1u);      // n0 - base_row neurons outside the hot set lie before this group
+                const size_t row = rest ? (size_t)(n0 - base_row + bit - below) : (size_t)(base_row + below);
+                const pi_block_q4_0 * wu = (rest ? Wup_rest : Wup) + row * nb + blk;
                 __builtin_memcpy(&du[j], &wu->d, 2);
                 __builtin_memcpy(qu[j], wu->qs + qoff, 8);
                 if (GATE) {
-                    const pi_block_q4_0 * wg = Wgate + row * nb + blk;
+                    const pi_block_q4_0 * wg = (rest ? Wgate_rest : Wgate) + row * nb + blk;
                     __builtin_memcpy(&dg[j], &wg->d, 2);
                     __builtin_memcpy(qg[j], wg->qs + qoff, 8);
                 }
@@ -1486,7 +1491,11 @@ constexpr int kAqGroups = 4;
 constexpr int kAqN = kAqGroups * 32;       // neurons per workgroup
 constexpr int kAqChunk = 16;               // rows in flight per wave
 
-__global__ __launch_bounds__(kPfBlock, 2) void axpy_q4_groups_kernel(const pi_block_q4_0 * __restrict__ Wd, const float * h, int ff,
+// SPLIT: rows of the neurons outside the hot words come from Wd_rest (those neurons' rows in ascending order, pinned host memory).
+constexpr int kAqRestFlag = 1 << 30;
+template <bool SPLIT>
+__global__ __launch_bounds__(kPfBlock, 2) void axpy_q4_groups_kernel(const pi_block_q4_0 * __restrict__ Wd, const pi_block_q4_0 * __restrict__ Wd_rest,
+                                                                     const float * h, int ff,
                                                                      const uint32_t * __restrict__ hot_words, const int32_t * __restrict__ hot_prefix,
                                                                      float * __restrict__ partial) {
     constexpr int cols = 4096, nb = cols / 32;
@@ -1510,11 +1519,13 @@ __global__ __launch_bounds__(kPfBlock, 2) void axpy_q4_groups_kernel(const pi_bl
             const int q = (int)rintf(__fmul_rn(hvv, id));
             const int g = nrn >> 5;
             const uint32_t hot = (nrn < ff) ? (hot_words ? hot_words[g] : 0xFFFFFFFFu) : 0u;
-            const bool take = q != 0 && ((hot >> (lane & 31)) & 1u);
+            const bool is_hot = (hot >> (lane & 31)) & 1u;
+            const bool take = q != 0 && (is_hot || (SPLIT && nrn < ff));
             const unsigned long long b = __ballot(take);
             if (take) {
                 const int pos = cnt + __popcll(b & ((1ull << lane) - 1ull));
-                lrow[pos] = (hot_prefix ? hot_prefix[g] : (nrn & ~31)) + __popc(hot & ((1u << (lane & 31)) - 1u));
+                const int base = hot_prefix ? hot_prefix[g] : (nrn & ~31), below = __popc(hot & ((1u << (lane & 31)) - 1u));
+                lrow[pos] = is_hot ? base + below : (((nrn & ~31) - base + (lane & 31) - below) | kAqRestFlag);
                 lq[pos] = q;
                 ld[pos] = pi_round_f16(d);
             }
@@ -1534,7 +1545,8 @@ __global__ __launch_bounds__(kPfBlock, 2) void axpy_q4_groups_kernel(const pi_bl
 #pragma unroll
         for (int j = 0; j < kAqChunk; ++j) {
             if (k0 + j < n) {
-                const pi_block_q4_0 * wb = Wd + (size_t)lrow[k0 + j] * nb + blk;
+                const int lr = lrow[k0 + j];
+                const pi_block_q4_0 * wb = ((SPLIT && (lr & kAqRestFlag)) ? Wd_rest + (size_t)(lr & ~kAqRestFlag) * nb : Wd + (size_t)lr * nb) + blk;
                 __builtin_memcpy(&dw[j], &wb->d, 2);
                 __builtin_memcpy(q[j], wb->qs + qoff, 8);
             }
@@ -3655,7 +3667,18 @@ int pi_k_pred_upgate_q4(const void * fc2_f16, int ff, int r, const float * hidde
                         const void * up_q4, const void * gate_q4, int cols, const float * x, const pi_norm * norm,
                         const uint32_t * hot_words, const int32_t * hot_prefix,
                         float * logits, float * h_dense, void * xq8_out, pi_workspace * ws, pi_stream_t stream) {
+    return pi_k_pred_upgate_q4_split(fc2_f16, ff, r, hidden, threshold, up_q4, gate_q4, nullptr, nullptr, cols, x, norm, hot_words, hot_prefix,
+                                     logits, h_dense, xq8_out, ws, stream);
+}
+
+int pi_k_pred_upgate_q4_split(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                              const void * up_q4, const void * gate_q4, const void * up_rest_q4, const void * gate_rest_q4,
+                              int cols, const float * x, const pi_norm * norm,
+                              const uint32_t * hot_words, const int32_t * hot_prefix,
+                              float * logits, float * h_dense, void * xq8_out, pi_workspace * ws, pi_stream_t stream) {
     if (!fc2_f16 || !hidden || !up_q4 || !x || !h_dense || !ws) return pi::fail(PI_E_ARG, "pi_k_pred_upgate_q4: null pointer");
+    if (up_rest_q4 && (!hot_words || (gate_q4 != nullptr) != (gate_rest_q4 != nullptr)))
+        return pi::fail(PI_E_ARG, "pi_k_pred_upgate_q4_split: the second matrices need hot_words / hot_prefix and a gate on both sides or on neither");
     if (!pi_k_pred_upgate_q4_supported(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_pred_upgate_q4: shape outside the fused kernel (cols 4096, r 512 or 1024, ff % 32 == 0)");
     if (ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_ARG, "pi_k_pred_upgate_q4: shape exceeds the workspace");
     if ((hot_words == nullptr) != (hot_prefix == nullptr)) return pi::fail(PI_E_ARG, "pi_k_pred_upgate_q4: hot_words and hot_prefix go together");
@@ -3665,20 +3688,33 @@ int pi_k_pred_upgate_q4(const void * fc2_f16, int ff, int r, const float * hidde
     const __half * w2 = (const __half *)fc2_f16;
     const pi_block_q4_0 * u = (const pi_block_q4_0 *)up_q4; const pi_block_q4_0 * g = (const pi_block_q4_0 *)gate_q4;
     const dim3 grid(ff / 32), block(kPfBlock);
-#define PI_PQ_LAUNCH(RCH, GATE) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, GATE>), grid, block, 0, st, w2, hidden, u, g, x, na, threshold, hot_words, hot_prefix, logits, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)xq8_out)
-    if (r == 1024) { if (g) PI_PQ_LAUNCH(2, true); else PI_PQ_LAUNCH(2, false); }
-    else           { if (g) PI_PQ_LAUNCH(1, true); else PI_PQ_LAUNCH(1, false); }
+    const pi_block_q4_0 * ur = (const pi_block_q4_0 *)up_rest_q4; const pi_block_q4_0 * gr = (const pi_block_q4_0 *)gate_rest_q4;
+#define PI_PQ_LAUNCH(RCH, GATE, SPLIT) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, GATE, SPLIT>), grid, block, 0, st, w2, hidden, u, g, ur, gr, x, na, threshold, hot_words, hot_prefix, logits, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)xq8_out)
+#define PI_PQ_LAUNCH_S(RCH, GATE) do { if (ur) PI_PQ_LAUNCH(RCH, GATE, true); else PI_PQ_LAUNCH(RCH, GATE, false); } while (0)
+    if (r == 1024) { if (g) PI_PQ_LAUNCH_S(2, true); else PI_PQ_LAUNCH_S(2, false); }
+    else           { if (g) PI_PQ_LAUNCH_S(1, true); else PI_PQ_LAUNCH_S(1, false); }
+#undef PI_PQ_LAUNCH_S
 #undef PI_PQ_LAUNCH
     return pi::check_launch("pi_k_pred_upgate_q4");
 }
 
 int pi_k_axpy_q4_partials(const void * down_t_q4, int cols, int ff, const float * h, const uint32_t * hot_words, const int32_t * hot_prefix,
                           pi_workspace * ws, pi_stream_t stream) {
+    return pi_k_axpy_q4_partials_split(down_t_q4, nullptr, cols, ff, h, hot_words, hot_prefix, ws, stream);
+}
+
+int pi_k_axpy_q4_partials_split(const void * down_t_q4, const void * down_t_rest_q4, int cols, int ff, const float * h,
+                                const uint32_t * hot_words, const int32_t * hot_prefix, pi_workspace * ws, pi_stream_t stream) {
     if (!down_t_q4 || !h || !ws) return pi::fail(PI_E_ARG, "pi_k_axpy_q4_partials: null pointer");
+    if (down_t_rest_q4 && !hot_words) return pi::fail(PI_E_ARG, "pi_k_axpy_q4_partials_split: the second matrix needs hot_words / hot_prefix");
     if (cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_UNSUPPORTED, "pi_k_axpy_q4_partials: cols must be 4096, ff % 32 == 0, within the workspace");
     if ((hot_words == nullptr) != (hot_prefix == nullptr)) return pi::fail(PI_E_ARG, "pi_k_axpy_q4_partials: hot_words and hot_prefix go together");
-    hipLaunchKernelGGL(axpy_q4_groups_kernel, dim3((ff + kAqN - 1) / kAqN), dim3(kPfBlock), 0, (hipStream_t)stream,
-                       (const pi_block_q4_0 *)down_t_q4, h, ff, hot_words, hot_prefix, ws->ffn_partial);
+    if (down_t_rest_q4)
+        hipLaunchKernelGGL(axpy_q4_groups_kernel<true>, dim3((ff + kAqN - 1) / kAqN), dim3(kPfBlock), 0, (hipStream_t)stream,
+                           (const pi_block_q4_0 *)down_t_q4, (const pi_block_q4_0 *)down_t_rest_q4, h, ff, hot_words, hot_prefix, ws->ffn_partial);
+    else
+        hipLaunchKernelGGL(axpy_q4_groups_kernel<false>, dim3((ff + kAqN - 1) / kAqN), dim3(kPfBlock), 0, (hipStream_t)stream,
+                           (const pi_block_q4_0 *)down_t_q4, (const pi_block_q4_0 *)nullptr, h, ff, hot_words, hot_prefix, ws->ffn_partial);
     return pi::check_launch("pi_k_axpy_q4_partials");
 }
 

@@ -61,6 +61,8 @@ _SIGS = {
     "pi_k_pred_upgate_q4_supported": (_i, [_i, _i, _i]),
     "pi_k_pred_upgate_q4": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_axpy_q4_partials": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_pred_upgate_q4_split": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_axpy_q4_partials_split": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_axpy_q4_reduce": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_k_shift": (_i, [_vp, _i, _i, _i, _i, _f, _vp, _i, _vp]),
     "pi_k_kv_compact": (_i, [_vp, _vp, _i, _i, _i, _vp, _i, _vp]),

@@ -36,6 +36,7 @@ def _declare(L):
     L.pi_model_decode.restype, L.pi_model_decode.argtypes = i, [vp, vp, i, i, vp]
     L.pi_model_generate.restype, L.pi_model_generate.argtypes = i, [vp, i, vp, C.POINTER(C.c_float)]
     L.pi_model_set_capture.restype, L.pi_model_set_capture.argtypes = i, [vp, i]
+    L.pi_model_set_rest_on_gpu.restype, L.pi_model_set_rest_on_gpu.argtypes = i, [vp, i]
     L.pi_model_get_capture.restype, L.pi_model_get_capture.argtypes = i, [vp, vp, vp, vp, vp]
     L.pi_model_step_active.restype, L.pi_model_step_active.argtypes = i, [vp, vp, i]
     L.pi_model_batch_init.restype, L.pi_model_batch_init.argtypes = i, [vp, i]
@@ -50,7 +51,7 @@ def _declare(L):
 
 ENGINE_SYMBOLS = ["pi_model_create", "pi_model_free", "pi_model_set_tensor", "pi_model_finalize", "pi_model_kv_clear",
                   "pi_model_kv_seq_rm", "pi_model_kv_seq_shift",
-                  "pi_model_decode", "pi_model_generate", "pi_model_set_capture", "pi_model_get_capture",
+                  "pi_model_decode", "pi_model_generate", "pi_model_set_capture", "pi_model_get_capture", "pi_model_set_rest_on_gpu",
                   "pi_model_step_active", "pi_model_time_section",
                   "pi_model_batch_init", "pi_model_batch_decode", "pi_model_batch_generate", "pi_model_batch_union",
                   "pi_model_batch_kv_seq_rm", "pi_model_batch_kv_seq_shift", "pi_model_batch_kv_seq_cp"]
@@ -85,6 +86,8 @@ class Model:
         self.h = self.L.pi_model_create(C.byref(c))
         if not self.h:
             raise pl.PiError("pi_model_create: " + self.L.pi_last_error().decode())
+        if hp.get("rest_on_gpu"):      # non-resident rows stay in pinned host memory and the GPU reads the active ones itself
+            check(self.L.pi_model_set_rest_on_gpu(self.h, 1), "set_rest_on_gpu")
         self._keep = []        # host arrays the engine borrows (hybrid layers)
         self.n_seq = 0         # sequences of batched decoding (batch_init)
 

@@ -310,6 +310,38 @@ def test_llama_7b_width_q4_two_layers(hot_frac):
     run_case(hp, n_prompt=6, n_gen=24, logit_tol=1.5e-1, min_same=0.5)
 
 
+@pytest.mark.timeout(300)
+def test_north_star_q4_split_rest_read_by_the_gpu():
+    """configs[2]'s split with the non-resident 40 % of each layer's rows in pinned host memory and the GPU reading the rows of
+    active neurons from there itself (pi_model_set_rest_on_gpu): same VRAM split, no host threads, the token loop is a graph
+    replay.  Same assertions as the host-thread variant."""
+    run_north_star(synth.hparams("llama-7b", n_layer=2, n_ctx=96, seed=SEED_7B_Q4, wtype=synth.Q4_0, hot_frac=0.6, rest_on_gpu=True, **NS))
+
+
+def test_q4_split_rest_read_by_the_gpu_matches_host_threads():
+    """The two ways of computing the non-resident neurons run the same arithmetic in the same order, so on one model and one
+    prompt their logits are bit-identical; and F16 layers, which the variant does not cover, are refused at finalize."""
+    from powerinfer_amd import lib as pl
+    from powerinfer_amd.model import Model
+    hp = synth.hparams("llama-7b", n_layer=2, n_ctx=64, seed=12, wtype=synth.Q4_0, hot_frac=0.6)
+    model = synth.make_model(hp)
+    prompt = np.random.default_rng(3).integers(0, hp.n_vocab, 6).astype(np.int32)
+    outs = []
+    for rest in (False, True):
+        hp2 = synth.HParams(hp)
+        hp2["rest_on_gpu"] = rest
+        gm = Model(hp2).load(model)
+        tok, lg = gm.decode(prompt, 0)
+        toks, _ = gm.generate(12)
+        outs.append((tok, lg, list(map(int, toks))))
+        gm.close()
+    assert outs[0][0] == outs[1][0] and outs[0][2] == outs[1][2]
+    assert np.array_equal(outs[0][1], outs[1][1])
+    hp3 = synth.hparams("llama-tiny", n_ctx=64, seed=8, hot_frac=0.6, rest_on_gpu=True)
+    with pytest.raises(pl.PiError):
+        Model(hp3).load(synth.make_model(hp3))
+
+
 @pytest.mark.parametrize("arch,wtype", [("llama-tiny", synth.F16), ("llama-tiny", synth.Q4_0), ("falcon-tiny", synth.F16)])
 def test_hybrid_split_matches_all_cold_oracle(arch, wtype):
     """Config-2 style partial split: the hottest 60 % of each layer's neurons live on the GPU (compact matrices +

@@ -477,12 +477,13 @@ def main():
             del keep2
         except Exception as e:
             out["rest_read_by_gpu"] = {"error": repr(e)[:200]}
-    if args.prompt_bench > 0 and not hybrid and hp.wtype == pl.F16:
+    if args.prompt_bench > 0:
         # prompt phase on its own: a fresh instance of the same model with room for the prompt, one untimed pass (allocations, the
         # transposed down projections, the library's mat-mul plans), then the timed pass from an empty cache; chunks of up to 512 tokens
         # per weight pass
         try:
-            hp2 = synth.hparams({1: "llama-7b", 4: "falcon-40b"}[args.config], n_layer=hp.n_layer, n_ctx=args.prompt_bench + 8, seed=1)
+            hp2 = synth.hparams({1: "llama-7b", 2: "llama-7b", 4: "falcon-40b"}[args.config], n_layer=hp.n_layer, n_ctx=args.prompt_bench + 8, seed=1,
+                                wtype=hp.wtype, hot_frac=hp.hot_frac)
             keep2 = []
             m2 = build_synthetic_on_device(hp2, keep2)
             ptoks = rng.integers(0, hp2.n_vocab, args.prompt_bench).astype(np.int32)
@@ -495,7 +496,9 @@ def main():
             dt = time.perf_counter() - t0
             out["prompt_phase"] = {"tokens": args.prompt_bench, "ms": round(dt * 1e3, 2), "tok_per_s": round(args.prompt_bench / dt, 1),
                                    "what": "pi_model_decode of the whole prompt: chunks of up to 512 tokens (dense mat-muls through hipBLASLt plans, each weight "
-                                           "row read once per chunk, predictor mask applied to h), last token through the single-token path"}
+                                           "row read once per chunk, predictor mask applied to h), last token through the single-token path"
+                                           + ("; Q4_0 matrices expanded to fp16 per chunk, activations through Q8_0 blocks" if hp.wtype != pl.F16 else "")
+                                           + ("; non-resident FFN rows read from pinned host memory once per chunk" if hybrid else "")}
             m2.close()
             del keep2
         except Exception as e:

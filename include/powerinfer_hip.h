@@ -288,6 +288,22 @@ PI_API int pi_k_gemm_wide_f16(const void * W_f16, int rows, int cols, const void
 PI_API int pi_k_ffn_h_f16(const float * up, const float * gate, const float * logits, float threshold, int T, int ff, void * h_f16, pi_stream_t stream);
 PI_API int pi_k_transpose_f16(const void * in_f16, int rows, int cols, void * out_f16, pi_stream_t stream);
 
+/* Q4_0 models in prompt chunks.  The CPU path multiplies Q4_0 rows with the Q8_0 form of the activations (ggml_vec_dot_q4_0_q8_0,
+ * ggml-quants.c:2512-2650; the down projection quantises h over blocks of 32 neurons, ggml.c:14465-14618).  The chunk path keeps
+ * those values and only changes the container: pi_k_norm_q8_round_f16 is pi_k_norm_round_f16 with the normalised row passed through
+ * Q8_0 blocks (value q * fp16(amax / 127)) before the fp16 rounding (cols % 32 == 0, cols <= 8192); pi_k_ffn_h_q8_f16 does the same
+ * to h (n_ff % 64 == 0); pi_k_dequant_q4_f16 writes a Q4_0 matrix as fp16 ((q - 8) * d), optionally assembling it from the compact
+ * matrix of the resident neurons and the matrix of the others (hot_words / hot_prefix as for pi_k_pred_upgate_q4_split).  The
+ * products then differ from the CPU path's only by the fp16 rounding of the two factors. */
+PI_API int pi_k_norm_q8_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, void * out_plain_f16, pi_stream_t stream);
+PI_API int pi_k_ffn_h_q8_f16(const float * up, const float * gate, const float * logits, float threshold, int T, int ff, void * h_f16, pi_stream_t stream);
+PI_API int pi_k_dequant_q4_f16(const void * W_q4, const void * W_rest_q4, const uint32_t * hot_words, const int32_t * hot_prefix, int rows, int cols,
+                               void * out_f16, pi_stream_t stream);
+/* the same assembly for an fp16 matrix of a hybrid layer (rows % 32 == 0, cols % 8 == 0), and the embedding rows of a chunk from a Q4_0 table */
+PI_API int pi_k_assemble_rows_f16(const void * W_f16, const void * W_rest_f16, const uint32_t * hot_words, const int32_t * hot_prefix, int rows, int cols,
+                                  void * out_f16, pi_stream_t stream);
+PI_API int pi_k_embed_batch_q4(const void * table_q4, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream);
+
 /* The same mat-mul for prompt chunks of any length through hipBLASLt (fp16 operands, fp32 accumulation and result), where the reference
  * calls cuBLAS (ggml_cuda_op_mul_mat_cublas, ggml-cuda.cu:7662-7756).  Arguments and epilogues as pi_k_gemm_f16; no limit on T or cols.
  * A pi_gemm_lib holds the library handle, its workspace and one plan per distinct (rows, cols, T) - at most 64 of them. */

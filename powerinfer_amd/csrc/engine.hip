@@ -452,6 +452,37 @@ int pi_model_set_tensor(pi_model * m, int layer, int kind, int type, const void 
     return upload_tensor(m, t, type, data, ne0, ne1, on_device);
 }
 
+}  // extern "C"
+
+namespace pi {
+// the up / gate / down rows of layer il's non-resident neurons, in ascending neuron order, in pinned host memory that kernels read directly
+int gather_rest_rows(pi_model * m, int il) {
+    const pi_hparams & hp = m->hp;
+    const int d = hp.n_embd, ff = hp.n_ff;
+    Tensor & bucket = m->L(il, PI_T_GPU_BUCKET);
+    if (!bucket.dev || m->rest_up[il]) return PI_OK;
+    const int32_t * gi = (const int32_t *)m->L(il, PI_T_GPU_IDX).host;
+    if (!gi) return pi::fail(PI_E_STATE, "gather_rest_rows: the layer has no gpu_idx");
+    std::vector<int> rest;
+    for (int j = 0; j < ff; ++j) if (gi[j] != 1) rest.push_back(j);
+    if ((int)rest.size() + (int)bucket.ne0 != ff) return pi::fail(PI_E_ARG, "gather_rest_rows: gpu_idx and gpu_bucket disagree");
+    for (int k : {PI_T_FFN_UP, PI_T_FFN_GATE, PI_T_FFN_DOWN_T}) {
+        if (k == PI_T_FFN_GATE && hp.arch == PI_ARCH_FALCON) continue;
+        Tensor & t = m->L(il, k);
+        if (!t.host) return pi::fail(PI_E_STATE, "gather_rest_rows: the host copy of the FFN matrices is needed");
+        const size_t rb = row_bytes(t.type, d);
+        void * pin = nullptr;
+        PI_HIP_TRY(hipHostMalloc(&pin, rb * (rest.empty() ? 1 : rest.size()), hipHostMallocDefault));
+        m->pinned.push_back(pin);
+        for (size_t i = 0; i < rest.size(); ++i) memcpy((unsigned char *)pin + rb * i, (const unsigned char *)t.host + rb * (size_t)rest[i], rb);
+        (k == PI_T_FFN_UP ? m->rest_up : k == PI_T_FFN_GATE ? m->rest_gate : m->rest_down)[il] = pin;
+    }
+    return PI_OK;
+}
+}  // namespace pi
+
+extern "C" {
+
 int pi_model_finalize(pi_model * m) {
     if (!m) return pi::fail(PI_E_ARG, "pi_model_finalize: null model");
     if (m->finalized) return PI_OK;
@@ -568,26 +599,10 @@ int pi_model_finalize(pi_model * m) {
     m->rest_up.assign(hp.n_layer, nullptr); m->rest_gate.assign(hp.n_layer, nullptr); m->rest_down.assign(hp.n_layer, nullptr);
     if (m->hybrid && m->rest_on_gpu) {
         for (int il = 0; il < hp.n_layer; ++il) {
-            Tensor & bucket = m->L(il, PI_T_GPU_BUCKET);
-            if (!bucket.dev) continue;
-            Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & fc1 = m->L(il, PI_T_FC1);
-            if (up.type != PI_TYPE_Q4_0 || !m->hot_words[il] || !pi_k_pred_upgate_q4_supported(ff, (int)fc1.ne1, d))
+            if (!m->L(il, PI_T_GPU_BUCKET).dev) continue;
+            if (m->L(il, PI_T_FFN_UP).type != PI_TYPE_Q4_0 || !m->hot_words[il] || !pi_k_pred_upgate_q4_supported(ff, (int)m->L(il, PI_T_FC1).ne1, d))
                 return pi::fail(PI_E_UNSUPPORTED, "pi_model_finalize: rest_on_gpu covers Q4_0 layers at n_embd 4096 with a predictor of rank 512 or 1024 and n_ff % 32 == 0");
-            const int32_t * gi = (const int32_t *)m->L(il, PI_T_GPU_IDX).host;
-            std::vector<int> rest;
-            for (int j = 0; j < ff; ++j) if (gi[j] != 1) rest.push_back(j);
-            if ((int)rest.size() + (int)bucket.ne0 != ff) return pi::fail(PI_E_ARG, "pi_model_finalize: gpu_idx and gpu_bucket disagree");
-            const size_t rb = row_bytes(up.type, d);
-            for (int k : {PI_T_FFN_UP, PI_T_FFN_GATE, PI_T_FFN_DOWN_T}) {
-                if (k == PI_T_FFN_GATE && hp.arch == PI_ARCH_FALCON) continue;
-                Tensor & t = m->L(il, k);
-                if (!t.host) return pi::fail(PI_E_STATE, "pi_model_finalize: rest_on_gpu needs the host copy of the FFN matrices");
-                void * pin = nullptr;
-                PI_HIP_TRY(hipHostMalloc(&pin, rb * (rest.empty() ? 1 : rest.size()), hipHostMallocDefault));
-                m->pinned.push_back(pin);
-                for (size_t i = 0; i < rest.size(); ++i) memcpy((unsigned char *)pin + rb * i, (const unsigned char *)t.host + rb * (size_t)rest[i], rb);
-                (k == PI_T_FFN_UP ? m->rest_up : k == PI_T_FFN_GATE ? m->rest_gate : m->rest_down)[il] = pin;
-            }
+            PI_TRY(pi::gather_rest_rows(m, il));
         }
     }
 
@@ -658,10 +673,11 @@ int pi_model_decode(pi_model * m, const int32_t * tokens, int n_tokens, int n_pa
     for (int i = 0; i < n_tokens; ++i)
         if (tokens[i] < 0 || tokens[i] >= m->hp.n_vocab) return pi::fail(PI_E_ARG, "pi_model_decode: token id out of range");
     int first = 0;
-    if (n_tokens > 2 && pi::prefill_supported(m)) {
+    if (n_tokens > 2) {
         // the prompt goes through in chunks (weights read once per chunk): up to 512 tokens where the dense chunk path covers the
-        // shape, up to 16 otherwise and for the remainder; the last token takes the single-token path below, which produces the logits
-        const bool wide = pi::prefill_wide_supported(m);
+        // model (F16 or Q4_0 matrices, hybrid layers included), up to 16 for the remainder of an F16 model that is whole on the
+        // device; what is left, and at least the last token, takes the single-token path below, which produces the logits
+        const bool wide = pi::prefill_wide_supported(m), small = pi::prefill_supported(m);
         const int wide_max = wide ? pi::prefill_wide_max(m) : 0;
         while (n_tokens - 1 - first >= 2) {
             const int left = n_tokens - 1 - first;
@@ -669,10 +685,12 @@ int pi_model_decode(pi_model * m, const int32_t * tokens, int n_tokens, int n_pa
                 const int T = left < wide_max ? left : wide_max;
                 PI_TRY(pi::prefill_wide_chunk(m, tokens + first, T, n_past + first));
                 first += T;
-            } else {
+            } else if (small) {
                 const int T = left < 16 ? left : 16;
                 PI_TRY(pi::prefill_chunk(m, tokens + first, T, n_past + first));
                 first += T;
+            } else {
+                break;
             }
         }
     }

@@ -6,6 +6,7 @@
 #include "runtime.hpp"
 
 #include <stdlib.h>
+#include <algorithm>
 #include <string.h>
 
 struct BatchState {
@@ -20,6 +21,7 @@ struct BatchState {
     int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_step = nullptr, *d_out_tokens = nullptr, *union_rows = nullptr, *n_union = nullptr;
     float *up_out = nullptr, *gate_out = nullptr;      // wide prompt chunks: dense gate/up products [T][n_ff]
     __half *h16 = nullptr;                             //                     and the FFN's hidden vector
+    __half *w16 = nullptr, *w16t = nullptr;            // wide prompt chunks of Q4_0 / hybrid layers: one matrix as fp16, and the down projection with the neurons contiguous
     hipGraphExec_t graph_exec = nullptr;
     hipGraph_t graph = nullptr;
     std::vector<std::vector<int32_t>> kv_pos;      // per sequence: cell positions while an edit left them non-contiguous
@@ -160,6 +162,35 @@ int chunk_gemm(pi_model * m, const void * W, int rows, int cols, const void * xn
     return pi_k_gemm_wide_f16(W, rows, cols, xn, T, epi, add1, add2, y, y16, m->stream);
 }
 
+// a matrix of layer il as fp16 rows for a chunk's mat-mul: an F16 matrix that is whole on the device as stored; a Q4_0 one expanded into
+// the chunk's scratch (values (q - 8) * d rounded to fp16); an FFN matrix of a hybrid layer assembled there from the compact matrix of the
+// resident neurons and the non-resident rows in pinned host memory, which the kernel reads over the host link once per chunk
+int chunk_weight(pi_model * m, BatchState * b, int il, int kind, int rows, int cols, const void ** out) {
+    Tensor & t = m->L(il, kind);
+    const bool ffn = kind == PI_T_FFN_UP || kind == PI_T_FFN_GATE || kind == PI_T_FFN_DOWN_T;
+    const bool split = ffn && m->L(il, PI_T_GPU_BUCKET).dev != nullptr;
+    const void * rest = !split ? nullptr : kind == PI_T_FFN_UP ? m->rest_up[il] : kind == PI_T_FFN_GATE ? m->rest_gate[il] : m->rest_down[il];
+    const uint32_t * hw = split ? m->hot_words[il] : nullptr;
+    const int32_t * hpx = split ? m->hot_prefix[il] : nullptr;
+    if (t.type == PI_TYPE_Q4_0) {
+        PI_TRY(pi_k_dequant_q4_f16(t.dev, rest, hw, hpx, rows, cols, b->w16, m->stream));
+        *out = b->w16;
+    } else if (split) {
+        PI_TRY(pi_k_assemble_rows_f16(t.dev, rest, hw, hpx, rows, cols, b->w16, m->stream));
+        *out = b->w16;
+    } else {
+        *out = t.dev;
+    }
+    return PI_OK;
+}
+
+// fp16 mat-mul input of a chunk for a matrix of the given type: the normalised rows rounded to fp16, for a Q4_0 matrix through Q8_0
+// blocks first (the CPU path multiplies Q4_0 rows with the Q8_0 form of the activations)
+int chunk_input(int wtype, const float * x, int T, int cols, const pi_norm * norm, void * out16, void * plain16, hipStream_t st) {
+    if (wtype == PI_TYPE_Q4_0) return pi_k_norm_q8_round_f16(x, T, cols, norm, out16, plain16, st);
+    return pi_k_norm_round_f16(x, T, cols, norm, out16, plain16, st);
+}
+
 int wide_layer(pi_model * m, BatchState * b, int il) {
     const pi_hparams & hp = m->hp;
     const int T = b->n_seq, d = hp.n_embd, ff = hp.n_ff, hd = m->hd, gqa = m->gqa;
@@ -167,45 +198,90 @@ int wide_layer(pi_model * m, BatchState * b, int il) {
     hipStream_t st = m->stream;
     Tensor & wqkv = m->L(il, PI_T_WQKV); Tensor & wo = m->L(il, PI_T_WO);
     Tensor & fc1 = m->L(il, PI_T_FC1); Tensor & fc2 = m->L(il, PI_T_FC2);
-    Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE);
+    Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
     const int r = (int)fc1.ne1;
     const size_t kv_off = (size_t)il * hp.n_head_kv * hp.n_ctx * hd;
     float * x = b->x;
+    const void * W = nullptr;
+    const pi_norm plain{0, 0.0f, nullptr, nullptr};
     pi_norm an;
     if (!falcon) an = mk_norm(1, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), nullptr);
     else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
     else an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
-    PI_TRY(pi_k_norm_round_f16(x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));
-    PI_TRY(chunk_gemm(m, wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr));
+    PI_TRY(chunk_input(wqkv.type, x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));
+    PI_TRY(chunk_weight(m, b, il, PI_T_WQKV, d + 2 * gqa, d, &W));
+    PI_TRY(chunk_gemm(m, W, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr));
     PI_TRY(pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, b->d_pos, hp.n_ctx, b->q_rot,
                            m->k_cache + kv_off, m->v_cache + kv_off, b->att, d, b->att16, st));
+    if (wo.type == PI_TYPE_Q4_0) PI_TRY(pi_k_norm_q8_round_f16(b->att, T, d, &plain, b->att16, nullptr, st));
+    PI_TRY(chunk_weight(m, b, il, PI_T_WO, d, d, &W));
     pi_norm fn;
+    const __half * ffn_x = b->xf16;
     if (!falcon) {
-        PI_TRY(chunk_gemm(m, wo.dev, d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, nullptr));
+        PI_TRY(chunk_gemm(m, W, d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, nullptr));
         fn = mk_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
-        PI_TRY(pi_k_norm_round_f16(b->ffn_inp, T, d, &fn, b->xf16, b->xp16, st));
+        PI_TRY(chunk_input(up.type, b->ffn_inp, T, d, &fn, b->xf16, b->xp16, st));
     } else {
-        PI_TRY(chunk_gemm(m, wo.dev, d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, nullptr));
+        PI_TRY(chunk_gemm(m, W, d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, nullptr));
         fn = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
-        if (m->L(il, PI_T_ATTN_NORM_2).dev) PI_TRY(pi_k_norm_round_f16(x, T, d, &fn, b->xf16, nullptr, st));
+        // the FFN branch reads the layer input under its own norm; with a single norm it shares the attention branch's rows unless
+        // the two matrices want different containers (fp16 against Q8_0 blocks)
+        if (m->L(il, PI_T_ATTN_NORM_2).dev || up.type != wqkv.type) PI_TRY(chunk_input(up.type, x, T, d, &fn, b->xf16, nullptr, st));
+        else ffn_x = b->xa16;
     }
-    const __half * ffn_x = (falcon && !m->L(il, PI_T_ATTN_NORM_2).dev) ? b->xa16 : b->xf16;
     PI_TRY(chunk_gemm(m, fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16));
     PI_TRY(chunk_gemm(m, fc2.dev, ff, r, b->hid16, T, PI_EPI_NONE, nullptr, nullptr, b->pred_logits, nullptr));
-    PI_TRY(chunk_gemm(m, up.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->up_out, nullptr));
-    if (!falcon) PI_TRY(chunk_gemm(m, gate.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->gate_out, nullptr));
-    PI_TRY(pi_k_ffn_h_f16(b->up_out, falcon ? nullptr : b->gate_out, b->pred_logits, hp.sparse_threshold, T, ff, b->h16, st));
-    if (!falcon) PI_TRY(chunk_gemm(m, m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD, b->ffn_inp, nullptr, b->x2, nullptr));
-    else         PI_TRY(chunk_gemm(m, m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD2, b->attn_out, x, b->x2, nullptr));
+    PI_TRY(chunk_weight(m, b, il, PI_T_FFN_UP, ff, d, &W));
+    PI_TRY(chunk_gemm(m, W, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->up_out, nullptr));
+    if (!falcon) {
+        PI_TRY(chunk_weight(m, b, il, PI_T_FFN_GATE, ff, d, &W));
+        PI_TRY(chunk_gemm(m, W, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->gate_out, nullptr));
+    }
+    if (down.type == PI_TYPE_Q4_0) PI_TRY(pi_k_ffn_h_q8_f16(b->up_out, falcon ? nullptr : b->gate_out, b->pred_logits, hp.sparse_threshold, T, ff, b->h16, st));
+    else                           PI_TRY(pi_k_ffn_h_f16(b->up_out, falcon ? nullptr : b->gate_out, b->pred_logits, hp.sparse_threshold, T, ff, b->h16, st));
+    const void * Wd = m->down_rows[il];
+    if (!Wd) {
+        PI_TRY(chunk_weight(m, b, il, PI_T_FFN_DOWN_T, ff, d, &W));
+        PI_TRY(pi_k_transpose_f16(W, ff, d, b->w16t, st));
+        Wd = b->w16t;
+    }
+    if (!falcon) PI_TRY(chunk_gemm(m, Wd, d, ff, b->h16, T, PI_EPI_ADD, b->ffn_inp, nullptr, b->x2, nullptr));
+    else         PI_TRY(chunk_gemm(m, Wd, d, ff, b->h16, T, PI_EPI_ADD2, b->attn_out, x, b->x2, nullptr));
     std::swap(b->x, b->x2);
     return PI_OK;
+}
+
+// why the model's prompts cannot go through wide chunks, or null
+const char * wide_unsupported(pi_model * m) {
+    const pi_hparams & hp = m->hp;
+    if (m->capture) return "capture hooks follow single tokens";
+    if (hp.n_embd % 256 || hp.n_ff % 256 || (int)m->L(0, PI_T_FC1).ne1 % 256) return "n_embd, n_ff and the predictor rank must be multiples of 256";
+    const int te = m->glob[PI_T_TOK_EMBD].type;
+    if (te != PI_TYPE_F16 && te != PI_TYPE_Q4_0) return "embedding table must be F16 or Q4_0";
+    for (int il = 0; il < hp.n_layer; ++il) {
+        for (int k : {PI_T_WQKV, PI_T_WO, PI_T_FFN_UP, PI_T_FFN_GATE, PI_T_FFN_DOWN_T}) {
+            if (k == PI_T_FFN_GATE && hp.arch == PI_ARCH_FALCON) continue;
+            const int ty = m->L(il, k).type;
+            if (ty != PI_TYPE_F16 && ty != PI_TYPE_Q4_0) return "matrices must be F16 or Q4_0";
+        }
+        if (m->L(il, PI_T_FC1).type != PI_TYPE_F16 || m->L(il, PI_T_FC2).type != PI_TYPE_F16 || (int)m->L(il, PI_T_FC1).ne1 != (int)m->L(0, PI_T_FC1).ne1)
+            return "predictors must be F16 and of one rank";
+        if (hp.arch != PI_ARCH_FALCON && m->L(il, PI_T_FFN_GATE).type != m->L(il, PI_T_FFN_UP).type) return "gate and up must share a type";
+        if (m->L(il, PI_T_GPU_BUCKET).dev) {
+            if (!m->hot_words[il]) return "hybrid layers need n_ff % 32 == 0";
+            for (int k : {PI_T_FFN_UP, PI_T_FFN_GATE, PI_T_FFN_DOWN_T})
+                if (!(k == PI_T_FFN_GATE && hp.arch == PI_ARCH_FALCON) && !m->L(il, k).host && !m->rest_up[il]) return "hybrid layers need the host copy of the FFN matrices";
+        }
+    }
+    return nullptr;
 }
 }  // namespace
 
 namespace pi {
 bool prefill_wide_supported(pi_model * m) {
     const char * off = getenv("PI_NO_PREFILL_WIDE");
-    return !(off && off[0] == '1') && prefill_supported(m) && m->hp.n_embd % 256 == 0 && m->hp.n_ff % 256 == 0 && (int)m->L(0, PI_T_FC1).ne1 % 256 == 0;
+    const char * off_all = getenv("PI_NO_PREFILL");
+    return !(off && off[0] == '1') && !(off_all && off_all[0] == '1') && wide_unsupported(m) == nullptr;
 }
 
 int prefill_wide_max(pi_model * m) {
@@ -229,14 +305,27 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
         b->gate_out = hp.arch == PI_ARCH_FALCON ? nullptr : m->alloc<float>((size_t)kMaxT * hp.n_ff);
         b->h16 = m->alloc<__half>((size_t)kMaxT * hp.n_ff);
         if (!b->up_out || (hp.arch != PI_ARCH_FALCON && !b->gate_out) || !b->h16) { delete b; return PI_E_HIP; }
-        // the down projection of a chunk is a mat-mul whose reduction runs over the neurons: one more copy of it with the neurons
-        // contiguous (n_embd x n_ff fp16 per layer; the decode loop keeps using the row-per-neuron layout)
+        // the down projection of a chunk is a mat-mul whose reduction runs over the neurons.  An F16 layer that is whole on the device
+        // gets one more copy of it with the neurons contiguous (n_embd x n_ff fp16; the decode loop keeps the row-per-neuron layout);
+        // Q4_0 and hybrid layers expand one matrix at a time into scratch instead, so that prompts leave the model's footprint as
+        // the quantisation and the VRAM split made it
+        size_t w16 = 0;
+        bool scratch = false;
         m->down_rows.assign(hp.n_layer, nullptr);
         for (int il = 0; il < hp.n_layer; ++il) {
+            const bool split = m->L(il, PI_T_GPU_BUCKET).dev != nullptr;
+            if (split) PI_TRY(gather_rest_rows(m, il));
+            if (m->L(il, PI_T_WQKV).type == PI_TYPE_Q4_0) w16 = std::max(w16, (size_t)(hp.n_embd + 2 * m->gqa) * hp.n_embd);
+            if (m->L(il, PI_T_WO).type == PI_TYPE_Q4_0) w16 = std::max(w16, (size_t)hp.n_embd * hp.n_embd);
+            if (split || m->L(il, PI_T_FFN_UP).type == PI_TYPE_Q4_0 || m->L(il, PI_T_FFN_DOWN_T).type == PI_TYPE_Q4_0) w16 = std::max(w16, (size_t)hp.n_ff * hp.n_embd);
+            if (split || m->L(il, PI_T_FFN_DOWN_T).type == PI_TYPE_Q4_0) { scratch = true; continue; }
             m->down_rows[il] = m->alloc<__half>((size_t)hp.n_embd * hp.n_ff);
             if (!m->down_rows[il]) { delete b; m->down_rows.clear(); return PI_E_HIP; }
             PI_TRY(pi_k_transpose_f16(m->L(il, PI_T_FFN_DOWN_T).dev, hp.n_ff, hp.n_embd, m->down_rows[il], m->stream));
         }
+        if (w16) b->w16 = m->alloc<__half>(w16);
+        if (scratch) b->w16t = m->alloc<__half>((size_t)hp.n_embd * hp.n_ff);
+        if ((w16 && !b->w16) || (scratch && !b->w16t)) { delete b; m->down_rows.clear(); return PI_E_HIP; }
         m->prefill_wide = b;
     }
     BatchState * b = m->prefill_wide;
@@ -246,7 +335,8 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
     PI_HIP_TRY(hipMemcpyAsync(b->d_tokens, tokens, sizeof(int32_t) * T, hipMemcpyHostToDevice, m->stream));
     PI_HIP_TRY(hipMemcpyAsync(b->d_pos, pos, sizeof(int32_t) * T, hipMemcpyHostToDevice, m->stream));
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
-    PI_TRY(pi_k_embed_batch(m->glob[PI_T_TOK_EMBD].dev, hp.n_embd, b->d_tokens, T, b->x, m->stream));
+    if (m->glob[PI_T_TOK_EMBD].type == PI_TYPE_Q4_0) PI_TRY(pi_k_embed_batch_q4(m->glob[PI_T_TOK_EMBD].dev, hp.n_embd, b->d_tokens, T, b->x, m->stream));
+    else PI_TRY(pi_k_embed_batch(m->glob[PI_T_TOK_EMBD].dev, hp.n_embd, b->d_tokens, T, b->x, m->stream));
     for (int il = 0; il < hp.n_layer; ++il) PI_TRY(wide_layer(m, b, il));
     return PI_OK;
 }

@@ -62,6 +62,7 @@ struct pi_model {
     BatchState * prefill_wide = nullptr;  // the same for chunks of up to 512 tokens (dense mat-muls, weights read once per chunk)
     pi_gemm_lib * gemm_lib = nullptr;     // hipBLASLt plans of those mat-muls (PI_PREFILL_GEMM=own keeps them on this library's kernel, 128 tokens a chunk)
     std::vector<__half *> down_rows;      // per layer: the down projection with the neurons contiguous ([n_embd][n_ff]), made at the first wide chunk
+                                          // (null for Q4_0 and hybrid layers, whose matrices are expanded into the chunk's scratch instead)
 
     Tensor & L(int il, int kind) { return layers[(size_t)il * PI_T_COUNT + kind]; }
 
@@ -77,7 +78,8 @@ int  kv_edit(pi_model * m, __half * k_cache, __half * v_cache, int32_t * d_pos, 
 void batch_destroy(pi_model * m);       // frees the batched-decoding state (graphs; device buffers belong to the model)
 bool prefill_supported(pi_model * m);   // F16 weights, every neuron on the GPU, shapes the multi-token kernels cover
 int  prefill_chunk(pi_model * m, const int32_t * tokens, int T, int n_past);
-bool prefill_wide_supported(pi_model * m);   // and additionally n_ff and the predictor rank multiples of 256
+bool prefill_wide_supported(pi_model * m);   // F16 or Q4_0 matrices (fp16 predictor), hybrid layers included; n_embd, n_ff and the predictor rank multiples of 256
+int  gather_rest_rows(pi_model * m, int il);  // hybrid layer: rows of the non-resident neurons into pinned host memory (rest_up / rest_gate / rest_down)
 int  prefill_wide_max(pi_model * m);         // longest chunk: 512 through the library mat-mul, 128 on this library's own kernel (PI_PREFILL_GEMM=own)
 int  prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past);     // 16 < T <= prefill_wide_max
 }

@@ -2379,8 +2379,10 @@ __global__ void embed_f16_kernel(const __half * __restrict__ table, int cols, co
     const __half * row = table + (size_t)(*token) * cols;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < cols; i += gridDim.x * blockDim.x) x[i] = __half2float(row[i]);
 }
+// blockIdx.y = token of a chunk (0 for a single token)
 __global__ void embed_q4_kernel(const pi_block_q4_0 * __restrict__ table, int cols, const int32_t * __restrict__ token, float * __restrict__ x) {
-    const pi_block_q4_0 * row = table + (size_t)(*token) * (cols / 32);
+    const pi_block_q4_0 * row = table + (size_t)token[blockIdx.y] * (cols / 32);
+    x += (size_t)blockIdx.y * cols;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < cols; i += gridDim.x * blockDim.x) {
         const pi_block_q4_0 * b = row + (i >> 5);
         uint16_t dbits; __builtin_memcpy(&dbits, &b->d, 2);
@@ -2471,8 +2473,20 @@ typedef _Float16 pi_h8 __attribute__((ext_vector_type(8)));
 typedef float    pi_f4 __attribute__((ext_vector_type(4)));
 constexpr int kBtMaxT = 16;
 
+// the value a Q8_0 block keeps of v: q * fp16(amax / 127) with q = rint(v * 127 / amax) and amax over the 32 consecutive elements
+// the 32 lanes of a half-wave hold (quantize_row_q8_0, x86 path, ggml-quants.c:702-760), rounded to fp16 for a mat-mul input
+__device__ __forceinline__ float q8_block_value(float v) {
+    float amax = fabsf(v);
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, PI_WAVE));
+    const float d = pi_round_f16(pi_div(amax, 127.0f)), id = (amax != 0.0f) ? pi_div(127.0f, amax) : 0.0f;
+    return __fmul_rn((float)(int)rintf(__fmul_rn(v, id)), d);
+}
+
+// q8 != 0 (cols % 32 == 0, cols <= 8192): the normalised row goes through Q8_0 blocks of 32 before the fp16 rounding, which is what
+// a Q4_0 mat-mul of the CPU path multiplies with (ggml_vec_dot_q4_0_q8_0, ggml-quants.c:2512-2650)
 __global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __restrict__ x, int cols, NormArgs na, __half * __restrict__ out,
-                                                              __half * __restrict__ out_plain) {
+                                                              __half * __restrict__ out_plain, int q8) {
     __shared__ double red[16];
     const float * xt = x + (size_t)blockIdx.x * cols;
     __half * ot = out + (size_t)blockIdx.x * cols;
@@ -2508,16 +2522,15 @@ __global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __re
 #pragma unroll
         for (int k = 0; k < 8; ++k) {
             const int i = threadIdx.x + k * 1024;
-            if (i < cols) {
-                float v = xv[k];
-                if (out_plain) out_plain[(size_t)blockIdx.x * cols + i] = __float2half_rn(v);
-                if (na.kind != 0) {
-                    v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
-                    if (na.w) v = __fmul_rn(v, wv[k]);
-                    if (na.b) v = __fadd_rn(v, bv[k]);
-                }
-                ot[i] = __float2half_rn(v);
+            float v = xv[k];
+            if (i < cols && out_plain) out_plain[(size_t)blockIdx.x * cols + i] = __float2half_rn(v);
+            if (na.kind != 0) {
+                v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
+                if (na.w) v = __fmul_rn(v, wv[k]);
+                if (na.b) v = __fadd_rn(v, bv[k]);
             }
+            if (q8) v = q8_block_value(i < cols ? v : 0.0f);          // every lane takes part in the block's maximum
+            if (i < cols) ot[i] = __float2half_rn(v);
         }
         return;
     }
@@ -2806,11 +2819,14 @@ __global__ __launch_bounds__(kBlock) void gemm_wide_f16_kernel(const __half * __
 }
 // h16[t][n] = fp16( !(logit[t][n] < thr) ? relu(gate[t][n]) * up[t][n] : 0 )   (relu(up) without a gate): the FFN's hidden vector of a
 // prompt chunk from the dense gate/up products; inactive neurons become exact zeros, which add nothing in the down projection
+// q8 != 0 (n % 64 == 0 and n_ff % 32 == 0): h goes through Q8_0 blocks of 32 neurons first, as the CPU path's Q4_0 down projection quantises it
+// (ggml.c:14465-14618)
 __global__ void ffn_h_f16_kernel(const float * __restrict__ up, const float * __restrict__ gate, const float * __restrict__ logits, float thr,
-                                 size_t n, __half * __restrict__ h16) {
+                                 size_t n, __half * __restrict__ h16, int q8) {
     for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
         float h = 0.0f;
         if (!(logits[i] < thr)) h = gate ? __fmul_rn(fmaxf(gate[i], 0.0f), up[i]) : fmaxf(up[i], 0.0f);
+        if (q8) h = q8_block_value(h);
         h16[i] = __float2half_rn(h);
     }
 }
@@ -3898,8 +3914,14 @@ int pi_k_sparse_ffn_noalloc(const void * fc2_f16, int ff, int r, const float * h
 
 int pi_k_norm_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, void * out_plain_f16, pi_stream_t stream) {
     if (!x || !out_f16 || T <= 0 || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_norm_round_f16: bad arguments");
-    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16, (__half *)out_plain_f16);
+    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16, (__half *)out_plain_f16, 0);
     return pi::check_launch("pi_k_norm_round_f16");
+}
+
+int pi_k_norm_q8_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, void * out_plain_f16, pi_stream_t stream) {
+    if (!x || !out_f16 || T <= 0 || cols <= 0 || cols % 32 || cols > 8 * 1024) return pi::fail(PI_E_ARG, "pi_k_norm_q8_round_f16: cols must be a multiple of 32, at most 8192");
+    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16, (__half *)out_plain_f16, 1);
+    return pi::check_launch("pi_k_norm_q8_round_f16");
 }
 
 static int gemm_launch(const char * who, const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
@@ -3945,8 +3967,78 @@ int pi_k_gemm_wide_f16(const void * W, int rows, int cols, const void * xn_f16, 
 }
 int pi_k_ffn_h_f16(const float * up, const float * gate, const float * logits, float threshold, int T, int ff, void * h_f16, pi_stream_t stream) {
     if (!up || !logits || !h_f16 || T <= 0 || ff <= 0) return pi::fail(PI_E_ARG, "pi_k_ffn_h_f16: bad arguments");
-    hipLaunchKernelGGL(ffn_h_f16_kernel, dim3(1024), dim3(256), 0, (hipStream_t)stream, up, gate, logits, threshold, (size_t)T * ff, (__half *)h_f16);
+    hipLaunchKernelGGL(ffn_h_f16_kernel, dim3(1024), dim3(256), 0, (hipStream_t)stream, up, gate, logits, threshold, (size_t)T * ff, (__half *)h_f16, 0);
     return pi::check_launch("pi_k_ffn_h_f16");
+}
+int pi_k_ffn_h_q8_f16(const float * up, const float * gate, const float * logits, float threshold, int T, int ff, void * h_f16, pi_stream_t stream) {
+    if (!up || !logits || !h_f16 || T <= 0 || ff <= 0 || ff % 64) return pi::fail(PI_E_ARG, "pi_k_ffn_h_q8_f16: n_ff must be a multiple of 64");
+    hipLaunchKernelGGL(ffn_h_f16_kernel, dim3(1024), dim3(256), 0, (hipStream_t)stream, up, gate, logits, threshold, (size_t)T * ff, (__half *)h_f16, 1);
+    return pi::check_launch("pi_k_ffn_h_q8_f16");
+}
+
+// W[rows][cols] in Q4_0 blocks -> fp16 (value (q - 8) * d, dequantize_row_q4_0, ggml-quants.c:1074-1092), one thread per block.  With hot
+// words the rows of resident neurons come from the compact matrix W and the others from W_rest (both in ascending neuron order).
+__global__ void dequant_q4_f16_kernel(const pi_block_q4_0 * __restrict__ W, const pi_block_q4_0 * __restrict__ W_rest,
+                                      const uint32_t * __restrict__ hot_words, const int32_t * __restrict__ hot_prefix,
+                                      int rows, int nb, __half * __restrict__ out) {
+    const size_t n = (size_t)rows * nb;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) {
+        const int row = (int)(idx / nb), blk = (int)(idx % nb);
+        const pi_block_q4_0 * src;
+        if (hot_words) {
+            const uint32_t hot = hot_words[row >> 5];
+            const int bit = row & 31, base = hot_prefix[row >> 5], below = __popc(hot & ((1u << bit) - 1u));
+            src = ((hot >> bit) & 1u) ? W + (size_t)(base + below) * nb : W_rest + (size_t)((row & ~31) - base + bit - below) * nb;
+        } else {
+            src = W + (size_t)row * nb;
+        }
+        src += blk;
+        uint16_t dbits; __builtin_memcpy(&dbits, &src->d, 2);
+        const float d = pi_f16_from_bits(dbits);
+        uint32_t qs[4]; __builtin_memcpy(qs, src->qs, 16);
+        __align__(16) __half o[32];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int b = (qs[j >> 2] >> ((j & 3) * 8)) & 0xFF;
+            o[j] = __float2half_rn(__fmul_rn((float)((b & 0x0F) - 8), d));
+            o[j + 16] = __float2half_rn(__fmul_rn((float)((b >> 4) - 8), d));
+        }
+        pi_u32x4 * dst = reinterpret_cast<pi_u32x4 *>(out + (size_t)row * nb * 32 + blk * 32);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) dst[k] = reinterpret_cast<const pi_u32x4 *>(o)[k];
+    }
+}
+int pi_k_dequant_q4_f16(const void * W_q4, const void * W_rest_q4, const uint32_t * hot_words, const int32_t * hot_prefix, int rows, int cols,
+                        void * out_f16, pi_stream_t stream) {
+    if (!W_q4 || !out_f16 || rows <= 0 || cols <= 0 || cols % 32) return pi::fail(PI_E_ARG, "pi_k_dequant_q4_f16: bad arguments");
+    if ((hot_words == nullptr) != (hot_prefix == nullptr) || (hot_words && !W_rest_q4) || (hot_words && rows % 32))
+        return pi::fail(PI_E_ARG, "pi_k_dequant_q4_f16: hot_words, hot_prefix and the second matrix go together (rows % 32 == 0)");
+    const size_t n = (size_t)rows * (cols / 32);
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(dequant_q4_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const pi_block_q4_0 *)W_q4, (const pi_block_q4_0 *)W_rest_q4,
+                       hot_words, hot_prefix, rows, cols / 32, (__half *)out_f16);
+    return pi::check_launch("pi_k_dequant_q4_f16");
+}
+// the full fp16 matrix of a hybrid layer from the compact matrix of the resident neurons and the matrix of the others (both in
+// ascending neuron order); one workgroup per row, 16 bytes per lane and pass
+__global__ void assemble_rows_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ W_rest, const uint32_t * __restrict__ hot_words,
+                                         const int32_t * __restrict__ hot_prefix, int cols, __half * __restrict__ out) {
+    const int row = blockIdx.x;
+    const uint32_t hot = hot_words[row >> 5];
+    const int bit = row & 31, base = hot_prefix[row >> 5], below = __popc(hot & ((1u << bit) - 1u));
+    const __half * src = ((hot >> bit) & 1u) ? W + (size_t)(base + below) * cols : W_rest + (size_t)((row & ~31) - base + bit - below) * cols;
+    const pi_u32x4 * s4 = reinterpret_cast<const pi_u32x4 *>(src);
+    pi_u32x4 * d4 = reinterpret_cast<pi_u32x4 *>(out + (size_t)row * cols);
+    for (int i = threadIdx.x; i < cols / 8; i += blockDim.x) d4[i] = s4[i];
+}
+int pi_k_assemble_rows_f16(const void * W_f16, const void * W_rest_f16, const uint32_t * hot_words, const int32_t * hot_prefix, int rows, int cols,
+                           void * out_f16, pi_stream_t stream) {
+    if (!W_f16 || !W_rest_f16 || !hot_words || !hot_prefix || !out_f16 || rows <= 0 || rows % 32 || cols <= 0 || cols % 8)
+        return pi::fail(PI_E_ARG, "pi_k_assemble_rows_f16: bad arguments (rows % 32 == 0, cols % 8 == 0)");
+    hipLaunchKernelGGL(assemble_rows_f16_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, (const __half *)W_f16, (const __half *)W_rest_f16,
+                       hot_words, hot_prefix, cols, (__half *)out_f16);
+    return pi::check_launch("pi_k_assemble_rows_f16");
 }
 int pi_k_transpose_f16(const void * in, int rows, int cols, void * out, pi_stream_t stream) {
     if (!in || !out || rows <= 0 || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_transpose_f16: bad arguments");
@@ -4164,6 +4256,12 @@ int pi_k_embed_batch(const void * table_f16, int cols, const int32_t * tokens, i
     if (!table_f16 || !tokens || !x || cols <= 0 || T <= 0 || T > kChunkMaxT) return pi::fail(PI_E_ARG, "pi_k_embed_batch: bad arguments");
     hipLaunchKernelGGL(embed_f16_batch_kernel, dim3((cols + 255) / 256, T), dim3(256), 0, (hipStream_t)stream, (const __half *)table_f16, cols, tokens, x);
     return pi::check_launch("pi_k_embed_batch");
+}
+
+int pi_k_embed_batch_q4(const void * table_q4, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream) {
+    if (!table_q4 || !tokens || !x || cols <= 0 || cols % 32 || T <= 0 || T > kChunkMaxT) return pi::fail(PI_E_ARG, "pi_k_embed_batch_q4: bad arguments");
+    hipLaunchKernelGGL(embed_q4_kernel, dim3((cols + 255) / 256, T), dim3(256), 0, (hipStream_t)stream, (const pi_block_q4_0 *)table_q4, cols, tokens, x);
+    return pi::check_launch("pi_k_embed_batch_q4");
 }
 
 int pi_k_argmax_batch(const float * logits, int n, int T, int32_t * tokens, int32_t * positions, int32_t * step, int32_t * out_tokens, int max_steps,

@@ -80,6 +80,11 @@ _SIGS = {
     "pi_k_gemm_wide_f16": (_i, [_vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_ffn_h_f16": (_i, [_vp, _vp, _vp, _f, _i, _i, _vp, _vp]),
     "pi_k_transpose_f16": (_i, [_vp, _i, _i, _vp, _vp]),
+    "pi_k_norm_q8_round_f16": (_i, [_vp, _i, _i, C.POINTER(Norm), _vp, _vp, _vp]),
+    "pi_k_ffn_h_q8_f16": (_i, [_vp, _vp, _vp, _f, _i, _i, _vp, _vp]),
+    "pi_k_dequant_q4_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
+    "pi_k_assemble_rows_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
+    "pi_k_embed_batch_q4": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
     "pi_gemm_lib_create": (_vp, [C.c_size_t]),
     "pi_gemm_lib_destroy": (_i, [_vp]),
     "pi_gemm_lib_f16": (_i, [_vp, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),

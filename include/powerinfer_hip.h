@@ -37,6 +37,10 @@ PI_API const char * pi_last_error(void);
 PI_API int          pi_device_name(char * buf, size_t n);
 PI_API void *       pi_malloc(size_t bytes);                 /* NULL on failure */
 PI_API int          pi_free(void * dptr);
+/* pinned host memory that kernels read and write directly over the host link (coherent: a kernel's stores are visible to the host once
+ * the kernel has completed or has released them at system scope); for the logits / h / output-share operands of hybrid layers */
+PI_API void *       pi_malloc_host(size_t bytes);            /* NULL on failure */
+PI_API int          pi_free_host(void * hptr);
 PI_API int          pi_memset(void * dptr, int byte, size_t bytes);
 PI_API int          pi_memcpy_h2d(void * dptr, const void * host, size_t bytes);
 PI_API int          pi_memcpy_d2h(void * host, const void * dptr, size_t bytes);
@@ -303,6 +307,24 @@ PI_API int pi_k_dequant_q4_f16(const void * W_q4, const void * W_rest_q4, const 
 PI_API int pi_k_assemble_rows_f16(const void * W_f16, const void * W_rest_f16, const uint32_t * hot_words, const int32_t * hot_prefix, int rows, int cols,
                                   void * out_f16, pi_stream_t stream);
 PI_API int pi_k_embed_batch_q4(const void * table_q4, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream);
+
+/* Hand-over points between the stream and host threads that compute the non-resident neurons of a hybrid layer (the CPU half of
+ * llm_build_sparse_mul_mat / llm_build_sparse_axpy, llama.cpp:4581-4593, 4635-4646) without the host launching anything in between.
+ * flags_pinned: 64 words of pinned host memory (words 0 and 8 written by the device, words 16 and 32 by the host, word 48 = the host's
+ * stop word); seq: a device word counting the hand-overs; status_pinned: one device or pinned word, non-zero after a wait gave up.
+ * pi_k_host_signal: flags[word] = *seq (after *seq += 1 when advance is set) once everything queued before it is complete.  pi_k_host_wait: holds the stream until
+ * flags[slot] has reached *seq, for at most limit_seconds (then *status = 1 and every later wait returns at once). */
+PI_API int pi_k_host_signal(uint32_t * seq, uint32_t * flags_pinned, int word, int advance, pi_stream_t stream);
+/* pi_k_pred_upgate_q4 cut in two for such a layer, so that the host threads start behind the predictor: pi_k_pred_q4_logits computes the
+ * logits (to `logits`, which may be pinned host memory, and to logits_dev), the mask words and the Q8_0 blocks of the normalised input;
+ * pi_k_upgate_q4_hot_rows reads logits_dev and writes h (or 0) for the neurons of the hot words only - the other entries of h_dense
+ * belong to the host. */
+PI_API int pi_k_pred_q4_logits(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
+                               float * logits, float * logits_dev, void * xq8_out, pi_workspace * ws, pi_stream_t stream);
+PI_API int pi_k_upgate_q4_hot_rows(int ff, float threshold, const void * up_q4, const void * gate_q4, int cols, const float * x, const pi_norm * norm,
+                                   const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense, pi_workspace * ws,
+                                   pi_stream_t stream);
+PI_API int pi_k_host_wait(const uint32_t * seq, const uint32_t * flags_pinned, int slot, uint32_t * status_pinned, double limit_seconds, pi_stream_t stream);
 
 /* The same mat-mul for prompt chunks of any length through hipBLASLt (fp16 operands, fp32 accumulation and result), where the reference
  * calls cuBLAS (ggml_cuda_op_mul_mat_cublas, ggml-cuda.cu:7662-7756).  Arguments and epilogues as pi_k_gemm_f16; no limit on T or cols.

@@ -27,6 +27,8 @@
 #define PI_COLD_SIMD 1
 #endif
 
+#define PI_TRY(expr) do { int _rc = (expr); if (_rc != PI_OK) return _rc; } while (0)
+
 namespace pi {
 
 namespace {
@@ -275,7 +277,29 @@ struct ColdPath {
     std::vector<BlockQ8> xq8, hq8;
     std::vector<int32_t> act;                   // active cold neurons of the current token
     int d = 0, ff = 0;
+
+    // Q4_0 layers served without the launching thread: the stream carries hand-over kernels (pi_k_host_signal / pi_k_host_wait),
+    // a service thread takes the posted layers in order, waits for the device's signal, computes the host share with the pool and
+    // answers through two flag words.  Device and host count the hand-overs in step.
+    pi_model * model = nullptr;
+    bool async = false;
+    std::vector<int> async_layers;              // hybrid layers that take this route, ascending
+    uint32_t * flags = nullptr;                 // pinned: [0] logits ready, [8] resident h ready (device -> host), [16] h complete, [32] output share complete, [48] stop word
+    bool split_pred = true;                     // the predictor is its own launch, so the host starts while the resident up/gate rows run
+    std::vector<float *> h_async;               // per layer, pinned: h of that variant; the device writes the resident neurons' entries, the host its own
+                                                // (one vector per layer, because the resident set differs from layer to layer)
+    std::vector<std::vector<int32_t>> prev_act; // per layer: the host's entries that are non-zero from the previous token
+    uint32_t * d_seq = nullptr, * d_status = nullptr;    // device words: hand-over count, non-zero once a device-side wait gave up
+    std::thread service;
+    std::vector<int> ring;                      // posted layer indices, single producer / single consumer
+    std::atomic<uint64_t> posted{0}, served{0};
+    std::atomic<bool> stop{false}, failed{false};
+    std::atomic<int> service_asleep{0};
+    std::mutex mu;
+    std::condition_variable cv;
 };
+
+namespace { void service_loop(ColdPath * c); }
 
 ColdPath * cold_create(pi_model * m) {
     ColdPath * c = new ColdPath();
@@ -313,6 +337,35 @@ ColdPath * cold_create(pi_model * m) {
     }
     c->xn.resize(c->d); c->x16.resize(c->d); c->xq8.resize(c->d / 32 + 1); c->hq8.resize(c->ff / 32 + 1);
     c->act.reserve(c->ff); c->hval.resize(c->ff);
+    c->model = m;
+    const char * sync_only = getenv("PI_COLD_SYNC");
+    if (!(sync_only && sync_only[0] == '1')) {
+        for (int il = 0; il < hp.n_layer; ++il) {
+            Tensor & up = m->L(il, PI_T_FFN_UP);
+            if (m->L(il, PI_T_GPU_BUCKET).dev && up.type == PI_TYPE_Q4_0 && m->L(il, PI_T_FC2).type == PI_TYPE_F16 && m->hot_words[il] &&
+                pi_k_pred_upgate_q4_supported(c->ff, (int)m->L(il, PI_T_FC1).ne1, c->d))
+                c->async_layers.push_back(il);
+        }
+    }
+    if (!c->async_layers.empty()) {
+        void * fl = nullptr;
+        if (hipHostMalloc(&fl, 64 * sizeof(uint32_t), hipHostMallocCoherent) != hipSuccess) { set_error("cold path: pinned host allocation failed"); cold_destroy(c); return nullptr; }
+        c->flags = (uint32_t *)fl;
+        memset(c->flags, 0, 64 * sizeof(uint32_t));
+        if (const char * e = getenv("PI_COLD_SPLIT")) c->split_pred = e[0] != '0';
+        c->h_async.assign(hp.n_layer, nullptr);
+        c->prev_act.resize(hp.n_layer);
+        for (int il : c->async_layers) {
+            c->h_async[il] = pin(c->ff);
+            if (!c->h_async[il]) { set_error("cold path: pinned host allocation failed"); cold_destroy(c); return nullptr; }
+            memset(c->h_async[il], 0, sizeof(float) * c->ff);
+        }
+        c->d_seq = m->alloc<uint32_t>(1); c->d_status = m->alloc<uint32_t>(1);
+        if (!c->d_seq || !c->d_status || pi_memset(c->d_seq, 0, 4) != PI_OK || pi_memset(c->d_status, 0, 4) != PI_OK) { cold_destroy(c); return nullptr; }
+        c->ring.resize(1 << 16);
+        c->async = true;
+        c->service = std::thread([c] { service_loop(c); });
+    }
     return c;
 }
 
@@ -323,6 +376,14 @@ void cold_destroy(ColdPath * c) {
         fprintf(stderr, "cold path, mean us per layer call over %lld calls: between calls %.1f | wait inputs %.1f | norm+list %.1f | up/gate %.1f | wait h + upload %.1f | down %.1f | merge launch %.1f | active cold neurons %.1f\n",
                 c->n_calls, c->t_between / n, c->t_phase[0] / n, c->t_phase[1] / n, c->t_phase[2] / n, c->t_phase[3] / n, c->t_phase[4] / n, c->t_phase[5] / n, (double)c->n_cold_active / n);
     }
+    if (c->service.joinable()) {
+        c->stop.store(true);
+        { std::lock_guard<std::mutex> g(c->mu); }
+        c->cv.notify_all();
+        c->service.join();
+    }
+    if (c->flags) (void)hipHostFree(c->flags);
+    for (float * p : c->h_async) if (p) (void)hipHostFree(p);
     delete c->pool;
     for (float * p : {c->logits, c->src, c->h_gpu, c->h_full[0], c->h_full[1], c->out[0], c->out[1]}) if (p) (void)hipHostFree(p);
     if (c->xq8_pin) (void)hipHostFree(c->xq8_pin);
@@ -670,6 +731,213 @@ int cold_layer_f16(ColdPath * c, int il, pi_model * m, hipStream_t st, bool capt
     lap(5);
     if (c->trace) { ++c->n_calls; c->n_cold_active += na; c->t_last_return = now(); }
     return rc;
+}
+
+
+// ---- Q4_0 hybrid layers without the launching thread in the loop -------------------------------------------------------------
+namespace {
+
+inline void relax() {
+#ifdef PI_COLD_SIMD
+    _mm_pause();
+#else
+    std::this_thread::yield();
+#endif
+}
+
+// the host share of one posted layer: what cold_layer_q4 does between its launches, started by the device's signal
+void serve_q4(ColdPath * c, int il, uint32_t seq) {
+    pi_model * m = c->model;
+    const pi_hparams & hp = m->hp;
+    const int d = c->d;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    ColdLayer & cl = c->layers[il];
+    Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
+    const float thr = hp.sparse_threshold;
+    float * hfull = c->split_pred ? c->h_async[il] : c->h_full[0];
+    float * out = c->out[0];
+    auto now = [] { return std::chrono::steady_clock::now(); };
+    auto us = [](std::chrono::steady_clock::time_point a, std::chrono::steady_clock::time_point b) { return std::chrono::duration<double, std::micro>(b - a).count(); };
+    std::chrono::steady_clock::time_point tp = now();
+    if (c->trace && c->n_calls) c->t_between += us(c->t_last_return, tp);
+    auto lap = [&](int i) { if (c->trace) { const auto t = now(); c->t_phase[i] += us(tp, t); tp = t; } };
+
+    // 1. logits, the Q8_0 blocks of the normalised input and the resident neurons' h are in pinned memory once the device says so
+    {
+        const auto t0 = now();
+        for (int it = 0; (int32_t)(__atomic_load_n(&c->flags[0], __ATOMIC_ACQUIRE) - seq) < 0; ++it) {
+            relax();
+            if ((it & 1023) == 1023 && (c->stop.load() || now() - t0 > std::chrono::seconds(20))) {
+                // the device never got here (a failed launch, a caller that gave up): release the stream's waits and stop serving
+                c->failed.store(true);
+                __atomic_store_n(&c->flags[48], 1u, __ATOMIC_RELEASE);
+                return;
+            }
+        }
+    }
+    lap(0);
+
+    // 2. active cold neurons, their up/gate rows against the same Q8_0 input
+    if (c->split_pred) {                        // this side's entries of the shared vector: the device never writes them
+        for (int j : c->prev_act[il]) hfull[j] = 0.f;
+        c->prev_act[il].clear();
+    }
+    c->act.clear();
+    for (int j : cl.cold_rows) if (!(c->logits[j] < thr)) c->act.push_back(j);
+    const int na = (int)c->act.size();
+    lap(1);
+    float * hval = c->hval.data();
+    const size_t rb = (size_t)(d / 32) * 18;
+    const unsigned char * wu = (const unsigned char *)up.host;
+    const unsigned char * wg = falcon ? nullptr : (const unsigned char *)gate.host;
+    const BlockQ8 * xq = c->xq8_pin;
+    c->pool->run([&](int t, int nt) {
+        for (int k = t; k < na; k += nt) {
+            const int j = c->act[k];
+            if (k + nt < na) { prefetch_bytes(wu + rb * c->act[k + nt], rb); if (wg) prefetch_bytes(wg + rb * c->act[k + nt], rb); }
+            const float u = dot_q4_q8(d, (const BlockQ4 *)(wu + rb * j), xq);
+            const float g = wg ? dot_q4_q8(d, (const BlockQ4 *)(wg + rb * j), xq) : 0.f;
+            hval[k] = wg ? (g > 0.f ? g : 0.f) * u : (u > 0.f ? u : 0.f);
+        }
+    });
+    for (int k = 0; k < na; ++k) hfull[c->act[k]] = hval[k];
+    if (c->split_pred) c->prev_act[il].assign(c->act.begin(), c->act.end());
+    __atomic_store_n(&c->flags[16], seq, __ATOMIC_RELEASE);          // the device's down projection may read the completed vector
+    lap(2);
+    if (c->split_pred) {
+        // the Q8_0 scales of h span resident and non-resident neurons: the resident ones' h must have arrived
+        const auto t0 = now();
+        for (int it = 0; (int32_t)(__atomic_load_n(&c->flags[8], __ATOMIC_ACQUIRE) - seq) < 0; ++it) {
+            relax();
+            if ((it & 1023) == 1023 && (c->stop.load() || now() - t0 > std::chrono::seconds(20))) {
+                c->failed.store(true);
+                __atomic_store_n(&c->flags[48], 1u, __ATOMIC_RELEASE);
+                return;
+            }
+        }
+    }
+
+    // 3. the host quantises h the same way and adds its neurons' down rows
+    for (int k = 0, last = -1; k < na; ++k) {
+        const int b = c->act[k] / 32;
+        if (b != last) { quantize_q8(hfull + b * 32, c->hq8.data() + b, 32); last = b; }
+    }
+    lap(3);
+    const unsigned char * wd = (const unsigned char *)down.host;
+    const int n_units = d / 32;
+    c->pool->run([&](int t, int nt) {
+        const int u0 = (int)((long long)n_units * t / nt), u1 = (int)((long long)n_units * (t + 1) / nt);
+        for (int i = u0 * 32; i < u1 * 32; ++i) out[i] = 0.f;
+        for (int k = 0; k < na; ++k) {
+            const int j = c->act[k];
+            const BlockQ8 & hb = c->hq8[j / 32];
+            const int a = hb.qs[j % 32];
+            if (k + 2 < na) prefetch_bytes(wd + rb * c->act[k + 2] + (size_t)u0 * 18, (size_t)(u1 - u0) * 18);
+            if (a == 0) continue;
+            axpy_q4_blocks((const BlockQ4 *)(wd + rb * j), u0, u1, a, h2f(hb.d), out);
+        }
+    });
+    __atomic_store_n(&c->flags[32], seq, __ATOMIC_RELEASE);          // the reduction may add the host share
+    lap(4);
+    if (c->trace) { ++c->n_calls; c->n_cold_active += na; c->t_last_return = now(); }
+}
+
+void service_loop(ColdPath * c) {
+    uint64_t next = 0;
+    uint32_t seq = 0;
+    for (;;) {
+        const auto t0 = std::chrono::steady_clock::now();
+        for (int it = 0; c->posted.load(std::memory_order_acquire) == next; ++it) {
+            if (c->stop.load()) return;
+            relax();
+            if ((it & 255) == 255 && std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(2000)) {
+                std::unique_lock<std::mutex> g(c->mu);
+                c->service_asleep.store(1);
+                c->cv.wait(g, [&] { return c->posted.load() != next || c->stop.load(); });
+                c->service_asleep.store(0);
+            }
+        }
+        if (c->stop.load()) return;
+        const int il = c->ring[next % c->ring.size()];
+        ++seq;
+        if (!c->failed.load()) serve_q4(c, il, seq);
+        c->served.store(++next, std::memory_order_release);
+    }
+}
+
+}  // namespace
+
+bool cold_async(const ColdPath * c) { return c && c->async; }
+bool cold_every_layer_async(const ColdPath * c) {
+    if (!c || !c->async) return false;
+    size_t hybrid = 0;
+    for (int il = 0; il < c->model->hp.n_layer; ++il) hybrid += c->model->L(il, PI_T_GPU_BUCKET).dev != nullptr;
+    return hybrid == c->async_layers.size();
+}
+
+// one token's hybrid layers, in the order the stream will reach them
+int cold_post_token(ColdPath * c) {
+    if (c->failed.load()) return fail(PI_E_STATE, "cold path: the host share stopped after a hand-over timed out");
+    for (int il : c->async_layers) {
+        const uint64_t p = c->posted.load(std::memory_order_relaxed);
+        while (p - c->served.load(std::memory_order_acquire) >= c->ring.size()) relax();
+        c->ring[p % c->ring.size()] = il;
+        c->posted.store(p + 1, std::memory_order_release);
+    }
+    if (c->service_asleep.load()) { { std::lock_guard<std::mutex> g(c->mu); } c->cv.notify_all(); }
+    return PI_OK;
+}
+
+// the stream has been synchronised: every posted layer has been answered, or something gave up
+int cold_drain(ColdPath * c) {
+    if (!c->async) return PI_OK;
+    const auto t0 = std::chrono::steady_clock::now();
+    while (c->served.load(std::memory_order_acquire) != c->posted.load() && !c->failed.load()) {
+        relax();
+        if (std::chrono::steady_clock::now() - t0 > std::chrono::seconds(30)) { c->failed.store(true); break; }
+    }
+    uint32_t status = 0;
+    if (pi_memcpy_d2h(&status, c->d_status, 4) != PI_OK) return PI_E_HIP;
+    if (status != 0 || c->failed.load()) return fail(PI_E_STATE, "cold path: a hand-over between the stream and the host threads timed out");
+    return PI_OK;
+}
+
+// the device half of such a layer, queued in one go: fc2 + mask + resident up/gate -> signal -> (wait for h) down projection ->
+// (wait for the host share) reduction with the merge folded in
+int cold_layer_q4_queue(ColdPath * c, int il, pi_model * m, hipStream_t st) {
+    const pi_hparams & hp = m->hp;
+    const int d = c->d, ff = c->ff;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
+    Tensor & fc1 = m->L(il, PI_T_FC1); Tensor & fc2 = m->L(il, PI_T_FC2);
+    const int r = (int)fc1.ne1;
+    float * hfull = c->h_full[0];
+    float * out = c->out[0];
+    const double limit = 5.0;
+    pi_norm fn;
+    fn.kind = falcon ? 2 : 1; fn.eps = hp.norm_eps;
+    fn.w = (const float *)m->L(il, falcon ? PI_T_ATTN_NORM : PI_T_FFN_NORM).dev;
+    fn.b = falcon ? (const float *)m->L(il, PI_T_ATTN_NORM_B).dev : nullptr;
+    const float * ffn_src = falcon ? m->x : m->ffn_inp;
+    if (c->split_pred) {
+        hfull = c->h_async[il];
+        PI_TRY(pi_k_pred_q4_logits(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, d, ffn_src, &fn, c->logits, m->pred_logits, c->xq8_pin, m->ws, st));
+        PI_TRY(pi_k_host_signal(c->d_seq, c->flags, 0, 1, st));
+        PI_TRY(pi_k_upgate_q4_hot_rows(ff, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, d, ffn_src, &fn, m->hot_words[il], m->hot_prefix[il],
+                                       m->pred_logits, hfull, m->ws, st));
+        PI_TRY(pi_k_host_signal(c->d_seq, c->flags, 8, 0, st));
+    } else {
+        PI_TRY(pi_k_pred_upgate_q4(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, d, ffn_src, &fn,
+                                   m->hot_words[il], m->hot_prefix[il], c->logits, hfull, c->xq8_pin, m->ws, st));
+        PI_TRY(pi_k_host_signal(c->d_seq, c->flags, 0, 1, st));
+    }
+    PI_TRY(pi_k_host_wait(c->d_seq, c->flags, 16, c->d_status, limit, st));
+    PI_TRY(pi_k_axpy_q4_partials(down.dev, d, ff, hfull, m->hot_words[il], m->hot_prefix[il], m->ws, st));
+    PI_TRY(pi_k_host_wait(c->d_seq, c->flags, 32, c->d_status, limit, st));
+    int32_t * n_act = m->n_active + il;
+    if (!falcon) return pi_k_axpy_q4_reduce(ff, d, PI_EPI_ADD2, out, m->ffn_inp, m->x2, n_act, m->ws, st);
+    PI_TRY(pi_k_axpy_q4_reduce(ff, d, PI_EPI_NONE, nullptr, nullptr, m->x2, n_act, m->ws, st));
+    return merge_shares(m->x2, out, m->x2, m->attn_out, m->x, nullptr, d, st);
 }
 
 }  // namespace pi

@@ -26,6 +26,16 @@ int        cold_layer_q4(ColdPath * c, int il, pi_model * m, hipStream_t st, boo
 // its whole FFN (gate/up/down partial vectors) is queued at once and only the final reduction waits for the host share.
 int        cold_layer_f16(ColdPath * c, int il, pi_model * m, hipStream_t st, bool capture);
 
+// Q4_0 hybrid layers with nothing launched between the two halves: the stream holds hand-over kernels, a service thread computes the
+// host share when the device signals and answers through flag words in pinned memory.  cold_post_token announces one token's
+// hybrid layers to the service thread (call it once per token whose kernels are queued with cold_layer_q4_queue), cold_drain
+// confirms after a stream synchronisation that every hand-over completed.  PI_COLD_SYNC=1 keeps the launching thread in the loop.
+bool       cold_async(const ColdPath * c);
+bool       cold_every_layer_async(const ColdPath * c);   // no hybrid layer needs the launching thread: the token loop can be one graph
+int        cold_post_token(ColdPath * c);
+int        cold_drain(ColdPath * c);
+int        cold_layer_q4_queue(ColdPath * c, int il, pi_model * m, hipStream_t st);
+
 int add_vec(float * y, const float * a, int n, hipStream_t st);
 // dst = ((cold + hot) + r1) [+ r2]; `cold` may be pinned host memory; `keep` (optional) receives cold + hot
 int merge_shares(float * dst, const float * cold, const float * hot, const float * r1, const float * r2, float * keep, int n, hipStream_t st);

@@ -229,7 +229,9 @@ int layer_forward(pi_model * m, int il, bool last_token) {
         const void * gp = falcon ? nullptr : gate.dev;
         const bool cap = m->capture && last_token;
         if (layer_hybrid && !m->rest_on_gpu) {
-            PI_TRY(pi::cold_layer_q4(m->cold, il, m, st, cap));
+            // nothing is launched between the two halves unless the parity hooks are on: the stream waits for the host threads itself
+            if (pi::cold_async(m->cold) && !m->capture) PI_TRY(pi::cold_layer_q4_queue(m->cold, il, m, st));
+            else PI_TRY(pi::cold_layer_q4(m->cold, il, m, st, cap));
         } else {
             // every neuron on the GPU, or the non-resident neurons' rows read from pinned host memory by the same two launches
             const uint32_t * hw = layer_hybrid ? m->hot_words[il] : nullptr;
@@ -297,6 +299,8 @@ int layer_forward(pi_model * m, int il, bool last_token) {
 int token_forward(pi_model * m, bool want_logits, bool last_token) {
     const pi_hparams & hp = m->hp;
     hipStream_t st = m->stream;
+    // the host threads expect this token's hybrid layers (a graph under construction runs nothing: its replays are announced one by one)
+    if (pi::cold_async(m->cold) && !m->capture && !m->building_graph) PI_TRY(pi::cold_post_token(m->cold));
     PI_TRY(pi_k_embed(m->glob[PI_T_TOK_EMBD].type, m->glob[PI_T_TOK_EMBD].dev, hp.n_embd, m->d_token, m->x, st));
     for (int il = 0; il < hp.n_layer; ++il) PI_TRY(layer_forward(m, il, last_token));
     if (want_logits) {
@@ -704,6 +708,7 @@ int pi_model_decode(pi_model * m, const int32_t * tokens, int n_tokens, int n_pa
     PI_HIP_TRY(hipMemsetAsync(m->d_step, 0, 4, m->stream));
     PI_TRY(launch_advance(m));
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    if (m->cold) PI_TRY(pi::cold_drain(m->cold));
     int32_t tok = -1;
     PI_TRY(pi_memcpy_d2h(&tok, m->d_token, 4));
     if (logits_out) PI_TRY(pi_memcpy_d2h(logits_out, m->logits, sizeof(float) * m->hp.n_vocab));
@@ -722,10 +727,15 @@ int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * m
 
     // PI_NO_GRAPH=1 issues the same launches eagerly (useful under tracing tools that cannot follow graph replays)
     const char * no_graph = getenv("PI_NO_GRAPH");
-    const bool use_graph = !(m->hybrid && !m->rest_on_gpu) && !m->capture && !(no_graph && no_graph[0] == '1');
+    // a model with host threads replays a graph too when every hybrid layer hands over through the stream's own wait kernels
+    const bool host_in_loop = m->hybrid && !m->rest_on_gpu && !pi::cold_every_layer_async(m->cold);
+    const bool use_graph = !host_in_loop && !m->capture && !(no_graph && no_graph[0] == '1');
+    const bool announce = use_graph && pi::cold_async(m->cold);
     if (use_graph && !m->graph_exec) {
         PI_HIP_TRY(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
+        m->building_graph = true;
         int rc = token_forward(m, true, false);
+        m->building_graph = false;
         if (rc == PI_OK) rc = launch_advance(m);
         hipGraph_t g = nullptr;
         const hipError_t e = hipStreamEndCapture(m->stream, &g);
@@ -737,6 +747,7 @@ int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * m
     PI_HIP_TRY(hipEventRecord(m->ev0, m->stream));
     for (int s = 0; s < n_steps; ++s) {
         if (use_graph) {
+            if (announce) PI_TRY(pi::cold_post_token(m->cold));
             PI_HIP_TRY(hipGraphLaunch(m->graph_exec, m->stream));
         } else {
             PI_TRY(token_forward(m, true, false));
@@ -745,6 +756,7 @@ int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * m
     }
     PI_HIP_TRY(hipEventRecord(m->ev1, m->stream));
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    if (m->cold) PI_TRY(pi::cold_drain(m->cold));
     if (ms_out) PI_HIP_TRY(hipEventElapsedTime(ms_out, m->ev0, m->ev1));
     PI_TRY(pi_memcpy_d2h(out_tokens, m->d_out_tokens, sizeof(int32_t) * n_steps));
     return PI_OK;

@@ -44,6 +44,7 @@ struct pi_model {
     hipGraph_t graph = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
 
+    bool building_graph = false;          // token_forward is being recorded into a graph, not run
     bool capture = false;
     float *cap_ffn = nullptr, *cap_logits = nullptr, *cap_src = nullptr;       // device
     pi::ColdPath * cold = nullptr;

@@ -1281,14 +1281,19 @@ struct __attribute__((packed)) pi_q8_host_block { uint16_t d; int8_t qs[32]; };
 
 // SPLIT: the neurons outside the hot words are computed here too, from a second pair of matrices that holds exactly those
 // neurons' rows in ascending order (rows in pinned host memory, fetched over the host link by the loads below).
-template <int RCH, bool GATE, bool SPLIT>
+// PHASE 1 / 2 cut the launch in two for a hybrid layer whose host share should start as early as possible: 1 stops behind the
+// logits (to `logits` and `logits2`), the mask words and the Q8_0 blocks of the input; 2 reads the logits back from `logits2`
+// instead of computing them, and writes h only for the neurons of the hot words (h or 0): the other entries of that vector
+// belong to the host.
+template <int RCH, bool GATE, bool SPLIT, int PHASE = 0>
 __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
                                                                      const pi_block_q4_0 * __restrict__ Wup, const pi_block_q4_0 * __restrict__ Wgate,
                                                                      const pi_block_q4_0 * __restrict__ Wup_rest, const pi_block_q4_0 * __restrict__ Wgate_rest,
                                                                      const float * __restrict__ x, NormArgs na, float thr,
                                                                      const uint32_t * __restrict__ hot_words, const int32_t * __restrict__ hot_prefix,
                                                                      float * __restrict__ logits, uint32_t * __restrict__ words, uint32_t * __restrict__ words_hot,
-                                                                     float * __restrict__ h_dense, pi_q8_host_block * __restrict__ xq_out) {
+                                                                     float * __restrict__ h_dense, pi_q8_host_block * __restrict__ xq_out,
+                                                                     float * __restrict__ logits2) {
     constexpr int cols = 4096, r = RCH * 512, nb = cols / 32, CH = kPfChunk;
     __shared__ float  lg[32];
     __shared__ double red[2][kPfWaves];
@@ -1300,15 +1305,20 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
 
     // ---- A: loads ------------------------------------------------------------------------------------------
     pi_u32x4 a[4][RCH];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < RCH; ++j) a[i][j] = pi_ld_stream(W2 + (size_t)(n0 + wave * 4 + i) * r + (j * PI_WAVE + lane) * 8);
     float4 hv[RCH][2];
+    float logit_in = 0.0f;
+    if (PHASE != 2) {
 #pragma unroll
-    for (int j = 0; j < RCH; ++j) {
-        hv[j][0] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8);
-        hv[j][1] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8 + 4);
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < RCH; ++j) a[i][j] = pi_ld_stream(W2 + (size_t)(n0 + wave * 4 + i) * r + (j * PI_WAVE + lane) * 8);
+#pragma unroll
+        for (int j = 0; j < RCH; ++j) {
+            hv[j][0] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8);
+            hv[j][1] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8 + 4);
+        }
+    } else {
+        logit_in = logits2[n0 + (lane & 31)];
     }
     const uint32_t hot = hot_words ? hot_words[blockIdx.x] : 0xFFFFFFFFu;
     const int base_row = hot_prefix ? hot_prefix[blockIdx.x] : n0;
@@ -1326,7 +1336,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
         }
     }
     // ---- A: logits (the CPU path rounds the hidden vector to fp16 before the dot, ggml.c:9703-9716) ------------
-    {
+    if (PHASE != 2) {
         pi_u32x4 hr[RCH];
 #pragma unroll
         for (int j = 0; j < RCH; ++j) {
@@ -1411,14 +1421,20 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
         if (sub == 0) { const uint16_t db = pi_f16_bits(dq); __builtin_memcpy(&ob->d, &db, 2); }
     }
     // ---- activity word (identical in every wave; lg is complete after the barrier above) -----------------------
-    const float my_logit = lg[lane & 31];
+    const float my_logit = PHASE == 2 ? logit_in : lg[lane & 31];
     const bool my_act = !(my_logit < thr);
     const uint32_t mask = (uint32_t)__ballot(my_act);
     const uint32_t sel = SPLIT ? mask : mask & hot;
     if (wave == 0) {
-        if (lane < 32) { if (logits) logits[n0 + lane] = my_logit; if (!((sel >> lane) & 1u)) h_dense[n0 + lane] = 0.0f; }
+        if (lane < 32) {
+            if (PHASE != 2 && logits) logits[n0 + lane] = my_logit;
+            if (PHASE == 1) logits2[n0 + lane] = my_logit;
+            if (PHASE == 0 && !((sel >> lane) & 1u)) h_dense[n0 + lane] = 0.0f;
+            if (PHASE == 2 && ((hot >> lane) & 1u) && !((sel >> lane) & 1u)) h_dense[n0 + lane] = 0.0f;
+        }
         if (lane == 0) { words[blockIdx.x] = mask; if (words_hot) words_hot[blockIdx.x] = sel; }
     }
+    if (PHASE == 1) return;
     // ---- B -------------------------------------------------------------------------------------------------
     const int n = __popc(sel);
     const int shift = (sub >> 1) * 4, qoff = (sub & 1) * 8;
@@ -3426,6 +3442,38 @@ __global__ __launch_bounds__(1024) void argmax_batch_kernel(const float * __rest
 
 __global__ void step_advance_kernel(int32_t * step) { if (threadIdx.x == 0) *step += 1; }
 
+// Hand-over points between the device and host threads that compute a share of a layer (hybrid layers).  Both sides count the
+// hand-overs; the device's count lives in *seq.  `flags` is pinned host memory: word 0 is written by the device, words 16 and 32
+// (their own cache lines) by the host, word 48 is the host's stop word; word 8 is a second device-written word.
+//   host_signal_kernel: everything queued before it on the stream is complete and visible to the host (a kernel boundary releases
+//                       at system scope): publish *seq in flags[word] (word 0 or 8), after advancing it when a new hand-over starts.
+//   host_wait_kernel:   returns once flags[slot] has reached *seq.  The wait is bounded: after `limit` ticks of the 100 MHz clock, or
+//                       when the host has set its stop word, the kernel records the failure in *status and returns, so the stream
+//                       always drains; later waits then return at once.
+__global__ void host_signal_kernel(uint32_t * __restrict__ seq, uint32_t * __restrict__ flags, int word, int advance) {
+    if (threadIdx.x == 0) {
+        uint32_t s = *seq;
+        if (advance) { s += 1u; *seq = s; }
+        __hip_atomic_store(flags + word, s, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
+}
+__global__ void host_wait_kernel(const uint32_t * __restrict__ seq, const uint32_t * __restrict__ flags, int slot, uint32_t * __restrict__ status,
+                                 unsigned long long limit) {
+    if (threadIdx.x != 0) return;
+    const uint32_t want = *seq;
+    if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0u) return;
+    const unsigned long long t0 = wall_clock64();
+    for (;;) {
+        const uint32_t v = __hip_atomic_load(flags + slot, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_SYSTEM);
+        if ((int32_t)(v - want) >= 0) return;
+        if (__hip_atomic_load(flags + 48, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0u || wall_clock64() - t0 > limit) {
+            __hip_atomic_store(status, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM);
+            return;
+        }
+        __builtin_amdgcn_s_sleep(4);
+    }
+}
+
 NormArgs to_norm(const pi_norm * n) {
     NormArgs a{0, 0.0f, nullptr, nullptr};
     if (n) { a.kind = n->kind; a.eps = n->eps; a.w = n->w; a.b = n->b; }
@@ -3705,13 +3753,42 @@ int pi_k_pred_upgate_q4_split(const void * fc2_f16, int ff, int r, const float *
     const pi_block_q4_0 * u = (const pi_block_q4_0 *)up_q4; const pi_block_q4_0 * g = (const pi_block_q4_0 *)gate_q4;
     const dim3 grid(ff / 32), block(kPfBlock);
     const pi_block_q4_0 * ur = (const pi_block_q4_0 *)up_rest_q4; const pi_block_q4_0 * gr = (const pi_block_q4_0 *)gate_rest_q4;
-#define PI_PQ_LAUNCH(RCH, GATE, SPLIT) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, GATE, SPLIT>), grid, block, 0, st, w2, hidden, u, g, ur, gr, x, na, threshold, hot_words, hot_prefix, logits, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)xq8_out)
+#define PI_PQ_LAUNCH(RCH, GATE, SPLIT) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, GATE, SPLIT>), grid, block, 0, st, w2, hidden, u, g, ur, gr, x, na, threshold, hot_words, hot_prefix, logits, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)xq8_out, nullptr)
 #define PI_PQ_LAUNCH_S(RCH, GATE) do { if (ur) PI_PQ_LAUNCH(RCH, GATE, true); else PI_PQ_LAUNCH(RCH, GATE, false); } while (0)
     if (r == 1024) { if (g) PI_PQ_LAUNCH_S(2, true); else PI_PQ_LAUNCH_S(2, false); }
     else           { if (g) PI_PQ_LAUNCH_S(1, true); else PI_PQ_LAUNCH_S(1, false); }
 #undef PI_PQ_LAUNCH_S
 #undef PI_PQ_LAUNCH
     return pi::check_launch("pi_k_pred_upgate_q4");
+}
+
+int pi_k_pred_q4_logits(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
+                        float * logits, float * logits_dev, void * xq8_out, pi_workspace * ws, pi_stream_t stream) {
+    if (!fc2_f16 || !hidden || !x || !logits_dev || !ws) return pi::fail(PI_E_ARG, "pi_k_pred_q4_logits: null pointer");
+    if (!pi_k_pred_upgate_q4_supported(ff, r, cols) || ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_UNSUPPORTED, "pi_k_pred_q4_logits: shape outside the fused kernel or the workspace");
+    const NormArgs na = to_norm(norm);
+    if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_pred_q4_logits: vectors must be 16-byte aligned");
+    const dim3 grid(ff / 32), block(kPfBlock);
+    const pi_block_q4_0 * none = nullptr;
+#define PI_PQ1(RCH) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, false, false, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, none, x, na, threshold, (const uint32_t *)nullptr, (const int32_t *)nullptr, logits, ws->words, (uint32_t *)nullptr, (float *)nullptr, (pi_q8_host_block *)xq8_out, logits_dev)
+    if (r == 1024) PI_PQ1(2); else PI_PQ1(1);
+#undef PI_PQ1
+    return pi::check_launch("pi_k_pred_q4_logits");
+}
+
+int pi_k_upgate_q4_hot_rows(int ff, float threshold, const void * up_q4, const void * gate_q4, int cols, const float * x, const pi_norm * norm,
+                            const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense, pi_workspace * ws, pi_stream_t stream) {
+    if (!up_q4 || !x || !hot_words || !hot_prefix || !logits_dev || !h_dense || !ws) return pi::fail(PI_E_ARG, "pi_k_upgate_q4_hot_rows: null pointer");
+    if (cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_UNSUPPORTED, "pi_k_upgate_q4_hot_rows: cols must be 4096, ff % 32 == 0, within the workspace");
+    const NormArgs na = to_norm(norm);
+    if ((((uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_upgate_q4_hot_rows: vectors must be 16-byte aligned");
+    const dim3 grid(ff / 32), block(kPfBlock);
+    const pi_block_q4_0 * none = nullptr;
+    const pi_block_q4_0 * u = (const pi_block_q4_0 *)up_q4; const pi_block_q4_0 * g = (const pi_block_q4_0 *)gate_q4;
+#define PI_PQ2(GATE) hipLaunchKernelGGL((pred_upgate_q4_kernel<1, GATE, false, 2>), grid, block, 0, (hipStream_t)stream, (const __half *)nullptr, (const float *)nullptr, u, g, none, none, x, na, threshold, hot_words, hot_prefix, (float *)nullptr, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)nullptr, const_cast<float *>(logits_dev))
+    if (g) PI_PQ2(true); else PI_PQ2(false);
+#undef PI_PQ2
+    return pi::check_launch("pi_k_upgate_q4_hot_rows");
 }
 
 int pi_k_axpy_q4_partials(const void * down_t_q4, int cols, int ff, const float * h, const uint32_t * hot_words, const int32_t * hot_prefix,
@@ -4256,6 +4333,19 @@ int pi_k_embed_batch(const void * table_f16, int cols, const int32_t * tokens, i
     if (!table_f16 || !tokens || !x || cols <= 0 || T <= 0 || T > kChunkMaxT) return pi::fail(PI_E_ARG, "pi_k_embed_batch: bad arguments");
     hipLaunchKernelGGL(embed_f16_batch_kernel, dim3((cols + 255) / 256, T), dim3(256), 0, (hipStream_t)stream, (const __half *)table_f16, cols, tokens, x);
     return pi::check_launch("pi_k_embed_batch");
+}
+
+int pi_k_host_signal(uint32_t * seq, uint32_t * flags_pinned, int word, int advance, pi_stream_t stream) {
+    if (!seq || !flags_pinned || (word != 0 && word != 8)) return pi::fail(PI_E_ARG, "pi_k_host_signal: bad arguments (word 0 or 8)");
+    hipLaunchKernelGGL(host_signal_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, seq, flags_pinned, word, advance);
+    return pi::check_launch("pi_k_host_signal");
+}
+int pi_k_host_wait(const uint32_t * seq, const uint32_t * flags_pinned, int slot, uint32_t * status_pinned, double limit_seconds, pi_stream_t stream) {
+    if (!seq || !flags_pinned || !status_pinned || (slot != 16 && slot != 32) || !(limit_seconds > 0.0) || limit_seconds > 60.0)
+        return pi::fail(PI_E_ARG, "pi_k_host_wait: bad arguments (slot 16 or 32, 0 < limit <= 60 s)");
+    hipLaunchKernelGGL(host_wait_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, seq, flags_pinned, slot, status_pinned,
+                       (unsigned long long)(limit_seconds * 1e8));
+    return pi::check_launch("pi_k_host_wait");
 }
 
 int pi_k_embed_batch_q4(const void * table_q4, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream) {

@@ -54,6 +54,13 @@ void * pi_malloc(size_t bytes) {
     return p;
 }
 int pi_free(void * dptr) { if (dptr) PI_HIP_TRY(hipFree(dptr)); return PI_OK; }
+void * pi_malloc_host(size_t bytes) {
+    void * p = nullptr;
+    const hipError_t e = hipHostMalloc(&p, bytes ? bytes : 1, hipHostMallocCoherent);
+    if (e != hipSuccess) { pi::hip_fail(e, "hipHostMalloc"); return nullptr; }
+    return p;
+}
+int pi_free_host(void * hptr) { if (hptr) PI_HIP_TRY(hipHostFree(hptr)); return PI_OK; }
 int pi_memset(void * dptr, int byte, size_t bytes) { PI_HIP_TRY(hipMemset(dptr, byte, bytes)); return PI_OK; }
 int pi_memcpy_h2d(void * dptr, const void * host, size_t bytes) { PI_HIP_TRY(hipMemcpy(dptr, host, bytes, hipMemcpyHostToDevice)); return PI_OK; }
 int pi_memcpy_d2h(void * host, const void * dptr, size_t bytes) { PI_HIP_TRY(hipMemcpy(host, dptr, bytes, hipMemcpyDeviceToHost)); return PI_OK; }

@@ -35,6 +35,8 @@ _SIGS = {
     "pi_device_name": (_i, [C.c_char_p, _sz]),
     "pi_malloc": (_vp, [_sz]),
     "pi_free": (_i, [_vp]),
+    "pi_malloc_host": (_vp, [_sz]),
+    "pi_free_host": (_i, [_vp]),
     "pi_memset": (_i, [_vp, _i, _sz]),
     "pi_memcpy_h2d": (_i, [_vp, _vp, _sz]),
     "pi_memcpy_d2h": (_i, [_vp, _vp, _sz]),
@@ -85,6 +87,10 @@ _SIGS = {
     "pi_k_dequant_q4_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "pi_k_assemble_rows_f16": (_i, [_vp, _vp, _vp, _vp, _i, _i, _vp, _vp]),
     "pi_k_embed_batch_q4": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
+    "pi_k_host_signal": (_i, [_vp, _vp, _i, _i, _vp]),
+    "pi_k_pred_q4_logits": (_i, [_vp, _i, _i, _vp, _f, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_upgate_q4_hot_rows": (_i, [_i, _f, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_host_wait": (_i, [_vp, _vp, _i, _vp, C.c_double, _vp]),
     "pi_gemm_lib_create": (_vp, [C.c_size_t]),
     "pi_gemm_lib_destroy": (_i, [_vp]),
     "pi_gemm_lib_f16": (_i, [_vp, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),

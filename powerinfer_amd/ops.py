@@ -198,6 +198,73 @@ class SparseFFN:
         return dict(logits=self.logits.download(np.float32), h=h, xq8=xq8.download(np.uint8),
                     n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32))
 
+    def forward_q4_handover(self, x_ffn, x_pred, host_h, host_out, limit_s=20.0):
+        """The same layer with the host share computed while the stream runs, nothing launched in between (what the decode loop
+        queues for a hybrid Q4_0 layer): pi_k_pred_q4_logits -> pi_k_host_signal -> pi_k_upgate_q4_hot_rows -> pi_k_host_signal ->
+        pi_k_host_wait -> pi_k_axpy_q4_partials (h in pinned memory) -> pi_k_host_wait -> pi_k_axpy_q4_reduce (+ the host share's
+        output from pinned memory).  Everything is queued first; then this thread plays the host side: once the logits have
+        arrived host_h(logits, xq8) returns {neuron: h} for the host's neurons, and once the resident neurons' h has arrived
+        host_out(h_full) returns the host share of the output.  Returns dict(logits, h, n_active, out, status)."""
+        import ctypes as C
+        import time
+        L = self.L
+        if self.wtype != pl.Q4_0 or not L.pi_k_pred_upgate_q4_supported(self.ff, self.r, self.d):
+            raise pl.PiError("forward_q4_handover: type or shape outside the fused kernels")
+        hw, hp = self._hot_tables()
+        if hw is None:
+            raise pl.PiError("forward_q4_handover: needs a hot/cold split")
+        p = lambda b: b.ptr if b is not None else None  # noqa: E731
+
+        def pinned(nbytes, dtype):
+            ptr = L.pi_malloc_host(nbytes)
+            if not ptr:
+                raise pl.PiError("pi_malloc_host: " + L.pi_last_error().decode())
+            arr = np.frombuffer((C.c_char * nbytes).from_address(ptr), dtype=dtype)
+            arr[...] = 0
+            return ptr, arr
+
+        flags_p, flags = pinned(64 * 4, np.uint32)
+        lg_p, lg = pinned(self.ff * 4, np.float32)
+        h_p, h = pinned(self.ff * 4, np.float32)
+        out_p, out_host = pinned(self.d * 4, np.float32)
+        xq_p, xq = pinned(self.d // 32 * 34, np.uint8)
+        seq, status, lg_dev = DevBuf.zeros(4), DevBuf.zeros(4), DevBuf(self.ff * 4)
+        try:
+            self.x.upload(np.asarray(x_ffn, np.float32))
+            self.xp.upload(np.asarray(x_pred, np.float32))
+            nrm = pl.norm_arg(self.norm_kind, self.eps, self.norm_w, self.norm_b)
+            check(L.pi_k_gemv(pl.F16, self.fc1.ptr, self.r, self.d, self.xp.ptr, None, pl.EPI_RELU, None, None, self.hidden.ptr, None), "fc1")
+            check(L.pi_k_pred_q4_logits(self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, self.d, self.x.ptr, nrm, lg_p, lg_dev.ptr, xq_p, self.ws, None), "pred_q4_logits")
+            check(L.pi_k_host_signal(seq.ptr, flags_p, 0, 1, None), "signal")
+            check(L.pi_k_upgate_q4_hot_rows(self.ff, self.thr, self.up.ptr, p(self.gate), self.d, self.x.ptr, nrm, hw.ptr, hp.ptr, lg_dev.ptr, h_p, self.ws, None), "hot_rows")
+            check(L.pi_k_host_signal(seq.ptr, flags_p, 8, 0, None), "signal")
+            check(L.pi_k_host_wait(seq.ptr, flags_p, 16, status.ptr, limit_s, None), "wait")
+            check(L.pi_k_axpy_q4_partials(self.down.ptr, self.d, self.ff, h_p, hw.ptr, hp.ptr, self.ws, None), "axpy_q4_partials")
+            check(L.pi_k_host_wait(seq.ptr, flags_p, 32, status.ptr, limit_s, None), "wait")
+            check(L.pi_k_axpy_q4_reduce(self.ff, self.d, pl.EPI_ADD, out_p, None, self.out.ptr, self.n_active.ptr, self.ws, None), "axpy_q4_reduce")
+
+            def wait_flag(word):
+                t0 = time.time()
+                while int(flags[word]) != 1:
+                    if time.time() - t0 > limit_s:
+                        flags[48] = 1
+                        raise pl.PiError("forward_q4_handover: the device never signalled word %d" % word)
+            wait_flag(0)
+            for j, v in host_h(lg.copy(), xq.copy()).items():
+                h[j] = v
+            flags[16] = 1
+            wait_flag(8)
+            out_host[...] = host_out(h.copy())
+            flags[32] = 1
+            pl.sync()
+            return dict(logits=lg.copy(), h=h.copy(), n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32),
+                        status=int(status.download(np.uint32)[0]))
+        finally:
+            pl.sync()
+            del flags, lg, h, out_host, xq
+            for ptr in (flags_p, lg_p, h_p, out_p, xq_p):
+                L.pi_free_host(ptr)
+
     def close(self):
         if self.ws:
             self.L.pi_workspace_destroy(self.ws)

@@ -285,6 +285,53 @@ def test_q4_fused_route_hybrid_share():
     ffn.close()
 
 
+def test_q4_hybrid_layer_with_stream_handovers():
+    """The hybrid Q4_0 layer as the decode loop queues it: predictor, signal, resident up/gate rows, signal, wait, down projection,
+    wait, reduction - all queued at once, the host share (here numpy, from the logits and the Q8_0 input the device wrote to pinned
+    memory) computed while the stream waits for it.  The resident share is bit-identical to the route with a launch boundary per
+    exchange (pi_k_pred_upgate_q4 -> fill h -> axpy -> reduce), and GPU share + host share equals every neuron on the CPU."""
+    from powerinfer_amd.ops import SparseFFN
+    d, ff, r = 4096, 4096, 512
+    L = synth.make_ffn_layer(seed=34, d=d, ff=ff, r=r, wtype=ol.Q4_0, mean_rate=0.15, T=1)
+    gid, bucket = synth.gpu_split(L["p"], 0.6)
+    cold = gid == 0
+    ffn = SparseFFN(d, ff, r, ol.Q4_0, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], bucket=bucket)
+    x = L["x"][0]
+    ref, got = {}, {}
+
+    def fill(h):
+        ref["full"] = under(L, d, ff, ol.Q4_0, True, x, ffn.logits.download(np.float32))
+        h[cold] = ref["full"]["h"][cold]
+        return h
+    base = ffn.forward_q4_fused(x, x, fill_h=fill)
+
+    def cold_share(hm):
+        q, dh = q8_blocks_np(hm)
+        rows = np.nonzero(cold & (q != 0))[0]
+        v, dw = q4_rows_np(L["down_t"], rows, d)
+        contrib = (v * q[rows, None]).astype(np.float32) * (np.repeat(dw, 32, axis=1) * dh[rows, None])
+        return contrib.sum(0, dtype=np.float32)
+
+    def host_h(logits, xq8):
+        assert np.array_equal(xq8, base["xq8"])                # the Q8_0 blocks of the normalised input, as the one-launch route writes them
+        got["full"] = under(L, d, ff, ol.Q4_0, True, x, logits)
+        act = np.nonzero(cold & ~(logits < 0.0))[0]
+        return {int(j): got["full"]["h"][j] for j in act}
+
+    def host_out(h_full):
+        got["h_full"] = h_full
+        return cold_share(h_full)
+    res = ffn.forward_q4_handover(x, x, host_h, host_out)
+    assert res["status"] == 0
+    assert np.array_equal(res["logits"], base["logits"])
+    hm = base["h"].copy(); hm[cold] = ref["full"]["h"][cold]
+    assert np.array_equal(got["h_full"], hm)                    # resident entries from the device, the others from the host, zeros elsewhere
+    assert res["n_active"] == base["n_active"]
+    assert np.array_equal(res["out"], base["out"] + cold_share(hm))      # same partial sums, host share added by the reduction
+    assert rel_err(res["out"], got["full"]["out"]) < FFN_REL_TOL
+    ffn.close()
+
+
 @pytest.mark.parametrize("wtype", [ol.F16, ol.Q4_0])
 def test_hybrid_split_gpu_share(wtype):
     """Config 2 split: the GPU holds the hottest 60 % of neurons (compact matrices + gpu_bucket) and

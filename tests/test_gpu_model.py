@@ -342,6 +342,36 @@ def test_q4_split_rest_read_by_the_gpu_matches_host_threads():
         Model(hp3).load(synth.make_model(hp3))
 
 
+@pytest.mark.parametrize("arch", ["llama-7b", "falcon-4096"])
+def test_q4_split_stream_handovers_match_launch_per_exchange(arch, monkeypatch):
+    """Hybrid Q4_0 layers hand over to the host threads through wait kernels in the stream (one graph replay per token, a service
+    thread on the host); PI_COLD_SYNC=1 keeps the launching thread in the loop with an event wait and a launch per exchange.  Same
+    kernels' arithmetic, same host arithmetic: logits and greedy tokens are bit-identical, across two generate calls."""
+    from powerinfer_amd.model import Model
+    if arch == "llama-7b":
+        hp = synth.hparams("llama-7b", n_layer=3, n_ctx=96, seed=14, wtype=synth.Q4_0, hot_frac=0.6)
+    else:
+        hp = synth.hparams("falcon-tiny", n_embd=4096, n_ff=8192, n_rank=512, n_head=64, n_head_kv=8, n_layer=2, n_vocab=4096,
+                           n_ctx=96, seed=15, wtype=synth.Q4_0, hot_frac=0.5)
+    model = synth.make_model(hp)
+    prompt = np.random.default_rng(5).integers(0, hp.n_vocab, 9).astype(np.int32)
+    outs = []
+    for sync in (False, True):
+        if sync:
+            monkeypatch.setenv("PI_COLD_SYNC", "1")
+        else:
+            monkeypatch.delenv("PI_COLD_SYNC", raising=False)
+        gm = Model(hp).load(model)
+        tok, lg = gm.decode(prompt, 0)
+        t1, _ = gm.generate(20)
+        t2, _ = gm.generate(7)
+        tok3, lg3 = gm.decode([int(t2[-1])], len(prompt) + 27)
+        outs.append((tok, lg, list(map(int, t1)) + list(map(int, t2)), tok3, lg3))
+        gm.close()
+    assert outs[0][0] == outs[1][0] and outs[0][2] == outs[1][2] and outs[0][3] == outs[1][3]
+    assert np.array_equal(outs[0][1], outs[1][1]) and np.array_equal(outs[0][4], outs[1][4])
+
+
 @pytest.mark.parametrize("arch,wtype", [("llama-tiny", synth.F16), ("llama-tiny", synth.Q4_0), ("falcon-tiny", synth.F16)])
 def test_hybrid_split_matches_all_cold_oracle(arch, wtype):
     """Config-2 style partial split: the hottest 60 % of each layer's neurons live on the GPU (compact matrices +

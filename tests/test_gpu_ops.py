@@ -308,3 +308,47 @@ def test_k_shift_and_compaction(mode):
     pl.sync()
     after = kd.download(np.float16).reshape(rows, n_ctx, hd)
     assert np.array_equal(after[:, :keep.size], got[:, keep])
+
+
+def test_host_signal_and_bounded_wait():
+    """The hand-over kernels between the stream and host threads: a signal publishes the hand-over count in pinned memory once the
+    work before it is complete; a wait returns when the host's word has reached that count, and gives up after its limit (here a
+    millisecond, with a host that never answers) by recording the failure, after which later waits return at once - the stream
+    always drains."""
+    import ctypes as C
+    import time
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    fp = L.pi_malloc_host(64 * 4)
+    assert fp
+    flags = np.frombuffer((C.c_char * 256).from_address(fp), dtype=np.uint32)
+    flags[...] = 0
+    seq, status = pl.DevBuf.zeros(4), pl.DevBuf.zeros(4)
+    try:
+        pl.check(L.pi_k_host_signal(seq.ptr, fp, 0, 1, None), "signal")
+        pl.check(L.pi_k_host_signal(seq.ptr, fp, 8, 0, None), "signal")
+        pl.sync()
+        assert int(flags[0]) == 1 and int(flags[8]) == 1 and int(seq.download(np.uint32)[0]) == 1
+        flags[16] = 1                                           # the host has already answered hand-over 1
+        pl.check(L.pi_k_host_wait(seq.ptr, fp, 16, status.ptr, 5.0, None), "wait")
+        pl.sync()
+        assert int(status.download(np.uint32)[0]) == 0
+        pl.check(L.pi_k_host_wait(seq.ptr, fp, 32, status.ptr, 5.0, None), "wait")      # answered while the kernel polls
+        time.sleep(0.05)
+        flags[32] = 1
+        pl.sync()
+        assert int(status.download(np.uint32)[0]) == 0
+        pl.check(L.pi_k_host_signal(seq.ptr, fp, 0, 1, None), "signal")                 # hand-over 2, never answered
+        t0 = time.time()
+        pl.check(L.pi_k_host_wait(seq.ptr, fp, 16, status.ptr, 1e-3, None), "wait")
+        pl.sync()
+        assert int(status.download(np.uint32)[0]) == 1 and int(flags[0]) == 2
+        pl.check(L.pi_k_host_wait(seq.ptr, fp, 32, status.ptr, 30.0, None), "wait")     # returns at once: the status word is set
+        pl.sync()
+        assert time.time() - t0 < 5.0
+        assert L.pi_k_host_wait(seq.ptr, fp, 7, status.ptr, 1.0, None) != 0
+        assert L.pi_k_host_wait(seq.ptr, fp, 16, status.ptr, 1e9, None) != 0
+    finally:
+        pl.sync()
+        del flags
+        L.pi_free_host(fp)

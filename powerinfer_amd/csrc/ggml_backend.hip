@@ -220,19 +220,22 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const float * x, floa
     const float inv = (float)(1.0 / (red[0] + red[1] + red[2] + red[3]));
     for (int i = threadIdx.x; i < n; i += 256) yr[i] = __fmul_rn(yr[i], inv);
 }
-// x [hd, n_head, T] contiguous, pos[T]; mode 0 adjacent pairs, 2 NeoX halves (ggml.c:11163-11325, no YaRN)
-__global__ void rope_kernel(const float * x, const int32_t * pos, float * y, int hd, int n_head, int n_dims, int mode, float theta_scale, float freq_scale) {
+// x [hd, n_head, T] with element strides s1 (head) and s2 (token), pos[T]; mode 0 adjacent pairs, 2 NeoX halves (ggml.c:11163-11325 for
+// fp32, :11327-11460 for fp16, no YaRN).  fp16 is what the K-shift graph runs in place over a layer's K cache (llama.cpp:4332-4381):
+// the same arithmetic with a conversion on either side.  A pair belongs to one thread, so y may be x.
+template <typename E>
+__global__ void rope_kernel(const E * x, const int32_t * pos, E * y, size_t s1, size_t s2, size_t d1, size_t d2, int n_dims, int mode, float theta_scale, float freq_scale) {
     const int t = blockIdx.y, h = blockIdx.x, i = threadIdx.x;         // i = pair index < n_dims/2
-    const float * s = x + ((size_t)t * n_head + h) * hd; float * o = y + ((size_t)t * n_head + h) * hd;
+    const E * s = x + (size_t)t * s2 + (size_t)h * s1; E * o = y + (size_t)t * d2 + (size_t)h * d1;
     float theta = (float)pos[t];
     if (mode & 2) theta = __fmul_rn(theta, freq_scale);
     for (int j = 0; j < i; ++j) theta = __fmul_rn(theta, theta_scale);
     const float th = __fmul_rn(freq_scale, theta);
     const float c = cosf(th), sn = sinf(th);
     const int i0 = (mode & 2) ? i : 2 * i, i1 = (mode & 2) ? i + n_dims / 2 : 2 * i + 1;
-    const float x0 = s[i0], x1 = s[i1];
-    o[i0] = __fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, sn));
-    o[i1] = __fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, c));
+    const float x0 = (float)s[i0], x1 = (float)s[i1];
+    o[i0] = (E)__fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, sn));
+    o[i1] = (E)__fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, c));
 }
 struct Shape { int64_t ne[4]; size_t nb[4]; };
 // element-wise copy with type conversion between two 4-D strided tensors of the same element count (ggml_cpy)
@@ -417,15 +420,26 @@ bool op_elementwise(ggml_tensor * dst) {
 
 bool op_rope(ggml_tensor * dst) {
     const ggml_tensor * a = dst->src[0]; const ggml_tensor * p = dst->src[1];
-    if (a->type != GGML_TYPE_F32 || !contiguous(a) || !contiguous(dst) || !p || p->type != GGML_TYPE_I32 || a->ne[3] != 1) return false;
+    if ((a->type != GGML_TYPE_F32 && a->type != GGML_TYPE_F16) || dst->type != a->type || !p || p->type != GGML_TYPE_I32 || a->ne[3] != 1) return false;
+    const size_t es = tsize(a->type);
+    // rows of one head contiguous; heads and tokens at any stride that is a whole number of elements (views into the KV cache)
+    if (a->nb[0] != es || dst->nb[0] != es || a->nb[1] % es || a->nb[2] % es || dst->nb[1] % es || dst->nb[2] % es) return false;
     const int n_dims = dst->op_params[1], mode = dst->op_params[2];
     float freq_base, freq_scale, ext_factor;
     memcpy(&freq_base, dst->op_params + 5, 4); memcpy(&freq_scale, dst->op_params + 6, 4); memcpy(&ext_factor, dst->op_params + 7, 4);
     if ((mode != 0 && mode != 2) || ext_factor != 0.0f || n_dims != a->ne[0] || n_dims / 2 > 1024) return false;       // no GLM / YaRN / partial rotation here
+    if (a->backend == GGML_BACKEND_CPU && !contiguous(a)) return false;                                                // staged operands are copied as one block
+    if (dst->backend == GGML_BACKEND_CPU && !contiguous(dst)) return false;
     Temps tmp;
-    const float * ad = (const float *)dev_in(a, tmp); const int32_t * pd = (const int32_t *)dev_in(p, tmp); float * y = (float *)dev_out(dst, tmp);
+    const void * ad = dev_in(a, tmp); const int32_t * pd = (const int32_t *)dev_in(p, tmp); void * y = dev_out(dst, tmp);
     const float theta_scale = powf(freq_base, -2.0f / n_dims);
-    hipLaunchKernelGGL(rope_kernel, dim3((unsigned)a->ne[1], (unsigned)a->ne[2]), dim3(n_dims / 2), 0, 0, ad, pd, y, (int)a->ne[0], (int)a->ne[1], n_dims, mode, theta_scale, freq_scale);
+    const dim3 grid((unsigned)a->ne[1], (unsigned)a->ne[2]), block(n_dims / 2);
+    if (a->type == GGML_TYPE_F32)
+        hipLaunchKernelGGL(rope_kernel<float>, grid, block, 0, 0, (const float *)ad, pd, (float *)y, a->nb[1] / es, a->nb[2] / es, dst->nb[1] / es, dst->nb[2] / es,
+                           n_dims, mode, theta_scale, freq_scale);
+    else
+        hipLaunchKernelGGL(rope_kernel<__half>, grid, block, 0, 0, (const __half *)ad, pd, (__half *)y, a->nb[1] / es, a->nb[2] / es, dst->nb[1] / es, dst->nb[2] / es,
+                           n_dims, mode, theta_scale, freq_scale);
     finish_out(dst, y);
     return true;
 }

@@ -144,6 +144,19 @@ class Graph:
         params = [0, n_dims, mode, 0, 0, self._f32(freq_base), self._f32(freq_scale), self._f32(0.0), self._f32(1.0), self._f32(32.0), self._f32(1.0)]
         return self._node("ROPE", F32, list(a.ne), [a, pos], name, params=params)
 
+    def rope_inplace(self, a, pos, n_dims, mode, freq_base=10000.0, freq_scale=1.0, name="rope_inplace"):
+        """ggml_rope_custom_inplace (ggml.c:5222-5262 with inplace = true): the result is a view of a, so the rotation overwrites it."""
+        t = self.view(a, [a.ne[i] for i in range(4)], [a.nb[i] for i in range(1, 4)], 0, name)
+        self.nodes.pop()
+        t.op = OP["ROPE"]
+        t.src[0], t.src[1] = C.pointer(a), C.pointer(pos)
+        params = [0, n_dims, mode, 0, 0, self._f32(freq_base), self._f32(freq_scale), self._f32(0.0), self._f32(1.0), self._f32(32.0), self._f32(1.0)]
+        for i, v in enumerate(params):
+            t.op_params[i] = v
+        t._srcs = [a, pos]
+        self.nodes.append(t)
+        return t
+
     def get_rows(self, a, ids, name="get_rows"):                                # ggml.c:4925
         return self._node("GET_ROWS", F32, [a.ne[0], ids.ne[0]], [a, ids], name)
 

@@ -54,6 +54,35 @@ def test_rope_modes(golden, mode):
     assert np.abs(G.host(y) - g[f"rope{mode}_y"]).max() < 2e-5   # position 300: cosf/sinf of the device vs the host's, angles identical
 
 
+@pytest.mark.parametrize("mode", [0, 2])
+def test_k_shift_rope_in_place_over_a_cache_view(mode):
+    """The K-shift graph (llama.cpp:4332-4381): ggml_rope_custom_inplace over a 3-D view [hd, n_head_kv, n_ctx] of one layer's fp16 K
+    cache, the position operand holding each cell's delta.  Against the oracle's RoPE on the fp32 values of the same cells, rounded
+    to fp16 as ggml_compute_forward_rope_f16 stores them (ggml.c:11327-11460); the other layer's cells must stay untouched."""
+    hd, nkv, nctx, n_layer, il = 64, 2, 24, 2, 1
+    gqa = hd * nkv
+    rng = np.random.default_rng(40 + mode)
+    cache = rng.standard_normal(n_layer * nctx * gqa).astype(np.float16)
+    delta = rng.integers(-9, 1, nctx).astype(np.int32)
+    G = graph()
+    kc = G.on_gpu(G.new(F16, [n_layer * nctx * gqa], cache.copy().view(np.uint16), "cache_k"))     # the tensor's host buffer is overwritten on read-back
+    G.L.ggml_cuda_copy_to_device(C.byref(kc))
+    kv = G.on_gpu(G.view(kc, [hd, nkv, nctx], [hd * 2, gqa * 2], il * nctx * gqa * 2, "k_view"))
+    pos = G.new(I32, [nctx], delta, "K_shift")
+    G.on_gpu(G.rope_inplace(kv, pos, hd, mode, name="K_shifted"))
+    G.compute()
+    assert not G.cpu_run, G.cpu_run
+    got = G.host(kc, np.uint16).view(np.float16).reshape(n_layer, nctx, nkv, hd)
+    O = ol.oracle()
+    x = np.ascontiguousarray(cache.reshape(n_layer, nctx, nkv, hd)[il].astype(np.float32))
+    want = np.zeros_like(x)
+    O.pio_rope(P(x), hd, nkv, nctx, P(delta), hd, mode, 10000.0, 1.0, P(want))
+    assert np.array_equal(got[0], cache.reshape(n_layer, nctx, nkv, hd)[0])
+    diff = np.abs(got[il].astype(np.float32) - want.astype(np.float16).astype(np.float32))
+    assert (diff > 0).mean() < 5e-3 and diff.max() <= 2e-3 * np.abs(want).max()      # a handful of fp16 rounding ties from the device's cosf / sinf
+    assert not np.array_equal(got[il], cache.reshape(n_layer, nctx, nkv, hd)[il])
+
+
 @pytest.mark.parametrize("wtype", [F16, Q4_0])
 def test_dense_mul_mat_two_tokens_and_get_rows(golden, wtype):
     g = golden("ops")

@@ -59,6 +59,8 @@ def run_reference(tmp_path, name, share, n_threads):
     split.write_gpuidx(path + ".generated.gpuidx", splits, split.required_bytes(hp, splits))
     toks = [str(int(t)) for t in g["consumed"]]                 # every step consumes the reference's token (teacher forcing)
     env = dict(os.environ, REF_VRAM_GB="2", REF_ONE_CORE="1" if n_threads > 1 else "0")
+    if "shift" in g and int(g["shift"][0]) >= 0:                # the fixture's context shift: seq_rm + seq_shift before that step
+        env.update(REF_SHIFT_AT=str(int(g["shift"][0])), REF_N_KEEP=str(int(g["shift"][1])), REF_N_DISCARD=str(int(g["shift"][2])))
     r = subprocess.run([BIN, path, str(hp.n_ctx), str(n_threads), "0", out] + toks, env=env, capture_output=True, text=True, timeout=110)
     log = r.stdout + r.stderr
     assert r.returncode == 0, log[-3000:]
@@ -84,3 +86,55 @@ def test_reference_llama_cpp_runs_on_this_backend(name, share, n_threads, tmp_pa
     assert errs.max() < 1e-2, errs
     assert np.median(errs) < 2e-3, errs
     assert int((greedy == g["greedy"]).sum()) >= len(errs) - 1, (greedy, g["greedy"])
+
+
+@pytest.mark.timeout(120)
+@pytest.mark.parametrize("name", ["llama_f16_shift", "falcon_f16_shift"])
+def test_reference_context_shift_on_this_backend(name, tmp_path):
+    """The reference's KV ring on this backend: before step 12 its driver removes cells [2, 6) of the sequence and shifts the cells
+    behind them by -4 (llama_kv_cache_seq_rm + llama_kv_cache_seq_shift, llama.cpp:1683-1848), which makes llama_decode_internal
+    build the K-shift graph (a RoPE over the whole K cache with per-cell deltas, llama.cpp:4332-4381), search the ring for free
+    slots and mask the cells by position; every node of that runs through ggml_cuda_compute_forward here, and the logits of all
+    steps, before and after the shift, must match what the same llama.cpp wrote on the CPU alone."""
+    g, hp, log, greedy, logits = run_reference(tmp_path, name, 1.0, 1)
+    assert int(g["shift"][0]) == 12
+    errs = np.abs(logits[:, g["sample_idx"]] - g["logits_sample"]).max(1) / g["logits_absmax"]
+    assert errs.max() < 1e-2, errs
+    assert np.median(errs) < 2e-3, errs
+    assert int((greedy == g["greedy"]).sum()) >= len(errs) - 1, (greedy, g["greedy"])
+
+
+@pytest.mark.timeout(120)
+def test_reference_multi_sequence_kv_cells_on_this_backend(tmp_path):
+    """Three sequence ids in one KV cache, decoded in lockstep batches of three, then seq_rm / seq_shift / seq_cp (cells shared by
+    two sequences after the copy) and one more lockstep step: the reference's own cell bookkeeping and masks
+    (llama_kv_cache_find_slot, llama.cpp:1683-1743; KQ mask :6506-6547), with every graph node on this backend.  The logits of the
+    first and of the last step are compared with the CPU run of the same llama.cpp (tests/golden/ref_llama_seq_edits.npz)."""
+    if not os.path.exists(BIN):
+        pytest.skip("oracle/_ref/ref_llama_gpu is not built (needs the reference sources at build time)")
+    from powerinfer_amd import synth
+    g = dict(np.load(os.path.join(ROOT, "tests", "golden", "ref_llama_seq_edits.npz")))
+    hp, toks, last_pos, lines = fx.seq_edit_case()
+    model = synth.make_model(hp)
+    if not np.array_equal(fx.model_sha(model), g["model_sha"]):
+        pytest.skip("numpy generates a different stream here than where the fixture was written")
+    assert np.array_equal(toks, g["tokens"])
+    path, out, script = str(tmp_path / "m.powerinfer.gguf"), str(tmp_path / "out.bin"), str(tmp_path / "script.txt")
+    gguf.write_model(path, model, gguf.synthetic_tokenizer_kv(hp.n_vocab))
+    splits = [(np.ones(hp.n_ff, np.int32), np.arange(hp.n_ff, dtype=np.int32)) for _ in range(hp.n_layer)]
+    split.write_gpuidx(path + ".generated.gpuidx", splits, split.required_bytes(hp, splits))
+    with open(script, "w") as f:
+        f.write("\n".join(lines) + "\n")
+    r = subprocess.run([BIN, path, str(hp.n_ctx), "1", "0", out, "0"], env=dict(os.environ, REF_VRAM_GB="2", REF_SCRIPT=script),
+                       capture_output=True, text=True, timeout=110)
+    log = r.stdout + r.stderr
+    assert r.returncode == 0, log[-3000:]
+    assert "offloading v cache to GPU" in log and "offloading k cache to GPU" in log, log[-3000:]
+    raw = np.fromfile(out, np.uint8)
+    n_rows, n_vocab = (int(v) for v in raw[:8].view(np.int32))
+    logits = raw[8:].view(np.float32).reshape(n_rows, n_vocab)
+    assert n_rows == 3 * 9
+    for got, want in ((logits[:3], g["logits_step0"]), (logits[-3:], g["logits_last"])):
+        err = np.abs(got - want).max(1) / np.abs(want).max(1)
+        assert err.max() < 1e-2, err
+        assert np.array_equal(got.argmax(1), want.argmax(1))

@@ -22,6 +22,14 @@ struct BatchState {
     float *up_out = nullptr, *gate_out = nullptr;      // wide prompt chunks: dense gate/up products [T][n_ff]
     __half *h16 = nullptr;                             //                     and the FFN's hidden vector
     __half *w16 = nullptr, *w16t = nullptr;            // wide prompt chunks of Q4_0 / hybrid layers: one matrix as fp16, and the down projection with the neurons contiguous
+    // hybrid layers in wide prompt chunks: the non-resident rows of the next layer travel from pinned host memory into one of two device
+    // staging buffers on a copy stream while this layer computes (up | gate | down, each n_rest rows)
+    unsigned char * stage[2] = {nullptr, nullptr};
+    size_t stage_rows = 0, stage_row_bytes = 0;
+    hipStream_t copy_stream = nullptr;
+    hipEvent_t ev_copied[2] = {nullptr, nullptr}, ev_free[2] = {nullptr, nullptr};
+    bool free_recorded[2] = {false, false};
+    int staged_layer[2] = {-1, -1};
     hipGraphExec_t graph_exec = nullptr;
     hipGraph_t graph = nullptr;
     std::vector<std::vector<int32_t>> kv_pos;      // per sequence: cell positions while an edit left them non-contiguous
@@ -170,6 +178,10 @@ int chunk_weight(pi_model * m, BatchState * b, int il, int kind, int rows, int c
     const bool ffn = kind == PI_T_FFN_UP || kind == PI_T_FFN_GATE || kind == PI_T_FFN_DOWN_T;
     const bool split = ffn && m->L(il, PI_T_GPU_BUCKET).dev != nullptr;
     const void * rest = !split ? nullptr : kind == PI_T_FFN_UP ? m->rest_up[il] : kind == PI_T_FFN_GATE ? m->rest_gate[il] : m->rest_down[il];
+    if (split && b->staged_layer[il & 1] == il) {      // the copy stream has brought this layer's rows into device memory
+        const int which = kind == PI_T_FFN_UP ? 0 : kind == PI_T_FFN_GATE ? 1 : 2;
+        rest = b->stage[il & 1] + (size_t)which * b->stage_rows * b->stage_row_bytes;
+    }
     const uint32_t * hw = split ? m->hot_words[il] : nullptr;
     const int32_t * hpx = split ? m->hot_prefix[il] : nullptr;
     if (t.type == PI_TYPE_Q4_0) {
@@ -277,6 +289,25 @@ const char * wide_unsupported(pi_model * m) {
 }
 }  // namespace
 
+namespace {
+// queues the copies of layer il's non-resident rows into its staging buffer on the copy stream (after the layer that used the
+// buffer last has finished with it) and marks the buffer; layers that are whole on the device need nothing
+int stage_rest_rows(pi_model * m, BatchState * b, int il) {
+    if (il >= m->hp.n_layer || !b->copy_stream || !m->L(il, PI_T_GPU_BUCKET).dev) return PI_OK;
+    const int s = il & 1;
+    const size_t n_rest = (size_t)m->hp.n_ff - (size_t)m->L(il, PI_T_GPU_BUCKET).ne0;
+    const size_t rb = m->L(il, PI_T_FFN_UP).type == PI_TYPE_Q4_0 ? (size_t)(m->hp.n_embd / 32) * 18 : (size_t)m->hp.n_embd * 2;
+    if (n_rest > b->stage_rows || rb > b->stage_row_bytes) return pi::fail(PI_E_STATE, "stage_rest_rows: staging buffer too small");
+    if (b->free_recorded[s]) PI_HIP_TRY(hipStreamWaitEvent(b->copy_stream, b->ev_free[s], 0));
+    const void * src[3] = {m->rest_up[il], m->hp.arch == PI_ARCH_FALCON ? nullptr : m->rest_gate[il], m->rest_down[il]};
+    for (int k = 0; k < 3; ++k)
+        if (src[k] && n_rest) PI_HIP_TRY(hipMemcpyAsync(b->stage[s] + (size_t)k * b->stage_rows * b->stage_row_bytes, src[k], n_rest * rb, hipMemcpyHostToDevice, b->copy_stream));
+    PI_HIP_TRY(hipEventRecord(b->ev_copied[s], b->copy_stream));
+    b->staged_layer[s] = il;
+    return PI_OK;
+}
+}  // namespace
+
 namespace pi {
 bool prefill_wide_supported(pi_model * m) {
     const char * off = getenv("PI_NO_PREFILL_WIDE");
@@ -326,6 +357,22 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
         if (w16) b->w16 = m->alloc<__half>(w16);
         if (scratch) b->w16t = m->alloc<__half>((size_t)hp.n_embd * hp.n_ff);
         if ((w16 && !b->w16) || (scratch && !b->w16t)) { delete b; m->down_rows.clear(); return PI_E_HIP; }
+        // two staging buffers for the non-resident rows of hybrid layers (the largest such layer decides their size)
+        for (int il = 0; il < hp.n_layer; ++il) {
+            if (!m->L(il, PI_T_GPU_BUCKET).dev) continue;
+            b->stage_rows = std::max(b->stage_rows, (size_t)hp.n_ff - (size_t)m->L(il, PI_T_GPU_BUCKET).ne0);
+            b->stage_row_bytes = std::max(b->stage_row_bytes, m->L(il, PI_T_FFN_UP).type == PI_TYPE_Q4_0 ? (size_t)(hp.n_embd / 32) * 18 : (size_t)hp.n_embd * 2);
+        }
+        const char * no_stage = getenv("PI_PREFILL_NO_STAGING");
+        if (b->stage_rows && !(no_stage && no_stage[0] == '1')) {
+            for (int i = 0; i < 2; ++i) {
+                b->stage[i] = m->alloc<unsigned char>(3 * b->stage_rows * b->stage_row_bytes);
+                if (!b->stage[i]) { delete b; m->down_rows.clear(); return PI_E_HIP; }
+                PI_HIP_TRY(hipEventCreateWithFlags(&b->ev_copied[i], hipEventDisableTiming));
+                PI_HIP_TRY(hipEventCreateWithFlags(&b->ev_free[i], hipEventDisableTiming));
+            }
+            PI_HIP_TRY(hipStreamCreateWithFlags(&b->copy_stream, hipStreamNonBlocking));
+        }
         m->prefill_wide = b;
     }
     BatchState * b = m->prefill_wide;
@@ -337,7 +384,15 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
     if (m->glob[PI_T_TOK_EMBD].type == PI_TYPE_Q4_0) PI_TRY(pi_k_embed_batch_q4(m->glob[PI_T_TOK_EMBD].dev, hp.n_embd, b->d_tokens, T, b->x, m->stream));
     else PI_TRY(pi_k_embed_batch(m->glob[PI_T_TOK_EMBD].dev, hp.n_embd, b->d_tokens, T, b->x, m->stream));
-    for (int il = 0; il < hp.n_layer; ++il) PI_TRY(wide_layer(m, b, il));
+    b->staged_layer[0] = b->staged_layer[1] = -1;
+    PI_TRY(stage_rest_rows(m, b, 0));
+    for (int il = 0; il < hp.n_layer; ++il) {
+        PI_TRY(stage_rest_rows(m, b, il + 1));                   // the next layer's rows cross the host link under this layer's mat-muls
+        const bool staged = b->staged_layer[il & 1] == il;
+        if (staged) PI_HIP_TRY(hipStreamWaitEvent(m->stream, b->ev_copied[il & 1], 0));
+        PI_TRY(wide_layer(m, b, il));
+        if (staged) { PI_HIP_TRY(hipEventRecord(b->ev_free[il & 1], m->stream)); b->free_recorded[il & 1] = true; }
+    }
     return PI_OK;
 }
 
@@ -369,7 +424,13 @@ int prefill_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) {
 
 void batch_destroy(pi_model * m) {
     if (m->prefill) { delete m->prefill; m->prefill = nullptr; }
-    if (m->prefill_wide) { delete m->prefill_wide; m->prefill_wide = nullptr; }
+    if (m->prefill_wide) {
+        BatchState * b = m->prefill_wide;
+        if (b->copy_stream) { (void)hipStreamSynchronize(b->copy_stream); (void)hipStreamDestroy(b->copy_stream); }
+        for (int i = 0; i < 2; ++i) { if (b->ev_copied[i]) (void)hipEventDestroy(b->ev_copied[i]); if (b->ev_free[i]) (void)hipEventDestroy(b->ev_free[i]); }
+        delete b;
+        m->prefill_wide = nullptr;
+    }
     if (m->gemm_lib) { (void)pi_gemm_lib_destroy(m->gemm_lib); m->gemm_lib = nullptr; }
     if (!m->batch) return;
     if (m->batch->graph_exec) (void)hipGraphExecDestroy(m->batch->graph_exec);

@@ -342,8 +342,10 @@ ColdPath * cold_create(pi_model * m) {
     if (!(sync_only && sync_only[0] == '1')) {
         for (int il = 0; il < hp.n_layer; ++il) {
             Tensor & up = m->L(il, PI_T_FFN_UP);
-            if (m->L(il, PI_T_GPU_BUCKET).dev && up.type == PI_TYPE_Q4_0 && m->L(il, PI_T_FC2).type == PI_TYPE_F16 && m->hot_words[il] &&
-                pi_k_pred_upgate_q4_supported(c->ff, (int)m->L(il, PI_T_FC1).ne1, c->d))
+            if (!m->L(il, PI_T_GPU_BUCKET).dev || m->L(il, PI_T_FC2).type != PI_TYPE_F16 || !m->hot_words[il]) continue;
+            const int r = (int)m->L(il, PI_T_FC1).ne1;
+            if ((up.type == PI_TYPE_Q4_0 && pi_k_pred_upgate_q4_supported(c->ff, r, c->d)) ||
+                (up.type == PI_TYPE_F16 && pi_k_sparse_ffn_two_phase_supported(c->ff, r, c->d)))
                 c->async_layers.push_back(il);
         }
     }
@@ -842,6 +844,79 @@ void serve_q4(ColdPath * c, int il, uint32_t seq) {
     if (c->trace) { ++c->n_calls; c->n_cold_active += na; c->t_last_return = now(); }
 }
 
+// the same for an F16 layer: the resident share needs nothing from the host, so there is one hand-over in each direction
+void serve_f16(ColdPath * c, int il, uint32_t seq) {
+    pi_model * m = c->model;
+    const pi_hparams & hp = m->hp;
+    const int d = c->d;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    ColdLayer & cl = c->layers[il];
+    Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
+    const float thr = hp.sparse_threshold;
+    float * out = c->out[0];
+    auto now = [] { return std::chrono::steady_clock::now(); };
+    auto us = [](std::chrono::steady_clock::time_point a, std::chrono::steady_clock::time_point b) { return std::chrono::duration<double, std::micro>(b - a).count(); };
+    std::chrono::steady_clock::time_point tp = now();
+    if (c->trace && c->n_calls) c->t_between += us(c->t_last_return, tp);
+    auto lap = [&](int i) { if (c->trace) { const auto t = now(); c->t_phase[i] += us(tp, t); tp = t; } };
+    {
+        const auto t0 = now();
+        for (int it = 0; (int32_t)(__atomic_load_n(&c->flags[0], __ATOMIC_ACQUIRE) - seq) < 0; ++it) {
+            relax();
+            if ((it & 1023) == 1023 && (c->stop.load() || now() - t0 > std::chrono::seconds(20))) {
+                c->failed.store(true);
+                __atomic_store_n(&c->flags[48], 1u, __ATOMIC_RELEASE);
+                return;
+            }
+        }
+    }
+    lap(0);
+    c->act.clear();
+    for (int j : cl.cold_rows) if (!(c->logits[j] < thr)) c->act.push_back(j);
+    const int na = (int)c->act.size();
+    lap(1);
+    float * hval = c->hval.data();
+    const size_t rb = (size_t)d * 2;
+    const unsigned char * wu = (const unsigned char *)up.host;
+    const unsigned char * wg = falcon ? nullptr : (const unsigned char *)gate.host;
+    const uint16_t * x16 = c->x16_pin;
+    c->pool->run([&](int t, int nt) {
+        for (int k = t; k < na; k += nt) {
+            const int j = c->act[k];
+            if (k + nt < na) { prefetch_bytes(wu + rb * c->act[k + nt], rb); if (wg) prefetch_bytes(wg + rb * c->act[k + nt], rb); }
+            const float u = dot_f16(d, (const uint16_t *)(wu + rb * j), x16);
+            const float g = wg ? dot_f16(d, (const uint16_t *)(wg + rb * j), x16) : 0.f;
+            hval[k] = wg ? (g > 0.f ? g : 0.f) * u : (u > 0.f ? u : 0.f);
+        }
+    });
+    lap(2);
+    lap(3);
+    const unsigned char * wd = (const unsigned char *)down.host;
+    const int n_units = d / 32;
+    c->pool->run([&](int t, int nt) {
+        const int u0 = (int)((long long)n_units * t / nt), u1 = (int)((long long)n_units * (t + 1) / nt);
+        const int c0 = u0 * 32, c1 = u1 * 32;
+        for (int i = c0; i < c1; ++i) out[i] = 0.f;
+        for (int k = 0; k < na; ++k) {
+            const uint16_t hb = f2h(hval[k]);
+            if (k + 2 < na) prefetch_bytes(wd + rb * c->act[k + 2] + (size_t)c0 * 2, (size_t)(c1 - c0) * 2);
+            if (hb == 0) continue;
+            const float a = h2f(hb);
+            const uint16_t * row = (const uint16_t *)(wd + rb * c->act[k]);
+#ifdef PI_COLD_SIMD
+            const __m256 av = _mm256_set1_ps(a);
+            for (int i = c0; i < c1; i += 8)
+                _mm256_storeu_ps(out + i, _mm256_fmadd_ps(_mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(row + i))), av, _mm256_loadu_ps(out + i)));
+#else
+            for (int i = c0; i < c1; ++i) out[i] = fmaf(h2f(row[i]), a, out[i]);
+#endif
+        }
+    });
+    __atomic_store_n(&c->flags[32], seq, __ATOMIC_RELEASE);          // the reduction may add the host share
+    lap(4);
+    if (c->trace) { ++c->n_calls; c->n_cold_active += na; c->t_last_return = now(); }
+}
+
 void service_loop(ColdPath * c) {
     uint64_t next = 0;
     uint32_t seq = 0;
@@ -860,7 +935,10 @@ void service_loop(ColdPath * c) {
         if (c->stop.load()) return;
         const int il = c->ring[next % c->ring.size()];
         ++seq;
-        if (!c->failed.load()) serve_q4(c, il, seq);
+        if (!c->failed.load()) {
+            if (c->model->L(il, PI_T_FFN_UP).type == PI_TYPE_Q4_0) serve_q4(c, il, seq);
+            else serve_f16(c, il, seq);
+        }
         c->served.store(++next, std::memory_order_release);
     }
 }
@@ -868,6 +946,11 @@ void service_loop(ColdPath * c) {
 }  // namespace
 
 bool cold_async(const ColdPath * c) { return c && c->async; }
+bool cold_layer_async(const ColdPath * c, int il) {
+    if (!c || !c->async) return false;
+    for (int a : c->async_layers) if (a == il) return true;
+    return false;
+}
 bool cold_every_layer_async(const ColdPath * c) {
     if (!c || !c->async) return false;
     size_t hybrid = 0;
@@ -937,6 +1020,34 @@ int cold_layer_q4_queue(ColdPath * c, int il, pi_model * m, hipStream_t st) {
     int32_t * n_act = m->n_active + il;
     if (!falcon) return pi_k_axpy_q4_reduce(ff, d, PI_EPI_ADD2, out, m->ffn_inp, m->x2, n_act, m->ws, st);
     PI_TRY(pi_k_axpy_q4_reduce(ff, d, PI_EPI_NONE, nullptr, nullptr, m->x2, n_act, m->ws, st));
+    return merge_shares(m->x2, out, m->x2, m->attn_out, m->x, nullptr, d, st);
+}
+
+// the device half of an F16 hybrid layer: predictor -> signal -> resident rows (gate / up / down partial vectors) -> (wait for the host
+// share) reduction with the merge folded in
+int cold_layer_f16_queue(ColdPath * c, int il, pi_model * m, hipStream_t st) {
+    const pi_hparams & hp = m->hp;
+    const int d = c->d, ff = c->ff;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
+    Tensor & fc1 = m->L(il, PI_T_FC1); Tensor & fc2 = m->L(il, PI_T_FC2);
+    const int r = (int)fc1.ne1;
+    float * out = c->out[0];
+    const double limit = 5.0;
+    pi_norm fn;
+    fn.kind = falcon ? 2 : 1; fn.eps = hp.norm_eps;
+    fn.w = (const float *)m->L(il, falcon ? PI_T_ATTN_NORM : PI_T_FFN_NORM).dev;
+    fn.b = falcon ? (const float *)m->L(il, PI_T_ATTN_NORM_B).dev : nullptr;
+    const float * ffn_src = falcon ? m->x : m->ffn_inp;
+    PI_TRY(pi_k_sparse_ffn_logits_hot(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, d, ffn_src, &fn, m->hot_words[il], m->hot_prefix[il],
+                                      c->logits, m->pred_logits, c->x16_pin, m->ws, st));
+    PI_TRY(pi_k_host_signal(c->d_seq, c->flags, 0, 1, st));
+    PI_TRY(pi_k_sparse_ffn_rows_hot(ff, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, down.dev, d, ffn_src, &fn, m->hot_words[il], m->hot_prefix[il],
+                                    m->pred_logits, nullptr, m->ws, st));
+    PI_TRY(pi_k_host_wait(c->d_seq, c->flags, 32, c->d_status, limit, st));
+    int32_t * n_act = m->n_active + il;
+    if (!falcon) return pi_k_sparse_ffn_reduce_hot(ff, d, PI_EPI_ADD2, out, m->ffn_inp, m->x2, n_act, m->ws, st);
+    PI_TRY(pi_k_sparse_ffn_reduce_hot(ff, d, PI_EPI_NONE, nullptr, nullptr, m->x2, n_act, m->ws, st));
     return merge_shares(m->x2, out, m->x2, m->attn_out, m->x, nullptr, d, st);
 }
 

@@ -26,7 +26,7 @@ int        cold_layer_q4(ColdPath * c, int il, pi_model * m, hipStream_t st, boo
 // its whole FFN (gate/up/down partial vectors) is queued at once and only the final reduction waits for the host share.
 int        cold_layer_f16(ColdPath * c, int il, pi_model * m, hipStream_t st, bool capture);
 
-// Q4_0 hybrid layers with nothing launched between the two halves: the stream holds hand-over kernels, a service thread computes the
+// Hybrid layers (Q4_0, and F16 at 4096 columns) with nothing launched between the two halves: the stream holds hand-over kernels, a service thread computes the
 // host share when the device signals and answers through flag words in pinned memory.  cold_post_token announces one token's
 // hybrid layers to the service thread (call it once per token whose kernels are queued with cold_layer_q4_queue), cold_drain
 // confirms after a stream synchronisation that every hand-over completed.  PI_COLD_SYNC=1 keeps the launching thread in the loop.
@@ -35,6 +35,8 @@ bool       cold_every_layer_async(const ColdPath * c);   // no hybrid layer need
 int        cold_post_token(ColdPath * c);
 int        cold_drain(ColdPath * c);
 int        cold_layer_q4_queue(ColdPath * c, int il, pi_model * m, hipStream_t st);
+int        cold_layer_f16_queue(ColdPath * c, int il, pi_model * m, hipStream_t st);     // F16 layers at 4096 columns: one hand-over each way
+bool       cold_layer_async(const ColdPath * c, int il);
 
 int add_vec(float * y, const float * a, int n, hipStream_t st);
 // dst = ((cold + hot) + r1) [+ r2]; `cold` may be pinned host memory; `keep` (optional) receives cold + hot

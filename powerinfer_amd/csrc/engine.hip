@@ -218,7 +218,8 @@ int layer_forward(pi_model * m, int il, bool last_token) {
         // F16 hybrid layer at a width the fused kernels cover: the resident share's whole FFN is one launch, the host share works
         // from the pinned buffers it fills, the reduction merges both
         const bool cap = m->capture && last_token;
-        PI_TRY(pi::cold_layer_f16(m->cold, il, m, st, cap));
+        if (pi::cold_layer_async(m->cold, il) && !m->capture) PI_TRY(pi::cold_layer_f16_queue(m->cold, il, m, st));
+        else PI_TRY(pi::cold_layer_f16(m->cold, il, m, st, cap));
         if (cap) PI_HIP_TRY(hipMemcpyAsync(m->cap_src + (size_t)il * d, ffn_in, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
         std::swap(m->x, m->x2);
         return PI_OK;
@@ -230,7 +231,7 @@ int layer_forward(pi_model * m, int il, bool last_token) {
         const bool cap = m->capture && last_token;
         if (layer_hybrid && !m->rest_on_gpu) {
             // nothing is launched between the two halves unless the parity hooks are on: the stream waits for the host threads itself
-            if (pi::cold_async(m->cold) && !m->capture) PI_TRY(pi::cold_layer_q4_queue(m->cold, il, m, st));
+            if (pi::cold_layer_async(m->cold, il) && !m->capture) PI_TRY(pi::cold_layer_q4_queue(m->cold, il, m, st));
             else PI_TRY(pi::cold_layer_q4(m->cold, il, m, st, cap));
         } else {
             // every neuron on the GPU, or the non-resident neurons' rows read from pinned host memory by the same two launches

@@ -990,7 +990,9 @@ __device__ __forceinline__ int select_nth_bit(uint32_t bits, int n);
 // HYB: a hot/cold split layer.  Only the GPU-resident neurons are computed (mask & hot word; weight row = hot prefix + rank among
 // the hot bits: the compact matrices of the bucket), the activity words of that share go to words_hot, and workgroup 0 hands the
 // fp16-rounded normalised input to the host share (xn_out; like logits it may be pinned host memory).
-template <int CPW, int RCH, bool GATE, int G, bool HYB>      // cols == 8 waves * CPW chunks * 512; r == RCH * 512; G groups of 32 neurons
+// PHASE 1 / 2 (G == 1) cut the launch in two for a hybrid layer whose host share should start behind the predictor: 1 stops after the
+// logits (to `logits` and `logits2`), the mask words and the fp16 input for the host; 2 reads the logits back from `logits2`.
+template <int CPW, int RCH, bool GATE, int G, bool HYB, int PHASE = 0>      // cols == 8 waves * CPW chunks * 512; r == RCH * 512; G groups of 32 neurons
 __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
                                                                    const __half * __restrict__ Wup, const __half * __restrict__ Wgate,
                                                                    const __half * __restrict__ Wdown,
@@ -998,7 +1000,9 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
                                                                    float * __restrict__ logits, uint32_t * __restrict__ words, float * __restrict__ h_dense,
                                                                    float * __restrict__ partial,
                                                                    const uint32_t * __restrict__ hot_words, const int32_t * __restrict__ hot_prefix,
-                                                                   uint32_t * __restrict__ words_hot, __half * __restrict__ xn_out) {
+                                                                   uint32_t * __restrict__ words_hot, __half * __restrict__ xn_out,
+                                                                   float * __restrict__ logits2) {
+    static_assert(PHASE == 0 || G == 1, "the two-phase form takes one group per workgroup");
     constexpr int cols = kPfWaves * CPW * 512, r = RCH * 512;
     constexpr int CH = kPfChunk / CPW;                 // active neurons per round trip: 3*CPW*CH (2*CPW*CH) loads in flight per lane
     __shared__ float  lg[2][32];
@@ -1010,15 +1014,20 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
 
     // ---- A: loads ------------------------------------------------------------------------------------------
     pi_u32x4 a[4][RCH];
-#pragma unroll
-    for (int i = 0; i < 4; ++i)
-#pragma unroll
-        for (int j = 0; j < RCH; ++j) a[i][j] = pi_ld_stream(W2 + (size_t)(n0 + wave * 4 + i) * r + (j * PI_WAVE + lane) * 8);
     float4 hv[RCH][2];
+    float logit_in = 0.0f;
+    if (PHASE != 2) {
 #pragma unroll
-    for (int j = 0; j < RCH; ++j) {
-        hv[j][0] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8);
-        hv[j][1] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8 + 4);
+        for (int i = 0; i < 4; ++i)
+#pragma unroll
+            for (int j = 0; j < RCH; ++j) a[i][j] = pi_ld_stream(W2 + (size_t)(n0 + wave * 4 + i) * r + (j * PI_WAVE + lane) * 8);
+#pragma unroll
+        for (int j = 0; j < RCH; ++j) {
+            hv[j][0] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8);
+            hv[j][1] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8 + 4);
+        }
+    } else {
+        logit_in = logits2[n0 + (lane & 31)];
     }
     float xs[CPW][8], ws[CPW][8], bs[CPW][8];
 #pragma unroll
@@ -1037,19 +1046,21 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
     }
     // ---- A: logits (the CPU path rounds the hidden vector to fp16 before the dot, ggml.c:9703-9716) ------------
     pi_u32x4 hr[RCH];
+    if (PHASE != 2) {
 #pragma unroll
-    for (int j = 0; j < RCH; ++j) {
-        __half2 hh[4] = {__floats2half2_rn(hv[j][0].x, hv[j][0].y), __floats2half2_rn(hv[j][0].z, hv[j][0].w),
-                         __floats2half2_rn(hv[j][1].x, hv[j][1].y), __floats2half2_rn(hv[j][1].z, hv[j][1].w)};
-        hr[j] = *reinterpret_cast<const pi_u32x4 *>(hh);
-    }
+        for (int j = 0; j < RCH; ++j) {
+            __half2 hh[4] = {__floats2half2_rn(hv[j][0].x, hv[j][0].y), __floats2half2_rn(hv[j][0].z, hv[j][0].w),
+                             __floats2half2_rn(hv[j][1].x, hv[j][1].y), __floats2half2_rn(hv[j][1].z, hv[j][1].w)};
+            hr[j] = *reinterpret_cast<const pi_u32x4 *>(hh);
+        }
 #pragma unroll
-    for (int i = 0; i < 4; ++i) {
-        float acc = 0.0f;
+        for (int i = 0; i < 4; ++i) {
+            float acc = 0.0f;
 #pragma unroll
-        for (int j = 0; j < RCH; ++j) acc = pi_dot8h(a[i][j], hr[j], acc);
-        acc = pi_wave_sum(acc);
-        if (lane == 0) lg[0][wave * 4 + i] = acc;
+            for (int j = 0; j < RCH; ++j) acc = pi_dot8h(a[i][j], hr[j], acc);
+            acc = pi_wave_sum(acc);
+            if (lane == 0) lg[0][wave * 4 + i] = acc;
+        }
     }
     if (G > 1) {       // the next group's predictor rows travel while this group's FFN rows are fetched and used
 #pragma unroll
@@ -1143,16 +1154,21 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
         __syncthreads();
     }
     // ---- activity word (identical in every wave; lg[g & 1] is complete after the barrier above) ----------------
-    const float my_logit = lg[g & 1][lane & 31];
+    const float my_logit = PHASE == 2 ? logit_in : lg[g & 1][lane & 31];
     const bool my_act = !(my_logit < thr);
     const uint32_t all = (uint32_t)__ballot(my_act);
     const uint32_t hot = HYB ? hot_words[blockIdx.x * G + g] : 0xFFFFFFFFu;
     const int base_row = HYB ? hot_prefix[blockIdx.x * G + g] : n0;
     const uint32_t mask = all & hot;
     if (wave == 0) {
-        if (lane < 32) { if (logits) logits[n0 + lane] = my_logit; if (h_dense && !((mask >> lane) & 1u)) h_dense[n0 + lane] = 0.0f; }
+        if (lane < 32) {
+            if (PHASE != 2 && logits) logits[n0 + lane] = my_logit;
+            if (PHASE == 1) logits2[n0 + lane] = my_logit;
+            if (PHASE != 1 && h_dense && !((mask >> lane) & 1u)) h_dense[n0 + lane] = 0.0f;
+        }
         if (lane == 0) { words[blockIdx.x * G + g] = all; if (HYB) words_hot[blockIdx.x * G + g] = mask; }
     }
+    if (PHASE == 1) return;
     // ---- B + C ---------------------------------------------------------------------------------------------
     const int n = __popc(mask);
     for (int c0 = 0; c0 < n; c0 += CH) {
@@ -3860,7 +3876,7 @@ static int sparse_ffn_partials_impl(const char * who, const void * fc2_f16, int 
     const int G = pf_groups(ff, cols);
     const dim3 grid(ff / (32 * G)), block(kPfBlock);
     const bool hyb = hot_words != nullptr;
-#define PI_PF_LAUNCH2(CPW, RCH, GATE, GG, HYB) hipLaunchKernelGGL((pred_ffn_f16_kernel<CPW, RCH, GATE, GG, HYB>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial, hot_words, hot_prefix, ws->words_hot, (__half *)xn_f16_out)
+#define PI_PF_LAUNCH2(CPW, RCH, GATE, GG, HYB) hipLaunchKernelGGL((pred_ffn_f16_kernel<CPW, RCH, GATE, GG, HYB>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial, hot_words, hot_prefix, ws->words_hot, (__half *)xn_f16_out, nullptr)
 #define PI_PF_LAUNCH(CPW, RCH, GATE, GG) do { if (hyb) PI_PF_LAUNCH2(CPW, RCH, GATE, GG, true); else PI_PF_LAUNCH2(CPW, RCH, GATE, GG, false); } while (0)
 #define PI_PF_WIDE(RCH, GATE) do { if (G == 4) PI_PF_LAUNCH(2, RCH, GATE, 4); else if (G == 2) PI_PF_LAUNCH(2, RCH, GATE, 2); else PI_PF_LAUNCH(2, RCH, GATE, 1); } while (0)
     const int cpw = cols / 4096, rch = r / 512;
@@ -3888,6 +3904,38 @@ int pi_k_sparse_ffn_partials_hot(const void * fc2_f16, int ff, int r, const floa
     if (!hot_words || !hot_prefix) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_partials_hot: hot words and prefix are required");
     return sparse_ffn_partials_impl("pi_k_sparse_ffn_partials_hot", fc2_f16, ff, r, hidden, threshold, up_f16, gate_f16, down_t_f16, cols, x, norm, logits, h_dense,
                                     hot_words, hot_prefix, xn_f16_out, ws, stream);
+}
+
+int pi_k_sparse_ffn_two_phase_supported(int ff, int r, int cols) { return pi_k_sparse_ffn_supported(ff, r, cols) && cols == 4096; }
+
+int pi_k_sparse_ffn_logits_hot(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
+                               const uint32_t * hot_words, const int32_t * hot_prefix, float * logits, float * logits_dev, void * xn_f16_out,
+                               pi_workspace * ws, pi_stream_t stream) {
+    if (!fc2_f16 || !hidden || !x || !hot_words || !hot_prefix || !logits_dev || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_logits_hot: null pointer");
+    if (!pi_k_sparse_ffn_two_phase_supported(ff, r, cols) || ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn_logits_hot: cols must be 4096, r 512 or 1024, ff % 32 == 0, within the workspace");
+    const NormArgs na = to_norm(norm);
+    if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b | (uintptr_t)xn_f16_out) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_logits_hot: vectors must be 16-byte aligned");
+    const dim3 grid(ff / 32), block(kPfBlock);
+    const __half * none = nullptr;
+#define PI_PF1(RCH) hipLaunchKernelGGL((pred_ffn_f16_kernel<1, RCH, false, 1, true, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, x, na, threshold, logits, ws->words, (float *)nullptr, (float *)nullptr, hot_words, hot_prefix, ws->words_hot, (__half *)xn_f16_out, logits_dev)
+    if (r == 1024) PI_PF1(2); else PI_PF1(1);
+#undef PI_PF1
+    return pi::check_launch("pi_k_sparse_ffn_logits_hot");
+}
+
+int pi_k_sparse_ffn_rows_hot(int ff, float threshold, const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x,
+                             const pi_norm * norm, const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense,
+                             pi_workspace * ws, pi_stream_t stream) {
+    if (!up_f16 || !down_t_f16 || !x || !hot_words || !hot_prefix || !logits_dev || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_rows_hot: null pointer");
+    if (cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn_rows_hot: cols must be 4096, ff % 32 == 0, within the workspace");
+    const NormArgs na = to_norm(norm);
+    if ((((uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_rows_hot: vectors must be 16-byte aligned");
+    const dim3 grid(ff / 32), block(kPfBlock);
+    const __half * u = (const __half *)up_f16; const __half * g = (const __half *)gate_f16; const __half * dn = (const __half *)down_t_f16;
+#define PI_PF2(GATE) hipLaunchKernelGGL((pred_ffn_f16_kernel<1, 1, GATE, 1, true, 2>), grid, block, 0, (hipStream_t)stream, (const __half *)nullptr, (const float *)nullptr, u, g, dn, x, na, threshold, (float *)nullptr, ws->words, h_dense, ws->ffn_partial, hot_words, hot_prefix, ws->words_hot, (__half *)nullptr, const_cast<float *>(logits_dev))
+    if (g) PI_PF2(true); else PI_PF2(false);
+#undef PI_PF2
+    return pi::check_launch("pi_k_sparse_ffn_rows_hot");
 }
 
 static int sparse_ffn_reduce_impl(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out, int32_t * n_active,

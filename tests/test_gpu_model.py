@@ -342,17 +342,18 @@ def test_q4_split_rest_read_by_the_gpu_matches_host_threads():
         Model(hp3).load(synth.make_model(hp3))
 
 
-@pytest.mark.parametrize("arch", ["llama-7b", "falcon-4096"])
-def test_q4_split_stream_handovers_match_launch_per_exchange(arch, monkeypatch):
-    """Hybrid Q4_0 layers hand over to the host threads through wait kernels in the stream (one graph replay per token, a service
-    thread on the host); PI_COLD_SYNC=1 keeps the launching thread in the loop with an event wait and a launch per exchange.  Same
-    kernels' arithmetic, same host arithmetic: logits and greedy tokens are bit-identical, across two generate calls."""
+@pytest.mark.parametrize("arch,wtype", [("llama-7b", synth.Q4_0), ("falcon-4096", synth.Q4_0), ("llama-7b", synth.F16), ("falcon-4096", synth.F16)])
+def test_split_stream_handovers_match_launch_per_exchange(arch, wtype, monkeypatch):
+    """Hybrid layers (Q4_0, and F16 at 4096 columns) hand over to the host threads through signal and wait kernels in the stream (one
+    graph replay per token, a service thread on the host); PI_COLD_SYNC=1 keeps the launching thread in the loop with an event wait
+    and a launch per exchange.  Same kernels' arithmetic, same host arithmetic: logits and greedy tokens are bit-identical, across
+    two generate calls."""
     from powerinfer_amd.model import Model
     if arch == "llama-7b":
-        hp = synth.hparams("llama-7b", n_layer=3, n_ctx=96, seed=14, wtype=synth.Q4_0, hot_frac=0.6)
+        hp = synth.hparams("llama-7b", n_layer=3, n_ctx=96, seed=14, wtype=wtype, hot_frac=0.6)
     else:
         hp = synth.hparams("falcon-tiny", n_embd=4096, n_ff=8192, n_rank=512, n_head=64, n_head_kv=8, n_layer=2, n_vocab=4096,
-                           n_ctx=96, seed=15, wtype=synth.Q4_0, hot_frac=0.5)
+                           n_ctx=96, seed=15, wtype=wtype, hot_frac=0.5)
     model = synth.make_model(hp)
     prompt = np.random.default_rng(5).integers(0, hp.n_vocab, 9).astype(np.int32)
     outs = []

@@ -407,6 +407,93 @@ hipError_t wait_event(hipEvent_t ev) {
 }
 }  // namespace
 
+namespace {
+// ---- the host share's three steps, shared by the variant that launches between them and the one that answers the stream's signals ----
+
+// neurons of this layer that are not GPU-resident and whose predictor logit reaches the threshold, ascending, into c->act
+int list_active_cold(ColdPath * c, const ColdLayer & cl, float thr) {
+    c->act.clear();
+    for (int j : cl.cold_rows) if (!(c->logits[j] < thr)) c->act.push_back(j);
+    return (int)c->act.size();
+}
+
+// h of the listed neurons into c->hval: up/gate dots on the input the device rounded (Q8_0 blocks for Q4_0 rows, fp16 for F16 rows;
+// ggml.c:14030-14282), the next neuron's rows prefetched while this one's are used
+void host_upgate(ColdPath * c, pi_model * m, int il, int na) {
+    const bool falcon = m->hp.arch == PI_ARCH_FALCON;
+    Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE);
+    const bool q4 = up.type == PI_TYPE_Q4_0;
+    const int d = c->d;
+    float * hval = c->hval.data();
+    const size_t rb = q4 ? (size_t)(d / 32) * 18 : (size_t)d * 2;
+    const unsigned char * wu = (const unsigned char *)up.host;
+    const unsigned char * wg = falcon ? nullptr : (const unsigned char *)gate.host;
+    const BlockQ8 * xq = c->xq8_pin;
+    const uint16_t * x16 = c->x16_pin;
+    c->pool->run([&](int t, int nt) {
+        for (int k = t; k < na; k += nt) {
+            const int j = c->act[k];
+            if (k + nt < na) { prefetch_bytes(wu + rb * c->act[k + nt], rb); if (wg) prefetch_bytes(wg + rb * c->act[k + nt], rb); }
+            float u, g = 0.f;
+            if (q4) {
+                u = dot_q4_q8(d, (const BlockQ4 *)(wu + rb * j), xq);
+                if (wg) g = dot_q4_q8(d, (const BlockQ4 *)(wg + rb * j), xq);
+            } else {
+                u = dot_f16(d, (const uint16_t *)(wu + rb * j), x16);
+                if (wg) g = dot_f16(d, (const uint16_t *)(wg + rb * j), x16);
+            }
+            hval[k] = wg ? (g > 0.f ? g : 0.f) * u : (u > 0.f ? u : 0.f);
+        }
+    });
+}
+
+// the listed neurons' share of the down projection into out[d]; threads split the output columns in blocks of 32, so no two threads
+// add into the same element.  Q4_0: h goes through the Q8_0 blocks of the completed vector hfull (only the blocks that hold a listed
+// neuron are quantised; ggml.c:14465-14618); F16: h rounded to fp16 (ggml.c:14420-14431).
+void host_down(ColdPath * c, pi_model * m, int il, int na, const float * hfull, float * out) {
+    Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
+    const bool q4 = down.type == PI_TYPE_Q4_0;
+    const int d = c->d;
+    const size_t rb = q4 ? (size_t)(d / 32) * 18 : (size_t)d * 2;
+    const unsigned char * wd = (const unsigned char *)down.host;
+    const float * hval = c->hval.data();
+    if (q4) {
+        for (int k = 0, last = -1; k < na; ++k) {               // act is ascending
+            const int b = c->act[k] / 32;
+            if (b != last) { quantize_q8(hfull + b * 32, c->hq8.data() + b, 32); last = b; }
+        }
+    }
+    const int n_units = d / 32;
+    c->pool->run([&](int t, int nt) {
+        const int u0 = (int)((long long)n_units * t / nt), u1 = (int)((long long)n_units * (t + 1) / nt);
+        const int c0 = u0 * 32, c1 = u1 * 32;
+        for (int i = c0; i < c1; ++i) out[i] = 0.f;
+        for (int k = 0; k < na; ++k) {
+            const int j = c->act[k];
+            if (k + 2 < na) prefetch_bytes(wd + rb * c->act[k + 2] + (q4 ? (size_t)u0 * 18 : (size_t)c0 * 2), q4 ? (size_t)(u1 - u0) * 18 : (size_t)(c1 - c0) * 2);
+            if (q4) {
+                const BlockQ8 & hb = c->hq8[j / 32];
+                const int a = hb.qs[j % 32];
+                if (a == 0) continue;
+                axpy_q4_blocks((const BlockQ4 *)(wd + rb * j), u0, u1, a, h2f(hb.d), out);
+            } else {
+                const uint16_t hb = f2h(hval[k]);
+                if (hb == 0) continue;
+                const float a = h2f(hb);
+                const uint16_t * row = (const uint16_t *)(wd + rb * j);
+#ifdef PI_COLD_SIMD
+                const __m256 av = _mm256_set1_ps(a);
+                for (int i = c0; i < c1; i += 8)
+                    _mm256_storeu_ps(out + i, _mm256_fmadd_ps(_mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(row + i))), av, _mm256_loadu_ps(out + i)));
+#else
+                for (int i = c0; i < c1; ++i) out[i] = fmaf(h2f(row[i]), a, out[i]);
+#endif
+            }
+        }
+    });
+}
+}  // namespace
+
 int cold_stage_inputs(ColdPath * c, int il, pi_model * m, hipStream_t st) {
     (void)il;
     const float * ffn_src = m->hp.arch == PI_ARCH_FALCON ? m->x : m->ffn_inp;
@@ -584,49 +671,17 @@ int cold_layer_q4(ColdPath * c, int il, pi_model * m, hipStream_t st, bool captu
     lap(0);
 
     // 2. active cold neurons, their up/gate rows against the same Q8_0 input
-    c->act.clear();
-    for (int j : cl.cold_rows) if (!(c->logits[j] < thr)) c->act.push_back(j);
-    const int na = (int)c->act.size();
+    const int na = list_active_cold(c, cl, thr);
     lap(1);
-    float * hval = c->hval.data();
-    const size_t rb = (size_t)(d / 32) * 18;
-    const unsigned char * wu = (const unsigned char *)up.host;
-    const unsigned char * wg = falcon ? nullptr : (const unsigned char *)gate.host;
-    const BlockQ8 * xq = c->xq8_pin;
-    c->pool->run([&](int t, int nt) {
-        for (int k = t; k < na; k += nt) {
-            const int j = c->act[k];
-            if (k + nt < na) { prefetch_bytes(wu + rb * c->act[k + nt], rb); if (wg) prefetch_bytes(wg + rb * c->act[k + nt], rb); }
-            const float u = dot_q4_q8(d, (const BlockQ4 *)(wu + rb * j), xq);
-            const float g = wg ? dot_q4_q8(d, (const BlockQ4 *)(wg + rb * j), xq) : 0.f;
-            hval[k] = wg ? (g > 0.f ? g : 0.f) * u : (u > 0.f ? u : 0.f);
-        }
-    });
-    for (int k = 0; k < na; ++k) hfull[c->act[k]] = hval[k];
+    host_upgate(c, m, il, na);
+    for (int k = 0; k < na; ++k) hfull[c->act[k]] = c->hval[k];
     lap(2);
 
     // 3. the GPU's down projection reads the completed vector from the pinned buffer; the host quantises it the same way
     rc = pi_k_axpy_q4_partials(down.dev, d, ff, hfull, m->hot_words[il], m->hot_prefix[il], m->ws, st);
     if (rc != PI_OK) return rc;
-    for (int k = 0, last = -1; k < na; ++k) {               // act is ascending: only the Q8_0 blocks of h that hold an active cold neuron
-        const int b = c->act[k] / 32;
-        if (b != last) { quantize_q8(hfull + b * 32, c->hq8.data() + b, 32); last = b; }
-    }
     lap(3);
-    const unsigned char * wd = (const unsigned char *)down.host;
-    const int n_units = d / 32;
-    c->pool->run([&](int t, int nt) {
-        const int u0 = (int)((long long)n_units * t / nt), u1 = (int)((long long)n_units * (t + 1) / nt);
-        for (int i = u0 * 32; i < u1 * 32; ++i) out[i] = 0.f;
-        for (int k = 0; k < na; ++k) {
-            const int j = c->act[k];
-            const BlockQ8 & hb = c->hq8[j / 32];
-            const int a = hb.qs[j % 32];
-            if (k + 2 < na) prefetch_bytes(wd + rb * c->act[k + 2] + (size_t)u0 * 18, (size_t)(u1 - u0) * 18);
-            if (a == 0) continue;
-            axpy_q4_blocks((const BlockQ4 *)(wd + rb * j), u0, u1, a, h2f(hb.d), out);
-        }
-    });
+    host_down(c, m, il, na, hfull, out);
     lap(4);
 
     // 4. (cold + hot) + residual(s), the reference's order (ggml_add(cpu, gpu), then the residual adds): folded into the
@@ -677,47 +732,12 @@ int cold_layer_f16(ColdPath * c, int il, pi_model * m, hipStream_t st, bool capt
     lap(0);
 
     // 2. active cold neurons: up/gate dots on the fp16 input (ggml.c:14030-14282), h rounded to fp16 for the axpy (ggml.c:14420-14431)
-    c->act.clear();
-    for (int j : cl.cold_rows) if (!(c->logits[j] < thr)) c->act.push_back(j);
-    const int na = (int)c->act.size();
+    const int na = list_active_cold(c, cl, thr);
     lap(1);
-    float * hval = c->hval.data();
-    const size_t rb = (size_t)d * 2;
-    const unsigned char * wu = (const unsigned char *)up.host;
-    const unsigned char * wg = falcon ? nullptr : (const unsigned char *)gate.host;
-    const uint16_t * x16 = c->x16_pin;
-    c->pool->run([&](int t, int nt) {
-        for (int k = t; k < na; k += nt) {
-            const int j = c->act[k];
-            if (k + nt < na) { prefetch_bytes(wu + rb * c->act[k + nt], rb); if (wg) prefetch_bytes(wg + rb * c->act[k + nt], rb); }
-            const float u = dot_f16(d, (const uint16_t *)(wu + rb * j), x16);
-            const float g = wg ? dot_f16(d, (const uint16_t *)(wg + rb * j), x16) : 0.f;
-            hval[k] = wg ? (g > 0.f ? g : 0.f) * u : (u > 0.f ? u : 0.f);
-        }
-    });
+    host_upgate(c, m, il, na);
     lap(2);
     lap(3);
-    const unsigned char * wd = (const unsigned char *)down.host;
-    const int n_units = d / 32;
-    c->pool->run([&](int t, int nt) {
-        const int u0 = (int)((long long)n_units * t / nt), u1 = (int)((long long)n_units * (t + 1) / nt);
-        const int c0 = u0 * 32, c1 = u1 * 32;
-        for (int i = c0; i < c1; ++i) out[i] = 0.f;
-        for (int k = 0; k < na; ++k) {
-            const uint16_t hb = f2h(hval[k]);
-            if (k + 2 < na) prefetch_bytes(wd + rb * c->act[k + 2] + (size_t)c0 * 2, (size_t)(c1 - c0) * 2);
-            if (hb == 0) continue;
-            const float a = h2f(hb);
-            const uint16_t * row = (const uint16_t *)(wd + rb * c->act[k]);
-#ifdef PI_COLD_SIMD
-            const __m256 av = _mm256_set1_ps(a);
-            for (int i = c0; i < c1; i += 8)
-                _mm256_storeu_ps(out + i, _mm256_fmadd_ps(_mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(row + i))), av, _mm256_loadu_ps(out + i)));
-#else
-            for (int i = c0; i < c1; ++i) out[i] = fmaf(h2f(row[i]), a, out[i]);
-#endif
-        }
-    });
+    host_down(c, m, il, na, nullptr, out);
     lap(4);
 
     // 3. (cold + hot) + residual(s), folded into the reduction of the GPU partials when there is one residual and nothing to keep
@@ -784,24 +804,10 @@ void serve_q4(ColdPath * c, int il, uint32_t seq) {
         for (int j : c->prev_act[il]) hfull[j] = 0.f;
         c->prev_act[il].clear();
     }
-    c->act.clear();
-    for (int j : cl.cold_rows) if (!(c->logits[j] < thr)) c->act.push_back(j);
-    const int na = (int)c->act.size();
+    const int na = list_active_cold(c, cl, thr);
     lap(1);
-    float * hval = c->hval.data();
-    const size_t rb = (size_t)(d / 32) * 18;
-    const unsigned char * wu = (const unsigned char *)up.host;
-    const unsigned char * wg = falcon ? nullptr : (const unsigned char *)gate.host;
-    const BlockQ8 * xq = c->xq8_pin;
-    c->pool->run([&](int t, int nt) {
-        for (int k = t; k < na; k += nt) {
-            const int j = c->act[k];
-            if (k + nt < na) { prefetch_bytes(wu + rb * c->act[k + nt], rb); if (wg) prefetch_bytes(wg + rb * c->act[k + nt], rb); }
-            const float u = dot_q4_q8(d, (const BlockQ4 *)(wu + rb * j), xq);
-            const float g = wg ? dot_q4_q8(d, (const BlockQ4 *)(wg + rb * j), xq) : 0.f;
-            hval[k] = wg ? (g > 0.f ? g : 0.f) * u : (u > 0.f ? u : 0.f);
-        }
-    });
+    host_upgate(c, m, il, na);
+    const float * hval = c->hval.data();
     for (int k = 0; k < na; ++k) hfull[c->act[k]] = hval[k];
     if (c->split_pred) c->prev_act[il].assign(c->act.begin(), c->act.end());
     __atomic_store_n(&c->flags[16], seq, __ATOMIC_RELEASE);          // the device's down projection may read the completed vector
@@ -820,25 +826,8 @@ void serve_q4(ColdPath * c, int il, uint32_t seq) {
     }
 
     // 3. the host quantises h the same way and adds its neurons' down rows
-    for (int k = 0, last = -1; k < na; ++k) {
-        const int b = c->act[k] / 32;
-        if (b != last) { quantize_q8(hfull + b * 32, c->hq8.data() + b, 32); last = b; }
-    }
     lap(3);
-    const unsigned char * wd = (const unsigned char *)down.host;
-    const int n_units = d / 32;
-    c->pool->run([&](int t, int nt) {
-        const int u0 = (int)((long long)n_units * t / nt), u1 = (int)((long long)n_units * (t + 1) / nt);
-        for (int i = u0 * 32; i < u1 * 32; ++i) out[i] = 0.f;
-        for (int k = 0; k < na; ++k) {
-            const int j = c->act[k];
-            const BlockQ8 & hb = c->hq8[j / 32];
-            const int a = hb.qs[j % 32];
-            if (k + 2 < na) prefetch_bytes(wd + rb * c->act[k + 2] + (size_t)u0 * 18, (size_t)(u1 - u0) * 18);
-            if (a == 0) continue;
-            axpy_q4_blocks((const BlockQ4 *)(wd + rb * j), u0, u1, a, h2f(hb.d), out);
-        }
-    });
+    host_down(c, m, il, na, hfull, out);
     __atomic_store_n(&c->flags[32], seq, __ATOMIC_RELEASE);          // the reduction may add the host share
     lap(4);
     if (c->trace) { ++c->n_calls; c->n_cold_active += na; c->t_last_return = now(); }
@@ -871,47 +860,12 @@ void serve_f16(ColdPath * c, int il, uint32_t seq) {
         }
     }
     lap(0);
-    c->act.clear();
-    for (int j : cl.cold_rows) if (!(c->logits[j] < thr)) c->act.push_back(j);
-    const int na = (int)c->act.size();
+    const int na = list_active_cold(c, cl, thr);
     lap(1);
-    float * hval = c->hval.data();
-    const size_t rb = (size_t)d * 2;
-    const unsigned char * wu = (const unsigned char *)up.host;
-    const unsigned char * wg = falcon ? nullptr : (const unsigned char *)gate.host;
-    const uint16_t * x16 = c->x16_pin;
-    c->pool->run([&](int t, int nt) {
-        for (int k = t; k < na; k += nt) {
-            const int j = c->act[k];
-            if (k + nt < na) { prefetch_bytes(wu + rb * c->act[k + nt], rb); if (wg) prefetch_bytes(wg + rb * c->act[k + nt], rb); }
-            const float u = dot_f16(d, (const uint16_t *)(wu + rb * j), x16);
-            const float g = wg ? dot_f16(d, (const uint16_t *)(wg + rb * j), x16) : 0.f;
-            hval[k] = wg ? (g > 0.f ? g : 0.f) * u : (u > 0.f ? u : 0.f);
-        }
-    });
+    host_upgate(c, m, il, na);
     lap(2);
     lap(3);
-    const unsigned char * wd = (const unsigned char *)down.host;
-    const int n_units = d / 32;
-    c->pool->run([&](int t, int nt) {
-        const int u0 = (int)((long long)n_units * t / nt), u1 = (int)((long long)n_units * (t + 1) / nt);
-        const int c0 = u0 * 32, c1 = u1 * 32;
-        for (int i = c0; i < c1; ++i) out[i] = 0.f;
-        for (int k = 0; k < na; ++k) {
-            const uint16_t hb = f2h(hval[k]);
-            if (k + 2 < na) prefetch_bytes(wd + rb * c->act[k + 2] + (size_t)c0 * 2, (size_t)(c1 - c0) * 2);
-            if (hb == 0) continue;
-            const float a = h2f(hb);
-            const uint16_t * row = (const uint16_t *)(wd + rb * c->act[k]);
-#ifdef PI_COLD_SIMD
-            const __m256 av = _mm256_set1_ps(a);
-            for (int i = c0; i < c1; i += 8)
-                _mm256_storeu_ps(out + i, _mm256_fmadd_ps(_mm256_cvtph_ps(_mm_loadu_si128((const __m128i *)(row + i))), av, _mm256_loadu_ps(out + i)));
-#else
-            for (int i = c0; i < c1; ++i) out[i] = fmaf(h2f(row[i]), a, out[i]);
-#endif
-        }
-    });
+    host_down(c, m, il, na, nullptr, out);
     __atomic_store_n(&c->flags[32], seq, __ATOMIC_RELEASE);          // the reduction may add the host share
     lap(4);
     if (c->trace) { ++c->n_calls; c->n_cold_active += na; c->t_last_return = now(); }

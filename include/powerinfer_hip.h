@@ -308,6 +308,19 @@ PI_API int pi_k_assemble_rows_f16(const void * W_f16, const void * W_rest_f16, c
                                   void * out_f16, pi_stream_t stream);
 PI_API int pi_k_embed_batch_q4(const void * table_q4, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream);
 
+/* The whole Q4_0 sparse FFN behind fc1 as one launch plus the reduction, for layers whose active neurons are all computed on the device
+ * (every neuron resident: no hot words, no second matrices; or the split of pi_k_pred_upgate_q4_split with the non-resident rows in
+ * pinned host memory).  A workgroup's 32 neurons are one Q8_0 block of h, so the launch of pi_k_pred_upgate_q4 goes on with the down rows
+ * of its own neurons (arithmetic of pi_k_axpy_q4_partials) and stores one partial output vector per workgroup;
+ * pi_k_sparse_ffn_q4_reduce adds the ff / 32 vectors in order plus the residual(s) and counts the active neurons. */
+PI_API int pi_k_sparse_ffn_q4_partials(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                                       const void * up_q4, const void * gate_q4, const void * down_t_q4,
+                                       const void * up_rest_q4, const void * gate_rest_q4, const void * down_t_rest_q4,
+                                       int cols, const float * x, const pi_norm * norm, const uint32_t * hot_words, const int32_t * hot_prefix,
+                                       float * logits, float * h_dense, pi_workspace * ws, pi_stream_t stream);
+PI_API int pi_k_sparse_ffn_q4_reduce(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out, int32_t * n_active,
+                                     pi_workspace * ws, pi_stream_t stream);
+
 /* Hand-over points between the stream and host threads that compute the non-resident neurons of a hybrid layer (the CPU half of
  * llm_build_sparse_mul_mat / llm_build_sparse_axpy, llama.cpp:4581-4593, 4635-4646) without the host launching anything in between.
  * flags_pinned: 64 words of pinned host memory (words 0 and 8 written by the device, words 16 and 32 by the host, word 48 = the host's

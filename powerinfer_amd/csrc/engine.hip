@@ -234,24 +234,24 @@ int layer_forward(pi_model * m, int il, bool last_token) {
             if (pi::cold_layer_async(m->cold, il) && !m->capture) PI_TRY(pi::cold_layer_q4_queue(m->cold, il, m, st));
             else PI_TRY(pi::cold_layer_q4(m->cold, il, m, st, cap));
         } else {
-            // every neuron on the GPU, or the non-resident neurons' rows read from pinned host memory by the same two launches
+            // every neuron on the GPU, or the non-resident neurons' rows read from pinned host memory: one launch carries the predictor,
+            // the up/gate rows and - a workgroup's 32 neurons being one Q8_0 block of h - the down rows; then the reduction
             const uint32_t * hw = layer_hybrid ? m->hot_words[il] : nullptr;
             const int32_t * hpx = layer_hybrid ? m->hot_prefix[il] : nullptr;
-            PI_TRY(pi_k_pred_upgate_q4_split(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, gp,
-                                             layer_hybrid ? m->rest_up[il] : nullptr, (layer_hybrid && !falcon) ? m->rest_gate[il] : nullptr,
-                                             d, ffn_in, &fn, hw, hpx, m->pred_logits, m->h_dense, nullptr, m->ws, st));
-            PI_TRY(pi_k_axpy_q4_partials_split(down.dev, layer_hybrid ? m->rest_down[il] : nullptr, d, ff, m->h_dense, hw, hpx, m->ws, st));
+            PI_TRY(pi_k_sparse_ffn_q4_partials(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, gp, down.dev,
+                                               layer_hybrid ? m->rest_up[il] : nullptr, (layer_hybrid && !falcon) ? m->rest_gate[il] : nullptr,
+                                               layer_hybrid ? m->rest_down[il] : nullptr, d, ffn_in, &fn, hw, hpx, m->pred_logits, m->h_dense, m->ws, st));
             if (cap) {
                 float * ffo = m->cap_ffn + (size_t)il * d;
-                PI_TRY(pi_k_axpy_q4_reduce(ff, d, PI_EPI_NONE, nullptr, nullptr, ffo, n_act, m->ws, st));
+                PI_TRY(pi_k_sparse_ffn_q4_reduce(ff, d, PI_EPI_NONE, nullptr, nullptr, ffo, n_act, m->ws, st));
                 PI_HIP_TRY(hipMemcpyAsync(m->x2, ffo, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
                 PI_TRY(pi::add_vec(m->x2, falcon ? m->attn_out : m->ffn_inp, d, st));
                 if (falcon) PI_TRY(pi::add_vec(m->x2, x, d, st));
                 PI_HIP_TRY(hipMemcpyAsync(m->cap_logits + (size_t)il * ff, m->pred_logits, sizeof(float) * ff, hipMemcpyDeviceToDevice, st));
             } else if (!falcon) {
-                PI_TRY(pi_k_axpy_q4_reduce(ff, d, PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, n_act, m->ws, st));
+                PI_TRY(pi_k_sparse_ffn_q4_reduce(ff, d, PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, n_act, m->ws, st));
             } else {
-                PI_TRY(pi_k_axpy_q4_reduce(ff, d, PI_EPI_ADD2, m->attn_out, x, m->x2, n_act, m->ws, st));
+                PI_TRY(pi_k_sparse_ffn_q4_reduce(ff, d, PI_EPI_ADD2, m->attn_out, x, m->x2, n_act, m->ws, st));
             }
         }
         if (cap) PI_HIP_TRY(hipMemcpyAsync(m->cap_src + (size_t)il * d, ffn_in, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
@@ -804,10 +804,9 @@ int pi_model_time_section(pi_model * m, int section, int rounds, float * ms_tota
                     continue;
                 }
                 if (q4 && fc2.type == PI_TYPE_F16 && pi_k_pred_upgate_q4_supported(ff, (int)fc1.ne1, d)) {
-                    PI_TRY(pi_k_pred_upgate_q4(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, d, fin, &fn,
-                                               nullptr, nullptr, m->pred_logits, m->h_dense, nullptr, m->ws, st));
-                    PI_TRY(pi_k_axpy_q4_partials(down.dev, d, ff, m->h_dense, nullptr, nullptr, m->ws, st));
-                    PI_TRY(pi_k_axpy_q4_reduce(ff, d, PI_EPI_ADD, fin, nullptr, m->x2, m->n_active + il, m->ws, st));
+                    PI_TRY(pi_k_sparse_ffn_q4_partials(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, down.dev,
+                                                       nullptr, nullptr, nullptr, d, fin, &fn, nullptr, nullptr, m->pred_logits, m->h_dense, m->ws, st));
+                    PI_TRY(pi_k_sparse_ffn_q4_reduce(ff, d, PI_EPI_ADD, fin, nullptr, m->x2, m->n_active + il, m->ws, st));
                     ++n;
                     continue;
                 }

@@ -1294,6 +1294,7 @@ __global__ __launch_bounds__(kPfBlock) void ffn_reduce_kernel(const float * __re
 // h_dense and the Q8_0 blocks may be pinned host memory (a hybrid layer's host share reads them after the launch).
 // ---------------------------------------------------------------------------------------------------
 struct __attribute__((packed)) pi_q8_host_block { uint16_t d; int8_t qs[32]; };
+constexpr int kAqChunkFused = 8;           // down rows in flight per wave in the fused form
 
 // SPLIT: the neurons outside the hot words are computed here too, from a second pair of matrices that holds exactly those
 // neurons' rows in ascending order (rows in pinned host memory, fetched over the host link by the loads below).
@@ -1301,7 +1302,11 @@ struct __attribute__((packed)) pi_q8_host_block { uint16_t d; int8_t qs[32]; };
 // logits (to `logits` and `logits2`), the mask words and the Q8_0 blocks of the input; 2 reads the logits back from `logits2`
 // instead of computing them, and writes h only for the neurons of the hot words (h or 0): the other entries of that vector
 // belong to the host.
-template <int RCH, bool GATE, bool SPLIT, int PHASE = 0>
+// FUSE: the workgroup's 32 neurons are exactly one Q8_0 block of h, so when every active neuron is computed here (all of them resident,
+// or SPLIT) the launch goes on with the down projection: h of the group is quantised as the CPU path quantises the dense vector
+// (ggml.c:14465-14618), and each wave adds its 512-column slice of the down rows of the neurons with a non-zero quant, in ascending
+// order and with axpy_q4_groups_kernel's arithmetic; the workgroup's partial output vector goes to `partial` for ffn_reduce_kernel.
+template <int RCH, bool GATE, bool SPLIT, int PHASE = 0, bool FUSE = false>
 __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
                                                                      const pi_block_q4_0 * __restrict__ Wup, const pi_block_q4_0 * __restrict__ Wgate,
                                                                      const pi_block_q4_0 * __restrict__ Wup_rest, const pi_block_q4_0 * __restrict__ Wgate_rest,
@@ -1309,8 +1314,12 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
                                                                      const uint32_t * __restrict__ hot_words, const int32_t * __restrict__ hot_prefix,
                                                                      float * __restrict__ logits, uint32_t * __restrict__ words, uint32_t * __restrict__ words_hot,
                                                                      float * __restrict__ h_dense, pi_q8_host_block * __restrict__ xq_out,
-                                                                     float * __restrict__ logits2) {
+                                                                     float * __restrict__ logits2,
+                                                                     const pi_block_q4_0 * __restrict__ Wd, const pi_block_q4_0 * __restrict__ Wd_rest,
+                                                                     float * __restrict__ partial) {
+    static_assert(!FUSE || PHASE == 0, "the fused form is one launch");
     constexpr int cols = 4096, r = RCH * 512, nb = cols / 32, CH = kPfChunk;
+    __shared__ float  hs[32];
     __shared__ float  lg[32];
     __shared__ double red[2][kPfWaves];
     __shared__ float  part[kPfWaves][CH][2];
@@ -1447,6 +1456,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
             if (PHASE == 1) logits2[n0 + lane] = my_logit;
             if (PHASE == 0 && !((sel >> lane) & 1u)) h_dense[n0 + lane] = 0.0f;
             if (PHASE == 2 && ((hot >> lane) & 1u) && !((sel >> lane) & 1u)) h_dense[n0 + lane] = 0.0f;
+            if (FUSE) hs[lane] = 0.0f;             // ordered before the h values below by the barrier inside the first chunk
         }
         if (lane == 0) { words[blockIdx.x] = mask; if (words_hot) words_hot[blockIdx.x] = sel; }
     }
@@ -1506,9 +1516,58 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
             int nj = 0;
 #pragma unroll
             for (int jj = 0; jj < CH; ++jj) if (jj == j) nj = nrn[jj];
-            h_dense[nj] = GATE ? __fmul_rn(fmaxf(g, 0.0f), u) : fmaxf(u, 0.0f);
+            const float hval = GATE ? __fmul_rn(fmaxf(g, 0.0f), u) : fmaxf(u, 0.0f);
+            h_dense[nj] = hval;
+            if (FUSE) hs[nj - n0] = hval;
         }
         if (c0 + CH < n) __syncthreads();                         // part[] is reused by the next chunk
+    }
+    if (FUSE) {
+        // ---- C: Q8_0 of the group's h, then the down rows ------------------------------------------------------------
+        __syncthreads();
+        const float hvv = hs[lane & 31];
+        float hmax = fabsf(hvv);
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) hmax = fmaxf(hmax, __shfl_xor(hmax, o, PI_WAVE));
+        const float dh = pi_round_f16(pi_div(hmax, 127.0f)), idh = (hmax != 0.0f) ? pi_div(127.0f, hmax) : 0.0f;
+        const int qh = (int)rintf(__fmul_rn(hvv, idh));
+        const uint32_t nz = (uint32_t)__ballot(qh != 0) & sel;     // neurons that add something, ascending
+        const int nrows = __popc(nz);
+        float acc[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+        for (int k0 = 0; k0 < nrows; k0 += kAqChunkFused) {
+            uint32_t q[kAqChunkFused][2];
+            uint16_t dw[kAqChunkFused];
+            int alpha[kAqChunkFused];
+#pragma unroll
+            for (int j = 0; j < kAqChunkFused; ++j) {
+                if (k0 + j < nrows) {
+                    const int bit = select_nth_bit(nz, k0 + j);
+                    alpha[j] = __builtin_amdgcn_readlane(qh, bit);
+                    const int below = __popc(hot & ((1u << bit) - 1u));
+                    const bool rest = SPLIT && !((hot >> bit) & 1u);
+                    const size_t row = rest ? (size_t)(n0 - base_row + bit - below) : (size_t)(base_row + below);
+                    const pi_block_q4_0 * wb = (rest ? Wd_rest : Wd) + row * nb + blk;
+                    __builtin_memcpy(&dw[j], &wb->d, 2);
+                    __builtin_memcpy(q[j], wb->qs + qoff, 8);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < kAqChunkFused; ++j) {
+                if (k0 + j < nrows) {
+                    const float d = __fmul_rn(pi_f16_from_bits(dw[j]), dh);
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) {
+                        const int v = (int)((q[j][i >> 2] >> ((i & 3) * 8 + shift)) & 0xF) - 8;
+                        acc[i] = __fadd_rn(acc[i], __fmul_rn((float)(v * alpha[j]), d));
+                    }
+                }
+            }
+        }
+        float4 * po = reinterpret_cast<float4 *>(partial + (size_t)blockIdx.x * cols + cbase);
+        po[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+        po[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
     }
 }
 
@@ -3769,13 +3828,49 @@ int pi_k_pred_upgate_q4_split(const void * fc2_f16, int ff, int r, const float *
     const pi_block_q4_0 * u = (const pi_block_q4_0 *)up_q4; const pi_block_q4_0 * g = (const pi_block_q4_0 *)gate_q4;
     const dim3 grid(ff / 32), block(kPfBlock);
     const pi_block_q4_0 * ur = (const pi_block_q4_0 *)up_rest_q4; const pi_block_q4_0 * gr = (const pi_block_q4_0 *)gate_rest_q4;
-#define PI_PQ_LAUNCH(RCH, GATE, SPLIT) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, GATE, SPLIT>), grid, block, 0, st, w2, hidden, u, g, ur, gr, x, na, threshold, hot_words, hot_prefix, logits, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)xq8_out, nullptr)
+#define PI_PQ_LAUNCH(RCH, GATE, SPLIT) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, GATE, SPLIT>), grid, block, 0, st, w2, hidden, u, g, ur, gr, x, na, threshold, hot_words, hot_prefix, logits, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)xq8_out, nullptr, nullptr, nullptr, nullptr)
 #define PI_PQ_LAUNCH_S(RCH, GATE) do { if (ur) PI_PQ_LAUNCH(RCH, GATE, true); else PI_PQ_LAUNCH(RCH, GATE, false); } while (0)
     if (r == 1024) { if (g) PI_PQ_LAUNCH_S(2, true); else PI_PQ_LAUNCH_S(2, false); }
     else           { if (g) PI_PQ_LAUNCH_S(1, true); else PI_PQ_LAUNCH_S(1, false); }
 #undef PI_PQ_LAUNCH_S
 #undef PI_PQ_LAUNCH
     return pi::check_launch("pi_k_pred_upgate_q4");
+}
+
+int pi_k_sparse_ffn_q4_partials(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
+                                const void * up_q4, const void * gate_q4, const void * down_t_q4,
+                                const void * up_rest_q4, const void * gate_rest_q4, const void * down_t_rest_q4,
+                                int cols, const float * x, const pi_norm * norm, const uint32_t * hot_words, const int32_t * hot_prefix,
+                                float * logits, float * h_dense, pi_workspace * ws, pi_stream_t stream) {
+    if (!fc2_f16 || !hidden || !up_q4 || !down_t_q4 || !x || !h_dense || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_q4_partials: null pointer");
+    const bool split = up_rest_q4 != nullptr;
+    if (split != (down_t_rest_q4 != nullptr) || (split && (!hot_words || !hot_prefix || (gate_q4 != nullptr) != (gate_rest_q4 != nullptr))) || (!split && hot_words))
+        return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_q4_partials: either every neuron's rows are in the first matrices (no hot words), or the second matrices and hot_words / hot_prefix come together");
+    if (!pi_k_pred_upgate_q4_supported(ff, r, cols) || ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn_q4_partials: shape outside the fused kernel (cols 4096, r 512 or 1024, ff % 32 == 0) or the workspace");
+    const NormArgs na = to_norm(norm);
+    if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_q4_partials: vectors must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    const __half * w2 = (const __half *)fc2_f16;
+    const pi_block_q4_0 * u = (const pi_block_q4_0 *)up_q4; const pi_block_q4_0 * g = (const pi_block_q4_0 *)gate_q4; const pi_block_q4_0 * dn = (const pi_block_q4_0 *)down_t_q4;
+    const pi_block_q4_0 * ur = (const pi_block_q4_0 *)up_rest_q4; const pi_block_q4_0 * gr = (const pi_block_q4_0 *)gate_rest_q4; const pi_block_q4_0 * dr = (const pi_block_q4_0 *)down_t_rest_q4;
+    const dim3 grid(ff / 32), block(kPfBlock);
+#define PI_PQF(RCH, GATE, SPLIT) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, GATE, SPLIT, 0, true>), grid, block, 0, st, w2, hidden, u, g, ur, gr, x, na, threshold, hot_words, hot_prefix, logits, ws->words, (uint32_t *)nullptr, h_dense, (pi_q8_host_block *)nullptr, (float *)nullptr, dn, dr, ws->ffn_partial)
+#define PI_PQF_S(RCH, GATE) do { if (split) PI_PQF(RCH, GATE, true); else PI_PQF(RCH, GATE, false); } while (0)
+    if (r == 1024) { if (g) PI_PQF_S(2, true); else PI_PQF_S(2, false); }
+    else           { if (g) PI_PQF_S(1, true); else PI_PQF_S(1, false); }
+#undef PI_PQF_S
+#undef PI_PQF
+    return pi::check_launch("pi_k_sparse_ffn_q4_partials");
+}
+
+int pi_k_sparse_ffn_q4_reduce(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out, int32_t * n_active,
+                              pi_workspace * ws, pi_stream_t stream) {
+    if (!out || !ws || cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_q4_reduce: bad arguments");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_q4_reduce: bad epilogue arguments");
+    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, ff / 32, cols,
+                       ws->words, ff / 32, n_active, epilogue, add1, add2, out);
+    return pi::check_launch("pi_k_sparse_ffn_q4_reduce");
 }
 
 int pi_k_pred_q4_logits(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
@@ -3786,7 +3881,7 @@ int pi_k_pred_q4_logits(const void * fc2_f16, int ff, int r, const float * hidde
     if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_pred_q4_logits: vectors must be 16-byte aligned");
     const dim3 grid(ff / 32), block(kPfBlock);
     const pi_block_q4_0 * none = nullptr;
-#define PI_PQ1(RCH) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, false, false, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, none, x, na, threshold, (const uint32_t *)nullptr, (const int32_t *)nullptr, logits, ws->words, (uint32_t *)nullptr, (float *)nullptr, (pi_q8_host_block *)xq8_out, logits_dev)
+#define PI_PQ1(RCH) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, false, false, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, none, x, na, threshold, (const uint32_t *)nullptr, (const int32_t *)nullptr, logits, ws->words, (uint32_t *)nullptr, (float *)nullptr, (pi_q8_host_block *)xq8_out, logits_dev, none, none, (float *)nullptr)
     if (r == 1024) PI_PQ1(2); else PI_PQ1(1);
 #undef PI_PQ1
     return pi::check_launch("pi_k_pred_q4_logits");
@@ -3801,7 +3896,7 @@ int pi_k_upgate_q4_hot_rows(int ff, float threshold, const void * up_q4, const v
     const dim3 grid(ff / 32), block(kPfBlock);
     const pi_block_q4_0 * none = nullptr;
     const pi_block_q4_0 * u = (const pi_block_q4_0 *)up_q4; const pi_block_q4_0 * g = (const pi_block_q4_0 *)gate_q4;
-#define PI_PQ2(GATE) hipLaunchKernelGGL((pred_upgate_q4_kernel<1, GATE, false, 2>), grid, block, 0, (hipStream_t)stream, (const __half *)nullptr, (const float *)nullptr, u, g, none, none, x, na, threshold, hot_words, hot_prefix, (float *)nullptr, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)nullptr, const_cast<float *>(logits_dev))
+#define PI_PQ2(GATE) hipLaunchKernelGGL((pred_upgate_q4_kernel<1, GATE, false, 2>), grid, block, 0, (hipStream_t)stream, (const __half *)nullptr, (const float *)nullptr, u, g, none, none, x, na, threshold, hot_words, hot_prefix, (float *)nullptr, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)nullptr, const_cast<float *>(logits_dev), none, none, (float *)nullptr)
     if (g) PI_PQ2(true); else PI_PQ2(false);
 #undef PI_PQ2
     return pi::check_launch("pi_k_upgate_q4_hot_rows");

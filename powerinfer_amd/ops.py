@@ -198,6 +198,35 @@ class SparseFFN:
         return dict(logits=self.logits.download(np.float32), h=h, xq8=xq8.download(np.uint8),
                     n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32))
 
+    def forward_q4_one_launch(self, x_ffn, x_pred, epilogue=pl.EPI_NONE, resid=None, rest=None):
+        """The Q4_0 layer as the decode loop runs it when every active neuron is computed on the device: fc1, then
+        pi_k_sparse_ffn_q4_partials (fc2 + mask + up/gate + down rows of each workgroup's 32 neurons) and pi_k_sparse_ffn_q4_reduce.
+        With a bucket, `rest` = (up, gate, down_t) rows of the neurons outside it in ascending order (the split form: those rows may
+        be pinned host memory in the engine).  Returns dict(logits, h, n_active, out)."""
+        L = self.L
+        if self.wtype != pl.Q4_0 or not L.pi_k_pred_upgate_q4_supported(self.ff, self.r, self.d):
+            raise pl.PiError("forward_q4_one_launch: type or shape outside the fused kernels")
+        hw, hp = self._hot_tables()
+        if (hw is None) != (rest is None):
+            raise pl.PiError("forward_q4_one_launch: a bucket and the other neurons' rows go together")
+        p = lambda b: b.ptr if b is not None else None  # noqa: E731
+        keep = [DevBuf(host=a) if a is not None else None for a in (rest or (None, None, None))]
+        self.x.upload(np.asarray(x_ffn, np.float32))
+        self.xp.upload(np.asarray(x_pred, np.float32))
+        if resid is not None:
+            self.resid.upload(np.asarray(resid, np.float32))
+        check(L.pi_memset(self.h_dense.ptr, 0xFF, self.h_dense.nbytes), "memset")      # the kernel must write every entry
+        nrm = pl.norm_arg(self.norm_kind, self.eps, self.norm_w, self.norm_b)
+        check(L.pi_k_gemv(pl.F16, self.fc1.ptr, self.r, self.d, self.xp.ptr, None, pl.EPI_RELU, None, None, self.hidden.ptr, None), "fc1")
+        check(L.pi_k_sparse_ffn_q4_partials(self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, self.up.ptr, p(self.gate), self.down.ptr,
+                                            p(keep[0]), p(keep[1]), p(keep[2]), self.d, self.x.ptr, nrm, p(hw), p(hp),
+                                            self.logits.ptr, self.h_dense.ptr, self.ws, None), "sparse_ffn_q4_partials")
+        check(L.pi_k_sparse_ffn_q4_reduce(self.ff, self.d, epilogue, self.resid.ptr if epilogue else None, None, self.out.ptr,
+                                          self.n_active.ptr, self.ws, None), "sparse_ffn_q4_reduce")
+        pl.sync()
+        return dict(logits=self.logits.download(np.float32), h=self.h_dense.download(np.float32),
+                    n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32))
+
     def forward_q4_handover(self, x_ffn, x_pred, host_h, host_out, limit_s=20.0):
         """The same layer with the host share computed while the stream runs, nothing launched in between (what the decode loop
         queues for a hybrid Q4_0 layer): pi_k_pred_q4_logits -> pi_k_host_signal -> pi_k_upgate_q4_hot_rows -> pi_k_host_signal ->

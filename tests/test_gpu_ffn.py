@@ -210,6 +210,47 @@ def test_q4_fused_route_7b_shape(has_gate, norm):
     ffn.close()
 
 
+@pytest.mark.parametrize("has_gate,norm,hot_frac", [(True, 1, 1.0), (False, 2, 1.0), (True, 1, 0.6), (False, 0, 0.5)])
+def test_q4_one_launch_route_7b_shape(has_gate, norm, hot_frac):
+    """pi_k_sparse_ffn_q4_partials + pi_k_sparse_ffn_q4_reduce: the Q4_0 layer in one launch plus the reduction, every neuron's rows
+    in one set of matrices or split into a compact resident set and the others (ascending).  Against the CPU reference evaluated
+    under the device's own logits, and against the two-launch route (same arithmetic per element, partial sums grouped by 32 neurons
+    instead of 128)."""
+    from powerinfer_amd import lib as pl
+    from powerinfer_amd.ops import SparseFFN
+    d, ff, r, T = 4096, 11008, 1024, 2
+    L = synth.make_ffn_layer(seed=70 + norm, d=d, ff=ff, r=r, wtype=ol.Q4_0, has_gate=has_gate, T=T)
+    rng = np.random.default_rng(7)
+    nw = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32) if norm else None
+    nb = (0.1 * rng.standard_normal(d)).astype(np.float32) if norm == 2 else None
+    eps = 1e-5
+    O, P = ol.oracle(), ol._ptr
+    bucket, rest = None, None
+    if hot_frac < 1.0:
+        gid, bucket = synth.gpu_split(L["p"], hot_frac)
+        cold = np.flatnonzero(gid != 1)
+        rest = (L["up"][cold], L["gate"][cold] if has_gate else None, L["down_t"][cold])
+    ffn = SparseFFN(d, ff, r, ol.Q4_0, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], bucket=bucket, norm_kind=norm, norm_w=nw, norm_b=nb, eps=eps)
+    ref2 = SparseFFN(d, ff, r, ol.Q4_0, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], norm_kind=norm, norm_w=nw, norm_b=nb, eps=eps)
+    for t in range(T):
+        x = np.ascontiguousarray(L["x"][t:t + 1], np.float32)
+        xn = x.copy()
+        if norm == 1:
+            O.pio_rms_norm(P(x), d, 1, eps, P(xn)); xn = np.ascontiguousarray(xn * nw, np.float32)
+        elif norm == 2:
+            O.pio_norm(P(x), d, 1, eps, P(xn)); xn = np.ascontiguousarray(xn * nw + nb, np.float32)
+        resid = rng.standard_normal(d).astype(np.float32)
+        res = ffn.forward_q4_one_launch(x[0], x[0], epilogue=pl.EPI_ADD, resid=resid, rest=rest)
+        two = ref2.forward_q4_fused(x[0], x[0], epilogue=pl.EPI_ADD, resid=resid)
+        assert np.array_equal(res["logits"], two["logits"]) and np.array_equal(res["h"], two["h"])
+        assert res["n_active"] == two["n_active"] == int((~(res["logits"] < 0.0)).sum())
+        assert rel_err(res["out"], two["out"]) < 1e-5
+        ou = under(L, d, ff, ol.Q4_0, has_gate, xn, res["logits"])
+        assert rel_err(res["h"], ou["h"]) < 1e-4
+        assert rel_err(res["out"] - resid, ou["out"]) < FFN_REL_TOL
+    ffn.close(), ref2.close()
+
+
 @pytest.mark.parametrize("has_gate,norm", [(True, 1), (False, 2)])
 def test_f16_fused_route_hybrid_share(has_gate, norm):
     """The fused F16 kernels on a hot/cold split at the 7B width: the resident 60 % come from compact matrices through the hot

@@ -4151,7 +4151,7 @@ static int gemm_launch(const char * who, const void * W, int rows, int cols, con
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
         return pi::fail(PI_E_ARG, "batched mat-mul: bad epilogue arguments");
     // row tiles per wave: enough workgroups to fill the chip first, then as few reads of the activations as possible
-    const int rt = rows >= 16384 ? 4 : rows >= 8192 ? 2 : 1;
+    const int rt = rows >= 16384 ? 4 : rows >= 5120 ? 2 : 1;      // (two tiles already at 5120 rows: the activations, re-read per row tile, are what limits one tile per wave)
 #define PI_GEMM_T16(RT) hipLaunchKernelGGL((gemm_t16_f16_kernel<RT>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(kBlock), 0, (hipStream_t)stream, \
                        (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any)
 #define PI_GEMM_LDS(RT) hipLaunchKernelGGL((gemm_t16_lds_f16_kernel<RT>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(kBlock), 0, (hipStream_t)stream, \

@@ -255,6 +255,7 @@ def main():
     ap.add_argument("--layers", type=int, default=32, help="only for quick trials; the reported workload uses 32")
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--prompt-bench", type=int, default=1024, help="length of the prompt timed for the prompt_phase entry (0 = skip)")
+    ap.add_argument("--no-q4", action="store_true", help="config 1: skip the extra object with the Q4_0 split model (configs[2]) measured in a child process (about 25 s)")
     ap.add_argument("--no-ref-host", action="store_true", help="skip the leg that runs the reference's llama.cpp on this backend (about 40 s)")
     ap.add_argument("--cpu-tokens", type=int, default=320, help="decode tokens timed on the host for the cpu_baseline leg (about 10 s of CPU work)")
     ap.add_argument("--config", type=int, default=1, choices=[1, 2, 3, 4],
@@ -503,6 +504,21 @@ def main():
             del keep2
         except Exception as e:
             out["prompt_phase"] = {"error": repr(e)[:200]}
+    if args.config == 1 and not hybrid and not args.no_q4:
+        # the Q4_0 half of the metric (configs[2]: hottest 60 % of neurons on the GPU, the rest on host threads) as an extra object:
+        # the same script in a child process, so that this process's line stays the FP16 one
+        try:
+            import subprocess
+            r = subprocess.run([sys.executable, os.path.abspath(__file__), "--config", "2", "--no-cpu", "--no-ref-host", "--steps", str(args.steps),
+                                "--warmup", str(args.warmup), "--prompt", str(args.prompt), "--layers", str(args.layers), "--prompt-bench", str(args.prompt_bench)],
+                               capture_output=True, text=True, timeout=600)
+            q = json.loads(r.stdout.strip().splitlines()[-1])
+            out["q4_0_split"] = {"value": q["value"], "unit": q["unit"], "ms_per_step": q["ms_per_step"], "workload": q["config"]["workload"],
+                                 "mean_active_per_layer": q["config"]["mean_active_per_layer"], "hbm_frac_touched": q["token_loop"]["hbm_frac_touched"],
+                                 "rest_read_by_gpu": {k: q["rest_read_by_gpu"].get(k) for k in ("value", "unit", "ms_per_step")} if "rest_read_by_gpu" in q else None,
+                                 "prompt_phase": {k: q["prompt_phase"].get(k) for k in ("tokens", "ms", "tok_per_s")} if "prompt_phase" in q else None}
+        except Exception as e:          # a reporting extra: never costs the bench line
+            out["q4_0_split"] = {"error": repr(e)[:200]}
     if not args.no_ref_host and args.config == 1:
         try:
             rh = reference_host_on_this_backend()

@@ -458,6 +458,66 @@ void pio_rope(const float * x, int n_embd_head, int n_head, int T, const int32_t
         }
 }
 
+/* RoPE with the scaling operands (ggml_compute_forward_rope_f32 with rope_yarn, ggml.c:11124-11161, 11163-11325): the angle is
+ * freq_scale * theta (linear scaling); with ext_factor != 0 it is mixed with the unscaled angle by a ramp over the pair index
+ * between the two correction dimensions, and cos / sin are multiplied by attn_factor * (1 + 0.1 ln(1 / freq_scale)).  NeoX mode
+ * hands the ramp the rotation fraction (ic / n_dims - ib) through an integer parameter, as the reference does: for ib == 0 that
+ * is always 0. */
+static float yarn_corr_dim(int n_dims, int n_orig_ctx, float n_rot, float base) {
+    return n_dims * logf(n_orig_ctx / (n_rot * 2 * (float)M_PI)) / (2 * logf(base));
+}
+static void yarn_angle(float theta_extrap, float freq_scale, const float corr[2], int64_t i0, float ext_factor, float mscale, float * c, float * sn) {
+    const float theta_interp = freq_scale * theta_extrap;
+    float theta = theta_interp;
+    if (ext_factor != 0.0f) {
+        const float y = (i0 / 2 - corr[0]) / fmaxf(0.001f, corr[1] - corr[0]);
+        const float ramp_mix = (1 - fminf(1, fmaxf(0, y))) * ext_factor;
+        theta = theta_interp * (1 - ramp_mix) + theta_extrap * ramp_mix;
+        mscale *= 1.0f + 0.1f * logf(1.0f / freq_scale);
+    }
+    *c = cosf(theta) * mscale;
+    *sn = sinf(theta) * mscale;
+}
+void pio_rope_ext(const float * x, int n_embd_head, int n_head, int T, const int32_t * pos, int n_dims, int mode, int n_orig_ctx,
+                  float freq_base, float freq_scale, float ext_factor, float attn_factor, float beta_fast, float beta_slow, float * out) {
+    const float theta_scale = powf(freq_base, -2.0f / n_dims);
+    const float inv_ndims = -1.0f / n_dims;
+    const int is_neox = mode & 2;
+    float corr[2];
+    corr[0] = fmaxf(0, floorf(yarn_corr_dim(n_dims, n_orig_ctx, beta_fast, freq_base)));
+    corr[1] = fminf(n_dims - 1, ceilf(yarn_corr_dim(n_dims, n_orig_ctx, beta_slow, freq_base)));
+    memcpy(out, x, sizeof(float) * (size_t)n_embd_head * n_head * T);
+    for (int t = 0; t < T; ++t)
+        for (int hd = 0; hd < n_head; ++hd) {
+            const float * s = x + ((size_t)t * n_head + hd) * n_embd_head;
+            float * o = out + ((size_t)t * n_head + hd) * n_embd_head;
+            float theta_base = (float)pos[t];
+            if (!is_neox) {
+                for (int i0 = 0; i0 < n_embd_head; i0 += 2) {
+                    float c, sn;
+                    yarn_angle(theta_base, freq_scale, corr, i0, ext_factor, attn_factor, &c, &sn);
+                    theta_base *= theta_scale;
+                    const float x0 = s[i0], x1 = s[i0 + 1];
+                    o[i0]     = x0 * c - x1 * sn;
+                    o[i0 + 1] = x0 * sn + x1 * c;
+                }
+            } else {
+                theta_base *= freq_scale;
+                for (int ib = 0; ib < n_embd_head / n_dims; ++ib)
+                    for (int ic = 0; ic < n_dims; ic += 2) {
+                        const float cur_rot = inv_ndims * ic - ib;
+                        float c, sn;
+                        yarn_angle(theta_base, freq_scale, corr, (int64_t)cur_rot, ext_factor, attn_factor, &c, &sn);
+                        theta_base *= theta_scale;
+                        const int i0 = ib * n_dims + ic / 2;
+                        const float x0 = s[i0], x1 = s[i0 + n_dims / 2];
+                        o[i0]              = x0 * c - x1 * sn;
+                        o[i0 + n_dims / 2] = x0 * sn + x1 * c;
+                    }
+            }
+        }
+}
+
 /* softmax: ggml_compute_forward_soft_max_f32, ggml.c:10708-10775.  exp goes through a table indexed
  * by the fp16 bit pattern of (x - max) holding fp16(expf(fp32(that fp16))) (table built at
  * ggml.c:2188-2196); the sum is in double; the row is scaled by (float)(1/sum). */

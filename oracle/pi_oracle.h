@@ -58,6 +58,9 @@ PIO_API void pio_norm(const float * x, int64_t n, int T, float eps, float * out)
 /* x [n_embd_head, n_head, T]; mode 0 = adjacent pairs (LLaMA), 2 = NeoX halves (Falcon) */
 PIO_API void pio_rope(const float * x, int n_embd_head, int n_head, int T, const int32_t * pos,
                       int n_dims, int mode, float freq_base, float freq_scale, float * out);
+/* the same with linear and YaRN scaling (ggml_rope_custom's operands; ext_factor 0 and attn_factor 1 give pio_rope) */
+PIO_API void pio_rope_ext(const float * x, int n_embd_head, int n_head, int T, const int32_t * pos, int n_dims, int mode, int n_orig_ctx,
+                          float freq_base, float freq_scale, float ext_factor, float attn_factor, float beta_fast, float beta_slow, float * out);
 PIO_API void pio_soft_max(const float * x, int64_t n, int64_t rows, float * out);
 
 /* ascending indices of idx[i] >= threshold; returns the count */

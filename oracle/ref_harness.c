@@ -171,6 +171,25 @@ REF_API int ref_rope(const float * x, int n_embd_head, int n_head, int T, const 
     return 0;
 }
 
+/* the same with the scaling operands of ggml_rope_custom: linear (freq_scale) and YaRN (n_orig_ctx, ext_factor, attn_factor, beta_fast, beta_slow) */
+REF_API int ref_rope_ext(const float * x, int n_embd_head, int n_head, int T, const int32_t * pos, int n_dims, int mode, int n_orig_ctx,
+                         float freq_base, float freq_scale, float ext_factor, float attn_factor, float beta_fast, float beta_slow, float * out) {
+    size_t n = (size_t)n_embd_head * n_head * T;
+    struct ggml_context * ctx = new_ctx(n * 16 + (1u << 20));
+    if (!ctx) return 1;
+    struct ggml_tensor * tx = ggml_new_tensor_3d(ctx, GGML_TYPE_F32, n_embd_head, n_head, T);
+    memcpy(tx->data, x, n * 4);
+    struct ggml_tensor * tp = ggml_new_tensor_1d(ctx, GGML_TYPE_I32, T);
+    memcpy(tp->data, pos, (size_t)T * 4);
+    struct ggml_tensor * r = ggml_rope_custom(ctx, tx, tp, n_dims, mode, 0, n_orig_ctx, freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow);
+    struct ggml_cgraph * gf = ggml_new_graph(ctx);
+    ggml_build_forward_expand(gf, r);
+    ggml_graph_compute_with_ctx(ctx, gf, 1);
+    memcpy(out, r->data, n * 4);
+    ggml_free(ctx);
+    return 0;
+}
+
 /* ggml_soft_max over rows of x [n, rows] */
 REF_API int ref_soft_max(const float * x, int n, int rows, float * out) {
     struct ggml_context * ctx = new_ctx((size_t)n * rows * 16 + (1u << 20));

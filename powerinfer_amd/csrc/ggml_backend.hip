@@ -221,17 +221,26 @@ __global__ __launch_bounds__(256) void softmax_rows_kernel(const float * x, floa
     for (int i = threadIdx.x; i < n; i += 256) yr[i] = __fmul_rn(yr[i], inv);
 }
 // x [hd, n_head, T] with element strides s1 (head) and s2 (token), pos[T]; mode 0 adjacent pairs, 2 NeoX halves (ggml.c:11163-11325 for
-// fp32, :11327-11460 for fp16, no YaRN).  fp16 is what the K-shift graph runs in place over a layer's K cache (llama.cpp:4332-4381):
-// the same arithmetic with a conversion on either side.  A pair belongs to one thread, so y may be x.
+// fp32, :11327-11460 for fp16).  fp16 is what the K-shift graph runs in place over a layer's K cache (llama.cpp:4332-4381): the same
+// arithmetic with a conversion on either side.  A pair belongs to one thread, so y may be x.  Scaling as rope_yarn does it
+// (ggml.c:11124-11146): the angle is freq_scale * theta; with ext != 0 it is mixed with the unscaled angle by a ramp over the pair
+// index between corr0 and corr1, and cos / sin carry the magnitude factor mscale.  NeoX mode hands the ramp the rotation fraction
+// through an integer parameter in the reference, which is 0 for every pair of a fully rotated head.
+struct RopeScale { float freq_scale, ext, mscale, corr0, corr1; };
 template <typename E>
-__global__ void rope_kernel(const E * x, const int32_t * pos, E * y, size_t s1, size_t s2, size_t d1, size_t d2, int n_dims, int mode, float theta_scale, float freq_scale) {
+__global__ void rope_kernel(const E * x, const int32_t * pos, E * y, size_t s1, size_t s2, size_t d1, size_t d2, int n_dims, int mode, float theta_scale, RopeScale rs) {
     const int t = blockIdx.y, h = blockIdx.x, i = threadIdx.x;         // i = pair index < n_dims/2
     const E * s = x + (size_t)t * s2 + (size_t)h * s1; E * o = y + (size_t)t * d2 + (size_t)h * d1;
     float theta = (float)pos[t];
-    if (mode & 2) theta = __fmul_rn(theta, freq_scale);
+    if (mode & 2) theta = __fmul_rn(theta, rs.freq_scale);
     for (int j = 0; j < i; ++j) theta = __fmul_rn(theta, theta_scale);
-    const float th = __fmul_rn(freq_scale, theta);
-    const float c = cosf(th), sn = sinf(th);
+    float th = __fmul_rn(rs.freq_scale, theta);
+    if (rs.ext != 0.0f) {
+        const float ramp_y = __fdiv_rn(__fsub_rn((float)((mode & 2) ? 0 : i), rs.corr0), fmaxf(0.001f, __fsub_rn(rs.corr1, rs.corr0)));
+        const float mix = __fmul_rn(__fsub_rn(1.0f, fminf(1.0f, fmaxf(0.0f, ramp_y))), rs.ext);
+        th = __fadd_rn(__fmul_rn(th, __fsub_rn(1.0f, mix)), __fmul_rn(theta, mix));
+    }
+    const float c = __fmul_rn(cosf(th), rs.mscale), sn = __fmul_rn(sinf(th), rs.mscale);
     const int i0 = (mode & 2) ? i : 2 * i, i1 = (mode & 2) ? i + n_dims / 2 : 2 * i + 1;
     const float x0 = (float)s[i0], x1 = (float)s[i1];
     o[i0] = (E)__fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, sn));
@@ -424,10 +433,19 @@ bool op_rope(ggml_tensor * dst) {
     const size_t es = tsize(a->type);
     // rows of one head contiguous; heads and tokens at any stride that is a whole number of elements (views into the KV cache)
     if (a->nb[0] != es || dst->nb[0] != es || a->nb[1] % es || a->nb[2] % es || dst->nb[1] % es || dst->nb[2] % es) return false;
-    const int n_dims = dst->op_params[1], mode = dst->op_params[2];
-    float freq_base, freq_scale, ext_factor;
+    const int n_dims = dst->op_params[1], mode = dst->op_params[2], n_orig_ctx = dst->op_params[4];
+    float freq_base, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow;
     memcpy(&freq_base, dst->op_params + 5, 4); memcpy(&freq_scale, dst->op_params + 6, 4); memcpy(&ext_factor, dst->op_params + 7, 4);
-    if ((mode != 0 && mode != 2) || ext_factor != 0.0f || n_dims != a->ne[0] || n_dims / 2 > 1024) return false;       // no GLM / YaRN / partial rotation here
+    memcpy(&attn_factor, dst->op_params + 8, 4); memcpy(&beta_fast, dst->op_params + 9, 4); memcpy(&beta_slow, dst->op_params + 10, 4);
+    if ((mode != 0 && mode != 2) || n_dims != a->ne[0] || n_dims / 2 > 1024) return false;       // no GLM / xPos / partial rotation here
+    // YaRN's correction dimensions and magnitude factor, as the host computes them (ggml_rope_yarn_corr_dims, ggml.c:11148-11161)
+    RopeScale rs{freq_scale, ext_factor, attn_factor, 0.0f, 0.0f};
+    if (ext_factor != 0.0f) {
+        auto corr_dim = [&](float n_rot) { return n_dims * logf(n_orig_ctx / (n_rot * 2 * (float)M_PI)) / (2 * logf(freq_base)); };
+        rs.corr0 = fmaxf(0.0f, floorf(corr_dim(beta_fast)));
+        rs.corr1 = fminf((float)(n_dims - 1), ceilf(corr_dim(beta_slow)));
+        rs.mscale = attn_factor * (1.0f + 0.1f * logf(1.0f / freq_scale));
+    }
     if (a->backend == GGML_BACKEND_CPU && !contiguous(a)) return false;                                                // staged operands are copied as one block
     if (dst->backend == GGML_BACKEND_CPU && !contiguous(dst)) return false;
     Temps tmp;
@@ -436,10 +454,10 @@ bool op_rope(ggml_tensor * dst) {
     const dim3 grid((unsigned)a->ne[1], (unsigned)a->ne[2]), block(n_dims / 2);
     if (a->type == GGML_TYPE_F32)
         hipLaunchKernelGGL(rope_kernel<float>, grid, block, 0, 0, (const float *)ad, pd, (float *)y, a->nb[1] / es, a->nb[2] / es, dst->nb[1] / es, dst->nb[2] / es,
-                           n_dims, mode, theta_scale, freq_scale);
+                           n_dims, mode, theta_scale, rs);
     else
         hipLaunchKernelGGL(rope_kernel<__half>, grid, block, 0, 0, (const __half *)ad, pd, (__half *)y, a->nb[1] / es, a->nb[2] / es, dst->nb[1] / es, dst->nb[2] / es,
-                           n_dims, mode, theta_scale, freq_scale);
+                           n_dims, mode, theta_scale, rs);
     finish_out(dst, y);
     return true;
 }

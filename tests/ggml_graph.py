@@ -140,8 +140,10 @@ class Graph:
     def soft_max(self, a, name="soft_max"):                                     # ggml.c:5171
         return self._node("SOFT_MAX", F32, list(a.ne), [a], name)
 
-    def rope(self, a, pos, n_dims, mode, freq_base=10000.0, freq_scale=1.0, name="rope"):      # ggml_rope_impl, ggml.c:5222-5262
-        params = [0, n_dims, mode, 0, 0, self._f32(freq_base), self._f32(freq_scale), self._f32(0.0), self._f32(1.0), self._f32(32.0), self._f32(1.0)]
+    def rope(self, a, pos, n_dims, mode, freq_base=10000.0, freq_scale=1.0, name="rope", n_orig_ctx=0, ext_factor=0.0, attn_factor=1.0,
+             beta_fast=32.0, beta_slow=1.0):                                                     # ggml_rope_impl, ggml.c:5222-5262
+        params = [0, n_dims, mode, 0, n_orig_ctx, self._f32(freq_base), self._f32(freq_scale), self._f32(ext_factor), self._f32(attn_factor),
+                  self._f32(beta_fast), self._f32(beta_slow)]
         return self._node("ROPE", F32, list(a.ne), [a, pos], name, params=params)
 
     def rope_inplace(self, a, pos, n_dims, mode, freq_base=10000.0, freq_scale=1.0, name="rope_inplace"):

@@ -130,12 +130,40 @@ def layer7b_case(R):
     print("layer7b active:", active.size, "of 11008")
 
 
+ROPE_SCALED_CASES = (     # (tag, mode, n_orig_ctx, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow)
+    ("lin0", 0, 0, 0.25, 0.0, 1.0, 32.0, 1.0),            # linear scaling, LLaMA pairs
+    ("lin2", 2, 0, 0.5, 0.0, 1.0, 32.0, 1.0),             # linear scaling, NeoX halves (the reference applies the factor twice there)
+    ("yarn0", 0, 256, 0.25, 1.0, 1.0, 32.0, 1.0),         # YaRN: ramp between the correction dimensions, magnitude correction
+    ("yarn0b", 0, 128, 0.125, 0.7, 1.3, 16.0, 2.0),
+    ("yarn2", 2, 256, 0.25, 1.0, 1.0, 32.0, 1.0),
+)
+
+
+def rope_scaled_case(R):
+    """ggml_rope_custom with its scaling operands (ggml.c:11124-11161): a file of its own, so that ops.npz keeps its random stream."""
+    P = ol._ptr
+    rng = np.random.default_rng(77)
+    hd, nh, T = 64, 3, 5
+    x = rng.standard_normal((T, nh, hd)).astype(np.float32)
+    pos = np.array([0, 1, 17, 300, 2047], np.int32)
+    out = dict(x=x, pos=pos)
+    for tag, mode, n_orig, fs, ext, attn, bf, bs in ROPE_SCALED_CASES:
+        y = np.zeros_like(x)
+        assert R.ref_rope_ext(P(x), hd, nh, T, P(pos), hd, mode, n_orig, 10000.0, fs, ext, attn, bf, bs, P(y)) == 0
+        out[tag] = y
+    save("rope_scaled", **out)
+
+
 if __name__ == "__main__":
     R = ol.ref()
     assert R is not None, "needs /root/reference"
+    if len(sys.argv) > 1 and sys.argv[1] == "rope_scaled":
+        rope_scaled_case(R)
+        sys.exit(0)
     ffn_case(R, "ffn_f16_gate", 11, 64, 1024, 32, 3, ol.F16, 1, 0.6)
     ffn_case(R, "ffn_f16_nogate", 12, 64, 1024, 32, 2, ol.F16, 0, 0.6)
     ffn_case(R, "ffn_q4_gate", 13, 64, 1024, 32, 3, ol.Q4_0, 1, 0.6)
     ffn_case(R, "ffn_q4_nogate", 14, 128, 1056, 32, 1, ol.Q4_0, 0, 0.6)
     ops_case(R)
+    rope_scaled_case(R)
     layer7b_case(R)

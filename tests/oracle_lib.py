@@ -55,6 +55,8 @@ def oracle():
         L.pio_rms_norm.argtypes = [_vp, _i64, _i, _f, _vp]
         L.pio_norm.argtypes = [_vp, _i64, _i, _f, _vp]
         L.pio_rope.argtypes = [_vp, _i, _i, _i, _vp, _i, _i, _f, _f, _vp]
+        L.pio_rope_ext.argtypes = [_vp, _i, _i, _i, _vp, _i, _i, _i, _f, _f, _f, _f, _f, _f, _vp]
+        L.pio_rope_ext.restype = None
         L.pio_soft_max.argtypes = [_vp, _i64, _i64, _vp]
         L.pio_active_list.argtypes = [_vp, _i64, _f, _vp]
         L.pio_ffn_sparse.argtypes = [_i] * 6 + [_vp] * 8 + [_f, _i] + [_vp] * 5
@@ -86,6 +88,8 @@ def ref():
         L.ref_mul_mat.argtypes = [_i, _vp, _i, _i, _vp, _i, _i, _vp]
         L.ref_norm.argtypes = [_i, _vp, _i, _i, _f, _vp]
         L.ref_rope.argtypes = [_vp, _i, _i, _i, _vp, _i, _i, _f, _f, _vp]
+        if hasattr(L, "ref_rope_ext"):
+            L.ref_rope_ext.argtypes = [_vp, _i, _i, _i, _vp, _i, _i, _i, _f, _f, _f, _f, _f, _f, _vp]
         L.ref_soft_max.argtypes = [_vp, _i, _i, _vp]
         L.ref_attention.argtypes = [_i] * 6 + [_vp] * 6
         for n in ("ref_quantize_row", "ref_quantize_row_fast", "ref_dequantize_row"):

@@ -54,6 +54,22 @@ def test_rope_modes(golden, mode):
     assert np.abs(G.host(y) - g[f"rope{mode}_y"]).max() < 2e-5   # position 300: cosf/sinf of the device vs the host's, angles identical
 
 
+@pytest.mark.parametrize("tag,mode,n_orig,fs,ext,attn,bf,bs", [("lin0", 0, 0, 0.25, 0.0, 1.0, 32.0, 1.0), ("lin2", 2, 0, 0.5, 0.0, 1.0, 32.0, 1.0),
+                                                               ("yarn0", 0, 256, 0.25, 1.0, 1.0, 32.0, 1.0), ("yarn0b", 0, 128, 0.125, 0.7, 1.3, 16.0, 2.0),
+                                                               ("yarn2", 2, 256, 0.25, 1.0, 1.0, 32.0, 1.0)])
+def test_rope_with_linear_and_yarn_scaling(golden, tag, mode, n_orig, fs, ext, attn, bf, bs):
+    """ROPE nodes as a model with a scaled context builds them (ggml_rope_custom, llama.cpp:4900-4960): linear scaling and YaRN
+    (rope_yarn, ggml.c:11124-11161), against what the compiled reference wrote (tests/golden/rope_scaled.npz)."""
+    g = golden("rope_scaled")
+    G = graph()
+    x = G.new(F32, [64, 3, 5], g["x"], "x")                      # [hd, n_head, T]
+    pos = G.new(I32, [5], g["pos"], "pos")
+    y = G.on_gpu(G.rope(x, pos, 64, mode, freq_scale=fs, n_orig_ctx=n_orig, ext_factor=ext, attn_factor=attn, beta_fast=bf, beta_slow=bs))
+    G.compute()
+    assert not G.cpu_run
+    assert np.abs(G.host(y) - g[tag]).max() < 3e-5               # positions up to 2047: cosf / sinf of the device against the host's
+
+
 @pytest.mark.parametrize("mode", [0, 2])
 def test_k_shift_rope_in_place_over_a_cache_view(mode):
     """The K-shift graph (llama.cpp:4332-4381): ggml_rope_custom_inplace over a 3-D view [hd, n_head_kv, n_ctx] of one layer's fp16 K

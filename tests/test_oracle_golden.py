@@ -72,6 +72,34 @@ def test_rope(golden):
         np.testing.assert_allclose(y, g[f"rope{mode}_y"], rtol=0, atol=1e-6)
 
 
+ROPE_SCALED_CASES = (     # as tests/golden/make_fixtures.py wrote them: (tag, mode, n_orig_ctx, freq_scale, ext_factor, attn_factor, beta_fast, beta_slow)
+    ("lin0", 0, 0, 0.25, 0.0, 1.0, 32.0, 1.0), ("lin2", 2, 0, 0.5, 0.0, 1.0, 32.0, 1.0), ("yarn0", 0, 256, 0.25, 1.0, 1.0, 32.0, 1.0),
+    ("yarn0b", 0, 128, 0.125, 0.7, 1.3, 16.0, 2.0), ("yarn2", 2, 256, 0.25, 1.0, 1.0, 32.0, 1.0))
+
+
+def test_rope_with_linear_and_yarn_scaling(golden):
+    """ggml_rope_custom's scaling operands against the compiled reference's outputs: linear scaling in both pairings (NeoX applies the
+    factor twice, as the reference does), YaRN with its ramp and magnitude correction; and the unscaled call reduces to pio_rope."""
+    g = golden("rope_scaled")
+    O = ol.oracle()
+    x, pos = g["x"], g["pos"]
+    T, nh, hd = x.shape
+    for tag, mode, n_orig, fs, ext, attn, bf, bs in ROPE_SCALED_CASES:
+        y = np.zeros_like(x)
+        O.pio_rope_ext(P(x), hd, nh, T, P(pos), hd, mode, n_orig, 10000.0, fs, ext, attn, bf, bs, P(y))
+        np.testing.assert_allclose(y, g[tag], rtol=0, atol=2e-6, err_msg=tag)
+        assert np.abs(y - x).max() > 0.1                              # the case rotates something
+    for mode in (0, 2):
+        a, b = np.zeros_like(x), np.zeros_like(x)
+        O.pio_rope(P(x), hd, nh, T, P(pos), hd, mode, 10000.0, 1.0, P(a))
+        O.pio_rope_ext(P(x), hd, nh, T, P(pos), hd, mode, 0, 10000.0, 1.0, 0.0, 1.0, 32.0, 1.0, P(b))
+        assert np.array_equal(a, b)
+    # the cases differ from one another and from the unscaled rotation: a dropped operand would not go unnoticed
+    a = np.zeros_like(x)
+    O.pio_rope(P(x), hd, nh, T, P(pos), hd, 0, 10000.0, 1.0, P(a))
+    assert np.abs(g["lin0"] - a).max() > 0.1 and np.abs(g["yarn0"] - g["lin0"]).max() > 0.05 and np.abs(g["yarn0b"] - g["yarn0"]).max() > 0.05
+
+
 def test_soft_max(golden):
     g = golden("ops")
     O = ol.oracle()

@@ -202,8 +202,9 @@ PI_API int pi_k_axpy_q4_partials_split(const void * down_t_q4, const void * down
 /* KV cache maintenance.  pi_k_k_shift replaces the graph of llm_build_k_shift (llama.cpp:4332-4381; the fp16 RoPE
  * ggml.c:11327-11478): cache [rows = layers x kv heads][n_ctx][hd] fp16, delta[n_cells] positions to rotate each cell by.
  * pi_k_kv_compact moves cell map[j] to cell j (map ascending) through `stage` ([rows][n_new][hd] fp16): this implementation keeps
- * the live cells contiguous instead of searching a ring for free slots (llama_kv_cache_find_slot, llama.cpp:1683-1736). */
-PI_API int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float theta_scale, const int32_t * delta, int n_cells, pi_stream_t stream);
+ * the live cells contiguous instead of searching a ring for free slots (llama_kv_cache_find_slot, llama.cpp:1683-1736).
+ * freq_scale: linear RoPE scaling as in pi_k_rope_kv_store. */
+PI_API int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float theta_scale, float freq_scale, const int32_t * delta, int n_cells, pi_stream_t stream);
 PI_API int pi_k_kv_compact(void * cache, void * stage, int rows, int n_ctx, int hd, const int32_t * map, int n_new, pi_stream_t stream);
 PI_API int pi_k_sparse_ffn_supported(int ff, int r, int cols);
 /* the two launches of pi_k_sparse_ffn on their own, for callers that overlap the block with an independent branch (Falcon's
@@ -380,7 +381,7 @@ PI_API int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void *
  * Head sizes 128 and 64 with 16 * n_ctx floats of scores within 156 KB of LDS (n_ctx up to about 1900) take 16 tokens per
  * workgroup on the matrix cores; other shapes one token per workgroup.  Same rounding points either way (llm_build_kqv on the
  * CPU path: fp16 q and K, fp16 in and out of exp, fp16 probabilities). */
-PI_API int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
+PI_API int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,
                            const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache,
                            float * out, int out_stride, void * out_f16, pi_stream_t stream);
 PI_API int pi_k_embed_batch(const void * table_f16, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream);
@@ -393,8 +394,11 @@ PI_API int pi_k_step_advance(int32_t * step, pi_stream_t stream);
  * cpy_f32_f16 :4944 for llm_build_kv_store, llama.cpp:4383).  qkv: fp32 [n_head*hd + 2*n_head_kv*hd]
  * (q | k | v).  mode 0 = adjacent pairs, 2 = NeoX halves.  The position is read from *pos (device).
  * Cache layout (this library's own): K and V are fp16 [n_head_kv][n_ctx][hd].
+ * theta_scale = freq_base^(-2/hd); freq_scale = linear RoPE scaling (llama_context_params.rope_freq_scale, 1 = none): the angle
+ * of a pair is freq_scale * theta as rope_yarn forms it with ext_factor 0 (ggml.c:11124-11146), and mode 2 multiplies the
+ * starting angle by freq_scale once more as the CPU path does (ggml.c:11292).
  */
-PI_API int pi_k_rope_kv_store(const float * qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
+PI_API int pi_k_rope_kv_store(const float * qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,
                               const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache, pi_stream_t stream);
 
 /*
@@ -407,10 +411,11 @@ PI_API int pi_k_attn_decode(const float * q_rot, const void * k_cache, const voi
                             int hd, int n_ctx, const int32_t * pos, float * out, pi_stream_t stream);
 
 /* cos/sin table for pi_k_attn_fused: float2 [n_ctx][hd/2], angles formed as the CPU path forms them
- * (theta advanced by repeated fp32 multiplication with theta_scale = base^(-2/hd), ggml.c:11196-11319).  A set-up call: the
+ * (theta advanced by repeated fp32 multiplication with theta_scale = base^(-2/hd), ggml.c:11196-11319; mode and freq_scale as in
+ * pi_k_rope_kv_store).  A set-up call: the
  * values are computed on the host with the C library's cosf / sinf (what the CPU path calls) and copied with a blocking copy
  * after the stream has drained. */
-PI_API int pi_k_rope_table(void * table, int n_ctx, int hd, float theta_scale, pi_stream_t stream);
+PI_API int pi_k_rope_table(void * table, int n_ctx, int hd, int mode, float theta_scale, float freq_scale, pi_stream_t stream);
 
 /* pi_k_rope_kv_store + pi_k_attn_decode in one launch (one workgroup per query head; the new cell is used
  * from LDS and stored by the first query head of each KV group).  Same arithmetic, same cache layout. */
@@ -438,6 +443,7 @@ typedef struct pi_hparams {
     int32_t arch;
     int32_t n_embd, n_ff, n_head, n_head_kv, n_layer, n_vocab, n_ctx;
     float   norm_eps, rope_freq_base, sparse_threshold;
+    float   rope_freq_scale;            /* linear RoPE scaling (llama_cparams.rope_freq_scale, llama.cpp:9857); 0 is read as 1 */
 } pi_hparams;
 
 /* tensor roles; names as llama.cpp:403-461 (blk.N.<role>.weight).  layer = -1 for the global ones. */

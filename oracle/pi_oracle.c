@@ -702,6 +702,7 @@ int pio_model_eval(pio_model * m, const int32_t * tokens, const int32_t * pos, c
     const pio_hparams * hp = &m->hp;
     const int d = hp->n_embd, ff = hp->n_ff, hd = d / hp->n_head, gqa = hd * hp->n_head_kv;
     const int falcon = hp->arch == PIO_ARCH_FALCON;
+    const float fscale = hp->rope_freq_scale == 0.0f ? 1.0f : hp->rope_freq_scale;      /* cparams.rope_freq_scale, llama.cpp:9857 */
     int rc = 0;
     const size_t nd = (size_t)d * T;
     float * inpL = (float *)malloc(sizeof(float) * nd);
@@ -736,8 +737,8 @@ int pio_model_eval(pio_model * m, const int32_t * tokens, const int32_t * pos, c
             rc |= mm(&L[PIO_T_WQ], nrm, T, q, n_threads);
             rc |= mm(&L[PIO_T_WK], nrm, T, k, n_threads);
             rc |= mm(&L[PIO_T_WV], nrm, T, v, n_threads);
-            pio_rope(q, hd, hp->n_head,    T, pos, hd, 0, hp->rope_freq_base, 1.0f, qr);
-            pio_rope(k, hd, hp->n_head_kv, T, pos, hd, 0, hp->rope_freq_base, 1.0f, kr);
+            pio_rope(q, hd, hp->n_head,    T, pos, hd, 0, hp->rope_freq_base, fscale, qr);
+            pio_rope(k, hd, hp->n_head_kv, T, pos, hd, 0, hp->rope_freq_base, fscale, kr);
             rc |= pio_attention(hd, hp->n_head, hp->n_head_kv, hp->n_ctx, n_kv, T, kv_slot, kq_mask, qr, kr, v, kc, vc, att);
             rc |= mm(&L[PIO_T_WO], att, T, cur, n_threads);
             for (size_t i = 0; i < nd; ++i) ffi[i] = cur[i] + inpL[i];                       /* ffn_inp */
@@ -761,8 +762,8 @@ int pio_model_eval(pio_model * m, const int32_t * tokens, const int32_t * pos, c
                 memcpy(k + (size_t)t * gqa, qkv + (size_t)t * w + d,       sizeof(float) * gqa);
                 memcpy(v + (size_t)t * gqa, qkv + (size_t)t * w + d + gqa, sizeof(float) * gqa);
             }
-            pio_rope(q, hd, hp->n_head,    T, pos, hd, 2, hp->rope_freq_base, 1.0f, qr);
-            pio_rope(k, hd, hp->n_head_kv, T, pos, hd, 2, hp->rope_freq_base, 1.0f, kr);
+            pio_rope(q, hd, hp->n_head,    T, pos, hd, 2, hp->rope_freq_base, fscale, qr);
+            pio_rope(k, hd, hp->n_head_kv, T, pos, hd, 2, hp->rope_freq_base, fscale, kr);
             rc |= pio_attention(hd, hp->n_head, hp->n_head_kv, hp->n_ctx, n_kv, T, kv_slot, kq_mask, qr, kr, v, kc, vc, att);
             rc |= mm(&L[PIO_T_WO], att, T, cur, n_threads);                                   /* ffn_inp = attention output */
             rc |= pio_ffn_sparse(d, ff, r, T, L[PIO_T_FFN_UP].type, 0,
@@ -795,15 +796,17 @@ int pio_model_k_shift(pio_model * m, const int32_t * delta) {
     const int hd = hp->n_embd / hp->n_head, gqa = hd * hp->n_head_kv;
     const int is_neox = hp->arch == 1;
     const float theta_scale = powf(hp->rope_freq_base, -2.0f / hd);
+    const float fscale = hp->rope_freq_scale == 0.0f ? 1.0f : hp->rope_freq_scale;
     for (int il = 0; il < hp->n_layer; ++il) {
         uint16_t * kc = m->k_cache + (size_t)il * hp->n_ctx * gqa;
         for (int c = 0; c < hp->n_ctx; ++c)
             for (int h = 0; h < hp->n_head_kv; ++h) {
                 uint16_t * row = kc + (size_t)c * gqa + (size_t)h * hd;
                 float theta_base = (float)delta[c];
-                if (is_neox) theta_base *= 1.0f;                       /* freq_scale, ggml.c:11447 */
+                if (is_neox) theta_base *= fscale;                     /* ggml.c:11447 */
                 for (int i = 0; i < hd / 2; ++i) {
-                    const float c_ = cosf(theta_base), s_ = sinf(theta_base);
+                    const float th = fscale * theta_base;              /* rope_yarn with ext_factor 0, ggml.c:11124-11146 */
+                    const float c_ = cosf(th), s_ = sinf(th);
                     theta_base *= theta_scale;
                     const int i0 = is_neox ? i : 2 * i, i1 = is_neox ? i + hd / 2 : 2 * i + 1;
                     const float x0 = H2F(row[i0]), x1 = H2F(row[i1]);

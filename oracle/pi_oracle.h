@@ -87,6 +87,7 @@ typedef struct pio_hparams {
     int32_t arch;
     int32_t n_embd, n_ff, n_head, n_head_kv, n_layer, n_vocab, n_ctx;
     float   norm_eps, rope_freq_base, sparse_threshold;
+    float   rope_freq_scale;            /* linear RoPE scaling (llama_cparams.rope_freq_scale, llama.cpp:9857); 0 is read as 1 */
 } pio_hparams;
 
 /* tensor kinds; layer = -1 for the three global tensors */

@@ -164,7 +164,7 @@ int layer_forward(pi_model * m, int il, bool last_token) {
         PI_TRY(pi_k_attn_fused(m->qkv, m->rope_table, m->k_cache + kv_off, m->v_cache + kv_off, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0,
                                hp.n_ctx, m->d_pos, m->att, st));
     } else {
-        PI_TRY(pi_k_rope_kv_store(m->qkv, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, m->d_pos, hp.n_ctx,
+        PI_TRY(pi_k_rope_kv_store(m->qkv, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, m->freq_scale, m->d_pos, hp.n_ctx,
                                   m->q_rot, m->k_cache + kv_off, m->v_cache + kv_off, st));
         PI_TRY(pi_k_attn_decode(m->q_rot, m->k_cache + kv_off, m->v_cache + kv_off, hp.n_head, hp.n_head_kv, hd, hp.n_ctx, m->d_pos, m->att, st));
     }
@@ -380,7 +380,7 @@ int kv_edit(pi_model * m, __half * k_cache, __half * v_cache, int32_t * d_pos, s
     if (!m->kv_map) { m->kv_map = m->alloc<int32_t>(hp.n_ctx); if (!m->kv_map) return PI_E_HIP; }
     if (any_shift) {
         PI_TRY(pi_memcpy_h2d(m->kv_map, dl.data(), sizeof(int32_t) * n_old));
-        PI_TRY(pi_k_k_shift(k_cache, rows, hp.n_ctx, m->hd, hp.arch == PI_ARCH_FALCON ? 2 : 0, m->theta_scale, m->kv_map, n_old, st));
+        PI_TRY(pi_k_k_shift(k_cache, rows, hp.n_ctx, m->hd, hp.arch == PI_ARCH_FALCON ? 2 : 0, m->theta_scale, m->freq_scale, m->kv_map, n_old, st));
         PI_HIP_TRY(hipStreamSynchronize(st));
     }
     bool moved = false;
@@ -420,6 +420,7 @@ pi_model * pi_model_create(const pi_hparams * hp) {
     m->gqa = m->hd * hp->n_head_kv;
     m->layers.resize((size_t)hp->n_layer * PI_T_COUNT);
     m->theta_scale = powf(hp->rope_freq_base, -2.0f / (float)m->hd);       // ggml.c:11196
+    m->freq_scale = hp->rope_freq_scale == 0.0f ? 1.0f : hp->rope_freq_scale;
     return m;
 }
 
@@ -636,7 +637,7 @@ int pi_model_finalize(pi_model * m) {
     if (pi_k_attn_fused_supported(m->hd, hp.n_ctx)) {
         m->rope_table = m->alloc<float>((size_t)hp.n_ctx * m->hd);
         if (!m->rope_table) return PI_E_HIP;
-        PI_TRY(pi_k_rope_table(m->rope_table, hp.n_ctx, m->hd, m->theta_scale, nullptr));
+        PI_TRY(pi_k_rope_table(m->rope_table, hp.n_ctx, m->hd, hp.arch == PI_ARCH_FALCON ? 2 : 0, m->theta_scale, m->freq_scale, nullptr));
     }
     else if (!pi_k_attn_decode_supported(m->hd, hp.n_ctx))
         return pi::fail(PI_E_UNSUPPORTED, "pi_model_finalize: head size or context outside both attention kernels (scores of every cell are kept in LDS: n_ctx up to about 13 000 at head size 128)");

@@ -64,7 +64,7 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     PI_TRY(pi_k_norm_round_f16(x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));       // Falcon: the predictor reads the raw layer input
     PI_TRY(pi_k_gemm_f16(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr, st));
     if (b->prefill)
-        PI_TRY(pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, b->d_pos, hp.n_ctx, b->q_rot,
+        PI_TRY(pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, m->freq_scale, b->d_pos, hp.n_ctx, b->q_rot,
                                m->k_cache + kv_off, m->v_cache + kv_off, b->att, d, b->att16, st));
     else
         PI_TRY(pi_k_attn_fused_batch(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
@@ -223,7 +223,7 @@ int wide_layer(pi_model * m, BatchState * b, int il) {
     PI_TRY(chunk_input(wqkv.type, x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));
     PI_TRY(chunk_weight(m, b, il, PI_T_WQKV, d + 2 * gqa, d, &W));
     PI_TRY(chunk_gemm(m, W, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr));
-    PI_TRY(pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, b->d_pos, hp.n_ctx, b->q_rot,
+    PI_TRY(pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, m->freq_scale, b->d_pos, hp.n_ctx, b->q_rot,
                            m->k_cache + kv_off, m->v_cache + kv_off, b->att, d, b->att16, st));
     if (wo.type == PI_TYPE_Q4_0) PI_TRY(pi_k_norm_q8_round_f16(b->att, T, d, &plain, b->att16, nullptr, st));
     PI_TRY(chunk_weight(m, b, il, PI_T_WO, d, d, &W));

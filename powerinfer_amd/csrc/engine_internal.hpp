@@ -32,6 +32,7 @@ struct pi_model {
     std::vector<hipEvent_t> ev_fork, ev_join;
     pi_workspace * ws = nullptr;
     float theta_scale = 0.0f;
+    float freq_scale = 1.0f;          // linear RoPE scaling (1 = none)
 
     float *x = nullptr, *x2 = nullptr, *qkv = nullptr, *q_rot = nullptr, *att = nullptr, *attn_out = nullptr, *ffn_inp = nullptr;
     float *hidden = nullptr, *pred_logits = nullptr, *h_c = nullptr, *h_dense = nullptr, *logits = nullptr, *cold_out = nullptr;

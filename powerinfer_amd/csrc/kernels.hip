@@ -2160,6 +2160,16 @@ __global__ __launch_bounds__(kBlock) void h_q8_gather_kernel(const float * __res
     }
 }
 
+// Angle of pair i at position p as the CPU path forms it (ggml.c:11196-11319, rope_yarn with ext_factor 0, ggml.c:11124-11146):
+// theta advanced from p by repeated fp32 multiplication with theta_scale, then multiplied by freq_scale (linear scaling); the
+// NeoX layout (mode 2) multiplies the starting angle by freq_scale as well (ggml.c:11292), so it is scaled twice there.  With
+// freq_scale 1 every extra product is exact.
+__host__ __device__ inline float rope_angle(float p, int i, int mode, float theta_scale, float freq_scale) {
+    float theta = (mode & 2) ? p * freq_scale : p;
+    for (int j = 0; j < i; ++j) theta = theta * theta_scale;
+    return freq_scale * theta;
+}
+
 // ---------------------------------------------------------------------------------------------------
 // K-shift (llm_build_k_shift, llama.cpp:4332-4381): cached K rows whose position changed by delta[cell] are rotated in place
 // by that many positions, the RoPE of fp16 data (ggml_compute_forward_rope_f16, ggml.c:11327-11478): fp16 -> fp32, angle
@@ -2167,14 +2177,13 @@ __global__ __launch_bounds__(kBlock) void h_q8_gather_kernel(const float * __res
 // row = (layer, kv head).  grid = (cells, rows), hd/2 threads; cells with delta 0 are left alone (the reference rotates them
 // by angle 0, which returns the same bits).
 // ---------------------------------------------------------------------------------------------------
-__global__ void k_shift_kernel(__half * __restrict__ k_cache, int n_ctx, int hd, int mode, float theta_scale,
+__global__ void k_shift_kernel(__half * __restrict__ k_cache, int n_ctx, int hd, int mode, float theta_scale, float freq_scale,
                                const int32_t * __restrict__ delta) {
     const int cell = blockIdx.x, i = threadIdx.x;
     const int dl = delta[cell];
     if (dl == 0) return;
     __half * row = k_cache + ((size_t)blockIdx.y * n_ctx + cell) * hd;
-    float theta = (float)dl;
-    for (int j = 0; j < i; ++j) theta = __fmul_rn(theta, theta_scale);
+    const float theta = rope_angle((float)dl, i, mode, theta_scale, freq_scale);
     const float c = cosf(theta), sn = sinf(theta);
     const int i0 = (mode & 2) ? i : 2 * i;
     const int i1 = (mode & 2) ? i + hd / 2 : 2 * i + 1;
@@ -2202,7 +2211,7 @@ __global__ void kv_place_kernel(__half * __restrict__ cache, const __half * __re
 // the CPU path does, so the angle is bit-identical and only cosf/sinf may differ in the last place).
 // grid = n_head + 2*n_head_kv blocks of hd/2 threads.
 // ---------------------------------------------------------------------------------------------------
-__global__ void rope_kv_store_kernel(const float * __restrict__ qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
+__global__ void rope_kv_store_kernel(const float * __restrict__ qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,
                                      const int32_t * __restrict__ pos_p, int n_ctx, float * __restrict__ q_rot,
                                      __half * __restrict__ k_cache, __half * __restrict__ v_cache, int qkv_stride, int q_stride) {
     // blockIdx.y = token of a prompt chunk (same sequence, its own position); 0 for single-token decoding
@@ -2213,8 +2222,7 @@ __global__ void rope_kv_store_kernel(const float * __restrict__ qkv, int n_head,
     const int pos = *pos_p;
     if (h < n_head + n_head_kv) {
         const float * src = qkv + (size_t)h * hd;
-        float theta = (float)pos;
-        for (int j = 0; j < i; ++j) theta = __fmul_rn(theta, theta_scale);
+        const float theta = rope_angle((float)pos, i, mode, theta_scale, freq_scale);
         const float c = cosf(theta), s = sinf(theta);
         const int i0 = (mode & 2) ? i : 2 * i;
         const int i1 = (mode & 2) ? i + hd / 2 : 2 * i + 1;
@@ -4330,13 +4338,13 @@ int pi_k_batch_sparse_axpy(const void * down_t_f16, int cols, int ff, const floa
     return pi::check_launch("pi_k_batch_sparse_axpy");
 }
 
-int pi_k_rope_kv_store(const float * qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
+int pi_k_rope_kv_store(const float * qkv, int n_head, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,
                        const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache, pi_stream_t stream) {
     if (!qkv || !pos || !q_rot || !k_cache || !v_cache) return pi::fail(PI_E_ARG, "pi_k_rope_kv_store: null pointer");
     if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd <= 0 || hd % 2 || hd / 2 > 1024 || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_rope_kv_store: bad head geometry or mode");
     hipLaunchKernelGGL(rope_kv_store_kernel, dim3(n_head + 2 * n_head_kv), dim3(hd / 2), 0, (hipStream_t)stream,
-                       qkv, n_head, n_head_kv, hd, mode, theta_scale, pos, n_ctx, q_rot, (__half *)k_cache, (__half *)v_cache, 0, 0);
+                       qkv, n_head, n_head_kv, hd, mode, theta_scale, freq_scale, pos, n_ctx, q_rot, (__half *)k_cache, (__half *)v_cache, 0, 0);
     return pi::check_launch("pi_k_rope_kv_store");
 }
 
@@ -4351,7 +4359,7 @@ int pi_k_attn_decode(const float * q_rot, const void * k_cache, const void * v_c
     return pi::check_launch("pi_k_attn_decode");
 }
 
-int pi_k_rope_table(void * table, int n_ctx, int hd, float theta_scale, pi_stream_t stream) {
+int pi_k_rope_table(void * table, int n_ctx, int hd, int mode, float theta_scale, float freq_scale, pi_stream_t stream) {
     if (!table || n_ctx <= 0 || hd <= 0 || hd % 2 || hd / 2 > 1024) return pi::fail(PI_E_ARG, "pi_k_rope_table: bad arguments");
     // A set-up call: the table is computed on the host with the C library's cosf / sinf -- the functions the CPU path itself calls
     // (ggml.c:11163-11325: theta = position, then *= theta_scale per pair) -- so rotated q and k start from bit-identical factors;
@@ -4359,10 +4367,11 @@ int pi_k_rope_table(void * table, int n_ctx, int hd, float theta_scale, pi_strea
     const int half = hd / 2;
     std::vector<float> host((size_t)n_ctx * hd);
     for (int p = 0; p < n_ctx; ++p) {
-        float theta = (float)p;
+        float theta = (mode & 2) ? (float)p * freq_scale : (float)p;             // rope_angle, one product per pair
         for (int i = 0; i < half; ++i) {
-            host[((size_t)p * half + i) * 2]     = cosf(theta);
-            host[((size_t)p * half + i) * 2 + 1] = sinf(theta);
+            const float th = freq_scale * theta;
+            host[((size_t)p * half + i) * 2]     = cosf(th);
+            host[((size_t)p * half + i) * 2 + 1] = sinf(th);
             theta *= theta_scale;
         }
     }
@@ -4414,7 +4423,7 @@ int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_t
     return pi::check_launch("pi_k_attn_fused_batch");
 }
 
-int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale,
+int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,
                     const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache, float * out, int out_stride, void * out_f16,
                     pi_stream_t stream) {
     if (!qkv || !pos || !q_rot || !k_cache || !v_cache || !out || T <= 0 || T > kChunkMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad arguments");
@@ -4423,7 +4432,7 @@ int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_
     hipStream_t st = (hipStream_t)stream;
     // all K/V rows of the chunk are in the cache before any token of the chunk attends
     hipLaunchKernelGGL(rope_kv_store_kernel, dim3(n_head + 2 * n_head_kv, T), dim3(hd / 2), 0, st,
-                       qkv, n_head, n_head_kv, hd, mode, theta_scale, pos, n_ctx, q_rot, (__half *)k_cache, (__half *)v_cache, qkv_stride, n_head * hd);
+                       qkv, n_head, n_head_kv, hd, mode, theta_scale, freq_scale, pos, n_ctx, q_rot, (__half *)k_cache, (__half *)v_cache, qkv_stride, n_head * hd);
     // 16 tokens per workgroup on the matrix cores where the head size and the context fit (scores of 16 tokens in LDS)
     const int s_stride = ((n_ctx + 31) & ~31) + 4;
     const size_t sh_mfma = sizeof(float) * 16 * (size_t)s_stride + (size_t)kWavesPerBlock * hd * kAcVtStride * 2;
@@ -4449,11 +4458,11 @@ int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_
     return pi::check_launch("pi_k_attn_chunk");
 }
 
-int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float theta_scale, const int32_t * delta, int n_cells, pi_stream_t stream) {
+int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float theta_scale, float freq_scale, const int32_t * delta, int n_cells, pi_stream_t stream) {
     if (!k_cache || !delta || rows <= 0 || n_ctx <= 0 || hd <= 0 || hd % 2 || hd / 2 > 1024 || n_cells < 0 || n_cells > n_ctx || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_k_shift: bad arguments");
     if (n_cells == 0) return PI_OK;
-    hipLaunchKernelGGL(k_shift_kernel, dim3(n_cells, rows), dim3(hd / 2), 0, (hipStream_t)stream, (__half *)k_cache, n_ctx, hd, mode, theta_scale, delta);
+    hipLaunchKernelGGL(k_shift_kernel, dim3(n_cells, rows), dim3(hd / 2), 0, (hipStream_t)stream, (__half *)k_cache, n_ctx, hd, mode, theta_scale, freq_scale, delta);
     return pi::check_launch("pi_k_k_shift");
 }
 

@@ -187,6 +187,9 @@ def write_model(path, model, tokenizer_kv):
         (f"{arch}.attention.layer_norm_rms_epsilon" if arch == "llama" else f"{arch}.attention.layer_norm_epsilon"): (T_F32, hp.norm_eps),
         "powerinfer.sparse_threshold": (T_F32, hp.sparse_threshold),
     }
+    if hp.get("rope_freq_scale", 1.0) != 1.0:             # stored as its inverse, with the scaling type the loader defaults to (llama.cpp:2316-2328)
+        kv[f"{arch}.rope.scaling.type"] = (T_STR, "linear")
+        kv[f"{arch}.rope.scaling.factor"] = (T_F32, 1.0 / hp.rope_freq_scale)
     kv.update(tokenizer_kv)
     tensors = {}
     for k, a in model["glob"].items():
@@ -207,11 +210,18 @@ def read_model(path, n_ctx=512):
         raise ValueError(f"{path}: architecture {arch!r} is outside this path (llama and falcon only)")
     g = lambda k, d=None: kv[k][1] if k in kv else d  # noqa: E731
     n_head = g(f"{arch}.attention.head_count")
+    # linear RoPE scaling: the file holds 1 / freq_scale under the new key or the old one (llama.cpp:2316-2328); type "none"
+    # switches it off (llama.cpp:9869-9871) and YaRN is outside the fused token loop
+    scaling = g(f"{arch}.rope.scaling.type", b"linear").decode()
+    if scaling not in ("linear", "none"):
+        raise ValueError(f"{path}: rope scaling type {scaling!r} is outside this path (linear only)")
+    factor = g(f"{arch}.rope.scaling.factor", 0.0) or g(f"{arch}.rope.scale_linear", 0.0)
+    freq_scale = 1.0 if scaling == "none" or factor == 0.0 else float(np.float32(1.0) / np.float32(factor))
     hp = synth.HParams(arch=arch, name=g("general.name", b"?").decode(), n_embd=g(f"{arch}.embedding_length"),
                        n_ff=g(f"{arch}.feed_forward_length"), n_head=n_head, n_head_kv=g(f"{arch}.attention.head_count_kv", n_head),
                        n_layer=g(f"{arch}.block_count"), n_vocab=tensors["token_embd.weight"][1][1], n_ctx=n_ctx,
                        norm_eps=g(f"{arch}.attention.layer_norm_rms_epsilon", g(f"{arch}.attention.layer_norm_epsilon", 1e-5)),
-                       rope_freq_base=g(f"{arch}.rope.freq_base", 10000.0), sparse_threshold=g("powerinfer.sparse_threshold", 0.0),
+                       rope_freq_base=g(f"{arch}.rope.freq_base", 10000.0), rope_freq_scale=freq_scale, sparse_threshold=g("powerinfer.sparse_threshold", 0.0),
                        sparse=(magic == b"PWRI"))
     hp["n_rank"] = tensors["blk.0.fc1.weight"][1][1]
     hp["wtype"] = tensors["blk.0.ffn_up.weight"][0]

@@ -66,7 +66,7 @@ _SIGS = {
     "pi_k_pred_upgate_q4_split": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_axpy_q4_partials_split": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_axpy_q4_reduce": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
-    "pi_k_k_shift": (_i, [_vp, _i, _i, _i, _i, _f, _vp, _i, _vp]),
+    "pi_k_k_shift": (_i, [_vp, _i, _i, _i, _i, _f, _f, _vp, _i, _vp]),
     "pi_k_kv_compact": (_i, [_vp, _vp, _i, _i, _i, _vp, _i, _vp]),
     "pi_k_sparse_ffn_partials": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_partials_hot": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
@@ -102,13 +102,13 @@ _SIGS = {
     "pi_k_batch_sparse_mul_mat": (_i, [_vp, _i, _i, _vp, _i, _vp, _f, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_batch_sparse_axpy": (_i, [_vp, _i, _i, _vp, _vp, _i, _f, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_attn_fused_batch": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),
-    "pi_k_attn_chunk": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
+    "pi_k_attn_chunk": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _f, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     "pi_k_embed_batch": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
     "pi_k_argmax_batch": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _i, _vp]),
     "pi_k_step_advance": (_i, [_vp, _vp]),
-    "pi_k_rope_kv_store": (_i, [_vp, _i, _i, _i, _i, _f, _vp, _i, _vp, _vp, _vp, _vp]),
+    "pi_k_rope_kv_store": (_i, [_vp, _i, _i, _i, _i, _f, _f, _vp, _i, _vp, _vp, _vp, _vp]),
     "pi_k_attn_decode": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _vp, _vp, _vp]),
-    "pi_k_rope_table": (_i, [_vp, _i, _i, _f, _vp]),
+    "pi_k_rope_table": (_i, [_vp, _i, _i, _i, _f, _f, _vp]),
     "pi_k_attn_fused_supported": (_i, [_i, _i]),
     "pi_k_attn_decode_supported": (_i, [_i, _i]),
     "pi_k_attn_fused": (_i, [_vp, _vp, _vp, _vp, _i, _i, _i, _i, _i, _vp, _vp, _vp]),

@@ -21,7 +21,7 @@ KIND = {k: i for i, k in enumerate(KINDS)}
 class HParamsC(C.Structure):
     _fields_ = [("arch", C.c_int32), ("n_embd", C.c_int32), ("n_ff", C.c_int32), ("n_head", C.c_int32),
                 ("n_head_kv", C.c_int32), ("n_layer", C.c_int32), ("n_vocab", C.c_int32), ("n_ctx", C.c_int32),
-                ("norm_eps", C.c_float), ("rope_freq_base", C.c_float), ("sparse_threshold", C.c_float)]
+                ("norm_eps", C.c_float), ("rope_freq_base", C.c_float), ("sparse_threshold", C.c_float), ("rope_freq_scale", C.c_float)]
 
 
 def _declare(L):
@@ -82,7 +82,7 @@ class Model:
         _declare(self.L)
         self.hp = hp
         c = HParamsC(ARCH[hp.arch], hp.n_embd, hp.n_ff, hp.n_head, hp.n_head_kv, hp.n_layer, hp.n_vocab, hp.n_ctx,
-                     hp.norm_eps, hp.rope_freq_base, hp.sparse_threshold)
+                     hp.norm_eps, hp.rope_freq_base, hp.sparse_threshold, hp.get("rope_freq_scale", 1.0))
         self.h = self.L.pi_model_create(C.byref(c))
         if not self.h:
             raise pl.PiError("pi_model_create: " + self.L.pi_last_error().decode())

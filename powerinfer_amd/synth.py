@@ -126,7 +126,7 @@ def hparams(name, **over):
         "falcon-tiny": dict(arch="falcon", n_embd=512, n_ff=4096, n_rank=128, n_head=8, n_head_kv=2, n_layer=3,
                             n_vocab=1024, mean_rate=0.15),
     }[name]
-    hp = HParams(base, name=name, n_ctx=512, wtype=F16, norm_eps=1e-5, rope_freq_base=10000.0, sparse_threshold=0.0,
+    hp = HParams(base, name=name, n_ctx=512, wtype=F16, norm_eps=1e-5, rope_freq_base=10000.0, rope_freq_scale=1.0, sparse_threshold=0.0,
                  hot_frac=1.0, seed=0)
     hp.update(over)
     return hp

@@ -28,6 +28,10 @@ CASES = {
     # the same models with a context shift before step 12 (llama_kv_cache_seq_rm + llama_kv_cache_seq_shift: K-shift, ring slots)
     "llama_f16_shift": dict(base="llama-tiny", vocab="ggml-vocab-llama.gguf", shift=(12, 2, 4), n_gen=14, over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=4, n_head_kv=4, n_layer=2, n_vocab=32000, n_ctx=64, seed=21)),
     "falcon_f16_shift": dict(base="falcon-tiny", vocab="ggml-vocab-falcon.gguf", shift=(12, 2, 4), n_gen=14, over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=8, n_head_kv=2, n_layer=2, n_vocab=65024, n_ctx=64, seed=23)),
+    # linear RoPE scaling (the file's rope.scaling.factor = 2, so rope_freq_scale = 0.5) through prompt, decode and a context shift:
+    # rope_yarn with ext_factor 0 (ggml.c:11124-11146), NeoX mode's second product (ggml.c:11292, 11447), the scaled K-shift
+    "llama_f16_scaled_shift": dict(base="llama-tiny", vocab="ggml-vocab-llama.gguf", shift=(12, 2, 4), n_gen=14, over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=4, n_head_kv=4, n_layer=2, n_vocab=32000, n_ctx=64, seed=24, rope_freq_scale=0.5)),
+    "falcon_f16_scaled_shift": dict(base="falcon-tiny", vocab="ggml-vocab-falcon.gguf", shift=(12, 2, 4), n_gen=14, over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=8, n_head_kv=2, n_layer=2, n_vocab=65024, n_ctx=64, seed=25, rope_freq_scale=0.5)),
     "falcon_f16": dict(base="falcon-tiny", vocab="ggml-vocab-falcon.gguf", over=dict(n_embd=256, n_ff=1024, n_rank=64, n_head=8, n_head_kv=2, n_layer=2, n_vocab=65024, n_ctx=64, seed=23)),
 }
 
@@ -83,9 +87,12 @@ def make_seq_edit_fixture():
     print("seq edits: greedy of the last step", logits[-3:].argmax(1).tolist())
 
 
-def main():
-    make_seq_edit_fixture()
+def main(only=()):
+    if not only:
+        make_seq_edit_fixture()
     for name, c in CASES.items():
+        if only and name not in only:
+            continue
         hp, model = case_model(name)
         _, vkv, _ = gguf.read_gguf(os.path.join(REF, "models", c["vocab"]))
         tok_kv = {k: v for k, v in vkv.items() if k.startswith("tokenizer.")}
@@ -115,4 +122,4 @@ def main():
 
 
 if __name__ == "__main__":
-    main()
+    main(sys.argv[1:])                                   # case names to write; none = every fixture

@@ -273,7 +273,7 @@ class KVCells:
 class HParamsC(C.Structure):
     _fields_ = [("arch", C.c_int32), ("n_embd", C.c_int32), ("n_ff", C.c_int32), ("n_head", C.c_int32),
                 ("n_head_kv", C.c_int32), ("n_layer", C.c_int32), ("n_vocab", C.c_int32), ("n_ctx", C.c_int32),
-                ("norm_eps", C.c_float), ("rope_freq_base", C.c_float), ("sparse_threshold", C.c_float)]
+                ("norm_eps", C.c_float), ("rope_freq_base", C.c_float), ("sparse_threshold", C.c_float), ("rope_freq_scale", C.c_float)]
 
 
 _KINDS = ["tok_embd", "output_norm", "output_norm_b", "output", "attn_norm", "attn_norm_b", "attn_norm_2", "attn_norm_2_b",
@@ -287,7 +287,7 @@ class OracleModel:
         hp = model["hp"]
         self.hp = hp
         c = HParamsC({"llama": 0, "falcon": 1}[hp.arch], hp.n_embd, hp.n_ff, hp.n_head, hp.n_head_kv, hp.n_layer, hp.n_vocab,
-                     hp.n_ctx, hp.norm_eps, hp.rope_freq_base, hp.sparse_threshold)
+                     hp.n_ctx, hp.norm_eps, hp.rope_freq_base, hp.sparse_threshold, hp.get("rope_freq_scale", 1.0))
         self.h = self.O.pio_model_new(C.byref(c))
         self._keep = []
 

@@ -43,7 +43,7 @@ def test_engine_from_gguf_matches_reference_llama_cpp(name, tmp_path):
     assert same >= len(errs) - 1, (same, len(errs))
 
 
-@pytest.mark.parametrize("name", ["llama_f16_shift", "falcon_f16_shift"])
+@pytest.mark.parametrize("name", ["llama_f16_shift", "falcon_f16_shift", "llama_f16_scaled_shift", "falcon_f16_scaled_shift"])
 def test_context_shift_matches_reference_llama_cpp(name):
     """llama_kv_cache_seq_rm + llama_kv_cache_seq_shift before step 12 (what examples/main does when the context is full): the
     engine squeezes the removed cells out and rotates the shifted K rows; the reference's logits after the shift are the check."""

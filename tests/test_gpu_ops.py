@@ -98,12 +98,13 @@ def test_gemv_rejects_bad_shapes():
     assert b"pi_k_gemv" in L.pi_last_error()
 
 
-@pytest.mark.parametrize("mode,hd,nh,nkv,chunks", [(0, 128, 4, 4, (37, 45)), (2, 64, 8, 2, (70, 17, 2)), (0, 128, 2, 1, (130,)), (0, 64, 4, 4, (16, 33))])
-def test_attention_of_prompt_chunks(mode, hd, nh, nkv, chunks, monkeypatch):
+@pytest.mark.parametrize("mode,hd,nh,nkv,chunks,fs", [(0, 128, 4, 4, (37, 45), 1.0), (2, 64, 8, 2, (70, 17, 2), 1.0), (0, 128, 2, 1, (130,), 1.0),
+                                                     (0, 64, 4, 4, (16, 33), 1.0), (0, 128, 4, 4, (37, 45), 0.25), (2, 64, 8, 2, (70, 17, 2), 0.5)])
+def test_attention_of_prompt_chunks(mode, hd, nh, nkv, chunks, fs, monkeypatch):
     """Prompt chunks through pi_k_attn_chunk (RoPE + KV store of the whole chunk, then causal attention of every token over the cache)
     against the oracle's rope + attention: the route on the matrix cores (16 tokens per workgroup; chunk lengths on and off that
     tile, caches filled by earlier chunks, grouped query heads) and the one-token-per-workgroup route, which must agree with
-    each other more closely than either has to agree with the CPU."""
+    each other more closely than either has to agree with the CPU.  fs = linear RoPE scaling (freq_scale)."""
     from powerinfer_amd import lib as pl
     L = pl.init()
     O = ol.oracle()
@@ -122,8 +123,8 @@ def test_attention_of_prompt_chunks(mode, hd, nh, nkv, chunks, monkeypatch):
         q, k, v = (np.ascontiguousarray(a) for a in (qkv[:, :d], qkv[:, d:d + gqa], qkv[:, d + gqa:]))
         pos = np.arange(n_past, n_past + T, dtype=np.int32)
         qr, kr = np.zeros_like(q), np.zeros_like(k)
-        O.pio_rope(P(q), hd, nh, T, P(pos), hd, mode, 10000.0, 1.0, P(qr))
-        O.pio_rope(P(k), hd, nkv, T, P(pos), hd, mode, 10000.0, 1.0, P(kr))
+        O.pio_rope(P(q), hd, nh, T, P(pos), hd, mode, 10000.0, fs, P(qr))
+        O.pio_rope(P(k), hd, nkv, T, P(pos), hd, mode, 10000.0, fs, P(kr))
         n_kv = (n_past + T + 31) // 32 * 32
         mask = np.where(np.arange(n_kv)[None, :] > pos[:, None], -np.inf, 0).astype(np.float32)
         want = np.zeros((T, d), np.float32)
@@ -137,7 +138,7 @@ def test_attention_of_prompt_chunks(mode, hd, nh, nkv, chunks, monkeypatch):
                 monkeypatch.delenv("PI_ATTN_CHUNK", raising=False)
             dqr, dout, dout16 = pl.DevBuf(T * d * 4), pl.DevBuf(T * d * 4), pl.DevBuf(T * d * 2)
             pl.check(L.pi_memset(dout.ptr, 0xFF, dout.nbytes), "memset")
-            pl.check(L.pi_k_attn_chunk(dq.ptr, d + 2 * gqa, T, nh, nkv, hd, mode, theta_scale, dpos.ptr, n_ctx, dqr.ptr, kc.ptr, vc.ptr,
+            pl.check(L.pi_k_attn_chunk(dq.ptr, d + 2 * gqa, T, nh, nkv, hd, mode, theta_scale, fs, dpos.ptr, n_ctx, dqr.ptr, kc.ptr, vc.ptr,
                                        dout.ptr, d, dout16.ptr, None), "attn_chunk")
             pl.sync()
             got[route] = dout.download(np.float32).reshape(T, d)
@@ -150,10 +151,11 @@ def test_attention_of_prompt_chunks(mode, hd, nh, nkv, chunks, monkeypatch):
     monkeypatch.delenv("PI_ATTN_CHUNK", raising=False)
 
 
-@pytest.mark.parametrize("mode,hd,nh,nkv", [(0, 128, 4, 4), (2, 64, 8, 2)])
-def test_rope_attention_sequence(mode, hd, nh, nkv):
+@pytest.mark.parametrize("mode,hd,nh,nkv,fs", [(0, 128, 4, 4, 1.0), (2, 64, 8, 2, 1.0), (0, 128, 4, 4, 0.25), (2, 64, 8, 2, 0.5)])
+def test_rope_attention_sequence(mode, hd, nh, nkv, fs):
     """Six decode steps: RoPE + KV store + attention on the GPU against the oracle's rope + attention with
-    the reference cache layout (K cell-major, V transposed)."""
+    the reference cache layout (K cell-major, V transposed).  fs = linear RoPE scaling (the oracle's rope is pinned against the
+    compiled reference for fs != 1 too, NeoX mode's double product included)."""
     from powerinfer_amd import lib as pl
     L = pl.init()
     O = ol.oracle()
@@ -166,21 +168,21 @@ def test_rope_attention_sequence(mode, hd, nh, nkv):
     theta_scale = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
     kc_f, vc_f = pl.DevBuf.zeros(nkv * n_ctx * hd * 2), pl.DevBuf.zeros(nkv * n_ctx * hd * 2)
     tab, dout_f = pl.DevBuf(n_ctx * hd * 4), pl.DevBuf(d * 4)
-    pl.check(L.pi_k_rope_table(tab.ptr, n_ctx, hd, theta_scale, None), "rope_table")
+    pl.check(L.pi_k_rope_table(tab.ptr, n_ctx, hd, mode, theta_scale, fs, None), "rope_table")
     for pos in range(6):
         qkv = rng.standard_normal(d + 2 * gqa).astype(np.float32)
         q, k, v = qkv[:d], qkv[d:d + gqa], qkv[d + gqa:]
         p = np.array([pos], np.int32)
         qr, kr = np.zeros_like(q), np.zeros_like(k)
-        O.pio_rope(P(q), hd, nh, 1, P(p), hd, mode, 10000.0, 1.0, P(qr))
-        O.pio_rope(P(k), hd, nkv, 1, P(p), hd, mode, 10000.0, 1.0, P(kr))
+        O.pio_rope(P(q), hd, nh, 1, P(p), hd, mode, 10000.0, fs, P(qr))
+        O.pio_rope(P(k), hd, nkv, 1, P(p), hd, mode, 10000.0, fs, P(kr))
         n_kv = max(32, pos + 1)
         mask = np.where(np.arange(n_kv)[None, :] > pos, -np.inf, 0).astype(np.float32)
         want = np.zeros(d, np.float32)
         assert O.pio_attention(hd, nh, nkv, n_ctx, n_kv, 1, P(p), P(mask), P(qr), P(kr), P(np.ascontiguousarray(v)), P(kc_o), P(vc_o), P(want)) == 0
         dq.upload(qkv)
         dpos.upload(p)
-        pl.check(L.pi_k_rope_kv_store(dq.ptr, nh, nkv, hd, mode, theta_scale, dpos.ptr, n_ctx, dqr.ptr, kc_g.ptr, vc_g.ptr, None), "rope")
+        pl.check(L.pi_k_rope_kv_store(dq.ptr, nh, nkv, hd, mode, theta_scale, fs, dpos.ptr, n_ctx, dqr.ptr, kc_g.ptr, vc_g.ptr, None), "rope")
         pl.check(L.pi_k_attn_decode(dqr.ptr, kc_g.ptr, vc_g.ptr, nh, nkv, hd, n_ctx, dpos.ptr, dout.ptr, None), "attn")
         pl.check(L.pi_k_attn_fused(dq.ptr, tab.ptr, kc_f.ptr, vc_f.ptr, nh, nkv, hd, mode, n_ctx, dpos.ptr, dout_f.ptr, None), "attn_fused")
         pl.sync()
@@ -213,7 +215,7 @@ def test_attention_long_context(mode, hd, nh, nkv):
     n_ctx, gqa, d = 768, nkv * hd, nh * hd
     theta_scale = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
     tab = pl.DevBuf(n_ctx * hd * 4)
-    pl.check(L.pi_k_rope_table(tab.ptr, n_ctx, hd, theta_scale, None), "rope_table")
+    pl.check(L.pi_k_rope_table(tab.ptr, n_ctx, hd, mode, theta_scale, 1.0, None), "rope_table")
     kfill = (rng.standard_normal((n_ctx, nkv, hd)) * 0.5).astype(np.float16)        # cell-major, as the oracle keeps K
     vfill = (rng.standard_normal((n_ctx, nkv, hd)) * 0.5).astype(np.float16)
     boundary = 4 * (1024 // (hd // 8))
@@ -238,7 +240,7 @@ def test_attention_long_context(mode, hd, nh, nkv):
             if fused:
                 pl.check(L.pi_k_attn_fused(dq.ptr, tab.ptr, kc.ptr, vc.ptr, nh, nkv, hd, mode, n_ctx, dpos.ptr, dout.ptr, None), "attn_fused")
             else:
-                pl.check(L.pi_k_rope_kv_store(dq.ptr, nh, nkv, hd, mode, theta_scale, dpos.ptr, n_ctx, dqr.ptr, kc.ptr, vc.ptr, None), "rope")
+                pl.check(L.pi_k_rope_kv_store(dq.ptr, nh, nkv, hd, mode, theta_scale, 1.0, dpos.ptr, n_ctx, dqr.ptr, kc.ptr, vc.ptr, None), "rope")
                 pl.check(L.pi_k_attn_decode(dqr.ptr, kc.ptr, vc.ptr, nh, nkv, hd, n_ctx, dpos.ptr, dout.ptr, None), "attn")
             pl.sync()
             assert rel_err(dout.download(np.float32), want) < 2e-3, (pos, fused)
@@ -268,10 +270,12 @@ def test_embed_and_argmax():
     assert dtok.download(np.int32)[0] == 123 == int(np.argmax(lg))
 
 
-@pytest.mark.parametrize("mode", [0, 2])
-def test_k_shift_and_compaction(mode):
+@pytest.mark.parametrize("mode,fs", [(0, 1.0), (2, 1.0), (0, 0.5), (2, 0.5)])
+def test_k_shift_and_compaction(mode, fs):
     """pi_k_k_shift against the fp16 RoPE of the reference's K-shift restated in numpy (ggml.c:11327-11478: fp16 in, fp32
-    rotation with theta advanced by repeated multiplication, fp16 out), and pi_k_kv_compact against a gather."""
+    rotation with theta advanced by repeated multiplication, fp16 out), and pi_k_kv_compact against a gather.  With linear
+    scaling (fs) the model-level fixtures written by the compiled reference are the check proper (tests/test_gpu_model_golden.py);
+    here the kernel is held to the same restatement."""
     from powerinfer_amd import lib as pl
     L = pl.init()
     rows, n_ctx, hd, n_cells = 6, 40, 64, 33
@@ -285,15 +289,18 @@ def test_k_shift_and_compaction(mode):
         if delta[c] == 0:
             continue
         th = np.float32(delta[c])
+        if mode == 2:
+            th = np.float32(th * np.float32(fs))
         for i in range(hd // 2):
-            cs, sn = np.float32(np.cos(th)), np.float32(np.sin(th))
+            ang = np.float32(np.float32(fs) * th)
+            cs, sn = np.float32(np.cos(ang)), np.float32(np.sin(ang))
             i0, i1 = (i, i + hd // 2) if mode == 2 else (2 * i, 2 * i + 1)
             x0, x1 = k[:, c, i0].astype(np.float32), k[:, c, i1].astype(np.float32)
             want[:, c, i0] = (x0 * cs - x1 * sn).astype(np.float16)
             want[:, c, i1] = (x0 * sn + x1 * cs).astype(np.float16)
             th = np.float32(th * theta_scale)
     kd, dd = pl.DevBuf(host=k), pl.DevBuf(host=delta)
-    pl.check(L.pi_k_k_shift(kd.ptr, rows, n_ctx, hd, mode, float(theta_scale), dd.ptr, n_cells, None), "k_shift")
+    pl.check(L.pi_k_k_shift(kd.ptr, rows, n_ctx, hd, mode, float(theta_scale), fs, dd.ptr, n_cells, None), "k_shift")
     pl.sync()
     got = kd.download(np.float16).reshape(rows, n_ctx, hd)
     assert np.array_equal(got[:, n_cells:], k[:, n_cells:])                       # cells beyond the live range untouched

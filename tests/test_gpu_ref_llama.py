@@ -89,7 +89,7 @@ def test_reference_llama_cpp_runs_on_this_backend(name, share, n_threads, tmp_pa
 
 
 @pytest.mark.timeout(120)
-@pytest.mark.parametrize("name", ["llama_f16_shift", "falcon_f16_shift"])
+@pytest.mark.parametrize("name", ["llama_f16_shift", "falcon_f16_shift", "llama_f16_scaled_shift", "falcon_f16_scaled_shift"])
 def test_reference_context_shift_on_this_backend(name, tmp_path):
     """The reference's KV ring on this backend: before step 12 its driver removes cells [2, 6) of the sequence and shifts the cells
     behind them by -4 (llama_kv_cache_seq_rm + llama_kv_cache_seq_shift, llama.cpp:1683-1848), which makes llama_decode_internal

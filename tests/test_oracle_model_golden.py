@@ -35,7 +35,7 @@ def test_model_eval_matches_reference_llama_cpp(name):
     om.close()
 
 
-@pytest.mark.parametrize("name", ["llama_f16_shift", "falcon_f16_shift"])
+@pytest.mark.parametrize("name", ["llama_f16_shift", "falcon_f16_shift", "llama_f16_scaled_shift", "falcon_f16_scaled_shift"])
 def test_context_shift_matches_reference_llama_cpp(name):
     """KV ring slots, cell mask and K-shift: before step 12 the reference removed positions [2, 6) and shifted the later cells by
     -4 (llama_kv_cache_seq_rm + llama_kv_cache_seq_shift); the next llama_decode rotated the cached K rows (llm_build_k_shift)

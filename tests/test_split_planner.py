@@ -102,3 +102,29 @@ def test_plan_split_roundtrip_through_the_split_file(tmp_path):
     assert kv["general.architecture"][1] == b"generic.gpu_index" and kv["split.vram_capacity"][1] == int(budget_gb * 1024 ** 3)
     with pytest.raises(ValueError):
         split.plan_split(hp, rates, base / 2 / 1024 ** 3, 64)
+
+
+def test_rope_scaling_keys_of_a_model_file(tmp_path):
+    """Linear RoPE scaling travels in the model file as the inverse of rope_freq_scale, under `rope.scaling.factor` or the
+    older `rope.scale_linear`; scaling type "none" switches it off and other types are refused (llama.cpp:2316-2328, 9857-9871).
+    That the reference's loader reads what write_model writes is shown by the compiled reference itself: the fixtures
+    ref_*_scaled_shift.npz come from such files."""
+    hp = synth.hparams("llama-tiny", n_layer=1, n_ctx=32, seed=3, rope_freq_scale=0.25)
+    model = synth.make_model(hp)
+    path = str(tmp_path / "m.powerinfer.gguf")
+    gguf.write_model(path, model, {})
+    _, kv, _ = gguf.read_gguf(path)
+    assert kv["llama.rope.scaling.factor"][1] == 4.0 and kv["llama.rope.scaling.type"][1] == b"linear"
+    assert gguf.read_model(path, n_ctx=32)[0].rope_freq_scale == 0.25
+    hp1 = synth.hparams("llama-tiny", n_layer=1, n_ctx=32, seed=3)
+    gguf.write_model(path, synth.make_model(hp1), {})
+    _, kv, _ = gguf.read_gguf(path)
+    assert "llama.rope.scaling.factor" not in kv
+    assert gguf.read_model(path, n_ctx=32)[0].rope_freq_scale == 1.0
+    for extra, want in (({"llama.rope.scale_linear": (gguf.T_F32, 2.0)}, 0.5),
+                        ({"llama.rope.scaling.type": (gguf.T_STR, "none"), "llama.rope.scaling.factor": (gguf.T_F32, 2.0)}, 1.0)):
+        gguf.write_model(path, synth.make_model(hp1), extra)
+        assert gguf.read_model(path, n_ctx=32)[0].rope_freq_scale == want
+    gguf.write_model(path, synth.make_model(hp1), {"llama.rope.scaling.type": (gguf.T_STR, "yarn")})
+    with pytest.raises(ValueError):
+        gguf.read_model(path, n_ctx=32)

@@ -327,29 +327,34 @@ PI_API int pi_k_sparse_ffn_q4_reduce(int ff, int cols, int epilogue, const float
  * flags_pinned: 64 words of pinned host memory (words 0 and 8 written by the device, words 16 and 32 by the host, word 48 = the host's
  * stop word); seq: a device word counting the hand-overs; status_pinned: one device or pinned word, non-zero after a wait gave up.
  * pi_k_host_signal: flags[word] = *seq (after *seq += 1 when advance is set) once everything queued before it is complete.  pi_k_host_wait: holds the stream until
- * flags[slot] has reached *seq, for at most limit_seconds (then *status = 1 and every later wait returns at once). */
+ * flags[slot] has reached *seq, for at most limit_seconds (then *status = 1 and every later wait returns at once).
+ * pi_k_host_signal_wait: a signal without advance (signal_word 0 or 8; -1 = none) and a wait in one launch. */
 PI_API int pi_k_host_signal(uint32_t * seq, uint32_t * flags_pinned, int word, int advance, pi_stream_t stream);
 /* pi_k_pred_upgate_q4 cut in two for such a layer, so that the host threads start behind the predictor: pi_k_pred_q4_logits computes the
  * logits (to `logits`, which may be pinned host memory, and to logits_dev), the mask words and the Q8_0 blocks of the normalised input;
  * pi_k_upgate_q4_hot_rows reads logits_dev and writes h (or 0) for the neurons of the hot words only - the other entries of h_dense
- * belong to the host. */
+ * belong to the host.  With announce_seq / announce_flags (both or neither) the first lane of that launch does what
+ * pi_k_host_signal(announce_seq, announce_flags, 0, 1) would have done right before it: the predictor's results are complete and
+ * visible to the host at the boundary in front of the launch, so the hand-over needs no launch of its own. */
 PI_API int pi_k_pred_q4_logits(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
                                float * logits, float * logits_dev, void * xq8_out, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_upgate_q4_hot_rows(int ff, float threshold, const void * up_q4, const void * gate_q4, int cols, const float * x, const pi_norm * norm,
-                                   const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense, pi_workspace * ws,
-                                   pi_stream_t stream);
+                                   const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense,
+                                   uint32_t * announce_seq, uint32_t * announce_flags, pi_workspace * ws, pi_stream_t stream);
 /* The fused F16 launch of a hybrid layer (pi_k_sparse_ffn_partials_hot) cut in two in the same way (cols 4096): pi_k_sparse_ffn_logits_hot
  * computes the logits (to `logits`, which may be pinned host memory, and to logits_dev), the mask words and the fp16 normalised input for
  * the host; pi_k_sparse_ffn_rows_hot reads logits_dev and computes the resident active neurons' gate / up / down rows into the partial
- * vectors that pi_k_sparse_ffn_reduce_hot adds. */
+ * vectors that pi_k_sparse_ffn_reduce_hot adds; announce_seq / announce_flags as for pi_k_upgate_q4_hot_rows. */
 PI_API int pi_k_sparse_ffn_two_phase_supported(int ff, int r, int cols);
 PI_API int pi_k_sparse_ffn_logits_hot(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
                                       const uint32_t * hot_words, const int32_t * hot_prefix, float * logits, float * logits_dev, void * xn_f16_out,
                                       pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_sparse_ffn_rows_hot(int ff, float threshold, const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x,
                                     const pi_norm * norm, const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense,
-                                    pi_workspace * ws, pi_stream_t stream);
+                                    uint32_t * announce_seq, uint32_t * announce_flags, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_host_wait(const uint32_t * seq, const uint32_t * flags_pinned, int slot, uint32_t * status_pinned, double limit_seconds, pi_stream_t stream);
+PI_API int pi_k_host_signal_wait(const uint32_t * seq, uint32_t * flags_pinned, int signal_word, int slot, uint32_t * status_pinned, double limit_seconds,
+                                 pi_stream_t stream);
 
 /* The same mat-mul for prompt chunks of any length through hipBLASLt (fp16 operands, fp32 accumulation and result), where the reference
  * calls cuBLAS (ggml_cuda_op_mul_mat_cublas, ggml-cuda.cu:7662-7756).  Arguments and epilogues as pi_k_gemm_f16; no limit on T or cols.

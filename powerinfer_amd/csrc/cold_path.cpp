@@ -959,16 +959,15 @@ int cold_layer_q4_queue(ColdPath * c, int il, pi_model * m, hipStream_t st) {
     if (c->split_pred) {
         hfull = c->h_async[il];
         PI_TRY(pi_k_pred_q4_logits(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, d, ffn_src, &fn, c->logits, m->pred_logits, c->xq8_pin, m->ws, st));
-        PI_TRY(pi_k_host_signal(c->d_seq, c->flags, 0, 1, st));
+        // the hand-over starts in the first lane of the next launch, and the second signal travels with the wait behind it
         PI_TRY(pi_k_upgate_q4_hot_rows(ff, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, d, ffn_src, &fn, m->hot_words[il], m->hot_prefix[il],
-                                       m->pred_logits, hfull, m->ws, st));
-        PI_TRY(pi_k_host_signal(c->d_seq, c->flags, 8, 0, st));
+                                       m->pred_logits, hfull, c->d_seq, c->flags, m->ws, st));
     } else {
         PI_TRY(pi_k_pred_upgate_q4(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, d, ffn_src, &fn,
                                    m->hot_words[il], m->hot_prefix[il], c->logits, hfull, c->xq8_pin, m->ws, st));
         PI_TRY(pi_k_host_signal(c->d_seq, c->flags, 0, 1, st));
     }
-    PI_TRY(pi_k_host_wait(c->d_seq, c->flags, 16, c->d_status, limit, st));
+    PI_TRY(pi_k_host_signal_wait(c->d_seq, c->flags, c->split_pred ? 8 : -1, 16, c->d_status, limit, st));
     PI_TRY(pi_k_axpy_q4_partials(down.dev, d, ff, hfull, m->hot_words[il], m->hot_prefix[il], m->ws, st));
     PI_TRY(pi_k_host_wait(c->d_seq, c->flags, 32, c->d_status, limit, st));
     int32_t * n_act = m->n_active + il;
@@ -995,9 +994,8 @@ int cold_layer_f16_queue(ColdPath * c, int il, pi_model * m, hipStream_t st) {
     const float * ffn_src = falcon ? m->x : m->ffn_inp;
     PI_TRY(pi_k_sparse_ffn_logits_hot(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, d, ffn_src, &fn, m->hot_words[il], m->hot_prefix[il],
                                       c->logits, m->pred_logits, c->x16_pin, m->ws, st));
-    PI_TRY(pi_k_host_signal(c->d_seq, c->flags, 0, 1, st));
     PI_TRY(pi_k_sparse_ffn_rows_hot(ff, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, down.dev, d, ffn_src, &fn, m->hot_words[il], m->hot_prefix[il],
-                                    m->pred_logits, nullptr, m->ws, st));
+                                    m->pred_logits, nullptr, c->d_seq, c->flags, m->ws, st));             // its first lane starts the hand-over
     PI_TRY(pi_k_host_wait(c->d_seq, c->flags, 32, c->d_status, limit, st));
     int32_t * n_act = m->n_active + il;
     if (!falcon) return pi_k_sparse_ffn_reduce_hot(ff, d, PI_EPI_ADD2, out, m->ffn_inp, m->x2, n_act, m->ws, st);

@@ -992,6 +992,9 @@ __device__ __forceinline__ int select_nth_bit(uint32_t bits, int n);
 // fp16-rounded normalised input to the host share (xn_out; like logits it may be pinned host memory).
 // PHASE 1 / 2 (G == 1) cut the launch in two for a hybrid layer whose host share should start behind the predictor: 1 stops after the
 // logits (to `logits` and `logits2`), the mask words and the fp16 input for the host; 2 reads the logits back from `logits2`.
+// a hand-over to the host announced by the first lane of a launch (see host_signal_kernel): device counter and word 0 of the pinned flags
+struct HostAnnounce { uint32_t * seq; uint32_t * flags; };
+
 template <int CPW, int RCH, bool GATE, int G, bool HYB, int PHASE = 0>      // cols == 8 waves * CPW chunks * 512; r == RCH * 512; G groups of 32 neurons
 __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
                                                                    const __half * __restrict__ Wup, const __half * __restrict__ Wgate,
@@ -1001,8 +1004,14 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
                                                                    float * __restrict__ partial,
                                                                    const uint32_t * __restrict__ hot_words, const int32_t * __restrict__ hot_prefix,
                                                                    uint32_t * __restrict__ words_hot, __half * __restrict__ xn_out,
-                                                                   float * __restrict__ logits2) {
+                                                                   float * __restrict__ logits2, HostAnnounce ann) {
     static_assert(PHASE == 0 || G == 1, "the two-phase form takes one group per workgroup");
+    if (PHASE == 2 && ann.flags && blockIdx.x == 0 && threadIdx.x == 0) {
+        // what was queued before this launch is complete and visible to the host: a new hand-over starts here, without a launch of its own
+        const uint32_t sq = *ann.seq + 1u;
+        *ann.seq = sq;
+        __hip_atomic_store(ann.flags, sq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
     constexpr int cols = kPfWaves * CPW * 512, r = RCH * 512;
     constexpr int CH = kPfChunk / CPW;                 // active neurons per round trip: 3*CPW*CH (2*CPW*CH) loads in flight per lane
     __shared__ float  lg[2][32];
@@ -1316,8 +1325,15 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
                                                                      float * __restrict__ h_dense, pi_q8_host_block * __restrict__ xq_out,
                                                                      float * __restrict__ logits2,
                                                                      const pi_block_q4_0 * __restrict__ Wd, const pi_block_q4_0 * __restrict__ Wd_rest,
-                                                                     float * __restrict__ partial) {
+                                                                     float * __restrict__ partial, HostAnnounce ann) {
     static_assert(!FUSE || PHASE == 0, "the fused form is one launch");
+    if (PHASE == 2 && ann.flags && blockIdx.x == 0 && threadIdx.x == 0) {
+        // what was queued before this launch is complete and visible to the host (the kernel boundary released at system scope):
+        // a new hand-over starts here, without a launch of its own
+        const uint32_t sq = *ann.seq + 1u;
+        *ann.seq = sq;
+        __hip_atomic_store(ann.flags, sq, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
+    }
     constexpr int cols = 4096, r = RCH * 512, nb = cols / 32, CH = kPfChunk;
     __shared__ float  hs[32];
     __shared__ float  lg[32];
@@ -3530,7 +3546,8 @@ __global__ void step_advance_kernel(int32_t * step) { if (threadIdx.x == 0) *ste
 // (their own cache lines) by the host, word 48 is the host's stop word; word 8 is a second device-written word.
 //   host_signal_kernel: everything queued before it on the stream is complete and visible to the host (a kernel boundary releases
 //                       at system scope): publish *seq in flags[word] (word 0 or 8), after advancing it when a new hand-over starts.
-//   host_wait_kernel:   returns once flags[slot] has reached *seq.  The wait is bounded: after `limit` ticks of the 100 MHz clock, or
+//   host_wait_kernel:   (publishes *seq in flags[signal_word] first when signal_word >= 0: a signal and a wait in one launch;)
+//                       returns once flags[slot] has reached *seq.  The wait is bounded: after `limit` ticks of the 100 MHz clock, or
 //                       when the host has set its stop word, the kernel records the failure in *status and returns, so the stream
 //                       always drains; later waits then return at once.
 __global__ void host_signal_kernel(uint32_t * __restrict__ seq, uint32_t * __restrict__ flags, int word, int advance) {
@@ -3540,10 +3557,11 @@ __global__ void host_signal_kernel(uint32_t * __restrict__ seq, uint32_t * __res
         __hip_atomic_store(flags + word, s, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);
     }
 }
-__global__ void host_wait_kernel(const uint32_t * __restrict__ seq, const uint32_t * __restrict__ flags, int slot, uint32_t * __restrict__ status,
-                                 unsigned long long limit) {
+__global__ void host_wait_kernel(const uint32_t * __restrict__ seq, uint32_t * __restrict__ flags, int slot, uint32_t * __restrict__ status,
+                                 unsigned long long limit, int signal_word) {
     if (threadIdx.x != 0) return;
     const uint32_t want = *seq;
+    if (signal_word >= 0) __hip_atomic_store(flags + signal_word, want, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_SYSTEM);     // host_signal_kernel without advance
     if (__hip_atomic_load(status, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_SYSTEM) != 0u) return;
     const unsigned long long t0 = wall_clock64();
     for (;;) {
@@ -3836,7 +3854,7 @@ int pi_k_pred_upgate_q4_split(const void * fc2_f16, int ff, int r, const float *
     const pi_block_q4_0 * u = (const pi_block_q4_0 *)up_q4; const pi_block_q4_0 * g = (const pi_block_q4_0 *)gate_q4;
     const dim3 grid(ff / 32), block(kPfBlock);
     const pi_block_q4_0 * ur = (const pi_block_q4_0 *)up_rest_q4; const pi_block_q4_0 * gr = (const pi_block_q4_0 *)gate_rest_q4;
-#define PI_PQ_LAUNCH(RCH, GATE, SPLIT) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, GATE, SPLIT>), grid, block, 0, st, w2, hidden, u, g, ur, gr, x, na, threshold, hot_words, hot_prefix, logits, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)xq8_out, nullptr, nullptr, nullptr, nullptr)
+#define PI_PQ_LAUNCH(RCH, GATE, SPLIT) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, GATE, SPLIT>), grid, block, 0, st, w2, hidden, u, g, ur, gr, x, na, threshold, hot_words, hot_prefix, logits, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)xq8_out, nullptr, nullptr, nullptr, nullptr, HostAnnounce{nullptr, nullptr})
 #define PI_PQ_LAUNCH_S(RCH, GATE) do { if (ur) PI_PQ_LAUNCH(RCH, GATE, true); else PI_PQ_LAUNCH(RCH, GATE, false); } while (0)
     if (r == 1024) { if (g) PI_PQ_LAUNCH_S(2, true); else PI_PQ_LAUNCH_S(2, false); }
     else           { if (g) PI_PQ_LAUNCH_S(1, true); else PI_PQ_LAUNCH_S(1, false); }
@@ -3862,7 +3880,7 @@ int pi_k_sparse_ffn_q4_partials(const void * fc2_f16, int ff, int r, const float
     const pi_block_q4_0 * u = (const pi_block_q4_0 *)up_q4; const pi_block_q4_0 * g = (const pi_block_q4_0 *)gate_q4; const pi_block_q4_0 * dn = (const pi_block_q4_0 *)down_t_q4;
     const pi_block_q4_0 * ur = (const pi_block_q4_0 *)up_rest_q4; const pi_block_q4_0 * gr = (const pi_block_q4_0 *)gate_rest_q4; const pi_block_q4_0 * dr = (const pi_block_q4_0 *)down_t_rest_q4;
     const dim3 grid(ff / 32), block(kPfBlock);
-#define PI_PQF(RCH, GATE, SPLIT) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, GATE, SPLIT, 0, true>), grid, block, 0, st, w2, hidden, u, g, ur, gr, x, na, threshold, hot_words, hot_prefix, logits, ws->words, (uint32_t *)nullptr, h_dense, (pi_q8_host_block *)nullptr, (float *)nullptr, dn, dr, ws->ffn_partial)
+#define PI_PQF(RCH, GATE, SPLIT) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, GATE, SPLIT, 0, true>), grid, block, 0, st, w2, hidden, u, g, ur, gr, x, na, threshold, hot_words, hot_prefix, logits, ws->words, (uint32_t *)nullptr, h_dense, (pi_q8_host_block *)nullptr, (float *)nullptr, dn, dr, ws->ffn_partial, HostAnnounce{nullptr, nullptr})
 #define PI_PQF_S(RCH, GATE) do { if (split) PI_PQF(RCH, GATE, true); else PI_PQF(RCH, GATE, false); } while (0)
     if (r == 1024) { if (g) PI_PQF_S(2, true); else PI_PQF_S(2, false); }
     else           { if (g) PI_PQF_S(1, true); else PI_PQF_S(1, false); }
@@ -3889,22 +3907,24 @@ int pi_k_pred_q4_logits(const void * fc2_f16, int ff, int r, const float * hidde
     if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_pred_q4_logits: vectors must be 16-byte aligned");
     const dim3 grid(ff / 32), block(kPfBlock);
     const pi_block_q4_0 * none = nullptr;
-#define PI_PQ1(RCH) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, false, false, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, none, x, na, threshold, (const uint32_t *)nullptr, (const int32_t *)nullptr, logits, ws->words, (uint32_t *)nullptr, (float *)nullptr, (pi_q8_host_block *)xq8_out, logits_dev, none, none, (float *)nullptr)
+#define PI_PQ1(RCH) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, false, false, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, none, x, na, threshold, (const uint32_t *)nullptr, (const int32_t *)nullptr, logits, ws->words, (uint32_t *)nullptr, (float *)nullptr, (pi_q8_host_block *)xq8_out, logits_dev, none, none, (float *)nullptr, HostAnnounce{nullptr, nullptr})
     if (r == 1024) PI_PQ1(2); else PI_PQ1(1);
 #undef PI_PQ1
     return pi::check_launch("pi_k_pred_q4_logits");
 }
 
 int pi_k_upgate_q4_hot_rows(int ff, float threshold, const void * up_q4, const void * gate_q4, int cols, const float * x, const pi_norm * norm,
-                            const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense, pi_workspace * ws, pi_stream_t stream) {
+                            const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense,
+                            uint32_t * announce_seq, uint32_t * announce_flags, pi_workspace * ws, pi_stream_t stream) {
     if (!up_q4 || !x || !hot_words || !hot_prefix || !logits_dev || !h_dense || !ws) return pi::fail(PI_E_ARG, "pi_k_upgate_q4_hot_rows: null pointer");
+    if ((announce_seq == nullptr) != (announce_flags == nullptr)) return pi::fail(PI_E_ARG, "pi_k_upgate_q4_hot_rows: announce_seq and announce_flags go together");
     if (cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_UNSUPPORTED, "pi_k_upgate_q4_hot_rows: cols must be 4096, ff % 32 == 0, within the workspace");
     const NormArgs na = to_norm(norm);
     if ((((uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_upgate_q4_hot_rows: vectors must be 16-byte aligned");
     const dim3 grid(ff / 32), block(kPfBlock);
     const pi_block_q4_0 * none = nullptr;
     const pi_block_q4_0 * u = (const pi_block_q4_0 *)up_q4; const pi_block_q4_0 * g = (const pi_block_q4_0 *)gate_q4;
-#define PI_PQ2(GATE) hipLaunchKernelGGL((pred_upgate_q4_kernel<1, GATE, false, 2>), grid, block, 0, (hipStream_t)stream, (const __half *)nullptr, (const float *)nullptr, u, g, none, none, x, na, threshold, hot_words, hot_prefix, (float *)nullptr, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)nullptr, const_cast<float *>(logits_dev), none, none, (float *)nullptr)
+#define PI_PQ2(GATE) hipLaunchKernelGGL((pred_upgate_q4_kernel<1, GATE, false, 2>), grid, block, 0, (hipStream_t)stream, (const __half *)nullptr, (const float *)nullptr, u, g, none, none, x, na, threshold, hot_words, hot_prefix, (float *)nullptr, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)nullptr, const_cast<float *>(logits_dev), none, none, (float *)nullptr, HostAnnounce{announce_seq, announce_flags})
     if (g) PI_PQ2(true); else PI_PQ2(false);
 #undef PI_PQ2
     return pi::check_launch("pi_k_upgate_q4_hot_rows");
@@ -3979,7 +3999,7 @@ static int sparse_ffn_partials_impl(const char * who, const void * fc2_f16, int 
     const int G = pf_groups(ff, cols);
     const dim3 grid(ff / (32 * G)), block(kPfBlock);
     const bool hyb = hot_words != nullptr;
-#define PI_PF_LAUNCH2(CPW, RCH, GATE, GG, HYB) hipLaunchKernelGGL((pred_ffn_f16_kernel<CPW, RCH, GATE, GG, HYB>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial, hot_words, hot_prefix, ws->words_hot, (__half *)xn_f16_out, nullptr)
+#define PI_PF_LAUNCH2(CPW, RCH, GATE, GG, HYB) hipLaunchKernelGGL((pred_ffn_f16_kernel<CPW, RCH, GATE, GG, HYB>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial, hot_words, hot_prefix, ws->words_hot, (__half *)xn_f16_out, nullptr, HostAnnounce{nullptr, nullptr})
 #define PI_PF_LAUNCH(CPW, RCH, GATE, GG) do { if (hyb) PI_PF_LAUNCH2(CPW, RCH, GATE, GG, true); else PI_PF_LAUNCH2(CPW, RCH, GATE, GG, false); } while (0)
 #define PI_PF_WIDE(RCH, GATE) do { if (G == 4) PI_PF_LAUNCH(2, RCH, GATE, 4); else if (G == 2) PI_PF_LAUNCH(2, RCH, GATE, 2); else PI_PF_LAUNCH(2, RCH, GATE, 1); } while (0)
     const int cpw = cols / 4096, rch = r / 512;
@@ -4020,7 +4040,7 @@ int pi_k_sparse_ffn_logits_hot(const void * fc2_f16, int ff, int r, const float 
     if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b | (uintptr_t)xn_f16_out) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_logits_hot: vectors must be 16-byte aligned");
     const dim3 grid(ff / 32), block(kPfBlock);
     const __half * none = nullptr;
-#define PI_PF1(RCH) hipLaunchKernelGGL((pred_ffn_f16_kernel<1, RCH, false, 1, true, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, x, na, threshold, logits, ws->words, (float *)nullptr, (float *)nullptr, hot_words, hot_prefix, ws->words_hot, (__half *)xn_f16_out, logits_dev)
+#define PI_PF1(RCH) hipLaunchKernelGGL((pred_ffn_f16_kernel<1, RCH, false, 1, true, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, x, na, threshold, logits, ws->words, (float *)nullptr, (float *)nullptr, hot_words, hot_prefix, ws->words_hot, (__half *)xn_f16_out, logits_dev, HostAnnounce{nullptr, nullptr})
     if (r == 1024) PI_PF1(2); else PI_PF1(1);
 #undef PI_PF1
     return pi::check_launch("pi_k_sparse_ffn_logits_hot");
@@ -4028,14 +4048,15 @@ int pi_k_sparse_ffn_logits_hot(const void * fc2_f16, int ff, int r, const float 
 
 int pi_k_sparse_ffn_rows_hot(int ff, float threshold, const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x,
                              const pi_norm * norm, const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense,
-                             pi_workspace * ws, pi_stream_t stream) {
+                             uint32_t * announce_seq, uint32_t * announce_flags, pi_workspace * ws, pi_stream_t stream) {
     if (!up_f16 || !down_t_f16 || !x || !hot_words || !hot_prefix || !logits_dev || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_rows_hot: null pointer");
+    if ((announce_seq == nullptr) != (announce_flags == nullptr)) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_rows_hot: announce_seq and announce_flags go together");
     if (cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn_rows_hot: cols must be 4096, ff % 32 == 0, within the workspace");
     const NormArgs na = to_norm(norm);
     if ((((uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_rows_hot: vectors must be 16-byte aligned");
     const dim3 grid(ff / 32), block(kPfBlock);
     const __half * u = (const __half *)up_f16; const __half * g = (const __half *)gate_f16; const __half * dn = (const __half *)down_t_f16;
-#define PI_PF2(GATE) hipLaunchKernelGGL((pred_ffn_f16_kernel<1, 1, GATE, 1, true, 2>), grid, block, 0, (hipStream_t)stream, (const __half *)nullptr, (const float *)nullptr, u, g, dn, x, na, threshold, (float *)nullptr, ws->words, h_dense, ws->ffn_partial, hot_words, hot_prefix, ws->words_hot, (__half *)nullptr, const_cast<float *>(logits_dev))
+#define PI_PF2(GATE) hipLaunchKernelGGL((pred_ffn_f16_kernel<1, 1, GATE, 1, true, 2>), grid, block, 0, (hipStream_t)stream, (const __half *)nullptr, (const float *)nullptr, u, g, dn, x, na, threshold, (float *)nullptr, ws->words, h_dense, ws->ffn_partial, hot_words, hot_prefix, ws->words_hot, (__half *)nullptr, const_cast<float *>(logits_dev), HostAnnounce{announce_seq, announce_flags})
     if (g) PI_PF2(true); else PI_PF2(false);
 #undef PI_PF2
     return pi::check_launch("pi_k_sparse_ffn_rows_hot");
@@ -4493,10 +4514,14 @@ int pi_k_host_signal(uint32_t * seq, uint32_t * flags_pinned, int word, int adva
     return pi::check_launch("pi_k_host_signal");
 }
 int pi_k_host_wait(const uint32_t * seq, const uint32_t * flags_pinned, int slot, uint32_t * status_pinned, double limit_seconds, pi_stream_t stream) {
+    return pi_k_host_signal_wait(seq, const_cast<uint32_t *>(flags_pinned), -1, slot, status_pinned, limit_seconds, stream);
+}
+int pi_k_host_signal_wait(const uint32_t * seq, uint32_t * flags_pinned, int signal_word, int slot, uint32_t * status_pinned, double limit_seconds, pi_stream_t stream) {
     if (!seq || !flags_pinned || !status_pinned || (slot != 16 && slot != 32) || !(limit_seconds > 0.0) || limit_seconds > 60.0)
         return pi::fail(PI_E_ARG, "pi_k_host_wait: bad arguments (slot 16 or 32, 0 < limit <= 60 s)");
+    if (signal_word != -1 && signal_word != 0 && signal_word != 8) return pi::fail(PI_E_ARG, "pi_k_host_signal_wait: signal word 0 or 8, or -1 for none");
     hipLaunchKernelGGL(host_wait_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, seq, flags_pinned, slot, status_pinned,
-                       (unsigned long long)(limit_seconds * 1e8));
+                       (unsigned long long)(limit_seconds * 1e8), signal_word);
     return pi::check_launch("pi_k_host_wait");
 }
 

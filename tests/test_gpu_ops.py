@@ -333,13 +333,12 @@ def test_host_signal_and_bounded_wait():
     seq, status = pl.DevBuf.zeros(4), pl.DevBuf.zeros(4)
     try:
         pl.check(L.pi_k_host_signal(seq.ptr, fp, 0, 1, None), "signal")
-        pl.check(L.pi_k_host_signal(seq.ptr, fp, 8, 0, None), "signal")
         pl.sync()
-        assert int(flags[0]) == 1 and int(flags[8]) == 1 and int(seq.download(np.uint32)[0]) == 1
+        assert int(flags[0]) == 1 and int(flags[8]) == 0 and int(seq.download(np.uint32)[0]) == 1
         flags[16] = 1                                           # the host has already answered hand-over 1
-        pl.check(L.pi_k_host_wait(seq.ptr, fp, 16, status.ptr, 5.0, None), "wait")
+        pl.check(L.pi_k_host_signal_wait(seq.ptr, fp, 8, 16, status.ptr, 5.0, None), "signal_wait")       # the second signal travels with the wait
         pl.sync()
-        assert int(status.download(np.uint32)[0]) == 0
+        assert int(status.download(np.uint32)[0]) == 0 and int(flags[8]) == 1
         pl.check(L.pi_k_host_wait(seq.ptr, fp, 32, status.ptr, 5.0, None), "wait")      # answered while the kernel polls
         time.sleep(0.05)
         flags[32] = 1
@@ -354,6 +353,7 @@ def test_host_signal_and_bounded_wait():
         pl.sync()
         assert time.time() - t0 < 5.0
         assert L.pi_k_host_wait(seq.ptr, fp, 7, status.ptr, 1.0, None) != 0
+        assert L.pi_k_host_signal_wait(seq.ptr, fp, 16, 32, status.ptr, 1.0, None) != 0                    # word 16 is the host's
         assert L.pi_k_host_wait(seq.ptr, fp, 16, status.ptr, 1e9, None) != 0
     finally:
         pl.sync()

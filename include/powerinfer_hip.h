@@ -331,13 +331,14 @@ PI_API int pi_k_sparse_ffn_q4_reduce(int ff, int cols, int epilogue, const float
  * pi_k_host_signal_wait: a signal without advance (signal_word 0 or 8; -1 = none) and a wait in one launch. */
 PI_API int pi_k_host_signal(uint32_t * seq, uint32_t * flags_pinned, int word, int advance, pi_stream_t stream);
 /* pi_k_pred_upgate_q4 cut in two for such a layer, so that the host threads start behind the predictor: pi_k_pred_q4_logits computes the
- * logits (to `logits`, which may be pinned host memory, and to logits_dev), the mask words and the Q8_0 blocks of the normalised input;
+ * logits (to `logits`, optional, which may be pinned host memory, and to logits_dev), the mask words (bit j of word w = neuron 32 w + j is
+ * active; also to words_out, optional, which may be pinned host memory) and the Q8_0 blocks of the normalised input;
  * pi_k_upgate_q4_hot_rows reads logits_dev and writes h (or 0) for the neurons of the hot words only - the other entries of h_dense
  * belong to the host.  With announce_seq / announce_flags (both or neither) the first lane of that launch does what
  * pi_k_host_signal(announce_seq, announce_flags, 0, 1) would have done right before it: the predictor's results are complete and
  * visible to the host at the boundary in front of the launch, so the hand-over needs no launch of its own. */
 PI_API int pi_k_pred_q4_logits(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
-                               float * logits, float * logits_dev, void * xq8_out, pi_workspace * ws, pi_stream_t stream);
+                               float * logits, float * logits_dev, void * xq8_out, uint32_t * words_out, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_upgate_q4_hot_rows(int ff, float threshold, const void * up_q4, const void * gate_q4, int cols, const float * x, const pi_norm * norm,
                                    const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense,
                                    uint32_t * announce_seq, uint32_t * announce_flags, pi_workspace * ws, pi_stream_t stream);

@@ -253,6 +253,7 @@ class Pool {
 struct ColdLayer {
     std::vector<float> norm_w, norm_b;          // host copies of the FFN-input norm
     std::vector<int32_t> cold_rows;             // neurons with gpu_idx == 0, ascending
+    std::vector<uint32_t> cold_words;           // the same as bits: bit j of word w = neuron 32 w + j
 };
 
 struct ColdPath {
@@ -263,6 +264,7 @@ struct ColdPath {
     float * h_full[2] = {nullptr, nullptr}, * out[2] = {nullptr, nullptr};   // host -> device, read by the GPU after the call returned: two sets, used in turn
     BlockQ8 * xq8_pin = nullptr;                // Q8_0 blocks of the normalised FFN input, written by the fused Q4_0 kernel
     uint16_t * x16_pin = nullptr;               // fp16 normalised FFN input, written by the fused F16 kernel
+    uint32_t * words_pin = nullptr;             // activity words of the layer in flight, written by the split-off Q4_0 predictor launch
     int flip = 0;
     hipEvent_t ev_in = nullptr, ev_h = nullptr;
     std::vector<float> hval;                    // h of the active cold neurons, in the order of act
@@ -324,14 +326,16 @@ ColdPath * cold_create(pi_model * m) {
             if (pi_memcpy_d2h(cl.norm_b.data(), m->L(il, PI_T_ATTN_NORM_B).dev, sizeof(float) * c->d) != PI_OK) { cold_destroy(c); return nullptr; }
         }
         const int32_t * gid = (const int32_t *)m->L(il, PI_T_GPU_IDX).host;
-        for (int j = 0; j < c->ff; ++j) if (gid[j] != 1) cl.cold_rows.push_back(j);
+        cl.cold_words.assign((size_t)(c->ff + 31) / 32, 0u);
+        for (int j = 0; j < c->ff; ++j) if (gid[j] != 1) { cl.cold_rows.push_back(j); cl.cold_words[j >> 5] |= 1u << (j & 31); }
     }
     auto pin = [](size_t n) { void * p = nullptr; return hipHostMalloc(&p, n * sizeof(float), hipHostMallocCoherent) == hipSuccess ? (float *)p : nullptr; };
     c->xq8_pin = (BlockQ8 *)pin((size_t)(c->d / 32 + 1) * sizeof(BlockQ8) / sizeof(float) + 1);
     c->x16_pin = (uint16_t *)pin((size_t)c->d / 2 + 8);
+    c->words_pin = (uint32_t *)pin((size_t)c->ff / 32 + 8);
     c->logits = pin(c->ff); c->src = pin(c->d); c->h_gpu = pin(c->ff);
     for (int i = 0; i < 2; ++i) { c->h_full[i] = pin(c->ff); c->out[i] = pin(c->d); }
-    if (!c->logits || !c->src || !c->h_gpu || !c->h_full[0] || !c->h_full[1] || !c->out[0] || !c->out[1] || !c->xq8_pin || !c->x16_pin) { set_error("cold path: pinned host allocation failed"); cold_destroy(c); return nullptr; }
+    if (!c->logits || !c->src || !c->h_gpu || !c->h_full[0] || !c->h_full[1] || !c->out[0] || !c->out[1] || !c->xq8_pin || !c->x16_pin || !c->words_pin) { set_error("cold path: pinned host allocation failed"); cold_destroy(c); return nullptr; }
     if (hipEventCreateWithFlags(&c->ev_in, hipEventDisableTiming) != hipSuccess || hipEventCreateWithFlags(&c->ev_h, hipEventDisableTiming) != hipSuccess) {
         set_error("cold path: event creation failed"); cold_destroy(c); return nullptr;
     }
@@ -390,6 +394,7 @@ void cold_destroy(ColdPath * c) {
     for (float * p : {c->logits, c->src, c->h_gpu, c->h_full[0], c->h_full[1], c->out[0], c->out[1]}) if (p) (void)hipHostFree(p);
     if (c->xq8_pin) (void)hipHostFree(c->xq8_pin);
     if (c->x16_pin) (void)hipHostFree(c->x16_pin);
+    if (c->words_pin) (void)hipHostFree(c->words_pin);
     if (c->ev_in) (void)hipEventDestroy(c->ev_in);
     if (c->ev_h) (void)hipEventDestroy(c->ev_h);
     delete c;
@@ -411,6 +416,16 @@ namespace {
 // ---- the host share's three steps, shared by the variant that launches between them and the one that answers the stream's signals ----
 
 // neurons of this layer that are not GPU-resident and whose predictor logit reaches the threshold, ascending, into c->act
+// the same list from the activity words the predictor launch left in pinned memory: 1.4 KB to read instead of a logit per cold neuron
+int list_active_cold_words(ColdPath * c, const ColdLayer & cl) {
+    c->act.clear();
+    const uint32_t * aw = c->words_pin;
+    const int nw = (int)cl.cold_words.size();
+    for (int w = 0; w < nw; ++w)
+        for (uint32_t bits = aw[w] & cl.cold_words[w]; bits; bits &= bits - 1) c->act.push_back(w * 32 + __builtin_ctz(bits));
+    return (int)c->act.size();
+}
+
 int list_active_cold(ColdPath * c, const ColdLayer & cl, float thr) {
     c->act.clear();
     for (int j : cl.cold_rows) if (!(c->logits[j] < thr)) c->act.push_back(j);
@@ -804,7 +819,7 @@ void serve_q4(ColdPath * c, int il, uint32_t seq) {
         for (int j : c->prev_act[il]) hfull[j] = 0.f;
         c->prev_act[il].clear();
     }
-    const int na = list_active_cold(c, cl, thr);
+    const int na = c->split_pred ? list_active_cold_words(c, cl) : list_active_cold(c, cl, thr);
     lap(1);
     host_upgate(c, m, il, na);
     const float * hval = c->hval.data();
@@ -958,7 +973,7 @@ int cold_layer_q4_queue(ColdPath * c, int il, pi_model * m, hipStream_t st) {
     const float * ffn_src = falcon ? m->x : m->ffn_inp;
     if (c->split_pred) {
         hfull = c->h_async[il];
-        PI_TRY(pi_k_pred_q4_logits(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, d, ffn_src, &fn, c->logits, m->pred_logits, c->xq8_pin, m->ws, st));
+        PI_TRY(pi_k_pred_q4_logits(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, d, ffn_src, &fn, nullptr, m->pred_logits, c->xq8_pin, c->words_pin, m->ws, st));
         // the hand-over starts in the first lane of the next launch, and the second signal travels with the wait behind it
         PI_TRY(pi_k_upgate_q4_hot_rows(ff, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, d, ffn_src, &fn, m->hot_words[il], m->hot_prefix[il],
                                        m->pred_logits, hfull, c->d_seq, c->flags, m->ws, st));

@@ -3900,14 +3900,14 @@ int pi_k_sparse_ffn_q4_reduce(int ff, int cols, int epilogue, const float * add1
 }
 
 int pi_k_pred_q4_logits(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
-                        float * logits, float * logits_dev, void * xq8_out, pi_workspace * ws, pi_stream_t stream) {
+                        float * logits, float * logits_dev, void * xq8_out, uint32_t * words_out, pi_workspace * ws, pi_stream_t stream) {
     if (!fc2_f16 || !hidden || !x || !logits_dev || !ws) return pi::fail(PI_E_ARG, "pi_k_pred_q4_logits: null pointer");
     if (!pi_k_pred_upgate_q4_supported(ff, r, cols) || ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_UNSUPPORTED, "pi_k_pred_q4_logits: shape outside the fused kernel or the workspace");
     const NormArgs na = to_norm(norm);
     if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_pred_q4_logits: vectors must be 16-byte aligned");
     const dim3 grid(ff / 32), block(kPfBlock);
     const pi_block_q4_0 * none = nullptr;
-#define PI_PQ1(RCH) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, false, false, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, none, x, na, threshold, (const uint32_t *)nullptr, (const int32_t *)nullptr, logits, ws->words, (uint32_t *)nullptr, (float *)nullptr, (pi_q8_host_block *)xq8_out, logits_dev, none, none, (float *)nullptr, HostAnnounce{nullptr, nullptr})
+#define PI_PQ1(RCH) hipLaunchKernelGGL((pred_upgate_q4_kernel<RCH, false, false, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, none, x, na, threshold, (const uint32_t *)nullptr, (const int32_t *)nullptr, logits, ws->words, words_out, (float *)nullptr, (pi_q8_host_block *)xq8_out, logits_dev, none, none, (float *)nullptr, HostAnnounce{nullptr, nullptr})
     if (r == 1024) PI_PQ1(2); else PI_PQ1(1);
 #undef PI_PQ1
     return pi::check_launch("pi_k_pred_q4_logits");

@@ -257,13 +257,14 @@ class SparseFFN:
         h_p, h = pinned(self.ff * 4, np.float32)
         out_p, out_host = pinned(self.d * 4, np.float32)
         xq_p, xq = pinned(self.d // 32 * 34, np.uint8)
+        words_p, words = pinned(self.ff // 32 * 4, np.uint32)
         seq, status, lg_dev = DevBuf.zeros(4), DevBuf.zeros(4), DevBuf(self.ff * 4)
         try:
             self.x.upload(np.asarray(x_ffn, np.float32))
             self.xp.upload(np.asarray(x_pred, np.float32))
             nrm = pl.norm_arg(self.norm_kind, self.eps, self.norm_w, self.norm_b)
             check(L.pi_k_gemv(pl.F16, self.fc1.ptr, self.r, self.d, self.xp.ptr, None, pl.EPI_RELU, None, None, self.hidden.ptr, None), "fc1")
-            check(L.pi_k_pred_q4_logits(self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, self.d, self.x.ptr, nrm, lg_p, lg_dev.ptr, xq_p, self.ws, None), "pred_q4_logits")
+            check(L.pi_k_pred_q4_logits(self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, self.d, self.x.ptr, nrm, lg_p, lg_dev.ptr, xq_p, words_p, self.ws, None), "pred_q4_logits")
             check(L.pi_k_upgate_q4_hot_rows(self.ff, self.thr, self.up.ptr, p(self.gate), self.d, self.x.ptr, nrm, hw.ptr, hp.ptr, lg_dev.ptr, h_p,
                                             seq.ptr, flags_p, self.ws, None), "hot_rows")
             check(L.pi_k_host_signal_wait(seq.ptr, flags_p, 8, 16, status.ptr, limit_s, None), "signal_wait")
@@ -286,11 +287,11 @@ class SparseFFN:
             flags[32] = 1
             pl.sync()
             return dict(logits=lg.copy(), h=h.copy(), n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32),
-                        status=int(status.download(np.uint32)[0]))
+                        status=int(status.download(np.uint32)[0]), words=words.copy())
         finally:
             pl.sync()
-            del flags, lg, h, out_host, xq
-            for ptr in (flags_p, lg_p, h_p, out_p, xq_p):
+            del flags, lg, h, out_host, xq, words
+            for ptr in (flags_p, lg_p, h_p, out_p, xq_p, words_p):
                 L.pi_free_host(ptr)
 
     def close(self):

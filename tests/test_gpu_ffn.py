@@ -365,6 +365,8 @@ def test_q4_hybrid_layer_with_stream_handovers():
     res = ffn.forward_q4_handover(x, x, host_h, host_out)
     assert res["status"] == 0
     assert np.array_equal(res["logits"], base["logits"])
+    thr_bits = np.packbits(~(base["logits"] < ffn.thr), bitorder="little").view(np.uint32)
+    assert np.array_equal(res["words"], thr_bits)               # the activity words the host lists its neurons from
     hm = base["h"].copy(); hm[cold] = ref["full"]["h"][cold]
     assert np.array_equal(got["h_full"], hm)                    # resident entries from the device, the others from the host, zeros elsewhere
     assert res["n_active"] == base["n_active"]

@@ -145,6 +145,34 @@ void axpy_q4_blocks(const BlockQ4 * row, int b0, int b1, int a, float sc, float 
     }
 }
 
+// The same sums with the loops exchanged: the 32 outputs of block b stay in registers while every listed row adds its product, in
+// list order, so each output sees the additions of axpy_q4_blocks row by row in the same order (bit-identical) without a load and
+// a store of the output per row.  rows[k] = start of row k, a[k] != 0 its Q8_0 value of h, sc[k] that block's scale.
+void axpy_q4_rows(const BlockQ4 * const * rows, const int * a, const float * sc, int n_rows, int b0, int b1, float * out) {
+#ifdef PI_COLD_SIMD
+    const __m128i lowmask = _mm_set1_epi8(0x0F), eight = _mm_set1_epi8(8);
+    for (int b = b0; b < b1; ++b) {
+        __m256 acc[4] = {_mm256_setzero_ps(), _mm256_setzero_ps(), _mm256_setzero_ps(), _mm256_setzero_ps()};
+        for (int k = 0; k < n_rows; ++k) {
+            const BlockQ4 & blk = rows[k][b];
+            const __m256 dv = _mm256_set1_ps(h2f(blk.d) * sc[k]);
+            const __m128i q = _mm_loadu_si128((const __m128i *)blk.qs);
+            const __m128i lo = _mm_sub_epi8(_mm_and_si128(q, lowmask), eight), hi = _mm_sub_epi8(_mm_and_si128(_mm_srli_epi16(q, 4), lowmask), eight);
+            const __m256i av = _mm256_set1_epi16((short)a[k]);
+            const __m256i plo = _mm256_mullo_epi16(_mm256_cvtepi8_epi16(lo), av), phi = _mm256_mullo_epi16(_mm256_cvtepi8_epi16(hi), av);
+            acc[0] = _mm256_add_ps(acc[0], _mm256_mul_ps(_mm256_cvtepi32_ps(_mm256_cvtepi16_epi32(_mm256_castsi256_si128(plo))), dv));
+            acc[1] = _mm256_add_ps(acc[1], _mm256_mul_ps(_mm256_cvtepi32_ps(_mm256_cvtepi16_epi32(_mm256_extracti128_si256(plo, 1))), dv));
+            acc[2] = _mm256_add_ps(acc[2], _mm256_mul_ps(_mm256_cvtepi32_ps(_mm256_cvtepi16_epi32(_mm256_castsi256_si128(phi))), dv));
+            acc[3] = _mm256_add_ps(acc[3], _mm256_mul_ps(_mm256_cvtepi32_ps(_mm256_cvtepi16_epi32(_mm256_extracti128_si256(phi, 1))), dv));
+        }
+        for (int i = 0; i < 4; ++i) _mm256_storeu_ps(out + b * 32 + 8 * i, acc[i]);
+    }
+#else
+    for (int i = b0 * 32; i < b1 * 32; ++i) out[i] = 0.f;
+    for (int k = 0; k < n_rows; ++k) axpy_q4_blocks(rows[k], b0, b1, a[k], sc[k], out);
+#endif
+}
+
 // the cold rows live in host DRAM and a token touches each of them once: fetch the next row while this one is used
 inline void prefetch_bytes(const void * p, size_t n) {
 #ifdef PI_COLD_SIMD
@@ -268,6 +296,7 @@ struct ColdPath {
     int flip = 0;
     hipEvent_t ev_in = nullptr, ev_h = nullptr;
     std::vector<float> hval;                    // h of the active cold neurons, in the order of act
+    std::vector<const BlockQ4 *> dn_rows; std::vector<int> dn_a; std::vector<float> dn_sc;    // the rows of one Q4_0 down projection
     // PI_COLD_TRACE=1: mean host time per phase of a layer call, printed when the model is freed
     bool trace = false;
     double t_phase[6] = {0, 0, 0, 0, 0, 0};
@@ -479,6 +508,23 @@ void host_down(ColdPath * c, pi_model * m, int il, int na, const float * hfull, 
         }
     }
     const int n_units = d / 32;
+    if (q4) {
+        // rows whose h rounds to 0 add nothing (skipped, as before); each thread takes a band of column blocks over all rows
+        c->dn_rows.clear(); c->dn_a.clear(); c->dn_sc.clear();
+        for (int k = 0; k < na; ++k) {
+            const int j = c->act[k];
+            const BlockQ8 & hb = c->hq8[j / 32];
+            if (hb.qs[j % 32] == 0) continue;
+            c->dn_rows.push_back((const BlockQ4 *)(wd + rb * j)); c->dn_a.push_back(hb.qs[j % 32]); c->dn_sc.push_back(h2f(hb.d));
+        }
+        const int nr = (int)c->dn_rows.size();
+        c->pool->run([&](int t, int nt) {
+            const int u0 = (int)((long long)n_units * t / nt), u1 = (int)((long long)n_units * (t + 1) / nt);
+            for (int k = 0; k < nr; ++k) prefetch_bytes((const unsigned char *)(c->dn_rows[k] + u0), (size_t)(u1 - u0) * 18);
+            axpy_q4_rows(c->dn_rows.data(), c->dn_a.data(), c->dn_sc.data(), nr, u0, u1, out);
+        });
+        return;
+    }
     c->pool->run([&](int t, int nt) {
         const int u0 = (int)((long long)n_units * t / nt), u1 = (int)((long long)n_units * (t + 1) / nt);
         const int c0 = u0 * 32, c1 = u1 * 32;

@@ -297,6 +297,8 @@ struct ColdPath {
     hipEvent_t ev_in = nullptr, ev_h = nullptr;
     std::vector<float> hval;                    // h of the active cold neurons, in the order of act
     std::vector<const BlockQ4 *> dn_rows; std::vector<int> dn_a; std::vector<float> dn_sc;    // the rows of one Q4_0 down projection
+    std::vector<int> act_down;                  // see list_active_cold_words
+    bool mixed_on_host = false;                 // Q4_0 hand-over layers: blocks with an active non-resident neuron are computed by the host as a whole
     // PI_COLD_TRACE=1: mean host time per phase of a layer call, printed when the model is freed
     bool trace = false;
     double t_phase[6] = {0, 0, 0, 0, 0, 0};
@@ -388,6 +390,11 @@ ColdPath * cold_create(pi_model * m) {
         c->flags = (uint32_t *)fl;
         memset(c->flags, 0, 64 * sizeof(uint32_t));
         if (const char * e = getenv("PI_COLD_SPLIT")) c->split_pred = e[0] != '0';
+        // PI_COLD_MIXED=host: 32-neuron blocks with an active non-resident neuron are computed by the host as a whole, so the device
+        // waits for the host once per layer instead of twice.  Measured slower with 8 host threads (the host's down projection
+        // grows from 84 to about 250 rows per 7B layer: 437 -> 381 tok/s), so the default keeps every resident row on the device.
+        const char * mx = getenv("PI_COLD_MIXED");
+        c->mixed_on_host = c->split_pred && mx && !strcmp(mx, "host");
         c->h_async.assign(hp.n_layer, nullptr);
         c->prev_act.resize(hp.n_layer);
         for (int il : c->async_layers) {
@@ -446,12 +453,19 @@ namespace {
 
 // neurons of this layer that are not GPU-resident and whose predictor logit reaches the threshold, ascending, into c->act
 // the same list from the activity words the predictor launch left in pinned memory: 1.4 KB to read instead of a logit per cold neuron
+// act_down: every active neuron, resident or not, of the blocks that hold an active non-resident one (the host's down rows when
+// such blocks are the host's as a whole)
 int list_active_cold_words(ColdPath * c, const ColdLayer & cl) {
     c->act.clear();
+    c->act_down.clear();
     const uint32_t * aw = c->words_pin;
     const int nw = (int)cl.cold_words.size();
-    for (int w = 0; w < nw; ++w)
-        for (uint32_t bits = aw[w] & cl.cold_words[w]; bits; bits &= bits - 1) c->act.push_back(w * 32 + __builtin_ctz(bits));
+    for (int w = 0; w < nw; ++w) {
+        const uint32_t all = aw[w];
+        if ((all & cl.cold_words[w]) == 0u) continue;
+        for (uint32_t bits = all & cl.cold_words[w]; bits; bits &= bits - 1) c->act.push_back(w * 32 + __builtin_ctz(bits));
+        if (c->mixed_on_host) for (uint32_t bits = all; bits; bits &= bits - 1) c->act_down.push_back(w * 32 + __builtin_ctz(bits));
+    }
     return (int)c->act.size();
 }
 
@@ -494,7 +508,7 @@ void host_upgate(ColdPath * c, pi_model * m, int il, int na) {
 // the listed neurons' share of the down projection into out[d]; threads split the output columns in blocks of 32, so no two threads
 // add into the same element.  Q4_0: h goes through the Q8_0 blocks of the completed vector hfull (only the blocks that hold a listed
 // neuron are quantised; ggml.c:14465-14618); F16: h rounded to fp16 (ggml.c:14420-14431).
-void host_down(ColdPath * c, pi_model * m, int il, int na, const float * hfull, float * out) {
+void host_down(ColdPath * c, pi_model * m, int il, int na, const float * hfull, float * out, bool whole_blocks = false) {
     Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
     const bool q4 = down.type == PI_TYPE_Q4_0;
     const int d = c->d;
@@ -511,8 +525,9 @@ void host_down(ColdPath * c, pi_model * m, int il, int na, const float * hfull, 
     if (q4) {
         // rows whose h rounds to 0 add nothing (skipped, as before); each thread takes a band of column blocks over all rows
         c->dn_rows.clear(); c->dn_a.clear(); c->dn_sc.clear();
-        for (int k = 0; k < na; ++k) {
-            const int j = c->act[k];
+        const std::vector<int> & rows_of = whole_blocks ? c->act_down : c->act;
+        for (size_t k = 0; k < rows_of.size(); ++k) {
+            const int j = rows_of[k];
             const BlockQ8 & hb = c->hq8[j / 32];
             if (hb.qs[j % 32] == 0) continue;
             c->dn_rows.push_back((const BlockQ4 *)(wd + rb * j)); c->dn_a.push_back(hb.qs[j % 32]); c->dn_sc.push_back(h2f(hb.d));
@@ -871,7 +886,8 @@ void serve_q4(ColdPath * c, int il, uint32_t seq) {
     const float * hval = c->hval.data();
     for (int k = 0; k < na; ++k) hfull[c->act[k]] = hval[k];
     if (c->split_pred) c->prev_act[il].assign(c->act.begin(), c->act.end());
-    __atomic_store_n(&c->flags[16], seq, __ATOMIC_RELEASE);          // the device's down projection may read the completed vector
+    const bool whole = c->split_pred && c->mixed_on_host;
+    if (!whole) __atomic_store_n(&c->flags[16], seq, __ATOMIC_RELEASE);          // the device's down projection may read the completed vector
     lap(2);
     if (c->split_pred) {
         // the Q8_0 scales of h span resident and non-resident neurons: the resident ones' h must have arrived
@@ -888,7 +904,7 @@ void serve_q4(ColdPath * c, int il, uint32_t seq) {
 
     // 3. the host quantises h the same way and adds its neurons' down rows
     lap(3);
-    host_down(c, m, il, na, hfull, out);
+    host_down(c, m, il, na, hfull, out, whole);
     __atomic_store_n(&c->flags[32], seq, __ATOMIC_RELEASE);          // the reduction may add the host share
     lap(4);
     if (c->trace) { ++c->n_calls; c->n_cold_active += na; c->t_last_return = now(); }
@@ -1022,7 +1038,15 @@ int cold_layer_q4_queue(ColdPath * c, int il, pi_model * m, hipStream_t st) {
         PI_TRY(pi_k_pred_q4_logits(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, d, ffn_src, &fn, nullptr, m->pred_logits, c->xq8_pin, c->words_pin, m->ws, st));
         // the hand-over starts in the first lane of the next launch, and the second signal travels with the wait behind it
         PI_TRY(pi_k_upgate_q4_hot_rows(ff, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, d, ffn_src, &fn, m->hot_words[il], m->hot_prefix[il],
-                                       m->pred_logits, hfull, c->d_seq, c->flags, m->ws, st));
+                                       m->pred_logits, hfull, c->d_seq, c->flags, c->mixed_on_host ? down.dev : nullptr, m->ws, st));
+        if (c->mixed_on_host) {
+            // blocks with an active non-resident neuron are the host's as a whole: nothing to wait for before the reduction
+            PI_TRY(pi_k_host_signal_wait(c->d_seq, c->flags, 8, 32, c->d_status, limit, st));
+            int32_t * n_act = m->n_active + il;
+            if (!falcon) return pi_k_sparse_ffn_q4_reduce_hot(ff, d, PI_EPI_ADD2, out, m->ffn_inp, m->x2, n_act, m->ws, st);
+            PI_TRY(pi_k_sparse_ffn_q4_reduce_hot(ff, d, PI_EPI_NONE, nullptr, nullptr, m->x2, n_act, m->ws, st));
+            return merge_shares(m->x2, out, m->x2, m->attn_out, m->x, nullptr, d, st);
+        }
     } else {
         PI_TRY(pi_k_pred_upgate_q4(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, d, ffn_src, &fn,
                                    m->hot_words[il], m->hot_prefix[il], c->logits, hfull, c->xq8_pin, m->ws, st));

@@ -350,13 +350,14 @@ PI_API int pi_k_upgate_q4_hot_rows(int ff, float threshold, const void * up_q4, 
                                    const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense,
                                    uint32_t * announce_seq, uint32_t * announce_flags, const void * down_t_q4, pi_workspace * ws, pi_stream_t stream);
 /* The fused F16 launch of a hybrid layer (pi_k_sparse_ffn_partials_hot) cut in two in the same way (cols 4096): pi_k_sparse_ffn_logits_hot
- * computes the logits (to `logits`, which may be pinned host memory, and to logits_dev), the mask words and the fp16 normalised input for
+ * computes the logits (to `logits`, optional, which may be pinned host memory, and to logits_dev), the mask words (also to words_out,
+ * optional, as pi_k_pred_q4_logits) and the fp16 normalised input for
  * the host; pi_k_sparse_ffn_rows_hot reads logits_dev and computes the resident active neurons' gate / up / down rows into the partial
  * vectors that pi_k_sparse_ffn_reduce_hot adds; announce_seq / announce_flags as for pi_k_upgate_q4_hot_rows. */
 PI_API int pi_k_sparse_ffn_two_phase_supported(int ff, int r, int cols);
 PI_API int pi_k_sparse_ffn_logits_hot(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
                                       const uint32_t * hot_words, const int32_t * hot_prefix, float * logits, float * logits_dev, void * xn_f16_out,
-                                      pi_workspace * ws, pi_stream_t stream);
+                                      uint32_t * words_out, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_sparse_ffn_rows_hot(int ff, float threshold, const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x,
                                     const pi_norm * norm, const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense,
                                     uint32_t * announce_seq, uint32_t * announce_flags, pi_workspace * ws, pi_stream_t stream);

@@ -918,7 +918,6 @@ void serve_f16(ColdPath * c, int il, uint32_t seq) {
     const bool falcon = hp.arch == PI_ARCH_FALCON;
     ColdLayer & cl = c->layers[il];
     Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
-    const float thr = hp.sparse_threshold;
     float * out = c->out[0];
     auto now = [] { return std::chrono::steady_clock::now(); };
     auto us = [](std::chrono::steady_clock::time_point a, std::chrono::steady_clock::time_point b) { return std::chrono::duration<double, std::micro>(b - a).count(); };
@@ -937,7 +936,7 @@ void serve_f16(ColdPath * c, int il, uint32_t seq) {
         }
     }
     lap(0);
-    const int na = list_active_cold(c, cl, thr);
+    const int na = list_active_cold_words(c, cl);
     lap(1);
     host_upgate(c, m, il, na);
     lap(2);
@@ -1078,7 +1077,7 @@ int cold_layer_f16_queue(ColdPath * c, int il, pi_model * m, hipStream_t st) {
     fn.b = falcon ? (const float *)m->L(il, PI_T_ATTN_NORM_B).dev : nullptr;
     const float * ffn_src = falcon ? m->x : m->ffn_inp;
     PI_TRY(pi_k_sparse_ffn_logits_hot(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, d, ffn_src, &fn, m->hot_words[il], m->hot_prefix[il],
-                                      c->logits, m->pred_logits, c->x16_pin, m->ws, st));
+                                      nullptr, m->pred_logits, c->x16_pin, c->words_pin, m->ws, st));
     PI_TRY(pi_k_sparse_ffn_rows_hot(ff, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, down.dev, d, ffn_src, &fn, m->hot_words[il], m->hot_prefix[il],
                                     m->pred_logits, nullptr, c->d_seq, c->flags, m->ws, st));             // its first lane starts the hand-over
     PI_TRY(pi_k_host_wait(c->d_seq, c->flags, 32, c->d_status, limit, st));

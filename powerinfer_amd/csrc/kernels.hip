@@ -993,7 +993,7 @@ __device__ __forceinline__ int select_nth_bit(uint32_t bits, int n);
 // PHASE 1 / 2 (G == 1) cut the launch in two for a hybrid layer whose host share should start behind the predictor: 1 stops after the
 // logits (to `logits` and `logits2`), the mask words and the fp16 input for the host; 2 reads the logits back from `logits2`.
 // a hand-over to the host announced by the first lane of a launch (see host_signal_kernel): device counter and word 0 of the pinned flags
-struct HostAnnounce { uint32_t * seq; uint32_t * flags; };
+struct HostAnnounce { uint32_t * seq; uint32_t * flags; uint32_t * words_out = nullptr; };    // words_out: a second copy of the activity words (pinned memory) for the logits-only launch
 
 template <int CPW, int RCH, bool GATE, int G, bool HYB, int PHASE = 0>      // cols == 8 waves * CPW chunks * 512; r == RCH * 512; G groups of 32 neurons
 __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
@@ -1175,7 +1175,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
             if (PHASE == 1) logits2[n0 + lane] = my_logit;
             if (PHASE != 1 && h_dense && !((mask >> lane) & 1u)) h_dense[n0 + lane] = 0.0f;
         }
-        if (lane == 0) { words[blockIdx.x * G + g] = all; if (HYB) words_hot[blockIdx.x * G + g] = mask; }
+        if (lane == 0) { words[blockIdx.x * G + g] = all; if (HYB) words_hot[blockIdx.x * G + g] = mask; if (PHASE == 1 && ann.words_out) ann.words_out[blockIdx.x * G + g] = all; }
     }
     if (PHASE == 1) return;
     // ---- B + C ---------------------------------------------------------------------------------------------
@@ -4047,14 +4047,14 @@ int pi_k_sparse_ffn_two_phase_supported(int ff, int r, int cols) { return pi_k_s
 
 int pi_k_sparse_ffn_logits_hot(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
                                const uint32_t * hot_words, const int32_t * hot_prefix, float * logits, float * logits_dev, void * xn_f16_out,
-                               pi_workspace * ws, pi_stream_t stream) {
+                               uint32_t * words_out, pi_workspace * ws, pi_stream_t stream) {
     if (!fc2_f16 || !hidden || !x || !hot_words || !hot_prefix || !logits_dev || !ws) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_logits_hot: null pointer");
     if (!pi_k_sparse_ffn_two_phase_supported(ff, r, cols) || ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn_logits_hot: cols must be 4096, r 512 or 1024, ff % 32 == 0, within the workspace");
     const NormArgs na = to_norm(norm);
     if ((((uintptr_t)hidden | (uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b | (uintptr_t)xn_f16_out) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_logits_hot: vectors must be 16-byte aligned");
     const dim3 grid(ff / 32), block(kPfBlock);
     const __half * none = nullptr;
-#define PI_PF1(RCH) hipLaunchKernelGGL((pred_ffn_f16_kernel<1, RCH, false, 1, true, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, x, na, threshold, logits, ws->words, (float *)nullptr, (float *)nullptr, hot_words, hot_prefix, ws->words_hot, (__half *)xn_f16_out, logits_dev, HostAnnounce{nullptr, nullptr})
+#define PI_PF1(RCH) hipLaunchKernelGGL((pred_ffn_f16_kernel<1, RCH, false, 1, true, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, x, na, threshold, logits, ws->words, (float *)nullptr, (float *)nullptr, hot_words, hot_prefix, ws->words_hot, (__half *)xn_f16_out, logits_dev, HostAnnounce{nullptr, nullptr, words_out})
     if (r == 1024) PI_PF1(2); else PI_PF1(1);
 #undef PI_PF1
     return pi::check_launch("pi_k_sparse_ffn_logits_hot");

@@ -89,7 +89,7 @@ _SIGS = {
     "pi_k_embed_batch_q4": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
     "pi_k_host_signal": (_i, [_vp, _vp, _i, _i, _vp]),
     "pi_k_sparse_ffn_two_phase_supported": (_i, [_i, _i, _i]),
-    "pi_k_sparse_ffn_logits_hot": (_i, [_vp, _i, _i, _vp, _f, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_sparse_ffn_logits_hot": (_i, [_vp, _i, _i, _vp, _f, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_rows_hot": (_i, [_i, _f, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_q4_partials": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_q4_reduce": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),

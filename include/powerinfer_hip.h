@@ -511,7 +511,7 @@ PI_API int pi_model_decode(pi_model * m, const int32_t * tokens, int n_tokens, i
 /*
  * The batch-1 greedy token loop of examples/main (main.cpp:462-623 with temp == 0): continues from the
  * state pi_model_decode left (next token = its greedy choice), generates n_steps tokens entirely on the
- * device (captured HIP graphs of eight tokens and of one token, replayed) and writes them to out_tokens (host).
+ * device (one captured HIP graph replayed per token) and writes them to out_tokens (host).
  * ms_out (optional) receives the device time of the loop measured with events on the model's stream.
  */
 PI_API int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, float * ms_out);

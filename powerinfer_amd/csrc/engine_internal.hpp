@@ -43,8 +43,6 @@ struct pi_model {
 
     hipGraphExec_t graph_exec = nullptr;
     hipGraph_t graph = nullptr;
-    hipGraphExec_t graph_exec_k = nullptr;   // the same token loop, kGraphTokens tokens per replay (tokens and positions advance on the device)
-    hipGraph_t graph_k = nullptr;
     hipEvent_t ev0 = nullptr, ev1 = nullptr;
 
     bool building_graph = false;          // token_forward is being recorded into a graph, not run

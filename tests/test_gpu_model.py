@@ -437,10 +437,10 @@ def test_vram_budget_split_matches_all_cold_oracle():
 
 
 @pytest.mark.parametrize("arch,wtype,n_layer", [("llama-tiny", synth.F16, 3), ("falcon-tiny", synth.Q4_0, 2), ("llama-7b", synth.F16, 3)])
-def test_generate_replays_of_several_tokens_match_single_token_calls(arch, wtype, n_layer):
-    """A generate call replays graphs that hold several tokens each (and single-token graphs for the remainder); tokens, positions
-    and the layer buffers' roles carry from one replay to the next on the device.  The same launches one token per call: tokens
-    and the logits after the last one are bit-identical, over call lengths that mix both graphs, with an odd layer count too."""
+def test_generate_replays_match_single_token_calls(arch, wtype, n_layer):
+    """A generate call replays one captured token per step; tokens, positions and the layer buffers' roles carry from one replay to
+    the next on the device.  The same launches one token per call: tokens and the logits after the last one are bit-identical, over
+    several calls, with an odd layer count too."""
     from powerinfer_amd.model import Model
     hp = synth.hparams(arch, n_layer=n_layer, n_ctx=96, seed=31, wtype=wtype)
     model = synth.make_model(hp)
@@ -449,7 +449,7 @@ def test_generate_replays_of_several_tokens_match_single_token_calls(arch, wtype
     tok_a, _ = ga.decode(prompt, 0)
     tok_b, _ = gb.decode(prompt, 0)
     assert tok_a == tok_b
-    toks = [int(t) for n in (21, 3, 16, 9) for t in ga.generate(n)[0]]            # 8+8+5, 3, 8+8, 8+1
+    toks = [int(t) for n in (21, 3, 16, 9) for t in ga.generate(n)[0]]
     n_past, cur, single = len(prompt), int(tok_b), []
     for _ in range(len(toks)):
         cur, lg_b = gb.decode([cur], n_past)

@@ -1596,7 +1596,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
 // waves each add their 512-column slice of those rows: acc += float((nibble - 8) * q) * (d_w * d_h), one fp32 multiply and
 // one fp32 add per element (ggml_axpy_q4_0_q8_0, ggml-quants.c:2426-2509), rows in ascending order.  One partial vector per
 // workgroup goes to `partial`; ffn_reduce_kernel adds them in workgroup order.
-constexpr int kAqGroups = 4;
+constexpr int kAqGroups = 1;               // the launch is all latency: more, smaller workgroups finish sooner (4 -> 1: 12.8 us -> about 9 per 7B layer)
 constexpr int kAqN = kAqGroups * 32;       // neurons per workgroup
 constexpr int kAqChunk = 16;               // rows in flight per wave
 
@@ -1618,8 +1618,9 @@ __global__ __launch_bounds__(kPfBlock, 2) void axpy_q4_groups_kernel(const pi_bl
     if (wave == 0) {
         int cnt = 0;
 #pragma unroll
-        for (int i = 0; i < kAqN / 64; ++i) {
-            const int nrn = n0 + i * 64 + lane;
+        for (int i = 0; i < (kAqN + 63) / 64; ++i) {
+            const bool mine = i * 64 + lane < kAqN;                  // kAqN == 32: the upper half of the wave idles
+            const int nrn = mine ? n0 + i * 64 + lane : ff;
             const float hvv = nrn < ff ? h[nrn] : 0.0f;
             float amax = fabsf(hvv);
 #pragma unroll

@@ -108,6 +108,7 @@ def build_synthetic_on_device(hp, keep):
             bias = pl.DevBuf(host=b)
             fc2 = normal(ff, r, bias, f16=True)
         put(il, "fc2", fc2, ff, r, f16=True)
+        m.set_tensor(il, "neuron_rate", p.astype(np.float32))      # the activation statistics the split planner works from
         if hybrid:
             gi, gb = synth.gpu_split(p, hp.hot_frac)
             m.set_tensor(il, "gpu_idx", gi)

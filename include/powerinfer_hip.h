@@ -207,6 +207,10 @@ PI_API int pi_k_axpy_q4_partials_split(const void * down_t_q4, const void * down
 PI_API int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float theta_scale, float freq_scale, const int32_t * delta, int n_cells, pi_stream_t stream);
 PI_API int pi_k_kv_compact(void * cache, void * stage, int rows, int n_ctx, int hd, const int32_t * map, int n_new, pi_stream_t stream);
 PI_API int pi_k_sparse_ffn_supported(int ff, int r, int cols);
+/* Workgroups of the fused launch for a layer that is whole on the device (0: shape not covered).  Workgroup b computes neurons
+ * [ff * b / n, ff * (b + 1) / n) and stores one partial output vector; a caller that arranges a layer's rows by firing rate deals
+ * them out over these ranges (pi_model_finalize does, from PI_T_NEURON_RATE). */
+PI_API int pi_k_sparse_ffn_workgroups(int ff, int r, int cols);
 /* the two launches of pi_k_sparse_ffn on their own, for callers that overlap the block with an independent branch (Falcon's
  * attention reads the same layer input): _partials may run on another stream, _reduce needs it and the residual operands done */
 PI_API int pi_k_sparse_ffn_partials(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
@@ -467,6 +471,7 @@ enum {
     PI_T_WQ, PI_T_WK, PI_T_WV, PI_T_WQKV, PI_T_WO,
     PI_T_FFN_NORM, PI_T_FFN_GATE, PI_T_FFN_UP, PI_T_FFN_DOWN_T,
     PI_T_FC1, PI_T_FC2, PI_T_GPU_IDX, PI_T_GPU_BUCKET,
+    PI_T_NEURON_RATE,
     PI_T_COUNT
 };
 
@@ -484,6 +489,13 @@ PI_API void       pi_model_free(pi_model * m);
  * FFN matrices of a layer that has a PI_T_GPU_BUCKET are given FULL-SIZE on the host: the bucket's rows are
  * sliced into compact device matrices (slice_ffn_mat_to_gpu, llama.cpp:2898-2967) and the host copy is
  * kept (borrowed, must outlive the model) for the cold neurons that run on the CPU.
+ * PI_T_NEURON_RATE (optional, host, F32 [n_ff], copied): each neuron's firing rate, the activation statistics the reference's offline
+ * solver places neurons with (powerinfer-py/powerinfer/solver.py:8-100, export_split.py:24-52).  For an F16 layer that is whole on
+ * the device and that the fused kernel covers, pi_model_finalize then deals the neurons out by rate over the 32-neuron groups of that
+ * kernel (group g, slot j holds the neuron of rank j * n_ff / 32 + g; fc2 / gate / up / down_t rows are moved alike into storage the
+ * model owns) so that every workgroup of that kernel carries the same expected number of active rows.  Results are those of the file
+ * order up to the order of the fp32 sums over neurons; everything the model reports per neuron (pi_model_get_capture) stays in file
+ * order.
  */
 PI_API int pi_model_set_tensor(pi_model * m, int layer, int kind, int type, const void * data,
                                int64_t ne0, int64_t ne1, int on_device);

@@ -14,6 +14,7 @@
 #include <stdlib.h>
 #include <string.h>
 
+#include <algorithm>
 #include <utility>
 #include <vector>
 
@@ -90,6 +91,14 @@ __global__ __launch_bounds__(1024) void argmax_advance_kernel(const float * __re
     }
 }
 
+// dst row i = src row perm[i]; rows of row_bytes (a multiple of 16) bytes, one workgroup per row
+__global__ __launch_bounds__(256) void gather_rows_kernel(const unsigned char * __restrict__ src, unsigned char * __restrict__ dst,
+                                                          const int32_t * __restrict__ perm, size_t row_bytes) {
+    const uint4 * s = reinterpret_cast<const uint4 *>(src + (size_t)perm[blockIdx.x] * row_bytes);
+    uint4 * d = reinterpret_cast<uint4 *>(dst + (size_t)blockIdx.x * row_bytes);
+    for (size_t i = threadIdx.x; i < row_bytes / 16; i += blockDim.x) d[i] = s[i];
+}
+
 __global__ void add_vec_kernel(float * __restrict__ y, const float * __restrict__ a, int n) {
     const int i = blockIdx.x * blockDim.x + threadIdx.x;
     if (i < n) y[i] = __fadd_rn(y[i], a[i]);
@@ -151,7 +160,7 @@ int layer_forward(pi_model * m, int il, bool last_token) {
         PI_HIP_TRY(hipStreamWaitEvent(m->stream2, m->ev_fork[il], 0));
         PI_TRY(pi_k_gemv(fc1.type, fc1.dev, r, d, x, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, m->stream2));
         PI_TRY(pi_k_sparse_ffn_partials(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, nullptr, down.dev, d, x, &fnb,
-                                        nullptr, nullptr, m->ws, m->stream2));
+                                               nullptr, nullptr, m->ws, m->stream2));
     }
 
     // attention
@@ -198,7 +207,7 @@ int layer_forward(pi_model * m, int il, bool last_token) {
         if (m->capture && last_token) {
             float * ffo = m->cap_ffn + (size_t)il * d;
             PI_TRY(pi_k_sparse_ffn(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, gp, down.dev, d, ffn_in, &fn,
-                                   PI_EPI_NONE, nullptr, nullptr, ffo, m->pred_logits, nullptr, n_act, m->ws, st));
+                                          PI_EPI_NONE, nullptr, nullptr, ffo, m->pred_logits, nullptr, n_act, m->ws, st));
             PI_HIP_TRY(hipMemcpyAsync(m->x2, ffo, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
             PI_TRY(pi::add_vec(m->x2, falcon ? m->attn_out : m->ffn_inp, d, st));
             if (falcon) PI_TRY(pi::add_vec(m->x2, x, d, st));
@@ -206,10 +215,10 @@ int layer_forward(pi_model * m, int il, bool last_token) {
             PI_HIP_TRY(hipMemcpyAsync(m->cap_src + (size_t)il * d, ffn_in, sizeof(float) * d, hipMemcpyDeviceToDevice, st));
         } else if (!falcon) {
             PI_TRY(pi_k_sparse_ffn(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, gp, down.dev, d, ffn_in, &fn,
-                                   PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, nullptr, nullptr, n_act, m->ws, st));
+                                          PI_EPI_ADD, m->ffn_inp, nullptr, m->x2, nullptr, nullptr, n_act, m->ws, st));
         } else {
             PI_TRY(pi_k_sparse_ffn(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, gp, down.dev, d, ffn_in, &fn,
-                                   PI_EPI_ADD2, m->attn_out, x, m->x2, nullptr, nullptr, n_act, m->ws, st));
+                                          PI_EPI_ADD2, m->attn_out, x, m->x2, nullptr, nullptr, n_act, m->ws, st));
         }
         std::swap(m->x, m->x2);
         return PI_OK;
@@ -454,11 +463,60 @@ int pi_model_set_tensor(pi_model * m, int layer, int kind, int type, const void 
         return PI_OK;
     }
     if (kind == PI_T_GPU_IDX) { t.type = type; t.ne0 = ne0; t.ne1 = ne1; t.host = data; return PI_OK; }   // host-only (cold path)
+    if (kind == PI_T_NEURON_RATE) {                                                                       // host-only, copied (finalize)
+        if (type != PI_TYPE_F32 || on_device || ne0 * ne1 != m->hp.n_ff) return pi::fail(PI_E_ARG, "pi_model_set_tensor: neuron rates are host F32 [n_ff]");
+        if (m->neuron_rate.empty()) m->neuron_rate.resize(m->hp.n_layer);
+        m->neuron_rate[layer].assign((const float *)data, (const float *)data + m->hp.n_ff);
+        return PI_OK;
+    }
     if (kind == PI_T_GPU_BUCKET) { t.host = data; }
     return upload_tensor(m, t, type, data, ne0, ne1, on_device);
 }
 
 }  // extern "C"
+
+namespace {
+// Deals the neurons of layer il out by firing rate over the workgroups of the fused F16 launch: the workgroup ranges take the neurons of
+// rank 0, 1, 2, ... in turn (first slot of every range, then the second, ...), so each range holds the same mix of busy and idle neurons
+// and every workgroup expects the same number of active rows.  fc2 / up / gate / down_t rows move alike into storage the model owns.
+int deal_neurons_by_rate(pi_model * m, int il) {
+    const pi_hparams & hp = m->hp;
+    const int d = hp.n_embd, ff = hp.n_ff;
+    const std::vector<float> & rate = m->neuron_rate[il];
+    Tensor & fc2 = m->L(il, PI_T_FC2); Tensor & up = m->L(il, PI_T_FFN_UP);
+    if (rate.empty() || m->L(il, PI_T_GPU_BUCKET).dev || up.type != PI_TYPE_F16 || fc2.type != PI_TYPE_F16) return PI_OK;
+    const int n_wg = pi_k_sparse_ffn_workgroups(ff, (int)fc2.ne0, d);
+    if (n_wg <= 0) return PI_OK;
+    std::vector<int32_t> order(ff);
+    for (int i = 0; i < ff; ++i) order[i] = i;
+    std::stable_sort(order.begin(), order.end(), [&](int32_t a, int32_t b) { return rate[a] > rate[b]; });
+    std::vector<int32_t> & perm = m->ffn_perm[il];
+    perm.resize(ff);
+    int next = 0;
+    for (int j = 0; next < ff; ++j)
+        for (int b = 0; b < n_wg; ++b) {
+            const int lo = (int)((long long)ff * b / n_wg), hi = (int)((long long)ff * (b + 1) / n_wg);
+            if (lo + j < hi) perm[lo + j] = order[next++];
+        }
+    int32_t * dperm = (int32_t *)pi_malloc(sizeof(int32_t) * ff);
+    if (!dperm) return PI_E_HIP;
+    int rc = pi_memcpy_h2d(dperm, perm.data(), sizeof(int32_t) * ff);
+    for (int k : {PI_T_FC2, PI_T_FFN_UP, PI_T_FFN_GATE, PI_T_FFN_DOWN_T}) {
+        Tensor & t = m->L(il, k);
+        if (rc != PI_OK || !t.dev) continue;                    // Falcon has no gate
+        const size_t rb = row_bytes(t.type, t.ne0);
+        unsigned char * moved = m->alloc<unsigned char>(rb * (size_t)ff);
+        if (!moved) { rc = PI_E_HIP; break; }
+        hipLaunchKernelGGL(gather_rows_kernel, dim3(ff), dim3(256), 0, nullptr, (const unsigned char *)t.dev, moved, dperm, rb);
+        rc = pi::check_launch("gather_rows");
+        if (rc == PI_OK && hipDeviceSynchronize() != hipSuccess) rc = pi::fail(PI_E_HIP, "gather_rows: device error");
+        if (t.owned) for (auto & o : m->owned) if (o == t.dev) { pi_free(o); o = nullptr; }
+        t.dev = moved; t.owned = true;
+    }
+    pi_free(dperm);
+    return rc;
+}
+}  // namespace
 
 namespace pi {
 // the up / gate / down rows of layer il's non-resident neurons, in ascending neuron order, in pinned host memory that kernels read directly
@@ -600,6 +658,10 @@ int pi_model_finalize(pi_model * m) {
             PI_TRY(pi_memcpy_h2d(m->hot_prefix[il], prefix.data(), sizeof(int32_t) * prefix.size()));
         }
     }
+
+    // neurons dealt out by firing rate for the fused F16 kernel (see PI_T_NEURON_RATE)
+    m->ffn_perm.assign(hp.n_layer, {});
+    for (int il = 0; il < hp.n_layer && !m->neuron_rate.empty(); ++il) PI_TRY(deal_neurons_by_rate(m, il));
 
     // non-resident rows the GPU is to read itself: gathered in ascending neuron order into pinned host memory
     m->rest_up.assign(hp.n_layer, nullptr); m->rest_gate.assign(hp.n_layer, nullptr); m->rest_down.assign(hp.n_layer, nullptr);
@@ -802,7 +864,7 @@ int pi_model_time_section(pi_model * m, int section, int rounds, float * ms_tota
                 PI_TRY(pi_k_gemv(fc1.type, fc1.dev, (int)fc1.ne1, d, fin, nullptr, PI_EPI_RELU, nullptr, nullptr, m->hidden, st));
                 if (!q4 && pi_k_sparse_ffn_supported(ff, (int)fc1.ne1, d)) {
                     PI_TRY(pi_k_sparse_ffn(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, down.dev, d,
-                                           fin, &fn, PI_EPI_ADD, fin, nullptr, m->x2, nullptr, nullptr, m->n_active + il, m->ws, st));
+                                                  fin, &fn, PI_EPI_ADD, fin, nullptr, m->x2, nullptr, nullptr, m->n_active + il, m->ws, st));
                     ++n;
                     continue;
                 }
@@ -831,7 +893,7 @@ int pi_model_time_section(pi_model * m, int section, int rounds, float * ms_tota
                 const float * fin = falcon ? m->x : m->ffn_inp;
                 if (section == 3)
                     PI_TRY(pi_k_sparse_ffn_partials(fc2.dev, ff, (int)fc1.ne1, m->hidden, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, down.dev, d,
-                                                    fin, &fn, nullptr, nullptr, m->ws, st));
+                                                           fin, &fn, nullptr, nullptr, m->ws, st));
                 else
                     PI_TRY(pi_k_sparse_ffn_reduce(ff, d, PI_EPI_ADD, fin, nullptr, m->x2, m->n_active + il, m->ws, st));
                 ++n;
@@ -864,7 +926,18 @@ int pi_model_get_capture(pi_model * m, float * ffn_out, float * pred_logits, int
     if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_get_capture: model not finalized");
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
     if (ffn_out) PI_TRY(pi_memcpy_d2h(ffn_out, m->cap_ffn, sizeof(float) * (size_t)m->hp.n_layer * m->hp.n_embd));
-    if (pred_logits) PI_TRY(pi_memcpy_d2h(pred_logits, m->cap_logits, sizeof(float) * (size_t)m->hp.n_layer * m->hp.n_ff));
+    if (pred_logits) {
+        PI_TRY(pi_memcpy_d2h(pred_logits, m->cap_logits, sizeof(float) * (size_t)m->hp.n_layer * m->hp.n_ff));
+        // layers whose neurons were dealt out by rate computed their logits in that order: hand them back in file order
+        std::vector<float> tmp;
+        for (int il = 0; il < m->hp.n_layer; ++il) {
+            const std::vector<int32_t> & perm = m->ffn_perm[il];
+            if (perm.empty()) continue;
+            float * row = pred_logits + (size_t)il * m->hp.n_ff;
+            tmp.assign(row, row + m->hp.n_ff);
+            for (int i = 0; i < m->hp.n_ff; ++i) row[perm[i]] = tmp[i];
+        }
+    }
     if (n_active) PI_TRY(pi_memcpy_d2h(n_active, m->n_active, sizeof(int32_t) * m->hp.n_layer));
     if (ffn_src) PI_TRY(pi_memcpy_d2h(ffn_src, m->cap_src, sizeof(float) * (size_t)m->hp.n_layer * m->hp.n_embd));
     return PI_OK;

@@ -59,6 +59,9 @@ struct pi_model {
     bool rest_on_gpu = false;
     std::vector<void *> rest_up, rest_gate, rest_down;
     std::vector<void *> pinned;           // hipHostMalloc allocations owned by the model
+    // layers whose neurons were dealt out by firing rate (PI_T_NEURON_RATE): position -> neuron of the file; empty: file order
+    std::vector<std::vector<float>>   neuron_rate;     // per layer, as given (empty: none)
+    std::vector<std::vector<int32_t>> ffn_perm;
     BatchState * batch = nullptr;         // per-sequence caches and step buffers of batched decoding
     BatchState * prefill = nullptr;       // step buffers for prompt chunks of the model's own sequence
     BatchState * prefill_wide = nullptr;  // the same for chunks of up to 512 tokens (dense mat-muls, weights read once per chunk)

@@ -1239,50 +1239,255 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_ffn_f16_kernel(const __half 
     }
 }
 
-// out[c] = epi( sum over workgroups b (ascending within a fixed tree) of partial[b][c] ).  A workgroup of 8 waves owns
-// 64 columns: 16 lanes x float4 cover them, the four 16-lane groups of a wave and the 8 waves split the rows of the
-// partial matrix; groups merge by DPP-free shuffles, waves through LDS in wave order.  Workgroup 0 also counts the
+// ---------------------------------------------------------------------------------------------------
+// The same block with the neurons spread evenly over the compute units (F16, cols == 4096, every neuron on the device).
+// What bounds a launch of this kind is the compute unit that has to pull the most bytes: a unit sustains about 1/256 of the
+// chip's HBM rate whatever it has in flight, so with ff / 32 workgroups of 32 neurons (344 on 256 units at ff 11008) the 88
+// units that hold two workgroups set the pace and the others idle.  Here the grid is one workgroup per unit and workgroup b
+// owns neurons [ff * b / n, ff * (b + 1) / n): up to 64 of them, so that one 64-lane ballot yields the activity mask.
+//   A  wave w computes the predictor logits of neurons w, w + 8, ... of the range (fc2 rows, r == 512 * RCH) and loads its
+//      eighth of the FFN input and norm weights; statistics and logits cross the waves through LDS.
+//   B  every wave derives the same 64-bit mask and loads ITS 512-column slice of the gate, up and down rows of up to
+//      kCuChunk active neurons at once; partial gate / up dots cross the waves through LDS; h = relu(g) * u.
+//   C  partial[b][512 w + 8 lane ..] += fp16(h) * down slice; one store per workgroup; ffn_reduce_kernel adds the n vectors.
+// A workgroup may use the whole register file of its unit (one workgroup per unit), which is what lets twelve active
+// neurons travel at once.  Logits and sums are those of pred_ffn_f16_kernel for the same rows.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kCuChunk = 12;
+
+__device__ __forceinline__ int select_nth_bit64(uint64_t bits, int n) {      // index of the n-th (0-based) set bit
+    for (int i = 0; i < n; ++i) bits &= bits - 1;
+    return __ffsll((unsigned long long)bits) - 1;
+}
+
+// KIND: 0 no norm, 1 RMSNorm * w, 2 LayerNorm * w + b (the launcher checks that the operands are there).  Every load of phase A is
+// unconditional - a wave without an ROWS-th row of its own requests the range's last row again, which its unit already has on the way -
+// because the compiler counts outstanding loads conservatively across branches and would otherwise hold the norm statistics back
+// until the last predictor row has landed.
+template <int RCH, bool GATE, int ROWS, int KIND>      // r == RCH * 512; ROWS fc2 rows per wave: at most 8 * ROWS neurons per workgroup
+__global__ __launch_bounds__(kPfBlock, 1) void ffn_cu_f16_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
+                                                                 const __half * __restrict__ Wup, const __half * __restrict__ Wgate,
+                                                                 const __half * __restrict__ Wdown,
+                                                                 const float * __restrict__ x, const float * __restrict__ nw, const float * __restrict__ nb, float eps,
+                                                                 float thr, int ff,
+                                                                 float * __restrict__ logits, uint32_t * __restrict__ words, float * __restrict__ h_dense,
+                                                                 float * __restrict__ partial) {
+    constexpr int cols = kPfWaves * 512, r = RCH * 512, CH = kCuChunk;
+    __shared__ float  lg[64];
+    __shared__ double red[2][kPfWaves];
+    __shared__ float  part[kPfWaves][CH][2];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n0 = (int)((long long)ff * blockIdx.x / gridDim.x);
+    const int np = (int)((long long)ff * (blockIdx.x + 1) / gridDim.x) - n0;       // <= 8 * ROWS <= 64 (the launcher's test)
+    const int cbase = wave * 512 + lane * 8;
+
+    // ---- A: loads.  Memory returns a wave's loads in the order it issued them: the small operands go first, so that the norm
+    // statistics, their exchange and the division run while the predictor rows are still on their way, and only the dot products
+    // and one barrier lie between the last predictor row and the first gate / up / down request. ------------------------------
+    float xs[8], ws[8], bs[8];
+    {
+        const float4 x0 = *reinterpret_cast<const float4 *>(x + cbase), x1 = *reinterpret_cast<const float4 *>(x + cbase + 4);
+        xs[0] = x0.x; xs[1] = x0.y; xs[2] = x0.z; xs[3] = x0.w; xs[4] = x1.x; xs[5] = x1.y; xs[6] = x1.z; xs[7] = x1.w;
+        if (KIND >= 1) {
+            const float4 w0 = *reinterpret_cast<const float4 *>(nw + cbase), w1 = *reinterpret_cast<const float4 *>(nw + cbase + 4);
+            ws[0] = w0.x; ws[1] = w0.y; ws[2] = w0.z; ws[3] = w0.w; ws[4] = w1.x; ws[5] = w1.y; ws[6] = w1.z; ws[7] = w1.w;
+        }
+        if (KIND == 2) {
+            const float4 b0 = *reinterpret_cast<const float4 *>(nb + cbase), b1 = *reinterpret_cast<const float4 *>(nb + cbase + 4);
+            bs[0] = b0.x; bs[1] = b0.y; bs[2] = b0.z; bs[3] = b0.w; bs[4] = b1.x; bs[5] = b1.y; bs[6] = b1.z; bs[7] = b1.w;
+        }
+    }
+    float4 hv[RCH][2];
+#pragma unroll
+    for (int j = 0; j < RCH; ++j) {
+        hv[j][0] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8);
+        hv[j][1] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8 + 4);
+    }
+    pi_u32x4 a[ROWS][RCH];
+#pragma unroll
+    for (int i = 0; i < ROWS; ++i) {
+        const int row = wave + 8 * i < np ? wave + 8 * i : np - 1;
+#pragma unroll
+        for (int j = 0; j < RCH; ++j) a[i][j] = pi_ld_stream(W2 + (size_t)(n0 + row) * r + (j * PI_WAVE + lane) * 8);
+    }
+    // ---- A: norm statistics across the 8 slices ---------------------------------------------------------------
+    float mean = 0.0f, scale = 1.0f;
+    if (KIND == 1) {
+        double sq = 0.0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) sq += (double)__fmul_rn(xs[k], xs[k]);
+        sq = pi_wave_sum_f64(sq);
+        if (lane == 0) red[0][wave] = sq;
+        __syncthreads();
+        double t = 0.0;
+#pragma unroll
+        for (int w = 0; w < kPfWaves; ++w) t += red[0][w];
+        scale = pi_inv_sqrt((float)(t / cols) + eps);
+    } else if (KIND == 2) {
+        double sm = 0.0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) sm += (double)xs[k];
+        sm = pi_wave_sum_f64(sm);
+        if (lane == 0) red[0][wave] = sm;
+        __syncthreads();
+        double t = 0.0;
+#pragma unroll
+        for (int w = 0; w < kPfWaves; ++w) t += red[0][w];
+        mean = (float)(t / cols);
+        double sq = 0.0;
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { const float v = __fsub_rn(xs[k], mean); sq += (double)__fmul_rn(v, v); }
+        sq = pi_wave_sum_f64(sq);
+        if (lane == 0) red[1][wave] = sq;
+        __syncthreads();
+        double t2 = 0.0;
+#pragma unroll
+        for (int w = 0; w < kPfWaves; ++w) t2 += red[1][w];
+        scale = pi_inv_sqrt((float)(t2 / cols) + eps);
+    }
+    pi_u32x4 xr;
+    {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            float v = xs[k];
+            if (KIND >= 1) v = __fmul_rn(__fmul_rn(KIND == 2 ? __fsub_rn(v, mean) : v, scale), ws[k]);
+            if (KIND == 2) v = __fadd_rn(v, bs[k]);
+            xs[k] = v;
+        }
+        __half2 hh[4] = {__floats2half2_rn(xs[0], xs[1]), __floats2half2_rn(xs[2], xs[3]),
+                         __floats2half2_rn(xs[4], xs[5]), __floats2half2_rn(xs[6], xs[7])};
+        xr = *reinterpret_cast<const pi_u32x4 *>(hh);
+    }
+    // ---- A: logits (the CPU path rounds the hidden vector to fp16 before the dot, ggml.c:9703-9716) ------------
+    {
+        pi_u32x4 hr[RCH];
+#pragma unroll
+        for (int j = 0; j < RCH; ++j) {
+            __half2 hh[4] = {__floats2half2_rn(hv[j][0].x, hv[j][0].y), __floats2half2_rn(hv[j][0].z, hv[j][0].w),
+                             __floats2half2_rn(hv[j][1].x, hv[j][1].y), __floats2half2_rn(hv[j][1].z, hv[j][1].w)};
+            hr[j] = *reinterpret_cast<const pi_u32x4 *>(hh);
+        }
+#pragma unroll
+        for (int i = 0; i < ROWS; ++i) {
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < RCH; ++j) acc = pi_dot8h(a[i][j], hr[j], acc);
+            acc = pi_wave_sum(acc);
+            if (lane == 0 && wave + 8 * i < np) lg[wave + 8 * i] = acc;
+        }
+    }
+    __syncthreads();
+    // ---- activity mask (identical in every wave; lg[] is complete after the barrier above) -----------------------
+    const float my_logit = lane < np ? lg[lane] : 0.0f;
+    const bool my_act = lane < np && !(my_logit < thr);
+    const uint64_t mask = (uint64_t)__ballot(my_act);
+    if (wave == 0) {
+        if (lane < np) {
+            if (logits) logits[n0 + lane] = my_logit;
+            if (h_dense && !my_act) h_dense[n0 + lane] = 0.0f;
+        }
+        if (lane == 0) { words[2 * blockIdx.x] = (uint32_t)mask; words[2 * blockIdx.x + 1] = (uint32_t)(mask >> 32); }
+    }
+    // ---- B + C ---------------------------------------------------------------------------------------------
+    float acc[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) acc[k] = 0.0f;
+    const int n = __popcll((unsigned long long)mask);
+    for (int c0 = 0; c0 < n; c0 += CH) {
+        const int nn = n - c0 < CH ? n - c0 : CH;
+        int rows[CH];
+        pi_u32x4 gu[CH], uu[CH], dd[CH];
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            if (j < nn) {
+                rows[j] = n0 + select_nth_bit64(mask, c0 + j);
+                const size_t off = (size_t)rows[j] * cols + cbase;
+                uu[j] = pi_ld_stream(Wup + off);
+                if (GATE) gu[j] = pi_ld_stream(Wgate + off);
+                dd[j] = pi_ld_stream(Wdown + off);
+            }
+        }
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            if (j < nn) {
+                float pu = pi_dot8h(uu[j], xr, 0.0f), pg = 0.0f;
+                if (GATE) pg = pi_dot8h(gu[j], xr, 0.0f);
+                pu = pi_wave_sum(pu);
+                if (GATE) pg = pi_wave_sum(pg);
+                if (lane == 0) { part[wave][j][0] = pu; part[wave][j][1] = pg; }
+            }
+        }
+        __syncthreads();
+#pragma unroll
+        for (int j = 0; j < CH; ++j) {
+            if (j < nn) {
+                float u = 0.0f, g = 0.0f;
+#pragma unroll
+                for (int w = 0; w < kPfWaves; ++w) { u += part[w][j][0]; if (GATE) g += part[w][j][1]; }
+                const float h = GATE ? __fmul_rn(fmaxf(g, 0.0f), u) : fmaxf(u, 0.0f);
+                if (h_dense && threadIdx.x == 0) h_dense[rows[j]] = h;
+                const float hq = pi_round_f16(h);                 // the CPU axpy rounds h to fp16 (ggml.c:14420-14431)
+                float wf[8];
+                pi_unpack8(dd[j], wf);
+#pragma unroll
+                for (int k = 0; k < 8; ++k) acc[k] = fmaf(wf[k], hq, acc[k]);
+            }
+        }
+        if (c0 + CH < n) __syncthreads();                         // part[] is reused by the next chunk
+    }
+    float4 * po = reinterpret_cast<float4 *>(partial + (size_t)blockIdx.x * cols + cbase);
+    po[0] = make_float4(acc[0], acc[1], acc[2], acc[3]);
+    po[1] = make_float4(acc[4], acc[5], acc[6], acc[7]);
+}
+
+// out[c] = epi( sum over workgroups b (within a fixed tree) of partial[b][c] ).  A workgroup of 8 waves owns kFrCols = 32
+// columns, one 128-byte line of every partial vector: 8 lanes x float4 cover them, the eight 8-lane groups of a wave and the
+// 8 waves split the rows of the partial matrix (64 rows per pass, all of a thread's rows requested at once); groups merge by
+// shuffles, waves through LDS in wave order.  cols / 32 workgroups: a compute unit sustains only about 1/256 of the chip's
+// HBM rate, so the partial matrix has to be spread over as many units as 128-byte lines allow.  Workgroup 0 also counts the
 // predictor's active neurons from the mask words.
-constexpr int kFrUn = 12;
+constexpr int kFrUn = 6, kFrCols = 32;
 __global__ __launch_bounds__(kPfBlock) void ffn_reduce_kernel(const float * __restrict__ partial, int n_part, int cols,
                                                               const uint32_t * __restrict__ words, int n_words, int32_t * __restrict__ n_active_out,
                                                               int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ out) {
-    __shared__ float redl[kPfWaves][64];
+    __shared__ float redl[kPfWaves][kFrCols];
     __shared__ int   sred[kPfWaves];
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const int sub = lane >> 4, col = blockIdx.x * 64 + (lane & 15) * 4;
+    const int sub = lane >> 3, col = blockIdx.x * kFrCols + (lane & 7) * 4;
     // the residual operands and the mask words do not depend on anything computed here: fetch them first
     float r1 = 0.0f, r2 = 0.0f;
-    if (tid < 64) {
-        if (epi >= PI_EPI_ADD) r1 = add1[blockIdx.x * 64 + tid];
-        if (epi == PI_EPI_ADD2) r2 = add2[blockIdx.x * 64 + tid];
+    if (tid < kFrCols) {
+        if (epi >= PI_EPI_ADD) r1 = add1[blockIdx.x * kFrCols + tid];
+        if (epi == PI_EPI_ADD2) r2 = add2[blockIdx.x * kFrCols + tid];
     }
     int cnt = 0;
     if (blockIdx.x == 0 && n_active_out)
         for (int w = tid; w < n_words; w += kPfBlock) cnt += __popc(words[w]);
     float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    for (int b0 = wave * 4 + sub; b0 < n_part; b0 += kPfWaves * 4 * kFrUn) {
+    for (int b0 = wave * 8 + sub; b0 < n_part; b0 += kPfWaves * 8 * kFrUn) {
         float4 v[kFrUn];
 #pragma unroll
         for (int u = 0; u < kFrUn; ++u) {
-            const int b = b0 + u * kPfWaves * 4;
+            const int b = b0 + u * kPfWaves * 8;
             v[u] = b < n_part ? *reinterpret_cast<const float4 *>(partial + (size_t)b * cols + col) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
         }
 #pragma unroll
         for (int u = 0; u < kFrUn; ++u) { acc.x += v[u].x; acc.y += v[u].y; acc.z += v[u].z; acc.w += v[u].w; }
     }
-    acc.x += __shfl_xor(acc.x, 16, PI_WAVE); acc.y += __shfl_xor(acc.y, 16, PI_WAVE); acc.z += __shfl_xor(acc.z, 16, PI_WAVE); acc.w += __shfl_xor(acc.w, 16, PI_WAVE);
-    acc.x += __shfl_xor(acc.x, 32, PI_WAVE); acc.y += __shfl_xor(acc.y, 32, PI_WAVE); acc.z += __shfl_xor(acc.z, 32, PI_WAVE); acc.w += __shfl_xor(acc.w, 32, PI_WAVE);
-    if (lane < 16) { redl[wave][lane * 4] = acc.x; redl[wave][lane * 4 + 1] = acc.y; redl[wave][lane * 4 + 2] = acc.z; redl[wave][lane * 4 + 3] = acc.w; }
+#pragma unroll
+    for (int o = 8; o < 64; o <<= 1) {
+        acc.x += __shfl_xor(acc.x, o, PI_WAVE); acc.y += __shfl_xor(acc.y, o, PI_WAVE); acc.z += __shfl_xor(acc.z, o, PI_WAVE); acc.w += __shfl_xor(acc.w, o, PI_WAVE);
+    }
+    if (lane < 8) { redl[wave][lane * 4] = acc.x; redl[wave][lane * 4 + 1] = acc.y; redl[wave][lane * 4 + 2] = acc.z; redl[wave][lane * 4 + 3] = acc.w; }
     if (blockIdx.x == 0 && n_active_out) { cnt = pi_wave_sum_i32(cnt); if (lane == 0) sred[wave] = cnt; }
     __syncthreads();
-    if (tid < 64) {
+    if (tid < kFrCols) {
         float sum = redl[0][tid];
 #pragma unroll
         for (int w = 1; w < kPfWaves; ++w) sum += redl[w][tid];
         if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, r1);
         else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, r1), r2);
-        out[blockIdx.x * 64 + tid] = sum;
+        out[blockIdx.x * kFrCols + tid] = sum;
     }
     if (blockIdx.x == 0 && n_active_out && tid == 0) { int t = 0; for (int w = 0; w < kPfWaves; ++w) t += sred[w]; *n_active_out = t; }
 }
@@ -3600,6 +3805,7 @@ struct pi_workspace {
     float *        ffn_partial;    // [max(max_ff/32, 32 * 16)][max_d]  partial outputs of the fused sparse FFN / of the batched axpy
     __half *       hc_batch;       // [16][max_ff + 16]  fp16 h of the union rows for a batched step, token-major
     unsigned char * row_any;       // [max_ff]  batched step: neuron active for at least one token
+    int            pf_parts, pf_words;   // partial vectors and activity words the last fused F16 launch left for its reduction
 };
 constexpr int kAxpyGroups = 32;
 
@@ -3609,7 +3815,8 @@ pi_workspace * pi_workspace_create(int max_ff, int max_d) {
     if (max_ff <= 0 || max_d <= 0 || (max_d + kAxpyTile - 1) / kAxpyTile > 62) { pi::set_error("pi_workspace_create: bad sizes"); return nullptr; }
     pi_workspace * ws = new pi_workspace{};
     ws->max_ff = max_ff; ws->max_d = max_d;
-    ws->words    = (uint32_t *)pi_malloc(sizeof(uint32_t) * (max_ff / 32 + 2));
+    const size_t n_words = (size_t)(max_ff / 32 + 2) > 2048 ? (size_t)(max_ff / 32 + 2) : 2048;       // groups of 32 neurons, or two words per compute unit
+    ws->words    = (uint32_t *)pi_malloc(sizeof(uint32_t) * n_words);
     ws->words_hot = (uint32_t *)pi_malloc(sizeof(uint32_t) * (max_ff / 32 + 2));
     ws->counters = (unsigned int *)pi_malloc(sizeof(unsigned int) * 64);
     ws->partial  = (float *)pi_malloc(sizeof(float) * (size_t)kAxpyGroups * max_d);
@@ -3897,7 +4104,7 @@ int pi_k_sparse_ffn_q4_reduce(int ff, int cols, int epilogue, const float * add1
     if (!out || !ws || cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_q4_reduce: bad arguments");
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
         return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_q4_reduce: bad epilogue arguments");
-    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, ff / 32, cols,
+    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / kFrCols), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, ff / 32, cols,
                        ws->words, ff / 32, n_active, epilogue, add1, add2, out);
     return pi::check_launch("pi_k_sparse_ffn_q4_reduce");
 }
@@ -3906,7 +4113,7 @@ int pi_k_sparse_ffn_q4_reduce_hot(int ff, int cols, int epilogue, const float * 
     if (!out || !ws || cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_q4_reduce_hot: bad arguments");
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
         return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_q4_reduce_hot: bad epilogue arguments");
-    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, ff / 32, cols,
+    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / kFrCols), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, ff / 32, cols,
                        ws->words_hot, ff / 32, n_active, epilogue, add1, add2, out);
     return pi::check_launch("pi_k_sparse_ffn_q4_reduce_hot");
 }
@@ -3970,7 +4177,7 @@ int pi_k_axpy_q4_reduce(int ff, int cols, int epilogue, const float * add1, cons
     if (!out || !ws || cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_axpy_q4_reduce: bad arguments");
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
         return pi::fail(PI_E_ARG, "pi_k_axpy_q4_reduce: bad epilogue arguments");
-    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, (ff + kAqN - 1) / kAqN, cols,
+    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / kFrCols), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, (ff + kAqN - 1) / kAqN, cols,
                        ws->words_hot, ff / 32, n_active, epilogue, add1, add2, out);
     return pi::check_launch("pi_k_axpy_q4_reduce");
 }
@@ -3989,6 +4196,8 @@ int pi_k_sparse_axpy_dense(const void * down_t_f16, int cols, int ff, const floa
 }
 
 int pi_k_sparse_ffn_supported(int ff, int r, int cols) { return (cols == 4096 || cols == 8192) && (r == 1024 || r == 512) && ff > 0 && ff % 32 == 0; }
+static int pf_parts(int ff, int cols, bool hyb);
+int pi_k_sparse_ffn_workgroups(int ff, int r, int cols) { return pi_k_sparse_ffn_supported(ff, r, cols) ? pf_parts(ff, cols, false) : 0; }
 
 // Groups of 32 neurons per workgroup of the fused sparse FFN.  Wide rows: a workgroup takes four groups in turn (the next
 // group's predictor rows travel during the current group's FFN rows) and stores one partial vector for all of them, which
@@ -3997,6 +4206,17 @@ static int pf_groups(int ff, int cols) {
     if (cols != 8192) return 1;                    // at 4096 columns one group per workgroup measured fastest
     return (ff % 128 == 0 && ff / 128 >= 256) ? 4 : 1;
 }
+
+// Workgroups of the one-per-compute-unit form (ffn_cu_f16_kernel), or 0 where the grouped form runs: 4096 columns, every neuron on
+// the device, and more than 32 but at most 64 neurons per unit (with 32 or fewer the groups of 32 already have a unit each).
+static int pf_cu_workgroups(int ff, int cols) {
+    if (cols != 4096) return 0;
+    const int n_cu = pi::compute_units();
+    if (n_cu <= 0 || ff <= 32 * n_cu || (ff + n_cu - 1) / n_cu > 64) return 0;
+    return n_cu;
+}
+// partial vectors the fused launch leaves for the reduction when nothing about the call rules the one-per-unit form out
+static int pf_parts(int ff, int cols, bool hyb) { const int n = hyb ? 0 : pf_cu_workgroups(ff, cols); return n ? n : ff / (32 * pf_groups(ff, cols)); }
 
 static int sparse_ffn_partials_impl(const char * who, const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
                                     const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x, const pi_norm * norm,
@@ -4011,9 +4231,25 @@ static int sparse_ffn_partials_impl(const char * who, const void * fc2_f16, int 
     hipStream_t st = (hipStream_t)stream;
     const __half * w2 = (const __half *)fc2_f16; const __half * u = (const __half *)up_f16; const __half * g = (const __half *)gate_f16;
     const __half * dn = (const __half *)down_t_f16;
+    const bool hyb = hot_words != nullptr;
+    // the one-workgroup-per-unit form takes the norm as a template parameter: it must carry what its kind needs
+    const bool cu_norm = na.kind == 0 || (na.kind == 1 && na.w && !na.b) || (na.kind == 2 && na.w && na.b);
+    if (const int n_wg = (hyb || !cu_norm) ? 0 : pf_cu_workgroups(ff, cols)) {
+        const int rows = ((ff + n_wg - 1) / n_wg + 7) / 8;              // fc2 rows per wave
+#define PI_CU_LAUNCH(RCH, GATE, ROWS, KIND) hipLaunchKernelGGL((ffn_cu_f16_kernel<RCH, GATE, ROWS, KIND>), dim3(n_wg), dim3(kPfBlock), 0, st, w2, hidden, u, g, dn, x, na.w, na.b, na.eps, threshold, ff, logits, ws->words, h_dense, ws->ffn_partial)
+#define PI_CU_KIND(RCH, GATE, ROWS) do { if (na.kind == 0) PI_CU_LAUNCH(RCH, GATE, ROWS, 0); else if (na.kind == 1) PI_CU_LAUNCH(RCH, GATE, ROWS, 1); else PI_CU_LAUNCH(RCH, GATE, ROWS, 2); } while (0)
+#define PI_CU_ROWS(RCH, GATE) do { if (rows <= 6) PI_CU_KIND(RCH, GATE, 6); else PI_CU_KIND(RCH, GATE, 8); } while (0)
+        if (r == 1024) { if (g) PI_CU_ROWS(2, true); else PI_CU_ROWS(2, false); }
+        else           { if (g) PI_CU_ROWS(1, true); else PI_CU_ROWS(1, false); }
+#undef PI_CU_ROWS
+#undef PI_CU_KIND
+#undef PI_CU_LAUNCH
+        ws->pf_parts = n_wg; ws->pf_words = 2 * n_wg;
+        return pi::check_launch(who);
+    }
+    ws->pf_parts = ff / (32 * pf_groups(ff, cols)); ws->pf_words = ff / 32;
     const int G = pf_groups(ff, cols);
     const dim3 grid(ff / (32 * G)), block(kPfBlock);
-    const bool hyb = hot_words != nullptr;
 #define PI_PF_LAUNCH2(CPW, RCH, GATE, GG, HYB) hipLaunchKernelGGL((pred_ffn_f16_kernel<CPW, RCH, GATE, GG, HYB>), grid, block, 0, st, w2, hidden, u, g, dn, x, na, threshold, logits, ws->words, h_dense, ws->ffn_partial, hot_words, hot_prefix, ws->words_hot, (__half *)xn_f16_out, nullptr, HostAnnounce{nullptr, nullptr})
 #define PI_PF_LAUNCH(CPW, RCH, GATE, GG) do { if (hyb) PI_PF_LAUNCH2(CPW, RCH, GATE, GG, true); else PI_PF_LAUNCH2(CPW, RCH, GATE, GG, false); } while (0)
 #define PI_PF_WIDE(RCH, GATE) do { if (G == 4) PI_PF_LAUNCH(2, RCH, GATE, 4); else if (G == 2) PI_PF_LAUNCH(2, RCH, GATE, 2); else PI_PF_LAUNCH(2, RCH, GATE, 1); } while (0)
@@ -4058,6 +4294,7 @@ int pi_k_sparse_ffn_logits_hot(const void * fc2_f16, int ff, int r, const float 
 #define PI_PF1(RCH) hipLaunchKernelGGL((pred_ffn_f16_kernel<1, RCH, false, 1, true, 1>), grid, block, 0, (hipStream_t)stream, (const __half *)fc2_f16, hidden, none, none, none, x, na, threshold, logits, ws->words, (float *)nullptr, (float *)nullptr, hot_words, hot_prefix, ws->words_hot, (__half *)xn_f16_out, logits_dev, HostAnnounce{nullptr, nullptr, words_out})
     if (r == 1024) PI_PF1(2); else PI_PF1(1);
 #undef PI_PF1
+    ws->pf_parts = ff / 32; ws->pf_words = ff / 32;
     return pi::check_launch("pi_k_sparse_ffn_logits_hot");
 }
 
@@ -4074,6 +4311,7 @@ int pi_k_sparse_ffn_rows_hot(int ff, float threshold, const void * up_f16, const
 #define PI_PF2(GATE) hipLaunchKernelGGL((pred_ffn_f16_kernel<1, 1, GATE, 1, true, 2>), grid, block, 0, (hipStream_t)stream, (const __half *)nullptr, (const float *)nullptr, u, g, dn, x, na, threshold, (float *)nullptr, ws->words, h_dense, ws->ffn_partial, hot_words, hot_prefix, ws->words_hot, (__half *)nullptr, const_cast<float *>(logits_dev), HostAnnounce{announce_seq, announce_flags})
     if (g) PI_PF2(true); else PI_PF2(false);
 #undef PI_PF2
+    ws->pf_parts = ff / 32; ws->pf_words = ff / 32;
     return pi::check_launch("pi_k_sparse_ffn_rows_hot");
 }
 
@@ -4095,8 +4333,10 @@ static int sparse_ffn_reduce_impl(int ff, int cols, int epilogue, const float * 
     if (!out || !ws || ff <= 0 || ff % 32 || ff > ws->max_ff || cols <= 0 || cols % 64 || cols > ws->max_d) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_reduce: bad arguments");
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
         return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_reduce: bad epilogue arguments");
-    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / 64), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, ff / (32 * pf_groups(ff, cols)), cols, hot ? ws->words_hot : ws->words, ff / 32, n_active,
-                       epilogue, add1, add2, out);
+    if (ws->pf_parts <= 0 || ws->pf_words <= 0 || ws->pf_words > ws->max_ff / 32 + 2048)
+        return pi::fail(PI_E_STATE, "pi_k_sparse_ffn_reduce: no fused launch has filled this workspace");
+    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / kFrCols), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, ws->pf_parts, cols, hot ? ws->words_hot : ws->words,
+                       ws->pf_words, n_active, epilogue, add1, add2, out);
     return pi::check_launch("pi_k_sparse_ffn_reduce");
 }
 
@@ -4152,8 +4392,8 @@ size_t pi_k_sparse_ffn_noalloc_scratch_bytes(void) { return kNaScratchBytes; }
 
 int pi_k_sparse_ffn_noalloc_supported(int ff, int r, int cols) {
     if (!pi_k_sparse_ffn_supported(ff, r, cols)) return 0;
-    const size_t parts = (size_t)(ff / (32 * pf_groups(ff, cols)));
-    return ff / 32 <= kNaMaxWords && parts * (size_t)cols * sizeof(float) <= kNaPartialBytes;
+    const size_t parts = (size_t)pf_parts(ff, cols, false);
+    return ff / 32 <= kNaMaxWords && 2 * parts <= (size_t)kNaMaxWords && parts * (size_t)cols * sizeof(float) <= kNaPartialBytes;
 }
 
 int pi_k_sparse_ffn_noalloc(const void * fc2_f16, int ff, int r, const float * hidden, float threshold,

@@ -22,6 +22,20 @@ int check_launch(const char * what) {
 
 }  // namespace pi
 
+namespace pi {
+int compute_units() {
+    static int cached[16] = {};
+    int dev = -1;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 16) return 0;
+    if (!cached[dev]) {
+        int n = 0;
+        if (hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) != hipSuccess) return 0;
+        cached[dev] = n;
+    }
+    return cached[dev];
+}
+}  // namespace pi
+
 extern "C" {
 
 const char * pi_last_error(void) { return pi::g_err; }
@@ -35,6 +49,7 @@ int pi_init(int device) {
     hipDeviceProp_t p;
     PI_HIP_TRY(hipGetDeviceProperties(&p, device));
     if (p.warpSize != 64) return pi::fail(PI_E_UNSUPPORTED, "pi_init: kernels are written for 64-wide wavefronts");
+    (void)pi::compute_units();
     return pi::noalloc_setup();
 }
 

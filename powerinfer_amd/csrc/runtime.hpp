@@ -9,6 +9,7 @@ void set_error(const char * msg);
 int  fail(int code, const char * msg);                 // records msg, returns code
 int  hip_fail(hipError_t e, const char * what);        // records "what: hipGetErrorString", returns PI_E_HIP
 int  check_launch(const char * what);                  // hipGetLastError() after a kernel launch
+int  compute_units();                                  // compute units of the current device (0 on error); cached per device, allocates nothing
 int  noalloc_setup();                                  // resolves the static scratch array of pi_k_sparse_ffn_noalloc on the current device
 
 }  // namespace pi

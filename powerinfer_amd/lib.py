@@ -56,6 +56,7 @@ _SIGS = {
     "pi_k_sparse_upgate": (_i, [_i, _vp, _vp, _i, _i, _vp, C.POINTER(Norm), _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_axpy": (_i, [_i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_supported": (_i, [_i, _i, _i]),
+    "pi_k_sparse_ffn_workgroups": (_i, [_i, _i, _i]),
     "pi_k_sparse_ffn": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_noalloc_scratch_bytes": (_sz, []),
     "pi_k_sparse_ffn_noalloc_supported": (_i, [_i, _i, _i]),

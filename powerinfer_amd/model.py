@@ -14,7 +14,7 @@ KINDS = ["tok_embd", "output_norm", "output_norm_b", "output",
          "attn_norm", "attn_norm_b", "attn_norm_2", "attn_norm_2_b",
          "wq", "wk", "wv", "wqkv", "wo",
          "ffn_norm", "ffn_gate", "ffn_up", "ffn_down_t",
-         "fc1", "fc2", "gpu_idx", "gpu_bucket"]
+         "fc1", "fc2", "gpu_idx", "gpu_bucket", "neuron_rate"]
 KIND = {k: i for i, k in enumerate(KINDS)}
 
 
@@ -109,6 +109,10 @@ class Model:
             for k, a in Lr.items():
                 if k in KIND and a is not None:
                     self.set_tensor(il, k, a)
+            if Lr.get("p") is not None and self.hp.get("use_rates", True):
+                # the neurons' firing rates (the activation statistics the reference's solver works from): the engine deals the
+                # neurons of a fully resident F16 layer out by rate over the groups of its fused kernel
+                self.set_tensor(il, "neuron_rate", np.asarray(Lr["p"], np.float32))
         self.finalize()
         return self
 

@@ -377,28 +377,51 @@ def main():
     n_mats = 2 if hp.arch == "falcon" else 3
     ffn_bytes = (d * hp.n_rank + hp.n_rank * hp.n_ff) * 2.0 + (act.mean() / hp.n_layer) * n_mats * d * wbytes
 
-    # the kernel next to it in time per token: fc2 rows of every neuron, the gate/up/down rows of the active ones, the input vector,
-    # the norm weights and the hidden vector in; the logits-free path writes one partial output vector per 32 neurons
+    # the fused sparse-FFN launch: ALGORITHMIC bytes only - the fc2 rows of every neuron and the gate / up / down rows of the active
+    # ones (fc2 + A * n_mats * R); the partial output vectors it writes for the reduction are overhead, not work
     a_layer = act.mean() / hp.n_layer
-    pf_bytes = hp.n_rank * hp.n_ff * 2.0 + a_layer * n_mats * d * 2.0 + (2 * d + hp.n_rank) * 4.0 + (hp.n_ff / 32.0) * d * 4.0
-    pf_traffic = None
-    try:
-        with open(os.path.join(ROOT, "profiles", "sparse_ffn_hbm_traffic.json")) as f:
-            pj = json.load(f)
-        if pj.get("shape") == [hp.n_ff, d, hp.n_rank] and args.config == 1:
-            pf_traffic = pj["traffic_bytes_per_launch"]
-    except (OSError, ValueError, KeyError):
-        pass
+    pf_bytes = hp.n_rank * hp.n_ff * 2.0 + a_layer * n_mats * d * 2.0
 
-    # HBM bytes per launch of that kernel from the FETCH_SIZE / WRITE_SIZE counter runs (profiles/qkv_gemv_hbm_traffic.md)
-    traffic = None
-    try:
-        with open(os.path.join(ROOT, "profiles", "qkv_gemv_hbm_traffic.json")) as f:
-            pj = json.load(f)
-        if pj.get("shape") == [d + 2 * gqa, d] and args.config == 1:
-            traffic = pj["traffic_bytes_per_launch"]
-    except (OSError, ValueError, KeyError):
-        pass
+    def profiled_traffic(name, shape):
+        """HBM bytes per launch from the FETCH_SIZE / WRITE_SIZE counter runs kept under profiles/ (a separate rocprofv3 --pmc run of
+        `bench.py --pmc-probe`, not measured by this run); None when no profile of this shape is there."""
+        try:
+            with open(os.path.join(ROOT, "profiles", name + ".json")) as f:
+                pj = json.load(f)
+            if pj.get("shape") == shape and args.config == 1:
+                return pj["traffic_bytes_per_launch"], "profiles/" + name + ".md (rocprofv3 --pmc FETCH_SIZE, WRITE_SIZE; a constant from that run, not measured here)"
+        except (OSError, ValueError, KeyError):
+            pass
+        return None, None
+
+    pf_traffic, pf_src = profiled_traffic("sparse_ffn_hbm_traffic", [hp.n_ff, d, hp.n_rank])
+    traffic, qkv_src = profiled_traffic("qkv_gemv_hbm_traffic", [d + 2 * gqa, d])
+    n_cu_form = d == 4096 and pl.load().pi_k_sparse_ffn_workgroups(hp.n_ff, hp.n_rank, d) != hp.n_ff // 32
+    roof_qkv = {
+        "bound": "hbm",
+        "kernel": {1: "gemv_f16_reg_kernel<8,1,0> (q|k|v projection, 12288 x 4096 fp16, fused RMSNorm)",
+                   2: "gemv_q4_kernel (q|k|v projection, 12288 x 4096 Q4_0, fused RMSNorm; not timed for a hybrid model)",
+                   4: "gemv_f16_reg_kernel<16,2,0> (q|k|v projection, 9216 x 8192 fp16, fused LayerNorm)"}[args.config],
+        "achieved": rnd(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": rnd(achieved / HBM_PEAK_GBPS, 4),
+        "traffic": traffic, "traffic_source": qkv_src,
+        "bytes_per_launch": qkv_bytes, "bytes_are": "weights + input vector + result (algorithmic)",
+        "us_per_launch": rnd(ms_qkv * 1e3, 2), "launches_timed": n_qkv,
+    }
+    roof_ffn = {
+        "bound": "hbm",
+        "kernel": {1: ("ffn_cu_f16_kernel<2,true,6,1>" if n_cu_form else "pred_ffn_f16_kernel<1,2,true,1,false>") +
+                      " (predictor fc2 11008 x 1024 + mask + gate/up/down rows of the active neurons, 7B layer)",
+                   2: "pred_upgate_q4_kernel (not timed for a hybrid model)",
+                   4: "pred_ffn_f16_kernel<2,2,false,4,false> (predictor fc2 32768 x 1024 + mask + up/down rows of the active neurons, Falcon-40B layer)"}[args.config],
+        "achieved": rnd(pf_bytes / (ms_pf * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
+        "frac": rnd(pf_bytes / (ms_pf * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
+        "traffic": pf_traffic, "traffic_source": pf_src,
+        "bytes_per_launch": round(pf_bytes),
+        "bytes_are": "fc2 rows of every neuron + gate/up/down rows of the measured mean of active neurons (algorithmic; the partial vectors written for the reduction are excluded)",
+        "us_per_launch": rnd(ms_pf * 1e3, 2), "reduce_us_per_launch": rnd(ms_fr * 1e3, 2), "launches_timed": n_pf,
+    }
+    # `roofline` names the kernel that takes the most time per token (one launch per layer each): whichever of the two is slower in this run
+    ffn_dominates = ms_pf == ms_pf and ms_pf >= ms_qkv
 
     out = {
         "metric": {1: "decode tok/s bs=1 ReLU-Llama2-7B FP16", 2: "decode tok/s bs=1 ReLU-Llama2-7B Q4_0 (60 % of neurons on the GPU)",
@@ -429,35 +452,9 @@ def main():
             "mean_active_per_layer": round(act.mean() / hp.n_layer, 1),
             "device": pl.device_name(),
         },
-        "roofline": {
-            "bound": "hbm",
-            "kernel": {1: "gemv_f16_reg_kernel<8,1,0> (q|k|v projection, 12288 x 4096 fp16, fused RMSNorm)",
-                       2: "gemv_q4_kernel (q|k|v projection, 12288 x 4096 Q4_0, fused RMSNorm; not timed for a hybrid model)",
-                       4: "gemv_f16_reg_kernel<16,2,0> (q|k|v projection, 9216 x 8192 fp16, fused LayerNorm)"}[args.config],
-            "achieved": rnd(achieved, 1),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": rnd(achieved / HBM_PEAK_GBPS, 4),
-            "traffic": traffic,
-            "bytes_per_launch": qkv_bytes,
-            "us_per_launch": rnd(ms_qkv * 1e3, 2),
-            "launches_timed": n_qkv,
-        },
-        "roofline_sparse_ffn": {
-            "bound": "hbm",
-            "kernel": {1: "pred_ffn_f16_kernel<1,2,true,1,false> (predictor fc2 11008 x 1024 + mask + gate/up/down rows of the active neurons, 7B layer)",
-                       2: "pred_upgate_q4_kernel (not timed for a hybrid model)",
-                       4: "pred_ffn_f16_kernel<2,2,false,4,false> (predictor fc2 32768 x 1024 + mask + up/down rows of the active neurons, Falcon-40B layer)"}[args.config],
-            "achieved": rnd(pf_bytes / (ms_pf * 1e-3) / 1e9, 1),
-            "peak": HBM_PEAK_GBPS,
-            "unit": "GB/s",
-            "frac": rnd(pf_bytes / (ms_pf * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
-            "traffic": pf_traffic,
-            "bytes_per_launch": round(pf_bytes),
-            "us_per_launch": rnd(ms_pf * 1e3, 2),
-            "reduce_us_per_launch": rnd(ms_fr * 1e3, 2),
-            "launches_timed": n_pf,
-        },
+        "roofline": dict(roof_ffn if ffn_dominates else roof_qkv),
+        "roofline_qkv": roof_qkv,
+        "roofline_sparse_ffn": roof_ffn,
         "token_loop": {
             "device_ms_per_step": round(ms_dev / args.steps, 4),
             "touched_GB_per_token": round(tok_bytes / 1e9, 4),

@@ -418,6 +418,10 @@ void cold_destroy(ColdPath * c) {
         fprintf(stderr, "cold path, mean us per layer call over %lld calls: between calls %.1f | wait inputs %.1f | norm+list %.1f | up/gate %.1f | wait h + upload %.1f | down %.1f | merge launch %.1f | active cold neurons %.1f\n",
                 c->n_calls, c->t_between / n, c->t_phase[0] / n, c->t_phase[1] / n, c->t_phase[2] / n, c->t_phase[3] / n, c->t_phase[4] / n, c->t_phase[5] / n, (double)c->n_cold_active / n);
     }
+    // wait kernels that are still queued (a decode that returned early) must not poll a host that is gone for their whole time limit:
+    // raise the host's stop word, which every wait kernel checks, let the stream drain, and only then stop the thread and free the flags
+    if (c->flags) __atomic_store_n(&c->flags[48], 1u, __ATOMIC_RELEASE);
+    if (c->model && c->model->stream) (void)hipStreamSynchronize(c->model->stream);
     if (c->service.joinable()) {
         c->stop.store(true);
         { std::lock_guard<std::mutex> g(c->mu); }
@@ -957,9 +961,13 @@ void service_loop(ColdPath * c) {
             relax();
             if ((it & 255) == 255 && std::chrono::steady_clock::now() - t0 > std::chrono::microseconds(2000)) {
                 std::unique_lock<std::mutex> g(c->mu);
-                c->service_asleep.store(1);
-                c->cv.wait(g, [&] { return c->posted.load() != next || c->stop.load(); });
-                c->service_asleep.store(0);
+                // the producer stores `posted` and then reads `service_asleep`; this side stores `service_asleep` and then reads
+                // `posted`: both pairs are sequentially consistent, so at least one side sees the other's store.  The bounded wait is
+                // a second line of defence: a wake-up that is lost all the same costs a few milliseconds, not the 5 s of the device's wait.
+                c->service_asleep.store(1, std::memory_order_seq_cst);
+                while (c->posted.load(std::memory_order_seq_cst) == next && !c->stop.load())
+                    c->cv.wait_for(g, std::chrono::milliseconds(2));
+                c->service_asleep.store(0, std::memory_order_seq_cst);
             }
         }
         if (c->stop.load()) return;
@@ -995,9 +1003,9 @@ int cold_post_token(ColdPath * c) {
         const uint64_t p = c->posted.load(std::memory_order_relaxed);
         while (p - c->served.load(std::memory_order_acquire) >= c->ring.size()) relax();
         c->ring[p % c->ring.size()] = il;
-        c->posted.store(p + 1, std::memory_order_release);
+        c->posted.store(p + 1, std::memory_order_seq_cst);
     }
-    if (c->service_asleep.load()) { { std::lock_guard<std::mutex> g(c->mu); } c->cv.notify_all(); }
+    if (c->service_asleep.load(std::memory_order_seq_cst)) { { std::lock_guard<std::mutex> g(c->mu); } c->cv.notify_all(); }
     return PI_OK;
 }
 

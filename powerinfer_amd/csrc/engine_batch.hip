@@ -325,17 +325,29 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
     if (T <= 16 || T > kMaxT) return pi::fail(PI_E_ARG, "prefill_wide_chunk: chunk length outside 17 .. prefill_wide_max");
     const pi_hparams & hp = m->hp;
     if (!m->prefill_wide) {
-        if (kMaxT > 128) {
+        if (kMaxT > 128 && !m->gemm_lib) {
             m->gemm_lib = pi_gemm_lib_create((size_t)64 << 20);
             if (!m->gemm_lib) return PI_E_HIP;
         }
         BatchState * b = batch_alloc(m, kMaxT, false);
         if (!b) return PI_E_HIP;
+        // until the state is complete every early return undoes what was created here (the device buffers stay with the model's
+        // allocation list; the mat-mul library is kept for the next attempt)
+        struct SetupGuard {
+            pi_model * m; BatchState * b; bool armed = true;
+            ~SetupGuard() {
+                if (!armed) return;
+                if (b->copy_stream) (void)hipStreamDestroy(b->copy_stream);
+                for (int i = 0; i < 2; ++i) { if (b->ev_copied[i]) (void)hipEventDestroy(b->ev_copied[i]); if (b->ev_free[i]) (void)hipEventDestroy(b->ev_free[i]); }
+                delete b;
+                m->down_rows.clear();
+            }
+        } guard{m, b};
         b->prefill = true;
         b->up_out = m->alloc<float>((size_t)kMaxT * hp.n_ff);
         b->gate_out = hp.arch == PI_ARCH_FALCON ? nullptr : m->alloc<float>((size_t)kMaxT * hp.n_ff);
         b->h16 = m->alloc<__half>((size_t)kMaxT * hp.n_ff);
-        if (!b->up_out || (hp.arch != PI_ARCH_FALCON && !b->gate_out) || !b->h16) { delete b; return PI_E_HIP; }
+        if (!b->up_out || (hp.arch != PI_ARCH_FALCON && !b->gate_out) || !b->h16) return PI_E_HIP;
         // the down projection of a chunk is a mat-mul whose reduction runs over the neurons.  An F16 layer that is whole on the device
         // gets one more copy of it with the neurons contiguous (n_embd x n_ff fp16; the decode loop keeps the row-per-neuron layout);
         // Q4_0 and hybrid layers expand one matrix at a time into scratch instead, so that prompts leave the model's footprint as
@@ -351,12 +363,12 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
             if (split || m->L(il, PI_T_FFN_UP).type == PI_TYPE_Q4_0 || m->L(il, PI_T_FFN_DOWN_T).type == PI_TYPE_Q4_0) w16 = std::max(w16, (size_t)hp.n_ff * hp.n_embd);
             if (split || m->L(il, PI_T_FFN_DOWN_T).type == PI_TYPE_Q4_0) { scratch = true; continue; }
             m->down_rows[il] = m->alloc<__half>((size_t)hp.n_embd * hp.n_ff);
-            if (!m->down_rows[il]) { delete b; m->down_rows.clear(); return PI_E_HIP; }
+            if (!m->down_rows[il]) return PI_E_HIP;
             PI_TRY(pi_k_transpose_f16(m->L(il, PI_T_FFN_DOWN_T).dev, hp.n_ff, hp.n_embd, m->down_rows[il], m->stream));
         }
         if (w16) b->w16 = m->alloc<__half>(w16);
         if (scratch) b->w16t = m->alloc<__half>((size_t)hp.n_embd * hp.n_ff);
-        if ((w16 && !b->w16) || (scratch && !b->w16t)) { delete b; m->down_rows.clear(); return PI_E_HIP; }
+        if ((w16 && !b->w16) || (scratch && !b->w16t)) return PI_E_HIP;
         // two staging buffers for the non-resident rows of hybrid layers (the largest such layer decides their size)
         for (int il = 0; il < hp.n_layer; ++il) {
             if (!m->L(il, PI_T_GPU_BUCKET).dev) continue;
@@ -367,12 +379,13 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
         if (b->stage_rows && !(no_stage && no_stage[0] == '1')) {
             for (int i = 0; i < 2; ++i) {
                 b->stage[i] = m->alloc<unsigned char>(3 * b->stage_rows * b->stage_row_bytes);
-                if (!b->stage[i]) { delete b; m->down_rows.clear(); return PI_E_HIP; }
+                if (!b->stage[i]) return PI_E_HIP;
                 PI_HIP_TRY(hipEventCreateWithFlags(&b->ev_copied[i], hipEventDisableTiming));
                 PI_HIP_TRY(hipEventCreateWithFlags(&b->ev_free[i], hipEventDisableTiming));
             }
             PI_HIP_TRY(hipStreamCreateWithFlags(&b->copy_stream, hipStreamNonBlocking));
         }
+        guard.armed = false;
         m->prefill_wide = b;
     }
     BatchState * b = m->prefill_wide;

@@ -16,6 +16,7 @@ namespace {
 struct Plan {
     int rows, cols, T;
     bool with_c;
+    uint64_t last_use;
     hipblasLtMatmulDesc_t op;
     hipblasLtMatrixLayout_t a, b, c;
     hipblasLtMatmulHeuristicResult_t heur;
@@ -38,8 +39,18 @@ struct pi_gemm_lib {
     hipblasLtHandle_t handle = nullptr;
     void * ws = nullptr;
     size_t ws_bytes = 0;
-    std::vector<Plan> plans;
+    std::vector<Plan> plans;          // at most kMaxPlans; the least recently used one makes room for a new shape
+    uint64_t clock = 0;
 };
+constexpr size_t kMaxPlans = 64;
+
+static void destroy_plan(Plan & p) {
+    if (p.a) (void)hipblasLtMatrixLayoutDestroy(p.a);
+    if (p.b) (void)hipblasLtMatrixLayoutDestroy(p.b);
+    if (p.c) (void)hipblasLtMatrixLayoutDestroy(p.c);
+    if (p.op) (void)hipblasLtMatmulDescDestroy(p.op);
+    p.a = p.b = p.c = nullptr; p.op = nullptr;
+}
 
 #define PI_TRY(expr) do { int _rc = (expr); if (_rc != PI_OK) return _rc; } while (0)
 #define PI_LT_TRY(expr)                                                                                                 \
@@ -52,30 +63,45 @@ struct pi_gemm_lib {
         }                                                                                                               \
     } while (0)
 
+// A plan is used only to enqueue its product (the descriptors are read at enqueue time), so evicting one between two calls is safe.
+// Prompt remainders of every length ask for their own plans: a server would otherwise run into the cap after a few dozen prompts.
 static int make_plan(pi_gemm_lib * g, int rows, int cols, int T, bool with_c, Plan ** out) {
     for (Plan & p : g->plans)
-        if (p.rows == rows && p.cols == cols && p.T == T && p.with_c == with_c) { *out = &p; return PI_OK; }
-    if (g->plans.size() >= 64) return pi::fail(PI_E_STATE, "pi_gemm_lib_f16: too many distinct shapes");      // pointers into plans stay valid
+        if (p.rows == rows && p.cols == cols && p.T == T && p.with_c == with_c) { p.last_use = ++g->clock; *out = &p; return PI_OK; }
     Plan p{};
     p.rows = rows; p.cols = cols; p.T = T; p.with_c = with_c;
-    // column-major view: D (rows x T, ld rows) = W^T-as-stored (cols x rows, ld cols) transposed  x  xn-as-stored (cols x T, ld cols)
-    PI_LT_TRY(hipblasLtMatmulDescCreate(&p.op, HIPBLAS_COMPUTE_32F, HIP_R_32F));
-    const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
-    PI_LT_TRY(hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof ta));
-    PI_LT_TRY(hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof tb));
-    PI_LT_TRY(hipblasLtMatrixLayoutCreate(&p.a, HIP_R_16F, cols, rows, cols));
-    PI_LT_TRY(hipblasLtMatrixLayoutCreate(&p.b, HIP_R_16F, cols, T, cols));
-    PI_LT_TRY(hipblasLtMatrixLayoutCreate(&p.c, HIP_R_32F, rows, T, rows));
-    hipblasLtMatmulPreference_t pref;
-    PI_LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
-    const uint64_t wsb = g->ws_bytes;
-    PI_LT_TRY(hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &wsb, sizeof wsb));
-    int found = 0;
-    const hipblasStatus_t hs = hipblasLtMatmulAlgoGetHeuristic(g->handle, p.op, p.a, p.b, p.c, p.c, pref, 1, &p.heur, &found);
-    (void)hipblasLtMatmulPreferenceDestroy(pref);
-    if (hs != HIPBLAS_STATUS_SUCCESS || found < 1) return pi::fail(PI_E_UNSUPPORTED, "pi_gemm_lib_f16: hipBLASLt offers no kernel for this shape");
-    g->plans.push_back(p);
-    *out = &g->plans.back();
+    const auto build = [&]() -> int {
+        // column-major view: D (rows x T, ld rows) = W^T-as-stored (cols x rows, ld cols) transposed  x  xn-as-stored (cols x T, ld cols)
+        PI_LT_TRY(hipblasLtMatmulDescCreate(&p.op, HIPBLAS_COMPUTE_32F, HIP_R_32F));
+        const hipblasOperation_t ta = HIPBLAS_OP_T, tb = HIPBLAS_OP_N;
+        PI_LT_TRY(hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_TRANSA, &ta, sizeof ta));
+        PI_LT_TRY(hipblasLtMatmulDescSetAttribute(p.op, HIPBLASLT_MATMUL_DESC_TRANSB, &tb, sizeof tb));
+        PI_LT_TRY(hipblasLtMatrixLayoutCreate(&p.a, HIP_R_16F, cols, rows, cols));
+        PI_LT_TRY(hipblasLtMatrixLayoutCreate(&p.b, HIP_R_16F, cols, T, cols));
+        PI_LT_TRY(hipblasLtMatrixLayoutCreate(&p.c, HIP_R_32F, rows, T, rows));
+        hipblasLtMatmulPreference_t pref;
+        PI_LT_TRY(hipblasLtMatmulPreferenceCreate(&pref));
+        const uint64_t wsb = g->ws_bytes;
+        hipblasStatus_t hs = hipblasLtMatmulPreferenceSetAttribute(pref, HIPBLASLT_MATMUL_PREF_MAX_WORKSPACE_BYTES, &wsb, sizeof wsb);
+        int found = 0;
+        if (hs == HIPBLAS_STATUS_SUCCESS) hs = hipblasLtMatmulAlgoGetHeuristic(g->handle, p.op, p.a, p.b, p.c, p.c, pref, 1, &p.heur, &found);
+        (void)hipblasLtMatmulPreferenceDestroy(pref);
+        if (hs != HIPBLAS_STATUS_SUCCESS || found < 1) return pi::fail(PI_E_UNSUPPORTED, "pi_gemm_lib_f16: hipBLASLt offers no kernel for this shape");
+        return PI_OK;
+    };
+    const int rc = build();
+    if (rc != PI_OK) { destroy_plan(p); return rc; }
+    p.last_use = ++g->clock;
+    if (g->plans.size() < kMaxPlans) {
+        g->plans.push_back(p);
+        *out = &g->plans.back();
+    } else {
+        size_t victim = 0;
+        for (size_t i = 1; i < g->plans.size(); ++i) if (g->plans[i].last_use < g->plans[victim].last_use) victim = i;
+        destroy_plan(g->plans[victim]);
+        g->plans[victim] = p;
+        *out = &g->plans[victim];
+    }
     return PI_OK;
 }
 
@@ -89,16 +115,13 @@ pi_gemm_lib * pi_gemm_lib_create(size_t workspace_bytes) {
         g->ws = pi_malloc(workspace_bytes);
         if (!g->ws) { (void)hipblasLtDestroy(g->handle); delete g; return nullptr; }
     }
-    g->plans.reserve(64);
+    g->plans.reserve(kMaxPlans);
     return g;
 }
 
 int pi_gemm_lib_destroy(pi_gemm_lib * g) {
     if (!g) return PI_OK;
-    for (Plan & p : g->plans) {
-        (void)hipblasLtMatrixLayoutDestroy(p.a); (void)hipblasLtMatrixLayoutDestroy(p.b); (void)hipblasLtMatrixLayoutDestroy(p.c);
-        (void)hipblasLtMatmulDescDestroy(p.op);
-    }
+    for (Plan & p : g->plans) destroy_plan(p);
     if (g->ws) { (void)pi_sync(); (void)pi_free(g->ws); }
     (void)hipblasLtDestroy(g->handle);
     delete g;

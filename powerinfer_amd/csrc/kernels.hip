@@ -4367,11 +4367,13 @@ constexpr int kNaMaxDevices = 16;
 unsigned char * g_na_ptr[kNaMaxDevices] = {};            // device address of `scratch` on each device (the name itself is not one)
 }
 
-// resolves the scratch array's address on the current device, once per device
-static int noalloc_setup_current_device(unsigned char ** out) {
+// the scratch array's address on the current device.  pi_init resolves it once per device (resolve = true: taking a symbol's address
+// may load the code object, which allocates); the entry point itself only looks it up, so that a call never reaches an allocator.
+static int noalloc_setup_current_device(unsigned char ** out, bool resolve) {
     int dev = -1;
     PI_HIP_TRY(hipGetDevice(&dev));
     if (dev < 0 || dev >= kNaMaxDevices) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn_noalloc: device index beyond 15");
+    if (!g_na_ptr[dev] && !resolve) return pi::fail(PI_E_STATE, "pi_k_sparse_ffn_noalloc: call pi_init on this device first (it resolves the scratch array's address)");
     if (!g_na_ptr[dev]) {
         unsigned char * p = nullptr;
         PI_HIP_TRY(hipGetSymbolAddress((void **)&p, HIP_SYMBOL(scratch)));
@@ -4383,7 +4385,7 @@ static int noalloc_setup_current_device(unsigned char ** out) {
 }
 
 namespace pi {
-int noalloc_setup() { return noalloc_setup_current_device(nullptr); }      // called by pi_init with the device current
+int noalloc_setup() { return noalloc_setup_current_device(nullptr, true); }      // called by pi_init with the device current
 }
 
 extern "C" {
@@ -4404,7 +4406,7 @@ int pi_k_sparse_ffn_noalloc(const void * fc2_f16, int ff, int r, const float * h
     if (!pi_k_sparse_ffn_noalloc_supported(ff, r, cols))
         return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn_noalloc: shape exceeds the static scratch (at most 8 MiB of partial vectors = (ff / 32 or ff / 128) * cols floats, ff <= 131072)");
     unsigned char * base = nullptr;
-    const int rc = noalloc_setup_current_device(&base);
+    const int rc = noalloc_setup_current_device(&base, false);
     if (rc != PI_OK) return rc;
     // a workspace view of the static array: only the members the fused route touches
     pi_workspace ws{};

@@ -475,3 +475,31 @@ def test_decode_rejects_bad_arguments():
     with pytest.raises(PiError):
         gm.generate(14)                              # would run past the context
     gm.close()
+
+
+def test_prompt_lengths_beyond_the_plan_cache():
+    """Prompt chunks of up to 512 tokens send their dense mat-muls to hipBLASLt, one plan per (matrix shape, chunk length); the cache
+    holds 64.  One engine instance decodes prompts of 16 distinct lengths (about 100 plans), then the same prompts in reverse order:
+    every call succeeds and reproduces its logits bit for bit, whether its plans survived or were rebuilt after an eviction."""
+    from powerinfer_amd.model import Model
+    hp = synth.hparams("llama-tiny", n_rank=256, n_ctx=128, seed=5, pred_margin=True)      # no neuron near the threshold: see run_north_star
+    model = synth.make_model(hp)
+    gm = Model(hp).load(model)
+    rng = np.random.default_rng(3)
+    prompt = rng.integers(0, hp.n_vocab, 64).astype(np.int32)
+    lengths = list(range(19, 51, 2))                          # the chunk is the prompt minus its last token: 18 .. 48, all above 16
+    first = {}
+    for n in lengths + lengths[::-1]:
+        gm.kv_clear()
+        tok, lg = gm.decode(prompt[:n], 0)
+        if n in first:
+            assert tok == first[n][0] and np.array_equal(lg, first[n][1]), n
+        else:
+            first[n] = (tok, lg)
+    # and the chunk path still agrees with the token-by-token path of the oracle on one of them
+    om = ol.OracleModel(model)
+    tok_o = lg_o = None
+    for i, t in enumerate(prompt[:33]):
+        tok_o, lg_o = om.eval([int(t)], i)
+    assert rel_err(first[33][1], lg_o) < 1e-2
+    gm.close(), om.close()

@@ -475,6 +475,14 @@ enum {
     PI_T_COUNT
 };
 
+/* The ggml_cuda_* boundary (include/ggml_backend_abi.h) keeps single-token nodes in a window until it knows whether they form a block
+ * it computes in one launch: llm_build_ffn_sparse's sequence (llama.cpp:4652-4757), with every neuron on the device, becomes pi_k_gemv +
+ * pi_k_sparse_ffn when its AXPY node arrives.  These two calls are not part of the reference's interface: the counters tell a test or
+ * a profile what the window did, the switch turns it off at run time (GGML_CUDA_NO_FUSION=1 in the environment does so from the start). */
+typedef struct pi_ggml_backend_stats { int64_t nodes_deferred, windows_flushed, ffn_blocks_fused; } pi_ggml_backend_stats;
+PI_API void pi_ggml_backend_get_stats(pi_ggml_backend_stats * out);
+PI_API void pi_ggml_backend_set_fusion(int enable);
+
 typedef struct pi_model pi_model;
 
 /* llama_load_model_from_file + llama_new_context_with_model (llama.cpp:9789, 9819) without the file

@@ -198,6 +198,36 @@ __global__ __launch_bounds__(256) void norm_rows_kernel(const float * x, float *
     const float scale = pi_inv_sqrt((float)(s / n) + eps);
     for (int i = threadIdx.x; i < n; i += 256) yr[i] = __fmul_rn(__fsub_rn(xr[i], mean), scale);
 }
+// norm -> * w -> (+ b) of one row in one launch (llm_build_norm's three nodes, llama.cpp:4420-4450, when each is computed in place of
+// the one before); same arithmetic as the three kernels: double statistics, one fp32 product per step
+__global__ __launch_bounds__(1024) void norm_affine_kernel(const float * x, const float * w, const float * b, float * y, int n, float eps, int kind) {
+    __shared__ double red[16];
+    auto bsum = [&](double v) {
+        v = pi_wave_sum_f64(v);
+        __syncthreads();
+        if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+        __syncthreads();
+        double t = 0.0;
+        for (int i = 0; i < 16; ++i) t += red[i];
+        return t;
+    };
+    float mean = 0.0f;
+    double s = 0.0;
+    if (kind == 0) { for (int i = threadIdx.x; i < n; i += 1024) s += (double)__fmul_rn(x[i], x[i]); s = bsum(s); }
+    else {
+        for (int i = threadIdx.x; i < n; i += 1024) s += (double)x[i];
+        mean = (float)(bsum(s) / n);
+        s = 0.0;
+        for (int i = threadIdx.x; i < n; i += 1024) { const float v = __fsub_rn(x[i], mean); s += (double)__fmul_rn(v, v); }
+        s = bsum(s);
+    }
+    const float scale = pi_inv_sqrt((float)(s / n) + eps);
+    for (int i = threadIdx.x; i < n; i += 1024) {
+        float v = __fmul_rn(__fmul_rn(__fsub_rn(x[i], mean), scale), w[i]);
+        if (b) v = __fadd_rn(v, b[i]);
+        y[i] = v;
+    }
+}
 // one workgroup per row; exp through the fp16 rounding of the CPU path's table (ggml.c:10747-10759)
 __global__ __launch_bounds__(256) void softmax_rows_kernel(const float * x, float * y, int n) {
     __shared__ double red[4];
@@ -487,6 +517,19 @@ bool op_get_rows(ggml_tensor * dst) {
     return true;
 }
 
+bool run_node(ggml_tensor * tensor) {
+    switch (tensor->op) {
+        case GGML_OP_MUL_MAT:        return op_mul_mat(tensor);
+        case GGML_OP_MUL_MAT_SPARSE: return sparse_common(tensor, false);
+        case GGML_OP_AXPY:           return sparse_common(tensor, true);
+        case GGML_OP_ROPE:           return op_rope(tensor);
+        case GGML_OP_CPY: case GGML_OP_CONT: case GGML_OP_DUP: return op_cpy(tensor);
+        case GGML_OP_GET_ROWS:       return op_get_rows(tensor);
+        case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE: return true;
+        default:                     return op_elementwise(tensor);
+    }
+}
+
 Extra * new_extra(void * p, bool owned) {
     Extra * e = new Extra();
     memset(e, 0, sizeof *e);
@@ -542,6 +585,181 @@ void assign(ggml_tensor * tensor, bool scratch, bool force_inplace, bool no_allo
     }
 }
 
+// ---- deferred nodes -----------------------------------------------------------------------------------------
+// The host hands over one node at a time, in graph order.  A single-token node that may turn out to be part of a block this library
+// computes in one launch is not run when it arrives: it joins a window of pending nodes.  The window only ever holds consecutive
+// nodes - the first node that cannot join it either consumes it (the AXPY node that completes llm_build_ffn_sparse's sequence,
+// llama.cpp:4652-4757: fc1 -> relu -> fc2 -> sparse up / gate -> relu * mul -> sparse down becomes pi_k_gemv + pi_k_sparse_ffn) or makes
+// every pending node run, in order, before it runs itself.  Running a node late but in order, with nothing else in between, is
+// the schedule the host's allocator planned for, so buffers it shares between nodes stay valid.
+// The fused block does not write the dense up / gate vectors and the predictor's hidden layer: in the reference's graph nothing
+// else reads them (they are locals of llm_build_ffn_sparse); the predictor logits and h are still written to their nodes.
+// GGML_CUDA_NO_FUSION=1 in the environment turns the window off (every node runs when it arrives).
+struct PendingNode { ggml_tensor * t; int op; const ggml_tensor * src[4]; void * extra; };
+std::vector<PendingNode> g_pending;
+bool g_fuse = true;
+pi_ggml_backend_stats g_stats{};
+constexpr size_t kMaxPending = 24;
+
+bool is_pending(const ggml_tensor * t) { for (const PendingNode & p : g_pending) if (p.t == t) return true; return false; }
+bool on_device(const ggml_tensor * t) { return t && t->backend != GGML_BACKEND_CPU && t->extra != nullptr && !((const Extra *)t->extra)->outside_scratch; }
+bool vec1(const ggml_tensor * t) { return t && t->type == GGML_TYPE_F32 && contiguous(t) && nrows(t) == 1; }
+bool avail(const ggml_tensor * t) { return vec1(t) && (is_pending(t) || on_device(t)); }
+bool weight_on_device(const ggml_tensor * a) {
+    return on_device(a) && a->ne[2] == 1 && a->ne[3] == 1 && a->nb[0] == tsize(a->type) && a->nb[1] == row_size(a) &&
+           (a->type == GGML_TYPE_F16 || a->type == GGML_TYPE_Q4_0) && a->ne[0] % (a->type == GGML_TYPE_F16 ? 8 : 32) == 0;
+}
+
+bool deferrable(const ggml_tensor * n) {
+    if (!g_fuse || g_pending.size() >= kMaxPending || n->backend != GGML_BACKEND_GPU || !vec1(n) || !on_device(n)) return false;
+    const ggml_tensor * a = n->src[0]; const ggml_tensor * b = n->src[1];
+    switch (n->op) {
+        case GGML_OP_RMS_NORM: case GGML_OP_NORM: return vec1(a) && on_device(a) && !is_pending(a) && nelem(a) == nelem(n);
+        case GGML_OP_MUL: case GGML_OP_ADD: return is_pending(a) && vec1(a) && avail(b) && nelem(b) == nelem(n) && nelem(a) == nelem(n);
+        case GGML_OP_UNARY: return n->op_params[0] == GGML_UNARY_OP_RELU && is_pending(a) && vec1(a);
+        case GGML_OP_MUL_MAT: return weight_on_device(a) && avail(b) && b->ne[0] == a->ne[0] && n->ne[0] == a->ne[1];
+        case GGML_OP_MUL_MAT_SPARSE:
+            return n->src[3] == nullptr && weight_on_device(a) && avail(b) && b->ne[0] == a->ne[0] && avail(n->src[2]) &&
+                   n->src[2]->ne[0] == a->ne[1] && n->ne[0] == a->ne[1];
+        default: return false;
+    }
+}
+void defer(ggml_tensor * n) { ++g_stats.nodes_deferred; g_pending.push_back(PendingNode{n, (int)n->op, {n->src[0], n->src[1], n->src[2], n->src[3]}, n->extra}); }
+// a node of an abandoned evaluation (the host rebuilt its graph in the same memory) no longer looks the way it was deferred
+bool still_valid(const PendingNode & p) {
+    return p.t->op == p.op && p.t->src[0] == p.src[0] && p.t->src[1] == p.src[1] && p.t->src[2] == p.src[2] && p.t->src[3] == p.src[3] && p.t->extra == p.extra;
+}
+
+// runs what is pending, in order.  Two peepholes: norm -> * w (-> + b) computed in place of one another is one launch, and a
+// mat-vec whose ReLU is computed in place of it takes the ReLU as its epilogue.
+void flush_pending() {
+    if (g_pending.empty()) return;
+    ++g_stats.windows_flushed;
+    std::vector<PendingNode> win;
+    win.swap(g_pending);
+    for (size_t i = 0; i < win.size(); ++i) {
+        if (!still_valid(win[i])) continue;
+        ggml_tensor * n = win[i].t;
+        if ((n->op == GGML_OP_RMS_NORM || n->op == GGML_OP_NORM) && i + 1 < win.size() && still_valid(win[i + 1])) {
+            ggml_tensor * m = win[i + 1].t;
+            if (m->op == GGML_OP_MUL && m->src[0] == n && on_device(m->src[1]) && dev_ptr(m) == dev_ptr(n)) {
+                ggml_tensor * last = m; const float * bias = nullptr; size_t used = 2;
+                if (i + 2 < win.size() && still_valid(win[i + 2])) {
+                    ggml_tensor * a = win[i + 2].t;
+                    if (a->op == GGML_OP_ADD && a->src[0] == m && on_device(a->src[1]) && dev_ptr(a) == dev_ptr(m)) { last = a; bias = (const float *)dev_ptr(a->src[1]); used = 3; }
+                }
+                float eps; memcpy(&eps, n->op_params, 4);
+                hipLaunchKernelGGL(norm_affine_kernel, dim3(1), dim3(1024), 0, 0, (const float *)dev_ptr(n->src[0]), (const float *)dev_ptr(m->src[1]), bias,
+                                   (float *)dev_ptr(last), (int)n->ne[0], eps, n->op == GGML_OP_NORM ? 1 : 0);
+                i += used - 1;
+                continue;
+            }
+        }
+        if (n->op == GGML_OP_MUL_MAT && i + 1 < win.size() && still_valid(win[i + 1])) {
+            ggml_tensor * r = win[i + 1].t;
+            const ggml_tensor * a = n->src[0];
+            if (r->op == GGML_OP_UNARY && r->src[0] == n && dev_ptr(r) == dev_ptr(n)) {
+                BK_PI(pi_k_gemv(a->type, dev_ptr(a), (int)a->ne[1], (int)a->ne[0], (const float *)dev_ptr(n->src[1]), nullptr, PI_EPI_RELU, nullptr, nullptr,
+                                (float *)dev_ptr(r), nullptr));
+                ++i;
+                continue;
+            }
+            // ... + residual, computed in place of the product (the attention output projection, llama.cpp:5022)
+            if (r->op == GGML_OP_ADD && r->src[0] == n && dev_ptr(r) == dev_ptr(n) && on_device(r->src[1]) && !is_pending(r->src[1]) && r->src[1] != n->src[1] &&
+                dev_ptr(r->src[1]) != dev_ptr(n)) {
+                BK_PI(pi_k_gemv(a->type, dev_ptr(a), (int)a->ne[1], (int)a->ne[0], (const float *)dev_ptr(n->src[1]), nullptr, PI_EPI_ADD, (const float *)dev_ptr(r->src[1]), nullptr,
+                                (float *)dev_ptr(r), nullptr));
+                ++i;
+                continue;
+            }
+        }
+        if (!run_node(n)) {
+            fprintf(stderr, "powerinfer-hip backend: deferred node '%s' (op %d) has a shape/type/stride this backend does not implement\n", n->name, (int)n->op);
+            exit(1);
+        }
+    }
+}
+
+const PendingNode * find_pending(const ggml_tensor * t) { for (const PendingNode & p : g_pending) if (p.t == t && still_valid(p)) return &p; return nullptr; }
+
+// The AXPY node that closes llm_build_ffn_sparse's sequence with every neuron on the device.  Returns false (nothing done) unless the
+// pending window is exactly that block.
+bool try_fused_ffn(ggml_tensor * axpy) {
+    const ggml_tensor * down = axpy->src[0]; const ggml_tensor * cur = axpy->src[1]; const ggml_tensor * idx = axpy->src[2];
+    if (axpy->src[3] != nullptr || !idx || !cur || !weight_on_device(down) || down->type != GGML_TYPE_F16 || !vec1(axpy) || axpy->backend != GGML_BACKEND_GPU || !on_device(axpy)) return false;
+    size_t used = 0;
+    auto take = [&](const ggml_tensor * t, int op) -> const ggml_tensor * {           // t is pending and has this operator
+        if (!t || !find_pending(t) || t->op != op) return nullptr;
+        ++used;
+        return t;
+    };
+    // h = relu(gate) * up, or relu(up)
+    const ggml_tensor * up_s = nullptr; const ggml_tensor * gate_s = nullptr;
+    if (take(cur, GGML_OP_MUL)) {
+        const ggml_tensor * ga = take(cur->src[0], GGML_OP_UNARY);
+        if (!ga) return false;
+        gate_s = take(ga->src[0], GGML_OP_MUL_MAT_SPARSE);
+        up_s = take(cur->src[1], GGML_OP_MUL_MAT_SPARSE);
+        if (!gate_s || !up_s || gate_s == up_s) return false;
+    } else if (take(cur, GGML_OP_UNARY)) {
+        up_s = take(cur->src[0], GGML_OP_MUL_MAT_SPARSE);
+        if (!up_s) return false;
+    } else return false;
+    const ggml_tensor * X = up_s->src[1];
+    if (up_s->src[2] != idx || (gate_s && (gate_s->src[1] != X || gate_s->src[2] != idx))) return false;
+    const ggml_tensor * up = up_s->src[0]; const ggml_tensor * gate = gate_s ? gate_s->src[0] : nullptr;
+    if (up->type != GGML_TYPE_F16 || (gate && gate->type != GGML_TYPE_F16)) return false;
+    // predictor: idx = fc2 . relu(fc1 . P)
+    if (!take(idx, GGML_OP_MUL_MAT)) return false;
+    const ggml_tensor * fc2 = idx->src[0];
+    const ggml_tensor * hid = take(idx->src[1], GGML_OP_UNARY);
+    if (!hid) return false;
+    const ggml_tensor * pre = take(hid->src[0], GGML_OP_MUL_MAT);
+    if (!pre) return false;
+    const ggml_tensor * fc1 = pre->src[0]; const ggml_tensor * P = pre->src[1];
+    if (is_pending(P) || !on_device(P) || fc2->type != GGML_TYPE_F16) return false;
+    // FFN input: norm(F) * w (+ b) still pending, or a vector that exists
+    pi_norm nrm{0, 0.0f, nullptr, nullptr};
+    const ggml_tensor * F = X;
+    if (is_pending(X)) {
+        const ggml_tensor * t = X;
+        if (t->op == GGML_OP_ADD) { if (!take(t, GGML_OP_ADD) || !on_device(t->src[1])) return false; nrm.b = (const float *)dev_ptr(t->src[1]); t = t->src[0]; }
+        if (!take(t, GGML_OP_MUL) || !on_device(t->src[1]) || is_pending(t->src[1])) return false;
+        nrm.w = (const float *)dev_ptr(t->src[1]);
+        t = t->src[0];
+        if (t->op != GGML_OP_RMS_NORM && t->op != GGML_OP_NORM) return false;
+        if (!take(t, t->op)) return false;
+        nrm.kind = t->op == GGML_OP_RMS_NORM ? 1 : 2;
+        memcpy(&nrm.eps, t->op_params, 4);
+        if ((nrm.kind == 1 && nrm.b) || (nrm.kind == 2 && !nrm.b)) return false;
+        F = t->src[0];
+        if (is_pending(F) || !on_device(F)) return false;
+    } else if (!on_device(X)) return false;
+    size_t live = 0;
+    for (const PendingNode & p : g_pending) live += still_valid(p) ? 1 : 0;
+    if (used != live) return false;                       // something else is pending: not the block
+    const int d = (int)down->ne[0], ff = (int)down->ne[1], r = (int)fc1->ne[1];
+    if (up->ne[0] != d || up->ne[1] != ff || (gate && (gate->ne[0] != d || gate->ne[1] != ff)) || fc2->ne[0] != r || fc2->ne[1] != ff || fc1->ne[0] != P->ne[0] ||
+        X->ne[0] != d || idx->ne[0] != ff || axpy->ne[0] != d || !pi_k_sparse_ffn_supported(ff, r, d)) return false;
+    g_pending.clear();
+    ++g_stats.ffn_blocks_fused;
+    pi_workspace * ws = workspace(ff, d);
+    // The rectified predictor layer goes to a buffer of this library's own: its node's buffer is dead in the host's plan once fc2 has
+    // "run", and the allocator may have handed the same bytes to one of the vectors this launch writes (the logits, h).
+    static float * hidden = nullptr;
+    static int hidden_n = 0;
+    if (r > hidden_n) {
+        if (hidden) { BK_PI(pi_sync()); pi_free(hidden); }
+        hidden = (float *)pi_malloc(sizeof(float) * (size_t)r);
+        if (!hidden) die("predictor buffer");
+        hidden_n = r;
+    }
+    BK_PI(pi_k_gemv(fc1->type, dev_ptr(fc1), r, (int)fc1->ne[0], (const float *)dev_ptr(P), nullptr, PI_EPI_RELU, nullptr, nullptr, hidden, nullptr));
+    BK_PI(pi_k_sparse_ffn(dev_ptr(fc2), ff, r, hidden, g_threshold, dev_ptr(up), gate ? dev_ptr(gate) : nullptr, dev_ptr(down), d, (const float *)dev_ptr(F),
+                          nrm.kind ? &nrm : nullptr, PI_EPI_NONE, nullptr, nullptr, (float *)dev_ptr(axpy), (float *)dev_ptr(idx), (float *)dev_ptr(cur), nullptr, ws, nullptr));
+    return true;
+}
+
 }  // namespace
 
 extern "C" {
@@ -550,6 +768,7 @@ void ggml_init_cublas(void) {
     std::lock_guard<std::mutex> g(g_mu);
     if (g_loaded) return;
     g_loaded = pi_init(0) == PI_OK;
+    { const char * nf = getenv("GGML_CUDA_NO_FUSION"); g_fuse = !(nf && nf[0] == '1'); }
     if (!g_loaded) fprintf(stderr, "powerinfer-hip backend: no usable HIP device (%s)\n", pi_last_error());
 }
 bool ggml_cublas_loaded(void) { return g_loaded; }
@@ -583,6 +802,7 @@ void ggml_cuda_alloc_tensor(struct ggml_tensor * tensor) {
 }
 void ggml_cuda_free_data(struct ggml_tensor * tensor) {
     if (!tensor || !tensor->extra) return;
+    flush_pending();
     Extra * e = (Extra *)tensor->extra;
     tensor->extra = nullptr;
     if (is_ring(e)) return;                        // a per-evaluation address: nothing is owned
@@ -618,15 +838,18 @@ void ggml_cuda_set_scratch_size(size_t scratch_size) {
     g_scratch_size = scratch_size;
 }
 void ggml_cuda_free_scratch(void) {
+    flush_pending();
     std::lock_guard<std::mutex> g(g_mu);
     if (g_scratch) { pi_free(g_scratch); g_scratch = nullptr; }
     if (g_arena.base) { pi_sync(); pi_free(g_arena.base); g_arena.base = nullptr; g_arena.cap = 0; }
     g_scratch_offset = 0;
 }
 void ggml_cuda_copy_to_device(struct ggml_tensor * tensor) {
+    flush_pending();
     BK_PI(pi_memcpy_h2d(dev_ptr(tensor), tensor->data, nbytes(tensor)));
 }
 void ggml_cuda_copy_to_host(struct ggml_tensor * tensor) {
+    flush_pending();
     BK_PI(pi_sync());
     BK_PI(pi_memcpy_d2h(tensor->data, dev_ptr(tensor), nbytes(tensor)));
 }
@@ -671,17 +894,19 @@ bool ggml_cuda_compute_forward(struct ggml_compute_params * params, struct ggml_
     }
     if (params->ith != 0) return true;
     if (params->type == GGML_TASK_INIT || params->type == GGML_TASK_FINALIZE) return true;
-    bool ok = true;
-    switch (tensor->op) {
-        case GGML_OP_MUL_MAT:        ok = op_mul_mat(tensor); break;
-        case GGML_OP_MUL_MAT_SPARSE: ok = sparse_common(tensor, false); break;
-        case GGML_OP_AXPY:           ok = sparse_common(tensor, true); break;
-        case GGML_OP_ROPE:           ok = op_rope(tensor); break;
-        case GGML_OP_CPY: case GGML_OP_CONT: case GGML_OP_DUP: ok = op_cpy(tensor); break;
-        case GGML_OP_GET_ROWS:       ok = op_get_rows(tensor); break;
-        case GGML_OP_RESHAPE: case GGML_OP_VIEW: case GGML_OP_PERMUTE: case GGML_OP_TRANSPOSE: break;
-        default:                     ok = op_elementwise(tensor); break;
+    const bool view = tensor->op == GGML_OP_RESHAPE || tensor->op == GGML_OP_VIEW || tensor->op == GGML_OP_PERMUTE || tensor->op == GGML_OP_TRANSPOSE;
+    if (!view) {                                         // views do nothing and neither join nor break the window
+        if (deferrable(tensor)) { defer(tensor); return true; }
+        if (!g_pending.empty()) {
+            if (tensor->op == GGML_OP_AXPY && try_fused_ffn(tensor)) {
+                if (pi::check_launch("ggml_cuda_compute_forward") != PI_OK) die("kernel launch");
+                return true;
+            }
+            flush_pending();
+            if (deferrable(tensor)) { defer(tensor); return true; }      // its operands exist now: it may open the next window
+        }
     }
+    const bool ok = run_node(tensor);
     if (!ok) {
         // the phase protocol has no way to hand a node back after INIT was claimed: refuse loudly rather than compute wrongly
         fprintf(stderr, "powerinfer-hip backend: node '%s' (op %d) has a shape/type/stride this backend does not implement\n", tensor->name, (int)tensor->op);
@@ -692,5 +917,8 @@ bool ggml_cuda_compute_forward(struct ggml_compute_params * params, struct ggml_
 }
 
 ggml_backend_t ggml_backend_cuda_init(void) { return nullptr; }
+
+void pi_ggml_backend_get_stats(pi_ggml_backend_stats * out) { if (out) *out = g_stats; }
+void pi_ggml_backend_set_fusion(int enable) { flush_pending(); g_fuse = enable != 0; }
 
 }  // extern "C"

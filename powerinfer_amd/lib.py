@@ -99,6 +99,8 @@ _SIGS = {
     "pi_k_upgate_q4_hot_rows": (_i, [_i, _f, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_host_wait": (_i, [_vp, _vp, _i, _vp, C.c_double, _vp]),
     "pi_k_host_signal_wait": (_i, [_vp, _vp, _i, _i, _vp, C.c_double, _vp]),
+    "pi_ggml_backend_get_stats": (None, [_vp]),
+    "pi_ggml_backend_set_fusion": (None, [_i]),
     "pi_gemm_lib_create": (_vp, [C.c_size_t]),
     "pi_gemm_lib_destroy": (_i, [_vp]),
     "pi_gemm_lib_f16": (_i, [_vp, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),

@@ -215,3 +215,110 @@ def test_reference_executor_drives_this_backend(wtype, hot_frac):
         assert (err.min(0) < 1e-4 * scale).all(), f"host node ffn_down_sparse: errors vs (both, thread 0, thread 1) {err.max(1) / scale}"
         raced += int((err[0] >= 1e-4 * scale).sum())
     print(f"host axpy groups of 8 floats that lost one thread's share: {raced} of {T * d // 8}")
+
+
+def backend_stats(L):
+    st = (C.c_int64 * 3)()
+    L.pi_ggml_backend_get_stats(st)
+    return dict(deferred=int(st[0]), flushed=int(st[1]), fused=int(st[2]))
+
+
+def build_decode_ffn(G, L, norm, has_gate, spoiler=None):
+    """One token through llm_build_norm + llm_build_ffn_sparse (llama.cpp:4420-4450, 4652-4757) with every tensor on the device, in the
+    node order the reference's graph has.  norm: 0 none (the FFN reads the vector as it is, Falcon's order of things), 1 RMSNorm * w,
+    2 LayerNorm * w + b.  spoiler: name of a node after which an unrelated node (a SCALE) is slipped in, which must break the window."""
+    d, ff, r = L["d"], L["ff"], L["r"]
+    F = G.weight_to_gpu(G.new(0, [d, 1], L["x"][:1], "ffn_inp"))
+    rng = np.random.default_rng(4)
+    nw = (1 + 0.1 * rng.standard_normal(d)).astype(np.float32)
+    nb = (0.1 * rng.standard_normal(d)).astype(np.float32)
+    if norm:
+        cur = G.on_gpu(G.rms_norm(F, 1e-5, "norm") if norm == 1 else G.norm(F, 1e-5, "norm"))
+        cur = G.on_gpu(G.mul(cur, G.weight_to_gpu(G.new(0, [d], nw, "ffn_norm.weight")), "norm_w"))
+        if norm == 2:
+            cur = G.on_gpu(G.add(cur, G.weight_to_gpu(G.new(0, [d], nb, "ffn_norm.bias")), "ffn_norm"))
+    else:
+        cur = F
+    one = G.weight_to_gpu(G.new(0, [1], np.ones(1, np.float32), "one"))
+    extra = []
+
+    def node(t):
+        G.on_gpu(t)
+        if spoiler and t.name.decode() == spoiler:
+            extra.append(G.on_gpu(G.scale(F, one, "unrelated")))
+        return t
+    fc1 = G.weight_to_gpu(G.new(1, [d, r], L["fc1"], "fc1"))
+    fc2 = G.weight_to_gpu(G.new(1, [r, ff], L["fc2"], "fc2"))
+    W = {n: G.weight_to_gpu(G.new(1, [d, ff], L[n], n + "_gpu")) for n in (("up", "gate", "down_t") if has_gate else ("up", "down_t"))}
+    idx = node(G.mul_mat(fc1, F, "mlp_pre_hidden"))
+    idx = node(G.relu(idx, "mlp_pre_relu"))
+    idx = node(G.mul_mat(fc2, idx, "mlp_pre_out"))
+    up = node(G.mul_mat_idx(W["up"], cur, idx, None, "ffn_up_sparse"))
+    if has_gate:
+        gate = node(G.mul_mat_idx(W["gate"], cur, idx, None, "ffn_gate_sparse"))
+        act = node(G.relu(gate, "ffn_gate_act"))
+        h = node(G.mul(act, up, "ffn_gate_par"))
+    else:
+        h = node(G.relu(up, "ffn_up_act"))
+    out = node(G.axpy(W["down_t"], h, idx, None, "ffn_down_sparse"))
+    res = G.on_gpu(G.add(out, F, "l_out"))
+    xn = ol.apply_norm(L["x"][0], norm, nw, nb if norm == 2 else None, 1e-5)
+    return dict(idx=idx, h=h, out=out, res=res, xn=xn, extra=extra)
+
+
+@pytest.mark.parametrize("d,ff,r,has_gate,norm", [(4096, 11008, 1024, True, 1), (4096, 2048, 512, False, 2), (8192, 4096, 512, False, 0),
+                                                  (4096, 2048, 512, True, 0)])
+def test_ffn_block_of_one_token_is_one_fused_launch(d, ff, r, has_gate, norm):
+    """The node window of the boundary: the single-token sequence llm_build_ffn_sparse emits is held back node by node and computed as
+    pi_k_gemv + pi_k_sparse_ffn when its AXPY node arrives.  The output, the predictor logits and h are those of the node-by-node
+    evaluation (and of the CPU oracle under the same logits); the counters show the block went through the fused path once."""
+    from powerinfer_amd import lib as pl
+    from ggml_graph import Graph
+    Lc = pl.load()
+    L = synth.make_ffn_layer(seed=17, d=d, ff=ff, r=r, wtype=ol.F16, has_gate=has_gate, T=1)
+    got = {}
+    for fuse in (1, 0):
+        G = Graph(Lc)
+        Lc.pi_ggml_backend_set_fusion(fuse)
+        s0 = backend_stats(Lc)
+        B = build_decode_ffn(G, L, norm, has_gate)
+        G.compute(0.0)
+        assert not G.cpu_run, G.cpu_run
+        got[fuse] = {k: G.host(B[k]).copy() for k in ("idx", "h", "out", "res")}
+        s1 = backend_stats(Lc)
+        assert s1["fused"] - s0["fused"] == fuse
+        if fuse:
+            assert s1["deferred"] - s0["deferred"] >= (6 if has_gate else 5) + (0 if norm == 0 else norm + 1)
+        else:
+            assert s1["deferred"] == s0["deferred"]
+        lg = got[fuse]["idx"]
+        o = ol.ffn_under_logits(ol.oracle(), d, ff, ol.F16, has_gate, L["up"], L["gate"], L["down_t"], B["xn"], lg, 0.0)
+        assert rel_err(got[fuse]["out"], o["out"]) < 1e-4
+        assert rel_err(got[fuse]["h"], o["h"]) < 1e-4 if "h" in o else True
+        assert rel_err(got[fuse]["res"], o["out"] + L["x"][0]) < 1e-4
+    Lc.pi_ggml_backend_set_fusion(1)
+    assert rel_err(got[1]["idx"], got[0]["idx"]) < 1e-5
+    assert ((got[1]["idx"] >= 0) == (got[0]["idx"] >= 0)).mean() >= 0.999
+    assert np.array_equal(got[1]["h"] != 0, (got[1]["idx"] >= 0) & (got[1]["h"] != 0))     # h is zero wherever the predictor says inactive
+
+
+@pytest.mark.parametrize("spoiler", ["mlp_pre_out", "ffn_up_sparse", "ffn_gate_act"])
+def test_an_unrelated_node_breaks_the_window(spoiler):
+    """A node that is not part of the block arrives in the middle of it: everything pending runs, in order, before it, nothing is
+    fused, and every intermediate vector exists as in a node-by-node evaluation."""
+    from powerinfer_amd import lib as pl
+    from ggml_graph import Graph
+    Lc = pl.load()
+    d, ff, r = 4096, 2048, 512
+    L = synth.make_ffn_layer(seed=19, d=d, ff=ff, r=r, wtype=ol.F16, has_gate=True, T=1)
+    Lc.pi_ggml_backend_set_fusion(1)
+    G = Graph(Lc)
+    s0 = backend_stats(Lc)
+    B = build_decode_ffn(G, L, 1, True, spoiler=spoiler)
+    G.compute(0.0)
+    s1 = backend_stats(Lc)
+    assert s1["fused"] == s0["fused"] and s1["flushed"] > s0["flushed"]
+    lg = G.host(B["idx"])
+    o = ol.ffn_under_logits(ol.oracle(), d, ff, ol.F16, True, L["up"], L["gate"], L["down_t"], B["xn"], lg, 0.0)
+    assert rel_err(G.host(B["out"]), o["out"]) < 1e-4
+    assert rel_err(G.host(B["extra"][0]), L["x"][0]) == 0.0

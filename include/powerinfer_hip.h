@@ -388,6 +388,30 @@ PI_API int pi_k_batch_sparse_mul_mat(const void * W_f16, int ff, int cols, const
 PI_API int pi_k_batch_sparse_axpy(const void * down_t_f16, int cols, int ff, const float * h, const float * idx, int T, float threshold,
                                   float * out, int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream);
 
+/* pi_k_attn_fused with the cache cells of every head split over n_parts workgroups, for contexts whose K / V rows one workgroup per
+ * head cannot pull fast enough (a compute unit sustains about 1/256 of the HBM rate) or whose scores do not fit one workgroup's LDS:
+ * part s takes cells [n_kv * s / n_parts, n_kv * (s + 1) / n_parts), keeps (max, sum, weighted V sum) of its cells in `scratch`
+ * (pi_k_attn_split_scratch_floats floats), and a second small launch merges the parts in order.  Each part rounds exp() to fp16
+ * relative to its own maximum, as the CPU path does relative to the global one (ggml.c:10747-10759), so outputs differ from
+ * pi_k_attn_fused in the last places of those roundings.  n_seq sequences as pi_k_attn_fused_batch (1 with strides 0 for one).
+ * The reference runs K.q, scale, mask, soft-max and V.p as separate nodes (llm_build_kqv, llama.cpp:4764-4850). */
+PI_API int    pi_k_attn_split_supported(int hd, int n_ctx, int n_parts);
+PI_API size_t pi_k_attn_split_scratch_floats(int n_seq, int n_head, int hd, int n_parts);
+PI_API int    pi_k_attn_split(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache, size_t cache_seq_stride,
+                              int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, int n_parts, const int32_t * pos, float * scratch,
+                              float * out, int out_stride, void * out_f16, pi_stream_t stream);
+/* pi_k_attn_chunk (below) for contexts beyond its kernels (pi_k_attn_chunk_supported tells): RoPE + KV store of the chunk's T tokens, then
+ * each token's cells split as above (scratch: pi_k_attn_split_scratch_floats(T, ...)).  No K / V tile is shared between the tokens of the
+ * chunk, so a long prompt costs T passes over the cache per chunk: it is the path that works at any context, not a fast one. */
+PI_API int    pi_k_attn_chunk_supported(int hd, int n_ctx);
+PI_API int    pi_k_attn_chunk_long(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,
+                                   const int32_t * pos, int n_ctx, int n_parts, float * scratch, float * q_rot, void * k_cache, void * v_cache,
+                                   float * out, void * out_f16, pi_stream_t stream);
+/* the same for tokens whose K / V rows are in the cache already and whose q is rotated (a prompt chunk after pi_k_rope_kv_store):
+ * q_rot fp32 [n_tok][n_head * hd], token t attends to cells [0, pos[t]] of the one cache */
+PI_API int    pi_k_attn_split_cached(const float * q_rot, const void * k_cache, const void * v_cache, int n_tok, int n_head, int n_head_kv, int hd,
+                                     int n_ctx, int n_parts, const int32_t * pos, float * scratch, float * out, pi_stream_t stream);
+
 /* per-sequence pieces of a batched step: sequence t owns token t, position pos[t] and the cache at t * cache_seq_stride
  * (elements), out_f16 (optional) receives fp16(out); pi_k_argmax_batch picks each sequence's next token (first maximum wins), stores it in tokens[t], adds 1 to
  * positions[t] and records it at out_tokens[*step][t]; pi_k_step_advance then moves *step on. */

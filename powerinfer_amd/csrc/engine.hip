@@ -169,7 +169,10 @@ int layer_forward(pi_model * m, int il, bool last_token) {
     else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
     else an = make_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
     PI_TRY(pi_k_gemv(wqkv.type, wqkv.dev, d + 2 * gqa, d, x, &an, PI_EPI_NONE, nullptr, nullptr, m->qkv, st));
-    if (m->rope_table) {
+    if (m->attn_parts > 1) {
+        PI_TRY(pi_k_attn_split(m->qkv, 0, m->rope_table, m->k_cache + kv_off, m->v_cache + kv_off, 0, 1, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0,
+                               hp.n_ctx, m->attn_parts, m->d_pos, m->attn_scratch, m->att, 0, nullptr, st));
+    } else if (m->rope_table) {
         PI_TRY(pi_k_attn_fused(m->qkv, m->rope_table, m->k_cache + kv_off, m->v_cache + kv_off, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0,
                                hp.n_ctx, m->d_pos, m->att, st));
     } else {
@@ -694,13 +697,28 @@ int pi_model_finalize(pi_model * m) {
     PI_TRY(pi_memset(m->v_cache, 0, kv * 2));
     // fused RoPE + attention when the head geometry and the context fit its single-pass kernel (the launcher's own test);
     // otherwise the rope_kv_store + attn_decode pair, whose smaller workgroup leaves room for a longer context
-    if (pi_k_attn_fused_supported(m->hd, hp.n_ctx)) {
+    // Long contexts (1024 cells and up, or more than one workgroup's LDS holds): the cells of every head are split over as many
+    // workgroups as fill the chip (a compute unit pulls about 1/256 of the HBM rate, so one workgroup per head leaves the K / V rows
+    // of a long context to n_head units), at least as many as bring a part's scores into LDS.
+    const bool fused_ok = pi_k_attn_fused_supported(m->hd, hp.n_ctx) != 0;
+    if (!fused_ok || hp.n_ctx >= 1024) {
+        const int n_cu = pi::compute_units();
+        int parts = 2;
+        while (parts < 8 && parts * 2 * hp.n_head <= n_cu) parts *= 2;
+        while (parts < 64 && !pi_k_attn_split_supported(m->hd, hp.n_ctx, parts)) parts *= 2;
+        if (pi_k_attn_split_supported(m->hd, hp.n_ctx, parts)) {
+            m->attn_parts = parts;
+            m->attn_scratch = m->alloc<float>(pi_k_attn_split_scratch_floats(1, hp.n_head, m->hd, parts));
+            if (!m->attn_scratch) return PI_E_HIP;
+        }
+    }
+    if (fused_ok || m->attn_parts > 1) {
         m->rope_table = m->alloc<float>((size_t)hp.n_ctx * m->hd);
         if (!m->rope_table) return PI_E_HIP;
         PI_TRY(pi_k_rope_table(m->rope_table, hp.n_ctx, m->hd, hp.arch == PI_ARCH_FALCON ? 2 : 0, m->theta_scale, m->freq_scale, nullptr));
     }
     else if (!pi_k_attn_decode_supported(m->hd, hp.n_ctx))
-        return pi::fail(PI_E_UNSUPPORTED, "pi_model_finalize: head size or context outside both attention kernels (scores of every cell are kept in LDS: n_ctx up to about 13 000 at head size 128)");
+        return pi::fail(PI_E_UNSUPPORTED, "pi_model_finalize: head size or context outside every attention kernel (head size a multiple of 8 that divides 512, at most 64 parts of the context per head)");
     PI_TRY(pi_memset(m->n_active, 0, sizeof(int32_t) * hp.n_layer));
     PI_TRY(pi_memset(m->d_step, 0, 4));
     PI_TRY(pi_memset(m->h_dense, 0, sizeof(float) * ff));

@@ -44,6 +44,22 @@ pi_norm mk_norm(int kind, float eps, const Tensor & w, const Tensor * b) {
     return n;
 }
 
+// attention of a prompt chunk of the model's own sequence: the chunk kernels where the context fits them, the split-over-cells path beyond
+int chunk_attention(pi_model * m, BatchState * b, int T, size_t kv_off) {
+    const pi_hparams & hp = m->hp;
+    const int d = hp.n_embd, hd = m->hd, gqa = m->gqa, mode = hp.arch == PI_ARCH_FALCON ? 2 : 0;
+    if (pi_k_attn_chunk_supported(hd, hp.n_ctx))
+        return pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, mode, m->theta_scale, m->freq_scale, b->d_pos, hp.n_ctx, b->q_rot,
+                               m->k_cache + kv_off, m->v_cache + kv_off, b->att, d, b->att16, m->stream);
+    const int parts = m->attn_parts > 1 ? m->attn_parts : 2;
+    if (!m->attn_scratch_chunk) {
+        m->attn_scratch_chunk = m->alloc<float>(pi_k_attn_split_scratch_floats(512, hp.n_head, hd, parts));
+        if (!m->attn_scratch_chunk) return PI_E_HIP;
+    }
+    return pi_k_attn_chunk_long(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, mode, m->theta_scale, m->freq_scale, b->d_pos, hp.n_ctx, parts,
+                                m->attn_scratch_chunk, b->q_rot, m->k_cache + kv_off, m->v_cache + kv_off, b->att, b->att16, m->stream);
+}
+
 int batch_layer(pi_model * m, BatchState * b, int il) {
     const pi_hparams & hp = m->hp;
     const int T = b->n_seq, d = hp.n_embd, ff = hp.n_ff, hd = m->hd, gqa = m->gqa;
@@ -64,8 +80,7 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     PI_TRY(pi_k_norm_round_f16(x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));       // Falcon: the predictor reads the raw layer input
     PI_TRY(pi_k_gemm_f16(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr, st));
     if (b->prefill)
-        PI_TRY(pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, m->freq_scale, b->d_pos, hp.n_ctx, b->q_rot,
-                               m->k_cache + kv_off, m->v_cache + kv_off, b->att, d, b->att16, st));
+        PI_TRY(chunk_attention(m, b, T, kv_off));
     else
         PI_TRY(pi_k_attn_fused_batch(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
                                      hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, hp.n_ctx, b->d_pos, b->att, d, b->att16, st));
@@ -223,8 +238,7 @@ int wide_layer(pi_model * m, BatchState * b, int il) {
     PI_TRY(chunk_input(wqkv.type, x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));
     PI_TRY(chunk_weight(m, b, il, PI_T_WQKV, d + 2 * gqa, d, &W));
     PI_TRY(chunk_gemm(m, W, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr));
-    PI_TRY(pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, m->theta_scale, m->freq_scale, b->d_pos, hp.n_ctx, b->q_rot,
-                           m->k_cache + kv_off, m->v_cache + kv_off, b->att, d, b->att16, st));
+    PI_TRY(chunk_attention(m, b, T, kv_off));
     if (wo.type == PI_TYPE_Q4_0) PI_TRY(pi_k_norm_q8_round_f16(b->att, T, d, &plain, b->att16, nullptr, st));
     PI_TRY(chunk_weight(m, b, il, PI_T_WO, d, d, &W));
     pi_norm fn;
@@ -459,7 +473,7 @@ int pi_model_batch_init(pi_model * m, int n_seq) {
     if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_batch_init: model not finalized");
     if (n_seq < 1 || n_seq > 16) return pi::fail(PI_E_ARG, "pi_model_batch_init: 1 <= n_seq <= 16");
     if (m->batch) return pi::fail(PI_E_STATE, "pi_model_batch_init: already initialised");
-    if (!m->rope_table) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: head size or context outside the fused attention kernel (pi_k_attn_fused_supported)");
+    if (!m->rope_table || !pi_k_attn_fused_supported(m->hd, m->hp.n_ctx)) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: head size or context outside the fused attention kernel (pi_k_attn_fused_supported)");
     if (const char * why = batch_unsupported(m)) { pi::set_error(why); return PI_E_UNSUPPORTED; }
     BatchState * b = batch_alloc(m, n_seq, true);
     if (!b) return PI_E_HIP;

@@ -39,7 +39,10 @@ struct pi_model {
     int32_t *list = nullptr, *n_active = nullptr, *d_token = nullptr, *d_pos = nullptr, *d_step = nullptr;
     int32_t *d_out_tokens = nullptr, *d_out_active = nullptr;
     __half *k_cache = nullptr, *v_cache = nullptr;
-    float *rope_table = nullptr;          // float2 [n_ctx][hd/2] (cos, sin), when the fused attention kernel is used
+    float *rope_table = nullptr;          // float2 [n_ctx][hd/2] (cos, sin), when the fused or the split attention kernel is used
+    int    attn_parts = 1;                // > 1: the cells of every head are split over this many workgroups (long contexts)
+    float *attn_scratch = nullptr;        // partial results of those workgroups for one token
+    float *attn_scratch_chunk = nullptr;  // and for a prompt chunk (allocated at the first chunk that needs it)
 
     hipGraphExec_t graph_exec = nullptr;
     hipGraph_t graph = nullptr;

@@ -2698,6 +2698,188 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// Attention of one token with the cache cells of a head split over several workgroups (grid: head x part x sequence).  A compute unit
+// pulls about 1/256 of the chip's HBM rate, so one workgroup per head leaves the K / V rows of a long context to 32 or 128 units
+// (18 us per 7B layer at 600 cells, growing by 2.4 us per 100 cells); with n_parts workgroups per head every unit takes a share and
+// the score buffer in LDS holds n_ctx / n_parts cells instead of all of them.
+// Part s owns cells [n_kv * s / n, n_kv * (s + 1) / n); the last part holds the new cell: it rotates and stores k, stores v, and
+// uses them from LDS.  Every part rotates q, computes its scores, e_i = fp16(exp(fp16(s_i - m))) with ITS maximum m (the rounding
+// points of the CPU path's table, ggml.c:10747-10759), l = sum e_i in double and acc = sum v_i * e_i, and hands (m, l, acc) to
+// attn_merge_kernel, which rescales by exp(m - M), adds the parts in order and divides by the total.  Against one workgroup per head,
+// which knows the global maximum before it rounds, results differ in the last places of the fp16 roundings (1e-4 of the output).
+// ---------------------------------------------------------------------------------------------------
+// FROM_CACHE: the token's own K / V row is in the cache already and qkv holds its rotated q only ([n_head * hd] per token; a prompt chunk
+// behind rope_kv_store_kernel): nothing is rotated or stored, every cell is read from the cache.
+constexpr int kAttnPartBlock = 512;
+constexpr int kAttnPartPre = 4;
+template <bool FROM_CACHE>
+__global__ __launch_bounds__(kAttnPartBlock) void attn_part_kernel(const float * __restrict__ qkv, const float2 * __restrict__ rope_table,
+                                                                   __half * __restrict__ k_cache, __half * __restrict__ v_cache,
+                                                                   int n_head, int n_head_kv, int hd, int mode, int n_ctx, int s_cap,
+                                                                   const int32_t * __restrict__ pos_p, float * __restrict__ part_acc, float * __restrict__ part_ml,
+                                                                   int qkv_stride, size_t cache_seq_stride) {
+    qkv += (size_t)blockIdx.z * qkv_stride;
+    k_cache += (size_t)blockIdx.z * cache_seq_stride;
+    v_cache += (size_t)blockIdx.z * cache_seq_stride;
+    pos_p += blockIdx.z;
+    extern __shared__ __align__(16) unsigned char smem[];
+    float * s    = reinterpret_cast<float *>(smem);               // [s_cap] scores of this part, then e_i
+    float * part = s + s_cap;                                     // [groups][hd]
+    float * qs   = part + (kAttnPartBlock / (hd / 8)) * hd;       // [hd] rotated q, rounded to fp16
+    float * kcur = qs + hd;                                       // [hd] rotated k of this position, rounded to fp16
+    float * vcur = kcur + hd;                                     // [hd]
+    __shared__ double red[16];
+    __shared__ float redf[16];
+    const int h = blockIdx.x, n_parts = gridDim.y, sp = blockIdx.y, grp_sz = n_head / n_head_kv, kvh = h / grp_sz;
+    const int tid = threadIdx.x;
+    const int pos = *pos_p, n_kv = pos + 1;
+    const int lo = (int)((long long)n_kv * sp / n_parts), hi = (int)((long long)n_kv * (sp + 1) / n_parts);
+    const bool owns_new = !FROM_CACHE && sp == n_parts - 1;        // hi == n_kv: the new cell is this part's last
+    const size_t slot = ((size_t)blockIdx.z * n_head + h) * n_parts + sp;
+    if (hi - lo > s_cap) return;                                  // cannot happen for pos < n_ctx (the launcher sizes s_cap); never write past LDS
+    const float * qsrc = qkv + (size_t)h * hd;
+    const float * ksrc = qkv + (size_t)(n_head + kvh) * hd;
+    const float * vsrc = qkv + (size_t)(n_head + n_head_kv + kvh) * hd;
+    const int lpp = hd / 8;
+    const int sub = tid % lpp, grp = tid / lpp, ngrp = kAttnPartBlock / lpp;
+    const __half * kb = k_cache + (size_t)kvh * n_ctx * hd;
+    const __half * vb = v_cache + (size_t)kvh * n_ctx * hd;
+    const int n_old = (owns_new ? hi - 1 : hi) - lo;              // cells of this part that live in the cache
+    pi_u32x4 kpre[kAttnPartPre], vpre[kAttnPartPre];
+#pragma unroll
+    for (int i = 0; i < kAttnPartPre; ++i) {
+        const int c = i * ngrp + grp;
+        if (c < n_old) { kpre[i] = pi_ld16(kb + (size_t)(lo + c) * hd + sub * 8); vpre[i] = pi_ld16(vb + (size_t)(lo + c) * hd + sub * 8); }
+    }
+    if (FROM_CACHE) {
+        if (tid < hd) qs[tid] = pi_round_f16(qsrc[tid]);
+    } else if (tid < hd / 2) {
+        const float2 cs = rope_table[(size_t)pos * (hd / 2) + tid];
+        const int i0 = (mode & 2) ? tid : 2 * tid;
+        const int i1 = (mode & 2) ? tid + hd / 2 : 2 * tid + 1;
+        const float q0 = qsrc[i0], q1 = qsrc[i1];
+        qs[i0] = pi_round_f16(__fsub_rn(__fmul_rn(q0, cs.x), __fmul_rn(q1, cs.y)));
+        qs[i1] = pi_round_f16(__fadd_rn(__fmul_rn(q0, cs.y), __fmul_rn(q1, cs.x)));
+        if (owns_new) {
+            const float k0 = ksrc[i0], k1 = ksrc[i1];
+            const __half ka = __float2half_rn(__fsub_rn(__fmul_rn(k0, cs.x), __fmul_rn(k1, cs.y)));
+            const __half kc = __float2half_rn(__fadd_rn(__fmul_rn(k0, cs.y), __fmul_rn(k1, cs.x)));
+            kcur[i0] = __half2float(ka); kcur[i1] = __half2float(kc);
+            if ((h % grp_sz) == 0) { __half * kdst = k_cache + ((size_t)kvh * n_ctx + pos) * hd; kdst[i0] = ka; kdst[i1] = kc; }
+        }
+    } else if (owns_new && tid < hd / 2 + hd) {
+        const int e = tid - hd / 2;
+        const __half v = __float2half_rn(vsrc[e]);
+        vcur[e] = __half2float(v);
+        if ((h % grp_sz) == 0) v_cache[((size_t)kvh * n_ctx + pos) * hd + e] = v;
+    }
+    __syncthreads();
+
+    const float scale = pi_inv_sqrt((float)hd);
+    const int n_mine = hi - lo;
+    float qf[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) qf[i] = qs[sub * 8 + i];
+#pragma unroll
+    for (int i = 0; i < kAttnPartPre; ++i) {
+        if (i * ngrp < n_mine) {
+            const int c = i * ngrp + grp;
+            float d = 0.0f;
+            if (c < n_old) d = pi_dot8(kpre[i], qf, 0.0f);
+            else if (c < n_mine) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) d = fmaf(kcur[sub * 8 + k], qf[k], d);
+            }
+            for (int o = lpp / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, PI_WAVE);
+            if (c < n_mine && sub == 0) s[c] = __fmul_rn(d, scale);
+        }
+    }
+    for (int c0 = kAttnPartPre * ngrp; c0 < n_mine; c0 += ngrp) {
+        const int c = c0 + grp;
+        float d = 0.0f;
+        if (c < n_old) d = pi_dot8(pi_ld16(kb + (size_t)(lo + c) * hd + sub * 8), qf, 0.0f);
+        else if (c < n_mine) {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) d = fmaf(kcur[sub * 8 + i], qf[i], d);
+        }
+        for (int o = lpp / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, PI_WAVE);
+        if (c < n_mine && sub == 0) s[c] = __fmul_rn(d, scale);
+    }
+    __syncthreads();
+
+    float mx = -INFINITY;
+    for (int c = tid; c < n_mine; c += kAttnPartBlock) mx = fmaxf(mx, s[c]);
+    mx = block_max_f32(mx, redf);
+    double sum = 0.0;
+    for (int c = tid; c < n_mine; c += kAttnPartBlock) {
+        const float e = pi_round_f16(expf(pi_round_f16(__fsub_rn(s[c], mx))));
+        s[c] = e;
+        sum += (double)e;
+    }
+    sum = block_sum_f64(sum, red);
+
+    float acc[8];
+#pragma unroll
+    for (int i = 0; i < 8; ++i) acc[i] = 0.0f;
+#pragma unroll
+    for (int i = 0; i < kAttnPartPre; ++i) {
+        const int c = i * ngrp + grp;
+        if (c < n_mine) {
+            const float p = s[c];
+            float vf[8];
+            if (c < n_old) pi_unpack8(vpre[i], vf);
+            else {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) vf[k] = vcur[sub * 8 + k];
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) acc[k] = fmaf(vf[k], p, acc[k]);
+        }
+    }
+    for (int c = kAttnPartPre * ngrp + grp; c < n_mine; c += ngrp) {
+        const float p = s[c];
+        float vf[8];
+        if (c < n_old) pi_unpack8(pi_ld16(vb + (size_t)(lo + c) * hd + sub * 8), vf);
+        else {
+#pragma unroll
+            for (int i = 0; i < 8; ++i) vf[i] = vcur[sub * 8 + i];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) acc[i] = fmaf(vf[i], p, acc[i]);
+    }
+#pragma unroll
+    for (int i = 0; i < 8; ++i) part[grp * hd + sub * 8 + i] = acc[i];
+    __syncthreads();
+    for (int e = tid; e < hd; e += kAttnPartBlock) {
+        float v = part[e];
+        for (int g = 1; g < ngrp; ++g) v += part[g * hd + e];
+        part_acc[slot * hd + e] = v;
+    }
+    if (tid == 0) { part_ml[slot * 2] = n_mine > 0 ? mx : -INFINITY; part_ml[slot * 2 + 1] = (float)sum; }
+}
+
+// out[h][e] = sum_s acc_s[e] * exp(m_s - M) / sum_s l_s * exp(m_s - M), parts in ascending order; one workgroup of hd threads per head
+__global__ void attn_merge_kernel(const float * __restrict__ part_acc, const float * __restrict__ part_ml, int n_parts, int hd,
+                                  float * __restrict__ out, int out_stride, __half * __restrict__ out16) {
+    const int h = blockIdx.x, n_head = gridDim.x, e = threadIdx.x;
+    const size_t slot0 = ((size_t)blockIdx.y * n_head + h) * n_parts;
+    float M = -INFINITY;
+    for (int sp = 0; sp < n_parts; ++sp) M = fmaxf(M, part_ml[(slot0 + sp) * 2]);
+    float L = 0.0f, v = 0.0f;
+    for (int sp = 0; sp < n_parts; ++sp) {
+        const float m = part_ml[(slot0 + sp) * 2], l = part_ml[(slot0 + sp) * 2 + 1];
+        if (l > 0.0f) {
+            const float w = expf(__fsub_rn(m, M));
+            L = fmaf(l, w, L);
+            v = fmaf(part_acc[(slot0 + sp) * hd + e], w, v);
+        }
+    }
+    v = pi_div(v, L);
+    out[(size_t)blockIdx.y * out_stride + (size_t)h * hd + e] = v;
+    if (out16) out16[(size_t)blockIdx.y * out_stride + (size_t)h * hd + e] = __float2half_rn(v);
+}
+
 __global__ void embed_f16_kernel(const __half * __restrict__ table, int cols, const int32_t * __restrict__ token, float * __restrict__ x) {
     const __half * row = table + (size_t)(*token) * cols;
     for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < cols; i += gridDim.x * blockDim.x) x[i] = __half2float(row[i]);
@@ -4688,6 +4870,49 @@ int pi_k_attn_fused(const float * qkv, const void * rope_table, void * k_cache, 
     return pi::check_launch("pi_k_attn_fused");
 }
 
+// ---- attention with the cells of a head split over n_parts workgroups --------------------------------------------
+static size_t attn_part_lds_bytes(int hd, int s_cap) {
+    return sizeof(float) * ((size_t)s_cap + (size_t)(kAttnPartBlock / (hd / 8)) * hd + 3 * (size_t)hd);
+}
+static bool attn_part_geometry_ok(int hd) {
+    return hd > 0 && hd % 8 == 0 && kAttnPartBlock % (hd / 8) == 0 && PI_WAVE % (hd / 8) == 0 && hd / 2 + hd <= kAttnPartBlock && hd <= 1024;
+}
+int pi_k_attn_split_supported(int hd, int n_ctx, int n_parts) {
+    return attn_part_geometry_ok(hd) && n_ctx > 0 && n_parts >= 1 && n_parts <= 64 && attn_part_lds_bytes(hd, (n_ctx + n_parts - 1) / n_parts + 1) <= kAttnLdsLimit;
+}
+size_t pi_k_attn_split_scratch_floats(int n_seq, int n_head, int hd, int n_parts) { return (size_t)n_seq * n_head * n_parts * ((size_t)hd + 2); }
+
+int pi_k_attn_split(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache, size_t cache_seq_stride,
+                    int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, int n_parts, const int32_t * pos, float * scratch,
+                    float * out, int out_stride, void * out_f16, pi_stream_t stream) {
+    if (!qkv || !rope_table || !k_cache || !v_cache || !pos || !out || !scratch || n_seq <= 0) return pi::fail(PI_E_ARG, "pi_k_attn_split: bad arguments");
+    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || (mode != 0 && mode != 2) || !pi_k_attn_split_supported(hd, n_ctx, n_parts))
+        return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_split: head size, context per part or part count outside the kernel (pi_k_attn_split_supported)");
+    const int s_cap = (n_ctx + n_parts - 1) / n_parts + 1;
+    float * acc = scratch;
+    float * ml = scratch + (size_t)n_seq * n_head * n_parts * hd;
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(attn_part_kernel<false>, dim3(n_head, n_parts, n_seq), dim3(kAttnPartBlock), attn_part_lds_bytes(hd, s_cap), st, qkv, (const float2 *)rope_table,
+                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, s_cap, pos, acc, ml, qkv_stride, cache_seq_stride);
+    hipLaunchKernelGGL(attn_merge_kernel, dim3(n_head, n_seq), dim3(hd), 0, st, acc, ml, n_parts, hd, out, out_stride, (__half *)out_f16);
+    return pi::check_launch("pi_k_attn_split");
+}
+
+int pi_k_attn_split_cached(const float * q_rot, const void * k_cache, const void * v_cache, int n_tok, int n_head, int n_head_kv, int hd,
+                           int n_ctx, int n_parts, const int32_t * pos, float * scratch, float * out, pi_stream_t stream) {
+    if (!q_rot || !k_cache || !v_cache || !pos || !out || !scratch || n_tok <= 0 || n_tok > 65535) return pi::fail(PI_E_ARG, "pi_k_attn_split_cached: bad arguments");
+    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || !pi_k_attn_split_supported(hd, n_ctx, n_parts))
+        return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_split_cached: head size, context per part or part count outside the kernel (pi_k_attn_split_supported)");
+    const int s_cap = (n_ctx + n_parts - 1) / n_parts + 1;
+    float * acc = scratch;
+    float * ml = scratch + (size_t)n_tok * n_head * n_parts * hd;
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(attn_part_kernel<true>, dim3(n_head, n_parts, n_tok), dim3(kAttnPartBlock), attn_part_lds_bytes(hd, s_cap), st, q_rot, (const float2 *)nullptr,
+                       (__half *)const_cast<void *>(k_cache), (__half *)const_cast<void *>(v_cache), n_head, n_head_kv, hd, 0, n_ctx, s_cap, pos, acc, ml, n_head * hd, (size_t)0);
+    hipLaunchKernelGGL(attn_merge_kernel, dim3(n_head, n_tok), dim3(hd), 0, st, acc, ml, n_parts, hd, out, n_head * hd, (__half *)nullptr);
+    return pi::check_launch("pi_k_attn_split_cached");
+}
+
 int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache, size_t cache_seq_stride,
                           int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, const int32_t * pos, float * out, int out_stride,
                           void * out_f16, pi_stream_t stream) {
@@ -4734,6 +4959,33 @@ int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_
     hipLaunchKernelGGL(attn_decode_kernel, dim3(n_head, T), dim3(kBlock), sh, st,
                        q_rot, (const __half *)k_cache, (const __half *)v_cache, n_head, n_head_kv, hd, n_ctx, pos, out, n_head * hd, out_stride, (__half *)out_f16);
     return pi::check_launch("pi_k_attn_chunk");
+}
+
+int pi_k_attn_chunk_supported(int hd, int n_ctx) {
+    if (hd <= 0 || hd % 8 || kBlock % (hd / 8) || PI_WAVE % (hd / 8) || n_ctx <= 0) return 0;
+    const int s_stride = ((n_ctx + 31) & ~31) + 4;
+    const size_t sh_mfma = sizeof(float) * 16 * (size_t)s_stride + (size_t)kWavesPerBlock * hd * kAcVtStride * 2;
+    if ((hd == 128 || hd == 64) && sh_mfma <= 156 * 1024) return 1;
+    return sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd) <= 60 * 1024;
+}
+
+// pi_k_attn_chunk for contexts beyond its kernels: RoPE + KV store of the chunk, then every token's cells split over n_parts workgroups
+int pi_k_attn_chunk_long(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,
+                         const int32_t * pos, int n_ctx, int n_parts, float * scratch, float * q_rot, void * k_cache, void * v_cache,
+                         float * out, void * out_f16, pi_stream_t stream) {
+    if (!qkv || !pos || !q_rot || !k_cache || !v_cache || !out || !scratch || T <= 0 || T > kChunkMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_chunk_long: bad arguments");
+    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || (mode != 0 && mode != 2) || hd % 2 || hd / 2 > 1024 || !pi_k_attn_split_supported(hd, n_ctx, n_parts))
+        return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_chunk_long: head size, context per part or part count outside the kernel (pi_k_attn_split_supported)");
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(rope_kv_store_kernel, dim3(n_head + 2 * n_head_kv, T), dim3(hd / 2), 0, st,
+                       qkv, n_head, n_head_kv, hd, mode, theta_scale, freq_scale, pos, n_ctx, q_rot, (__half *)k_cache, (__half *)v_cache, qkv_stride, n_head * hd);
+    const int s_cap = (n_ctx + n_parts - 1) / n_parts + 1;
+    float * acc = scratch;
+    float * ml = scratch + (size_t)T * n_head * n_parts * hd;
+    hipLaunchKernelGGL(attn_part_kernel<true>, dim3(n_head, n_parts, T), dim3(kAttnPartBlock), attn_part_lds_bytes(hd, s_cap), st, q_rot, (const float2 *)nullptr,
+                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, 0, n_ctx, s_cap, pos, acc, ml, n_head * hd, (size_t)0);
+    hipLaunchKernelGGL(attn_merge_kernel, dim3(n_head, T), dim3(hd), 0, st, acc, ml, n_parts, hd, out, n_head * hd, (__half *)out_f16);
+    return pi::check_launch("pi_k_attn_chunk_long");
 }
 
 int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float theta_scale, float freq_scale, const int32_t * delta, int n_cells, pi_stream_t stream) {

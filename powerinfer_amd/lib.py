@@ -106,6 +106,12 @@ _SIGS = {
     "pi_gemm_lib_f16": (_i, [_vp, _vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_batch_sparse_mul_mat": (_i, [_vp, _i, _i, _vp, _i, _vp, _f, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_batch_sparse_axpy": (_i, [_vp, _i, _i, _vp, _vp, _i, _f, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_attn_split_supported": (_i, [_i, _i, _i]),
+    "pi_k_attn_split_scratch_floats": (_sz, [_i, _i, _i, _i]),
+    "pi_k_attn_split": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _vp, _vp]),
+    "pi_k_attn_chunk_supported": (_i, [_i, _i]),
+    "pi_k_attn_chunk_long": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _f, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_attn_split_cached": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "pi_k_attn_fused_batch": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),
     "pi_k_attn_chunk": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _f, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     "pi_k_embed_batch": (_i, [_vp, _i, _vp, _i, _vp, _vp]),

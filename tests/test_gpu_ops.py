@@ -250,6 +250,80 @@ def test_attention_long_context(mode, hd, nh, nkv):
             assert np.array_equal(after[:, untouched], kg[:, untouched])
 
 
+@pytest.mark.parametrize("mode,hd,nh,nkv,n_ctx,parts", [(0, 128, 4, 4, 8192, 8), (2, 64, 8, 2, 32768, 4), (0, 128, 2, 1, 32768, 16)])
+def test_attention_split_over_cells(mode, hd, nh, nkv, n_ctx, parts):
+    """pi_k_attn_split: the cells of every head divided among `parts` workgroups and merged by a second launch, at contexts of 8 k and 32 k
+    cells that one workgroup's LDS cannot hold.  Positions with fewer cells than parts (empty parts), around the prefetch boundary of a
+    part and at the end of the context are compared with the oracle; where the single-workgroup kernel can run, the two agree to the
+    last places of the fp16 roundings; and only the new cell is written.  The chunk form (K / V already stored, q already rotated)
+    must return the same numbers as the decode form."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    O = ol.oracle()
+    rng = np.random.default_rng(7 * mode + hd + parts)
+    gqa, d = nkv * hd, nh * hd
+    assert L.pi_k_attn_split_supported(hd, n_ctx, parts) == 1 and L.pi_k_attn_fused_supported(hd, n_ctx) == 0
+    theta_scale = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
+    tab = pl.DevBuf(n_ctx * hd * 4)
+    pl.check(L.pi_k_rope_table(tab.ptr, n_ctx, hd, mode, theta_scale, 1.0, None), "rope_table")
+    kfill = (rng.standard_normal((n_ctx, nkv, hd)) * 0.5).astype(np.float16)
+    vfill = (rng.standard_normal((n_ctx, nkv, hd)) * 0.5).astype(np.float16)
+    kg = np.ascontiguousarray(kfill.transpose(1, 0, 2))
+    vg = np.ascontiguousarray(vfill.transpose(1, 0, 2))
+    kc_o = np.ascontiguousarray(kfill.reshape(n_ctx, gqa)).view(np.uint16)
+    vc_o = np.ascontiguousarray(vfill.reshape(n_ctx, gqa).T).view(np.uint16)
+    scratch = pl.DevBuf(4 * L.pi_k_attn_split_scratch_floats(1, nh, hd, parts))
+    per_pass = 512 // (hd // 8)
+    for pos in (0, 1, parts - 1, parts + 3, 4 * per_pass * parts - 1, 4 * per_pass * parts + 77, 5000, n_ctx - 1):
+        qkv = rng.standard_normal(d + 2 * gqa).astype(np.float32)
+        q, k, v = qkv[:d], qkv[d:d + gqa], qkv[d + gqa:]
+        p = np.array([pos], np.int32)
+        qr, kr = np.zeros_like(q), np.zeros_like(k)
+        O.pio_rope(P(q), hd, nh, 1, P(p), hd, mode, 10000.0, 1.0, P(qr))
+        O.pio_rope(P(k), hd, nkv, 1, P(p), hd, mode, 10000.0, 1.0, P(kr))
+        n_kv = pos + 1
+        mask = np.zeros((1, n_kv), np.float32)
+        want = np.zeros(d, np.float32)
+        ko, vo = kc_o.copy(), vc_o.copy()
+        assert O.pio_attention(hd, nh, nkv, n_ctx, n_kv, 1, P(p), P(mask), P(qr), P(kr), P(np.ascontiguousarray(v)), P(ko), P(vo), P(want)) == 0
+        dq, dpos = pl.DevBuf(host=qkv), pl.DevBuf(host=p)
+        kc, vc, dout = pl.DevBuf(host=kg), pl.DevBuf(host=vg), pl.DevBuf(d * 4)
+        pl.check(L.pi_k_attn_split(dq.ptr, 0, tab.ptr, kc.ptr, vc.ptr, 0, 1, nh, nkv, hd, mode, n_ctx, parts, dpos.ptr, scratch.ptr, dout.ptr, 0, None, None), "attn_split")
+        pl.sync()
+        got = dout.download(np.float32)
+        assert rel_err(got, want) < 2e-3, (pos, rel_err(got, want))
+        after_k = kc.download(np.float16).reshape(nkv, n_ctx, hd)
+        untouched = np.ones(n_ctx, bool); untouched[pos] = False
+        assert np.array_equal(after_k[:, untouched], kg[:, untouched])
+        assert np.array_equal(vc.download(np.float16).reshape(nkv, n_ctx, hd)[:, untouched], vg[:, untouched])
+        # the chunk form on the cache the decode form left behind (the new cell is in it now)
+        dqr, dout2 = pl.DevBuf(host=qr), pl.DevBuf(d * 4)
+        pl.check(L.pi_k_attn_split_cached(dqr.ptr, kc.ptr, vc.ptr, 1, nh, nkv, hd, n_ctx, parts, dpos.ptr, scratch.ptr, dout2.ptr, None), "attn_split_cached")
+        pl.sync()
+        assert rel_err(dout2.download(np.float32), got) < 1e-5, pos
+    # against the single-workgroup kernel, at a context both can run
+    n_small = 2048
+    tab2 = pl.DevBuf(n_small * hd * 4)
+    pl.check(L.pi_k_rope_table(tab2.ptr, n_small, hd, mode, theta_scale, 1.0, None), "rope_table")
+    kg2, vg2 = np.ascontiguousarray(kg[:, :n_small]), np.ascontiguousarray(vg[:, :n_small])
+    for pos in (5, 700, n_small - 1):
+        qkv = rng.standard_normal(d + 2 * gqa).astype(np.float32)
+        dq, dpos = pl.DevBuf(host=qkv), pl.DevBuf(host=np.array([pos], np.int32))
+        outs = []
+        for split in (False, True):
+            kc, vc, dout = pl.DevBuf(host=kg2), pl.DevBuf(host=vg2), pl.DevBuf(d * 4)
+            if split:
+                pl.check(L.pi_k_attn_split(dq.ptr, 0, tab2.ptr, kc.ptr, vc.ptr, 0, 1, nh, nkv, hd, mode, n_small, parts, dpos.ptr, scratch.ptr, dout.ptr, 0, None, None), "attn_split")
+            else:
+                pl.check(L.pi_k_attn_fused(dq.ptr, tab2.ptr, kc.ptr, vc.ptr, nh, nkv, hd, mode, n_small, dpos.ptr, dout.ptr, None), "attn_fused")
+            pl.sync()
+            outs.append(dout.download(np.float32))
+        # each part rounds its exp arguments to fp16 relative to its own maximum, the single workgroup relative to the global one:
+        # the two differ by those roundings (a few 2^-11 of a score), no more
+        assert rel_err(outs[1], outs[0]) < 1.5e-3, (pos, rel_err(outs[1], outs[0]))
+    assert L.pi_k_attn_split_supported(hd, n_ctx, 65) == 0 and L.pi_k_attn_split_supported(24, n_ctx, parts) == 0
+
+
 def test_embed_and_argmax():
     from powerinfer_amd import lib as pl
     L = pl.init()

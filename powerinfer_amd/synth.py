@@ -53,6 +53,47 @@ def predictor_fc2_margin(ff, r, p, rng, sigma=0.02, kappa=0.5):
     return (eps + (b / np.sqrt(r)).astype(np.float32)[:, None]).astype(np.float16)
 
 
+# ---- a predictor whose active set moves with the token and still keeps a margin -------------------------------------------------
+# Five coordinates of the residual stream are a side channel (MARK_DIMS): coordinate d-5 carries a constant for every token, coordinates
+# d-4 .. d-1 carry a constant for token 0 .. 3 only (make_model writes them into the embeddings, keeps the attention output and the
+# down projection away from them and hides them from the output matrix).  Five rows of fc1 read those coordinates, so the last five
+# hidden units are MARK_GAIN * MARK_VALUE for the constant one and for the current token's own one (tokens 0..3), about zero otherwise.
+MARK_DIMS, MARK_VALUE, MARK_GAIN = 5, 1.0, 8.0          # small enough to leave the norms alone (nothing else writes the channel: no noise to beat)
+
+
+def predictor_fc2_moving(ff, r, p, rng, sigma=0.02, kappa=0.5, group_div=48):
+    """Two classes of rows.  Four groups of ff // group_div neurons read only the marker units: row = g * (e_t - e_c / 2) for
+    group t, so logit = g * MARK_GAIN * MARK_VALUE * (+1/2 if the current token is t, -1/2 otherwise): the group is active exactly
+    while token t is being decoded (tokens 0..3, which is where the greedy path of a head_pair model lives), with a margin that does
+    not depend on the layer or the input.  The other rows are predictor_fc2_margin's static-sign rows over the ordinary units, of
+    which round(mean * ff) - ff // group_div are active for every token, so that a decoding step fires about mean * ff neurons.
+    (With larger groups the token's own group dominates the block's output and the greedy path of a synthetic model settles on one
+    token at once.)  Returns (fc2 fp16 [ff][r], rates [ff]): the rate of a moving neuron is 1/4 in groups 0 and 1 and next to nothing
+    in groups 2 and 3, so that a split by rate (gpu_split) puts the first two on the device and the other two with the host share,
+    which then has rows to compute whenever token 2 or 3 is decoded."""
+    g = ff // group_div
+    moving = np.sort(rng.permutation(ff)[:4 * g])
+    static = np.setdiff1d(np.arange(ff), moving)
+    n_on = max(int(round(float(np.mean(p)) * ff)) - g, 1)
+    on = np.zeros(ff, bool)
+    on[static[np.argsort(-p[static], kind="stable")[:n_on]]] = True
+    ro = r - MARK_DIMS                                                     # ordinary hidden units
+    b = np.where(on, 1.0, -1.0) * sigma * np.sqrt(np.pi) * (0.5 + rng.random(ff))
+    eps = (rng.random((ff, ro), dtype=np.float32) * 2 - 1) * (kappa * np.abs(b) / np.sqrt(ro)).astype(np.float32)[:, None]
+    w = np.zeros((ff, r), np.float32)
+    w[:, :ro] = eps + (b / np.sqrt(ro)).astype(np.float32)[:, None]
+    gain = np.float32(0.25)
+    for t in range(4):
+        rows = moving[t * g:(t + 1) * g]
+        w[rows] = 0.0
+        w[rows, ro] = -0.5 * gain                                          # the constant marker
+        w[rows, ro + 1 + t] = gain                                         # token t's marker
+    rates = np.where(on, 0.98, 1e-4)
+    rates[moving[:2 * g]] = 0.25
+    rates[moving[2 * g:]] = 1e-5            # groups 2 and 3 pass for rarely active: a hot/cold split by rate leaves them to the host
+    return w.astype(np.float16), rates
+
+
 def quantize_q4_0(x):
     """ggml Q4_0 (ggml-quants.c:428-463) in numpy: float32 [..., n] -> uint8 [..., n/32*18]."""
     x = np.ascontiguousarray(x, np.float32)
@@ -160,28 +201,50 @@ def make_model(hp):
             output[2 * k], output[2 * k + 1] = w.astype(np.float16), (-w).astype(np.float16)
         for t in range(4):
             tok_embd[t] = (tok_embd[t].astype(np.float32) * np.float32(0.05)).astype(np.float16)
+    moving = bool(hp.get("pred_moving"))
+    if moving:
+        assert hp.get("head_pair"), "pred_moving marks tokens 0..3, the tokens a head_pair model decodes"
+        tok_embd[:, d - MARK_DIMS:] = 0
+        tok_embd[:, d - MARK_DIMS] = MARK_VALUE
+        for t in range(4):
+            tok_embd[t, d - MARK_DIMS + 1 + t] = MARK_VALUE
+        output[:, d - MARK_DIMS:] = 0                                      # the greedy choice does not look at the side channel
     glob = dict(tok_embd=enc(tok_embd), output_norm=np.ones(d, np.float32), output=enc(output))
     if falcon:
         glob["output_norm_b"] = np.zeros(d, np.float32)
     layers = []
     for _ in range(hp.n_layer):
         L = dict(attn_norm=np.ones(d, np.float32))
+        def blind(w):                                                      # a matrix that does not read the side channel
+            if moving:
+                w[:, d - MARK_DIMS:] = 0
+            return w
         if falcon:
             L["attn_norm_b"] = np.zeros(d, np.float32)
             if hp.n_head_kv != hp.n_head and hp.get("two_norms", True):
                 L["attn_norm_2"] = np.ones(d, np.float32)
                 L["attn_norm_2_b"] = np.zeros(d, np.float32)
-            L["wqkv"] = enc(nrm(d + 2 * gqa, d))
+            L["wqkv"] = enc(blind(nrm(d + 2 * gqa, d)))
         else:
-            L["wq"], L["wk"], L["wv"] = enc(nrm(d, d)), enc(nrm(gqa, d)), enc(nrm(gqa, d))
+            L["wq"], L["wk"], L["wv"] = enc(blind(nrm(d, d))), enc(blind(nrm(gqa, d))), enc(blind(nrm(gqa, d)))
             L["ffn_norm"] = np.ones(d, np.float32)
-            L["ffn_gate"] = enc(nrm(ff, d))
-        L["wo"] = enc(nrm(d, d))
-        L["ffn_up"] = enc(nrm(ff, d))
-        L["ffn_down_t"] = enc(nrm(ff, d))
-        L["fc1"] = nrm(r, d)
+            L["ffn_gate"] = enc(blind(nrm(ff, d)))
+        wo, up, down_t, fc1 = nrm(d, d), blind(nrm(ff, d)), nrm(ff, d), blind(nrm(r, d))
+        if moving:                                                         # nothing writes into the side channel; only fc1's last rows read it
+            wo[d - MARK_DIMS:, :] = 0
+            down_t[:, d - MARK_DIMS:] = 0
+            fc1[r - MARK_DIMS:, :] = 0
+            for k in range(MARK_DIMS):
+                fc1[r - MARK_DIMS + k, d - MARK_DIMS + k] = MARK_GAIN
+        L["wo"] = enc(wo)
+        L["ffn_up"] = enc(up)
+        L["ffn_down_t"] = enc(down_t)
+        L["fc1"] = fc1
         p, _ = zipf_rates(ff, hp.mean_rate, rng)
-        L["fc2"] = predictor_fc2_margin(ff, r, p, rng) if hp.get("pred_margin") else predictor_fc2(ff, r, p, rng)
+        if moving:
+            L["fc2"], p = predictor_fc2_moving(ff, r, p, rng)
+        else:
+            L["fc2"] = predictor_fc2_margin(ff, r, p, rng) if hp.get("pred_margin") else predictor_fc2(ff, r, p, rng)
         L["p"] = p
         if hp.hot_frac < 1.0:
             L["gpu_idx"], L["gpu_bucket"] = gpu_split(p, hp.hot_frac)

@@ -120,6 +120,17 @@ def run_case(hp, n_prompt=12, n_gen=64, logit_tol=1e-2, min_same=0.9):
     return same
 
 
+def predictor_margin(model, il, src, logits, thr):
+    """Smallest distance of a predictor logit from the threshold, relative to what that row can move: |logit_j - thr| over
+    sum_k |fc2_jk| * h_k with h = relu(fc1 . src).  The arithmetic of two implementations differs by a few fp32 roundings of that sum, so a
+    value far above 1e-6 means no neuron's decision can depend on the order of the additions.  (A margin relative to the largest logit
+    of the layer would be misleading: rows of very different scale sit side by side.)"""
+    L = model["layers"][il]
+    h = np.maximum(L["fc1"].astype(np.float32) @ np.asarray(src, np.float32).astype(np.float16).astype(np.float32), 0.0)
+    reach = np.abs(L["fc2"].astype(np.float32)) @ h
+    return float((np.abs(np.asarray(logits) - thr) / np.maximum(reach, 1e-30)).min())
+
+
 def run_north_star(hp, n_prompt=8, n_gen=64, model=None):
     """The stated tolerances, verbatim, on a model whose decisions keep a margin:
       * predictor (synth.predictor_fc2_margin): every logit stays away from the threshold, so no neuron can flip and nothing
@@ -128,11 +139,14 @@ def run_north_star(hp, n_prompt=8, n_gen=64, model=None):
         the final state and the runner-up comes close only where their magnitudes happen to agree, which the test rules out for
         its seed by measuring it (with i.i.d. random output rows two correct implementations disagree on one greedy token in
         a few hundred, because the two largest of tens of thousands of logits come that close).
-    Asserted: predictor masks identical; every layer's FFN output within 2e-3 of the reference's block on the same input (and
-    the free-running trajectories within 2e-3 of each other for F16 weights); the logits of EVERY token within 1e-2 (maximum,
-    not median; for Q4_0 weights the median, see note()); 64 greedy tokens of the two sides, each running free on its own choices, identical -- and, so that this
-    identity is implied rather than lucky, the oracle's top-2 gap at every step more than 2.5 times the largest logit
-    difference of that step."""
+    Asserted: predictor masks identical; every layer's FFN output within 2e-3 of the reference's block on the same input; the logits
+    of EVERY token within 1e-2 (maximum, not median; for Q4_0 weights the median, see note()); 64 greedy tokens of the two sides, each
+    running free on its own choices, identical -- and, so that this identity is implied rather than lucky, the oracle's top-2 gap at
+    every step more than 2.5 times the largest logit difference of that step.
+    With hparams pred_moving the active set depends on the token being decoded (synth.predictor_fc2_moving) and the generated path
+    must show it: more than one distinct mask, and their union larger than any single one.
+    Returns what it measured; "trajectory" is the largest distance between the two sides' FFN outputs of a layer along the prompt,
+    each side on its own history -- not one of the stated criteria (a legal change of summation order moves it), so the caller decides."""
     from powerinfer_amd.model import Model
     assert hp.get("pred_margin") and hp.get("head_pair")
     model = model or synth.make_model(hp)
@@ -143,7 +157,7 @@ def run_north_star(hp, n_prompt=8, n_gen=64, model=None):
     thr = hp.sparse_threshold
     gm.set_capture(True)
     om.capture(1)
-    n_past, margins, gaps, diffs, errs = 0, [], [], [], []
+    n_past, margins, gaps, diffs, errs, traj = 0, [], [], [], [], []
     q4 = hp.wtype != synth.F16
 
     def note(lg_g, lg_o):
@@ -162,42 +176,54 @@ def run_north_star(hp, n_prompt=8, n_gen=64, model=None):
         ffn_g, plg_g, na_g, src_g = gm.get_capture()
         for il in range(hp.n_layer):
             assert np.array_equal(~(plg_g[il] < thr), ~(om.cap_lg[il, 0] < thr)), (n_past, il)          # masks identical
-            margins.append(float(np.abs(om.cap_lg[il, 0] - thr).min() / np.abs(om.cap_lg[il, 0]).max()))
-            # per-layer FFN output: the reference's block on the input this layer actually received, and the two trajectories
-            # side by side.  With Q4_0 weights the reference rounds activations to int8 per block of 32, so a last-place
-            # difference upstream can move one rounding step; the trajectories then differ by that step and what it grows into,
-            # while each layer, given the same input, still agrees to 2e-3.
+            margins.append(predictor_margin(model, il, src_g[il], om.cap_lg[il, 0], thr))
+            # per-layer FFN output: the reference's block on the input this layer actually received (the stated criterion); the
+            # distance between the two sides' own trajectories is only recorded.  With Q4_0 weights the reference rounds activations
+            # to int8 per block of 32, so a last-place difference upstream can move one rounding step; the trajectories then differ by
+            # that step and what it grows into, while each layer, given the same input, still agrees to 2e-3.
             ou = oracle_ffn_under(model, il, src_g[il], plg_g[il])
             assert rel_err(ffn_g[il], ou["out"]) < 2e-3, (n_past, il, rel_err(ffn_g[il], ou["out"]))
-            assert q4 or rel_err(ffn_g[il], om.cap_ffn[il, 0]) < 2e-3, (n_past, il)
+            traj.append(rel_err(ffn_g[il], om.cap_ffn[il, 0]))
         note(lg_g, lg_o)
         assert tok_g == tok_o
         n_past += 1
     assert min(margins) > 1e-3, min(margins)                    # the predictor's margin, far above any arithmetic difference
     gm.set_capture(False)
     toks_g, _ = gm.generate(n_gen)                              # free-running on the device: one HIP-graph replay per token
-    cur, toks_o = int(tok_o), []
+    cur, toks_o, masks_o = int(tok_o), [], []
     for s in range(n_gen):                                      # free-running on the CPU
         cur, _ = om.eval([cur], n_past + s)
         toks_o.append(int(cur))
+        masks_o.append(~(om.cap_lg[0, 0] < thr))
+    if hp.get("pred_moving"):                                   # the active set really moved along the path
+        m = np.array(masks_o)
+        assert len({row.tobytes() for row in m}) >= 2 and m.any(0).sum() > m.sum(1).max(), (m.sum(1).max(), m.any(0).sum())
     assert list(map(int, toks_g)) == toks_o
     assert len(set(toks_o)) >= 2 and max(toks_o.count(t) for t in set(toks_o)) <= n_gen - 3, toks_o      # the path is not one token repeated
     # the same path once more, token by token with logits (a second engine instance continues from an identical prefix)
     gm2 = Model(hp).load(model)
     gm2.decode(prompt, 0, want_logits=False)
+    gm2.set_capture(True)
     om.O.pio_model_kv_clear(om.h)
     om.capture(n_prompt)                                        # the capture buffers hold one row per token of a call
     om.eval([int(t) for t in prompt], 0)
+    om.capture(1)                                               # ... laid out for that call's token count: single tokens from here on
     cur = int(tok_o)
     for s in range(n_gen):
         _, lg_o = om.eval([cur], n_past + s)
         _, lg_g = gm2.decode([cur], n_past + s)
+        ffn_g, plg_g, _, src_g = gm2.get_capture()
+        for il in range(hp.n_layer):                            # along the generated path the masks move (pred_moving) and still agree
+            assert np.array_equal(~(plg_g[il] < thr), ~(om.cap_lg[il, 0] < thr)), (n_past + s, il)
+            if s % 8 == 0:
+                assert rel_err(ffn_g[il], oracle_ffn_under(model, il, src_g[il], plg_g[il])["out"]) < 2e-3, (n_past + s, il)
         note(lg_g, lg_o)
         cur = toks_o[s]
     assert np.median(errs) < 1e-2, errs
     ratio = min(g / max(e, 1e-30) for g, e in zip(gaps, diffs))
     assert ratio > 2.5, ratio        # identical greedy tokens are implied once the winner leads by more than twice the largest difference
     gm.close(), gm2.close(), om.close()
+    return dict(trajectory=max(traj), logits=max(errs), margin=min(margins))
 
 
 NS = dict(pred_margin=True, head_pair=2048)
@@ -222,10 +248,10 @@ def test_north_star_f16_7b_width():
 def test_north_star_f16_7b_full_depth():
     """configs[1] at its full size: all 32 layers of the 7B shape, 13 GB of weights.  The weights are generated in HBM (bench.py's
     builder, with the margin predictor and the four-row head), copied back for the oracle, and the same assertions run: masks
-    identical, every layer's FFN within 2e-3 on the same input and along the free-running trajectories, every token's logits
-    within 1e-2, 64 greedy tokens identical with the oracle's top-2 gap above 2.5 times the largest difference.  The trajectory
-    comparison is the fragile one at this depth: of seeds 1..11, three part by more than 2e-3 between layers 20 and 24 of some
-    prompt token (each layer still agreeing on the same input), three settle on one repeated token, five pass everything."""
+    identical, every layer's FFN within 2e-3 on the same input, every token's logits within 1e-2, 64 greedy tokens identical with
+    the oracle's top-2 gap above 2.5 times the largest difference.  The distance between the two sides' own trajectories (each on
+    its own history; not a stated criterion) grows with depth: a few 1e-3 between layers 20 and 30 depending on the seed and on the
+    order of the partial sums, so it is bounded here at 1e-2, which a flipped neuron or a wrong row would exceed by far."""
     import bench
     hp = synth.hparams("llama-7b", n_layer=32, n_ctx=96, seed=SEED_7B_FULL, **NS)
     keep = []
@@ -234,7 +260,8 @@ def test_north_star_f16_7b_full_depth():
     gm.close()
     del gm
     keep.clear()
-    run_north_star(hp, model=model)
+    r = run_north_star(hp, model=model)
+    assert r["trajectory"] < 1e-2, r
 
 
 @pytest.mark.timeout(300)
@@ -249,6 +276,75 @@ def test_north_star_falcon_40b_width():
     LayerNorm, parallel attention + FFN block, vocab 65024, two layers: the 8192-column mat-vec with the fused LayerNorm, the
     GQA attention and the four-groups-per-workgroup FFN instantiation all run here."""
     run_north_star(synth.hparams("falcon-40b", n_layer=2, n_ctx=80, seed=SEED_F40, **NS), n_prompt=6, n_gen=64)
+
+
+NSM = dict(pred_margin=True, pred_moving=True, head_pair=2048)
+# seeds whose greedy path (a CPU-oracle property) alternates between tokens of the pair, so that the active set moves along it
+SEED_TINY_MOVING = {"llama-tiny": 31, "falcon-tiny": 3}
+SEED_7B_MOVING, SEED_7B_Q4_MOVING = 44, 46
+
+
+@pytest.mark.parametrize("arch", ["llama-tiny", "falcon-tiny"])
+def test_north_star_moving_mask_tiny(arch):
+    """The stated tolerances on a predictor whose active set depends on the token being decoded (synth.predictor_fc2_moving): four groups
+    of neurons fire only while their own token is decoded, every decision with a margin.  Masks identical along the prompt AND along
+    the generated path, on which they change from step to step."""
+    run_north_star(synth.hparams(arch, n_ctx=96, seed=SEED_TINY_MOVING[arch], **NSM))
+
+
+@pytest.mark.timeout(300)
+def test_north_star_moving_mask_f16_7b_width():
+    """configs[1]'s layer shape, two layers, every neuron on the GPU, the active set moving with the token."""
+    run_north_star(synth.hparams("llama-7b", n_layer=2, n_ctx=96, seed=SEED_7B_MOVING, **NSM))
+
+
+@pytest.mark.timeout(300)
+def test_north_star_moving_mask_q4_split_7b_width():
+    """configs[2]: Q4_0, the hottest 60 % of each layer's neurons on the GPU, the rest on host threads.  Two of the four moving groups
+    sit in the host share (their profiled rate is low), so the host threads have active rows whenever token 2 or 3 is decoded and
+    the device's whenever token 0 or 1 is: both shares of the merge carry part of the moving mask."""
+    run_north_star(synth.hparams("llama-7b", n_layer=2, n_ctx=96, seed=SEED_7B_Q4_MOVING, wtype=synth.Q4_0, hot_frac=0.6, **NSM))
+
+
+@pytest.mark.parametrize("arch,seed", [("llama-tiny", 23), ("falcon-tiny", 22)])
+def test_free_running_trajectories_stay_close(arch, seed):
+    """Not a stated criterion: the FFN outputs of the two sides, each running on its own history, stay within 2e-3 of each other along
+    the prompt on these small models.  Kept apart from the north-star tests so that a change in the order of a sum, which moves this
+    number, cannot hide behind or block them."""
+    r = run_north_star(synth.hparams(arch, n_ctx=96, seed=seed, **NS))
+    assert r["trajectory"] < 2e-3, r
+
+
+@pytest.mark.parametrize("arch,seed", [("llama-tiny", 23), ("falcon-tiny", 22)])
+def test_north_star_long_context_allocation(arch, seed):
+    """A context of 1100 cells and up makes the engine split every head's cells over several workgroups (pi_k_attn_split) in the
+    token loop: the stated tolerances hold on that path as on the single-workgroup one."""
+    run_north_star(synth.hparams(arch, n_ctx=1100, seed=seed, **NS))
+
+
+@pytest.mark.timeout(600)
+def test_prompt_and_decode_at_a_context_beyond_the_chunk_kernels():
+    """n_ctx 16384: the scores of a prompt chunk no longer fit the chunk kernels' LDS, so the prompt goes through pi_k_attn_chunk_long and
+    the token loop through pi_k_attn_split.  A 300-token prompt and 12 decoded tokens against the oracle, token by token."""
+    from powerinfer_amd.model import Model
+    hp = synth.hparams("llama-tiny", n_ctx=16384, seed=23, **NS)
+    model = synth.make_model(hp)
+    gm, om = Model(hp).load(model), ol.OracleModel(model)
+    rng = np.random.default_rng(11)
+    prompt = rng.integers(0, hp.n_vocab, 300).astype(np.int32)
+    tok_g, lg_g = gm.decode(prompt, 0)
+    tok_o = lg_o = None
+    for i, t in enumerate(prompt):
+        tok_o, lg_o = om.eval([int(t)], i)
+    assert rel_err(lg_g, lg_o) < 1e-2 and tok_g == tok_o
+    cur = int(tok_o)
+    for s in range(12):
+        nxt_o, lg_o = om.eval([cur], 300 + s)
+        nxt_g, lg_g = gm.decode([cur], 300 + s)
+        assert rel_err(lg_g, lg_o) < 1e-2, (s, rel_err(lg_g, lg_o))
+        assert nxt_g == nxt_o
+        cur = int(nxt_o)
+    gm.close(), om.close()
 
 
 @pytest.mark.parametrize("wtype", [synth.F16, synth.Q4_0])

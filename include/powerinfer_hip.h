@@ -325,10 +325,6 @@ PI_API int pi_k_sparse_ffn_q4_partials(const void * fc2_f16, int ff, int r, cons
                                        float * logits, float * h_dense, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_sparse_ffn_q4_reduce(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out, int32_t * n_active,
                                      pi_workspace * ws, pi_stream_t stream);
-/* the same reduction behind pi_k_upgate_q4_hot_rows with down rows (a hybrid layer): n_active counts the resident active neurons */
-PI_API int pi_k_sparse_ffn_q4_reduce_hot(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out, int32_t * n_active,
-                                         pi_workspace * ws, pi_stream_t stream);
-
 /* Hand-over points between the stream and host threads that compute the non-resident neurons of a hybrid layer (the CPU half of
  * llm_build_sparse_mul_mat / llm_build_sparse_axpy, llama.cpp:4581-4593, 4635-4646) without the host launching anything in between.
  * flags_pinned: 64 words of pinned host memory (words 0 and 8 written by the device, words 16 and 32 by the host, word 48 = the host's
@@ -343,16 +339,12 @@ PI_API int pi_k_host_signal(uint32_t * seq, uint32_t * flags_pinned, int word, i
  * pi_k_upgate_q4_hot_rows reads logits_dev and writes h (or 0) for the neurons of the hot words only - the other entries of h_dense
  * belong to the host.  With announce_seq / announce_flags (both or neither) the first lane of that launch does what
  * pi_k_host_signal(announce_seq, announce_flags, 0, 1) would have done right before it: the predictor's results are complete and
- * visible to the host at the boundary in front of the launch, so the hand-over needs no launch of its own.
- * With down_t_q4 (the resident rows of the down projection, optional) the same launch also adds the down rows of every 32-neuron block
- * whose active neurons are all resident, one partial vector per block for pi_k_sparse_ffn_q4_reduce; a block with an active neuron
- * outside the hot words is left to the host as a whole, because its Q8_0 scale of h needs that neuron's value (the host holds every row
- * and reads the resident neurons' h from h_dense) - the device then needs nothing from the host before the reduction. */
+ * visible to the host at the boundary in front of the launch, so the hand-over needs no launch of its own. */
 PI_API int pi_k_pred_q4_logits(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
                                float * logits, float * logits_dev, void * xq8_out, uint32_t * words_out, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_upgate_q4_hot_rows(int ff, float threshold, const void * up_q4, const void * gate_q4, int cols, const float * x, const pi_norm * norm,
                                    const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense,
-                                   uint32_t * announce_seq, uint32_t * announce_flags, const void * down_t_q4, pi_workspace * ws, pi_stream_t stream);
+                                   uint32_t * announce_seq, uint32_t * announce_flags, pi_workspace * ws, pi_stream_t stream);
 /* The fused F16 launch of a hybrid layer (pi_k_sparse_ffn_partials_hot) cut in two in the same way (cols 4096): pi_k_sparse_ffn_logits_hot
  * computes the logits (to `logits`, optional, which may be pinned host memory, and to logits_dev), the mask words (also to words_out,
  * optional, as pi_k_pred_q4_logits) and the fp16 normalised input for

@@ -297,8 +297,6 @@ struct ColdPath {
     hipEvent_t ev_in = nullptr, ev_h = nullptr;
     std::vector<float> hval;                    // h of the active cold neurons, in the order of act
     std::vector<const BlockQ4 *> dn_rows; std::vector<int> dn_a; std::vector<float> dn_sc;    // the rows of one Q4_0 down projection
-    std::vector<int> act_down;                  // see list_active_cold_words
-    bool mixed_on_host = false;                 // Q4_0 hand-over layers: blocks with an active non-resident neuron are computed by the host as a whole
     // PI_COLD_TRACE=1: mean host time per phase of a layer call, printed when the model is freed
     bool trace = false;
     double t_phase[6] = {0, 0, 0, 0, 0, 0};
@@ -318,7 +316,6 @@ struct ColdPath {
     bool async = false;
     std::vector<int> async_layers;              // hybrid layers that take this route, ascending
     uint32_t * flags = nullptr;                 // pinned: [0] logits ready, [8] resident h ready (device -> host), [16] h complete, [32] output share complete, [48] stop word
-    bool split_pred = true;                     // the predictor is its own launch, so the host starts while the resident up/gate rows run
     std::vector<float *> h_async;               // per layer, pinned: h of that variant; the device writes the resident neurons' entries, the host its own
                                                 // (one vector per layer, because the resident set differs from layer to layer)
     std::vector<std::vector<int32_t>> prev_act; // per layer: the host's entries that are non-zero from the previous token
@@ -389,12 +386,6 @@ ColdPath * cold_create(pi_model * m) {
         if (hipHostMalloc(&fl, 64 * sizeof(uint32_t), hipHostMallocCoherent) != hipSuccess) { set_error("cold path: pinned host allocation failed"); cold_destroy(c); return nullptr; }
         c->flags = (uint32_t *)fl;
         memset(c->flags, 0, 64 * sizeof(uint32_t));
-        if (const char * e = getenv("PI_COLD_SPLIT")) c->split_pred = e[0] != '0';
-        // PI_COLD_MIXED=host: 32-neuron blocks with an active non-resident neuron are computed by the host as a whole, so the device
-        // waits for the host once per layer instead of twice.  Measured slower with 8 host threads (the host's down projection
-        // grows from 84 to about 250 rows per 7B layer: 437 -> 381 tok/s), so the default keeps every resident row on the device.
-        const char * mx = getenv("PI_COLD_MIXED");
-        c->mixed_on_host = c->split_pred && mx && !strcmp(mx, "host");
         c->h_async.assign(hp.n_layer, nullptr);
         c->prev_act.resize(hp.n_layer);
         for (int il : c->async_layers) {
@@ -457,18 +448,14 @@ namespace {
 
 // neurons of this layer that are not GPU-resident and whose predictor logit reaches the threshold, ascending, into c->act
 // the same list from the activity words the predictor launch left in pinned memory: 1.4 KB to read instead of a logit per cold neuron
-// act_down: every active neuron, resident or not, of the blocks that hold an active non-resident one (the host's down rows when
-// such blocks are the host's as a whole)
 int list_active_cold_words(ColdPath * c, const ColdLayer & cl) {
     c->act.clear();
-    c->act_down.clear();
     const uint32_t * aw = c->words_pin;
     const int nw = (int)cl.cold_words.size();
     for (int w = 0; w < nw; ++w) {
         const uint32_t all = aw[w];
         if ((all & cl.cold_words[w]) == 0u) continue;
         for (uint32_t bits = all & cl.cold_words[w]; bits; bits &= bits - 1) c->act.push_back(w * 32 + __builtin_ctz(bits));
-        if (c->mixed_on_host) for (uint32_t bits = all; bits; bits &= bits - 1) c->act_down.push_back(w * 32 + __builtin_ctz(bits));
     }
     return (int)c->act.size();
 }
@@ -512,7 +499,7 @@ void host_upgate(ColdPath * c, pi_model * m, int il, int na) {
 // the listed neurons' share of the down projection into out[d]; threads split the output columns in blocks of 32, so no two threads
 // add into the same element.  Q4_0: h goes through the Q8_0 blocks of the completed vector hfull (only the blocks that hold a listed
 // neuron are quantised; ggml.c:14465-14618); F16: h rounded to fp16 (ggml.c:14420-14431).
-void host_down(ColdPath * c, pi_model * m, int il, int na, const float * hfull, float * out, bool whole_blocks = false) {
+void host_down(ColdPath * c, pi_model * m, int il, int na, const float * hfull, float * out) {
     Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
     const bool q4 = down.type == PI_TYPE_Q4_0;
     const int d = c->d;
@@ -529,7 +516,7 @@ void host_down(ColdPath * c, pi_model * m, int il, int na, const float * hfull, 
     if (q4) {
         // rows whose h rounds to 0 add nothing (skipped, as before); each thread takes a band of column blocks over all rows
         c->dn_rows.clear(); c->dn_a.clear(); c->dn_sc.clear();
-        const std::vector<int> & rows_of = whole_blocks ? c->act_down : c->act;
+        const std::vector<int> & rows_of = c->act;
         for (size_t k = 0; k < rows_of.size(); ++k) {
             const int j = rows_of[k];
             const BlockQ8 & hb = c->hq8[j / 32];
@@ -856,7 +843,7 @@ void serve_q4(ColdPath * c, int il, uint32_t seq) {
     ColdLayer & cl = c->layers[il];
     Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
     const float thr = hp.sparse_threshold;
-    float * hfull = c->split_pred ? c->h_async[il] : c->h_full[0];
+    float * hfull = c->h_async[il];
     float * out = c->out[0];
     auto now = [] { return std::chrono::steady_clock::now(); };
     auto us = [](std::chrono::steady_clock::time_point a, std::chrono::steady_clock::time_point b) { return std::chrono::duration<double, std::micro>(b - a).count(); };
@@ -880,35 +867,30 @@ void serve_q4(ColdPath * c, int il, uint32_t seq) {
     lap(0);
 
     // 2. active cold neurons, their up/gate rows against the same Q8_0 input
-    if (c->split_pred) {                        // this side's entries of the shared vector: the device never writes them
-        for (int j : c->prev_act[il]) hfull[j] = 0.f;
-        c->prev_act[il].clear();
-    }
-    const int na = c->split_pred ? list_active_cold_words(c, cl) : list_active_cold(c, cl, thr);
+    for (int j : c->prev_act[il]) hfull[j] = 0.f;        // this side's entries of the shared vector: the device never writes them
+    c->prev_act[il].clear();
+    const int na = list_active_cold_words(c, cl);
     lap(1);
     host_upgate(c, m, il, na);
     const float * hval = c->hval.data();
     for (int k = 0; k < na; ++k) hfull[c->act[k]] = hval[k];
-    if (c->split_pred) c->prev_act[il].assign(c->act.begin(), c->act.end());
-    const bool whole = c->split_pred && c->mixed_on_host;
-    if (!whole) __atomic_store_n(&c->flags[16], seq, __ATOMIC_RELEASE);          // the device's down projection may read the completed vector
+    c->prev_act[il].assign(c->act.begin(), c->act.end());
+    __atomic_store_n(&c->flags[16], seq, __ATOMIC_RELEASE);          // the device's down projection may read the completed vector
     lap(2);
-    if (c->split_pred) {
-        // the Q8_0 scales of h span resident and non-resident neurons: the resident ones' h must have arrived
-        const auto t0 = now();
-        for (int it = 0; (int32_t)(__atomic_load_n(&c->flags[8], __ATOMIC_ACQUIRE) - seq) < 0; ++it) {
-            relax();
-            if ((it & 1023) == 1023 && (c->stop.load() || now() - t0 > std::chrono::seconds(20))) {
-                c->failed.store(true);
-                __atomic_store_n(&c->flags[48], 1u, __ATOMIC_RELEASE);
-                return;
-            }
+    // the Q8_0 scales of h span resident and non-resident neurons: the resident ones' h must have arrived
+    const auto t0 = now();
+    for (int it = 0; (int32_t)(__atomic_load_n(&c->flags[8], __ATOMIC_ACQUIRE) - seq) < 0; ++it) {
+        relax();
+        if ((it & 1023) == 1023 && (c->stop.load() || now() - t0 > std::chrono::seconds(20))) {
+            c->failed.store(true);
+            __atomic_store_n(&c->flags[48], 1u, __ATOMIC_RELEASE);
+            return;
         }
     }
 
     // 3. the host quantises h the same way and adds its neurons' down rows
     lap(3);
-    host_down(c, m, il, na, hfull, out, whole);
+    host_down(c, m, il, na, hfull, out);
     __atomic_store_n(&c->flags[32], seq, __ATOMIC_RELEASE);          // the reduction may add the host share
     lap(4);
     if (c->trace) { ++c->n_calls; c->n_cold_active += na; c->t_last_return = now(); }
@@ -1032,7 +1014,7 @@ int cold_layer_q4_queue(ColdPath * c, int il, pi_model * m, hipStream_t st) {
     Tensor & up = m->L(il, PI_T_FFN_UP); Tensor & gate = m->L(il, PI_T_FFN_GATE); Tensor & down = m->L(il, PI_T_FFN_DOWN_T);
     Tensor & fc1 = m->L(il, PI_T_FC1); Tensor & fc2 = m->L(il, PI_T_FC2);
     const int r = (int)fc1.ne1;
-    float * hfull = c->h_full[0];
+    float * hfull = c->h_async[il];
     float * out = c->out[0];
     const double limit = 5.0;
     pi_norm fn;
@@ -1040,26 +1022,11 @@ int cold_layer_q4_queue(ColdPath * c, int il, pi_model * m, hipStream_t st) {
     fn.w = (const float *)m->L(il, falcon ? PI_T_ATTN_NORM : PI_T_FFN_NORM).dev;
     fn.b = falcon ? (const float *)m->L(il, PI_T_ATTN_NORM_B).dev : nullptr;
     const float * ffn_src = falcon ? m->x : m->ffn_inp;
-    if (c->split_pred) {
-        hfull = c->h_async[il];
-        PI_TRY(pi_k_pred_q4_logits(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, d, ffn_src, &fn, nullptr, m->pred_logits, c->xq8_pin, c->words_pin, m->ws, st));
-        // the hand-over starts in the first lane of the next launch, and the second signal travels with the wait behind it
-        PI_TRY(pi_k_upgate_q4_hot_rows(ff, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, d, ffn_src, &fn, m->hot_words[il], m->hot_prefix[il],
-                                       m->pred_logits, hfull, c->d_seq, c->flags, c->mixed_on_host ? down.dev : nullptr, m->ws, st));
-        if (c->mixed_on_host) {
-            // blocks with an active non-resident neuron are the host's as a whole: nothing to wait for before the reduction
-            PI_TRY(pi_k_host_signal_wait(c->d_seq, c->flags, 8, 32, c->d_status, limit, st));
-            int32_t * n_act = m->n_active + il;
-            if (!falcon) return pi_k_sparse_ffn_q4_reduce_hot(ff, d, PI_EPI_ADD2, out, m->ffn_inp, m->x2, n_act, m->ws, st);
-            PI_TRY(pi_k_sparse_ffn_q4_reduce_hot(ff, d, PI_EPI_NONE, nullptr, nullptr, m->x2, n_act, m->ws, st));
-            return merge_shares(m->x2, out, m->x2, m->attn_out, m->x, nullptr, d, st);
-        }
-    } else {
-        PI_TRY(pi_k_pred_upgate_q4(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, d, ffn_src, &fn,
-                                   m->hot_words[il], m->hot_prefix[il], c->logits, hfull, c->xq8_pin, m->ws, st));
-        PI_TRY(pi_k_host_signal(c->d_seq, c->flags, 0, 1, st));
-    }
-    PI_TRY(pi_k_host_signal_wait(c->d_seq, c->flags, c->split_pred ? 8 : -1, 16, c->d_status, limit, st));
+    PI_TRY(pi_k_pred_q4_logits(fc2.dev, ff, r, m->hidden, hp.sparse_threshold, d, ffn_src, &fn, nullptr, m->pred_logits, c->xq8_pin, c->words_pin, m->ws, st));
+    // the hand-over starts in the first lane of the next launch, and the second signal travels with the wait behind it
+    PI_TRY(pi_k_upgate_q4_hot_rows(ff, hp.sparse_threshold, up.dev, falcon ? nullptr : gate.dev, d, ffn_src, &fn, m->hot_words[il], m->hot_prefix[il],
+                                   m->pred_logits, hfull, c->d_seq, c->flags, m->ws, st));
+    PI_TRY(pi_k_host_signal_wait(c->d_seq, c->flags, 8, 16, c->d_status, limit, st));
     PI_TRY(pi_k_axpy_q4_partials(down.dev, d, ff, hfull, m->hot_words[il], m->hot_prefix[il], m->ws, st));
     PI_TRY(pi_k_host_wait(c->d_seq, c->flags, 32, c->d_status, limit, st));
     int32_t * n_act = m->n_active + il;

@@ -324,9 +324,8 @@ int stage_rest_rows(pi_model * m, BatchState * b, int il) {
 
 namespace pi {
 bool prefill_wide_supported(pi_model * m) {
-    const char * off = getenv("PI_NO_PREFILL_WIDE");
-    const char * off_all = getenv("PI_NO_PREFILL");
-    return !(off && off[0] == '1') && !(off_all && off_all[0] == '1') && wide_unsupported(m) == nullptr;
+    const char * off = getenv("PI_NO_PREFILL_WIDE");          // the comparison side of the chunk tests: prompts in steps of 16 tokens
+    return !(off && off[0] == '1') && wide_unsupported(m) == nullptr;
 }
 
 int prefill_wide_max(pi_model * m) {
@@ -389,8 +388,7 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
             b->stage_rows = std::max(b->stage_rows, (size_t)hp.n_ff - (size_t)m->L(il, PI_T_GPU_BUCKET).ne0);
             b->stage_row_bytes = std::max(b->stage_row_bytes, m->L(il, PI_T_FFN_UP).type == PI_TYPE_Q4_0 ? (size_t)(hp.n_embd / 32) * 18 : (size_t)hp.n_embd * 2);
         }
-        const char * no_stage = getenv("PI_PREFILL_NO_STAGING");
-        if (b->stage_rows && !(no_stage && no_stage[0] == '1')) {
+        if (b->stage_rows) {
             for (int i = 0; i < 2; ++i) {
                 b->stage[i] = m->alloc<unsigned char>(3 * b->stage_rows * b->stage_row_bytes);
                 if (!b->stage[i]) return PI_E_HIP;
@@ -424,8 +422,7 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
 }
 
 bool prefill_supported(pi_model * m) {
-    const char * off = getenv("PI_NO_PREFILL");
-    return !(off && off[0] == '1') && !m->capture && batch_unsupported(m) == nullptr;
+    return !m->capture && batch_unsupported(m) == nullptr;
 }
 
 // T <= 16 consecutive prompt tokens of the model's own sequence in one step: the weights are read once for the chunk

@@ -1531,7 +1531,7 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
                                                                      float * __restrict__ logits2,
                                                                      const pi_block_q4_0 * __restrict__ Wd, const pi_block_q4_0 * __restrict__ Wd_rest,
                                                                      float * __restrict__ partial, HostAnnounce ann) {
-    static_assert(!FUSE || PHASE != 1, "the logits-only launch has no rows");
+    static_assert(!FUSE || PHASE == 0, "the two-phase form of a hybrid layer leaves the down projection to its own launch");
     if (PHASE == 2 && ann.flags && blockIdx.x == 0 && threadIdx.x == 0) {
         // what was queued before this launch is complete and visible to the host (the kernel boundary released at system scope):
         // a new hand-over starts here, without a launch of its own
@@ -1752,9 +1752,8 @@ __global__ __launch_bounds__(kPfBlock, 2) void pred_upgate_q4_kernel(const __hal
         for (int o = 16; o > 0; o >>= 1) hmax = fmaxf(hmax, __shfl_xor(hmax, o, PI_WAVE));
         const float dh = pi_round_f16(pi_div(hmax, 127.0f)), idh = (hmax != 0.0f) ? pi_div(127.0f, hmax) : 0.0f;
         const int qh = (int)rintf(__fmul_rn(hvv, idh));
-        // neurons that add something, ascending.  In the second launch of a hybrid layer (PHASE 2) a block with an active neuron outside
-        // the hot set belongs to the host as a whole (its Q8_0 scale needs that neuron's h): this workgroup then adds nothing.
-        const uint32_t nz = (PHASE == 2 && (mask & ~hot) != 0u) ? 0u : (uint32_t)__ballot(qh != 0) & sel;
+        // neurons that add something, ascending
+        const uint32_t nz = (uint32_t)__ballot(qh != 0) & sel;
         const int nrows = __popc(nz);
         float acc[8];
 #pragma unroll
@@ -4290,15 +4289,6 @@ int pi_k_sparse_ffn_q4_reduce(int ff, int cols, int epilogue, const float * add1
                        ws->words, ff / 32, n_active, epilogue, add1, add2, out);
     return pi::check_launch("pi_k_sparse_ffn_q4_reduce");
 }
-int pi_k_sparse_ffn_q4_reduce_hot(int ff, int cols, int epilogue, const float * add1, const float * add2, float * out, int32_t * n_active,
-                                  pi_workspace * ws, pi_stream_t stream) {
-    if (!out || !ws || cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_q4_reduce_hot: bad arguments");
-    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
-        return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_q4_reduce_hot: bad epilogue arguments");
-    hipLaunchKernelGGL(ffn_reduce_kernel, dim3(cols / kFrCols), dim3(kPfBlock), 0, (hipStream_t)stream, ws->ffn_partial, ff / 32, cols,
-                       ws->words_hot, ff / 32, n_active, epilogue, add1, add2, out);
-    return pi::check_launch("pi_k_sparse_ffn_q4_reduce_hot");
-}
 
 int pi_k_pred_q4_logits(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
                         float * logits, float * logits_dev, void * xq8_out, uint32_t * words_out, pi_workspace * ws, pi_stream_t stream) {
@@ -4316,7 +4306,7 @@ int pi_k_pred_q4_logits(const void * fc2_f16, int ff, int r, const float * hidde
 
 int pi_k_upgate_q4_hot_rows(int ff, float threshold, const void * up_q4, const void * gate_q4, int cols, const float * x, const pi_norm * norm,
                             const uint32_t * hot_words, const int32_t * hot_prefix, const float * logits_dev, float * h_dense,
-                            uint32_t * announce_seq, uint32_t * announce_flags, const void * down_t_q4, pi_workspace * ws, pi_stream_t stream) {
+                            uint32_t * announce_seq, uint32_t * announce_flags, pi_workspace * ws, pi_stream_t stream) {
     if (!up_q4 || !x || !hot_words || !hot_prefix || !logits_dev || !h_dense || !ws) return pi::fail(PI_E_ARG, "pi_k_upgate_q4_hot_rows: null pointer");
     if ((announce_seq == nullptr) != (announce_flags == nullptr)) return pi::fail(PI_E_ARG, "pi_k_upgate_q4_hot_rows: announce_seq and announce_flags go together");
     if (cols != 4096 || ff <= 0 || ff % 32 || ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_UNSUPPORTED, "pi_k_upgate_q4_hot_rows: cols must be 4096, ff % 32 == 0, within the workspace");
@@ -4326,10 +4316,7 @@ int pi_k_upgate_q4_hot_rows(int ff, float threshold, const void * up_q4, const v
     const pi_block_q4_0 * none = nullptr;
     const pi_block_q4_0 * u = (const pi_block_q4_0 *)up_q4; const pi_block_q4_0 * g = (const pi_block_q4_0 *)gate_q4;
 #define PI_PQ2(GATE) hipLaunchKernelGGL((pred_upgate_q4_kernel<1, GATE, false, 2>), grid, block, 0, (hipStream_t)stream, (const __half *)nullptr, (const float *)nullptr, u, g, none, none, x, na, threshold, hot_words, hot_prefix, (float *)nullptr, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)nullptr, const_cast<float *>(logits_dev), none, none, (float *)nullptr, HostAnnounce{announce_seq, announce_flags})
-#define PI_PQ2F(GATE) hipLaunchKernelGGL((pred_upgate_q4_kernel<1, GATE, false, 2, true>), grid, block, 0, (hipStream_t)stream, (const __half *)nullptr, (const float *)nullptr, u, g, none, none, x, na, threshold, hot_words, hot_prefix, (float *)nullptr, ws->words, ws->words_hot, h_dense, (pi_q8_host_block *)nullptr, const_cast<float *>(logits_dev), (const pi_block_q4_0 *)down_t_q4, none, ws->ffn_partial, HostAnnounce{announce_seq, announce_flags})
-    if (down_t_q4) { if (g) PI_PQ2F(true); else PI_PQ2F(false); }
-    else           { if (g) PI_PQ2(true); else PI_PQ2(false); }
-#undef PI_PQ2F
+    if (g) PI_PQ2(true); else PI_PQ2(false);
 #undef PI_PQ2
     return pi::check_launch("pi_k_upgate_q4_hot_rows");
 }

@@ -94,9 +94,8 @@ _SIGS = {
     "pi_k_sparse_ffn_rows_hot": (_i, [_i, _f, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_q4_partials": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_q4_reduce": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
-    "pi_k_sparse_ffn_q4_reduce_hot": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_pred_q4_logits": (_i, [_vp, _i, _i, _vp, _f, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp]),
-    "pi_k_upgate_q4_hot_rows": (_i, [_i, _f, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_upgate_q4_hot_rows": (_i, [_i, _f, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_host_wait": (_i, [_vp, _vp, _i, _vp, C.c_double, _vp]),
     "pi_k_host_signal_wait": (_i, [_vp, _vp, _i, _i, _vp, C.c_double, _vp]),
     "pi_ggml_backend_get_stats": (None, [_vp]),

@@ -227,17 +227,13 @@ class SparseFFN:
         return dict(logits=self.logits.download(np.float32), h=self.h_dense.download(np.float32),
                     n_active=int(self.n_active.download(np.int32)[0]), out=self.out.download(np.float32))
 
-    def forward_q4_handover(self, x_ffn, x_pred, host_h, host_out, limit_s=20.0, whole_blocks=False):
+    def forward_q4_handover(self, x_ffn, x_pred, host_h, host_out, limit_s=20.0):
         """The same layer with the host share computed while the stream runs, nothing launched in between (what the decode loop
         queues for a hybrid Q4_0 layer): pi_k_pred_q4_logits -> pi_k_upgate_q4_hot_rows (its first lane starts the hand-over) ->
         pi_k_host_signal_wait -> pi_k_axpy_q4_partials (h in pinned memory) -> pi_k_host_wait -> pi_k_axpy_q4_reduce (+ the host
         share's output from pinned memory).  Everything is queued first; then this thread plays the host side: once the logits have
         arrived host_h(logits, xq8) returns {neuron: h} for the host's neurons, and once the resident neurons' h has arrived
-        host_out(h_full) returns the host share of the output.  Returns dict(logits, h, n_active, out, status).
-        whole_blocks: the arrangement the decode loop uses under PI_COLD_MIXED=host - the launch that computes the resident neurons' h also adds
-        the down rows of every 32-neuron block whose active neurons are all resident, the host owns the other blocks as a whole
-        (host_out must add their resident neurons' rows too), and the stream waits for the host once: pi_k_pred_q4_logits ->
-        pi_k_upgate_q4_hot_rows(down) -> pi_k_host_signal_wait -> pi_k_sparse_ffn_q4_reduce_hot."""
+        host_out(h_full) returns the host share of the output.  Returns dict(logits, h, n_active, out, status)."""
         import ctypes as C
         import time
         L = self.L
@@ -270,15 +266,11 @@ class SparseFFN:
             check(L.pi_k_gemv(pl.F16, self.fc1.ptr, self.r, self.d, self.xp.ptr, None, pl.EPI_RELU, None, None, self.hidden.ptr, None), "fc1")
             check(L.pi_k_pred_q4_logits(self.fc2.ptr, self.ff, self.r, self.hidden.ptr, self.thr, self.d, self.x.ptr, nrm, lg_p, lg_dev.ptr, xq_p, words_p, self.ws, None), "pred_q4_logits")
             check(L.pi_k_upgate_q4_hot_rows(self.ff, self.thr, self.up.ptr, p(self.gate), self.d, self.x.ptr, nrm, hw.ptr, hp.ptr, lg_dev.ptr, h_p,
-                                            seq.ptr, flags_p, self.down.ptr if whole_blocks else None, self.ws, None), "hot_rows")
-            if whole_blocks:
-                check(L.pi_k_host_signal_wait(seq.ptr, flags_p, 8, 32, status.ptr, limit_s, None), "signal_wait")
-                check(L.pi_k_sparse_ffn_q4_reduce_hot(self.ff, self.d, pl.EPI_ADD, out_p, None, self.out.ptr, self.n_active.ptr, self.ws, None), "sparse_ffn_q4_reduce_hot")
-            else:
-                check(L.pi_k_host_signal_wait(seq.ptr, flags_p, 8, 16, status.ptr, limit_s, None), "signal_wait")
-                check(L.pi_k_axpy_q4_partials(self.down.ptr, self.d, self.ff, h_p, hw.ptr, hp.ptr, self.ws, None), "axpy_q4_partials")
-                check(L.pi_k_host_wait(seq.ptr, flags_p, 32, status.ptr, limit_s, None), "wait")
-                check(L.pi_k_axpy_q4_reduce(self.ff, self.d, pl.EPI_ADD, out_p, None, self.out.ptr, self.n_active.ptr, self.ws, None), "axpy_q4_reduce")
+                                            seq.ptr, flags_p, self.ws, None), "hot_rows")
+            check(L.pi_k_host_signal_wait(seq.ptr, flags_p, 8, 16, status.ptr, limit_s, None), "signal_wait")
+            check(L.pi_k_axpy_q4_partials(self.down.ptr, self.d, self.ff, h_p, hw.ptr, hp.ptr, self.ws, None), "axpy_q4_partials")
+            check(L.pi_k_host_wait(seq.ptr, flags_p, 32, status.ptr, limit_s, None), "wait")
+            check(L.pi_k_axpy_q4_reduce(self.ff, self.d, pl.EPI_ADD, out_p, None, self.out.ptr, self.n_active.ptr, self.ws, None), "axpy_q4_reduce")
 
             def wait_flag(word):
                 t0 = time.time()

@@ -373,28 +373,6 @@ def test_q4_hybrid_layer_with_stream_handovers():
     assert np.array_equal(res["out"], base["out"] + cold_share(hm))      # same partial sums, host share added by the reduction
     assert rel_err(res["out"], got["full"]["out"]) < FFN_REL_TOL
 
-    # The decode loop under PI_COLD_MIXED=host: a block of 32 neurons with an active non-resident neuron is the host's as a whole (the Q8_0 scale of
-    # its h needs that neuron's value), the device adds every other block in the launch that computes its h and waits for the host
-    # once.  Every active neuron's row is added exactly once, by one side or the other: device share + host share is the full layer,
-    # and the device share alone is the full layer's sum over the neurons of the blocks it owns.
-    act_all = ~(base["logits"] < ffn.thr)
-    mixed_block = (act_all & cold).reshape(-1, 32).any(1)
-    host_rows_mask = np.repeat(mixed_block, 32)
-
-    def share(hm, mask):
-        q, dh = q8_blocks_np(hm)
-        rows = np.nonzero(mask & (q != 0))[0]
-        v, dw = q4_rows_np(L["down_t"], rows, d)
-        contrib = (v * q[rows, None]).astype(np.float32) * (np.repeat(dw, 32, axis=1) * dh[rows, None])
-        return contrib.sum(0, dtype=np.float32)
-    res2 = ffn.forward_q4_handover(x, x, host_h, lambda h_full: share(h_full, host_rows_mask), whole_blocks=True)
-    assert res2["status"] == 0 and res2["n_active"] == base["n_active"]
-    assert 0 < mixed_block.sum() < mixed_block.size and (act_all & ~cold & host_rows_mask).any()      # the host took resident neurons' rows too
-    assert np.array_equal(res2["h"], hm)
-    dev_only = res2["out"] - share(hm, host_rows_mask)
-    assert rel_err(dev_only, share(hm, ~host_rows_mask)) < 1e-5, rel_err(dev_only, share(hm, ~host_rows_mask))
-    assert rel_err(res2["out"], res["out"]) < 1e-5, rel_err(res2["out"], res["out"])
-    assert rel_err(res2["out"], got["full"]["out"]) < FFN_REL_TOL
     ffn.close()
 
 

@@ -453,7 +453,6 @@ def test_split_stream_handovers_match_launch_per_exchange(arch, wtype, monkeypat
     model = synth.make_model(hp)
     prompt = np.random.default_rng(5).integers(0, hp.n_vocab, 9).astype(np.int32)
     outs = []
-    monkeypatch.delenv("PI_COLD_MIXED", raising=False)
     for sync in (False, True):
         if sync:
             monkeypatch.setenv("PI_COLD_SYNC", "1")
@@ -468,45 +467,6 @@ def test_split_stream_handovers_match_launch_per_exchange(arch, wtype, monkeypat
         gm.close()
     assert outs[0][0] == outs[1][0] and outs[0][2] == outs[1][2] and outs[0][3] == outs[1][3]
     assert np.array_equal(outs[0][1], outs[1][1]) and np.array_equal(outs[0][4], outs[1][4])
-    if wtype != synth.Q4_0:
-        return
-    # PI_COLD_MIXED=host (Q4_0): a block of 32 neurons with an active non-resident neuron is the host's as a whole (the Q8_0 scale of
-    # its h needs that neuron's value), every other block is added by the device in the launch that computes its h, and the device waits
-    # for the host once per layer.  Same products, another order of the sums: the prompt's logits agree to rounding, and the graph replays
-    # agree bit for bit with the same launches issued one token per call.
-    monkeypatch.delenv("PI_COLD_SYNC", raising=False)
-    monkeypatch.setenv("PI_COLD_MIXED", "host")
-    ga, gb = Model(hp).load(model), Model(hp).load(model)
-    tok_a, lg_a = ga.decode(prompt, 0)
-    tok_b, _ = gb.decode(prompt, 0)
-    # another order of the sums moves last places, and over three Q4_0 layers and nine tokens some of those flip an int8 rounding of
-    # the activations downstream (tests/test_oracle_math.py::test_reference_arithmetic_is_chaotic_under_last_bit_noise); the
-    # one-layer comparison below has no such amplifier and holds the two arrangements to rounding
-    assert rel_err(lg_a, outs[1][1]) < 3e-2, rel_err(lg_a, outs[1][1])
-    assert tok_a == tok_b
-    toks = [int(t) for n in (20, 7) for t in ga.generate(n)[0]]
-    cur, n_past, single = int(tok_b), len(prompt), []
-    for _ in toks:
-        cur, _ = gb.decode([cur], n_past)
-        single.append(int(cur))
-        n_past += 1
-    assert toks == single
-    assert np.array_equal(ga.decode([toks[-1]], n_past)[1], gb.decode([single[-1]], n_past)[1])
-    ga.close(), gb.close()
-    hp1 = synth.HParams(hp)
-    hp1["n_layer"] = 1
-    model1 = dict(model, hp=hp1, layers=model["layers"][:1])
-    one = []
-    for mixed in (None, "host"):
-        if mixed:
-            monkeypatch.setenv("PI_COLD_MIXED", mixed)
-        else:
-            monkeypatch.delenv("PI_COLD_MIXED", raising=False)
-        g1 = Model(hp1).load(model1)
-        one.append([g1.decode([int(t)], i)[1] for i, t in enumerate(prompt[:4])])
-        g1.close()
-    worst = max(rel_err(a, b) for a, b in zip(one[1], one[0]))
-    assert worst < 5e-4, worst
 
 
 @pytest.mark.parametrize("arch,wtype", [("llama-tiny", synth.F16), ("llama-tiny", synth.Q4_0), ("falcon-tiny", synth.F16)])

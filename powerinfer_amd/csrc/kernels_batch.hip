@@ -1,0 +1,1000 @@
+// Steps of several tokens: 2..16 sequences in lockstep or a prompt chunk of one sequence.  Dense and sparse mat-muls on the matrix
+// cores, the union of the tokens' active rows, norm + rounding passes, Q4_0 expansion and row assembly for prompt chunks.
+#include "kernels_common.hpp"
+
+namespace {
+
+// =====================================================================================================
+// Batched decode (2..16 tokens per step, one per sequence).  Weights are still streamed once per step, so the
+// roofline stays HBM, but 16 dot products per weight would make the VALU the limit: the dense mat-muls and the
+// sparse gate/up run on the matrix cores (v_mfma_f32_16x16x32_f16: a tile of 16 weight rows x 16 tokens x 32
+// columns per instruction, fp32 accumulate).  Lane l holds, for row (token) l % 16, the 8 columns
+// 8 * (l / 16) .. + 8 of the 32-column slab of both operands, i.e. one 16-byte load each; the accumulator lane l
+// holds rows 4 * (l / 16) .. + 4 of column (token) l % 16.
+// Activations are normalised and rounded to fp16 once per mat-mul input by norm_round_f16_kernel (the CPU path rounds
+// them to fp16 before every dot, ggml.c:9703-9716) and read by every tile from L2.
+// =====================================================================================================
+
+// the value a Q8_0 block keeps of v: q * fp16(amax / 127) with q = rint(v * 127 / amax) and amax over the 32 consecutive elements
+// the 32 lanes of a half-wave hold (quantize_row_q8_0, x86 path, ggml-quants.c:702-760), rounded to fp16 for a mat-mul input
+__device__ __forceinline__ float q8_block_value(float v) {
+    float amax = fabsf(v);
+#pragma unroll
+    for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, PI_WAVE));
+    const float d = pi_round_f16(pi_div(amax, 127.0f)), id = (amax != 0.0f) ? pi_div(127.0f, amax) : 0.0f;
+    return __fmul_rn((float)(int)rintf(__fmul_rn(v, id)), d);
+}
+
+// q8 != 0 (cols % 32 == 0, cols <= 8192): the normalised row goes through Q8_0 blocks of 32 before the fp16 rounding, which is what
+// a Q4_0 mat-mul of the CPU path multiplies with (ggml_vec_dot_q4_0_q8_0, ggml-quants.c:2512-2650)
+__global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __restrict__ x, int cols, NormArgs na, __half * __restrict__ out,
+                                                              __half * __restrict__ out_plain, int q8) {
+    __shared__ double red[16];
+    const float * xt = x + (size_t)blockIdx.x * cols;
+    __half * ot = out + (size_t)blockIdx.x * cols;
+    float mean = 0.0f, scale = 1.0f;
+    if (cols <= 8 * 1024) {
+        // one memory round trip: the row, the norm weights and the bias are requested together and stay in registers
+        float xv[8], wv[8], bv[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int i = threadIdx.x + k * 1024;
+            xv[k] = i < cols ? xt[i] : 0.0f;
+            wv[k] = (na.kind != 0 && na.w && i < cols) ? na.w[i] : 1.0f;
+            bv[k] = (na.kind != 0 && na.b && i < cols) ? na.b[i] : 0.0f;
+        }
+        if (na.kind == 1) {
+            double s = 0.0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) s += (double)__fmul_rn(xv[k], xv[k]);
+            s = block_sum_f64(s, red);
+            scale = pi_inv_sqrt((float)(s / cols) + na.eps);
+        } else if (na.kind == 2) {
+            double s = 0.0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) s += (double)xv[k];
+            s = block_sum_f64(s, red);
+            mean = (float)(s / cols);
+            double s2 = 0.0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) { const int i = threadIdx.x + k * 1024; const float v = __fsub_rn(xv[k], mean); if (i < cols) s2 += (double)__fmul_rn(v, v); }
+            s2 = block_sum_f64(s2, red);
+            scale = pi_inv_sqrt((float)(s2 / cols) + na.eps);
+        }
+#pragma unroll
+        for (int k = 0; k < 8; ++k) {
+            const int i = threadIdx.x + k * 1024;
+            float v = xv[k];
+            if (i < cols && out_plain) out_plain[(size_t)blockIdx.x * cols + i] = __float2half_rn(v);
+            if (na.kind != 0) {
+                v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
+                if (na.w) v = __fmul_rn(v, wv[k]);
+                if (na.b) v = __fadd_rn(v, bv[k]);
+            }
+            if (q8) v = q8_block_value(i < cols ? v : 0.0f);          // every lane takes part in the block's maximum
+            if (i < cols) ot[i] = __float2half_rn(v);
+        }
+        return;
+    }
+    if (na.kind == 1) {
+        double s = 0.0;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = xt[i]; s += (double)__fmul_rn(v, v); }
+        s = block_sum_f64(s, red);
+        scale = pi_inv_sqrt((float)(s / cols) + na.eps);
+    } else if (na.kind == 2) {
+        double s = 0.0;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) s += (double)xt[i];
+        s = block_sum_f64(s, red);
+        mean = (float)(s / cols);
+        double s2 = 0.0;
+        for (int i = threadIdx.x; i < cols; i += blockDim.x) { const float v = __fsub_rn(xt[i], mean); s2 += (double)__fmul_rn(v, v); }
+        s2 = block_sum_f64(s2, red);
+        scale = pi_inv_sqrt((float)(s2 / cols) + na.eps);
+    }
+    for (int i = threadIdx.x; i < cols; i += blockDim.x) {
+        float v = xt[i];
+        if (out_plain) out_plain[(size_t)blockIdx.x * cols + i] = __float2half_rn(v);
+        if (na.kind != 0) {
+            v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
+            if (na.w) v = __fmul_rn(v, na.w[i]);
+            if (na.b) v = __fadd_rn(v, na.b[i]);
+        }
+        ot[i] = __float2half_rn(v);
+    }
+}
+
+// y[t][row] = epi( W[row] . xn[t] ), t < T <= 16.  A workgroup owns 16*RT rows; its four waves split the columns in
+// quarters (cols % 128 == 0) and merge their 16 x 16 accumulator tiles through LDS in wave order.  A wave loads each
+// activation fragment once per 32-column step and uses it for its RT row tiles (the activations of a step are 16 x cols
+// fp16, as many bytes per row tile as the weights, so re-reading them per tile would double the L2 -> CU traffic);
+// 16 weight loads of 16 B per lane are in flight.
+template <int RT>
+__global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
+                                                              int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y,
+                                                              __half * __restrict__ y16, float thr, unsigned char * __restrict__ row_any) {
+    __shared__ float cs[kWavesPerBlock][16][17];
+    constexpr int SU = 16 / RT;                     // steps per batch of loads
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;
+    const int row0 = blockIdx.x * 16 * RT;
+    const int tok = i < T ? i : T - 1;
+    const int kw = cols / kWavesPerBlock;
+    const __half * ap[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        const int row = row0 + rt * 16 + i < rows ? row0 + rt * 16 + i : rows - 1;
+        ap[rt] = W + (size_t)row * cols + wave * kw + g * 8;
+    }
+    const __half * bp = xn + (size_t)tok * cols + wave * kw + g * 8;
+    pi_f4 acc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    const int steps = kw / 32;
+    for (int s0 = 0; s0 < steps; s0 += SU) {
+        pi_u32x4 a[SU][RT], b[SU];
+#pragma unroll
+        for (int u = 0; u < SU; ++u)
+            if (s0 + u < steps) {
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) a[u][rt] = pi_ld_stream(ap[rt] + (s0 + u) * 32);
+                b[u] = pi_ld16(bp + (s0 + u) * 32);
+            }
+#pragma unroll
+        for (int u = 0; u < SU; ++u)
+            if (s0 + u < steps) {
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt)
+                    acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a[u][rt]), __builtin_bit_cast(pi_h8, b[u]), acc[rt], 0, 0, 0);
+            }
+    }
+    const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        if (rt > 0) __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 4; ++r) cs[wave][4 * g + r][i] = acc[rt][r];
+        __syncthreads();
+        const int row = row0 + rt * 16 + rr;
+        bool act = false;
+        if (row < rows && t < T) {
+            float sum = cs[0][rr][t];
+#pragma unroll
+            for (int w = 1; w < kWavesPerBlock; ++w) sum += cs[w][rr][t];
+            const size_t o = (size_t)t * rows + row;
+            if (epi == PI_EPI_RELU) sum = fmaxf(sum, 0.0f);
+            else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
+            else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[o]), add2[o]);
+            y[o] = sum;
+            if (y16) y16[o] = __float2half_rn(sum);
+            act = !(sum < thr);
+        }
+        if (row_any) {      // predictor logits: is the row active for at least one token of the step?  (16 lanes = 16 tokens of a row)
+            const unsigned long long m = __ballot(act);
+            if (t == 0 && row < rows) row_any[row] = ((m >> (16 * (lane >> 4))) & 0xffffull) ? 1 : 0;
+        }
+    }
+}
+
+// The same mat-mul with row-contiguous global reads (cols % 256 == 0).  The MFMA operand layout wants lane l to hold
+// row l % 16, which makes a direct load instruction touch 16 rows x 64 B; here a wave instead reads 2 rows x 512 B per
+// instruction (8 instructions = its 16 rows x 256 columns), drops the tile into a wave-private LDS buffer with a padded
+// row stride (conflict-free both ways) and reads it back in operand layout.  No workgroup barrier is involved: the
+// buffer belongs to one wave and LDS operations of a wave complete in order.  Two 256-column tiles of loads are in flight.
+constexpr int kGlStride = 512 + 16;               // bytes per LDS row: 256 fp16 + one 16-byte pad
+template <int RT>
+__global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
+                                                                  int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y,
+                                                                  __half * __restrict__ y16, float thr, unsigned char * __restrict__ row_any) {
+    __shared__ __align__(16) unsigned char tile[kWavesPerBlock][16 * kGlStride];
+    __shared__ float cs[kWavesPerBlock][16][17];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;
+    const int lr = lane >> 5, lc = lane & 31;           // load role: row within the pair, 16-byte chunk within the 512-byte row piece
+    const int row0 = blockIdx.x * 16 * RT;
+    const int tok = i < T ? i : T - 1;
+    // the 256-column super-steps of a row are dealt round-robin to the four waves: wave w takes steps w, w + 4, ...
+    const __half * bp = xn + (size_t)tok * cols + g * 8;
+    unsigned char * mytile = tile[wave];
+    pi_f4 acc[RT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) acc[rt] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    const int n_ss = (cols / 256 - wave + kWavesPerBlock - 1) / kWavesPerBlock;      // super-steps of this wave
+    pi_u32x4 ld[2][RT][8];
+    auto issue = [&](int buf, int ss) {
+        if (ss < n_ss) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    int r = row0 + rt * 16 + 2 * j + lr;
+                    r = r < rows ? r : rows - 1;
+                    ld[buf][rt][j] = pi_ld_stream(W + (size_t)r * cols + (wave + ss * kWavesPerBlock) * 256 + lc * 8);
+                }
+        }
+    };
+    issue(0, 0);
+    issue(1, 1);
+    for (int ss = 0; ss < n_ss; ss += 2) {
+#pragma unroll
+        for (int buf = 0; buf < 2; ++buf) {
+            const int cur = ss + buf;
+            if (cur < n_ss) {
+                pi_u32x4 b[8];
+#pragma unroll
+                for (int st = 0; st < 8; ++st) b[st] = pi_ld16(bp + (wave + cur * kWavesPerBlock) * 256 + st * 32);
+#pragma unroll
+                for (int rt = 0; rt < RT; ++rt) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (2 * j + lr) * kGlStride + lc * 16) = ld[buf][rt][j];
+#pragma unroll
+                    for (int st = 0; st < 8; ++st) {
+                        const pi_u32x4 a = *reinterpret_cast<const pi_u32x4 *>(mytile + i * kGlStride + (4 * st + g) * 16);
+                        acc[rt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a), __builtin_bit_cast(pi_h8, b[st]), acc[rt], 0, 0, 0);
+                    }
+                }
+            }
+            issue(buf, cur + 2);
+        }
+    }
+    const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt) {
+        if (rt > 0) __syncthreads();
+#pragma unroll
+        for (int r = 0; r < 4; ++r) cs[wave][4 * g + r][i] = acc[rt][r];
+        __syncthreads();
+        const int row = row0 + rt * 16 + rr;
+        bool act = false;
+        if (row < rows && t < T) {
+            float sum = cs[0][rr][t];
+#pragma unroll
+            for (int w = 1; w < kWavesPerBlock; ++w) sum += cs[w][rr][t];
+            const size_t o = (size_t)t * rows + row;
+            if (epi == PI_EPI_RELU) sum = fmaxf(sum, 0.0f);
+            else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
+            else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[o]), add2[o]);
+            y[o] = sum;
+            if (y16) y16[o] = __float2half_rn(sum);
+            act = !(sum < thr);
+        }
+        if (row_any) {
+            const unsigned long long m = __ballot(act);
+            if (t == 0 && row < rows) row_any[row] = ((m >> (16 * (lane >> 4))) & 0xffffull) ? 1 : 0;
+        }
+    }
+}
+
+// Prompt chunks of up to 128 tokens: the same mat-mul with NT token tiles of 16 per row tile, so a weight row is read once per chunk
+// instead of once per 16 tokens.  A wave keeps its RT x 16 rows of a 256-column super-step in its private LDS tile (row-contiguous
+// global reads, as above; the load registers are free again once the tile is written, so the next super-step's loads are issued at
+// once and travel during the MFMAs) and streams the activations of all NT x 16 tokens past it, one 32-column step ahead.
+// K is split over the four waves of a workgroup (super-steps w, w + 4, ...); their partial tiles meet in LDS in wave order.
+template <int RT, int NT>
+__global__ __launch_bounds__(kBlock) void gemm_wide_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
+                                                               int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y,
+                                                               __half * __restrict__ y16) {
+    __shared__ __align__(16) unsigned char tile[kWavesPerBlock][RT * 16 * kGlStride];
+    __shared__ float cs[kWavesPerBlock][16][17];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;
+    const int lr = lane >> 5, lc = lane & 31;
+    const int row0 = blockIdx.x * 16 * RT;
+    // blockIdx.y: group of NT x 16 tokens (matrices with few rows are spread over more workgroups by splitting the chunk's tokens)
+    const int t_base = blockIdx.y * NT * 16;
+    xn += (size_t)t_base * cols; y += (size_t)t_base * rows; T -= t_base;
+    if (y16) y16 += (size_t)t_base * rows;
+    if (add1) add1 += (size_t)t_base * rows;
+    if (add2) add2 += (size_t)t_base * rows;
+    const __half * bp[NT];
+#pragma unroll
+    for (int nt = 0; nt < NT; ++nt) { const int tok = nt * 16 + i; bp[nt] = xn + (size_t)(tok < T ? tok : T - 1) * cols + g * 8; }
+    unsigned char * mytile = tile[wave];
+    pi_f4 acc[RT][NT];
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    const int n_ss = (cols / 256 - wave + kWavesPerBlock - 1) / kWavesPerBlock;
+    pi_u32x4 ld[RT][8];
+    auto issue = [&](int ss) {
+        if (ss < n_ss) {
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+                for (int j = 0; j < 8; ++j) {
+                    int r = row0 + rt * 16 + 2 * j + lr;
+                    r = r < rows ? r : rows - 1;
+                    ld[rt][j] = pi_ld_stream(W + (size_t)r * cols + (wave + ss * kWavesPerBlock) * 256 + lc * 8);
+                }
+        }
+    };
+    issue(0);
+    for (int ss = 0; ss < n_ss; ++ss) {
+        const int k0 = (wave + ss * kWavesPerBlock) * 256;
+        pi_u32x4 b[2][NT];
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) b[0][nt] = pi_ld16(bp[nt] + k0);
+#pragma unroll
+        for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+            for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (rt * 16 + 2 * j + lr) * kGlStride + lc * 16) = ld[rt][j];
+        issue(ss + 1);
+#pragma unroll
+        for (int st = 0; st < 8; ++st) {
+            if (st + 1 < 8) {
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) b[(st + 1) & 1][nt] = pi_ld16(bp[nt] + k0 + (st + 1) * 32);
+            }
+#pragma unroll
+            for (int rt = 0; rt < RT; ++rt) {
+                const pi_u32x4 a = *reinterpret_cast<const pi_u32x4 *>(mytile + (rt * 16 + i) * kGlStride + (4 * st + g) * 16);
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+                    acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a), __builtin_bit_cast(pi_h8, b[st & 1][nt]), acc[rt][nt], 0, 0, 0);
+            }
+        }
+    }
+    const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
+#pragma unroll
+    for (int rt = 0; rt < RT; ++rt)
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            __syncthreads();
+#pragma unroll
+            for (int r = 0; r < 4; ++r) cs[wave][4 * g + r][i] = acc[rt][nt][r];
+            __syncthreads();
+            const int row = row0 + rt * 16 + rr, tok = nt * 16 + t;
+            if (row < rows && tok < T) {
+                float sum = cs[0][rr][t];
+#pragma unroll
+                for (int w = 1; w < kWavesPerBlock; ++w) sum += cs[w][rr][t];
+                const size_t o = (size_t)tok * rows + row;
+                if (epi == PI_EPI_RELU) sum = fmaxf(sum, 0.0f);
+                else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
+                else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[o]), add2[o]);
+                y[o] = sum;
+                if (y16) y16[o] = __float2half_rn(sum);
+            }
+        }
+}
+// h16[t][n] = fp16( !(logit[t][n] < thr) ? relu(gate[t][n]) * up[t][n] : 0 )   (relu(up) without a gate): the FFN's hidden vector of a
+// prompt chunk from the dense gate/up products; inactive neurons become exact zeros, which add nothing in the down projection
+// q8 != 0 (n % 64 == 0 and n_ff % 32 == 0): h goes through Q8_0 blocks of 32 neurons first, as the CPU path's Q4_0 down projection quantises it
+// (ggml.c:14465-14618)
+__global__ void ffn_h_f16_kernel(const float * __restrict__ up, const float * __restrict__ gate, const float * __restrict__ logits, float thr,
+                                 size_t n, __half * __restrict__ h16, int q8) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        float h = 0.0f;
+        if (!(logits[i] < thr)) h = gate ? __fmul_rn(fmaxf(gate[i], 0.0f), up[i]) : fmaxf(up[i], 0.0f);
+        if (q8) h = q8_block_value(h);
+        h16[i] = __float2half_rn(h);
+    }
+}
+// out[c][r] = in[r][c] for an fp16 matrix [rows][cols] (32 x 32 tiles through LDS)
+__global__ void transpose_f16_kernel(const __half * __restrict__ in, int rows, int cols, __half * __restrict__ out) {
+    __shared__ __half t[32][33];
+    const int c0 = blockIdx.x * 32, r0 = blockIdx.y * 32;
+    for (int j = threadIdx.y; j < 32; j += blockDim.y) {
+        const int r = r0 + j, c = c0 + threadIdx.x;
+        if (r < rows && c < cols) t[j][threadIdx.x] = in[(size_t)r * cols + c];
+    }
+    __syncthreads();
+    for (int j = threadIdx.y; j < 32; j += blockDim.y) {
+        const int c = c0 + j, r = r0 + threadIdx.x;
+        if (r < rows && c < cols) out[(size_t)c * rows + r] = t[threadIdx.x][j];
+    }
+}
+
+// the operator boundary hands over the predictor's output instead of running the predictor: row_any[n] = some token has !(idx[t][n] < thr)
+__global__ void batch_flag_any_kernel(const float * __restrict__ idx, int T, int ff, float thr, unsigned char * __restrict__ row_any) {
+    const int n = blockIdx.x * blockDim.x + threadIdx.x;
+    if (n >= ff) return;
+    bool any = false;
+    for (int t = 0; t < T; ++t) any = any || !(idx[(size_t)t * ff + n] < thr);
+    row_any[n] = any ? 1 : 0;
+}
+// hc[t][u] = fp16(h[t][row_u]) where the row is active for token t, 0 elsewhere and in the padding up to the next multiple of 16
+__global__ void batch_gather_h_kernel(const float * __restrict__ h, const float * __restrict__ idx, int T, int ff, float thr,
+                                      const int32_t * __restrict__ list, const int32_t * __restrict__ n_union, __half * __restrict__ hc, int hstride) {
+    const int n = *n_union, n_pad = (n + 15) & ~15;
+    const int t = blockIdx.y;
+    for (int u = blockIdx.x * blockDim.x + threadIdx.x; u < n_pad; u += gridDim.x * blockDim.x) {
+        float v = 0.0f;
+        if (u < n && t < T) { const int row = list[u]; if (!(idx[(size_t)t * ff + row] < thr)) v = h[(size_t)t * ff + row]; }
+        hc[(size_t)t * hstride + u] = __float2half_rn(v);
+    }
+}
+__global__ void zero_f32_kernel(float * __restrict__ p, size_t n) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) p[i] = 0.0f;
+}
+
+// union over the tokens of the step of the predictor's active sets: ascending list of the neurons whose flag the
+// predictor's mat-mul epilogue raised (single workgroup: wave ballot per 64 neurons, popcount prefix over the mask words)
+__global__ __launch_bounds__(1024) void union_active_kernel(const unsigned char * __restrict__ row_any, int ff,
+                                                            uint32_t * __restrict__ words, int32_t * __restrict__ list, int32_t * __restrict__ n_union) {
+    __shared__ int sred[17];
+    const int lane = threadIdx.x & 63;
+    if ((ff & 31) == 0) {
+        // a thread takes 16 neurons (one 16-byte load); 16384 neurons per pass
+        int base = 0;
+        for (int i0 = 0; i0 < ff; i0 += 16 * 1024) {
+            const int i = i0 + threadIdx.x * 16;
+            uint32_t m = 0;
+            if (i < ff) {
+                const pi_u32x4 v = *reinterpret_cast<const pi_u32x4 *>(row_any + i);
+                const uint32_t d[4] = {v.x, v.y, v.z, v.w};
+#pragma unroll
+                for (int k = 0; k < 16; ++k) m |= (((d[k >> 2] >> ((k & 3) * 8)) & 0xFFu) != 0u ? 1u : 0u) << k;
+            }
+            const uint32_t hi = (uint32_t)__shfl_down((int)m, 1, PI_WAVE);
+            if ((threadIdx.x & 1) == 0 && i < ff) words[i >> 5] = m | (hi << 16);
+            int tot;
+            int off = base + block_exclusive_scan_i32(__popc(m), &tot, sred);
+            while (m) { const int b = __ffs(m) - 1; m &= m - 1; list[off++] = i + b; }
+            base += tot;
+            __syncthreads();
+        }
+        if (threadIdx.x == 0) *n_union = base;
+        return;
+    }
+    for (int i0 = 0; i0 < ff; i0 += blockDim.x) {
+        const int i = i0 + threadIdx.x;
+        const bool act = i < ff && row_any[i] != 0;
+        const unsigned long long m = __ballot(act);
+        if (lane == 0 && i < ff) words[i >> 5] = (uint32_t)m;
+        if (lane == 32 && i < ff) words[i >> 5] = (uint32_t)(m >> 32);
+    }
+    __syncthreads();
+    compact_from_words(words, ff, nullptr, 0, list, n_union, sred);
+}
+
+// sparse gate/up for the union rows: a workgroup gathers 16 rows of the union list into one MFMA tile (lane l reads
+// the row of list entry 16 * tile + l % 16), the four waves split the columns, then
+// hc[u][t] = active(t, row_u) ? relu(gate . x_t) * (up . x_t) : 0  (relu(up . x_t) without a gate).
+__global__ __launch_bounds__(kBlock) void batch_upgate_f16_kernel(const __half * __restrict__ Wup, const __half * __restrict__ Wgate, int cols,
+                                                                  const __half * __restrict__ xn, int T, const float * __restrict__ logits, int ff, float thr,
+                                                                  const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
+                                                                  __half * __restrict__ hc, int hstride) {
+    // hc[t][u] (token-major, stride hstride) holds h already rounded to fp16: the CPU axpy rounds h before use (ggml.c:14420-14431)
+    __shared__ float cu[kWavesPerBlock][16][17], cg[kWavesPerBlock][16][17];
+    const int n = *n_union;
+    const int u0 = blockIdx.x * 16;
+    if (u0 >= n) return;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;
+    const int row = list[u0 + i < n ? u0 + i : n - 1];
+    const int tok = i < T ? i : T - 1;
+    const int kw = cols / kWavesPerBlock;
+    const size_t aoff = (size_t)row * cols + wave * kw + g * 8;
+    const __half * bp = xn + (size_t)tok * cols + wave * kw + g * 8;
+    pi_f4 au = {0.0f, 0.0f, 0.0f, 0.0f}, ag = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int steps = kw / 32;
+    constexpr int UN = 4;
+    for (int s0 = 0; s0 < steps; s0 += UN) {
+        pi_u32x4 a[UN], c[UN], b[UN];
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+            if (s0 + u < steps) {
+                a[u] = pi_ld_stream(Wup + aoff + (s0 + u) * 32);
+                if (Wgate) c[u] = pi_ld_stream(Wgate + aoff + (s0 + u) * 32);
+                b[u] = pi_ld16(bp + (s0 + u) * 32);
+            }
+#pragma unroll
+        for (int u = 0; u < UN; ++u)
+            if (s0 + u < steps) {
+                au = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a[u]), __builtin_bit_cast(pi_h8, b[u]), au, 0, 0, 0);
+                if (Wgate) ag = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, c[u]), __builtin_bit_cast(pi_h8, b[u]), ag, 0, 0, 0);
+            }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) { cu[wave][4 * g + r][i] = au[r]; cg[wave][4 * g + r][i] = ag[r]; }
+    __syncthreads();
+    const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
+    float h = 0.0f;
+    if (u0 + rr < n && t < T) {
+        const int rrow = list[u0 + rr];
+        if (!(logits[(size_t)t * ff + rrow] < thr)) {
+            float su = cu[0][rr][t], sg = cg[0][rr][t];
+#pragma unroll
+            for (int w = 1; w < kWavesPerBlock; ++w) { su += cu[w][rr][t]; sg += cg[w][rr][t]; }
+            h = Wgate ? __fmul_rn(fmaxf(sg, 0.0f), su) : fmaxf(su, 0.0f);
+        }
+    }
+    hc[(size_t)t * hstride + u0 + rr] = __float2half_rn(h);
+}
+
+// sparse gate/up with row-contiguous reads (cols % 256 == 0): the loader of gemm_t16_lds_f16_kernel applied to the gathered
+// rows of the union list; the gate tile and the up tile of a 256-column step pass through the same wave-private LDS buffer.
+__global__ __launch_bounds__(kBlock) void batch_upgate_lds_f16_kernel(const __half * __restrict__ Wup, const __half * __restrict__ Wgate, int cols,
+                                                                      const __half * __restrict__ xn, int T, const float * __restrict__ logits, int ff, float thr,
+                                                                      const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
+                                                                      __half * __restrict__ hc, int hstride, float * __restrict__ raw) {
+    // raw != nullptr: the plain product of ONE matrix (Wgate == nullptr) for the operator boundary: raw[t][row] = Wup[row] . xn[t] for
+    // the tokens the row is active for and 0 for the others (rows outside the union list are zeroed by the caller); hc is not written
+    __shared__ __align__(16) unsigned char tile[kWavesPerBlock][16 * kGlStride];
+    __shared__ float cu[kWavesPerBlock][16][17], cg[kWavesPerBlock][16][17];
+    const int n = *n_union;
+    const int u0 = blockIdx.x * 16;
+    if (u0 >= n) return;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;
+    const int lr = lane >> 5, lc = lane & 31;
+    const int tok = i < T ? i : T - 1;
+    const __half * bp = xn + (size_t)tok * cols + g * 8;       // super-steps w, w + 4, ... of the row belong to wave w
+    unsigned char * mytile = tile[wave];
+    size_t roff[8];                                       // row offsets of the 8 load instructions of this lane
+#pragma unroll
+    for (int j = 0; j < 8; ++j) {
+        const int u = u0 + 2 * j + lr;
+        roff[j] = (size_t)list[u < n ? u : n - 1] * cols + wave * 256 + lc * 8;
+    }
+    const bool has_gate = Wgate != nullptr;
+    pi_f4 au = {0.0f, 0.0f, 0.0f, 0.0f}, ag = {0.0f, 0.0f, 0.0f, 0.0f};
+    const int n_ss = (cols / 256 - wave + kWavesPerBlock - 1) / kWavesPerBlock;
+    pi_u32x4 lu[2][8], lg[2][8];
+    auto issue = [&](int buf, int ss) {
+        if (ss < n_ss) {
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                lu[buf][j] = pi_ld_stream(Wup + roff[j] + ss * kWavesPerBlock * 256);
+                if (has_gate) lg[buf][j] = pi_ld_stream(Wgate + roff[j] + ss * kWavesPerBlock * 256);
+            }
+        }
+    };
+    issue(0, 0);
+    issue(1, 1);
+    for (int ss = 0; ss < n_ss; ss += 2) {
+#pragma unroll
+        for (int buf = 0; buf < 2; ++buf) {
+            const int cur = ss + buf;
+            if (cur < n_ss) {
+                pi_u32x4 b[8];
+#pragma unroll
+                for (int st = 0; st < 8; ++st) b[st] = pi_ld16(bp + (wave + cur * kWavesPerBlock) * 256 + st * 32);
+#pragma unroll
+                for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (2 * j + lr) * kGlStride + lc * 16) = lu[buf][j];
+#pragma unroll
+                for (int st = 0; st < 8; ++st) {
+                    const pi_u32x4 a = *reinterpret_cast<const pi_u32x4 *>(mytile + i * kGlStride + (4 * st + g) * 16);
+                    au = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a), __builtin_bit_cast(pi_h8, b[st]), au, 0, 0, 0);
+                }
+                if (has_gate) {
+#pragma unroll
+                    for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (2 * j + lr) * kGlStride + lc * 16) = lg[buf][j];
+#pragma unroll
+                    for (int st = 0; st < 8; ++st) {
+                        const pi_u32x4 a = *reinterpret_cast<const pi_u32x4 *>(mytile + i * kGlStride + (4 * st + g) * 16);
+                        ag = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a), __builtin_bit_cast(pi_h8, b[st]), ag, 0, 0, 0);
+                    }
+                }
+            }
+            issue(buf, cur + 2);
+        }
+    }
+#pragma unroll
+    for (int r = 0; r < 4; ++r) { cu[wave][4 * g + r][i] = au[r]; cg[wave][4 * g + r][i] = ag[r]; }
+    __syncthreads();
+    const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
+    float h = 0.0f, su = 0.0f;
+    int rrow = -1;
+    if (u0 + rr < n && t < T) {
+        rrow = list[u0 + rr];
+        if (!(logits[(size_t)t * ff + rrow] < thr)) {
+            float sg = cg[0][rr][t];
+            su = cu[0][rr][t];
+#pragma unroll
+            for (int w = 1; w < kWavesPerBlock; ++w) { su += cu[w][rr][t]; sg += cg[w][rr][t]; }
+            h = has_gate ? __fmul_rn(fmaxf(sg, 0.0f), su) : fmaxf(su, 0.0f);
+        }
+    }
+    if (raw) { if (rrow >= 0) raw[(size_t)t * ff + rrow] = su; }
+    else hc[(size_t)t * hstride + u0 + rr] = __float2half_rn(h);
+}
+
+// sparse down projection for the step: partial[g][t][c] = sum over the union entries of row group g of hc[u][t] * down[row_u][c].
+// A workgroup of 8 waves owns 256 columns (4 per lane, one 8-byte load per row) and one of G row groups; wave w of group g
+// walks entries u = 8g + w, + 8G, ...: a whole wave works on ONE row at a time, so the row's 16 h values are wave-uniform
+// and arrive through the scalar cache.  The 8 waves then add their 16 x 256 tiles into LDS one after the other (fixed order).
+constexpr int kBaGroups = 8;
+constexpr int kBaBlock = 512;
+constexpr int kBaWaves = kBaBlock / PI_WAVE;
+constexpr int kBaTile = 256;
+__global__ __launch_bounds__(kBaBlock) void batch_axpy_f16_kernel(const __half * __restrict__ Wd, int cols, const __half * __restrict__ hc, int hstride,
+                                                                  const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
+                                                                  float * __restrict__ partial) {
+    __shared__ float tile[kBtMaxT][kBaTile];
+    const int n = *n_union;
+    const int wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6), lane = threadIdx.x & 63;
+    const int c0 = blockIdx.x * kBaTile + lane * 4;
+    const int stride = kBaGroups * kBaWaves;
+    float acc[kBtMaxT][4];
+#pragma unroll
+    for (int t = 0; t < kBtMaxT; ++t)
+#pragma unroll
+        for (int k = 0; k < 4; ++k) acc[t][k] = 0.0f;
+    constexpr int UN = 8;
+    for (int u0 = blockIdx.y * kBaWaves + wave; u0 < n; u0 += stride * UN) {
+        pi_u32x2 w[UN];
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            const int u = u0 + j * stride;
+            w[j] = u < n ? __builtin_nontemporal_load(reinterpret_cast<const pi_u32x2 *>(Wd + (size_t)list[u] * cols + c0)) : pi_u32x2{0u, 0u};
+        }
+#pragma unroll
+        for (int j = 0; j < UN; ++j) {
+            const int u = u0 + j * stride;
+            if (u < n) {
+                const __half2 * hw = reinterpret_cast<const __half2 *>(&w[j]);
+                const float2 w01 = __half22float2(hw[0]), w23 = __half22float2(hw[1]);
+#pragma unroll
+                for (int t = 0; t < kBtMaxT; ++t) {
+                    const float h = __half2float(hc[(size_t)t * hstride + u]);
+                    acc[t][0] = fmaf(w01.x, h, acc[t][0]); acc[t][1] = fmaf(w01.y, h, acc[t][1]);
+                    acc[t][2] = fmaf(w23.x, h, acc[t][2]); acc[t][3] = fmaf(w23.y, h, acc[t][3]);
+                }
+            }
+        }
+    }
+    for (int w = 0; w < kBaWaves; ++w) {
+        if (wave == w) {
+#pragma unroll
+            for (int t = 0; t < kBtMaxT; ++t) {
+                float4 * p = reinterpret_cast<float4 *>(&tile[t][lane * 4]);
+                float4 v = w == 0 ? make_float4(0.0f, 0.0f, 0.0f, 0.0f) : *p;
+                v.x += acc[t][0]; v.y += acc[t][1]; v.z += acc[t][2]; v.w += acc[t][3];
+                *p = v;
+            }
+        }
+        __syncthreads();
+    }
+    for (int i = threadIdx.x; i < kBtMaxT * kBaTile / 4; i += kBaBlock) {
+        const int t = i / (kBaTile / 4), c4 = i % (kBaTile / 4);
+        *reinterpret_cast<float4 *>(partial + ((size_t)blockIdx.y * kBtMaxT + t) * cols + blockIdx.x * kBaTile + c4 * 4) =
+            *reinterpret_cast<const float4 *>(&tile[t][c4 * 4]);
+    }
+}
+
+// The down projection on the matrix cores (cols % 256 == 0).  out[t][c] = sum_u h[t][u] * down[row_u][c] has the union rows as its
+// reduction dimension, along which the weight matrix is NOT contiguous, so the operand layout cannot be loaded directly: a wave
+// reads 16 union rows x 256 columns row-contiguously (2 rows x 512 B per instruction), drops them into its private LDS tile and
+// reads the B fragments column-wise (4 rows of one column per lane: four 2-byte LDS reads) for 16 column tiles of
+// v_mfma_f32_16x16x16_f16; the A fragment is 4 consecutive entries of h[t][.] (one 8-byte load from the token-major h).
+// grid = (cols / 1024, G row groups); wave w of a workgroup owns columns 256 w .. 256 w + 255 of the workgroup's 1024 and walks
+// the 16-row steps g, g + G, ...; partial[g][t][c] is summed by batch_reduce_kernel.
+typedef _Float16 pi_h4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(kBlock) void batch_axpy_mfma_f16_kernel(const __half * __restrict__ Wd, int cols, const __half * __restrict__ hc, int hstride,
+                                                                     const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
+                                                                     float * __restrict__ partial) {
+    __shared__ __align__(16) unsigned char tile[kWavesPerBlock][16 * kGlStride];
+    const int n = *n_union;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;
+    const int lr = lane >> 5, lc = lane & 31;
+    const int c0 = blockIdx.x * 1024 + wave * 256;
+    if (c0 >= cols) return;                               // no workgroup barrier below: waves are independent
+    unsigned char * mytile = tile[wave];
+    pi_f4 acc[16];
+#pragma unroll
+    for (int ct = 0; ct < 16; ++ct) acc[ct] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    const int n_steps = (n + 15) / 16;
+    pi_u32x4 ld[2][8];
+    pi_u32x2 af[2];
+    auto issue = [&](int buf, int ks) {
+        if (ks < n_steps) {
+            const int u0 = ks * 16;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                const int u = u0 + 2 * j + lr;
+                ld[buf][j] = pi_ld_stream(Wd + (size_t)list[u < n ? u : n - 1] * cols + c0 + lc * 8);
+            }
+            af[buf] = *reinterpret_cast<const pi_u32x2 *>(hc + (size_t)i * hstride + u0 + 4 * g);      // zeros beyond n (written by the gate/up kernel)
+        }
+    };
+    issue(0, blockIdx.y);
+    issue(1, blockIdx.y + kBmGroups);
+    for (int ks = blockIdx.y; ks < n_steps; ks += 2 * kBmGroups) {
+#pragma unroll
+        for (int buf = 0; buf < 2; ++buf) {
+            const int cur = ks + buf * kBmGroups;
+            if (cur < n_steps) {
+#pragma unroll
+                for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (2 * j + lr) * kGlStride + lc * 16) = ld[buf][j];
+                const pi_h4 a = __builtin_bit_cast(pi_h4, af[buf]);
+#pragma unroll
+                for (int ct = 0; ct < 16; ++ct) {
+                    const unsigned char * bp = mytile + (4 * g) * kGlStride + (ct * 16 + i) * 2;
+                    const uint32_t e0 = *reinterpret_cast<const uint16_t *>(bp), e1 = *reinterpret_cast<const uint16_t *>(bp + kGlStride);
+                    const uint32_t e2 = *reinterpret_cast<const uint16_t *>(bp + 2 * kGlStride), e3 = *reinterpret_cast<const uint16_t *>(bp + 3 * kGlStride);
+                    const pi_u32x2 bw = {e0 | (e1 << 16), e2 | (e3 << 16)};
+                    acc[ct] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, __builtin_bit_cast(pi_h4, bw), acc[ct], 0, 0, 0);
+                }
+            }
+            issue(buf, cur + 2 * kBmGroups);
+        }
+    }
+    // accumulator lane l: tokens 4 * (l / 16) .. + 3 of column l % 16 of every column tile
+#pragma unroll
+    for (int ct = 0; ct < 16; ++ct)
+#pragma unroll
+        for (int r = 0; r < 4; ++r)
+            partial[((size_t)blockIdx.y * kBtMaxT + 4 * g + r) * cols + c0 + ct * 16 + i] = acc[ct][r];
+}
+
+__global__ __launch_bounds__(kBlock) void batch_reduce_kernel(const float * __restrict__ partial, int n_groups, int T, int cols, int epi,
+                                                              const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ out) {
+    const int idx = (blockIdx.x * blockDim.x + threadIdx.x) * 4;          // cols % 4 == 0: four columns of one token
+    if (idx >= T * cols) return;
+    const int t = idx / cols, c = idx - t * cols;
+    const size_t gstride = (size_t)kBtMaxT * cols;
+    const float * p = partial + (size_t)t * cols + c;
+    float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (int g0 = 0; g0 < n_groups; g0 += 8) {
+        float4 v[8];
+#pragma unroll
+        for (int j = 0; j < 8; ++j) v[j] = g0 + j < n_groups ? *reinterpret_cast<const float4 *>(p + (size_t)(g0 + j) * gstride) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+        for (int j = 0; j < 8; ++j) { sum.x += v[j].x; sum.y += v[j].y; sum.z += v[j].z; sum.w += v[j].w; }
+    }
+    if (epi >= PI_EPI_ADD) { const float4 a = *reinterpret_cast<const float4 *>(add1 + idx); sum.x = __fadd_rn(sum.x, a.x); sum.y = __fadd_rn(sum.y, a.y); sum.z = __fadd_rn(sum.z, a.z); sum.w = __fadd_rn(sum.w, a.w); }
+    if (epi == PI_EPI_ADD2) { const float4 a = *reinterpret_cast<const float4 *>(add2 + idx); sum.x = __fadd_rn(sum.x, a.x); sum.y = __fadd_rn(sum.y, a.y); sum.z = __fadd_rn(sum.z, a.z); sum.w = __fadd_rn(sum.w, a.w); }
+    *reinterpret_cast<float4 *>(out + idx) = sum;
+}
+
+__global__ void embed_f16_batch_kernel(const __half * __restrict__ table, int cols, const int32_t * __restrict__ tokens, float * __restrict__ x) {
+    const int c = blockIdx.x * blockDim.x + threadIdx.x;
+    if (c < cols) x[(size_t)blockIdx.y * cols + c] = __half2float(table[(size_t)tokens[blockIdx.y] * cols + c]);
+}
+
+// greedy choice per sequence (first maximum wins, llama.cpp:8617-8631), then the sequence's state moves on: its next token,
+// its position + 1; workgroup 0 also advances the step counter after recording the step's tokens.
+__global__ __launch_bounds__(1024) void argmax_batch_kernel(const float * __restrict__ logits, int n, int T, int32_t * __restrict__ tokens,
+                                                            int32_t * __restrict__ positions, int32_t * __restrict__ step,
+                                                            int32_t * __restrict__ out_tokens, int max_steps) {
+    __shared__ float bv[16];
+    __shared__ int   bi[16];
+    const int t = blockIdx.x;
+    const float * lg = logits + (size_t)t * n;
+    float best = -INFINITY; int idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) { const float v = lg[i]; if (v > best) { best = v; idx = i; } }
+    for (int o = 32; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, PI_WAVE); const int oi = __shfl_xor(idx, o, PI_WAVE);
+        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+    }
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) { bv[wave] = best; bi[wave] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < 16; ++w) if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
+        if (idx >= n) idx = 0;             // no logit compared greater than -inf (all NaN or -inf): a valid row for the next embedding lookup
+        tokens[t] = idx;
+        if (positions) positions[t] += 1;
+        const int s = step ? *step : 0;
+        if (out_tokens && s < max_steps) out_tokens[(size_t)s * T + t] = idx;
+    }
+}
+
+__global__ void step_advance_kernel(int32_t * step) { if (threadIdx.x == 0) *step += 1; }
+
+}  // namespace
+
+extern "C" {
+
+int pi_k_norm_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, void * out_plain_f16, pi_stream_t stream) {
+    if (!x || !out_f16 || T <= 0 || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_norm_round_f16: bad arguments");
+    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16, (__half *)out_plain_f16, 0);
+    return pi::check_launch("pi_k_norm_round_f16");
+}
+
+int pi_k_norm_q8_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, void * out_plain_f16, pi_stream_t stream) {
+    if (!x || !out_f16 || T <= 0 || cols <= 0 || cols % 32 || cols > 8 * 1024) return pi::fail(PI_E_ARG, "pi_k_norm_q8_round_f16: cols must be a multiple of 32, at most 8192");
+    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16, (__half *)out_plain_f16, 1);
+    return pi::check_launch("pi_k_norm_q8_round_f16");
+}
+
+static int gemm_launch(const char * who, const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
+                       float * y, void * y_f16, float thr, unsigned char * row_any, pi_stream_t stream) {
+    if (!W || !xn_f16 || !y || rows <= 0) return pi::fail(PI_E_ARG, who);
+    if (T < 1 || T > kBtMaxT || cols <= 0 || cols % 128) return pi::fail(PI_E_ARG, "batched mat-mul: 1 <= T <= 16 and cols % 128 == 0 required");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "batched mat-mul: bad epilogue arguments");
+    // row tiles per wave: enough workgroups to fill the chip first, then as few reads of the activations as possible
+    const int rt = rows >= 16384 ? 4 : rows >= 5120 ? 2 : 1;      // (two tiles already at 5120 rows: the activations, re-read per row tile, are what limits one tile per wave)
+#define PI_GEMM_T16(RT) hipLaunchKernelGGL((gemm_t16_f16_kernel<RT>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(kBlock), 0, (hipStream_t)stream, \
+                       (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any)
+#define PI_GEMM_LDS(RT) hipLaunchKernelGGL((gemm_t16_lds_f16_kernel<RT>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(kBlock), 0, (hipStream_t)stream, \
+                       (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any)
+    if (cols % 256 == 0) { if (rt >= 2) PI_GEMM_LDS(2); else PI_GEMM_LDS(1); }
+    else if (rt == 4) PI_GEMM_T16(4); else if (rt == 2) PI_GEMM_T16(2); else PI_GEMM_T16(1);
+#undef PI_GEMM_LDS
+#undef PI_GEMM_T16
+    return pi::check_launch(who);
+}
+
+int pi_k_gemm_f16(const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
+                  float * y, void * y_f16, pi_stream_t stream) {
+    return gemm_launch("pi_k_gemm_f16", W, rows, cols, xn_f16, T, epilogue, add1, add2, y, y_f16, 0.0f, nullptr, stream);
+}
+
+int pi_k_gemm_wide_f16(const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
+                       float * y, void * y_f16, pi_stream_t stream) {
+    if (!W || !xn_f16 || !y || rows <= 0) return pi::fail(PI_E_ARG, "pi_k_gemm_wide_f16: null pointer or empty shape");
+    if (T < 1 || T > kWideMaxT || cols <= 0 || cols % 256) return pi::fail(PI_E_ARG, "pi_k_gemm_wide_f16: 1 <= T <= 128 and cols % 256 == 0 required");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_gemm_wide_f16: bad epilogue arguments");
+    if (T <= kBtMaxT) return gemm_launch("pi_k_gemm_wide_f16", W, rows, cols, xn_f16, T, epilogue, add1, add2, y, y_f16, 0.0f, nullptr, stream);
+#define PI_GEMM_WIDE(RT, NT) hipLaunchKernelGGL((gemm_wide_f16_kernel<RT, NT>), dim3((rows + 16 * RT - 1) / (16 * RT), (T + 16 * NT - 1) / (16 * NT)), dim3(kBlock), 0, \
+        (hipStream_t)stream, (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16)
+    // tile shape by row count: wide matrices take 64 rows x the whole chunk per workgroup; narrower ones split the chunk's tokens over
+    // several workgroups so that the grid still covers the chip (their weights then pass through L2 once per token group)
+    if (rows >= 8192) { if (T <= 32) PI_GEMM_WIDE(2, 2); else if (T <= 64) PI_GEMM_WIDE(4, 4); else PI_GEMM_WIDE(4, 8); }
+    else if (rows > 2048) { if (T <= 32) PI_GEMM_WIDE(2, 2); else PI_GEMM_WIDE(2, 4); }
+    else PI_GEMM_WIDE(1, 2);
+#undef PI_GEMM_WIDE
+    return pi::check_launch("pi_k_gemm_wide_f16");
+}
+int pi_k_ffn_h_f16(const float * up, const float * gate, const float * logits, float threshold, int T, int ff, void * h_f16, pi_stream_t stream) {
+    if (!up || !logits || !h_f16 || T <= 0 || ff <= 0) return pi::fail(PI_E_ARG, "pi_k_ffn_h_f16: bad arguments");
+    hipLaunchKernelGGL(ffn_h_f16_kernel, dim3(1024), dim3(256), 0, (hipStream_t)stream, up, gate, logits, threshold, (size_t)T * ff, (__half *)h_f16, 0);
+    return pi::check_launch("pi_k_ffn_h_f16");
+}
+int pi_k_ffn_h_q8_f16(const float * up, const float * gate, const float * logits, float threshold, int T, int ff, void * h_f16, pi_stream_t stream) {
+    if (!up || !logits || !h_f16 || T <= 0 || ff <= 0 || ff % 64) return pi::fail(PI_E_ARG, "pi_k_ffn_h_q8_f16: n_ff must be a multiple of 64");
+    hipLaunchKernelGGL(ffn_h_f16_kernel, dim3(1024), dim3(256), 0, (hipStream_t)stream, up, gate, logits, threshold, (size_t)T * ff, (__half *)h_f16, 1);
+    return pi::check_launch("pi_k_ffn_h_q8_f16");
+}
+
+// W[rows][cols] in Q4_0 blocks -> fp16 (value (q - 8) * d, dequantize_row_q4_0, ggml-quants.c:1074-1092), one thread per block.  With hot
+// words the rows of resident neurons come from the compact matrix W and the others from W_rest (both in ascending neuron order).
+__global__ void dequant_q4_f16_kernel(const pi_block_q4_0 * __restrict__ W, const pi_block_q4_0 * __restrict__ W_rest,
+                                      const uint32_t * __restrict__ hot_words, const int32_t * __restrict__ hot_prefix,
+                                      int rows, int nb, __half * __restrict__ out) {
+    const size_t n = (size_t)rows * nb;
+    for (size_t idx = (size_t)blockIdx.x * blockDim.x + threadIdx.x; idx < n; idx += (size_t)gridDim.x * blockDim.x) {
+        const int row = (int)(idx / nb), blk = (int)(idx % nb);
+        const pi_block_q4_0 * src;
+        if (hot_words) {
+            const uint32_t hot = hot_words[row >> 5];
+            const int bit = row & 31, base = hot_prefix[row >> 5], below = __popc(hot & ((1u << bit) - 1u));
+            src = ((hot >> bit) & 1u) ? W + (size_t)(base + below) * nb : W_rest + (size_t)((row & ~31) - base + bit - below) * nb;
+        } else {
+            src = W + (size_t)row * nb;
+        }
+        src += blk;
+        uint16_t dbits; __builtin_memcpy(&dbits, &src->d, 2);
+        const float d = pi_f16_from_bits(dbits);
+        uint32_t qs[4]; __builtin_memcpy(qs, src->qs, 16);
+        __align__(16) __half o[32];
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int b = (qs[j >> 2] >> ((j & 3) * 8)) & 0xFF;
+            o[j] = __float2half_rn(__fmul_rn((float)((b & 0x0F) - 8), d));
+            o[j + 16] = __float2half_rn(__fmul_rn((float)((b >> 4) - 8), d));
+        }
+        pi_u32x4 * dst = reinterpret_cast<pi_u32x4 *>(out + (size_t)row * nb * 32 + blk * 32);
+#pragma unroll
+        for (int k = 0; k < 4; ++k) dst[k] = reinterpret_cast<const pi_u32x4 *>(o)[k];
+    }
+}
+int pi_k_dequant_q4_f16(const void * W_q4, const void * W_rest_q4, const uint32_t * hot_words, const int32_t * hot_prefix, int rows, int cols,
+                        void * out_f16, pi_stream_t stream) {
+    if (!W_q4 || !out_f16 || rows <= 0 || cols <= 0 || cols % 32) return pi::fail(PI_E_ARG, "pi_k_dequant_q4_f16: bad arguments");
+    if ((hot_words == nullptr) != (hot_prefix == nullptr) || (hot_words && !W_rest_q4) || (hot_words && rows % 32))
+        return pi::fail(PI_E_ARG, "pi_k_dequant_q4_f16: hot_words, hot_prefix and the second matrix go together (rows % 32 == 0)");
+    const size_t n = (size_t)rows * (cols / 32);
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 8192) blocks = 8192;
+    hipLaunchKernelGGL(dequant_q4_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (const pi_block_q4_0 *)W_q4, (const pi_block_q4_0 *)W_rest_q4,
+                       hot_words, hot_prefix, rows, cols / 32, (__half *)out_f16);
+    return pi::check_launch("pi_k_dequant_q4_f16");
+}
+// the full fp16 matrix of a hybrid layer from the compact matrix of the resident neurons and the matrix of the others (both in
+// ascending neuron order); one workgroup per row, 16 bytes per lane and pass
+__global__ void assemble_rows_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ W_rest, const uint32_t * __restrict__ hot_words,
+                                         const int32_t * __restrict__ hot_prefix, int cols, __half * __restrict__ out) {
+    const int row = blockIdx.x;
+    const uint32_t hot = hot_words[row >> 5];
+    const int bit = row & 31, base = hot_prefix[row >> 5], below = __popc(hot & ((1u << bit) - 1u));
+    const __half * src = ((hot >> bit) & 1u) ? W + (size_t)(base + below) * cols : W_rest + (size_t)((row & ~31) - base + bit - below) * cols;
+    const pi_u32x4 * s4 = reinterpret_cast<const pi_u32x4 *>(src);
+    pi_u32x4 * d4 = reinterpret_cast<pi_u32x4 *>(out + (size_t)row * cols);
+    for (int i = threadIdx.x; i < cols / 8; i += blockDim.x) d4[i] = s4[i];
+}
+int pi_k_assemble_rows_f16(const void * W_f16, const void * W_rest_f16, const uint32_t * hot_words, const int32_t * hot_prefix, int rows, int cols,
+                           void * out_f16, pi_stream_t stream) {
+    if (!W_f16 || !W_rest_f16 || !hot_words || !hot_prefix || !out_f16 || rows <= 0 || rows % 32 || cols <= 0 || cols % 8)
+        return pi::fail(PI_E_ARG, "pi_k_assemble_rows_f16: bad arguments (rows % 32 == 0, cols % 8 == 0)");
+    hipLaunchKernelGGL(assemble_rows_f16_kernel, dim3(rows), dim3(256), 0, (hipStream_t)stream, (const __half *)W_f16, (const __half *)W_rest_f16,
+                       hot_words, hot_prefix, cols, (__half *)out_f16);
+    return pi::check_launch("pi_k_assemble_rows_f16");
+}
+int pi_k_transpose_f16(const void * in, int rows, int cols, void * out, pi_stream_t stream) {
+    if (!in || !out || rows <= 0 || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_transpose_f16: bad arguments");
+    hipLaunchKernelGGL(transpose_f16_kernel, dim3((cols + 31) / 32, (rows + 31) / 32), dim3(32, 8), 0, (hipStream_t)stream, (const __half *)in, rows, cols, (__half *)out);
+    return pi::check_launch("pi_k_transpose_f16");
+}
+
+int pi_k_batch_predictor_fc2(const void * fc2_f16, int ff, int r, const void * hidden_f16, int T, float threshold, float * logits,
+                             pi_workspace * ws, pi_stream_t stream) {
+    if (!ws || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_batch_predictor_fc2: ff exceeds the workspace");
+    return gemm_launch("pi_k_batch_predictor_fc2", fc2_f16, ff, r, hidden_f16, T, PI_EPI_NONE, nullptr, nullptr, logits, nullptr, threshold, ws->row_any, stream);
+}
+
+int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, const void * up_f16, const void * gate_f16, const void * down_t_f16,
+                          int cols, const void * xn_f16, int epilogue, const float * add1, const float * add2, float * out,
+                          int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream) {
+    if (!logits || !up_f16 || !down_t_f16 || !xn_f16 || !out || !union_rows || !n_union || !ws) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: null pointer");
+    if (T < 1 || T > kBtMaxT || ff <= 0 || ff > ws->max_ff || cols <= 0 || cols > ws->max_d || cols % kBaTile || cols % 128)
+        return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: 1 <= T <= 16, ff <= workspace, cols % 256 == 0 and cols <= workspace required");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: bad epilogue arguments");
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, ws->row_any, ff, ws->words, union_rows, n_union);
+    const int hstride = ws->max_ff + 16;
+    if (cols % 256 == 0) {
+        hipLaunchKernelGGL(batch_upgate_lds_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
+                           (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride, (float *)nullptr);
+        hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3((cols + 1023) / 1024, kBmGroups), dim3(kBlock), 0, st, (const __half *)down_t_f16, cols,
+                           ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
+        hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBmGroups, T, cols, epilogue, add1, add2, out);
+    } else {
+        hipLaunchKernelGGL(batch_upgate_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
+                           (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
+        hipLaunchKernelGGL(batch_axpy_f16_kernel, dim3(cols / kBaTile, kBaGroups), dim3(kBaBlock), 0, st, (const __half *)down_t_f16, cols,
+                           ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
+        hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBaGroups, T, cols, epilogue, add1, add2, out);
+    }
+    return pi::check_launch("pi_k_batch_sparse_ffn");
+}
+
+// The two sparse operators of a step of T <= 16 tokens AS OPERATORS (the reference's mul_mat_batch_sparse / axpy at batch size > 1,
+// ggml-cuda.cu:6994-7034, 8787-8814): the caller supplies the predictor output idx [T][ff]; each weight row is read once for the step.
+int pi_k_batch_sparse_mul_mat(const void * W_f16, int ff, int cols, const void * xn_f16, int T, const float * idx, float threshold,
+                              float * y, int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream) {
+    if (!W_f16 || !xn_f16 || !idx || !y || !union_rows || !n_union || !ws) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_mul_mat: null pointer");
+    if (T < 1 || T > kBtMaxT || ff <= 0 || ff > ws->max_ff || cols <= 0 || cols % 256) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_mul_mat: 1 <= T <= 16, ff <= workspace and cols % 256 == 0 required");
+    hipStream_t st = (hipStream_t)stream;
+    hipLaunchKernelGGL(batch_flag_any_kernel, dim3((ff + 255) / 256), dim3(256), 0, st, idx, T, ff, threshold, ws->row_any);
+    hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, ws->row_any, ff, ws->words, union_rows, n_union);
+    hipLaunchKernelGGL(zero_f32_kernel, dim3(256), dim3(256), 0, st, y, (size_t)T * ff);
+    hipLaunchKernelGGL(batch_upgate_lds_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)W_f16, (const __half *)nullptr, cols,
+                       (const __half *)xn_f16, T, idx, ff, threshold, union_rows, n_union, ws->hc_batch, ws->max_ff + 16, y);
+    return pi::check_launch("pi_k_batch_sparse_mul_mat");
+}
+int pi_k_batch_sparse_axpy(const void * down_t_f16, int cols, int ff, const float * h, const float * idx, int T, float threshold,
+                           float * out, int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream) {
+    if (!down_t_f16 || !h || !idx || !out || !union_rows || !n_union || !ws) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_axpy: null pointer");
+    if (T < 1 || T > kBtMaxT || ff <= 0 || ff > ws->max_ff || cols <= 0 || cols > ws->max_d || cols % 256)
+        return pi::fail(PI_E_ARG, "pi_k_batch_sparse_axpy: 1 <= T <= 16, ff and cols within the workspace and cols % 256 == 0 required");
+    hipStream_t st = (hipStream_t)stream;
+    const int hstride = ws->max_ff + 16;
+    hipLaunchKernelGGL(batch_flag_any_kernel, dim3((ff + 255) / 256), dim3(256), 0, st, idx, T, ff, threshold, ws->row_any);
+    hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, ws->row_any, ff, ws->words, union_rows, n_union);
+    hipLaunchKernelGGL(batch_gather_h_kernel, dim3(32, kBtMaxT), dim3(256), 0, st, h, idx, T, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
+    hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3((cols + 1023) / 1024, kBmGroups), dim3(kBlock), 0, st, (const __half *)down_t_f16, cols,
+                       ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
+    hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBmGroups, T, cols, PI_EPI_NONE,
+                       (const float *)nullptr, (const float *)nullptr, out);
+    return pi::check_launch("pi_k_batch_sparse_axpy");
+}
+
+int pi_k_step_advance(int32_t * step, pi_stream_t stream) {
+    if (!step) return pi::fail(PI_E_ARG, "pi_k_step_advance: null pointer");
+    hipLaunchKernelGGL(step_advance_kernel, dim3(1), dim3(64), 0, (hipStream_t)stream, step);
+    return pi::check_launch("pi_k_step_advance");
+}
+
+int pi_k_embed_batch(const void * table_f16, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream) {
+    if (!table_f16 || !tokens || !x || cols <= 0 || T <= 0 || T > kChunkMaxT) return pi::fail(PI_E_ARG, "pi_k_embed_batch: bad arguments");
+    hipLaunchKernelGGL(embed_f16_batch_kernel, dim3((cols + 255) / 256, T), dim3(256), 0, (hipStream_t)stream, (const __half *)table_f16, cols, tokens, x);
+    return pi::check_launch("pi_k_embed_batch");
+}
+
+
+int pi_k_argmax_batch(const float * logits, int n, int T, int32_t * tokens, int32_t * positions, int32_t * step, int32_t * out_tokens, int max_steps,
+                      pi_stream_t stream) {
+    if (!logits || !tokens || n <= 0 || T <= 0 || T > kBtMaxT) return pi::fail(PI_E_ARG, "pi_k_argmax_batch: bad arguments");
+    hipLaunchKernelGGL(argmax_batch_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, logits, n, T, tokens, positions, step, out_tokens, max_steps);
+    return pi::check_launch("pi_k_argmax_batch");
+}
+
+}  // extern "C"

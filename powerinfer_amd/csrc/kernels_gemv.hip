@@ -1,0 +1,702 @@
+// Mat-vecs of one token (fp16 and Q4_0 rows, fused norm prologue, ReLU / residual epilogues), embedding rows, greedy argmax, the
+// random fills of synthetic models, and the workspace of the pi_k_* launchers.  gfx950, wave64.  Citations are file:line into the
+// reference tree.
+#include "kernels_common.hpp"
+
+namespace {
+
+// ---------------------------------------------------------------------------------------------------
+// Dense F16 mat-vec.  A fixed grid of about two workgroups per CU (what a pure streaming read needs to reach
+// HBM speed on this chip), each wave walking row groups g = wave_id, wave_id + n_waves, ...  A group is RPW
+// consecutive rows; lane l reads 16 B (8 halfs) at column 8*l + 512*c of each row (chunk c), i.e. 1 KiB
+// contiguous per row per load instruction.  The (group, chunk) space of a wave is flattened into steps of U
+// chunks with one step of loads always in flight; the first step is issued before the activations are
+// staged (weights do not depend on them).  Fast path: cols % 512 == 0 and rows % RPW == 0 (no guards).
+// TAG only separates instantiations by role so that kernel traces can tell them apart.
+// ---------------------------------------------------------------------------------------------------
+constexpr int kGemvBlocks = 512;
+
+template <int RPW, int U, int TAG>
+__global__ __launch_bounds__(kBlock) void gemv_f16_kernel(const __half * __restrict__ W, const float * __restrict__ x, NormArgs na,
+                                                          int epi, const float * add1, const float * add2,
+                                                          float * __restrict__ y, int rows, int cols) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    float * lds = reinterpret_cast<float *>(smem);
+    __half * xs = reinterpret_cast<__half *>(smem + (size_t)cols * 8);
+    __shared__ double red[16];
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n_waves = gridDim.x * kWavesPerBlock, wid = blockIdx.x * kWavesPerBlock + wave;
+    const int n_groups = rows / RPW;
+    const int spg = cols / (PI_WAVE * 8 * U);                              // steps per group
+    const int my_groups = wid < n_groups ? (n_groups - wid + n_waves - 1) / n_waves : 0;
+    const int T = my_groups * spg;
+
+    stage_fast_issue(lds, x, na, cols);
+
+    pi_u32x4 buf[RPW][U], nxt[RPW][U];
+    const __half * wp = W + (size_t)wid * RPW * cols + lane * 8;           // this wave's position in the (group, step) walk
+    int sig = 0;                                                           // step within the current group
+    auto issue = [&](pi_u32x4 (&dst)[RPW][U]) {
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int i = 0; i < RPW; ++i) dst[i][u] = pi_ld_stream(wp + (size_t)i * cols + u * (PI_WAVE * 8));
+        wp += U * PI_WAVE * 8;
+        if (++sig == spg) { sig = 0; wp += (size_t)(n_waves * RPW - 1) * cols; }   // next group: (n_waves*RPW) rows down, back to column 0
+    };
+    if (T > 0) issue(buf);
+    // the direct-to-LDS loads were issued first and complete in order: allow only the weight loads to remain in flight
+    asm volatile("s_waitcnt vmcnt(%0)" ::"n"(RPW * U) : "memory");
+    __syncthreads();
+    stage_fast_finish(xs, lds, na, cols, red);
+
+    float acc[RPW];
+#pragma unroll
+    for (int i = 0; i < RPW; ++i) acc[i] = 0.0f;
+    int row = wid * RPW, c = lane * 8, s_in = 0;
+    for (int t = 0; t < T; ++t) {
+        if (t + 1 < T) issue(nxt);
+#pragma unroll
+        for (int u = 0; u < U; ++u) {
+            float xf[8];
+            pi_unpack8(pi_ld16(xs + c + u * (PI_WAVE * 8)), xf);
+#pragma unroll
+            for (int i = 0; i < RPW; ++i) acc[i] = pi_dot8(buf[i][u], xf, acc[i]);
+        }
+        c += U * PI_WAVE * 8;
+        if (++s_in == spg) {
+#pragma unroll
+            for (int i = 0; i < RPW; ++i) {
+                const float sum = pi_wave_sum(acc[i]);
+                if (lane == 0) y[row + i] = apply_epilogue(sum, epi, add1, add2, row + i);
+                acc[i] = 0.0f;
+            }
+            s_in = 0; c = lane * 8; row += n_waves * RPW;
+        }
+#pragma unroll
+        for (int u = 0; u < U; ++u)
+#pragma unroll
+            for (int i = 0; i < RPW; ++i) buf[i][u] = nxt[i][u];
+    }
+}
+
+// Register-resident variant for cols == 512 * NCH (4096, 5120, 8192): a wave owns whole rows
+// (row = wave_id, wave_id + n_waves, ...), lane l holds the activations of columns 8*l + 512*j as packed fp16 in
+// registers, so the row loop touches neither LDS nor a workgroup barrier.  The prologue is shared by the four
+// waves of a workgroup: wave w loads and normalises chunks w, w+4, ... of the vector (statistics cross the waves
+// through LDS in wave order), the packed fp16 result meets in LDS and every wave reads all of it back once.
+// 16 weight loads of 16 B per lane are in flight throughout (two rows, or the two halves of a wide row) and
+// are issued before the prologue starts.  The residual operands of the epilogue travel with the row.
+// KIND: 0 no norm, 1 RMSNorm * w, 2 LayerNorm * w + b.  TAG only names the role in kernel traces.
+template <int NCH, int KIND, int TAG>
+__global__ __launch_bounds__(kBlock, 2) void gemv_f16_reg_kernel(const __half * __restrict__ W, const float * __restrict__ x,
+                                                              const float * __restrict__ nw, const float * __restrict__ nb, float eps,
+                                                              int epi, const float * __restrict__ add1, const float * __restrict__ add2,
+                                                              float * __restrict__ y, int rows) {
+    constexpr int cols = NCH * 512;
+    constexpr bool kWide = NCH > 8;               // wide rows: the two buffers hold the halves of one row
+    constexpr int CPB = kWide ? NCH / 2 : NCH;
+    static_assert(!kWide || NCH % 2 == 0, "wide rows are split in two halves");
+    constexpr int MYCH = (NCH + kWavesPerBlock - 1) / kWavesPerBlock;      // chunks a wave normalises
+    __shared__ __align__(16) __half xs[cols];
+    __shared__ double red[2][kWavesPerBlock];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n_waves = gridDim.x * kWavesPerBlock, wid = blockIdx.x * kWavesPerBlock + wave;
+    pi_u32x4 buf[2][CPB];
+    float r1[2] = {0.0f, 0.0f}, r2[2] = {0.0f, 0.0f};
+    auto issue = [&](int b, int r) {
+        if (r < rows) {
+            const __half * wp = W + (size_t)r * cols + lane * 8 + (kWide ? b * CPB * 512 : 0);
+#pragma unroll
+            for (int j = 0; j < CPB; ++j) buf[b][j] = pi_ld_stream(wp + j * 512);
+            if (!kWide || b == 0) {
+                if (epi >= PI_EPI_ADD) r1[b] = add1[r];
+                if (epi == PI_EPI_ADD2) r2[b] = add2[r];
+            }
+        }
+    };
+    issue(0, wid);
+    issue(1, kWide ? wid : wid + n_waves);
+
+    // ---- shared prologue ---------------------------------------------------------------------------------
+    {
+        float xv[MYCH][8], wv[MYCH][8], bv[MYCH][8];
+#pragma unroll
+        for (int i = 0; i < MYCH; ++i) {
+            const int j = wave + i * kWavesPerBlock;
+            if (j < NCH) {
+                const int o = j * 512 + lane * 8;
+                const float4 a = *reinterpret_cast<const float4 *>(x + o), b = *reinterpret_cast<const float4 *>(x + o + 4);
+                xv[i][0] = a.x; xv[i][1] = a.y; xv[i][2] = a.z; xv[i][3] = a.w; xv[i][4] = b.x; xv[i][5] = b.y; xv[i][6] = b.z; xv[i][7] = b.w;
+                if (KIND >= 1) {
+                    const float4 c = *reinterpret_cast<const float4 *>(nw + o), e = *reinterpret_cast<const float4 *>(nw + o + 4);
+                    wv[i][0] = c.x; wv[i][1] = c.y; wv[i][2] = c.z; wv[i][3] = c.w; wv[i][4] = e.x; wv[i][5] = e.y; wv[i][6] = e.z; wv[i][7] = e.w;
+                }
+                if (KIND == 2) {
+                    const float4 c = *reinterpret_cast<const float4 *>(nb + o), e = *reinterpret_cast<const float4 *>(nb + o + 4);
+                    bv[i][0] = c.x; bv[i][1] = c.y; bv[i][2] = c.z; bv[i][3] = c.w; bv[i][4] = e.x; bv[i][5] = e.y; bv[i][6] = e.z; bv[i][7] = e.w;
+                }
+            }
+        }
+        float mean = 0.0f, scale = 1.0f;
+        if (KIND >= 1) {
+            double s = 0.0;
+#pragma unroll
+            for (int i = 0; i < MYCH; ++i)
+                if (wave + i * kWavesPerBlock < NCH) {
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) s += KIND == 1 ? (double)__fmul_rn(xv[i][k], xv[i][k]) : (double)xv[i][k];
+                }
+            s = pi_wave_sum_f64(s);
+            if (lane == 0) red[0][wave] = s;
+            __syncthreads();
+            double t = 0.0;
+#pragma unroll
+            for (int w = 0; w < kWavesPerBlock; ++w) t += red[0][w];
+            if (KIND == 1) scale = pi_inv_sqrt((float)(t / cols) + eps);
+            else {
+                mean = (float)(t / cols);
+                double s2 = 0.0;
+#pragma unroll
+                for (int i = 0; i < MYCH; ++i)
+                    if (wave + i * kWavesPerBlock < NCH) {
+#pragma unroll
+                        for (int k = 0; k < 8; ++k) { const float v = __fsub_rn(xv[i][k], mean); s2 += (double)__fmul_rn(v, v); }
+                    }
+                s2 = pi_wave_sum_f64(s2);
+                if (lane == 0) red[1][wave] = s2;
+                __syncthreads();
+                double t2 = 0.0;
+#pragma unroll
+                for (int w = 0; w < kWavesPerBlock; ++w) t2 += red[1][w];
+                scale = pi_inv_sqrt((float)(t2 / cols) + eps);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MYCH; ++i) {
+            const int j = wave + i * kWavesPerBlock;
+            if (j < NCH) {
+#pragma unroll
+                for (int k = 0; k < 8; ++k) {
+                    float v = xv[i][k];
+                    if (KIND >= 1) v = __fmul_rn(__fmul_rn(KIND == 2 ? __fsub_rn(v, mean) : v, scale), wv[i][k]);
+                    if (KIND == 2) v = __fadd_rn(v, bv[i][k]);
+                    xv[i][k] = v;
+                }
+                __half2 hh[4] = {__floats2half2_rn(xv[i][0], xv[i][1]), __floats2half2_rn(xv[i][2], xv[i][3]),
+                                 __floats2half2_rn(xv[i][4], xv[i][5]), __floats2half2_rn(xv[i][6], xv[i][7])};
+                *reinterpret_cast<pi_u32x4 *>(xs + j * 512 + lane * 8) = *reinterpret_cast<const pi_u32x4 *>(hh);
+            }
+        }
+        __syncthreads();
+    }
+    pi_u32x4 xr[NCH];
+#pragma unroll
+    for (int j = 0; j < NCH; ++j) xr[j] = *reinterpret_cast<const pi_u32x4 *>(xs + j * 512 + lane * 8);
+
+    auto finish = [&](float acc, float a1, float a2, int r) {
+        acc = pi_wave_sum(acc);
+        if (epi == PI_EPI_RELU) acc = fmaxf(acc, 0.0f);
+        else if (epi == PI_EPI_ADD) acc = __fadd_rn(acc, a1);
+        else if (epi == PI_EPI_ADD2) acc = __fadd_rn(__fadd_rn(acc, a1), a2);
+        if (lane == 0) y[r] = acc;
+    };
+    if constexpr (kWide) {
+        for (int r = wid; r < rows; r += n_waves) {
+            // keep the activations packed: widening them once outside the loop would double their register footprint
+#pragma unroll
+            for (int j = 0; j < NCH; ++j) asm volatile("" : "+v"(xr[j].x), "+v"(xr[j].y), "+v"(xr[j].z), "+v"(xr[j].w));
+            float acc = 0.0f;
+#pragma unroll
+            for (int j = 0; j < CPB; ++j) acc = pi_dot8h(buf[0][j], xr[j], acc);
+            const float a1 = r1[0], a2 = r2[0];
+            issue(0, r + n_waves);
+#pragma unroll
+            for (int j = 0; j < CPB; ++j) acc = pi_dot8h(buf[1][j], xr[CPB + j], acc);
+            issue(1, r + n_waves);
+            finish(acc, a1, a2, r);
+        }
+    } else {
+        for (int r = wid; r < rows; r += 2 * n_waves) {
+#pragma unroll
+            for (int b = 0; b < 2; ++b) {
+                const int rr = r + b * n_waves;
+                if (rr < rows) {
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < NCH; ++j) acc = pi_dot8h(buf[b][j], xr[j], acc);
+                    finish(acc, r1[b], r2[b], rr);
+                }
+                issue(b, rr + 2 * n_waves);
+            }
+        }
+    }
+}
+
+// ---------------------------------------------------------------------------------------------------
+// Register-resident Q4_0 mat-vec for cols == 4096 * CB.  A Q4_0 row of 4096 weights is 128 blocks of 18 bytes =
+// 2304 bytes = 64 lanes x 36 bytes: lane l reads the block pair (2l, 2l+1) of each 4096-column group with two
+// 16-byte loads and one 4-byte load (4-byte aligned) and meets it with the matching 64 int8 activations, their two
+// Q8_0 scales and block sums, all held in registers.  The nibbles are used unsigned through v_dot4_i32_i8 and
+// 8 * sum(x) is subtracted per block, which is exact in int32; the result is scaled by d_w * d_x in fp32 as
+// vec_dot_q4_0_q8_0 does (ggml-quants.c:2512-2650).  The prologue (norm, then Q8_0 quantisation as the x86
+// quantize_row_q8_0 does: d = amax / 127 kept as fp16, q = rint(x * 127 / amax), ggml-quants.c:702-760) is shared by
+// the four waves through LDS.  Four rows (two for CB = 2) of loads are in flight per lane.
+// ---------------------------------------------------------------------------------------------------
+typedef uint32_t pi_u32x4_a4 __attribute__((ext_vector_type(4), aligned(4)));
+
+template <int CB, int KIND, int TAG>
+__global__ __launch_bounds__(kBlock, 2) void gemv_q4_reg_kernel(const unsigned char * __restrict__ W, const float * __restrict__ x,
+                                                             const float * __restrict__ nw, const float * __restrict__ nb, float eps,
+                                                             int epi, const float * __restrict__ add1, const float * __restrict__ add2,
+                                                             float * __restrict__ y, int rows) {
+    constexpr int cols = CB * 4096, NCH = cols / 512, nblk = cols / 32;
+    constexpr int NBUF = 4 / CB;
+    constexpr int MYCH = NCH / kWavesPerBlock;
+    constexpr size_t row_bytes = (size_t)nblk * 18;
+    __shared__ __align__(16) int8_t xq[cols];
+    __shared__ float xd[nblk];
+    __shared__ int   xsum[nblk];
+    __shared__ double red[2][kWavesPerBlock];
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int n_waves = gridDim.x * kWavesPerBlock, wid = blockIdx.x * kWavesPerBlock + wave;
+
+    uint32_t D[NBUF][CB][9];
+    float r1[NBUF], r2[NBUF];
+    auto issue = [&](int b, int r) {
+        if (r < rows) {
+#pragma unroll
+            for (int g = 0; g < CB; ++g) {
+                const unsigned char * p = W + (size_t)r * row_bytes + g * 2304 + lane * 36;
+                const pi_u32x4_a4 v0 = __builtin_nontemporal_load(reinterpret_cast<const pi_u32x4_a4 *>(p));
+                const pi_u32x4_a4 v1 = __builtin_nontemporal_load(reinterpret_cast<const pi_u32x4_a4 *>(p + 16));
+                D[b][g][0] = v0.x; D[b][g][1] = v0.y; D[b][g][2] = v0.z; D[b][g][3] = v0.w;
+                D[b][g][4] = v1.x; D[b][g][5] = v1.y; D[b][g][6] = v1.z; D[b][g][7] = v1.w;
+                D[b][g][8] = __builtin_nontemporal_load(reinterpret_cast<const uint32_t *>(p + 32));
+            }
+            if (epi >= PI_EPI_ADD) r1[b] = add1[r];
+            if (epi == PI_EPI_ADD2) r2[b] = add2[r];
+        }
+    };
+#pragma unroll
+    for (int b = 0; b < NBUF; ++b) { r1[b] = 0.0f; r2[b] = 0.0f; issue(b, wid + b * n_waves); }
+
+    // ---- shared prologue: norm, Q8_0 quantisation -------------------------------------------------------------
+    {
+        float xv[MYCH][8], wv[MYCH][8], bv[MYCH][8];
+#pragma unroll
+        for (int i = 0; i < MYCH; ++i) {
+            const int o = (wave + i * kWavesPerBlock) * 512 + lane * 8;
+            const float4 a = *reinterpret_cast<const float4 *>(x + o), b = *reinterpret_cast<const float4 *>(x + o + 4);
+            xv[i][0] = a.x; xv[i][1] = a.y; xv[i][2] = a.z; xv[i][3] = a.w; xv[i][4] = b.x; xv[i][5] = b.y; xv[i][6] = b.z; xv[i][7] = b.w;
+            if (KIND >= 1) {
+                const float4 c = *reinterpret_cast<const float4 *>(nw + o), e = *reinterpret_cast<const float4 *>(nw + o + 4);
+                wv[i][0] = c.x; wv[i][1] = c.y; wv[i][2] = c.z; wv[i][3] = c.w; wv[i][4] = e.x; wv[i][5] = e.y; wv[i][6] = e.z; wv[i][7] = e.w;
+            }
+            if (KIND == 2) {
+                const float4 c = *reinterpret_cast<const float4 *>(nb + o), e = *reinterpret_cast<const float4 *>(nb + o + 4);
+                bv[i][0] = c.x; bv[i][1] = c.y; bv[i][2] = c.z; bv[i][3] = c.w; bv[i][4] = e.x; bv[i][5] = e.y; bv[i][6] = e.z; bv[i][7] = e.w;
+            }
+        }
+        float mean = 0.0f, scale = 1.0f;
+        if (KIND >= 1) {
+            double s = 0.0;
+#pragma unroll
+            for (int i = 0; i < MYCH; ++i)
+#pragma unroll
+                for (int k = 0; k < 8; ++k) s += KIND == 1 ? (double)__fmul_rn(xv[i][k], xv[i][k]) : (double)xv[i][k];
+            s = pi_wave_sum_f64(s);
+            if (lane == 0) red[0][wave] = s;
+            __syncthreads();
+            double t = 0.0;
+#pragma unroll
+            for (int w = 0; w < kWavesPerBlock; ++w) t += red[0][w];
+            if (KIND == 1) scale = pi_inv_sqrt((float)(t / cols) + eps);
+            else {
+                mean = (float)(t / cols);
+                double s2 = 0.0;
+#pragma unroll
+                for (int i = 0; i < MYCH; ++i)
+#pragma unroll
+                    for (int k = 0; k < 8; ++k) { const float v = __fsub_rn(xv[i][k], mean); s2 += (double)__fmul_rn(v, v); }
+                s2 = pi_wave_sum_f64(s2);
+                if (lane == 0) red[1][wave] = s2;
+                __syncthreads();
+                double t2 = 0.0;
+#pragma unroll
+                for (int w = 0; w < kWavesPerBlock; ++w) t2 += red[1][w];
+                scale = pi_inv_sqrt((float)(t2 / cols) + eps);
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < MYCH; ++i) {
+            const int j = wave + i * kWavesPerBlock;
+            float amax = 0.0f;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                float v = xv[i][k];
+                if (KIND >= 1) v = __fmul_rn(__fmul_rn(KIND == 2 ? __fsub_rn(v, mean) : v, scale), wv[i][k]);
+                if (KIND == 2) v = __fadd_rn(v, bv[i][k]);
+                xv[i][k] = v;
+                amax = fmaxf(amax, fabsf(v));
+            }
+            // a quad of lanes holds one block of 32 values
+            amax = fmaxf(amax, pi_dpp_f32<PI_DPP_XOR1, 0xF>(amax));
+            amax = fmaxf(amax, pi_dpp_f32<PI_DPP_XOR2, 0xF>(amax));
+            const float d = pi_div(amax, 127.0f);
+            const float id = (amax != 0.0f) ? pi_div(127.0f, amax) : 0.0f;
+            int q[8], qs = 0;
+#pragma unroll
+            for (int k = 0; k < 8; ++k) { q[k] = (int)rintf(__fmul_rn(xv[i][k], id)); qs += q[k]; }
+            qs += pi_dpp_i32<PI_DPP_XOR1, 0xF>(qs);
+            qs += pi_dpp_i32<PI_DPP_XOR2, 0xF>(qs);
+            const uint32_t p0 = (uint32_t)(q[0] & 0xff) | ((uint32_t)(q[1] & 0xff) << 8) | ((uint32_t)(q[2] & 0xff) << 16) | ((uint32_t)(q[3] & 0xff) << 24);
+            const uint32_t p1 = (uint32_t)(q[4] & 0xff) | ((uint32_t)(q[5] & 0xff) << 8) | ((uint32_t)(q[6] & 0xff) << 16) | ((uint32_t)(q[7] & 0xff) << 24);
+            *reinterpret_cast<pi_u32x2 *>(xq + j * 512 + lane * 8) = pi_u32x2{p0, p1};
+            if ((lane & 3) == 0) { xd[j * 16 + (lane >> 2)] = pi_round_f16(d); xsum[j * 16 + (lane >> 2)] = qs; }
+        }
+        __syncthreads();
+    }
+    int   X[CB][16];
+    float dx[CB][2];
+    int   sx[CB][2];
+#pragma unroll
+    for (int g = 0; g < CB; ++g) {
+        const int b0 = g * 128 + 2 * lane;
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const pi_u32x4 v = *reinterpret_cast<const pi_u32x4 *>(xq + b0 * 32 + k * 16);
+            X[g][4 * k] = (int)v.x; X[g][4 * k + 1] = (int)v.y; X[g][4 * k + 2] = (int)v.z; X[g][4 * k + 3] = (int)v.w;
+        }
+        dx[g][0] = xd[b0]; dx[g][1] = xd[b0 + 1];
+        sx[g][0] = xsum[b0]; sx[g][1] = xsum[b0 + 1];
+    }
+
+    for (int r = wid; r < rows; r += NBUF * n_waves) {
+#pragma unroll
+        for (int b = 0; b < NBUF; ++b) {
+            const int rr = r + b * n_waves;
+            if (rr < rows) {
+                float acc = 0.0f;
+#pragma unroll
+                for (int g = 0; g < CB; ++g) {
+                    const uint32_t * d9 = D[b][g];
+                    int s0 = 0, s1 = 0;
+#pragma unroll
+                    for (int k = 0; k < 4; ++k) {
+                        const uint32_t q0 = __builtin_amdgcn_alignbit(d9[k + 1], d9[k], 16);       // bytes 2 + 4k .. 5 + 4k of the pair
+                        s0 = __builtin_amdgcn_sdot4((int)(q0 & 0x0F0F0F0Fu), X[g][k], s0, false);
+                        s0 = __builtin_amdgcn_sdot4((int)((q0 >> 4) & 0x0F0F0F0Fu), X[g][4 + k], s0, false);
+                        const uint32_t q1 = d9[5 + k];
+                        s1 = __builtin_amdgcn_sdot4((int)(q1 & 0x0F0F0F0Fu), X[g][8 + k], s1, false);
+                        s1 = __builtin_amdgcn_sdot4((int)((q1 >> 4) & 0x0F0F0F0Fu), X[g][12 + k], s1, false);
+                    }
+                    s0 -= 8 * sx[g][0];
+                    s1 -= 8 * sx[g][1];
+                    acc = fmaf(__fmul_rn(pi_f16_from_bits((uint16_t)(d9[0] & 0xffffu)), dx[g][0]), (float)s0, acc);
+                    acc = fmaf(__fmul_rn(pi_f16_from_bits((uint16_t)(d9[4] >> 16)), dx[g][1]), (float)s1, acc);
+                }
+                acc = pi_wave_sum(acc);
+                if (epi == PI_EPI_RELU) acc = fmaxf(acc, 0.0f);
+                else if (epi == PI_EPI_ADD) acc = __fadd_rn(acc, r1[b]);
+                else if (epi == PI_EPI_ADD2) acc = __fadd_rn(__fadd_rn(acc, r1[b]), r2[b]);
+                if (lane == 0) y[rr] = acc;
+            }
+            issue(b, rr + NBUF * n_waves);
+        }
+    }
+}
+
+// any shape with cols % 8 == 0: one wave per row, grid-stride
+__global__ __launch_bounds__(kBlock) void gemv_f16_generic_kernel(const __half * __restrict__ W, const float * __restrict__ x, NormArgs na,
+                                                                  int epi, const float * add1, const float * add2,
+                                                                  float * __restrict__ y, int rows, int cols) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    __half * xs = reinterpret_cast<__half *>(smem);
+    __shared__ double red[16];
+    stage_x_f16(xs, x, cols, na, red);
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    for (int r = blockIdx.x * kWavesPerBlock + wave; r < rows; r += gridDim.x * kWavesPerBlock) {
+        float acc = 0.0f;
+#pragma unroll 4
+        for (int c = lane * 8; c < cols; c += PI_WAVE * 8) {
+            float xf[8];
+            pi_unpack8(pi_ld16(xs + c), xf);
+            acc = pi_dot8(pi_ld_stream(W + (size_t)r * cols + c), xf, acc);
+        }
+        acc = pi_wave_sum(acc);
+        if (lane == 0) y[r] = apply_epilogue(acc, epi, add1, add2, r);
+    }
+}
+
+
+// Dense Q4_0 mat-vec: one wave per RPW rows, lane l owns blocks l, l+64, ...
+template <int RPW>
+__global__ __launch_bounds__(kBlock) void gemv_q4_kernel(const pi_block_q4_0 * __restrict__ W, const float * __restrict__ x, NormArgs na,
+                                                         int epi, const float * add1, const float * add2,
+                                                         float * __restrict__ y, int rows, int cols) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    int8_t * xq   = reinterpret_cast<int8_t *>(smem);
+    float  * xd   = reinterpret_cast<float *>(smem + cols);
+    float  * xtmp = reinterpret_cast<float *>(smem + cols + (cols / 32) * 4);
+    __shared__ double red[16];
+    stage_x_q8(xq, xd, x, cols, na, red, xtmp);
+
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int nb = cols / 32;
+    const int n_groups = (rows + RPW - 1) / RPW;
+    for (int g = blockIdx.x * kWavesPerBlock + wave; g < n_groups; g += gridDim.x * kWavesPerBlock) {
+        const int r0 = g * RPW;
+        float acc[RPW];
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) acc[i] = 0.0f;
+        for (int b = lane; b < nb; b += PI_WAVE) {
+            const float dx = xd[b];
+#pragma unroll
+            for (int i = 0; i < RPW; ++i)
+                if (r0 + i < rows) acc[i] = q4_block_dot(W + (size_t)(r0 + i) * nb + b, xq + b * 32, dx, acc[i]);
+        }
+#pragma unroll
+        for (int i = 0; i < RPW; ++i) {
+            const float s = pi_wave_sum(acc[i]);
+            if (lane == 0 && r0 + i < rows) y[r0 + i] = apply_epilogue(s, epi, add1, add2, r0 + i);
+        }
+    }
+}
+
+__global__ void embed_f16_kernel(const __half * __restrict__ table, int cols, const int32_t * __restrict__ token, float * __restrict__ x) {
+    const __half * row = table + (size_t)(*token) * cols;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < cols; i += gridDim.x * blockDim.x) x[i] = __half2float(row[i]);
+}
+// blockIdx.y = token of a chunk (0 for a single token)
+__global__ void embed_q4_kernel(const pi_block_q4_0 * __restrict__ table, int cols, const int32_t * __restrict__ token, float * __restrict__ x) {
+    const pi_block_q4_0 * row = table + (size_t)token[blockIdx.y] * (cols / 32);
+    x += (size_t)blockIdx.y * cols;
+    for (int i = blockIdx.x * blockDim.x + threadIdx.x; i < cols; i += gridDim.x * blockDim.x) {
+        const pi_block_q4_0 * b = row + (i >> 5);
+        uint16_t dbits; __builtin_memcpy(&dbits, &b->d, 2);
+        const int j = i & 31;
+        const int q = (j < 16) ? (b->qs[j] & 0x0F) : (b->qs[j - 16] >> 4);
+        x[i] = __fmul_rn((float)(q - 8), pi_f16_from_bits(dbits));
+    }
+}
+
+// first maximum wins (std::max_element, llama.cpp:8617-8631)
+__global__ __launch_bounds__(1024) void argmax_kernel(const float * __restrict__ logits, int n, int32_t * __restrict__ token_out) {
+    __shared__ float bv[16];
+    __shared__ int   bi[16];
+    float best = -INFINITY; int idx = 0x7fffffff;
+    for (int i = threadIdx.x; i < n; i += blockDim.x) { const float v = logits[i]; if (v > best) { best = v; idx = i; } }
+    if (idx == 0x7fffffff) { idx = n; }                          // thread saw nothing above -inf
+#pragma unroll
+    for (int o = PI_WAVE / 2; o > 0; o >>= 1) {
+        const float ov = __shfl_xor(best, o, PI_WAVE); const int oi = __shfl_xor(idx, o, PI_WAVE);
+        if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }
+    }
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    if (lane == 0) { bv[wave] = best; bi[wave] = idx; }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+        for (int w = 1; w < (int)(blockDim.x >> 6); ++w)
+            if (bv[w] > best || (bv[w] == best && bi[w] < idx)) { best = bv[w]; idx = bi[w]; }
+        *token_out = idx < n ? idx : 0;
+    }
+}
+
+// counter-based N(0, std^2): two 32-bit hashes -> Box-Muller; deterministic in (seed, index)
+__device__ __forceinline__ uint64_t mix64(uint64_t z) {
+    z += 0x9E3779B97F4A7C15ull;
+    z = (z ^ (z >> 30)) * 0xBF58476D1CE4E5B9ull;
+    z = (z ^ (z >> 27)) * 0x94D049BB133111EBull;
+    return z ^ (z >> 31);
+}
+__global__ void fill_normal_f16_kernel(__half * __restrict__ p, size_t n, uint64_t seed, float std, const float * __restrict__ row_bias, int cols) {
+    for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n; i += (size_t)gridDim.x * blockDim.x) {
+        const uint64_t r = mix64(seed * 0xD1342543DE82EF95ull + i);
+        const float u1 = ((uint32_t)(r >> 32) + 1.0f) * (1.0f / 4294967296.0f);
+        const float u2 = (uint32_t)r * (1.0f / 4294967296.0f);
+        float v = sqrtf(-2.0f * logf(u1)) * cosf(6.28318530718f * u2) * std;
+        if (row_bias) v += row_bias[i / cols];
+        p[i] = __float2half_rn(v);
+    }
+}
+
+// N(0, std^2) values quantised to Q4_0 exactly as quantize_row_q4_0_reference does (ggml-quants.c:428-463): the
+// element of largest magnitude (first one wins) sets d = max / -8, q = min(15, (int)(x / d + 8.5)).  One thread per block.
+__global__ void fill_normal_q4_0_kernel(pi_block_q4_0 * __restrict__ p, size_t n_blocks, uint64_t seed, float std) {
+    for (size_t b = (size_t)blockIdx.x * blockDim.x + threadIdx.x; b < n_blocks; b += (size_t)gridDim.x * blockDim.x) {
+        float v[32];
+        float amax = 0.0f, mx = 0.0f;
+#pragma unroll
+        for (int j = 0; j < 32; ++j) {
+            const uint64_t r = mix64(seed * 0xD1342543DE82EF95ull + b * 32 + j);
+            const float u1 = ((uint32_t)(r >> 32) + 1.0f) * (1.0f / 4294967296.0f);
+            const float u2 = (uint32_t)r * (1.0f / 4294967296.0f);
+            v[j] = pi_round_f16(sqrtf(-2.0f * logf(u1)) * cosf(6.28318530718f * u2) * std);
+            if (fabsf(v[j]) > amax) { amax = fabsf(v[j]); mx = v[j]; }
+        }
+        const float d = mx / -8.0f;
+        const float id = d != 0.0f ? pi_div(1.0f, d) : 0.0f;
+        pi_block_q4_0 blk;
+        blk.d = pi_f16_bits(d);
+#pragma unroll
+        for (int j = 0; j < 16; ++j) {
+            const int q0 = min(15, (int)(v[j] * id + 8.5f)), q1 = min(15, (int)(v[j + 16] * id + 8.5f));
+            blk.qs[j] = (uint8_t)(q0 | (q1 << 4));
+        }
+        p[b] = blk;
+    }
+}
+
+}  // namespace
+
+extern "C" {
+
+pi_workspace * pi_workspace_create(int max_ff, int max_d) {
+    if (max_ff <= 0 || max_d <= 0 || (max_d + kAxpyTile - 1) / kAxpyTile > 62) { pi::set_error("pi_workspace_create: bad sizes"); return nullptr; }
+    pi_workspace * ws = new pi_workspace{};
+    ws->max_ff = max_ff; ws->max_d = max_d;
+    const size_t n_words = (size_t)(max_ff / 32 + 2) > 2048 ? (size_t)(max_ff / 32 + 2) : 2048;       // groups of 32 neurons, or two words per compute unit
+    ws->words    = (uint32_t *)pi_malloc(sizeof(uint32_t) * n_words);
+    ws->words_hot = (uint32_t *)pi_malloc(sizeof(uint32_t) * (max_ff / 32 + 2));
+    ws->counters = (unsigned int *)pi_malloc(sizeof(unsigned int) * 64);
+    ws->partial  = (float *)pi_malloc(sizeof(float) * (size_t)kAxpyGroups * max_d);
+    ws->hq       = (int32_t *)pi_malloc(sizeof(int32_t) * max_ff);
+    ws->hd       = (float *)pi_malloc(sizeof(float) * max_ff);
+    const size_t n_part = (size_t)((max_ff + 31) / 32) > (size_t)kBmGroups * kBtMaxT ? (size_t)((max_ff + 31) / 32) : (size_t)kBmGroups * kBtMaxT;
+    ws->ffn_partial = (float *)pi_malloc(sizeof(float) * n_part * max_d);
+    ws->hc_batch = (__half *)pi_malloc(sizeof(__half) * ((size_t)max_ff + 16) * kBtMaxT);
+    ws->row_any = (unsigned char *)pi_malloc((size_t)max_ff + 16);
+    if (!ws->words || !ws->words_hot || !ws->counters || !ws->partial || !ws->hq || !ws->hd || !ws->ffn_partial || !ws->hc_batch || !ws->row_any) {
+        pi_workspace_destroy(ws); return nullptr;
+    }
+    pi_memset(ws->counters, 0, sizeof(unsigned int) * 64);
+    return ws;
+}
+int pi_workspace_destroy(pi_workspace * ws) {
+    if (!ws) return PI_OK;
+    pi_free(ws->words); pi_free(ws->words_hot); pi_free(ws->counters); pi_free(ws->partial); pi_free(ws->hq); pi_free(ws->hd); pi_free(ws->ffn_partial); pi_free(ws->hc_batch); pi_free(ws->row_any);
+    delete ws;
+    return PI_OK;
+}
+
+int pi_k_gemv(int wtype, const void * W, int rows, int cols, const float * x, const pi_norm * norm,
+              int epilogue, const float * add1, const float * add2, float * y, pi_stream_t stream) {
+    if (!W || !x || !y || rows <= 0 || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_gemv: null pointer or empty shape");
+    if (epilogue < 0 || epilogue > PI_EPI_ADD2 || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
+        return pi::fail(PI_E_ARG, "pi_k_gemv: bad epilogue arguments");
+    hipStream_t st = (hipStream_t)stream;
+    const NormArgs na = to_norm(norm);
+    // rows per wave group / chunks per step: 8 x 16 B loads in flight per lane per step, and at least one
+    // group for each of the grid's waves
+    const int n_waves = kGemvBlocks * kWavesPerBlock;
+    const int rpw = rows >= 4 * n_waves ? 4 : rows >= 2 * n_waves ? 2 : 1;
+    const int n_groups = (rows + rpw - 1) / rpw;
+    int blocks = (n_groups + kWavesPerBlock - 1) / kWavesPerBlock;
+    if (blocks > kGemvBlocks) blocks = kGemvBlocks;
+    if (wtype == PI_TYPE_F16) {
+        if (cols % 8) return pi::fail(PI_E_ARG, "pi_k_gemv: F16 needs cols % 8 == 0");
+        const __half * w = (const __half *)W;
+        const int u = 8 / rpw;
+        const bool fast = cols % (PI_WAVE * 8 * u) == 0 && rows % rpw == 0 && stage_fast_lds_bytes(cols) <= 64 * 1024 &&
+                          (((uintptr_t)x | (uintptr_t)(norm ? norm->w : nullptr)) & 15) == 0;
+        const bool aligned = (((uintptr_t)x | (uintptr_t)(norm ? norm->w : nullptr) | (uintptr_t)(norm ? norm->b : nullptr)) & 15) == 0;
+        const int rblocks = rows >= n_waves ? kGemvBlocks : (rows + kWavesPerBlock - 1) / kWavesPerBlock;
+        // register-resident kernel: the norm must carry what its kind needs (RMSNorm a weight, LayerNorm weight and bias)
+        const bool reg_ok = aligned && (cols == 4096 || cols == 5120 || cols == 8192) &&
+                            (na.kind == 0 || (na.kind == 1 && na.w && !na.b) || (na.kind == 2 && na.w && na.b));
+        if (reg_ok) {
+            // the tag only names the role in kernel traces: 1 = lm-head sized, 2 = fewer rows than the grid has waves
+            const int tag = rows >= 16384 ? 1 : rows < n_waves ? 2 : 0;
+#define PI_GEMV_REG(NCH, KIND, TAG) hipLaunchKernelGGL((gemv_f16_reg_kernel<NCH, KIND, TAG>), dim3(rblocks), dim3(kBlock), 0, st, w, x, na.w, na.b, na.eps, epilogue, add1, add2, y, rows)
+#define PI_GEMV_REG_K(NCH, KIND) do { if (tag == 1) PI_GEMV_REG(NCH, KIND, 1); else if (tag == 2) PI_GEMV_REG(NCH, KIND, 2); else PI_GEMV_REG(NCH, KIND, 0); } while (0)
+#define PI_GEMV_REG_N(NCH) do { if (na.kind == 0) PI_GEMV_REG_K(NCH, 0); else if (na.kind == 1) PI_GEMV_REG_K(NCH, 1); else PI_GEMV_REG_K(NCH, 2); } while (0)
+            if (cols == 4096) PI_GEMV_REG_N(8); else if (cols == 5120) PI_GEMV_REG_N(10); else PI_GEMV_REG_N(16);
+#undef PI_GEMV_REG_N
+#undef PI_GEMV_REG_K
+#undef PI_GEMV_REG
+        } else if (fast) {
+            const size_t sh = stage_fast_lds_bytes(cols);
+            if (rows >= 16384) hipLaunchKernelGGL((gemv_f16_kernel<4, 2, 1>), dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+            else if (rpw == 4) hipLaunchKernelGGL((gemv_f16_kernel<4, 2, 0>), dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+            else if (rpw == 2) hipLaunchKernelGGL((gemv_f16_kernel<2, 4, 0>), dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+            else               hipLaunchKernelGGL((gemv_f16_kernel<1, 8, 0>), dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        } else {
+            const size_t sh = (size_t)cols * 2;
+            if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv: cols too large for LDS staging");
+            int gb = (rows + kWavesPerBlock - 1) / kWavesPerBlock;
+            if (gb > 2048) gb = 2048;
+            hipLaunchKernelGGL(gemv_f16_generic_kernel, dim3(gb), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        }
+    } else if (wtype == PI_TYPE_Q4_0) {
+        if (cols % 32) return pi::fail(PI_E_ARG, "pi_k_gemv: Q4_0 needs cols % 32 == 0");
+        const size_t sh = (size_t)cols + (size_t)(cols / 32) * 4 + (size_t)cols * 4;
+        if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv: cols too large for LDS staging");
+        const pi_block_q4_0 * w = (const pi_block_q4_0 *)W;
+        const bool aligned = (((uintptr_t)x | (uintptr_t)(norm ? norm->w : nullptr) | (uintptr_t)(norm ? norm->b : nullptr)) & 15) == 0 && ((uintptr_t)W & 3) == 0;
+        const bool reg_ok = aligned && (cols == 4096 || cols == 8192) &&
+                            (na.kind == 0 || (na.kind == 1 && na.w && !na.b) || (na.kind == 2 && na.w && na.b));
+        if (reg_ok) {
+            const int rblocks = rows >= n_waves ? kGemvBlocks : (rows + kWavesPerBlock - 1) / kWavesPerBlock;
+            const int tag = rows >= 16384 ? 1 : 0;
+            const unsigned char * wb = (const unsigned char *)W;
+#define PI_GEMV_Q4(CB, KIND, TAG) hipLaunchKernelGGL((gemv_q4_reg_kernel<CB, KIND, TAG>), dim3(rblocks), dim3(kBlock), 0, st, wb, x, na.w, na.b, na.eps, epilogue, add1, add2, y, rows)
+#define PI_GEMV_Q4_K(CB, KIND) do { if (tag == 1) PI_GEMV_Q4(CB, KIND, 1); else PI_GEMV_Q4(CB, KIND, 0); } while (0)
+#define PI_GEMV_Q4_N(CB) do { if (na.kind == 0) PI_GEMV_Q4_K(CB, 0); else if (na.kind == 1) PI_GEMV_Q4_K(CB, 1); else PI_GEMV_Q4_K(CB, 2); } while (0)
+            if (cols == 4096) PI_GEMV_Q4_N(1); else PI_GEMV_Q4_N(2);
+#undef PI_GEMV_Q4_N
+#undef PI_GEMV_Q4_K
+#undef PI_GEMV_Q4
+            return pi::check_launch("pi_k_gemv");
+        }
+        if (rpw == 8)      hipLaunchKernelGGL(gemv_q4_kernel<8>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        else if (rpw == 4) hipLaunchKernelGGL(gemv_q4_kernel<4>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        else if (rpw == 2) hipLaunchKernelGGL(gemv_q4_kernel<2>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+        else               hipLaunchKernelGGL(gemv_q4_kernel<1>, dim3(blocks), dim3(kBlock), sh, st, w, x, na, epilogue, add1, add2, y, rows, cols);
+    } else {
+        return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv: weight type must be F16 or Q4_0");
+    }
+    return pi::check_launch("pi_k_gemv");
+}
+
+int pi_k_embed_batch_q4(const void * table_q4, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream) {
+    if (!table_q4 || !tokens || !x || cols <= 0 || cols % 32 || T <= 0 || T > kChunkMaxT) return pi::fail(PI_E_ARG, "pi_k_embed_batch_q4: bad arguments");
+    hipLaunchKernelGGL(embed_q4_kernel, dim3((cols + 255) / 256, T), dim3(256), 0, (hipStream_t)stream, (const pi_block_q4_0 *)table_q4, cols, tokens, x);
+    return pi::check_launch("pi_k_embed_batch_q4");
+}
+
+int pi_k_embed(int wtype, const void * table, int cols, const int32_t * token, float * x, pi_stream_t stream) {
+    if (!table || !token || !x || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_embed: bad arguments");
+    const int blocks = (cols + 255) / 256;
+    if (wtype == PI_TYPE_F16)       hipLaunchKernelGGL(embed_f16_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const __half *)table, cols, token, x);
+    else if (wtype == PI_TYPE_Q4_0) hipLaunchKernelGGL(embed_q4_kernel, dim3(blocks), dim3(256), 0, (hipStream_t)stream, (const pi_block_q4_0 *)table, cols, token, x);
+    else return pi::fail(PI_E_UNSUPPORTED, "pi_k_embed: table type must be F16 or Q4_0");
+    return pi::check_launch("pi_k_embed");
+}
+
+int pi_k_argmax(const float * logits, int n, int32_t * token_out, pi_stream_t stream) {
+    if (!logits || !token_out || n <= 0) return pi::fail(PI_E_ARG, "pi_k_argmax: bad arguments");
+    hipLaunchKernelGGL(argmax_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, logits, n, token_out);
+    return pi::check_launch("pi_k_argmax");
+}
+
+int pi_fill_normal_f16(void * dptr, size_t n, uint64_t seed, float std, const float * row_bias, int cols, pi_stream_t stream) {
+    if (!dptr || (row_bias && cols <= 0)) return pi::fail(PI_E_ARG, "pi_fill_normal_f16: bad arguments");
+    if (n == 0) return PI_OK;
+    size_t blocks = (n + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(fill_normal_f16_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (__half *)dptr, n, seed, std, row_bias, cols);
+    return pi::check_launch("pi_fill_normal_f16");
+}
+
+int pi_fill_normal_q4_0(void * dptr, size_t n_weights, uint64_t seed, float std, pi_stream_t stream) {
+    if (!dptr || n_weights % 32) return pi::fail(PI_E_ARG, "pi_fill_normal_q4_0: null pointer or a weight count that is not a multiple of 32");
+    if (n_weights == 0) return PI_OK;
+    size_t blocks = (n_weights / 32 + 255) / 256;
+    if (blocks > 65536) blocks = 65536;
+    hipLaunchKernelGGL(fill_normal_q4_0_kernel, dim3((unsigned)blocks), dim3(256), 0, (hipStream_t)stream, (pi_block_q4_0 *)dptr, n_weights / 32, seed, std);
+    return pi::check_launch("pi_fill_normal_q4_0");
+}
+
+}  // extern "C"

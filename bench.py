@@ -292,6 +292,7 @@ def main():
                     help="BASELINE configs index: 1 (default, the reported metric) 7B FP16 all on the GPU; 2 the same shape in "
                          "Q4_0 with the hottest 60 %% of neurons on the GPU and the rest on host threads; 3 ProSparse-LLaMA-2-13B shape FP16, "
                          "16 sequences decoded in lockstep; 4 Falcon-40B shape FP16")
+    ap.add_argument("--n-seq", type=int, default=16, choices=[1, 16], help="config 3: 16 sequences in lockstep (configs[3]) or the same model at batch 1")
     ap.add_argument("--rest-on-gpu", action="store_true", help="config 2: the GPU reads the non-resident neurons' rows from pinned host memory itself instead of handing those neurons to host threads")
     ap.add_argument("--hot-frac", type=float, default=None, help="configs 1 and 2: share of each layer's neurons on the GPU (default 1.0 and 0.6)")
     ap.add_argument("--pmc-probe", action="store_true",
@@ -330,10 +331,10 @@ def main():
         hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_ctx, seed=1, wtype=pl.Q4_0, hot_frac=0.6 if args.hot_frac is None else args.hot_frac,
                            rest_on_gpu=bool(args.rest_on_gpu))
     elif args.config == 3:
-        hp = None
+        hp = None if args.n_seq != 1 else synth.hparams("llama-13b", n_layer=40 if args.layers == 32 else args.layers, n_ctx=n_ctx, seed=1)
     else:
         hp = synth.hparams("falcon-40b", n_layer=60 if args.layers == 32 else args.layers, n_ctx=n_ctx, seed=1)
-    if args.config == 3:
+    if args.config == 3 and args.n_seq != 1:
         return bench_batched(args)
     hybrid = hp.hot_frac < 1.0
     keep = []
@@ -401,6 +402,7 @@ def main():
         "bound": "hbm",
         "kernel": {1: "gemv_f16_reg_kernel<8,1,0> (q|k|v projection, 12288 x 4096 fp16, fused RMSNorm)",
                    2: "gemv_q4_kernel (q|k|v projection, 12288 x 4096 Q4_0, fused RMSNorm; not timed for a hybrid model)",
+                   3: "gemv_f16_reg_kernel<10,1,0> (q|k|v projection, 15360 x 5120 fp16, fused RMSNorm)",
                    4: "gemv_f16_reg_kernel<16,2,0> (q|k|v projection, 9216 x 8192 fp16, fused LayerNorm)"}[args.config],
         "achieved": rnd(achieved, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s", "frac": rnd(achieved / HBM_PEAK_GBPS, 4),
         "traffic": traffic, "traffic_source": qkv_src,
@@ -409,9 +411,10 @@ def main():
     }
     roof_ffn = {
         "bound": "hbm",
-        "kernel": {1: ("ffn_cu_f16_kernel<2,true,6,1>" if n_cu_form else "pred_ffn_f16_kernel<1,2,true,1,false>") +
+        "kernel": {1: ("ffn_cu_f16_kernel<8,1024,true,6,1>" if n_cu_form else "pred_ffn_f16_kernel<1,2,true,1,false>") +
                       " (predictor fc2 11008 x 1024 + mask + gate/up/down rows of the active neurons, 7B layer)",
                    2: "pred_upgate_q4_kernel (not timed for a hybrid model)",
+                   3: "ffn_cu_f16_kernel<10,1280,true,6,1> (predictor fc2 13824 x 1280 + mask + gate/up/down rows of the active neurons, 13B layer)",
                    4: "pred_ffn_f16_kernel<2,2,false,4,false> (predictor fc2 32768 x 1024 + mask + up/down rows of the active neurons, Falcon-40B layer)"}[args.config],
         "achieved": rnd(pf_bytes / (ms_pf * 1e-3) / 1e9, 1), "peak": HBM_PEAK_GBPS, "unit": "GB/s",
         "frac": rnd(pf_bytes / (ms_pf * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4),
@@ -425,7 +428,7 @@ def main():
 
     out = {
         "metric": {1: "decode tok/s bs=1 ReLU-Llama2-7B FP16", 2: "decode tok/s bs=1 ReLU-Llama2-7B Q4_0 (60 % of neurons on the GPU)",
-                   4: "decode tok/s bs=1 ReLU-Falcon-40B FP16"}[args.config],
+                   3: "decode tok/s bs=1 ProSparse-Llama2-13B shape FP16", 4: "decode tok/s bs=1 ReLU-Falcon-40B FP16"}[args.config],
         "value": round(1e3 / ms_per_step, 2),
         "unit": "tok/s",
         "n_gpus": 1,
@@ -445,6 +448,8 @@ def main():
                 2: "configs[2]: ReLU-LLaMA-2-7B shape, random-init weights quantised to Q4_0 (predictors FP16), per layer the hottest "
                    f"60 % of neurons on the GPU and the rest " + ("in pinned host memory, their active rows read by the GPU itself" if hp.get("rest_on_gpu") else "on host threads")
                    + f", {hp.n_layer} layers, {args.prompt}-token random prompt, greedy decode at batch 1",
+                3: "configs[3]'s model at batch 1: ProSparse-LLaMA-2-13B shape (d 5120, ff 13824, 40 heads, vocab 32000, predictor rank 1280), "
+                   f"{hp.n_layer} layers, random-init FP16 weights, all neurons on the GPU, {args.prompt}-token random prompt, greedy decode at batch 1",
                 4: "configs[4]: ReLU-Falcon-40B shape (d 8192, ff 32768 up/down only, 128 heads / 8 KV heads, vocab 65024, predictor "
                    f"rank 1024), {hp.n_layer} layers, random-init FP16 weights, all neurons on the GPU, {args.prompt}-token random "
                    "prompt, greedy decode at batch 1"}[args.config],

@@ -206,7 +206,11 @@ PI_API int pi_k_axpy_q4_partials_split(const void * down_t_q4, const void * down
  * freq_scale: linear RoPE scaling as in pi_k_rope_kv_store. */
 PI_API int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float theta_scale, float freq_scale, const int32_t * delta, int n_cells, pi_stream_t stream);
 PI_API int pi_k_kv_compact(void * cache, void * stage, int rows, int n_ctx, int hd, const int32_t * map, int n_new, pi_stream_t stream);
+/* Shapes of the fused block: cols 4096 or 8192 with a predictor of rank 512 or 1024 and ff % 32 == 0; cols 5120 with rank 1280 (the
+ * 13B shape) where ff gives every compute unit 33..60 neurons, with a norm that carries its weights (or none).  Needs pi_init
+ * (the answer depends on the device's compute units).  _hot_supported: the shapes of the hybrid forms below (the first group only). */
 PI_API int pi_k_sparse_ffn_supported(int ff, int r, int cols);
+PI_API int pi_k_sparse_ffn_hot_supported(int ff, int r, int cols);
 /* Workgroups of the fused launch for a layer that is whole on the device (0: shape not covered).  Workgroup b computes neurons
  * [ff * b / n, ff * (b + 1) / n) and stores one partial output vector; a caller that arranges a layer's rows by firing rate deals
  * them out over these ranges (pi_model_finalize does, from PI_T_NEURON_RATE). */
@@ -395,7 +399,7 @@ PI_API int    pi_k_attn_split(const float * qkv, int qkv_stride, const void * ro
 /* pi_k_attn_chunk (below) for contexts beyond its kernels (pi_k_attn_chunk_supported tells): RoPE + KV store of the chunk's T tokens, then
  * each token's cells split as above (scratch: pi_k_attn_split_scratch_floats(T, ...)).  No K / V tile is shared between the tokens of the
  * chunk, so a long prompt costs T passes over the cache per chunk: it is the path that works at any context, not a fast one. */
-PI_API int    pi_k_attn_chunk_supported(int hd, int n_ctx);
+PI_API int    pi_k_attn_chunk_supported(int hd, int n_ctx, int n_kv_max);
 PI_API int    pi_k_attn_chunk_long(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,
                                    const int32_t * pos, int n_ctx, int n_parts, float * scratch, float * q_rot, void * k_cache, void * v_cache,
                                    float * out, void * out_f16, pi_stream_t stream);
@@ -412,11 +416,12 @@ PI_API int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void *
                                  const int32_t * pos, float * out, int out_stride, void * out_f16, pi_stream_t stream);
 /* prompt chunk of ONE sequence: T <= 512 consecutive tokens at positions pos[t]; RoPE + KV store of the whole chunk first, then
  * every token attends to the cells up to its own position (the causal mask of llama.cpp:6506-6531).  q_rot: fp32 [T][n_head*hd].
- * Head sizes 128 and 64 with 16 * n_ctx floats of scores within 156 KB of LDS (n_ctx up to about 1900) take 16 tokens per
- * workgroup on the matrix cores; other shapes one token per workgroup.  Same rounding points either way (llm_build_kqv on the
- * CPU path: fp16 q and K, fp16 in and out of exp, fp16 probabilities). */
+ * n_kv_max: an upper bound of max(pos) + 1, the cells the chunk's furthest token attends (<= 0: n_ctx); positions beyond it are
+ * clamped.  Head sizes 128 and 64 with 16 * n_kv_max floats of scores within 156 KB of LDS (about 1850 cells, whatever the cache's
+ * n_ctx) take 16 tokens per workgroup on the matrix cores; other shapes one token per workgroup (n_ctx up to about 11 k).  Same
+ * rounding points either way (llm_build_kqv on the CPU path: fp16 q and K, fp16 in and out of exp, fp16 probabilities). */
 PI_API int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,
-                           const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache,
+                           const int32_t * pos, int n_ctx, int n_kv_max, float * q_rot, void * k_cache, void * v_cache,
                            float * out, int out_stride, void * out_f16, pi_stream_t stream);
 PI_API int pi_k_embed_batch(const void * table_f16, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream);
 PI_API int pi_k_argmax_batch(const float * logits, int n, int T, int32_t * tokens, int32_t * positions, int32_t * step,

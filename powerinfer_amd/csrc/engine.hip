@@ -226,7 +226,7 @@ int layer_forward(pi_model * m, int il, bool last_token) {
         std::swap(m->x, m->x2);
         return PI_OK;
     }
-    if (layer_hybrid && !q4 && m->hot_words[il] && up.type == PI_TYPE_F16 && fc2.type == PI_TYPE_F16 && pi_k_sparse_ffn_supported(ff, r, d)) {
+    if (layer_hybrid && !q4 && m->hot_words[il] && up.type == PI_TYPE_F16 && fc2.type == PI_TYPE_F16 && pi_k_sparse_ffn_hot_supported(ff, r, d)) {
         // F16 hybrid layer at a width the fused kernels cover: the resident share's whole FFN is one launch, the host share works
         // from the pinned buffers it fills, the reduction merges both
         const bool cap = m->capture && last_token;

@@ -11,6 +11,7 @@
 
 struct BatchState {
     int n_seq = 0, max_steps = 4096;
+    int kv_hi = 0;                        // prompt chunks: cells the chunk's last token attends (its position + 1)
     bool prefill = false;                 // prompt chunks of the model's own sequence: tokens share the model's KV cache
     float * q_rot = nullptr;
     size_t cache_seq_stride = 0;          // elements per sequence: n_layer * n_head_kv * n_ctx * hd
@@ -48,8 +49,8 @@ pi_norm mk_norm(int kind, float eps, const Tensor & w, const Tensor * b) {
 int chunk_attention(pi_model * m, BatchState * b, int T, size_t kv_off) {
     const pi_hparams & hp = m->hp;
     const int d = hp.n_embd, hd = m->hd, gqa = m->gqa, mode = hp.arch == PI_ARCH_FALCON ? 2 : 0;
-    if (pi_k_attn_chunk_supported(hd, hp.n_ctx))
-        return pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, mode, m->theta_scale, m->freq_scale, b->d_pos, hp.n_ctx, b->q_rot,
+    if (pi_k_attn_chunk_supported(hd, hp.n_ctx, b->kv_hi))
+        return pi_k_attn_chunk(b->qkv, d + 2 * gqa, T, hp.n_head, hp.n_head_kv, hd, mode, m->theta_scale, m->freq_scale, b->d_pos, hp.n_ctx, b->kv_hi, b->q_rot,
                                m->k_cache + kv_off, m->v_cache + kv_off, b->att, d, b->att16, m->stream);
     const int parts = m->attn_parts > 1 ? m->attn_parts : 2;
     if (!m->attn_scratch_chunk) {
@@ -402,6 +403,7 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
     }
     BatchState * b = m->prefill_wide;
     b->n_seq = T;
+    b->kv_hi = n_past + T;
     int32_t pos[512];
     for (int t = 0; t < T; ++t) pos[t] = n_past + t;
     PI_HIP_TRY(hipMemcpyAsync(b->d_tokens, tokens, sizeof(int32_t) * T, hipMemcpyHostToDevice, m->stream));
@@ -436,6 +438,7 @@ int prefill_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) {
     }
     BatchState * b = m->prefill;
     b->n_seq = T;
+    b->kv_hi = n_past + T;
     int32_t pos[16];
     for (int t = 0; t < T; ++t) pos[t] = n_past + t;
     PI_HIP_TRY(hipMemcpyAsync(b->d_tokens, tokens, sizeof(int32_t) * T, hipMemcpyHostToDevice, m->stream));

@@ -520,6 +520,7 @@ __global__ __launch_bounds__(kBlock) void attn_chunk_mfma_kernel(const float * _
     // cells the furthest-reaching token of the tile sees
     int n_kv = pos_p[min(t0 + i, T - 1)] + 1;
     for (int o = 8; o > 0; o >>= 1) n_kv = max(n_kv, __shfl_xor(n_kv, o, PI_WAVE));
+    n_kv = min(n_kv, s_stride - 4);                // the launcher sized the scores for the cells its caller announced
     const int n_t16 = (n_kv + 15) / 16, n_t32 = (n_kv + 31) / 32;
 
     // ---- 1. scores --------------------------------------------------------------------------------------------------------
@@ -566,7 +567,7 @@ __global__ __launch_bounds__(kBlock) void attn_chunk_mfma_kernel(const float * _
     // ---- 2. softmax: 16 lanes per token, four cells per lane and step ------------------------------------------------------------
     {
         const int q = threadIdx.x >> 4, j = threadIdx.x & 15;
-        const int nq = pos_p[min(t0 + q, T - 1)] + 1;
+        const int nq = min(pos_p[min(t0 + q, T - 1)] + 1, n_kv);
         float * sq = s + (size_t)q * s_stride;
         float mx = -INFINITY;
         for (int c = 4 * j; c < nq; c += 64) {
@@ -813,9 +814,10 @@ int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_t
 }
 
 int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,
-                    const int32_t * pos, int n_ctx, float * q_rot, void * k_cache, void * v_cache, float * out, int out_stride, void * out_f16,
+                    const int32_t * pos, int n_ctx, int n_kv_max, float * q_rot, void * k_cache, void * v_cache, float * out, int out_stride, void * out_f16,
                     pi_stream_t stream) {
     if (!qkv || !pos || !q_rot || !k_cache || !v_cache || !out || T <= 0 || T > kChunkMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad arguments");
+    if (n_kv_max <= 0 || n_kv_max > n_ctx) n_kv_max = n_ctx;                  // cells the furthest token of the chunk attends: what the scores in LDS are sized for
     if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || hd <= 0 || hd % 8 || hd / 2 > 1024 || kBlock % (hd / 8) || PI_WAVE % (hd / 8) || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_attn_chunk: bad head geometry or mode");
     hipStream_t st = (hipStream_t)stream;
@@ -823,7 +825,7 @@ int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_
     hipLaunchKernelGGL(rope_kv_store_kernel, dim3(n_head + 2 * n_head_kv, T), dim3(hd / 2), 0, st,
                        qkv, n_head, n_head_kv, hd, mode, theta_scale, freq_scale, pos, n_ctx, q_rot, (__half *)k_cache, (__half *)v_cache, qkv_stride, n_head * hd);
     // 16 tokens per workgroup on the matrix cores where the head size and the context fit (scores of 16 tokens in LDS)
-    const int s_stride = ((n_ctx + 31) & ~31) + 4;
+    const int s_stride = ((n_kv_max + 31) & ~31) + 4;
     const size_t sh_mfma = sizeof(float) * 16 * (size_t)s_stride + (size_t)kWavesPerBlock * hd * kAcVtStride * 2;
     const char * own = getenv("PI_ATTN_CHUNK");
     if ((hd == 128 || hd == 64) && T > 1 && sh_mfma <= 156 * 1024 && !(own && !strcmp(own, "scalar"))) {
@@ -841,15 +843,16 @@ int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_
         return pi::check_launch("pi_k_attn_chunk");
     }
     const size_t sh = sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd);
-    if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_chunk: context too long for the single-pass kernel");
+    if (sh > 60 * 1024) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_chunk: context too long for the single-pass kernel (pi_k_attn_chunk_supported)");
     hipLaunchKernelGGL(attn_decode_kernel, dim3(n_head, T), dim3(kBlock), sh, st,
                        q_rot, (const __half *)k_cache, (const __half *)v_cache, n_head, n_head_kv, hd, n_ctx, pos, out, n_head * hd, out_stride, (__half *)out_f16);
     return pi::check_launch("pi_k_attn_chunk");
 }
 
-int pi_k_attn_chunk_supported(int hd, int n_ctx) {
+int pi_k_attn_chunk_supported(int hd, int n_ctx, int n_kv_max) {
     if (hd <= 0 || hd % 8 || kBlock % (hd / 8) || PI_WAVE % (hd / 8) || n_ctx <= 0) return 0;
-    const int s_stride = ((n_ctx + 31) & ~31) + 4;
+    if (n_kv_max <= 0 || n_kv_max > n_ctx) n_kv_max = n_ctx;
+    const int s_stride = ((n_kv_max + 31) & ~31) + 4;
     const size_t sh_mfma = sizeof(float) * 16 * (size_t)s_stride + (size_t)kWavesPerBlock * hd * kAcVtStride * 2;
     if ((hd == 128 || hd == 64) && sh_mfma <= 156 * 1024) return 1;
     return sizeof(float) * ((size_t)n_ctx + (size_t)(kBlock / (hd / 8)) * hd) <= 60 * 1024;

@@ -303,21 +303,25 @@ __device__ __forceinline__ int select_nth_bit64(uint64_t bits, int n) {      // 
 // unconditional - a wave without an ROWS-th row of its own requests the range's last row again, which its unit already has on the way -
 // because the compiler counts outstanding loads conservatively across branches and would otherwise hold the norm statistics back
 // until the last predictor row has landed.
-template <int RCH, bool GATE, int ROWS, int KIND>      // r == RCH * 512; ROWS fc2 rows per wave: at most 8 * ROWS neurons per workgroup
-__global__ __launch_bounds__(kPfBlock, 1) void ffn_cu_f16_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
+// NW waves of 512 columns each (8: 4096 columns, 10: 5120); R = predictor rank, a multiple of 256 (a last half chunk of 512 is read by
+// half the lanes, the others re-read the row's start against a zero of the hidden vector).  Ten waves are three on two of the four
+// SIMDs, which leaves each 168 registers: eight active neurons travel at once instead of twelve.
+template <int NW, int R, bool GATE, int ROWS, int KIND>      // ROWS fc2 rows per wave: at most NW * ROWS neurons per workgroup
+__global__ __launch_bounds__(NW * 64, 1) void ffn_cu_f16_kernel(const __half * __restrict__ W2, const float * __restrict__ hidden,
                                                                  const __half * __restrict__ Wup, const __half * __restrict__ Wgate,
                                                                  const __half * __restrict__ Wdown,
                                                                  const float * __restrict__ x, const float * __restrict__ nw, const float * __restrict__ nb, float eps,
                                                                  float thr, int ff,
                                                                  float * __restrict__ logits, uint32_t * __restrict__ words, float * __restrict__ h_dense,
                                                                  float * __restrict__ partial) {
-    constexpr int cols = kPfWaves * 512, r = RCH * 512, CH = kCuChunk;
+    constexpr int cols = NW * 512, r = R, RCH = (R + 511) / 512, CH = NW == 8 ? kCuChunk : 8;
+    static_assert(R % 256 == 0 && NW * ROWS <= 64 + NW - 1, "rank in half chunks; one 64-bit mask per workgroup");
     __shared__ float  lg[64];
-    __shared__ double red[2][kPfWaves];
-    __shared__ float  part[kPfWaves][CH][2];
+    __shared__ double red[2][NW];
+    __shared__ float  part[NW][CH][2];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int n0 = (int)((long long)ff * blockIdx.x / gridDim.x);
-    const int np = (int)((long long)ff * (blockIdx.x + 1) / gridDim.x) - n0;       // <= 8 * ROWS <= 64 (the launcher's test)
+    const int np = (int)((long long)ff * (blockIdx.x + 1) / gridDim.x) - n0;       // <= NW * ROWS and <= 64 (the launcher's test)
     const int cbase = wave * 512 + lane * 8;
 
     // ---- A: loads.  Memory returns a wave's loads in the order it issued them: the small operands go first, so that the norm
@@ -337,19 +341,23 @@ __global__ __launch_bounds__(kPfBlock, 1) void ffn_cu_f16_kernel(const __half * 
         }
     }
     float4 hv[RCH][2];
+    int roff[RCH];
 #pragma unroll
     for (int j = 0; j < RCH; ++j) {
-        hv[j][0] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8);
-        hv[j][1] = *reinterpret_cast<const float4 *>(hidden + j * 512 + lane * 8 + 4);
+        const bool in = (j + 1) * 512 <= R || (j * PI_WAVE + lane) * 8 < R;          // the last chunk may be half a chunk
+        roff[j] = in ? (j * PI_WAVE + lane) * 8 : 0;
+        hv[j][0] = *reinterpret_cast<const float4 *>(hidden + roff[j]);
+        hv[j][1] = *reinterpret_cast<const float4 *>(hidden + roff[j] + 4);
+        if (!in) hv[j][0] = hv[j][1] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
     }
     pi_u32x4 a[ROWS][RCH];
 #pragma unroll
     for (int i = 0; i < ROWS; ++i) {
-        const int row = wave + 8 * i < np ? wave + 8 * i : np - 1;
+        const int row = wave + NW * i < np ? wave + NW * i : np - 1;
 #pragma unroll
-        for (int j = 0; j < RCH; ++j) a[i][j] = pi_ld_stream(W2 + (size_t)(n0 + row) * r + (j * PI_WAVE + lane) * 8);
+        for (int j = 0; j < RCH; ++j) a[i][j] = pi_ld_stream(W2 + (size_t)(n0 + row) * r + roff[j]);
     }
-    // ---- A: norm statistics across the 8 slices ---------------------------------------------------------------
+    // ---- A: norm statistics across the NW slices ---------------------------------------------------------------
     float mean = 0.0f, scale = 1.0f;
     if (KIND == 1) {
         double sq = 0.0;
@@ -360,7 +368,7 @@ __global__ __launch_bounds__(kPfBlock, 1) void ffn_cu_f16_kernel(const __half * 
         __syncthreads();
         double t = 0.0;
 #pragma unroll
-        for (int w = 0; w < kPfWaves; ++w) t += red[0][w];
+        for (int w = 0; w < NW; ++w) t += red[0][w];
         scale = pi_inv_sqrt((float)(t / cols) + eps);
     } else if (KIND == 2) {
         double sm = 0.0;
@@ -371,7 +379,7 @@ __global__ __launch_bounds__(kPfBlock, 1) void ffn_cu_f16_kernel(const __half * 
         __syncthreads();
         double t = 0.0;
 #pragma unroll
-        for (int w = 0; w < kPfWaves; ++w) t += red[0][w];
+        for (int w = 0; w < NW; ++w) t += red[0][w];
         mean = (float)(t / cols);
         double sq = 0.0;
 #pragma unroll
@@ -381,7 +389,7 @@ __global__ __launch_bounds__(kPfBlock, 1) void ffn_cu_f16_kernel(const __half * 
         __syncthreads();
         double t2 = 0.0;
 #pragma unroll
-        for (int w = 0; w < kPfWaves; ++w) t2 += red[1][w];
+        for (int w = 0; w < NW; ++w) t2 += red[1][w];
         scale = pi_inv_sqrt((float)(t2 / cols) + eps);
     }
     pi_u32x4 xr;
@@ -412,7 +420,7 @@ __global__ __launch_bounds__(kPfBlock, 1) void ffn_cu_f16_kernel(const __half * 
 #pragma unroll
             for (int j = 0; j < RCH; ++j) acc = pi_dot8h(a[i][j], hr[j], acc);
             acc = pi_wave_sum(acc);
-            if (lane == 0 && wave + 8 * i < np) lg[wave + 8 * i] = acc;
+            if (lane == 0 && wave + NW * i < np) lg[wave + NW * i] = acc;
         }
     }
     __syncthreads();
@@ -462,7 +470,7 @@ __global__ __launch_bounds__(kPfBlock, 1) void ffn_cu_f16_kernel(const __half * 
             if (j < nn) {
                 float u = 0.0f, g = 0.0f;
 #pragma unroll
-                for (int w = 0; w < kPfWaves; ++w) { u += part[w][j][0]; if (GATE) g += part[w][j][1]; }
+                for (int w = 0; w < NW; ++w) { u += part[w][j][0]; if (GATE) g += part[w][j][1]; }
                 const float h = GATE ? __fmul_rn(fmaxf(g, 0.0f), u) : fmaxf(u, 0.0f);
                 if (h_dense && threadIdx.x == 0) h_dense[rows[j]] = h;
                 const float hq = pi_round_f16(h);                 // the CPU axpy rounds h to fp16 (ggml.c:14420-14431)
@@ -1096,9 +1104,14 @@ int pi_k_axpy_q4_reduce(int ff, int cols, int epilogue, const float * add1, cons
     return pi::check_launch("pi_k_axpy_q4_reduce");
 }
 
-int pi_k_sparse_ffn_supported(int ff, int r, int cols) { return (cols == 4096 || cols == 8192) && (r == 1024 || r == 512) && ff > 0 && ff % 32 == 0; }
-static int pf_parts(int ff, int cols, bool hyb);
-int pi_k_sparse_ffn_workgroups(int ff, int r, int cols) { return pi_k_sparse_ffn_supported(ff, r, cols) ? pf_parts(ff, cols, false) : 0; }
+static int pf_cu_workgroups(int ff, int r, int cols);
+// the grouped form (a workgroup per 32 G neurons) and the two-phase forms of hybrid layers
+static bool pf_grouped_shape(int ff, int r, int cols) { return (cols == 4096 || cols == 8192) && (r == 1024 || r == 512) && ff > 0 && ff % 32 == 0; }
+// 5120 columns with a predictor of rank 1280 (the 13B shape) exist in the one-workgroup-per-unit form only: every neuron resident,
+// at most 60 neurons per compute unit
+int pi_k_sparse_ffn_supported(int ff, int r, int cols) { return pf_grouped_shape(ff, r, cols) || pf_cu_workgroups(ff, r, cols) > 0; }
+static int pf_parts(int ff, int r, int cols, bool hyb);
+int pi_k_sparse_ffn_workgroups(int ff, int r, int cols) { return pi_k_sparse_ffn_supported(ff, r, cols) ? pf_parts(ff, r, cols, false) : 0; }
 
 // Groups of 32 neurons per workgroup of the fused sparse FFN.  Wide rows: a workgroup takes four groups in turn (the next
 // group's predictor rows travel during the current group's FFN rows) and stores one partial vector for all of them, which
@@ -1110,21 +1123,22 @@ static int pf_groups(int ff, int cols) {
 
 // Workgroups of the one-per-compute-unit form (ffn_cu_f16_kernel), or 0 where the grouped form runs: 4096 columns, every neuron on
 // the device, and more than 32 but at most 64 neurons per unit (with 32 or fewer the groups of 32 already have a unit each).
-static int pf_cu_workgroups(int ff, int cols) {
-    if (cols != 4096) return 0;
+static int pf_cu_workgroups(int ff, int r, int cols) {
+    const bool wide = cols == 5120 && r == 1280;
+    if (!wide && !(cols == 4096 && (r == 1024 || r == 512))) return 0;
     const int n_cu = pi::compute_units();
-    if (n_cu <= 0 || ff <= 32 * n_cu || (ff + n_cu - 1) / n_cu > 64) return 0;
+    if (n_cu <= 0 || ff <= 32 * n_cu || (ff + n_cu - 1) / n_cu > (wide ? 60 : 64)) return 0;
     return n_cu;
 }
 // partial vectors the fused launch leaves for the reduction when nothing about the call rules the one-per-unit form out
-static int pf_parts(int ff, int cols, bool hyb) { const int n = hyb ? 0 : pf_cu_workgroups(ff, cols); return n ? n : ff / (32 * pf_groups(ff, cols)); }
+static int pf_parts(int ff, int r, int cols, bool hyb) { const int n = hyb ? 0 : pf_cu_workgroups(ff, r, cols); return n ? n : ff / (32 * pf_groups(ff, cols)); }
 
 static int sparse_ffn_partials_impl(const char * who, const void * fc2_f16, int ff, int r, const float * hidden, float threshold,
                                     const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const float * x, const pi_norm * norm,
                                     float * logits, float * h_dense, const uint32_t * hot_words, const int32_t * hot_prefix, void * xn_f16_out,
                                     pi_workspace * ws, pi_stream_t stream) {
     if (!fc2_f16 || !hidden || !up_f16 || !down_t_f16 || !x || !ws) return pi::fail(PI_E_ARG, who);
-    if (!pi_k_sparse_ffn_supported(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn: shape outside the fused kernel (cols 4096 or 8192, r 512 or 1024, ff % 32 == 0)");
+    if (!pi_k_sparse_ffn_supported(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn: shape outside the fused kernels (cols 4096 or 8192 with r 512 or 1024 and ff % 32 == 0; cols 5120 with r 1280 and 33..60 neurons per compute unit)");
     if (ff > ws->max_ff || cols > ws->max_d) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: shape exceeds the workspace");
     if ((hot_words == nullptr) != (hot_prefix == nullptr)) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn: hot_words and hot_prefix go together");
     const NormArgs na = to_norm(norm);
@@ -1135,19 +1149,22 @@ static int sparse_ffn_partials_impl(const char * who, const void * fc2_f16, int 
     const bool hyb = hot_words != nullptr;
     // the one-workgroup-per-unit form takes the norm as a template parameter: it must carry what its kind needs
     const bool cu_norm = na.kind == 0 || (na.kind == 1 && na.w && !na.b) || (na.kind == 2 && na.w && na.b);
-    if (const int n_wg = (hyb || !cu_norm) ? 0 : pf_cu_workgroups(ff, cols)) {
-        const int rows = ((ff + n_wg - 1) / n_wg + 7) / 8;              // fc2 rows per wave
-#define PI_CU_LAUNCH(RCH, GATE, ROWS, KIND) hipLaunchKernelGGL((ffn_cu_f16_kernel<RCH, GATE, ROWS, KIND>), dim3(n_wg), dim3(kPfBlock), 0, st, w2, hidden, u, g, dn, x, na.w, na.b, na.eps, threshold, ff, logits, ws->words, h_dense, ws->ffn_partial)
-#define PI_CU_KIND(RCH, GATE, ROWS) do { if (na.kind == 0) PI_CU_LAUNCH(RCH, GATE, ROWS, 0); else if (na.kind == 1) PI_CU_LAUNCH(RCH, GATE, ROWS, 1); else PI_CU_LAUNCH(RCH, GATE, ROWS, 2); } while (0)
-#define PI_CU_ROWS(RCH, GATE) do { if (rows <= 6) PI_CU_KIND(RCH, GATE, 6); else PI_CU_KIND(RCH, GATE, 8); } while (0)
-        if (r == 1024) { if (g) PI_CU_ROWS(2, true); else PI_CU_ROWS(2, false); }
-        else           { if (g) PI_CU_ROWS(1, true); else PI_CU_ROWS(1, false); }
+    if (const int n_wg = (hyb || !cu_norm) ? 0 : pf_cu_workgroups(ff, r, cols)) {
+        const int nw = cols / 512;
+        const int rows = ((ff + n_wg - 1) / n_wg + nw - 1) / nw;         // fc2 rows per wave
+#define PI_CU_LAUNCH(NW, R, GATE, ROWS, KIND) hipLaunchKernelGGL((ffn_cu_f16_kernel<NW, R, GATE, ROWS, KIND>), dim3(n_wg), dim3(NW * 64), 0, st, w2, hidden, u, g, dn, x, na.w, na.b, na.eps, threshold, ff, logits, ws->words, h_dense, ws->ffn_partial)
+#define PI_CU_KIND(NW, R, GATE, ROWS) do { if (na.kind == 0) PI_CU_LAUNCH(NW, R, GATE, ROWS, 0); else if (na.kind == 1) PI_CU_LAUNCH(NW, R, GATE, ROWS, 1); else PI_CU_LAUNCH(NW, R, GATE, ROWS, 2); } while (0)
+#define PI_CU_ROWS(NW, R, GATE) do { if (rows <= 6) PI_CU_KIND(NW, R, GATE, 6); else PI_CU_KIND(NW, R, GATE, 8); } while (0)
+        if (cols == 5120)   { if (g) PI_CU_KIND(10, 1280, true, 6); else PI_CU_KIND(10, 1280, false, 6); }
+        else if (r == 1024) { if (g) PI_CU_ROWS(8, 1024, true); else PI_CU_ROWS(8, 1024, false); }
+        else                { if (g) PI_CU_ROWS(8, 512, true); else PI_CU_ROWS(8, 512, false); }
 #undef PI_CU_ROWS
 #undef PI_CU_KIND
 #undef PI_CU_LAUNCH
         ws->pf_parts = n_wg; ws->pf_words = 2 * n_wg;
         return pi::check_launch(who);
     }
+    if (!pf_grouped_shape(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn: this shape runs only with every neuron resident and a norm the kernel carries (5120 columns, rank 1280)");
     ws->pf_parts = ff / (32 * pf_groups(ff, cols)); ws->pf_words = ff / 32;
     const int G = pf_groups(ff, cols);
     const dim3 grid(ff / (32 * G)), block(kPfBlock);
@@ -1177,11 +1194,13 @@ int pi_k_sparse_ffn_partials_hot(const void * fc2_f16, int ff, int r, const floa
                                  const uint32_t * hot_words, const int32_t * hot_prefix, float * logits, float * h_dense, void * xn_f16_out,
                                  pi_workspace * ws, pi_stream_t stream) {
     if (!hot_words || !hot_prefix) return pi::fail(PI_E_ARG, "pi_k_sparse_ffn_partials_hot: hot words and prefix are required");
+    if (!pf_grouped_shape(ff, r, cols)) return pi::fail(PI_E_UNSUPPORTED, "pi_k_sparse_ffn_partials_hot: shape outside the fused kernel of hybrid layers (pi_k_sparse_ffn_hot_supported)");
     return sparse_ffn_partials_impl("pi_k_sparse_ffn_partials_hot", fc2_f16, ff, r, hidden, threshold, up_f16, gate_f16, down_t_f16, cols, x, norm, logits, h_dense,
                                     hot_words, hot_prefix, xn_f16_out, ws, stream);
 }
 
-int pi_k_sparse_ffn_two_phase_supported(int ff, int r, int cols) { return pi_k_sparse_ffn_supported(ff, r, cols) && cols == 4096; }
+int pi_k_sparse_ffn_hot_supported(int ff, int r, int cols) { return pf_grouped_shape(ff, r, cols); }
+int pi_k_sparse_ffn_two_phase_supported(int ff, int r, int cols) { return pf_grouped_shape(ff, r, cols) && cols == 4096; }
 
 int pi_k_sparse_ffn_logits_hot(const void * fc2_f16, int ff, int r, const float * hidden, float threshold, int cols, const float * x, const pi_norm * norm,
                                const uint32_t * hot_words, const int32_t * hot_prefix, float * logits, float * logits_dev, void * xn_f16_out,
@@ -1295,7 +1314,7 @@ size_t pi_k_sparse_ffn_noalloc_scratch_bytes(void) { return kNaScratchBytes; }
 
 int pi_k_sparse_ffn_noalloc_supported(int ff, int r, int cols) {
     if (!pi_k_sparse_ffn_supported(ff, r, cols)) return 0;
-    const size_t parts = (size_t)pf_parts(ff, cols, false);
+    const size_t parts = (size_t)pf_parts(ff, r, cols, false);
     return ff / 32 <= kNaMaxWords && 2 * parts <= (size_t)kNaMaxWords && parts * (size_t)cols * sizeof(float) <= kNaPartialBytes;
 }
 

@@ -56,6 +56,7 @@ _SIGS = {
     "pi_k_sparse_upgate": (_i, [_i, _vp, _vp, _i, _i, _vp, C.POINTER(Norm), _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_axpy": (_i, [_i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_supported": (_i, [_i, _i, _i]),
+    "pi_k_sparse_ffn_hot_supported": (_i, [_i, _i, _i]),
     "pi_k_sparse_ffn_workgroups": (_i, [_i, _i, _i]),
     "pi_k_sparse_ffn": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_noalloc_scratch_bytes": (_sz, []),
@@ -108,11 +109,11 @@ _SIGS = {
     "pi_k_attn_split_supported": (_i, [_i, _i, _i]),
     "pi_k_attn_split_scratch_floats": (_sz, [_i, _i, _i, _i]),
     "pi_k_attn_split": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _vp, _vp]),
-    "pi_k_attn_chunk_supported": (_i, [_i, _i]),
+    "pi_k_attn_chunk_supported": (_i, [_i, _i, _i]),
     "pi_k_attn_chunk_long": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _f, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_attn_split_cached": (_i, [_vp, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "pi_k_attn_fused_batch": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _vp]),
-    "pi_k_attn_chunk": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _f, _vp, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
+    "pi_k_attn_chunk": (_i, [_vp, _i, _i, _i, _i, _i, _i, _f, _f, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _vp, _vp]),
     "pi_k_embed_batch": (_i, [_vp, _i, _vp, _i, _vp, _vp]),
     "pi_k_argmax_batch": (_i, [_vp, _i, _i, _vp, _vp, _vp, _vp, _i, _vp]),
     "pi_k_step_advance": (_i, [_vp, _vp]),

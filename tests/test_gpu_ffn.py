@@ -106,6 +106,17 @@ def test_one_launch_route_wide_rows(has_gate, norm):
     run_fused_route(has_gate, norm, "one", 8192, 4096, 512)
 
 
+@pytest.mark.parametrize("has_gate,norm", [(True, 1), (False, 2), (True, 0)])
+def test_one_launch_route_13b_layer(has_gate, norm):
+    """One FFN block at the 13B shape (13824 x 5120, predictor rank 1280 = two and a half chunks of 512): ten waves per workgroup, one
+    workgroup per compute unit, the last half chunk of the predictor rows read by half the lanes."""
+    from powerinfer_amd import lib as pl
+    assert pl.load().pi_k_sparse_ffn_supported(13824, 1280, 5120) == 1
+    assert pl.load().pi_k_sparse_ffn_hot_supported(13824, 1280, 5120) == 0          # hybrid layers of this width keep the list kernels
+    assert pl.load().pi_k_sparse_ffn_workgroups(13824, 1280, 5120) == 256
+    run_fused_route(has_gate, norm, "one", 5120, 13824, 1280, T=2)
+
+
 def test_one_launch_route_falcon40b_layer():
     """One FFN block at the full Falcon-40B shape (32768 x 8192, no gate, LayerNorm, rank 1024): the instantiation in which a
     workgroup takes four groups of 32 neurons and stores one partial vector for all of them."""

@@ -228,7 +228,7 @@ def run_north_star(hp, n_prompt=8, n_gen=64, model=None):
 
 NS = dict(pred_margin=True, head_pair=2048)
 # seeds whose greedy path (a CPU-oracle property) visits both tokens of the pair
-SEED_7B_F16, SEED_7B_Q4, SEED_F40, SEED_7B_FULL = 35, 40, 44, 3
+SEED_7B_F16, SEED_7B_Q4, SEED_F40, SEED_7B_FULL, SEED_13B = 35, 40, 44, 3, 45
 
 
 # (Q4_0 at this width is left to run_case: 256-wide activations make one int8 rounding step a visible share of a dot product, and
@@ -268,6 +268,13 @@ def test_north_star_f16_7b_full_depth():
 def test_north_star_q4_split_7b_width():
     """configs[2]: the same shape in Q4_0 with the hottest 60 % of each layer's neurons on the GPU and the rest on host threads."""
     run_north_star(synth.hparams("llama-7b", n_layer=2, n_ctx=96, seed=SEED_7B_Q4, wtype=synth.Q4_0, hot_frac=0.6, **NS))
+
+
+@pytest.mark.timeout(600)
+def test_north_star_13b_width_single_sequence():
+    """configs[3]'s layer shape at batch 1 (d 5120, 40 heads, ff 13824, predictor rank 1280, two layers) through the token loop: the
+    5120-column mat-vecs and the ten-wave fused FFN, neurons dealt out by rate."""
+    run_north_star(synth.hparams("llama-13b", n_layer=2, n_ctx=96, seed=SEED_13B, **NS))
 
 
 @pytest.mark.timeout(600)
@@ -323,24 +330,25 @@ def test_north_star_long_context_allocation(arch, seed):
 
 
 @pytest.mark.timeout(600)
-def test_prompt_and_decode_at_a_context_beyond_the_chunk_kernels():
-    """n_ctx 16384: the scores of a prompt chunk no longer fit the chunk kernels' LDS, so the prompt goes through pi_k_attn_chunk_long and
-    the token loop through pi_k_attn_split.  A 300-token prompt and 12 decoded tokens against the oracle, token by token."""
+@pytest.mark.parametrize("n_prompt", [300, 2200])
+def test_prompt_and_decode_at_a_context_beyond_the_chunk_kernels(n_prompt):
+    """n_ctx 16384, far more cells than the chunk kernels' LDS holds.  What a chunk needs is sized by the cells it attends, not by the
+    cache: a 300-token prompt still runs 16 tokens per workgroup on the matrix cores; a 2200-token prompt starts there and, from about
+    1850 cells on, goes through pi_k_attn_chunk_long (every token's cells split over several workgroups).  The token loop takes
+    pi_k_attn_split.  Prompt and 12 decoded tokens against the oracle, token by token."""
     from powerinfer_amd.model import Model
     hp = synth.hparams("llama-tiny", n_ctx=16384, seed=23, **NS)
     model = synth.make_model(hp)
     gm, om = Model(hp).load(model), ol.OracleModel(model)
     rng = np.random.default_rng(11)
-    prompt = rng.integers(0, hp.n_vocab, 300).astype(np.int32)
+    prompt = rng.integers(0, hp.n_vocab, n_prompt).astype(np.int32)
     tok_g, lg_g = gm.decode(prompt, 0)
-    tok_o = lg_o = None
-    for i, t in enumerate(prompt):
-        tok_o, lg_o = om.eval([int(t)], i)
+    tok_o, lg_o = om.eval([int(t) for t in prompt], 0)
     assert rel_err(lg_g, lg_o) < 1e-2 and tok_g == tok_o
     cur = int(tok_o)
     for s in range(12):
-        nxt_o, lg_o = om.eval([cur], 300 + s)
-        nxt_g, lg_g = gm.decode([cur], 300 + s)
+        nxt_o, lg_o = om.eval([cur], n_prompt + s)
+        nxt_g, lg_g = gm.decode([cur], n_prompt + s)
         assert rel_err(lg_g, lg_o) < 1e-2, (s, rel_err(lg_g, lg_o))
         assert nxt_g == nxt_o
         cur = int(nxt_o)

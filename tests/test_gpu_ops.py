@@ -138,8 +138,9 @@ def test_attention_of_prompt_chunks(mode, hd, nh, nkv, chunks, fs, monkeypatch):
                 monkeypatch.delenv("PI_ATTN_CHUNK", raising=False)
             dqr, dout, dout16 = pl.DevBuf(T * d * 4), pl.DevBuf(T * d * 4), pl.DevBuf(T * d * 2)
             pl.check(L.pi_memset(dout.ptr, 0xFF, dout.nbytes), "memset")
-            pl.check(L.pi_k_attn_chunk(dq.ptr, d + 2 * gqa, T, nh, nkv, hd, mode, theta_scale, fs, dpos.ptr, n_ctx, dqr.ptr, kc.ptr, vc.ptr,
-                                       dout.ptr, d, dout16.ptr, None), "attn_chunk")
+            # the scores in LDS are sized for the cells the chunk attends (mfma) or for the whole cache (n_kv_max 0)
+            pl.check(L.pi_k_attn_chunk(dq.ptr, d + 2 * gqa, T, nh, nkv, hd, mode, theta_scale, fs, dpos.ptr, n_ctx, n_past + T if route == "mfma" else 0,
+                                       dqr.ptr, kc.ptr, vc.ptr, dout.ptr, d, dout16.ptr, None), "attn_chunk")
             pl.sync()
             got[route] = dout.download(np.float32).reshape(T, d)
             assert np.array_equal(dout16.download(np.float16).reshape(T, d), got[route].astype(np.float16))
@@ -149,6 +150,9 @@ def test_attention_of_prompt_chunks(mode, hd, nh, nkv, chunks, fs, monkeypatch):
         assert not np.array_equal(got["mfma"], got["scalar"])         # two routes, two summation orders
         n_past += T
     monkeypatch.delenv("PI_ATTN_CHUNK", raising=False)
+    # which kernel a chunk gets depends on the cells it attends, not on the size of the cache
+    assert L.pi_k_attn_chunk_supported(128, 32768, 0) == 0 and L.pi_k_attn_chunk_supported(128, 32768, 1800) == 1
+    assert L.pi_k_attn_chunk_supported(128, 32768, 2400) == 0 and L.pi_k_attn_chunk_supported(128, 8192, 2400) == 1      # one token per workgroup
 
 
 @pytest.mark.parametrize("mode,hd,nh,nkv,fs", [(0, 128, 4, 4, 1.0), (2, 64, 8, 2, 1.0), (0, 128, 4, 4, 0.25), (2, 64, 8, 2, 0.5)])

@@ -202,35 +202,48 @@ def cpu_reference(model, prompt, n_prompt, n_decode, threads):
         shutil.rmtree(td, ignore_errors=True)
 
 
-def reference_host_on_this_backend(n_layer=4, n_prompt=8, n_gen=48):
-    """The cost of per-node dispatch as a number: the reference's own llama.cpp (loader, ggml-alloc, graph builder, executor)
-    compiled against this library in place of ggml-cuda.cu (oracle/_ref/ref_llama_gpu, test infrastructure) decodes a 7B-wide,
-    n_layer-deep synthetic model with every tensor on the GPU, one ggml_cuda_compute_forward call per graph node."""
+def reference_host_on_this_backend(n_prompt=8, n_gen=48):
+    """The drop-in path as a number: the reference's own llama.cpp (loader, ggml-alloc, graph builder, executor) compiled against this
+    library in place of ggml-cuda.cu (oracle/_ref/ref_llama_gpu, test infrastructure) decodes 7B-wide synthetic models of 4 and of 8
+    layers with every tensor on the GPU, one ggml_cuda_compute_forward call per graph node.  The difference between the two runs is
+    what one more layer costs; the 4-layer figure also carries what the host does once per token (graph construction, the
+    inputs' upload, the lm-head and the logits' way back)."""
     import subprocess
     import tempfile
     from powerinfer_amd import gguf, split, synth
     exe = os.path.join(ROOT, "oracle", "_ref", "ref_llama_gpu")
     if not os.path.exists(exe):
         return None
-    hp = synth.hparams("llama-7b", n_layer=n_layer, n_ctx=128, seed=3)
-    model = synth.make_model(hp)
-    with tempfile.TemporaryDirectory() as td:
-        path, out = os.path.join(td, "m.powerinfer.gguf"), os.path.join(td, "out.bin")
-        gguf.write_model(path, model, gguf.synthetic_tokenizer_kv(hp.n_vocab))
-        splits = [(np.ones(hp.n_ff, np.int32), np.arange(hp.n_ff, dtype=np.int32)) for _ in range(hp.n_layer)]
-        split.write_gpuidx(path + ".generated.gpuidx", splits, split.required_bytes(hp, splits))
-        del model
-        toks = [str(int(t)) for t in np.random.default_rng(5).integers(0, hp.n_vocab, n_prompt)]
-        r = subprocess.run([exe, path, "128", "1", str(n_gen), out] + toks, env=dict(os.environ, REF_VRAM_GB="16"),
-                           capture_output=True, text=True, timeout=240)
-    if r.returncode != 0:
-        return {"error": (r.stdout + r.stderr)[-300:]}
-    ms = [float(l.split()[1]) for l in r.stdout.splitlines() if l.startswith("decode_ms_per_token")]
-    if not ms:
-        return {"error": "no timing line"}
-    return {"ms_per_token": round(ms[0], 3), "n_layer": n_layer, "ms_per_token_per_layer": round(ms[0] / n_layer, 4), "host_threads": 1,
+    ms_of, stats = {}, {}
+    for n_layer in (4, 8):
+        hp = synth.hparams("llama-7b", n_layer=n_layer, n_ctx=128, seed=3)
+        model = synth.make_model(hp)
+        with tempfile.TemporaryDirectory() as td:
+            path, out = os.path.join(td, "m.powerinfer.gguf"), os.path.join(td, "out.bin")
+            gguf.write_model(path, model, gguf.synthetic_tokenizer_kv(hp.n_vocab))
+            splits = [(np.ones(hp.n_ff, np.int32), np.arange(hp.n_ff, dtype=np.int32)) for _ in range(hp.n_layer)]
+            split.write_gpuidx(path + ".generated.gpuidx", splits, split.required_bytes(hp, splits))
+            del model
+            toks = [str(int(t)) for t in np.random.default_rng(5).integers(0, hp.n_vocab, n_prompt)]
+            r = subprocess.run([exe, path, "128", "1", str(n_gen), out] + toks, env=dict(os.environ, REF_VRAM_GB="16"),
+                               capture_output=True, text=True, timeout=240)
+        if r.returncode != 0:
+            return {"error": (r.stdout + r.stderr)[-300:]}
+        ms = [float(l.split()[1]) for l in r.stdout.splitlines() if l.startswith("decode_ms_per_token")]
+        if not ms:
+            return {"error": "no timing line"}
+        ms_of[n_layer] = ms[0]
+        for l in r.stdout.splitlines():
+            if l.startswith("backend_stats"):
+                w = l.split()
+                stats[n_layer] = {w[i]: int(w[i + 1]) for i in range(1, len(w), 2)}
+    return {"ms_per_token": round(ms_of[4], 3), "n_layer": 4, "ms_per_token_per_layer": round(ms_of[4] / 4, 4),
+            "ms_per_token_8_layers": round(ms_of[8], 3), "ms_per_additional_layer": round((ms_of[8] - ms_of[4]) / 4, 4),
+            "backend_stats_8_layers": stats.get(8), "host_threads": 1,
             "what": "reference llama.cpp + ggml executor linked to libpowerinfer_hip.so (oracle/_ref/ref_llama_gpu), 7B-wide layers, "
-                    "all tensors and the KV cache on the GPU, one backend call per graph node; includes the lm-head once per token"}
+                    "all tensors and the KV cache on the GPU, one backend call per graph node (single-token nodes wait in a window: an "
+                    "attention block runs as three launches, an FFN block as three); ms_per_token includes the lm-head and the host's "
+                    "per-token work once, ms_per_additional_layer is (8 layers - 4 layers) / 4"}
 
 
 def bench_batched(args):

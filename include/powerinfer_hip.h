@@ -82,6 +82,11 @@ enum { PI_EPI_NONE = 0, PI_EPI_RELU = 1, PI_EPI_ADD = 2, PI_EPI_ADD2 = 3 };
  */
 PI_API int pi_k_gemv(int wtype, const void * W, int rows, int cols, const float * x, const pi_norm * norm,
                      int epilogue, const float * add1, const float * add2, float * y, pi_stream_t stream);
+/* up to three F16 matrices of the same width against one vector in one launch: y[i][rows[i]] = W[i] . fp16(norm(x)).  For hosts that
+ * keep the q, k and v projections as separate tensors (llama.cpp:4989-4995: three mul_mat nodes on the same normalised input); cols
+ * 4096, 5120 or 8192.  Every product is the one pi_k_gemv computes for that matrix. */
+PI_API int pi_k_gemv_multi_f16(const void * const * W, const int * rows, int n_mat, int cols, const float * x, const pi_norm * norm,
+                               float * const * y, pi_stream_t stream);
 
 /* scratch shared by the predictor / sparse kernels of one stream; sized for the largest ff and d used */
 typedef struct pi_workspace pi_workspace;
@@ -408,6 +413,17 @@ PI_API int    pi_k_attn_chunk_long(const float * qkv, int qkv_stride, int T, int
 PI_API int    pi_k_attn_split_cached(const float * q_rot, const void * k_cache, const void * v_cache, int n_tok, int n_head, int n_head_kv, int hd,
                                      int n_ctx, int n_parts, const int32_t * pos, float * scratch, float * out, pi_stream_t stream);
 
+/* One token's attention on the reference's own cache layouts, for the ggml_cuda_* boundary: what llm_build_kv_store and llm_build_kqv
+ * (llama.cpp:4383-4418, 4764-4850) build from two ROPE, two CPY, K.q, SCALE, ADD(mask), SOFT_MAX, V.p and CONT nodes, in one launch.
+ * q [n_head * hd], k, v [n_head_kv * hd]: the token's projections before RoPE (fp32); pos: its position (device, one int32);
+ * k_cache: the layer's cells [n_kv][n_head_kv * hd] fp16; v_cache: the layer's transposed values [n_head_kv * hd][n_ctx] fp16;
+ * cell: where the token's rows are stored (< n_kv); kq_scale: one float; kq_mask: n_kv floats added to the scaled scores (-inf hides a
+ * cell); out fp32 [n_head * hd].  mode 0 / 2 and theta_scale, freq_scale, mscale as the ROPE node carries them (no YaRN mixing). */
+PI_API int pi_k_attn_ggml_supported(int hd, int n_ctx, int n_kv);
+PI_API int pi_k_attn_ggml(const float * q, const float * k, const float * v, const int32_t * pos, int mode, float theta_scale, float freq_scale, float mscale,
+                          void * k_cache, void * v_cache, int n_head, int n_head_kv, int hd, int n_ctx, int n_kv, int cell,
+                          const float * kq_scale, const float * kq_mask, float * out, pi_stream_t stream);
+
 /* per-sequence pieces of a batched step: sequence t owns token t, position pos[t] and the cache at t * cache_seq_stride
  * (elements), out_f16 (optional) receives fp16(out); pi_k_argmax_batch picks each sequence's next token (first maximum wins), stores it in tokens[t], adds 1 to
  * positions[t] and records it at out_tokens[*step][t]; pi_k_step_advance then moves *step on. */
@@ -500,7 +516,7 @@ enum {
  * it computes in one launch: llm_build_ffn_sparse's sequence (llama.cpp:4652-4757), with every neuron on the device, becomes pi_k_gemv +
  * pi_k_sparse_ffn when its AXPY node arrives.  These two calls are not part of the reference's interface: the counters tell a test or
  * a profile what the window did, the switch turns it off at run time (GGML_CUDA_NO_FUSION=1 in the environment does so from the start). */
-typedef struct pi_ggml_backend_stats { int64_t nodes_deferred, windows_flushed, ffn_blocks_fused; } pi_ggml_backend_stats;
+typedef struct pi_ggml_backend_stats { int64_t nodes_deferred, windows_flushed, ffn_blocks_fused, attn_blocks_fused; } pi_ggml_backend_stats;
 PI_API void pi_ggml_backend_get_stats(pi_ggml_backend_stats * out);
 PI_API void pi_ggml_backend_set_fusion(int enable);
 

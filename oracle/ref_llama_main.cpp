@@ -37,6 +37,9 @@
 #include <execinfo.h>
 #include <sched.h>
 #include <unistd.h>
+#ifdef GGML_USE_CUBLAS
+extern "C" void pi_ggml_backend_get_stats(int64_t * out);      // libpowerinfer_hip.so: four counters
+#endif
 
 // a crash of the host side names its call chain on stderr (the binary is linked with -rdynamic)
 static void on_fatal_signal(int sig, siginfo_t * info, void *) {
@@ -157,6 +160,13 @@ int main(int argc, char ** argv) {
     }
     fclose(f);
     if (n_gen > 0) printf("decode_ms_per_token %.4f\n", gen_ms / n_gen);
+#ifdef GGML_USE_CUBLAS
+    {   // what the backend library's window of deferred nodes did over the run (its own counters, not part of the reference's interface)
+        int64_t st[4] = {0, 0, 0, 0};
+        pi_ggml_backend_get_stats(st);
+        printf("backend_stats deferred %lld flushed %lld ffn_fused %lld attn_fused %lld\n", (long long)st[0], (long long)st[1], (long long)st[2], (long long)st[3]);
+    }
+#endif
     llama_free(ctx);
     llama_free_model(model);
     llama_backend_free();

@@ -113,6 +113,37 @@ struct Temps {
     }
 };
 
+// Small host -> device transfers (a token's position, mask, scale and embedding row arrive this way for every evaluation) go through
+// a ring of pinned slots: the bytes are copied into a slot and from there by an asynchronous transfer on the launch stream, so the host
+// does not wait for the device (a plain hipMemcpy from pageable memory returns only when the device has the data, after everything
+// queued before it).  A slot is reused once the event behind its last transfer has passed.
+struct PinRing {
+    static constexpr size_t kSlot = 64u << 10;
+    static constexpr int kSlots = 32;
+    char * base = nullptr;
+    hipEvent_t ev[kSlots];
+    bool used[kSlots] = {};
+    int next = 0;
+};
+PinRing g_pin;
+void h2d(void * dst, const void * src, size_t n) {
+    if (n == 0) return;
+    if (n > PinRing::kSlot) { BK_PI(pi_memcpy_h2d(dst, src, n)); return; }
+    if (!g_pin.base) {
+        g_pin.base = (char *)pi_malloc_host(PinRing::kSlot * PinRing::kSlots);
+        if (!g_pin.base) die("pinned staging ring");
+        for (int i = 0; i < PinRing::kSlots; ++i) BK_HIP(hipEventCreateWithFlags(&g_pin.ev[i], hipEventDisableTiming));
+    }
+    const int slot = g_pin.next;
+    g_pin.next = (g_pin.next + 1) % PinRing::kSlots;
+    if (g_pin.used[slot]) BK_HIP(hipEventSynchronize(g_pin.ev[slot]));
+    char * stage = g_pin.base + (size_t)slot * PinRing::kSlot;
+    memcpy(stage, src, n);
+    BK_HIP(hipMemcpyAsync(dst, stage, n, hipMemcpyHostToDevice, nullptr));
+    BK_HIP(hipEventRecord(g_pin.ev[slot], nullptr));
+    g_pin.used[slot] = true;
+}
+
 void * dev_ptr(const ggml_tensor * t) {
     const Extra * e = (const Extra *)t->extra;
     if (!e || !e->data_device[0]) { fprintf(stderr, "powerinfer-hip backend: tensor '%s' is marked GPU but has no device buffer\n", t->name); exit(1); }
@@ -123,7 +154,7 @@ void * dev_in(const ggml_tensor * t, Temps & tmp) {
     if (t->backend != GGML_BACKEND_CPU) return dev_ptr(t);
     const size_t n = nbytes(t);
     void * p = tmp.get(n);
-    BK_PI(pi_memcpy_h2d(p, t->data, n));
+    h2d(p, t->data, n);
     return p;
 }
 void * dev_out(ggml_tensor * t, Temps & tmp) {
@@ -593,7 +624,9 @@ void assign(ggml_tensor * tensor, bool scratch, bool force_inplace, bool no_allo
 // every pending node run, in order, before it runs itself.  Running a node late but in order, with nothing else in between, is
 // the schedule the host's allocator planned for, so buffers it shares between nodes stay valid.
 // The fused block does not write the dense up / gate vectors and the predictor's hidden layer: in the reference's graph nothing
-// else reads them (they are locals of llm_build_ffn_sparse); the predictor logits and h are still written to their nodes.
+// else reads them (they are locals of llm_build_ffn_sparse); the predictor logits and h are still written to their nodes.  When the
+// node behind the AXPY node adds the residual to its result (llama.cpp:5063, 5443), that add is the block's epilogue and only the
+// sum is written.
 // GGML_CUDA_NO_FUSION=1 in the environment turns the window off (every node runs when it arrives).
 struct PendingNode { ggml_tensor * t; int op; const ggml_tensor * src[4]; void * extra; };
 std::vector<PendingNode> g_pending;
@@ -610,8 +643,35 @@ bool weight_on_device(const ggml_tensor * a) {
            (a->type == GGML_TYPE_F16 || a->type == GGML_TYPE_Q4_0) && a->ne[0] % (a->type == GGML_TYPE_F16 ? 8 : 32) == 0;
 }
 
+// through reshapes, permutes, transposes and views to the node that computes the data
+const ggml_tensor * base_of(const ggml_tensor * t) { while (t && view_like(t->op) && t->src[0]) t = t->src[0]; return t; }
+// an fp32 result of one token: contiguous, at most two dimensions larger than one
+bool one_token(const ggml_tensor * t) { return t && t->type == GGML_TYPE_F32 && contiguous(t) && t->ne[3] == 1 && (t->ne[1] == 1 || t->ne[2] == 1); }
+
+// The nodes between the q / k / v projections and the output projection of one token's attention (llm_build_kv_store, llm_build_kqv:
+// ROPE, CPY into the cache, K.q, SCALE, + mask, SOFT_MAX, V.p, CONT) join a window that the attention norm opened, so that the block can
+// run as three launches when the window is flushed (try_fused_attn); on their own they run as they always did, in order.
+bool deferrable_attn(const ggml_tensor * n) {
+    // (the node of a copy into the cache is a view of its destination and is never read through its own address)
+    if (g_pending.empty() || n->backend != GGML_BACKEND_GPU || (n->op != GGML_OP_CPY && !on_device(n))) return false;
+    const ggml_tensor * a = n->src[0]; const ggml_tensor * b = n->src[1];
+    if (!a) return false;
+    const ggml_tensor * ab = base_of(a);
+    switch (n->op) {
+        case GGML_OP_ROPE: return one_token(n) && a->type == GGML_TYPE_F32 && is_pending(ab) && b && on_device(b) && !is_pending(b);
+        case GGML_OP_CPY:  return b && on_device(b) && is_pending(ab) && nelem(a) == nelem(b) && nelem(a) <= 16384;
+        case GGML_OP_MUL_MAT: return one_token(n) && b && is_pending(base_of(b)) && b->type == GGML_TYPE_F32 && on_device(a) && !is_pending(ab) && a->type == GGML_TYPE_F16;
+        case GGML_OP_SCALE: return one_token(n) && is_pending(a) && b && on_device(b) && !is_pending(b);
+        case GGML_OP_ADD: return one_token(n) && is_pending(a) && b && on_device(b) && !is_pending(b) && b->type == GGML_TYPE_F32 && b->ne[0] == a->ne[0];
+        case GGML_OP_SOFT_MAX: return one_token(n) && is_pending(a);
+        case GGML_OP_CONT: return one_token(n) && is_pending(ab) && a->type == GGML_TYPE_F32;
+        default: return false;
+    }
+}
+
 bool deferrable(const ggml_tensor * n) {
-    if (!g_fuse || g_pending.size() >= kMaxPending || n->backend != GGML_BACKEND_GPU || !vec1(n) || !on_device(n)) return false;
+    if (!g_fuse || g_pending.size() >= kMaxPending) return false;
+    if (n->backend != GGML_BACKEND_GPU || !vec1(n) || !on_device(n)) return deferrable_attn(n);
     const ggml_tensor * a = n->src[0]; const ggml_tensor * b = n->src[1];
     switch (n->op) {
         case GGML_OP_RMS_NORM: case GGML_OP_NORM: return vec1(a) && on_device(a) && !is_pending(a) && nelem(a) == nelem(n);
@@ -621,7 +681,7 @@ bool deferrable(const ggml_tensor * n) {
         case GGML_OP_MUL_MAT_SPARSE:
             return n->src[3] == nullptr && weight_on_device(a) && avail(b) && b->ne[0] == a->ne[0] && avail(n->src[2]) &&
                    n->src[2]->ne[0] == a->ne[1] && n->ne[0] == a->ne[1];
-        default: return false;
+        default: return deferrable_attn(n);
     }
 }
 void defer(ggml_tensor * n) { ++g_stats.nodes_deferred; g_pending.push_back(PendingNode{n, (int)n->op, {n->src[0], n->src[1], n->src[2], n->src[3]}, n->extra}); }
@@ -630,13 +690,161 @@ bool still_valid(const PendingNode & p) {
     return p.t->op == p.op && p.t->src[0] == p.src[0] && p.t->src[1] == p.src[1] && p.t->src[2] == p.src[2] && p.t->src[3] == p.src[3] && p.t->extra == p.extra;
 }
 
+// One token's attention block of build_llama (llama.cpp:4977-5022): attention norm, the q / k / v projections, RoPE, the two copies into
+// the KV cache, K.q, scale, + mask, soft-max, V.p, the gather of the heads, the output projection and the residual - seventeen nodes
+// (fourteen to sixteen in the first layer, whose norm and residual read the embedding from the host and run on their own).
+// When the window holds exactly those, they run as three launches: the three projections with the norm as their prologue
+// (pi_k_gemv_multi_f16), the attention on the cache's own layouts (pi_k_attn_ggml), the output projection with the residual as its
+// epilogue.  q, k and v pass through a buffer of this library's own (their nodes' buffers may have been handed on by the host's plan
+// by the time the attention reads them).  Returns false, with nothing done, for any other window.
+bool try_fused_attn(const std::vector<PendingNode> & win) {
+    auto in_win = [&](const ggml_tensor * t) -> const ggml_tensor * {
+        if (!t) return nullptr;
+        for (const PendingNode & p : win) if (p.t == t && still_valid(p)) return t;
+        return nullptr;
+    };
+    auto with_op = [&](const ggml_tensor * t, int op) -> const ggml_tensor * { return (in_win(t) && t->op == op) ? t : nullptr; };
+    size_t live = 0;
+    const ggml_tensor * sm = nullptr;
+    for (const PendingNode & p : win) {
+        if (!still_valid(p)) continue;
+        ++live;
+        if (p.t->op == GGML_OP_SOFT_MAX) { if (sm) return false; sm = p.t; }
+    }
+    if (!sm || live < 14 || live > 17) return false;
+    const ggml_tensor * addm = with_op(sm->src[0], GGML_OP_ADD);
+    const ggml_tensor * scl = addm ? with_op(addm->src[0], GGML_OP_SCALE) : nullptr;
+    const ggml_tensor * kq = scl ? with_op(scl->src[0], GGML_OP_MUL_MAT) : nullptr;
+    if (!kq) return false;
+    const ggml_tensor * mask = addm->src[1]; const ggml_tensor * kq_scale = scl->src[1];
+    const ggml_tensor * kview = kq->src[0];
+    const ggml_tensor * ropeq = with_op(base_of(kq->src[1]), GGML_OP_ROPE);
+    const ggml_tensor * kcpy = kview ? with_op(kview->src[1], GGML_OP_CPY) : nullptr;
+    const ggml_tensor * ropek = kcpy ? with_op(base_of(kcpy->src[0]), GGML_OP_ROPE) : nullptr;
+    if (!ropeq || !ropek || kview->op != GGML_OP_VIEW) return false;
+    const ggml_tensor * mmq = with_op(base_of(ropeq->src[0]), GGML_OP_MUL_MAT);
+    const ggml_tensor * mmk = with_op(base_of(ropek->src[0]), GGML_OP_MUL_MAT);
+    const ggml_tensor * kqv = nullptr; const ggml_tensor * cont = nullptr; const ggml_tensor * mmo = nullptr; const ggml_tensor * addr = nullptr;
+    for (const PendingNode & p : win) {
+        if (!still_valid(p)) continue;
+        if (p.t->op == GGML_OP_MUL_MAT && p.t->src[1] == sm) kqv = p.t;
+    }
+    if (!mmq || !mmk || !kqv) return false;
+    for (const PendingNode & p : win) {
+        if (!still_valid(p)) continue;
+        if (p.t->op == GGML_OP_CONT && base_of(p.t->src[0]) == kqv) cont = p.t;
+    }
+    if (!cont) return false;
+    for (const PendingNode & p : win) {
+        if (!still_valid(p)) continue;
+        if (p.t->op == GGML_OP_MUL_MAT && p.t->src[1] == cont) mmo = p.t;
+    }
+    if (!mmo) return false;
+    for (const PendingNode & p : win) {
+        if (!still_valid(p)) continue;
+        if (p.t->op == GGML_OP_ADD && p.t->src[0] == mmo) addr = p.t;
+    }
+    const ggml_tensor * vview = kqv->src[0];
+    const ggml_tensor * vcpy = vview ? with_op(vview->src[1], GGML_OP_CPY) : nullptr;
+    const ggml_tensor * mmv = vcpy ? with_op(base_of(vcpy->src[0]), GGML_OP_MUL_MAT) : nullptr;
+    if (!mmv || vview->op != GGML_OP_VIEW) return false;
+    const ggml_tensor * X = mmq->src[1];
+    if (mmk->src[1] != X || mmv->src[1] != X) return false;
+    // the projections' input: norm(F) * w with both nodes in the window (the norm becomes the projections' prologue), or a vector
+    // that exists (the first layer's norm reads the embedding from the host and has run already)
+    const ggml_tensor * mulw = with_op(X, GGML_OP_MUL);
+    const ggml_tensor * nrm = mulw ? in_win(mulw->src[0]) : nullptr;
+    const ggml_tensor * F = X;
+    if (mulw) {
+        if (!nrm || (nrm->op != GGML_OP_RMS_NORM) || !on_device(mulw->src[1]) || in_win(mulw->src[1])) return false;
+        F = nrm->src[0];
+    } else if (in_win(X)) return false;
+    if (!F || !on_device(F) || in_win(F)) return false;
+    // 3 projections, 2 rope, 2 cpy, kq, scale, add, soft-max, kqv, cont, wo; the norm's two nodes and the residual add where they are pending
+    if (live != (size_t)(14 + (mulw ? 2 : 0) + (addr ? 1 : 0))) return false;
+    // ---- shapes, types, layouts ----
+    const ggml_tensor * wq = mmq->src[0]; const ggml_tensor * wk = mmk->src[0]; const ggml_tensor * wv = mmv->src[0]; const ggml_tensor * wo = mmo->src[0];
+    if (!weight_on_device(wq) || !weight_on_device(wk) || !weight_on_device(wv) || !weight_on_device(wo)) return false;
+    if (wq->type != GGML_TYPE_F16 || wk->type != GGML_TYPE_F16 || wv->type != GGML_TYPE_F16) return false;
+    const int d = (int)wq->ne[0];
+    if ((d != 4096 && d != 5120 && d != 8192) || wk->ne[0] != d || wv->ne[0] != d || F->ne[0] != d || !vec1(F)) return false;
+    const int hd = (int)ropeq->ne[0], n_head = (int)ropeq->ne[1], n_head_kv = (int)ropek->ne[1], gqa = n_head_kv * hd;
+    if (ropeq->ne[2] != 1 || ropek->ne[2] != 1 || ropek->ne[0] != hd || wq->ne[1] != (int64_t)n_head * hd || wk->ne[1] != gqa || wv->ne[1] != gqa || n_head_kv <= 0 || n_head % n_head_kv) return false;
+    if (wo->ne[0] != (int64_t)n_head * hd || nelem(cont) != (int64_t)n_head * hd) return false;
+    if (memcmp(ropeq->op_params, ropek->op_params, sizeof(int32_t) * 11) != 0 || ropeq->src[1] != ropek->src[1]) return false;
+    const int n_dims = ropeq->op_params[1], mode = ropeq->op_params[2];
+    float freq_base, freq_scale, ext_factor, attn_factor;
+    memcpy(&freq_base, ropeq->op_params + 5, 4); memcpy(&freq_scale, ropeq->op_params + 6, 4); memcpy(&ext_factor, ropeq->op_params + 7, 4); memcpy(&attn_factor, ropeq->op_params + 8, 4);
+    const ggml_tensor * pos = ropeq->src[1];
+    if (n_dims != hd || (mode != 0 && mode != 2) || ext_factor != 0.0f || !pos || pos->type != GGML_TYPE_I32 || !on_device(pos) || in_win(pos)) return false;
+    // K cells [cell][gqa], V transposed [gqa][n_ctx]; the copies' destinations name the cell
+    if (kview->type != GGML_TYPE_F16 || vview->type != GGML_TYPE_F16 || !on_device(kview) || !on_device(vview)) return false;
+    const int n_kv = (int)kview->ne[1];
+    if (kview->ne[0] != hd || kview->ne[2] != n_head_kv || kview->nb[0] != 2 || kview->nb[1] != (size_t)gqa * 2 || kview->nb[2] != (size_t)hd * 2) return false;
+    if (vview->ne[0] != n_kv || vview->ne[1] != hd || vview->ne[2] != n_head_kv || vview->nb[0] != 2 || vview->nb[1] % 2 || vview->nb[2] != vview->nb[1] * hd) return false;
+    const int n_ctx = (int)(vview->nb[1] / 2);
+    const ggml_tensor * kdst = kcpy->src[1]; const ggml_tensor * vdst = vcpy->src[1];
+    if (!kdst || !vdst || kdst->type != GGML_TYPE_F16 || vdst->type != GGML_TYPE_F16 || !on_device(kdst) || !on_device(vdst) || nelem(kdst) != gqa || nelem(vdst) != gqa) return false;
+    const ptrdiff_t koff = (char *)dev_ptr(kdst) - (char *)dev_ptr(kview), voff = (char *)dev_ptr(vdst) - (char *)dev_ptr(vview);
+    if (koff < 0 || koff % ((ptrdiff_t)gqa * 2) || voff < 0 || voff % 2) return false;
+    const int cell = (int)(koff / ((ptrdiff_t)gqa * 2));
+    if (cell >= n_kv || voff / 2 != cell || vdst->ne[0] != 1 || vdst->nb[1] != vview->nb[1] || !contiguous(kdst)) return false;
+    if (!pi_k_attn_ggml_supported(hd, n_ctx, n_kv)) return false;
+    if (!mask || mask->type != GGML_TYPE_F32 || !on_device(mask) || in_win(mask) || mask->ne[0] != n_kv || nrows(mask) != 1 || !contiguous(mask)) return false;
+    if (!kq_scale || kq_scale->type != GGML_TYPE_F32 || !on_device(kq_scale) || in_win(kq_scale) || nelem(kq_scale) != 1) return false;
+    if (kq->ne[0] != n_kv || kq->ne[2] != n_head || kqv->ne[0] != hd || kqv->ne[2] != n_head) return false;
+    const ggml_tensor * resid = addr ? addr->src[1] : nullptr;
+    if (addr && (!vec1(resid) || !on_device(resid) || in_win(resid) || nelem(resid) != wo->ne[1] || dev_ptr(resid) == dev_ptr(cont))) return false;
+    if ((((uintptr_t)dev_ptr(F) | (uintptr_t)(mulw ? dev_ptr(mulw->src[1]) : nullptr) | (uintptr_t)dev_ptr(kview) | (uintptr_t)dev_ptr(vview)) & 15) != 0) return false;
+    // ---- run ----
+    ++g_stats.attn_blocks_fused;
+    static float * qkv = nullptr;
+    static size_t qkv_n = 0;
+    const size_t need = (size_t)n_head * hd + 2 * (size_t)gqa;
+    if (need > qkv_n) {
+        if (qkv) { BK_PI(pi_sync()); pi_free(qkv); }
+        qkv = (float *)pi_malloc(sizeof(float) * need);
+        if (!qkv) die("attention buffer");
+        qkv_n = need;
+    }
+    pi_norm na{0, 0.0f, nullptr, nullptr};
+    if (mulw) { na.kind = 1; na.w = (const float *)dev_ptr(mulw->src[1]); memcpy(&na.eps, nrm->op_params, 4); }
+    const void * Ws[3] = {dev_ptr(wq), dev_ptr(wk), dev_ptr(wv)};
+    const int rows[3] = {n_head * hd, gqa, gqa};
+    float * ys[3] = {qkv, qkv + (size_t)n_head * hd, qkv + (size_t)n_head * hd + gqa};
+    BK_PI(pi_k_gemv_multi_f16(Ws, rows, 3, d, (const float *)dev_ptr(F), mulw ? &na : nullptr, ys, nullptr));
+    BK_PI(pi_k_attn_ggml(ys[0], ys[1], ys[2], (const int32_t *)dev_ptr(pos), mode, powf(freq_base, -2.0f / n_dims), freq_scale, attn_factor,
+                         dev_ptr(kview), dev_ptr(vview), n_head, n_head_kv, hd, n_ctx, n_kv, cell, (const float *)dev_ptr(kq_scale), (const float *)dev_ptr(mask),
+                         (float *)dev_ptr(cont), nullptr));
+    if (addr) BK_PI(pi_k_gemv(wo->type, dev_ptr(wo), (int)wo->ne[1], (int)wo->ne[0], (const float *)dev_ptr(cont), nullptr, PI_EPI_ADD, (const float *)dev_ptr(resid), nullptr,
+                              (float *)dev_ptr(addr), nullptr));
+    else      BK_PI(pi_k_gemv(wo->type, dev_ptr(wo), (int)wo->ne[1], (int)wo->ne[0], (const float *)dev_ptr(cont), nullptr, PI_EPI_NONE, nullptr, nullptr, (float *)dev_ptr(mmo), nullptr));
+    return true;
+}
+
+bool try_fused_ffn(const ggml_tensor * axpy, const ggml_tensor * add, bool axpy_pending, bool execute);
+
 // runs what is pending, in order.  Two peepholes: norm -> * w (-> + b) computed in place of one another is one launch, and a
 // mat-vec whose ReLU is computed in place of it takes the ReLU as its epilogue.
 void flush_pending() {
     if (g_pending.empty()) return;
     ++g_stats.windows_flushed;
+    {   // an FFN block whose AXPY node joined the window, with or without the residual add behind it
+        const ggml_tensor * axpy = nullptr; const ggml_tensor * add = nullptr;
+        for (const PendingNode & p : g_pending) {
+            if (!still_valid(p)) continue;
+            if (p.t->op == GGML_OP_AXPY) { axpy = p.t; add = nullptr; }
+            else if (axpy && !add && p.t->op == GGML_OP_ADD && p.t->src[0] == axpy) add = p.t;
+            else if (axpy) { axpy = nullptr; break; }                 // something else came behind it: no block
+        }
+        if (axpy && try_fused_ffn(axpy, add, true, true)) {
+            if (pi::check_launch("ggml_cuda_compute_forward") != PI_OK) die("kernel launch");
+            return;
+        }
+    }
     std::vector<PendingNode> win;
     win.swap(g_pending);
+    if (try_fused_attn(win)) return;
     for (size_t i = 0; i < win.size(); ++i) {
         if (!still_valid(win[i])) continue;
         ggml_tensor * n = win[i].t;
@@ -683,8 +891,10 @@ void flush_pending() {
 const PendingNode * find_pending(const ggml_tensor * t) { for (const PendingNode & p : g_pending) if (p.t == t && still_valid(p)) return &p; return nullptr; }
 
 // The AXPY node that closes llm_build_ffn_sparse's sequence with every neuron on the device.  Returns false (nothing done) unless the
-// pending window is exactly that block.
-bool try_fused_ffn(ggml_tensor * axpy) {
+// pending window is exactly that block.  The node is asked about twice: when it arrives (execute false: does the window before it
+// hold the block?  then it joins the window, so that the residual add behind it can follow), and when the window is flushed
+// (axpy_pending true, execute true; add: the pending node behind it that adds the residual to its result, or null).
+bool try_fused_ffn(const ggml_tensor * axpy, const ggml_tensor * add, bool axpy_pending, bool execute) {
     const ggml_tensor * down = axpy->src[0]; const ggml_tensor * cur = axpy->src[1]; const ggml_tensor * idx = axpy->src[2];
     if (axpy->src[3] != nullptr || !idx || !cur || !weight_on_device(down) || down->type != GGML_TYPE_F16 || !vec1(axpy) || axpy->backend != GGML_BACKEND_GPU || !on_device(axpy)) return false;
     size_t used = 0;
@@ -737,10 +947,13 @@ bool try_fused_ffn(ggml_tensor * axpy) {
     } else if (!on_device(X)) return false;
     size_t live = 0;
     for (const PendingNode & p : g_pending) live += still_valid(p) ? 1 : 0;
-    if (used != live) return false;                       // something else is pending: not the block
+    if (used + (axpy_pending ? 1 : 0) + (add ? 1 : 0) != live) return false;                       // something else is pending: not the block
+    const ggml_tensor * resid = add ? add->src[1] : nullptr;
+    if (add && (add->src[0] != axpy || !vec1(add) || !on_device(add) || !vec1(resid) || !on_device(resid) || is_pending(resid) || nelem(resid) != nelem(axpy))) return false;
     const int d = (int)down->ne[0], ff = (int)down->ne[1], r = (int)fc1->ne[1];
     if (up->ne[0] != d || up->ne[1] != ff || (gate && (gate->ne[0] != d || gate->ne[1] != ff)) || fc2->ne[0] != r || fc2->ne[1] != ff || fc1->ne[0] != P->ne[0] ||
         X->ne[0] != d || idx->ne[0] != ff || axpy->ne[0] != d || !pi_k_sparse_ffn_supported(ff, r, d)) return false;
+    if (!execute) return true;
     g_pending.clear();
     ++g_stats.ffn_blocks_fused;
     pi_workspace * ws = workspace(ff, d);
@@ -756,7 +969,8 @@ bool try_fused_ffn(ggml_tensor * axpy) {
     }
     BK_PI(pi_k_gemv(fc1->type, dev_ptr(fc1), r, (int)fc1->ne[0], (const float *)dev_ptr(P), nullptr, PI_EPI_RELU, nullptr, nullptr, hidden, nullptr));
     BK_PI(pi_k_sparse_ffn(dev_ptr(fc2), ff, r, hidden, g_threshold, dev_ptr(up), gate ? dev_ptr(gate) : nullptr, dev_ptr(down), d, (const float *)dev_ptr(F),
-                          nrm.kind ? &nrm : nullptr, PI_EPI_NONE, nullptr, nullptr, (float *)dev_ptr(axpy), (float *)dev_ptr(idx), (float *)dev_ptr(cur), nullptr, ws, nullptr));
+                          nrm.kind ? &nrm : nullptr, add ? PI_EPI_ADD : PI_EPI_NONE, add ? (const float *)dev_ptr(resid) : nullptr, nullptr,
+                          (float *)dev_ptr(add ? add : axpy), (float *)dev_ptr(idx), (float *)dev_ptr(cur), nullptr, ws, nullptr));
     return true;
 }
 
@@ -846,7 +1060,7 @@ void ggml_cuda_free_scratch(void) {
 }
 void ggml_cuda_copy_to_device(struct ggml_tensor * tensor) {
     flush_pending();
-    BK_PI(pi_memcpy_h2d(dev_ptr(tensor), tensor->data, nbytes(tensor)));
+    h2d(dev_ptr(tensor), tensor->data, nbytes(tensor));
 }
 void ggml_cuda_copy_to_host(struct ggml_tensor * tensor) {
     flush_pending();
@@ -898,10 +1112,9 @@ bool ggml_cuda_compute_forward(struct ggml_compute_params * params, struct ggml_
     if (!view) {                                         // views do nothing and neither join nor break the window
         if (deferrable(tensor)) { defer(tensor); return true; }
         if (!g_pending.empty()) {
-            if (tensor->op == GGML_OP_AXPY && try_fused_ffn(tensor)) {
-                if (pi::check_launch("ggml_cuda_compute_forward") != PI_OK) die("kernel launch");
-                return true;
-            }
+            // the AXPY node that completes an FFN block joins the window: the block runs when the window is flushed, with the residual
+            // add as its epilogue if that is what comes next
+            if (g_fuse && tensor->op == GGML_OP_AXPY && try_fused_ffn(tensor, nullptr, false, false)) { defer(tensor); return true; }
             flush_pending();
             if (deferrable(tensor)) { defer(tensor); return true; }      // its operands exist now: it may open the next window
         }

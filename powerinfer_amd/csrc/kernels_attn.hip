@@ -681,6 +681,150 @@ __global__ __launch_bounds__(kBlock) void attn_chunk_mfma_kernel(const float * _
     }
 }
 
+// ---------------------------------------------------------------------------------------------------
+// One token's attention on the layouts of the reference's own KV cache (llm_build_kv_store / llm_build_kqv, llama.cpp:4383-4418,
+// 4764-4850): K cells [cell][n_head_kv * hd] fp16, V transposed [n_head_kv * hd][n_ctx] fp16.  What its graph spreads over eleven nodes
+// - RoPE of q and k, the two copies into the cache, K.q, scale, + mask, soft-max, V.p and the gather of the heads - is one launch, one
+// workgroup per query head, with the CPU path's rounding points: q and p rounded to fp16 in front of their products (the mat-muls
+// against fp16 operands, ggml.c:9703-9716), exp through fp16 on both sides (ggml.c:10747-10759), the sum of the exponentials in double.
+// The new cell's K and V rows are used from LDS (every head of a group computes them, the group's first head stores them), so no
+// workgroup depends on another's stores.  Cells whose mask entry is -inf get probability 0 whatever the cache holds there.
+// RoPE as rope_kernel of the boundary computes it: angle advanced by repeated fp32 multiplication, cosf / sinf, * mscale.
+// ---------------------------------------------------------------------------------------------------
+__global__ __launch_bounds__(kBlock) void attn_ggml_kernel(const float * __restrict__ q, const float * __restrict__ k, const float * __restrict__ v,
+                                                           const int32_t * __restrict__ pos, int mode, float theta_scale, float freq_scale, float mscale,
+                                                           __half * __restrict__ k_cache, __half * __restrict__ v_cache,
+                                                           int n_head, int n_head_kv, int hd, int n_ctx, int n_kv, int cell,
+                                                           const float * __restrict__ kq_scale, const float * __restrict__ kq_mask, float * __restrict__ out) {
+    extern __shared__ __align__(16) unsigned char smem[];
+    const int n_kv8 = (n_kv + 7) & ~7;                                     // the V rows are read eight cells at a time
+    float * sc = reinterpret_cast<float *>(smem);                          // [n_kv8] scores, then probabilities (zeros behind n_kv)
+    __half * q16 = reinterpret_cast<__half *>(sc + n_kv8);                 // [hd] each
+    __half * k16 = q16 + hd;
+    __half * v16 = k16 + hd;
+    __shared__ double red[kWavesPerBlock];
+    __shared__ float  redf[kWavesPerBlock];
+    const int h = blockIdx.x, kvh = h / (n_head / n_head_kv), gqa = n_head_kv * hd;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    const bool owner = h % (n_head / n_head_kv) == 0;                      // this head's workgroup stores the group's new K / V rows
+    if (tid < hd / 2) {
+        const int i = tid;
+        float theta = (float)pos[0];
+        if (mode & 2) theta = __fmul_rn(theta, freq_scale);
+        for (int j = 0; j < i; ++j) theta = __fmul_rn(theta, theta_scale);
+        const float th = __fmul_rn(freq_scale, theta);
+        const float c = __fmul_rn(cosf(th), mscale), sn = __fmul_rn(sinf(th), mscale);
+        const int i0 = (mode & 2) ? i : 2 * i, i1 = (mode & 2) ? i + hd / 2 : 2 * i + 1;
+        const float q0 = q[h * hd + i0], q1 = q[h * hd + i1];
+        q16[i0] = __float2half_rn(__fsub_rn(__fmul_rn(q0, c), __fmul_rn(q1, sn)));
+        q16[i1] = __float2half_rn(__fadd_rn(__fmul_rn(q0, sn), __fmul_rn(q1, c)));
+        const float k0 = k[kvh * hd + i0], k1 = k[kvh * hd + i1];
+        const __half r0 = __float2half_rn(__fsub_rn(__fmul_rn(k0, c), __fmul_rn(k1, sn)));
+        const __half r1 = __float2half_rn(__fadd_rn(__fmul_rn(k0, sn), __fmul_rn(k1, c)));
+        k16[i0] = r0; k16[i1] = r1;
+        if (owner) { k_cache[(size_t)cell * gqa + kvh * hd + i0] = r0; k_cache[(size_t)cell * gqa + kvh * hd + i1] = r1; }
+    }
+    if (tid < hd) {
+        const __half r = __float2half_rn(v[kvh * hd + tid]);
+        v16[tid] = r;
+        if (owner) v_cache[(size_t)(kvh * hd + tid) * n_ctx + cell] = r;
+    }
+    __syncthreads();
+
+    // ---- scores: hd / 8 lanes per cell, 16 bytes of the cell's row each; four cells' rows in flight per lane -----------------
+    const int lpc = hd / 8, cpw = PI_WAVE / lpc;                          // lanes per cell, cells per wave and pass
+    const int sub = lane / lpc, l = lane % lpc;
+    const pi_u32x4 qv = *reinterpret_cast<const pi_u32x4 *>(q16 + l * 8);
+    const float scale = kq_scale[0];
+    constexpr int SU = 4;
+    const int cstep = kWavesPerBlock * cpw;
+    for (int c0 = wave * cpw + sub; c0 < n_kv; c0 += SU * cstep) {
+        pi_u32x4 kr[SU];
+        float m[SU];
+#pragma unroll
+        for (int u = 0; u < SU; ++u) {
+            const int c = c0 + u * cstep;
+            const int cc = c < n_kv ? c : n_kv - 1;                          // (clamped requests keep the loads unconditional)
+            m[u] = kq_mask[cc];
+            kr[u] = pi_ld16(k_cache + (size_t)cc * gqa + kvh * hd + l * 8);
+        }
+#pragma unroll
+        for (int u = 0; u < SU; ++u) {
+            const int c = c0 + u * cstep;
+            if (c == cell) kr[u] = *reinterpret_cast<const pi_u32x4 *>(k16 + l * 8);
+            float d = pi_dot8h(kr[u], qv, 0.0f);
+            for (int o = 1; o < lpc; o <<= 1) d += __shfl_xor(d, o, PI_WAVE);
+            if (c < n_kv && l == 0) sc[c] = m[u] == -INFINITY ? -INFINITY : __fadd_rn(__fmul_rn(d, scale), m[u]);
+        }
+    }
+    __syncthreads();
+    // ---- soft-max over the cells -------------------------------------------------------------------------------------------
+    float mx = -INFINITY;
+    for (int c = tid; c < n_kv; c += kBlock) mx = fmaxf(mx, sc[c]);
+    mx = pi_wave_max(mx);
+    if (lane == 0) redf[wave] = mx;
+    __syncthreads();
+    mx = redf[0];
+    for (int w = 1; w < kWavesPerBlock; ++w) mx = fmaxf(mx, redf[w]);
+    double sum = 0.0;
+    for (int c = tid; c < n_kv; c += kBlock) {
+        const float e = sc[c] == -INFINITY ? 0.0f : pi_round_f16(expf(pi_round_f16(__fsub_rn(sc[c], mx))));
+        sc[c] = e; sum += (double)e;
+    }
+    sum = pi_wave_sum_f64(sum);
+    if (lane == 0) red[wave] = sum;
+    __syncthreads();
+    double tot = 0.0;
+    for (int w = 0; w < kWavesPerBlock; ++w) tot += red[w];
+    const float inv = (float)(1.0 / tot);
+    for (int c = tid; c < n_kv8; c += kBlock) sc[c] = c < n_kv ? __fmul_rn(sc[c], inv) : 0.0f;
+    __syncthreads();
+    // ---- out[dim] = sum over cells of fp16(p[cell]) * V[dim][cell].  Thread t owns column t % hd and every (kBlock / hd)-th group of
+    // eight cells of it, four groups in flight; the column's partial sums meet in LDS (the scores' first floats are free by then
+    // only after everyone has read its probabilities, hence the barrier in between) ------------------------------------------------
+    {
+        const int dim = tid % hd, part = tid / hd, nparts = kBlock / hd;      // hd <= kBlock and divides it (the launcher's test)
+        const __half * vr = v_cache + (size_t)(kvh * hd + dim) * n_ctx;
+        const __half vn = v16[dim];
+        float acc = 0.0f;
+        constexpr int VU = 4;
+        for (int g0 = part; g0 * 8 < n_kv; g0 += VU * nparts) {
+            pi_u32x4 vv[VU];
+#pragma unroll
+            for (int u = 0; u < VU; ++u) {
+                const int c0 = (g0 + u * nparts) * 8;
+                vv[u] = pi_ld16(vr + (c0 < n_kv ? c0 : 0));
+            }
+#pragma unroll
+            for (int u = 0; u < VU; ++u) {
+                const int c0 = (g0 + u * nparts) * 8;
+                if (c0 < n_kv) {
+                    if (cell >= c0 && cell < c0 + 8) reinterpret_cast<__half *>(&vv[u])[cell - c0] = vn;
+                    const float4 p0 = *reinterpret_cast<const float4 *>(sc + c0), p1 = *reinterpret_cast<const float4 *>(sc + c0 + 4);
+                    __half2 ph[4] = {__floats2half2_rn(p0.x, p0.y), __floats2half2_rn(p0.z, p0.w), __floats2half2_rn(p1.x, p1.y), __floats2half2_rn(p1.z, p1.w)};
+                    // a cell without probability contributes nothing, whatever its (possibly never written) V entry holds
+                    const uint32_t * pw = reinterpret_cast<const uint32_t *>(ph);
+                    uint32_t * vw = reinterpret_cast<uint32_t *>(&vv[u]);
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) {
+                        if ((pw[j] & 0x0000ffffu) == 0u) vw[j] &= 0xffff0000u;
+                        if ((pw[j] & 0xffff0000u) == 0u) vw[j] &= 0x0000ffffu;
+                    }
+                    acc = pi_dot8h(vv[u], *reinterpret_cast<const pi_u32x4 *>(ph), acc);
+                }
+            }
+        }
+        float * pacc = reinterpret_cast<float *>(v16 + hd);                   // [kBlock] floats behind the three fp16 rows
+        pacc[tid] = acc;
+        __syncthreads();
+        if (tid < hd) {
+            float t = pacc[tid];
+            for (int w = 1; w < nparts; ++w) t += pacc[tid + w * hd];
+            out[h * hd + tid] = t;
+        }
+    }
+}
+
 }  // namespace
 
 extern "C" {
@@ -875,6 +1019,24 @@ int pi_k_attn_chunk_long(const float * qkv, int qkv_stride, int T, int n_head, i
                        (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, 0, n_ctx, s_cap, pos, acc, ml, n_head * hd, (size_t)0);
     hipLaunchKernelGGL(attn_merge_kernel, dim3(n_head, T), dim3(hd), 0, st, acc, ml, n_parts, hd, out, n_head * hd, (__half *)out_f16);
     return pi::check_launch("pi_k_attn_chunk_long");
+}
+
+int pi_k_attn_ggml_supported(int hd, int n_ctx, int n_kv) {
+    return hd > 0 && hd % 8 == 0 && hd <= kBlock && kBlock % hd == 0 && PI_WAVE % (hd / 8) == 0 && n_kv > 0 && n_ctx % 8 == 0 && n_kv <= n_ctx &&
+           sizeof(float) * (size_t)((n_kv + 7) & ~7) + 6 * (size_t)hd + sizeof(float) * kBlock <= 60 * 1024;
+}
+
+int pi_k_attn_ggml(const float * q, const float * k, const float * v, const int32_t * pos, int mode, float theta_scale, float freq_scale, float mscale,
+                   void * k_cache, void * v_cache, int n_head, int n_head_kv, int hd, int n_ctx, int n_kv, int cell,
+                   const float * kq_scale, const float * kq_mask, float * out, pi_stream_t stream) {
+    if (!q || !k || !v || !pos || !k_cache || !v_cache || !kq_scale || !kq_mask || !out) return pi::fail(PI_E_ARG, "pi_k_attn_ggml: null pointer");
+    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || (mode != 0 && mode != 2) || cell < 0 || cell >= n_kv || !pi_k_attn_ggml_supported(hd, n_ctx, n_kv))
+        return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_ggml: head geometry, cell or context outside the kernel (pi_k_attn_ggml_supported)");
+    if ((((uintptr_t)k_cache | (uintptr_t)v_cache) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_attn_ggml: the caches must be 16-byte aligned");
+    const size_t sh = sizeof(float) * (size_t)((n_kv + 7) & ~7) + 6 * (size_t)hd + sizeof(float) * kBlock;
+    hipLaunchKernelGGL(attn_ggml_kernel, dim3(n_head), dim3(kBlock), sh, (hipStream_t)stream, q, k, v, pos, mode, theta_scale, freq_scale, mscale,
+                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, n_ctx, n_kv, cell, kq_scale, kq_mask, out);
+    return pi::check_launch("pi_k_attn_ggml");
 }
 
 int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float theta_scale, float freq_scale, const int32_t * delta, int n_cells, pi_stream_t stream) {

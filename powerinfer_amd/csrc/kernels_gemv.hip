@@ -89,12 +89,29 @@ __global__ __launch_bounds__(kBlock) void gemv_f16_kernel(const __half * __restr
 // 16 weight loads of 16 B per lane are in flight throughout (two rows, or the two halves of a wide row) and
 // are issued before the prologue starts.  The residual operands of the epilogue travel with the row.
 // KIND: 0 no norm, 1 RMSNorm * w, 2 LayerNorm * w + b.  TAG only names the role in kernel traces.
-template <int NCH, int KIND, int TAG>
-__global__ __launch_bounds__(kBlock, 2) void gemv_f16_reg_kernel(const __half * __restrict__ W, const float * __restrict__ x,
-                                                              const float * __restrict__ nw, const float * __restrict__ nb, float eps,
-                                                              int epi, const float * __restrict__ add1, const float * __restrict__ add2,
-                                                              float * __restrict__ y, int rows) {
+// MULTI: up to three matrices of the same width against the one vector in a single launch (the q, k and v projections of a host
+// that keeps them as separate tensors): row r of the launch is row r of the first matrix, or row r - rows[0] of the second, ...
+struct GemvMulti { const __half * W[3]; float * y[3]; int rows[3]; };
+template <int NCH, int KIND, bool MULTI>
+__device__ __forceinline__ void gemv_f16_reg_body(const __half * __restrict__ W, const float * __restrict__ x,
+                                                  const float * __restrict__ nw, const float * __restrict__ nb, float eps,
+                                                  int epi, const float * __restrict__ add1, const float * __restrict__ add2,
+                                                  float * __restrict__ y, int rows, const GemvMulti & mm) {
     constexpr int cols = NCH * 512;
+    auto row_base = [&](int r) -> const __half * {
+        if (!MULTI) return W + (size_t)r * cols;
+        if (r < mm.rows[0]) return mm.W[0] + (size_t)r * cols;
+        r -= mm.rows[0];
+        if (r < mm.rows[1]) return mm.W[1] + (size_t)r * cols;
+        return mm.W[2] + (size_t)(r - mm.rows[1]) * cols;
+    };
+    auto out_ptr = [&](int r) -> float * {
+        if (!MULTI) return y + r;
+        if (r < mm.rows[0]) return mm.y[0] + r;
+        r -= mm.rows[0];
+        if (r < mm.rows[1]) return mm.y[1] + r;
+        return mm.y[2] + (r - mm.rows[1]);
+    };
     constexpr bool kWide = NCH > 8;               // wide rows: the two buffers hold the halves of one row
     constexpr int CPB = kWide ? NCH / 2 : NCH;
     static_assert(!kWide || NCH % 2 == 0, "wide rows are split in two halves");
@@ -107,7 +124,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemv_f16_reg_kernel(const __half * 
     float r1[2] = {0.0f, 0.0f}, r2[2] = {0.0f, 0.0f};
     auto issue = [&](int b, int r) {
         if (r < rows) {
-            const __half * wp = W + (size_t)r * cols + lane * 8 + (kWide ? b * CPB * 512 : 0);
+            const __half * wp = row_base(r) + lane * 8 + (kWide ? b * CPB * 512 : 0);
 #pragma unroll
             for (int j = 0; j < CPB; ++j) buf[b][j] = pi_ld_stream(wp + j * 512);
             if (!kWide || b == 0) {
@@ -200,7 +217,7 @@ __global__ __launch_bounds__(kBlock, 2) void gemv_f16_reg_kernel(const __half * 
         if (epi == PI_EPI_RELU) acc = fmaxf(acc, 0.0f);
         else if (epi == PI_EPI_ADD) acc = __fadd_rn(acc, a1);
         else if (epi == PI_EPI_ADD2) acc = __fadd_rn(__fadd_rn(acc, a1), a2);
-        if (lane == 0) y[r] = acc;
+        if (lane == 0) *out_ptr(r) = acc;
     };
     if constexpr (kWide) {
         for (int r = wid; r < rows; r += n_waves) {
@@ -232,6 +249,19 @@ __global__ __launch_bounds__(kBlock, 2) void gemv_f16_reg_kernel(const __half * 
             }
         }
     }
+}
+
+template <int NCH, int KIND, int TAG>
+__global__ __launch_bounds__(kBlock, 2) void gemv_f16_reg_kernel(const __half * __restrict__ W, const float * __restrict__ x,
+                                                              const float * __restrict__ nw, const float * __restrict__ nb, float eps,
+                                                              int epi, const float * __restrict__ add1, const float * __restrict__ add2,
+                                                              float * __restrict__ y, int rows) {
+    gemv_f16_reg_body<NCH, KIND, false>(W, x, nw, nb, eps, epi, add1, add2, y, rows, GemvMulti{});
+}
+template <int NCH, int KIND>
+__global__ __launch_bounds__(kBlock, 2) void gemv_multi_f16_reg_kernel(GemvMulti mm, const float * __restrict__ x,
+                                                                    const float * __restrict__ nw, const float * __restrict__ nb, float eps, int rows) {
+    gemv_f16_reg_body<NCH, KIND, true>(nullptr, x, nw, nb, eps, PI_EPI_NONE, nullptr, nullptr, nullptr, rows, mm);
 }
 
 // ---------------------------------------------------------------------------------------------------
@@ -658,6 +688,32 @@ int pi_k_gemv(int wtype, const void * W, int rows, int cols, const float * x, co
         return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv: weight type must be F16 or Q4_0");
     }
     return pi::check_launch("pi_k_gemv");
+}
+
+int pi_k_gemv_multi_f16(const void * const * W, const int * rows, int n_mat, int cols, const float * x, const pi_norm * norm, float * const * y,
+                        pi_stream_t stream) {
+    if (!W || !rows || !y || !x || n_mat < 1 || n_mat > 3) return pi::fail(PI_E_ARG, "pi_k_gemv_multi_f16: one to three matrices");
+    const NormArgs na = to_norm(norm);
+    GemvMulti mm{};
+    int total = 0;
+    for (int i = 0; i < 3; ++i) {
+        if (i < n_mat) {
+            if (!W[i] || !y[i] || rows[i] <= 0) return pi::fail(PI_E_ARG, "pi_k_gemv_multi_f16: null matrix or result, or no rows");
+            mm.W[i] = (const __half *)W[i]; mm.y[i] = y[i]; mm.rows[i] = rows[i]; total += rows[i];
+        }
+    }
+    const bool aligned = (((uintptr_t)x | (uintptr_t)na.w | (uintptr_t)na.b) & 15) == 0;
+    if (!aligned || (cols != 4096 && cols != 5120 && cols != 8192) || !(na.kind == 0 || (na.kind == 1 && na.w && !na.b) || (na.kind == 2 && na.w && na.b)))
+        return pi::fail(PI_E_UNSUPPORTED, "pi_k_gemv_multi_f16: cols 4096, 5120 or 8192, 16-byte aligned vectors, a norm that carries its weights");
+    hipStream_t st = (hipStream_t)stream;
+    const int n_waves = kGemvBlocks * kWavesPerBlock;
+    const int rblocks = total >= n_waves ? kGemvBlocks : (total + kWavesPerBlock - 1) / kWavesPerBlock;
+#define PI_GEMV_M(NCH, KIND) hipLaunchKernelGGL((gemv_multi_f16_reg_kernel<NCH, KIND>), dim3(rblocks), dim3(kBlock), 0, st, mm, x, na.w, na.b, na.eps, total)
+#define PI_GEMV_M_N(NCH) do { if (na.kind == 0) PI_GEMV_M(NCH, 0); else if (na.kind == 1) PI_GEMV_M(NCH, 1); else PI_GEMV_M(NCH, 2); } while (0)
+    if (cols == 4096) PI_GEMV_M_N(8); else if (cols == 5120) PI_GEMV_M_N(10); else PI_GEMV_M_N(16);
+#undef PI_GEMV_M_N
+#undef PI_GEMV_M
+    return pi::check_launch("pi_k_gemv_multi_f16");
 }
 
 int pi_k_embed_batch_q4(const void * table_q4, int cols, const int32_t * tokens, int T, float * x, pi_stream_t stream) {

@@ -138,3 +138,58 @@ def test_reference_multi_sequence_kv_cells_on_this_backend(tmp_path):
         err = np.abs(got - want).max(1) / np.abs(want).max(1)
         assert err.max() < 1e-2, err
         assert np.array_equal(got.argmax(1), want.argmax(1))
+
+
+def run_binary(exe, path, n_ctx, toks, n_gen, out, env):
+    r = subprocess.run([exe, path, str(n_ctx), "1", str(n_gen), out] + [str(int(t)) for t in toks], env=env, capture_output=True, text=True, timeout=280)
+    log = r.stdout + r.stderr
+    assert r.returncode == 0, log[-3000:]
+    raw = np.fromfile(out, np.uint8)
+    n_steps, n_vocab = (int(v) for v in raw[:8].view(np.int32))
+    rec = raw[8:].reshape(n_steps, 8 + 4 * n_vocab)
+    stats = {}
+    for line in log.splitlines():
+        if line.startswith("backend_stats"):
+            w = line.split()
+            stats = {w[i]: int(w[i + 1]) for i in range(1, len(w), 2)}
+    return rec[:, 4:8].copy().view(np.int32)[:, 0], rec[:, 8:].copy().view(np.float32), stats
+
+
+@pytest.mark.timeout(300)
+def test_reference_llama_cpp_at_7b_width_runs_as_fused_blocks(tmp_path):
+    """Two 7B-wide layers through the reference's own llama.cpp on this backend: every token's attention block (norm, three
+    projections, two RoPEs, two cache copies, K.q, scale, mask, soft-max, V.p, gather, output projection, residual: 17 graph nodes)
+    must have run as three launches and every FFN block as two, and the logits must be those of the reference's CPU-only run of
+    the same file, and those of this backend with one launch per node (GGML_CUDA_NO_FUSION=1).  The model keeps margins
+    (predictor_fc2_margin, head_pair), so the greedy continuations of the three runs are the same tokens."""
+    from powerinfer_amd import synth
+    cpu = os.path.join(ROOT, "oracle", "_ref", "ref_llama")
+    if not os.path.exists(BIN) or not os.path.exists(cpu):
+        pytest.skip("oracle/_ref/ref_llama(_gpu) are not built (they need the reference sources at build time)")
+    hp = synth.hparams("llama-7b", n_layer=2, n_ctx=128, seed=35, pred_margin=True, head_pair=2048)
+    model = synth.make_model(hp)
+    path = str(tmp_path / "m.powerinfer.gguf")
+    gguf.write_model(path, model, gguf.synthetic_tokenizer_kv(hp.n_vocab))
+    splits = [(np.ones(hp.n_ff, np.int32), np.arange(hp.n_ff, dtype=np.int32)) for _ in range(hp.n_layer)]
+    split.write_gpuidx(path + ".generated.gpuidx", splits, split.required_bytes(hp, splits))
+    del model
+    toks = np.random.default_rng(42).integers(0, hp.n_vocab, 6)
+    n_gen = 40                      # 46 steps: from the 33rd on the number of attended cells is no multiple of 8 or 32
+    env = dict(os.environ, REF_VRAM_GB="16")
+    g_f, l_f, st_f = run_binary(BIN, path, hp.n_ctx, toks, n_gen, str(tmp_path / "f.bin"), env)
+    g_n, l_n, st_n = run_binary(BIN, path, hp.n_ctx, toks, n_gen, str(tmp_path / "n.bin"), dict(env, GGML_CUDA_NO_FUSION="1"))
+    os.remove(path + ".generated.gpuidx")                       # the CPU build loads the same file without a split
+    g_c, l_c, _ = run_binary(cpu, path, hp.n_ctx, toks, n_gen, str(tmp_path / "c.bin"), dict(os.environ))
+    n_steps = len(toks) + n_gen
+    assert st_f["attn_fused"] == hp.n_layer * n_steps and st_f["ffn_fused"] == hp.n_layer * n_steps, st_f
+    assert st_n["attn_fused"] == 0 and st_n["ffn_fused"] == 0 and st_n["deferred"] == 0, st_n
+    assert np.array_equal(g_f, g_c) and np.array_equal(g_n, g_c), (g_f, g_n, g_c)
+    scale = np.abs(l_c).max(1)
+    e_fc = np.abs(l_f - l_c).max(1) / scale
+    e_nc = np.abs(l_n - l_c).max(1) / scale
+    e_fn = np.abs(l_f - l_n).max(1) / scale
+    # the north star's logits tolerance on every step, for both arrangements against the CPU and against each other (another order
+    # of the sums in the attention and the projections; what is left grows with the number of cached cells)
+    assert e_fc.max() < 1e-2 and np.median(e_fc) < 2e-3, e_fc
+    assert e_nc.max() < 1e-2 and np.median(e_nc) < 2e-3, e_nc
+    assert e_fn.max() < 1e-2 and np.median(e_fn) < 2e-3, e_fn

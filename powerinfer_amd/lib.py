@@ -49,6 +49,7 @@ _SIGS = {
     "pi_event_elapsed_ms": (_i, [_vp, _vp, C.POINTER(_f)]),
     "pi_event_destroy": (_i, [_vp]),
     "pi_k_gemv": (_i, [_i, _vp, _i, _i, _vp, C.POINTER(Norm), _i, _vp, _vp, _vp, _vp]),
+    "pi_k_gemv_multi_f16": (_i, [_vp, _vp, _i, _i, _vp, C.POINTER(Norm), _vp, _vp]),
     "pi_workspace_create": (_vp, [_i, _i]),
     "pi_workspace_destroy": (_i, [_vp]),
     "pi_k_predictor_fc2": (_i, [_vp, _i, _i, _vp, _f, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
@@ -107,6 +108,8 @@ _SIGS = {
     "pi_k_batch_sparse_mul_mat": (_i, [_vp, _i, _i, _vp, _i, _vp, _f, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_batch_sparse_axpy": (_i, [_vp, _i, _i, _vp, _vp, _i, _f, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_attn_split_supported": (_i, [_i, _i, _i]),
+    "pi_k_attn_ggml_supported": (_i, [_i, _i, _i]),
+    "pi_k_attn_ggml": (_i, [_vp, _vp, _vp, _vp, _i, _f, _f, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
     "pi_k_attn_split_scratch_floats": (_sz, [_i, _i, _i, _i]),
     "pi_k_attn_split": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _vp, _vp]),
     "pi_k_attn_chunk_supported": (_i, [_i, _i, _i]),

@@ -328,6 +328,74 @@ def test_attention_split_over_cells(mode, hd, nh, nkv, n_ctx, parts):
     assert L.pi_k_attn_split_supported(hd, n_ctx, 65) == 0 and L.pi_k_attn_split_supported(24, n_ctx, parts) == 0
 
 
+@pytest.mark.parametrize("cols,kind", [(4096, 1), (5120, 0), (8192, 2)])
+def test_gemv_of_three_matrices_in_one_launch(cols, kind):
+    """pi_k_gemv_multi_f16: the q, k and v projections of a host that keeps them as three tensors, one launch against one normalised
+    vector.  Every product is bit for bit the one pi_k_gemv computes for that matrix alone."""
+    import ctypes as C
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    rng = np.random.default_rng(cols + kind)
+    rows = [cols, 1024, 520]
+    Ws = [pl.DevBuf(host=(rng.standard_normal((r, cols)) * 0.02).astype(np.float16)) for r in rows]
+    x = pl.DevBuf(host=rng.standard_normal(cols).astype(np.float32))
+    nw = pl.DevBuf(host=(1 + 0.1 * rng.standard_normal(cols)).astype(np.float32)) if kind else None
+    nb = pl.DevBuf(host=(0.1 * rng.standard_normal(cols)).astype(np.float32)) if kind == 2 else None
+    nrm = pl.norm_arg(kind, 1e-5, nw, nb) if kind else None
+    ys = [pl.DevBuf(r * 4) for r in rows]
+    pl.check(L.pi_k_gemv_multi_f16((C.c_void_p * 3)(*[w.ptr for w in Ws]), (C.c_int * 3)(*rows), 3, cols, x.ptr, nrm, (C.c_void_p * 3)(*[y.ptr for y in ys]), None), "gemv_multi")
+    pl.sync()
+    for W, r, y in zip(Ws, rows, ys):
+        one = pl.DevBuf(r * 4)
+        pl.check(L.pi_k_gemv(pl.F16, W.ptr, r, cols, x.ptr, nrm, 0, None, None, one.ptr, None), "gemv")
+        pl.sync()
+        assert np.array_equal(y.download(np.float32), one.download(np.float32))
+    assert L.pi_k_gemv_multi_f16((C.c_void_p * 3)(*[w.ptr for w in Ws]), (C.c_int * 3)(*rows), 3, 4000, x.ptr, nrm, (C.c_void_p * 3)(*[y.ptr for y in ys]), None) != 0
+
+
+@pytest.mark.parametrize("mode,hd,nh,nkv", [(0, 128, 4, 4), (2, 64, 8, 2)])
+def test_attention_on_the_reference_cache_layouts(mode, hd, nh, nkv):
+    """pi_k_attn_ggml: one token's attention with K cells [cell][n_embd_gqa] and V transposed [n_embd_gqa][n_ctx], as the reference's
+    llm_build_kv_store / llm_build_kqv lay the cache out, RoPE and both cache stores included.  Forty tokens one after the other
+    against the oracle's rope + attention on the same layouts: outputs within 2e-3, the two caches identical up to the last bit of
+    the rotated K values; cells are handed out in a scrambled order and hidden cells carry -inf in the mask, as a ring with holes does;
+    the number of attended cells passes through values that are no multiple of 8."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    O = ol.oracle()
+    rng = np.random.default_rng(mode + hd)
+    n_ctx, gqa, d = 64, nkv * hd, nh * hd
+    assert L.pi_k_attn_ggml_supported(hd, n_ctx, 33) == 1 and L.pi_k_attn_ggml_supported(hd, 63, 33) == 0
+    kc_o, vc_o = np.zeros((n_ctx, gqa), np.uint16), np.zeros((gqa, n_ctx), np.uint16)
+    kc, vc = pl.DevBuf.zeros(n_ctx * gqa * 2), pl.DevBuf.zeros(n_ctx * gqa * 2)
+    theta_scale = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
+    scale = pl.DevBuf(host=np.array([1.0 / np.sqrt(hd)], np.float32))
+    cells = rng.permutation(40)                                  # token t lives in cell cells[t]
+    used = np.zeros(n_ctx, bool)
+    for t in range(40):
+        cell = int(cells[t])
+        used[cell] = True
+        n_kv = max(int(np.flatnonzero(used).max()) + 1, 5)       # cells up to the highest one in use are attended, the unused ones masked
+        q, k, v = (rng.standard_normal(n).astype(np.float32) for n in (d, gqa, gqa))
+        pos = np.array([t], np.int32)
+        mask = np.where(used[:n_kv], 0.0, -np.inf).astype(np.float32)
+        qr, kr = np.zeros_like(q), np.zeros_like(k)
+        O.pio_rope(P(q), hd, nh, 1, P(pos), hd, mode, 10000.0, 1.0, P(qr))
+        O.pio_rope(P(k), hd, nkv, 1, P(pos), hd, mode, 10000.0, 1.0, P(kr))
+        want = np.zeros(d, np.float32)
+        slot = np.array([cell], np.int32)
+        assert O.pio_attention(hd, nh, nkv, n_ctx, n_kv, 1, P(slot), P(mask), P(qr), P(kr), P(v), P(kc_o), P(vc_o), P(want)) == 0
+        dq, dk, dv, dpos, dmask, dout = pl.DevBuf(host=q), pl.DevBuf(host=k), pl.DevBuf(host=v), pl.DevBuf(host=pos), pl.DevBuf(host=mask), pl.DevBuf(d * 4)
+        pl.check(L.pi_k_attn_ggml(dq.ptr, dk.ptr, dv.ptr, dpos.ptr, mode, theta_scale, 1.0, 1.0, kc.ptr, vc.ptr, nh, nkv, hd, n_ctx, n_kv, cell,
+                                  scale.ptr, dmask.ptr, dout.ptr, None), "attn_ggml")
+        pl.sync()
+        assert rel_err(dout.download(np.float32), want) < 2e-3, (t, rel_err(dout.download(np.float32), want))
+    kg = kc.download(np.float16).reshape(n_ctx, gqa).astype(np.float32)
+    vg = vc.download(np.uint16).reshape(gqa, n_ctx)
+    assert np.array_equal(vg, vc_o)
+    assert np.abs(kg - kc_o.view(np.float16).astype(np.float32)).max() <= 2e-3 * np.abs(kg).max()
+
+
 def test_embed_and_argmax():
     from powerinfer_amd import lib as pl
     L = pl.init()

@@ -252,10 +252,13 @@ def bench_batched(args):
     n_seq = 16
     n_prompt = 512 if args.prompt == 64 else args.prompt
     steps = 128 if args.steps == 256 else args.steps
-    hp = synth.hparams("llama-13b", n_layer=40 if args.layers == 32 else args.layers, n_ctx=n_prompt + args.warmup + steps + 8, seed=1)
+    over = {} if args.mean_rate is None else {"mean_rate": args.mean_rate}
+    hp = synth.hparams("llama-13b", n_layer=40 if args.layers == 32 else args.layers, n_ctx=n_prompt + args.warmup + steps + 8, seed=1, **over)
     keep = []
     m = build_synthetic_on_device(hp, keep)
     m.batch_init(n_seq)
+    if args.dense_above is not None:
+        m.batch_set_dense_above(args.dense_above)
     rng = np.random.default_rng(2024)
     prompt = rng.integers(0, hp.n_vocab, (n_prompt, n_seq)).astype(np.int32)
     for s in range(n_prompt):                                   # prompt phase (not timed): one position of every sequence per step
@@ -280,7 +283,8 @@ def bench_batched(args):
                                f"{hp.n_layer} layers, random-init FP16 weights, all neurons on the GPU, {n_seq} sequences with {n_prompt}-token random "
                                "prompts, greedy decode in lockstep (one token per sequence per step)",
                    "n_layer": hp.n_layer, "n_seq": n_seq, "prompt_tokens": n_prompt, "n_ctx": hp.n_ctx,
-                   "mean_union_rows_per_layer": round(union.mean(), 1), "device": pl.device_name()},
+                   "mean_union_rows_per_layer": round(union.mean(), 1), "union_fraction": round(union.mean() / hp.n_ff, 3),
+                   "layers_run_dense": m.batch_dense_layers(), "device": pl.device_name()},
         "token_loop": {"device_ms_per_step": round(ms_dev / steps, 4), "touched_GB_per_step": round(step_bytes / 1e9, 3),
                        "effective_GBps": round(step_bytes / (ms_step * 1e-3) / 1e9, 1),
                        "hbm_frac_touched": round(step_bytes / (ms_step * 1e-3) / 1e9 / HBM_PEAK_GBPS, 4)},
@@ -306,6 +310,8 @@ def main():
                          "Q4_0 with the hottest 60 %% of neurons on the GPU and the rest on host threads; 3 ProSparse-LLaMA-2-13B shape FP16, "
                          "16 sequences decoded in lockstep; 4 Falcon-40B shape FP16")
     ap.add_argument("--n-seq", type=int, default=16, choices=[1, 16], help="config 3: 16 sequences in lockstep (configs[3]) or the same model at batch 1")
+    ap.add_argument("--mean-rate", type=float, default=None, help="config 3: mean firing rate of the synthetic predictors (default: the model's own, 0.11)")
+    ap.add_argument("--dense-above", type=float, default=None, help="config 3: union fraction above which a layer's FFN runs dense (library default 0.65; 0 always, 1 never)")
     ap.add_argument("--rest-on-gpu", action="store_true", help="config 2: the GPU reads the non-resident neurons' rows from pinned host memory itself instead of handing those neurons to host threads")
     ap.add_argument("--hot-frac", type=float, default=None, help="configs 1 and 2: share of each layer's neurons on the GPU (default 1.0 and 0.6)")
     ap.add_argument("--pmc-probe", action="store_true",

@@ -290,6 +290,8 @@ PI_API int pi_k_gemm_f16(const void * W_f16, int rows, int cols, const void * xn
                          const float * add1, const float * add2, float * y, void * y_f16, pi_stream_t stream);
 PI_API int pi_k_batch_predictor_fc2(const void * fc2_f16, int ff, int r, const void * hidden_f16, int T, float threshold, float * logits,
                                     pi_workspace * ws, pi_stream_t stream);
+/* the union list and count alone, from the flags pi_k_batch_predictor_fc2 left in the workspace */
+PI_API int pi_k_batch_union_count(int ff, int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold,
                                  const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const void * xn_f16,
                                  int epilogue, const float * add1, const float * add2, float * out,
@@ -593,7 +595,16 @@ PI_API int pi_model_batch_generate(pi_model * m, int n_steps, int32_t * out_toke
 PI_API int pi_model_batch_kv_seq_rm(pi_model * m, int seq, int p0, int p1);
 PI_API int pi_model_batch_kv_seq_shift(pi_model * m, int seq, int p0, int p1, int delta);
 PI_API int pi_model_batch_kv_seq_cp(pi_model * m, int src, int dst, int p0, int p1);
-PI_API int pi_model_batch_union(pi_model * m, int32_t * n_union_per_layer);   /* union sizes of the last step, [n_layer] */
+PI_API int pi_model_batch_union(pi_model * m, int32_t * n_union_per_layer); /* Dense cross-over of lockstep decoding (the reference leaves its batch-sparse kernels for a plain mat-mul when a step has many
+ * tokens, ggml-cuda.cu:8787-8814, 7717-7756; here the switch is the union of the sequences' active rows): a layer whose union in the
+ * last step exceeded fraction * n_ff computes its FFN in the next step as dense gate / up mat-muls, h with the predictor's mask, and a
+ * dense down mat-mul (one more copy of that layer's down projection with the neurons contiguous, made on first use).  Default 0.9:
+ * on the 13B shape with 16 sequences the union kernels are faster up to a union of about 0.9 of n_ff (7.46 against 9.18 ms per step at
+ * 0.41, 9.60 against 9.38 at 0.99); <= 0: always dense, >= 1: never.
+ * pi_model_batch_dense_layers: how many layers the next step runs dense. */
+PI_API int pi_model_batch_set_dense_above(pi_model * m, float fraction);
+PI_API int pi_model_batch_dense_layers(pi_model * m);
+  /* union sizes of the last step, [n_layer] */
 
 /* Before pi_model_finalize: layers with a gpu_bucket keep their non-resident rows in pinned host memory and the GPU reads the
  * rows of active neurons from there itself (pi_k_pred_upgate_q4_split) instead of handing those neurons to host threads; the

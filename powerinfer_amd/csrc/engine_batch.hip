@@ -12,6 +12,9 @@
 struct BatchState {
     int n_seq = 0, max_steps = 4096;
     int kv_hi = 0;                        // prompt chunks: cells the chunk's last token attends (its position + 1)
+    // lockstep decoding: layers whose union of active rows was above dense_above * n_ff in the last step run their FFN dense
+    std::vector<char> dense_ffn, graph_dense;
+    float dense_above = 0.9f;
     bool prefill = false;                 // prompt chunks of the model's own sequence: tokens share the model's KV cache
     float * q_rot = nullptr;
     size_t cache_seq_stride = 0;          // elements per sequence: n_layer * n_head_kv * n_ctx * hd
@@ -61,6 +64,17 @@ int chunk_attention(pi_model * m, BatchState * b, int T, size_t kv_off) {
                                 m->attn_scratch_chunk, b->q_rot, m->k_cache + kv_off, m->v_cache + kv_off, b->att, b->att16, m->stream);
 }
 
+// the down projection of layer il with the neurons contiguous ([n_embd][n_ff] fp16), made on first use: a dense mat-mul over the
+// neurons wants them along the rows' contiguous dimension (the decode kernels keep the row-per-neuron layout)
+int ensure_down_rows(pi_model * m, int il) {
+    const pi_hparams & hp = m->hp;
+    if ((int)m->down_rows.size() != hp.n_layer) m->down_rows.assign(hp.n_layer, nullptr);
+    if (m->down_rows[il]) return PI_OK;
+    m->down_rows[il] = m->alloc<__half>((size_t)hp.n_embd * hp.n_ff);
+    if (!m->down_rows[il]) return PI_E_HIP;
+    return pi_k_transpose_f16(m->L(il, PI_T_FFN_DOWN_T).dev, hp.n_ff, hp.n_embd, m->down_rows[il], m->stream);
+}
+
 int batch_layer(pi_model * m, BatchState * b, int il) {
     const pi_hparams & hp = m->hp;
     const int T = b->n_seq, d = hp.n_embd, ff = hp.n_ff, hd = m->hd, gqa = m->gqa;
@@ -100,6 +114,21 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     // predictor
     PI_TRY(pi_k_gemm_f16(fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16, st));
     PI_TRY(pi_k_batch_predictor_fc2(fc2.dev, ff, r, b->hid16, T, hp.sparse_threshold, b->pred_logits, m->ws, st));
+    // Dense cross-over (the reference's switch from its batch-sparse kernels to a plain mat-mul, ggml-cuda.cu:8787-8814, 7717-7756):
+    // when the sequences' active sets together cover nearly all of the layer, gathering rows costs more than streaming all of them.
+    // Measured on the 13B shape, 40 layers, 16 sequences (ms per step, union kernels / dense): union 0.41 of n_ff 7.46 / 9.18,
+    // 0.61 8.27 / 9.26, 0.75 8.63 / 9.24, 0.91 9.40 / 9.29, 0.99 9.60 / 9.38 - the union kernels lose only beyond 0.9.  The choice
+    // is made from the union the previous step measured (the count below keeps that statistic alive while the layer runs dense).
+    if (!b->prefill && il < (int)b->dense_ffn.size() && b->dense_ffn[il]) {
+        PI_TRY(pi_k_batch_union_count(ff, b->union_rows, b->n_union + il, m->ws, st));
+        PI_TRY(pi_k_gemm_f16(up.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->up_out, nullptr, st));
+        if (!falcon) PI_TRY(pi_k_gemm_f16(gate.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->gate_out, nullptr, st));
+        PI_TRY(pi_k_ffn_h_f16(b->up_out, falcon ? nullptr : b->gate_out, b->pred_logits, hp.sparse_threshold, T, ff, b->h16, st));
+        if (!falcon) PI_TRY(pi_k_gemm_f16(m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD, b->ffn_inp, nullptr, b->x2, nullptr, st));
+        else         PI_TRY(pi_k_gemm_f16(m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD2, b->attn_out, x, b->x2, nullptr, st));
+        std::swap(b->x, b->x2);
+        return PI_OK;
+    }
     // sparse FFN over the union of the sequences' active sets
     if (!falcon)
         PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, gate.dev, down.dev, d, ffn_x, PI_EPI_ADD, b->ffn_inp, nullptr,
@@ -165,6 +194,11 @@ BatchState * batch_alloc(pi_model * m, int T, bool with_caches) {
     b->att16 = m->alloc<__half>(n * d); b->hid16 = m->alloc<__half>(n * r);
     b->d_tokens = m->alloc<int32_t>(n); b->d_pos = m->alloc<int32_t>(n); b->d_step = m->alloc<int32_t>(1);
     b->d_out_tokens = m->alloc<int32_t>((size_t)b->max_steps * n); b->union_rows = m->alloc<int32_t>(ff); b->n_union = m->alloc<int32_t>(hp.n_layer);
+    if (with_caches) {                                 // the dense form of a step's FFN (dense_ffn)
+        b->up_out = m->alloc<float>(n * ff); b->gate_out = m->alloc<float>(n * ff); b->h16 = m->alloc<__half>(n * ff);
+        ok = ok && b->up_out && b->gate_out && b->h16;
+        b->dense_ffn.assign(hp.n_layer, 0);
+    }
     if (!ok || !b->x || !b->x2 || !b->qkv || !b->att || !b->attn_out || !b->ffn_inp || !b->hidden || !b->pred_logits || !b->logits ||
         !b->xa16 || !b->xf16 || !b->xp16 || !b->att16 || !b->hid16 || !b->d_tokens || !b->d_pos || !b->d_step || !b->d_out_tokens || !b->union_rows || !b->n_union) {
         delete b;
@@ -368,7 +402,7 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
         // the quantisation and the VRAM split made it
         size_t w16 = 0;
         bool scratch = false;
-        m->down_rows.assign(hp.n_layer, nullptr);
+        if ((int)m->down_rows.size() != hp.n_layer) m->down_rows.assign(hp.n_layer, nullptr);
         for (int il = 0; il < hp.n_layer; ++il) {
             const bool split = m->L(il, PI_T_GPU_BUCKET).dev != nullptr;
             if (split) PI_TRY(gather_rest_rows(m, il));
@@ -376,9 +410,7 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
             if (m->L(il, PI_T_WO).type == PI_TYPE_Q4_0) w16 = std::max(w16, (size_t)hp.n_embd * hp.n_embd);
             if (split || m->L(il, PI_T_FFN_UP).type == PI_TYPE_Q4_0 || m->L(il, PI_T_FFN_DOWN_T).type == PI_TYPE_Q4_0) w16 = std::max(w16, (size_t)hp.n_ff * hp.n_embd);
             if (split || m->L(il, PI_T_FFN_DOWN_T).type == PI_TYPE_Q4_0) { scratch = true; continue; }
-            m->down_rows[il] = m->alloc<__half>((size_t)hp.n_embd * hp.n_ff);
-            if (!m->down_rows[il]) return PI_E_HIP;
-            PI_TRY(pi_k_transpose_f16(m->L(il, PI_T_FFN_DOWN_T).dev, hp.n_ff, hp.n_embd, m->down_rows[il], m->stream));
+            PI_TRY(ensure_down_rows(m, il));
         }
         if (w16) b->w16 = m->alloc<__half>(w16);
         if (scratch) b->w16t = m->alloc<__half>((size_t)hp.n_embd * hp.n_ff);
@@ -467,7 +499,37 @@ void batch_destroy(pi_model * m) {
 }
 }  // namespace pi
 
+namespace {
+// after a step has completed: which layers run their FFN dense in the next one
+int choose_dense_layers(pi_model * m, BatchState * b) {
+    const pi_hparams & hp = m->hp;
+    if (hp.n_ff % 128 || hp.n_embd % 128) return PI_OK;            // the dense mat-muls' shapes
+    std::vector<int32_t> u(hp.n_layer);
+    PI_TRY(pi_memcpy_d2h(u.data(), b->n_union, sizeof(int32_t) * hp.n_layer));
+    for (int il = 0; il < hp.n_layer; ++il) {
+        const bool dense = b->dense_above <= 0.0f || (b->dense_above < 1.0f && (float)u[il] > b->dense_above * (float)hp.n_ff);
+        if (dense) PI_TRY(ensure_down_rows(m, il));
+        b->dense_ffn[il] = dense ? 1 : 0;
+    }
+    return PI_OK;
+}
+}  // namespace
+
 extern "C" {
+
+int pi_model_batch_set_dense_above(pi_model * m, float fraction) {
+    if (!m || !m->batch) return pi::fail(PI_E_STATE, "pi_model_batch_set_dense_above: pi_model_batch_init first");
+    m->batch->dense_above = fraction;
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    return choose_dense_layers(m, m->batch);
+}
+
+int pi_model_batch_dense_layers(pi_model * m) {
+    if (!m || !m->batch) return pi::fail(PI_E_STATE, "pi_model_batch_dense_layers: pi_model_batch_init first");
+    int n = 0;
+    for (char c : m->batch->dense_ffn) n += c ? 1 : 0;
+    return n;
+}
 
 int pi_model_batch_init(pi_model * m, int n_seq) {
     if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_batch_init: model not finalized");
@@ -480,6 +542,7 @@ int pi_model_batch_init(pi_model * m, int n_seq) {
     const size_t T = n_seq;
     PI_HIP_TRY(hipMemsetAsync(b->k_cache, 0, sizeof(__half) * b->cache_seq_stride * T, m->stream));
     PI_HIP_TRY(hipMemsetAsync(b->v_cache, 0, sizeof(__half) * b->cache_seq_stride * T, m->stream));
+    PI_HIP_TRY(hipMemsetAsync(b->n_union, 0, sizeof(int32_t) * m->hp.n_layer, m->stream));
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
     m->batch = b;
     return PI_OK;
@@ -500,6 +563,7 @@ int pi_model_batch_decode(pi_model * m, const int32_t * tokens, const int32_t * 
     PI_HIP_TRY(hipStreamSynchronize(m->stream));          // the host arrays may be pageable: finish the copies before returning control
     PI_TRY(batch_step(m));
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    PI_TRY(choose_dense_layers(m, b));
     if (next_tokens) PI_TRY(pi_memcpy_d2h(next_tokens, b->d_tokens, sizeof(int32_t) * b->n_seq));
     if (logits_out) PI_TRY(pi_memcpy_d2h(logits_out, b->logits, sizeof(float) * (size_t)b->n_seq * m->hp.n_vocab));
     return PI_OK;
@@ -518,7 +582,12 @@ int pi_model_batch_generate(pi_model * m, int n_steps, int32_t * out_tokens, flo
     PI_HIP_TRY(hipMemsetAsync(b->d_step, 0, 4, m->stream));
     const char * no_graph = getenv("PI_NO_GRAPH");
     const bool use_graph = !(no_graph && no_graph[0] == '1');
+    if (b->graph_exec && b->graph_dense != b->dense_ffn) {          // the captured step runs other layers dense than the next one should
+        (void)hipGraphExecDestroy(b->graph_exec); b->graph_exec = nullptr;
+        if (b->graph) { (void)hipGraphDestroy(b->graph); b->graph = nullptr; }
+    }
     if (use_graph && !b->graph_exec) {
+        b->graph_dense = b->dense_ffn;
         PI_HIP_TRY(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
         const int rc = batch_step(m);
         hipGraph_t g = nullptr;
@@ -537,7 +606,7 @@ int pi_model_batch_generate(pi_model * m, int n_steps, int32_t * out_tokens, flo
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
     if (ms_out) PI_HIP_TRY(hipEventElapsedTime(ms_out, m->ev0, m->ev1));
     PI_TRY(pi_memcpy_d2h(out_tokens, b->d_out_tokens, sizeof(int32_t) * (size_t)n_steps * b->n_seq));
-    return PI_OK;
+    return choose_dense_layers(m, b);
 }
 
 // llama_kv_cache_seq_rm / _seq_shift / _seq_cp for one sequence of the batch (llama.cpp:1757-1848).  Every sequence owns a cache,

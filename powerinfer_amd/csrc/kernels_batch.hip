@@ -946,6 +946,14 @@ int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, 
     return pi::check_launch("pi_k_batch_sparse_ffn");
 }
 
+// the union of the step's active rows alone (list and count from the flags pi_k_batch_predictor_fc2 left in the workspace): the statistic
+// a caller keeps when it runs the step's FFN dense
+int pi_k_batch_union_count(int ff, int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream) {
+    if (!union_rows || !n_union || !ws || ff <= 0 || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_batch_union_count: bad arguments");
+    hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, (hipStream_t)stream, ws->row_any, ff, ws->words, union_rows, n_union);
+    return pi::check_launch("pi_k_batch_union_count");
+}
+
 // The two sparse operators of a step of T <= 16 tokens AS OPERATORS (the reference's mul_mat_batch_sparse / axpy at batch size > 1,
 // ggml-cuda.cu:6994-7034, 8787-8814): the caller supplies the predictor output idx [T][ff]; each weight row is read once for the step.
 int pi_k_batch_sparse_mul_mat(const void * W_f16, int ff, int cols, const void * xn_f16, int T, const float * idx, float threshold,

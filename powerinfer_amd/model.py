@@ -46,6 +46,8 @@ def _declare(L):
     L.pi_model_batch_kv_seq_shift.restype, L.pi_model_batch_kv_seq_shift.argtypes = i, [vp, i, i, i, i]
     L.pi_model_batch_kv_seq_cp.restype, L.pi_model_batch_kv_seq_cp.argtypes = i, [vp, i, i, i, i]
     L.pi_model_batch_union.restype, L.pi_model_batch_union.argtypes = i, [vp, vp]
+    L.pi_model_batch_set_dense_above.restype, L.pi_model_batch_set_dense_above.argtypes = i, [vp, C.c_float]
+    L.pi_model_batch_dense_layers.restype, L.pi_model_batch_dense_layers.argtypes = i, [vp]
     L.pi_model_time_section.restype, L.pi_model_time_section.argtypes = i, [vp, i, i, C.POINTER(C.c_float), C.POINTER(C.c_int)]
 
 
@@ -54,6 +56,7 @@ ENGINE_SYMBOLS = ["pi_model_create", "pi_model_free", "pi_model_set_tensor", "pi
                   "pi_model_decode", "pi_model_generate", "pi_model_set_capture", "pi_model_get_capture", "pi_model_set_rest_on_gpu",
                   "pi_model_step_active", "pi_model_time_section",
                   "pi_model_batch_init", "pi_model_batch_decode", "pi_model_batch_generate", "pi_model_batch_union",
+                  "pi_model_batch_set_dense_above", "pi_model_batch_dense_layers",
                   "pi_model_batch_kv_seq_rm", "pi_model_batch_kv_seq_shift", "pi_model_batch_kv_seq_cp"]
 
 
@@ -218,6 +221,16 @@ class Model:
         out = np.empty(self.hp.n_layer, np.int32)
         check(self.L.pi_model_batch_union(self.h, out.ctypes.data_as(C.c_void_p)), "pi_model_batch_union")
         return out
+
+    def batch_set_dense_above(self, fraction):
+        """Layers whose union of active rows exceeded fraction * n_ff in the last step run their FFN dense (<= 0: always, >= 1: never)."""
+        check(self.L.pi_model_batch_set_dense_above(self.h, float(fraction)), "pi_model_batch_set_dense_above")
+
+    def batch_dense_layers(self):
+        n = self.L.pi_model_batch_dense_layers(self.h)
+        if n < 0:
+            check(n, "pi_model_batch_dense_layers")
+        return n
 
     def close(self):
         if self.h:

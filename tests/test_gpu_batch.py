@@ -390,6 +390,61 @@ def test_batched_decode_matches_per_sequence_oracle(arch):
         m.close()
 
 
+@pytest.mark.parametrize("arch", ["llama-tiny", "falcon-tiny"])
+def test_lockstep_decoding_crosses_over_to_dense_ffn(arch):
+    """The dense cross-over of batched decoding: with an active set that covers 95 % of every layer the union of the sequences' rows
+    is above the switch (90 % of n_ff), so from the second step on every layer computes its FFN as dense gate / up mat-muls, h under
+    the predictor's mask, and a dense down mat-mul.  The first step has no statistic yet and runs the union kernels.  Both forms
+    against the CPU oracle per sequence (margin-protected model: logits within 1e-2 at every step, identical greedy tokens), against
+    each other (an engine that never switches), and through the captured graph, which is re-captured when the choice changes."""
+    from powerinfer_amd.model import Model
+    hp = synth.hparams(arch, seed=6, n_ctx=48, mean_rate=0.95, pred_margin=True, head_pair=2048)
+    model = synth.make_model(hp)
+    n_seq, n_steps = 4, 6
+    toks = np.random.default_rng(3).integers(0, hp.n_vocab, (n_steps, n_seq)).astype(np.int32)
+    auto, never, always = Model(hp).load(model), Model(hp).load(model), Model(hp).load(model)
+    for g in (auto, never, always):
+        g.batch_init(n_seq)
+    never.batch_set_dense_above(1.0)
+    always.batch_set_dense_above(0.0)
+    assert auto.batch_dense_layers() == 0 and never.batch_dense_layers() == 0 and always.batch_dense_layers() == hp.n_layer
+    oms = [ol.OracleModel(model) for _ in range(n_seq)]
+    nxt = None
+    for s in range(n_steps):
+        pos = np.full(n_seq, s, np.int32)
+        nxt, lg_a = auto.batch_decode(toks[s], pos)
+        nxt_n, lg_n = never.batch_decode(toks[s], pos)
+        nxt_d, lg_d = always.batch_decode(toks[s], pos)
+        assert auto.batch_dense_layers() == hp.n_layer and never.batch_dense_layers() == 0          # the statistic of this step decides the next
+        assert np.all(auto.batch_union() > 0.9 * hp.n_ff) and np.array_equal(auto.batch_union(), never.batch_union())
+        for t in range(n_seq):
+            tok_o, lg_o = oms[t].eval([int(toks[s, t])], s)
+            for lg in (lg_a, lg_n, lg_d):
+                assert rel_err(lg[t], lg_o) < 1e-2, (s, t, rel_err(lg[t], lg_o))
+            assert int(nxt[t]) == tok_o and int(nxt_n[t]) == tok_o and int(nxt_d[t]) == tok_o, (s, t)
+            assert rel_err(lg_d[t], lg_n[t]) < 2e-3
+        if s >= 1:                                                  # `auto` runs what `always` runs now, on a cache whose first cell came from the union kernels
+            assert rel_err(lg_a, lg_d) < 2e-3
+    # free-running on the device: `auto` captures its graph with the dense layers, `never` with the union kernels; same tokens
+    gen_a, _ = auto.batch_generate(5)
+    gen_n, _ = never.batch_generate(5)
+    assert np.array_equal(gen_a, gen_n)
+    for t in range(n_seq):
+        cur = int(nxt[t])
+        for s in range(5):
+            cur, _ = oms[t].eval([cur], n_steps + s)
+            assert int(gen_a[s, t]) == cur, (t, s)
+        oms[t].close()
+    # the choice changes under a captured graph: the next call captures again and continues from the same state
+    auto.batch_set_dense_above(1.0)
+    assert auto.batch_dense_layers() == 0
+    more_a, _ = auto.batch_generate(3)
+    more_n, _ = never.batch_generate(3)
+    assert np.array_equal(more_a, more_n)
+    for g in (auto, never, always):
+        g.close()
+
+
 SEED_13B_MOVING = 53       # a seed whose sixteen greedy paths spread over all four marker tokens, keep their top-2 gaps, and never pass a step where both head pairs project near zero (the logit tolerance is relative to the largest logit)
 
 

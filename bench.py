@@ -311,7 +311,7 @@ def main():
                          "16 sequences decoded in lockstep; 4 Falcon-40B shape FP16")
     ap.add_argument("--n-seq", type=int, default=16, choices=[1, 16], help="config 3: 16 sequences in lockstep (configs[3]) or the same model at batch 1")
     ap.add_argument("--mean-rate", type=float, default=None, help="config 3: mean firing rate of the synthetic predictors (default: the model's own, 0.11)")
-    ap.add_argument("--dense-above", type=float, default=None, help="config 3: union fraction above which a layer's FFN runs dense (library default 0.65; 0 always, 1 never)")
+    ap.add_argument("--dense-above", type=float, default=None, help="config 3: union fraction above which a layer's FFN runs dense (library default 0.9; 0 always, 1 never)")
     ap.add_argument("--rest-on-gpu", action="store_true", help="config 2: the GPU reads the non-resident neurons' rows from pinned host memory itself instead of handing those neurons to host threads")
     ap.add_argument("--hot-frac", type=float, default=None, help="configs 1 and 2: share of each layer's neurons on the GPU (default 1.0 and 0.6)")
     ap.add_argument("--pmc-probe", action="store_true",
@@ -560,7 +560,8 @@ def main():
             pl.sync()
             dt = time.perf_counter() - t0
             out["prompt_phase"] = {"tokens": args.prompt_bench, "ms": round(dt * 1e3, 2), "tok_per_s": round(args.prompt_bench / dt, 1),
-                                   "what": "pi_model_decode of the whole prompt: chunks of up to 512 tokens (dense mat-muls through hipBLASLt plans, each weight "
+                                   "gemm": "own LDS-tiled MFMA kernel" if os.environ.get("PI_PREFILL_GEMM") == "own" else "hipBLASLt plans",
+                                   "what": "pi_model_decode of the whole prompt: chunks of up to 512 tokens (dense mat-muls through hipBLASLt plans, or on this library's own kernel with PI_PREFILL_GEMM=own; each weight "
                                            "row read once per chunk, predictor mask applied to h), last token through the single-token path"
                                            + ("; Q4_0 matrices expanded to fp16 per chunk, activations through Q8_0 blocks" if hp.wtype != pl.F16 else "")
                                            + ("; non-resident FFN rows read from pinned host memory once per chunk" if hybrid else "")}

@@ -217,7 +217,7 @@ namespace {
 int chunk_gemm(pi_model * m, const void * W, int rows, int cols, const void * xn, int T, int epi, const float * add1, const float * add2,
                float * y, void * y16) {
     if (m->gemm_lib) return pi_gemm_lib_f16(m->gemm_lib, W, rows, cols, xn, T, epi, add1, add2, y, y16, m->stream);
-    return pi_k_gemm_wide_f16(W, rows, cols, xn, T, epi, add1, add2, y, y16, m->stream);
+    return pi_k_gemm_tile_f16(W, rows, cols, xn, T, epi, add1, add2, y, y16, 0, m->stream);
 }
 
 // a matrix of layer il as fp16 rows for a chunk's mat-mul: an F16 matrix that is whole on the device as stored; a Q4_0 one expanded into
@@ -363,9 +363,12 @@ bool prefill_wide_supported(pi_model * m) {
     return !(off && off[0] == '1') && wide_unsupported(m) == nullptr;
 }
 
-int prefill_wide_max(pi_model * m) {
+int prefill_wide_max(pi_model * m) { (void)m; return 512; }      // the longest chunk of the attention, embedding and elementwise kernels
+
+// PI_PREFILL_GEMM=own: the dense mat-muls of prompt chunks run on this library's LDS-tiled MFMA kernel instead of hipBLASLt plans
+static bool prefill_own_gemm() {
     const char * own = getenv("PI_PREFILL_GEMM");
-    return (own && !strcmp(own, "own")) ? 128 : 512;
+    return own && !strcmp(own, "own");
 }
 
 int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) {
@@ -373,7 +376,7 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
     if (T <= 16 || T > kMaxT) return pi::fail(PI_E_ARG, "prefill_wide_chunk: chunk length outside 17 .. prefill_wide_max");
     const pi_hparams & hp = m->hp;
     if (!m->prefill_wide) {
-        if (kMaxT > 128 && !m->gemm_lib) {
+        if (!prefill_own_gemm() && !m->gemm_lib) {
             m->gemm_lib = pi_gemm_lib_create((size_t)64 << 20);
             if (!m->gemm_lib) return PI_E_HIP;
         }

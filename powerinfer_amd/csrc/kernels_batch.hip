@@ -1,6 +1,7 @@
 // Steps of several tokens: 2..16 sequences in lockstep or a prompt chunk of one sequence.  Dense and sparse mat-muls on the matrix
 // cores, the union of the tokens' active rows, norm + rounding passes, Q4_0 expansion and row assembly for prompt chunks.
 #include "kernels_common.hpp"
+#include <type_traits>
 
 namespace {
 
@@ -264,99 +265,152 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
     }
 }
 
-// Prompt chunks of up to 128 tokens: the same mat-mul with NT token tiles of 16 per row tile, so a weight row is read once per chunk
-// instead of once per 16 tokens.  A wave keeps its RT x 16 rows of a 256-column super-step in its private LDS tile (row-contiguous
-// global reads, as above; the load registers are free again once the tile is written, so the next super-step's loads are issued at
-// once and travel during the MFMAs) and streams the activations of all NT x 16 tokens past it, one 32-column step ahead.
-// K is split over the four waves of a workgroup (super-steps w, w + 4, ...); their partial tiles meet in LDS in wave order.
-template <int RT, int NT>
-__global__ __launch_bounds__(kBlock) void gemm_wide_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
-                                                               int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y,
-                                                               __half * __restrict__ y16) {
-    __shared__ __align__(16) unsigned char tile[kWavesPerBlock][RT * 16 * kGlStride];
-    __shared__ float cs[kWavesPerBlock][16][17];
-    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
-    const int i = lane & 15, g = lane >> 4;
-    const int lr = lane >> 5, lc = lane & 31;
-    const int row0 = blockIdx.x * 16 * RT;
-    // blockIdx.y: group of NT x 16 tokens (matrices with few rows are spread over more workgroups by splitting the chunk's tokens)
-    const int t_base = blockIdx.y * NT * 16;
-    xn += (size_t)t_base * cols; y += (size_t)t_base * rows; T -= t_base;
-    if (y16) y16 += (size_t)t_base * rows;
-    if (add1) add1 += (size_t)t_base * rows;
-    if (add2) add2 += (size_t)t_base * rows;
-    const __half * bp[NT];
+// ---------------------------------------------------------------------------------------------------
+// Prompt chunks of any length on the matrix cores with both operands staged in LDS: y[t][row] = epi(W[row] . xn[t]).
+// A workgroup of four waves owns BM weight rows x BN tokens; the reduction dimension advances 64 columns at a time through two
+// LDS stages, and two more stages travel in registers as 16-byte global loads (one stage of MFMAs lasts about 0.2 us, less than a
+// trip to HBM); one barrier per stage.  Both operands are stored row by row with the reduction dimension contiguous, which is
+// the matrix cores' operand layout (eight consecutive columns per lane), so a fragment is one ds_read_b128.  A row is 128 bytes;
+// its eight 16-byte pieces are stored at piece ^ (row & 7), so that the 16 rows a quarter wave reads the same piece of, and the
+// eight pieces of a row that eight neighbouring lanes write, fall on different banks (the bank-conflict counter reads 0; with
+// rows padded to 144 bytes instead it read a third of the LDS cycles).  A wave computes (BM/2) x (BN/2) outputs as 16 x 16
+// tiles; per 32-column step it reads BM/32 + BN/32 fragments for (BM/32) * (BN/32) MFMAs.  Workgroups are numbered so that the
+// token tiles of one row tile run on the same XCD back to back: the row tile's weights cross HBM once and are re-read from that
+// XCD's L2.  cols % 64 == 0; rows and T need not fill the tiles (requests past the edge re-read the last row, results are not
+// stored).
+// ---------------------------------------------------------------------------------------------------
+constexpr int kGtBK = 64;                        // columns per stage
+constexpr int kGtRow = kGtBK * 2;                // bytes per LDS row
+template <int BM, int BN>
+__global__ __launch_bounds__(kBlock, (BM + BN <= 192 ? 3 : 2)) void gemm_tile_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
+                                                                  int nx, int ny, int epi, const float * __restrict__ add1, const float * __restrict__ add2,
+                                                                  float * __restrict__ y, __half * __restrict__ y16) {
+    constexpr int WM = BM / 2, WN = BN / 2, MT = WM / 16, NT = WN / 16;
+    constexpr int ACH = BM * kGtBK * 2 / 16 / kBlock, BCH = BN * kGtBK * 2 / 16 / kBlock;      // 16-byte chunks per thread and stage
+    extern __shared__ __align__(16) unsigned char smem[];
+    unsigned char * sa = smem;                                     // [2][BM][kGtRow]
+    unsigned char * sb = smem + 2 * BM * kGtRow;                   // [2][BN][kGtRow]
+    // workgroup -> (row tile, token tile): XCD x takes row tiles x, x + 8, ... and walks each one's token tiles in turn
+    const int xcd = blockIdx.x % 8, slot = blockIdx.x / 8;
+    const int tx = (slot / ny) * 8 + xcd, ty = slot % ny;
+    if (tx >= nx) return;
+    const int row0 = tx * BM, tok0 = ty * BN;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 15, g = lane >> 4;
+    const int wm = wave & 1, wn = wave >> 1;
+    auto lds_off = [](int r, int kc) { return r * kGtRow + ((kc ^ (r & 7)) * 16); };
+    const __half * ga[ACH]; const __half * gb[BCH];
+    int la[ACH], lb[BCH];
 #pragma unroll
-    for (int nt = 0; nt < NT; ++nt) { const int tok = nt * 16 + i; bp[nt] = xn + (size_t)(tok < T ? tok : T - 1) * cols + g * 8; }
-    unsigned char * mytile = tile[wave];
-    pi_f4 acc[RT][NT];
-#pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) acc[rt][nt] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
-    const int n_ss = (cols / 256 - wave + kWavesPerBlock - 1) / kWavesPerBlock;
-    pi_u32x4 ld[RT][8];
-    auto issue = [&](int ss) {
-        if (ss < n_ss) {
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-                for (int j = 0; j < 8; ++j) {
-                    int r = row0 + rt * 16 + 2 * j + lr;
-                    r = r < rows ? r : rows - 1;
-                    ld[rt][j] = pi_ld_stream(W + (size_t)r * cols + (wave + ss * kWavesPerBlock) * 256 + lc * 8);
-                }
-        }
-    };
-    issue(0);
-    for (int ss = 0; ss < n_ss; ++ss) {
-        const int k0 = (wave + ss * kWavesPerBlock) * 256;
-        pi_u32x4 b[2][NT];
-#pragma unroll
-        for (int nt = 0; nt < NT; ++nt) b[0][nt] = pi_ld16(bp[nt] + k0);
-#pragma unroll
-        for (int rt = 0; rt < RT; ++rt)
-#pragma unroll
-            for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (rt * 16 + 2 * j + lr) * kGlStride + lc * 16) = ld[rt][j];
-        issue(ss + 1);
-#pragma unroll
-        for (int st = 0; st < 8; ++st) {
-            if (st + 1 < 8) {
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt) b[(st + 1) & 1][nt] = pi_ld16(bp[nt] + k0 + (st + 1) * 32);
-            }
-#pragma unroll
-            for (int rt = 0; rt < RT; ++rt) {
-                const pi_u32x4 a = *reinterpret_cast<const pi_u32x4 *>(mytile + (rt * 16 + i) * kGlStride + (4 * st + g) * 16);
-#pragma unroll
-                for (int nt = 0; nt < NT; ++nt)
-                    acc[rt][nt] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a), __builtin_bit_cast(pi_h8, b[st & 1][nt]), acc[rt][nt], 0, 0, 0);
-            }
-        }
+    for (int j = 0; j < ACH; ++j) {
+        const int kc = tid % 8, r = j * 32 + tid / 8;
+        const int rr = row0 + r < rows ? row0 + r : rows - 1;
+        ga[j] = W + (size_t)rr * cols + kc * 8; la[j] = lds_off(r, kc);
     }
-    const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
 #pragma unroll
-    for (int rt = 0; rt < RT; ++rt)
+    for (int j = 0; j < BCH; ++j) {
+        const int kc = tid % 8, r = j * 32 + tid / 8;
+        const int tt = tok0 + r < T ? tok0 + r : T - 1;
+        gb[j] = xn + (size_t)tt * cols + kc * 8; lb[j] = lds_off(r, kc);
+    }
+    pi_f4 acc[MT][NT];
 #pragma unroll
-        for (int nt = 0; nt < NT; ++nt) {
-            __syncthreads();
+    for (int m = 0; m < MT; ++m)
 #pragma unroll
-            for (int r = 0; r < 4; ++r) cs[wave][4 * g + r][i] = acc[rt][nt][r];
-            __syncthreads();
-            const int row = row0 + rt * 16 + rr, tok = nt * 16 + t;
-            if (row < rows && tok < T) {
-                float sum = cs[0][rr][t];
+        for (int n = 0; n < NT; ++n) acc[m][n] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
+    // Two column stages travel in registers while a third is being multiplied: stage kt sits in LDS half kt & 1, stages kt + 1 and
+    // kt + 2 are in flight (one stage of MFMAs is about 0.2 us, less than a trip to HBM).
+    pi_u32x4 ra[2][ACH], rb[2][BCH];
+    const int nk = cols / kGtBK;
+    auto fetch = [&](auto slot, int kt) {
+        constexpr int S = decltype(slot)::value;
 #pragma unroll
-                for (int w = 1; w < kWavesPerBlock; ++w) sum += cs[w][rr][t];
-                const size_t o = (size_t)tok * rows + row;
-                if (epi == PI_EPI_RELU) sum = fmaxf(sum, 0.0f);
-                else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
-                else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[o]), add2[o]);
-                y[o] = sum;
-                if (y16) y16[o] = __float2half_rn(sum);
+        for (int j = 0; j < ACH; ++j) ra[S][j] = pi_ld16(ga[j] + (size_t)kt * kGtBK);
+#pragma unroll
+        for (int j = 0; j < BCH; ++j) rb[S][j] = pi_ld16(gb[j] + (size_t)kt * kGtBK);
+    };
+    auto stash = [&](auto slot) {              // registers of slot S -> LDS half S
+        constexpr int S = decltype(slot)::value;
+        unsigned char * na = sa + S * BM * kGtRow; unsigned char * nb = sb + S * BN * kGtRow;
+#pragma unroll
+        for (int j = 0; j < ACH; ++j) *reinterpret_cast<pi_u32x4 *>(na + la[j]) = ra[S][j];
+#pragma unroll
+        for (int j = 0; j < BCH; ++j) *reinterpret_cast<pi_u32x4 *>(nb + lb[j]) = rb[S][j];
+    };
+    const std::integral_constant<int, 0> c0; const std::integral_constant<int, 1> c1;
+    // every fetch and stash below is unconditional (past the last stage the last one is fetched again and stashed where nobody
+    // reads): the count of loads in flight is then the same on every path, and the waits name exactly the loads they need
+    const int last = nk - 1;
+    fetch(c0, 0);
+    fetch(c1, min(1, last));
+    stash(c0);
+    fetch(c0, min(2, last));
+    __syncthreads();
+    // the lane's two pieces (columns 8g.. of each 32-column step) of fragment row i: every 16-row tile starts on a multiple of 8
+    const int koff[2] = {(g ^ (i & 7)) * 16, ((4 + g) ^ (i & 7)) * 16};
+    const int frag_a = (wm * WM + i) * kGtRow, frag_b = (wn * WN + i) * kGtRow;
+    auto step = [&](auto par, int kt) {
+        constexpr int P = decltype(par)::value;
+        const unsigned char * ca = sa + P * BM * kGtRow + frag_a;
+        const unsigned char * cb = sb + P * BN * kGtRow + frag_b;
+        pi_u32x4 fa[2][MT], fb[2][NT];
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks) {
+#pragma unroll
+            for (int m = 0; m < MT; ++m) fa[ks][m] = *reinterpret_cast<const pi_u32x4 *>(ca + m * 16 * kGtRow + koff[ks]);
+#pragma unroll
+            for (int n = 0; n < NT; ++n) fb[ks][n] = *reinterpret_cast<const pi_u32x4 *>(cb + n * 16 * kGtRow + koff[ks]);
+        }
+#pragma unroll
+        for (int ks = 0; ks < 2; ++ks)
+#pragma unroll
+            for (int m = 0; m < MT; ++m)
+#pragma unroll
+                for (int n = 0; n < NT; ++n)
+                    acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, fa[ks][m]), __builtin_bit_cast(pi_h8, fb[ks][n]), acc[m][n], 0, 0, 0);
+        stash(std::integral_constant<int, P ^ 1>());
+        fetch(std::integral_constant<int, P ^ 1>(), min(kt + 3, last));
+        __syncthreads();
+    };
+    int kt = 0;
+    for (; kt + 1 < nk; kt += 2) { step(c0, kt); step(c1, kt + 1); }
+    if (kt < nk) step(c0, kt);
+    // acc[m][n][r] = y[token tok0 + wn*WN + n*16 + i][row row0 + wm*WM + m*16 + 4g + r]: four consecutive rows per lane
+#pragma unroll
+    for (int m = 0; m < MT; ++m)
+#pragma unroll
+        for (int n = 0; n < NT; ++n) {
+            const int row = row0 + wm * WM + m * 16 + 4 * g, tok = tok0 + wn * WN + n * 16 + i;
+            if (tok >= T || row >= rows) continue;
+            const size_t o = (size_t)tok * rows + row;
+            float v[4] = {acc[m][n][0], acc[m][n][1], acc[m][n][2], acc[m][n][3]};
+            if (row + 4 <= rows && (rows & 3) == 0) {
+                if (epi == PI_EPI_RELU) { for (int r = 0; r < 4; ++r) v[r] = fmaxf(v[r], 0.0f); }
+                else if (epi >= PI_EPI_ADD) {
+                    const float4 a1 = *reinterpret_cast<const float4 *>(add1 + o);
+                    v[0] = __fadd_rn(v[0], a1.x); v[1] = __fadd_rn(v[1], a1.y); v[2] = __fadd_rn(v[2], a1.z); v[3] = __fadd_rn(v[3], a1.w);
+                    if (epi == PI_EPI_ADD2) {
+                        const float4 a2 = *reinterpret_cast<const float4 *>(add2 + o);
+                        v[0] = __fadd_rn(v[0], a2.x); v[1] = __fadd_rn(v[1], a2.y); v[2] = __fadd_rn(v[2], a2.z); v[3] = __fadd_rn(v[3], a2.w);
+                    }
+                }
+                *reinterpret_cast<float4 *>(y + o) = make_float4(v[0], v[1], v[2], v[3]);
+                if (y16) {
+                    __half2 h2[2] = {__floats2half2_rn(v[0], v[1]), __floats2half2_rn(v[2], v[3])};
+                    *reinterpret_cast<uint2 *>(y16 + o) = *reinterpret_cast<const uint2 *>(h2);
+                }
+            } else {
+                for (int r = 0; r < 4 && row + r < rows; ++r) {
+                    float s = v[r];
+                    if (epi == PI_EPI_RELU) s = fmaxf(s, 0.0f);
+                    else if (epi == PI_EPI_ADD) s = __fadd_rn(s, add1[o + r]);
+                    else if (epi == PI_EPI_ADD2) s = __fadd_rn(__fadd_rn(s, add1[o + r]), add2[o + r]);
+                    y[o + r] = s;
+                    if (y16) y16[o + r] = __float2half_rn(s);
+                }
             }
         }
 }
+
 // h16[t][n] = fp16( !(logit[t][n] < thr) ? relu(gate[t][n]) * up[t][n] : 0 )   (relu(up) without a gate): the FFN's hidden vector of a
 // prompt chunk from the dense gate/up products; inactive neurons become exact zeros, which add nothing in the down projection
 // q8 != 0 (n % 64 == 0 and n_ff % 32 == 0): h goes through Q8_0 blocks of 32 neurons first, as the CPU path's Q4_0 down projection quantises it
@@ -815,22 +869,56 @@ int pi_k_gemm_f16(const void * W, int rows, int cols, const void * xn_f16, int T
     return gemm_launch("pi_k_gemm_f16", W, rows, cols, xn_f16, T, epilogue, add1, add2, y, y_f16, 0.0f, nullptr, stream);
 }
 
-int pi_k_gemm_wide_f16(const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
-                       float * y, void * y_f16, pi_stream_t stream) {
-    if (!W || !xn_f16 || !y || rows <= 0) return pi::fail(PI_E_ARG, "pi_k_gemm_wide_f16: null pointer or empty shape");
-    if (T < 1 || T > kWideMaxT || cols <= 0 || cols % 256) return pi::fail(PI_E_ARG, "pi_k_gemm_wide_f16: 1 <= T <= 128 and cols % 256 == 0 required");
+// Output tiles the kernel is built for (weight rows x tokens per workgroup); two workgroups share a compute unit.
+// Output tiles the kernel is built for (weight rows x tokens per workgroup).
+constexpr int kGtNShapes = 5;
+static const int kGtShapes[kGtNShapes][2] = {{128, 128}, {96, 128}, {128, 64}, {64, 128}, {64, 64}};
+// Relative time per output of one workgroup (LDS and L2 bytes per MFMA grow as the tile shrinks); measured on 7B and 13B shapes.
+static const float kGtCost[kGtNShapes] = {1.00f, 1.05f, 1.25f, 1.25f, 1.45f};
+
+// The device spreads workgroups over its compute units, so a launch lasts as long as the unit with the most workgroups:
+// ceil(workgroups / units) tiles one after the other (or side by side at the same total rate).
+static int gt_choose(int rows, int T, int n_cu) {
+    int best = 0; double best_t = 1e30;
+    for (int s = 0; s < kGtNShapes; ++s) {
+        const int bm = kGtShapes[s][0], bn = kGtShapes[s][1];
+        const long long wgs = (long long)((rows + bm - 1) / bm) * ((T + bn - 1) / bn);
+        const double t = (double)((wgs + n_cu - 1) / n_cu) * bm * bn * kGtCost[s];
+        if (t < best_t) { best_t = t; best = s; }
+    }
+    return best;
+}
+
+int pi_k_gemm_tile_f16(const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
+                       float * y, void * y_f16, int tile, pi_stream_t stream) {
+    if (!W || !xn_f16 || !y || rows <= 0 || T <= 0) return pi::fail(PI_E_ARG, "pi_k_gemm_tile_f16: null pointer or empty shape");
+    if (cols <= 0 || cols % kGtBK) return pi::fail(PI_E_ARG, "pi_k_gemm_tile_f16: cols % 64 == 0 required");
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
-        return pi::fail(PI_E_ARG, "pi_k_gemm_wide_f16: bad epilogue arguments");
-    if (T <= kBtMaxT) return gemm_launch("pi_k_gemm_wide_f16", W, rows, cols, xn_f16, T, epilogue, add1, add2, y, y_f16, 0.0f, nullptr, stream);
-#define PI_GEMM_WIDE(RT, NT) hipLaunchKernelGGL((gemm_wide_f16_kernel<RT, NT>), dim3((rows + 16 * RT - 1) / (16 * RT), (T + 16 * NT - 1) / (16 * NT)), dim3(kBlock), 0, \
-        (hipStream_t)stream, (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16)
-    // tile shape by row count: wide matrices take 64 rows x the whole chunk per workgroup; narrower ones split the chunk's tokens over
-    // several workgroups so that the grid still covers the chip (their weights then pass through L2 once per token group)
-    if (rows >= 8192) { if (T <= 32) PI_GEMM_WIDE(2, 2); else if (T <= 64) PI_GEMM_WIDE(4, 4); else PI_GEMM_WIDE(4, 8); }
-    else if (rows > 2048) { if (T <= 32) PI_GEMM_WIDE(2, 2); else PI_GEMM_WIDE(2, 4); }
-    else PI_GEMM_WIDE(1, 2);
-#undef PI_GEMM_WIDE
-    return pi::check_launch("pi_k_gemm_wide_f16");
+        return pi::fail(PI_E_ARG, "pi_k_gemm_tile_f16: bad epilogue arguments");
+    if ((((uintptr_t)W | (uintptr_t)xn_f16 | (uintptr_t)y | (uintptr_t)add1 | (uintptr_t)add2) & 15) != 0 || ((uintptr_t)y_f16 & 7) != 0)
+        return pi::fail(PI_E_ARG, "pi_k_gemm_tile_f16: operands must be 16-byte aligned");
+    hipStream_t st = (hipStream_t)stream;
+    int shape = -1;
+    if (tile == 0) shape = gt_choose(rows, T, pi::compute_units());
+    else for (int s = 0; s < kGtNShapes; ++s) if (tile == kGtShapes[s][0] * 1000 + kGtShapes[s][1]) shape = s;
+    if (shape < 0) return pi::fail(PI_E_ARG, "pi_k_gemm_tile_f16: tile must be 0 or one of 128128, 96128, 128064, 64128, 64064");
+#define PI_GEMM_TILE(BM, BN) do {                                                                                                         \
+        const int nx = (rows + BM - 1) / BM, ny = (T + BN - 1) / BN;                                                                      \
+        const size_t sh = (size_t)2 * (BM + BN) * kGtRow;                                                                                 \
+        static bool raised = false;                                                                                                       \
+        if (!raised && sh > 64 * 1024) { PI_HIP_TRY(hipFuncSetAttribute((const void *)gemm_tile_f16_kernel<BM, BN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh)); raised = true; } \
+        hipLaunchKernelGGL((gemm_tile_f16_kernel<BM, BN>), dim3(8 * ((nx + 7) / 8) * ny), dim3(kBlock), sh, st, (const __half *)W, (const __half *)xn_f16, T, rows, cols,   \
+                           nx, ny, epilogue, add1, add2, y, (__half *)y_f16);                                                             \
+    } while (0)
+    switch (shape) {
+        case 0: PI_GEMM_TILE(128, 128); break;
+        case 1: PI_GEMM_TILE(96, 128); break;
+        case 2: PI_GEMM_TILE(128, 64); break;
+        case 3: PI_GEMM_TILE(64, 128); break;
+        default: PI_GEMM_TILE(64, 64); break;
+    }
+#undef PI_GEMM_TILE
+    return pi::check_launch("pi_k_gemm_tile_f16");
 }
 int pi_k_ffn_h_f16(const float * up, const float * gate, const float * logits, float threshold, int T, int ff, void * h_f16, pi_stream_t stream) {
     if (!up || !logits || !h_f16 || T <= 0 || ff <= 0) return pi::fail(PI_E_ARG, "pi_k_ffn_h_f16: bad arguments");

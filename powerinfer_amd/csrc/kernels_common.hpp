@@ -187,7 +187,6 @@ __device__ __forceinline__ float apply_epilogue(float v, int epi, const float * 
 typedef _Float16 pi_h8 __attribute__((ext_vector_type(8)));
 typedef float    pi_f4 __attribute__((ext_vector_type(4)));
 constexpr int kBtMaxT = 16;
-constexpr int kWideMaxT = 128;            // longest chunk of gemm_wide_f16_kernel
 constexpr int kChunkMaxT = 512;           // longest chunk of the attention, embedding and elementwise kernels of a prompt chunk
 constexpr int kBmGroups = 32;
 constexpr int kAxpyTile = PI_WAVE * 8;

@@ -57,11 +57,14 @@ def test_gemm_matches_oracle(rows, cols, T):
     assert np.array_equal(dy16.download(np.float16).reshape(T, rows), got.astype(np.float16))
 
 
-@pytest.mark.parametrize("rows,cols,T", [(3000, 5120, 128), (4104, 4096, 100), (1024, 11008, 128), (520, 512, 17), (2048, 1024, 40), (4096, 4096, 64)])
-def test_gemm_wide_matches_oracle(rows, cols, T):
-    """The prompt-chunk mat-mul (up to 128 tokens per weight pass): token counts on and off the tile sizes (17 -> 2 tiles, 40 -> 4,
-    100 and 128 -> 8), row counts off the 32-row workgroup tile, the FFN-wide reduction dimension of the down projection, every
-    epilogue, and the transposition that feeds the down projection."""
+@pytest.mark.parametrize("tile", [0, 128128, 96128, 128064, 64128, 64064])
+@pytest.mark.parametrize("rows,cols,T", [(3000, 5120, 300), (4104, 4096, 512), (1024, 11008, 130), (520, 512, 17), (64, 64, 1), (130, 192, 129),
+                                         (2048, 1024, 40), (12288, 4096, 512)])
+def test_gemm_tile_matches_oracle(rows, cols, T, tile):
+    """This library's LDS-tiled mat-mul of prompt chunks against the reference's CPU mat-mul on the same fp16-rounded activations, on
+    every output tile it is built for and on the one the library picks: token and row counts on and off the tile sizes (a single
+    token, one past a tile, 512 tokens), a reduction dimension of one stage and of 172, every epilogue, the fp16 copy, and the
+    transposition that feeds the down projection."""
     from powerinfer_amd import lib as pl
     L = pl.init()
     rng = np.random.default_rng(rows + cols + T)
@@ -73,23 +76,30 @@ def test_gemm_wide_matches_oracle(rows, cols, T):
     dn = gpu_norm_round(pl, L, x)
     dw, dy, d1, d2 = pl.DevBuf(host=w), pl.DevBuf(T * rows * 4), pl.DevBuf(host=a1), pl.DevBuf(host=a2)
     pl.check(L.pi_memset(dy.ptr, 0xFF, dy.nbytes), "memset")
-    pl.check(L.pi_k_gemm_wide_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_NONE, None, None, dy.ptr, None, None), "gemm_wide")
+    pl.check(L.pi_k_gemm_tile_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_NONE, None, None, dy.ptr, None, tile, None), "gemm_tile")
     pl.sync()
     got = dy.download(np.float32).reshape(T, rows)
     assert rel_err(got, want) < 5e-6
-    pl.check(L.pi_k_gemm_wide_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_ADD2, d1.ptr, d2.ptr, dy.ptr, None, None), "gemm_wide")
+    pl.check(L.pi_k_gemm_tile_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_ADD, d1.ptr, None, dy.ptr, None, tile, None), "gemm_tile")
+    pl.sync()
+    assert rel_err(dy.download(np.float32).reshape(T, rows), want + a1) < 5e-6
+    pl.check(L.pi_k_gemm_tile_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_ADD2, d1.ptr, d2.ptr, dy.ptr, None, tile, None), "gemm_tile")
     pl.sync()
     assert rel_err(dy.download(np.float32).reshape(T, rows), (want + a1) + a2) < 5e-6
     dy16 = pl.DevBuf(T * rows * 2)
-    pl.check(L.pi_k_gemm_wide_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_RELU, None, None, dy.ptr, dy16.ptr, None), "gemm_wide")
+    pl.check(L.pi_k_gemm_tile_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_RELU, None, None, dy.ptr, dy16.ptr, tile, None), "gemm_tile")
     pl.sync()
     got = dy.download(np.float32).reshape(T, rows)
     assert rel_err(got, np.maximum(want, 0)) < 5e-6
     assert np.array_equal(dy16.download(np.float16).reshape(T, rows), got.astype(np.float16))
-    dt = pl.DevBuf(rows * cols * 2)
-    pl.check(L.pi_k_transpose_f16(dw.ptr, rows, cols, dt.ptr, None), "transpose")
-    pl.sync()
-    assert np.array_equal(dt.download(np.float16).reshape(cols, rows), w.T)
+    if tile == 0:
+        dt = pl.DevBuf(rows * cols * 2)
+        pl.check(L.pi_k_transpose_f16(dw.ptr, rows, cols, dt.ptr, None), "transpose")
+        pl.sync()
+        assert np.array_equal(dt.download(np.float16).reshape(cols, rows), w.T)
+        assert L.pi_k_gemm_tile_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_NONE, None, None, dy.ptr, None, 32032, None) != 0        # no such tile
+        assert L.pi_k_gemm_tile_f16(dw.ptr, rows, cols - 8, dn.ptr, T, pl.EPI_NONE, None, None, dy.ptr, None, 0, None) != 0       # cols % 64
+        assert L.pi_k_gemm_tile_f16(dw.ptr, rows, cols, dn.ptr, T, pl.EPI_ADD, None, None, dy.ptr, None, 0, None) != 0            # residual missing
 
 
 @pytest.mark.parametrize("rows,cols,T", [(3000, 5120, 300), (4104, 4096, 512), (1024, 11008, 130), (520, 512, 17), (12288, 4096, 512)])
@@ -612,14 +622,15 @@ def test_prompt_chunks_match_token_by_token(arch):
 @pytest.mark.timeout(300)
 @pytest.mark.parametrize("name,kw,n_prompt,gemm", [("llama-tiny", dict(n_rank=256, n_ctx=192), 150, "own"), ("falcon-tiny", dict(n_rank=256, n_ctx=192), 150, "own"),
                                                    ("llama-tiny", dict(n_rank=256, n_ctx=192), 40, "own"),
-                                                   ("llama-7b", dict(n_layer=2, n_ctx=160), 140, "own"),
+                                                   ("llama-7b", dict(n_layer=2, n_ctx=160), 140, "own"), ("llama-7b", dict(n_layer=2, n_ctx=640), 600, "own"),
+                                                   ("falcon-tiny", dict(n_rank=256, n_ctx=640), 600, "own"),
                                                    ("llama-tiny", dict(n_rank=256, n_ctx=192), 150, "lib"), ("falcon-tiny", dict(n_rank=256, n_ctx=640), 600, "lib"),
                                                    ("llama-tiny", dict(n_rank=256, n_ctx=192), 40, "lib"),
                                                    ("llama-7b", dict(n_layer=2, n_ctx=640), 600, "lib")])
 def test_wide_prompt_chunks_match_the_oracle(name, kw, n_prompt, gemm, monkeypatch):
-    """Prompts longer than 16 tokens go through chunks of up to 512 (dense mat-muls through the library, every weight row read once
-    per chunk, the predictor's mask applied as zeros of h; chunks of up to 128 on this library's own mat-mul kernel with
-    PI_PREFILL_GEMM=own), then chunks of 16, then the last token alone.  On a margin-protected model (no neuron can flip, greedy
+    """Prompts longer than 16 tokens go through chunks of up to 512 (dense mat-muls through the library, or on this library's own
+    LDS-tiled mat-mul kernel with PI_PREFILL_GEMM=own; every weight row read once per chunk, the predictor's mask applied as zeros
+    of h), then chunks of 16, then the last token alone.  On a margin-protected model (no neuron can flip, greedy
     decisions keep their distance) the logits after the prompt and of the steps behind it agree with the CPU oracle within the
     stated tolerance, and with the same engine fed 16 tokens at a time."""
     import os

@@ -348,28 +348,41 @@ __global__ __launch_bounds__(kBlock, (BM + BN <= 192 ? 3 : 2)) void gemm_tile_f1
     // the lane's two pieces (columns 8g.. of each 32-column step) of fragment row i: every 16-row tile starts on a multiple of 8
     const int koff[2] = {(g ^ (i & 7)) * 16, ((4 + g) ^ (i & 7)) * 16};
     const int frag_a = (wm * WM + i) * kGtRow, frag_b = (wn * WN + i) * kGtRow;
+    // The fragments of a stage's first 32 columns are read while the previous stage's second 32 are multiplied, those of its second
+    // 32 while its first are: every LDS read has a block of MFMAs between its issue and its use.
+    pi_u32x4 f0a[MT], f0b[NT], f1a[MT], f1b[NT];
+    auto frags = [&](auto par, auto half, pi_u32x4 * fa, pi_u32x4 * fb) {
+        constexpr int P = decltype(par)::value, KS = decltype(half)::value;
+        const unsigned char * ca = sa + P * BM * kGtRow + frag_a + koff[KS];
+        const unsigned char * cb = sb + P * BN * kGtRow + frag_b + koff[KS];
+#pragma unroll
+        for (int m = 0; m < MT; ++m) fa[m] = *reinterpret_cast<const pi_u32x4 *>(ca + m * 16 * kGtRow);
+#pragma unroll
+        for (int n = 0; n < NT; ++n) fb[n] = *reinterpret_cast<const pi_u32x4 *>(cb + n * 16 * kGtRow);
+    };
+    auto mfmas = [&](const pi_u32x4 * fa, const pi_u32x4 * fb) {
+#pragma unroll
+        for (int m = 0; m < MT; ++m)
+#pragma unroll
+            for (int n = 0; n < NT; ++n)
+                acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, fa[m]), __builtin_bit_cast(pi_h8, fb[n]), acc[m][n], 0, 0, 0);
+    };
+    frags(c0, c0, f0a, f0b);
     auto step = [&](auto par, int kt) {
         constexpr int P = decltype(par)::value;
-        const unsigned char * ca = sa + P * BM * kGtRow + frag_a;
-        const unsigned char * cb = sb + P * BN * kGtRow + frag_b;
-        pi_u32x4 fa[2][MT], fb[2][NT];
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks) {
-#pragma unroll
-            for (int m = 0; m < MT; ++m) fa[ks][m] = *reinterpret_cast<const pi_u32x4 *>(ca + m * 16 * kGtRow + koff[ks]);
-#pragma unroll
-            for (int n = 0; n < NT; ++n) fb[ks][n] = *reinterpret_cast<const pi_u32x4 *>(cb + n * 16 * kGtRow + koff[ks]);
-        }
-#pragma unroll
-        for (int ks = 0; ks < 2; ++ks)
-#pragma unroll
-            for (int m = 0; m < MT; ++m)
-#pragma unroll
-                for (int n = 0; n < NT; ++n)
-                    acc[m][n] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, fa[ks][m]), __builtin_bit_cast(pi_h8, fb[ks][n]), acc[m][n], 0, 0, 0);
-        stash(std::integral_constant<int, P ^ 1>());
-        fetch(std::integral_constant<int, P ^ 1>(), min(kt + 3, last));
+        const std::integral_constant<int, P ^ 1> other;
+        frags(par, c1, f1a, f1b);
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(f0a, f0b);
+        stash(other);
+        fetch(other, min(kt + 3, last));
+        __builtin_amdgcn_sched_barrier(0);
         __syncthreads();
+        __builtin_amdgcn_sched_barrier(0);
+        frags(other, c0, f0a, f0b);           // past the last stage: the re-stashed last stage, read and not used
+        __builtin_amdgcn_sched_barrier(0);
+        mfmas(f1a, f1b);
+        __builtin_amdgcn_sched_barrier(0);
     };
     int kt = 0;
     for (; kt + 1 < nk; kt += 2) { step(c0, kt); step(c1, kt + 1); }

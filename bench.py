@@ -253,7 +253,11 @@ def bench_batched(args):
     n_prompt = 512 if args.prompt == 64 else args.prompt
     steps = 128 if args.steps == 256 else args.steps
     over = {} if args.mean_rate is None else {"mean_rate": args.mean_rate}
-    hp = synth.hparams("llama-13b", n_layer=40 if args.layers == 32 else args.layers, n_ctx=n_prompt + args.warmup + steps + 8, seed=1, **over)
+    q4 = args.batch_model == "llama-7b-q4"
+    if q4:      # the Q4_0 model of configs[2] with every neuron on the GPU, sixteen sequences on the fp16 form of its matrices
+        hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_prompt + args.warmup + steps + 8, seed=1, wtype=pl.Q4_0, **over)
+    else:
+        hp = synth.hparams("llama-13b", n_layer=40 if args.layers == 32 else args.layers, n_ctx=n_prompt + args.warmup + steps + 8, seed=1, **over)
     keep = []
     m = build_synthetic_on_device(hp, keep)
     m.batch_init(n_seq)
@@ -276,11 +280,12 @@ def bench_batched(args):
     step_bytes = hp.n_layer * (4 * d * d * 2.0 + (d * r + r * ff) * 2.0 + n_seq * 2 * n_kv * d * 2.0) + union.sum() * 3 * d * 2.0 + hp.n_vocab * d * 2.0
     ms_step = wall * 1e3 / steps
     out = {
-        "metric": "decode tok/s, 16 sequences, ProSparse-Llama2-13B shape FP16", "value": round(n_seq * 1e3 / ms_step, 1), "unit": "tok/s",
+        "metric": "decode tok/s, 16 sequences, " + ("ReluLLaMA-7B shape Q4_0 (matrices expanded to fp16 at batch_init)" if q4 else "ProSparse-Llama2-13B shape FP16"), "value": round(n_seq * 1e3 / ms_step, 1), "unit": "tok/s",
         "n_gpus": 1, "steps": steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak",
         "vs_baseline": None, "dtype": "f16", "data": "synthetic",
-        "config": {"workload": "configs[3]: ProSparse-LLaMA-2-13B shape (d 5120, ff 13824, 40 heads, vocab 32000, predictor rank 1280), "
-                               f"{hp.n_layer} layers, random-init FP16 weights, all neurons on the GPU, {n_seq} sequences with {n_prompt}-token random "
+        "config": {"workload": ("configs[2]'s model in lockstep: ReluLLaMA-7B shape (d 4096, ff 11008, 32 heads, vocab 32000, predictor rank 1024), " if q4 else
+                                "configs[3]: ProSparse-LLaMA-2-13B shape (d 5120, ff 13824, 40 heads, vocab 32000, predictor rank 1280), ") +
+                               f"{hp.n_layer} layers, random-init {'Q4_0' if q4 else 'FP16'} weights, all neurons on the GPU, {n_seq} sequences with {n_prompt}-token random "
                                "prompts, greedy decode in lockstep (one token per sequence per step)",
                    "n_layer": hp.n_layer, "n_seq": n_seq, "prompt_tokens": n_prompt, "n_ctx": hp.n_ctx,
                    "mean_union_rows_per_layer": round(union.mean(), 1), "union_fraction": round(union.mean() / hp.n_ff, 3),
@@ -310,6 +315,7 @@ def main():
                          "Q4_0 with the hottest 60 %% of neurons on the GPU and the rest on host threads; 3 ProSparse-LLaMA-2-13B shape FP16, "
                          "16 sequences decoded in lockstep; 4 Falcon-40B shape FP16")
     ap.add_argument("--n-seq", type=int, default=16, choices=[1, 16], help="config 3: 16 sequences in lockstep (configs[3]) or the same model at batch 1")
+    ap.add_argument("--batch-model", default="llama-13b", choices=["llama-13b", "llama-7b-q4"], help="config 3 with 16 sequences: configs[3]'s model, or the Q4_0 7B model in lockstep")
     ap.add_argument("--mean-rate", type=float, default=None, help="config 3: mean firing rate of the synthetic predictors (default: the model's own, 0.11)")
     ap.add_argument("--dense-above", type=float, default=None, help="config 3: union fraction above which a layer's FFN runs dense (library default 0.9; 0 always, 1 never)")
     ap.add_argument("--rest-on-gpu", action="store_true", help="config 2: the GPU reads the non-resident neurons' rows from pinned host memory itself instead of handing those neurons to host threads")

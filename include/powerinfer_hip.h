@@ -584,7 +584,9 @@ PI_API int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, fl
  * the norm; it is also the predictor's input).  Any output pointer may be NULL. */
 /*
  * Batched greedy decoding: n_seq <= 16 independent sequences advance one token per step (examples/batched/batched.cpp:100-260).
- * F16 models with every neuron on the GPU.  pi_model_batch_init allocates one KV cache per sequence and the step buffers;
+ * F16 or Q4_0 models with every neuron on the GPU (a Q4_0 matrix is expanded to fp16 rows once, at pi_model_batch_init, and kept
+ * beside its Q4_0 form; activations pass through the CPU path's Q8_0 values).  pi_model_batch_init allocates one KV cache per
+ * sequence and the step buffers;
  * pi_model_batch_decode feeds tokens[t] of sequence t at positions[t] and returns each sequence's greedy next token (and,
  * if logits_out != NULL, the [n_seq][n_vocab] logits); pi_model_batch_generate continues greedily from that state for
  * n_steps steps and returns out_tokens[n_steps][n_seq].

@@ -349,13 +349,22 @@ def test_batch_sparse_ffn_none_and_all_active(thr):
     L.pi_workspace_destroy(ws)
 
 
+@pytest.mark.parametrize("wtype", [synth.F16, synth.Q4_0], ids=["f16", "q4_0"])
 @pytest.mark.parametrize("arch", ["llama-tiny", "falcon-tiny"])
-def test_batched_decode_matches_per_sequence_oracle(arch):
+def test_batched_decode_matches_per_sequence_oracle(arch, wtype):
     """Four sequences with different prompts advance in lockstep (examples/batched/batched.cpp).  Sequences do not interact,
     so sequence t of the batch must reproduce a single-sequence run on the same tokens: against the CPU oracle (teacher
-    forced, the trajectory-level criteria of the single-sequence tests) and against this library's own batch-1 engine."""
+    forced, the trajectory-level criteria of the single-sequence tests) and against this library's own batch-1 engine.
+    A Q4_0 model steps on the fp16 form of its matrices ((q - 8) * d, made once at batch_init) with the activations passed
+    through the CPU path's Q8_0 blocks.  Both factors are then rounded to fp16 (2^-11 each), which moves a few per cent of the next
+    stage's int8 roundings by one step; the single-token path, whose integer dots reproduce the CPU's activations bit for bit,
+    sits at a median distance of 0 from the oracle on these models, the lockstep path at about 1e-2.  Its bound is therefore
+    3e-2 on the median and 2e-1 on single steps (the reference's own batch kernel for Q4_0 rows, dequantize_mul_mat_batch_sparse,
+    ggml-cuda.cu:4757-4758 and 5390-5397, multiplies dequantised weights with unquantised activations: a larger difference of the
+    same kind), on a model whose predictors and greedy choices keep a margin."""
     from powerinfer_amd.model import Model
-    hp = synth.hparams(arch, seed=5, n_ctx=64)
+    q4 = wtype != synth.F16
+    hp = synth.hparams(arch, seed=5, n_ctx=64, wtype=wtype, **(dict(pred_margin=True, head_pair=2048) if q4 else {}))
     model = synth.make_model(hp)
     n_seq, n_steps = 4, 10
     rng = np.random.default_rng(11)
@@ -381,8 +390,9 @@ def test_batched_decode_matches_per_sequence_oracle(arch):
             same += int(batch_next[s, t] == tok_o)
         om.close()
     errs_o, errs_g = np.array(errs_o), np.array(errs_g)
-    assert np.median(errs_o) < 1e-2, errs_o
-    assert np.median(errs_g) < 1e-2, errs_g
+    assert np.median(errs_o) < (3e-2 if q4 else 1e-2), errs_o
+    assert np.median(errs_g) < (3e-2 if q4 else 1e-2), errs_g
+    assert not q4 or max(errs_o.max(), errs_g.max()) < 2e-1, (errs_o, errs_g)
     assert same >= 0.9 * n_seq * n_steps, same
     # greedy continuation on the device equals stepping the same state by hand
     gm2 = Model(hp).load(model)
@@ -456,6 +466,7 @@ def test_lockstep_decoding_crosses_over_to_dense_ffn(arch):
 
 
 SEED_13B_MOVING = 53       # a seed whose sixteen greedy paths spread over all four marker tokens, keep their top-2 gaps, and never pass a step where both head pairs project near zero (the logit tolerance is relative to the largest logit)
+SEED_7B_Q4_BATCH = 44       # the 7B-width Q4_0 lockstep test's model
 
 
 @pytest.mark.timeout(600)
@@ -511,6 +522,46 @@ def test_batched_decode_13b_width_16_sequences(moving):
         assert np.array_equal(union, m.any(0).sum(-1)), (union, m.any(0).sum(-1))
         assert np.all(union > m.sum(-1).max(0)), (union, m.sum(-1).max(0))
     gm.close()
+
+
+@pytest.mark.timeout(600)
+def test_batched_decode_7b_q4_width_16_sequences():
+    """A Q4_0 model at the 7B width (d 4096, ff 11008, predictor rank 1024, vocab 32000, two layers), sixteen sequences in lockstep
+    on the fp16 form of the matrices: per sequence against the CPU oracle, teacher forced, with the Q4_0 bounds of
+    test_batched_decode_matches_per_sequence_oracle (median 3e-2, single steps 2e-1, nine greedy tokens in ten equal), then the
+    free-running continuation on the device against stepping the same state by hand."""
+    from powerinfer_amd.model import Model
+    hp = synth.hparams("llama-7b", n_layer=2, n_ctx=32, seed=SEED_7B_Q4_BATCH, wtype=synth.Q4_0, pred_margin=True, head_pair=2048)
+    model = synth.make_model(hp)
+    n_seq, n_steps = 16, 6
+    rng = np.random.default_rng(23)
+    toks = rng.integers(0, hp.n_vocab, (n_steps, n_seq)).astype(np.int32)
+    gm = Model(hp).load(model)
+    gm.batch_init(n_seq)
+    oms = [ol.OracleModel(model) for _ in range(n_seq)]
+    errs, same = [], 0
+    for s in range(n_steps):
+        nxt, lg = gm.batch_decode(toks[s], np.full(n_seq, s, np.int32))
+        for t in range(n_seq):
+            tok_o, lg_o = oms[t].eval([int(toks[s, t])], s)
+            errs.append(rel_err(lg[t], lg_o))
+            same += int(nxt[t] == tok_o)
+    for om in oms:
+        om.close()
+    errs = np.array(errs)
+    assert np.median(errs) < 3e-2 and errs.max() < 2e-1, errs
+    assert same >= 0.9 * n_seq * n_steps, same
+    assert np.all(gm.batch_union() > 0)
+    gen, _ = gm.batch_generate(4)
+    gm2 = Model(hp).load(model)
+    gm2.batch_init(n_seq)
+    cur = None
+    for s in range(n_steps):
+        cur, _ = gm2.batch_decode(toks[s], np.full(n_seq, s, np.int32))
+    for s in range(4):
+        cur, _ = gm2.batch_decode(cur, np.full(n_seq, n_steps + s, np.int32))
+        assert np.array_equal(gen[s], cur), s
+    gm.close(), gm2.close()
 
 
 def test_batch_kv_sequence_edits():
@@ -575,7 +626,7 @@ def test_batch_kv_sequence_edits():
 def test_batch_init_rejects_unsupported_models():
     from powerinfer_amd import lib as pl
     from powerinfer_amd.model import Model
-    hp = synth.hparams("llama-tiny", seed=2, n_ctx=32, wtype=ol.Q4_0)
+    hp = synth.hparams("llama-tiny", seed=2, n_ctx=32, hot_frac=0.5)          # a VRAM split: the host computes part of every layer
     m = Model(hp).load(synth.make_model(hp))
     with pytest.raises(pl.PiError):
         m.batch_init(4)

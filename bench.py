@@ -254,7 +254,7 @@ def bench_batched(args):
     steps = 128 if args.steps == 256 else args.steps
     over = {} if args.mean_rate is None else {"mean_rate": args.mean_rate}
     q4 = args.batch_model == "llama-7b-q4"
-    if q4:      # the Q4_0 model of configs[2] with every neuron on the GPU, sixteen sequences on the fp16 form of its matrices
+    if q4:      # the Q4_0 model of configs[2] with every neuron on the GPU, sixteen sequences in lockstep
         hp = synth.hparams("llama-7b", n_layer=args.layers, n_ctx=n_prompt + args.warmup + steps + 8, seed=1, wtype=pl.Q4_0, **over)
     else:
         hp = synth.hparams("llama-13b", n_layer=40 if args.layers == 32 else args.layers, n_ctx=n_prompt + args.warmup + steps + 8, seed=1, **over)
@@ -280,9 +280,9 @@ def bench_batched(args):
     step_bytes = hp.n_layer * (4 * d * d * 2.0 + (d * r + r * ff) * 2.0 + n_seq * 2 * n_kv * d * 2.0) + union.sum() * 3 * d * 2.0 + hp.n_vocab * d * 2.0
     ms_step = wall * 1e3 / steps
     out = {
-        "metric": "decode tok/s, 16 sequences, " + ("ReluLLaMA-7B shape Q4_0 (matrices expanded to fp16 at batch_init)" if q4 else "ProSparse-Llama2-13B shape FP16"), "value": round(n_seq * 1e3 / ms_step, 1), "unit": "tok/s",
+        "metric": "decode tok/s, 16 sequences, " + ("ReluLLaMA-7B shape Q4_0 (integer matrix-core kernels on Q4_0 x Q8_0 blocks)" if q4 else "ProSparse-Llama2-13B shape FP16"), "value": round(n_seq * 1e3 / ms_step, 1), "unit": "tok/s",
         "n_gpus": 1, "steps": steps, "warmup": args.warmup, "ms_per_step": round(ms_step, 4), "higher_is_better": True, "scaling": "weak",
-        "vs_baseline": None, "dtype": "f16", "data": "synthetic",
+        "vs_baseline": None, "dtype": "q4_0 x q8_0 (int8 MFMA, fp32 scale)" if q4 else "f16", "data": "synthetic",
         "config": {"workload": ("configs[2]'s model in lockstep: ReluLLaMA-7B shape (d 4096, ff 11008, 32 heads, vocab 32000, predictor rank 1024), " if q4 else
                                 "configs[3]: ProSparse-LLaMA-2-13B shape (d 5120, ff 13824, 40 heads, vocab 32000, predictor rank 1280), ") +
                                f"{hp.n_layer} layers, random-init {'Q4_0' if q4 else 'FP16'} weights, all neurons on the GPU, {n_seq} sequences with {n_prompt}-token random "

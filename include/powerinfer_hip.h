@@ -308,6 +308,26 @@ PI_API int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float thre
  * contiguous). */
 PI_API int pi_k_gemm_tile_f16(const void * W_f16, int rows, int cols, const void * xn_f16, int T, int epilogue,
                               const float * add1, const float * add2, float * y, void * y_f16, int tile, pi_stream_t stream);
+/* Steps of up to 16 tokens on Q4_0 weights with the CPU path's arithmetic (ggml_vec_dot_q4_0_q8_0, ggml-quants.c:2512-2650; in the reference's
+ * CUDA backend the mul_mat_q tiles and dequantize_mul_mat_batch_sparse, ggml-cuda.cu:3524-4308, 4757-4830): one integer matrix-core
+ * instruction per pair of a Q4_0 weight block and a Q8_0 activation block gives the exact int32 sum, scaled by d_w * d_x in fp32.
+ * pi_k_q4_split writes a Q4_0 matrix [rows][cols / 32] blocks as two arrays, quants (16 bytes per block, the dwords of four consecutive
+ * blocks interleaved: [row][block / 4][dword][block % 4]) and scales [rows][cols / 32] fp16 (cols % 256 == 0); pi_k_norm_q8_blocks
+ * normalises T <= 16 rows and quantises them as quantize_row_q8_0 does (ggml-quants.c:702-760) into q int8 [T][cols], d float
+ * [cols / 32][16] and s8 = 8 * sum(q) int32 [cols / 32][16] (token innermost; cols <= 8192), and, if plain_f16 != NULL, also writes the
+ * rows before the norm as fp16 (the predictor's input); pi_k_gemm_q4_t16 is y[t][row] = epilogue(W[row] . x[t]) on those forms; pi_k_batch_sparse_ffn_q4 is
+ * pi_k_batch_sparse_ffn on them: the union list from the flags pi_k_batch_predictor_fc2 left in the workspace, up/gate dots of the
+ * union rows, h [16][ff] under the predictor's mask, hq = the values h's Q8_0 blocks keep (blocks of 32 consecutive neurons, as the
+ * CPU path's axpy reads them, ggml.c:14436-14470), and the down projection over the union rows on fp32 matrix cores.
+ * h and hq are caller-provided scratch of 16 * ff floats each. */
+PI_API int pi_k_q4_split(const void * W_q4, int rows, int cols, void * quants, void * scales, pi_stream_t stream);
+PI_API int pi_k_norm_q8_blocks(const float * x, int T, int cols, const pi_norm * norm, void * q, float * d, int32_t * s8, void * plain_f16, pi_stream_t stream);
+PI_API int pi_k_gemm_q4_t16(const void * quants, const void * scales, int rows, int cols, const void * xq, const float * xd, const int32_t * xs8, int T,
+                            int epilogue, const float * add1, const float * add2, float * y, pi_stream_t stream);
+PI_API int pi_k_batch_sparse_ffn_q4(const float * logits, int T, int ff, float threshold, const void * up_quants, const void * up_scales,
+                                    const void * gate_quants, const void * gate_scales, const void * down_quants, const void * down_scales, int cols,
+                                    const void * xq, const float * xd, const int32_t * xs8, int epilogue, const float * add1, const float * add2, float * out,
+                                    float * h, float * hq, int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream);
 PI_API int pi_k_ffn_h_f16(const float * up, const float * gate, const float * logits, float threshold, int T, int ff, void * h_f16, pi_stream_t stream);
 PI_API int pi_k_transpose_f16(const void * in_f16, int rows, int cols, void * out_f16, pi_stream_t stream);
 
@@ -584,9 +604,9 @@ PI_API int pi_model_generate(pi_model * m, int n_steps, int32_t * out_tokens, fl
  * the norm; it is also the predictor's input).  Any output pointer may be NULL. */
 /*
  * Batched greedy decoding: n_seq <= 16 independent sequences advance one token per step (examples/batched/batched.cpp:100-260).
- * F16 or Q4_0 models with every neuron on the GPU (a Q4_0 matrix is expanded to fp16 rows once, at pi_model_batch_init, and kept
- * beside its Q4_0 form; activations pass through the CPU path's Q8_0 values).  pi_model_batch_init allocates one KV cache per
- * sequence and the step buffers;
+ * F16 models, or Q4_0 models with F16 predictors, with every neuron on the GPU (Q4_0: integer matrix-core kernels on the Q4_0 x Q8_0
+ * blocks, pi_k_gemm_q4_t16 / pi_k_batch_sparse_ffn_q4, from a split copy of the quants made at pi_model_batch_init).
+ * pi_model_batch_init allocates one KV cache per sequence and the step buffers;
  * pi_model_batch_decode feeds tokens[t] of sequence t at positions[t] and returns each sequence's greedy next token (and,
  * if logits_out != NULL, the [n_seq][n_vocab] logits); pi_model_batch_generate continues greedily from that state for
  * n_steps steps and returns out_tokens[n_steps][n_seq].

@@ -26,8 +26,10 @@ struct BatchState {
     int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_step = nullptr, *d_out_tokens = nullptr, *union_rows = nullptr, *n_union = nullptr;
     float *up_out = nullptr, *gate_out = nullptr;      // wide prompt chunks: dense gate/up products [T][n_ff]
     __half *h16 = nullptr;                             //                     and the FFN's hidden vector
-    // lockstep decoding of a Q4_0 model: every Q4_0 matrix once more as fp16 rows ((q - 8) * d), made at pi_model_batch_init
-    std::unordered_map<const Tensor *, const void *> as_f16;
+    // steps of a Q4_0 model on integer matrix cores: Q8_0 blocks of the attention-side and of the FFN-side mat-mul input (int8 quants
+    // [16][n_embd], scales and 8 * sums [n_embd / 32][16]), h and the values its Q8_0 blocks keep [16][n_ff]
+    void *qa = nullptr, *qf = nullptr; float *da = nullptr, *df = nullptr; int32_t *sa = nullptr, *sf = nullptr;
+    float *h32 = nullptr, *hq32 = nullptr;
     __half *w16 = nullptr, *w16t = nullptr;            // wide prompt chunks of Q4_0 / hybrid layers: one matrix as fp16, and the down projection with the neurons contiguous
     // hybrid layers in wide prompt chunks: the non-resident rows of the next layer travel from pinned host memory into one of two device
     // staging buffers on a copy stream while this layer computes (up | gate | down, each n_rest rows)
@@ -67,17 +69,103 @@ int chunk_attention(pi_model * m, BatchState * b, int T, size_t kv_off) {
                                 m->attn_scratch_chunk, b->q_rot, m->k_cache + kv_off, m->v_cache + kv_off, b->att, b->att16, m->stream);
 }
 
-// a matrix as fp16 rows for a lockstep step: an F16 matrix as stored, a Q4_0 one in the fp16 form made at pi_model_batch_init
-const void * batch_weight(pi_model * m, Tensor & t) {
-    if (m->batch) { auto it = m->batch->as_f16.find(&t); if (it != m->batch->as_f16.end()) return it->second; }
-    return t.dev;
-}
-
 // fp16 mat-mul input for a matrix of the given type: rounded to fp16, for a Q4_0 matrix through Q8_0 blocks first (the CPU path
 // multiplies Q4_0 rows with the Q8_0 form of the activations)
 int batch_input(int wtype, const float * x, int T, int cols, const pi_norm * norm, void * out16, void * plain16, hipStream_t st) {
     if (wtype == PI_TYPE_Q4_0) return pi_k_norm_q8_round_f16(x, T, cols, norm, out16, plain16, st);
     return pi_k_norm_round_f16(x, T, cols, norm, out16, plain16, st);
+}
+
+// why the model's multi-token steps cannot run on the integer matrix-core kernels, or null
+const char * q4_steps_unsupported(pi_model * m) {
+    const pi_hparams & hp = m->hp;
+    if (m->hybrid || m->capture) return "hybrid models and capture hooks follow single tokens";
+    if (hp.n_embd % 512 || hp.n_embd > 8192 || hp.n_ff % 32 || (int)m->L(0, PI_T_FC1).ne1 % 128) return "n_embd % 512 == 0, n_embd <= 8192, n_ff % 32 == 0 and predictor rank % 128 == 0 required";
+    for (int il = 0; il < hp.n_layer; ++il) {
+        for (int k : {PI_T_WQKV, PI_T_WO, PI_T_FFN_UP, PI_T_FFN_GATE, PI_T_FFN_DOWN_T}) {
+            if (k == PI_T_FFN_GATE && hp.arch == PI_ARCH_FALCON) continue;
+            if (m->L(il, k).type != PI_TYPE_Q4_0) return "every attention and FFN matrix must be Q4_0";
+        }
+        if (m->L(il, PI_T_FC1).type != PI_TYPE_F16 || m->L(il, PI_T_FC2).type != PI_TYPE_F16) return "predictors must be F16";
+    }
+    const int te = m->glob[PI_T_TOK_EMBD].type, to = m->glob[PI_T_OUTPUT].type;
+    if ((te != PI_TYPE_F16 && te != PI_TYPE_Q4_0) || (to != PI_TYPE_F16 && to != PI_TYPE_Q4_0)) return "embedding and output matrix must be F16 or Q4_0";
+    return nullptr;
+}
+
+// the split form of every Q4_0 matrix the steps multiply with, made once
+int ensure_q4_split(pi_model * m) {
+    if (m->q4_steps) return PI_OK;
+    auto split = [&](Tensor & t) -> int {
+        if (t.type != PI_TYPE_Q4_0 || !t.dev || m->q4_split.count(&t)) return PI_OK;
+        const size_t nb = (size_t)t.ne1 * (t.ne0 / 32);
+        unsigned char * q = m->alloc<unsigned char>(nb * 16);
+        __half * d = m->alloc<__half>(nb);
+        if (!q || !d) return PI_E_HIP;
+        PI_TRY(pi_k_q4_split(t.dev, (int)t.ne1, (int)t.ne0, q, d, m->stream));
+        m->q4_split[&t] = pi_model::Q4Split{q, d};
+        return PI_OK;
+    };
+    PI_TRY(split(m->glob[PI_T_OUTPUT]));
+    for (int il = 0; il < m->hp.n_layer; ++il)
+        for (int k : {PI_T_WQKV, PI_T_WO, PI_T_FFN_UP, PI_T_FFN_GATE, PI_T_FFN_DOWN_T}) PI_TRY(split(m->L(il, k)));
+    m->q4_steps = true;
+    return PI_OK;
+}
+
+int chunk_attention(pi_model * m, BatchState * b, int T, size_t kv_off);
+
+// One layer of a step of up to 16 tokens of a Q4_0 model: the mat-muls of the Q4_0 matrices on integer matrix cores against the
+// Q8_0 blocks of their inputs (the CPU path's arithmetic), the F16 predictor as in an F16 model.
+int batch_layer_q4(pi_model * m, BatchState * b, int il) {
+    const pi_hparams & hp = m->hp;
+    const int T = b->n_seq, d = hp.n_embd, ff = hp.n_ff, hd = m->hd, gqa = m->gqa;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    hipStream_t st = m->stream;
+    auto W = [&](int kind) { return m->q4_split.at(&m->L(il, kind)); };
+    Tensor & fc1 = m->L(il, PI_T_FC1); Tensor & fc2 = m->L(il, PI_T_FC2);
+    const int r = (int)fc1.ne1;
+    const size_t kv_off = (size_t)il * hp.n_head_kv * hp.n_ctx * hd;
+    float * x = b->x;
+    const pi_norm plain{0, 0.0f, nullptr, nullptr};
+    pi_norm an;
+    if (!falcon) an = mk_norm(1, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), nullptr);
+    else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
+    else an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
+    PI_TRY(pi_k_norm_q8_blocks(x, T, d, &an, b->qa, b->da, b->sa, falcon ? b->xp16 : nullptr, st));      // Falcon: the predictor reads the layer input as plain fp16
+    if (falcon) {
+        // the FFN branch reads the layer input too, under its own norm (with a single norm: the attention's)
+        pi_norm fn = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
+        PI_TRY(pi_k_norm_q8_blocks(x, T, d, m->L(il, PI_T_ATTN_NORM_2).dev ? &fn : &an, b->qf, b->df, b->sf, nullptr, st));
+    }
+    const auto wqkv = W(PI_T_WQKV), wo = W(PI_T_WO);
+    PI_TRY(pi_k_gemm_q4_t16(wqkv.quants, wqkv.scales, d + 2 * gqa, d, b->qa, b->da, b->sa, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, st));
+    if (b->prefill)
+        PI_TRY(chunk_attention(m, b, T, kv_off));
+    else
+        PI_TRY(pi_k_attn_fused_batch(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
+                                     hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, hp.n_ctx, b->d_pos, b->att, d, b->att16, st));
+    PI_TRY(pi_k_norm_q8_blocks(b->att, T, d, &plain, b->qa, b->da, b->sa, nullptr, st));
+    if (!falcon) {
+        PI_TRY(pi_k_gemm_q4_t16(wo.quants, wo.scales, d, d, b->qa, b->da, b->sa, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, st));       // ffn_inp = wo.att + x
+        pi_norm fn = mk_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
+        PI_TRY(pi_k_norm_q8_blocks(b->ffn_inp, T, d, &fn, b->qf, b->df, b->sf, b->xp16, st));                                        // the predictor reads the rows before the norm
+    } else {
+        PI_TRY(pi_k_gemm_q4_t16(wo.quants, wo.scales, d, d, b->qa, b->da, b->sa, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, st));
+    }
+    PI_TRY(pi_k_gemm_f16(fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16, st));
+    PI_TRY(pi_k_batch_predictor_fc2(fc2.dev, ff, r, b->hid16, T, hp.sparse_threshold, b->pred_logits, m->ws, st));
+    const auto up = W(PI_T_FFN_UP), down = W(PI_T_FFN_DOWN_T);
+    if (!falcon) {
+        const auto gate = W(PI_T_FFN_GATE);
+        PI_TRY(pi_k_batch_sparse_ffn_q4(b->pred_logits, T, ff, hp.sparse_threshold, up.quants, up.scales, gate.quants, gate.scales, down.quants, down.scales, d,
+                                        b->qf, b->df, b->sf, PI_EPI_ADD, b->ffn_inp, nullptr, b->x2, b->h32, b->hq32, b->union_rows, b->n_union + il, m->ws, st));
+    } else {
+        PI_TRY(pi_k_batch_sparse_ffn_q4(b->pred_logits, T, ff, hp.sparse_threshold, up.quants, up.scales, nullptr, nullptr, down.quants, down.scales, d,
+                                        b->qf, b->df, b->sf, PI_EPI_ADD2, b->attn_out, x, b->x2, b->h32, b->hq32, b->union_rows, b->n_union + il, m->ws, st));
+    }
+    std::swap(b->x, b->x2);
+    return PI_OK;
 }
 
 // the down projection of layer il with the neurons contiguous ([n_embd][n_ff] fp16), made on first use: a dense mat-mul over the
@@ -88,10 +176,11 @@ int ensure_down_rows(pi_model * m, int il) {
     if (m->down_rows[il]) return PI_OK;
     m->down_rows[il] = m->alloc<__half>((size_t)hp.n_embd * hp.n_ff);
     if (!m->down_rows[il]) return PI_E_HIP;
-    return pi_k_transpose_f16(batch_weight(m, m->L(il, PI_T_FFN_DOWN_T)), hp.n_ff, hp.n_embd, m->down_rows[il], m->stream);
+    return pi_k_transpose_f16(m->L(il, PI_T_FFN_DOWN_T).dev, hp.n_ff, hp.n_embd, m->down_rows[il], m->stream);
 }
 
 int batch_layer(pi_model * m, BatchState * b, int il) {
+    if (m->q4_steps) return batch_layer_q4(m, b, il);
     const pi_hparams & hp = m->hp;
     const int T = b->n_seq, d = hp.n_embd, ff = hp.n_ff, hd = m->hd, gqa = m->gqa;
     const bool falcon = hp.arch == PI_ARCH_FALCON;
@@ -104,42 +193,32 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     float * x = b->x;
 
     // attention
-    const pi_norm plain{0, 0.0f, nullptr, nullptr};
     pi_norm an;
     if (!falcon) an = mk_norm(1, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), nullptr);
     else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
     else an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
-    // Falcon: the predictor reads the raw layer input (plain fp16 for an F16 predictor; a Q4_0 one gets its own pass below)
-    PI_TRY(batch_input(wqkv.type, x, T, d, &an, b->xa16, falcon && fc1.type != PI_TYPE_Q4_0 ? b->xp16 : nullptr, st));
-    if (falcon && fc1.type == PI_TYPE_Q4_0) PI_TRY(pi_k_norm_q8_round_f16(x, T, d, &plain, b->xp16, nullptr, st));
-    PI_TRY(pi_k_gemm_f16(batch_weight(m, wqkv), d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr, st));
+    PI_TRY(pi_k_norm_round_f16(x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));       // Falcon: the predictor reads the raw layer input
+    PI_TRY(pi_k_gemm_f16(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr, st));
     if (b->prefill)
         PI_TRY(chunk_attention(m, b, T, kv_off));
     else
         PI_TRY(pi_k_attn_fused_batch(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
                                      hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, hp.n_ctx, b->d_pos, b->att, d, b->att16, st));
-    if (wo.type == PI_TYPE_Q4_0) PI_TRY(pi_k_norm_q8_round_f16(b->att, T, d, &plain, b->att16, nullptr, st));
 
     pi_norm fn;
-    const __half * ffn_x = b->xf16;
     if (!falcon) {
-        PI_TRY(pi_k_gemm_f16(batch_weight(m, wo), d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, nullptr, st));       // ffn_inp = wo.att + x
+        PI_TRY(pi_k_gemm_f16(wo.dev, d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, nullptr, st));       // ffn_inp = wo.att + x
         fn = mk_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
-        // FFN input and predictor input (the rows before the norm) in one pass; a Q4_0 predictor wants its rows through Q8_0 blocks
-        PI_TRY(batch_input(up.type, b->ffn_inp, T, d, &fn, b->xf16, fc1.type == PI_TYPE_Q4_0 ? nullptr : b->xp16, st));
-        if (fc1.type == PI_TYPE_Q4_0) PI_TRY(pi_k_norm_q8_round_f16(b->ffn_inp, T, d, &plain, b->xp16, nullptr, st));
+        PI_TRY(pi_k_norm_round_f16(b->ffn_inp, T, d, &fn, b->xf16, b->xp16, st));                                // FFN input and predictor input in one pass
     } else {
-        PI_TRY(pi_k_gemm_f16(batch_weight(m, wo), d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, nullptr, st));
+        PI_TRY(pi_k_gemm_f16(wo.dev, d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, nullptr, st));
         fn = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
-        // two norms: the FFN has its own; a single norm is shared with the attention branch unless the two matrices want different
-        // containers (fp16 against Q8_0 blocks)
-        if (m->L(il, PI_T_ATTN_NORM_2).dev || up.type != wqkv.type) PI_TRY(batch_input(up.type, x, T, d, &fn, b->xf16, nullptr, st));
-        else ffn_x = b->xa16;
+        if (m->L(il, PI_T_ATTN_NORM_2).dev) PI_TRY(pi_k_norm_round_f16(x, T, d, &fn, b->xf16, nullptr, st));     // two norms: the FFN has its own
     }
+    const __half * ffn_x = (falcon && !m->L(il, PI_T_ATTN_NORM_2).dev) ? b->xa16 : b->xf16;                        // single-norm Falcon: attention and FFN share it
     // predictor
-    PI_TRY(pi_k_gemm_f16(batch_weight(m, fc1), r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16, st));
-    if (fc2.type == PI_TYPE_Q4_0) PI_TRY(pi_k_norm_q8_round_f16(b->hidden, T, r, &plain, b->hid16, nullptr, st));
-    PI_TRY(pi_k_batch_predictor_fc2(batch_weight(m, fc2), ff, r, b->hid16, T, hp.sparse_threshold, b->pred_logits, m->ws, st));
+    PI_TRY(pi_k_gemm_f16(fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16, st));
+    PI_TRY(pi_k_batch_predictor_fc2(fc2.dev, ff, r, b->hid16, T, hp.sparse_threshold, b->pred_logits, m->ws, st));
     // Dense cross-over (the reference's switch from its batch-sparse kernels to a plain mat-mul, ggml-cuda.cu:8787-8814, 7717-7756):
     // when the sequences' active sets together cover nearly all of the layer, gathering rows costs more than streaming all of them.
     // Measured on the 13B shape, 40 layers, 16 sequences (ms per step, union kernels / dense): union 0.41 of n_ff 7.46 / 9.18,
@@ -147,23 +226,21 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     // is made from the union the previous step measured (the count below keeps that statistic alive while the layer runs dense).
     if (!b->prefill && il < (int)b->dense_ffn.size() && b->dense_ffn[il]) {
         PI_TRY(pi_k_batch_union_count(ff, b->union_rows, b->n_union + il, m->ws, st));
-        PI_TRY(pi_k_gemm_f16(batch_weight(m, up), ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->up_out, nullptr, st));
-        if (!falcon) PI_TRY(pi_k_gemm_f16(batch_weight(m, gate), ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->gate_out, nullptr, st));
-        if (down.type == PI_TYPE_Q4_0) PI_TRY(pi_k_ffn_h_q8_f16(b->up_out, falcon ? nullptr : b->gate_out, b->pred_logits, hp.sparse_threshold, T, ff, b->h16, st));
-        else                           PI_TRY(pi_k_ffn_h_f16(b->up_out, falcon ? nullptr : b->gate_out, b->pred_logits, hp.sparse_threshold, T, ff, b->h16, st));
+        PI_TRY(pi_k_gemm_f16(up.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->up_out, nullptr, st));
+        if (!falcon) PI_TRY(pi_k_gemm_f16(gate.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->gate_out, nullptr, st));
+        PI_TRY(pi_k_ffn_h_f16(b->up_out, falcon ? nullptr : b->gate_out, b->pred_logits, hp.sparse_threshold, T, ff, b->h16, st));
         if (!falcon) PI_TRY(pi_k_gemm_f16(m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD, b->ffn_inp, nullptr, b->x2, nullptr, st));
         else         PI_TRY(pi_k_gemm_f16(m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD2, b->attn_out, x, b->x2, nullptr, st));
         std::swap(b->x, b->x2);
         return PI_OK;
     }
-    // sparse FFN over the union of the sequences' active sets (the hidden vector stays fp16 between gate/up and down: for a Q4_0
-    // down projection the CPU path would pass it through Q8_0 blocks, a difference of at most half an int8 step per element)
+    // sparse FFN over the union of the sequences' active sets
     if (!falcon)
-        PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, batch_weight(m, up), batch_weight(m, gate), batch_weight(m, down), d, ffn_x,
-                                     PI_EPI_ADD, b->ffn_inp, nullptr, b->x2, b->union_rows, b->n_union + il, m->ws, st));
+        PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, gate.dev, down.dev, d, ffn_x, PI_EPI_ADD, b->ffn_inp, nullptr,
+                                     b->x2, b->union_rows, b->n_union + il, m->ws, st));
     else
-        PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, batch_weight(m, up), nullptr, batch_weight(m, down), d, ffn_x,
-                                     PI_EPI_ADD2, b->attn_out, x, b->x2, b->union_rows, b->n_union + il, m->ws, st));
+        PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, nullptr, down.dev, d, ffn_x, PI_EPI_ADD2, b->attn_out, x,
+                                     b->x2, b->union_rows, b->n_union + il, m->ws, st));
     std::swap(b->x, b->x2);
     return PI_OK;
 }
@@ -178,8 +255,14 @@ int batch_step(pi_model * m) {
     else PI_TRY(pi_k_embed_batch(m->glob[PI_T_TOK_EMBD].dev, d, b->d_tokens, T, b->x, st));
     for (int il = 0; il < hp.n_layer; ++il) PI_TRY(batch_layer(m, b, il));
     pi_norm on = mk_norm(falcon ? 2 : 1, hp.norm_eps, m->glob[PI_T_OUTPUT_NORM], falcon ? &m->glob[PI_T_OUTPUT_NORM_B] : nullptr);
-    PI_TRY(batch_input(m->glob[PI_T_OUTPUT].type, b->x, T, d, &on, b->xa16, nullptr, st));
-    PI_TRY(pi_k_gemm_f16(batch_weight(m, m->glob[PI_T_OUTPUT]), hp.n_vocab, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->logits, nullptr, st));
+    if (m->q4_steps && m->glob[PI_T_OUTPUT].type == PI_TYPE_Q4_0) {
+        const auto wout = m->q4_split.at(&m->glob[PI_T_OUTPUT]);
+        PI_TRY(pi_k_norm_q8_blocks(b->x, T, d, &on, b->qa, b->da, b->sa, nullptr, st));
+        PI_TRY(pi_k_gemm_q4_t16(wout.quants, wout.scales, hp.n_vocab, d, b->qa, b->da, b->sa, T, PI_EPI_NONE, nullptr, nullptr, b->logits, st));
+    } else {
+        PI_TRY(pi_k_norm_round_f16(b->x, T, d, &on, b->xa16, nullptr, st));
+        PI_TRY(pi_k_gemm_f16(m->glob[PI_T_OUTPUT].dev, hp.n_vocab, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->logits, nullptr, st));
+    }
     PI_TRY(pi_k_argmax_batch(b->logits, hp.n_vocab, T, b->d_tokens, b->d_pos, b->d_step, b->d_out_tokens, b->max_steps, st));
     PI_TRY(pi_k_step_advance(b->d_step, st));
     return PI_OK;
@@ -189,18 +272,14 @@ int batch_step(pi_model * m) {
 
 namespace {
 
-// why the model cannot take multi-token steps, or null.  q4_too: Q4_0 matrices count as supported (lockstep decoding keeps an fp16
-// form of them; prompt chunks of up to 16 tokens of a Q4_0 model stay on the single-token path and its integer dot)
-const char * batch_unsupported(pi_model * m, bool q4_too = false) {
+// why the model cannot take multi-token steps on the F16 kernels, or null
+const char * batch_unsupported(pi_model * m) {
     const pi_hparams & hp = m->hp;
     if (m->hybrid) return "hybrid models decode one token at a time";
-    auto ok = [&](int ty) { return ty == PI_TYPE_F16 || (q4_too && ty == PI_TYPE_Q4_0); };
     for (int il = 0; il < hp.n_layer; ++il)
-        for (int k : {PI_T_WQKV, PI_T_WO, PI_T_FC1, PI_T_FC2, PI_T_FFN_UP, PI_T_FFN_GATE, PI_T_FFN_DOWN_T}) {
-            if (k == PI_T_FFN_GATE && hp.arch == PI_ARCH_FALCON) continue;
-            if (!ok(m->L(il, k).type)) return q4_too ? "multi-token steps need F16 or Q4_0 weights" : "multi-token steps need F16 weights";
-        }
-    if (!ok(m->glob[PI_T_TOK_EMBD].type) || !ok(m->glob[PI_T_OUTPUT].type)) return q4_too ? "multi-token steps need F16 or Q4_0 weights" : "multi-token steps need F16 weights";
+        for (int k : {PI_T_WQKV, PI_T_WO, PI_T_FC1, PI_T_FC2, PI_T_FFN_UP, PI_T_FFN_DOWN_T})
+            if (m->L(il, k).type != PI_TYPE_F16) return "multi-token steps need F16 weights, or Q4_0 matrices with F16 predictors";
+    if (m->glob[PI_T_TOK_EMBD].type != PI_TYPE_F16 || m->glob[PI_T_OUTPUT].type != PI_TYPE_F16) return "multi-token steps need F16 weights, or Q4_0 matrices with F16 predictors";
     if (hp.n_embd % 512 || (int)m->L(0, PI_T_FC1).ne1 % 128) return "n_embd % 512 == 0 and predictor rank % 128 == 0 required";
     return nullptr;
 }
@@ -228,6 +307,15 @@ BatchState * batch_alloc(pi_model * m, int T, bool with_caches) {
     b->att16 = m->alloc<__half>(n * d); b->hid16 = m->alloc<__half>(n * r);
     b->d_tokens = m->alloc<int32_t>(n); b->d_pos = m->alloc<int32_t>(n); b->d_step = m->alloc<int32_t>(1);
     b->d_out_tokens = m->alloc<int32_t>((size_t)b->max_steps * n); b->union_rows = m->alloc<int32_t>(ff); b->n_union = m->alloc<int32_t>(hp.n_layer);
+    if (m->L(0, PI_T_WQKV).type == PI_TYPE_Q4_0 && d % 32 == 0) {          // steps of a Q4_0 model on integer matrix cores
+        b->qa = m->alloc<unsigned char>((size_t)16 * d); b->qf = m->alloc<unsigned char>((size_t)16 * d);
+        b->da = m->alloc<float>((size_t)d / 32 * 16); b->df = m->alloc<float>((size_t)d / 32 * 16);
+        b->sa = m->alloc<int32_t>((size_t)d / 32 * 16); b->sf = m->alloc<int32_t>((size_t)d / 32 * 16);
+        b->h32 = m->alloc<float>((size_t)16 * ff); b->hq32 = m->alloc<float>((size_t)16 * ff);
+        ok = ok && b->qa && b->qf && b->da && b->df && b->sa && b->sf && b->h32 && b->hq32;
+        if (ok) ok = hipMemsetAsync(b->qa, 0, (size_t)16 * d, m->stream) == hipSuccess && hipMemsetAsync(b->qf, 0, (size_t)16 * d, m->stream) == hipSuccess &&
+                     hipMemsetAsync(b->hq32, 0, sizeof(float) * 16 * ff, m->stream) == hipSuccess && hipMemsetAsync(b->h32, 0, sizeof(float) * 16 * ff, m->stream) == hipSuccess;
+    }
     if (with_caches) {                                 // the dense form of a step's FFN (dense_ffn)
         b->up_out = m->alloc<float>(n * ff); b->gate_out = m->alloc<float>(n * ff); b->h16 = m->alloc<__half>(n * ff);
         ok = ok && b->up_out && b->gate_out && b->h16;
@@ -486,13 +574,14 @@ int prefill_wide_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) 
 }
 
 bool prefill_supported(pi_model * m) {
-    return !m->capture && batch_unsupported(m) == nullptr;
+    return !m->capture && (batch_unsupported(m) == nullptr || q4_steps_unsupported(m) == nullptr);
 }
 
 // T <= 16 consecutive prompt tokens of the model's own sequence in one step: the weights are read once for the chunk
 // (the prompt-phase counterpart of llama_decode with n_tokens > 1; the reference's batch kernels, ggml-cuda.cu:6994-7034)
 int prefill_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) {
     if (T < 1 || T > 16) return pi::fail(PI_E_ARG, "prefill_chunk: 1 <= T <= 16");
+    if (batch_unsupported(m) != nullptr) PI_TRY(ensure_q4_split(m));          // a Q4_0 model: the integer matrix-core route
     if (!m->prefill) {
         m->prefill = batch_alloc(m, 16, false);
         if (!m->prefill) return PI_E_HIP;
@@ -506,7 +595,8 @@ int prefill_chunk(pi_model * m, const int32_t * tokens, int T, int n_past) {
     PI_HIP_TRY(hipMemcpyAsync(b->d_tokens, tokens, sizeof(int32_t) * T, hipMemcpyHostToDevice, m->stream));
     PI_HIP_TRY(hipMemcpyAsync(b->d_pos, pos, sizeof(int32_t) * T, hipMemcpyHostToDevice, m->stream));
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
-    PI_TRY(pi_k_embed_batch(m->glob[PI_T_TOK_EMBD].dev, m->hp.n_embd, b->d_tokens, T, b->x, m->stream));
+    if (m->glob[PI_T_TOK_EMBD].type == PI_TYPE_Q4_0) PI_TRY(pi_k_embed_batch_q4(m->glob[PI_T_TOK_EMBD].dev, m->hp.n_embd, b->d_tokens, T, b->x, m->stream));
+    else PI_TRY(pi_k_embed_batch(m->glob[PI_T_TOK_EMBD].dev, m->hp.n_embd, b->d_tokens, T, b->x, m->stream));
     for (int il = 0; il < m->hp.n_layer; ++il) PI_TRY(batch_layer(m, b, il));
     return PI_OK;
 }
@@ -533,7 +623,7 @@ namespace {
 // after a step has completed: which layers run their FFN dense in the next one
 int choose_dense_layers(pi_model * m, BatchState * b) {
     const pi_hparams & hp = m->hp;
-    if (hp.n_ff % 128 || hp.n_embd % 128) return PI_OK;            // the dense mat-muls' shapes
+    if (hp.n_ff % 128 || hp.n_embd % 128 || m->q4_steps) return PI_OK;            // the dense mat-muls' shapes; the integer route has no dense form
     std::vector<int32_t> u(hp.n_layer);
     PI_TRY(pi_memcpy_d2h(u.data(), b->n_union, sizeof(int32_t) * hp.n_layer));
     for (int il = 0; il < hp.n_layer; ++il) {
@@ -566,25 +656,11 @@ int pi_model_batch_init(pi_model * m, int n_seq) {
     if (n_seq < 1 || n_seq > 16) return pi::fail(PI_E_ARG, "pi_model_batch_init: 1 <= n_seq <= 16");
     if (m->batch) return pi::fail(PI_E_STATE, "pi_model_batch_init: already initialised");
     if (!m->rope_table || !pi_k_attn_fused_supported(m->hd, m->hp.n_ctx)) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: head size or context outside the fused attention kernel (pi_k_attn_fused_supported)");
-    if (const char * why = batch_unsupported(m, true)) { pi::set_error(why); return PI_E_UNSUPPORTED; }
+    const bool q4_route = q4_steps_unsupported(m) == nullptr;
+    if (!q4_route) if (const char * why = batch_unsupported(m)) { pi::set_error(why); return PI_E_UNSUPPORTED; }
+    if (q4_route) PI_TRY(ensure_q4_split(m));
     BatchState * b = batch_alloc(m, n_seq, true);
     if (!b) return PI_E_HIP;
-    // Q4_0 matrices once more as fp16 rows: a lockstep step then runs on the same matrix-core kernels as an F16 model, with the
-    // activations passed through the CPU path's Q8_0 blocks (3.6 times the bytes of the Q4_0 form, which this device has room for)
-    auto expand = [&](Tensor & t) -> int {
-        if (t.type != PI_TYPE_Q4_0 || !t.dev) return PI_OK;
-        if (t.ne0 % 32) return pi::fail(PI_E_UNSUPPORTED, "pi_model_batch_init: Q4_0 rows must be whole blocks");
-        __half * w = m->alloc<__half>((size_t)t.ne0 * t.ne1);
-        if (!w) return PI_E_HIP;
-        PI_TRY(pi_k_dequant_q4_f16(t.dev, nullptr, nullptr, nullptr, (int)t.ne1, (int)t.ne0, w, m->stream));
-        b->as_f16[&t] = w;
-        return PI_OK;
-    };
-    int rc = expand(m->glob[PI_T_OUTPUT]);
-    for (int il = 0; il < m->hp.n_layer && rc == PI_OK; ++il)
-        for (int k : {PI_T_WQKV, PI_T_WO, PI_T_FC1, PI_T_FC2, PI_T_FFN_UP, PI_T_FFN_GATE, PI_T_FFN_DOWN_T})
-            if (rc == PI_OK) rc = expand(m->L(il, k));
-    if (rc != PI_OK) { delete b; return rc; }
     const size_t T = n_seq;
     PI_HIP_TRY(hipMemsetAsync(b->k_cache, 0, sizeof(__half) * b->cache_seq_stride * T, m->stream));
     PI_HIP_TRY(hipMemsetAsync(b->v_cache, 0, sizeof(__half) * b->cache_seq_stride * T, m->stream));

@@ -7,6 +7,7 @@
 #include <hip/hip_runtime.h>
 #include <hip/hip_fp16.h>
 
+#include <unordered_map>
 #include <vector>
 
 struct Tensor {
@@ -69,6 +70,11 @@ struct pi_model {
     BatchState * prefill = nullptr;       // step buffers for prompt chunks of the model's own sequence
     BatchState * prefill_wide = nullptr;  // the same for chunks of up to 512 tokens (dense mat-muls, weights read once per chunk)
     pi_gemm_lib * gemm_lib = nullptr;     // hipBLASLt plans of those mat-muls (PI_PREFILL_GEMM=own keeps them on this library's kernel, 128 tokens a chunk)
+    // multi-token steps of a Q4_0 model on integer matrix cores: every Q4_0 matrix once more as 16-byte-aligned quants and fp16
+    // scales (pi_k_q4_split), made at the first such step; q4_steps says the model takes that route
+    struct Q4Split { const void * quants; const void * scales; };
+    std::unordered_map<const Tensor *, Q4Split> q4_split;
+    bool q4_steps = false;
     std::vector<__half *> down_rows;      // per layer: the down projection with the neurons contiguous ([n_embd][n_ff]), made at the first wide chunk
                                           // (null for Q4_0 and hybrid layers, whose matrices are expanded into the chunk's scratch instead)
 

@@ -844,6 +844,15 @@ __global__ void step_advance_kernel(int32_t * step) { if (threadIdx.x == 0) *ste
 
 }  // namespace
 
+namespace pi {
+void launch_union_active(const unsigned char * row_any, int ff, uint32_t * words, int32_t * union_rows, int32_t * n_union, hipStream_t st) {
+    hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, row_any, ff, words, union_rows, n_union);
+}
+void launch_batch_reduce(const float * partial, int n_groups, int T, int cols, int epilogue, const float * add1, const float * add2, float * out, hipStream_t st) {
+    hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, partial, n_groups, T, cols, epilogue, add1, add2, out);
+}
+}  // namespace pi
+
 extern "C" {
 
 int pi_k_norm_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, void * out_plain_f16, pi_stream_t stream) {

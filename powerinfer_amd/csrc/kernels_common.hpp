@@ -294,3 +294,9 @@ struct pi_workspace {
     int            pf_parts, pf_words;   // partial vectors and activity words the last fused F16 launch left for its reduction
 };
 constexpr int kAxpyGroups = 32;
+
+// launches of kernels_batch.hip that the Q4_0 step kernels reuse
+namespace pi {
+void launch_union_active(const unsigned char * row_any, int ff, uint32_t * words, int32_t * union_rows, int32_t * n_union, hipStream_t st);
+void launch_batch_reduce(const float * partial, int n_groups, int T, int cols, int epilogue, const float * add1, const float * add2, float * out, hipStream_t st);
+}

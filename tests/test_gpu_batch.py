@@ -318,6 +318,136 @@ def test_batch_sparse_ffn_matches_oracle(shape, has_gate, T):
     L.pi_workspace_destroy(ws)
 
 
+def q4_split_on_device(pl, L, wq4, rows, cols):
+    dw = pl.DevBuf(host=wq4)
+    qs, ds = pl.DevBuf(rows * cols // 2), pl.DevBuf(rows * cols // 32 * 2)
+    pl.check(L.pi_k_q4_split(dw.ptr, rows, cols, qs.ptr, ds.ptr, None), "q4 split")
+    return qs, ds
+
+
+def q8_blocks_on_device(pl, L, x, norm=None):
+    import ctypes as C
+    T, cols = x.shape
+    dx = pl.DevBuf(host=np.ascontiguousarray(x, np.float32))
+    q, d, s = pl.DevBuf(16 * cols), pl.DevBuf(cols // 32 * 16 * 4), pl.DevBuf(cols // 32 * 16 * 4)
+    keep, na = [], pl.Norm(0, 0.0, None, None)
+    if norm is not None:
+        kind, eps, nw, nb = norm
+        bw = pl.DevBuf(host=nw) if nw is not None else None
+        bb = pl.DevBuf(host=nb) if nb is not None else None
+        keep += [bw, bb]
+        na = pl.Norm(kind, eps, bw.ptr if bw else None, bb.ptr if bb else None)
+    pl.check(L.pi_k_norm_q8_blocks(dx.ptr, T, cols, C.byref(na), q.ptr, d.ptr, s.ptr, None, None), "q8 blocks")
+    pl.sync()
+    return q, d, s
+
+
+@pytest.mark.parametrize("rows,cols,T", [(64, 256, 1), (520, 512, 5), (4096, 4096, 16), (12288, 4096, 16), (32000, 4096, 7), (1030, 1024, 16), (5120, 5120, 16)])
+def test_gemm_q4_t16_matches_oracle(rows, cols, T):
+    """The Q4_0 mat-mul of a step of up to 16 tokens on integer matrix cores against the reference's CPU mat-mul (Q4_0 rows times
+    the Q8_0 blocks of the activations): the block sums are exact integers on both sides, what differs is the order in which the
+    128 scaled block sums of a row are added in fp32, hence 1e-5.  One and two row tiles per workgroup, a row count off the tile,
+    a single token, the residual epilogue."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    rng = np.random.default_rng(rows + cols + T)
+    wq = synth.encode((rng.standard_normal((rows, cols)) * 0.02).astype(np.float32), ol.Q4_0)
+    x = rng.standard_normal((T, cols)).astype(np.float32)
+    a1 = rng.standard_normal((T, rows)).astype(np.float32)
+    want = np.zeros((T, rows), np.float32)
+    assert ol.oracle().pio_mul_mat(ol.Q4_0, P(wq), rows, cols, P(x), T, P(want), 8) == 0
+    qs, ds = q4_split_on_device(pl, L, wq, rows, cols)
+    q, d, s = q8_blocks_on_device(pl, L, x)
+    y, d1 = pl.DevBuf(T * rows * 4), pl.DevBuf(host=a1)
+    pl.check(L.pi_memset(y.ptr, 0xFF, y.nbytes), "memset")
+    pl.check(L.pi_k_gemm_q4_t16(qs.ptr, ds.ptr, rows, cols, q.ptr, d.ptr, s.ptr, T, pl.EPI_NONE, None, None, y.ptr, None), "gemm q4")
+    pl.sync()
+    assert rel_err(y.download(np.float32).reshape(T, rows), want) < 1e-5
+    pl.check(L.pi_k_gemm_q4_t16(qs.ptr, ds.ptr, rows, cols, q.ptr, d.ptr, s.ptr, T, pl.EPI_ADD, d1.ptr, None, y.ptr, None), "gemm q4")
+    pl.sync()
+    assert rel_err(y.download(np.float32).reshape(T, rows), want + a1) < 1e-5
+    assert L.pi_k_gemm_q4_t16(qs.ptr, ds.ptr, rows, cols, q.ptr, d.ptr, s.ptr, 17, pl.EPI_NONE, None, None, y.ptr, None) != 0       # T > 16
+    assert L.pi_k_gemm_q4_t16(qs.ptr, ds.ptr, rows, cols, q.ptr, d.ptr, s.ptr, T, pl.EPI_ADD, None, None, y.ptr, None) != 0         # residual missing
+
+
+@pytest.mark.parametrize("kind", [1, 2])
+def test_norm_q8_blocks_match_the_reference_quantiser(kind):
+    """Norm + Q8_0 blocks of a step's rows against the oracle's norm followed by quantize_row_q8_0: quants and scales bit for bit,
+    and the block sums the mat-mul subtracts."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    O = ol.oracle()
+    T, cols = 5, 4096
+    rng = np.random.default_rng(kind)
+    x = rng.standard_normal((T, cols)).astype(np.float32) * 3
+    nw = (1 + 0.1 * rng.standard_normal(cols)).astype(np.float32)
+    nb = (0.1 * rng.standard_normal(cols)).astype(np.float32) if kind == 2 else None
+    q, d, s = q8_blocks_on_device(pl, L, x, (kind, 1e-5, nw, nb))
+    normed = np.zeros_like(x)
+    (O.pio_rms_norm if kind == 1 else O.pio_norm)(P(x), cols, T, 1e-5, P(normed))
+    normed = normed * nw
+    if nb is not None:
+        normed = normed + nb
+    normed = np.ascontiguousarray(normed, np.float32)
+    blocks = np.zeros((T, cols // 32, 34), np.uint8)
+    for t in range(T):
+        O.pio_quantize_row_q8_0(P(normed[t]), P(blocks[t]), cols)
+    want_d = blocks[:, :, :2].copy().view(np.float16).reshape(T, cols // 32).astype(np.float32)
+    want_q = blocks[:, :, 2:].copy().view(np.int8).reshape(T, cols)
+    # the quants sit in the integer MFMA's operand layout: [block][group g][token][8 bytes], the group's bytes being elements 4g .. 4g + 3
+    # and 16 + 4g .. 16 + 4g + 3 of the block
+    raw = q.download(np.int8).reshape(cols // 32, 4, 16, 2, 4)                # [blk][g][t][half][byte]
+    got_q = raw.transpose(2, 0, 3, 1, 4).reshape(16, cols)[:T]               # [t][blk][half][g][byte] = element 16 * half + 4 * g + byte
+    got_d = d.download(np.float32).reshape(cols // 32, 16).T[:T]
+    got_s = s.download(np.int32).reshape(cols // 32, 16).T[:T]
+    assert np.array_equal(got_d, want_d)
+    assert (got_q != want_q).mean() < 1e-3           # a value on a rounding boundary after the norm's last bit
+    assert np.array_equal(got_s, 8 * got_q.reshape(T, cols // 32, 32).astype(np.int32).sum(-1))
+
+
+@pytest.mark.parametrize("shape,has_gate,T", [((4096, 11008, 1024), True, 16), ((4096, 11008, 1024), False, 5), ((1024, 1024, 128), True, 3)])
+def test_batch_sparse_ffn_q4_matches_oracle(shape, has_gate, T):
+    """The sparse FFN of a step on Q4_0 weights (7B shape, 16 tokens; a gate-less layer; a small one): union list, up/gate dots of the
+    union rows on integer matrix cores, h under the predictor's mask, its Q8_0 values, and the down projection over the union rows
+    on fp32 matrix cores, against the CPU kernels under the same logits (GGML_OP_MUL_MAT_SPARSE, GGML_OP_AXPY with Q4_0 rows)."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    O = ol.oracle()
+    d, ff, r = shape
+    Lr = synth.make_ffn_layer(seed=31 + T, d=d, ff=ff, r=r, wtype=ol.Q4_0, has_gate=has_gate, mean_rate=0.11, T=T)
+    x = Lr["x"]
+    ws = L.pi_workspace_create(ff, d)
+    assert ws
+    fc1, fc2 = pl.DevBuf(host=Lr["fc1"]), pl.DevBuf(host=Lr["fc2"])
+    upq, ups = q4_split_on_device(pl, L, Lr["up"], ff, d)
+    dnq, dns = q4_split_on_device(pl, L, Lr["down_t"], ff, d)
+    gq, gs = q4_split_on_device(pl, L, Lr["gate"], ff, d) if has_gate else (None, None)
+    xn = gpu_norm_round(pl, L, x)
+    q, dd, s = q8_blocks_on_device(pl, L, x)
+    hidden, hid16 = pl.DevBuf(T * r * 4), pl.DevBuf(T * r * 2)
+    logits, out = pl.DevBuf(T * ff * 4), pl.DevBuf(T * d * 4)
+    union, n_union = pl.DevBuf(ff * 4), pl.DevBuf.zeros(4)
+    h, hq = pl.DevBuf.zeros(16 * ff * 4), pl.DevBuf.zeros(16 * ff * 4)
+    resid = np.random.default_rng(3).standard_normal((T, d)).astype(np.float32)
+    dres = pl.DevBuf(host=resid)
+    pl.check(L.pi_k_gemm_f16(fc1.ptr, r, d, xn.ptr, T, pl.EPI_RELU, None, None, hidden.ptr, hid16.ptr, None), "fc1")
+    for rep in range(2):                                       # the second pass finds the first one's h in the scratch buffers
+        pl.check(L.pi_k_batch_predictor_fc2(fc2.ptr, ff, r, hid16.ptr, T, 0.0, logits.ptr, ws, None), "fc2")
+        pl.check(L.pi_k_batch_sparse_ffn_q4(logits.ptr, T, ff, 0.0, upq.ptr, ups.ptr, gq.ptr if gq else None, gs.ptr if gs else None, dnq.ptr, dns.ptr, d,
+                                            q.ptr, dd.ptr, s.ptr, pl.EPI_ADD, dres.ptr, None, out.ptr, h.ptr, hq.ptr, union.ptr, n_union.ptr, ws, None), "ffn q4")
+    pl.sync()
+    lg = logits.download(np.float32).reshape(T, ff)
+    n = int(n_union.download(np.int32)[0])
+    assert np.array_equal(union.download(np.int32, n), np.nonzero((~(lg < 0.0)).any(0))[0])
+    got = out.download(np.float32).reshape(T, d) - resid
+    hh = h.download(np.float32).reshape(16, ff)
+    for t in range(T):
+        ou = ol.ffn_under_logits(O, d, ff, ol.Q4_0, has_gate, Lr["up"], Lr["gate"], Lr["down_t"], x[t], lg[t], 0.0)
+        assert rel_err(np.where(~(lg[t] < 0.0), hh[t], 0), ou["h"]) < 1e-5
+        assert rel_err(got[t], ou["out"]) < 1e-4
+    L.pi_workspace_destroy(ws)
+
+
 @pytest.mark.parametrize("thr", [1e9, -1e9])
 def test_batch_sparse_ffn_none_and_all_active(thr):
     """Empty union (zero output, residual only) and the full union (every row of every matrix read once: the dense FFN)."""
@@ -355,16 +485,13 @@ def test_batched_decode_matches_per_sequence_oracle(arch, wtype):
     """Four sequences with different prompts advance in lockstep (examples/batched/batched.cpp).  Sequences do not interact,
     so sequence t of the batch must reproduce a single-sequence run on the same tokens: against the CPU oracle (teacher
     forced, the trajectory-level criteria of the single-sequence tests) and against this library's own batch-1 engine.
-    A Q4_0 model steps on the fp16 form of its matrices ((q - 8) * d, made once at batch_init) with the activations passed
-    through the CPU path's Q8_0 blocks.  Both factors are then rounded to fp16 (2^-11 each), which moves a few per cent of the next
-    stage's int8 roundings by one step; the single-token path, whose integer dots reproduce the CPU's activations bit for bit,
-    sits at a median distance of 0 from the oracle on these models, the lockstep path at about 1e-2.  Its bound is therefore
-    3e-2 on the median and 2e-1 on single steps (the reference's own batch kernel for Q4_0 rows, dequantize_mul_mat_batch_sparse,
-    ggml-cuda.cu:4757-4758 and 5390-5397, multiplies dequantised weights with unquantised activations: a larger difference of the
-    same kind), on a model whose predictors and greedy choices keep a margin."""
+    A Q4_0 model steps on the integer matrix-core kernels (one MFMA per pair of a Q4_0 weight block and a Q8_0 activation block,
+    the CPU path's arithmetic): same criteria on the median; single steps of a Q4_0 model may sit further out (the single-token
+    path itself is up to 4e-2 from the oracle on these models: one int8 rounding step of an activation is a visible share of a dot
+    product, tests/test_oracle_math.py::test_q4_reference_departs_from_itself_beyond_the_logit_tolerance), so they are held to 1e-1."""
     from powerinfer_amd.model import Model
     q4 = wtype != synth.F16
-    hp = synth.hparams(arch, seed=5, n_ctx=64, wtype=wtype, **(dict(pred_margin=True, head_pair=2048) if q4 else {}))
+    hp = synth.hparams(arch, seed=5, n_ctx=64, wtype=wtype, **(dict(pred_margin=True, head_pair=2048) if q4 else {}))          # Q4_0: a margin model, so that no neuron flips on a rounding step
     model = synth.make_model(hp)
     n_seq, n_steps = 4, 10
     rng = np.random.default_rng(11)
@@ -390,9 +517,9 @@ def test_batched_decode_matches_per_sequence_oracle(arch, wtype):
             same += int(batch_next[s, t] == tok_o)
         om.close()
     errs_o, errs_g = np.array(errs_o), np.array(errs_g)
-    assert np.median(errs_o) < (3e-2 if q4 else 1e-2), errs_o
-    assert np.median(errs_g) < (3e-2 if q4 else 1e-2), errs_g
-    assert not q4 or max(errs_o.max(), errs_g.max()) < 2e-1, (errs_o, errs_g)
+    assert np.median(errs_o) < 1e-2, errs_o
+    assert np.median(errs_g) < 1e-2, errs_g
+    assert not q4 or max(errs_o.max(), errs_g.max()) < 1e-1, (errs_o, errs_g)
     assert same >= 0.9 * n_seq * n_steps, same
     # greedy continuation on the device equals stepping the same state by hand
     gm2 = Model(hp).load(model)
@@ -527,9 +654,9 @@ def test_batched_decode_13b_width_16_sequences(moving):
 @pytest.mark.timeout(600)
 def test_batched_decode_7b_q4_width_16_sequences():
     """A Q4_0 model at the 7B width (d 4096, ff 11008, predictor rank 1024, vocab 32000, two layers), sixteen sequences in lockstep
-    on the fp16 form of the matrices: per sequence against the CPU oracle, teacher forced, with the Q4_0 bounds of
-    test_batched_decode_matches_per_sequence_oracle (median 3e-2, single steps 2e-1, nine greedy tokens in ten equal), then the
-    free-running continuation on the device against stepping the same state by hand."""
+    on the integer matrix-core kernels: per sequence against the CPU oracle, teacher forced (median of the logit distances 1e-2,
+    single steps 1e-1, nine greedy tokens in ten equal), then the free-running continuation on the device against stepping the
+    same state by hand."""
     from powerinfer_amd.model import Model
     hp = synth.hparams("llama-7b", n_layer=2, n_ctx=32, seed=SEED_7B_Q4_BATCH, wtype=synth.Q4_0, pred_margin=True, head_pair=2048)
     model = synth.make_model(hp)
@@ -549,7 +676,7 @@ def test_batched_decode_7b_q4_width_16_sequences():
     for om in oms:
         om.close()
     errs = np.array(errs)
-    assert np.median(errs) < 3e-2 and errs.max() < 2e-1, errs
+    assert np.median(errs) < 1e-2 and errs.max() < 1e-1, errs
     assert same >= 0.9 * n_seq * n_steps, same
     assert np.all(gm.batch_union() > 0)
     gen, _ = gm.batch_generate(4)
@@ -635,15 +762,19 @@ def test_batch_init_rejects_unsupported_models():
     m.close()
 
 
+@pytest.mark.parametrize("wtype", [synth.F16, synth.Q4_0], ids=["f16", "q4_0"])
 @pytest.mark.parametrize("arch", ["llama-tiny", "falcon-tiny"])
-def test_prompt_chunks_match_token_by_token(arch):
+def test_prompt_chunks_match_token_by_token(arch, wtype):
     """A prompt handed over in one call is evaluated in chunks of up to 16 tokens (weights read once per chunk, causal attention
     inside the chunk); the result must agree with the CPU oracle evaluating the whole prompt as one batch (llama_decode with
     n_tokens > 1) and with feeding the same tokens one at a time.  As in the single-token model tests one predictor logit on
     the threshold can flip a neuron in either path (a few percent of one layer's output with these random predictors), so
-    the criterion is the median over several prompts."""
+    the criterion is the median over several prompts.  A Q4_0 model's chunks run on the integer matrix-core kernels
+    (pi_k_gemm_q4_t16, pi_k_batch_sparse_ffn_q4): same criteria, on a model whose predictors keep a margin - without one the
+    int8 rounding steps of Q4_0 activations flip neurons in either path, and the single-token path, whose dots are the CPU's bit
+    for bit, is then as far from the oracle's batch evaluation (1.4e-2 median on this model) as the chunks are (1.5e-2)."""
     from powerinfer_amd.model import Model
-    hp = synth.hparams(arch, seed=12, n_ctx=64)
+    hp = synth.hparams(arch, seed=12, n_ctx=64, wtype=wtype, **(dict(pred_margin=True, head_pair=2048) if wtype != synth.F16 else {}))
     model = synth.make_model(hp)
     rng = np.random.default_rng(4)
     err_oracle, err_single, err_after = [], [], []

@@ -128,15 +128,10 @@ __global__ __launch_bounds__(kBlock) void gemm_q4_t16_kernel(const uint32_t * __
     for (int m = 0; m < NM; ++m)
 #pragma unroll
         for (int r = 0; r < 4; ++r) acc[m][r] = 0.0f;
-    // the activations' scales and block sums for every block: [blk][16 tokens], staged once per workgroup
+    // LDS: the activations' scales and block sums for every block, [blk][16 tokens]
     extern __shared__ __align__(16) unsigned char q4_smem[];
     float * sdx = reinterpret_cast<float *>(q4_smem);
     int * ssx = reinterpret_cast<int *>(q4_smem + (size_t)nblk * 64);
-    for (int k = threadIdx.x; k < nblk * 4; k += kBlock) {
-        reinterpret_cast<pi_u32x4 *>(sdx)[k] = pi_ld16(dx + (size_t)k * 4);
-        reinterpret_cast<pi_u32x4 *>(ssx)[k] = pi_ld16(sx8 + (size_t)k * 4);
-    }
-    __syncthreads();
     const unsigned long * qx64 = reinterpret_cast<const unsigned long *>(qx) + g * 16 + i;      // + block * 64
     const int ngroups = nblk / kQ4Group;
     struct Loads { pi_u32x4 w0[NM], w1[NM], wd[NM]; unsigned long a[kQ4Group]; };
@@ -175,15 +170,25 @@ __global__ __launch_bounds__(kBlock) void gemm_q4_t16_kernel(const uint32_t * __
             }
         }
     };
-    // the next group's loads travel while this one is multiplied
-    Loads cur, nxt;
-    int grp = wave;
-    if (grp < ngroups) fetch(cur, grp);
-    for (; grp < ngroups; grp += kWavesPerBlock) {
-        const bool more = grp + kWavesPerBlock < ngroups;
-        if (more) fetch(nxt, grp + kWavesPerBlock);
-        multiply(cur, grp);
-        if (more) cur = nxt;
+    // A wave's groups (wave, wave + 4, ...) go in rounds of four: all loads of a round are issued before its first multiply, so
+    // a row of 4096 columns costs one trip to memory per wave instead of four; the first round's loads are already under way
+    // while the workgroup stages the scales.
+    constexpr int kRound = 4;
+    Loads L[kRound];
+#pragma unroll
+    for (int u = 0; u < kRound; ++u) if (wave + u * kWavesPerBlock < ngroups) fetch(L[u], wave + u * kWavesPerBlock);
+    for (int k = threadIdx.x; k < nblk * 4; k += kBlock) {
+        reinterpret_cast<pi_u32x4 *>(sdx)[k] = pi_ld16(dx + (size_t)k * 4);
+        reinterpret_cast<pi_u32x4 *>(ssx)[k] = pi_ld16(sx8 + (size_t)k * 4);
+    }
+    __syncthreads();
+    for (int g0 = wave; g0 < ngroups; g0 += kRound * kWavesPerBlock) {
+        if (g0 != wave) {
+#pragma unroll
+            for (int u = 0; u < kRound; ++u) if (g0 + u * kWavesPerBlock < ngroups) fetch(L[u], g0 + u * kWavesPerBlock);
+        }
+#pragma unroll
+        for (int u = 0; u < kRound; ++u) if (g0 + u * kWavesPerBlock < ngroups) multiply(L[u], g0 + u * kWavesPerBlock);
     }
 #pragma unroll
     for (int m = 0; m < NM; ++m)
@@ -267,7 +272,7 @@ __global__ __launch_bounds__(kBlock) void batch_axpy_q4_kernel(const uint32_t * 
     for (int e = 0; e < 8; ++e) acc[e] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
     const int nquads = (nu + 3) / 4;
     const int stride = kQ4AxpyGroups * kWavesPerBlock;
-    // quad q of this wave's u-th slot: (blockIdx.y * 4 + wave) + (it * kQ4AxpyUnroll + u) * stride
+    // quad of this wave's u-th slot in iteration it: (blockIdx.y * 4 + wave) + (it * kQ4AxpyUnroll + u) * stride
     int rows_next[kQ4AxpyUnroll];
     auto rows_of = [&](int it, int * out) {
 #pragma unroll
@@ -276,26 +281,33 @@ __global__ __launch_bounds__(kBlock) void batch_axpy_q4_kernel(const uint32_t * 
             out[u] = k < nu ? union_rows[k] : -1;
         }
     };
-    rows_of(0, rows_next);
-    for (int it = 0; ((int)blockIdx.y * kWavesPerBlock + wave) + it * kQ4AxpyUnroll * stride < nquads; ++it) {
-        int n[kQ4AxpyUnroll];
-        uint32_t w[kQ4AxpyUnroll]; float dw[kQ4AxpyUnroll], a[kQ4AxpyUnroll];
+    // two iterations ahead: the union rows; one ahead: the rows' quants, scales and h values
+    struct Quad { uint32_t w[kQ4AxpyUnroll]; float dw[kQ4AxpyUnroll], a[kQ4AxpyUnroll]; };
+    auto fetch = [&](Quad & Q, const int * n) {
 #pragma unroll
         for (int u = 0; u < kQ4AxpyUnroll; ++u) {
-            n[u] = rows_next[u];
             const size_t row = (size_t)(n[u] < 0 ? 0 : n[u]);
-            w[u] = qs[(row * nblk + (size_t)blockIdx.x * 4) * 4 + i];
-            dw[u] = n[u] < 0 ? 0.0f : pi_f16_from_bits(ds[row * nblk + cb]);
-            a[u] = n[u] < 0 ? 0.0f : hq[row * kBtMaxT + i];        // token i (entries of tokens beyond T are stale and feed discarded rows)
+            Q.w[u] = qs[(row * nblk + (size_t)blockIdx.x * 4) * 4 + i];
+            Q.dw[u] = n[u] < 0 ? 0.0f : pi_f16_from_bits(ds[row * nblk + cb]);
+            Q.a[u] = n[u] < 0 ? 0.0f : hq[row * kBtMaxT + i];      // token i (entries of tokens beyond T are stale and feed discarded rows)
         }
-        rows_of(it + 1, rows_next);
+    };
+    const int q0 = (int)blockIdx.y * kWavesPerBlock + wave;
+    rows_of(0, rows_next);
+    Quad cur, nxt;
+    fetch(cur, rows_next);
+    rows_of(1, rows_next);
+    for (int it = 0; q0 + it * kQ4AxpyUnroll * stride < nquads; ++it) {
+        fetch(nxt, rows_next);                                     // past the end: rows_of gave -1, the loads read row 0 and count as zeros
+        rows_of(it + 2, rows_next);
 #pragma unroll
         for (int u = 0; u < kQ4AxpyUnroll; ++u)
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const int nib = e < 4 ? (int)((w[u] >> (8 * e)) & 0xF) : (int)((w[u] >> (8 * (e - 4) + 4)) & 0xF);
-                acc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a[u], __fmul_rn(dw[u], (float)(nib - 8)), acc[e], 0, 0, 0);
+                const int nib = e < 4 ? (int)((cur.w[u] >> (8 * e)) & 0xF) : (int)((cur.w[u] >> (8 * (e - 4) + 4)) & 0xF);
+                acc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.a[u], __fmul_rn(cur.dw[u], (float)(nib - 8)), acc[e], 0, 0, 0);
             }
+        cur = nxt;
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e)

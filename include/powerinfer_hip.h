@@ -301,8 +301,8 @@ PI_API int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float thre
 /* Prompt chunks on this library's own mat-mul kernel (the prompt phase of llama_decode, where the reference goes through cuBLAS and
  * its batch kernels, ggml-cuda.cu:7662-7756, 6994-7034): pi_k_gemm_tile_f16 is pi_k_gemm_f16 for chunks of any length, both operands
  * tiled through LDS (64 columns per stage, two stages in LDS and two more in flight): cols % 64 == 0, operands 16-byte aligned.
- * tile = 0 lets the library choose the output tile from the number of workgroups it gives the device; 128128, 96128, 128064, 64128,
- * 64064 (weight rows x 1000 + tokens) forces one, for tests and measurement.  pi_k_ffn_h_f16 forms h_f16[t][n] = fp16(relu(gate) * up)
+ * tile = 0 lets the library choose the output tile from the number of workgroups it gives the device; 256128, 192128 (eight waves per
+ * workgroup), 128128, 96128, 128064, 64128, 64064 (four waves; weight rows x 1000 + tokens) forces one, for tests and measurement.  pi_k_ffn_h_f16 forms h_f16[t][n] = fp16(relu(gate) * up)
  * where !(logits[t][n] < threshold) and 0 elsewhere from dense gate/up products (gate may be NULL: relu(up)); pi_k_transpose_f16 writes
  * out[cols][rows] of an fp16 matrix in[rows][cols] (the down projection of a chunk is a mat-mul over the neurons and wants them
  * contiguous). */

@@ -281,12 +281,14 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
 // ---------------------------------------------------------------------------------------------------
 constexpr int kGtBK = 64;                        // columns per stage
 constexpr int kGtRow = kGtBK * 2;                // bytes per LDS row
-template <int BM, int BN>
-__global__ __launch_bounds__(kBlock, (BM + BN <= 192 ? 3 : 2)) void gemm_tile_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
+template <int BM, int BN, int WGM = 2, int WGN = 2>      // output tile and the waves' grid over it (WGM x WGN waves)
+__global__ __launch_bounds__(64 * WGM * WGN, (WGM * WGN > 4 ? 1 : BM + BN <= 192 ? 3 : 2)) void gemm_tile_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
                                                                   int nx, int ny, int epi, const float * __restrict__ add1, const float * __restrict__ add2,
                                                                   float * __restrict__ y, __half * __restrict__ y16) {
-    constexpr int WM = BM / 2, WN = BN / 2, MT = WM / 16, NT = WN / 16;
-    constexpr int ACH = BM * kGtBK * 2 / 16 / kBlock, BCH = BN * kGtBK * 2 / 16 / kBlock;      // 16-byte chunks per thread and stage
+    constexpr int kThreads = 64 * WGM * WGN;
+    constexpr int WM = BM / WGM, WN = BN / WGN, MT = WM / 16, NT = WN / 16;
+    constexpr int ACH = BM * kGtBK * 2 / 16 / kThreads, BCH = BN * kGtBK * 2 / 16 / kThreads;  // 16-byte chunks per thread and stage
+    static_assert(WM % 16 == 0 && WN % 16 == 0 && ACH * kThreads * 16 == BM * kGtBK * 2 && BCH * kThreads * 16 == BN * kGtBK * 2, "tile does not divide among the waves");
     extern __shared__ __align__(16) unsigned char smem[];
     unsigned char * sa = smem;                                     // [2][BM][kGtRow]
     unsigned char * sb = smem + 2 * BM * kGtRow;                   // [2][BN][kGtRow]
@@ -296,19 +298,19 @@ __global__ __launch_bounds__(kBlock, (BM + BN <= 192 ? 3 : 2)) void gemm_tile_f1
     if (tx >= nx) return;
     const int row0 = tx * BM, tok0 = ty * BN;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, i = lane & 15, g = lane >> 4;
-    const int wm = wave & 1, wn = wave >> 1;
+    const int wm = wave % WGM, wn = wave / WGM;
     auto lds_off = [](int r, int kc) { return r * kGtRow + ((kc ^ (r & 7)) * 16); };
     const __half * ga[ACH]; const __half * gb[BCH];
     int la[ACH], lb[BCH];
 #pragma unroll
     for (int j = 0; j < ACH; ++j) {
-        const int kc = tid % 8, r = j * 32 + tid / 8;
+        const int kc = tid % 8, r = j * (kThreads / 8) + tid / 8;
         const int rr = row0 + r < rows ? row0 + r : rows - 1;
         ga[j] = W + (size_t)rr * cols + kc * 8; la[j] = lds_off(r, kc);
     }
 #pragma unroll
     for (int j = 0; j < BCH; ++j) {
-        const int kc = tid % 8, r = j * 32 + tid / 8;
+        const int kc = tid % 8, r = j * (kThreads / 8) + tid / 8;
         const int tt = tok0 + r < T ? tok0 + r : T - 1;
         gb[j] = xn + (size_t)tt * cols + kc * 8; lb[j] = lds_off(r, kc);
     }
@@ -892,11 +894,11 @@ int pi_k_gemm_f16(const void * W, int rows, int cols, const void * xn_f16, int T
 }
 
 // Output tiles the kernel is built for (weight rows x tokens per workgroup); two workgroups share a compute unit.
-// Output tiles the kernel is built for (weight rows x tokens per workgroup).
-constexpr int kGtNShapes = 5;
-static const int kGtShapes[kGtNShapes][2] = {{128, 128}, {96, 128}, {128, 64}, {64, 128}, {64, 64}};
+// Output tiles the kernel is built for (weight rows x tokens per workgroup); the first two run eight waves, one workgroup per unit.
+constexpr int kGtNShapes = 7;
+static const int kGtShapes[kGtNShapes][2] = {{256, 128}, {192, 128}, {128, 128}, {96, 128}, {128, 64}, {64, 128}, {64, 64}};
 // Relative time per output of one workgroup (LDS and L2 bytes per MFMA grow as the tile shrinks); measured on 7B and 13B shapes.
-static const float kGtCost[kGtNShapes] = {1.00f, 1.05f, 1.25f, 1.25f, 1.45f};
+static const float kGtCost[kGtNShapes] = {0.95f, 0.95f, 1.00f, 1.05f, 1.25f, 1.25f, 1.45f};
 
 // The device spreads workgroups over its compute units, so a launch lasts as long as the unit with the most workgroups:
 // ceil(workgroups / units) tiles one after the other (or side by side at the same total rate).
@@ -923,21 +925,23 @@ int pi_k_gemm_tile_f16(const void * W, int rows, int cols, const void * xn_f16, 
     int shape = -1;
     if (tile == 0) shape = gt_choose(rows, T, pi::compute_units());
     else for (int s = 0; s < kGtNShapes; ++s) if (tile == kGtShapes[s][0] * 1000 + kGtShapes[s][1]) shape = s;
-    if (shape < 0) return pi::fail(PI_E_ARG, "pi_k_gemm_tile_f16: tile must be 0 or one of 128128, 96128, 128064, 64128, 64064");
-#define PI_GEMM_TILE(BM, BN) do {                                                                                                         \
+    if (shape < 0) return pi::fail(PI_E_ARG, "pi_k_gemm_tile_f16: tile must be 0 or one of 256128, 192128, 128128, 96128, 128064, 64128, 64064");
+#define PI_GEMM_TILE(BM, BN, WGM, WGN) do {                                                                                               \
         const int nx = (rows + BM - 1) / BM, ny = (T + BN - 1) / BN;                                                                      \
         const size_t sh = (size_t)2 * (BM + BN) * kGtRow;                                                                                 \
         static bool raised = false;                                                                                                       \
-        if (!raised && sh > 64 * 1024) { PI_HIP_TRY(hipFuncSetAttribute((const void *)gemm_tile_f16_kernel<BM, BN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh)); raised = true; } \
-        hipLaunchKernelGGL((gemm_tile_f16_kernel<BM, BN>), dim3(8 * ((nx + 7) / 8) * ny), dim3(kBlock), sh, st, (const __half *)W, (const __half *)xn_f16, T, rows, cols,   \
+        if (!raised && sh > 64 * 1024) { PI_HIP_TRY(hipFuncSetAttribute((const void *)gemm_tile_f16_kernel<BM, BN, WGM, WGN>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)sh)); raised = true; } \
+        hipLaunchKernelGGL((gemm_tile_f16_kernel<BM, BN, WGM, WGN>), dim3(8 * ((nx + 7) / 8) * ny), dim3(64 * WGM * WGN), sh, st, (const __half *)W, (const __half *)xn_f16, T, rows, cols,   \
                            nx, ny, epilogue, add1, add2, y, (__half *)y_f16);                                                             \
     } while (0)
     switch (shape) {
-        case 0: PI_GEMM_TILE(128, 128); break;
-        case 1: PI_GEMM_TILE(96, 128); break;
-        case 2: PI_GEMM_TILE(128, 64); break;
-        case 3: PI_GEMM_TILE(64, 128); break;
-        default: PI_GEMM_TILE(64, 64); break;
+        case 0: PI_GEMM_TILE(256, 128, 4, 2); break;
+        case 1: PI_GEMM_TILE(192, 128, 4, 2); break;
+        case 2: PI_GEMM_TILE(128, 128, 2, 2); break;
+        case 3: PI_GEMM_TILE(96, 128, 2, 2); break;
+        case 4: PI_GEMM_TILE(128, 64, 2, 2); break;
+        case 5: PI_GEMM_TILE(64, 128, 2, 2); break;
+        default: PI_GEMM_TILE(64, 64, 2, 2); break;
     }
 #undef PI_GEMM_TILE
     return pi::check_launch("pi_k_gemm_tile_f16");

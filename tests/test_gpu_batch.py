@@ -57,7 +57,7 @@ def test_gemm_matches_oracle(rows, cols, T):
     assert np.array_equal(dy16.download(np.float16).reshape(T, rows), got.astype(np.float16))
 
 
-@pytest.mark.parametrize("tile", [0, 128128, 96128, 128064, 64128, 64064])
+@pytest.mark.parametrize("tile", [0, 256128, 192128, 128128, 96128, 128064, 64128, 64064])
 @pytest.mark.parametrize("rows,cols,T", [(3000, 5120, 300), (4104, 4096, 512), (1024, 11008, 130), (520, 512, 17), (64, 64, 1), (130, 192, 129),
                                          (2048, 1024, 40), (12288, 4096, 512)])
 def test_gemm_tile_matches_oracle(rows, cols, T, tile):

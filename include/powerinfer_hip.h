@@ -620,7 +620,26 @@ PI_API int pi_model_batch_generate(pi_model * m, int n_steps, int32_t * out_toke
 PI_API int pi_model_batch_kv_seq_rm(pi_model * m, int seq, int p0, int p1);
 PI_API int pi_model_batch_kv_seq_shift(pi_model * m, int seq, int p0, int p1, int delta);
 PI_API int pi_model_batch_kv_seq_cp(pi_model * m, int src, int dst, int p0, int p1);
-PI_API int pi_model_batch_union(pi_model * m, int32_t * n_union_per_layer); /* Dense cross-over of lockstep decoding (the reference leaves its batch-sparse kernels for a plain mat-mul when a step has many
+/* One KV cache whose cells are shared between sequences: llama_kv_cell / llama_kv_cache (llama.cpp:1381-1420), llama_kv_cache_find_slot (:1683-1730),
+ * _seq_rm / _seq_cp / _seq_keep / _clear (:1745-1822), the visibility mask of llama_decode (:6506-6531) and the cell range a step looks
+ * at (:1735-1743, 6842).  A cell holds a position and a set of sequence ids (0..31, one bit each); a step of up to 16 tokens takes a run
+ * of free cells found from the ring's head, every token attends the cells of its (first) sequence at positions not beyond its own;
+ * _seq_cp makes the cells of src visible to dst without copying anything (a prompt evaluated once serves every continuation).
+ * F16 models, or Q4_0 models with F16 predictors, with every neuron on the GPU; n_cells a multiple of 32.  Tokens of one sequence
+ * come in ascending positions within a step.  _decode returns PI_E_STATE when no run of free cells is left (the reference's
+ * llama_decode returns 1), each token's greedy next token and, if logits_out != NULL, its logits [n_tokens][n_vocab].
+ * _state copies the cells' positions (-1: free) and sequence bit sets and the ring's head out (tests, monitoring); returns n_cells.
+ * Position shifts (llama_kv_cache_seq_shift) exist for the per-sequence caches only (pi_model_kv_seq_shift, pi_model_batch_kv_seq_shift). */
+PI_API int pi_model_kv_cells_init(pi_model * m, int n_cells);
+PI_API int pi_model_kv_cells_decode(pi_model * m, const int32_t * tokens, const int32_t * positions, const uint32_t * seq_masks, int n_tokens,
+                                    int32_t * next_tokens, float * logits_out);
+PI_API int pi_model_kv_cells_seq_rm(pi_model * m, int seq, int p0, int p1);
+PI_API int pi_model_kv_cells_seq_cp(pi_model * m, int src, int dst, int p0, int p1);
+PI_API int pi_model_kv_cells_seq_keep(pi_model * m, int seq);
+PI_API int pi_model_kv_cells_clear(pi_model * m);
+PI_API int pi_model_kv_cells_state(pi_model * m, int32_t * cell_pos, uint32_t * cell_seq, int32_t * head);
+PI_API int pi_model_batch_union(pi_model * m, int32_t * n_union_per_layer);   /* union sizes of the last step, [n_layer] */
+/* Dense cross-over of lockstep decoding (the reference leaves its batch-sparse kernels for a plain mat-mul when a step has many
  * tokens, ggml-cuda.cu:8787-8814, 7717-7756; here the switch is the union of the sequences' active rows): a layer whose union in the
  * last step exceeded fraction * n_ff computes its FFN in the next step as dense gate / up mat-muls, h with the predictor's mask, and a
  * dense down mat-mul (one more copy of that layer's down projection with the neurons contiguous, made on first use).  Default 0.9:
@@ -629,7 +648,6 @@ PI_API int pi_model_batch_union(pi_model * m, int32_t * n_union_per_layer); /* D
  * pi_model_batch_dense_layers: how many layers the next step runs dense. */
 PI_API int pi_model_batch_set_dense_above(pi_model * m, float fraction);
 PI_API int pi_model_batch_dense_layers(pi_model * m);
-  /* union sizes of the last step, [n_layer] */
 
 /* Before pi_model_finalize: layers with a gpu_bucket keep their non-resident rows in pinned host memory and the GPU reads the
  * rows of active neurons from there itself (pi_k_pred_upgate_q4_split) instead of handing those neurons to host threads; the

@@ -5,6 +5,8 @@
 #include "engine_internal.hpp"
 #include "runtime.hpp"
 
+#include <math.h>
+#include <stdint.h>
 #include <stdlib.h>
 #include <algorithm>
 #include <unordered_map>
@@ -26,6 +28,16 @@ struct BatchState {
     int32_t *d_tokens = nullptr, *d_pos = nullptr, *d_step = nullptr, *d_out_tokens = nullptr, *union_rows = nullptr, *n_union = nullptr;
     float *up_out = nullptr, *gate_out = nullptr;      // wide prompt chunks: dense gate/up products [T][n_ff]
     __half *h16 = nullptr;                             //                     and the FFN's hidden vector
+    // One KV cache whose cells are shared between sequences (llama_kv_cache, llama.cpp:1683-1848): a cell holds a position and a set of
+    // sequence ids; K cells [n_layer][n_cells][n_embd_gqa] and transposed values [n_layer][n_embd_gqa][n_cells] as the reference lays them
+    // out.  Host side: the cells' positions (-1: free), sequence sets (bit s) and the ring's search start.
+    bool unified = false;
+    int n_cells = 0, head = 0, n_kv = 0;
+    std::vector<int32_t> cell_pos;
+    std::vector<uint32_t> cell_seq;
+    __half *cells_k = nullptr, *cells_v = nullptr;
+    float *cells_mask = nullptr, *kq_scale = nullptr;  // device: [16][n_cells] mask rows of a step, 1 / sqrt(head size)
+    int slot[16] = {0};                                // the cells the step's tokens were given
     // steps of a Q4_0 model on integer matrix cores: Q8_0 blocks of the attention-side and of the FFN-side mat-mul input (int8 quants
     // [16][n_embd], scales and 8 * sums [n_embd / 32][16]), h and the values its Q8_0 blocks keep [16][n_ff]
     void *qa = nullptr, *qf = nullptr; float *da = nullptr, *df = nullptr; int32_t *sa = nullptr, *sf = nullptr;
@@ -74,6 +86,23 @@ int chunk_attention(pi_model * m, BatchState * b, int T, size_t kv_off) {
 int batch_input(int wtype, const float * x, int T, int cols, const pi_norm * norm, void * out16, void * plain16, hipStream_t st) {
     if (wtype == PI_TYPE_Q4_0) return pi_k_norm_q8_round_f16(x, T, cols, norm, out16, plain16, st);
     return pi_k_norm_round_f16(x, T, cols, norm, out16, plain16, st);
+}
+
+// attention of a step whose tokens live in the shared-cell cache: token t's K / V rows go to cell slot[t], and it attends the cells its
+// mask row leaves visible (same sequence, position not beyond its own: llama.cpp:6506-6531).  One launch per token, in the order
+// of the batch: a token may attend an earlier token of the same step, whose rows are then already in place.
+int cells_attention(pi_model * m, BatchState * b, int il, int T) {
+    const pi_hparams & hp = m->hp;
+    const int d = hp.n_embd, gqa = m->gqa, stride = d + 2 * gqa;
+    const bool falcon = hp.arch == PI_ARCH_FALCON;
+    __half * k = b->cells_k + (size_t)il * b->n_cells * gqa;
+    __half * v = b->cells_v + (size_t)il * gqa * b->n_cells;
+    for (int t = 0; t < T; ++t)
+        PI_TRY(pi_k_attn_ggml(b->qkv + (size_t)t * stride, b->qkv + (size_t)t * stride + d, b->qkv + (size_t)t * stride + d + gqa, b->d_pos + t,
+                              falcon ? 2 : 0, m->theta_scale, m->freq_scale, 1.0f, k, v, hp.n_head, hp.n_head_kv, m->hd, b->n_cells, b->n_kv, b->slot[t],
+                              b->kq_scale, b->cells_mask + (size_t)t * b->n_cells, b->att + (size_t)t * d, m->stream));
+    const pi_norm plain{0, 0.0f, nullptr, nullptr};
+    return pi_k_norm_round_f16(b->att, T, d, &plain, b->att16, nullptr, m->stream);
 }
 
 // why the model's multi-token steps cannot run on the integer matrix-core kernels, or null
@@ -140,7 +169,9 @@ int batch_layer_q4(pi_model * m, BatchState * b, int il) {
     }
     const auto wqkv = W(PI_T_WQKV), wo = W(PI_T_WO);
     PI_TRY(pi_k_gemm_q4_t16(wqkv.quants, wqkv.scales, d + 2 * gqa, d, b->qa, b->da, b->sa, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, st));
-    if (b->prefill)
+    if (b->unified)
+        PI_TRY(cells_attention(m, b, il, T));
+    else if (b->prefill)
         PI_TRY(chunk_attention(m, b, T, kv_off));
     else
         PI_TRY(pi_k_attn_fused_batch(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
@@ -199,7 +230,9 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     else an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
     PI_TRY(pi_k_norm_round_f16(x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));       // Falcon: the predictor reads the raw layer input
     PI_TRY(pi_k_gemm_f16(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr, st));
-    if (b->prefill)
+    if (b->unified)
+        PI_TRY(cells_attention(m, b, il, T));
+    else if (b->prefill)
         PI_TRY(chunk_attention(m, b, T, kv_off));
     else
         PI_TRY(pi_k_attn_fused_batch(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
@@ -224,7 +257,7 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     // Measured on the 13B shape, 40 layers, 16 sequences (ms per step, union kernels / dense): union 0.41 of n_ff 7.46 / 9.18,
     // 0.61 8.27 / 9.26, 0.75 8.63 / 9.24, 0.91 9.40 / 9.29, 0.99 9.60 / 9.38 - the union kernels lose only beyond 0.9.  The choice
     // is made from the union the previous step measured (the count below keeps that statistic alive while the layer runs dense).
-    if (!b->prefill && il < (int)b->dense_ffn.size() && b->dense_ffn[il]) {
+    if (!b->prefill && !b->unified && il < (int)b->dense_ffn.size() && b->dense_ffn[il]) {
         PI_TRY(pi_k_batch_union_count(ff, b->union_rows, b->n_union + il, m->ws, st));
         PI_TRY(pi_k_gemm_f16(up.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->up_out, nullptr, st));
         if (!falcon) PI_TRY(pi_k_gemm_f16(gate.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->gate_out, nullptr, st));
@@ -245,8 +278,7 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     return PI_OK;
 }
 
-int batch_step(pi_model * m) {
-    BatchState * b = m->batch;
+int batch_step(pi_model * m, BatchState * b) {
     const pi_hparams & hp = m->hp;
     const int T = b->n_seq, d = hp.n_embd;
     const bool falcon = hp.arch == PI_ARCH_FALCON;
@@ -611,6 +643,7 @@ void batch_destroy(pi_model * m) {
         m->prefill_wide = nullptr;
     }
     if (m->gemm_lib) { (void)pi_gemm_lib_destroy(m->gemm_lib); m->gemm_lib = nullptr; }
+    if (m->cells) { delete m->cells; m->cells = nullptr; }
     if (!m->batch) return;
     if (m->batch->graph_exec) (void)hipGraphExecDestroy(m->batch->graph_exec);
     if (m->batch->graph) (void)hipGraphDestroy(m->batch->graph);
@@ -683,7 +716,7 @@ int pi_model_batch_decode(pi_model * m, const int32_t * tokens, const int32_t * 
     PI_HIP_TRY(hipMemcpyAsync(b->d_pos, positions, sizeof(int32_t) * b->n_seq, hipMemcpyHostToDevice, m->stream));
     PI_HIP_TRY(hipMemsetAsync(b->d_step, 0, 4, m->stream));
     PI_HIP_TRY(hipStreamSynchronize(m->stream));          // the host arrays may be pageable: finish the copies before returning control
-    PI_TRY(batch_step(m));
+    PI_TRY(batch_step(m, m->batch));
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
     PI_TRY(choose_dense_layers(m, b));
     if (next_tokens) PI_TRY(pi_memcpy_d2h(next_tokens, b->d_tokens, sizeof(int32_t) * b->n_seq));
@@ -711,7 +744,7 @@ int pi_model_batch_generate(pi_model * m, int n_steps, int32_t * out_tokens, flo
     if (use_graph && !b->graph_exec) {
         b->graph_dense = b->dense_ffn;
         PI_HIP_TRY(hipStreamBeginCapture(m->stream, hipStreamCaptureModeThreadLocal));
-        const int rc = batch_step(m);
+        const int rc = batch_step(m, m->batch);
         hipGraph_t g = nullptr;
         const hipError_t e = hipStreamEndCapture(m->stream, &g);
         if (rc != PI_OK) { if (g) (void)hipGraphDestroy(g); return rc; }
@@ -722,7 +755,7 @@ int pi_model_batch_generate(pi_model * m, int n_steps, int32_t * out_tokens, flo
     PI_HIP_TRY(hipEventRecord(m->ev0, m->stream));
     for (int s = 0; s < n_steps; ++s) {
         if (use_graph) PI_HIP_TRY(hipGraphLaunch(b->graph_exec, m->stream));
-        else PI_TRY(batch_step(m));
+        else PI_TRY(batch_step(m, m->batch));
     }
     PI_HIP_TRY(hipEventRecord(m->ev1, m->stream));
     PI_HIP_TRY(hipStreamSynchronize(m->stream));
@@ -772,6 +805,157 @@ int pi_model_batch_kv_seq_cp(pi_model * m, int src, int dst, int p0, int p1) {
     const int32_t n = p1;
     PI_TRY(pi_memcpy_h2d(b->d_pos + dst, &n, 4));
     return p1;
+}
+
+// ---- one KV cache with cells shared between sequences ----------------------------------------------------------------------------
+int pi_model_kv_cells_init(pi_model * m, int n_cells) {
+    if (!m || !m->finalized) return pi::fail(PI_E_STATE, "pi_model_kv_cells_init: model not finalized");
+    if (m->cells) return pi::fail(PI_E_STATE, "pi_model_kv_cells_init: already initialised");
+    if (n_cells < 32 || n_cells % 32) return pi::fail(PI_E_ARG, "pi_model_kv_cells_init: n_cells must be a multiple of 32, at least 32");
+    const bool q4_route = q4_steps_unsupported(m) == nullptr;
+    if (!q4_route) if (const char * why = batch_unsupported(m)) { pi::set_error(why); return PI_E_UNSUPPORTED; }
+    if (!pi_k_attn_ggml_supported(m->hd, n_cells, n_cells)) return pi::fail(PI_E_UNSUPPORTED, "pi_model_kv_cells_init: head size or cell count outside pi_k_attn_ggml");
+    if (q4_route) PI_TRY(ensure_q4_split(m));
+    BatchState * b = batch_alloc(m, 16, false);
+    if (!b) return PI_E_HIP;
+    b->unified = true;
+    b->n_cells = n_cells;
+    b->cell_pos.assign(n_cells, -1);
+    b->cell_seq.assign(n_cells, 0u);
+    const size_t per_layer = (size_t)n_cells * m->gqa;
+    b->cells_k = m->alloc<__half>(per_layer * m->hp.n_layer); b->cells_v = m->alloc<__half>(per_layer * m->hp.n_layer);
+    b->cells_mask = m->alloc<float>((size_t)16 * n_cells); b->kq_scale = m->alloc<float>(1);
+    if (!b->cells_k || !b->cells_v || !b->cells_mask || !b->kq_scale) { delete b; return PI_E_HIP; }
+    const float scale = 1.0f / sqrtf((float)m->hd);
+    PI_HIP_TRY(hipMemsetAsync(b->cells_k, 0, sizeof(__half) * per_layer * m->hp.n_layer, m->stream));
+    PI_HIP_TRY(hipMemsetAsync(b->cells_v, 0, sizeof(__half) * per_layer * m->hp.n_layer, m->stream));
+    PI_HIP_TRY(hipMemcpyAsync(b->kq_scale, &scale, 4, hipMemcpyHostToDevice, m->stream));
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    m->cells = b;
+    return PI_OK;
+}
+
+// llama_kv_cache_find_slot (llama.cpp:1683-1730): n contiguous free cells, searched from the ring's head, wrapping once
+static bool cells_find_slot(BatchState * b, int n) {
+    const int n_ctx = b->n_cells;
+    if (n > n_ctx) return false;
+    int n_tested = 0;
+    while (true) {
+        if (b->head + n > n_ctx) { n_tested += n_ctx - b->head; b->head = 0; continue; }
+        bool found = true;
+        for (int i = 0; i < n; ++i)
+            if (b->cell_pos[b->head + i] >= 0) { found = false; b->head += i + 1; n_tested += i + 1; break; }
+        if (found) return true;
+        if (n_tested >= n_ctx) return false;
+    }
+}
+
+int pi_model_kv_cells_decode(pi_model * m, const int32_t * tokens, const int32_t * positions, const uint32_t * seq_masks, int n_tokens,
+                             int32_t * next_tokens, float * logits_out) {
+    if (!m || !m->cells) return pi::fail(PI_E_STATE, "pi_model_kv_cells_decode: pi_model_kv_cells_init first");
+    if (!tokens || !positions || !seq_masks || n_tokens < 1 || n_tokens > 16) return pi::fail(PI_E_ARG, "pi_model_kv_cells_decode: 1 <= n_tokens <= 16");
+    BatchState * b = m->cells;
+    for (int t = 0; t < n_tokens; ++t) {
+        if (tokens[t] < 0 || tokens[t] >= m->hp.n_vocab) return pi::fail(PI_E_ARG, "pi_model_kv_cells_decode: token id out of range");
+        if (positions[t] < 0 || seq_masks[t] == 0) return pi::fail(PI_E_ARG, "pi_model_kv_cells_decode: a token needs a position and at least one sequence");
+        // a token may attend an earlier token of the same step (its rows are written first), never a later one
+        for (int u = 0; u < t; ++u)
+            if ((seq_masks[u] & seq_masks[t]) && positions[u] > positions[t])
+                return pi::fail(PI_E_ARG, "pi_model_kv_cells_decode: tokens of one sequence must come in ascending positions");
+    }
+    if (!cells_find_slot(b, n_tokens)) return pi::fail(PI_E_STATE, "pi_model_kv_cells_decode: no run of free cells for the step (llama_kv_cache_find_slot failed)");
+    for (int t = 0; t < n_tokens; ++t) {
+        b->slot[t] = b->head + t;
+        b->cell_pos[b->head + t] = positions[t];
+        b->cell_seq[b->head + t] |= seq_masks[t];
+    }
+    // the cells a step looks at: up to the last one in use, at least 32 (llama_kv_cache_cell_max, llama.cpp:1735-1743, 6842)
+    int cell_max = 0;
+    for (int i = b->n_cells - 1; i > 0; --i) if (b->cell_pos[i] >= 0 && b->cell_seq[i]) { cell_max = i + 1; break; }
+    b->n_kv = std::min(b->n_cells, std::max(32, cell_max));
+    // mask rows (llama.cpp:6506-6531): a cell is hidden from token t unless it belongs to t's sequence and its position is not beyond t's
+    std::vector<float> mask((size_t)n_tokens * b->n_cells, 0.0f);
+    for (int t = 0; t < n_tokens; ++t) {
+        const int seq = __builtin_ctz(seq_masks[t]);               // the reference masks by the token's first sequence id
+        for (int i = 0; i < b->n_kv; ++i)
+            if (!(b->cell_seq[i] >> seq & 1u) || b->cell_pos[i] > positions[t]) mask[(size_t)t * b->n_cells + i] = -INFINITY;
+    }
+    b->n_seq = n_tokens;
+    PI_HIP_TRY(hipMemcpyAsync(b->d_tokens, tokens, sizeof(int32_t) * n_tokens, hipMemcpyHostToDevice, m->stream));
+    PI_HIP_TRY(hipMemcpyAsync(b->d_pos, positions, sizeof(int32_t) * n_tokens, hipMemcpyHostToDevice, m->stream));
+    PI_HIP_TRY(hipMemcpyAsync(b->cells_mask, mask.data(), sizeof(float) * mask.size(), hipMemcpyHostToDevice, m->stream));
+    PI_HIP_TRY(hipMemsetAsync(b->d_step, 0, 4, m->stream));
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    PI_TRY(batch_step(m, b));
+    PI_HIP_TRY(hipStreamSynchronize(m->stream));
+    b->head += n_tokens;                                          // llama_decode moves the ring's head past the step's cells and wraps it
+    if (b->head >= b->n_cells) b->head = 0;                       // (llama.cpp:6936-6943)
+    if (next_tokens) PI_TRY(pi_memcpy_d2h(next_tokens, b->d_tokens, sizeof(int32_t) * n_tokens));
+    if (logits_out) PI_TRY(pi_memcpy_d2h(logits_out, b->logits, sizeof(float) * (size_t)n_tokens * m->hp.n_vocab));
+    return PI_OK;
+}
+
+// llama_kv_cache_seq_rm (llama.cpp:1757-1785): seq < 0 removes the range from every sequence; p1 < 0: to the end
+int pi_model_kv_cells_seq_rm(pi_model * m, int seq, int p0, int p1) {
+    if (!m || !m->cells || seq >= 32) return pi::fail(PI_E_ARG, "pi_model_kv_cells_seq_rm: bad arguments");
+    BatchState * b = m->cells;
+    int new_head = b->n_cells;
+    if (p0 < 0) p0 = 0;
+    if (p1 < 0) p1 = INT32_MAX;
+    for (int i = 0; i < b->n_cells; ++i) {
+        if (b->cell_pos[i] >= p0 && b->cell_pos[i] < p1) {
+            if (seq < 0) b->cell_seq[i] = 0;
+            else if (b->cell_seq[i] >> seq & 1u) b->cell_seq[i] &= ~(1u << seq);
+            else continue;
+            if (b->cell_seq[i] == 0) { b->cell_pos[i] = -1; if (new_head == b->n_cells) new_head = i; }
+        }
+    }
+    if (new_head != b->n_cells) b->head = new_head;
+    return PI_OK;
+}
+
+// llama_kv_cache_seq_cp (llama.cpp:1787-1803): the cells of src in [p0, p1) join dst as well; nothing is copied
+int pi_model_kv_cells_seq_cp(pi_model * m, int src, int dst, int p0, int p1) {
+    if (!m || !m->cells || src < 0 || dst < 0 || src >= 32 || dst >= 32) return pi::fail(PI_E_ARG, "pi_model_kv_cells_seq_cp: bad arguments");
+    BatchState * b = m->cells;
+    if (p0 < 0) p0 = 0;
+    if (p1 < 0) p1 = INT32_MAX;
+    b->head = 0;
+    for (int i = 0; i < b->n_cells; ++i)
+        if ((b->cell_seq[i] >> src & 1u) && b->cell_pos[i] >= p0 && b->cell_pos[i] < p1) b->cell_seq[i] |= 1u << dst;
+    return PI_OK;
+}
+
+// llama_kv_cache_seq_keep (llama.cpp:1805-1822)
+int pi_model_kv_cells_seq_keep(pi_model * m, int seq) {
+    if (!m || !m->cells || seq < 0 || seq >= 32) return pi::fail(PI_E_ARG, "pi_model_kv_cells_seq_keep: bad arguments");
+    BatchState * b = m->cells;
+    int new_head = b->n_cells;
+    for (int i = 0; i < b->n_cells; ++i) {
+        if (!(b->cell_seq[i] >> seq & 1u)) { b->cell_pos[i] = -1; b->cell_seq[i] = 0; if (new_head == b->n_cells) new_head = i; }
+        else b->cell_seq[i] = 1u << seq;
+    }
+    if (new_head != b->n_cells) b->head = new_head;
+    return PI_OK;
+}
+
+// llama_kv_cache_clear (llama.cpp:1745-1751)
+int pi_model_kv_cells_clear(pi_model * m) {
+    if (!m || !m->cells) return pi::fail(PI_E_ARG, "pi_model_kv_cells_clear: bad arguments");
+    BatchState * b = m->cells;
+    std::fill(b->cell_pos.begin(), b->cell_pos.end(), -1);
+    std::fill(b->cell_seq.begin(), b->cell_seq.end(), 0u);
+    b->head = 0;
+    return PI_OK;
+}
+
+int pi_model_kv_cells_state(pi_model * m, int32_t * cell_pos, uint32_t * cell_seq, int32_t * head) {
+    if (!m || !m->cells) return pi::fail(PI_E_ARG, "pi_model_kv_cells_state: bad arguments");
+    BatchState * b = m->cells;
+    if (cell_pos) memcpy(cell_pos, b->cell_pos.data(), sizeof(int32_t) * b->n_cells);
+    if (cell_seq) memcpy(cell_seq, b->cell_seq.data(), sizeof(uint32_t) * b->n_cells);
+    if (head) *head = b->head;
+    return b->n_cells;
 }
 
 int pi_model_batch_union(pi_model * m, int32_t * n_union_per_layer) {

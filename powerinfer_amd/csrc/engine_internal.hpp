@@ -67,6 +67,7 @@ struct pi_model {
     std::vector<std::vector<float>>   neuron_rate;     // per layer, as given (empty: none)
     std::vector<std::vector<int32_t>> ffn_perm;
     BatchState * batch = nullptr;         // per-sequence caches and step buffers of batched decoding
+    BatchState * cells = nullptr;         // the KV cache with cells shared between sequences and its step buffers (pi_model_kv_cells_*)
     BatchState * prefill = nullptr;       // step buffers for prompt chunks of the model's own sequence
     BatchState * prefill_wide = nullptr;  // the same for chunks of up to 512 tokens (dense mat-muls, weights read once per chunk)
     pi_gemm_lib * gemm_lib = nullptr;     // hipBLASLt plans of those mat-muls (PI_PREFILL_GEMM=own keeps them on this library's kernel, 128 tokens a chunk)

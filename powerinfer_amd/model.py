@@ -48,6 +48,13 @@ def _declare(L):
     L.pi_model_batch_union.restype, L.pi_model_batch_union.argtypes = i, [vp, vp]
     L.pi_model_batch_set_dense_above.restype, L.pi_model_batch_set_dense_above.argtypes = i, [vp, C.c_float]
     L.pi_model_batch_dense_layers.restype, L.pi_model_batch_dense_layers.argtypes = i, [vp]
+    L.pi_model_kv_cells_init.restype, L.pi_model_kv_cells_init.argtypes = i, [vp, i]
+    L.pi_model_kv_cells_decode.restype, L.pi_model_kv_cells_decode.argtypes = i, [vp, vp, vp, vp, i, vp, vp]
+    L.pi_model_kv_cells_seq_rm.restype, L.pi_model_kv_cells_seq_rm.argtypes = i, [vp, i, i, i]
+    L.pi_model_kv_cells_seq_cp.restype, L.pi_model_kv_cells_seq_cp.argtypes = i, [vp, i, i, i, i]
+    L.pi_model_kv_cells_seq_keep.restype, L.pi_model_kv_cells_seq_keep.argtypes = i, [vp, i]
+    L.pi_model_kv_cells_clear.restype, L.pi_model_kv_cells_clear.argtypes = i, [vp]
+    L.pi_model_kv_cells_state.restype, L.pi_model_kv_cells_state.argtypes = i, [vp, vp, vp, vp]
     L.pi_model_time_section.restype, L.pi_model_time_section.argtypes = i, [vp, i, i, C.POINTER(C.c_float), C.POINTER(C.c_int)]
 
 
@@ -57,7 +64,9 @@ ENGINE_SYMBOLS = ["pi_model_create", "pi_model_free", "pi_model_set_tensor", "pi
                   "pi_model_step_active", "pi_model_time_section",
                   "pi_model_batch_init", "pi_model_batch_decode", "pi_model_batch_generate", "pi_model_batch_union",
                   "pi_model_batch_set_dense_above", "pi_model_batch_dense_layers",
-                  "pi_model_batch_kv_seq_rm", "pi_model_batch_kv_seq_shift", "pi_model_batch_kv_seq_cp"]
+                  "pi_model_batch_kv_seq_rm", "pi_model_batch_kv_seq_shift", "pi_model_batch_kv_seq_cp",
+                  "pi_model_kv_cells_init", "pi_model_kv_cells_decode", "pi_model_kv_cells_seq_rm", "pi_model_kv_cells_seq_cp",
+                  "pi_model_kv_cells_seq_keep", "pi_model_kv_cells_clear", "pi_model_kv_cells_state"]
 
 
 def _type_of(a, hint):
@@ -216,6 +225,50 @@ class Model:
         n = self.L.pi_model_batch_kv_seq_cp(self.h, src, dst, p0, p1)
         check(min(n, 0), "pi_model_batch_kv_seq_cp")
         return n
+
+    # ---- one KV cache with cells shared between sequences (llama_kv_cache) ----
+    def kv_cells_init(self, n_cells):
+        check(self.L.pi_model_kv_cells_init(self.h, int(n_cells)), "pi_model_kv_cells_init")
+        self.n_cells = int(n_cells)
+
+    def kv_cells_decode(self, tokens, positions, seqs, want_logits=True):
+        """One step of up to 16 tokens.  seqs[t]: a sequence id, or a list of ids the token's cell belongs to with the lowest first
+        (the token attends the cells of its first sequence, as the reference masks by seq_id[t][0]).  Returns (greedy next token per
+        token, logits [n_tokens][n_vocab] or None)."""
+        tokens = np.ascontiguousarray(tokens, np.int32)
+        positions = np.ascontiguousarray(positions, np.int32)
+        masks = np.zeros(tokens.size, np.uint32)
+        for t, sq in enumerate(seqs):
+            ids = [int(sq)] if np.isscalar(sq) else [int(v) for v in sq]
+            if min(ids) != ids[0]:
+                raise pl.PiError("kv_cells_decode: list a token's lowest sequence id first")
+            for v in ids:
+                masks[t] |= np.uint32(1 << v)
+        nxt = np.empty(tokens.size, np.int32)
+        logits = np.empty((tokens.size, self.hp.n_vocab), np.float32) if want_logits else None
+        check(self.L.pi_model_kv_cells_decode(self.h, tokens.ctypes.data_as(C.c_void_p), positions.ctypes.data_as(C.c_void_p),
+                                              masks.ctypes.data_as(C.c_void_p), int(tokens.size), nxt.ctypes.data_as(C.c_void_p),
+                                              logits.ctypes.data_as(C.c_void_p) if want_logits else None), "pi_model_kv_cells_decode")
+        return nxt, logits
+
+    def kv_cells_seq_rm(self, seq, p0, p1):
+        check(self.L.pi_model_kv_cells_seq_rm(self.h, seq, p0, p1), "pi_model_kv_cells_seq_rm")
+
+    def kv_cells_seq_cp(self, src, dst, p0, p1):
+        check(self.L.pi_model_kv_cells_seq_cp(self.h, src, dst, p0, p1), "pi_model_kv_cells_seq_cp")
+
+    def kv_cells_seq_keep(self, seq):
+        check(self.L.pi_model_kv_cells_seq_keep(self.h, seq), "pi_model_kv_cells_seq_keep")
+
+    def kv_cells_clear(self):
+        check(self.L.pi_model_kv_cells_clear(self.h), "pi_model_kv_cells_clear")
+
+    def kv_cells_state(self):
+        """(positions [n_cells] (-1: free), sequence bit sets [n_cells], head of the ring)"""
+        pos, seq, head = np.empty(self.n_cells, np.int32), np.empty(self.n_cells, np.uint32), C.c_int32(0)
+        n = self.L.pi_model_kv_cells_state(self.h, pos.ctypes.data_as(C.c_void_p), seq.ctypes.data_as(C.c_void_p), C.byref(head))
+        check(min(n, 0), "pi_model_kv_cells_state")
+        return pos, seq, int(head.value)
 
     def batch_union(self):
         out = np.empty(self.hp.n_layer, np.int32)

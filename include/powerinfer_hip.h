@@ -448,6 +448,13 @@ PI_API int pi_k_attn_ggml_supported(int hd, int n_ctx, int n_kv);
 PI_API int pi_k_attn_ggml(const float * q, const float * k, const float * v, const int32_t * pos, int mode, float theta_scale, float freq_scale, float mscale,
                           void * k_cache, void * v_cache, int n_head, int n_head_kv, int hd, int n_ctx, int n_kv, int cell,
                           const float * kq_scale, const float * kq_mask, float * out, pi_stream_t stream);
+/* the same for a step of T <= 16 tokens whose rows go to the consecutive cells cell0 .. cell0 + T - 1 (the run llama_kv_cache_find_slot
+ * returns): token u's projections at qkv + u * qkv_stride ([q | k | v]), its position pos[u], its mask row at kq_mask + u * mask_stride,
+ * its result at out + u * out_stride.  Every token sees the step's other new cells where its mask row allows, as if the whole batch
+ * had been stored first (llm_build_kv_store runs ahead of llm_build_kqv, llama.cpp:4383-4418, 4764-4850). */
+PI_API int pi_k_attn_ggml_step(const float * qkv, int qkv_stride, const int32_t * pos, int mode, float theta_scale, float freq_scale, float mscale,
+                               void * k_cache, void * v_cache, int n_head, int n_head_kv, int hd, int n_ctx, int n_kv, int T, int cell0,
+                               const float * kq_scale, const float * kq_mask, int mask_stride, float * out, int out_stride, pi_stream_t stream);
 
 /* per-sequence pieces of a batched step: sequence t owns token t, position pos[t] and the cache at t * cache_seq_stride
  * (elements), out_f16 (optional) receives fp16(out); pi_k_argmax_batch picks each sequence's next token (first maximum wins), stores it in tokens[t], adds 1 to
@@ -625,8 +632,7 @@ PI_API int pi_model_batch_kv_seq_cp(pi_model * m, int src, int dst, int p0, int 
  * at (:1735-1743, 6842).  A cell holds a position and a set of sequence ids (0..31, one bit each); a step of up to 16 tokens takes a run
  * of free cells found from the ring's head, every token attends the cells of its (first) sequence at positions not beyond its own;
  * _seq_cp makes the cells of src visible to dst without copying anything (a prompt evaluated once serves every continuation).
- * F16 models, or Q4_0 models with F16 predictors, with every neuron on the GPU; n_cells a multiple of 32.  Tokens of one sequence
- * come in ascending positions within a step.  _decode returns PI_E_STATE when no run of free cells is left (the reference's
+ * F16 models, or Q4_0 models with F16 predictors, with every neuron on the GPU; n_cells a multiple of 32.  _decode returns PI_E_STATE when no run of free cells is left (the reference's
  * llama_decode returns 1), each token's greedy next token and, if logits_out != NULL, its logits [n_tokens][n_vocab].
  * _state copies the cells' positions (-1: free) and sequence bit sets and the ring's head out (tests, monitoring); returns n_cells.
  * Position shifts (llama_kv_cache_seq_shift) exist for the per-sequence caches only (pi_model_kv_seq_shift, pi_model_batch_kv_seq_shift). */

@@ -88,19 +88,16 @@ int batch_input(int wtype, const float * x, int T, int cols, const pi_norm * nor
     return pi_k_norm_round_f16(x, T, cols, norm, out16, plain16, st);
 }
 
-// attention of a step whose tokens live in the shared-cell cache: token t's K / V rows go to cell slot[t], and it attends the cells its
-// mask row leaves visible (same sequence, position not beyond its own: llama.cpp:6506-6531).  One launch per token, in the order
-// of the batch: a token may attend an earlier token of the same step, whose rows are then already in place.
+// attention of a step whose tokens live in the shared-cell cache: token t's K / V rows go to cell slot[0] + t, and it attends the cells
+// its mask row leaves visible (same sequence, position not beyond its own: llama.cpp:6506-6531), the step's other new cells included
 int cells_attention(pi_model * m, BatchState * b, int il, int T) {
     const pi_hparams & hp = m->hp;
-    const int d = hp.n_embd, gqa = m->gqa, stride = d + 2 * gqa;
+    const int d = hp.n_embd, gqa = m->gqa;
     const bool falcon = hp.arch == PI_ARCH_FALCON;
     __half * k = b->cells_k + (size_t)il * b->n_cells * gqa;
     __half * v = b->cells_v + (size_t)il * gqa * b->n_cells;
-    for (int t = 0; t < T; ++t)
-        PI_TRY(pi_k_attn_ggml(b->qkv + (size_t)t * stride, b->qkv + (size_t)t * stride + d, b->qkv + (size_t)t * stride + d + gqa, b->d_pos + t,
-                              falcon ? 2 : 0, m->theta_scale, m->freq_scale, 1.0f, k, v, hp.n_head, hp.n_head_kv, m->hd, b->n_cells, b->n_kv, b->slot[t],
-                              b->kq_scale, b->cells_mask + (size_t)t * b->n_cells, b->att + (size_t)t * d, m->stream));
+    PI_TRY(pi_k_attn_ggml_step(b->qkv, d + 2 * gqa, b->d_pos, falcon ? 2 : 0, m->theta_scale, m->freq_scale, 1.0f, k, v, hp.n_head, hp.n_head_kv, m->hd,
+                               b->n_cells, b->n_kv, T, b->slot[0], b->kq_scale, b->cells_mask, b->n_cells, b->att, d, m->stream));
     const pi_norm plain{0, 0.0f, nullptr, nullptr};
     return pi_k_norm_round_f16(b->att, T, d, &plain, b->att16, nullptr, m->stream);
 }
@@ -858,10 +855,6 @@ int pi_model_kv_cells_decode(pi_model * m, const int32_t * tokens, const int32_t
     for (int t = 0; t < n_tokens; ++t) {
         if (tokens[t] < 0 || tokens[t] >= m->hp.n_vocab) return pi::fail(PI_E_ARG, "pi_model_kv_cells_decode: token id out of range");
         if (positions[t] < 0 || seq_masks[t] == 0) return pi::fail(PI_E_ARG, "pi_model_kv_cells_decode: a token needs a position and at least one sequence");
-        // a token may attend an earlier token of the same step (its rows are written first), never a later one
-        for (int u = 0; u < t; ++u)
-            if ((seq_masks[u] & seq_masks[t]) && positions[u] > positions[t])
-                return pi::fail(PI_E_ARG, "pi_model_kv_cells_decode: tokens of one sequence must come in ascending positions");
     }
     if (!cells_find_slot(b, n_tokens)) return pi::fail(PI_E_STATE, "pi_model_kv_cells_decode: no run of free cells for the step (llama_kv_cache_find_slot failed)");
     for (int t = 0; t < n_tokens; ++t) {

@@ -691,43 +691,56 @@ __global__ __launch_bounds__(kBlock) void attn_chunk_mfma_kernel(const float * _
 // workgroup depends on another's stores.  Cells whose mask entry is -inf get probability 0 whatever the cache holds there.
 // RoPE as rope_kernel of the boundary computes it: angle advanced by repeated fp32 multiplication, cosf / sinf, * mscale.
 // ---------------------------------------------------------------------------------------------------
-__global__ __launch_bounds__(kBlock) void attn_ggml_kernel(const float * __restrict__ q, const float * __restrict__ k, const float * __restrict__ v,
+// A step of T tokens (grid.y; token u's q, k, v at stride tok_stride, its cell cell0 + u, its mask row at mask_stride, its output at
+// out_stride): the K and V rows of all T new cells are formed in LDS by every workgroup, so a token attends the other tokens of its
+// step (where its mask allows) without waiting for their stores - what the reference gets by storing the whole batch first.
+__global__ __launch_bounds__(kBlock) void attn_ggml_kernel(const float * __restrict__ q, const float * __restrict__ k, const float * __restrict__ v, int tok_stride,
                                                            const int32_t * __restrict__ pos, int mode, float theta_scale, float freq_scale, float mscale,
                                                            __half * __restrict__ k_cache, __half * __restrict__ v_cache,
-                                                           int n_head, int n_head_kv, int hd, int n_ctx, int n_kv, int cell,
-                                                           const float * __restrict__ kq_scale, const float * __restrict__ kq_mask, float * __restrict__ out) {
+                                                           int n_head, int n_head_kv, int hd, int n_ctx, int n_kv, int T, int cell0,
+                                                           const float * __restrict__ kq_scale, const float * __restrict__ kq_mask, int mask_stride,
+                                                           float * __restrict__ out, int out_stride) {
     extern __shared__ __align__(16) unsigned char smem[];
     const int n_kv8 = (n_kv + 7) & ~7;                                     // the V rows are read eight cells at a time
     float * sc = reinterpret_cast<float *>(smem);                          // [n_kv8] scores, then probabilities (zeros behind n_kv)
-    __half * q16 = reinterpret_cast<__half *>(sc + n_kv8);                 // [hd] each
-    __half * k16 = q16 + hd;
-    __half * v16 = k16 + hd;
+    __half * q16 = reinterpret_cast<__half *>(sc + n_kv8);                 // [hd]
+    __half * k16 = q16 + hd;                                               // [T][hd] the step's new K rows
+    __half * v16 = k16 + (size_t)T * hd;                                   // [T][hd] and V rows
     __shared__ double red[kWavesPerBlock];
     __shared__ float  redf[kWavesPerBlock];
-    const int h = blockIdx.x, kvh = h / (n_head / n_head_kv), gqa = n_head_kv * hd;
+    const int h = blockIdx.x, tok = blockIdx.y, kvh = h / (n_head / n_head_kv), gqa = n_head_kv * hd;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
-    const bool owner = h % (n_head / n_head_kv) == 0;                      // this head's workgroup stores the group's new K / V rows
+    const bool owner = h % (n_head / n_head_kv) == 0;                      // this head's workgroup stores the group's new K / V rows of its token
+    const int cell = cell0 + tok;
+    kq_mask += (size_t)tok * mask_stride;
+    out += (size_t)tok * out_stride;
     if (tid < hd / 2) {
         const int i = tid;
-        float theta = (float)pos[0];
-        if (mode & 2) theta = __fmul_rn(theta, freq_scale);
-        for (int j = 0; j < i; ++j) theta = __fmul_rn(theta, theta_scale);
-        const float th = __fmul_rn(freq_scale, theta);
-        const float c = __fmul_rn(cosf(th), mscale), sn = __fmul_rn(sinf(th), mscale);
         const int i0 = (mode & 2) ? i : 2 * i, i1 = (mode & 2) ? i + hd / 2 : 2 * i + 1;
-        const float q0 = q[h * hd + i0], q1 = q[h * hd + i1];
-        q16[i0] = __float2half_rn(__fsub_rn(__fmul_rn(q0, c), __fmul_rn(q1, sn)));
-        q16[i1] = __float2half_rn(__fadd_rn(__fmul_rn(q0, sn), __fmul_rn(q1, c)));
-        const float k0 = k[kvh * hd + i0], k1 = k[kvh * hd + i1];
-        const __half r0 = __float2half_rn(__fsub_rn(__fmul_rn(k0, c), __fmul_rn(k1, sn)));
-        const __half r1 = __float2half_rn(__fadd_rn(__fmul_rn(k0, sn), __fmul_rn(k1, c)));
-        k16[i0] = r0; k16[i1] = r1;
-        if (owner) { k_cache[(size_t)cell * gqa + kvh * hd + i0] = r0; k_cache[(size_t)cell * gqa + kvh * hd + i1] = r1; }
+        for (int u = 0; u < T; ++u) {
+            float theta = (float)pos[u];
+            if (mode & 2) theta = __fmul_rn(theta, freq_scale);
+            for (int j = 0; j < i; ++j) theta = __fmul_rn(theta, theta_scale);
+            const float th = __fmul_rn(freq_scale, theta);
+            const float c = __fmul_rn(cosf(th), mscale), sn = __fmul_rn(sinf(th), mscale);
+            if (u == tok) {
+                const float q0 = q[(size_t)u * tok_stride + h * hd + i0], q1 = q[(size_t)u * tok_stride + h * hd + i1];
+                q16[i0] = __float2half_rn(__fsub_rn(__fmul_rn(q0, c), __fmul_rn(q1, sn)));
+                q16[i1] = __float2half_rn(__fadd_rn(__fmul_rn(q0, sn), __fmul_rn(q1, c)));
+            }
+            const float k0 = k[(size_t)u * tok_stride + kvh * hd + i0], k1 = k[(size_t)u * tok_stride + kvh * hd + i1];
+            const __half r0 = __float2half_rn(__fsub_rn(__fmul_rn(k0, c), __fmul_rn(k1, sn)));
+            const __half r1 = __float2half_rn(__fadd_rn(__fmul_rn(k0, sn), __fmul_rn(k1, c)));
+            k16[u * hd + i0] = r0; k16[u * hd + i1] = r1;
+            if (owner && u == tok) { k_cache[(size_t)cell * gqa + kvh * hd + i0] = r0; k_cache[(size_t)cell * gqa + kvh * hd + i1] = r1; }
+        }
     }
     if (tid < hd) {
-        const __half r = __float2half_rn(v[kvh * hd + tid]);
-        v16[tid] = r;
-        if (owner) v_cache[(size_t)(kvh * hd + tid) * n_ctx + cell] = r;
+        for (int u = 0; u < T; ++u) {
+            const __half r = __float2half_rn(v[(size_t)u * tok_stride + kvh * hd + tid]);
+            v16[u * hd + tid] = r;
+            if (owner && u == tok) v_cache[(size_t)(kvh * hd + tid) * n_ctx + cell] = r;
+        }
     }
     __syncthreads();
 
@@ -751,7 +764,7 @@ __global__ __launch_bounds__(kBlock) void attn_ggml_kernel(const float * __restr
 #pragma unroll
         for (int u = 0; u < SU; ++u) {
             const int c = c0 + u * cstep;
-            if (c == cell) kr[u] = *reinterpret_cast<const pi_u32x4 *>(k16 + l * 8);
+            if (c >= cell0 && c < cell0 + T) kr[u] = *reinterpret_cast<const pi_u32x4 *>(k16 + (c - cell0) * hd + l * 8);
             float d = pi_dot8h(kr[u], qv, 0.0f);
             for (int o = 1; o < lpc; o <<= 1) d += __shfl_xor(d, o, PI_WAVE);
             if (c < n_kv && l == 0) sc[c] = m[u] == -INFINITY ? -INFINITY : __fadd_rn(__fmul_rn(d, scale), m[u]);
@@ -785,7 +798,6 @@ __global__ __launch_bounds__(kBlock) void attn_ggml_kernel(const float * __restr
     {
         const int dim = tid % hd, part = tid / hd, nparts = kBlock / hd;      // hd <= kBlock and divides it (the launcher's test)
         const __half * vr = v_cache + (size_t)(kvh * hd + dim) * n_ctx;
-        const __half vn = v16[dim];
         float acc = 0.0f;
         constexpr int VU = 4;
         for (int g0 = part; g0 * 8 < n_kv; g0 += VU * nparts) {
@@ -799,7 +811,8 @@ __global__ __launch_bounds__(kBlock) void attn_ggml_kernel(const float * __restr
             for (int u = 0; u < VU; ++u) {
                 const int c0 = (g0 + u * nparts) * 8;
                 if (c0 < n_kv) {
-                    if (cell >= c0 && cell < c0 + 8) reinterpret_cast<__half *>(&vv[u])[cell - c0] = vn;
+                    for (int w = c0 > cell0 ? c0 - cell0 : 0; w < T && cell0 + w < c0 + 8; ++w)      // the step's own cells come from LDS
+                        reinterpret_cast<__half *>(&vv[u])[cell0 + w - c0] = v16[w * hd + dim];
                     const float4 p0 = *reinterpret_cast<const float4 *>(sc + c0), p1 = *reinterpret_cast<const float4 *>(sc + c0 + 4);
                     __half2 ph[4] = {__floats2half2_rn(p0.x, p0.y), __floats2half2_rn(p0.z, p0.w), __floats2half2_rn(p1.x, p1.y), __floats2half2_rn(p1.z, p1.w)};
                     // a cell without probability contributes nothing, whatever its (possibly never written) V entry holds
@@ -814,7 +827,7 @@ __global__ __launch_bounds__(kBlock) void attn_ggml_kernel(const float * __restr
                 }
             }
         }
-        float * pacc = reinterpret_cast<float *>(v16 + hd);                   // [kBlock] floats behind the three fp16 rows
+        float * pacc = reinterpret_cast<float *>(v16 + (size_t)T * hd);       // [kBlock] floats behind the fp16 rows
         pacc[tid] = acc;
         __syncthreads();
         if (tid < hd) {
@@ -1021,9 +1034,12 @@ int pi_k_attn_chunk_long(const float * qkv, int qkv_stride, int T, int n_head, i
     return pi::check_launch("pi_k_attn_chunk_long");
 }
 
+static size_t attn_ggml_lds(int hd, int n_kv, int T) {
+    return sizeof(float) * (size_t)((n_kv + 7) & ~7) + 2 * (size_t)hd * (1 + 2 * (size_t)T) + sizeof(float) * kBlock;
+}
 int pi_k_attn_ggml_supported(int hd, int n_ctx, int n_kv) {
     return hd > 0 && hd % 8 == 0 && hd <= kBlock && kBlock % hd == 0 && PI_WAVE % (hd / 8) == 0 && n_kv > 0 && n_ctx % 8 == 0 && n_kv <= n_ctx &&
-           sizeof(float) * (size_t)((n_kv + 7) & ~7) + 6 * (size_t)hd + sizeof(float) * kBlock <= 60 * 1024;
+           attn_ggml_lds(hd, n_kv, kBtMaxT) <= 60 * 1024;
 }
 
 int pi_k_attn_ggml(const float * q, const float * k, const float * v, const int32_t * pos, int mode, float theta_scale, float freq_scale, float mscale,
@@ -1033,10 +1049,23 @@ int pi_k_attn_ggml(const float * q, const float * k, const float * v, const int3
     if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || (mode != 0 && mode != 2) || cell < 0 || cell >= n_kv || !pi_k_attn_ggml_supported(hd, n_ctx, n_kv))
         return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_ggml: head geometry, cell or context outside the kernel (pi_k_attn_ggml_supported)");
     if ((((uintptr_t)k_cache | (uintptr_t)v_cache) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_attn_ggml: the caches must be 16-byte aligned");
-    const size_t sh = sizeof(float) * (size_t)((n_kv + 7) & ~7) + 6 * (size_t)hd + sizeof(float) * kBlock;
-    hipLaunchKernelGGL(attn_ggml_kernel, dim3(n_head), dim3(kBlock), sh, (hipStream_t)stream, q, k, v, pos, mode, theta_scale, freq_scale, mscale,
-                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, n_ctx, n_kv, cell, kq_scale, kq_mask, out);
+    hipLaunchKernelGGL(attn_ggml_kernel, dim3(n_head, 1), dim3(kBlock), attn_ggml_lds(hd, n_kv, 1), (hipStream_t)stream, q, k, v, 0, pos, mode, theta_scale, freq_scale, mscale,
+                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, n_ctx, n_kv, 1, cell, kq_scale, kq_mask, 0, out, 0);
     return pi::check_launch("pi_k_attn_ggml");
+}
+
+int pi_k_attn_ggml_step(const float * qkv, int qkv_stride, const int32_t * pos, int mode, float theta_scale, float freq_scale, float mscale,
+                        void * k_cache, void * v_cache, int n_head, int n_head_kv, int hd, int n_ctx, int n_kv, int T, int cell0,
+                        const float * kq_scale, const float * kq_mask, int mask_stride, float * out, int out_stride, pi_stream_t stream) {
+    if (!qkv || !pos || !k_cache || !v_cache || !kq_scale || !kq_mask || !out) return pi::fail(PI_E_ARG, "pi_k_attn_ggml_step: null pointer");
+    if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || (mode != 0 && mode != 2) || T < 1 || T > kBtMaxT || cell0 < 0 || cell0 + T > n_kv ||
+        qkv_stride < (n_head + 2 * n_head_kv) * hd || mask_stride < n_kv || out_stride < n_head * hd || !pi_k_attn_ggml_supported(hd, n_ctx, n_kv))
+        return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_ggml_step: head geometry, cells, strides or context outside the kernel (pi_k_attn_ggml_supported)");
+    if ((((uintptr_t)k_cache | (uintptr_t)v_cache) & 15) != 0) return pi::fail(PI_E_ARG, "pi_k_attn_ggml_step: the caches must be 16-byte aligned");
+    hipLaunchKernelGGL(attn_ggml_kernel, dim3(n_head, T), dim3(kBlock), attn_ggml_lds(hd, n_kv, T), (hipStream_t)stream, qkv, qkv + (size_t)n_head * hd,
+                       qkv + (size_t)(n_head + n_head_kv) * hd, qkv_stride, pos, mode, theta_scale, freq_scale, mscale, (__half *)k_cache, (__half *)v_cache,
+                       n_head, n_head_kv, hd, n_ctx, n_kv, T, cell0, kq_scale, kq_mask, mask_stride, out, out_stride);
+    return pi::check_launch("pi_k_attn_ggml_step");
 }
 
 int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float theta_scale, float freq_scale, const int32_t * delta, int n_cells, pi_stream_t stream) {

@@ -115,6 +115,7 @@ _SIGS = {
     "pi_k_attn_split_supported": (_i, [_i, _i, _i]),
     "pi_k_attn_ggml_supported": (_i, [_i, _i, _i]),
     "pi_k_attn_ggml": (_i, [_vp, _vp, _vp, _vp, _i, _f, _f, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _vp]),
+    "pi_k_attn_ggml_step": (_i, [_vp, _i, _vp, _i, _f, _f, _f, _vp, _vp, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _i, _vp, _i, _vp]),
     "pi_k_attn_split_scratch_floats": (_sz, [_i, _i, _i, _i]),
     "pi_k_attn_split": (_i, [_vp, _i, _vp, _vp, _vp, _sz, _i, _i, _i, _i, _i, _i, _i, _vp, _vp, _vp, _i, _vp, _vp]),
     "pi_k_attn_chunk_supported": (_i, [_i, _i, _i]),

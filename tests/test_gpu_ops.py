@@ -396,6 +396,64 @@ def test_attention_on_the_reference_cache_layouts(mode, hd, nh, nkv):
     assert np.abs(kg - kc_o.view(np.float16).astype(np.float32)).max() <= 2e-3 * np.abs(kg).max()
 
 
+@pytest.mark.parametrize("mode,hd,nh,nkv,T", [(0, 128, 4, 4, 16), (2, 64, 8, 2, 5), (0, 128, 8, 8, 1)])
+def test_attention_of_a_step_on_the_reference_cache_layouts(mode, hd, nh, nkv, T):
+    """pi_k_attn_ggml_step: T tokens whose rows go to a run of consecutive cells, each under its own mask row, in one launch, against
+    the oracle's llm_build_kv_store + llm_build_kqv for the same batch (which stores every token's rows before anyone attends).
+    Three steps into a cache that already holds cells: tokens of two interleaved sequences (a token does not see the other
+    sequence's cells, old or new), causal inside the step, and in the last step the tokens come in descending positions, so that a
+    token attends rows of tokens behind it in the batch."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    O = ol.oracle()
+    rng = np.random.default_rng(mode + hd + T)
+    n_ctx, gqa, d = 96, nkv * hd, nh * hd
+    stride = d + 2 * gqa + 8                                     # tokens' [q | k | v] rows with a gap between them
+    kc_o, vc_o = np.zeros((n_ctx, gqa), np.uint16), np.zeros((gqa, n_ctx), np.uint16)
+    kc, vc = pl.DevBuf.zeros(n_ctx * gqa * 2), pl.DevBuf.zeros(n_ctx * gqa * 2)
+    theta_scale = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
+    scale = pl.DevBuf(host=np.array([1.0 / np.sqrt(hd)], np.float32))
+    cell_seq, cell_pos = np.full(n_ctx, -1), np.full(n_ctx, -1)
+    next_pos = [0, 0]
+    cell0 = 3                                                    # the first run does not start at cell 0
+    for step in range(3):
+        seqs = rng.integers(0, 2, T)
+        pos = np.zeros(T, np.int32)
+        for t in range(T):
+            pos[t] = next_pos[seqs[t]]
+            next_pos[seqs[t]] += 1
+        if step == 2:
+            seqs, pos = seqs[::-1].copy(), pos[::-1].copy()
+        cell_seq[cell0:cell0 + T], cell_pos[cell0:cell0 + T] = seqs, pos
+        n_kv = cell0 + T + (3 if step == 1 else 0)               # a range that is no multiple of 8 and reaches past the cells in use
+        mask = np.zeros((T, n_kv), np.float32)
+        for t in range(T):
+            hidden = (cell_seq[:n_kv] != seqs[t]) | (cell_pos[:n_kv] > pos[t]) | (cell_pos[:n_kv] < 0)
+            mask[t, hidden] = -np.inf
+        qkv = rng.standard_normal((T, stride)).astype(np.float32)
+        q, k, v = (np.ascontiguousarray(qkv[:, a:b]) for a, b in ((0, d), (d, d + gqa), (d + gqa, d + 2 * gqa)))
+        qr, kr = np.zeros_like(q), np.zeros_like(k)
+        O.pio_rope(P(q), hd, nh, T, P(pos), hd, mode, 10000.0, 1.0, P(qr))
+        O.pio_rope(P(k), hd, nkv, T, P(pos), hd, mode, 10000.0, 1.0, P(kr))
+        want = np.zeros((T, d), np.float32)
+        slots = np.arange(cell0, cell0 + T, dtype=np.int32)
+        assert O.pio_attention(hd, nh, nkv, n_ctx, n_kv, T, P(slots), P(mask), P(qr), P(kr), P(v), P(kc_o), P(vc_o), P(want)) == 0
+        dqkv, dpos, dmask, dout = pl.DevBuf(host=qkv), pl.DevBuf(host=pos), pl.DevBuf(host=mask), pl.DevBuf(T * (d + 4) * 4)
+        pl.check(L.pi_k_attn_ggml_step(dqkv.ptr, stride, dpos.ptr, mode, theta_scale, 1.0, 1.0, kc.ptr, vc.ptr, nh, nkv, hd, n_ctx, n_kv, T, cell0,
+                                       scale.ptr, dmask.ptr, n_kv, dout.ptr, d + 4, None), "attn_ggml_step")
+        pl.sync()
+        got = dout.download(np.float32).reshape(T, d + 4)[:, :d]
+        for t in range(T):
+            assert rel_err(got[t], want[t]) < 2e-3, (step, t, rel_err(got[t], want[t]))
+        cell0 += T + (2 if step == 0 else 0)                     # a hole of two free cells behind the first run
+    vg = vc.download(np.uint16).reshape(gqa, n_ctx)
+    assert np.array_equal(vg, vc_o)
+    kg = kc.download(np.float16).reshape(n_ctx, gqa).astype(np.float32)
+    assert np.abs(kg - kc_o.view(np.float16).astype(np.float32)).max() <= 2e-3 * np.abs(kg).max()
+    assert L.pi_k_attn_ggml_step(dqkv.ptr, stride, dpos.ptr, mode, theta_scale, 1.0, 1.0, kc.ptr, vc.ptr, nh, nkv, hd, n_ctx, 40, 17, 0,
+                                 scale.ptr, dmask.ptr, 40, dout.ptr, d + 4, None) != 0                   # more than 16 tokens
+
+
 def test_embed_and_argmax():
     from powerinfer_amd import lib as pl
     L = pl.init()

@@ -211,6 +211,10 @@ PI_API int pi_k_axpy_q4_partials_split(const void * down_t_q4, const void * down
  * freq_scale: linear RoPE scaling as in pi_k_rope_kv_store. */
 PI_API int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float theta_scale, float freq_scale, const int32_t * delta, int n_cells, pi_stream_t stream);
 PI_API int pi_k_kv_compact(void * cache, void * stage, int rows, int n_ctx, int hd, const int32_t * map, int n_new, pi_stream_t stream);
+/* the K-shift on the reference's own cache layout, K cells [n_layer][n_cells][n_head_kv][hd] (the strided view llm_build_k_shift rotates,
+ * llama.cpp:4366-4378): every cell's rows are rotated by delta[cell] positions, cells with delta 0 are left alone */
+PI_API int pi_k_k_shift_cells(void * k_cache, int n_layer, int n_cells, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,
+                              const int32_t * delta, pi_stream_t stream);
 /* Shapes of the fused block: cols 4096 or 8192 with a predictor of rank 512 or 1024 and ff % 32 == 0; cols 5120 with rank 1280 (the
  * 13B shape) where ff gives every compute unit 33..60 neurons, with a norm that carries its weights (or none).  Needs pi_init
  * (the answer depends on the device's compute units).  _hot_supported: the shapes of the hybrid forms below (the first group only). */
@@ -628,20 +632,23 @@ PI_API int pi_model_batch_kv_seq_rm(pi_model * m, int seq, int p0, int p1);
 PI_API int pi_model_batch_kv_seq_shift(pi_model * m, int seq, int p0, int p1, int delta);
 PI_API int pi_model_batch_kv_seq_cp(pi_model * m, int src, int dst, int p0, int p1);
 /* One KV cache whose cells are shared between sequences: llama_kv_cell / llama_kv_cache (llama.cpp:1381-1420), llama_kv_cache_find_slot (:1683-1730),
- * _seq_rm / _seq_cp / _seq_keep / _clear (:1745-1822), the visibility mask of llama_decode (:6506-6531) and the cell range a step looks
+ * _seq_rm / _seq_cp / _seq_keep / _seq_shift / _clear (:1745-1848), the visibility mask of llama_decode (:6506-6531) and the cell range a step looks
  * at (:1735-1743, 6842).  A cell holds a position and a set of sequence ids (0..31, one bit each); a step of up to 16 tokens takes a run
  * of free cells found from the ring's head, every token attends the cells of its (first) sequence at positions not beyond its own;
  * _seq_cp makes the cells of src visible to dst without copying anything (a prompt evaluated once serves every continuation).
  * F16 models, or Q4_0 models with F16 predictors, with every neuron on the GPU; n_cells a multiple of 32.  _decode returns PI_E_STATE when no run of free cells is left (the reference's
  * llama_decode returns 1), each token's greedy next token and, if logits_out != NULL, its logits [n_tokens][n_vocab].
  * _state copies the cells' positions (-1: free) and sequence bit sets and the ring's head out (tests, monitoring); returns n_cells.
- * Position shifts (llama_kv_cache_seq_shift) exist for the per-sequence caches only (pi_model_kv_seq_shift, pi_model_batch_kv_seq_shift). */
+ * _seq_shift moves the positions of a sequence's cells in [p0, p1) by delta (llama_kv_cache_seq_shift, :1824-1848; a cell whose position
+ * falls below 0 is freed); the K rows are rotated at the start of the next step (llm_build_k_shift, :4332-4381), after which the pending
+ * deltas are cleared (:6925-6932). */
 PI_API int pi_model_kv_cells_init(pi_model * m, int n_cells);
 PI_API int pi_model_kv_cells_decode(pi_model * m, const int32_t * tokens, const int32_t * positions, const uint32_t * seq_masks, int n_tokens,
                                     int32_t * next_tokens, float * logits_out);
 PI_API int pi_model_kv_cells_seq_rm(pi_model * m, int seq, int p0, int p1);
 PI_API int pi_model_kv_cells_seq_cp(pi_model * m, int src, int dst, int p0, int p1);
 PI_API int pi_model_kv_cells_seq_keep(pi_model * m, int seq);
+PI_API int pi_model_kv_cells_seq_shift(pi_model * m, int seq, int p0, int p1, int delta);
 PI_API int pi_model_kv_cells_clear(pi_model * m);
 PI_API int pi_model_kv_cells_state(pi_model * m, int32_t * cell_pos, uint32_t * cell_seq, int32_t * head);
 PI_API int pi_model_batch_union(pi_model * m, int32_t * n_union_per_layer);   /* union sizes of the last step, [n_layer] */

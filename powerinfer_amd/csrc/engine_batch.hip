@@ -35,6 +35,9 @@ struct BatchState {
     int n_cells = 0, head = 0, n_kv = 0;
     std::vector<int32_t> cell_pos;
     std::vector<uint32_t> cell_seq;
+    std::vector<int32_t> cell_delta;                   // position shifts not yet applied to the K rows
+    bool has_shift = false;
+    int32_t * d_delta = nullptr;
     __half *cells_k = nullptr, *cells_v = nullptr;
     float *cells_mask = nullptr, *kq_scale = nullptr;  // device: [16][n_cells] mask rows of a step, 1 / sqrt(head size)
     int slot[16] = {0};                                // the cells the step's tokens were given
@@ -819,10 +822,11 @@ int pi_model_kv_cells_init(pi_model * m, int n_cells) {
     b->n_cells = n_cells;
     b->cell_pos.assign(n_cells, -1);
     b->cell_seq.assign(n_cells, 0u);
+    b->cell_delta.assign(n_cells, 0);
     const size_t per_layer = (size_t)n_cells * m->gqa;
     b->cells_k = m->alloc<__half>(per_layer * m->hp.n_layer); b->cells_v = m->alloc<__half>(per_layer * m->hp.n_layer);
-    b->cells_mask = m->alloc<float>((size_t)16 * n_cells); b->kq_scale = m->alloc<float>(1);
-    if (!b->cells_k || !b->cells_v || !b->cells_mask || !b->kq_scale) { delete b; return PI_E_HIP; }
+    b->cells_mask = m->alloc<float>((size_t)16 * n_cells); b->kq_scale = m->alloc<float>(1); b->d_delta = m->alloc<int32_t>(n_cells);
+    if (!b->cells_k || !b->cells_v || !b->cells_mask || !b->kq_scale || !b->d_delta) { delete b; return PI_E_HIP; }
     const float scale = 1.0f / sqrtf((float)m->hd);
     PI_HIP_TRY(hipMemsetAsync(b->cells_k, 0, sizeof(__half) * per_layer * m->hp.n_layer, m->stream));
     PI_HIP_TRY(hipMemsetAsync(b->cells_v, 0, sizeof(__half) * per_layer * m->hp.n_layer, m->stream));
@@ -874,6 +878,14 @@ int pi_model_kv_cells_decode(pi_model * m, const int32_t * tokens, const int32_t
             if (!(b->cell_seq[i] >> seq & 1u) || b->cell_pos[i] > positions[t]) mask[(size_t)t * b->n_cells + i] = -INFINITY;
     }
     b->n_seq = n_tokens;
+    if (b->has_shift) {          // pending position shifts: the K rows are rotated ahead of the step's layers (llm_build_k_shift runs first in the graph)
+        PI_HIP_TRY(hipMemcpyAsync(b->d_delta, b->cell_delta.data(), sizeof(int32_t) * b->n_cells, hipMemcpyHostToDevice, m->stream));
+        PI_HIP_TRY(hipStreamSynchronize(m->stream));
+        PI_TRY(pi_k_k_shift_cells(b->cells_k, m->hp.n_layer, b->n_cells, m->hp.n_head_kv, m->hd, m->hp.arch == PI_ARCH_FALCON ? 2 : 0, m->theta_scale,
+                                  m->freq_scale, b->d_delta, m->stream));
+        b->has_shift = false;
+        std::fill(b->cell_delta.begin(), b->cell_delta.end(), 0);
+    }
     PI_HIP_TRY(hipMemcpyAsync(b->d_tokens, tokens, sizeof(int32_t) * n_tokens, hipMemcpyHostToDevice, m->stream));
     PI_HIP_TRY(hipMemcpyAsync(b->d_pos, positions, sizeof(int32_t) * n_tokens, hipMemcpyHostToDevice, m->stream));
     PI_HIP_TRY(hipMemcpyAsync(b->cells_mask, mask.data(), sizeof(float) * mask.size(), hipMemcpyHostToDevice, m->stream));
@@ -929,6 +941,25 @@ int pi_model_kv_cells_seq_keep(pi_model * m, int seq) {
         else b->cell_seq[i] = 1u << seq;
     }
     if (new_head != b->n_cells) b->head = new_head;
+    return PI_OK;
+}
+
+// llama_kv_cache_seq_shift (llama.cpp:1824-1848): the positions move now, the K rows at the start of the next step
+int pi_model_kv_cells_seq_shift(pi_model * m, int seq, int p0, int p1, int delta) {
+    if (!m || !m->cells || seq < 0 || seq >= 32) return pi::fail(PI_E_ARG, "pi_model_kv_cells_seq_shift: bad arguments");
+    BatchState * b = m->cells;
+    int new_head = b->n_cells;
+    if (p0 < 0) p0 = 0;
+    if (p1 < 0) p1 = INT32_MAX;
+    for (int i = 0; i < b->n_cells; ++i) {
+        if ((b->cell_seq[i] >> seq & 1u) && b->cell_pos[i] >= p0 && b->cell_pos[i] < p1) {
+            b->has_shift = true;
+            b->cell_pos[i] += delta;
+            b->cell_delta[i] += delta;
+            if (b->cell_pos[i] < 0) { b->cell_pos[i] = -1; b->cell_seq[i] = 0; if (new_head == b->n_cells) new_head = i; }
+        }
+    }
+    b->head = new_head != b->n_cells ? new_head : 0;
     return PI_OK;
 }
 

@@ -26,6 +26,23 @@ __global__ void k_shift_kernel(__half * __restrict__ k_cache, int n_ctx, int hd,
     row[i1] = __float2half_rn(__fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, c)));
 }
 
+// the same on the reference's own layout, K cells [layer][cell][kv head][hd]: grid = (cells, layers * kv heads)
+__global__ void k_shift_cells_kernel(__half * __restrict__ k_cache, int n_cells, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,
+                                     const int32_t * __restrict__ delta) {
+    const int cell = blockIdx.x, i = threadIdx.x;
+    const int dl = delta[cell];
+    if (dl == 0) return;
+    const int layer = blockIdx.y / n_head_kv, kvh = blockIdx.y % n_head_kv;
+    __half * row = k_cache + (((size_t)layer * n_cells + cell) * n_head_kv + kvh) * hd;
+    const float theta = rope_angle((float)dl, i, mode, theta_scale, freq_scale);
+    const float c = cosf(theta), sn = sinf(theta);
+    const int i0 = (mode & 2) ? i : 2 * i;
+    const int i1 = (mode & 2) ? i + hd / 2 : 2 * i + 1;
+    const float x0 = __half2float(row[i0]), x1 = __half2float(row[i1]);
+    row[i0] = __float2half_rn(__fsub_rn(__fmul_rn(x0, c), __fmul_rn(x1, sn)));
+    row[i1] = __float2half_rn(__fadd_rn(__fmul_rn(x0, sn), __fmul_rn(x1, c)));
+}
+
 // Cell compaction of one cache (K or V) after cells were removed: new cell j takes old cell map[j] (map ascending, so the cells
 // keep their order).  Two launches through a staging buffer [rows][n_new][hd] because source and destination ranges overlap.
 // grid = (n_new, rows), hd/8 threads (16 bytes each).
@@ -1074,6 +1091,15 @@ int pi_k_k_shift(void * k_cache, int rows, int n_ctx, int hd, int mode, float th
     if (n_cells == 0) return PI_OK;
     hipLaunchKernelGGL(k_shift_kernel, dim3(n_cells, rows), dim3(hd / 2), 0, (hipStream_t)stream, (__half *)k_cache, n_ctx, hd, mode, theta_scale, freq_scale, delta);
     return pi::check_launch("pi_k_k_shift");
+}
+
+int pi_k_k_shift_cells(void * k_cache, int n_layer, int n_cells, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale, const int32_t * delta,
+                       pi_stream_t stream) {
+    if (!k_cache || !delta || n_layer <= 0 || n_cells <= 0 || n_head_kv <= 0 || hd <= 0 || hd % 2 || hd / 2 > 1024 || (mode != 0 && mode != 2))
+        return pi::fail(PI_E_ARG, "pi_k_k_shift_cells: bad arguments");
+    hipLaunchKernelGGL(k_shift_cells_kernel, dim3(n_cells, n_layer * n_head_kv), dim3(hd / 2), 0, (hipStream_t)stream, (__half *)k_cache, n_cells, n_head_kv, hd, mode,
+                       theta_scale, freq_scale, delta);
+    return pi::check_launch("pi_k_k_shift_cells");
 }
 
 int pi_k_kv_compact(void * cache, void * stage, int rows, int n_ctx, int hd, const int32_t * map, int n_new, pi_stream_t stream) {

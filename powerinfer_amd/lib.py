@@ -70,6 +70,7 @@ _SIGS = {
     "pi_k_axpy_q4_partials_split": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_axpy_q4_reduce": (_i, [_i, _i, _i, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_k_shift": (_i, [_vp, _i, _i, _i, _i, _f, _f, _vp, _i, _vp]),
+    "pi_k_k_shift_cells": (_i, [_vp, _i, _i, _i, _i, _i, _f, _f, _vp, _vp]),
     "pi_k_kv_compact": (_i, [_vp, _vp, _i, _i, _i, _vp, _i, _vp]),
     "pi_k_sparse_ffn_partials": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp]),
     "pi_k_sparse_ffn_partials_hot": (_i, [_vp, _i, _i, _vp, _f, _vp, _vp, _vp, _i, _vp, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp, _vp, _vp]),

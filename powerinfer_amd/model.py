@@ -53,6 +53,7 @@ def _declare(L):
     L.pi_model_kv_cells_seq_rm.restype, L.pi_model_kv_cells_seq_rm.argtypes = i, [vp, i, i, i]
     L.pi_model_kv_cells_seq_cp.restype, L.pi_model_kv_cells_seq_cp.argtypes = i, [vp, i, i, i, i]
     L.pi_model_kv_cells_seq_keep.restype, L.pi_model_kv_cells_seq_keep.argtypes = i, [vp, i]
+    L.pi_model_kv_cells_seq_shift.restype, L.pi_model_kv_cells_seq_shift.argtypes = i, [vp, i, i, i, i]
     L.pi_model_kv_cells_clear.restype, L.pi_model_kv_cells_clear.argtypes = i, [vp]
     L.pi_model_kv_cells_state.restype, L.pi_model_kv_cells_state.argtypes = i, [vp, vp, vp, vp]
     L.pi_model_time_section.restype, L.pi_model_time_section.argtypes = i, [vp, i, i, C.POINTER(C.c_float), C.POINTER(C.c_int)]
@@ -66,7 +67,7 @@ ENGINE_SYMBOLS = ["pi_model_create", "pi_model_free", "pi_model_set_tensor", "pi
                   "pi_model_batch_set_dense_above", "pi_model_batch_dense_layers",
                   "pi_model_batch_kv_seq_rm", "pi_model_batch_kv_seq_shift", "pi_model_batch_kv_seq_cp",
                   "pi_model_kv_cells_init", "pi_model_kv_cells_decode", "pi_model_kv_cells_seq_rm", "pi_model_kv_cells_seq_cp",
-                  "pi_model_kv_cells_seq_keep", "pi_model_kv_cells_clear", "pi_model_kv_cells_state"]
+                  "pi_model_kv_cells_seq_keep", "pi_model_kv_cells_seq_shift", "pi_model_kv_cells_clear", "pi_model_kv_cells_state"]
 
 
 def _type_of(a, hint):
@@ -259,6 +260,9 @@ class Model:
 
     def kv_cells_seq_keep(self, seq):
         check(self.L.pi_model_kv_cells_seq_keep(self.h, seq), "pi_model_kv_cells_seq_keep")
+
+    def kv_cells_seq_shift(self, seq, p0, p1, delta):
+        check(self.L.pi_model_kv_cells_seq_shift(self.h, seq, p0, p1, delta), "pi_model_kv_cells_seq_shift")
 
     def kv_cells_clear(self):
         check(self.L.pi_model_kv_cells_clear(self.h), "pi_model_kv_cells_clear")

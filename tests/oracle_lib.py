@@ -194,10 +194,18 @@ class KVCells:
         self.delta = np.zeros(n_ctx, np.int64)
         self.seq = [set() for _ in range(n_ctx)]
 
+    @staticmethod
+    def _ids(seq_id, n):
+        """one id for every token, one per token, or a list of ids per token -> a list of id lists"""
+        per_token = list(seq_id) if isinstance(seq_id, (list, tuple, np.ndarray)) else [seq_id] * n
+        return [[int(v) for v in t] if isinstance(t, (list, tuple, set, np.ndarray)) else [int(t)] for t in per_token]
+
     def find_slot(self, positions, seq_id=0):          # llama_kv_cache_find_slot, llama.cpp:1683-1736
-        """seq_id: one id for every token, or one per token."""
-        seq_ids = list(seq_id) if np.ndim(seq_id) else [seq_id] * len(positions)
+        """seq_id: one id for every token, one per token, or a list of ids per token."""
+        seq_ids = self._ids(seq_id, len(positions))
         n, tested = len(positions), 0
+        if n > self.size:
+            raise RuntimeError("no KV slot")
         while True:
             if self.head + n > self.size:
                 tested += self.size - self.head
@@ -212,8 +220,45 @@ class KVCells:
                 raise RuntimeError("no KV slot")
         for i, p in enumerate(positions):
             self.pos[self.head + i] = p
-            self.seq[self.head + i].add(seq_ids[i])
+            self.seq[self.head + i].update(seq_ids[i])
         return self.head
+
+    def decode(self, positions, seq_id=0):             # the cache's part of llama_decode_internal, llama.cpp:6834-6842, 6925-6943
+        """slot for the step, the cell range it looks at, its mask; pending shifts count as applied; then the head moves past the step.
+        Returns (first cell, n_kv, mask [n_tokens][n_kv]) or None when no run of free cells is left (llama_decode returns 1)."""
+        try:
+            first = self.find_slot(positions, seq_id)
+        except RuntimeError:
+            return None
+        n_kv = min(self.size, max(32, self.cell_max()))
+        m = self.mask(positions, n_kv, seq_id)
+        self.has_shift = False
+        self.delta[:] = 0
+        self.head += len(positions)
+        if self.head >= self.size:
+            self.head = 0
+        return first, n_kv, m
+
+    def seq_keep(self, seq_id):                         # llama_kv_cache_seq_keep, llama.cpp:1805-1822
+        new_head = self.size
+        for i in range(self.size):
+            if seq_id not in self.seq[i]:
+                self.pos[i] = -1
+                self.seq[i] = set()
+                new_head = min(new_head, i)
+            else:
+                self.seq[i] = {seq_id}
+        if new_head != self.size:
+            self.head = new_head
+
+    def clear(self):                                    # llama_kv_cache_clear, llama.cpp:1745-1751
+        self.pos[:] = -1
+        self.seq = [set() for _ in range(self.size)]
+        self.head = 0
+
+    def state(self):
+        """(positions, sequence sets as bit masks, head) as arrays"""
+        return self.pos.astype(np.int32), np.array([sum(1 << s for s in c) for c in self.seq], np.uint32), int(self.head)
 
     def cell_max(self):                                 # llama_kv_cache_cell_max, llama.cpp:1739-1747
         for i in range(self.size - 1, 0, -1):
@@ -257,8 +302,8 @@ class KVCells:
                     new_head = min(new_head, i)
         self.head = new_head if new_head != self.size else 0
 
-    def mask(self, positions, n_kv, seq_id=0):          # KQ_mask, llama.cpp:6506-6531
-        seq_ids = list(seq_id) if np.ndim(seq_id) else [seq_id] * len(positions)
+    def mask(self, positions, n_kv, seq_id=0):          # KQ_mask, llama.cpp:6506-6531 (by the token's first sequence id)
+        seq_ids = [t[0] for t in self._ids(seq_id, len(positions))]
         m = np.zeros((len(positions), n_kv), np.float32)
         for j, p in enumerate(positions):
             for i in range(n_kv):

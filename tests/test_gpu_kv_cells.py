@@ -1,16 +1,11 @@
 """One KV cache with cells shared between sequences (pi_model_kv_cells_*): the cells' bookkeeping against the restatement of
-llama_kv_cache (oracle/kv_cells.py), and the logits of sequences that share cells against the CPU oracle evaluating every
+llama_kv_cache (oracle_lib.KVCells), and the logits of sequences that share cells against the CPU oracle evaluating every
 sequence on its own."""
-import os
-import sys
-
 import numpy as np
 import pytest
 
-sys.path.insert(0, os.path.join(os.path.dirname(os.path.abspath(__file__)), "..", "oracle"))
-import kv_cells  # noqa: E402
-import oracle_lib as ol  # noqa: E402
-from powerinfer_amd import synth  # noqa: E402
+import oracle_lib as ol
+from powerinfer_amd import synth
 
 pytestmark = pytest.mark.gpu
 
@@ -20,7 +15,8 @@ def rel_err(a, b):
 
 
 def test_cells_follow_the_reference_bookkeeping():
-    """A random walk of steps (one to six tokens, one or several sequences per token), removals, copies and keeps on a 64-cell cache:
+    """A random walk of steps (one to six tokens, one or several sequences per token), removals, copies, keeps and position shifts on a
+    64-cell cache:
     after every operation the cells' positions, sequence sets and the ring's head equal the restatement's, and a step finds no slot
     exactly when the restatement finds none."""
     from powerinfer_amd import lib as pl
@@ -28,12 +24,12 @@ def test_cells_follow_the_reference_bookkeeping():
     hp = synth.hparams("llama-tiny", seed=3, n_ctx=64)
     gm = Model(hp).load(synth.make_model(hp))
     gm.kv_cells_init(64)
-    ref = kv_cells.KvCells(64)
+    ref = ol.KVCells(64)
     rng = np.random.default_rng(7)
     next_pos = [0] * 6
     n_fail = 0
     for it in range(140):
-        op = rng.choice(["step", "step", "step", "rm", "cp", "keep"], p=[0.3, 0.3, 0.2, 0.1, 0.07, 0.03])
+        op = rng.choice(["step", "step", "step", "rm", "cp", "keep", "shift"], p=[0.3, 0.3, 0.15, 0.1, 0.07, 0.03, 0.05])
         if op == "step":
             n = int(rng.integers(1, 7))
             seqs, pos = [], []
@@ -61,6 +57,11 @@ def test_cells_follow_the_reference_bookkeeping():
             a, b = (int(v) for v in rng.choice(6, 2, replace=False))
             ref.seq_cp(a, b, 0, -1)
             gm.kv_cells_seq_cp(a, b, 0, -1)
+        elif op == "shift":
+            s, p0, dl = int(rng.integers(0, 6)), int(rng.integers(0, 6)), int(rng.integers(-4, 3))
+            ref.seq_shift(s, p0, -1, dl)
+            gm.kv_cells_seq_shift(s, p0, -1, dl)
+            next_pos[s] = max(0, next_pos[s] + dl)
         else:
             s = int(rng.integers(0, 6))
             ref.seq_keep(s)
@@ -131,6 +132,40 @@ def test_a_prompt_evaluated_once_serves_every_continuation(arch, wtype):
     for om in oms + [om3]:
         om.close()
     gm.close()
+
+
+@pytest.mark.parametrize("arch", ["llama-tiny", "falcon-tiny"])
+def test_a_context_shift_in_the_shared_cell_cache(arch):
+    """The context shift of examples/main (llama_kv_cache_seq_rm of a range, llama_kv_cache_seq_shift of what lies behind it): the
+    positions move at once, the K rows are rotated at the start of the next step (llm_build_k_shift on the reference's cache layout).
+    The steps after the shift against this library's per-sequence cache doing the same edit (pi_model_kv_seq_rm / _seq_shift, which
+    the reference's own context-shift logits pin, tests/test_gpu_model.py), and a second sequence that shares the shifted cells."""
+    from powerinfer_amd.model import Model
+    hp = synth.hparams(arch, seed=9, n_ctx=64, pred_margin=True, head_pair=2048)      # no neuron on the threshold: the two attention kernels round differently
+    model = synth.make_model(hp)
+    rng = np.random.default_rng(5)
+    toks = rng.integers(0, hp.n_vocab, 20)
+    ga, gb = Model(hp).load(model), Model(hp).load(model)
+    gb.kv_cells_init(32)
+    for i in range(12):
+        _, la = ga.decode([int(toks[i])], i)
+        _, lb = gb.kv_cells_decode([toks[i]], [i], [0])
+        assert rel_err(lb[0], la) < 1e-2, (i, rel_err(lb[0], la))
+    gb.kv_cells_seq_cp(0, 1, 0, -1)                              # sequence 1 shares every cell: the shift below moves them for both
+    ga.kv_seq_rm(2, 6)
+    ga.kv_seq_shift(6, -1, -4)
+    gb.kv_cells_seq_rm(0, 2, 6)
+    gb.kv_cells_seq_rm(1, 2, 6)
+    gb.kv_cells_seq_shift(0, 6, -1, -4)
+    pos, seq, head = gb.kv_cells_state()
+    assert list(pos[:12]) == [0, 1, -1, -1, -1, -1, 2, 3, 4, 5, 6, 7] and np.all(seq[6:12] == 0b11) and head == 0
+    for i in range(12, 16):
+        _, la = ga.decode([int(toks[i])], i - 4)
+        nxt, lb = gb.kv_cells_decode([toks[i], toks[i]], [i - 4, i - 4], [0, 1])      # both sequences take the same token: same logits
+        assert rel_err(lb[0], la) < 1e-2 and rel_err(lb[1], la) < 1e-2, (i, rel_err(lb[0], la), rel_err(lb[1], la))
+    pos, _, _ = gb.kv_cells_state()
+    assert list(pos[2:6]) == [8, 8, 9, 9]                        # the freed cells were found again, two per step
+    ga.close(), gb.close()
 
 
 def test_kv_cells_refuse_what_they_cannot_hold():

@@ -893,7 +893,6 @@ int pi_k_gemm_f16(const void * W, int rows, int cols, const void * xn_f16, int T
     return gemm_launch("pi_k_gemm_f16", W, rows, cols, xn_f16, T, epilogue, add1, add2, y, y_f16, 0.0f, nullptr, stream);
 }
 
-// Output tiles the kernel is built for (weight rows x tokens per workgroup); two workgroups share a compute unit.
 // Output tiles the kernel is built for (weight rows x tokens per workgroup); the first two run eight waves, one workgroup per unit.
 constexpr int kGtNShapes = 7;
 static const int kGtShapes[kGtNShapes][2] = {{256, 128}, {192, 128}, {128, 128}, {96, 128}, {128, 64}, {64, 128}, {64, 64}};

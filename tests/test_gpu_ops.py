@@ -454,6 +454,32 @@ def test_attention_of_a_step_on_the_reference_cache_layouts(mode, hd, nh, nkv, T
                                  scale.ptr, dmask.ptr, 40, dout.ptr, d + 4, None) != 0                   # more than 16 tokens
 
 
+@pytest.mark.parametrize("mode,fs", [(0, 1.0), (2, 0.5)])
+def test_k_shift_on_the_reference_cache_layout(mode, fs):
+    """pi_k_k_shift_cells rotates K cells laid out [layer][cell][kv head][hd] (the view llm_build_k_shift rotates): the same data
+    permuted into [layer * kv head][cell][hd] and sent through pi_k_k_shift, which test_k_shift_and_compaction holds to the
+    reference's fp16 RoPE, must come out bit for bit the same; cells with delta 0 keep their bits."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    n_layer, n_cells, nkv, hd = 3, 40, 2, 64
+    rng = np.random.default_rng(3 + mode)
+    k = rng.standard_normal((n_layer, n_cells, nkv, hd)).astype(np.float16)
+    delta = rng.integers(-9, 10, n_cells).astype(np.int32)
+    delta[::3] = 0
+    theta_scale = float(np.float32(10000.0) ** np.float32(-2.0 / hd))
+    ka = pl.DevBuf(host=k)
+    kb = pl.DevBuf(host=np.ascontiguousarray(k.transpose(0, 2, 1, 3)))          # [layer][kv head][cell][hd]
+    dd = pl.DevBuf(host=delta)
+    pl.check(L.pi_k_k_shift_cells(ka.ptr, n_layer, n_cells, nkv, hd, mode, theta_scale, fs, dd.ptr, None), "k_shift_cells")
+    pl.check(L.pi_k_k_shift(kb.ptr, n_layer * nkv, n_cells, hd, mode, theta_scale, fs, dd.ptr, n_cells, None), "k_shift")
+    pl.sync()
+    got = ka.download(np.float16).reshape(n_layer, n_cells, nkv, hd)
+    want = kb.download(np.float16).reshape(n_layer, nkv, n_cells, hd).transpose(0, 2, 1, 3)
+    assert np.array_equal(got.view(np.uint16), want.view(np.uint16))
+    assert np.array_equal(got[:, delta == 0].view(np.uint16), k[:, delta == 0].view(np.uint16))
+    assert not np.array_equal(got[:, delta != 0].view(np.uint16), k[:, delta != 0].view(np.uint16))
+
+
 def test_embed_and_argmax():
     from powerinfer_amd import lib as pl
     L = pl.init()

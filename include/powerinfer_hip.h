@@ -318,7 +318,7 @@ PI_API int pi_k_gemm_tile_f16(const void * W_f16, int rows, int cols, const void
  * pi_k_q4_split writes a Q4_0 matrix [rows][cols / 32] blocks as two arrays, quants (16 bytes per block, the dwords of four consecutive
  * blocks interleaved: [row][block / 4][dword][block % 4]) and scales [rows][cols / 32] fp16 (cols % 256 == 0); pi_k_norm_q8_blocks
  * normalises T <= 16 rows and quantises them as quantize_row_q8_0 does (ggml-quants.c:702-760) into q int8 [T][cols], d float
- * [cols / 32][16] and s8 = 8 * sum(q) int32 [cols / 32][16] (token innermost; cols <= 8192), and, if plain_f16 != NULL, also writes the
+ * [cols / 32][16] and s8 = -8 * sum(q) int32 [cols / 32][16] (token innermost; cols <= 8192), and, if plain_f16 != NULL, also writes the
  * rows before the norm as fp16 (the predictor's input); pi_k_gemm_q4_t16 is y[t][row] = epilogue(W[row] . x[t]) on those forms; pi_k_batch_sparse_ffn_q4 is
  * pi_k_batch_sparse_ffn on them: the union list from the flags pi_k_batch_predictor_fc2 left in the workspace, up/gate dots of the
  * union rows, h [16][ff] under the predictor's mask, hq = the values h's Q8_0 blocks keep (blocks of 32 consecutive neurons, as the

@@ -9,7 +9,8 @@
 // the integer MFMA reads its dword of four blocks as one 16-byte load, and a wave's 16 rows x 64 bytes per load are whole half
 // cache lines whose other half the next load takes.
 // Activations come as Q8_0 blocks in three arrays (pi_k_norm_q8_blocks): int8 quants in the MFMA's operand layout, scale d [nblk][16] and
-// 8 * sum(q) [nblk][16] - the nibbles go into the MFMA unsigned, and sum((q - 8) * x) = sum(q * x) - 8 * sum(x) stays exact in int32.
+// -8 * sum(q) [nblk][16] - the nibbles go into the MFMA unsigned and the MFMA's accumulator input carries -8 * sum(x), so that
+// sum((q - 8) * x) = sum(q * x) - 8 * sum(x) comes out of the instruction, exact in int32.
 #include "kernels_common.hpp"
 
 namespace {
@@ -29,7 +30,7 @@ __global__ void q4_split_kernel(const pi_block_q4_0 * __restrict__ w, size_t n_b
 }
 
 // One row per workgroup: norm (as norm_round_f16_kernel), then Q8_0 blocks of 32 (quantize_row_q8_0, ggml-quants.c:702-760):
-// d = fp16(amax / 127), q = rint(v * (127 / amax)).  Outputs: q in the MFMA's operand layout (below), d and 8 * sum(q) as [blk][16]
+// d = fp16(amax / 127), q = rint(v * (127 / amax)).  Outputs: q in the MFMA's operand layout (below), d and -8 * sum(q) as [blk][16]
 // (token innermost).
 __global__ __launch_bounds__(1024) void norm_q8_blocks_kernel(const float * __restrict__ x, int cols, NormArgs na, int8_t * __restrict__ q_out,
                                                               float * __restrict__ d_out, int * __restrict__ s8_out, __half * __restrict__ plain16) {
@@ -65,6 +66,7 @@ __global__ __launch_bounds__(1024) void norm_q8_blocks_kernel(const float * __re
     }
 #pragma unroll
     for (int k = 0; k < 8; ++k) {
+        if (k * 1024 >= cols) break;                              // uniform: the row ends before this slot
         const int i = threadIdx.x + k * 1024;
         float v = xv[k];
         if (plain16 && i < cols) plain16[(size_t)t * cols + i] = __float2half_rn(v);
@@ -88,7 +90,7 @@ __global__ __launch_bounds__(1024) void norm_q8_blocks_kernel(const float * __re
             // 16 + 4g .. 16 + 4g + 3 of the block, so that a lane's 8-byte operand is one load and a wave's 64 lanes read 512 contiguous bytes
             const int e = i & 31;
             q_out[(((size_t)(i >> 5) * 4 + ((e & 15) >> 2)) * 16 + t) * 8 + (e >> 4) * 4 + (e & 3)] = (int8_t)q;
-            if ((i & 31) == 0) { d_out[(size_t)(i >> 5) * 16 + t] = d; s8_out[(size_t)(i >> 5) * 16 + t] = 8 * s; }
+            if ((i & 31) == 0) { d_out[(size_t)(i >> 5) * 16 + t] = d; s8_out[(size_t)(i >> 5) * 16 + t] = -8 * s; }
         }
     }
 }
@@ -160,20 +162,21 @@ __global__ __launch_bounds__(kBlock) void gemm_q4_t16_kernel(const uint32_t * __
             for (int m = 0; m < NM; ++m) {
                 const uint32_t w = u < 4 ? L.w0[m][u & 3] : L.w1[m][u & 3];
                 const unsigned long lo = w & 0x0F0F0F0Fu, hi = (w >> 4) & 0x0F0F0F0Fu;
-                const pi_i4 sum = __builtin_amdgcn_mfma_i32_16x16x32_i8((long)L.a[u], (long)((hi << 32) | lo), pi_i4{0, 0, 0, 0}, 0, 0, 0);
+                // the accumulator input carries -8 * sum(x) of the activation block: the result is sum((q - 8) * x), exact in int32
+                const pi_i4 sum = __builtin_amdgcn_mfma_i32_16x16x32_i8((long)L.a[u], (long)((hi << 32) | lo), sxs, 0, 0, 0);
                 const uint32_t dpair = L.wd[m][u >> 1];
                 const float dw = pi_f16_from_bits((uint16_t)((u & 1) ? (dpair >> 16) : (dpair & 0xFFFFu)));
-                acc[m][0] = fmaf(__fmul_rn(dw, dxs.x), (float)(sum[0] - sxs[0]), acc[m][0]);
-                acc[m][1] = fmaf(__fmul_rn(dw, dxs.y), (float)(sum[1] - sxs[1]), acc[m][1]);
-                acc[m][2] = fmaf(__fmul_rn(dw, dxs.z), (float)(sum[2] - sxs[2]), acc[m][2]);
-                acc[m][3] = fmaf(__fmul_rn(dw, dxs.w), (float)(sum[3] - sxs[3]), acc[m][3]);
+                acc[m][0] = fmaf(__fmul_rn(dw, dxs.x), (float)sum[0], acc[m][0]);
+                acc[m][1] = fmaf(__fmul_rn(dw, dxs.y), (float)sum[1], acc[m][1]);
+                acc[m][2] = fmaf(__fmul_rn(dw, dxs.z), (float)sum[2], acc[m][2]);
+                acc[m][3] = fmaf(__fmul_rn(dw, dxs.w), (float)sum[3], acc[m][3]);
             }
         }
     };
     // A wave's groups (wave, wave + 4, ...) go in rounds of four: all loads of a round are issued before its first multiply, so
     // a row of 4096 columns costs one trip to memory per wave instead of four; the first round's loads are already under way
     // while the workgroup stages the scales.
-    constexpr int kRound = 4;
+    constexpr int kRound = 2;
     Loads L[kRound];
 #pragma unroll
     for (int u = 0; u < kRound; ++u) if (wave + u * kWavesPerBlock < ngroups) fetch(L[u], wave + u * kWavesPerBlock);

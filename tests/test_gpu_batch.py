@@ -402,7 +402,7 @@ def test_norm_q8_blocks_match_the_reference_quantiser(kind):
     got_s = s.download(np.int32).reshape(cols // 32, 16).T[:T]
     assert np.array_equal(got_d, want_d)
     assert (got_q != want_q).mean() < 1e-3           # a value on a rounding boundary after the norm's last bit
-    assert np.array_equal(got_s, 8 * got_q.reshape(T, cols // 32, 32).astype(np.int32).sum(-1))
+    assert np.array_equal(got_s, -8 * got_q.reshape(T, cols // 32, 32).astype(np.int32).sum(-1))
 
 
 @pytest.mark.parametrize("shape,has_gate,T", [((4096, 11008, 1024), True, 16), ((4096, 11008, 1024), False, 5), ((1024, 1024, 128), True, 3)])

@@ -724,69 +724,88 @@ __global__ __launch_bounds__(kBaBlock) void batch_axpy_f16_kernel(const __half *
 }
 
 // The down projection on the matrix cores (cols % 256 == 0).  out[t][c] = sum_u h[t][u] * down[row_u][c] has the union rows as its
-// reduction dimension, along which the weight matrix is NOT contiguous, so the operand layout cannot be loaded directly: a wave
-// reads 16 union rows x 256 columns row-contiguously (2 rows x 512 B per instruction), drops them into its private LDS tile and
-// reads the B fragments column-wise (4 rows of one column per lane: four 2-byte LDS reads) for 16 column tiles of
-// v_mfma_f32_16x16x16_f16; the A fragment is 4 consecutive entries of h[t][.] (one 8-byte load from the token-major h).
-// grid = (cols / 1024, G row groups); wave w of a workgroup owns columns 256 w .. 256 w + 255 of the workgroup's 1024 and walks
-// the 16-row steps g, g + G, ...; partial[g][t][c] is summed by batch_reduce_kernel.
+// reduction dimension, along which the weight matrix is NOT contiguous, while the B operand of v_mfma_f32_16x16x16_f16 wants four
+// consecutive k (rows) of ONE column per lane.  The operand's column index is free to name any column, though: lane (i, g) loads
+// 16 bytes = columns 8 i .. 8 i + 7 of rows 4 g .. 4 g + 3 (per instruction 4 rows x 256 contiguous bytes), and the e-th of eight
+// MFMAs takes column 8 i + e of those four rows, two v_perm_b32 per operand and no trip through LDS; accumulator e then holds
+// out[4 g + r][8 i + e], eight consecutive columns per lane for the store.  The A fragment is 4 consecutive entries of h[t][.]
+// (one 8-byte load from the token-major h).
+// grid = (cols / 512, G row groups), two waves a workgroup; a wave owns 256 columns (two 128-column halves) and walks the 16-row
+// steps g, g + G, ...; partial[g][t][c] is summed by batch_reduce_kernel.  At 5120 columns and 5720 union rows a launch takes
+// 15.5 us for 58.6 MB of rows and 10.5 MB of partial sums; four waves a workgroup, or 250 workgroups held one to a compute
+// unit, take the same time, one wave a workgroup with 128 columns and eight steps in flight takes 18 us.
 typedef _Float16 pi_h4 __attribute__((ext_vector_type(4)));
 __global__ __launch_bounds__(kBlock) void batch_axpy_mfma_f16_kernel(const __half * __restrict__ Wd, int cols, const __half * __restrict__ hc, int hstride,
                                                                      const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
                                                                      float * __restrict__ partial) {
-    __shared__ __align__(16) unsigned char tile[kWavesPerBlock][16 * kGlStride];
     const int n = *n_union;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int i = lane & 15, g = lane >> 4;
-    const int lr = lane >> 5, lc = lane & 31;
-    const int c0 = blockIdx.x * 1024 + wave * 256;
+    const int c0 = (blockIdx.x * (blockDim.x >> 6) + wave) * 256;
     if (c0 >= cols) return;                               // no workgroup barrier below: waves are independent
-    unsigned char * mytile = tile[wave];
     pi_f4 acc[16];
 #pragma unroll
     for (int ct = 0; ct < 16; ++ct) acc[ct] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
     const int n_steps = (n + 15) / 16;
-    pi_u32x4 ld[2][8];
-    pi_u32x2 af[2];
-    auto issue = [&](int buf, int ks) {
-        if (ks < n_steps) {
-            const int u0 = ks * 16;
+    // Four 16-row steps of loads in flight per wave: a wave is alone on its SIMD most of the time, so what it has requested is all
+    // that hides the trip to memory.  Two things keep the requests in flight: the row numbers come through the scalar unit (sixteen
+    // uniform loads and a select on g; a vector load of them would sit between the weight loads in the in-order counter and every
+    // wait for a row number would drain the weights before it), and every round issues all of its loads unconditionally (steps
+    // behind the group's last re-read that step, a cache hit), so the wait before a step's first MFMA is an exact count.
+    constexpr int NB = 4;
+    const int G = gridDim.y;
+    const int my_steps = (n_steps - (int)blockIdx.y + G - 1) / G;                           // steps blockIdx.y, + G, ... of this group
+    pi_u32x4 ld[NB][8];
+    pi_u32x2 af[NB];
+    auto issue = [&](int buf, int s) {
+        const int u0 = ((int)blockIdx.y + (s < my_steps ? s : my_steps - 1) * G) * 16;
 #pragma unroll
-            for (int j = 0; j < 8; ++j) {
-                const int u = u0 + 2 * j + lr;
-                ld[buf][j] = pi_ld_stream(Wd + (size_t)list[u < n ? u : n - 1] * cols + c0 + lc * 8);
-            }
-            af[buf] = *reinterpret_cast<const pi_u32x2 *>(hc + (size_t)i * hstride + u0 + 4 * g);      // zeros beyond n (written by the gate/up kernel)
+        for (int r = 0; r < 4; ++r) {
+            // (readfirstlane pins the four loads to the scalar unit, ahead of the select)
+            const int r0 = __builtin_amdgcn_readfirstlane(list[u0 + r < n ? u0 + r : n - 1]);
+            const int r1 = __builtin_amdgcn_readfirstlane(list[u0 + 4 + r < n ? u0 + 4 + r : n - 1]);
+            const int r2 = __builtin_amdgcn_readfirstlane(list[u0 + 8 + r < n ? u0 + 8 + r : n - 1]);
+            const int r3 = __builtin_amdgcn_readfirstlane(list[u0 + 12 + r < n ? u0 + 12 + r : n - 1]);
+            const __half * wp = Wd + (size_t)(g == 0 ? r0 : g == 1 ? r1 : g == 2 ? r2 : r3) * cols + c0 + 8 * i;
+            ld[buf][2 * r]     = pi_ld_stream(wp);
+            ld[buf][2 * r + 1] = pi_ld_stream(wp + 128);
         }
+        af[buf] = *reinterpret_cast<const pi_u32x2 *>(hc + (size_t)i * hstride + u0 + 4 * g);      // zeros beyond n (written by the gate/up kernel)
     };
-    issue(0, blockIdx.y);
-    issue(1, blockIdx.y + kBmGroups);
-    for (int ks = blockIdx.y; ks < n_steps; ks += 2 * kBmGroups) {
+    auto consume = [&](int buf) {
+        const pi_h4 a = __builtin_bit_cast(pi_h4, af[buf]);
 #pragma unroll
-        for (int buf = 0; buf < 2; ++buf) {
-            const int cur = ks + buf * kBmGroups;
-            if (cur < n_steps) {
+        for (int half = 0; half < 2; ++half)
 #pragma unroll
-                for (int j = 0; j < 8; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (2 * j + lr) * kGlStride + lc * 16) = ld[buf][j];
-                const pi_h4 a = __builtin_bit_cast(pi_h4, af[buf]);
-#pragma unroll
-                for (int ct = 0; ct < 16; ++ct) {
-                    const unsigned char * bp = mytile + (4 * g) * kGlStride + (ct * 16 + i) * 2;
-                    const uint32_t e0 = *reinterpret_cast<const uint16_t *>(bp), e1 = *reinterpret_cast<const uint16_t *>(bp + kGlStride);
-                    const uint32_t e2 = *reinterpret_cast<const uint16_t *>(bp + 2 * kGlStride), e3 = *reinterpret_cast<const uint16_t *>(bp + 3 * kGlStride);
-                    const pi_u32x2 bw = {e0 | (e1 << 16), e2 | (e3 << 16)};
-                    acc[ct] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, __builtin_bit_cast(pi_h4, bw), acc[ct], 0, 0, 0);
-                }
+            for (int e2 = 0; e2 < 4; ++e2) {
+                const uint32_t w0 = ld[buf][half][e2], w1 = ld[buf][2 + half][e2], w2 = ld[buf][4 + half][e2], w3 = ld[buf][6 + half][e2];
+                const pi_u32x2 lo = {__builtin_amdgcn_perm(w1, w0, 0x05040100u), __builtin_amdgcn_perm(w3, w2, 0x05040100u)};
+                const pi_u32x2 hi = {__builtin_amdgcn_perm(w1, w0, 0x07060302u), __builtin_amdgcn_perm(w3, w2, 0x07060302u)};
+                acc[half * 8 + 2 * e2]     = __builtin_amdgcn_mfma_f32_16x16x16f16(a, __builtin_bit_cast(pi_h4, lo), acc[half * 8 + 2 * e2], 0, 0, 0);
+                acc[half * 8 + 2 * e2 + 1] = __builtin_amdgcn_mfma_f32_16x16x16f16(a, __builtin_bit_cast(pi_h4, hi), acc[half * 8 + 2 * e2 + 1], 0, 0, 0);
             }
-            issue(buf, cur + 2 * kBmGroups);
+    };
+    if (my_steps > 0) {
+#pragma unroll
+        for (int buf = 0; buf < NB; ++buf) issue(buf, buf);
+        int s = 0;
+        for (; s + NB < my_steps; s += NB) {
+#pragma unroll
+            for (int buf = 0; buf < NB; ++buf) { consume(buf); issue(buf, s + buf + NB); }
         }
+#pragma unroll
+        for (int buf = 0; buf < NB; ++buf)
+            if (s + buf < my_steps) consume(buf);
     }
-    // accumulator lane l: tokens 4 * (l / 16) .. + 3 of column l % 16 of every column tile
+    // accumulator e of a half, lane (i, g): tokens 4 g .. 4 g + 3 of column 8 i + e of the half
 #pragma unroll
-    for (int ct = 0; ct < 16; ++ct)
+    for (int r = 0; r < 4; ++r)
 #pragma unroll
-        for (int r = 0; r < 4; ++r)
-            partial[((size_t)blockIdx.y * kBtMaxT + 4 * g + r) * cols + c0 + ct * 16 + i] = acc[ct][r];
+        for (int half = 0; half < 2; ++half) {
+            float * dst = partial + ((size_t)blockIdx.y * kBtMaxT + 4 * g + r) * cols + c0 + half * 128 + 8 * i;
+            *reinterpret_cast<float4 *>(dst)     = make_float4(acc[half * 8][r], acc[half * 8 + 1][r], acc[half * 8 + 2][r], acc[half * 8 + 3][r]);
+            *reinterpret_cast<float4 *>(dst + 4) = make_float4(acc[half * 8 + 4][r], acc[half * 8 + 5][r], acc[half * 8 + 6][r], acc[half * 8 + 7][r]);
+        }
 }
 
 __global__ __launch_bounds__(kBlock) void batch_reduce_kernel(const float * __restrict__ partial, int n_groups, int T, int cols, int epi,
@@ -1046,7 +1065,7 @@ int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, 
     if (cols % 256 == 0) {
         hipLaunchKernelGGL(batch_upgate_lds_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
                            (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride, (float *)nullptr);
-        hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3((cols + 1023) / 1024, kBmGroups), dim3(kBlock), 0, st, (const __half *)down_t_f16, cols,
+        hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3((cols + 511) / 512, kBmGroups), dim3(128), 0, st, (const __half *)down_t_f16, cols,
                            ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
         hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBmGroups, T, cols, epilogue, add1, add2, out);
     } else {
@@ -1091,7 +1110,7 @@ int pi_k_batch_sparse_axpy(const void * down_t_f16, int cols, int ff, const floa
     hipLaunchKernelGGL(batch_flag_any_kernel, dim3((ff + 255) / 256), dim3(256), 0, st, idx, T, ff, threshold, ws->row_any);
     hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, ws->row_any, ff, ws->words, union_rows, n_union);
     hipLaunchKernelGGL(batch_gather_h_kernel, dim3(32, kBtMaxT), dim3(256), 0, st, h, idx, T, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
-    hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3((cols + 1023) / 1024, kBmGroups), dim3(kBlock), 0, st, (const __half *)down_t_f16, cols,
+    hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3((cols + 511) / 512, kBmGroups), dim3(128), 0, st, (const __half *)down_t_f16, cols,
                        ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
     hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBmGroups, T, cols, PI_EPI_NONE,
                        (const float *)nullptr, (const float *)nullptr, out);

@@ -275,42 +275,67 @@ __global__ __launch_bounds__(kBlock) void batch_axpy_q4_kernel(const uint32_t * 
     for (int e = 0; e < 8; ++e) acc[e] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
     const int nquads = (nu + 3) / 4;
     const int stride = kQ4AxpyGroups * kWavesPerBlock;
-    // quad of this wave's u-th slot in iteration it: (blockIdx.y * 4 + wave) + (it * kQ4AxpyUnroll + u) * stride
-    int rows_next[kQ4AxpyUnroll];
-    auto rows_of = [&](int it, int * out) {
+    // quad of this wave's u-th slot in iteration it: q0 + (it * kQ4AxpyUnroll + u) * stride.  The loads of three iterations are in flight
+    // while a fourth is multiplied.  What keeps them in flight: a quad's four row numbers come through the scalar unit (one
+    // 16-byte load; vector loads of them would sit in the in-order counter of the weight loads, and waiting for a row number would
+    // drain the weights requested before it), and every load is unconditional - a slot behind the list's end reads the wave's last quad again (every
+    // wave reading ONE row there would queue up on that row's memory channel) and counts with h = 0 - so that the wait before an iteration's first MFMA is an exact count.  (union_rows holds ff entries and ff % 4 == 0.)
+    const int q0 = (int)blockIdx.y * kWavesPerBlock + __builtin_amdgcn_readfirstlane(wave);
+    const int q_last = q0 < nquads ? q0 + (nquads - 1 - q0) / stride * stride : 0;       // this wave's last quad
+    struct Quad { uint32_t w[kQ4AxpyUnroll]; uint16_t dw[kQ4AxpyUnroll]; float a[kQ4AxpyUnroll]; bool live[kQ4AxpyUnroll]; };
+    int4 rn[kQ4AxpyUnroll];                                        // the row numbers of the next fetch's quads (uniform: scalar registers)
+    auto fetch_rows = [&](int it) {
 #pragma unroll
         for (int u = 0; u < kQ4AxpyUnroll; ++u) {
-            const int k = (((int)blockIdx.y * kWavesPerBlock + wave) + (it * kQ4AxpyUnroll + u) * stride) * 4 + g;
-            out[u] = k < nu ? union_rows[k] : -1;
+            const int q = q0 + (it * kQ4AxpyUnroll + u) * stride;
+            rn[u] = *reinterpret_cast<const int4 *>(union_rows + 4 * (q < nquads ? q : q_last));
         }
     };
-    // two iterations ahead: the union rows; one ahead: the rows' quants, scales and h values
-    struct Quad { uint32_t w[kQ4AxpyUnroll]; float dw[kQ4AxpyUnroll], a[kQ4AxpyUnroll]; };
-    auto fetch = [&](Quad & Q, const int * n) {
+    auto fetch = [&](Quad & Q, int it) {                            // uses the row numbers requested one fetch earlier, requests the next ones
 #pragma unroll
         for (int u = 0; u < kQ4AxpyUnroll; ++u) {
-            const size_t row = (size_t)(n[u] < 0 ? 0 : n[u]);
-            Q.w[u] = qs[(row * nblk + (size_t)blockIdx.x * 4) * 4 + i];
-            Q.dw[u] = n[u] < 0 ? 0.0f : pi_f16_from_bits(ds[row * nblk + cb]);
-            Q.a[u] = n[u] < 0 ? 0.0f : hq[row * kBtMaxT + i];      // token i (entries of tokens beyond T are stale and feed discarded rows)
+            const int q = q0 + (it * kQ4AxpyUnroll + u) * stride;
+            const int r0 = __builtin_amdgcn_readfirstlane(rn[u].x), r1 = __builtin_amdgcn_readfirstlane(rn[u].y);
+            const int r2 = __builtin_amdgcn_readfirstlane(rn[u].z), r3 = __builtin_amdgcn_readfirstlane(rn[u].w);
+            Q.live[u] = q < nquads && 4 * q + g < nu;
+            const int qq = q < nquads ? q : q_last;                 // entry 4 qq of the list is a row of the union
+            const size_t row = (size_t)(4 * qq + g < nu ? (g == 0 ? r0 : g == 1 ? r1 : g == 2 ? r2 : r3) : r0);
+            Q.w[u]  = qs[(row * nblk + (size_t)blockIdx.x * 4) * 4 + i];
+            Q.dw[u] = ds[row * nblk + cb];
+            Q.a[u]  = hq[row * kBtMaxT + i];                       // token i (entries of tokens beyond T are stale and feed discarded rows)
         }
+        fetch_rows(it + 1);
     };
-    const int q0 = (int)blockIdx.y * kWavesPerBlock + wave;
-    rows_of(0, rows_next);
-    Quad cur, nxt;
-    fetch(cur, rows_next);
-    rows_of(1, rows_next);
-    for (int it = 0; q0 + it * kQ4AxpyUnroll * stride < nquads; ++it) {
-        fetch(nxt, rows_next);                                     // past the end: rows_of gave -1, the loads read row 0 and count as zeros
-        rows_of(it + 2, rows_next);
+    auto consume = [&](const Quad & Q) {
 #pragma unroll
-        for (int u = 0; u < kQ4AxpyUnroll; ++u)
+        for (int u = 0; u < kQ4AxpyUnroll; ++u) {
+            const float a = Q.live[u] ? Q.a[u] : 0.0f, dw = pi_f16_from_bits(Q.dw[u]), m8 = -8.0f * dw;
+            // d_w * (q - 8) as fma(q, d_w, -8 d_w): the same single rounding of the same exact product (8 d_w is exact), and a byte of
+            // the masked dword converts to float in one instruction: two VALU operations per MFMA instead of four
+            const uint32_t lo = Q.w[u] & 0x0F0F0F0Fu, hi = (Q.w[u] >> 4) & 0x0F0F0F0Fu;
 #pragma unroll
             for (int e = 0; e < 8; ++e) {
-                const int nib = e < 4 ? (int)((cur.w[u] >> (8 * e)) & 0xF) : (int)((cur.w[u] >> (8 * (e - 4) + 4)) & 0xF);
-                acc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(cur.a[u], __fmul_rn(cur.dw[u], (float)(nib - 8)), acc[e], 0, 0, 0);
+                const float nib = (float)(((e < 4 ? lo : hi) >> (8 * (e & 3))) & 0xFFu);
+                acc[e] = __builtin_amdgcn_mfma_f32_16x16x4f32(a, fmaf(nib, dw, m8), acc[e], 0, 0, 0);
             }
-        cur = nxt;
+        }
+    };
+    const int n_it = q0 < nquads ? (nquads - q0 + kQ4AxpyUnroll * stride - 1) / (kQ4AxpyUnroll * stride) : 0;
+    if (n_it > 0) {
+        // three iterations of loads in flight behind the one being multiplied
+        Quad S0, S1, S2, S3;
+        fetch_rows(0);
+        fetch(S0, 0); fetch(S1, 1); fetch(S2, 2);
+        int it = 0;
+        for (; it + 4 <= n_it; it += 4) {
+            fetch(S3, it + 3); consume(S0);
+            fetch(S0, it + 4); consume(S1);
+            fetch(S1, it + 5); consume(S2);
+            fetch(S2, it + 6); consume(S3);
+        }
+        if (it < n_it) consume(S0);                                 // the last one to three iterations: their loads are on the way
+        if (it + 1 < n_it) consume(S1);
+        if (it + 2 < n_it) consume(S2);
     }
 #pragma unroll
     for (int e = 0; e < 8; ++e)

@@ -660,6 +660,127 @@ __global__ __launch_bounds__(kBlock) void batch_upgate_lds_f16_kernel(const __ha
     else hc[(size_t)t * hstride + u0 + rr] = __float2half_rn(h);
 }
 
+// The same product with the union rows dealt evenly to the compute units.  What bounds these kernels is the unit that has to pull
+// the most bytes (a unit sustains about 1/256 of the chip's rate, weights and activations alike): with one workgroup per 16 union
+// rows, 5720 rows are 358 workgroups, 102 units hold two of them and set the pace, and every workgroup pulls the step's whole
+// activation matrix for its 16 rows.  Here the grid is one workgroup per unit and workgroup b owns union entries [b R, (b + 1) R)
+// with R = n / grid rounded up to even (2 <= R <= 32: two MFMA row tiles that share the activation fragments; beyond 32 * grid
+// union rows a workgroup walks several such chunks).  Eight waves split the 128-column super-steps of the rows (w, w + 8, ...);
+// a wave reads 4 rows x 256 B per instruction, has two super-steps in flight and passes the tiles through its own LDS buffer as
+// batch_upgate_lds_f16_kernel does.  Every load is unconditional, so that the in-order counter gives exact waits: a lane whose row
+// lies behind the chunk's end reads what another lane of the same instruction reads (one request), or the chunk's first 16 bytes.
+constexpr int kUbWaves = 8, kUbBlock = kUbWaves * PI_WAVE, kUbRows = 32, kUbStep = 128, kUbStride = kUbStep * 2 + 16;
+template <bool GATE>
+__global__ __launch_bounds__(kUbBlock, 1) void batch_upgate_bal_f16_kernel(const __half * __restrict__ Wup, const __half * __restrict__ Wgate, int cols,
+                                                                           const __half * __restrict__ xn, int T, const float * __restrict__ logits, int ff, float thr,
+                                                                           const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
+                                                                           __half * __restrict__ hc, int hstride) {
+    __shared__ __align__(16) unsigned char tile[kUbWaves][16 * kUbStride];
+    __shared__ float cu[kUbWaves][kUbRows][17], cg[GATE ? kUbWaves : 1][kUbRows][17];
+    const int n = *n_union;
+    const int G = gridDim.x;
+    int R = (n + G - 1) / G;
+    R = (R + 1) & ~1;
+    R = R < 2 ? 2 : R > kUbRows ? kUbRows : R;
+    const int n_chunks = (n + R - 1) / R;
+    const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
+    const int i = lane & 15, g = lane >> 4;                        // MFMA role: row (token) i, k group g
+    const int lr = lane >> 4, lc = lane & 15;                      // load role: row within the instruction's four, 16-byte piece of the 256-byte row piece
+    const int tok = i < T ? i : T - 1;
+    const char * bp = reinterpret_cast<const char *>(xn + (size_t)tok * cols + g * 8);
+    unsigned char * mytile = tile[wave];
+    const int n_steps = cols / kUbStep;
+    const int n_ss = (n_steps - wave + kUbWaves - 1) / kUbWaves;   // super-steps wave, wave + 8, ... of this wave
+    for (int c = blockIdx.x; c < n_chunks; c += G) {
+        const int u0 = c * R;
+        const int Rc = n - u0 < R ? n - u0 : R;                    // rows of this chunk (the list's last chunk may be short, and odd)
+        uint32_t roff[8];                                          // byte offsets of this lane's 8 load instructions (< 2^32: the launcher's test)
+#pragma unroll
+        for (int j = 0; j < 8; ++j) {
+            const int k = 4 * j + lr;
+            const int kk = k < Rc ? k : 4 * j < Rc ? 4 * j : 0;
+            roff[j] = ((uint32_t)list[u0 + kk] * (uint32_t)cols + (4 * j < Rc ? lc * 8 : 0)) * 2;
+        }
+        pi_f4 au[2], ag[2];
+#pragma unroll
+        for (int t = 0; t < 2; ++t) au[t] = ag[t] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
+        // The weights of two super-steps are in flight; the activations of a super-step are requested when the previous one has been
+        // multiplied, BEFORE the weights that replace it (requested after them, the wait for the activations would drain them).
+        pi_u32x4 lu[2][8], lg[2][8], bb[4];
+        auto issue_b = [&](int s) {
+            const size_t so = (size_t)(wave + (s < n_ss ? s : n_ss - 1) * kUbWaves) * (kUbStep * 2);
+#pragma unroll
+            for (int st = 0; st < 4; ++st) bb[st] = pi_ld16(bp + so + st * 64);
+        };
+        auto issue = [&](int buf, int s) {                         // a super-step behind the wave's last reads the last one again
+            const size_t so = (size_t)(wave + (s < n_ss ? s : n_ss - 1) * kUbWaves) * (kUbStep * 2);
+            const char * wu = reinterpret_cast<const char *>(Wup) + so, * wg = reinterpret_cast<const char *>(Wgate) + so;
+#pragma unroll
+            for (int j = 0; j < 8; ++j) {
+                lu[buf][j] = pi_ld_stream(wu + roff[j]);
+                if (GATE) lg[buf][j] = pi_ld_stream(wg + roff[j]);
+            }
+        };
+        auto consume = [&](int buf) {
+#pragma unroll
+            for (int t = 0; t < 2; ++t) {                          // (the second tile also where the chunk has 16 rows or fewer: straight-line code keeps the waits exact)
+                {
+#pragma unroll
+                    for (int j = 0; j < 4; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (4 * j + lr) * kUbStride + lc * 16) = lu[buf][4 * t + j];
+#pragma unroll
+                    for (int st = 0; st < 4; ++st) {
+                        const pi_u32x4 a = *reinterpret_cast<const pi_u32x4 *>(mytile + i * kUbStride + (4 * st + g) * 16);
+                        au[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a), __builtin_bit_cast(pi_h8, bb[st]), au[t], 0, 0, 0);
+                    }
+                    if (GATE) {
+#pragma unroll
+                        for (int j = 0; j < 4; ++j) *reinterpret_cast<pi_u32x4 *>(mytile + (4 * j + lr) * kUbStride + lc * 16) = lg[buf][4 * t + j];
+#pragma unroll
+                        for (int st = 0; st < 4; ++st) {
+                            const pi_u32x4 a = *reinterpret_cast<const pi_u32x4 *>(mytile + i * kUbStride + (4 * st + g) * 16);
+                            ag[t] = __builtin_amdgcn_mfma_f32_16x16x32_f16(__builtin_bit_cast(pi_h8, a), __builtin_bit_cast(pi_h8, bb[st]), ag[t], 0, 0, 0);
+                        }
+                    }
+                }
+            }
+        };
+        if (n_ss > 0) {
+            issue(0, 0);
+            __builtin_amdgcn_sched_barrier(0);
+            issue_b(0);
+            __builtin_amdgcn_sched_barrier(0);
+            issue(1, 1);
+            __builtin_amdgcn_sched_barrier(0);
+            int s = 0;
+            for (; s + 2 < n_ss; s += 2) {        // (the scheduling barriers keep a phase's loads from rising into the MFMAs that free their registers)
+                consume(0); __builtin_amdgcn_sched_barrier(0); issue_b(s + 1); __builtin_amdgcn_sched_barrier(0); issue(0, s + 2); __builtin_amdgcn_sched_barrier(0);
+                consume(1); __builtin_amdgcn_sched_barrier(0); issue_b(s + 2); __builtin_amdgcn_sched_barrier(0); issue(1, s + 3); __builtin_amdgcn_sched_barrier(0);
+            }
+            consume(0);
+            if (s + 1 < n_ss) { __builtin_amdgcn_sched_barrier(0); issue_b(s + 1); consume(1); }
+        }
+#pragma unroll
+        for (int t = 0; t < 2; ++t)
+#pragma unroll
+            for (int r = 0; r < 4; ++r) { cu[wave][16 * t + 4 * g + r][i] = au[t][r]; if (GATE) cg[wave][16 * t + 4 * g + r][i] = ag[t][r]; }
+        __syncthreads();
+        const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;     // 512 threads: 32 rows x 16 tokens
+        if (rr < Rc) {
+            float h = 0.0f;
+            if (t < T && !(logits[(size_t)t * ff + list[u0 + rr]] < thr)) {
+                float su = cu[0][rr][t], sg = GATE ? cg[0][rr][t] : 0.0f;
+#pragma unroll
+                for (int w = 1; w < kUbWaves; ++w) { su += cu[w][rr][t]; if (GATE) sg += cg[w][rr][t]; }
+                h = GATE ? __fmul_rn(fmaxf(sg, 0.0f), su) : fmaxf(su, 0.0f);
+            }
+            hc[(size_t)t * hstride + u0 + rr] = __float2half_rn(h);
+        }
+        // the down projection reads h in steps of 16 union entries: zeros behind the list's end
+        if (c == n_chunks - 1 && rr < ((n + 15) & ~15) - n) hc[(size_t)t * hstride + n + rr] = __float2half_rn(0.0f);
+        __syncthreads();                                           // cu / cg are reused by the next chunk
+    }
+}
+
 // sparse down projection for the step: partial[g][t][c] = sum over the union entries of row group g of hc[u][t] * down[row_u][c].
 // A workgroup of 8 waves owns 256 columns (4 per lane, one 8-byte load per row) and one of G row groups; wave w of group g
 // walks entries u = 8g + w, + 8G, ...: a whole wave works on ONE row at a time, so the row's 16 h values are wave-uniform
@@ -1063,8 +1184,15 @@ int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, 
     hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, ws->row_any, ff, ws->words, union_rows, n_union);
     const int hstride = ws->max_ff + 16;
     if (cols % 256 == 0) {
-        hipLaunchKernelGGL(batch_upgate_lds_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
-                           (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride, (float *)nullptr);
+        const int n_cu = pi::compute_units();
+        if (n_cu > 0 && (size_t)ff * cols * 2 < ((size_t)1 << 32)) {
+            if (gate_f16) hipLaunchKernelGGL(batch_upgate_bal_f16_kernel<true>, dim3(n_cu), dim3(kUbBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
+                                             (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
+            else hipLaunchKernelGGL(batch_upgate_bal_f16_kernel<false>, dim3(n_cu), dim3(kUbBlock), 0, st, (const __half *)up_f16, (const __half *)nullptr, cols,
+                                    (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
+        } else
+            hipLaunchKernelGGL(batch_upgate_lds_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
+                               (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride, (float *)nullptr);
         hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3((cols + 511) / 512, kBmGroups), dim3(128), 0, st, (const __half *)down_t_f16, cols,
                            ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
         hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBmGroups, T, cols, epilogue, add1, add2, out);

@@ -767,14 +767,14 @@ def test_batch_init_rejects_unsupported_models():
 def test_prompt_chunks_match_token_by_token(arch, wtype):
     """A prompt handed over in one call is evaluated in chunks of up to 16 tokens (weights read once per chunk, causal attention
     inside the chunk); the result must agree with the CPU oracle evaluating the whole prompt as one batch (llama_decode with
-    n_tokens > 1) and with feeding the same tokens one at a time.  As in the single-token model tests one predictor logit on
-    the threshold can flip a neuron in either path (a few percent of one layer's output with these random predictors), so
-    the criterion is the median over several prompts.  A Q4_0 model's chunks run on the integer matrix-core kernels
-    (pi_k_gemm_q4_t16, pi_k_batch_sparse_ffn_q4): same criteria, on a model whose predictors keep a margin - without one the
-    int8 rounding steps of Q4_0 activations flip neurons in either path, and the single-token path, whose dots are the CPU's bit
-    for bit, is then as far from the oracle's batch evaluation (1.4e-2 median on this model) as the chunks are (1.5e-2)."""
+    n_tokens > 1) and with feeding the same tokens one at a time.  The models' predictors keep a margin (no logit on the
+    threshold, so no neuron flips on the order of a sum): an F16 model then agrees to 5e-3 for every prompt and every later
+    step.  A Q4_0 model's chunks run on the integer matrix-core kernels (pi_k_gemm_q4_t16, pi_k_batch_sparse_ffn_q4), where one
+    int8 rounding step of a Q8_0 activation still moves a logit by up to a per cent in either path (the single-token path,
+    whose dots are the CPU's bit for bit, is as far from the oracle's batch evaluation as the chunks are), so its criterion
+    is the median over several prompts."""
     from powerinfer_amd.model import Model
-    hp = synth.hparams(arch, seed=12, n_ctx=64, wtype=wtype, **(dict(pred_margin=True, head_pair=2048) if wtype != synth.F16 else {}))
+    hp = synth.hparams(arch, seed=12, n_ctx=64, wtype=wtype, pred_margin=True, head_pair=2048)
     model = synth.make_model(hp)
     rng = np.random.default_rng(4)
     err_oracle, err_single, err_after = [], [], []
@@ -796,9 +796,12 @@ def test_prompt_chunks_match_token_by_token(arch, wtype):
         om.close()
         ga.close()
         gb.close()
-    assert np.median(err_oracle) < 1e-2, err_oracle
-    assert np.median(err_after) < 1e-2, err_after
-    assert np.median(err_single) < 5e-2 and max(err_single) < 0.3, err_single
+    if wtype == synth.F16:
+        assert max(err_oracle) < 5e-3 and max(err_after) < 5e-3 and max(err_single) < 5e-3, (err_oracle, err_after, err_single)
+    else:
+        assert np.median(err_oracle) < 1e-2, err_oracle
+        assert np.median(err_after) < 1e-2, err_after
+        assert np.median(err_single) < 5e-2 and max(err_single) < 0.3, err_single
 
 
 @pytest.mark.timeout(300)

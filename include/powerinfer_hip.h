@@ -301,6 +301,27 @@ PI_API int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float thre
                                  int epilogue, const float * add1, const float * add2, float * out,
                                  int32_t * union_rows, int32_t * n_union,
                                  pi_workspace * ws, pi_stream_t stream);
+/*
+ * The same four with the step's fp16 activations in the operand layout of the matrix cores instead of [T][cols]: 16 token slots
+ * (whatever T is) laid out [cols / 8][16][8], element (t, c) at ((c / 8) * 16 + t) * 8 + c % 8, so that the fragment a wave loads
+ * for a 32-column step is one contiguous kilobyte instead of 16 token rows x 64 bytes.  Same arithmetic, bit for bit; a buffer holds
+ * 16 * cols fp16 values.  No counterpart in the reference (its batch kernels read ggml's row-major src1, ggml-cuda.cu:6994-7034): the
+ * layout exists because the activation loads, not the weight loads, were what the vector L1 of a compute unit spent its cycles on.
+ *   pi_k_norm_round_f16_ol: both outputs in the operand layout (cols % 8 == 0).
+ *   pi_k_gemm_f16_ol: xn_ol read and y_ol (optional, rows % 8 == 0) written in it; y, add1, add2 stay [T][rows] fp32.
+ *   pi_k_batch_predictor_fc2_ol: hidden_ol in it (the y_ol of the fc1 mat-mul).
+ *   pi_k_batch_sparse_ffn_ol: xn_ol in it (cols % 256 == 0 and ff * cols < 2^31 required).
+ */
+PI_API int pi_k_norm_round_f16_ol(const float * x, int T, int cols, const pi_norm * norm, void * out_ol, void * out_plain_ol, pi_stream_t stream);
+PI_API int pi_k_gemm_f16_ol(const void * W_f16, int rows, int cols, const void * xn_ol, int T, int epilogue,
+                            const float * add1, const float * add2, float * y, void * y_ol, pi_stream_t stream);
+PI_API int pi_k_batch_predictor_fc2_ol(const void * fc2_f16, int ff, int r, const void * hidden_ol, int T, float threshold, float * logits,
+                                       pi_workspace * ws, pi_stream_t stream);
+PI_API int pi_k_batch_sparse_ffn_ol(const float * logits, int T, int ff, float threshold,
+                                    const void * up_f16, const void * gate_f16, const void * down_t_f16, int cols, const void * xn_ol,
+                                    int epilogue, const float * add1, const float * add2, float * out,
+                                    int32_t * union_rows, int32_t * n_union,
+                                    pi_workspace * ws, pi_stream_t stream);
 
 /* Prompt chunks on this library's own mat-mul kernel (the prompt phase of llama_decode, where the reference goes through cuBLAS and
  * its batch kernels, ggml-cuda.cu:7662-7756, 6994-7034): pi_k_gemm_tile_f16 is pi_k_gemm_f16 for chunks of any length, both operands

@@ -228,8 +228,10 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     if (!falcon) an = mk_norm(1, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), nullptr);
     else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
     else an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
-    PI_TRY(pi_k_norm_round_f16(x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));       // Falcon: the predictor reads the raw layer input
-    PI_TRY(pi_k_gemm_f16(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr, st));
+    // the fp16 inputs of the step's mat-muls (xa16, xf16, xp16, hid16) are kept in the matrix cores' operand layout; the attention
+    // kernels write theirs (att16) token-major
+    PI_TRY(pi_k_norm_round_f16_ol(x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));    // Falcon: the predictor reads the raw layer input
+    PI_TRY(pi_k_gemm_f16_ol(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr, st));
     if (b->unified)
         PI_TRY(cells_attention(m, b, il, T));
     else if (b->prefill)
@@ -242,16 +244,16 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     if (!falcon) {
         PI_TRY(pi_k_gemm_f16(wo.dev, d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, nullptr, st));       // ffn_inp = wo.att + x
         fn = mk_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
-        PI_TRY(pi_k_norm_round_f16(b->ffn_inp, T, d, &fn, b->xf16, b->xp16, st));                                // FFN input and predictor input in one pass
+        PI_TRY(pi_k_norm_round_f16_ol(b->ffn_inp, T, d, &fn, b->xf16, b->xp16, st));                             // FFN input and predictor input in one pass
     } else {
         PI_TRY(pi_k_gemm_f16(wo.dev, d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, nullptr, st));
         fn = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
-        if (m->L(il, PI_T_ATTN_NORM_2).dev) PI_TRY(pi_k_norm_round_f16(x, T, d, &fn, b->xf16, nullptr, st));     // two norms: the FFN has its own
+        if (m->L(il, PI_T_ATTN_NORM_2).dev) PI_TRY(pi_k_norm_round_f16_ol(x, T, d, &fn, b->xf16, nullptr, st));  // two norms: the FFN has its own
     }
     const __half * ffn_x = (falcon && !m->L(il, PI_T_ATTN_NORM_2).dev) ? b->xa16 : b->xf16;                        // single-norm Falcon: attention and FFN share it
     // predictor
-    PI_TRY(pi_k_gemm_f16(fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16, st));
-    PI_TRY(pi_k_batch_predictor_fc2(fc2.dev, ff, r, b->hid16, T, hp.sparse_threshold, b->pred_logits, m->ws, st));
+    PI_TRY(pi_k_gemm_f16_ol(fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16, st));
+    PI_TRY(pi_k_batch_predictor_fc2_ol(fc2.dev, ff, r, b->hid16, T, hp.sparse_threshold, b->pred_logits, m->ws, st));
     // Dense cross-over (the reference's switch from its batch-sparse kernels to a plain mat-mul, ggml-cuda.cu:8787-8814, 7717-7756):
     // when the sequences' active sets together cover nearly all of the layer, gathering rows costs more than streaming all of them.
     // Measured on the 13B shape, 40 layers, 16 sequences (ms per step, union kernels / dense): union 0.41 of n_ff 7.46 / 9.18,
@@ -259,8 +261,8 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     // is made from the union the previous step measured (the count below keeps that statistic alive while the layer runs dense).
     if (!b->prefill && !b->unified && il < (int)b->dense_ffn.size() && b->dense_ffn[il]) {
         PI_TRY(pi_k_batch_union_count(ff, b->union_rows, b->n_union + il, m->ws, st));
-        PI_TRY(pi_k_gemm_f16(up.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->up_out, nullptr, st));
-        if (!falcon) PI_TRY(pi_k_gemm_f16(gate.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->gate_out, nullptr, st));
+        PI_TRY(pi_k_gemm_f16_ol(up.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->up_out, nullptr, st));
+        if (!falcon) PI_TRY(pi_k_gemm_f16_ol(gate.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->gate_out, nullptr, st));
         PI_TRY(pi_k_ffn_h_f16(b->up_out, falcon ? nullptr : b->gate_out, b->pred_logits, hp.sparse_threshold, T, ff, b->h16, st));
         if (!falcon) PI_TRY(pi_k_gemm_f16(m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD, b->ffn_inp, nullptr, b->x2, nullptr, st));
         else         PI_TRY(pi_k_gemm_f16(m->down_rows[il], d, ff, b->h16, T, PI_EPI_ADD2, b->attn_out, x, b->x2, nullptr, st));
@@ -269,10 +271,10 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     }
     // sparse FFN over the union of the sequences' active sets
     if (!falcon)
-        PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, gate.dev, down.dev, d, ffn_x, PI_EPI_ADD, b->ffn_inp, nullptr,
+        PI_TRY(pi_k_batch_sparse_ffn_ol(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, gate.dev, down.dev, d, ffn_x, PI_EPI_ADD, b->ffn_inp, nullptr,
                                      b->x2, b->union_rows, b->n_union + il, m->ws, st));
     else
-        PI_TRY(pi_k_batch_sparse_ffn(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, nullptr, down.dev, d, ffn_x, PI_EPI_ADD2, b->attn_out, x,
+        PI_TRY(pi_k_batch_sparse_ffn_ol(b->pred_logits, T, ff, hp.sparse_threshold, up.dev, nullptr, down.dev, d, ffn_x, PI_EPI_ADD2, b->attn_out, x,
                                      b->x2, b->union_rows, b->n_union + il, m->ws, st));
     std::swap(b->x, b->x2);
     return PI_OK;
@@ -292,8 +294,8 @@ int batch_step(pi_model * m, BatchState * b) {
         PI_TRY(pi_k_norm_q8_blocks(b->x, T, d, &on, b->qa, b->da, b->sa, nullptr, st));
         PI_TRY(pi_k_gemm_q4_t16(wout.quants, wout.scales, hp.n_vocab, d, b->qa, b->da, b->sa, T, PI_EPI_NONE, nullptr, nullptr, b->logits, st));
     } else {
-        PI_TRY(pi_k_norm_round_f16(b->x, T, d, &on, b->xa16, nullptr, st));
-        PI_TRY(pi_k_gemm_f16(m->glob[PI_T_OUTPUT].dev, hp.n_vocab, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->logits, nullptr, st));
+        PI_TRY(pi_k_norm_round_f16_ol(b->x, T, d, &on, b->xa16, nullptr, st));
+        PI_TRY(pi_k_gemm_f16_ol(m->glob[PI_T_OUTPUT].dev, hp.n_vocab, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->logits, nullptr, st));
     }
     PI_TRY(pi_k_argmax_batch(b->logits, hp.n_vocab, T, b->d_tokens, b->d_pos, b->d_step, b->d_out_tokens, b->max_steps, st));
     PI_TRY(pi_k_step_advance(b->d_step, st));
@@ -335,8 +337,9 @@ BatchState * batch_alloc(pi_model * m, int T, bool with_caches) {
     b->x = m->alloc<float>(n * d); b->x2 = m->alloc<float>(n * d); b->qkv = m->alloc<float>(n * (d + 2 * m->gqa));
     b->att = m->alloc<float>(n * d); b->attn_out = m->alloc<float>(n * d); b->ffn_inp = m->alloc<float>(n * d);
     b->hidden = m->alloc<float>(n * r); b->pred_logits = m->alloc<float>(n * ff); b->logits = m->alloc<float>(n * hp.n_vocab);
-    b->xa16 = m->alloc<__half>(n * d); b->xf16 = m->alloc<__half>(n * d); b->xp16 = m->alloc<__half>(n * d);
-    b->att16 = m->alloc<__half>(n * d); b->hid16 = m->alloc<__half>(n * r);
+    const size_t n16 = n < 16 ? 16 : n;                            // steps of up to 16 tokens keep these in the operand layout: 16 token slots
+    b->xa16 = m->alloc<__half>(n16 * d); b->xf16 = m->alloc<__half>(n16 * d); b->xp16 = m->alloc<__half>(n16 * d);
+    b->att16 = m->alloc<__half>(n * d); b->hid16 = m->alloc<__half>(n16 * r);
     b->d_tokens = m->alloc<int32_t>(n); b->d_pos = m->alloc<int32_t>(n); b->d_step = m->alloc<int32_t>(1);
     b->d_out_tokens = m->alloc<int32_t>((size_t)b->max_steps * n); b->union_rows = m->alloc<int32_t>(ff); b->n_union = m->alloc<int32_t>(hp.n_layer);
     if (m->L(0, PI_T_WQKV).type == PI_TYPE_Q4_0 && d % 32 == 0) {          // steps of a Q4_0 model on integer matrix cores

@@ -26,13 +26,21 @@ __device__ __forceinline__ float q8_block_value(float v) {
     return __fmul_rn((float)(int)rintf(__fmul_rn(v, id)), d);
 }
 
+// Operand layout of a step's fp16 activations ([16 token slots][cols], T <= 16): [cols / 8][16][8], i.e. the eight consecutive columns
+// a lane of v_mfma_f32_16x16x32_f16 holds, token after token.  The B fragments of a 32-column step are then one contiguous kilobyte
+// (lane (token i, group g) reads 16 bytes at ((4 step + g) * 16 + i) * 8 halves) instead of 16 token rows x 64 bytes, which halves the
+// cache lines an activation load touches: with [token][cols] the activation loads cost the vector L1 as many line accesses as the
+// weight loads of two row tiles, and the L1 is what these kernels wait for.
+__device__ __forceinline__ size_t pi_ol_index(int t, int col) { return ((size_t)(col >> 3) * 16 + t) * 8 + (col & 7); }
+
 // q8 != 0 (cols % 32 == 0, cols <= 8192): the normalised row goes through Q8_0 blocks of 32 before the fp16 rounding, which is what
 // a Q4_0 mat-mul of the CPU path multiplies with (ggml_vec_dot_q4_0_q8_0, ggml-quants.c:2512-2650)
+// ol != 0: both outputs in the operand layout of the 16-token mat-muls (pi_ol_index) instead of [token][cols].
 __global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __restrict__ x, int cols, NormArgs na, __half * __restrict__ out,
-                                                              __half * __restrict__ out_plain, int q8) {
+                                                              __half * __restrict__ out_plain, int q8, int ol) {
     __shared__ double red[16];
     const float * xt = x + (size_t)blockIdx.x * cols;
-    __half * ot = out + (size_t)blockIdx.x * cols;
+    auto at = [&](int i) -> size_t { return ol ? pi_ol_index(blockIdx.x, i) : (size_t)blockIdx.x * cols + i; };
     float mean = 0.0f, scale = 1.0f;
     if (cols <= 8 * 1024) {
         // one memory round trip: the row, the norm weights and the bias are requested together and stay in registers
@@ -66,14 +74,14 @@ __global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __re
         for (int k = 0; k < 8; ++k) {
             const int i = threadIdx.x + k * 1024;
             float v = xv[k];
-            if (i < cols && out_plain) out_plain[(size_t)blockIdx.x * cols + i] = __float2half_rn(v);
+            if (i < cols && out_plain) out_plain[at(i)] = __float2half_rn(v);
             if (na.kind != 0) {
                 v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
                 if (na.w) v = __fmul_rn(v, wv[k]);
                 if (na.b) v = __fadd_rn(v, bv[k]);
             }
             if (q8) v = q8_block_value(i < cols ? v : 0.0f);          // every lane takes part in the block's maximum
-            if (i < cols) ot[i] = __float2half_rn(v);
+            if (i < cols) out[at(i)] = __float2half_rn(v);
         }
         return;
     }
@@ -94,13 +102,13 @@ __global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __re
     }
     for (int i = threadIdx.x; i < cols; i += blockDim.x) {
         float v = xt[i];
-        if (out_plain) out_plain[(size_t)blockIdx.x * cols + i] = __float2half_rn(v);
+        if (out_plain) out_plain[at(i)] = __float2half_rn(v);
         if (na.kind != 0) {
             v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
             if (na.w) v = __fmul_rn(v, na.w[i]);
             if (na.b) v = __fadd_rn(v, na.b[i]);
         }
-        ot[i] = __float2half_rn(v);
+        out[at(i)] = __float2half_rn(v);
     }
 }
 
@@ -112,7 +120,8 @@ __global__ __launch_bounds__(1024) void norm_round_f16_kernel(const float * __re
 template <int RT>
 __global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
                                                               int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y,
-                                                              __half * __restrict__ y16, float thr, unsigned char * __restrict__ row_any) {
+                                                              __half * __restrict__ y16, float thr, unsigned char * __restrict__ row_any, int lay) {
+    // lay bit 0: xn in the operand layout (pi_ol_index); bit 1: y16 in the operand layout (the next mat-mul's input)
     __shared__ float cs[kWavesPerBlock][16][17];
     constexpr int SU = 16 / RT;                     // steps per batch of loads
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -126,7 +135,8 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __r
         const int row = row0 + rt * 16 + i < rows ? row0 + rt * 16 + i : rows - 1;
         ap[rt] = W + (size_t)row * cols + wave * kw + g * 8;
     }
-    const __half * bp = xn + (size_t)tok * cols + wave * kw + g * 8;
+    const __half * bp = (lay & 1) ? xn + ((size_t)(wave * kw / 32) * 64 + g * 16 + i) * 8 : xn + (size_t)tok * cols + wave * kw + g * 8;
+    const int bstep = (lay & 1) ? 512 : 32;        // halves from one 32-column step's fragment to the next
     pi_f4 acc[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
@@ -138,7 +148,7 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __r
             if (s0 + u < steps) {
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) a[u][rt] = pi_ld_stream(ap[rt] + (s0 + u) * 32);
-                b[u] = pi_ld16(bp + (s0 + u) * 32);
+                b[u] = pi_ld16(bp + (s0 + u) * bstep);
             }
 #pragma unroll
         for (int u = 0; u < SU; ++u)
@@ -166,7 +176,7 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __r
             else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
             else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[o]), add2[o]);
             y[o] = sum;
-            if (y16) y16[o] = __float2half_rn(sum);
+            if (y16) y16[(lay & 2) ? pi_ol_index(t, row) : o] = __float2half_rn(sum);
             act = !(sum < thr);
         }
         if (row_any) {      // predictor logits: is the row active for at least one token of the step?  (16 lanes = 16 tokens of a row)
@@ -185,7 +195,7 @@ constexpr int kGlStride = 512 + 16;               // bytes per LDS row: 256 fp16
 template <int RT>
 __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
                                                                   int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y,
-                                                                  __half * __restrict__ y16, float thr, unsigned char * __restrict__ row_any) {
+                                                                  __half * __restrict__ y16, float thr, unsigned char * __restrict__ row_any, int lay) {
     __shared__ __align__(16) unsigned char tile[kWavesPerBlock][16 * kGlStride];
     __shared__ float cs[kWavesPerBlock][16][17];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -194,7 +204,8 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
     const int row0 = blockIdx.x * 16 * RT;
     const int tok = i < T ? i : T - 1;
     // the 256-column super-steps of a row are dealt round-robin to the four waves: wave w takes steps w, w + 4, ...
-    const __half * bp = xn + (size_t)tok * cols + g * 8;
+    const __half * bp = (lay & 1) ? xn + (g * 16 + i) * 8 : xn + (size_t)tok * cols + g * 8;
+    const int bstep = (lay & 1) ? 512 : 32;        // halves from one 32-column step's fragment to the next
     unsigned char * mytile = tile[wave];
     pi_f4 acc[RT];
 #pragma unroll
@@ -222,7 +233,7 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
             if (cur < n_ss) {
                 pi_u32x4 b[8];
 #pragma unroll
-                for (int st = 0; st < 8; ++st) b[st] = pi_ld16(bp + (wave + cur * kWavesPerBlock) * 256 + st * 32);
+                for (int st = 0; st < 8; ++st) b[st] = pi_ld16(bp + ((wave + cur * kWavesPerBlock) * 8 + st) * bstep);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
@@ -255,7 +266,7 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
             else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
             else if (epi == PI_EPI_ADD2) sum = __fadd_rn(__fadd_rn(sum, add1[o]), add2[o]);
             y[o] = sum;
-            if (y16) y16[o] = __float2half_rn(sum);
+            if (y16) y16[(lay & 2) ? pi_ol_index(t, row) : o] = __float2half_rn(sum);
             act = !(sum < thr);
         }
         if (row_any) {
@@ -674,7 +685,8 @@ template <bool GATE>
 __global__ __launch_bounds__(kUbBlock, 1) void batch_upgate_bal_f16_kernel(const __half * __restrict__ Wup, const __half * __restrict__ Wgate, int cols,
                                                                            const __half * __restrict__ xn, int T, const float * __restrict__ logits, int ff, float thr,
                                                                            const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
-                                                                           __half * __restrict__ hc, int hstride) {
+                                                                           __half * __restrict__ hc, int hstride, int xol) {
+    // xol != 0: xn in the operand layout (pi_ol_index)
     __shared__ __align__(16) unsigned char tile[kUbWaves][16 * kUbStride];
     __shared__ float cu[kUbWaves][kUbRows][17], cg[GATE ? kUbWaves : 1][kUbRows][17];
     const int n = *n_union;
@@ -687,7 +699,8 @@ __global__ __launch_bounds__(kUbBlock, 1) void batch_upgate_bal_f16_kernel(const
     const int i = lane & 15, g = lane >> 4;                        // MFMA role: row (token) i, k group g
     const int lr = lane >> 4, lc = lane & 15;                      // load role: row within the instruction's four, 16-byte piece of the 256-byte row piece
     const int tok = i < T ? i : T - 1;
-    const char * bp = reinterpret_cast<const char *>(xn + (size_t)tok * cols + g * 8);
+    const char * bp = reinterpret_cast<const char *>(xol ? xn + (g * 16 + i) * 8 : xn + (size_t)tok * cols + g * 8);
+    const int bs_step = xol ? 4096 : kUbStep * 2, bs_frag = xol ? 1024 : 64;      // bytes from a 128-column step to the next, and between its four 32-column fragments
     unsigned char * mytile = tile[wave];
     const int n_steps = cols / kUbStep;
     const int n_ss = (n_steps - wave + kUbWaves - 1) / kUbWaves;   // super-steps wave, wave + 8, ... of this wave
@@ -707,13 +720,17 @@ __global__ __launch_bounds__(kUbBlock, 1) void batch_upgate_bal_f16_kernel(const
         // The weights of two super-steps are in flight; the activations of a super-step are requested when the previous one has been
         // multiplied, BEFORE the weights that replace it (requested after them, the wait for the activations would drain them).
         pi_u32x4 lu[2][8], lg[2][8], bb[4];
+        // workgroup b starts its walk over the columns b super-steps further on (and wraps): the units run in step, and all of them
+        // asking for the same kilobytes of the activations at the same time queue up on one L2 channel
+        const int rot0 = n_ss > 0 ? (int)(blockIdx.x % (unsigned)n_ss) : 0;
+        auto rot = [&](int s) { const int v = s + rot0; return v >= n_ss ? v - n_ss : v; };
         auto issue_b = [&](int s) {
-            const size_t so = (size_t)(wave + (s < n_ss ? s : n_ss - 1) * kUbWaves) * (kUbStep * 2);
+            const size_t so = (size_t)(wave + rot(s < n_ss ? s : n_ss - 1) * kUbWaves) * bs_step;
 #pragma unroll
-            for (int st = 0; st < 4; ++st) bb[st] = pi_ld16(bp + so + st * 64);
+            for (int st = 0; st < 4; ++st) bb[st] = pi_ld16(bp + so + st * bs_frag);
         };
         auto issue = [&](int buf, int s) {                         // a super-step behind the wave's last reads the last one again
-            const size_t so = (size_t)(wave + (s < n_ss ? s : n_ss - 1) * kUbWaves) * (kUbStep * 2);
+            const size_t so = (size_t)(wave + rot(s < n_ss ? s : n_ss - 1) * kUbWaves) * (kUbStep * 2);
             const char * wu = reinterpret_cast<const char *>(Wup) + so, * wg = reinterpret_cast<const char *>(Wgate) + so;
 #pragma unroll
             for (int j = 0; j < 8; ++j) {
@@ -999,18 +1016,25 @@ extern "C" {
 
 int pi_k_norm_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, void * out_plain_f16, pi_stream_t stream) {
     if (!x || !out_f16 || T <= 0 || cols <= 0) return pi::fail(PI_E_ARG, "pi_k_norm_round_f16: bad arguments");
-    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16, (__half *)out_plain_f16, 0);
+    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16, (__half *)out_plain_f16, 0, 0);
     return pi::check_launch("pi_k_norm_round_f16");
+}
+
+int pi_k_norm_round_f16_ol(const float * x, int T, int cols, const pi_norm * norm, void * out_ol, void * out_plain_ol, pi_stream_t stream) {
+    if (!x || !out_ol || T <= 0 || T > kBtMaxT || cols <= 0 || cols % 8) return pi::fail(PI_E_ARG, "pi_k_norm_round_f16_ol: 1 <= T <= 16 and cols % 8 == 0 required");
+    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_ol, (__half *)out_plain_ol, 0, 1);
+    return pi::check_launch("pi_k_norm_round_f16_ol");
 }
 
 int pi_k_norm_q8_round_f16(const float * x, int T, int cols, const pi_norm * norm, void * out_f16, void * out_plain_f16, pi_stream_t stream) {
     if (!x || !out_f16 || T <= 0 || cols <= 0 || cols % 32 || cols > 8 * 1024) return pi::fail(PI_E_ARG, "pi_k_norm_q8_round_f16: cols must be a multiple of 32, at most 8192");
-    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16, (__half *)out_plain_f16, 1);
+    hipLaunchKernelGGL(norm_round_f16_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (__half *)out_f16, (__half *)out_plain_f16, 1, 0);
     return pi::check_launch("pi_k_norm_q8_round_f16");
 }
 
+// lay bit 0: xn_f16 in the operand layout of the step's activations (pi_ol_index), bit 1: y_f16 written in it
 static int gemm_launch(const char * who, const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
-                       float * y, void * y_f16, float thr, unsigned char * row_any, pi_stream_t stream) {
+                       float * y, void * y_f16, float thr, unsigned char * row_any, pi_stream_t stream, int lay = 0) {
     if (!W || !xn_f16 || !y || rows <= 0) return pi::fail(PI_E_ARG, who);
     if (T < 1 || T > kBtMaxT || cols <= 0 || cols % 128) return pi::fail(PI_E_ARG, "batched mat-mul: 1 <= T <= 16 and cols % 128 == 0 required");
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
@@ -1018,9 +1042,9 @@ static int gemm_launch(const char * who, const void * W, int rows, int cols, con
     // row tiles per wave: enough workgroups to fill the chip first, then as few reads of the activations as possible
     const int rt = rows >= 16384 ? 4 : rows >= 5120 ? 2 : 1;      // (two tiles already at 5120 rows: the activations, re-read per row tile, are what limits one tile per wave)
 #define PI_GEMM_T16(RT) hipLaunchKernelGGL((gemm_t16_f16_kernel<RT>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(kBlock), 0, (hipStream_t)stream, \
-                       (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any)
+                       (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any, lay)
 #define PI_GEMM_LDS(RT) hipLaunchKernelGGL((gemm_t16_lds_f16_kernel<RT>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(kBlock), 0, (hipStream_t)stream, \
-                       (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any)
+                       (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any, lay)
     if (cols % 256 == 0) { if (rt >= 2) PI_GEMM_LDS(2); else PI_GEMM_LDS(1); }
     else if (rt == 4) PI_GEMM_T16(4); else if (rt == 2) PI_GEMM_T16(2); else PI_GEMM_T16(1);
 #undef PI_GEMM_LDS
@@ -1031,6 +1055,12 @@ static int gemm_launch(const char * who, const void * W, int rows, int cols, con
 int pi_k_gemm_f16(const void * W, int rows, int cols, const void * xn_f16, int T, int epilogue, const float * add1, const float * add2,
                   float * y, void * y_f16, pi_stream_t stream) {
     return gemm_launch("pi_k_gemm_f16", W, rows, cols, xn_f16, T, epilogue, add1, add2, y, y_f16, 0.0f, nullptr, stream);
+}
+
+int pi_k_gemm_f16_ol(const void * W, int rows, int cols, const void * xn_ol, int T, int epilogue, const float * add1, const float * add2,
+                     float * y, void * y_ol, pi_stream_t stream) {
+    if (y_ol && rows % 8) return pi::fail(PI_E_ARG, "pi_k_gemm_f16_ol: rows % 8 == 0 required for the fp16 copy in the operand layout");
+    return gemm_launch("pi_k_gemm_f16_ol", W, rows, cols, xn_ol, T, epilogue, add1, add2, y, y_ol, 0.0f, nullptr, stream, 3);
 }
 
 // Output tiles the kernel is built for (weight rows x tokens per workgroup); the first two run eight waves, one workgroup per unit.
@@ -1172,9 +1202,15 @@ int pi_k_batch_predictor_fc2(const void * fc2_f16, int ff, int r, const void * h
     return gemm_launch("pi_k_batch_predictor_fc2", fc2_f16, ff, r, hidden_f16, T, PI_EPI_NONE, nullptr, nullptr, logits, nullptr, threshold, ws->row_any, stream);
 }
 
-int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, const void * up_f16, const void * gate_f16, const void * down_t_f16,
-                          int cols, const void * xn_f16, int epilogue, const float * add1, const float * add2, float * out,
-                          int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream) {
+int pi_k_batch_predictor_fc2_ol(const void * fc2_f16, int ff, int r, const void * hidden_ol, int T, float threshold, float * logits,
+                                pi_workspace * ws, pi_stream_t stream) {
+    if (!ws || ff > ws->max_ff) return pi::fail(PI_E_ARG, "pi_k_batch_predictor_fc2_ol: ff exceeds the workspace");
+    return gemm_launch("pi_k_batch_predictor_fc2_ol", fc2_f16, ff, r, hidden_ol, T, PI_EPI_NONE, nullptr, nullptr, logits, nullptr, threshold, ws->row_any, stream, 1);
+}
+
+static int batch_sparse_ffn(const float * logits, int T, int ff, float threshold, const void * up_f16, const void * gate_f16, const void * down_t_f16,
+                            int cols, const void * xn_f16, int epilogue, const float * add1, const float * add2, float * out,
+                            int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream, int xol) {
     if (!logits || !up_f16 || !down_t_f16 || !xn_f16 || !out || !union_rows || !n_union || !ws) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: null pointer");
     if (T < 1 || T > kBtMaxT || ff <= 0 || ff > ws->max_ff || cols <= 0 || cols > ws->max_d || cols % kBaTile || cols % 128)
         return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: 1 <= T <= 16, ff <= workspace, cols % 256 == 0 and cols <= workspace required");
@@ -1187,16 +1223,18 @@ int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, 
         const int n_cu = pi::compute_units();
         if (n_cu > 0 && (size_t)ff * cols * 2 < ((size_t)1 << 32)) {
             if (gate_f16) hipLaunchKernelGGL(batch_upgate_bal_f16_kernel<true>, dim3(n_cu), dim3(kUbBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
-                                             (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
+                                             (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride, xol);
             else hipLaunchKernelGGL(batch_upgate_bal_f16_kernel<false>, dim3(n_cu), dim3(kUbBlock), 0, st, (const __half *)up_f16, (const __half *)nullptr, cols,
-                                    (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
-        } else
+                                    (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride, xol);
+        } else if (xol) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn_ol: the operand layout needs the one-workgroup-per-unit kernel (ff * cols * 2 < 4 GiB)");
+        else
             hipLaunchKernelGGL(batch_upgate_lds_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
                                (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride, (float *)nullptr);
         hipLaunchKernelGGL(batch_axpy_mfma_f16_kernel, dim3((cols + 511) / 512, kBmGroups), dim3(128), 0, st, (const __half *)down_t_f16, cols,
                            ws->hc_batch, hstride, union_rows, n_union, ws->ffn_partial);
         hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBmGroups, T, cols, epilogue, add1, add2, out);
     } else {
+        if (xol) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn_ol: cols % 256 == 0 required");
         hipLaunchKernelGGL(batch_upgate_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
                            (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride);
         hipLaunchKernelGGL(batch_axpy_f16_kernel, dim3(cols / kBaTile, kBaGroups), dim3(kBaBlock), 0, st, (const __half *)down_t_f16, cols,
@@ -1204,6 +1242,18 @@ int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, 
         hipLaunchKernelGGL(batch_reduce_kernel, dim3((T * cols / 4 + kBlock - 1) / kBlock), dim3(kBlock), 0, st, ws->ffn_partial, kBaGroups, T, cols, epilogue, add1, add2, out);
     }
     return pi::check_launch("pi_k_batch_sparse_ffn");
+}
+
+int pi_k_batch_sparse_ffn(const float * logits, int T, int ff, float threshold, const void * up_f16, const void * gate_f16, const void * down_t_f16,
+                          int cols, const void * xn_f16, int epilogue, const float * add1, const float * add2, float * out,
+                          int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream) {
+    return batch_sparse_ffn(logits, T, ff, threshold, up_f16, gate_f16, down_t_f16, cols, xn_f16, epilogue, add1, add2, out, union_rows, n_union, ws, stream, 0);
+}
+
+int pi_k_batch_sparse_ffn_ol(const float * logits, int T, int ff, float threshold, const void * up_f16, const void * gate_f16, const void * down_t_f16,
+                             int cols, const void * xn_ol, int epilogue, const float * add1, const float * add2, float * out,
+                             int32_t * union_rows, int32_t * n_union, pi_workspace * ws, pi_stream_t stream) {
+    return batch_sparse_ffn(logits, T, ff, threshold, up_f16, gate_f16, down_t_f16, cols, xn_ol, epilogue, add1, add2, out, union_rows, n_union, ws, stream, 1);
 }
 
 // the union of the step's active rows alone (list and count from the flags pi_k_batch_predictor_fc2 left in the workspace): the statistic

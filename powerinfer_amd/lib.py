@@ -83,6 +83,10 @@ _SIGS = {
     "pi_k_gemm_f16": (_i, [_vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_batch_predictor_fc2": (_i, [_vp, _i, _i, _vp, _i, _f, _vp, _vp, _vp]),
     "pi_k_batch_sparse_ffn": (_i, [_vp, _i, _i, _f, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_norm_round_f16_ol": (_i, [_vp, _i, _i, C.POINTER(Norm), _vp, _vp, _vp]),
+    "pi_k_gemm_f16_ol": (_i, [_vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_batch_predictor_fc2_ol": (_i, [_vp, _i, _i, _vp, _i, _f, _vp, _vp, _vp]),
+    "pi_k_batch_sparse_ffn_ol": (_i, [_vp, _i, _i, _f, _vp, _vp, _vp, _i, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_batch_union_count": (_i, [_i, _vp, _vp, _vp, _vp]),
     "pi_k_q4_split": (_i, [_vp, _i, _i, _vp, _vp, _vp]),
     "pi_k_norm_q8_blocks": (_i, [_vp, _i, _i, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp]),

@@ -318,6 +318,54 @@ def test_batch_sparse_ffn_matches_oracle(shape, has_gate, T):
     L.pi_workspace_destroy(ws)
 
 
+def from_operand_layout(buf, T, cols):
+    """[cols / 8][16 token slots][8] fp16 -> [T][cols] (the layout pi_k_norm_round_f16_ol and pi_k_gemm_f16_ol write)."""
+    return buf.download(np.float16, 16 * cols).reshape(cols // 8, 16, 8)[:, :T, :].transpose(1, 0, 2).reshape(T, cols)
+
+
+@pytest.mark.parametrize("shape,has_gate,T", [((5120, 13824, 1280), True, 16), ((4096, 11008, 1024), False, 5), ((1024, 1024, 128), True, 3)])
+def test_operand_layout_entry_points_match_the_token_major_ones_bit_for_bit(shape, has_gate, T):
+    """The *_ol entry points keep a step's fp16 activations in the operand layout of the matrix cores ([cols / 8][16][8]); only the
+    addresses of the activation loads and stores differ, so the FFN block of a step - norm + rounding, predictor fc1 (with its fp16
+    copy for fc2), fc2 and its flags, union list, gate / up, down projection - must give the same bits either way."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    d, ff, r = shape
+    Lr = synth.make_ffn_layer(seed=17 + T, d=d, ff=ff, r=r, wtype=ol.F16, has_gate=has_gate, mean_rate=0.11, T=T)
+    x = Lr["x"]
+    nw = (1.0 + 0.1 * np.random.default_rng(5).standard_normal(d)).astype(np.float32)
+    dx, dw = pl.DevBuf(host=np.ascontiguousarray(x, np.float32)), pl.DevBuf(host=nw)
+    na = pl.norm_arg(1, 1e-5, dw, None)
+    up, down, fc1, fc2 = (pl.DevBuf(host=Lr[k]) for k in ("up", "down_t", "fc1", "fc2"))
+    gate = pl.DevBuf(host=Lr["gate"]) if has_gate else None
+    resid = np.random.default_rng(3).standard_normal((T, d)).astype(np.float32)
+    dres = pl.DevBuf(host=resid)
+    ws = L.pi_workspace_create(ff, d)
+    assert ws
+    got = {}
+    for tag, sfx in (("plain", ""), ("ol", "_ol")):
+        fn = lambda name: getattr(L, name + sfx)
+        slots = 16 if sfx else T
+        xn, xp = pl.DevBuf.zeros(slots * d * 2), pl.DevBuf.zeros(slots * d * 2)
+        hidden, hid16 = pl.DevBuf(T * r * 4), pl.DevBuf.zeros(slots * r * 2)
+        logits, out = pl.DevBuf(T * ff * 4), pl.DevBuf(T * d * 4)
+        union, n_union = pl.DevBuf(ff * 4), pl.DevBuf.zeros(4)
+        pl.check(fn("pi_k_norm_round_f16")(dx.ptr, T, d, na, xn.ptr, xp.ptr, None), "norm")
+        pl.check(fn("pi_k_gemm_f16")(fc1.ptr, r, d, xp.ptr, T, pl.EPI_RELU, None, None, hidden.ptr, hid16.ptr, None), "fc1")
+        pl.check(fn("pi_k_batch_predictor_fc2")(fc2.ptr, ff, r, hid16.ptr, T, 0.0, logits.ptr, ws, None), "fc2")
+        pl.check(fn("pi_k_batch_sparse_ffn")(logits.ptr, T, ff, 0.0, up.ptr, gate.ptr if gate else None, down.ptr, d, xn.ptr,
+                                             pl.EPI_ADD, dres.ptr, None, out.ptr, union.ptr, n_union.ptr, ws, None), "ffn")
+        pl.sync()
+        n = int(n_union.download(np.int32)[0])
+        unpack = (lambda b, c: from_operand_layout(b, T, c)) if sfx else (lambda b, c: b.download(np.float16, T * c).reshape(T, c))
+        got[tag] = dict(xn=unpack(xn, d), xp=unpack(xp, d), hid16=unpack(hid16, r), hidden=hidden.download(np.float32), logits=logits.download(np.float32),
+                        out=out.download(np.float32), union=union.download(np.int32, n))
+    assert len(got["plain"]["union"]) > 0 and np.abs(got["plain"]["out"] - resid.ravel()).max() > 0
+    for k in got["plain"]:
+        assert np.array_equal(got["plain"][k].view(np.uint8), got["ol"][k].view(np.uint8)), k
+    L.pi_workspace_destroy(ws)
+
+
 def q4_split_on_device(pl, L, wq4, rows, cols):
     dw = pl.DevBuf(host=wq4)
     qs, ds = pl.DevBuf(rows * cols // 2), pl.DevBuf(rows * cols // 32 * 2)

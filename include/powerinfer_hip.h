@@ -487,6 +487,10 @@ PI_API int pi_k_attn_ggml_step(const float * qkv, int qkv_stride, const int32_t 
 PI_API int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache,
                                  size_t cache_seq_stride, int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx,
                                  const int32_t * pos, float * out, int out_stride, void * out_f16, pi_stream_t stream);
+/* the same with the fp16 copy in the operand layout of pi_k_gemm_f16_ol (16 sequence slots of n_head * hd columns; out stays [n_seq][out_stride]) */
+PI_API int pi_k_attn_fused_batch_ol(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache,
+                                    size_t cache_seq_stride, int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx,
+                                    const int32_t * pos, float * out, int out_stride, void * out_ol, pi_stream_t stream);
 /* prompt chunk of ONE sequence: T <= 512 consecutive tokens at positions pos[t]; RoPE + KV store of the whole chunk first, then
  * every token attends to the cells up to its own position (the causal mask of llama.cpp:6506-6531).  q_rot: fp32 [T][n_head*hd].
  * n_kv_max: an upper bound of max(pos) + 1, the cells the chunk's furthest token attends (<= 0: n_ctx); positions beyond it are

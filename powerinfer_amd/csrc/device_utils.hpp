@@ -121,3 +121,10 @@ __device__ __forceinline__ pi_u32x4 pi_ld_stream(const void * p) {
     return __builtin_nontemporal_load(reinterpret_cast<const pi_u32x4 *>(p));
 }
 __device__ __forceinline__ pi_u32x4 pi_ld16(const void * p) { return *reinterpret_cast<const pi_u32x4 *>(p); }
+
+// Operand layout of a step's fp16 activations ([16 token slots][cols], T <= 16): [cols / 8][16][8], i.e. the eight consecutive columns
+// a lane of v_mfma_f32_16x16x32_f16 holds, token after token.  The B fragments of a 32-column step are then one contiguous kilobyte
+// (lane (token i, group g) reads 16 bytes at ((4 step + g) * 16 + i) * 8 halves) instead of 16 token rows x 64 bytes, which halves the
+// cache lines an activation load touches: with [token][cols] the activation loads cost the vector L1 as many line accesses as the
+// weight loads of two row tiles, and the L1 is what these kernels wait for.
+__device__ __forceinline__ size_t pi_ol_index(int t, int col) { return ((size_t)(col >> 3) * 16 + t) * 8 + (col & 7); }

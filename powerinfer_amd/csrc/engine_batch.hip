@@ -228,8 +228,8 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     if (!falcon) an = mk_norm(1, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), nullptr);
     else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
     else an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
-    // the fp16 inputs of the step's mat-muls (xa16, xf16, xp16, hid16) are kept in the matrix cores' operand layout; the attention
-    // kernels write theirs (att16) token-major
+    // the fp16 inputs of the step's mat-muls (xa16, xf16, xp16, hid16, and att16 of a lockstep step) are kept in the matrix cores'
+    // operand layout; the attention of a prompt chunk and of the shared-cell cache write att16 token-major
     PI_TRY(pi_k_norm_round_f16_ol(x, T, d, &an, b->xa16, falcon ? b->xp16 : nullptr, st));    // Falcon: the predictor reads the raw layer input
     PI_TRY(pi_k_gemm_f16_ol(wqkv.dev, d + 2 * gqa, d, b->xa16, T, PI_EPI_NONE, nullptr, nullptr, b->qkv, nullptr, st));
     if (b->unified)
@@ -237,16 +237,18 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     else if (b->prefill)
         PI_TRY(chunk_attention(m, b, T, kv_off));
     else
-        PI_TRY(pi_k_attn_fused_batch(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
-                                     hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, hp.n_ctx, b->d_pos, b->att, d, b->att16, st));
+        PI_TRY(pi_k_attn_fused_batch_ol(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
+                                        hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, hp.n_ctx, b->d_pos, b->att, d, b->att16, st));
+    const bool att_ol = !b->unified && !b->prefill;               // the lockstep attention writes its fp16 copy in the operand layout
+    auto wo_gemm = att_ol ? pi_k_gemm_f16_ol : pi_k_gemm_f16;
 
     pi_norm fn;
     if (!falcon) {
-        PI_TRY(pi_k_gemm_f16(wo.dev, d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, nullptr, st));       // ffn_inp = wo.att + x
+        PI_TRY(wo_gemm(wo.dev, d, d, b->att16, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, nullptr, st));             // ffn_inp = wo.att + x
         fn = mk_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
         PI_TRY(pi_k_norm_round_f16_ol(b->ffn_inp, T, d, &fn, b->xf16, b->xp16, st));                             // FFN input and predictor input in one pass
     } else {
-        PI_TRY(pi_k_gemm_f16(wo.dev, d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, nullptr, st));
+        PI_TRY(wo_gemm(wo.dev, d, d, b->att16, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, nullptr, st));
         fn = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
         if (m->L(il, PI_T_ATTN_NORM_2).dev) PI_TRY(pi_k_norm_round_f16_ol(x, T, d, &fn, b->xf16, nullptr, st));  // two norms: the FFN has its own
     }
@@ -339,7 +341,7 @@ BatchState * batch_alloc(pi_model * m, int T, bool with_caches) {
     b->hidden = m->alloc<float>(n * r); b->pred_logits = m->alloc<float>(n * ff); b->logits = m->alloc<float>(n * hp.n_vocab);
     const size_t n16 = n < 16 ? 16 : n;                            // steps of up to 16 tokens keep these in the operand layout: 16 token slots
     b->xa16 = m->alloc<__half>(n16 * d); b->xf16 = m->alloc<__half>(n16 * d); b->xp16 = m->alloc<__half>(n16 * d);
-    b->att16 = m->alloc<__half>(n * d); b->hid16 = m->alloc<__half>(n16 * r);
+    b->att16 = m->alloc<__half>(n16 * d); b->hid16 = m->alloc<__half>(n16 * r);
     b->d_tokens = m->alloc<int32_t>(n); b->d_pos = m->alloc<int32_t>(n); b->d_step = m->alloc<int32_t>(1);
     b->d_out_tokens = m->alloc<int32_t>((size_t)b->max_steps * n); b->union_rows = m->alloc<int32_t>(ff); b->n_union = m->alloc<int32_t>(hp.n_layer);
     if (m->L(0, PI_T_WQKV).type == PI_TYPE_Q4_0 && d % 32 == 0) {          // steps of a Q4_0 model on integer matrix cores

@@ -186,13 +186,14 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
                                                             __half * __restrict__ k_cache, __half * __restrict__ v_cache,
                                                             int n_head, int n_head_kv, int hd, int mode, int n_ctx,
                                                             const int32_t * __restrict__ pos_p, float * __restrict__ out,
-                                                            int qkv_stride, size_t cache_seq_stride, int out_stride, __half * __restrict__ out16) {
+                                                            int qkv_stride, size_t cache_seq_stride, int out_stride, __half * __restrict__ out16, int out16_ol) {
     // blockIdx.y = sequence of a batched step (its own token, position and cache); 0 for single-sequence decoding
+    // out16_ol != 0: the fp16 copy in the operand layout of the 16-token mat-muls (pi_ol_index) instead of [sequence][out_stride]
     qkv += (size_t)blockIdx.y * qkv_stride;
     k_cache += (size_t)blockIdx.y * cache_seq_stride;
     v_cache += (size_t)blockIdx.y * cache_seq_stride;
     out += (size_t)blockIdx.y * out_stride;
-    if (out16) out16 += (size_t)blockIdx.y * out_stride;      // optional fp16 copy: the input of the next mat-mul of a batched step
+    if (out16 && !out16_ol) out16 += (size_t)blockIdx.y * out_stride;      // optional fp16 copy: the input of the next mat-mul of a batched step
     pos_p += blockIdx.y;
     extern __shared__ __align__(16) unsigned char smem[];
     float * s    = reinterpret_cast<float *>(smem);               // [n_ctx] scores, then probabilities
@@ -321,7 +322,7 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
         float v = part[e];
         for (int g = 1; g < ngrp; ++g) v += part[g * hd + e];
         out[(size_t)h * hd + e] = v;
-        if (out16) out16[(size_t)h * hd + e] = __float2half_rn(v);
+        if (out16) out16[out16_ol ? pi_ol_index(blockIdx.y, h * hd + e) : (size_t)h * hd + e] = __float2half_rn(v);
     }
 }
 
@@ -927,7 +928,7 @@ int pi_k_attn_fused(const float * qkv, const void * rope_table, void * k_cache, 
     const size_t sh = attn_fused_lds_bytes(hd, n_ctx);
     if (sh > kAttnLdsLimit) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused: context too long for the single-pass kernel");
     hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
-                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, 0, (size_t)0, 0, nullptr);
+                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, 0, (size_t)0, 0, nullptr, 0);
     return pi::check_launch("pi_k_attn_fused");
 }
 
@@ -974,17 +975,29 @@ int pi_k_attn_split_cached(const float * q_rot, const void * k_cache, const void
     return pi::check_launch("pi_k_attn_split_cached");
 }
 
-int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache, size_t cache_seq_stride,
-                          int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, const int32_t * pos, float * out, int out_stride,
-                          void * out_f16, pi_stream_t stream) {
+static int attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache, size_t cache_seq_stride,
+                            int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, const int32_t * pos, float * out, int out_stride,
+                            void * out_f16, pi_stream_t stream, int out16_ol) {
     if (!qkv || !rope_table || !k_cache || !v_cache || !pos || !out || n_seq <= 0 || n_seq > kBtMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch: bad arguments");
     if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || !attn_fused_geometry_ok(hd) || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch: head size must be 8 * (a divisor of 64), at most 128; mode 0 or 2");
     const size_t sh = attn_fused_lds_bytes(hd, n_ctx);
     if (sh > kAttnLdsLimit) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused_batch: context too long for the single-pass kernel");
     hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head, n_seq), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
-                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride, (__half *)out_f16);
+                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride, (__half *)out_f16, out16_ol);
     return pi::check_launch("pi_k_attn_fused_batch");
+}
+
+int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache, size_t cache_seq_stride,
+                          int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, const int32_t * pos, float * out, int out_stride,
+                          void * out_f16, pi_stream_t stream) {
+    return attn_fused_batch(qkv, qkv_stride, rope_table, k_cache, v_cache, cache_seq_stride, n_seq, n_head, n_head_kv, hd, mode, n_ctx, pos, out, out_stride, out_f16, stream, 0);
+}
+
+int pi_k_attn_fused_batch_ol(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache, size_t cache_seq_stride,
+                             int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, const int32_t * pos, float * out, int out_stride,
+                             void * out_ol, pi_stream_t stream) {
+    return attn_fused_batch(qkv, qkv_stride, rope_table, k_cache, v_cache, cache_seq_stride, n_seq, n_head, n_head_kv, hd, mode, n_ctx, pos, out, out_stride, out_ol, stream, 1);
 }
 
 int pi_k_attn_chunk(const float * qkv, int qkv_stride, int T, int n_head, int n_head_kv, int hd, int mode, float theta_scale, float freq_scale,

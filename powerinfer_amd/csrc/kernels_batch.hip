@@ -26,13 +26,6 @@ __device__ __forceinline__ float q8_block_value(float v) {
     return __fmul_rn((float)(int)rintf(__fmul_rn(v, id)), d);
 }
 
-// Operand layout of a step's fp16 activations ([16 token slots][cols], T <= 16): [cols / 8][16][8], i.e. the eight consecutive columns
-// a lane of v_mfma_f32_16x16x32_f16 holds, token after token.  The B fragments of a 32-column step are then one contiguous kilobyte
-// (lane (token i, group g) reads 16 bytes at ((4 step + g) * 16 + i) * 8 halves) instead of 16 token rows x 64 bytes, which halves the
-// cache lines an activation load touches: with [token][cols] the activation loads cost the vector L1 as many line accesses as the
-// weight loads of two row tiles, and the L1 is what these kernels wait for.
-__device__ __forceinline__ size_t pi_ol_index(int t, int col) { return ((size_t)(col >> 3) * 16 + t) * 8 + (col & 7); }
-
 // q8 != 0 (cols % 32 == 0, cols <= 8192): the normalised row goes through Q8_0 blocks of 32 before the fp16 rounding, which is what
 // a Q4_0 mat-mul of the CPU path multiplies with (ggml_vec_dot_q4_0_q8_0, ggml-quants.c:2512-2650)
 // ol != 0: both outputs in the operand layout of the 16-token mat-muls (pi_ol_index) instead of [token][cols].

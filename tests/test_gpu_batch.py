@@ -366,6 +366,35 @@ def test_operand_layout_entry_points_match_the_token_major_ones_bit_for_bit(shap
     L.pi_workspace_destroy(ws)
 
 
+@pytest.mark.parametrize("nh,nkv,hd,n_seq", [(8, 8, 128, 5), (16, 2, 64, 16)])
+def test_lockstep_attention_writes_the_same_fp16_copy_in_either_layout(nh, nkv, hd, n_seq):
+    """pi_k_attn_fused_batch_ol differs from pi_k_attn_fused_batch only in where the fp16 copy of the output lands (the operand layout
+    of the output projection's mat-mul): same fp32 output, same fp16 values, same cache rows, over three steps of n_seq sequences."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    rng = np.random.default_rng(nh + n_seq)
+    n_ctx, gqa, d = 32, nkv * hd, nh * hd
+    stride = nkv * n_ctx * hd
+    tab = pl.DevBuf(n_ctx * hd * 4)
+    pl.check(L.pi_k_rope_table(tab.ptr, n_ctx, hd, 0, float(np.float32(10000.0) ** np.float32(-2.0 / hd)), 1.0, None), "rope_table")
+    caches = {k: (pl.DevBuf.zeros(n_seq * stride * 2), pl.DevBuf.zeros(n_seq * stride * 2)) for k in ("plain", "ol")}
+    dq, dpos = pl.DevBuf(n_seq * (d + 2 * gqa) * 4), pl.DevBuf(n_seq * 4)
+    for step in range(3):
+        dq.upload(rng.standard_normal(n_seq * (d + 2 * gqa)).astype(np.float32))
+        dpos.upload(np.full(n_seq, step, np.int32))
+        res = {}
+        for tag, fn in (("plain", L.pi_k_attn_fused_batch), ("ol", L.pi_k_attn_fused_batch_ol)):
+            out, out16 = pl.DevBuf(n_seq * d * 4), pl.DevBuf.zeros(16 * d * 2)
+            kc, vc = caches[tag]
+            pl.check(fn(dq.ptr, d + 2 * gqa, tab.ptr, kc.ptr, vc.ptr, stride, n_seq, nh, nkv, hd, 0, n_ctx, dpos.ptr, out.ptr, d, out16.ptr, None), tag)
+            pl.sync()
+            h = from_operand_layout(out16, n_seq, d) if tag == "ol" else out16.download(np.float16, n_seq * d).reshape(n_seq, d)
+            res[tag] = (out.download(np.float32), h, kc.download(np.uint16), vc.download(np.uint16))
+        for a, b in zip(res["plain"], res["ol"]):
+            assert np.array_equal(a.view(np.uint8), b.view(np.uint8))
+        assert np.abs(res["plain"][0]).max() > 0
+
+
 def q4_split_on_device(pl, L, wq4, rows, cols):
     dw = pl.DevBuf(host=wq4)
     qs, ds = pl.DevBuf(rows * cols // 2), pl.DevBuf(rows * cols // 32 * 2)

@@ -864,7 +864,8 @@ __global__ __launch_bounds__(kBaBlock) void batch_axpy_f16_kernel(const __half *
 // grid = (cols / 512, G row groups), two waves a workgroup; a wave owns 256 columns (two 128-column halves) and walks the 16-row
 // steps g, g + G, ...; partial[g][t][c] is summed by batch_reduce_kernel.  At 5120 columns and 5720 union rows a launch takes
 // 15.5 us for 58.6 MB of rows and 10.5 MB of partial sums; four waves a workgroup, or 250 workgroups held one to a compute
-// unit, take the same time, one wave a workgroup with 128 columns and eight steps in flight takes 18 us.
+// unit, take the same time; one wave a workgroup with 128 columns and eight steps in flight takes 18 us, and so do eight waves a
+// workgroup (one workgroup per unit, four waves per column half adding their tiles through LDS).
 typedef _Float16 pi_h4 __attribute__((ext_vector_type(4)));
 __global__ __launch_bounds__(kBlock) void batch_axpy_mfma_f16_kernel(const __half * __restrict__ Wd, int cols, const __half * __restrict__ hc, int hstride,
                                                                      const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,

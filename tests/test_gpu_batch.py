@@ -525,12 +525,14 @@ def test_batch_sparse_ffn_q4_matches_oracle(shape, has_gate, T):
     L.pi_workspace_destroy(ws)
 
 
-@pytest.mark.parametrize("thr", [1e9, -1e9])
-def test_batch_sparse_ffn_none_and_all_active(thr):
-    """Empty union (zero output, residual only) and the full union (every row of every matrix read once: the dense FFN)."""
+@pytest.mark.parametrize("thr,ff", [(1e9, 1024), (-1e9, 1024), (-1e9, 12288), (-1e9, 8200)])
+def test_batch_sparse_ffn_none_and_all_active(thr, ff):
+    """Empty union (zero output, residual only) and the full union (every row of every matrix read once: the dense FFN).  With
+    12288 and 8200 union rows the gate / up kernel, one workgroup per compute unit with at most 32 rows at a time, walks more than
+    one chunk per workgroup (the second shape: a last chunk of 8 rows, on some of the units only)."""
     from powerinfer_amd import lib as pl
     L = pl.init()
-    d, ff, r, T = 1024, 1024, 128, 3
+    d, r, T = 1024, 128, 3
     Lr = synth.make_ffn_layer(seed=5, d=d, ff=ff, r=r, wtype=ol.F16, has_gate=True, T=T)
     x = Lr["x"]
     o = ol.ffn_sparse(ol.oracle(), d, ff, r, T, ol.F16, True, Lr["up"], Lr["gate"], Lr["down_t"], Lr["fc1"], Lr["fc2"], x, x,

@@ -677,12 +677,42 @@ constexpr int kUbWaves = 8, kUbBlock = kUbWaves * PI_WAVE, kUbRows = 32, kUbStep
 template <bool GATE>
 __global__ __launch_bounds__(kUbBlock, 1) void batch_upgate_bal_f16_kernel(const __half * __restrict__ Wup, const __half * __restrict__ Wgate, int cols,
                                                                            const __half * __restrict__ xn, int T, const float * __restrict__ logits, int ff, float thr,
-                                                                           const int32_t * __restrict__ list, const int32_t * __restrict__ n_union,
-                                                                           __half * __restrict__ hc, int hstride, int xol) {
-    // xol != 0: xn in the operand layout (pi_ol_index)
+                                                                           int32_t * __restrict__ list, int32_t * __restrict__ n_union,
+                                                                           __half * __restrict__ hc, int hstride, int xol, const unsigned char * __restrict__ row_any) {
+    // xol != 0: xn in the operand layout (pi_ol_index).
+    // row_any != nullptr (ff <= 32 flags x 512 threads, ff % 16 == 0): the union list is made HERE from the per-neuron flags the
+    // predictor's mat-mul left (a byte each, 0 or 1) instead of by a launch of its own: every workgroup counts all the flags (a thread
+    // takes 32, a scan over the workgroup gives its rank), picks the rows of its own chunk out of them and writes them to `list` for the
+    // down projection; workgroup 0 writes the count.  The flags are requested where the list entries would have been, so the
+    // launch is no deeper; at 13824 neurons it grows by 3 us (256 workgroups reading the same 13.8 KB) and the list kernel's 4.8 us go.
     __shared__ __align__(16) unsigned char tile[kUbWaves][16 * kUbStride];
     __shared__ float cu[kUbWaves][kUbRows][17], cg[GATE ? kUbWaves : 1][kUbRows][17];
-    const int n = *n_union;
+    __shared__ int s_wtot[kUbWaves], s_rows[kUbRows];
+    int n, fl_excl = 0, fl_cnt = 0;
+    uint32_t fl[8] = {0u, 0u, 0u, 0u, 0u, 0u, 0u, 0u};                 // this thread's 32 flags: neurons 32 t .. 32 t + 31
+    if (row_any) {
+        const int f0 = (int)threadIdx.x * 32;
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+            if (f0 + 16 * q < ff) {
+                const pi_u32x4 v = *reinterpret_cast<const pi_u32x4 *>(row_any + f0 + 16 * q);
+                fl[4 * q] = v.x; fl[4 * q + 1] = v.y; fl[4 * q + 2] = v.z; fl[4 * q + 3] = v.w;
+            }
+#pragma unroll
+        for (int q = 0; q < 8; ++q) fl_cnt += __popc(fl[q] & 0x01010101u);
+        int incl = fl_cnt;
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) { const int v = __shfl_up(incl, o, PI_WAVE); if ((int)(threadIdx.x & 63) >= o) incl += v; }
+        if ((threadIdx.x & 63) == 63) s_wtot[threadIdx.x >> 6] = incl;
+        __syncthreads();
+        n = 0;
+#pragma unroll
+        for (int w = 0; w < kUbWaves; ++w) { if (w < (int)(threadIdx.x >> 6)) fl_excl += s_wtot[w]; n += s_wtot[w]; }
+        fl_excl += incl - fl_cnt;
+        if (blockIdx.x == 0 && threadIdx.x == 0) *n_union = n;
+    } else {
+        n = *n_union;
+    }
     const int G = gridDim.x;
     int R = (n + G - 1) / G;
     R = (R + 1) & ~1;
@@ -700,12 +730,27 @@ __global__ __launch_bounds__(kUbBlock, 1) void batch_upgate_bal_f16_kernel(const
     for (int c = blockIdx.x; c < n_chunks; c += G) {
         const int u0 = c * R;
         const int Rc = n - u0 < R ? n - u0 : R;                    // rows of this chunk (the list's last chunk may be short, and odd)
+        if (row_any) {                                             // this chunk's rows out of the flags: ranks u0 .. u0 + Rc - 1
+            if (fl_excl < u0 + Rc && fl_excl + fl_cnt > u0) {
+                int k = fl_excl;
+#pragma unroll
+                for (int q = 0; q < 8; ++q)
+#pragma unroll
+                    for (int e = 0; e < 4; ++e)
+                        if ((fl[q] >> (8 * e)) & 1u) {
+                            if (k >= u0 && k < u0 + Rc) { const int row = (int)threadIdx.x * 32 + 4 * q + e; s_rows[k - u0] = row; list[k] = row; }
+                            ++k;
+                        }
+            }
+            __syncthreads();
+        }
         uint32_t roff[8];                                          // byte offsets of this lane's 8 load instructions (< 2^32: the launcher's test)
 #pragma unroll
         for (int j = 0; j < 8; ++j) {
             const int k = 4 * j + lr;
             const int kk = k < Rc ? k : 4 * j < Rc ? 4 * j : 0;
-            roff[j] = ((uint32_t)list[u0 + kk] * (uint32_t)cols + (4 * j < Rc ? lc * 8 : 0)) * 2;
+            const int row = row_any ? s_rows[kk] : list[u0 + kk];
+            roff[j] = ((uint32_t)row * (uint32_t)cols + (4 * j < Rc ? lc * 8 : 0)) * 2;
         }
         pi_f4 au[2], ag[2];
 #pragma unroll
@@ -777,7 +822,7 @@ __global__ __launch_bounds__(kUbBlock, 1) void batch_upgate_bal_f16_kernel(const
         const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;     // 512 threads: 32 rows x 16 tokens
         if (rr < Rc) {
             float h = 0.0f;
-            if (t < T && !(logits[(size_t)t * ff + list[u0 + rr]] < thr)) {
+            if (t < T && !(logits[(size_t)t * ff + (row_any ? s_rows[rr] : list[u0 + rr])] < thr)) {
                 float su = cu[0][rr][t], sg = GATE ? cg[0][rr][t] : 0.0f;
 #pragma unroll
                 for (int w = 1; w < kUbWaves; ++w) { su += cu[w][rr][t]; if (GATE) sg += cg[w][rr][t]; }
@@ -1211,15 +1256,18 @@ static int batch_sparse_ffn(const float * logits, int T, int ff, float threshold
     if (epilogue < 0 || epilogue > PI_EPI_ADD2 || epilogue == PI_EPI_RELU || (epilogue >= PI_EPI_ADD && !add1) || (epilogue == PI_EPI_ADD2 && !add2))
         return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn: bad epilogue arguments");
     hipStream_t st = (hipStream_t)stream;
-    hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, ws->row_any, ff, ws->words, union_rows, n_union);
+    const int n_cu = pi::compute_units();
+    const bool balanced = cols % 256 == 0 && n_cu > 0 && (size_t)ff * cols * 2 < ((size_t)1 << 32);
+    // the one-workgroup-per-unit gate / up kernel makes the union list itself where its threads can hold all the flags
+    const unsigned char * flags = (balanced && ff <= 32 * kUbBlock && ff % 16 == 0) ? ws->row_any : nullptr;
+    if (!flags) hipLaunchKernelGGL(union_active_kernel, dim3(1), dim3(1024), 0, st, ws->row_any, ff, ws->words, union_rows, n_union);
     const int hstride = ws->max_ff + 16;
     if (cols % 256 == 0) {
-        const int n_cu = pi::compute_units();
-        if (n_cu > 0 && (size_t)ff * cols * 2 < ((size_t)1 << 32)) {
+        if (balanced) {
             if (gate_f16) hipLaunchKernelGGL(batch_upgate_bal_f16_kernel<true>, dim3(n_cu), dim3(kUbBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,
-                                             (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride, xol);
+                                             (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride, xol, flags);
             else hipLaunchKernelGGL(batch_upgate_bal_f16_kernel<false>, dim3(n_cu), dim3(kUbBlock), 0, st, (const __half *)up_f16, (const __half *)nullptr, cols,
-                                    (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride, xol);
+                                    (const __half *)xn_f16, T, logits, ff, threshold, union_rows, n_union, ws->hc_batch, hstride, xol, flags);
         } else if (xol) return pi::fail(PI_E_ARG, "pi_k_batch_sparse_ffn_ol: the operand layout needs the one-workgroup-per-unit kernel (ff * cols * 2 < 4 GiB)");
         else
             hipLaunchKernelGGL(batch_upgate_lds_f16_kernel, dim3((ff + 15) / 16), dim3(kBlock), 0, st, (const __half *)up_f16, (const __half *)gate_f16, cols,

@@ -182,7 +182,12 @@ __global__ __launch_bounds__(kBlock) void attn_decode_kernel(const float * __res
 // ---------------------------------------------------------------------------------------------------
 constexpr int kAttnBlock = 1024;        // 16 waves per head: 64 (hd 128) or 128 (hd 64) cache cells per pass
 constexpr int kAttnPre = 4;             // passes whose K and V rows are requested before the prologue
-__global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __restrict__ qkv, const float2 * __restrict__ rope_table,
+constexpr int kAttnBatch = 4;           // passes behind those whose rows are requested together
+// BLOCK threads per head: kAttnBlock for a single sequence and for steps whose workgroups all fit on the chip at once (two of 1024
+// threads per compute unit); half of that where they do not (16 sequences x 40 heads are 640 workgroups against 512 places: a
+// quarter of the units ran a second round, 48 us at 530 cells; with 512 threads four fit a unit and all 640 run together).
+template <int BLOCK>
+__global__ __launch_bounds__(BLOCK, 8) void attn_fused_kernel(const float * __restrict__ qkv, const float2 * __restrict__ rope_table,
                                                             __half * __restrict__ k_cache, __half * __restrict__ v_cache,
                                                             int n_head, int n_head_kv, int hd, int mode, int n_ctx,
                                                             const int32_t * __restrict__ pos_p, float * __restrict__ out,
@@ -198,7 +203,7 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
     extern __shared__ __align__(16) unsigned char smem[];
     float * s    = reinterpret_cast<float *>(smem);               // [n_ctx] scores, then probabilities
     float * part = s + n_ctx;                                     // [groups][hd]
-    float * qs   = part + (kAttnBlock / (hd / 8)) * hd;               // [hd] rotated q, rounded to fp16
+    float * qs   = part + (BLOCK / (hd / 8)) * hd;                    // [hd] rotated q, rounded to fp16
     float * kcur = qs + hd;                                       // [hd] rotated k of this position, rounded to fp16
     float * vcur = kcur + hd;                                     // [hd]
     __shared__ double red[16];
@@ -215,7 +220,7 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
     // the cache cells of the first kAttnPre passes do not depend on anything computed here: their K and V rows are requested
     // now and travel during the rotation, the scores and the softmax (one memory round trip instead of three in a row)
     const int lpp = hd / 8;
-    const int sub = tid % lpp, grp = tid / lpp, ngrp = kAttnBlock / lpp;
+    const int sub = tid % lpp, grp = tid / lpp, ngrp = BLOCK / lpp;
     const __half * kb = k_cache + (size_t)kvh * n_ctx * hd;
     const __half * vb = v_cache + (size_t)kvh * n_ctx * hd;
     pi_u32x4 kpre[kAttnPre], vpre[kAttnPre];
@@ -261,24 +266,37 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
             if (c < n_kv && sub == 0) s[c] = __fmul_rn(d, scale);
         }
     }
-    for (int c0 = kAttnPre * ngrp; c0 < n_kv; c0 += ngrp) {
-        const int c = c0 + grp;
-        float d = 0.0f;
-        if (c < pos) d = pi_dot8(pi_ld16(kb + (size_t)c * hd + sub * 8), qf, 0.0f);
-        else if (c == pos) {
+    // the passes behind the prefetched ones, kAttnBatch at a time: their rows are requested together and cost one trip to memory
+    // instead of one each (the same dots in the same order)
+    for (int c0 = kAttnPre * ngrp; c0 < n_kv; c0 += kAttnBatch * ngrp) {
+        pi_u32x4 kk[kAttnBatch];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) d = fmaf(kcur[sub * 8 + i], qf[i], d);
+        for (int u = 0; u < kAttnBatch; ++u) {
+            const int c = c0 + u * ngrp + grp;
+            if (c < pos) kk[u] = pi_ld16(kb + (size_t)c * hd + sub * 8);
         }
-        for (int o = lpp / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, PI_WAVE);
-        if (c < n_kv && sub == 0) s[c] = __fmul_rn(d, scale);
+#pragma unroll
+        for (int u = 0; u < kAttnBatch; ++u) {
+            if (c0 + u * ngrp < n_kv) {
+                const int c = c0 + u * ngrp + grp;
+                float d = 0.0f;
+                if (c < pos) d = pi_dot8(kk[u], qf, 0.0f);
+                else if (c == pos) {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) d = fmaf(kcur[sub * 8 + i], qf[i], d);
+                }
+                for (int o = lpp / 2; o > 0; o >>= 1) d += __shfl_xor(d, o, PI_WAVE);
+                if (c < n_kv && sub == 0) s[c] = __fmul_rn(d, scale);
+            }
+        }
     }
     __syncthreads();
 
     float mx = -INFINITY;
-    for (int c = tid; c < n_kv; c += kAttnBlock) mx = fmaxf(mx, s[c]);
+    for (int c = tid; c < n_kv; c += BLOCK) mx = fmaxf(mx, s[c]);
     mx = block_max_f32(mx, redf);
     double sum = 0.0;
-    for (int c = tid; c < n_kv; c += kAttnBlock) {
+    for (int c = tid; c < n_kv; c += BLOCK) {
         const float e = pi_round_f16(expf(pi_round_f16(__fsub_rn(s[c], mx))));
         s[c] = e;
         sum += (double)e;
@@ -304,21 +322,33 @@ __global__ __launch_bounds__(kAttnBlock) void attn_fused_kernel(const float * __
             for (int k = 0; k < 8; ++k) acc[k] = fmaf(vf[k], p, acc[k]);
         }
     }
-    for (int c = kAttnPre * ngrp + grp; c < n_kv; c += ngrp) {
-        const float p = pi_round_f16(__fmul_rn(s[c], inv));
-        float vf[8];
-        if (c < pos) pi_unpack8(pi_ld16(vb + (size_t)c * hd + sub * 8), vf);
-        else {
+    for (int c0 = kAttnPre * ngrp; c0 < n_kv; c0 += kAttnBatch * ngrp) {
+        pi_u32x4 vv[kAttnBatch];
 #pragma unroll
-            for (int i = 0; i < 8; ++i) vf[i] = vcur[sub * 8 + i];
+        for (int u = 0; u < kAttnBatch; ++u) {
+            const int c = c0 + u * ngrp + grp;
+            if (c < pos) vv[u] = pi_ld16(vb + (size_t)c * hd + sub * 8);
         }
 #pragma unroll
-        for (int i = 0; i < 8; ++i) acc[i] = fmaf(vf[i], p, acc[i]);
+        for (int u = 0; u < kAttnBatch; ++u) {
+            const int c = c0 + u * ngrp + grp;
+            if (c < n_kv) {
+                const float p = pi_round_f16(__fmul_rn(s[c], inv));
+                float vf[8];
+                if (c < pos) pi_unpack8(vv[u], vf);
+                else {
+#pragma unroll
+                    for (int i = 0; i < 8; ++i) vf[i] = vcur[sub * 8 + i];
+                }
+#pragma unroll
+                for (int i = 0; i < 8; ++i) acc[i] = fmaf(vf[i], p, acc[i]);
+            }
+        }
     }
 #pragma unroll
     for (int i = 0; i < 8; ++i) part[grp * hd + sub * 8 + i] = acc[i];
     __syncthreads();
-    for (int e = tid; e < hd; e += kAttnBlock) {
+    for (int e = tid; e < hd; e += BLOCK) {
         float v = part[e];
         for (int g = 1; g < ngrp; ++g) v += part[g * hd + e];
         out[(size_t)h * hd + e] = v;
@@ -904,10 +934,10 @@ int pi_k_rope_table(void * table, int n_ctx, int hd, int mode, float theta_scale
 
 // LDS of attn_fused_kernel: the scores of every cell, one partial output row per group of hd/8 lanes, and q, k, v of the new cell
 static bool attn_fused_geometry_ok(int hd) {
-    return hd > 0 && hd % 8 == 0 && kAttnBlock % (hd / 8) == 0 && PI_WAVE % (hd / 8) == 0 && hd / 2 + hd <= kAttnBlock;
+    return hd > 0 && hd % 8 == 0 && (kAttnBlock / 2) % (hd / 8) == 0 && PI_WAVE % (hd / 8) == 0 && hd / 2 + hd <= kAttnBlock / 2;
 }
-static size_t attn_fused_lds_bytes(int hd, int n_ctx) {
-    return sizeof(float) * ((size_t)n_ctx + (size_t)(kAttnBlock / (hd / 8)) * hd + 3 * (size_t)hd);
+static size_t attn_fused_lds_bytes(int hd, int n_ctx, int block = kAttnBlock) {
+    return sizeof(float) * ((size_t)n_ctx + (size_t)(block / (hd / 8)) * hd + 3 * (size_t)hd);
 }
 constexpr size_t kAttnLdsLimit = 60 * 1024;
 
@@ -927,7 +957,7 @@ int pi_k_attn_fused(const float * qkv, const void * rope_table, void * k_cache, 
         return pi::fail(PI_E_ARG, "pi_k_attn_fused: head size must be 8 * (a divisor of 64), at most 128; mode 0 or 2");
     const size_t sh = attn_fused_lds_bytes(hd, n_ctx);
     if (sh > kAttnLdsLimit) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused: context too long for the single-pass kernel");
-    hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
+    hipLaunchKernelGGL(attn_fused_kernel<kAttnBlock>, dim3(n_head), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
                        (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, 0, (size_t)0, 0, nullptr, 0);
     return pi::check_launch("pi_k_attn_fused");
 }
@@ -983,8 +1013,13 @@ static int attn_fused_batch(const float * qkv, int qkv_stride, const void * rope
         return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch: head size must be 8 * (a divisor of 64), at most 128; mode 0 or 2");
     const size_t sh = attn_fused_lds_bytes(hd, n_ctx);
     if (sh > kAttnLdsLimit) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused_batch: context too long for the single-pass kernel");
-    hipLaunchKernelGGL(attn_fused_kernel, dim3(n_head, n_seq), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
-                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride, (__half *)out_f16, out16_ol);
+    const int n_cu = pi::compute_units();
+    if (n_cu > 0 && n_seq * n_head > 2 * n_cu)
+        hipLaunchKernelGGL(attn_fused_kernel<kAttnBlock / 2>, dim3(n_head, n_seq), dim3(kAttnBlock / 2), attn_fused_lds_bytes(hd, n_ctx, kAttnBlock / 2), (hipStream_t)stream, qkv, (const float2 *)rope_table,
+                           (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride, (__half *)out_f16, out16_ol);
+    else
+        hipLaunchKernelGGL(attn_fused_kernel<kAttnBlock>, dim3(n_head, n_seq), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
+                           (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride, (__half *)out_f16, out16_ol);
     return pi::check_launch("pi_k_attn_fused_batch");
 }
 

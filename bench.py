@@ -317,7 +317,7 @@ def main():
     ap.add_argument("--n-seq", type=int, default=16, choices=[1, 16], help="config 3: 16 sequences in lockstep (configs[3]) or the same model at batch 1")
     ap.add_argument("--batch-model", default="llama-13b", choices=["llama-13b", "llama-7b-q4"], help="config 3 with 16 sequences: configs[3]'s model, or the Q4_0 7B model in lockstep")
     ap.add_argument("--mean-rate", type=float, default=None, help="config 3: mean firing rate of the synthetic predictors (default: the model's own, 0.11)")
-    ap.add_argument("--dense-above", type=float, default=None, help="config 3: union fraction above which a layer's FFN runs dense (library default 0.9; 0 always, 1 never)")
+    ap.add_argument("--dense-above", type=float, default=None, help="config 3: union fraction above which a layer's FFN runs dense (0 always, 1 never: the library's default)")
     ap.add_argument("--rest-on-gpu", action="store_true", help="config 2: the GPU reads the non-resident neurons' rows from pinned host memory itself instead of handing those neurons to host threads")
     ap.add_argument("--hot-frac", type=float, default=None, help="configs 1 and 2: share of each layer's neurons on the GPU (default 1.0 and 0.6)")
     ap.add_argument("--pmc-probe", action="store_true",

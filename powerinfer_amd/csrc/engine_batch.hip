@@ -16,8 +16,9 @@ struct BatchState {
     int n_seq = 0, max_steps = 4096;
     int kv_hi = 0;                        // prompt chunks: cells the chunk's last token attends (its position + 1)
     // lockstep decoding: layers whose union of active rows was above dense_above * n_ff in the last step run their FFN dense
+    // (>= 1: never, the default: the union kernels are the faster ones at every union fraction measured, see batch_layer)
     std::vector<char> dense_ffn, graph_dense;
-    float dense_above = 0.9f;
+    float dense_above = 1.0f;
     bool prefill = false;                 // prompt chunks of the model's own sequence: tokens share the model's KV cache
     float * q_rot = nullptr;
     size_t cache_seq_stride = 0;          // elements per sequence: n_layer * n_head_kv * n_ctx * hd
@@ -258,9 +259,11 @@ int batch_layer(pi_model * m, BatchState * b, int il) {
     PI_TRY(pi_k_batch_predictor_fc2_ol(fc2.dev, ff, r, b->hid16, T, hp.sparse_threshold, b->pred_logits, m->ws, st));
     // Dense cross-over (the reference's switch from its batch-sparse kernels to a plain mat-mul, ggml-cuda.cu:8787-8814, 7717-7756):
     // when the sequences' active sets together cover nearly all of the layer, gathering rows costs more than streaming all of them.
-    // Measured on the 13B shape, 40 layers, 16 sequences (ms per step, union kernels / dense): union 0.41 of n_ff 7.46 / 9.18,
-    // 0.61 8.27 / 9.26, 0.75 8.63 / 9.24, 0.91 9.40 / 9.29, 0.99 9.60 / 9.38 - the union kernels lose only beyond 0.9.  The choice
-    // is made from the union the previous step measured (the count below keeps that statistic alive while the layer runs dense).
+    // Measured on the 13B shape, 40 layers, 16 sequences, 128-token prompts (ms per step, union kernels / dense): union 0.41 of n_ff
+    // 5.59 / 7.61, 0.61 7.03 / 7.66, 0.75 7.26 / 7.68, 0.92 7.44 / 7.74, 0.99 7.55 / 7.77 - the union kernels win everywhere (they lost
+    // beyond 0.9, 9.60 / 9.38 at 0.99, before the union rows were dealt evenly to the units and the down projection stopped going
+    // through LDS), so the switch is off unless the caller sets a fraction (pi_model_batch_set_dense_above).  The choice is made from
+    // the union the previous step measured (the count below keeps that statistic alive while the layer runs dense).
     if (!b->prefill && !b->unified && il < (int)b->dense_ffn.size() && b->dense_ffn[il]) {
         PI_TRY(pi_k_batch_union_count(ff, b->union_rows, b->n_union + il, m->ws, st));
         PI_TRY(pi_k_gemm_f16_ol(up.dev, ff, d, ffn_x, T, PI_EPI_NONE, nullptr, nullptr, b->up_out, nullptr, st));

@@ -619,7 +619,7 @@ def test_batched_decode_matches_per_sequence_oracle(arch, wtype):
 @pytest.mark.parametrize("arch", ["llama-tiny", "falcon-tiny"])
 def test_lockstep_decoding_crosses_over_to_dense_ffn(arch):
     """The dense cross-over of batched decoding: with an active set that covers 95 % of every layer the union of the sequences' rows
-    is above the switch (90 % of n_ff), so from the second step on every layer computes its FFN as dense gate / up mat-muls, h under
+    is above a switch set to 90 % of n_ff, so from the second step on every layer computes its FFN as dense gate / up mat-muls, h under
     the predictor's mask, and a dense down mat-mul.  The first step has no statistic yet and runs the union kernels.  Both forms
     against the CPU oracle per sequence (margin-protected model: logits within 1e-2 at every step, identical greedy tokens), against
     each other (an engine that never switches), and through the captured graph, which is re-captured when the choice changes."""
@@ -631,6 +631,7 @@ def test_lockstep_decoding_crosses_over_to_dense_ffn(arch):
     auto, never, always = Model(hp).load(model), Model(hp).load(model), Model(hp).load(model)
     for g in (auto, never, always):
         g.batch_init(n_seq)
+    auto.batch_set_dense_above(0.9)                                # (the library's default is never)
     never.batch_set_dense_above(1.0)
     always.batch_set_dense_above(0.0)
     assert auto.batch_dense_layers() == 0 and never.batch_dense_layers() == 0 and always.batch_dense_layers() == hp.n_layer

@@ -323,6 +323,34 @@ def from_operand_layout(buf, T, cols):
     return buf.download(np.float16, 16 * cols).reshape(cols // 8, 16, 8)[:, :T, :].transpose(1, 0, 2).reshape(T, cols)
 
 
+@pytest.mark.parametrize("rows,cols,T", [(72, 128, 1), (520, 640, 7), (1032, 384, 16), (4096, 4096, 16), (3000, 5120, 9)])
+def test_gemm_in_the_operand_layout_matches_the_token_major_one_bit_for_bit(rows, cols, T):
+    """pi_k_gemm_f16_ol against pi_k_gemm_f16 on shapes of both kernels behind them (column counts that are and are not multiples of
+    256), one token, a ragged last row tile, every epilogue, and the fp16 copy in either layout."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    rng = np.random.default_rng(rows + T)
+    w = (0.05 * rng.standard_normal((rows, cols))).astype(np.float16)
+    x = rng.standard_normal((T, cols)).astype(np.float32)
+    a1, a2 = rng.standard_normal((T, rows)).astype(np.float32), rng.standard_normal((T, rows)).astype(np.float32)
+    dw, dx, d1, d2 = pl.DevBuf(host=w), pl.DevBuf(host=x), pl.DevBuf(host=a1), pl.DevBuf(host=a2)
+    na = pl.norm_arg(0, 0.0, None, None)
+    xn, xo = pl.DevBuf.zeros(T * cols * 2), pl.DevBuf.zeros(16 * cols * 2)
+    pl.check(L.pi_k_norm_round_f16(dx.ptr, T, cols, na, xn.ptr, None, None), "norm")
+    pl.check(L.pi_k_norm_round_f16_ol(dx.ptr, T, cols, na, xo.ptr, None, None), "norm ol")
+    for epi, p1, p2 in ((pl.EPI_NONE, None, None), (pl.EPI_RELU, None, None), (pl.EPI_ADD, d1.ptr, None), (pl.EPI_ADD2, d1.ptr, d2.ptr)):
+        y, y16 = pl.DevBuf(T * rows * 4), pl.DevBuf.zeros(T * rows * 2)
+        yo, yo16 = pl.DevBuf(T * rows * 4), pl.DevBuf.zeros(16 * rows * 2)
+        pl.check(L.pi_k_gemm_f16(dw.ptr, rows, cols, xn.ptr, T, epi, p1, p2, y.ptr, y16.ptr, None), "gemm")
+        pl.check(L.pi_k_gemm_f16_ol(dw.ptr, rows, cols, xo.ptr, T, epi, p1, p2, yo.ptr, yo16.ptr, None), "gemm ol")
+        pl.sync()
+        assert np.array_equal(y.download(np.float32).view(np.uint32), yo.download(np.float32).view(np.uint32)), epi
+        assert np.array_equal(y16.download(np.float16, T * rows).reshape(T, rows).view(np.uint16), from_operand_layout(yo16, T, rows).view(np.uint16)), epi
+    assert np.abs(y.download(np.float32)).max() > 0
+    assert L.pi_k_gemm_f16_ol(dw.ptr, rows - 4, cols, xo.ptr, T, pl.EPI_NONE, None, None, yo.ptr, yo16.ptr, None) != 0          # fp16 copy: rows % 8
+    assert L.pi_k_norm_round_f16_ol(dx.ptr, 17, cols, na, xo.ptr, None, None) != 0                                               # 16 token slots
+
+
 @pytest.mark.parametrize("shape,has_gate,T", [((5120, 13824, 1280), True, 16), ((4096, 11008, 1024), False, 5), ((1024, 1024, 128), True, 3)])
 def test_operand_layout_entry_points_match_the_token_major_ones_bit_for_bit(shape, has_gate, T):
     """The *_ol entry points keep a step's fp16 activations in the operand layout of the matrix cores ([cols / 8][16][8]); only the

@@ -487,6 +487,13 @@ PI_API int pi_k_attn_ggml_step(const float * qkv, int qkv_stride, const int32_t 
 PI_API int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache,
                                  size_t cache_seq_stride, int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx,
                                  const int32_t * pos, float * out, int out_stride, void * out_f16, pi_stream_t stream);
+/* the same for a Q4_0 output projection: instead of an fp16 copy, the output as the Q8_0 blocks pi_k_gemm_q4_t16 multiplies with (what
+ * pi_k_norm_q8_blocks without a norm makes of `out`, bit for bit: blocks in the MFMA operand layout, scales and -8 * sums as [block][16]);
+ * head size % 32 == 0 */
+PI_API int pi_k_attn_fused_batch_q8(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache,
+                                    size_t cache_seq_stride, int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx,
+                                    const int32_t * pos, float * out, int out_stride, void * q8_quants, float * q8_scales, int32_t * q8_sums,
+                                    pi_stream_t stream);
 /* the same with the fp16 copy in the operand layout of pi_k_gemm_f16_ol (16 sequence slots of n_head * hd columns; out stays [n_seq][out_stride]) */
 PI_API int pi_k_attn_fused_batch_ol(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache,
                                     size_t cache_seq_stride, int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx,

@@ -174,10 +174,13 @@ int batch_layer_q4(pi_model * m, BatchState * b, int il) {
         PI_TRY(cells_attention(m, b, il, T));
     else if (b->prefill)
         PI_TRY(chunk_attention(m, b, T, kv_off));
+    else if (hd % 32 == 0)                                         // lockstep: the attention writes the Q8_0 blocks of its output itself
+        PI_TRY(pi_k_attn_fused_batch_q8(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
+                                        hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, hp.n_ctx, b->d_pos, b->att, d, b->qa, b->da, b->sa, st));
     else
         PI_TRY(pi_k_attn_fused_batch(b->qkv, d + 2 * gqa, m->rope_table, b->k_cache + kv_off, b->v_cache + kv_off, b->cache_seq_stride, T,
                                      hp.n_head, hp.n_head_kv, hd, falcon ? 2 : 0, hp.n_ctx, b->d_pos, b->att, d, b->att16, st));
-    PI_TRY(pi_k_norm_q8_blocks(b->att, T, d, &plain, b->qa, b->da, b->sa, nullptr, st));
+    if (b->unified || b->prefill || hd % 32 != 0) PI_TRY(pi_k_norm_q8_blocks(b->att, T, d, &plain, b->qa, b->da, b->sa, nullptr, st));
     if (!falcon) {
         PI_TRY(pi_k_gemm_q4_t16(wo.quants, wo.scales, d, d, b->qa, b->da, b->sa, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, st));       // ffn_inp = wo.att + x
         pi_norm fn = mk_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);

@@ -191,7 +191,10 @@ __global__ __launch_bounds__(BLOCK, 8) void attn_fused_kernel(const float * __re
                                                             __half * __restrict__ k_cache, __half * __restrict__ v_cache,
                                                             int n_head, int n_head_kv, int hd, int mode, int n_ctx,
                                                             const int32_t * __restrict__ pos_p, float * __restrict__ out,
-                                                            int qkv_stride, size_t cache_seq_stride, int out_stride, __half * __restrict__ out16, int out16_ol) {
+                                                            int qkv_stride, size_t cache_seq_stride, int out_stride, __half * __restrict__ out16, int out16_ol,
+                                                            int8_t * __restrict__ q8_q, float * __restrict__ q8_d, int * __restrict__ q8_s) {
+    // q8_q != nullptr: the output also as the Q8_0 blocks an integer mat-mul of a Q4_0 matrix multiplies with (the blocks, scales and
+    // -8 * sums pi_k_norm_q8_blocks makes of the same values: a head's hd outputs are whole blocks of 32, one per half-wave)
     // blockIdx.y = sequence of a batched step (its own token, position and cache); 0 for single-sequence decoding
     // out16_ol != 0: the fp16 copy in the operand layout of the 16-token mat-muls (pi_ol_index) instead of [sequence][out_stride]
     qkv += (size_t)blockIdx.y * qkv_stride;
@@ -353,6 +356,19 @@ __global__ __launch_bounds__(BLOCK, 8) void attn_fused_kernel(const float * __re
         for (int g = 1; g < ngrp; ++g) v += part[g * hd + e];
         out[(size_t)h * hd + e] = v;
         if (out16) out16[out16_ol ? pi_ol_index(blockIdx.y, h * hd + e) : (size_t)h * hd + e] = __float2half_rn(v);
+        if (q8_q) {                                               // (hd % 32 == 0: the lanes of a block run this together)
+            float amax = fabsf(v);
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, PI_WAVE));
+            const float d = pi_round_f16(pi_div(amax, 127.0f)), id = (amax != 0.0f) ? pi_div(127.0f, amax) : 0.0f;
+            const int q = (int)rintf(__fmul_rn(v, id));
+            int sq = q;
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) sq += __shfl_xor(sq, o, PI_WAVE);
+            const int i = h * hd + e, eb = i & 31, t = blockIdx.y;
+            q8_q[(((size_t)(i >> 5) * 4 + ((eb & 15) >> 2)) * 16 + t) * 8 + (eb >> 4) * 4 + (eb & 3)] = (int8_t)q;
+            if (eb == 0) { q8_d[(size_t)(i >> 5) * 16 + t] = d; q8_s[(size_t)(i >> 5) * 16 + t] = -8 * sq; }
+        }
     }
 }
 
@@ -958,7 +974,7 @@ int pi_k_attn_fused(const float * qkv, const void * rope_table, void * k_cache, 
     const size_t sh = attn_fused_lds_bytes(hd, n_ctx);
     if (sh > kAttnLdsLimit) return pi::fail(PI_E_UNSUPPORTED, "pi_k_attn_fused: context too long for the single-pass kernel");
     hipLaunchKernelGGL(attn_fused_kernel<kAttnBlock>, dim3(n_head), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
-                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, 0, (size_t)0, 0, nullptr, 0);
+                       (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, 0, (size_t)0, 0, nullptr, 0, nullptr, nullptr, nullptr);
     return pi::check_launch("pi_k_attn_fused");
 }
 
@@ -1007,7 +1023,8 @@ int pi_k_attn_split_cached(const float * q_rot, const void * k_cache, const void
 
 static int attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache, size_t cache_seq_stride,
                             int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, const int32_t * pos, float * out, int out_stride,
-                            void * out_f16, pi_stream_t stream, int out16_ol) {
+                            void * out_f16, pi_stream_t stream, int out16_ol, void * q8_q = nullptr, float * q8_d = nullptr, int32_t * q8_s = nullptr) {
+    if (q8_q && (hd % 32 || !q8_d || !q8_s)) return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch_q8: head size % 32 == 0 and all three outputs required");
     if (!qkv || !rope_table || !k_cache || !v_cache || !pos || !out || n_seq <= 0 || n_seq > kBtMaxT) return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch: bad arguments");
     if (n_head <= 0 || n_head_kv <= 0 || n_head % n_head_kv || !attn_fused_geometry_ok(hd) || (mode != 0 && mode != 2))
         return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch: head size must be 8 * (a divisor of 64), at most 128; mode 0 or 2");
@@ -1016,10 +1033,10 @@ static int attn_fused_batch(const float * qkv, int qkv_stride, const void * rope
     const int n_cu = pi::compute_units();
     if (n_cu > 0 && n_seq * n_head > 2 * n_cu)
         hipLaunchKernelGGL(attn_fused_kernel<kAttnBlock / 2>, dim3(n_head, n_seq), dim3(kAttnBlock / 2), attn_fused_lds_bytes(hd, n_ctx, kAttnBlock / 2), (hipStream_t)stream, qkv, (const float2 *)rope_table,
-                           (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride, (__half *)out_f16, out16_ol);
+                           (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride, (__half *)out_f16, out16_ol, (int8_t *)q8_q, q8_d, q8_s);
     else
         hipLaunchKernelGGL(attn_fused_kernel<kAttnBlock>, dim3(n_head, n_seq), dim3(kAttnBlock), sh, (hipStream_t)stream, qkv, (const float2 *)rope_table,
-                           (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride, (__half *)out_f16, out16_ol);
+                           (__half *)k_cache, (__half *)v_cache, n_head, n_head_kv, hd, mode, n_ctx, pos, out, qkv_stride, cache_seq_stride, out_stride, (__half *)out_f16, out16_ol, (int8_t *)q8_q, q8_d, q8_s);
     return pi::check_launch("pi_k_attn_fused_batch");
 }
 
@@ -1027,6 +1044,14 @@ int pi_k_attn_fused_batch(const float * qkv, int qkv_stride, const void * rope_t
                           int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, const int32_t * pos, float * out, int out_stride,
                           void * out_f16, pi_stream_t stream) {
     return attn_fused_batch(qkv, qkv_stride, rope_table, k_cache, v_cache, cache_seq_stride, n_seq, n_head, n_head_kv, hd, mode, n_ctx, pos, out, out_stride, out_f16, stream, 0);
+}
+
+int pi_k_attn_fused_batch_q8(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache, size_t cache_seq_stride,
+                             int n_seq, int n_head, int n_head_kv, int hd, int mode, int n_ctx, const int32_t * pos, float * out, int out_stride,
+                             void * q8_quants, float * q8_scales, int32_t * q8_sums, pi_stream_t stream) {
+    if (!q8_quants) return pi::fail(PI_E_ARG, "pi_k_attn_fused_batch_q8: null pointer");
+    return attn_fused_batch(qkv, qkv_stride, rope_table, k_cache, v_cache, cache_seq_stride, n_seq, n_head, n_head_kv, hd, mode, n_ctx, pos, out, out_stride, nullptr, stream, 0,
+                            q8_quants, q8_scales, q8_sums);
 }
 
 int pi_k_attn_fused_batch_ol(const float * qkv, int qkv_stride, const void * rope_table, void * k_cache, void * v_cache, size_t cache_seq_stride,

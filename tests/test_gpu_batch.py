@@ -423,6 +423,45 @@ def test_lockstep_attention_writes_the_same_fp16_copy_in_either_layout(nh, nkv, 
         assert np.abs(res["plain"][0]).max() > 0
 
 
+@pytest.mark.parametrize("nh,nkv,hd,n_seq", [(8, 8, 128, 5), (16, 2, 64, 16)])
+def test_lockstep_attention_writes_the_q8_blocks_of_its_output(nh, nkv, hd, n_seq):
+    """pi_k_attn_fused_batch_q8 leaves the Q8_0 blocks of the attention output (operand layout of the integer mat-mul, scales,
+    -8 * sums) that pi_k_norm_q8_blocks without a norm makes of the fp32 output of pi_k_attn_fused_batch: the same bytes, so the
+    Q4_0 steps need no launch between the attention and the output projection."""
+    import ctypes as C
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    rng = np.random.default_rng(nh + n_seq + 1)
+    n_ctx, gqa, d = 32, nkv * hd, nh * hd
+    stride = nkv * n_ctx * hd
+    tab = pl.DevBuf(n_ctx * hd * 4)
+    pl.check(L.pi_k_rope_table(tab.ptr, n_ctx, hd, 0, float(np.float32(10000.0) ** np.float32(-2.0 / hd)), 1.0, None), "rope_table")
+    caches = {k: (pl.DevBuf.zeros(n_seq * stride * 2), pl.DevBuf.zeros(n_seq * stride * 2)) for k in ("two", "one")}
+    dq, dpos = pl.DevBuf(n_seq * (d + 2 * gqa) * 4), pl.DevBuf(n_seq * 4)
+    na = pl.Norm(0, 0.0, None, None)
+    for step in range(3):
+        dq.upload(rng.standard_normal(n_seq * (d + 2 * gqa)).astype(np.float32))
+        dpos.upload(np.full(n_seq, step, np.int32))
+        res = {}
+        for tag in ("two", "one"):
+            out = pl.DevBuf(n_seq * d * 4)
+            q, dd, ss = pl.DevBuf.zeros(16 * d), pl.DevBuf.zeros(d // 32 * 16 * 4), pl.DevBuf.zeros(d // 32 * 16 * 4)
+            kc, vc = caches[tag]
+            if tag == "two":
+                pl.check(L.pi_k_attn_fused_batch(dq.ptr, d + 2 * gqa, tab.ptr, kc.ptr, vc.ptr, stride, n_seq, nh, nkv, hd, 0, n_ctx, dpos.ptr, out.ptr, d, None, None), tag)
+                pl.check(L.pi_k_norm_q8_blocks(out.ptr, n_seq, d, C.byref(na), q.ptr, dd.ptr, ss.ptr, None, None), "q8 blocks")
+            else:
+                pl.check(L.pi_k_attn_fused_batch_q8(dq.ptr, d + 2 * gqa, tab.ptr, kc.ptr, vc.ptr, stride, n_seq, nh, nkv, hd, 0, n_ctx, dpos.ptr, out.ptr, d,
+                                                    q.ptr, dd.ptr, ss.ptr, None), tag)
+            pl.sync()
+            # token slots behind n_seq are never written by either
+            qv = q.download(np.uint8).reshape(d // 32, 4, 16, 8)[:, :, :n_seq]
+            res[tag] = (out.download(np.float32).view(np.uint32), qv, dd.download(np.uint32).reshape(-1, 16)[:, :n_seq], ss.download(np.int32).reshape(-1, 16)[:, :n_seq])
+        for a, b in zip(res["two"], res["one"]):
+            assert np.array_equal(a, b)
+        assert res["one"][1].any()
+
+
 def q4_split_on_device(pl, L, wq4, rows, cols):
     dw = pl.DevBuf(host=wq4)
     qs, ds = pl.DevBuf(rows * cols // 2), pl.DevBuf(rows * cols // 32 * 2)

@@ -347,6 +347,8 @@ PI_API int pi_k_gemm_tile_f16(const void * W_f16, int rows, int cols, const void
  * h and hq are caller-provided scratch of 16 * ff floats each. */
 PI_API int pi_k_q4_split(const void * W_q4, int rows, int cols, void * quants, void * scales, pi_stream_t stream);
 PI_API int pi_k_norm_q8_blocks(const float * x, int T, int cols, const pi_norm * norm, void * q, float * d, int32_t * s8, void * plain_f16, pi_stream_t stream);
+/* the same with the fp16 copy of the un-normalised rows in the operand layout of pi_k_gemm_f16_ol (16 token slots) */
+PI_API int pi_k_norm_q8_blocks_ol(const float * x, int T, int cols, const pi_norm * norm, void * q, float * d, int32_t * s8, void * plain_ol, pi_stream_t stream);
 PI_API int pi_k_gemm_q4_t16(const void * quants, const void * scales, int rows, int cols, const void * xq, const float * xd, const int32_t * xs8, int T,
                             int epilogue, const float * add1, const float * add2, float * y, pi_stream_t stream);
 PI_API int pi_k_batch_sparse_ffn_q4(const float * logits, int T, int ff, float threshold, const void * up_quants, const void * up_scales,

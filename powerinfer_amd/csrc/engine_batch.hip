@@ -162,7 +162,8 @@ int batch_layer_q4(pi_model * m, BatchState * b, int il) {
     if (!falcon) an = mk_norm(1, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), nullptr);
     else if (m->L(il, PI_T_ATTN_NORM_2).dev) an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM_2), &m->L(il, PI_T_ATTN_NORM_2_B));
     else an = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
-    PI_TRY(pi_k_norm_q8_blocks(x, T, d, &an, b->qa, b->da, b->sa, falcon ? b->xp16 : nullptr, st));      // Falcon: the predictor reads the layer input as plain fp16
+    // (the predictor's fp16 inputs, xp16 and hid16, are kept in the operand layout of the 16-token fp16 mat-muls)
+    PI_TRY(pi_k_norm_q8_blocks_ol(x, T, d, &an, b->qa, b->da, b->sa, falcon ? b->xp16 : nullptr, st));   // Falcon: the predictor reads the layer input as plain fp16
     if (falcon) {
         // the FFN branch reads the layer input too, under its own norm (with a single norm: the attention's)
         pi_norm fn = mk_norm(2, hp.norm_eps, m->L(il, PI_T_ATTN_NORM), &m->L(il, PI_T_ATTN_NORM_B));
@@ -184,12 +185,12 @@ int batch_layer_q4(pi_model * m, BatchState * b, int il) {
     if (!falcon) {
         PI_TRY(pi_k_gemm_q4_t16(wo.quants, wo.scales, d, d, b->qa, b->da, b->sa, T, PI_EPI_ADD, x, nullptr, b->ffn_inp, st));       // ffn_inp = wo.att + x
         pi_norm fn = mk_norm(1, hp.norm_eps, m->L(il, PI_T_FFN_NORM), nullptr);
-        PI_TRY(pi_k_norm_q8_blocks(b->ffn_inp, T, d, &fn, b->qf, b->df, b->sf, b->xp16, st));                                        // the predictor reads the rows before the norm
+        PI_TRY(pi_k_norm_q8_blocks_ol(b->ffn_inp, T, d, &fn, b->qf, b->df, b->sf, b->xp16, st));                                     // the predictor reads the rows before the norm
     } else {
         PI_TRY(pi_k_gemm_q4_t16(wo.quants, wo.scales, d, d, b->qa, b->da, b->sa, T, PI_EPI_NONE, nullptr, nullptr, b->attn_out, st));
     }
-    PI_TRY(pi_k_gemm_f16(fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16, st));
-    PI_TRY(pi_k_batch_predictor_fc2(fc2.dev, ff, r, b->hid16, T, hp.sparse_threshold, b->pred_logits, m->ws, st));
+    PI_TRY(pi_k_gemm_f16_ol(fc1.dev, r, d, b->xp16, T, PI_EPI_RELU, nullptr, nullptr, b->hidden, b->hid16, st));
+    PI_TRY(pi_k_batch_predictor_fc2_ol(fc2.dev, ff, r, b->hid16, T, hp.sparse_threshold, b->pred_logits, m->ws, st));
     const auto up = W(PI_T_FFN_UP), down = W(PI_T_FFN_DOWN_T);
     if (!falcon) {
         const auto gate = W(PI_T_FFN_GATE);

@@ -33,7 +33,8 @@ __global__ void q4_split_kernel(const pi_block_q4_0 * __restrict__ w, size_t n_b
 // d = fp16(amax / 127), q = rint(v * (127 / amax)).  Outputs: q in the MFMA's operand layout (below), d and -8 * sum(q) as [blk][16]
 // (token innermost).
 __global__ __launch_bounds__(1024) void norm_q8_blocks_kernel(const float * __restrict__ x, int cols, NormArgs na, int8_t * __restrict__ q_out,
-                                                              float * __restrict__ d_out, int * __restrict__ s8_out, __half * __restrict__ plain16) {
+                                                              float * __restrict__ d_out, int * __restrict__ s8_out, __half * __restrict__ plain16, int plain_ol) {
+    // plain_ol != 0: plain16 in the operand layout of the 16-token fp16 mat-muls (pi_ol_index) instead of [token][cols]
     __shared__ double red[16];
     const int t = blockIdx.x;
     const float * xt = x + (size_t)t * cols;
@@ -69,7 +70,7 @@ __global__ __launch_bounds__(1024) void norm_q8_blocks_kernel(const float * __re
         if (k * 1024 >= cols) break;                              // uniform: the row ends before this slot
         const int i = threadIdx.x + k * 1024;
         float v = xv[k];
-        if (plain16 && i < cols) plain16[(size_t)t * cols + i] = __float2half_rn(v);
+        if (plain16 && i < cols) plain16[plain_ol ? pi_ol_index(t, i) : (size_t)t * cols + i] = __float2half_rn(v);
         if (na.kind != 0) {
             v = __fmul_rn(na.kind == 2 ? __fsub_rn(v, mean) : v, scale);
             if (na.w) v = __fmul_rn(v, wv[k]);
@@ -370,8 +371,15 @@ int pi_k_q4_split(const void * W_q4, int rows, int cols, void * quants, void * s
 int pi_k_norm_q8_blocks(const float * x, int T, int cols, const pi_norm * norm, void * q, float * d, int32_t * s8, void * plain_f16, pi_stream_t stream) {
     if (!x || !norm || !q || !d || !s8 || T < 1 || T > kBtMaxT || cols <= 0 || cols % 32 || cols > 8192)
         return pi::fail(PI_E_ARG, "pi_k_norm_q8_blocks: 1 <= T <= 16, cols % 32 == 0 and cols <= 8192 required");
-    hipLaunchKernelGGL(norm_q8_blocks_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (int8_t *)q, d, s8, (__half *)plain_f16);
+    hipLaunchKernelGGL(norm_q8_blocks_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (int8_t *)q, d, s8, (__half *)plain_f16, 0);
     return pi::check_launch("pi_k_norm_q8_blocks");
+}
+
+int pi_k_norm_q8_blocks_ol(const float * x, int T, int cols, const pi_norm * norm, void * q, float * d, int32_t * s8, void * plain_ol, pi_stream_t stream) {
+    if (!x || !norm || !q || !d || !s8 || T < 1 || T > kBtMaxT || cols <= 0 || cols % 32 || cols > 8192)
+        return pi::fail(PI_E_ARG, "pi_k_norm_q8_blocks_ol: 1 <= T <= 16, cols % 32 == 0 and cols <= 8192 required");
+    hipLaunchKernelGGL(norm_q8_blocks_kernel, dim3(T), dim3(1024), 0, (hipStream_t)stream, x, cols, to_norm(norm), (int8_t *)q, d, s8, (__half *)plain_ol, 1);
+    return pi::check_launch("pi_k_norm_q8_blocks_ol");
 }
 
 int pi_k_gemm_q4_t16(const void * quants, const void * scales, int rows, int cols, const void * xq, const float * xd, const int32_t * xs8, int T,

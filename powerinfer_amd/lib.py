@@ -90,6 +90,7 @@ _SIGS = {
     "pi_k_batch_union_count": (_i, [_i, _vp, _vp, _vp, _vp]),
     "pi_k_q4_split": (_i, [_vp, _i, _i, _vp, _vp, _vp]),
     "pi_k_norm_q8_blocks": (_i, [_vp, _i, _i, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp]),
+    "pi_k_norm_q8_blocks_ol": (_i, [_vp, _i, _i, C.POINTER(Norm), _vp, _vp, _vp, _vp, _vp]),
     "pi_k_gemm_q4_t16": (_i, [_vp, _vp, _i, _i, _vp, _vp, _vp, _i, _i, _vp, _vp, _vp, _vp]),
     "pi_k_batch_sparse_ffn_q4": (_i, [_vp, _i, _i, _f, _vp, _vp, _vp, _vp, _vp, _vp, _i, _vp, _vp, _vp, _i, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp, _vp]),
     "pi_k_gemm_tile_f16": (_i, [_vp, _i, _i, _vp, _i, _i, _vp, _vp, _vp, _vp, _i, _vp]),

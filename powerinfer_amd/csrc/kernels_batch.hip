@@ -185,25 +185,24 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_f16_kernel(const __half * __r
 // row stride (conflict-free both ways) and reads it back in operand layout.  No workgroup barrier is involved: the
 // buffer belongs to one wave and LDS operations of a wave complete in order.  Two 256-column tiles of loads are in flight.
 constexpr int kGlStride = 512 + 16;               // bytes per LDS row: 256 fp16 + one 16-byte pad
-template <int RT>
-__global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
+template <int RT, int NW>
+__global__ __launch_bounds__(64 * NW) void gemm_t16_lds_f16_kernel(const __half * __restrict__ W, const __half * __restrict__ xn, int T, int rows, int cols,
                                                                   int epi, const float * __restrict__ add1, const float * __restrict__ add2, float * __restrict__ y,
                                                                   __half * __restrict__ y16, float thr, unsigned char * __restrict__ row_any, int lay) {
-    __shared__ __align__(16) unsigned char tile[kWavesPerBlock][16 * kGlStride];
-    __shared__ float cs[kWavesPerBlock][16][17];
+    __shared__ __align__(16) unsigned char tile[NW][16 * kGlStride];
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
     const int i = lane & 15, g = lane >> 4;
     const int lr = lane >> 5, lc = lane & 31;           // load role: row within the pair, 16-byte chunk within the 512-byte row piece
     const int row0 = blockIdx.x * 16 * RT;
     const int tok = i < T ? i : T - 1;
-    // the 256-column super-steps of a row are dealt round-robin to the four waves: wave w takes steps w, w + 4, ...
+    // the 256-column super-steps of a row are dealt round-robin to the NW waves: wave w takes steps w, w + NW, ...
     const __half * bp = (lay & 1) ? xn + (g * 16 + i) * 8 : xn + (size_t)tok * cols + g * 8;
     const int bstep = (lay & 1) ? 512 : 32;        // halves from one 32-column step's fragment to the next
     unsigned char * mytile = tile[wave];
     pi_f4 acc[RT];
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) acc[rt] = pi_f4{0.0f, 0.0f, 0.0f, 0.0f};
-    const int n_ss = (cols / 256 - wave + kWavesPerBlock - 1) / kWavesPerBlock;      // super-steps of this wave
+    const int n_ss = (cols / 256 - wave + NW - 1) / NW;      // super-steps of this wave
     pi_u32x4 ld[2][RT][8];
     auto issue = [&](int buf, int ss) {
         if (ss < n_ss) {
@@ -213,7 +212,7 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
                 for (int j = 0; j < 8; ++j) {
                     int r = row0 + rt * 16 + 2 * j + lr;
                     r = r < rows ? r : rows - 1;
-                    ld[buf][rt][j] = pi_ld_stream(W + (size_t)r * cols + (wave + ss * kWavesPerBlock) * 256 + lc * 8);
+                    ld[buf][rt][j] = pi_ld_stream(W + (size_t)r * cols + (wave + ss * NW) * 256 + lc * 8);
                 }
         }
     };
@@ -226,7 +225,7 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
             if (cur < n_ss) {
                 pi_u32x4 b[8];
 #pragma unroll
-                for (int st = 0; st < 8; ++st) b[st] = pi_ld16(bp + ((wave + cur * kWavesPerBlock) * 8 + st) * bstep);
+                for (int st = 0; st < 8; ++st) b[st] = pi_ld16(bp + ((wave + cur * NW) * 8 + st) * bstep);
 #pragma unroll
                 for (int rt = 0; rt < RT; ++rt) {
 #pragma unroll
@@ -241,19 +240,22 @@ __global__ __launch_bounds__(kBlock) void gemm_t16_lds_f16_kernel(const __half *
             issue(buf, cur + 2);
         }
     }
+    // the waves' accumulator tiles meet in LDS, each in the front of its wave's own (now idle) staging buffer
+    auto cs = [&](int w, int r, int c) -> float & { return reinterpret_cast<float *>(tile[w])[r * 17 + c]; };
     const int rr = threadIdx.x >> 4, t = threadIdx.x & 15;
 #pragma unroll
     for (int rt = 0; rt < RT; ++rt) {
         if (rt > 0) __syncthreads();
 #pragma unroll
-        for (int r = 0; r < 4; ++r) cs[wave][4 * g + r][i] = acc[rt][r];
+        for (int r = 0; r < 4; ++r) cs(wave, 4 * g + r, i) = acc[rt][r];
         __syncthreads();
+        if (threadIdx.x >= 256) continue;         // 16 rows x 16 tokens: the first four waves write the tile out
         const int row = row0 + rt * 16 + rr;
         bool act = false;
         if (row < rows && t < T) {
-            float sum = cs[0][rr][t];
+            float sum = cs(0, rr, t);
 #pragma unroll
-            for (int w = 1; w < kWavesPerBlock; ++w) sum += cs[w][rr][t];
+            for (int w = 1; w < NW; ++w) sum += cs(w, rr, t);
             const size_t o = (size_t)t * rows + row;
             if (epi == PI_EPI_RELU) sum = fmaxf(sum, 0.0f);
             else if (epi == PI_EPI_ADD) sum = __fadd_rn(sum, add1[o]);
@@ -1082,9 +1084,16 @@ static int gemm_launch(const char * who, const void * W, int rows, int cols, con
     const int rt = rows >= 16384 ? 4 : rows >= 5120 ? 2 : 1;      // (two tiles already at 5120 rows: the activations, re-read per row tile, are what limits one tile per wave)
 #define PI_GEMM_T16(RT) hipLaunchKernelGGL((gemm_t16_f16_kernel<RT>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(kBlock), 0, (hipStream_t)stream, \
                        (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any, lay)
-#define PI_GEMM_LDS(RT) hipLaunchKernelGGL((gemm_t16_lds_f16_kernel<RT>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(kBlock), 0, (hipStream_t)stream, \
+#define PI_GEMM_LDS(RT, NW) hipLaunchKernelGGL((gemm_t16_lds_f16_kernel<RT, NW>), dim3((rows + 16 * RT - 1) / (16 * RT)), dim3(64 * NW), 0, (hipStream_t)stream, \
                        (const __half *)W, (const __half *)xn_f16, T, rows, cols, epilogue, add1, add2, y, (__half *)y_f16, thr, row_any, lay)
-    if (cols % 256 == 0) { if (rt >= 2) PI_GEMM_LDS(2); else PI_GEMM_LDS(1); }
+    if (cols % 256 == 0) {
+        // waves per workgroup: when every workgroup has a compute unit to itself (at most one per unit), eight waves keep twice
+        // the loads in flight per unit; with more workgroups than units the chip is full with four
+        const int rtl = rt >= 2 ? 2 : 1;
+        const bool wide = (rows + 16 * rtl - 1) / (16 * rtl) <= pi::compute_units();
+        if (rtl == 2) { if (wide) PI_GEMM_LDS(2, 8); else PI_GEMM_LDS(2, 4); }
+        else { if (wide) PI_GEMM_LDS(1, 8); else PI_GEMM_LDS(1, 4); }
+    }
     else if (rt == 4) PI_GEMM_T16(4); else if (rt == 2) PI_GEMM_T16(2); else PI_GEMM_T16(1);
 #undef PI_GEMM_LDS
 #undef PI_GEMM_T16

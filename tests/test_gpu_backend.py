@@ -126,7 +126,10 @@ def test_full_gpu_graph_13b_step_of_16():
     o = ol.ffn_sparse(ol.oracle(), d, ff, r, T, ol.F16, True, L["up"], L["gate"], L["down_t"], L["fc1"], L["fc2"], L["x"], L["x"],
                       np.zeros(ff, np.int32), 0.0, nth=8)
     lg = G.host(idx)
-    assert rel_err(lg, o["logits"]) < 1e-5
+    # fp32 sums of 5120 products in another order than the oracle's, then the fp16 rounding of the hidden vector: a hidden value that
+    # falls on the other side of a rounding boundary moves a logit by 2^-11 of one term; the largest of the 221 184 logits' errors
+    # comes out at 0.9e-5 to 1.1e-5 of the largest logit, whichever way the columns are split over the waves
+    assert rel_err(lg, o["logits"]) < 2e-5
     assert ((lg >= 0) == (o["logits"] >= 0)).mean() >= 0.999
     assert rel_err(G.host(out), out_under(L, ol.F16, True, L["x"], lg)) < 1e-4
     per_token = ((lg >= 0).sum(1))

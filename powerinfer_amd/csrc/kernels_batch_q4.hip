@@ -174,25 +174,29 @@ __global__ __launch_bounds__(kBlock) void gemm_q4_t16_kernel(const uint32_t * __
             }
         }
     };
-    // A wave's groups (wave, wave + 4, ...) go in rounds of four: all loads of a round are issued before its first multiply, so
-    // a row of 4096 columns costs one trip to memory per wave instead of four; the first round's loads are already under way
-    // while the workgroup stages the scales.
-    constexpr int kRound = 2;
-    Loads L[kRound];
-#pragma unroll
-    for (int u = 0; u < kRound; ++u) if (wave + u * kWavesPerBlock < ngroups) fetch(L[u], wave + u * kWavesPerBlock);
+    // A wave's groups (wave, wave + 4, ...) pass through two register buffers: a buffer is requested again as soon as it has been
+    // multiplied, so one group is always on its way while the other is multiplied.  Every load of the loop is unconditional (a
+    // request behind the wave's last group reads that group again and is not used), which lets the waits be exact counts instead
+    // of waits for everything in flight; the first two groups are already under way while the workgroup stages the scales.
+    const int my_n = (ngroups - wave + kWavesPerBlock - 1) / kWavesPerBlock;          // groups of this wave (0 for a wave behind a short row's end)
+    auto grp_of = [&](int k) { return wave + (k < my_n ? k : my_n - 1) * kWavesPerBlock; };
+    Loads L0, L1;
+    if (my_n > 0) { fetch(L0, grp_of(0)); fetch(L1, grp_of(1)); }
     for (int k = threadIdx.x; k < nblk * 4; k += kBlock) {
         reinterpret_cast<pi_u32x4 *>(sdx)[k] = pi_ld16(dx + (size_t)k * 4);
         reinterpret_cast<pi_u32x4 *>(ssx)[k] = pi_ld16(sx8 + (size_t)k * 4);
     }
     __syncthreads();
-    for (int g0 = wave; g0 < ngroups; g0 += kRound * kWavesPerBlock) {
-        if (g0 != wave) {
-#pragma unroll
-            for (int u = 0; u < kRound; ++u) if (g0 + u * kWavesPerBlock < ngroups) fetch(L[u], g0 + u * kWavesPerBlock);
+    if (my_n > 0) {
+        int k = 0;
+        for (; k + 2 < my_n; k += 2) {
+            multiply(L0, grp_of(k));
+            fetch(L0, grp_of(k + 2));
+            multiply(L1, grp_of(k + 1));
+            fetch(L1, grp_of(k + 3));
         }
-#pragma unroll
-        for (int u = 0; u < kRound; ++u) if (g0 + u * kWavesPerBlock < ngroups) multiply(L[u], g0 + u * kWavesPerBlock);
+        multiply(L0, grp_of(k));
+        if (k + 1 < my_n) multiply(L1, grp_of(k + 1));
     }
 #pragma unroll
     for (int m = 0; m < NM; ++m)

@@ -1022,7 +1022,32 @@ __global__ __launch_bounds__(1024) void argmax_batch_kernel(const float * __rest
     const int t = blockIdx.x;
     const float * lg = logits + (size_t)t * n;
     float best = -INFINITY; int idx = 0x7fffffff;
-    for (int i = threadIdx.x; i < n; i += blockDim.x) { const float v = lg[i]; if (v > best) { best = v; idx = i; } }
+    if (n % 4 == 0 && ((uintptr_t)lg & 15) == 0) {
+        // eight 16-byte loads per thread requested together (a row of 32 000 logits is one such round: one trip to memory instead
+        // of one per element); a thread's indices ascend, so the strict comparison keeps its first maximum
+        const float4 * lg4 = reinterpret_cast<const float4 *>(lg);
+        const int n4 = n / 4;
+        for (int i0 = threadIdx.x; i0 < n4; i0 += 8 * (int)blockDim.x) {
+            float4 v[8];
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int i4 = i0 + u * (int)blockDim.x;
+                v[u] = lg4[i4 < n4 ? i4 : n4 - 1];
+            }
+#pragma unroll
+            for (int u = 0; u < 8; ++u) {
+                const int i4 = i0 + u * (int)blockDim.x;
+                if (i4 < n4) {
+                    if (v[u].x > best) { best = v[u].x; idx = 4 * i4; }
+                    if (v[u].y > best) { best = v[u].y; idx = 4 * i4 + 1; }
+                    if (v[u].z > best) { best = v[u].z; idx = 4 * i4 + 2; }
+                    if (v[u].w > best) { best = v[u].w; idx = 4 * i4 + 3; }
+                }
+            }
+        }
+    } else {
+        for (int i = threadIdx.x; i < n; i += blockDim.x) { const float v = lg[i]; if (v > best) { best = v; idx = i; } }
+    }
     for (int o = 32; o > 0; o >>= 1) {
         const float ov = __shfl_xor(best, o, PI_WAVE); const int oi = __shfl_xor(idx, o, PI_WAVE);
         if (ov > best || (ov == best && oi < idx)) { best = ov; idx = oi; }

@@ -1046,3 +1046,31 @@ def test_wide_prompt_chunks_of_q4_and_hybrid_models(name, wtype, hot_frac, kw, n
     assert rel_err(lg_a, lg_b) < (5e-2 if q4 else 1e-2), rel_err(lg_a, lg_b)
     assert not np.array_equal(lg_a, lg_b)                     # identical bits would mean the chunk route did not run
     ga.close(), gb.close()
+
+
+@pytest.mark.parametrize("n", [32000, 32001, 1000, 7])
+def test_argmax_batch_takes_the_first_maximum(n):
+    """pi_k_argmax_batch against numpy's argmax (the first maximum wins, as the greedy sampler's loop does, llama.cpp:8617-8631): ties
+    inside one thread's 16-byte load, across threads and across waves, a row of -inf (token 0), a row with NaNs (never greater),
+    row widths that take the 16-byte path (n % 4 == 0) and the element-wise one; positions advance, the step's tokens are recorded."""
+    from powerinfer_amd import lib as pl
+    L = pl.init()
+    T = 16
+    rng = np.random.default_rng(n)
+    lg = rng.standard_normal((T, n)).astype(np.float32)
+    lg[1, :] = 0.25                                                  # every element ties: token 0
+    lg[2, [n - 1, n // 2, 3 % n]] = 9.0                                # ties far apart: the lowest index
+    lg[3, min(5, n - 1)] = 9.0; lg[3, min(6, n - 1)] = 9.0           # ties within one 16-byte load
+    lg[4, :] = -np.inf                                                # nothing compares greater: token 0
+    lg[5, ::3] = np.nan                                               # NaNs never win
+    lg[6, n - 1] = 50.0                                               # the last element
+    want = np.array([int(np.nanargmax(np.where(np.isnan(r), -np.inf, r))) if np.isfinite(r[~np.isnan(r)]).any() else 0 for r in lg], np.int32)
+    dl, dt = pl.DevBuf(host=lg), pl.DevBuf(T * 4)
+    dp, ds, do = pl.DevBuf(host=np.arange(T, dtype=np.int32)), pl.DevBuf(host=np.array([1], np.int32)), pl.DevBuf(host=np.full(3 * T, -1, np.int32))
+    pl.check(L.pi_k_argmax_batch(dl.ptr, n, T, dt.ptr, dp.ptr, ds.ptr, do.ptr, 3, None), "argmax")
+    pl.sync()
+    got = dt.download(np.int32)
+    assert np.array_equal(got, want), (got, want)
+    assert np.array_equal(dp.download(np.int32), np.arange(T) + 1)
+    rec = do.download(np.int32).reshape(3, T)
+    assert np.array_equal(rec[1], want) and np.all(rec[0] == -1) and np.all(rec[2] == -1)

@@ -994,16 +994,26 @@ __global__ __launch_bounds__(kBlock) void batch_reduce_kernel(const float * __re
     const int t = idx / cols, c = idx - t * cols;
     const size_t gstride = (size_t)kBtMaxT * cols;
     const float * p = partial + (size_t)t * cols + c;
+    // the residual operands are requested with the first partial sums, and 16 partial sums travel together: two trips to memory
+    // for 32 groups (the sums are added in group order whatever the batching)
+    float4 a1 = make_float4(0.0f, 0.0f, 0.0f, 0.0f), a2 = a1;
+    if (epi >= PI_EPI_ADD) a1 = *reinterpret_cast<const float4 *>(add1 + idx);
+    if (epi == PI_EPI_ADD2) a2 = *reinterpret_cast<const float4 *>(add2 + idx);
     float4 sum = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-    for (int g0 = 0; g0 < n_groups; g0 += 8) {
-        float4 v[8];
+    int g0 = 0;
+    for (; g0 + 16 <= n_groups; g0 += 16) {
+        float4 v[16];
 #pragma unroll
-        for (int j = 0; j < 8; ++j) v[j] = g0 + j < n_groups ? *reinterpret_cast<const float4 *>(p + (size_t)(g0 + j) * gstride) : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        for (int j = 0; j < 16; ++j) v[j] = *reinterpret_cast<const float4 *>(p + (size_t)(g0 + j) * gstride);
 #pragma unroll
-        for (int j = 0; j < 8; ++j) { sum.x += v[j].x; sum.y += v[j].y; sum.z += v[j].z; sum.w += v[j].w; }
+        for (int j = 0; j < 16; ++j) { sum.x += v[j].x; sum.y += v[j].y; sum.z += v[j].z; sum.w += v[j].w; }
     }
-    if (epi >= PI_EPI_ADD) { const float4 a = *reinterpret_cast<const float4 *>(add1 + idx); sum.x = __fadd_rn(sum.x, a.x); sum.y = __fadd_rn(sum.y, a.y); sum.z = __fadd_rn(sum.z, a.z); sum.w = __fadd_rn(sum.w, a.w); }
-    if (epi == PI_EPI_ADD2) { const float4 a = *reinterpret_cast<const float4 *>(add2 + idx); sum.x = __fadd_rn(sum.x, a.x); sum.y = __fadd_rn(sum.y, a.y); sum.z = __fadd_rn(sum.z, a.z); sum.w = __fadd_rn(sum.w, a.w); }
+    for (; g0 < n_groups; ++g0) {
+        const float4 v = *reinterpret_cast<const float4 *>(p + (size_t)g0 * gstride);
+        sum.x += v.x; sum.y += v.y; sum.z += v.z; sum.w += v.w;
+    }
+    if (epi >= PI_EPI_ADD) { sum.x = __fadd_rn(sum.x, a1.x); sum.y = __fadd_rn(sum.y, a1.y); sum.z = __fadd_rn(sum.z, a1.z); sum.w = __fadd_rn(sum.w, a1.w); }
+    if (epi == PI_EPI_ADD2) { sum.x = __fadd_rn(sum.x, a2.x); sum.y = __fadd_rn(sum.y, a2.y); sum.z = __fadd_rn(sum.z, a2.z); sum.w = __fadd_rn(sum.w, a2.w); }
     *reinterpret_cast<float4 *>(out + idx) = sum;
 }
 

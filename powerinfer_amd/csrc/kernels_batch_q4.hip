@@ -252,7 +252,10 @@ __global__ __launch_bounds__(256) void h_q8_values_kernel(const float * __restri
                                                           float * __restrict__ hq) {
     const int blk = (int)blockIdx.x * 8 + (threadIdx.x >> 5), t = blockIdx.y, n = blk * 32 + (threadIdx.x & 31);
     const bool in = n < ff;
-    float v = (in && row_any[n]) ? h[(size_t)t * ff + n] : 0.0f;
+    // both operands requested at once (a neuron outside the union holds a stale h, which the flag deselects): one trip to memory
+    const float hv = in ? h[(size_t)t * ff + n] : 0.0f;
+    const unsigned char any = in ? row_any[n] : (unsigned char)0;
+    float v = any ? hv : 0.0f;
     float amax = fabsf(v);
 #pragma unroll
     for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, PI_WAVE));

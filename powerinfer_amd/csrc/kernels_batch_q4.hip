@@ -115,13 +115,21 @@ __global__ __launch_bounds__(kBlock) void gemm_q4_t16_kernel(const uint32_t * __
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63, i = lane & 15, g = lane >> 4;
     const int cols = nblk * 32;
     int nu = rows;
-    if (SPARSE) { nu = *n_union; if ((int)blockIdx.x * 16 >= nu) return; }
+    // SPARSE: the list entry of this lane is requested together with the list's length (the list has one entry per row of the
+    // matrix, so the address is good whatever the length; an entry behind the end is stale and is replaced by the last one)
+    int listed = 0;
+    if (SPARSE) {
+        listed = union_rows[(int)blockIdx.x * 16 + i];
+        nu = *n_union;
+        if ((int)blockIdx.x * 16 >= nu) return;
+        if ((int)blockIdx.x * 16 + i >= nu) listed = union_rows[nu - 1];
+    }
     size_t wrow[NM];
     int my_row[NM];
 #pragma unroll
     for (int m = 0; m < NM; ++m) {
         int r = SPARSE ? (int)blockIdx.x * 16 + i : ((int)blockIdx.x * RT + m) * 16 + i;
-        if (SPARSE) r = union_rows[r < nu ? r : nu - 1];
+        if (SPARSE) r = listed;
         else r = r < rows ? r : rows - 1;
         my_row[m] = r;
         wrow[m] = (size_t)r * nblk;

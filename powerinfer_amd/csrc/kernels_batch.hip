@@ -936,20 +936,30 @@ __global__ __launch_bounds__(kBlock) void batch_axpy_mfma_f16_kernel(const __hal
     const int my_steps = (n_steps - (int)blockIdx.y + G - 1) / G;                           // steps blockIdx.y, + G, ... of this group
     pi_u32x4 ld[NB][8];
     pi_u32x2 af[NB];
+    // the 16 row numbers of the NEXT step to be requested (steps are requested in order): they are asked for right behind a step's
+    // weight loads and have arrived when the next step's addresses are made, instead of holding every request up for a trip of
+    // their own
+    int rn[16];
+    auto fetch_rows = [&](int s) {
+        const int u0 = ((int)blockIdx.y + (s < my_steps ? s : my_steps - 1) * G) * 16;
+#pragma unroll
+        for (int k = 0; k < 16; ++k) rn[k] = list[u0 + k < n ? u0 + k : n - 1];
+    };
     auto issue = [&](int buf, int s) {
         const int u0 = ((int)blockIdx.y + (s < my_steps ? s : my_steps - 1) * G) * 16;
 #pragma unroll
         for (int r = 0; r < 4; ++r) {
-            // (readfirstlane pins the four loads to the scalar unit, ahead of the select)
-            const int r0 = __builtin_amdgcn_readfirstlane(list[u0 + r < n ? u0 + r : n - 1]);
-            const int r1 = __builtin_amdgcn_readfirstlane(list[u0 + 4 + r < n ? u0 + 4 + r : n - 1]);
-            const int r2 = __builtin_amdgcn_readfirstlane(list[u0 + 8 + r < n ? u0 + 8 + r : n - 1]);
-            const int r3 = __builtin_amdgcn_readfirstlane(list[u0 + 12 + r < n ? u0 + 12 + r : n - 1]);
+            // (readfirstlane keeps the row numbers on the scalar unit, ahead of the select)
+            const int r0 = __builtin_amdgcn_readfirstlane(rn[r]);
+            const int r1 = __builtin_amdgcn_readfirstlane(rn[4 + r]);
+            const int r2 = __builtin_amdgcn_readfirstlane(rn[8 + r]);
+            const int r3 = __builtin_amdgcn_readfirstlane(rn[12 + r]);
             const __half * wp = Wd + (size_t)(g == 0 ? r0 : g == 1 ? r1 : g == 2 ? r2 : r3) * cols + c0 + 8 * i;
             ld[buf][2 * r]     = pi_ld_stream(wp);
             ld[buf][2 * r + 1] = pi_ld_stream(wp + 128);
         }
         af[buf] = *reinterpret_cast<const pi_u32x2 *>(hc + (size_t)i * hstride + u0 + 4 * g);      // zeros beyond n (written by the gate/up kernel)
+        fetch_rows(s + 1);
     };
     auto consume = [&](int buf) {
         const pi_h4 a = __builtin_bit_cast(pi_h4, af[buf]);
@@ -965,6 +975,7 @@ __global__ __launch_bounds__(kBlock) void batch_axpy_mfma_f16_kernel(const __hal
             }
     };
     if (my_steps > 0) {
+        fetch_rows(0);
 #pragma unroll
         for (int buf = 0; buf < NB; ++buf) issue(buf, buf);
         int s = 0;
